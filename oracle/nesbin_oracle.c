@@ -1,0 +1,144 @@
+/*
+ * TEST INFRASTRUCTURE ONLY.  CPU oracle for the packed binary forward path of
+ * jamesal1/NESgpu: a plain-C restatement of the reference kernels' arithmetic.
+ * Only tests, the smoke check and the benchmark's cpu_baseline leg load this
+ * library; the product (libnesbin.so) never links or calls it.
+ *
+ * What pins each function (checked by the CPU test-suite):
+ *   pack / unpack        numpy.packbits(bitorder="little") closed form + round trip
+ *   int8pack             numpy little-endian byte view of a zero-padded row
+ *   im2col               independent numpy gather over unpacked, explicitly padded bits
+ *   bmm / bmm_act        integer matmul on +-1 values: 2*popc - K == a.(-b)
+ *                        (booloptests.py:150-160) and brute force on bits
+ *   conv / conv_act      grouped torch.conv2d on +-1 with pad value -1 and
+ *                        sign-inverted filters (booloptests.py:150-155,157-160)
+ *   max_pool2d           pack(F.max_pool2d(bits)) for 2x2/s2 (booloptests.py:94-95,138-141)
+ *                        and an OR-of-window brute force for padded cases
+ *   sample_from_words    numpy (words < thresh) + packbits; rate check mean ~= p
+ *   seeded_bmv           must equal bmm(sample_from_words(...), x)
+ *   philox4x32_10        Random123 known-answer vectors and rocRAND's host engine
+ *   weighted_sum         float64 numpy einsum over unpacked bits (tolerance)
+ * The cuRAND XORWOW stream of the reference samplers (sample_bits.cu:23-25,54) is NOT
+ * reproduced anywhere: parity unpinned for that stream; supplied-word parity replaces it.
+ *
+ * Build: make -C oracle   (gcc -O2 -fopenmp, see Makefile)
+ */
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+#define CAT_(a, b) a##b
+#define CAT(a, b) CAT_(a, b)
+
+#define WORD uint64_t
+#define WBITS 64
+#define POPC(x) __builtin_popcountll(x)
+#define FN(x) CAT(x, _i64)
+#include "nesbin_oracle_impl.h"
+#undef WORD
+#undef WBITS
+#undef POPC
+#undef FN
+
+#define WORD uint32_t
+#define WBITS 32
+#define POPC(x) __builtin_popcount(x)
+#define FN(x) CAT(x, _i32)
+#include "nesbin_oracle_impl.h"
+#undef WORD
+#undef WBITS
+#undef POPC
+#undef FN
+
+/* booleanOperations.py:162-166 -- conv = bmm(im2col(input), filter); filter is
+ * [D, fx*fy*Cw, O] (modules/binary.py:136-137).  Done one member at a time so the
+ * column buffer stays small.  out is [D, h, w, O] int32. */
+#define DEFINE_CONV(SUF, WORD_T)                                                                   \
+    void nbo_conv_##SUF(int32_t *out, const WORD_T *in, const WORD_T *filt, int64_t D, int64_t H,  \
+                        int64_t W, int64_t Cw, int64_t O, int fx, int fy, int px, int py, int sx,  \
+                        int sy)                                                                    \
+    {                                                                                              \
+        const int64_t h = (H - fx + 2 * px) / sx + 1, w = (W - fy + 2 * py) / sy + 1;              \
+        const int64_t K = (int64_t)fx * fy * Cw;                                                   \
+        _Pragma("omp parallel")                                                                    \
+        {                                                                                          \
+            WORD_T *cols = (WORD_T *)malloc(sizeof(WORD_T) * (size_t)(h * w * K + 1));             \
+            _Pragma("omp for schedule(static)")                                                    \
+            for (int64_t d = 0; d < D; d++) {                                                      \
+                nbo_im2col_##SUF(cols, in + d * H * W * Cw, 1, H, W, Cw, fx, fy, px, py, sx, sy);  \
+                nbo_bmm_##SUF(out + d * h * w * O, cols, filt + d * K * O, 1, h * w, K, O);        \
+            }                                                                                      \
+            free(cols);                                                                            \
+        }                                                                                          \
+    }                                                                                              \
+    /* booleanOperations.py:168-172 -- conv_act = bmm_act(im2col(input), filter, thresh). */       \
+    void nbo_conv_act_##SUF(uint8_t *out, const WORD_T *in, const WORD_T *filt,                    \
+                            const int32_t *thresh, int64_t D, int64_t H, int64_t W, int64_t Cw,    \
+                            int64_t O, int fx, int fy, int px, int py, int sx, int sy)             \
+    {                                                                                              \
+        const int64_t h = (H - fx + 2 * px) / sx + 1, w = (W - fy + 2 * py) / sy + 1;              \
+        const int64_t K = (int64_t)fx * fy * Cw;                                                   \
+        _Pragma("omp parallel")                                                                    \
+        {                                                                                          \
+            WORD_T *cols = (WORD_T *)malloc(sizeof(WORD_T) * (size_t)(h * w * K + 1));             \
+            _Pragma("omp for schedule(static)")                                                    \
+            for (int64_t d = 0; d < D; d++) {                                                      \
+                nbo_im2col_##SUF(cols, in + d * H * W * Cw, 1, H, W, Cw, fx, fy, px, py, sx, sy);  \
+                nbo_bmm_act_##SUF(out + d * h * w * O, cols, filt + d * K * O, thresh + d * O, 1,  \
+                                  h * w, K, O);                                                    \
+            }                                                                                      \
+            free(cols);                                                                            \
+        }                                                                                          \
+    }
+
+DEFINE_CONV(i64, uint64_t)
+DEFINE_CONV(i32, uint32_t)
+
+/* Philox4x32-10 (Salmon, Moraes, Dror, Shaw: "Parallel random numbers: as easy as 1, 2, 3",
+ * SC'11).  Not part of the reference (it draws from cuRAND XORWOW, sample_bits.cu:23-25);
+ * this is the generator the replacement uses when the random words are not supplied.
+ * ctr[4], key[2] -> out[4]. */
+void nbo_philox4x32_10(uint32_t out[4], const uint32_t ctr[4], const uint32_t key[2])
+{
+    uint32_t c0 = ctr[0], c1 = ctr[1], c2 = ctr[2], c3 = ctr[3];
+    uint32_t k0 = key[0], k1 = key[1];
+    for (int r = 0; r < 10; r++) {
+        const uint64_t p0 = (uint64_t)0xD2511F53u * c0;
+        const uint64_t p1 = (uint64_t)0xCD9E8D57u * c2;
+        const uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0;
+        const uint32_t n1 = (uint32_t)p1;
+        const uint32_t n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1;
+        const uint32_t n3 = (uint32_t)p0;
+        c0 = n0; c1 = n1; c2 = n2; c3 = n3;
+        k0 += 0x9E3779B9u;
+        k1 += 0xBB67AE85u;
+    }
+    out[0] = c0; out[1] = c1; out[2] = c2; out[3] = c3;
+}
+
+/* The word stream the replacement's generator mode defines: word number g (a flat index into
+ * the [n, R, C] draw tensor, plus first) is lane g%4 of the Philox block with counter
+ * (lo32(g/4), hi32(g/4), lo32(subseq), hi32(subseq)) and key (lo32(seed), hi32(seed)). */
+void nbo_philox_words(uint32_t *out, uint64_t seed, uint64_t subseq, uint64_t first, int64_t count)
+{
+    const uint32_t key[2] = {(uint32_t)seed, (uint32_t)(seed >> 32)};
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < count; i++) {
+        const uint64_t g = first + (uint64_t)i;
+        const uint64_t blk = g >> 2;
+        const uint32_t ctr[4] = {(uint32_t)blk, (uint32_t)(blk >> 32), (uint32_t)subseq,
+                                 (uint32_t)(subseq >> 32)};
+        uint32_t o[4];
+        nbo_philox4x32_10(o, ctr, key);
+        out[i] = o[g & 3];
+    }
+}
+
+#ifdef _OPENMP
+#include <omp.h>
+int nbo_max_threads(void) { return omp_get_max_threads(); }
+void nbo_set_threads(int n) { omp_set_num_threads(n); }
+#else
+int nbo_max_threads(void) { return 1; }
+void nbo_set_threads(int n) { (void)n; }
+#endif

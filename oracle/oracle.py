@@ -1,0 +1,227 @@
+"""TEST INFRASTRUCTURE ONLY: numpy front-end of the C oracle (``libnesbin_oracle.so``).
+
+Only tests, ``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of ``bench.py`` may import
+this module.  Every function takes and returns numpy arrays; packed words are ``int64`` or
+``int32`` arrays holding the bit patterns (LSB-first, extensions/src/pack.cu:26).
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB = None
+
+
+def build(force=False):
+    """Compile the oracle with gcc (a few hundred ms)."""
+    so = os.path.join(_HERE, "libnesbin_oracle.so")
+    if force or not os.path.exists(so):
+        subprocess.check_call(["make", "-C", _HERE, "-B" if force else "-s", "libnesbin_oracle.so"])
+    return so
+
+
+def lib():
+    global _LIB
+    if _LIB is None:
+        name = os.environ.get("NESBIN_ORACLE_LIB") or build()
+        _LIB = ctypes.CDLL(name)
+    return _LIB
+
+
+def _suf(dtype):
+    dtype = np.dtype(dtype)
+    if dtype == np.int64 or dtype == np.uint64:
+        return "i64", 64, np.int64
+    if dtype == np.int32 or dtype == np.uint32:
+        return "i32", 32, np.int32
+    raise TypeError("word dtype must be int64 or int32, got %r" % (dtype,))
+
+
+def _p(a):
+    return ctypes.c_void_p(a.ctypes.data) if a is not None else ctypes.c_void_p(0)
+
+
+def _c(a, dtype=None):
+    a = np.ascontiguousarray(a) if dtype is None else np.ascontiguousarray(a, dtype=dtype)
+    return a
+
+
+def _i64(v):
+    return ctypes.c_int64(int(v))
+
+
+def out_hw(H, W, fx, fy, px, py, sx, sy):
+    """Output size formula of booleanOperations.py:83-84."""
+    return (H - fx + 2 * px) // sx + 1, (W - fy + 2 * py) // sy + 1
+
+
+def pack(bits, dtype=np.int64):
+    suf, wb, wt = _suf(dtype)
+    bits = _c(bits).view(np.uint8)
+    R, C = bits.shape
+    out = np.empty((R, (C + wb - 1) // wb), dtype=wt)
+    getattr(lib(), "nbo_pack_" + suf)(_p(out), _p(bits), _i64(R), _i64(C))
+    return out
+
+
+def unpack(words):
+    suf, wb, _ = _suf(words.dtype)
+    words = _c(words)
+    R, Rw = words.shape
+    out = np.empty((R, Rw * wb), dtype=np.uint8)
+    getattr(lib(), "nbo_unpack_" + suf)(_p(out), _p(words), _i64(R), _i64(Rw))
+    return out.view(np.bool_)
+
+
+def int8pack(data, dtype=np.int64):
+    suf, wb, wt = _suf(dtype)
+    data = _c(data, np.uint8)
+    R, C = data.shape
+    per = wb // 8
+    out = np.empty((R, (C + per - 1) // per), dtype=wt)
+    getattr(lib(), "nbo_int8pack_" + suf)(_p(out), _p(data), _i64(R), _i64(C))
+    return out
+
+
+def batch_im2col(x, fx, fy, px, py, sx, sy):
+    suf, _, wt = _suf(x.dtype)
+    x = _c(x)
+    B, H, W, Cw = x.shape
+    h, w = out_hw(H, W, fx, fy, px, py, sx, sy)
+    out = np.empty((B, h * w, fx * fy * Cw), dtype=wt)
+    getattr(lib(), "nbo_im2col_" + suf)(_p(out), _p(x), _i64(B), _i64(H), _i64(W), _i64(Cw),
+                                         fx, fy, px, py, sx, sy)
+    return out
+
+
+def bmm(A, B):
+    suf, _, _ = _suf(A.dtype)
+    A, B = _c(A), _c(B)
+    assert A.dtype == B.dtype and A.ndim == 3 and B.ndim == 3
+    Z, M, K = A.shape
+    assert B.shape[0] == Z and B.shape[1] == K
+    N = B.shape[2]
+    out = np.empty((Z, M, N), dtype=np.int32)
+    getattr(lib(), "nbo_bmm_" + suf)(_p(out), _p(A), _p(B), _i64(Z), _i64(M), _i64(K), _i64(N))
+    return out
+
+
+def bmm_act(A, B, thresh):
+    suf, _, _ = _suf(A.dtype)
+    A, B, thresh = _c(A), _c(B), _c(thresh, np.int32)
+    Z, M, K = A.shape
+    N = B.shape[2]
+    assert thresh.shape == (Z, N)
+    out = np.empty((Z, M, N), dtype=np.uint8)
+    getattr(lib(), "nbo_bmm_act_" + suf)(_p(out), _p(A), _p(B), _p(thresh), _i64(Z), _i64(M), _i64(K), _i64(N))
+    return out.view(np.bool_)
+
+
+def conv(x, filt, fx, fy, px, py, sx, sy):
+    suf, _, _ = _suf(x.dtype)
+    x, filt = _c(x), _c(filt)
+    D, H, W, Cw = x.shape
+    O = filt.shape[2]
+    assert filt.shape[:2] == (D, fx * fy * Cw) and filt.dtype == x.dtype
+    h, w = out_hw(H, W, fx, fy, px, py, sx, sy)
+    out = np.empty((D, h, w, O), dtype=np.int32)
+    getattr(lib(), "nbo_conv_" + suf)(_p(out), _p(x), _p(filt), _i64(D), _i64(H), _i64(W), _i64(Cw), _i64(O),
+                                       fx, fy, px, py, sx, sy)
+    return out
+
+
+def conv_act(x, filt, thresh, fx, fy, px, py, sx, sy):
+    suf, _, _ = _suf(x.dtype)
+    x, filt, thresh = _c(x), _c(filt), _c(thresh, np.int32)
+    D, H, W, Cw = x.shape
+    O = filt.shape[2]
+    h, w = out_hw(H, W, fx, fy, px, py, sx, sy)
+    out = np.empty((D, h, w, O), dtype=np.uint8)
+    getattr(lib(), "nbo_conv_act_" + suf)(_p(out), _p(x), _p(filt), _p(thresh), _i64(D), _i64(H), _i64(W),
+                                           _i64(Cw), _i64(O), fx, fy, px, py, sx, sy)
+    return out.view(np.bool_)
+
+
+def max_pool2d(x, fx, fy, px, py, sx, sy):
+    suf, _, wt = _suf(x.dtype)
+    x = _c(x)
+    B, H, W, Cw = x.shape
+    h, w = out_hw(H, W, fx, fy, px, py, sx, sy)
+    out = np.empty((B, h, w, Cw), dtype=wt)
+    getattr(lib(), "nbo_max_pool2d_" + suf)(_p(out), _p(x), _i64(B), _i64(H), _i64(W), _i64(Cw),
+                                             fx, fy, px, py, sx, sy)
+    return out
+
+
+def _thr_args(thresh):
+    if np.isscalar(thresh) or (isinstance(thresh, np.ndarray) and thresh.ndim == 0):
+        return None, ctypes.c_uint32(int(thresh))
+    return _c(thresh, np.uint32), ctypes.c_uint32(0)
+
+
+def sample_from_words(thresh, words, dtype=np.int64, base=None):
+    """bit = words[m,r,c] < thresh[r,c] (or a scalar); optional base [R,Rw] is XORed on."""
+    suf, wb, wt = _suf(dtype)
+    words = _c(words, np.uint32)
+    n, R, C = words.shape
+    tarr, tsc = _thr_args(thresh)
+    if tarr is not None:
+        assert tarr.shape == (R, C)
+    if base is not None:
+        base = _c(base)
+        assert base.dtype == wt and base.shape == (R, (C + wb - 1) // wb)
+    out = np.empty((n, R, (C + wb - 1) // wb), dtype=wt)
+    getattr(lib(), "nbo_sample_from_words_" + suf)(_p(out), _p(base), _p(tarr), tsc, _p(words),
+                                                    _i64(n), _i64(R), _i64(C))
+    return out
+
+
+def seeded_bmv_from_words(thresh, x, words, base=None):
+    suf, wb, wt = _suf(x.dtype)
+    x = _c(x)
+    words = _c(words, np.uint32)
+    n, R, C = words.shape
+    assert x.shape == (n, (C + wb - 1) // wb)
+    tarr, tsc = _thr_args(thresh)
+    if base is not None:
+        base = _c(base)
+        assert base.dtype == wt
+    out = np.empty((n, R), dtype=np.int32)
+    getattr(lib(), "nbo_seeded_bmv_from_words_" + suf)(_p(out), _p(base), _p(tarr), tsc, _p(x), _p(words),
+                                                        _i64(n), _i64(R), _i64(C))
+    return out
+
+
+def weighted_sum(words, w, zbits):
+    suf, _, _ = _suf(words.dtype)
+    words = _c(words)
+    w = _c(w, np.float32)
+    n, R, Rw = words.shape
+    out = np.empty((R, zbits), dtype=np.float32)
+    getattr(lib(), "nbo_weighted_sum_" + suf)(_p(out), _p(words), _p(w), _i64(n), _i64(R), _i64(Rw), _i64(zbits))
+    return out
+
+
+def philox4x32_10(ctr, key):
+    ctr = _c(ctr, np.uint32)
+    key = _c(key, np.uint32)
+    out = np.empty(4, dtype=np.uint32)
+    lib().nbo_philox4x32_10(_p(out), _p(ctr), _p(key))
+    return out
+
+
+def philox_words(seed, subseq, first, count):
+    out = np.empty(int(count), dtype=np.uint32)
+    lib().nbo_philox_words(_p(out), ctypes.c_uint64(int(seed)), ctypes.c_uint64(int(subseq)),
+                           ctypes.c_uint64(int(first)), _i64(count))
+    return out
+
+
+def max_threads():
+    return int(lib().nbo_max_threads())
+
+
+def set_threads(n):
+    lib().nbo_set_threads(int(n))

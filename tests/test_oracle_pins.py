@@ -1,0 +1,249 @@
+"""Pins the C oracle (oracle/nesbin_oracle.c) against independent statements of the same
+arithmetic: numpy.packbits, +-1 integer matmul, torch.conv2d / max_pool2d in the form the
+reference's check script uses (booloptests.py:94-163), brute force and special cases.
+CPU only."""
+import itertools
+
+import numpy as np
+import pytest
+
+from oracle import unpacked as U
+
+WORD_DTYPES = [np.int64, np.int32]
+
+
+def rng(seed):
+    return np.random.default_rng(seed)
+
+
+@pytest.mark.parametrize("dtype", WORD_DTYPES)
+@pytest.mark.parametrize("R,C", [(1, 1), (3, 3), (5, 31), (4, 32), (7, 33), (2, 63), (9, 64), (3, 65),
+                                 (6, 127), (5, 128), (2, 200), (1, 1024), (17, 576)])
+def test_pack_matches_packbits_and_roundtrips(oracle, dtype, R, C):
+    bits = rng(R * 1000 + C).integers(0, 2, size=(R, C)).astype(bool)
+    got = oracle.pack(bits, dtype)
+    assert got.dtype == dtype
+    np.testing.assert_array_equal(got, U.pack_bits(bits, dtype))
+    un = oracle.unpack(got)
+    wb = np.dtype(dtype).itemsize * 8
+    assert un.shape == (R, got.shape[1] * wb)
+    np.testing.assert_array_equal(un[:, :C], bits)
+    assert not un[:, C:].any()                      # zero tail (pack.cu:17)
+    np.testing.assert_array_equal(un, U.unpack_bits(got))
+
+
+def test_pack_bit_order_and_sign_bit(oracle):
+    # bit i of word y is column y*bits+i (pack.cu:26); bit 63 makes the int64 negative
+    bits = np.zeros((1, 128), dtype=bool)
+    bits[0, 0] = True
+    bits[0, 63] = True
+    bits[0, 64 + 5] = True
+    w = oracle.pack(bits, np.int64)
+    assert w[0, 0] == np.int64(-(2 ** 63) + 1)
+    assert w[0, 1] == 32
+    w32 = oracle.pack(bits, np.int32)
+    assert list(w32[0]) == [1, -(2 ** 31), 32, 0]
+
+
+@pytest.mark.parametrize("dtype", WORD_DTYPES)
+def test_int8pack_is_little_endian_view(oracle, dtype):
+    per = np.dtype(dtype).itemsize
+    for R, C in [(3, 1), (2, per), (4, per + 3), (5, 3 * per)]:
+        data = rng(C).integers(0, 256, size=(R, C)).astype(np.uint8)
+        Rw = (C + per - 1) // per
+        padded = np.zeros((R, Rw * per), dtype=np.uint8)
+        padded[:, :C] = data
+        want = padded.view(np.dtype(dtype).newbyteorder("<")).astype(dtype)
+        np.testing.assert_array_equal(oracle.int8pack(data, dtype), want)
+
+
+@pytest.mark.parametrize("dtype", WORD_DTYPES)
+@pytest.mark.parametrize("Z,M,K,N", [(1, 1, 1, 1), (3, 5, 7, 2), (2, 33, 70, 9), (4, 16, 64, 1), (2, 1, 130, 35),
+                                     (5, 9, 200, 3)])
+def test_bmm_matches_pm1_matmul(oracle, dtype, Z, M, K, N):
+    g = rng(Z + 10 * M + 100 * K + N)
+    a = g.integers(0, 2, size=(Z, M, K)).astype(bool)
+    b = g.integers(0, 2, size=(Z, K, N)).astype(bool)
+    A = U.pack_bits(a.reshape(Z * M, K), dtype).reshape(Z, M, -1)
+    # B is [Z, Kw, N]: pack along K for every (z, n), then put N last
+    Bp = U.pack_bits(b.transpose(0, 2, 1).reshape(Z * N, K), dtype).reshape(Z, N, -1).transpose(0, 2, 1)
+    got = oracle.bmm(A, np.ascontiguousarray(Bp))
+    want = U.popc_bmm_bits(a, b)
+    np.testing.assert_array_equal(got, want)
+    # brute force: number of differing positions
+    brute = (a[:, :, :, None] != b[:, None, :, :]).sum(axis=2).astype(np.int32)
+    np.testing.assert_array_equal(got, brute)
+
+
+@pytest.mark.parametrize("dtype", WORD_DTYPES)
+def test_bmm_special_cases(oracle, dtype):
+    wb = np.dtype(dtype).itemsize * 8
+    g = rng(7)
+    K = 2 * wb + 5
+    a = g.integers(0, 2, size=(3, 6, K)).astype(bool)
+    A = U.pack_bits(a.reshape(18, K), dtype).reshape(3, 6, -1)
+    Kw = A.shape[2]
+    zeros = np.zeros((3, Kw, 4), dtype=dtype)
+    # B == 0: popc counts the ones of A
+    np.testing.assert_array_equal(oracle.bmm(A, zeros), np.repeat(a.sum(2)[:, :, None], 4, axis=2))
+    # A == B: 0 ; B == ~A on the valid bits: K
+    same = np.ascontiguousarray(A[:, 2:3, :].transpose(0, 2, 1))
+    assert np.all(oracle.bmm(A[:, 2:3, :], same) == 0)
+    inv = U.pack_bits(~a.reshape(18, K), dtype).reshape(3, 6, -1)
+    invb = np.ascontiguousarray(inv[:, 2:3, :].transpose(0, 2, 1))
+    assert np.all(oracle.bmm(A[:, 2:3, :], invb) == K)
+    # all-ones words against zero: full word width per word (bit 63 / sign bit counted)
+    ones = np.full((1, 1, 3), -1, dtype=dtype)
+    assert oracle.bmm(ones, np.zeros((1, 3, 1), dtype=dtype))[0, 0, 0] == 3 * wb
+
+
+@pytest.mark.parametrize("dtype", WORD_DTYPES)
+def test_bmm_act_is_threshold_of_bmm(oracle, dtype):
+    g = rng(11)
+    Z, M, K, N = 3, 10, 150, 7
+    A = g.integers(-2 ** 31, 2 ** 31, size=(Z, M, 3)).astype(dtype)
+    B = g.integers(-2 ** 31, 2 ** 31, size=(Z, 3, N)).astype(dtype)
+    popc = oracle.bmm(A, B)
+    thr = (g.integers(0, 2 * popc.max() + 3, size=(Z, N)) - 1).astype(np.int32)
+    got = oracle.bmm_act(A, B, thr)
+    np.testing.assert_array_equal(got, 2 * popc > thr[:, None, :])     # booloptests.py:157-159
+    assert got.any() and not got.all()
+
+
+SWEEP = list(itertools.product([1, 3, 7], [0, 1, 2], [1, 2, 3]))      # booloptests.py:122-124
+
+
+@pytest.mark.parametrize("dtype", WORD_DTYPES)
+@pytest.mark.parametrize("C", [1, 3, 16, 64, 70])
+def test_conv_sweep_matches_torch_grouped_conv(oracle, dtype, C):
+    """The reference's own identity (booloptests.py:150-160) over its sweep of filter size x
+    padding x stride, on a 10x10 input (booloptests.py:116)."""
+    D, O, S = 3, 5, 10
+    for fs, pad, stride in SWEEP:
+        g = rng(fs * 100 + pad * 10 + stride + C)
+        xb = g.integers(0, 2, size=(D, S, S, C)).astype(bool)
+        fb = g.integers(0, 2, size=(D, O, fs, fs, C)).astype(bool)
+        xp = U.pack_bits(xb.reshape(-1, C), dtype).reshape(D, S, S, -1)
+        fp = U.pack_bits(fb.reshape(-1, C), dtype).reshape(D, O, fs, fs, -1)
+        # modules/binary.py:136-137 / booloptests.py:62: [D,O,fx,fy,Cw] -> [D, fx*fy*Cw, O]
+        fr = np.ascontiguousarray(fp.transpose(0, 2, 3, 4, 1).reshape(D, -1, O))
+        got = oracle.conv(xp, fr, fs, fs, pad, pad, stride, stride)
+        want = U.conv_popc_torch(xb, fb, pad, stride)
+        np.testing.assert_array_equal(got, want, err_msg=str((fs, pad, stride)))
+        K = fs * fs * C
+        thr = (g.integers(0, K, size=(D, O)) - K // 2 + K).astype(np.int32)   # booloptests.py:130,133
+        act = oracle.conv_act(xp, fr, thr, fs, fs, pad, pad, stride, stride)
+        np.testing.assert_array_equal(act, 2 * want > thr[:, None, None, :])
+
+
+@pytest.mark.parametrize("dtype", WORD_DTYPES)
+def test_im2col_matches_slicing_and_1x1_conv_is_bmm(oracle, dtype):
+    g = rng(5)
+    B, H, W, C = 2, 6, 9, 70
+    xb = g.integers(0, 2, size=(B, H, W, C)).astype(bool)
+    xp = U.pack_bits(xb.reshape(-1, C), dtype).reshape(B, H, W, -1)
+    Cw = xp.shape[3]
+    wb = np.dtype(dtype).itemsize * 8
+    for fx, fy, px, py, sx, sy in [(3, 3, 1, 1, 1, 1), (1, 1, 0, 0, 1, 1), (2, 3, 0, 2, 2, 1), (3, 2, 2, 0, 1, 3),
+                                   (5, 5, 2, 2, 2, 2)]:
+        got = oracle.batch_im2col(xp, fx, fy, px, py, sx, sy)
+        cols_bits = U.im2col_bits(xb, fx, fy, px, py, sx, sy)             # [B, hw, taps*C]
+        hw = cols_bits.shape[1]
+        # pack per tap so that the word layout is (tap, channel word)
+        per_tap = cols_bits.reshape(B * hw * fx * fy, C)
+        want = U.pack_bits(per_tap, dtype).reshape(B, hw, fx * fy * Cw)
+        np.testing.assert_array_equal(got, want)
+    # 1x1 / no pad / stride 1: im2col is the identity reshape, conv is bmm
+    filt = g.integers(-2 ** 31, 2 ** 31, size=(B, Cw, 4)).astype(dtype)
+    filt &= np.array(-1, dtype=dtype)  # any bits: padding bits of the input are zero anyway
+    np.testing.assert_array_equal(oracle.batch_im2col(xp, 1, 1, 0, 0, 1, 1), xp.reshape(B, H * W, Cw))
+    np.testing.assert_array_equal(oracle.conv(xp, filt, 1, 1, 0, 0, 1, 1).reshape(B, H * W, 4),
+                                  oracle.bmm(xp.reshape(B, H * W, Cw), filt))
+    assert wb in (32, 64)
+
+
+@pytest.mark.parametrize("dtype", WORD_DTYPES)
+def test_max_pool_matches_torch_and_or_window(oracle, dtype):
+    g = rng(3)
+    for C in [1, 16, 64, 100]:
+        for S in [10, 7]:
+            xb = g.integers(0, 2, size=(3, S, S, C)).astype(bool)
+            xp = U.pack_bits(xb.reshape(-1, C), dtype).reshape(3, S, S, -1)
+            # booloptests.py:138-141: 2x2 stride 2 no padding against F.max_pool2d
+            got = oracle.max_pool2d(xp, 2, 2, 0, 0, 2, 2)
+            want_bits = U.max_pool_bits_torch(xb)
+            want = U.pack_bits(want_bits.reshape(-1, C), dtype).reshape(got.shape)
+            np.testing.assert_array_equal(got, want)
+            for fx, fy, px, py, sx, sy in [(2, 2, 1, 1, 2, 2), (2, 2, 0, 1, 1, 2), (3, 3, 1, 1, 2, 2), (2, 2, 0, 0, 1, 1),
+                                           (2, 2, 1, 0, 3, 3)]:
+                got = oracle.max_pool2d(xp, fx, fy, px, py, sx, sy)
+                wb_ = U.or_pool2x2_bits(xb, fx, fy, px, py, sx, sy)
+                want = U.pack_bits(wb_.reshape(-1, C), dtype).reshape(got.shape)
+                np.testing.assert_array_equal(got, want, err_msg=str((C, S, fx, fy, px, py, sx, sy)))
+    # padded torch pooling agrees where the 2x2 window is what the caller asked for
+    xb = g.integers(0, 2, size=(2, 8, 8, 5)).astype(bool)
+    xp = U.pack_bits(xb.reshape(-1, 5), dtype).reshape(2, 8, 8, -1)
+    got = oracle.max_pool2d(xp, 2, 2, 1, 1, 2, 2)
+    want = U.pack_bits(U.max_pool_bits_torch(xb, 2, 1, 2).reshape(-1, 5), dtype).reshape(got.shape)
+    np.testing.assert_array_equal(got, want)
+
+
+@pytest.mark.parametrize("dtype", WORD_DTYPES)
+@pytest.mark.parametrize("n,R,C", [(3, 4, 64), (2, 3, 1), (5, 2, 63), (2, 5, 65), (3, 2, 200), (1, 1, 256)])
+def test_sample_from_words_closed_form(oracle, dtype, n, R, C):
+    g = rng(n * 7 + R * 3 + C)
+    words = g.integers(0, 2 ** 32, size=(n, R, C), dtype=np.uint64).astype(np.uint32)
+    thr = g.integers(0, 2 ** 32, size=(R, C), dtype=np.uint64).astype(np.uint32)
+    got = oracle.sample_from_words(thr, words, dtype)
+    want = U.pack_bits((words < thr[None]).reshape(n * R, C), dtype).reshape(n, R, -1)
+    np.testing.assert_array_equal(got, want)
+    # scalar threshold + base (flip form): weights = base ^ mask
+    T = 214748364                                              # floor(0.05 * 2**32)
+    base_bits = g.integers(0, 2, size=(R, C)).astype(bool)
+    base = U.pack_bits(base_bits, dtype)
+    got = oracle.sample_from_words(T, words, dtype, base=base)
+    want = U.pack_bits(((words < T) ^ base_bits[None]).reshape(n * R, C), dtype).reshape(n, R, -1)
+    np.testing.assert_array_equal(got, want)
+    # edge thresholds: 0 never fires; 2**32-1 fires unless the word is 0xFFFFFFFF
+    assert not oracle.sample_from_words(0, words, dtype).any()
+    allw = np.full((1, 1, C), 0xFFFFFFFF, dtype=np.uint32)
+    assert not oracle.sample_from_words(0xFFFFFFFF, allw, dtype).any()
+
+
+def test_sample_rate_is_p(oracle):
+    g = rng(0)
+    words = g.integers(0, 2 ** 32, size=(64, 16, 256), dtype=np.uint64).astype(np.uint32)
+    for p in [0.01, 0.02, 0.05, 0.5]:
+        T = int(p * 2 ** 32)
+        m = oracle.sample_from_words(T, words, np.int64)
+        rate = U.unpack_bits(m.reshape(-1, 4)).mean()
+        assert abs(rate - p) < 4 * np.sqrt(p * (1 - p) / words.size) + 1e-4
+
+
+@pytest.mark.parametrize("dtype", WORD_DTYPES)
+@pytest.mark.parametrize("n,R,C", [(3, 4, 64), (4, 7, 100), (2, 3, 31), (2, 2, 300)])
+def test_seeded_bmv_equals_materialised(oracle, dtype, n, R, C):
+    g = rng(C)
+    words = g.integers(0, 2 ** 32, size=(n, R, C), dtype=np.uint64).astype(np.uint32)
+    xb = g.integers(0, 2, size=(n, C)).astype(bool)
+    x = U.pack_bits(xb, dtype)
+    base = U.pack_bits(g.integers(0, 2, size=(R, C)).astype(bool), dtype)
+    T = int(0.05 * 2 ** 32)
+    thr = g.integers(0, 2 ** 32, size=(R, C), dtype=np.uint64).astype(np.uint32)
+    for kw in [dict(thresh=T, base=base), dict(thresh=thr, base=None), dict(thresh=thr, base=base)]:
+        W = oracle.sample_from_words(kw["thresh"], words, dtype, base=kw["base"])
+        want = oracle.bmm(W, x.reshape(n, -1, 1))[:, :, 0]
+        got = oracle.seeded_bmv_from_words(kw["thresh"], x, words, base=kw["base"])
+        np.testing.assert_array_equal(got, want)
+
+
+@pytest.mark.parametrize("dtype", WORD_DTYPES)
+def test_weighted_sum_matches_einsum(oracle, dtype):
+    g = rng(2)
+    n, R, C = 37, 5, 100
+    bits = g.integers(0, 2, size=(n, R, C)).astype(bool)
+    words = U.pack_bits(bits.reshape(n * R, C), dtype).reshape(n, R, -1)
+    w = g.standard_normal(n).astype(np.float32)
+    got = oracle.weighted_sum(words, w, C)
+    want = np.einsum("n,nrc->rc", w.astype(np.float64), bits.astype(np.float64))
+    np.testing.assert_allclose(got, want, rtol=1e-4, atol=1e-4)
