@@ -1,0 +1,174 @@
+/*
+ * nesbin.h -- C ABI of libnesbin.so: population-batched packed binary layer forward ops for
+ * AMD Instinct MI355X (gfx950), a from-scratch replacement for the CUDA/CuPy kernels behind
+ * jamesal1/NESgpu's extensions/booleanOperations.py, boolop_cuda and boolutil_cuda.
+ *
+ * Conventions (all entry points)
+ *   - every pointer is a DEVICE pointer into dense row-major memory owned by the caller; the
+ *     library allocates nothing and keeps no state between calls (re-entrant);
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream); launches are
+ *     asynchronous on it and the call never synchronises;
+ *   - packed words are LSB-first: bit i of word y of a row is element y*bits+i
+ *     (extensions/src/pack.cu:26); `_i64` entry points use 64-bit words, `_i32` 32-bit words
+ *     (the reference retargets its kernels the same way, extensions/booleanOperations.py:10-11);
+ *   - the return value is 0 on success, NB_ERR_* for rejected arguments (nothing launched), or
+ *     NB_ERR_HIP_BASE + hipError_t when the runtime refused a launch.  Nothing throws.
+ *     nb_last_error_string() describes the last failure on the calling thread.
+ */
+#ifndef NESBIN_H
+#define NESBIN_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define NB_OK 0
+#define NB_ERR_NULL 1        /* a required pointer is NULL */
+#define NB_ERR_SHAPE 2       /* negative / inconsistent / too large dimension */
+#define NB_ERR_ALIGN 3       /* pointer not aligned to its element size */
+#define NB_ERR_UNSUPPORTED 4 /* combination this build has no kernel for */
+#define NB_ERR_HIP_BASE 1000
+
+typedef void *nb_stream_t;
+
+int nb_version(void);
+const char *nb_last_error_string(void);
+
+/* ---- pack / unpack -------------------------------------------------------------------
+ * pack: bool bytes [R, C] -> words [R, ceil(C/bits)], zero-filled tail.
+ *   replaces extensions/booleanOperations.py:175-187 (pack_kernel, extensions/src/pack.cu:4-30)
+ *   and boolutil_cuda.pack (extensions/booleanUtilities.cpp:36-40). */
+int nb_pack_i64(int64_t *out, const uint8_t *in, int64_t R, int64_t C, nb_stream_t stream);
+int nb_pack_i32(int32_t *out, const uint8_t *in, int64_t R, int64_t C, nb_stream_t stream);
+/* unpack: words [R, Rw] -> bool bytes [R, Rw*bits].
+ *   replaces boolutil_cuda.unpack (extensions/booleanUtilities.cpp:43-46,
+ *   extensions/booleanUtilitiesCuda.cu:77-90,182-195). */
+int nb_unpack_i64(uint8_t *out, const int64_t *in, int64_t R, int64_t Rw, nb_stream_t stream);
+int nb_unpack_i32(uint8_t *out, const int32_t *in, int64_t R, int64_t Rw, nb_stream_t stream);
+/* int8pack: uint8 [R, C] -> words [R, ceil(C/(bits/8))], little-endian bytes, zero tail.
+ *   replaces extensions/booleanOperations.py:189-201 (extensions/src/int8pack.cu:4-30). */
+int nb_int8pack_i64(int64_t *out, const uint8_t *in, int64_t R, int64_t C, nb_stream_t stream);
+int nb_int8pack_i32(int32_t *out, const uint8_t *in, int64_t R, int64_t C, nb_stream_t stream);
+
+/* ---- XOR-popcount batched matmul --------------------------------------------------------
+ * C[z,x,y] = sum_k popcount(A[z,x,k] ^ B[z,k,y]);  A [Z,M,Kw], B [Z,Kw,N], C [Z,M,N] int32.
+ *   replaces extensions/booleanOperations.py:107-129 (bmm_kernel, extensions/src/bmm.cu:5-58)
+ *   and boolop_cuda.binary_bmm (extensions/booleanOperations.cpp:34-41). */
+int nb_bmm_i64(int32_t *C, const int64_t *A, const int64_t *B, int64_t Z, int64_t M, int64_t Kw, int64_t N,
+               nb_stream_t stream);
+int nb_bmm_i32(int32_t *C, const int32_t *A, const int32_t *B, int64_t Z, int64_t M, int64_t Kw, int64_t N,
+               nb_stream_t stream);
+/* same with the output (2*popc > thresh[z,y]) as bool bytes; thresh [Z,N] int32.
+ *   replaces extensions/booleanOperations.py:131-158 (extensions/src/bmm_act.cu:5-63). */
+int nb_bmm_act_i64(uint8_t *C, const int64_t *A, const int64_t *B, const int32_t *thresh, int64_t Z, int64_t M,
+                   int64_t Kw, int64_t N, nb_stream_t stream);
+int nb_bmm_act_i32(uint8_t *C, const int32_t *A, const int32_t *B, const int32_t *thresh, int64_t Z, int64_t M,
+                   int64_t Kw, int64_t N, nb_stream_t stream);
+
+/* ---- packed im2col / conv -----------------------------------------------------------------
+ * Geometry: input [D,H,W,Cw] (channels-last packed), fx taps along H, fy taps along W,
+ * h=(H-fx+2px)/sx+1, w=(W-fy+2py)/sy+1, out-of-range taps read the zero word.
+ * im2col: -> [D, h*w, fx*fy*Cw], element (i*fy+j)*Cw+c.
+ *   replaces extensions/booleanOperations.py:82-102 (extensions/src/batch_im2col.cu:3-33) and
+ *   boolop_cuda.batch_im2col (extensions/booleanOperations.cpp:52-55). */
+int nb_im2col_i64(int64_t *out, const int64_t *in, int64_t D, int64_t H, int64_t W, int64_t Cw, int fx, int fy,
+                  int px, int py, int sx, int sy, nb_stream_t stream);
+int nb_im2col_i32(int32_t *out, const int32_t *in, int64_t D, int64_t H, int64_t W, int64_t Cw, int fx, int fy,
+                  int px, int py, int sx, int sy, nb_stream_t stream);
+/* conv: filt [D, fx*fy*Cw, O] -> out [D,h,w,O] int32 popcount sums; equals
+ * bmm(im2col(in), filt) without materialising the columns.
+ *   replaces extensions/booleanOperations.py:162-166 and boolop_cuda.binary_batch_conv2d
+ *   (extensions/booleanOperations.cpp:43-50, extensions/booleanOperationsCuda.cu:295-298). */
+int nb_conv_i64(int32_t *out, const int64_t *in, const int64_t *filt, int64_t D, int64_t H, int64_t W, int64_t Cw,
+                int64_t O, int fx, int fy, int px, int py, int sx, int sy, nb_stream_t stream);
+int nb_conv_i32(int32_t *out, const int32_t *in, const int32_t *filt, int64_t D, int64_t H, int64_t W, int64_t Cw,
+                int64_t O, int fx, int fy, int px, int py, int sx, int sy, nb_stream_t stream);
+/* conv_act: out [D,h,w,O] bool bytes = 2*popc > thresh[d,o]; thresh [D,O] int32.
+ *   replaces extensions/booleanOperations.py:168-172. */
+int nb_conv_act_i64(uint8_t *out, const int64_t *in, const int64_t *filt, const int32_t *thresh, int64_t D,
+                    int64_t H, int64_t W, int64_t Cw, int64_t O, int fx, int fy, int px, int py, int sx, int sy,
+                    nb_stream_t stream);
+int nb_conv_act_i32(uint8_t *out, const int32_t *in, const int32_t *filt, const int32_t *thresh, int64_t D,
+                    int64_t H, int64_t W, int64_t Cw, int64_t O, int fx, int fy, int px, int py, int sx, int sy,
+                    nb_stream_t stream);
+/* conv_act_pack: the same bits packed along O into [D,h,w,ceil(O/bits)] words; with pool != 0
+ * the 2x2 / stride-2 / no-padding OR-pool of those words, [D,h/2,w/2,ceil(O/bits)].
+ * Equals pack(conv_act(...)) followed (pool) by max_pool2d(.,2,2,0,0,2,2); it fuses the chain
+ * conv_act -> pack -> max_pool2d of modules/binary.py:156-157,141-142,177-182 so the bool map
+ * never reaches memory.  No single counterpart in the reference. */
+int nb_conv_act_pack_i64(int64_t *out, const int64_t *in, const int64_t *filt, const int32_t *thresh, int64_t D,
+                         int64_t H, int64_t W, int64_t Cw, int64_t O, int fx, int fy, int px, int py, int sx,
+                         int sy, int pool, nb_stream_t stream);
+int nb_conv_act_pack_i32(int32_t *out, const int32_t *in, const int32_t *filt, const int32_t *thresh, int64_t D,
+                         int64_t H, int64_t W, int64_t Cw, int64_t O, int fx, int fy, int px, int py, int sx,
+                         int sy, int pool, nb_stream_t stream);
+
+/* ---- packed max-pool -------------------------------------------------------------------------
+ * [B,H,W,Cw] -> [B,h,w,Cw]; bitwise OR over the 2x2 window anchored at (xo*sx-px, yo*sy-py),
+ * zero outside.  fx, fy only set the output size, as in the reference kernel whose window
+ * loops are fixed at 2 (extensions/src/max_pool2d.cu:21-23).
+ *   replaces extensions/booleanOperations.py:232-252 (extensions/src/max_pool2d.cu:3-36). */
+int nb_max_pool2d_i64(int64_t *out, const int64_t *in, int64_t B, int64_t H, int64_t W, int64_t Cw, int fx, int fy,
+                      int px, int py, int sx, int sy, nb_stream_t stream);
+int nb_max_pool2d_i32(int32_t *out, const int32_t *in, int64_t B, int64_t H, int64_t W, int64_t Cw, int fx, int fy,
+                      int px, int py, int sx, int sy, nb_stream_t stream);
+
+/* ---- Bernoulli bit sampling ------------------------------------------------------------------
+ * Law and layout of sample_bits (extensions/booleanOperations.py:203-215,
+ * extensions/src/sample_bits.cu:47-57; boolutil_cuda.sample_bits,
+ * extensions/booleanUtilities.cpp:49-52): out [n,R,ceil(C/bits)], one independent draw per
+ * (member, row, column), tail bits zero.  The cuRAND XORWOW draw is replaced by a uint32 word:
+ *     bit(m,r,c) = word(m,r,c) < threshold(r,c)
+ * threshold(r,c) = thresh[r*C+c] if thresh != NULL else thr_scalar.  If base != NULL
+ * ([R,ceil(C/bits)]) the sampled mask is XORed onto it: out = base ^ mask (bit-flip form).
+ * from_words: word(m,r,c) = words[(m*R+r)*C+c], supplied by the caller.
+ * philox:     word(m,r,c) = lane g%4 of Philox4x32-10(counter=(lo(g/4),hi(g/4),lo(subseq),
+ *             hi(subseq)), key=(lo(seed),hi(seed))), g = first + (m*R+r)*C+c  -- the same
+ *             numbers nb_philox_words writes, so the two forms agree bit for bit. */
+int nb_sample_from_words_i64(int64_t *out, const int64_t *base, const uint32_t *thresh, uint32_t thr_scalar,
+                             const uint32_t *words, int64_t n, int64_t R, int64_t C, nb_stream_t stream);
+int nb_sample_from_words_i32(int32_t *out, const int32_t *base, const uint32_t *thresh, uint32_t thr_scalar,
+                             const uint32_t *words, int64_t n, int64_t R, int64_t C, nb_stream_t stream);
+int nb_sample_philox_i64(int64_t *out, const int64_t *base, const uint32_t *thresh, uint32_t thr_scalar,
+                         uint64_t seed, uint64_t subseq, uint64_t first, int64_t n, int64_t R, int64_t C,
+                         nb_stream_t stream);
+int nb_sample_philox_i32(int32_t *out, const int32_t *base, const uint32_t *thresh, uint32_t thr_scalar,
+                         uint64_t seed, uint64_t subseq, uint64_t first, int64_t n, int64_t R, int64_t C,
+                         nb_stream_t stream);
+int nb_philox_words(uint32_t *out, uint64_t seed, uint64_t subseq, uint64_t first, int64_t count,
+                    nb_stream_t stream);
+
+/* ---- fused sample + XOR-popcount matrix-vector product -------------------------------------------
+ * C[m,r] = sum_k popcount(w(m,r,k) ^ x[m,k]) where w is what nb_sample_* would have written;
+ * the per-member weights never exist in memory.  x [n,ceil(C/bits)], C [n,R] int32.
+ *   replaces boolop_cuda.binary_seeded_bmv (extensions/booleanOperations.cpp:58-63,
+ *   extensions/booleanOperationsCuda.cu:172-202,301-322). */
+int nb_seeded_bmv_from_words_i64(int32_t *C, const int64_t *base, const uint32_t *thresh, uint32_t thr_scalar,
+                                 const int64_t *x, const uint32_t *words, int64_t n, int64_t R, int64_t Cbits,
+                                 nb_stream_t stream);
+int nb_seeded_bmv_from_words_i32(int32_t *C, const int32_t *base, const uint32_t *thresh, uint32_t thr_scalar,
+                                 const int32_t *x, const uint32_t *words, int64_t n, int64_t R, int64_t Cbits,
+                                 nb_stream_t stream);
+int nb_seeded_bmv_philox_i64(int32_t *C, const int64_t *base, const uint32_t *thresh, uint32_t thr_scalar,
+                             const int64_t *x, uint64_t seed, uint64_t subseq, uint64_t first, int64_t n, int64_t R,
+                             int64_t Cbits, nb_stream_t stream);
+int nb_seeded_bmv_philox_i32(int32_t *C, const int32_t *base, const uint32_t *thresh, uint32_t thr_scalar,
+                             const int32_t *x, uint64_t seed, uint64_t subseq, uint64_t first, int64_t n, int64_t R,
+                             int64_t Cbits, nb_stream_t stream);
+
+/* ---- weighted sum of packed masks (update step) ---------------------------------------------------
+ * ret[r,z] = fp16( sum_m float(w[m]) * bit(in[m,r,z/bits], z%bits) ), fp32 accumulation in member
+ * order; in [n,R,Rw], w [n] fp16, ret [R,zbits] fp16.
+ *   replaces extensions/booleanOperations.py:218-229 (extensions/src/weighted_sum.cu:8-48) and
+ *   boolutil_cuda.binary_weighted_sum (extensions/booleanUtilities.cpp:54-59). */
+int nb_weighted_sum_i64(uint16_t *ret, const int64_t *in, const uint16_t *w, int64_t n, int64_t R, int64_t Rw,
+                        int64_t zbits, nb_stream_t stream);
+int nb_weighted_sum_i32(uint16_t *ret, const int32_t *in, const uint16_t *w, int64_t n, int64_t R, int64_t Rw,
+                        int64_t zbits, nb_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NESBIN_H */

@@ -1,0 +1,84 @@
+"""ctypes binding of libnesbin.so (the C ABI declared in include/nesbin.h).
+
+The library is loaded lazily on first use and there is no fallback: if it has not been built
+(`python -c "import __graft_entry__ as g; g.build()"` or `make -C nesgpu_amd/csrc`) every op
+raises ``RuntimeError``.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libnesbin.so")
+_lib = None
+
+NB_OK = 0
+NB_ERR_HIP_BASE = 1000
+
+_I64, _I32, _U32, _U64, _PTR = ctypes.c_int64, ctypes.c_int, ctypes.c_uint32, ctypes.c_uint64, ctypes.c_void_p
+_GEOM = [_I32] * 6
+
+# name -> argument types (without the `_i64`/`_i32` suffix expansion); every entry returns int
+_SUFFIXED = {
+    "nb_pack": [_PTR, _PTR, _I64, _I64, _PTR],
+    "nb_unpack": [_PTR, _PTR, _I64, _I64, _PTR],
+    "nb_int8pack": [_PTR, _PTR, _I64, _I64, _PTR],
+    "nb_bmm": [_PTR, _PTR, _PTR, _I64, _I64, _I64, _I64, _PTR],
+    "nb_bmm_act": [_PTR, _PTR, _PTR, _PTR, _I64, _I64, _I64, _I64, _PTR],
+    "nb_im2col": [_PTR, _PTR, _I64, _I64, _I64, _I64] + _GEOM + [_PTR],
+    "nb_conv": [_PTR, _PTR, _PTR, _I64, _I64, _I64, _I64, _I64] + _GEOM + [_PTR],
+    "nb_conv_act": [_PTR, _PTR, _PTR, _PTR, _I64, _I64, _I64, _I64, _I64] + _GEOM + [_PTR],
+    "nb_conv_act_pack": [_PTR, _PTR, _PTR, _PTR, _I64, _I64, _I64, _I64, _I64] + _GEOM + [_I32, _PTR],
+    "nb_max_pool2d": [_PTR, _PTR, _I64, _I64, _I64, _I64] + _GEOM + [_PTR],
+    "nb_sample_from_words": [_PTR, _PTR, _PTR, _U32, _PTR, _I64, _I64, _I64, _PTR],
+    "nb_sample_philox": [_PTR, _PTR, _PTR, _U32, _U64, _U64, _U64, _I64, _I64, _I64, _PTR],
+    "nb_seeded_bmv_from_words": [_PTR, _PTR, _PTR, _U32, _PTR, _PTR, _I64, _I64, _I64, _PTR],
+    "nb_seeded_bmv_philox": [_PTR, _PTR, _PTR, _U32, _PTR, _U64, _U64, _U64, _I64, _I64, _I64, _PTR],
+    "nb_weighted_sum": [_PTR, _PTR, _PTR, _I64, _I64, _I64, _I64, _PTR],
+}
+_PLAIN = {
+    "nb_philox_words": [_PTR, _U64, _U64, _U64, _I64, _PTR],
+}
+
+
+def exported_symbols():
+    """Every symbol include/nesbin.h declares."""
+    names = ["nb_version", "nb_last_error_string"] + list(_PLAIN)
+    for base in _SUFFIXED:
+        names += [base + "_i64", base + "_i32"]
+    return names
+
+
+def load():
+    global _lib
+    if _lib is not None:
+        return _lib
+    path = os.environ.get("NESBIN_LIB", LIB_PATH)
+    if not os.path.exists(path):
+        raise RuntimeError(
+            "libnesbin.so is not built (looked at %s); run `make -C nesgpu_amd/csrc` or "
+            "`python -c 'import __graft_entry__ as g; g.build()'`. There is no CPU fallback." % path)
+    lib = ctypes.CDLL(path)
+    lib.nb_version.restype = ctypes.c_int
+    lib.nb_version.argtypes = []
+    lib.nb_last_error_string.restype = ctypes.c_char_p
+    lib.nb_last_error_string.argtypes = []
+    for base, args in _SUFFIXED.items():
+        for suf in ("_i64", "_i32"):
+            fn = getattr(lib, base + suf)
+            fn.restype = ctypes.c_int
+            fn.argtypes = args
+    for name, args in _PLAIN.items():
+        fn = getattr(lib, name)
+        fn.restype = ctypes.c_int
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+def call(name, *args):
+    """Call an entry point and turn a non-zero status into RuntimeError."""
+    lib = load()
+    rc = getattr(lib, name)(*args)
+    if rc != NB_OK:
+        msg = lib.nb_last_error_string().decode("utf-8", "replace")
+        raise RuntimeError("%s failed with status %d: %s" % (name, rc, msg))

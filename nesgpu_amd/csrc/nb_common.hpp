@@ -1,0 +1,93 @@
+// Shared definitions for the gfx950 kernels of libnesbin.so.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/nesbin.h"
+
+namespace nb {
+
+constexpr int kWave = 64;  // CDNA4 wavefront width
+
+template <typename W>
+struct WordTraits;
+template <>
+struct WordTraits<uint64_t> {
+    static constexpr int bits = 64;
+    static constexpr int log2bits = 6;
+};
+template <>
+struct WordTraits<uint32_t> {
+    static constexpr int bits = 32;
+    static constexpr int log2bits = 5;
+};
+
+// XOR + popcount of one packed word.  A 64-bit word compiles to two v_xor_b32 and two
+// v_bcnt_u32_b32; the add into `acc` folds into v_bcnt's accumulate operand.
+__device__ __forceinline__ int popc_xor(uint64_t a, uint64_t b) { return __popcll(a ^ b); }
+__device__ __forceinline__ int popc_xor(uint32_t a, uint32_t b) { return __popc(a ^ b); }
+
+// Philox4x32-10 (Salmon et al., SC'11): counter-based generator used when the caller does not
+// supply the random words.
+__device__ __forceinline__ uint4 philox4x32_10(uint4 c, uint2 k)
+{
+#pragma unroll
+    for (int r = 0; r < 10; r++) {
+        const uint32_t lo0 = 0xD2511F53u * c.x, hi0 = __umulhi(0xD2511F53u, c.x);
+        const uint32_t lo1 = 0xCD9E8D57u * c.z, hi1 = __umulhi(0xCD9E8D57u, c.z);
+        c = make_uint4(hi1 ^ c.y ^ k.x, lo1, hi0 ^ c.w ^ k.y, lo0);
+        k.x += 0x9E3779B9u;
+        k.y += 0xBB67AE85u;
+    }
+    return c;
+}
+
+struct PhiloxKey {
+    uint64_t seed, subseq, first;
+};
+
+// Block number `blk` (= word index / 4) of the stream described by `key`.
+__device__ __forceinline__ uint4 philox_block(const PhiloxKey &key, uint64_t blk)
+{
+    return philox4x32_10(make_uint4((uint32_t)blk, (uint32_t)(blk >> 32), (uint32_t)key.subseq,
+                                    (uint32_t)(key.subseq >> 32)),
+                         make_uint2((uint32_t)key.seed, (uint32_t)(key.seed >> 32)));
+}
+
+__device__ __forceinline__ uint32_t philox_word(const PhiloxKey &key, uint64_t g)
+{
+    const uint4 b = philox_block(key, g >> 2);
+    const uint32_t e = (uint32_t)g & 3u;
+    return e == 0 ? b.x : e == 1 ? b.y : e == 2 ? b.z : b.w;
+}
+
+// ---- host side -----------------------------------------------------------------------------
+void set_error(const char *fmt, ...);
+int fail(int code, const char *fmt, ...);
+int check_launch(const char *what);
+
+inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+inline bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+inline hipStream_t as_stream(nb_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
+
+// Largest grid dimension we ever request in x; y/z are limited to 65535 by the runtime.
+constexpr int64_t kMaxGridX = 2147483647LL;
+constexpr int64_t kMaxGridYZ = 65535;
+
+// Output size of a strided window op (extensions/booleanOperations.py:83-84,234-235).
+inline int64_t out_dim(int64_t in, int f, int p, int s) { return (in - f + 2 * (int64_t)p) / s + 1; }
+
+}  // namespace nb
+
+#define NB_REQUIRE_PTR(p)                                            \
+    do {                                                             \
+        if ((p) == nullptr) return nb::fail(NB_ERR_NULL, "%s: %s is NULL", __func__, #p); \
+    } while (0)
+#define NB_REQUIRE_ALIGNED(p, a)                                                                        \
+    do {                                                                                                \
+        if (!nb::aligned((p), (a))) return nb::fail(NB_ERR_ALIGN, "%s: %s is not %d-byte aligned", __func__, #p, (int)(a)); \
+    } while (0)
+#define NB_REQUIRE(cond, ...)                                        \
+    do {                                                             \
+        if (!(cond)) return nb::fail(NB_ERR_SHAPE, __VA_ARGS__);     \
+    } while (0)

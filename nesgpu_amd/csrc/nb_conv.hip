@@ -1,0 +1,287 @@
+// Packed im2col, implicit-im2col binary conv (int32 / bool / packed / packed+pooled outputs) and
+// the packed-bit max-pool.
+#include "nb_rowlane.hpp"
+
+namespace nb {
+
+// ---- im2col (kept for API parity; conv itself never materialises the columns) ----------------
+// One thread per output word; consecutive threads write consecutive words.
+template <typename W>
+__global__ __launch_bounds__(256) void im2col_kernel(W *__restrict__ out, const W *__restrict__ in, int64_t total,
+                                                     ConvGeom g)
+{
+    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (t >= total) return;
+    const int K = g.fx * g.fy * g.Cw;
+    const int64_t rowi = t / K;  // (b, loc)
+    const int e = (int)(t - rowi * K);
+    const int hw = g.h * g.w;
+    const int64_t b = rowi / hw;
+    const int loc = (int)(rowi - b * hw);
+    const int xo = loc / g.w, yo = loc - xo * g.w;
+    const int tap = e / g.Cw, c = e - tap * g.Cw;
+    const int i = tap / g.fy, j = tap - i * g.fy;
+    const int xi = i + xo * g.sx - g.px, yi = j + yo * g.sy - g.py;
+    const bool ok = xi >= 0 && xi < g.H && yi >= 0 && yi < g.Wd;
+    out[t] = ok ? in[((b * g.H + xi) * g.Wd + yi) * g.Cw + c] : (W)0;
+}
+
+// ---- max-pool: OR over the fixed 2x2 window (extensions/src/max_pool2d.cu:19-32) ---------------
+template <typename W>
+__global__ __launch_bounds__(256) void max_pool_kernel(W *__restrict__ out, const W *__restrict__ in, int64_t total,
+                                                       ConvGeom g)
+{
+    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (t >= total) return;
+    const int64_t pix = t / g.Cw;
+    const int c = (int)(t - pix * g.Cw);
+    const int hw = g.h * g.w;
+    const int64_t b = pix / hw;
+    const int loc = (int)(pix - b * hw);
+    const int xo = loc / g.w, yo = loc - xo * g.w;
+    const W *img = in + b * (int64_t)g.H * g.Wd * g.Cw;
+    W v = 0;
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            const int xi = i + xo * g.sx - g.px, yi = j + yo * g.sy - g.py;
+            if (xi >= 0 && xi < g.H && yi >= 0 && yi < g.Wd) v |= img[((int64_t)xi * g.Wd + yi) * g.Cw + c];
+        }
+    out[t] = v;
+}
+
+// ---- conv: row-per-lane kernel with the implicit-im2col loader ----------------------------------
+// POOLMAP: lanes 4q..4q+3 hold the 2x2 window of pooled pixel q (needed by EpiPack<.,true>);
+// otherwise lane p of a member is output pixel p in row-major order.
+template <typename W, int KC, int NT, bool SINGLE, bool POOLMAP, class Epi>
+__global__ __launch_bounds__(256) void conv_rowlane_kernel(ConvA<W> al, const W *__restrict__ filt, Epi epi,
+                                                           int pblocks, int N)
+{
+    const ConvGeom &g = al.g;
+    const int64_t z = blockIdx.x / pblocks;
+    const int p = (int)(blockIdx.x - z * pblocks) * 256 + threadIdx.x;
+    int yo, xo;
+    bool valid;
+    int64_t orow;
+    if (POOLMAP) {
+        const int h2 = g.h >> 1, w2 = g.w >> 1;
+        const int q = p >> 2, sub = p & 3;
+        valid = q < h2 * w2;
+        const int qy = q / w2, qx = q - qy * w2;
+        yo = 2 * qy + (sub >> 1);
+        xo = 2 * qx + (sub & 1);
+        orow = z * (int64_t)(h2 * w2) + q;
+    } else {
+        valid = p < g.h * g.w;
+        yo = p / g.w;
+        xo = p - yo * g.w;
+        orow = z * (int64_t)(g.h * g.w) + p;
+    }
+    const typename ConvA<W>::Lane lane = al.lane_at(z, yo, xo, valid);
+    const int Kw = g.fx * g.fy * g.Cw;
+    const W *__restrict__ Fz = filt + z * (int64_t)Kw * N;
+    rowlane_body<W, KC, NT, SINGLE>(al, lane, Fz, epi, orow, z, Kw, N);
+}
+
+template <typename W, bool POOLMAP, class Epi>
+static void dispatch_conv(const ConvA<W> &al, const W *filt, const Epi &epi, int64_t D, int64_t lanes_per_member,
+                          int N, hipStream_t s)
+{
+    const int Kw = al.g.fx * al.g.fy * al.g.Cw;
+    const int pblocks = (int)ceil_div(lanes_per_member, 256);
+    const dim3 grid((unsigned)(D * pblocks)), block(256);
+    if (Kw <= 4)
+        conv_rowlane_kernel<W, 4, 16, true, POOLMAP, Epi><<<grid, block, 0, s>>>(al, filt, epi, pblocks, N);
+    else if (Kw <= 9)
+        conv_rowlane_kernel<W, 9, 16, true, POOLMAP, Epi><<<grid, block, 0, s>>>(al, filt, epi, pblocks, N);
+    else if (Kw <= 18)
+        conv_rowlane_kernel<W, 18, 16, true, POOLMAP, Epi><<<grid, block, 0, s>>>(al, filt, epi, pblocks, N);
+    else
+        conv_rowlane_kernel<W, 16, 16, false, POOLMAP, Epi><<<grid, block, 0, s>>>(al, filt, epi, pblocks, N);
+}
+
+static int geom_check(ConvGeom *g, int64_t D, int64_t H, int64_t Wd, int64_t Cw, int fx, int fy, int px, int py,
+                      int sx, int sy, const char *who)
+{
+    NB_REQUIRE(D >= 0 && H >= 0 && Wd >= 0 && Cw >= 0, "%s: negative shape D=%lld H=%lld W=%lld Cw=%lld", who,
+               (long long)D, (long long)H, (long long)Wd, (long long)Cw);
+    NB_REQUIRE(fx >= 1 && fy >= 1 && sx >= 1 && sy >= 1 && px >= 0 && py >= 0,
+               "%s: bad window fx=%d fy=%d px=%d py=%d sx=%d sy=%d", who, fx, fy, px, py, sx, sy);
+    NB_REQUIRE(H <= 32768 && Wd <= 32768 && Cw <= 32768 && fx <= 1024 && fy <= 1024 && px <= 32768 && py <= 32768,
+               "%s: dimension too large (H=%lld W=%lld Cw=%lld fx=%d fy=%d)", who, (long long)H, (long long)Wd,
+               (long long)Cw, fx, fy);
+    const int64_t h = out_dim(H, fx, px, sx), w = out_dim(Wd, fy, py, sy);
+    NB_REQUIRE(H - fx + 2 * (int64_t)px >= 0 && Wd - fy + 2 * (int64_t)py >= 0,
+               "%s: window %dx%d larger than padded input %lldx%lld", who, fx, fy, (long long)(H + 2 * px),
+               (long long)(Wd + 2 * py));
+    NB_REQUIRE(h * w < (1LL << 30) && (int64_t)fx * fy * Cw < (1LL << 24), "%s: output %lldx%lld too large", who,
+               (long long)h, (long long)w);
+    g->H = (int)H;
+    g->Wd = (int)Wd;
+    g->Cw = (int)Cw;
+    g->fx = fx;
+    g->fy = fy;
+    g->px = px;
+    g->py = py;
+    g->sx = sx;
+    g->sy = sy;
+    g->h = (int)h;
+    g->w = (int)w;
+    return NB_OK;
+}
+
+template <typename W>
+int im2col_impl(W *out, const W *in, int64_t D, int64_t H, int64_t Wd, int64_t Cw, int fx, int fy, int px, int py,
+                int sx, int sy, nb_stream_t stream, const char *who)
+{
+    ConvGeom g;
+    if (int rc = geom_check(&g, D, H, Wd, Cw, fx, fy, px, py, sx, sy, who)) return rc;
+    const int64_t total = D * g.h * g.w * (int64_t)fx * fy * Cw;
+    if (total == 0) return NB_OK;
+    NB_REQUIRE_PTR(out);
+    NB_REQUIRE_PTR(in);
+    NB_REQUIRE_ALIGNED(out, sizeof(W));
+    NB_REQUIRE_ALIGNED(in, sizeof(W));
+    const int64_t blocks = ceil_div(total, 256);
+    NB_REQUIRE(blocks <= kMaxGridX, "%s: %lld output words exceed one launch", who, (long long)total);
+    im2col_kernel<W><<<dim3((unsigned)blocks), dim3(256), 0, as_stream(stream)>>>(out, in, total, g);
+    return check_launch(who);
+}
+
+template <typename W>
+int max_pool_impl(W *out, const W *in, int64_t B, int64_t H, int64_t Wd, int64_t Cw, int fx, int fy, int px, int py,
+                  int sx, int sy, nb_stream_t stream, const char *who)
+{
+    ConvGeom g;
+    if (int rc = geom_check(&g, B, H, Wd, Cw, fx, fy, px, py, sx, sy, who)) return rc;
+    const int64_t total = B * g.h * g.w * Cw;
+    if (total == 0) return NB_OK;
+    NB_REQUIRE_PTR(out);
+    NB_REQUIRE_PTR(in);
+    NB_REQUIRE_ALIGNED(out, sizeof(W));
+    NB_REQUIRE_ALIGNED(in, sizeof(W));
+    const int64_t blocks = ceil_div(total, 256);
+    NB_REQUIRE(blocks <= kMaxGridX, "%s: %lld output words exceed one launch", who, (long long)total);
+    max_pool_kernel<W><<<dim3((unsigned)blocks), dim3(256), 0, as_stream(stream)>>>(out, in, total, g);
+    return check_launch(who);
+}
+
+// mode 0: int32 sums, 1: bool bytes, 2: packed words, 3: packed + 2x2 pooled words
+template <typename W>
+int conv_impl(void *out, const W *in, const W *filt, const int32_t *thresh, int64_t D, int64_t H, int64_t Wd,
+              int64_t Cw, int64_t O, int fx, int fy, int px, int py, int sx, int sy, int mode, nb_stream_t stream,
+              const char *who)
+{
+    constexpr int bits = WordTraits<W>::bits;
+    ConvGeom g;
+    if (int rc = geom_check(&g, D, H, Wd, Cw, fx, fy, px, py, sx, sy, who)) return rc;
+    NB_REQUIRE(O >= 0 && O <= (1 << 24), "%s: bad output channel count %lld", who, (long long)O);
+    const int64_t hw = (int64_t)g.h * g.w;
+    const int64_t h2w2 = (int64_t)(g.h >> 1) * (g.w >> 1);
+    const int64_t lanes = mode == 3 ? 4 * h2w2 : hw;
+    if (D * lanes * O == 0) return NB_OK;
+    NB_REQUIRE_PTR(out);
+    if (Cw > 0) {
+        NB_REQUIRE_PTR(in);
+        NB_REQUIRE_PTR(filt);
+        NB_REQUIRE_ALIGNED(in, sizeof(W));
+        NB_REQUIRE_ALIGNED(filt, sizeof(W));
+    }
+    if (mode != 0) {
+        NB_REQUIRE_PTR(thresh);
+        NB_REQUIRE_ALIGNED(thresh, 4);
+    }
+    NB_REQUIRE(D * ceil_div(lanes, 256) <= kMaxGridX, "%s: %lld members x %lld pixels exceed one launch", who,
+               (long long)D, (long long)lanes);
+    ConvA<W> al{in, g};
+    hipStream_t s = as_stream(stream);
+    const int N = (int)O;
+    if (mode == 0) {
+        NB_REQUIRE_ALIGNED(out, 4);
+        EpiI32 epi{static_cast<int32_t *>(out), (N & 3) == 0 && aligned(out, 16)};
+        dispatch_conv<W, false, EpiI32>(al, filt, epi, D, lanes, N, s);
+    } else if (mode == 1) {
+        EpiBool epi{static_cast<uint8_t *>(out), thresh, (N & 3) == 0 && aligned(out, 4)};
+        dispatch_conv<W, false, EpiBool>(al, filt, epi, D, lanes, N, s);
+    } else if (mode == 2) {
+        NB_REQUIRE_ALIGNED(out, sizeof(W));
+        EpiPack<W, false> epi{static_cast<W *>(out), thresh, (int)ceil_div(O, bits)};
+        dispatch_conv<W, false, EpiPack<W, false>>(al, filt, epi, D, lanes, N, s);
+    } else {
+        NB_REQUIRE_ALIGNED(out, sizeof(W));
+        EpiPack<W, true> epi{static_cast<W *>(out), thresh, (int)ceil_div(O, bits)};
+        dispatch_conv<W, true, EpiPack<W, true>>(al, filt, epi, D, lanes, N, s);
+    }
+    return check_launch(who);
+}
+
+}  // namespace nb
+
+#define W64(p) reinterpret_cast<const uint64_t *>(p)
+#define W32(p) reinterpret_cast<const uint32_t *>(p)
+
+extern "C" {
+int nb_im2col_i64(int64_t *out, const int64_t *in, int64_t D, int64_t H, int64_t W, int64_t Cw, int fx, int fy, int px,
+                  int py, int sx, int sy, nb_stream_t s)
+{
+    return nb::im2col_impl<uint64_t>(reinterpret_cast<uint64_t *>(out), W64(in), D, H, W, Cw, fx, fy, px, py, sx, sy, s,
+                                     "nb_im2col_i64");
+}
+int nb_im2col_i32(int32_t *out, const int32_t *in, int64_t D, int64_t H, int64_t W, int64_t Cw, int fx, int fy, int px,
+                  int py, int sx, int sy, nb_stream_t s)
+{
+    return nb::im2col_impl<uint32_t>(reinterpret_cast<uint32_t *>(out), W32(in), D, H, W, Cw, fx, fy, px, py, sx, sy, s,
+                                     "nb_im2col_i32");
+}
+int nb_max_pool2d_i64(int64_t *out, const int64_t *in, int64_t B, int64_t H, int64_t W, int64_t Cw, int fx, int fy,
+                      int px, int py, int sx, int sy, nb_stream_t s)
+{
+    return nb::max_pool_impl<uint64_t>(reinterpret_cast<uint64_t *>(out), W64(in), B, H, W, Cw, fx, fy, px, py, sx, sy,
+                                       s, "nb_max_pool2d_i64");
+}
+int nb_max_pool2d_i32(int32_t *out, const int32_t *in, int64_t B, int64_t H, int64_t W, int64_t Cw, int fx, int fy,
+                      int px, int py, int sx, int sy, nb_stream_t s)
+{
+    return nb::max_pool_impl<uint32_t>(reinterpret_cast<uint32_t *>(out), W32(in), B, H, W, Cw, fx, fy, px, py, sx, sy,
+                                       s, "nb_max_pool2d_i32");
+}
+int nb_conv_i64(int32_t *out, const int64_t *in, const int64_t *filt, int64_t D, int64_t H, int64_t W, int64_t Cw,
+                int64_t O, int fx, int fy, int px, int py, int sx, int sy, nb_stream_t s)
+{
+    return nb::conv_impl<uint64_t>(out, W64(in), W64(filt), nullptr, D, H, W, Cw, O, fx, fy, px, py, sx, sy, 0, s,
+                                   "nb_conv_i64");
+}
+int nb_conv_i32(int32_t *out, const int32_t *in, const int32_t *filt, int64_t D, int64_t H, int64_t W, int64_t Cw,
+                int64_t O, int fx, int fy, int px, int py, int sx, int sy, nb_stream_t s)
+{
+    return nb::conv_impl<uint32_t>(out, W32(in), W32(filt), nullptr, D, H, W, Cw, O, fx, fy, px, py, sx, sy, 0, s,
+                                   "nb_conv_i32");
+}
+int nb_conv_act_i64(uint8_t *out, const int64_t *in, const int64_t *filt, const int32_t *thresh, int64_t D, int64_t H,
+                    int64_t W, int64_t Cw, int64_t O, int fx, int fy, int px, int py, int sx, int sy, nb_stream_t s)
+{
+    return nb::conv_impl<uint64_t>(out, W64(in), W64(filt), thresh, D, H, W, Cw, O, fx, fy, px, py, sx, sy, 1, s,
+                                   "nb_conv_act_i64");
+}
+int nb_conv_act_i32(uint8_t *out, const int32_t *in, const int32_t *filt, const int32_t *thresh, int64_t D, int64_t H,
+                    int64_t W, int64_t Cw, int64_t O, int fx, int fy, int px, int py, int sx, int sy, nb_stream_t s)
+{
+    return nb::conv_impl<uint32_t>(out, W32(in), W32(filt), thresh, D, H, W, Cw, O, fx, fy, px, py, sx, sy, 1, s,
+                                   "nb_conv_act_i32");
+}
+int nb_conv_act_pack_i64(int64_t *out, const int64_t *in, const int64_t *filt, const int32_t *thresh, int64_t D,
+                         int64_t H, int64_t W, int64_t Cw, int64_t O, int fx, int fy, int px, int py, int sx, int sy,
+                         int pool, nb_stream_t s)
+{
+    return nb::conv_impl<uint64_t>(out, W64(in), W64(filt), thresh, D, H, W, Cw, O, fx, fy, px, py, sx, sy,
+                                   pool ? 3 : 2, s, "nb_conv_act_pack_i64");
+}
+int nb_conv_act_pack_i32(int32_t *out, const int32_t *in, const int32_t *filt, const int32_t *thresh, int64_t D,
+                         int64_t H, int64_t W, int64_t Cw, int64_t O, int fx, int fy, int px, int py, int sx, int sy,
+                         int pool, nb_stream_t s)
+{
+    return nb::conv_impl<uint32_t>(out, W32(in), W32(filt), thresh, D, H, W, Cw, O, fx, fy, px, py, sx, sy,
+                                   pool ? 3 : 2, s, "nb_conv_act_pack_i32");
+}
+}

@@ -1,0 +1,186 @@
+// pack / unpack / int8pack: HBM-bound layout conversions between bool bytes and packed words.
+#include "nb_common.hpp"
+
+namespace nb {
+
+// 4 bool bytes of a dword -> 4 bits.  Any non-zero byte counts as 1.
+__device__ __forceinline__ uint32_t nibble_of_bools(uint32_t v)
+{
+    // high bit of every byte := byte != 0
+    const uint32_t nz = (((v & 0x7F7F7F7Fu) + 0x7F7F7F7Fu) | v) & 0x80808080u;
+    const uint32_t t = nz >> 7;                 // b0@0 b1@8 b2@16 b3@24
+    const uint32_t y = (t << 7) | t;            // b0@7 b1@8 ...
+    const uint32_t z = (y << 14) | y;           // b0@21 b1@22 b2@23 b3@24
+    return (z >> 21) & 0xFu;
+}
+
+__device__ __forceinline__ uint32_t bits16_of_bools(uint4 v)
+{
+    return nibble_of_bools(v.x) | (nibble_of_bools(v.y) << 4) | (nibble_of_bools(v.z) << 8) |
+           (nibble_of_bools(v.w) << 12);
+}
+
+// One thread per output word, 16-byte loads.  Requires C % 16 == 0 and a 16-byte aligned input,
+// so every 16-byte chunk lies inside one row.
+template <typename W>
+__global__ __launch_bounds__(256) void pack_vec16_kernel(W *__restrict__ out, const uint8_t *__restrict__ in,
+                                                         int64_t total_words, int Rw, int64_t C)
+{
+    constexpr int bits = WordTraits<W>::bits;
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= total_words) return;
+    const int64_t row = t / Rw;
+    const int y = (int)(t - row * Rw);
+    const int64_t col0 = (int64_t)y * bits;
+    const uint4 *src = reinterpret_cast<const uint4 *>(in + row * C + col0);
+    int64_t left = C - col0;
+    const int chunks = (int)((left < bits ? left : bits) >> 4);
+    W w = 0;
+#pragma unroll
+    for (int c = 0; c < bits / 16; c++) {
+        if (c < chunks) w |= (W)bits16_of_bools(src[c]) << (16 * c);
+    }
+    out[t] = w;
+}
+
+// Generic: one thread per output word, byte loads, any C.
+template <typename W>
+__global__ __launch_bounds__(256) void pack_generic_kernel(W *__restrict__ out, const uint8_t *__restrict__ in,
+                                                           int64_t total_words, int Rw, int64_t C)
+{
+    constexpr int bits = WordTraits<W>::bits;
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= total_words) return;
+    const int64_t row = t / Rw;
+    const int y = (int)(t - row * Rw);
+    const int64_t col0 = (int64_t)y * bits;
+    const uint8_t *src = in + row * C + col0;
+    int64_t left = C - col0;
+    const int nb_ = (int)(left < bits ? left : bits);
+    W w = 0;
+    for (int i = 0; i < nb_; i++) w |= (W)(src[i] != 0) << i;
+    out[t] = w;
+}
+
+// One thread per 16 output bytes (16 bits of a word).
+template <typename W>
+__global__ __launch_bounds__(256) void unpack_kernel(uint8_t *__restrict__ out, const W *__restrict__ in,
+                                                     int64_t total_chunks)
+{
+    constexpr int bits = WordTraits<W>::bits;
+    constexpr int per = bits / 16;
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= total_chunks) return;
+    const W w = in[t / per];
+    const uint32_t h = (uint32_t)(w >> (16 * (int)(t % per))) & 0xFFFFu;
+    uint32_t d[4];
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        const uint32_t nib = (h >> (4 * q)) & 0xFu;
+        d[q] = (nib * 0x00204081u) & 0x01010101u;   // bit j -> byte j
+    }
+    reinterpret_cast<uint4 *>(out)[t] = make_uint4(d[0], d[1], d[2], d[3]);
+}
+
+template <typename W>
+__global__ __launch_bounds__(256) void int8pack_kernel(W *__restrict__ out, const uint8_t *__restrict__ in,
+                                                       int64_t total_words, int Rw, int64_t C)
+{
+    constexpr int per = WordTraits<W>::bits / 8;
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= total_words) return;
+    const int64_t row = t / Rw;
+    const int y = (int)(t - row * Rw);
+    const int64_t col0 = (int64_t)y * per;
+    const uint8_t *src = in + row * C + col0;
+    int64_t left = C - col0;
+    const int nb_ = (int)(left < per ? left : per);
+    W w = 0;
+    for (int i = 0; i < nb_; i++) w |= (W)src[i] << (8 * i);
+    out[t] = w;
+}
+
+template <typename W>
+int pack_impl(W *out, const uint8_t *in, int64_t R, int64_t C, nb_stream_t stream, const char *who)
+{
+    constexpr int bits = WordTraits<W>::bits;
+    NB_REQUIRE(R >= 0 && C >= 0, "%s: negative shape R=%lld C=%lld", who, (long long)R, (long long)C);
+    const int64_t Rw = ceil_div(C, bits);
+    const int64_t total = R * Rw;
+    if (total == 0) return NB_OK;
+    NB_REQUIRE_PTR(out);
+    NB_REQUIRE_PTR(in);
+    NB_REQUIRE_ALIGNED(out, sizeof(W));
+    NB_REQUIRE(Rw <= 2147483647LL, "%s: row of %lld words is too long", who, (long long)Rw);
+    const int64_t blocks = ceil_div(total, 256);
+    NB_REQUIRE(blocks <= kMaxGridX, "%s: %lld output words exceed one launch", who, (long long)total);
+    if ((C & 15) == 0 && aligned(in, 16))
+        pack_vec16_kernel<W><<<dim3((unsigned)blocks), dim3(256), 0, as_stream(stream)>>>(out, in, total, (int)Rw, C);
+    else
+        pack_generic_kernel<W><<<dim3((unsigned)blocks), dim3(256), 0, as_stream(stream)>>>(out, in, total, (int)Rw, C);
+    return check_launch(who);
+}
+
+template <typename W>
+int unpack_impl(uint8_t *out, const W *in, int64_t R, int64_t Rw, nb_stream_t stream, const char *who)
+{
+    constexpr int bits = WordTraits<W>::bits;
+    NB_REQUIRE(R >= 0 && Rw >= 0, "%s: negative shape R=%lld Rw=%lld", who, (long long)R, (long long)Rw);
+    const int64_t chunks = R * Rw * (bits / 16);
+    if (chunks == 0) return NB_OK;
+    NB_REQUIRE_PTR(out);
+    NB_REQUIRE_PTR(in);
+    NB_REQUIRE_ALIGNED(in, sizeof(W));
+    NB_REQUIRE_ALIGNED(out, 16);
+    const int64_t blocks = ceil_div(chunks, 256);
+    NB_REQUIRE(blocks <= kMaxGridX, "%s: %lld words exceed one launch", who, (long long)(R * Rw));
+    unpack_kernel<W><<<dim3((unsigned)blocks), dim3(256), 0, as_stream(stream)>>>(out, in, chunks);
+    return check_launch(who);
+}
+
+template <typename W>
+int int8pack_impl(W *out, const uint8_t *in, int64_t R, int64_t C, nb_stream_t stream, const char *who)
+{
+    constexpr int per = WordTraits<W>::bits / 8;
+    NB_REQUIRE(R >= 0 && C >= 0, "%s: negative shape R=%lld C=%lld", who, (long long)R, (long long)C);
+    const int64_t Rw = ceil_div(C, per);
+    const int64_t total = R * Rw;
+    if (total == 0) return NB_OK;
+    NB_REQUIRE_PTR(out);
+    NB_REQUIRE_PTR(in);
+    NB_REQUIRE_ALIGNED(out, sizeof(W));
+    NB_REQUIRE(Rw <= 2147483647LL, "%s: row of %lld words is too long", who, (long long)Rw);
+    const int64_t blocks = ceil_div(total, 256);
+    NB_REQUIRE(blocks <= kMaxGridX, "%s: %lld output words exceed one launch", who, (long long)total);
+    int8pack_kernel<W><<<dim3((unsigned)blocks), dim3(256), 0, as_stream(stream)>>>(out, in, total, (int)Rw, C);
+    return check_launch(who);
+}
+
+}  // namespace nb
+
+extern "C" {
+int nb_pack_i64(int64_t *out, const uint8_t *in, int64_t R, int64_t C, nb_stream_t s)
+{
+    return nb::pack_impl<uint64_t>(reinterpret_cast<uint64_t *>(out), in, R, C, s, "nb_pack_i64");
+}
+int nb_pack_i32(int32_t *out, const uint8_t *in, int64_t R, int64_t C, nb_stream_t s)
+{
+    return nb::pack_impl<uint32_t>(reinterpret_cast<uint32_t *>(out), in, R, C, s, "nb_pack_i32");
+}
+int nb_unpack_i64(uint8_t *out, const int64_t *in, int64_t R, int64_t Rw, nb_stream_t s)
+{
+    return nb::unpack_impl<uint64_t>(out, reinterpret_cast<const uint64_t *>(in), R, Rw, s, "nb_unpack_i64");
+}
+int nb_unpack_i32(uint8_t *out, const int32_t *in, int64_t R, int64_t Rw, nb_stream_t s)
+{
+    return nb::unpack_impl<uint32_t>(out, reinterpret_cast<const uint32_t *>(in), R, Rw, s, "nb_unpack_i32");
+}
+int nb_int8pack_i64(int64_t *out, const uint8_t *in, int64_t R, int64_t C, nb_stream_t s)
+{
+    return nb::int8pack_impl<uint64_t>(reinterpret_cast<uint64_t *>(out), in, R, C, s, "nb_int8pack_i64");
+}
+int nb_int8pack_i32(int32_t *out, const uint8_t *in, int64_t R, int64_t C, nb_stream_t s)
+{
+    return nb::int8pack_impl<uint32_t>(reinterpret_cast<uint32_t *>(out), in, R, C, s, "nb_int8pack_i32");
+}
+}

@@ -1,0 +1,234 @@
+// "Row per lane" XOR-popcount tile kernel shared by bmm and the implicit-im2col conv.
+//
+// Mapping: one lane owns one row x of the product (an output pixel for conv) and keeps that
+// row's packed words a[k] in VGPRs.  All lanes of a workgroup belong to the same member z, so
+// the second operand B[z,k,y] is wave-uniform: the compiler fetches it with scalar loads and
+// feeds it to v_xor_b32 as an SGPR operand -- no LDS staging and no per-lane traffic for B.
+// Per 64-bit word and output the VALU work is 2 v_xor_b32 + 2 accumulating v_bcnt_u32_b32.
+#pragma once
+#include "nb_common.hpp"
+
+namespace nb {
+
+// ---- A-operand loaders ---------------------------------------------------------------------
+// Explicit rows: A [Z, M, Kw].
+template <typename W>
+struct RowsA {
+    const W *__restrict__ A;
+    int64_t M;
+    int Kw;
+    struct Lane {
+        const W *row;
+        bool valid;
+    };
+    __device__ __forceinline__ Lane lane(int64_t z, int64_t m) const
+    {
+        Lane l;
+        l.valid = m < M;
+        l.row = A + (z * M + (l.valid ? m : 0)) * Kw;
+        return l;
+    }
+    template <int KC>
+    __device__ __forceinline__ void load(const Lane &l, int k0, W (&a)[KC]) const
+    {
+#pragma unroll
+        for (int i = 0; i < KC; i++) a[i] = (l.valid && k0 + i < Kw) ? l.row[k0 + i] : (W)0;
+    }
+};
+
+// Implicit im2col: input [D, H, W, Cw]; word k of output pixel (yo, xo) is channel word k%Cw
+// of tap k/Cw = i*fy + j at input position (i + yo*sx - px, j + xo*sy - py), zero outside
+// (extensions/src/batch_im2col.cu:14-29).
+struct ConvGeom {
+    int H, Wd, Cw, fx, fy, px, py, sx, sy, h, w;
+};
+
+template <typename W>
+struct ConvA {
+    const W *__restrict__ in;
+    ConvGeom g;
+    struct Lane {
+        const W *img;
+        int y0, x0;
+        bool valid;
+    };
+    // (yo, xo) output pixel of this lane
+    __device__ __forceinline__ Lane lane_at(int64_t z, int yo, int xo, bool valid) const
+    {
+        Lane l;
+        l.valid = valid;
+        l.img = in + z * (int64_t)g.H * g.Wd * g.Cw;
+        l.y0 = yo * g.sx - g.px;
+        l.x0 = xo * g.sy - g.py;
+        return l;
+    }
+    template <int KC>
+    __device__ __forceinline__ void load(const Lane &l, int k0, W (&a)[KC]) const
+    {
+        const int Kw = g.fx * g.fy * g.Cw;
+        // tap counters for k0, then advanced incrementally (all wave-uniform)
+        const int cw = g.Cw > 0 ? g.Cw : 1;
+        int tap = k0 / cw;
+        int c = k0 - tap * cw;
+        int ti = tap / g.fy;
+        int tj = tap - ti * g.fy;
+#pragma unroll
+        for (int i = 0; i < KC; i++) {
+            const int y = l.y0 + ti, x = l.x0 + tj;
+            const bool ok = l.valid && (k0 + i < Kw) && y >= 0 && y < g.H && x >= 0 && x < g.Wd;
+            a[i] = ok ? l.img[((int64_t)y * g.Wd + x) * g.Cw + c] : (W)0;
+            if (++c == g.Cw) {
+                c = 0;
+                if (++tj == g.fy) {
+                    tj = 0;
+                    ++ti;
+                }
+            }
+        }
+    }
+};
+
+// ---- accumulate one K-chunk into an N-tile ----------------------------------------------------
+template <typename W, int KC, int NT>
+__device__ __forceinline__ void mac_chunk(int (&acc)[NT], const W (&a)[KC], const W *__restrict__ Bz, int k0, int Kw,
+                                          int n0, int N)
+{
+    if (n0 + NT <= N) {
+#pragma unroll
+        for (int i = 0; i < KC; i++) {
+            if (k0 + i < Kw) {
+                const W *__restrict__ brow = Bz + (int64_t)(k0 + i) * N + n0;
+#pragma unroll
+                for (int j = 0; j < NT; j++) acc[j] += popc_xor(a[i], brow[j]);
+            }
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < KC; i++) {
+            if (k0 + i < Kw) {
+                const W *__restrict__ brow = Bz + (int64_t)(k0 + i) * N + n0;
+#pragma unroll
+                for (int j = 0; j < NT; j++)
+                    if (n0 + j < N) acc[j] += popc_xor(a[i], brow[j]);
+            }
+        }
+    }
+}
+
+// ---- epilogues -----------------------------------------------------------------------------------
+// int32 popcount sums, C [Z, M, N].
+struct EpiI32 {
+    int32_t *__restrict__ C;
+    bool vec;  // rows are 16-byte aligned and N % 4 == 0: store int4
+    struct State {};
+    template <int NT>
+    __device__ __forceinline__ void tile(State &, int64_t row, bool valid, int64_t z, int n0, int N,
+                                         const int (&acc)[NT]) const
+    {
+        if (!valid) return;
+        int32_t *dst = C + row * N + n0;
+        if (n0 + NT <= N && vec) {
+#pragma unroll
+            for (int j = 0; j < NT; j += 4)
+                *reinterpret_cast<int4 *>(dst + j) = make_int4(acc[j], acc[j + 1], acc[j + 2], acc[j + 3]);
+        } else {
+#pragma unroll
+            for (int j = 0; j < NT; j++)
+                if (n0 + j < N) dst[j] = acc[j];
+        }
+    }
+    __device__ __forceinline__ void finish(State &, int64_t, bool) const {}
+};
+
+// bool bytes (2*popc > thresh[z,y]), C [Z, M, N]   (extensions/src/bmm_act.cu:56)
+struct EpiBool {
+    uint8_t *__restrict__ C;
+    const int32_t *__restrict__ thresh;
+    bool vec;  // rows are 4-byte aligned and N % 4 == 0: store four bools per dword
+    struct State {};
+    template <int NT>
+    __device__ __forceinline__ void tile(State &, int64_t row, bool valid, int64_t z, int n0, int N,
+                                         const int (&acc)[NT]) const
+    {
+        const int32_t *__restrict__ t = thresh + z * N + n0;
+        uint8_t *dst = C + row * N + n0;
+        if (n0 + NT <= N && vec) {
+#pragma unroll
+            for (int j = 0; j < NT; j += 4) {
+                uint32_t v = 0;
+#pragma unroll
+                for (int q = 0; q < 4; q++) v |= (uint32_t)(2 * acc[j + q] > t[j + q]) << (8 * q);
+                if (valid) *reinterpret_cast<uint32_t *>(dst + j) = v;
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < NT; j++)
+                if (n0 + j < N && valid) dst[j] = (uint8_t)(2 * acc[j] > t[j]);
+        }
+    }
+    __device__ __forceinline__ void finish(State &, int64_t, bool) const {}
+};
+
+// Threshold bits packed along y into words, out [rows, Ow]; with POOL the four lanes of a quad
+// hold the 2x2 window of one pooled pixel and their words are ORed before lane 0 stores
+// (extensions/src/bmm_act.cu:56 + extensions/src/pack.cu:26 + extensions/src/max_pool2d.cu:19-32).
+template <typename W, bool POOL>
+struct EpiPack {
+    W *__restrict__ out;
+    const int32_t *__restrict__ thresh;
+    int Ow;
+    struct State {
+        W cur = 0;
+    };
+    template <int NT>
+    __device__ __forceinline__ void tile(State &st, int64_t row, bool valid, int64_t z, int n0, int N,
+                                         const int (&acc)[NT]) const
+    {
+        constexpr int bits = WordTraits<W>::bits;
+        static_assert(bits % NT == 0, "an N-tile must not straddle two output words");
+        const int32_t *__restrict__ t = thresh + z * N + n0;
+#pragma unroll
+        for (int j = 0; j < NT; j++)
+            if (n0 + j < N) st.cur |= (W)(2 * acc[j] > t[j]) << ((n0 + j) & (bits - 1));
+        if (((n0 + NT) & (bits - 1)) == 0 || n0 + NT >= N) {
+            W v = valid ? st.cur : (W)0;
+            bool writer = valid;
+            if (POOL) {
+                v |= __shfl_xor(v, 1);
+                v |= __shfl_xor(v, 2);
+                writer = valid && (threadIdx.x & 3) == 0;
+            }
+            if (writer) out[row * Ow + n0 / bits] = v;
+            st.cur = 0;
+        }
+    }
+    __device__ __forceinline__ void finish(State &, int64_t, bool) const {}
+};
+
+// The loop nest shared by every row-per-lane kernel.
+template <typename W, int KC, int NT, bool SINGLE, class ALoad, class Epi>
+__device__ __forceinline__ void rowlane_body(const ALoad &al, const typename ALoad::Lane &lane,
+                                             const W *__restrict__ Bz, const Epi &epi, int64_t orow, int64_t z,
+                                             int Kw, int N)
+{
+    typename Epi::State st;
+    W a[KC];
+    if (SINGLE) al.template load<KC>(lane, 0, a);
+    for (int n0 = 0; n0 < N; n0 += NT) {
+        int acc[NT];
+#pragma unroll
+        for (int j = 0; j < NT; j++) acc[j] = 0;
+        if (SINGLE) {
+            mac_chunk<W, KC, NT>(acc, a, Bz, 0, Kw, n0, N);
+        } else {
+            for (int k0 = 0; k0 < Kw; k0 += KC) {
+                al.template load<KC>(lane, k0, a);
+                mac_chunk<W, KC, NT>(acc, a, Bz, k0, Kw, n0, N);
+            }
+        }
+        epi.template tile<NT>(st, orow, lane.valid, z, n0, N, acc);
+    }
+    epi.finish(st, orow, lane.valid);
+}
+
+}  // namespace nb

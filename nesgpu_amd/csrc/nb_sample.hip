@@ -1,0 +1,348 @@
+// Bernoulli bit sampling by threshold compare, materialised ([n,R,Rw] packed words) or fused into
+// the XOR-popcount matrix-vector product so the per-member weights never reach memory.
+//
+// The draw for (member m, row r, column c) is one uint32 word: either words[(m*R+r)*C+c]
+// (supplied) or word first+(m*R+r)*C+c of a Philox4x32-10 stream.  The supplied stream is
+// 4 bytes per weight bit, so these kernels are HBM-bound on it: lanes read it with 16-byte
+// loads at consecutive addresses and every word is touched exactly once.
+#include "nb_common.hpp"
+
+namespace nb {
+
+struct WordsSrc {
+    const uint32_t *__restrict__ p;
+    // four words starting at flat index g (g % 4 == 0, p 16-byte aligned)
+    __device__ __forceinline__ uint4 load4(int64_t g) const { return *reinterpret_cast<const uint4 *>(p + g); }
+    __device__ __forceinline__ uint32_t load1(int64_t g) const { return p[g]; }
+};
+
+struct PhiloxSrc {
+    PhiloxKey key;
+    // (first + g) % 4 == 0 is guaranteed by the host for load4
+    __device__ __forceinline__ uint4 load4(int64_t g) const { return philox_block(key, (key.first + (uint64_t)g) >> 2); }
+    __device__ __forceinline__ uint32_t load1(int64_t g) const { return philox_word(key, key.first + (uint64_t)g); }
+};
+
+// threshold of columns c..c+3 of row r
+__device__ __forceinline__ uint4 thr4(const uint32_t *__restrict__ thresh, uint32_t ts, int64_t idx)
+{
+    return thresh ? *reinterpret_cast<const uint4 *>(thresh + idx) : make_uint4(ts, ts, ts, ts);
+}
+
+__device__ __forceinline__ uint32_t nibble_lt(uint4 w, uint4 t)
+{
+    return (uint32_t)(w.x < t.x) | ((uint32_t)(w.y < t.y) << 1) | ((uint32_t)(w.z < t.z) << 2) |
+           ((uint32_t)(w.w < t.w) << 3);
+}
+
+// ---- materialised sampler, wide path: C % bits == 0 and 16-byte aligned streams ------------------
+// One lane per 4 columns; bits/4 neighbouring lanes assemble one output word by OR-ing their
+// shifted nibbles across the lane group.
+template <typename W, class Src>
+__global__ __launch_bounds__(256) void sample_wide_kernel(W *__restrict__ out, const W *__restrict__ base,
+                                                          const uint32_t *__restrict__ thresh, uint32_t ts, Src src,
+                                                          int64_t total_quads, int64_t RC4, int C4)
+{
+    constexpr int bits = WordTraits<W>::bits;
+    constexpr int G = bits / 4;  // lanes per output word
+    const int64_t q = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const bool live = q < total_quads;
+    W v = 0;
+    int64_t rq = 0;
+    if (live) {
+        rq = q % RC4;  // quad index inside one member: row * C4 + c4
+        const uint4 w = src.load4(q * 4);
+        const uint4 t = thr4(thresh, ts, rq * 4);
+        v = (W)nibble_lt(w, t) << (4 * (int)(q & (G - 1)));
+    }
+#pragma unroll
+    for (int off = 1; off < G; off <<= 1) v |= __shfl_xor(v, off);
+    if (live && (q & (G - 1)) == 0) {
+        const int64_t wi = q / G;  // flat output word index (C % bits == 0)
+        if (base) v ^= base[rq / G];
+        out[wi] = v;
+    }
+}
+
+// ---- materialised sampler, generic path: one wave per (member,row), ballot builds the words ------
+template <typename W, class Src>
+__global__ __launch_bounds__(256) void sample_ballot_kernel(W *__restrict__ out, const W *__restrict__ base,
+                                                            const uint32_t *__restrict__ thresh, uint32_t ts, Src src,
+                                                            int64_t nrows, int64_t R, int C, int Rw)
+{
+    constexpr int bits = WordTraits<W>::bits;
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);  // (m, r) flattened
+    if (row >= nrows) return;                                          // wave-uniform exit
+    const int64_t r = row % R;
+    for (int c0 = 0; c0 < C; c0 += 64) {
+        const int c = c0 + lane;
+        bool bit = false;
+        if (c < C) {
+            const uint32_t t = thresh ? thresh[r * C + c] : ts;
+            bit = src.load1(row * C + c) < t;
+        }
+        const uint64_t m = __ballot(bit);
+        if (lane == 0) {
+            if (bits == 64) {
+                const int wi = c0 >> 6;
+                out[row * Rw + wi] = (W)m ^ (base ? base[r * Rw + wi] : (W)0);
+            } else {
+                const int wi = c0 >> 5;
+                out[row * Rw + wi] = (W)m ^ (base ? base[r * Rw + wi] : (W)0);
+                if (wi + 1 < Rw) out[row * Rw + wi + 1] = (W)(m >> 32) ^ (base ? base[r * Rw + wi + 1] : (W)0);
+            }
+        }
+    }
+}
+
+// ---- fused sample + XOR-popcount matrix-vector product -------------------------------------------------
+// Wide path (C % 4 == 0, aligned streams): one wave per RPW consecutive rows of one member; lane
+// l covers columns 4*(l+64*it)..+3.  The lane XORs its 4 sampled bits with the matching nibbles
+// of base[r] and x[m] and counts; a wave reduction per row finishes the sum.
+template <typename W, class Src, int RPW>
+__global__ __launch_bounds__(256) void seeded_bmv_wide_kernel(int32_t *__restrict__ Cout, const W *__restrict__ base,
+                                                              const uint32_t *__restrict__ thresh, uint32_t ts,
+                                                              const W *__restrict__ x, Src src, int64_t n, int64_t R,
+                                                              int C4, int Rw, int64_t groups_per_member)
+{
+    constexpr int bits = WordTraits<W>::bits;
+    constexpr int G = bits / 4;
+    const int lane = threadIdx.x & 63;
+    const int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int64_t m = wave / groups_per_member;
+    if (m >= n) return;  // wave-uniform
+    const int64_t r0 = (wave - m * groups_per_member) * RPW;
+    int acc[RPW];
+#pragma unroll
+    for (int q = 0; q < RPW; q++) acc[q] = 0;
+    const int64_t C = (int64_t)C4 * 4;
+    for (int c4 = lane; c4 < C4; c4 += 64) {
+        const int wi = c4 / G, sh = 4 * (c4 & (G - 1));
+        const uint32_t xn = (uint32_t)(x[m * Rw + wi] >> sh) & 0xFu;
+#pragma unroll
+        for (int q = 0; q < RPW; q++) {
+            const int64_t r = r0 + q;
+            if (r < R) {
+                const uint4 w = src.load4((m * R + r) * C + 4 * (int64_t)c4);
+                const uint4 t = thr4(thresh, ts, r * C + 4 * (int64_t)c4);
+                uint32_t nib = nibble_lt(w, t) ^ xn;
+                if (base) nib ^= (uint32_t)(base[r * Rw + wi] >> sh) & 0xFu;
+                acc[q] += __popc(nib);
+            }
+        }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+#pragma unroll
+        for (int q = 0; q < RPW; q++) acc[q] += __shfl_xor(acc[q], off);
+    }
+    if (lane == 0) {
+#pragma unroll
+        for (int q = 0; q < RPW; q++)
+            if (r0 + q < R) Cout[m * R + r0 + q] = acc[q];
+    }
+}
+
+// Generic path: one wave per (member,row), one column per lane and step.
+template <typename W, class Src>
+__global__ __launch_bounds__(256) void seeded_bmv_generic_kernel(int32_t *__restrict__ Cout,
+                                                                 const W *__restrict__ base,
+                                                                 const uint32_t *__restrict__ thresh, uint32_t ts,
+                                                                 const W *__restrict__ x, Src src, int64_t nrows,
+                                                                 int64_t R, int C, int Rw)
+{
+    constexpr int lb = WordTraits<W>::log2bits;
+    constexpr int bits = WordTraits<W>::bits;
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= nrows) return;  // wave-uniform
+    const int64_t m = row / R, r = row - m * R;
+    int acc = 0;
+    for (int c = lane; c < C; c += 64) {
+        const uint32_t t = thresh ? thresh[r * C + c] : ts;
+        uint32_t bit = src.load1(row * C + c) < t;
+        const int wi = c >> lb, sh = c & (bits - 1);
+        bit ^= (uint32_t)(x[m * Rw + wi] >> sh) & 1u;
+        if (base) bit ^= (uint32_t)(base[r * Rw + wi] >> sh) & 1u;
+        acc += bit;
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off);
+    if (lane == 0) Cout[row] = acc;
+}
+
+__global__ __launch_bounds__(256) void philox_words_kernel(uint32_t *__restrict__ out, PhiloxKey key, int64_t count)
+{
+    // one thread per aligned block of the stream; head/tail blocks are partial
+    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const uint64_t blk0 = key.first >> 2;
+    const uint64_t blk = blk0 + (uint64_t)t;
+    const uint64_t gbeg = blk << 2;
+    if (gbeg >= key.first + (uint64_t)count) return;
+    const uint4 b = philox_block(key, blk);
+    const uint32_t v[4] = {b.x, b.y, b.z, b.w};
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        const uint64_t g = gbeg + e;
+        if (g >= key.first && g < key.first + (uint64_t)count) out[g - key.first] = v[e];
+    }
+}
+
+template <typename W>
+static int sample_check(const void *out, const W *base, const uint32_t *thresh, int64_t n, int64_t R, int64_t C,
+                        const char *who, bool *empty)
+{
+    NB_REQUIRE(n >= 0 && R >= 0 && C >= 0, "%s: negative shape n=%lld R=%lld C=%lld", who, (long long)n, (long long)R,
+               (long long)C);
+    *empty = (n * R * C == 0);
+    if (*empty) return NB_OK;
+    NB_REQUIRE_PTR(out);
+    NB_REQUIRE(C <= (1 << 30), "%s: C=%lld too large", who, (long long)C);
+    NB_REQUIRE(n * R <= (1LL << 40) && ceil_div(n * R, 4) <= kMaxGridX, "%s: n*R=%lld rows exceed one launch", who,
+               (long long)(n * R));
+    if (base) NB_REQUIRE_ALIGNED(base, sizeof(W));
+    if (thresh) NB_REQUIRE_ALIGNED(thresh, 4);
+    return NB_OK;
+}
+
+template <typename W, class Src>
+int sample_impl(W *out, const W *base, const uint32_t *thresh, uint32_t ts, Src src, bool src_vec_ok, int64_t n,
+                int64_t R, int64_t C, nb_stream_t stream, const char *who)
+{
+    constexpr int bits = WordTraits<W>::bits;
+    bool empty;
+    if (int rc = sample_check<W>(out, base, thresh, n, R, C, who, &empty)) return rc;
+    if (empty) return NB_OK;
+    NB_REQUIRE_ALIGNED(out, sizeof(W));
+    hipStream_t s = as_stream(stream);
+    const int64_t Rw = ceil_div(C, bits);
+    const int64_t quads = n * R * (C / 4);
+    if (C % bits == 0 && src_vec_ok && (!thresh || aligned(thresh, 16)) && ceil_div(quads, 256) <= kMaxGridX) {
+        sample_wide_kernel<W, Src><<<dim3((unsigned)ceil_div(quads, 256)), dim3(256), 0, s>>>(
+            out, base, thresh, ts, src, quads, R * (C / 4), (int)(C / 4));
+    } else {
+        sample_ballot_kernel<W, Src><<<dim3((unsigned)ceil_div(n * R, 4)), dim3(256), 0, s>>>(
+            out, base, thresh, ts, src, n * R, R, (int)C, (int)Rw);
+    }
+    return check_launch(who);
+}
+
+template <typename W, class Src>
+int seeded_bmv_impl(int32_t *Cout, const W *base, const uint32_t *thresh, uint32_t ts, const W *x, Src src,
+                    bool src_vec_ok, int64_t n, int64_t R, int64_t C, nb_stream_t stream, const char *who)
+{
+    constexpr int bits = WordTraits<W>::bits;
+    NB_REQUIRE(n >= 0 && R >= 0 && C >= 0, "%s: negative shape n=%lld R=%lld C=%lld", who, (long long)n, (long long)R,
+               (long long)C);
+    if (n * R == 0) return NB_OK;
+    NB_REQUIRE_PTR(Cout);
+    NB_REQUIRE_ALIGNED(Cout, 4);
+    NB_REQUIRE(C <= (1 << 30), "%s: C=%lld too large", who, (long long)C);
+    NB_REQUIRE(n * R <= (1LL << 40) && ceil_div(n * R, 4) <= kMaxGridX, "%s: n*R=%lld rows exceed one launch", who,
+               (long long)(n * R));
+    if (C > 0) {
+        NB_REQUIRE_PTR(x);
+        NB_REQUIRE_ALIGNED(x, sizeof(W));
+    }
+    if (base) NB_REQUIRE_ALIGNED(base, sizeof(W));
+    if (thresh) NB_REQUIRE_ALIGNED(thresh, 4);
+    hipStream_t s = as_stream(stream);
+    const int64_t Rw = ceil_div(C, bits);
+    constexpr int RPW = 4;
+    if (C > 0 && (C & 3) == 0 && src_vec_ok && (!thresh || aligned(thresh, 16))) {
+        const int64_t gpm = ceil_div(R, RPW);
+        const int64_t waves = n * gpm;
+        seeded_bmv_wide_kernel<W, Src, RPW><<<dim3((unsigned)ceil_div(waves, 4)), dim3(256), 0, s>>>(
+            Cout, base, thresh, ts, x, src, n, R, (int)(C / 4), (int)Rw, gpm);
+    } else {
+        seeded_bmv_generic_kernel<W, Src><<<dim3((unsigned)ceil_div(n * R, 4)), dim3(256), 0, s>>>(
+            Cout, base, thresh, ts, x, src, n * R, R, (int)C, (int)Rw);
+    }
+    return check_launch(who);
+}
+
+}  // namespace nb
+
+using nb::PhiloxSrc;
+using nb::WordsSrc;
+#define U64(p) reinterpret_cast<uint64_t *>(p)
+#define U32(p) reinterpret_cast<uint32_t *>(p)
+#define CU64(p) reinterpret_cast<const uint64_t *>(p)
+#define CU32(p) reinterpret_cast<const uint32_t *>(p)
+
+extern "C" {
+int nb_sample_from_words_i64(int64_t *out, const int64_t *base, const uint32_t *thresh, uint32_t ts,
+                             const uint32_t *words, int64_t n, int64_t R, int64_t C, nb_stream_t s)
+{
+    if (n * R * C > 0 && !words) return nb::fail(NB_ERR_NULL, "nb_sample_from_words_i64: words is NULL");
+    return nb::sample_impl<uint64_t, WordsSrc>(U64(out), CU64(base), thresh, ts, WordsSrc{words},
+                                               nb::aligned(words, 16) && (C & 3) == 0, n, R, C, s,
+                                               "nb_sample_from_words_i64");
+}
+int nb_sample_from_words_i32(int32_t *out, const int32_t *base, const uint32_t *thresh, uint32_t ts,
+                             const uint32_t *words, int64_t n, int64_t R, int64_t C, nb_stream_t s)
+{
+    if (n * R * C > 0 && !words) return nb::fail(NB_ERR_NULL, "nb_sample_from_words_i32: words is NULL");
+    return nb::sample_impl<uint32_t, WordsSrc>(U32(out), CU32(base), thresh, ts, WordsSrc{words},
+                                               nb::aligned(words, 16) && (C & 3) == 0, n, R, C, s,
+                                               "nb_sample_from_words_i32");
+}
+int nb_sample_philox_i64(int64_t *out, const int64_t *base, const uint32_t *thresh, uint32_t ts, uint64_t seed,
+                         uint64_t subseq, uint64_t first, int64_t n, int64_t R, int64_t C, nb_stream_t s)
+{
+    return nb::sample_impl<uint64_t, PhiloxSrc>(U64(out), CU64(base), thresh, ts, PhiloxSrc{{seed, subseq, first}},
+                                                (first & 3) == 0 && (C & 3) == 0, n, R, C, s, "nb_sample_philox_i64");
+}
+int nb_sample_philox_i32(int32_t *out, const int32_t *base, const uint32_t *thresh, uint32_t ts, uint64_t seed,
+                         uint64_t subseq, uint64_t first, int64_t n, int64_t R, int64_t C, nb_stream_t s)
+{
+    return nb::sample_impl<uint32_t, PhiloxSrc>(U32(out), CU32(base), thresh, ts, PhiloxSrc{{seed, subseq, first}},
+                                                (first & 3) == 0 && (C & 3) == 0, n, R, C, s, "nb_sample_philox_i32");
+}
+int nb_philox_words(uint32_t *out, uint64_t seed, uint64_t subseq, uint64_t first, int64_t count, nb_stream_t s)
+{
+    if (count < 0) return nb::fail(NB_ERR_SHAPE, "nb_philox_words: negative count");
+    if (count == 0) return NB_OK;
+    if (!out) return nb::fail(NB_ERR_NULL, "nb_philox_words: out is NULL");
+    if (!nb::aligned(out, 4)) return nb::fail(NB_ERR_ALIGN, "nb_philox_words: out is not 4-byte aligned");
+    const int64_t blocks4 = (int64_t)(((first + (uint64_t)count + 3) >> 2) - (first >> 2));
+    if (nb::ceil_div(blocks4, 256) > nb::kMaxGridX)
+        return nb::fail(NB_ERR_SHAPE, "nb_philox_words: %lld words exceed one launch", (long long)count);
+    nb::philox_words_kernel<<<dim3((unsigned)nb::ceil_div(blocks4, 256)), dim3(256), 0, nb::as_stream(s)>>>(
+        out, nb::PhiloxKey{seed, subseq, first}, count);
+    return nb::check_launch("nb_philox_words");
+}
+int nb_seeded_bmv_from_words_i64(int32_t *C, const int64_t *base, const uint32_t *thresh, uint32_t ts, const int64_t *x,
+                                 const uint32_t *words, int64_t n, int64_t R, int64_t Cbits, nb_stream_t s)
+{
+    if (n * R * Cbits > 0 && !words) return nb::fail(NB_ERR_NULL, "nb_seeded_bmv_from_words_i64: words is NULL");
+    return nb::seeded_bmv_impl<uint64_t, WordsSrc>(C, CU64(base), thresh, ts, CU64(x), WordsSrc{words},
+                                                   nb::aligned(words, 16), n, R, Cbits, s,
+                                                   "nb_seeded_bmv_from_words_i64");
+}
+int nb_seeded_bmv_from_words_i32(int32_t *C, const int32_t *base, const uint32_t *thresh, uint32_t ts, const int32_t *x,
+                                 const uint32_t *words, int64_t n, int64_t R, int64_t Cbits, nb_stream_t s)
+{
+    if (n * R * Cbits > 0 && !words) return nb::fail(NB_ERR_NULL, "nb_seeded_bmv_from_words_i32: words is NULL");
+    return nb::seeded_bmv_impl<uint32_t, WordsSrc>(C, CU32(base), thresh, ts, CU32(x), WordsSrc{words},
+                                                   nb::aligned(words, 16), n, R, Cbits, s,
+                                                   "nb_seeded_bmv_from_words_i32");
+}
+int nb_seeded_bmv_philox_i64(int32_t *C, const int64_t *base, const uint32_t *thresh, uint32_t ts, const int64_t *x,
+                             uint64_t seed, uint64_t subseq, uint64_t first, int64_t n, int64_t R, int64_t Cbits,
+                             nb_stream_t s)
+{
+    return nb::seeded_bmv_impl<uint64_t, PhiloxSrc>(C, CU64(base), thresh, ts, CU64(x),
+                                                    PhiloxSrc{{seed, subseq, first}}, (first & 3) == 0, n, R, Cbits, s,
+                                                    "nb_seeded_bmv_philox_i64");
+}
+int nb_seeded_bmv_philox_i32(int32_t *C, const int32_t *base, const uint32_t *thresh, uint32_t ts, const int32_t *x,
+                             uint64_t seed, uint64_t subseq, uint64_t first, int64_t n, int64_t R, int64_t Cbits,
+                             nb_stream_t s)
+{
+    return nb::seeded_bmv_impl<uint32_t, PhiloxSrc>(C, CU32(base), thresh, ts, CU32(x),
+                                                    PhiloxSrc{{seed, subseq, first}}, (first & 3) == 0, n, R, Cbits, s,
+                                                    "nb_seeded_bmv_philox_i32");
+}
+}

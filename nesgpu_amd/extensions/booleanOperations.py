@@ -1,0 +1,413 @@
+"""Drop-in replacement for the reference's ``extensions/booleanOperations.py``.
+
+Same function names, positional order, defaults and return shapes/dtypes as the reference module
+(extensions/booleanOperations.py:82-252), but every op is one call into libnesbin.so -- hand-written
+gfx950 kernels behind the C ABI of include/nesbin.h -- on the CURRENT torch stream (the reference
+captures the stream once at import, extensions/booleanOperations.py:3-4).  Nothing is compiled or read
+from disk at import, and there is no CPU path: tensors must live on the GPU.
+
+Error behaviour follows the reference: shape/rank mistakes raise ``AssertionError``
+(extensions/booleanOperations.py:108-111,132-138,176,204,219-220,233), an unsupported word dtype raises
+``TypeError`` (what ``raise NotImplemented`` at :28,80 surfaces as), and -- from the torch-extension
+half of the reference (extensions/booleanOperations.cpp:13-15) -- non-CUDA or non-contiguous inputs raise
+``RuntimeError`` instead of being read through a wrong stride.
+
+Additions that the reference lacks are grouped at the end (supplied-word / Philox sampling, the fused
+sample+popcount product with a flip base, the fused conv->threshold->pack(->pool) op).
+"""
+import torch
+
+from .. import _lib
+
+__all__ = [
+    "batch_im2col", "bmm", "bmm_act", "conv", "conv_act", "pack", "int8pack", "sample_bits", "weighted_sum",
+    "max_pool2d", "next_pow2_clip", "ceil_div", "unpack", "thresholds_from_p", "sample_bits_from_words",
+    "flip_from_words", "sample_bits_philox", "flip_philox", "seeded_bmv_from_words", "seeded_bmv_philox",
+    "philox_words", "conv_act_pack",
+]
+
+
+def next_pow2_clip(v, cap):
+    """Launch-shape helper kept for API parity (extensions/booleanOperations.py:57-67)."""
+    if v > cap // 2:
+        return cap
+    p = 1
+    while p < v:
+        p *= 2
+    return p
+
+
+def ceil_div(a, b):
+    return (a + b - 1) // b
+
+
+# --------------------------------------------------------------------------------------------
+def _suffix(dtype):
+    if dtype == torch.int64:
+        return "_i64", 64
+    if dtype == torch.int32:
+        return "_i32", 32
+    # the reference executes `raise NotImplemented`, which Python turns into a TypeError
+    raise TypeError("packed word dtype must be torch.int64 or torch.int32, got %r" % (dtype,))
+
+
+def _check(t, name):
+    if not isinstance(t, torch.Tensor):
+        raise TypeError("%s must be a torch.Tensor" % name)
+    if not t.is_cuda:
+        raise RuntimeError("%s must be a CUDA tensor" % name)       # booleanOperations.cpp:13
+    if not t.is_contiguous():
+        raise RuntimeError("%s must be contiguous" % name)           # booleanOperations.cpp:14
+    return t
+
+
+def _same_device(a, b):
+    if a.device != b.device:
+        raise RuntimeError("Tensors are on different devices")       # booleanOperations.cpp:39
+
+
+def _stream(t):
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _out_hw(inp, filterx, filtery, padx, pady, stridex, stridey):
+    h = (inp.size(1) - filterx + 2 * padx) // stridex + 1
+    w = (inp.size(2) - filtery + 2 * pady) // stridey + 1
+    return h, w
+
+
+# ---- reference API ----------------------------------------------------------------------------
+def batch_im2col(input, filterx, filtery, padx, pady, stridex, stridey, REPEAT=128):
+    """[B,H,W,Cw] -> [B, h*w, filterx*filtery*Cw] (extensions/booleanOperations.py:82-102).
+    ``REPEAT`` was a launch-shape knob of the reference kernel; accepted and ignored."""
+    _check(input, "input")
+    assert len(input.shape) == 4
+    suf, _ = _suffix(input.dtype)
+    h, w = _out_hw(input, filterx, filtery, padx, pady, stridex, stridey)
+    out = torch.empty((input.size(0), h * w, filterx * filtery * input.size(3)), dtype=input.dtype,
+                      device=input.device)
+    with torch.cuda.device(input.device):
+        _lib.call("nb_im2col" + suf, out.data_ptr(), input.data_ptr(), input.size(0), input.size(1), input.size(2),
+                  input.size(3), filterx, filtery, padx, pady, stridex, stridey, _stream(input))
+    return out
+
+
+def bmm(A, B):
+    """C[z,x,y] = sum_k popcount(A[z,x,k] ^ B[z,k,y]), int32 (extensions/booleanOperations.py:107-129)."""
+    assert len(A.shape) == 3
+    assert len(B.shape) == 3
+    assert A.size(0) == B.size(0)
+    assert A.size(2) == B.size(1)
+    _check(A, "A")
+    _check(B, "B")
+    _same_device(A, B)
+    assert A.dtype == B.dtype
+    suf, _ = _suffix(A.dtype)
+    C = torch.empty((A.size(0), A.size(1), B.size(2)), dtype=torch.int32, device=A.device)
+    with torch.cuda.device(A.device):
+        _lib.call("nb_bmm" + suf, C.data_ptr(), A.data_ptr(), B.data_ptr(), A.size(0), A.size(1), A.size(2), B.size(2),
+                  _stream(A))
+    return C
+
+
+def bmm_act(A, B, threshold):
+    """bool = 2*popc > threshold[z,y] (extensions/booleanOperations.py:131-158)."""
+    assert len(A.shape) == 3
+    assert len(B.shape) == 3
+    assert len(threshold.shape) == 2
+    assert A.size(0) == B.size(0) == threshold.size(0)
+    assert A.size(2) == B.size(1)
+    assert threshold.size(1) == B.size(2)
+    assert threshold.dtype == torch.int32
+    _check(A, "A")
+    _check(B, "B")
+    _check(threshold, "threshold")
+    _same_device(A, B)
+    _same_device(A, threshold)
+    assert A.dtype == B.dtype
+    suf, _ = _suffix(A.dtype)
+    C = torch.empty((A.size(0), A.size(1), B.size(2)), dtype=torch.bool, device=A.device)
+    with torch.cuda.device(A.device):
+        _lib.call("nb_bmm_act" + suf, C.data_ptr(), A.data_ptr(), B.data_ptr(), threshold.data_ptr(), A.size(0),
+                  A.size(1), A.size(2), B.size(2), _stream(A))
+    return C
+
+
+def _conv_args(input, filter, filterx, filtery):
+    _check(input, "input")
+    _check(filter, "filter")
+    _same_device(input, filter)
+    assert len(input.shape) == 4
+    assert len(filter.shape) == 3
+    assert input.size(0) == filter.size(0)                       # "Batch dim doesn't match", booleanOperations.cpp:46
+    assert input.dtype == filter.dtype                           # booleanOperations.cpp:48
+    assert filter.size(1) == filterx * filtery * input.size(3)   # the bmm contraction assert (:111)
+    return _suffix(input.dtype)
+
+
+def conv(input, filter, filterx, filtery, padx, pady, stridex, stridey):
+    """bmm(batch_im2col(input), filter).view(D,h,w,O) without materialising the columns
+    (extensions/booleanOperations.py:162-166).  filter is [D, filterx*filtery*Cw, O]."""
+    suf, _ = _conv_args(input, filter, filterx, filtery)
+    h, w = _out_hw(input, filterx, filtery, padx, pady, stridex, stridey)
+    out = torch.empty((input.size(0), h, w, filter.size(2)), dtype=torch.int32, device=input.device)
+    with torch.cuda.device(input.device):
+        _lib.call("nb_conv" + suf, out.data_ptr(), input.data_ptr(), filter.data_ptr(), input.size(0), input.size(1),
+                  input.size(2), input.size(3), filter.size(2), filterx, filtery, padx, pady, stridex, stridey,
+                  _stream(input))
+    return out
+
+
+def conv_act(input, filter, threshold, filterx, filtery, padx, pady, stridex, stridey):
+    """bmm_act(batch_im2col(input), filter, threshold).view(D,h,w,O) (extensions/booleanOperations.py:168-172)."""
+    suf, _ = _conv_args(input, filter, filterx, filtery)
+    _check(threshold, "threshold")
+    _same_device(input, threshold)
+    assert len(threshold.shape) == 2
+    assert threshold.size(0) == input.size(0)
+    assert threshold.size(1) == filter.size(2)
+    assert threshold.dtype == torch.int32
+    h, w = _out_hw(input, filterx, filtery, padx, pady, stridex, stridey)
+    out = torch.empty((input.size(0), h, w, filter.size(2)), dtype=torch.bool, device=input.device)
+    with torch.cuda.device(input.device):
+        _lib.call("nb_conv_act" + suf, out.data_ptr(), input.data_ptr(), filter.data_ptr(), threshold.data_ptr(),
+                  input.size(0), input.size(1), input.size(2), input.size(3), filter.size(2), filterx, filtery, padx,
+                  pady, stridex, stridey, _stream(input))
+    return out
+
+
+def pack(input, dtype=torch.int32):
+    """bool [R,C] -> words [R, ceil(C/bits)], LSB first (extensions/booleanOperations.py:175-187).
+    The default word type is int32, as in the reference; the layers pass int64."""
+    assert len(input.shape) == 2
+    _check(input, "input")
+    if input.dtype != torch.bool:
+        raise TypeError("pack expects a torch.bool tensor, got %r" % (input.dtype,))
+    suf, bits = _suffix(dtype)
+    ret = torch.empty((input.size(0), ceil_div(input.shape[1], bits)), dtype=dtype, device=input.device)
+    with torch.cuda.device(input.device):
+        _lib.call("nb_pack" + suf, ret.data_ptr(), input.data_ptr(), input.size(0), input.size(1), _stream(input))
+    return ret
+
+
+def int8pack(input, dtype=torch.int32):
+    """uint8 [R,C] -> words [R, ceil(C/(bits/8))], little-endian bytes (extensions/booleanOperations.py:189-201)."""
+    assert len(input.shape) == 2
+    _check(input, "input")
+    if input.dtype not in (torch.uint8, torch.int8):
+        raise TypeError("int8pack expects a uint8 tensor, got %r" % (input.dtype,))
+    suf, bits = _suffix(dtype)
+    ret = torch.empty((input.size(0), ceil_div(input.shape[1], bits // 8)), dtype=dtype, device=input.device)
+    with torch.cuda.device(input.device):
+        _lib.call("nb_int8pack" + suf, ret.data_ptr(), input.data_ptr(), input.size(0), input.size(1), _stream(input))
+    return ret
+
+
+def sample_bits(p, n, dtype, seed):
+    """ret[m,r,z] bit i = Bernoulli(p[r, z*bits+i]), n independent members
+    (extensions/booleanOperations.py:203-215, extensions/src/sample_bits.cu:47-57).
+
+    Same law, layout and tail rule as the reference; the random stream is Philox4x32-10 keyed by
+    ``seed`` instead of cuRAND XORWOW (whose exact bitstream no reference test pins)."""
+    assert len(p.shape) == 2
+    return sample_bits_philox(thresholds_from_p(p), n, dtype, seed)
+
+
+def weighted_sum(input, weights, zbits):
+    """ret[r,z] = fp16(sum_m weights[m] * bit(input[m,r,z/bits], z%bits)), fp32 accumulation
+    (extensions/booleanOperations.py:218-229, extensions/src/weighted_sum.cu:28-46)."""
+    assert len(input.shape) == 3
+    assert input.size(0) == weights.size(0)
+    _check(input, "input")
+    _check(weights, "weights")
+    _same_device(input, weights)
+    assert weights.dtype == torch.float16 and len(weights.shape) == 1
+    suf, bits = _suffix(input.dtype)
+    assert zbits <= input.size(2) * bits
+    ret = torch.empty((input.size(1), zbits), dtype=torch.float16, device=input.device)
+    with torch.cuda.device(input.device):
+        _lib.call("nb_weighted_sum" + suf, ret.data_ptr(), input.data_ptr(), weights.data_ptr(), input.size(0),
+                  input.size(1), input.size(2), zbits, _stream(input))
+    return ret
+
+
+def max_pool2d(input, filterx, filtery, padx, pady, stridex, stridey, REPEAT=128):
+    """[D,H,W,Cw] -> [D,h,w,Cw], bitwise OR over a 2x2 window (extensions/booleanOperations.py:232-252).
+    As in the reference kernel the window is always 2x2 (extensions/src/max_pool2d.cu:21-23); filterx and
+    filtery only enter the output size.  ``REPEAT`` is accepted and ignored."""
+    assert len(input.shape) == 4
+    _check(input, "input")
+    suf, _ = _suffix(input.dtype)
+    h, w = _out_hw(input, filterx, filtery, padx, pady, stridex, stridey)
+    out = torch.empty((input.size(0), h, w, input.size(3)), dtype=input.dtype, device=input.device)
+    with torch.cuda.device(input.device):
+        _lib.call("nb_max_pool2d" + suf, out.data_ptr(), input.data_ptr(), input.size(0), input.size(1), input.size(2),
+                  input.size(3), filterx, filtery, padx, pady, stridex, stridey, _stream(input))
+    return out
+
+
+# ---- additions ----------------------------------------------------------------------------------
+def unpack(input):
+    """words [R,Rw] -> bool [R, Rw*bits] (boolutil_cuda.unpack, extensions/booleanUtilitiesCuda.cu:77-90,182-195)."""
+    assert len(input.shape) == 2
+    _check(input, "input")
+    suf, bits = _suffix(input.dtype)
+    ret = torch.empty((input.size(0), input.size(1) * bits), dtype=torch.bool, device=input.device)
+    with torch.cuda.device(input.device):
+        _lib.call("nb_unpack" + suf, ret.data_ptr(), input.data_ptr(), input.size(0), input.size(1), _stream(input))
+    return ret
+
+
+def thresholds_from_p(p):
+    """Probabilities -> uint32 thresholds T with P(word < T) = T / 2**32 ~= p:
+    T = min(floor(p * 2**32), 2**32 - 1), computed exactly in float64.  p = 1.0 therefore fails only
+    for the single word 0xFFFFFFFF, like ``p > u`` with u in (0, 1] in the reference
+    (extensions/src/sample_bits.cu:54)."""
+    t = torch.floor(p.detach().to(torch.float64) * 4294967296.0).clamp_(0.0, 4294967295.0)
+    return t.to(torch.int64).to(torch.uint32)
+
+
+def _thr_args(threshold, R, C, device):
+    """-> (tensor kept alive or None, pointer or None, scalar)"""
+    if isinstance(threshold, torch.Tensor):
+        _check(threshold, "threshold")
+        assert tuple(threshold.shape) == (R, C)
+        if threshold.dtype != torch.uint32:
+            raise TypeError("threshold tensor must be torch.uint32 (see thresholds_from_p)")
+        if threshold.device != device:
+            raise RuntimeError("Tensors are on different devices")
+        return threshold, threshold.data_ptr(), 0
+    t = int(threshold)
+    if not 0 <= t <= 0xFFFFFFFF:
+        raise ValueError("scalar threshold must fit in uint32")
+    return None, None, t
+
+
+def _words_check(words):
+    _check(words, "words")
+    assert len(words.shape) == 3
+    if words.dtype not in (torch.uint32, torch.int32):
+        raise TypeError("random words must be torch.uint32 (or int32 holding the same bit patterns)")
+
+
+def _base_check(base, R, Rw, dtype, device):
+    if base is None:
+        return None
+    _check(base, "base")
+    assert tuple(base.shape) == (R, Rw) and base.dtype == dtype
+    if base.device != device:
+        raise RuntimeError("Tensors are on different devices")
+    return base.data_ptr()
+
+
+def sample_bits_from_words(threshold, words, dtype, base=None):
+    """ret[m,r,z] bit i = words[m,r,z*bits+i] < threshold[r,z*bits+i]  (threshold: uint32 [R,C] tensor or a
+    Python int); with ``base`` ([R,Rw] packed) the result is ``base ^ mask``."""
+    _words_check(words)
+    suf, bits = _suffix(dtype)
+    n, R, C = words.shape
+    keep, tptr, ts = _thr_args(threshold, R, C, words.device)
+    Rw = ceil_div(C, bits)
+    bptr = _base_check(base, R, Rw, dtype, words.device)
+    ret = torch.empty((n, R, Rw), dtype=dtype, device=words.device)
+    with torch.cuda.device(words.device):
+        _lib.call("nb_sample_from_words" + suf, ret.data_ptr(), bptr, tptr, ts, words.data_ptr(), n, R, C,
+                  _stream(words))
+    return ret
+
+
+def flip_from_words(base_packed, words, threshold):
+    """Per-member weights = base XOR Bernoulli flip mask: ret[m] = base ^ pack(words[m] < threshold)."""
+    return sample_bits_from_words(threshold, words, base_packed.dtype, base=base_packed)
+
+
+def sample_bits_philox(threshold, n, dtype, seed, subsequence=0, first=0, base=None, shape=None):
+    """Like :func:`sample_bits_from_words` with the words generated in-kernel: word (m,r,c) is element
+    ``first + (m*R+r)*C + c`` of the Philox4x32-10 stream (seed, subsequence) -- exactly what
+    :func:`philox_words` returns, so both forms agree bit for bit."""
+    suf, bits = _suffix(dtype)
+    if isinstance(threshold, torch.Tensor):
+        R, C = threshold.shape
+        device = threshold.device
+    else:
+        R, C = shape
+        device = base.device if base is not None else torch.device("cuda", torch.cuda.current_device())
+    keep, tptr, ts = _thr_args(threshold, R, C, device)
+    Rw = ceil_div(C, bits)
+    bptr = _base_check(base, R, Rw, dtype, device)
+    ret = torch.empty((n, R, Rw), dtype=dtype, device=device)
+    with torch.cuda.device(device):
+        _lib.call("nb_sample_philox" + suf, ret.data_ptr(), bptr, tptr, ts, int(seed) & (2 ** 64 - 1),
+                  int(subsequence), int(first), n, R, C, torch.cuda.current_stream(device).cuda_stream)
+    return ret
+
+
+def flip_philox(base_packed, in_bits, n, threshold, seed, subsequence=0, first=0):
+    """base XOR in-kernel Philox flip mask; ``in_bits`` is the true column count C of a row."""
+    return sample_bits_philox(threshold, n, base_packed.dtype, seed, subsequence, first, base=base_packed,
+                              shape=(base_packed.size(0), in_bits))
+
+
+def seeded_bmv_from_words(threshold, x_packed, words, base=None):
+    """C[m,r] = sum_k popcount(w(m,r,k) ^ x[m,k]) with w = base ^ (words < threshold) never materialised
+    (the fused op of boolop_cuda.binary_seeded_bmv, extensions/booleanOperationsCuda.cu:172-202)."""
+    _words_check(words)
+    _check(x_packed, "x_packed")
+    suf, bits = _suffix(x_packed.dtype)
+    n, R, C = words.shape
+    Rw = ceil_div(C, bits)
+    assert tuple(x_packed.shape) == (n, Rw)
+    _same_device(words, x_packed)
+    keep, tptr, ts = _thr_args(threshold, R, C, words.device)
+    bptr = _base_check(base, R, Rw, x_packed.dtype, words.device)
+    out = torch.empty((n, R), dtype=torch.int32, device=words.device)
+    with torch.cuda.device(words.device):
+        _lib.call("nb_seeded_bmv_from_words" + suf, out.data_ptr(), bptr, tptr, ts, x_packed.data_ptr(),
+                  words.data_ptr(), n, R, C, _stream(words))
+    return out
+
+
+def seeded_bmv_philox(threshold, x_packed, rows, in_bits, seed, subsequence=0, first=0, base=None):
+    """:func:`seeded_bmv_from_words` with in-kernel Philox words."""
+    _check(x_packed, "x_packed")
+    suf, bits = _suffix(x_packed.dtype)
+    n = x_packed.size(0)
+    R, C = rows, in_bits
+    Rw = ceil_div(C, bits)
+    assert tuple(x_packed.shape) == (n, Rw)
+    keep, tptr, ts = _thr_args(threshold, R, C, x_packed.device)
+    bptr = _base_check(base, R, Rw, x_packed.dtype, x_packed.device)
+    out = torch.empty((n, R), dtype=torch.int32, device=x_packed.device)
+    with torch.cuda.device(x_packed.device):
+        _lib.call("nb_seeded_bmv_philox" + suf, out.data_ptr(), bptr, tptr, ts, x_packed.data_ptr(),
+                  int(seed) & (2 ** 64 - 1), int(subsequence), int(first), n, R, C, _stream(x_packed))
+    return out
+
+
+def philox_words(count, seed, subsequence=0, first=0, device=None):
+    """uint32 [count]: elements first..first+count-1 of the Philox4x32-10 stream (seed, subsequence)."""
+    device = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+    out = torch.empty((count,), dtype=torch.uint32, device=device)
+    with torch.cuda.device(device):
+        _lib.call("nb_philox_words", out.data_ptr(), int(seed) & (2 ** 64 - 1), int(subsequence), int(first), count,
+                  torch.cuda.current_stream(device).cuda_stream)
+    return out
+
+
+def conv_act_pack(input, filter, threshold, filterx, filtery, padx, pady, stridex, stridey, pool=False):
+    """pack(conv_act(...)) along the channel axis -> [D,h,w,ceil(O/bits)]; with ``pool`` followed by the
+    2x2/stride-2 OR-pool -> [D,h//2,w//2,ceil(O/bits)].  One kernel; the bool map never reaches memory."""
+    suf, bits = _conv_args(input, filter, filterx, filtery)
+    _check(threshold, "threshold")
+    _same_device(input, threshold)
+    assert tuple(threshold.shape) == (input.size(0), filter.size(2))
+    assert threshold.dtype == torch.int32
+    h, w = _out_hw(input, filterx, filtery, padx, pady, stridex, stridey)
+    Ow = ceil_div(filter.size(2), bits)
+    shape = (input.size(0), h // 2, w // 2, Ow) if pool else (input.size(0), h, w, Ow)
+    out = torch.empty(shape, dtype=input.dtype, device=input.device)
+    with torch.cuda.device(input.device):
+        _lib.call("nb_conv_act_pack" + suf, out.data_ptr(), input.data_ptr(), filter.data_ptr(), threshold.data_ptr(),
+                  input.size(0), input.size(1), input.size(2), input.size(3), filter.size(2), filterx, filtery, padx,
+                  pady, stridex, stridey, 1 if pool else 0, _stream(input))
+    return out

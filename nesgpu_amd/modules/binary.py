@@ -1,0 +1,221 @@
+"""Binarized perturbed layers with the API of the reference's ``modules/binary.py``:
+``BinarizedLinear`` (:80-109), ``BinarizedConv2d`` (:112-166), ``BinarizedMaxPool2d`` (:168-182),
+``AsType`` (:11-18), ``ExtractBits`` (:20-29), on top of ``Binarized`` (:32-77).
+
+Constructor signatures, attribute names, tensor layouts and the arithmetic of ``forward`` follow the
+reference; the ops come from :mod:`nesgpu_amd.extensions.booleanOperations` (gfx950 kernels).  Known
+defects of the reference snapshot are not reproduced: construction order (``Perturbed.__init__`` reading
+``self.bias`` too early, modules/base.py:54,107) and ``threshold`` landing in the ``antithetic`` slot
+(modules/binary.py:36 vs modules/base.py:47).
+
+Additions, all opt-in: ``set_noise(words=...)`` samples from caller-supplied uint32 words (bit-exact
+parity mode), and ``BinarizedConv2d(pack_output=True[, pool_output=True])`` returns the thresholded map
+already packed along channels (and 2x2 OR-pooled) from one fused kernel instead of a bool map.
+"""
+import torch
+from torch import nn
+from torch.nn.parameter import Parameter
+
+from ..extensions import booleanOperations
+from .base import Perturbed, PerturbedModel  # noqa: F401
+
+
+class AsType(nn.Module):
+    """modules/binary.py:11-18."""
+
+    def __init__(self, dtype):
+        super().__init__()
+        self.dtype = dtype
+
+    def forward(self, x):
+        return x.type(self.dtype)
+
+
+class ExtractBits(nn.Module):
+    """Expands every integer into its bits, LSB first, along the last axis (modules/binary.py:20-29)."""
+
+    def __init__(self, dtype):
+        nn.Module.__init__(self)
+        self.dtype = dtype
+        self.bitlength = torch.iinfo(dtype).bits
+        # 1 << i; the top bit of a signed type is the sign bit, built by shifting rather than 2 ** i
+        self.mask = torch.ones(self.bitlength, dtype=dtype) << torch.arange(self.bitlength, dtype=dtype)
+
+    def forward(self, input):
+        mask = self.mask.to(input.device)
+        return ((input.unsqueeze(-1) & mask) != 0).view(*input.shape[:-1], -1)
+
+
+class Binarized(Perturbed, nn.Module):
+    """Common part of the binary layers (modules/binary.py:32-77).
+
+    ``weight`` is a latent fp16 matrix [rows, in_degree]; a member's binary weights are drawn per bit with
+    probability sigmoid(5 * w / (mean|w| + 1e-5)) (modules/binary.py:59-62) and stored packed as
+    ``weight_noise`` [directions, rows, ceil(in_degree/bits)]."""
+
+    def __init__(self, in_degree, out_degree, directions, threshold=False, dtype=torch.int64, device="cuda"):
+        nn.Module.__init__(self)
+        Perturbed.__init__(self, directions)
+        self.in_degree = in_degree
+        self.out_degree = out_degree
+        self.dtype = dtype
+        self.threshold = threshold
+        self.device = device
+        self.directions = directions
+        self.bias = None
+
+    def reset_parameters(self):
+        with torch.no_grad():
+            self.weight.fill_(0)
+            if self.threshold:
+                self.bias.fill_(0)
+
+    def probabilities(self):
+        """fp16 [rows, in_degree] per-bit probabilities of a 1 (modules/binary.py:59-60)."""
+        norm_weight = self.weight / (self.weight.abs().mean() + 1e-5) * 5
+        return torch.sigmoid(norm_weight.float()).half()
+
+    def set_noise(self, noise_scale=None, words=None):
+        """modules/binary.py:54-64.  ``words`` (uint32 [directions, rows, in_degree]) replaces the
+        generator: bit = words < floor(P * 2**32)."""
+        if self.seed is None:
+            self.set_seed()
+        if noise_scale is not None:
+            self.set_noise_scale(noise_scale)
+        P = self.probabilities()
+        if words is None:
+            self.weight_noise = booleanOperations.sample_bits(P, self.directions, self.dtype, self.seed)
+        else:
+            self.weight_noise = booleanOperations.sample_bits_from_words(
+                booleanOperations.thresholds_from_p(P), words, self.dtype)
+        if self.threshold:
+            gen = torch.Generator(device=self.weight.device)
+            gen.manual_seed(int(self.seed))
+            self.bias_noise = (torch.rand(size=(self.directions, self.out_degree), dtype=torch.float16,
+                                          device=self.weight.device, generator=gen) - .5) * 6
+        else:
+            self.bias_noise = None
+
+    def update(self, weights, l1=0, l2=1e-3):
+        """modules/binary.py:67-77."""
+        weights = weights.type(torch.float16)
+        weights = (weights - weights.mean())
+        self.weight.grad = booleanOperations.weighted_sum(self.weight_noise, weights.contiguous(), self.in_degree)
+        if l1:
+            self.weight.grad += l1 * torch.sign(self.weight)
+        if l2:
+            self.weight.grad += l2 * self.weight
+        if self.threshold:
+            self.bias.grad = weights @ self.bias_noise
+
+
+class BinarizedLinear(Binarized):
+    """modules/binary.py:80-109.  Input [directions, in_features] bool or [directions, Kw] packed: one input
+    row per member (a batched matrix-VECTOR product, modules/binary.py:97)."""
+
+    def __init__(self, in_features, out_features, directions, threshold=True, batch_norm=False, dtype=torch.int64,
+                 device="cuda"):
+        Binarized.__init__(self, in_features, out_features, directions, threshold, dtype, device)
+        self.in_features = in_features
+        self.out_features = out_features
+        self.weight = Parameter(torch.zeros(out_features, in_features, dtype=torch.float16, device=device))
+        if threshold:
+            self.bias = Parameter(torch.zeros(out_features, dtype=torch.float16, device=device))
+        self.batch_norm = batch_norm
+        self.reset_parameters()
+
+    def forward(self, input):
+        if not self.perturbed_flag:
+            raise NotImplementedError                     # modules/binary.py:108-109: no inference path
+        packed_input = booleanOperations.pack(input, self.dtype) if input.dtype == torch.bool else input
+        popc = booleanOperations.bmm(self.weight_noise, packed_input.view(self.directions, -1, 1))
+        activation = 2 * popc.squeeze(dim=2) - self.in_features
+        if self.threshold:
+            thresh = (self.bias + self.bias_noise)
+            if self.batch_norm:
+                thresh = thresh + activation.type(torch.float16).mean(dim=0, keepdim=True)
+            return activation > thresh
+        return activation
+
+
+class BinarizedConv2d(Binarized):
+    """modules/binary.py:112-166.  Input [directions, H, W, C] bool (channels last) or
+    [directions, H, W, Cw] packed; ``weight`` is [out*kx*ky, in]."""
+
+    def __init__(self, in_channels, out_channels, directions, kernel_size, stride=1, padding=0, dilation=1, groups=1,
+                 threshold=True, batch_norm=True, padding_mode='zeros', dtype=torch.int64, device="cuda",
+                 pack_output=False, pool_output=False):
+        Binarized.__init__(self, in_channels, out_channels, directions, threshold, dtype, device)
+        if dilation != 1 or groups != 1 or padding_mode != "zeros":
+            raise NotImplementedError
+        self.in_channels = in_channels
+        self.out_channels = out_channels
+        self.stride = stride
+        self.padding = padding
+        self.kernel_size = (kernel_size, kernel_size) if isinstance(kernel_size, int) else kernel_size
+        self.weight = Parameter(torch.zeros(out_channels * self.kernel_size[0] * self.kernel_size[1], in_channels,
+                                            dtype=torch.float16, device=device))
+        if threshold:
+            self.bias = Parameter(torch.zeros(out_channels, dtype=torch.float16, device=device))
+        self.batch_norm = batch_norm
+        self.pack_output = pack_output
+        self.pool_output = pool_output
+        if (pack_output or pool_output) and (batch_norm or not threshold):
+            raise NotImplementedError("packed output needs threshold=True, batch_norm=False")
+        self.weight_noise_reshaped = None
+        self.reset_parameters()
+
+    def reset_parameters(self):
+        Binarized.reset_parameters(self)
+
+    def set_noise(self, noise_scale=None, words=None):
+        """modules/binary.py:134-137: [D, out*kx*ky, Cw] -> [D, kx*ky*Cw, out], out contiguous."""
+        Binarized.set_noise(self, noise_scale, words)
+        r = self.weight_noise.view(self.directions, self.out_channels, *self.kernel_size, -1)
+        self.weight_noise_reshaped = r.permute([0, 2, 3, 4, 1]).reshape(self.directions, -1,
+                                                                       self.out_channels).contiguous()
+
+    def forward(self, input):
+        if not self.perturbed_flag:
+            raise NotImplementedError
+        if input.dtype == torch.bool:
+            packed_input = booleanOperations.pack(input.reshape(-1, self.in_channels), self.dtype).view(
+                *input.shape[:3], -1)
+        else:
+            packed_input = input
+        offset = self.in_channels * self.kernel_size[0] * self.kernel_size[1]
+        geom = (*self.kernel_size, self.padding, self.padding, self.stride, self.stride)
+        if self.threshold:
+            if self.batch_norm:
+                activation = 2 * booleanOperations.conv(packed_input, self.weight_noise_reshaped, *geom) - offset
+                thresh = self.bias + self.bias_noise + activation.type(torch.float16).mean(dim=[1, 2])
+                return activation > thresh.unsqueeze(1).unsqueeze(1)
+            thresh = (self.bias + self.bias_noise).type(torch.int32) + offset
+            if self.pack_output or self.pool_output:
+                return booleanOperations.conv_act_pack(packed_input, self.weight_noise_reshaped, thresh, *geom,
+                                                       pool=self.pool_output)
+            return booleanOperations.conv_act(packed_input, self.weight_noise_reshaped, thresh, *geom)
+        return 2 * booleanOperations.conv(packed_input, self.weight_noise_reshaped, *geom) - offset
+
+    def free_memory(self):
+        Perturbed.free_memory(self)
+        self.weight_noise_reshaped = None
+
+
+class BinarizedMaxPool2d(nn.Module):
+    """modules/binary.py:168-182."""
+
+    def __init__(self, kernel_size=(2, 2), padding=(0, 0), stride=(2, 2), dtype=torch.int64):
+        nn.Module.__init__(self)
+        self.kernel_size = kernel_size
+        self.padding = padding
+        self.stride = stride
+        self.dtype = dtype
+
+    def forward(self, input):
+        if input.dtype == torch.bool:
+            packed_input = booleanOperations.pack(input.reshape(-1, input.size(3)), self.dtype).view(
+                *input.shape[:3], -1)
+        else:
+            packed_input = input
+        return booleanOperations.max_pool2d(packed_input, *self.kernel_size, *self.padding, *self.stride)

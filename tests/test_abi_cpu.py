@@ -1,0 +1,107 @@
+"""The C-ABI shared library without a GPU: it loads, exports every symbol include/nesbin.h declares, and
+rejects bad arguments with a status code before launching anything.  No compute calls here."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "nesbin.h")
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from nesgpu_amd import _lib
+    if not os.path.exists(_lib.LIB_PATH):
+        import __graft_entry__ as g
+        g.build()
+    return _lib.load()
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(nb_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_what_the_binding_lists():
+    from nesgpu_amd import _lib
+    assert declared_symbols() == sorted(_lib.exported_symbols())
+
+
+def test_every_declared_symbol_is_exported(lib):
+    for name in declared_symbols():
+        assert hasattr(lib, name), name
+
+
+def test_version_and_error_string(lib):
+    assert lib.nb_version() >= 100
+    assert isinstance(lib.nb_last_error_string(), bytes)
+
+
+def test_bad_arguments_are_rejected_without_a_launch(lib):
+    from nesgpu_amd import _lib
+    one = ctypes.c_void_p(8)          # a non-NULL, 8-byte aligned dummy; never dereferenced on these paths
+    odd = ctypes.c_void_p(12)
+    # negative shape
+    assert lib.nb_pack_i64(one, one, -1, 3, None) == 2
+    assert b"negative" in lib.nb_last_error_string()
+    # NULL pointer with a non-empty shape
+    assert lib.nb_bmm_i64(None, one, one, 1, 1, 1, 1, None) == 1
+    assert lib.nb_bmm_i64(one, None, one, 1, 1, 1, 2, None) == 1
+    # misaligned words
+    assert lib.nb_bmm_i64(one, odd, one, 1, 1, 1, 2, None) == 3
+    # conv window larger than the padded input
+    assert lib.nb_conv_i64(one, one, one, 1, 2, 2, 1, 1, 5, 5, 0, 0, 1, 1, None) == 2
+    # zero stride
+    assert lib.nb_max_pool2d_i64(one, one, 1, 4, 4, 1, 2, 2, 0, 0, 0, 2, None) == 2
+    # empty problems succeed without touching the pointers
+    assert lib.nb_pack_i64(None, None, 0, 64, None) == 0
+    assert lib.nb_bmm_i32(None, None, None, 0, 5, 5, 5, None) == 0
+    assert lib.nb_conv_i64(None, None, None, 0, 8, 8, 1, 4, 3, 3, 1, 1, 1, 1, None) == 0
+    assert lib.nb_sample_from_words_i64(None, None, None, 0, None, 0, 3, 64, None) == 0
+    with pytest.raises(RuntimeError, match="negative"):
+        _lib.call("nb_unpack_i32", one, one, -2, 1, None)
+
+
+def test_python_ops_refuse_cpu_tensors():
+    import torch
+    from nesgpu_amd.extensions import booleanOperations as ops
+    x = torch.zeros(4, 64, dtype=torch.bool)
+    with pytest.raises(RuntimeError, match="CUDA"):
+        ops.pack(x, torch.int64)
+    with pytest.raises(AssertionError):
+        ops.pack(torch.zeros(4, dtype=torch.bool), torch.int64)          # rank check first, as the reference
+    with pytest.raises(TypeError):
+        ops._suffix(torch.int8)
+    a = torch.zeros(2, 3, 4, dtype=torch.int64)
+    with pytest.raises(AssertionError):
+        ops.bmm(a, torch.zeros(2, 5, 1, dtype=torch.int64))             # contraction mismatch
+    assert ops.next_pow2_clip(9, 512) == 16 and ops.next_pow2_clip(300, 512) == 512 and ops.ceil_div(7, 2) == 4
+
+
+def test_layer_construction_and_lifecycle_on_cpu():
+    import torch
+    from nesgpu_amd.modules import binary
+    lin = binary.BinarizedLinear(100, 10, 8, device="cpu")
+    conv = binary.BinarizedConv2d(16, 32, 8, 3, padding=1, device="cpu")
+    pool = binary.BinarizedMaxPool2d()
+    assert lin.weight.shape == (10, 100) and lin.weight.dtype == torch.float16 and lin.bias.shape == (10,)
+    assert conv.weight.shape == (32 * 9, 16) and conv.kernel_size == (3, 3)
+    assert pool.kernel_size == (2, 2) and pool.stride == (2, 2)
+    model = torch.nn.Sequential(conv, pool, torch.nn.Flatten(), lin)
+    pm = binary.PerturbedModel(model, 8)
+    assert pm.perturbed_layers == [conv, lin]
+    pm.set_seed(5)
+    assert conv.seed == 5 and lin.seed == 5
+    pm.free_memory()
+    assert lin.weight_noise is None and conv.weight_noise_reshaped is None
+    with pytest.raises(NotImplementedError):
+        lin(torch.zeros(8, 100, dtype=torch.bool))                        # not in perturbed mode
+    with pytest.raises(NotImplementedError):
+        binary.BinarizedConv2d(3, 3, 2, 3, dilation=2, device="cpu")
+    eb = binary.ExtractBits(torch.int64)
+    v = torch.tensor([[5, -1]], dtype=torch.int64)
+    bits = eb(v)
+    assert bits.shape == (1, 128) and bits[0, :3].tolist() == [True, False, True] and bits[0, 64:].all()

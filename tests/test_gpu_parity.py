@@ -1,0 +1,364 @@
+"""GPU parity tests: the HIP kernels, called through the Python op layer (ctypes -> C ABI of
+include/nesbin.h), against the committed golden fixtures and the CPU oracle on the same seeded inputs.
+Integer / bit results must match exactly."""
+import itertools
+
+import numpy as np
+import pytest
+import torch
+
+from golden_util import (BMM_CASES, CONV_CASES, PACK_WIDTHS, POOL_CASES, SMP_CASES, TAGS, load_ops, load_philox)
+
+pytestmark = pytest.mark.gpu
+
+G = load_ops()
+TDT = {"i64": torch.int64, "i32": torch.int32}
+NDT = {torch.int64: np.int64, torch.int32: np.int32}
+
+
+@pytest.fixture(scope="module")
+def ops():
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    from nesgpu_amd.extensions import booleanOperations
+    return booleanOperations
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def host(t):
+    return t.cpu().numpy()
+
+
+def rng(seed):
+    return np.random.default_rng(seed)
+
+
+def rand_words(g, shape, dtype):
+    return g.integers(-2 ** 63, 2 ** 63, size=shape, dtype=np.int64).astype(dtype)
+
+
+# ---------------------------------------------------------------------------------------------- golden
+@pytest.mark.parametrize("tag", TAGS)
+def test_golden_pack_unpack(ops, tag):
+    for C in PACK_WIDTHS:
+        bits = G[f"pack_{tag}_C{C}_in"]
+        got = ops.pack(dev(bits), TDT[tag])
+        np.testing.assert_array_equal(host(got), G[f"pack_{tag}_C{C}_out"])
+        un = host(ops.unpack(got))
+        np.testing.assert_array_equal(un[:, :C], bits)
+        assert not un[:, C:].any()
+
+
+@pytest.mark.parametrize("tag", TAGS)
+@pytest.mark.parametrize("case", BMM_CASES)
+def test_golden_bmm(ops, tag, case):
+    A, B = dev(G[f"bmm_{tag}_{case}_A"]), dev(G[f"bmm_{tag}_{case}_B"])
+    np.testing.assert_array_equal(host(ops.bmm(A, B)), G[f"bmm_{tag}_{case}_C"])
+    act = ops.bmm_act(A, B, dev(G[f"bmm_{tag}_{case}_thr"]))
+    assert act.dtype == torch.bool
+    np.testing.assert_array_equal(host(act), G[f"bmm_{tag}_{case}_act"])
+
+
+@pytest.mark.parametrize("tag", TAGS)
+@pytest.mark.parametrize("case", CONV_CASES)
+def test_golden_conv(ops, tag, case):
+    x, f = dev(G[f"conv_{tag}_{case}_x"]), dev(G[f"conv_{tag}_{case}_f"])
+    thr = dev(G[f"conv_{tag}_{case}_thr"])
+    geom = [int(v) for v in G[f"conv_{tag}_{case}_geom"]]
+    np.testing.assert_array_equal(host(ops.batch_im2col(x, *geom)), G[f"conv_{tag}_{case}_cols"])
+    popc = ops.conv(x, f, *geom)
+    assert popc.dtype == torch.int32
+    np.testing.assert_array_equal(host(popc), G[f"conv_{tag}_{case}_popc"])
+    np.testing.assert_array_equal(host(ops.conv_act(x, f, thr, *geom)), G[f"conv_{tag}_{case}_act"])
+
+
+@pytest.mark.parametrize("tag", TAGS)
+@pytest.mark.parametrize("case", POOL_CASES)
+def test_golden_pool(ops, tag, case):
+    geom = [int(v) for v in G[f"pool_{tag}_{case}_geom"]]
+    got = ops.max_pool2d(dev(G[f"pool_{tag}_{case}_x"]), *geom)
+    np.testing.assert_array_equal(host(got), G[f"pool_{tag}_{case}_out"])
+
+
+@pytest.mark.parametrize("tag", TAGS)
+@pytest.mark.parametrize("case", SMP_CASES)
+def test_golden_sampling(ops, tag, case):
+    p = f"smp_{tag}_{case}_"
+    words, thr, base, x = dev(G[p + "words"]), dev(G[p + "thr"]), dev(G[p + "base"]), dev(G[p + "x"])
+    T = 214748364
+    np.testing.assert_array_equal(host(ops.sample_bits_from_words(thr, words, TDT[tag])), G[p + "sample"])
+    np.testing.assert_array_equal(host(ops.flip_from_words(base, words, T)), G[p + "flip"])
+    np.testing.assert_array_equal(host(ops.seeded_bmv_from_words(thr, x, words)), G[p + "bmv_sample"])
+    np.testing.assert_array_equal(host(ops.seeded_bmv_from_words(T, x, words, base=base)), G[p + "bmv_flip"])
+
+
+def test_golden_philox(ops):
+    P = load_philox()
+    for case in P["rocrand"]:
+        got = ops.philox_words(len(case["words"]), case["seed"], case["subsequence"], case["offset"])
+        assert [int(v) for v in host(got)] == case["words"]
+
+
+# ---------------------------------------------------------------------------------------------- vs oracle
+@pytest.mark.parametrize("dtype", [torch.int64, torch.int32])
+@pytest.mark.parametrize("R,C", [(1, 16), (5, 64), (300, 128), (1000, 16), (77, 48), (33, 256), (9, 8192), (4097, 3),
+                                 (64, 80), (2, 1), (513, 576)])
+def test_pack_unpack_vs_oracle(ops, oracle, dtype, R, C):
+    bits = rng(R + C).integers(0, 2, size=(R, C)).astype(bool)
+    want = oracle.pack(bits, NDT[dtype])
+    got = ops.pack(dev(bits), dtype)
+    np.testing.assert_array_equal(host(got), want)
+    np.testing.assert_array_equal(host(ops.unpack(got)), oracle.unpack(want))
+
+
+def test_pack_counts_any_nonzero_byte_as_one(ops):
+    raw = rng(1).integers(0, 256, size=(8, 64)).astype(np.uint8)
+    t = dev(raw).view(torch.bool)
+    got = host(ops.pack(t, torch.int64))
+    want = np.packbits(raw != 0, axis=1, bitorder="little").view("<i8")
+    np.testing.assert_array_equal(got, want)
+
+
+def test_pack_misaligned_rows_take_the_generic_path(ops, oracle):
+    bits = rng(3).integers(0, 2, size=(41, 64)).astype(bool)
+    big = dev(np.concatenate([np.zeros(3, dtype=bool), bits.ravel()]))
+    view = big[3:].view(41, 64)                         # data pointer not 16-byte aligned
+    np.testing.assert_array_equal(host(ops.pack(view, torch.int64)), oracle.pack(bits, np.int64))
+
+
+@pytest.mark.parametrize("dtype", [torch.int64, torch.int32])
+def test_int8pack_vs_oracle(ops, oracle, dtype):
+    for R, C in [(3, 1), (50, 8), (7, 13), (100, 784)]:
+        data = rng(C).integers(0, 256, size=(R, C)).astype(np.uint8)
+        np.testing.assert_array_equal(host(ops.int8pack(dev(data), dtype)), oracle.int8pack(data, NDT[dtype]))
+
+
+LINEAR_SHAPES = [(8, 256, 4), (5, 10, 16), (3, 1000, 128), (7, 33, 9), (4, 64, 1), (2, 3, 200), (9, 1, 2), (1, 5, 31),
+                 (6, 130, 6)]
+
+
+@pytest.mark.parametrize("dtype", [torch.int64, torch.int32])
+@pytest.mark.parametrize("Z,M,Kw", LINEAR_SHAPES)
+def test_bmm_matrix_vector_form_vs_oracle(ops, oracle, dtype, Z, M, Kw):
+    g = rng(Z * 31 + M * 7 + Kw)
+    A = rand_words(g, (Z, M, Kw), NDT[dtype])
+    x = rand_words(g, (Z, Kw, 1), NDT[dtype])
+    np.testing.assert_array_equal(host(ops.bmm(dev(A), dev(x))), oracle.bmm(A, x))
+
+
+def test_bmm_matrix_vector_unaligned_operands(ops, oracle):
+    g = rng(17)
+    A = rand_words(g, (3, 20, 4), np.int64)
+    x = rand_words(g, (3, 4, 1), np.int64)
+    bigA = dev(np.concatenate([np.zeros(1, np.int64), A.ravel()]))[1:].view(3, 20, 4)      # 8- but not 16-byte aligned
+    np.testing.assert_array_equal(host(ops.bmm(bigA, dev(x))), oracle.bmm(A, x))
+
+
+GENERAL_SHAPES = [(2, 300, 9, 64), (3, 65, 4, 16), (2, 257, 18, 5), (2, 40, 40, 33), (1, 1, 1, 2), (2, 513, 3, 128),
+                  (3, 7, 17, 17), (2, 100, 0, 4)]
+
+
+@pytest.mark.parametrize("dtype", [torch.int64, torch.int32])
+@pytest.mark.parametrize("Z,M,Kw,N", GENERAL_SHAPES)
+def test_bmm_general_and_act_vs_oracle(ops, oracle, dtype, Z, M, Kw, N):
+    g = rng(Z + M + Kw + N)
+    A = rand_words(g, (Z, M, Kw), NDT[dtype])
+    B = rand_words(g, (Z, Kw, N), NDT[dtype])
+    want = oracle.bmm(A, B)
+    np.testing.assert_array_equal(host(ops.bmm(dev(A), dev(B))), want)
+    hi = max(int(want.max()), 1)
+    thr = (g.integers(0, 2 * hi + 2, size=(Z, N)) - 1).astype(np.int32)
+    np.testing.assert_array_equal(host(ops.bmm_act(dev(A), dev(B), dev(thr))), oracle.bmm_act(A, B, thr))
+
+
+def test_bmm_special_cases(ops):
+    g = rng(4)
+    A = rand_words(g, (2, 70, 5), np.int64)
+    At = np.ascontiguousarray(A.transpose(0, 2, 1))
+    got = host(ops.bmm(dev(A), dev(At)))
+    assert (got[:, np.arange(70), np.arange(70)] == 0).all()                  # a ^ a
+    got = host(ops.bmm(dev(A), dev(~At)))
+    assert (got[:, np.arange(70), np.arange(70)] == 5 * 64).all()             # a ^ ~a, sign bits included
+    zeros = np.zeros((2, 5, 3), np.int64)
+    ones = np.unpackbits(A.view(np.uint8), axis=2).sum(axis=2)
+    np.testing.assert_array_equal(host(ops.bmm(dev(A), dev(zeros))), np.repeat(ones[:, :, None], 3, 2))
+
+
+SWEEP = list(itertools.product([1, 3, 7], [0, 1, 2], [1, 2, 3]))                # booloptests.py:122-124
+
+
+@pytest.mark.parametrize("dtype", [torch.int32, torch.int64])
+@pytest.mark.parametrize("C,O", [(1, 64), (16, 16), (64, 5), (70, 33), (130, 8)])
+def test_conv_reference_sweep_vs_oracle(ops, oracle, dtype, C, O):
+    """The reference's check_result sweep (filter x padding x stride on a 10x10 input, booloptests.py:113-124)."""
+    D, S = 5, 10
+    bits = torch.iinfo(dtype).bits
+    Cw = (C + bits - 1) // bits
+    for fs, pad, st in SWEEP:
+        g = rng(fs * 100 + pad * 10 + st + C)
+        xb = g.integers(0, 2, size=(D * S * S, C)).astype(bool)
+        x = oracle.pack(xb, NDT[dtype]).reshape(D, S, S, Cw)
+        fb = g.integers(0, 2, size=(D * O * fs * fs, C)).astype(bool)
+        f5 = oracle.pack(fb, NDT[dtype]).reshape(D, O, fs, fs, Cw)
+        f = np.ascontiguousarray(f5.transpose(0, 2, 3, 4, 1).reshape(D, -1, O))
+        K = fs * fs * C
+        thr = (g.integers(0, K, size=(D, O)) - K // 2 + K).astype(np.int32)
+        geom = (fs, fs, pad, pad, st, st)
+        xd, fd, td = dev(x), dev(f), dev(thr)
+        want = oracle.conv(x, f, *geom)
+        np.testing.assert_array_equal(host(ops.conv(xd, fd, *geom)), want, err_msg=str(geom))
+        np.testing.assert_array_equal(host(ops.conv_act(xd, fd, td, *geom)), 2 * want > thr[:, None, None, :])
+        np.testing.assert_array_equal(host(ops.batch_im2col(xd, *geom)), oracle.batch_im2col(x, *geom))
+        # fused conv -> threshold -> pack (-> pool) against the op chain of the oracle
+        act = oracle.conv_act(x, f, thr, *geom)
+        h, w = act.shape[1:3]
+        packed = oracle.pack(act.reshape(-1, O), NDT[dtype]).reshape(D, h, w, -1)
+        np.testing.assert_array_equal(host(ops.conv_act_pack(xd, fd, td, *geom)), packed)
+        if h >= 2 and w >= 2:
+            pooled = oracle.max_pool2d(packed, 2, 2, 0, 0, 2, 2)
+            np.testing.assert_array_equal(host(ops.conv_act_pack(xd, fd, td, *geom, pool=True)), pooled)
+
+
+def test_conv_rectangular_window_and_image(ops, oracle):
+    g = rng(8)
+    D, H, W, Cw, O = 3, 9, 13, 2, 20
+    x = rand_words(g, (D, H, W, Cw), np.int64)
+    for fx, fy, px, py, sx, sy in [(3, 2, 1, 0, 1, 2), (1, 5, 0, 2, 2, 1), (4, 4, 3, 3, 3, 2)]:
+        f = rand_words(g, (D, fx * fy * Cw, O), np.int64)
+        want = oracle.conv(x, f, fx, fy, px, py, sx, sy)
+        np.testing.assert_array_equal(host(ops.conv(dev(x), dev(f), fx, fy, px, py, sx, sy)), want)
+
+
+@pytest.mark.parametrize("dtype", [torch.int64, torch.int32])
+def test_max_pool_vs_oracle(ops, oracle, dtype):
+    g = rng(12)
+    for B, H, W, Cw in [(3, 10, 10, 1), (2, 7, 9, 3), (5, 64, 64, 1), (1, 2, 2, 1), (2, 33, 5, 2)]:
+        x = rand_words(g, (B, H, W, Cw), NDT[dtype])
+        for geom in [(2, 2, 0, 0, 2, 2), (2, 2, 1, 1, 2, 2), (3, 3, 1, 1, 2, 2), (2, 2, 0, 0, 1, 1), (2, 2, 0, 1, 3, 2)]:
+            if H - geom[0] + 2 * geom[2] < 0 or W - geom[1] + 2 * geom[3] < 0:
+                continue
+            np.testing.assert_array_equal(host(ops.max_pool2d(dev(x), *geom)), oracle.max_pool2d(x, *geom),
+                                          err_msg=str((B, H, W, Cw, geom)))
+
+
+SAMPLE_SHAPES = [(3, 4, 64), (2, 3, 1), (5, 2, 63), (2, 5, 65), (3, 2, 200), (4, 7, 256), (2, 576, 64), (3, 10, 1024),
+                 (2, 9, 16), (3, 5, 128), (2, 3, 100)]
+
+
+@pytest.mark.parametrize("dtype", [torch.int64, torch.int32])
+@pytest.mark.parametrize("n,R,C", SAMPLE_SHAPES)
+def test_sampling_from_words_vs_oracle(ops, oracle, dtype, n, R, C):
+    g = rng(n * 7 + R * 3 + C)
+    words = g.integers(0, 2 ** 32, size=(n, R, C), dtype=np.uint64).astype(np.uint32)
+    thr = g.integers(0, 2 ** 32, size=(R, C), dtype=np.uint64).astype(np.uint32)
+    T = int(0.05 * 2 ** 32)
+    nd = NDT[dtype]
+    wb = np.dtype(nd).itemsize * 8
+    base = rand_words(g, (R, (C + wb - 1) // wb), nd)
+    if C % wb:
+        base[:, -1] &= nd((1 << (C % wb)) - 1)
+    x = rand_words(g, (n, (C + wb - 1) // wb), nd)
+    if C % wb:
+        x[:, -1] &= nd((1 << (C % wb)) - 1)          # tail bits are zero by contract (pack.cu:17)
+    wd, td, bd, xd = dev(words), dev(thr), dev(base), dev(x)
+    np.testing.assert_array_equal(host(ops.sample_bits_from_words(td, wd, dtype)), oracle.sample_from_words(thr, words, nd))
+    np.testing.assert_array_equal(host(ops.flip_from_words(bd, wd, T)), oracle.sample_from_words(T, words, nd, base=base))
+    np.testing.assert_array_equal(host(ops.sample_bits_from_words(td, wd, dtype, base=bd)),
+                                  oracle.sample_from_words(thr, words, nd, base=base))
+    for kw in (dict(base=None, thr=thr), dict(base=base, thr=T), dict(base=base, thr=thr)):
+        want = oracle.seeded_bmv_from_words(kw["thr"], x, words, base=kw["base"])
+        tarr = td if isinstance(kw["thr"], np.ndarray) else kw["thr"]
+        got = ops.seeded_bmv_from_words(tarr, xd, wd, base=None if kw["base"] is None else bd)
+        np.testing.assert_array_equal(host(got), want)
+        # fused == materialise + bmm on the GPU as well
+        Wm = ops.sample_bits_from_words(tarr, wd, dtype, base=None if kw["base"] is None else bd)
+        np.testing.assert_array_equal(host(ops.bmm(Wm, xd.view(n, -1, 1)))[:, :, 0], want)
+
+
+@pytest.mark.parametrize("dtype", [torch.int64, torch.int32])
+@pytest.mark.parametrize("n,R,C,first", [(3, 4, 64, 0), (2, 5, 100, 0), (2, 3, 256, 8), (2, 3, 64, 5), (3, 2, 63, 2),
+                                         (2, 7, 1024, 4 * 0xFFFFFFFE)])
+def test_philox_mode_equals_supplied_words_mode(ops, oracle, dtype, n, R, C, first):
+    """Generator mode is defined as: the words nb_philox_words writes, fed to the supplied-words kernels."""
+    seed, sub = 0x1234ABCD5678EF01, 3
+    g = rng(C + first % 97)
+    nd = NDT[dtype]
+    wb = np.dtype(nd).itemsize * 8
+    words_gpu = ops.philox_words(n * R * C, seed, sub, first)
+    words_cpu = oracle.philox_words(seed, sub, first, n * R * C)
+    np.testing.assert_array_equal(host(words_gpu), words_cpu)
+    words = words_gpu.view(n, R, C)
+    thr = dev(g.integers(0, 2 ** 32, size=(R, C), dtype=np.uint64).astype(np.uint32))
+    base = rand_words(g, (R, (C + wb - 1) // wb), nd)
+    if C % wb:
+        base[:, -1] &= nd((1 << (C % wb)) - 1)
+    bd = dev(base)
+    xh = rand_words(g, (n, (C + wb - 1) // wb), nd)
+    if C % wb:
+        xh[:, -1] &= nd((1 << (C % wb)) - 1)
+    x = dev(xh)
+    T = int(0.02 * 2 ** 32)
+    a = ops.sample_bits_philox(thr, n, dtype, seed, sub, first)
+    assert torch.equal(a, ops.sample_bits_from_words(thr, words, dtype))
+    a = ops.flip_philox(bd, C, n, T, seed, sub, first)
+    assert torch.equal(a, ops.flip_from_words(bd, words, T))
+    a = ops.seeded_bmv_philox(T, x, R, C, seed, sub, first, base=bd)
+    assert torch.equal(a, ops.seeded_bmv_from_words(T, x, words, base=bd))
+    a = ops.seeded_bmv_philox(thr, x, R, C, seed, sub, first)
+    assert torch.equal(a, ops.seeded_bmv_from_words(thr, x, words))
+
+
+def test_sample_bits_law_and_layout(ops):
+    """sample_bits(p, n, dtype, seed): shape [n,R,ceil(C/bits)], zero tail bits, rate ~= p, seed-reproducible."""
+    p = torch.tensor([[0.0] * 100, [1.0] * 100, [0.25] * 100, [0.5] * 100], dtype=torch.float16, device="cuda")
+    a = ops.sample_bits(p, 512, torch.int64, 999)
+    assert a.shape == (512, 4, 2) and a.dtype == torch.int64
+    assert torch.equal(a, ops.sample_bits(p, 512, torch.int64, 999))
+    assert not torch.equal(a, ops.sample_bits(p, 512, torch.int64, 1000))
+    bits = host(ops.unpack(a.view(-1, 2))).reshape(512, 4, 128)
+    assert not bits[:, :, 100:].any()
+    assert not bits[:, 0].any() and bits[:, 1, :100].all()
+    assert abs(bits[:, 2, :100].mean() - 0.25) < 0.01 and abs(bits[:, 3, :100].mean() - 0.5) < 0.01
+
+
+@pytest.mark.parametrize("dtype", [torch.int64, torch.int32])
+def test_weighted_sum_vs_oracle(ops, oracle, dtype):
+    g = rng(21)
+    for n, R, C in [(37, 5, 100), (128, 16, 64), (64, 3, 256)]:
+        nd = NDT[dtype]
+        wb = np.dtype(nd).itemsize * 8
+        words = rand_words(g, (n, R, (C + wb - 1) // wb), nd)
+        w = g.standard_normal(n).astype(np.float16)
+        got = host(ops.weighted_sum(dev(words), dev(w), C)).astype(np.float32)
+        want = oracle.weighted_sum(words, w.astype(np.float32), C)
+        # same fp32 additions in the same order, then one rounding to fp16
+        np.testing.assert_array_equal(got, want.astype(np.float16).astype(np.float32))
+
+
+def test_ops_run_on_the_current_stream(ops, oracle):
+    g = rng(2)
+    A = rand_words(g, (4, 100, 9), np.int64)
+    B = rand_words(g, (4, 9, 16), np.int64)
+    s = torch.cuda.Stream()
+    with torch.cuda.stream(s):
+        Ad, Bd = dev(A), dev(B)
+        out = ops.bmm(Ad, Bd)
+    s.synchronize()
+    np.testing.assert_array_equal(host(out), oracle.bmm(A, B))
+
+
+def test_errors_match_the_reference_conventions(ops):
+    a = torch.zeros(2, 3, 4, dtype=torch.int64, device="cuda")
+    with pytest.raises(AssertionError):
+        ops.bmm(a, torch.zeros(3, 4, 1, dtype=torch.int64, device="cuda"))
+    with pytest.raises(RuntimeError, match="contiguous"):
+        ops.bmm(a.transpose(1, 2), torch.zeros(2, 3, 1, dtype=torch.int64, device="cuda"))
+    with pytest.raises(TypeError):
+        ops.bmm(a.to(torch.int16), torch.zeros(2, 4, 1, dtype=torch.int16, device="cuda"))
+    with pytest.raises(RuntimeError):
+        ops.conv(torch.zeros(1, 2, 2, 1, dtype=torch.int64, device="cuda"),
+                 torch.zeros(1, 25, 4, dtype=torch.int64, device="cuda"), 5, 5, 0, 0, 1, 1)
+    assert ops.bmm(torch.zeros(0, 3, 4, dtype=torch.int64, device="cuda"),
+                   torch.zeros(0, 4, 2, dtype=torch.int64, device="cuda")).shape == (0, 3, 2)
