@@ -1,0 +1,188 @@
+#!/usr/bin/env python3
+"""Benchmark of the population-batched binary forward path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--extra 1,3,4,5] [--no-cpu]
+
+Headline workload (BASELINE configs[1]): binary linear 1024x1024, population 1024, one input row per member,
+p = 0.05 flip masks sampled by threshold compare from SUPPLIED uint32 words, fused into the XOR-popcount
+product.  A step is one such population forward with every operand resident in HBM.  Prints one JSON line.
+
+value      packed binary TOPS = 2 * valid bit-MACs / s (whole job, one GPU)
+roofline   the dominant kernel against MI355X's published HBM bandwidth: algorithmic bytes per launch
+           (4 B per weight bit of random words + base + inputs + int32 outputs) / average launch duration
+cpu_baseline  the C oracle (a port of the same arithmetic) timed on this box's host cores on a subset of
+           the members of the same workload
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--extra", type=str, default="1,3,4,5",
+                    help="other configurations to time as well (reported under other_configs); '' for none")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-calib", action="store_true", help="skip the measured copy / popcount ceilings")
+    ap.add_argument("--cpu-members", type=int, default=256, help="members of the workload the CPU baseline runs")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU time the baseline leg accumulates")
+    ap.add_argument("--only-calib", action="store_true", help="run only the calibration kernels (for counter runs)")
+    return ap.parse_args()
+
+
+def time_steps(torch, step, steps, warmup):
+    """W untimed steps, then K steps bracketed by synchronize; wall clock and HIP events on the launch stream."""
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+        step()
+    e1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    return wall / steps, e0.elapsed_time(e1) * 1e-3 / steps
+
+
+def cpu_baseline(wl, members, seconds):
+    """Oracle (port) on the first `members` members of the headline workload; words regenerated on the host from
+    the same Philox stream the GPU words came from."""
+    import numpy as np
+    from oracle import oracle as O
+    m = wl.meta
+    out_f, in_f = m["out_f"], m["in_f"]
+    members = min(members, wl.population)
+    words = O.philox_words(m["seed"], m["subsequence"], 0, members * out_f * in_f).reshape(members, out_f, in_f)
+    base = wl.tensors["base"].cpu().numpy()
+    x = wl.tensors["x"][:members].cpu().numpy()
+    times = []
+    got = None
+    total = 0.0
+    while total < seconds or len(times) < 3:
+        t0 = time.perf_counter()
+        got = O.seeded_bmv_from_words(m["T"], x, words, base=base)
+        dt = time.perf_counter() - t0
+        times.append(dt)
+        total += dt
+    gpu = wl.step()[:members].cpu().numpy()
+    if not np.array_equal(gpu, got):
+        raise SystemExit("bench: GPU result differs from the CPU oracle on the baseline sample")
+    macs = members * out_f * in_f
+    med = sorted(times)[len(times) // 2]
+    return {"value": round(2 * macs / med / 1e12, 6), "unit": "binary TOPS", "cores": O.max_threads(), "kind": "port",
+            "sample": "first %d of %d members of the same workload, %d passes over %.1f s, median %.4f s per pass, "
+                      "OpenMP over members; output checked equal to the GPU's" % (members, wl.population, len(times),
+                                                                                  total, med)}
+
+
+def calibrate(torch):
+    """Measured ceilings reported beside the datasheet peaks: streaming copy, streaming read, xor+bcnt loop."""
+    import ctypes
+    path = os.path.join(ROOT, "nesgpu_amd", "libnesbin_calib.so")
+    if not os.path.exists(path):
+        return None
+    lib = ctypes.CDLL(path)
+    vp, i64, i32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
+    lib.nb_calib_copy.argtypes = [vp, vp, i64, i32, vp]
+    lib.nb_calib_read.argtypes = [vp, vp, i64, vp]
+    lib.nb_calib_popc.argtypes = [vp, vp, i32, i32, vp]
+    st = torch.cuda.current_stream().cuda_stream
+    nbytes = 2 << 30
+    src = torch.empty(nbytes, dtype=torch.uint8, device="cuda").fill_(1)
+    dst = torch.empty_like(src)
+    sink = torch.zeros(4, dtype=torch.int32, device="cuda")
+    res = {}
+    per, ev = time_steps(torch, lambda: lib.nb_calib_copy(dst.data_ptr(), src.data_ptr(), nbytes, 256 * 32, st), 10, 2)
+    res["copy_GBps"] = round(2 * nbytes / ev / 1e9, 1)
+    per, ev = time_steps(torch, lambda: lib.nb_calib_read(sink.data_ptr(), src.data_ptr(), nbytes, st), 10, 2)
+    res["read_GBps"] = round(nbytes / ev / 1e9, 1)
+    blocks, iters = 256 * 32, 2000
+    s = torch.randint(0, 2 ** 31, (1024,), dtype=torch.int32, device="cuda")
+    out = torch.empty(blocks * 256, dtype=torch.int32, device="cuda")
+    per, ev = time_steps(torch, lambda: lib.nb_calib_popc(out.data_ptr(), s.data_ptr(), blocks, iters, st), 5, 1)
+    lane_ops = blocks * 256 * iters * 8 * 16 * 2
+    res["xor_bcnt_lane_ops_per_s"] = float("%.4g" % (lane_ops / ev))
+    res["xor_bcnt_binary_TOPS"] = round(2 * (lane_ops / 4 * 64) / ev / 1e12, 1)
+    return res
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU; population sharding over several GPUs is design-only "
+              "(run with --gpus 1)", file=sys.stderr)
+        return 2
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 2
+    from nesgpu_amd import _lib, workloads
+    _lib.load()                                                   # fail loudly if the HIP library is missing
+    torch.cuda.set_device(0)
+    if args.only_calib:
+        print(json.dumps({"measured_ceilings": calibrate(torch)}))
+        return 0
+
+    wl = workloads.linear_flip_fused()
+    per_wall, per_ev = time_steps(torch, wl.step, args.steps, args.warmup)
+    tops = 2 * wl.bit_macs / per_wall / 1e12
+    achieved = wl.algo_bytes / per_ev / 1e9
+    line = {
+        "metric": "packed binary TOPS (2 x valid bit-MACs / s) per population forward",
+        "value": round(tops, 4), "unit": "binary TOPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(per_wall * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "u64", "data": "synthetic (seed 0; inputs/base from torch CPU generator, random words from "
+                                "Philox4x32-10)",
+        "config": {"workload": wl.name, "population": wl.population, "word_bits": 64,
+                   "bit_macs_per_step": wl.bit_macs},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": workloads.HBM_PEAK / 1e9, "unit": "GB/s",
+                     "frac": round(achieved * 1e9 / workloads.HBM_PEAK, 4), "traffic": None,
+                     "kernel": "seeded_bmv_wide_kernel", "algorithmic_bytes_per_launch": wl.algo_bytes,
+                     "avg_launch_ms": round(per_ev * 1e3, 4)},
+    }
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline(wl, args.cpu_members, args.cpu_seconds)
+    del wl
+    torch.cuda.empty_cache()
+
+    others = []
+    for tok in [t for t in args.extra.split(",") if t.strip()]:
+        cfg = int(tok)
+        if cfg == 2:
+            continue
+        w = workloads.BUILDERS[cfg]()
+        steps = max(3, args.steps // 2) if cfg == 5 else args.steps
+        pw, pe = time_steps(torch, w.step, steps, args.warmup)
+        entry = {"config": cfg, "workload": w.name, "ms_per_step": round(pw * 1e3, 4),
+                 "binary_TOPS": round(2 * w.bit_macs / pw / 1e12, 3), "bound": w.bound}
+        if w.bound == "hbm":
+            entry["roofline_frac"] = round(w.algo_bytes / pe / workloads.HBM_PEAK, 4)
+        else:
+            entry["roofline_frac"] = round(w.bit_macs / pe / workloads.VALU_POPC_PEAK, 4)
+        others.append(entry)
+        del w
+        torch.cuda.empty_cache()
+    if others:
+        line["other_configs"] = others
+    if not args.no_calib:
+        cal = calibrate(torch)
+        if cal:
+            line["measured_ceilings"] = cal
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -10,39 +10,45 @@
 
 namespace nb {
 
-template <typename W, int L, int V, int RPG>
-__global__ __launch_bounds__(256) void bmv_kernel(int32_t *__restrict__ C, const W *__restrict__ A,
-                                                  const W *__restrict__ X, int64_t rows, int64_t M, int Kw)
+template <typename W, int L, int V, int RPG, int BS>
+__global__ __launch_bounds__(BS) void bmv_kernel(int32_t *__restrict__ C, const W *__restrict__ A,
+                                                 const W *__restrict__ X, int64_t rows, int64_t M, int Kw)
 {
-    const int64_t gid = ((int64_t)blockIdx.x * 256 + threadIdx.x) / L;
+    typedef W WV __attribute__((ext_vector_type(V == 2 ? 2 : 1)));
+    const int64_t gid = ((int64_t)blockIdx.x * BS + threadIdx.x) / L;
     const int sub = threadIdx.x % L;
     const int64_t r0 = gid * RPG;
     int acc[RPG];
 #pragma unroll
     for (int q = 0; q < RPG; q++) acc[q] = 0;
-    const int64_t z0 = r0 < rows ? r0 / M : 0;
-    const int64_t m0 = r0 - z0 * M;
-    for (int k = sub * V; k < Kw; k += L * V) {
+    // rows past the end are clamped (recomputed, never stored) so that the loads need no branches
+    int64_t rr[RPG], zz[RPG];
+    {
+        const int64_t last = rows - 1;
+        const int64_t rc = r0 < last ? r0 : last;
+        int64_t z = rc / M, m = rc - z * M;
 #pragma unroll
         for (int q = 0; q < RPG; q++) {
-            const int64_t r = r0 + q;
-            if (r < rows) {
-                int64_t z = z0, m = m0 + q;
-                while (m >= M) {
-                    m -= M;
-                    z++;
-                }
-                const W *ap = A + r * Kw + k;
-                const W *xp = X + z * Kw + k;
-                if (V == 2) {
-                    typedef W W2 __attribute__((ext_vector_type(2)));
-                    const W2 av = *reinterpret_cast<const W2 *>(ap);
-                    const W2 xv = *reinterpret_cast<const W2 *>(xp);
-                    acc[q] += popc_xor(av.x, xv.x) + popc_xor(av.y, xv.y);
-                } else {
-                    acc[q] += popc_xor(*ap, *xp);
-                }
+            rr[q] = r0 + q < last ? r0 + q : last;
+            zz[q] = z;
+            if (r0 + q < last && ++m == M) {
+                m = 0;
+                z++;
             }
+        }
+    }
+    for (int k = sub * V; k < Kw; k += L * V) {
+        WV av[RPG], xv[RPG];
+#pragma unroll
+        for (int q = 0; q < RPG; q++) xv[q] = *reinterpret_cast<const WV *>(X + zz[q] * Kw + k);
+#pragma unroll
+        for (int q = 0; q < RPG; q++)
+            av[q] = __builtin_nontemporal_load(reinterpret_cast<const WV *>(A + rr[q] * Kw + k));  // read once
+        __builtin_amdgcn_sched_barrier(0);  // all loads of the step in flight before the first use
+#pragma unroll
+        for (int q = 0; q < RPG; q++) {
+            if (V == 2) acc[q] += popc_xor(av[q][0], xv[q][0]) + popc_xor(av[q][V - 1], xv[q][V - 1]);
+            else acc[q] += popc_xor(av[q][0], xv[q][0]);
         }
     }
 #pragma unroll
@@ -71,10 +77,10 @@ __global__ __launch_bounds__(256) void bmm_rowlane_kernel(RowsA<W> al, const W *
 template <typename W, int L, int V>
 static void launch_bmv(int32_t *C, const W *A, const W *X, int64_t rows, int64_t M, int Kw, hipStream_t s)
 {
-    constexpr int RPG = 4;
+    constexpr int RPG = 4, BS = 1024;
     const int64_t groups = ceil_div(rows, RPG);
-    const int64_t blocks = ceil_div(groups * L, 256);
-    bmv_kernel<W, L, V, RPG><<<dim3((unsigned)blocks), dim3(256), 0, s>>>(C, A, X, rows, M, Kw);
+    const int64_t blocks = ceil_div(groups * L, BS);
+    bmv_kernel<W, L, V, RPG, BS><<<dim3((unsigned)blocks), dim3(BS), 0, s>>>(C, A, X, rows, M, Kw);
 }
 
 template <typename W, int V>

@@ -10,20 +10,22 @@ template <typename W>
 __global__ __launch_bounds__(256) void im2col_kernel(W *__restrict__ out, const W *__restrict__ in, int64_t total,
                                                      ConvGeom g)
 {
-    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (t >= total) return;
-    const int K = g.fx * g.fy * g.Cw;
-    const int64_t rowi = t / K;  // (b, loc)
-    const int e = (int)(t - rowi * K);
-    const int hw = g.h * g.w;
-    const int64_t b = rowi / hw;
-    const int loc = (int)(rowi - b * hw);
-    const int xo = loc / g.w, yo = loc - xo * g.w;
-    const int tap = e / g.Cw, c = e - tap * g.Cw;
-    const int i = tap / g.fy, j = tap - i * g.fy;
-    const int xi = i + xo * g.sx - g.px, yi = j + yo * g.sy - g.py;
-    const bool ok = xi >= 0 && xi < g.H && yi >= 0 && yi < g.Wd;
-    out[t] = ok ? in[((b * g.H + xi) * g.Wd + yi) * g.Cw + c] : (W)0;
+    NB_FLAT_LOOP(t, total)
+    {
+        if (t >= total) continue;
+        const int K = g.fx * g.fy * g.Cw;
+        const int64_t rowi = t / K;  // (b, loc)
+        const int e = (int)(t - rowi * K);
+        const int hw = g.h * g.w;
+        const int64_t b = rowi / hw;
+        const int loc = (int)(rowi - b * hw);
+        const int xo = loc / g.w, yo = loc - xo * g.w;
+        const int tap = e / g.Cw, c = e - tap * g.Cw;
+        const int i = tap / g.fy, j = tap - i * g.fy;
+        const int xi = i + xo * g.sx - g.px, yi = j + yo * g.sy - g.py;
+        const bool ok = xi >= 0 && xi < g.H && yi >= 0 && yi < g.Wd;
+        out[t] = ok ? in[((b * g.H + xi) * g.Wd + yi) * g.Cw + c] : (W)0;
+    }
 }
 
 // ---- max-pool: OR over the fixed 2x2 window (extensions/src/max_pool2d.cu:19-32) ---------------
@@ -31,24 +33,26 @@ template <typename W>
 __global__ __launch_bounds__(256) void max_pool_kernel(W *__restrict__ out, const W *__restrict__ in, int64_t total,
                                                        ConvGeom g)
 {
-    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (t >= total) return;
-    const int64_t pix = t / g.Cw;
-    const int c = (int)(t - pix * g.Cw);
-    const int hw = g.h * g.w;
-    const int64_t b = pix / hw;
-    const int loc = (int)(pix - b * hw);
-    const int xo = loc / g.w, yo = loc - xo * g.w;
-    const W *img = in + b * (int64_t)g.H * g.Wd * g.Cw;
-    W v = 0;
+    NB_FLAT_LOOP(t, total)
+    {
+        if (t >= total) continue;
+        const int64_t pix = t / g.Cw;
+        const int c = (int)(t - pix * g.Cw);
+        const int hw = g.h * g.w;
+        const int64_t b = pix / hw;
+        const int loc = (int)(pix - b * hw);
+        const int xo = loc / g.w, yo = loc - xo * g.w;
+        const W *img = in + b * (int64_t)g.H * g.Wd * g.Cw;
+        W v = 0;
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+        for (int i = 0; i < 2; i++)
 #pragma unroll
-        for (int j = 0; j < 2; j++) {
-            const int xi = i + xo * g.sx - g.px, yi = j + yo * g.sy - g.py;
-            if (xi >= 0 && xi < g.H && yi >= 0 && yi < g.Wd) v |= img[((int64_t)xi * g.Wd + yi) * g.Cw + c];
-        }
-    out[t] = v;
+            for (int j = 0; j < 2; j++) {
+                const int xi = i + xo * g.sx - g.px, yi = j + yo * g.sy - g.py;
+                if (xi >= 0 && xi < g.H && yi >= 0 && yi < g.Wd) v |= img[((int64_t)xi * g.Wd + yi) * g.Cw + c];
+            }
+        out[t] = v;
+    }
 }
 
 // ---- conv: row-per-lane kernel with the implicit-im2col loader ----------------------------------
@@ -143,9 +147,8 @@ int im2col_impl(W *out, const W *in, int64_t D, int64_t H, int64_t Wd, int64_t C
     NB_REQUIRE_PTR(in);
     NB_REQUIRE_ALIGNED(out, sizeof(W));
     NB_REQUIRE_ALIGNED(in, sizeof(W));
-    const int64_t blocks = ceil_div(total, 256);
-    NB_REQUIRE(blocks <= kMaxGridX, "%s: %lld output words exceed one launch", who, (long long)total);
-    im2col_kernel<W><<<dim3((unsigned)blocks), dim3(256), 0, as_stream(stream)>>>(out, in, total, g);
+    const unsigned blocks = grid_for(total);
+    im2col_kernel<W><<<dim3(blocks), dim3(256), 0, as_stream(stream)>>>(out, in, total, g);
     return check_launch(who);
 }
 
@@ -161,9 +164,8 @@ int max_pool_impl(W *out, const W *in, int64_t B, int64_t H, int64_t Wd, int64_t
     NB_REQUIRE_PTR(in);
     NB_REQUIRE_ALIGNED(out, sizeof(W));
     NB_REQUIRE_ALIGNED(in, sizeof(W));
-    const int64_t blocks = ceil_div(total, 256);
-    NB_REQUIRE(blocks <= kMaxGridX, "%s: %lld output words exceed one launch", who, (long long)total);
-    max_pool_kernel<W><<<dim3((unsigned)blocks), dim3(256), 0, as_stream(stream)>>>(out, in, total, g);
+    const unsigned blocks = grid_for(total);
+    max_pool_kernel<W><<<dim3(blocks), dim3(256), 0, as_stream(stream)>>>(out, in, total, g);
     return check_launch(who);
 }
 

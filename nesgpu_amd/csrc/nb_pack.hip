@@ -27,20 +27,22 @@ __global__ __launch_bounds__(256) void pack_vec16_kernel(W *__restrict__ out, co
                                                          int64_t total_words, int Rw, int64_t C)
 {
     constexpr int bits = WordTraits<W>::bits;
-    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (t >= total_words) return;
-    const int64_t row = t / Rw;
-    const int y = (int)(t - row * Rw);
-    const int64_t col0 = (int64_t)y * bits;
-    const uint4 *src = reinterpret_cast<const uint4 *>(in + row * C + col0);
-    int64_t left = C - col0;
-    const int chunks = (int)((left < bits ? left : bits) >> 4);
-    W w = 0;
+    NB_FLAT_LOOP(t, total_words)
+    {
+        if (t >= total_words) continue;
+        const int64_t row = t / Rw;
+        const int y = (int)(t - row * Rw);
+        const int64_t col0 = (int64_t)y * bits;
+        const uint4 *src = reinterpret_cast<const uint4 *>(in + row * C + col0);
+        int64_t left = C - col0;
+        const int chunks = (int)((left < bits ? left : bits) >> 4);
+        W w = 0;
 #pragma unroll
-    for (int c = 0; c < bits / 16; c++) {
-        if (c < chunks) w |= (W)bits16_of_bools(src[c]) << (16 * c);
+        for (int c = 0; c < bits / 16; c++) {
+            if (c < chunks) w |= (W)bits16_of_bools(src[c]) << (16 * c);
+        }
+        out[t] = w;
     }
-    out[t] = w;
 }
 
 // Generic: one thread per output word, byte loads, any C.
@@ -49,17 +51,19 @@ __global__ __launch_bounds__(256) void pack_generic_kernel(W *__restrict__ out, 
                                                            int64_t total_words, int Rw, int64_t C)
 {
     constexpr int bits = WordTraits<W>::bits;
-    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (t >= total_words) return;
-    const int64_t row = t / Rw;
-    const int y = (int)(t - row * Rw);
-    const int64_t col0 = (int64_t)y * bits;
-    const uint8_t *src = in + row * C + col0;
-    int64_t left = C - col0;
-    const int nb_ = (int)(left < bits ? left : bits);
-    W w = 0;
-    for (int i = 0; i < nb_; i++) w |= (W)(src[i] != 0) << i;
-    out[t] = w;
+    NB_FLAT_LOOP(t, total_words)
+    {
+        if (t >= total_words) continue;
+        const int64_t row = t / Rw;
+        const int y = (int)(t - row * Rw);
+        const int64_t col0 = (int64_t)y * bits;
+        const uint8_t *src = in + row * C + col0;
+        int64_t left = C - col0;
+        const int nb_ = (int)(left < bits ? left : bits);
+        W w = 0;
+        for (int i = 0; i < nb_; i++) w |= (W)(src[i] != 0) << i;
+        out[t] = w;
+    }
 }
 
 // One thread per 16 output bytes (16 bits of a word).
@@ -69,17 +73,19 @@ __global__ __launch_bounds__(256) void unpack_kernel(uint8_t *__restrict__ out, 
 {
     constexpr int bits = WordTraits<W>::bits;
     constexpr int per = bits / 16;
-    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (t >= total_chunks) return;
-    const W w = in[t / per];
-    const uint32_t h = (uint32_t)(w >> (16 * (int)(t % per))) & 0xFFFFu;
-    uint32_t d[4];
+    NB_FLAT_LOOP(t, total_chunks)
+    {
+        if (t >= total_chunks) continue;
+        const W w = in[t / per];
+        const uint32_t h = (uint32_t)(w >> (16 * (int)(t % per))) & 0xFFFFu;
+        uint32_t d[4];
 #pragma unroll
-    for (int q = 0; q < 4; q++) {
-        const uint32_t nib = (h >> (4 * q)) & 0xFu;
-        d[q] = (nib * 0x00204081u) & 0x01010101u;   // bit j -> byte j
+        for (int q = 0; q < 4; q++) {
+            const uint32_t nib = (h >> (4 * q)) & 0xFu;
+            d[q] = (nib * 0x00204081u) & 0x01010101u;   // bit j -> byte j
+        }
+        reinterpret_cast<uint4 *>(out)[t] = make_uint4(d[0], d[1], d[2], d[3]);
     }
-    reinterpret_cast<uint4 *>(out)[t] = make_uint4(d[0], d[1], d[2], d[3]);
 }
 
 template <typename W>
@@ -87,17 +93,19 @@ __global__ __launch_bounds__(256) void int8pack_kernel(W *__restrict__ out, cons
                                                        int64_t total_words, int Rw, int64_t C)
 {
     constexpr int per = WordTraits<W>::bits / 8;
-    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (t >= total_words) return;
-    const int64_t row = t / Rw;
-    const int y = (int)(t - row * Rw);
-    const int64_t col0 = (int64_t)y * per;
-    const uint8_t *src = in + row * C + col0;
-    int64_t left = C - col0;
-    const int nb_ = (int)(left < per ? left : per);
-    W w = 0;
-    for (int i = 0; i < nb_; i++) w |= (W)src[i] << (8 * i);
-    out[t] = w;
+    NB_FLAT_LOOP(t, total_words)
+    {
+        if (t >= total_words) continue;
+        const int64_t row = t / Rw;
+        const int y = (int)(t - row * Rw);
+        const int64_t col0 = (int64_t)y * per;
+        const uint8_t *src = in + row * C + col0;
+        int64_t left = C - col0;
+        const int nb_ = (int)(left < per ? left : per);
+        W w = 0;
+        for (int i = 0; i < nb_; i++) w |= (W)src[i] << (8 * i);
+        out[t] = w;
+    }
 }
 
 template <typename W>
@@ -112,12 +120,11 @@ int pack_impl(W *out, const uint8_t *in, int64_t R, int64_t C, nb_stream_t strea
     NB_REQUIRE_PTR(in);
     NB_REQUIRE_ALIGNED(out, sizeof(W));
     NB_REQUIRE(Rw <= 2147483647LL, "%s: row of %lld words is too long", who, (long long)Rw);
-    const int64_t blocks = ceil_div(total, 256);
-    NB_REQUIRE(blocks <= kMaxGridX, "%s: %lld output words exceed one launch", who, (long long)total);
+    const unsigned blocks = grid_for(total);
     if ((C & 15) == 0 && aligned(in, 16))
-        pack_vec16_kernel<W><<<dim3((unsigned)blocks), dim3(256), 0, as_stream(stream)>>>(out, in, total, (int)Rw, C);
+        pack_vec16_kernel<W><<<dim3(blocks), dim3(256), 0, as_stream(stream)>>>(out, in, total, (int)Rw, C);
     else
-        pack_generic_kernel<W><<<dim3((unsigned)blocks), dim3(256), 0, as_stream(stream)>>>(out, in, total, (int)Rw, C);
+        pack_generic_kernel<W><<<dim3(blocks), dim3(256), 0, as_stream(stream)>>>(out, in, total, (int)Rw, C);
     return check_launch(who);
 }
 
@@ -132,9 +139,8 @@ int unpack_impl(uint8_t *out, const W *in, int64_t R, int64_t Rw, nb_stream_t st
     NB_REQUIRE_PTR(in);
     NB_REQUIRE_ALIGNED(in, sizeof(W));
     NB_REQUIRE_ALIGNED(out, 16);
-    const int64_t blocks = ceil_div(chunks, 256);
-    NB_REQUIRE(blocks <= kMaxGridX, "%s: %lld words exceed one launch", who, (long long)(R * Rw));
-    unpack_kernel<W><<<dim3((unsigned)blocks), dim3(256), 0, as_stream(stream)>>>(out, in, chunks);
+    const unsigned blocks = grid_for(chunks);
+    unpack_kernel<W><<<dim3(blocks), dim3(256), 0, as_stream(stream)>>>(out, in, chunks);
     return check_launch(who);
 }
 
@@ -150,9 +156,8 @@ int int8pack_impl(W *out, const uint8_t *in, int64_t R, int64_t C, nb_stream_t s
     NB_REQUIRE_PTR(in);
     NB_REQUIRE_ALIGNED(out, sizeof(W));
     NB_REQUIRE(Rw <= 2147483647LL, "%s: row of %lld words is too long", who, (long long)Rw);
-    const int64_t blocks = ceil_div(total, 256);
-    NB_REQUIRE(blocks <= kMaxGridX, "%s: %lld output words exceed one launch", who, (long long)total);
-    int8pack_kernel<W><<<dim3((unsigned)blocks), dim3(256), 0, as_stream(stream)>>>(out, in, total, (int)Rw, C);
+    const unsigned blocks = grid_for(total);
+    int8pack_kernel<W><<<dim3(blocks), dim3(256), 0, as_stream(stream)>>>(out, in, total, (int)Rw, C);
     return check_launch(who);
 }
 

@@ -12,8 +12,11 @@ namespace nb {
 struct WordsSrc {
     const uint32_t *__restrict__ p;
     // four words starting at flat index g (g % 4 == 0, p 16-byte aligned)
-    __device__ __forceinline__ uint4 load4(int64_t g) const { return *reinterpret_cast<const uint4 *>(p + g); }
-    __device__ __forceinline__ uint32_t load1(int64_t g) const { return p[g]; }
+    __device__ __forceinline__ uint4 load4(int64_t g) const { return load_stream16(p + g); }
+    __device__ __forceinline__ uint32_t load1(int64_t g) const { return load_stream4(p + g); }
+    // wave-uniform row start `row0` (flat index) plus a 32-bit per-lane offset: lets the load use a
+    // scalar base register and a 32-bit vector offset
+    __device__ __forceinline__ uint4 load4(int64_t row0, uint32_t off) const { return load_stream16(p + row0 + off); }
 };
 
 struct PhiloxSrc {
@@ -21,6 +24,7 @@ struct PhiloxSrc {
     // (first + g) % 4 == 0 is guaranteed by the host for load4
     __device__ __forceinline__ uint4 load4(int64_t g) const { return philox_block(key, (key.first + (uint64_t)g) >> 2); }
     __device__ __forceinline__ uint32_t load1(int64_t g) const { return philox_word(key, key.first + (uint64_t)g); }
+    __device__ __forceinline__ uint4 load4(int64_t row0, uint32_t off) const { return load4(row0 + off); }
 };
 
 // threshold of columns c..c+3 of row r
@@ -38,29 +42,37 @@ __device__ __forceinline__ uint32_t nibble_lt(uint4 w, uint4 t)
 // ---- materialised sampler, wide path: C % bits == 0 and 16-byte aligned streams ------------------
 // One lane per 4 columns; bits/4 neighbouring lanes assemble one output word by OR-ing their
 // shifted nibbles across the lane group.
-template <typename W, class Src>
-__global__ __launch_bounds__(256) void sample_wide_kernel(W *__restrict__ out, const W *__restrict__ base,
-                                                          const uint32_t *__restrict__ thresh, uint32_t ts, Src src,
-                                                          int64_t total_quads, int64_t RC4, int C4)
+template <typename W, class Src, int U, int BS, bool HAS_THR>
+__global__ __launch_bounds__(BS) void sample_wide_kernel(W *__restrict__ out, const W *__restrict__ base,
+                                                         const uint32_t *__restrict__ thresh, uint32_t ts, Src src,
+                                                         int64_t total_quads, int64_t RC4)
 {
     constexpr int bits = WordTraits<W>::bits;
     constexpr int G = bits / 4;  // lanes per output word
-    const int64_t q = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    const bool live = q < total_quads;
-    W v = 0;
-    int64_t rq = 0;
-    if (live) {
-        rq = q % RC4;  // quad index inside one member: row * C4 + c4
-        const uint4 w = src.load4(q * 4);
-        const uint4 t = thr4(thresh, ts, rq * 4);
-        v = (W)nibble_lt(w, t) << (4 * (int)(q & (G - 1)));
-    }
+    // a workgroup walks tiles of BS*U consecutive quads; thread t owns quads tile + u*BS + t
+    for (int64_t tile = (int64_t)blockIdx.x * (BS * U); tile < total_quads; tile += (int64_t)gridDim.x * (BS * U)) {
+        uint4 w[U], t[U];
+        int64_t rq[U];
 #pragma unroll
-    for (int off = 1; off < G; off <<= 1) v |= __shfl_xor(v, off);
-    if (live && (q & (G - 1)) == 0) {
-        const int64_t wi = q / G;  // flat output word index (C % bits == 0)
-        if (base) v ^= base[rq / G];
-        out[wi] = v;
+        for (int u = 0; u < U; u++) {
+            const int64_t q = tile + (int64_t)u * BS + threadIdx.x;
+            const int64_t qc = q < total_quads ? q : total_quads - 1;  // clamp: no branch around the load
+            rq[u] = qc % RC4;                                          // quad index inside one member
+            t[u] = HAS_THR ? *reinterpret_cast<const uint4 *>(thresh + rq[u] * 4) : make_uint4(ts, ts, ts, ts);
+            w[u] = src.load4(qc * 4);
+        }
+        __builtin_amdgcn_sched_barrier(0);  // all U stream loads in flight before the first use
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int64_t q = tile + (int64_t)u * BS + threadIdx.x;
+            W v = (W)nibble_lt(w[u], t[u]) << (4 * (int)(q & (G - 1)));
+#pragma unroll
+            for (int off = 1; off < G; off <<= 1) v |= __shfl_xor(v, off);
+            if (q < total_quads && (q & (G - 1)) == 0) {
+                if (base) v ^= base[rq[u] / G];
+                out[q / G] = v;  // flat output word index (C % bits == 0)
+            }
+        }
     }
 }
 
@@ -72,25 +84,26 @@ __global__ __launch_bounds__(256) void sample_ballot_kernel(W *__restrict__ out,
 {
     constexpr int bits = WordTraits<W>::bits;
     const int lane = threadIdx.x & 63;
-    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);  // (m, r) flattened
-    if (row >= nrows) return;                                          // wave-uniform exit
-    const int64_t r = row % R;
-    for (int c0 = 0; c0 < C; c0 += 64) {
-        const int c = c0 + lane;
-        bool bit = false;
-        if (c < C) {
-            const uint32_t t = thresh ? thresh[r * C + c] : ts;
-            bit = src.load1(row * C + c) < t;
-        }
-        const uint64_t m = __ballot(bit);
-        if (lane == 0) {
-            if (bits == 64) {
-                const int wi = c0 >> 6;
-                out[row * Rw + wi] = (W)m ^ (base ? base[r * Rw + wi] : (W)0);
-            } else {
-                const int wi = c0 >> 5;
-                out[row * Rw + wi] = (W)m ^ (base ? base[r * Rw + wi] : (W)0);
-                if (wi + 1 < Rw) out[row * Rw + wi + 1] = (W)(m >> 32) ^ (base ? base[r * Rw + wi + 1] : (W)0);
+    // one wave per (m, r) row; wave-uniform stride loop
+    for (int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6); row < nrows; row += (int64_t)gridDim.x * 4) {
+        const int64_t r = row % R;
+        for (int c0 = 0; c0 < C; c0 += 64) {
+            const int c = c0 + lane;
+            bool bit = false;
+            if (c < C) {
+                const uint32_t t = thresh ? thresh[r * C + c] : ts;
+                bit = src.load1(row * C + c) < t;
+            }
+            const uint64_t m = __ballot(bit);
+            if (lane == 0) {
+                if (bits == 64) {
+                    const int wi = c0 >> 6;
+                    out[row * Rw + wi] = (W)m ^ (base ? base[r * Rw + wi] : (W)0);
+                } else {
+                    const int wi = c0 >> 5;
+                    out[row * Rw + wi] = (W)m ^ (base ? base[r * Rw + wi] : (W)0);
+                    if (wi + 1 < Rw) out[row * Rw + wi + 1] = (W)(m >> 32) ^ (base ? base[r * Rw + wi + 1] : (W)0);
+                }
             }
         }
     }
@@ -111,7 +124,7 @@ __global__ __launch_bounds__(256) void seeded_bmv_wide_kernel(int32_t *__restric
     const int lane = threadIdx.x & 63;
     const int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     const int64_t m = wave / groups_per_member;
-    if (m >= n) return;  // wave-uniform
+    if (m >= n) return;  // wave-uniform; the host keeps n * groups_per_member within one launch
     const int64_t r0 = (wave - m * groups_per_member) * RPW;
     int acc[RPW];
 #pragma unroll
@@ -142,6 +155,92 @@ __global__ __launch_bounds__(256) void seeded_bmv_wide_kernel(int32_t *__restric
         for (int q = 0; q < RPW; q++)
             if (r0 + q < R) Cout[m * R + r0 + q] = acc[q];
     }
+}
+
+// Streaming path (C % 256 == 0, aligned streams): every lane issues RPW*ITU independent 16-byte loads of
+// the word stream before it consumes any of them, a 1024-thread workgroup covers a contiguous span of
+// rows, and the per-lane work is four compares, a nibble XOR and one v_bcnt per load.
+template <typename W, class Src, int RPW, int ITU, bool HAS_THR, bool HAS_BASE>
+__global__ __launch_bounds__(1024) void seeded_bmv_stream_kernel(int32_t *__restrict__ Cout,
+                                                                 const W *__restrict__ base,
+                                                                 const uint32_t *__restrict__ thresh, uint32_t ts,
+                                                                 const W *__restrict__ x, Src src, int64_t n, int R,
+                                                                 int C4, int Rw, int groups_per_member)
+{
+    constexpr int bits = WordTraits<W>::bits;
+    constexpr int G = bits / 4;
+    const int lane = threadIdx.x & 63;
+    // wave-uniform quantities are forced into scalar registers (the host keeps n*groups below 2^31)
+    const uint32_t wave = blockIdx.x * 16u + (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const uint32_t m32 = wave / (uint32_t)groups_per_member;
+    if (m32 >= n) return;
+    const int64_t m = m32;
+    const int r0 = (int)(wave - m32 * (uint32_t)groups_per_member) * RPW;
+    const int64_t C = (int64_t)C4 * 4;
+    int rows[RPW];
+#pragma unroll
+    for (int q = 0; q < RPW; q++) rows[q] = r0 + q < R ? r0 + q : R - 1;  // tail rows are recomputed, not stored
+    int acc[RPW];
+#pragma unroll
+    for (int q = 0; q < RPW; q++) acc[q] = 0;
+    const int sh = 4 * (lane & (G - 1));
+    for (int c40 = 0; c40 < C4; c40 += 64 * ITU) {
+        // Issue every load of this step before consuming any: the small cached operands (x, base,
+        // thresholds) first, then the RPW*ITU 16-byte loads of the word stream.
+        W bx[RPW][ITU];
+        uint4 t[RPW][ITU];
+        uint4 w[RPW][ITU];
+#pragma unroll
+        for (int it = 0; it < ITU; it++) {
+            const int c4 = c40 + it * 64 + lane;
+            const int wi = c4 / G;
+            const W xw = x[m * Rw + wi];
+#pragma unroll
+            for (int q = 0; q < RPW; q++) {
+                bx[q][it] = HAS_BASE ? (W)(xw ^ base[(int64_t)rows[q] * Rw + wi]) : xw;
+                t[q][it] = HAS_THR ? *reinterpret_cast<const uint4 *>(thresh + rows[q] * C + 4 * (int64_t)c4)
+                                   : make_uint4(ts, ts, ts, ts);
+            }
+        }
+#pragma unroll
+        for (int q = 0; q < RPW; q++)
+#pragma unroll
+            for (int it = 0; it < ITU; it++)
+                w[q][it] = src.load4((m * R + rows[q]) * C, 4u * (uint32_t)(c40 + it * 64 + lane));
+        __builtin_amdgcn_sched_barrier(0);  // do not let the scheduler sink a load next to its use
+#pragma unroll
+        for (int it = 0; it < ITU; it++)
+#pragma unroll
+            for (int q = 0; q < RPW; q++)
+                acc[q] += __popc(nibble_lt(w[q][it], t[q][it]) ^ ((uint32_t)(bx[q][it] >> sh) & 0xFu));
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+#pragma unroll
+        for (int q = 0; q < RPW; q++) acc[q] += __shfl_xor(acc[q], off);
+    }
+    if (lane == 0) {
+#pragma unroll
+        for (int q = 0; q < RPW; q++)
+            if (r0 + q < R) Cout[m * R + r0 + q] = acc[q];
+    }
+}
+
+template <typename W, class Src, int RPW, int ITU>
+static void launch_bmv_stream(int32_t *Cout, const W *base, const uint32_t *thresh, uint32_t ts, const W *x, Src src,
+                              int64_t n, int64_t R, int64_t C, int Rw, hipStream_t s)
+{
+    const int gpm = (int)ceil_div(R, RPW);
+    const int64_t waves = n * gpm;
+    const dim3 grid((unsigned)ceil_div(waves, 16)), block(1024);
+#define NB_LAUNCH_STREAM(T, B)                                                                                   \
+    seeded_bmv_stream_kernel<W, Src, RPW, ITU, T, B><<<grid, block, 0, s>>>(Cout, base, thresh, ts, x, src, n, (int)R, \
+                                                                            (int)(C / 4), Rw, gpm)
+    if (thresh && base) NB_LAUNCH_STREAM(true, true);
+    else if (thresh) NB_LAUNCH_STREAM(true, false);
+    else if (base) NB_LAUNCH_STREAM(false, true);
+    else NB_LAUNCH_STREAM(false, false);
+#undef NB_LAUNCH_STREAM
 }
 
 // Generic path: one wave per (member,row), one column per lane and step.
@@ -175,17 +274,20 @@ __global__ __launch_bounds__(256) void seeded_bmv_generic_kernel(int32_t *__rest
 __global__ __launch_bounds__(256) void philox_words_kernel(uint32_t *__restrict__ out, PhiloxKey key, int64_t count)
 {
     // one thread per aligned block of the stream; head/tail blocks are partial
-    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
     const uint64_t blk0 = key.first >> 2;
-    const uint64_t blk = blk0 + (uint64_t)t;
-    const uint64_t gbeg = blk << 2;
-    if (gbeg >= key.first + (uint64_t)count) return;
-    const uint4 b = philox_block(key, blk);
-    const uint32_t v[4] = {b.x, b.y, b.z, b.w};
+    const int64_t nblk = (int64_t)(((key.first + (uint64_t)count + 3) >> 2) - blk0);
+    NB_FLAT_LOOP(t, nblk)
+    {
+        if (t >= nblk) continue;
+        const uint64_t blk = blk0 + (uint64_t)t;
+        const uint64_t gbeg = blk << 2;
+        const uint4 b = philox_block(key, blk);
+        const uint32_t v[4] = {b.x, b.y, b.z, b.w};
 #pragma unroll
-    for (int e = 0; e < 4; e++) {
-        const uint64_t g = gbeg + e;
-        if (g >= key.first && g < key.first + (uint64_t)count) out[g - key.first] = v[e];
+        for (int e = 0; e < 4; e++) {
+            const uint64_t g = gbeg + e;
+            if (g >= key.first && g < key.first + (uint64_t)count) out[g - key.first] = v[e];
+        }
     }
 }
 
@@ -199,8 +301,7 @@ static int sample_check(const void *out, const W *base, const uint32_t *thresh, 
     if (*empty) return NB_OK;
     NB_REQUIRE_PTR(out);
     NB_REQUIRE(C <= (1 << 30), "%s: C=%lld too large", who, (long long)C);
-    NB_REQUIRE(n * R <= (1LL << 40) && ceil_div(n * R, 4) <= kMaxGridX, "%s: n*R=%lld rows exceed one launch", who,
-               (long long)(n * R));
+    NB_REQUIRE(n * R <= (1LL << 40), "%s: n*R=%lld rows is too many", who, (long long)(n * R));
     if (base) NB_REQUIRE_ALIGNED(base, sizeof(W));
     if (thresh) NB_REQUIRE_ALIGNED(thresh, 4);
     return NB_OK;
@@ -218,11 +319,18 @@ int sample_impl(W *out, const W *base, const uint32_t *thresh, uint32_t ts, Src 
     hipStream_t s = as_stream(stream);
     const int64_t Rw = ceil_div(C, bits);
     const int64_t quads = n * R * (C / 4);
-    if (C % bits == 0 && src_vec_ok && (!thresh || aligned(thresh, 16)) && ceil_div(quads, 256) <= kMaxGridX) {
-        sample_wide_kernel<W, Src><<<dim3((unsigned)ceil_div(quads, 256)), dim3(256), 0, s>>>(
-            out, base, thresh, ts, src, quads, R * (C / 4), (int)(C / 4));
+    if (C % bits == 0 && src_vec_ok && (!thresh || aligned(thresh, 16))) {
+        constexpr int U = 4, BS = 1024;
+        const int64_t tiles = ceil_div(quads, (int64_t)BS * U);
+        const dim3 grid((unsigned)(tiles < kMaxBlocks ? tiles : kMaxBlocks)), block(BS);
+        if (thresh)
+            sample_wide_kernel<W, Src, U, BS, true><<<grid, block, 0, s>>>(out, base, thresh, ts, src, quads,
+                                                                           R * (C / 4));
+        else
+            sample_wide_kernel<W, Src, U, BS, false><<<grid, block, 0, s>>>(out, base, thresh, ts, src, quads,
+                                                                            R * (C / 4));
     } else {
-        sample_ballot_kernel<W, Src><<<dim3((unsigned)ceil_div(n * R, 4)), dim3(256), 0, s>>>(
+        sample_ballot_kernel<W, Src><<<dim3(grid_for(n * R * 64)), dim3(256), 0, s>>>(
             out, base, thresh, ts, src, n * R, R, (int)C, (int)Rw);
     }
     return check_launch(who);
@@ -250,7 +358,14 @@ int seeded_bmv_impl(int32_t *Cout, const W *base, const uint32_t *thresh, uint32
     hipStream_t s = as_stream(stream);
     const int64_t Rw = ceil_div(C, bits);
     constexpr int RPW = 4;
-    if (C > 0 && (C & 3) == 0 && src_vec_ok && (!thresh || aligned(thresh, 16))) {
+    const bool vec_ok = C > 0 && (C & 3) == 0 && src_vec_ok && (!thresh || aligned(thresh, 16));
+    if (vec_ok && (C & 255) == 0 && n * R < (1LL << 31) && ceil_div(n * R, 16) <= kMaxBlocks) {
+        const int64_t it = C / 256;  // wave-steps per row
+        if ((it & 7) == 0) launch_bmv_stream<W, Src, 1, 8>(Cout, base, thresh, ts, x, src, n, R, C, (int)Rw, s);
+        else if ((it & 3) == 0) launch_bmv_stream<W, Src, 2, 4>(Cout, base, thresh, ts, x, src, n, R, C, (int)Rw, s);
+        else if ((it & 1) == 0) launch_bmv_stream<W, Src, 4, 2>(Cout, base, thresh, ts, x, src, n, R, C, (int)Rw, s);
+        else launch_bmv_stream<W, Src, 8, 1>(Cout, base, thresh, ts, x, src, n, R, C, (int)Rw, s);
+    } else if (vec_ok) {
         const int64_t gpm = ceil_div(R, RPW);
         const int64_t waves = n * gpm;
         seeded_bmv_wide_kernel<W, Src, RPW><<<dim3((unsigned)ceil_div(waves, 4)), dim3(256), 0, s>>>(
@@ -307,9 +422,7 @@ int nb_philox_words(uint32_t *out, uint64_t seed, uint64_t subseq, uint64_t firs
     if (!out) return nb::fail(NB_ERR_NULL, "nb_philox_words: out is NULL");
     if (!nb::aligned(out, 4)) return nb::fail(NB_ERR_ALIGN, "nb_philox_words: out is not 4-byte aligned");
     const int64_t blocks4 = (int64_t)(((first + (uint64_t)count + 3) >> 2) - (first >> 2));
-    if (nb::ceil_div(blocks4, 256) > nb::kMaxGridX)
-        return nb::fail(NB_ERR_SHAPE, "nb_philox_words: %lld words exceed one launch", (long long)count);
-    nb::philox_words_kernel<<<dim3((unsigned)nb::ceil_div(blocks4, 256)), dim3(256), 0, nb::as_stream(s)>>>(
+    nb::philox_words_kernel<<<dim3(nb::grid_for(blocks4)), dim3(256), 0, nb::as_stream(s)>>>(
         out, nb::PhiloxKey{seed, subseq, first}, count);
     return nb::check_launch("nb_philox_words");
 }

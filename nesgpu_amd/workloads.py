@@ -1,0 +1,179 @@
+"""The five benchmark configurations as seeded synthetic workloads on one GPU.
+
+Every builder returns a :class:`Workload` whose ``step()`` launches the population forward of that
+configuration (inputs already resident in HBM) and returns its output tensor.  Small operands (inputs,
+base weights) come from ``torch.Generator().manual_seed(seed)`` on the CPU; the per-bit random words come
+from the library's Philox4x32-10 stream (seed, subsequence) so that a CPU checker can regenerate exactly the
+same words for any subset of members without moving gigabytes over PCIe.
+
+Bit convention: +1 <-> bit 1.  Ops return raw popcount sums ``popc``; the reference layer applies
+``2*popc - K`` (modules/binary.py:97,145).
+"""
+from dataclasses import dataclass, field
+from typing import Callable, Dict
+
+import torch
+
+from .extensions import booleanOperations as ops
+
+# floor(p * 2**32) for the flip probabilities the configurations name
+T_P01 = 42949672
+T_P02 = 85899345
+T_P05 = 214748364
+
+HBM_PEAK = 8.0e12                     # B/s, MI355X datasheet
+VALU_POPC_PEAK = 6.29e14              # bit-MAC/s: 256 CU x 64 lanes x 2.4 GHz / (4 lane-ops per 64 bits) x 64
+
+
+@dataclass
+class Workload:
+    name: str
+    population: int
+    bit_macs: int                      # valid bit-MACs per step (word padding never counted)
+    algo_bytes: int                    # algorithmic HBM bytes per step of the dominant kernel
+    bound: str                         # "hbm" or "valu"
+    step: Callable[[], torch.Tensor]
+    tensors: Dict[str, torch.Tensor] = field(default_factory=dict)
+    meta: Dict[str, object] = field(default_factory=dict)
+
+
+def _gen(seed):
+    g = torch.Generator(device="cpu")
+    g.manual_seed(seed)
+    return g
+
+
+def _bits(g, shape):
+    return torch.randint(0, 2, shape, generator=g, dtype=torch.uint8).bool()
+
+
+def linear_flip_materialised(D=1024, out_f=256, in_f=256, T=T_P01, seed=0, dtype=torch.int64, device="cuda"):
+    """Config 1: per-member weights = base ^ flips are materialised once (outside the step); the step is the
+    batched matrix-vector XOR-popcount product, one input row per member."""
+    g = _gen(seed)
+    base_bits = _bits(g, (out_f, in_f))
+    x_bits = _bits(g, (D, in_f))
+    base = ops.pack(base_bits.to(device), dtype)
+    x = ops.pack(x_bits.to(device), dtype)
+    W = ops.flip_philox(base, in_f, D, T, seed, subsequence=1)
+    xv = x.view(D, -1, 1)
+    Kw = W.size(2)
+    w = Workload(
+        name="linear %dx%d D=%d N=1 p-flip materialised weights" % (out_f, in_f, D),
+        population=D, bit_macs=D * out_f * in_f,
+        algo_bytes=W.numel() * W.element_size() + x.numel() * x.element_size() + D * out_f * 4,
+        bound="hbm", step=lambda: ops.bmm(W, xv),
+        tensors=dict(base=base, x=x, W=W), meta=dict(T=T, seed=seed, subsequence=1, in_f=in_f, out_f=out_f, Kw=Kw))
+    return w
+
+
+def linear_flip_fused(D=1024, out_f=1024, in_f=1024, T=T_P05, seed=0, dtype=torch.int64, device="cuda"):
+    """Config 2: flip masks are sampled from SUPPLIED uint32 words (threshold compare) inside the XOR-popcount
+    product; the words are the only large operand (4 bytes per weight bit)."""
+    g = _gen(seed)
+    base_bits = _bits(g, (out_f, in_f))
+    x_bits = _bits(g, (D, in_f))
+    base = ops.pack(base_bits.to(device), dtype)
+    x = ops.pack(x_bits.to(device), dtype)
+    words = ops.philox_words(D * out_f * in_f, seed, subsequence=2, device=device).view(D, out_f, in_f)
+    w = Workload(
+        name="linear %dx%d D=%d N=1 p=0.05 flips from supplied uint32 words, fused" % (out_f, in_f, D),
+        population=D, bit_macs=D * out_f * in_f,
+        algo_bytes=words.numel() * 4 + base.numel() * base.element_size() + x.numel() * x.element_size()
+        + D * out_f * 4,
+        bound="hbm", step=lambda: ops.seeded_bmv_from_words(T, x, words, base=base),
+        tensors=dict(base=base, x=x, words=words), meta=dict(T=T, seed=seed, subsequence=2, in_f=in_f, out_f=out_f))
+    return w
+
+
+def _conv_filters(base_bits, D, O, k, C, T, seed, subseq, dtype, device):
+    """base_bits [O*k*k, C] (rows ordered (out, kx, ky), modules/binary.py:125) -> per-member filters
+    [D, k*k*Cw, O] (modules/binary.py:136-137)."""
+    base = ops.pack(base_bits.to(device), dtype)                                  # [O*k*k, Cw]
+    Wn = ops.flip_philox(base, C, D, T, seed, subsequence=subseq)                # [D, O*k*k, Cw]
+    filt = Wn.view(D, O, k, k, -1).permute(0, 2, 3, 4, 1).reshape(D, -1, O).contiguous()
+    return base, Wn, filt
+
+
+def conv_int32(D=1024, C=64, O=64, S=32, k=3, pad=1, T=T_P02, seed=0, dtype=torch.int64, device="cuda"):
+    """Config 3: batched binary conv, int32 popcount maps out."""
+    g = _gen(seed)
+    x_bits = _bits(g, (D, S, S, C))
+    base_bits = _bits(g, (O * k * k, C))
+    x = ops.pack(x_bits.view(-1, C).to(device), dtype).view(D, S, S, -1)
+    base, Wn, filt = _conv_filters(base_bits, D, O, k, C, T, seed, 3, dtype, device)
+    h = S + 2 * pad - k + 1
+    w = Workload(
+        name="conv %d->%d %dx%d pad %d on %dx%d D=%d int32 out" % (C, O, k, k, pad, S, S, D),
+        population=D, bit_macs=D * h * h * O * k * k * C,
+        algo_bytes=x.numel() * x.element_size() + filt.numel() * filt.element_size() + D * h * h * O * 4,
+        bound="valu", step=lambda: ops.conv(x, filt, k, k, pad, pad, 1, 1),
+        tensors=dict(x=x, base=base, Wn=Wn, filt=filt), meta=dict(T=T, seed=seed, subsequence=3, C=C, O=O, k=k,
+                                                                   pad=pad))
+    return w
+
+
+def conv_sign_pool(D=1024, C=16, O=16, S=64, k=3, pad=1, T=T_P02, seed=0, dtype=torch.int64, device="cuda"):
+    """Config 4: conv -> sign (2*popc - K > 0) -> pack along channels -> 2x2/s2 OR-pool, one fused kernel."""
+    g = _gen(seed)
+    x_bits = _bits(g, (D, S, S, C))
+    base_bits = _bits(g, (O * k * k, C))
+    x = ops.pack(x_bits.view(-1, C).to(device), dtype).view(D, S, S, -1)
+    base, Wn, filt = _conv_filters(base_bits, D, O, k, C, T, seed, 4, dtype, device)
+    K = k * k * C
+    thr = torch.full((D, O), K, dtype=torch.int32, device=device)                # 2*popc > K  <=>  2*popc - K > 0
+    h = S + 2 * pad - k + 1
+    out_words = D * (h // 2) * (h // 2) * ((O + 63) // 64)
+    w = Workload(
+        name="conv %d->%d %dx%d pad %d on %dx%d D=%d -> sign -> 2x2 OR-pool, packed out" % (C, O, k, k, pad, S, S, D),
+        population=D, bit_macs=D * h * h * O * K,
+        algo_bytes=x.numel() * x.element_size() + filt.numel() * filt.element_size() + out_words * 8,
+        bound="valu", step=lambda: ops.conv_act_pack(x, filt, thr, k, k, pad, pad, 1, 1, pool=True),
+        tensors=dict(x=x, base=base, Wn=Wn, filt=filt, thr=thr), meta=dict(T=T, seed=seed, subsequence=4, C=C, O=O,
+                                                                             k=k, pad=pad))
+    return w
+
+
+def cifar_net(D=4096, T=T_P01, seed=0, dtype=torch.int64, device="cuda", classes=10):
+    """Config 5: conv3->64, conv64->64, pool, conv64->128, pool, linear 8192->1024, linear 1024->10 on 3x32x32
+    inputs binarised at their per-channel mean; sign threshold 0 between layers; int32 logits (raw popc)."""
+    g = _gen(seed)
+    z = torch.randn((D, 3, 32, 32), generator=g)
+    x_bits = (z > z.mean(dim=(0, 2, 3), keepdim=True)).permute(0, 2, 3, 1).contiguous()      # [D,32,32,3]
+    x = ops.pack(x_bits.view(-1, 3).to(device), dtype).view(D, 32, 32, 1)
+    layers = []
+    macs = 0
+    subseq = 10
+    for (C, O, S) in ((3, 64, 32), (64, 64, 32), (64, 128, 16)):
+        base_bits = _bits(g, (O * 9, C))
+        base, Wn, filt = _conv_filters(base_bits, D, O, 3, C, T, seed, subseq, dtype, device)
+        del Wn
+        thr = torch.full((D, O), 9 * C, dtype=torch.int32, device=device)
+        layers.append((filt, thr))
+        macs += D * S * S * O * 9 * C
+        subseq += 1
+    b4 = ops.pack(_bits(g, (1024, 8192)).to(device), dtype)
+    W4 = ops.flip_philox(b4, 8192, D, T, seed, subsequence=subseq)              # [D,1024,128]: 4 GiB at D=4096
+    b5 = ops.pack(_bits(g, (classes, 1024)).to(device), dtype)
+    W5 = ops.flip_philox(b5, 1024, D, T, seed, subsequence=subseq + 1)
+    macs += D * 1024 * 8192 + D * classes * 1024
+
+    def step():
+        a = ops.conv_act_pack(x, layers[0][0], layers[0][1], 3, 3, 1, 1, 1, 1)                 # [D,32,32,1]
+        a = ops.conv_act_pack(a, layers[1][0], layers[1][1], 3, 3, 1, 1, 1, 1, pool=True)      # [D,16,16,1]
+        a = ops.conv_act_pack(a, layers[2][0], layers[2][1], 3, 3, 1, 1, 1, 1, pool=True)      # [D,8,8,2]
+        a = a.view(D, -1, 1)                                                                    # [D,128,1]
+        p4 = ops.bmm(W4, a).squeeze(2)                                                          # [D,1024]
+        a = ops.pack(2 * p4 > 8192, dtype).view(D, -1, 1)                                       # [D,16,1]
+        return ops.bmm(W5, a).squeeze(2)                                                        # [D,classes] popc
+
+    w = Workload(
+        name="CIFAR-shaped binary net D=%d (conv3-64, conv64-64, pool, conv64-128, pool, fc8192-1024, fc1024-%d)"
+             % (D, classes),
+        population=D, bit_macs=macs, algo_bytes=W4.numel() * 8, bound="valu", step=step,
+        tensors=dict(x=x, f1=layers[0][0], f2=layers[1][0], f3=layers[2][0], W4=W4, W5=W5),
+        meta=dict(T=T, seed=seed))
+    return w
+
+
+BUILDERS = {1: linear_flip_materialised, 2: linear_flip_fused, 3: conv_int32, 4: conv_sign_pool, 5: cifar_net}

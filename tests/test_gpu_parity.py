@@ -244,7 +244,7 @@ def test_max_pool_vs_oracle(ops, oracle, dtype):
 
 
 SAMPLE_SHAPES = [(3, 4, 64), (2, 3, 1), (5, 2, 63), (2, 5, 65), (3, 2, 200), (4, 7, 256), (2, 576, 64), (3, 10, 1024),
-                 (2, 9, 16), (3, 5, 128), (2, 3, 100)]
+                 (2, 9, 16), (3, 5, 128), (2, 3, 100), (2, 5, 256), (2, 7, 512), (2, 3, 768), (2, 3, 2048), (3, 33, 1024)]
 
 
 @pytest.mark.parametrize("dtype", [torch.int64, torch.int32])
