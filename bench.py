@@ -36,6 +36,7 @@ def parse_args():
     ap.add_argument("--cpu-members", type=int, default=256, help="members of the workload the CPU baseline runs")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU time the baseline leg accumulates")
     ap.add_argument("--only-calib", action="store_true", help="run only the calibration kernels (for counter runs)")
+    ap.add_argument("--only", type=int, default=0, help="time just this configuration (for profiler runs)")
     return ap.parse_args()
 
 
@@ -133,6 +134,16 @@ def main():
     torch.cuda.set_device(0)
     if args.only_calib:
         print(json.dumps({"measured_ceilings": calibrate(torch)}))
+        return 0
+
+    if args.only:
+        w = workloads.BUILDERS[args.only]()
+        pw, pe = time_steps(torch, w.step, args.steps, args.warmup)
+        peak = workloads.HBM_PEAK if w.bound == "hbm" else workloads.VALU_POPC_PEAK
+        work = w.algo_bytes if w.bound == "hbm" else w.bit_macs
+        print(json.dumps({"config": args.only, "workload": w.name, "ms_per_step": round(pw * 1e3, 4),
+                          "event_ms_per_step": round(pe * 1e3, 4), "binary_TOPS": round(2 * w.bit_macs / pw / 1e12, 3),
+                          "bound": w.bound, "roofline_frac": round(work / pe / peak, 4)}))
         return 0
 
     wl = workloads.linear_flip_fused()

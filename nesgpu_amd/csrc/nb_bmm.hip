@@ -63,7 +63,7 @@ __global__ __launch_bounds__(BS) void bmv_kernel(int32_t *__restrict__ C, const 
     }
 }
 
-template <typename W, int KC, int NT, bool SINGLE, class Epi>
+template <typename W, int KC, int NT, bool SINGLE, bool EXACT, class Epi>
 __global__ __launch_bounds__(256) void bmm_rowlane_kernel(RowsA<W> al, const W *__restrict__ Bm, Epi epi, int mblocks,
                                                           int N)
 {
@@ -71,7 +71,7 @@ __global__ __launch_bounds__(256) void bmm_rowlane_kernel(RowsA<W> al, const W *
     const int64_t m = (int64_t)(blockIdx.x - z * mblocks) * 256 + threadIdx.x;
     const typename RowsA<W>::Lane lane = al.lane(z, m);
     const W *__restrict__ Bz = Bm + z * al.Kw * (int64_t)N;
-    rowlane_body<W, KC, NT, SINGLE>(al, lane, Bz, epi, z * al.M + m, z, al.Kw, N);
+    rowlane_body<W, KC, NT, SINGLE, EXACT>(al, lane, Bz, epi, z * al.M + m, z, al.Kw, N);
 }
 
 template <typename W, int L, int V>
@@ -102,10 +102,12 @@ static void dispatch_rowlane(const RowsA<W> &al, const W *B, const Epi &epi, int
 {
     const int mblocks = (int)ceil_div(M, 256);
     const dim3 grid((unsigned)(Z * mblocks)), block(256);
-    if (Kw <= 4) bmm_rowlane_kernel<W, 4, 16, true, Epi><<<grid, block, 0, s>>>(al, B, epi, mblocks, N);
-    else if (Kw <= 9) bmm_rowlane_kernel<W, 9, 16, true, Epi><<<grid, block, 0, s>>>(al, B, epi, mblocks, N);
-    else if (Kw <= 18) bmm_rowlane_kernel<W, 18, 16, true, Epi><<<grid, block, 0, s>>>(al, B, epi, mblocks, N);
-    else bmm_rowlane_kernel<W, 16, 16, false, Epi><<<grid, block, 0, s>>>(al, B, epi, mblocks, N);
+    if (Kw == 9) bmm_rowlane_kernel<W, 9, 16, true, true, Epi><<<grid, block, 0, s>>>(al, B, epi, mblocks, N);
+    else if (Kw == 18) bmm_rowlane_kernel<W, 18, 16, true, true, Epi><<<grid, block, 0, s>>>(al, B, epi, mblocks, N);
+    else if (Kw <= 4) bmm_rowlane_kernel<W, 4, 16, true, false, Epi><<<grid, block, 0, s>>>(al, B, epi, mblocks, N);
+    else if (Kw <= 9) bmm_rowlane_kernel<W, 9, 16, true, false, Epi><<<grid, block, 0, s>>>(al, B, epi, mblocks, N);
+    else if (Kw <= 18) bmm_rowlane_kernel<W, 18, 16, true, false, Epi><<<grid, block, 0, s>>>(al, B, epi, mblocks, N);
+    else bmm_rowlane_kernel<W, 16, 16, false, false, Epi><<<grid, block, 0, s>>>(al, B, epi, mblocks, N);
 }
 
 template <typename W>

@@ -27,6 +27,22 @@ struct WordTraits<uint32_t> {
 __device__ __forceinline__ int popc_xor(uint64_t a, uint64_t b) { return __popcll(a ^ b); }
 __device__ __forceinline__ int popc_xor(uint32_t a, uint32_t b) { return __popc(a ^ b); }
 
+// acc += popcount(a ^ b).  The v_bcnt_u32_b32 is emitted by hand so that its third operand carries the
+// running sum: per 32-bit half exactly one v_xor_b32 and one v_bcnt_u32_b32, no separate add (the
+// compiler otherwise rewrites the sum of two popcounts and the accumulator into bcnt,bcnt,v_add3).
+__device__ __forceinline__ int bcnt_acc(uint32_t x, int acc)
+{
+    int r;
+    asm("v_bcnt_u32_b32 %0, %1, %2" : "=v"(r) : "v"(x), "v"(acc));
+    return r;
+}
+__device__ __forceinline__ void acc_popc_xor(int &acc, uint64_t a, uint64_t b)
+{
+    acc = bcnt_acc((uint32_t)a ^ (uint32_t)b, acc);
+    acc = bcnt_acc((uint32_t)(a >> 32) ^ (uint32_t)(b >> 32), acc);
+}
+__device__ __forceinline__ void acc_popc_xor(int &acc, uint32_t a, uint32_t b) { acc = bcnt_acc(a ^ b, acc); }
+
 // Streaming (read-once) loads: the non-temporal hint keeps a multi-GiB stream from displacing the small
 // reused operands in L2 and measurably raises achieved HBM bandwidth on MI355X.
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));

@@ -58,7 +58,7 @@ __global__ __launch_bounds__(256) void max_pool_kernel(W *__restrict__ out, cons
 // ---- conv: row-per-lane kernel with the implicit-im2col loader ----------------------------------
 // POOLMAP: lanes 4q..4q+3 hold the 2x2 window of pooled pixel q (needed by EpiPack<.,true>);
 // otherwise lane p of a member is output pixel p in row-major order.
-template <typename W, int KC, int NT, bool SINGLE, bool POOLMAP, class Epi>
+template <typename W, int KC, int NT, bool SINGLE, bool EXACT, bool POOLMAP, class Epi>
 __global__ __launch_bounds__(256) void conv_rowlane_kernel(ConvA<W> al, const W *__restrict__ filt, Epi epi,
                                                            int pblocks, int N)
 {
@@ -85,7 +85,7 @@ __global__ __launch_bounds__(256) void conv_rowlane_kernel(ConvA<W> al, const W 
     const typename ConvA<W>::Lane lane = al.lane_at(z, yo, xo, valid);
     const int Kw = g.fx * g.fy * g.Cw;
     const W *__restrict__ Fz = filt + z * (int64_t)Kw * N;
-    rowlane_body<W, KC, NT, SINGLE>(al, lane, Fz, epi, orow, z, Kw, N);
+    rowlane_body<W, KC, NT, SINGLE, EXACT>(al, lane, Fz, epi, orow, z, Kw, N);
 }
 
 template <typename W, bool POOLMAP, class Epi>
@@ -95,14 +95,18 @@ static void dispatch_conv(const ConvA<W> &al, const W *filt, const Epi &epi, int
     const int Kw = al.g.fx * al.g.fy * al.g.Cw;
     const int pblocks = (int)ceil_div(lanes_per_member, 256);
     const dim3 grid((unsigned)(D * pblocks)), block(256);
-    if (Kw <= 4)
-        conv_rowlane_kernel<W, 4, 16, true, POOLMAP, Epi><<<grid, block, 0, s>>>(al, filt, epi, pblocks, N);
+    if (Kw == 9)
+        conv_rowlane_kernel<W, 9, 16, true, true, POOLMAP, Epi><<<grid, block, 0, s>>>(al, filt, epi, pblocks, N);
+    else if (Kw == 18)
+        conv_rowlane_kernel<W, 18, 16, true, true, POOLMAP, Epi><<<grid, block, 0, s>>>(al, filt, epi, pblocks, N);
+    else if (Kw <= 4)
+        conv_rowlane_kernel<W, 4, 16, true, false, POOLMAP, Epi><<<grid, block, 0, s>>>(al, filt, epi, pblocks, N);
     else if (Kw <= 9)
-        conv_rowlane_kernel<W, 9, 16, true, POOLMAP, Epi><<<grid, block, 0, s>>>(al, filt, epi, pblocks, N);
+        conv_rowlane_kernel<W, 9, 16, true, false, POOLMAP, Epi><<<grid, block, 0, s>>>(al, filt, epi, pblocks, N);
     else if (Kw <= 18)
-        conv_rowlane_kernel<W, 18, 16, true, POOLMAP, Epi><<<grid, block, 0, s>>>(al, filt, epi, pblocks, N);
+        conv_rowlane_kernel<W, 18, 16, true, false, POOLMAP, Epi><<<grid, block, 0, s>>>(al, filt, epi, pblocks, N);
     else
-        conv_rowlane_kernel<W, 16, 16, false, POOLMAP, Epi><<<grid, block, 0, s>>>(al, filt, epi, pblocks, N);
+        conv_rowlane_kernel<W, 16, 16, false, false, POOLMAP, Epi><<<grid, block, 0, s>>>(al, filt, epi, pblocks, N);
 }
 
 static int geom_check(ConvGeom *g, int64_t D, int64_t H, int64_t Wd, int64_t Cw, int fx, int fy, int px, int py,

@@ -89,53 +89,92 @@ struct ConvA {
 };
 
 // ---- accumulate one K-chunk into an N-tile ----------------------------------------------------
-template <typename W, int KC, int NT>
+// EXACT: the chunk is complete (k0 + KC <= Kw), so the k-steps carry no guards and the scalar loads of
+// later steps can be issued while earlier steps compute.
+template <typename W, int KC, int NT, bool EXACT>
 __device__ __forceinline__ void mac_chunk(int (&acc)[NT], const W (&a)[KC], const W *__restrict__ Bz, int k0, int Kw,
                                           int n0, int N)
 {
-    if (n0 + NT <= N) {
+    if (EXACT && n0 + NT <= N) {
+        // software pipeline over k: the scalar loads of step i+1 are issued before step i computes
+        const W *__restrict__ brow = Bz + (int64_t)k0 * N + n0;
+        W bcur[NT], bnxt[NT];
+#pragma unroll
+        for (int j = 0; j < NT; j++) bcur[j] = brow[j];
 #pragma unroll
         for (int i = 0; i < KC; i++) {
-            if (k0 + i < Kw) {
+            if (i + 1 < KC) {
+#pragma unroll
+                for (int j = 0; j < NT; j++) bnxt[j] = brow[(int64_t)(i + 1) * N + j];
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int j = 0; j < NT; j++) acc_popc_xor(acc[j], a[i], bcur[j]);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int j = 0; j < NT; j++) bcur[j] = bnxt[j];
+        }
+    } else if (n0 + NT <= N) {
+#pragma unroll
+        for (int i = 0; i < KC; i++) {
+            if (EXACT || k0 + i < Kw) {
                 const W *__restrict__ brow = Bz + (int64_t)(k0 + i) * N + n0;
 #pragma unroll
-                for (int j = 0; j < NT; j++) acc[j] += popc_xor(a[i], brow[j]);
+                for (int j = 0; j < NT; j++) acc_popc_xor(acc[j], a[i], brow[j]);
             }
         }
     } else {
 #pragma unroll
         for (int i = 0; i < KC; i++) {
-            if (k0 + i < Kw) {
+            if (EXACT || k0 + i < Kw) {
                 const W *__restrict__ brow = Bz + (int64_t)(k0 + i) * N + n0;
 #pragma unroll
                 for (int j = 0; j < NT; j++)
-                    if (n0 + j < N) acc[j] += popc_xor(a[i], brow[j]);
+                    if (n0 + j < N) acc_popc_xor(acc[j], a[i], brow[j]);
             }
         }
     }
 }
 
 // ---- epilogues -----------------------------------------------------------------------------------
-// int32 popcount sums, C [Z, M, N].
+// int32 popcount sums, C [Z, M, N].  A full N-tile is transposed through LDS so that every store
+// instruction of a wave writes whole 64-byte row segments (4 lanes x int4 per row), and the stores are
+// non-temporal: the output is written once and never re-read by this kernel.  The lanes of a wave own
+// consecutive rows (row - lane is the wave's first row).
+typedef int nb_i32x4 __attribute__((ext_vector_type(4)));
 struct EpiI32 {
     int32_t *__restrict__ C;
-    bool vec;  // rows are 16-byte aligned and N % 4 == 0: store int4
+    bool vec;  // rows are 16-byte aligned and N % 4 == 0
     struct State {};
     template <int NT>
     __device__ __forceinline__ void tile(State &, int64_t row, bool valid, int64_t z, int n0, int N,
                                          const int (&acc)[NT]) const
     {
+        static_assert(NT == 16, "the transposed store assumes 16-wide tiles");
+        const int wv = threadIdx.x >> 6, lane = threadIdx.x & 63;
+        const bool full = __all(valid);
+        if (n0 + NT <= N && vec && full) {
+            __shared__ int stage[4][64][NT + 1];  // +1: conflict-free column writes
+#pragma unroll
+            for (int j = 0; j < NT; j++) stage[wv][lane][j] = acc[j];
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            const int64_t row0 = row - lane;
+#pragma unroll
+            for (int p = 0; p < 4; p++) {
+                const int r = p * 16 + (lane >> 2), c = (lane & 3) * 4;
+                const nb_i32x4 v = {stage[wv][r][c], stage[wv][r][c + 1], stage[wv][r][c + 2], stage[wv][r][c + 3]};
+                __builtin_nontemporal_store(v, reinterpret_cast<nb_i32x4 *>(C + (row0 + r) * N + n0 + c));
+            }
+            __builtin_amdgcn_wave_barrier();
+            return;
+        }
         if (!valid) return;
         int32_t *dst = C + row * N + n0;
-        if (n0 + NT <= N && vec) {
 #pragma unroll
-            for (int j = 0; j < NT; j += 4)
-                *reinterpret_cast<int4 *>(dst + j) = make_int4(acc[j], acc[j + 1], acc[j + 2], acc[j + 3]);
-        } else {
-#pragma unroll
-            for (int j = 0; j < NT; j++)
-                if (n0 + j < N) dst[j] = acc[j];
-        }
+        for (int j = 0; j < NT; j++)
+            if (n0 + j < N) dst[j] = acc[j];
     }
     __device__ __forceinline__ void finish(State &, int64_t, bool) const {}
 };
@@ -206,7 +245,8 @@ struct EpiPack {
 };
 
 // The loop nest shared by every row-per-lane kernel.
-template <typename W, int KC, int NT, bool SINGLE, class ALoad, class Epi>
+// SINGLE: Kw <= KC (one chunk, A words stay in registers for every N-tile); EXACT: Kw == KC.
+template <typename W, int KC, int NT, bool SINGLE, bool EXACT, class ALoad, class Epi>
 __device__ __forceinline__ void rowlane_body(const ALoad &al, const typename ALoad::Lane &lane,
                                              const W *__restrict__ Bz, const Epi &epi, int64_t orow, int64_t z,
                                              int Kw, int N)
@@ -219,11 +259,16 @@ __device__ __forceinline__ void rowlane_body(const ALoad &al, const typename ALo
 #pragma unroll
         for (int j = 0; j < NT; j++) acc[j] = 0;
         if (SINGLE) {
-            mac_chunk<W, KC, NT>(acc, a, Bz, 0, Kw, n0, N);
+            mac_chunk<W, KC, NT, EXACT>(acc, a, Bz, 0, Kw, n0, N);
         } else {
-            for (int k0 = 0; k0 < Kw; k0 += KC) {
+            int k0 = 0;
+            for (; k0 + KC <= Kw; k0 += KC) {
                 al.template load<KC>(lane, k0, a);
-                mac_chunk<W, KC, NT>(acc, a, Bz, k0, Kw, n0, N);
+                mac_chunk<W, KC, NT, true>(acc, a, Bz, k0, Kw, n0, N);
+            }
+            if (k0 < Kw) {
+                al.template load<KC>(lane, k0, a);
+                mac_chunk<W, KC, NT, false>(acc, a, Bz, k0, Kw, n0, N);
             }
         }
         epi.template tile<NT>(st, orow, lane.valid, z, n0, N, acc);
