@@ -72,8 +72,9 @@ class Binarized(Perturbed, nn.Module):
 
     def probabilities(self):
         """fp16 [rows, in_degree] per-bit probabilities of a 1 (modules/binary.py:59-60)."""
-        norm_weight = self.weight / (self.weight.abs().mean() + 1e-5) * 5
-        return torch.sigmoid(norm_weight.float()).half()
+        with torch.no_grad():
+            norm_weight = self.weight / (self.weight.abs().mean() + 1e-5) * 5
+            return torch.sigmoid(norm_weight.float()).half()
 
     def set_noise(self, noise_scale=None, words=None):
         """modules/binary.py:54-64.  ``words`` (uint32 [directions, rows, in_degree]) replaces the

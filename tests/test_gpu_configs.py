@@ -1,0 +1,141 @@
+"""The five benchmark configurations at their FULL sizes on the GPU.
+
+Each is checked two ways: (1) a size-independent identity over the whole population computed by a second,
+independent GPU path (fused == materialise-then-bmm, implicit conv == bmm(im2col), fused epilogue == op
+chain), and (2) bit-exact agreement with the CPU oracle on a few members, whose random words are regenerated
+on the host from the same Philox stream (oracle/nesbin_oracle.c: nbo_philox_words)."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+MEMBERS = (0, 1, 511, 1023)
+
+
+@pytest.fixture(scope="module")
+def wk():
+    assert torch.cuda.is_available()
+    from nesgpu_amd import workloads
+    return workloads
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from nesgpu_amd.extensions import booleanOperations
+    return booleanOperations
+
+
+def host_member_weights(oracle, base, in_bits, rows, T, seed, subseq, m):
+    """base ^ flips of member m, regenerated on the host."""
+    words = oracle.philox_words(seed, subseq, m * rows * in_bits, rows * in_bits).reshape(1, rows, in_bits)
+    return oracle.sample_from_words(T, words, np.int64, base=base)[0]
+
+
+def test_config1_linear_256_materialised(wk, ops, oracle):
+    w = wk.linear_flip_materialised()
+    out = w.step()
+    assert tuple(out.shape) == (1024, 256, 1) and out.dtype == torch.int32
+    base, x, W = (w.tensors[k].cpu().numpy() for k in ("base", "x", "W"))
+    # whole population against the oracle (small enough)
+    words = oracle.philox_words(0, 1, 0, 1024 * 256 * 256).reshape(1024, 256, 256)
+    Wn = oracle.sample_from_words(wk.T_P01, words, np.int64, base=base)
+    np.testing.assert_array_equal(W, Wn)
+    popc = oracle.bmm(Wn, x.reshape(1024, 4, 1))
+    np.testing.assert_array_equal(out.cpu().numpy(), popc)
+    flips = oracle.unpack((Wn ^ base[None]).reshape(-1, 4)).mean()
+    assert abs(flips - 0.01) < 2e-4                                         # Bernoulli(p = 0.01)
+    # the configuration's stated output K - 2*popcount(x XOR w) is the XNOR reading of the same sum
+    xb = oracle.unpack(x)[:, :256]
+    wb = oracle.unpack(Wn[7])[:, :256]
+    dot = ((2 * xb[7].astype(int) - 1) * (2 * wb.astype(int) - 1)).sum(1)
+    np.testing.assert_array_equal(256 - 2 * popc[7, :, 0], dot)
+
+
+def test_config2_linear_1024_fused_from_words(wk, ops, oracle):
+    w = wk.linear_flip_fused()
+    out = w.step()
+    assert tuple(out.shape) == (1024, 1024) and out.dtype == torch.int32
+    base, x, words = w.tensors["base"], w.tensors["x"], w.tensors["words"]
+    # identity over the whole population: fused == materialise + bmm (two different kernels)
+    ref = torch.empty_like(out)
+    for lo in range(0, 1024, 256):
+        Wm = ops.flip_from_words(base, words[lo:lo + 256], wk.T_P05)
+        ref[lo:lo + 256] = ops.bmm(Wm, x[lo:lo + 256].view(256, -1, 1)).squeeze(2)
+    assert torch.equal(out, ref)
+    # generator mode reproduces the same numbers without reading any words
+    assert torch.equal(ops.seeded_bmv_philox(wk.T_P05, x, 1024, 1024, 0, subsequence=2, base=base), out)
+    # oracle on a few members
+    bh, xh = base.cpu().numpy(), x.cpu().numpy()
+    for m in MEMBERS:
+        wm = oracle.philox_words(0, 2, m * 1024 * 1024, 1024 * 1024).reshape(1, 1024, 1024)
+        want = oracle.seeded_bmv_from_words(wk.T_P05, xh[m:m + 1], wm, base=bh)
+        np.testing.assert_array_equal(out[m].cpu().numpy(), want[0])
+    rate = (ops.unpack((ops.flip_from_words(base, words[:8], wk.T_P05) ^ base).view(-1, 16)).float().mean().item())
+    assert abs(rate - 0.05) < 5e-4
+
+
+def test_config3_conv_64_int32(wk, ops, oracle):
+    w = wk.conv_int32()
+    out = w.step()
+    assert tuple(out.shape) == (1024, 32, 32, 64) and out.dtype == torch.int32
+    x, filt, base = w.tensors["x"], w.tensors["filt"], w.tensors["base"]
+    for lo in range(0, 1024, 256):                                          # implicit conv == bmm(im2col)
+        cols = ops.batch_im2col(x[lo:lo + 256], 3, 3, 1, 1, 1, 1)
+        assert torch.equal(ops.bmm(cols, filt[lo:lo + 256]).view(256, 32, 32, 64), out[lo:lo + 256])
+    bh = base.cpu().numpy()
+    for m in MEMBERS:
+        Wn = host_member_weights(oracle, bh, 64, 576, wk.T_P02, 0, 3, m)                 # [576, 1]
+        f = np.ascontiguousarray(Wn.reshape(1, 64, 3, 3, 1).transpose(0, 2, 3, 4, 1).reshape(1, 9, 64))
+        np.testing.assert_array_equal(filt[m].cpu().numpy(), f[0])
+        want = oracle.conv(x[m:m + 1].cpu().numpy(), f, 3, 3, 1, 1, 1, 1)
+        np.testing.assert_array_equal(out[m].cpu().numpy(), want[0])
+    # padding is the zero word = every padded bit -1: a corner pixel only sees 4 real taps
+    xm, fm = x[0].cpu().numpy().view(np.uint64), filt[0].cpu().numpy().view(np.uint64)
+    taps = [(1, 1, 0, 0), (1, 2, 0, 1), (2, 1, 1, 0), (2, 2, 1, 1)]                     # (i, j, y, x)
+    for o in (0, 63):
+        s = sum(bin(int(xm[y, xx, 0] ^ fm[i * 3 + j, o])).count("1") for i, j, y, xx in taps)
+        s += sum(bin(int(fm[i * 3 + j, o])).count("1") for i in range(3) for j in range(3)
+                 if (i, j) not in [(t[0], t[1]) for t in taps])
+        assert int(out[0, 0, 0, o]) == s
+
+
+def test_config4_conv_16_sign_pool(wk, ops, oracle):
+    w = wk.conv_sign_pool()
+    out = w.step()
+    assert tuple(out.shape) == (1024, 32, 32, 1) and out.dtype == torch.int64
+    x, filt, thr = w.tensors["x"], w.tensors["filt"], w.tensors["thr"]
+    for lo in range(0, 1024, 256):                                          # fused == conv_act -> pack -> max_pool2d
+        act = ops.conv_act(x[lo:lo + 256], filt[lo:lo + 256], thr[lo:lo + 256], 3, 3, 1, 1, 1, 1)
+        sign = 2 * ops.conv(x[lo:lo + 256], filt[lo:lo + 256], 3, 3, 1, 1, 1, 1) - 144 > 0
+        assert torch.equal(act, sign)                                       # threshold K <=> sign of 2*popc - K
+        packed = ops.pack(act.view(-1, 16), torch.int64).view(256, 64, 64, 1)
+        assert torch.equal(ops.max_pool2d(packed, 2, 2, 0, 0, 2, 2), out[lo:lo + 256])
+    assert int((out >> 16).abs().max()) == 0                               # only 16 channel bits per word
+    for m in MEMBERS:
+        xm, fm = x[m:m + 1].cpu().numpy(), filt[m:m + 1].cpu().numpy()
+        act = oracle.conv_act(xm, fm, np.full((1, 16), 144, np.int32), 3, 3, 1, 1, 1, 1)
+        want = oracle.max_pool2d(oracle.pack(act.reshape(-1, 16), np.int64).reshape(1, 64, 64, 1), 2, 2, 0, 0, 2, 2)
+        np.testing.assert_array_equal(out[m].cpu().numpy(), want[0])
+
+
+def test_config5_cifar_net(wk, ops, oracle):
+    D = 4096
+    w = wk.cifar_net(D=D)
+    out = w.step()
+    assert tuple(out.shape) == (D, 10) and out.dtype == torch.int32
+    assert torch.equal(w.step(), out)                                      # deterministic
+    t = w.tensors
+    for m in (0, 2047, 4095):
+        a = t["x"][m:m + 1].cpu().numpy()                                  # [1,32,32,1]
+        for name, C, O, pool in (("f1", 3, 64, False), ("f2", 64, 64, True), ("f3", 64, 128, True)):
+            f = t[name][m:m + 1].cpu().numpy()
+            act = oracle.conv_act(a, f, np.full((1, O), 9 * C, np.int32), 3, 3, 1, 1, 1, 1)
+            a = oracle.pack(act.reshape(-1, O), np.int64).reshape(1, act.shape[1], act.shape[2], -1)
+            if pool:
+                a = oracle.max_pool2d(a, 2, 2, 0, 0, 2, 2)
+        a = a.reshape(1, 128, 1)
+        p4 = oracle.bmm(t["W4"][m:m + 1].cpu().numpy(), a)[:, :, 0]        # [1,1024]
+        a5 = oracle.pack(2 * p4 > 8192, np.int64).reshape(1, 16, 1)
+        want = oracle.bmm(t["W5"][m:m + 1].cpu().numpy(), a5)[:, :, 0]
+        np.testing.assert_array_equal(out[m].cpu().numpy(), want[0])

@@ -1,0 +1,207 @@
+"""GPU tests of the layer API (nesgpu_amd.modules.binary) against the CPU oracle: the layers are driven with
+caller-supplied random words so that every sampled weight bit is reproducible on the host."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def binary():
+    assert torch.cuda.is_available()
+    from nesgpu_amd.modules import binary as b
+    return b
+
+
+def rng(seed):
+    return np.random.default_rng(seed)
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def host_thresholds(layer):
+    """uint32 thresholds the layer samples with, recomputed on the host from the fp16 probabilities
+    (T = min(floor(P * 2**32), 2**32 - 1))."""
+    P = layer.probabilities().cpu().numpy().astype(np.float64)
+    return np.minimum(np.floor(P * 4294967296.0), 4294967295.0).astype(np.uint32)
+
+
+def randomise(layer, g):
+    with torch.no_grad():
+        layer.weight.copy_(dev(g.standard_normal(tuple(layer.weight.shape)).astype(np.float16)))
+        if layer.bias is not None:
+            layer.bias.copy_(dev((g.standard_normal(tuple(layer.bias.shape)) * 4).astype(np.float16)))
+
+
+@pytest.mark.parametrize("dtype", [torch.int64, torch.int32])
+@pytest.mark.parametrize("in_f,out_f", [(256, 64), (100, 10), (1024, 33)])
+def test_linear_forward(binary, oracle, dtype, in_f, out_f):
+    D = 16
+    g = rng(in_f + out_f)
+    nd = np.int64 if dtype == torch.int64 else np.int32
+    for threshold, batch_norm in [(False, False), (True, False), (True, True)]:
+        layer = binary.BinarizedLinear(in_f, out_f, D, threshold=threshold, batch_norm=batch_norm, dtype=dtype)
+        randomise(layer, g)
+        words = g.integers(0, 2 ** 32, size=(D, out_f, in_f), dtype=np.uint64).astype(np.uint32)
+        layer.set_seed(11)
+        layer.set_noise(words=dev(words))
+        T = host_thresholds(layer)
+        Wn = oracle.sample_from_words(T, words, nd)
+        np.testing.assert_array_equal(layer.weight_noise.cpu().numpy(), Wn)           # modules/binary.py:62
+        xb = g.integers(0, 2, size=(D, in_f)).astype(bool)
+        layer.perturbed_flag = True
+        out = layer(dev(xb))
+        popc = oracle.bmm(Wn, oracle.pack(xb, nd).reshape(D, -1, 1))[:, :, 0]
+        act = 2 * popc - in_f                                                          # modules/binary.py:97
+        # same +-1 reading as the reference's check: x = 2b-1, w = 1-2b
+        want_dot = ((2 * xb.astype(np.int64) - 1)[:, None, :] *
+                    (1 - 2 * oracle.unpack(Wn.reshape(D * out_f, -1))[:, :in_f].reshape(D, out_f, in_f).astype(np.int64))
+                    ).sum(2)
+        np.testing.assert_array_equal(act, want_dot)
+        if not threshold:
+            assert out.dtype == torch.int32
+            np.testing.assert_array_equal(out.cpu().numpy(), act)
+            continue
+        assert out.dtype == torch.bool and tuple(out.shape) == (D, out_f)
+        assert tuple(layer.bias_noise.shape) == (D, out_f) and layer.bias_noise.dtype == torch.float16
+        assert float(layer.bias_noise.abs().max()) <= 3.0                              # (rand - .5) * 6
+        act_t = torch.from_numpy(act.astype(np.int32)).cuda()
+        thresh = layer.bias + layer.bias_noise
+        if batch_norm:
+            thresh = thresh + act_t.type(torch.float16).mean(dim=0, keepdim=True)      # modules/binary.py:101
+        assert torch.equal(out, act_t > thresh)
+        # packed input is accepted as is (modules/binary.py:95)
+        assert torch.equal(layer(dev(oracle.pack(xb, nd))), out)
+
+
+@pytest.mark.parametrize("dtype", [torch.int64, torch.int32])
+@pytest.mark.parametrize("C,O,k,pad,stride", [(16, 16, 3, 1, 1), (64, 70, 3, 1, 1), (3, 8, 5, 2, 2), (100, 4, 1, 0, 1)])
+def test_conv_forward(binary, oracle, dtype, C, O, k, pad, stride):
+    D, S = 6, 12
+    g = rng(C * 3 + O + k)
+    nd = np.int64 if dtype == torch.int64 else np.int32
+    K = C * k * k
+    xb = g.integers(0, 2, size=(D, S, S, C)).astype(bool)
+    xp = oracle.pack(xb.reshape(-1, C), nd).reshape(D, S, S, -1)
+    geom = (k, k, pad, pad, stride, stride)
+    for threshold, batch_norm in [(False, False), (True, False), (True, True)]:
+        layer = binary.BinarizedConv2d(C, O, D, k, stride=stride, padding=pad, threshold=threshold,
+                                       batch_norm=batch_norm, dtype=dtype)
+        randomise(layer, g)
+        words = g.integers(0, 2 ** 32, size=(D, O * k * k, C), dtype=np.uint64).astype(np.uint32)
+        layer.set_seed(5)
+        layer.set_noise(words=dev(words))
+        Wn = oracle.sample_from_words(host_thresholds(layer), words, nd)             # [D, O*k*k, Cw]
+        filt = np.ascontiguousarray(Wn.reshape(D, O, k, k, -1).transpose(0, 2, 3, 4, 1).reshape(D, -1, O))
+        np.testing.assert_array_equal(layer.weight_noise_reshaped.cpu().numpy(), filt)   # modules/binary.py:136-137
+        popc = oracle.conv(xp, filt, *geom)
+        act = 2 * popc - K                                                              # modules/binary.py:145,158
+        layer.perturbed_flag = True
+        out = layer(dev(xb))
+        if not threshold:
+            np.testing.assert_array_equal(out.cpu().numpy(), act)
+            continue
+        assert out.dtype == torch.bool and tuple(out.shape) == act.shape
+        if batch_norm:
+            act_t = torch.from_numpy(act.astype(np.int32)).cuda()
+            thresh = layer.bias + layer.bias_noise + act_t.type(torch.float16).mean(dim=[1, 2])   # :151
+            assert torch.equal(out, act_t > thresh.unsqueeze(1).unsqueeze(1))
+        else:
+            thr = (layer.bias + layer.bias_noise).type(torch.int32).cpu().numpy() + K          # :156
+            np.testing.assert_array_equal(out.cpu().numpy(), oracle.conv_act(xp, filt, thr, *geom))
+            assert torch.equal(layer(dev(xp)), out)                                            # packed input
+            # fused packed / pooled outputs of the same layer
+            layer.pack_output = True
+            packed = layer(dev(xp))
+            want = oracle.pack(out.cpu().numpy().reshape(-1, O), nd).reshape(*out.shape[:3], -1)
+            np.testing.assert_array_equal(packed.cpu().numpy(), want)
+            if out.shape[1] >= 2:
+                layer.pool_output = True
+                np.testing.assert_array_equal(layer(dev(xp)).cpu().numpy(), oracle.max_pool2d(want, 2, 2, 0, 0, 2, 2))
+                pool = binary.BinarizedMaxPool2d(dtype=dtype)
+                assert torch.equal(pool(out), layer(dev(xp)))                                   # bool input gets packed
+
+
+def test_maxpool_module(binary, oracle):
+    g = rng(9)
+    xb = g.integers(0, 2, size=(4, 10, 10, 70)).astype(bool)
+    pool = binary.BinarizedMaxPool2d()
+    want = oracle.max_pool2d(oracle.pack(xb.reshape(-1, 70), np.int64).reshape(4, 10, 10, 2), 2, 2, 0, 0, 2, 2)
+    np.testing.assert_array_equal(pool(dev(xb)).cpu().numpy(), want)
+    np.testing.assert_array_equal(pool(dev(oracle.pack(xb.reshape(-1, 70), np.int64).reshape(4, 10, 10, 2))).cpu().numpy(),
+                                  want)
+
+
+def test_perturbed_model_step(binary):
+    """set_seed -> set_noise -> forward -> update on a small conv/pool/linear stack through PerturbedModel
+    (the NES step of cifar10test.py:150-179 restricted to the binary layers)."""
+    D = 32
+    model = torch.nn.Sequential(
+        binary.BinarizedConv2d(16, 64, D, 3, padding=1, batch_norm=True),
+        binary.BinarizedMaxPool2d(),
+        binary.BinarizedConv2d(64, 64, D, 3, padding=1, batch_norm=False),
+        binary.BinarizedMaxPool2d(),
+        torch.nn.Flatten(),
+        binary.BinarizedLinear(64 * 2 * 2, 10, D, threshold=False),
+    )
+    pm = binary.PerturbedModel(model, D)
+    assert len(pm.perturbed_layers) == 3
+    g = rng(0)
+    for layer in pm.perturbed_layers:
+        randomise(layer, g)
+    pm.set_seed(123)
+    pm.set_noise()
+    x = dev(g.integers(0, 2, size=(D, 8, 8, 16)).astype(bool))
+    out = pm.forward(x)
+    assert tuple(out.shape) == (D, 10) and out.dtype == torch.int32
+    assert all(not l.perturbed_flag for l in pm.perturbed_layers)
+    assert int(out.abs().max()) <= 256 and (out % 2 == 0).all()               # 2*popc - K with K even
+    # same seed -> same noise -> same output; another seed -> different weights
+    w0 = [l.weight_noise.clone() for l in pm.perturbed_layers]
+    pm.set_noise()
+    assert all(torch.equal(a, l.weight_noise) for a, l in zip(w0, pm.perturbed_layers))
+    assert torch.equal(pm.forward(x), out)
+    pm.set_seed(124)
+    pm.set_noise()
+    assert not torch.equal(w0[0], pm.perturbed_layers[0].weight_noise)
+    # update: gradients with the parameter shapes (modules/binary.py:67-77)
+    fitness = dev(g.standard_normal(D).astype(np.float32))
+    pm.update(fitness)
+    for l in pm.perturbed_layers:
+        assert l.weight.grad.shape == l.weight.shape and l.weight.grad.dtype == torch.float16
+        assert torch.isfinite(l.weight.grad.float()).all()
+        if l.threshold:
+            assert l.bias.grad.shape == l.bias.shape
+    # the weight gradient is the fitness-weighted sum of the sampled bits
+    lin = pm.perturbed_layers[2]
+    from nesgpu_amd.extensions import booleanOperations as ops
+    bits = ops.unpack(lin.weight_noise.view(-1, lin.weight_noise.size(2)))[:, :lin.in_features].view(D, 10, -1)
+    f16 = fitness.type(torch.float16)
+    f16 = f16 - f16.mean()
+    want = torch.einsum("d,doi->oi", f16.float(), bits.float()) + 1e-3 * lin.weight.float()
+    assert torch.allclose(lin.weight.grad.float(), want, rtol=1e-2, atol=2e-2)     # tolerance of booloptests.py:284
+    pm.free_memory()
+    assert all(l.weight_noise is None for l in pm.perturbed_layers)
+
+
+def test_reference_import_names_resolve(binary):
+    import sys
+    import nesgpu_amd
+    saved = {k: sys.modules.get(k) for k in ("extensions", "extensions.booleanOperations", "modules", "modules.binary")}
+    try:
+        for k in saved:
+            sys.modules.pop(k, None)
+        nesgpu_amd.install_as_reference_modules()
+        from extensions import booleanOperations as ref_ops       # the reference's import lines
+        from modules import binary as ref_binary
+        assert ref_ops.bmm is nesgpu_amd.extensions.booleanOperations.bmm
+        assert ref_binary.BinarizedLinear is binary.BinarizedLinear
+    finally:
+        for k, v in saved.items():
+            if v is None:
+                sys.modules.pop(k, None)
+            else:
+                sys.modules[k] = v
