@@ -43,6 +43,8 @@ def parse_args():
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU time the baseline leg accumulates")
     ap.add_argument("--only-calib", action="store_true", help="run only the calibration kernels (for counter runs)")
     ap.add_argument("--only", type=int, default=0, help="time just this configuration (for profiler runs)")
+    ap.add_argument("--kernels", action="store_true",
+                    help="time the HBM-bound helper kernels (pack, unpack, samplers, max-pool, im2col) on their own")
     return ap.parse_args()
 
 
@@ -125,6 +127,52 @@ def calibrate(torch):
     return res
 
 
+def hbm_kernels(torch, steps, warmup):
+    """Each HBM-bound kernel of the path alone, at a configuration-sized shape: algorithmic bytes / event time."""
+    from nesgpu_amd import workloads
+    from nesgpu_amd.extensions import booleanOperations as ops
+    dev = "cuda"
+    res = []
+
+    def run(name, fn, nbytes):
+        pw, pe = time_steps(torch, fn, steps, warmup)
+        res.append({"kernel": name, "us": round(pe * 1e6, 2), "GBps": round(nbytes / pe / 1e9, 1),
+                    "hbm_frac": round(nbytes / pe / workloads.HBM_PEAK, 4), "algorithmic_bytes": nbytes})
+
+    g = torch.Generator(device=dev)
+    g.manual_seed(0)
+    # pack: config 3 activations [1024*32*32, 64] bool -> 1 word per pixel; and a wide row case
+    b = torch.randint(0, 2, (1024 * 32 * 32, 64), device=dev, generator=g, dtype=torch.uint8).bool()
+    run("pack [1048576,64] -> i64", lambda: ops.pack(b, torch.int64), b.numel() + b.numel() // 8)
+    b2 = torch.randint(0, 2, (65536, 1024), device=dev, generator=g, dtype=torch.uint8).bool()
+    run("pack [65536,1024] -> i64", lambda: ops.pack(b2, torch.int64), b2.numel() + b2.numel() // 8)
+    b3 = torch.randint(0, 2, (1024 * 64 * 64, 16), device=dev, generator=g, dtype=torch.uint8).bool()
+    run("pack [4194304,16] -> i64", lambda: ops.pack(b3, torch.int64), b3.numel() + b3.size(0) * 8)
+    p2 = ops.pack(b2, torch.int64)
+    run("unpack [65536,16] i64", lambda: ops.unpack(p2), p2.numel() * 8 + p2.numel() * 64)
+    del b, b2, b3
+    # samplers from supplied words: config 1 (linear 256x256, D=1024) and config 3 filters (576 x 64, D=1024)
+    for (n, R, C, T) in ((1024, 256, 256, workloads.T_P01), (1024, 576, 64, workloads.T_P02), (256, 1024, 1024, workloads.T_P05)):
+        words = ops.philox_words(n * R * C, 0, 7).view(n, R, C)
+        base = ops.pack(torch.randint(0, 2, (R, C), device=dev, generator=g, dtype=torch.uint8).bool(), torch.int64)
+        nb = words.numel() * 4 + n * R * ((C + 63) // 64) * 8
+        run("flip_from_words [%d,%d,%d]" % (n, R, C), lambda: ops.flip_from_words(base, words, T), nb)
+        thr = ops.thresholds_from_p(torch.rand(R, C, device=dev, generator=g).half())
+        run("sample_bits_from_words [%d,%d,%d]" % (n, R, C), lambda: ops.sample_bits_from_words(thr, words, torch.int64), nb)
+        del words
+    # max-pool 2x2/s2 on config 4's thresholded map [1024,64,64,1] and on a 2-word map
+    for shape in ((1024, 64, 64, 1), (4096, 16, 16, 2), (1024, 64, 64, 4)):
+        x = torch.randint(-2 ** 62, 2 ** 62, shape, device=dev, generator=g, dtype=torch.int64)
+        run("max_pool2d %s" % (list(shape),), lambda: ops.max_pool2d(x, 2, 2, 0, 0, 2, 2), x.numel() * 8 * 5 // 4)
+    x = torch.randint(-2 ** 62, 2 ** 62, (1024, 32, 32, 1), device=dev, generator=g, dtype=torch.int64)
+    run("batch_im2col [1024,32,32,1] 3x3 p1", lambda: ops.batch_im2col(x, 3, 3, 1, 1, 1, 1), x.numel() * 8 * 10)
+    # linear matrix-vector product streaming materialised weights (config 5's 8192 -> 1024 layer at D=1024)
+    W = torch.randint(-2 ** 62, 2 ** 62, (1024, 1024, 128), device=dev, generator=g, dtype=torch.int64)
+    xv = torch.randint(-2 ** 62, 2 ** 62, (1024, 128, 1), device=dev, generator=g, dtype=torch.int64)
+    run("bmm N=1 [1024,1024,128]", lambda: ops.bmm(W, xv), W.numel() * 8 + xv.numel() * 8 + 1024 * 1024 * 4)
+    return res
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -142,6 +190,9 @@ def main():
         print(json.dumps({"measured_ceilings": calibrate(torch)}))
         return 0
 
+    if args.kernels:
+        print(json.dumps({"hbm_kernels": hbm_kernels(torch, args.steps, args.warmup)}))
+        return 0
     if args.only:
         w = workloads.BUILDERS[args.only]()
         pw, pe = time_steps(torch, w.step, args.steps, args.warmup)

@@ -54,6 +54,30 @@ __device__ __forceinline__ uint4 load_stream16(const void *p)
 }
 __device__ __forceinline__ uint32_t load_stream4(const uint32_t *p) { return __builtin_nontemporal_load(p); }
 
+// OR-reduction over aligned groups of G lanes (G = 4, 8 or 16) with DPP lane permutes instead of
+// LDS-crossbar shuffles: xor-1 and xor-2 inside a quad, then the mirrored half-row and row.
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_mov(uint32_t v)
+{
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xF, 0xF, true);
+}
+template <int G>
+__device__ __forceinline__ uint32_t or_reduce_group(uint32_t v)
+{
+    static_assert(G == 4 || G == 8 || G == 16, "group must be 4, 8 or 16 lanes");
+    v |= dpp_mov<0xB1>(v);               // quad_perm [1,0,3,2]
+    v |= dpp_mov<0x4E>(v);               // quad_perm [2,3,0,1]
+    if (G >= 8) v |= dpp_mov<0x141>(v);  // row_half_mirror: lane i <-> 7-i within 8
+    if (G >= 16) v |= dpp_mov<0x140>(v); // row_mirror: lane i <-> 15-i within 16
+    return v;
+}
+template <int G>
+__device__ __forceinline__ uint64_t or_reduce_group(uint64_t v)
+{
+    const uint32_t lo = or_reduce_group<G>((uint32_t)v), hi = or_reduce_group<G>((uint32_t)(v >> 32));
+    return ((uint64_t)hi << 32) | lo;
+}
+
 // Philox4x32-10 (Salmon et al., SC'11): counter-based generator used when the caller does not
 // supply the random words.
 __device__ __forceinline__ uint4 philox4x32_10(uint4 c, uint2 k)

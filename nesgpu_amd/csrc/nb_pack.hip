@@ -45,6 +45,38 @@ __global__ __launch_bounds__(256) void pack_vec16_kernel(W *__restrict__ out, co
     }
 }
 
+// 64-bit words, C % 64 == 0, 16-byte aligned input: a wave converts 4 KiB of bools (64 words) per step.
+// Load i (0..3) takes the 1 KiB slice i with lanes at consecutive 16-byte chunks (fully coalesced); the four
+// lanes of a quad then hold the four 16-bit quarters of word i*16 + lane/4 and OR them together, and lane
+// 4q+i stores word i*16+q, so one store instruction writes the 64 finished words.
+__global__ __launch_bounds__(256) void pack_quad_kernel(uint64_t *__restrict__ out, const uint8_t *__restrict__ in,
+                                                        int64_t total_words)
+{
+    const int lane = threadIdx.x & 63;
+    const int64_t nwaves = (int64_t)gridDim.x * 4;
+    for (int64_t w0 = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * 64; w0 < total_words; w0 += nwaves * 64) {
+        const uint8_t *src = in + w0 * 64;
+        const int64_t left = total_words - w0;  // words left from w0 (>= 1)
+        uint4 v[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            int64_t word = i * 16 + (lane >> 2);
+            if (word >= left) word = left - 1;  // clamp: tail lanes re-read a valid word and do not store
+            v[i] = load_stream16(src + word * 64 + (lane & 3) * 16);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        uint64_t mine = 0;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            uint64_t q = (uint64_t)bits16_of_bools(v[i]) << (16 * (lane & 3));
+            q = or_reduce_group<4>(q);
+            if ((lane & 3) == i) mine = q;
+        }
+        const int64_t word = (lane & 3) * 16 + (lane >> 2);
+        if (word < left) out[w0 + word] = mine;
+    }
+}
+
 // Generic: one thread per output word, byte loads, any C.
 template <typename W>
 __global__ __launch_bounds__(256) void pack_generic_kernel(W *__restrict__ out, const uint8_t *__restrict__ in,
@@ -121,7 +153,10 @@ int pack_impl(W *out, const uint8_t *in, int64_t R, int64_t C, nb_stream_t strea
     NB_REQUIRE_ALIGNED(out, sizeof(W));
     NB_REQUIRE(Rw <= 2147483647LL, "%s: row of %lld words is too long", who, (long long)Rw);
     const unsigned blocks = grid_for(total);
-    if ((C & 15) == 0 && aligned(in, 16))
+    if (bits == 64 && (C & 63) == 0 && aligned(in, 16)) {
+        const unsigned qb = grid_for(ceil_div(total, 64) * 64);  // one wave per 64 words
+        pack_quad_kernel<<<dim3(qb), dim3(256), 0, as_stream(stream)>>>(reinterpret_cast<uint64_t *>(out), in, total);
+    } else if ((C & 15) == 0 && aligned(in, 16))
         pack_vec16_kernel<W><<<dim3(blocks), dim3(256), 0, as_stream(stream)>>>(out, in, total, (int)Rw, C);
     else
         pack_generic_kernel<W><<<dim3(blocks), dim3(256), 0, as_stream(stream)>>>(out, in, total, (int)Rw, C);

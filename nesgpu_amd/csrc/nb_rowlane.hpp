@@ -233,8 +233,7 @@ struct EpiPack {
             W v = valid ? st.cur : (W)0;
             bool writer = valid;
             if (POOL) {
-                v |= __shfl_xor(v, 1);
-                v |= __shfl_xor(v, 2);
+                v = or_reduce_group<4>(v);
                 writer = valid && (threadIdx.x & 3) == 0;
             }
             if (writer) out[row * Ow + n0 / bits] = v;

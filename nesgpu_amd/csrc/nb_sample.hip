@@ -42,36 +42,39 @@ __device__ __forceinline__ uint32_t nibble_lt(uint4 w, uint4 t)
 // ---- materialised sampler, wide path: C % bits == 0 and 16-byte aligned streams ------------------
 // One lane per 4 columns; bits/4 neighbouring lanes assemble one output word by OR-ing their
 // shifted nibbles across the lane group.
-template <typename W, class Src, int U, int BS, bool HAS_THR>
+// A workgroup owns BS consecutive quads of the [R, C] plane and U consecutive members: the thresholds and
+// the base word of a quad are fetched once and reused for the U members, whose stream loads (U independent
+// 16-byte non-temporal loads per lane, 16 KiB contiguous per member and workgroup) are all issued before
+// the first use.
+template <typename W, class Src, int U, int BS, bool HAS_THR, bool HAS_BASE>
 __global__ __launch_bounds__(BS) void sample_wide_kernel(W *__restrict__ out, const W *__restrict__ base,
                                                          const uint32_t *__restrict__ thresh, uint32_t ts, Src src,
-                                                         int64_t total_quads, int64_t RC4)
+                                                         int64_t n, uint32_t RC4, uint32_t plane_tiles,
+                                                         int64_t total_blocks)
 {
     constexpr int bits = WordTraits<W>::bits;
     constexpr int G = bits / 4;  // lanes per output word
-    // a workgroup walks tiles of BS*U consecutive quads; thread t owns quads tile + u*BS + t
-    for (int64_t tile = (int64_t)blockIdx.x * (BS * U); tile < total_quads; tile += (int64_t)gridDim.x * (BS * U)) {
-        uint4 w[U], t[U];
-        int64_t rq[U];
+    for (int64_t b = blockIdx.x; b < total_blocks; b += gridDim.x) {  // block-uniform
+        const int64_t mg = b / plane_tiles;
+        const uint32_t pt = (uint32_t)(b - mg * plane_tiles);
+        const uint32_t p = pt * BS + threadIdx.x;           // quad inside the plane
+        const uint32_t pc = p < RC4 ? p : RC4 - 1;          // clamp: no branch around the loads
+        const uint4 t = HAS_THR ? *reinterpret_cast<const uint4 *>(thresh + (int64_t)pc * 4) : make_uint4(ts, ts, ts, ts);
+        const W bw = HAS_BASE ? base[pc / G] : (W)0;
+        uint4 w[U];
 #pragma unroll
         for (int u = 0; u < U; u++) {
-            const int64_t q = tile + (int64_t)u * BS + threadIdx.x;
-            const int64_t qc = q < total_quads ? q : total_quads - 1;  // clamp: no branch around the load
-            rq[u] = qc % RC4;                                          // quad index inside one member
-            t[u] = HAS_THR ? *reinterpret_cast<const uint4 *>(thresh + rq[u] * 4) : make_uint4(ts, ts, ts, ts);
-            w[u] = src.load4(qc * 4);
+            int64_t m = mg * U + u;
+            m = m < n ? m : n - 1;
+            w[u] = src.load4(m * RC4 * 4, pc * 4u);
         }
-        __builtin_amdgcn_sched_barrier(0);  // all U stream loads in flight before the first use
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int u = 0; u < U; u++) {
-            const int64_t q = tile + (int64_t)u * BS + threadIdx.x;
-            W v = (W)nibble_lt(w[u], t[u]) << (4 * (int)(q & (G - 1)));
-#pragma unroll
-            for (int off = 1; off < G; off <<= 1) v |= __shfl_xor(v, off);
-            if (q < total_quads && (q & (G - 1)) == 0) {
-                if (base) v ^= base[rq[u] / G];
-                out[q / G] = v;  // flat output word index (C % bits == 0)
-            }
+            const int64_t m = mg * U + u;
+            W v = (W)nibble_lt(w[u], t) << (4 * (int)(p & (G - 1)));
+            v = or_reduce_group<G>(v) ^ bw;
+            if (m < n && p < RC4 && (p & (G - 1)) == 0) out[m * (RC4 / G) + p / G] = v;  // C % bits == 0
         }
     }
 }
@@ -318,17 +321,20 @@ int sample_impl(W *out, const W *base, const uint32_t *thresh, uint32_t ts, Src 
     NB_REQUIRE_ALIGNED(out, sizeof(W));
     hipStream_t s = as_stream(stream);
     const int64_t Rw = ceil_div(C, bits);
-    const int64_t quads = n * R * (C / 4);
-    if (C % bits == 0 && src_vec_ok && (!thresh || aligned(thresh, 16))) {
-        constexpr int U = 4, BS = 1024;
-        const int64_t tiles = ceil_div(quads, (int64_t)BS * U);
-        const dim3 grid((unsigned)(tiles < kMaxBlocks ? tiles : kMaxBlocks)), block(BS);
-        if (thresh)
-            sample_wide_kernel<W, Src, U, BS, true><<<grid, block, 0, s>>>(out, base, thresh, ts, src, quads,
-                                                                           R * (C / 4));
-        else
-            sample_wide_kernel<W, Src, U, BS, false><<<grid, block, 0, s>>>(out, base, thresh, ts, src, quads,
-                                                                            R * (C / 4));
+    if (C % bits == 0 && src_vec_ok && (!thresh || aligned(thresh, 16)) && R * (C / 4) < (1LL << 31)) {
+        constexpr int U = 8, BS = 1024;
+        const uint32_t rc4 = (uint32_t)(R * (C / 4));
+        const uint32_t plane_tiles = (uint32_t)ceil_div(rc4, BS);
+        const int64_t total_blocks = ceil_div(n, U) * plane_tiles;
+        const dim3 grid((unsigned)(total_blocks < kMaxBlocks ? total_blocks : kMaxBlocks)), block(BS);
+#define NB_LAUNCH_WIDE(T, B)                                                                                   \
+    sample_wide_kernel<W, Src, U, BS, T, B><<<grid, block, 0, s>>>(out, base, thresh, ts, src, n, rc4, plane_tiles, \
+                                                                   total_blocks)
+        if (thresh && base) NB_LAUNCH_WIDE(true, true);
+        else if (thresh) NB_LAUNCH_WIDE(true, false);
+        else if (base) NB_LAUNCH_WIDE(false, true);
+        else NB_LAUNCH_WIDE(false, false);
+#undef NB_LAUNCH_WIDE
     } else {
         sample_ballot_kernel<W, Src><<<dim3(grid_for(n * R * 64)), dim3(256), 0, s>>>(
             out, base, thresh, ts, src, n * R, R, (int)C, (int)Rw);
