@@ -80,19 +80,23 @@ int nb_im2col_i32(int32_t *out, const int32_t *in, int64_t D, int64_t H, int64_t
 /* conv: filt [D, fx*fy*Cw, O] -> out [D,h,w,O] int32 popcount sums; equals
  * bmm(im2col(in), filt) without materialising the columns.
  *   replaces extensions/booleanOperations.py:162-166 and boolop_cuda.binary_batch_conv2d
- *   (extensions/booleanOperations.cpp:43-50, extensions/booleanOperationsCuda.cu:295-298). */
+ *   (extensions/booleanOperations.cpp:43-50, extensions/booleanOperationsCuda.cu:295-298).
+ * tap_bits (all conv entry points): 0 = the layout above.  tap_bits = C > 0 declares that Cw == 1 and only
+ * the low C <= bits/2 bits of every input word are used (C true channels, zero tail as pack writes it); filt
+ * must then be the TAP-PACKED filter [D, ceil(fx*fy/T), O], T = bits/C, produced by nb_tap_pack_filter_*.
+ * T taps share a word, the sums are identical, the work is T times smaller. */
 int nb_conv_i64(int32_t *out, const int64_t *in, const int64_t *filt, int64_t D, int64_t H, int64_t W, int64_t Cw,
-                int64_t O, int fx, int fy, int px, int py, int sx, int sy, nb_stream_t stream);
+                int64_t O, int fx, int fy, int px, int py, int sx, int sy, int tap_bits, nb_stream_t stream);
 int nb_conv_i32(int32_t *out, const int32_t *in, const int32_t *filt, int64_t D, int64_t H, int64_t W, int64_t Cw,
-                int64_t O, int fx, int fy, int px, int py, int sx, int sy, nb_stream_t stream);
+                int64_t O, int fx, int fy, int px, int py, int sx, int sy, int tap_bits, nb_stream_t stream);
 /* conv_act: out [D,h,w,O] bool bytes = 2*popc > thresh[d,o]; thresh [D,O] int32.
  *   replaces extensions/booleanOperations.py:168-172. */
 int nb_conv_act_i64(uint8_t *out, const int64_t *in, const int64_t *filt, const int32_t *thresh, int64_t D,
                     int64_t H, int64_t W, int64_t Cw, int64_t O, int fx, int fy, int px, int py, int sx, int sy,
-                    nb_stream_t stream);
+                    int tap_bits, nb_stream_t stream);
 int nb_conv_act_i32(uint8_t *out, const int32_t *in, const int32_t *filt, const int32_t *thresh, int64_t D,
                     int64_t H, int64_t W, int64_t Cw, int64_t O, int fx, int fy, int px, int py, int sx, int sy,
-                    nb_stream_t stream);
+                    int tap_bits, nb_stream_t stream);
 /* conv_act_pack: the same bits packed along O into [D,h,w,ceil(O/bits)] words; with pool != 0
  * the 2x2 / stride-2 / no-padding OR-pool of those words, [D,h/2,w/2,ceil(O/bits)].
  * Equals pack(conv_act(...)) followed (pool) by max_pool2d(.,2,2,0,0,2,2); it fuses the chain
@@ -100,10 +104,17 @@ int nb_conv_act_i32(uint8_t *out, const int32_t *in, const int32_t *filt, const 
  * never reaches memory.  No single counterpart in the reference. */
 int nb_conv_act_pack_i64(int64_t *out, const int64_t *in, const int64_t *filt, const int32_t *thresh, int64_t D,
                          int64_t H, int64_t W, int64_t Cw, int64_t O, int fx, int fy, int px, int py, int sx,
-                         int sy, int pool, nb_stream_t stream);
+                         int sy, int pool, int tap_bits, nb_stream_t stream);
 int nb_conv_act_pack_i32(int32_t *out, const int32_t *in, const int32_t *filt, const int32_t *thresh, int64_t D,
                          int64_t H, int64_t W, int64_t Cw, int64_t O, int fx, int fy, int px, int py, int sx,
-                         int sy, int pool, nb_stream_t stream);
+                         int sy, int pool, int tap_bits, nb_stream_t stream);
+/* tap_pack_filter: filt [D, taps, O] (one word per tap, Cw == 1) -> out [D, ceil(taps/T), O], T = bits/tap_bits,
+ * out[d,w,o] = OR_t (filt[d,w*T+t,o] & (2^tap_bits - 1)) << (tap_bits*t).  A layout transform of the
+ * per-member filters of modules/binary.py:136-137; no counterpart in the reference. */
+int nb_tap_pack_filter_i64(int64_t *out, const int64_t *filt, int64_t D, int64_t taps, int64_t O, int tap_bits,
+                           nb_stream_t stream);
+int nb_tap_pack_filter_i32(int32_t *out, const int32_t *filt, int64_t D, int64_t taps, int64_t O, int tap_bits,
+                           nb_stream_t stream);
 
 /* ---- packed max-pool -------------------------------------------------------------------------
  * [B,H,W,Cw] -> [B,h,w,Cw]; bitwise OR over the 2x2 window anchored at (xo*sx-px, yo*sy-py),

@@ -25,9 +25,10 @@ _SUFFIXED = {
     "nb_bmm": [_PTR, _PTR, _PTR, _I64, _I64, _I64, _I64, _PTR],
     "nb_bmm_act": [_PTR, _PTR, _PTR, _PTR, _I64, _I64, _I64, _I64, _PTR],
     "nb_im2col": [_PTR, _PTR, _I64, _I64, _I64, _I64] + _GEOM + [_PTR],
-    "nb_conv": [_PTR, _PTR, _PTR, _I64, _I64, _I64, _I64, _I64] + _GEOM + [_PTR],
-    "nb_conv_act": [_PTR, _PTR, _PTR, _PTR, _I64, _I64, _I64, _I64, _I64] + _GEOM + [_PTR],
-    "nb_conv_act_pack": [_PTR, _PTR, _PTR, _PTR, _I64, _I64, _I64, _I64, _I64] + _GEOM + [_I32, _PTR],
+    "nb_conv": [_PTR, _PTR, _PTR, _I64, _I64, _I64, _I64, _I64] + _GEOM + [_I32, _PTR],
+    "nb_conv_act": [_PTR, _PTR, _PTR, _PTR, _I64, _I64, _I64, _I64, _I64] + _GEOM + [_I32, _PTR],
+    "nb_conv_act_pack": [_PTR, _PTR, _PTR, _PTR, _I64, _I64, _I64, _I64, _I64] + _GEOM + [_I32, _I32, _PTR],
+    "nb_tap_pack_filter": [_PTR, _PTR, _I64, _I64, _I64, _I32, _PTR],
     "nb_max_pool2d": [_PTR, _PTR, _I64, _I64, _I64, _I64] + _GEOM + [_PTR],
     "nb_sample_from_words": [_PTR, _PTR, _PTR, _U32, _PTR, _I64, _I64, _I64, _PTR],
     "nb_sample_philox": [_PTR, _PTR, _PTR, _U32, _U64, _U64, _U64, _I64, _I64, _I64, _PTR],

@@ -1,6 +1,6 @@
 // Packed im2col, implicit-im2col binary conv (int32 / bool / packed / packed+pooled outputs) and
 // the packed-bit max-pool.
-#include "nb_rowlane.hpp"
+#include "nb_conv_common.hpp"
 
 namespace nb {
 
@@ -55,88 +55,23 @@ __global__ __launch_bounds__(256) void max_pool_kernel(W *__restrict__ out, cons
     }
 }
 
-// ---- conv: row-per-lane kernel with the implicit-im2col loader ----------------------------------
-// POOLMAP: lanes 4q..4q+3 hold the 2x2 window of pooled pixel q (needed by EpiPack<.,true>);
-// otherwise lane p of a member is output pixel p in row-major order.
-template <typename W, int KC, int NT, bool SINGLE, bool EXACT, bool POOLMAP, class Epi>
-__global__ __launch_bounds__(256) void conv_rowlane_kernel(ConvA<W> al, const W *__restrict__ filt, Epi epi,
-                                                           int pblocks, int N)
-{
-    const ConvGeom &g = al.g;
-    const int64_t z = blockIdx.x / pblocks;
-    const int p = (int)(blockIdx.x - z * pblocks) * 256 + threadIdx.x;
-    int yo, xo;
-    bool valid;
-    int64_t orow;
-    if (POOLMAP) {
-        const int h2 = g.h >> 1, w2 = g.w >> 1;
-        const int q = p >> 2, sub = p & 3;
-        valid = q < h2 * w2;
-        const int qy = q / w2, qx = q - qy * w2;
-        yo = 2 * qy + (sub >> 1);
-        xo = 2 * qx + (sub & 1);
-        orow = z * (int64_t)(h2 * w2) + q;
-    } else {
-        valid = p < g.h * g.w;
-        yo = p / g.w;
-        xo = p - yo * g.w;
-        orow = z * (int64_t)(g.h * g.w) + p;
-    }
-    const typename ConvA<W>::Lane lane = al.lane_at(z, yo, xo, valid);
-    const int Kw = g.fx * g.fy * g.Cw;
-    const W *__restrict__ Fz = filt + z * (int64_t)Kw * N;
-    rowlane_body<W, KC, NT, SINGLE, EXACT>(al, lane, Fz, epi, orow, z, Kw, N);
-}
-
 template <typename W, bool POOLMAP, class Epi>
 static void dispatch_conv(const ConvA<W> &al, const W *filt, const Epi &epi, int64_t D, int64_t lanes_per_member,
                           int N, hipStream_t s)
 {
+    typedef ConvA<W> AL;
     const int Kw = al.g.fx * al.g.fy * al.g.Cw;
     const int pblocks = (int)ceil_div(lanes_per_member, 256);
     const dim3 grid((unsigned)(D * pblocks)), block(256);
-    if (Kw == 9)
-        conv_rowlane_kernel<W, 9, 16, true, true, POOLMAP, Epi><<<grid, block, 0, s>>>(al, filt, epi, pblocks, N);
-    else if (Kw == 18)
-        conv_rowlane_kernel<W, 18, 16, true, true, POOLMAP, Epi><<<grid, block, 0, s>>>(al, filt, epi, pblocks, N);
-    else if (Kw <= 4)
-        conv_rowlane_kernel<W, 4, 16, true, false, POOLMAP, Epi><<<grid, block, 0, s>>>(al, filt, epi, pblocks, N);
-    else if (Kw <= 9)
-        conv_rowlane_kernel<W, 9, 16, true, false, POOLMAP, Epi><<<grid, block, 0, s>>>(al, filt, epi, pblocks, N);
-    else if (Kw <= 18)
-        conv_rowlane_kernel<W, 18, 16, true, false, POOLMAP, Epi><<<grid, block, 0, s>>>(al, filt, epi, pblocks, N);
-    else
-        conv_rowlane_kernel<W, 16, 16, false, false, POOLMAP, Epi><<<grid, block, 0, s>>>(al, filt, epi, pblocks, N);
-}
-
-static int geom_check(ConvGeom *g, int64_t D, int64_t H, int64_t Wd, int64_t Cw, int fx, int fy, int px, int py,
-                      int sx, int sy, const char *who)
-{
-    NB_REQUIRE(D >= 0 && H >= 0 && Wd >= 0 && Cw >= 0, "%s: negative shape D=%lld H=%lld W=%lld Cw=%lld", who,
-               (long long)D, (long long)H, (long long)Wd, (long long)Cw);
-    NB_REQUIRE(fx >= 1 && fy >= 1 && sx >= 1 && sy >= 1 && px >= 0 && py >= 0,
-               "%s: bad window fx=%d fy=%d px=%d py=%d sx=%d sy=%d", who, fx, fy, px, py, sx, sy);
-    NB_REQUIRE(H <= 32768 && Wd <= 32768 && Cw <= 32768 && fx <= 1024 && fy <= 1024 && px <= 32768 && py <= 32768,
-               "%s: dimension too large (H=%lld W=%lld Cw=%lld fx=%d fy=%d)", who, (long long)H, (long long)Wd,
-               (long long)Cw, fx, fy);
-    const int64_t h = out_dim(H, fx, px, sx), w = out_dim(Wd, fy, py, sy);
-    NB_REQUIRE(H - fx + 2 * (int64_t)px >= 0 && Wd - fy + 2 * (int64_t)py >= 0,
-               "%s: window %dx%d larger than padded input %lldx%lld", who, fx, fy, (long long)(H + 2 * px),
-               (long long)(Wd + 2 * py));
-    NB_REQUIRE(h * w < (1LL << 30) && (int64_t)fx * fy * Cw < (1LL << 24), "%s: output %lldx%lld too large", who,
-               (long long)h, (long long)w);
-    g->H = (int)H;
-    g->Wd = (int)Wd;
-    g->Cw = (int)Cw;
-    g->fx = fx;
-    g->fy = fy;
-    g->px = px;
-    g->py = py;
-    g->sx = sx;
-    g->sy = sy;
-    g->h = (int)h;
-    g->w = (int)w;
-    return NB_OK;
+#define NB_CONV(KC, SINGLE, EXACT) \
+    conv_rowlane_kernel<W, AL, KC, 16, SINGLE, EXACT, POOLMAP, Epi><<<grid, block, 0, s>>>(al, filt, epi, pblocks, Kw, N)
+    if (Kw == 9) NB_CONV(9, true, true);
+    else if (Kw == 18) NB_CONV(18, true, true);
+    else if (Kw <= 4) NB_CONV(4, true, false);
+    else if (Kw <= 9) NB_CONV(9, true, false);
+    else if (Kw <= 18) NB_CONV(18, true, false);
+    else NB_CONV(16, false, false);
+#undef NB_CONV
 }
 
 template <typename W>
@@ -176,8 +111,8 @@ int max_pool_impl(W *out, const W *in, int64_t B, int64_t H, int64_t Wd, int64_t
 // mode 0: int32 sums, 1: bool bytes, 2: packed words, 3: packed + 2x2 pooled words
 template <typename W>
 int conv_impl(void *out, const W *in, const W *filt, const int32_t *thresh, int64_t D, int64_t H, int64_t Wd,
-              int64_t Cw, int64_t O, int fx, int fy, int px, int py, int sx, int sy, int mode, nb_stream_t stream,
-              const char *who)
+              int64_t Cw, int64_t O, int fx, int fy, int px, int py, int sx, int sy, int mode, int tap_bits,
+              nb_stream_t stream, const char *who)
 {
     constexpr int bits = WordTraits<W>::bits;
     ConvGeom g;
@@ -203,6 +138,15 @@ int conv_impl(void *out, const W *in, const W *filt, const int32_t *thresh, int6
     ConvA<W> al{in, g};
     hipStream_t s = as_stream(stream);
     const int N = (int)O;
+    NB_REQUIRE(tap_bits >= 0, "%s: negative tap_bits", who);
+    if (tap_bits > 0) {
+        NB_REQUIRE(Cw == 1 && 2 * tap_bits <= bits, "%s: tap packing needs Cw == 1 and tap_bits <= %d (got Cw=%lld, %d)",
+                   who, bits / 2, (long long)Cw, tap_bits);
+        if (mode == 0) NB_REQUIRE_ALIGNED(out, 4);
+        if (mode >= 2) NB_REQUIRE_ALIGNED(out, sizeof(W));
+        conv_tap_launch<W>(out, in, filt, thresh, g, D, lanes, N, tap_bits, mode, s);
+        return check_launch(who);
+    }
     if (mode == 0) {
         NB_REQUIRE_ALIGNED(out, 4);
         EpiI32 epi{static_cast<int32_t *>(out), (N & 3) == 0 && aligned(out, 16)};
@@ -253,41 +197,43 @@ int nb_max_pool2d_i32(int32_t *out, const int32_t *in, int64_t B, int64_t H, int
                                        s, "nb_max_pool2d_i32");
 }
 int nb_conv_i64(int32_t *out, const int64_t *in, const int64_t *filt, int64_t D, int64_t H, int64_t W, int64_t Cw,
-                int64_t O, int fx, int fy, int px, int py, int sx, int sy, nb_stream_t s)
+                int64_t O, int fx, int fy, int px, int py, int sx, int sy, int tap_bits, nb_stream_t s)
 {
-    return nb::conv_impl<uint64_t>(out, W64(in), W64(filt), nullptr, D, H, W, Cw, O, fx, fy, px, py, sx, sy, 0, s,
-                                   "nb_conv_i64");
+    return nb::conv_impl<uint64_t>(out, W64(in), W64(filt), nullptr, D, H, W, Cw, O, fx, fy, px, py, sx, sy, 0,
+                                   tap_bits, s, "nb_conv_i64");
 }
 int nb_conv_i32(int32_t *out, const int32_t *in, const int32_t *filt, int64_t D, int64_t H, int64_t W, int64_t Cw,
-                int64_t O, int fx, int fy, int px, int py, int sx, int sy, nb_stream_t s)
+                int64_t O, int fx, int fy, int px, int py, int sx, int sy, int tap_bits, nb_stream_t s)
 {
-    return nb::conv_impl<uint32_t>(out, W32(in), W32(filt), nullptr, D, H, W, Cw, O, fx, fy, px, py, sx, sy, 0, s,
-                                   "nb_conv_i32");
+    return nb::conv_impl<uint32_t>(out, W32(in), W32(filt), nullptr, D, H, W, Cw, O, fx, fy, px, py, sx, sy, 0,
+                                   tap_bits, s, "nb_conv_i32");
 }
 int nb_conv_act_i64(uint8_t *out, const int64_t *in, const int64_t *filt, const int32_t *thresh, int64_t D, int64_t H,
-                    int64_t W, int64_t Cw, int64_t O, int fx, int fy, int px, int py, int sx, int sy, nb_stream_t s)
+                    int64_t W, int64_t Cw, int64_t O, int fx, int fy, int px, int py, int sx, int sy, int tap_bits,
+                    nb_stream_t s)
 {
-    return nb::conv_impl<uint64_t>(out, W64(in), W64(filt), thresh, D, H, W, Cw, O, fx, fy, px, py, sx, sy, 1, s,
-                                   "nb_conv_act_i64");
+    return nb::conv_impl<uint64_t>(out, W64(in), W64(filt), thresh, D, H, W, Cw, O, fx, fy, px, py, sx, sy, 1,
+                                   tap_bits, s, "nb_conv_act_i64");
 }
 int nb_conv_act_i32(uint8_t *out, const int32_t *in, const int32_t *filt, const int32_t *thresh, int64_t D, int64_t H,
-                    int64_t W, int64_t Cw, int64_t O, int fx, int fy, int px, int py, int sx, int sy, nb_stream_t s)
+                    int64_t W, int64_t Cw, int64_t O, int fx, int fy, int px, int py, int sx, int sy, int tap_bits,
+                    nb_stream_t s)
 {
-    return nb::conv_impl<uint32_t>(out, W32(in), W32(filt), thresh, D, H, W, Cw, O, fx, fy, px, py, sx, sy, 1, s,
-                                   "nb_conv_act_i32");
+    return nb::conv_impl<uint32_t>(out, W32(in), W32(filt), thresh, D, H, W, Cw, O, fx, fy, px, py, sx, sy, 1,
+                                   tap_bits, s, "nb_conv_act_i32");
 }
 int nb_conv_act_pack_i64(int64_t *out, const int64_t *in, const int64_t *filt, const int32_t *thresh, int64_t D,
                          int64_t H, int64_t W, int64_t Cw, int64_t O, int fx, int fy, int px, int py, int sx, int sy,
-                         int pool, nb_stream_t s)
+                         int pool, int tap_bits, nb_stream_t s)
 {
     return nb::conv_impl<uint64_t>(out, W64(in), W64(filt), thresh, D, H, W, Cw, O, fx, fy, px, py, sx, sy,
-                                   pool ? 3 : 2, s, "nb_conv_act_pack_i64");
+                                   pool ? 3 : 2, tap_bits, s, "nb_conv_act_pack_i64");
 }
 int nb_conv_act_pack_i32(int32_t *out, const int32_t *in, const int32_t *filt, const int32_t *thresh, int64_t D,
                          int64_t H, int64_t W, int64_t Cw, int64_t O, int fx, int fy, int px, int py, int sx, int sy,
-                         int pool, nb_stream_t s)
+                         int pool, int tap_bits, nb_stream_t s)
 {
     return nb::conv_impl<uint32_t>(out, W32(in), W32(filt), thresh, D, H, W, Cw, O, fx, fy, px, py, sx, sy,
-                                   pool ? 3 : 2, s, "nb_conv_act_pack_i32");
+                                   pool ? 3 : 2, tap_bits, s, "nb_conv_act_pack_i32");
 }
 }

@@ -1,0 +1,77 @@
+// Shared by the conv translation units: geometry validation and the row-per-lane conv kernel.
+#pragma once
+#include "nb_rowlane.hpp"
+
+namespace nb {
+
+inline int geom_check(ConvGeom *g, int64_t D, int64_t H, int64_t Wd, int64_t Cw, int fx, int fy, int px, int py,
+                      int sx, int sy, const char *who)
+{
+    NB_REQUIRE(D >= 0 && H >= 0 && Wd >= 0 && Cw >= 0, "%s: negative shape D=%lld H=%lld W=%lld Cw=%lld", who,
+               (long long)D, (long long)H, (long long)Wd, (long long)Cw);
+    NB_REQUIRE(fx >= 1 && fy >= 1 && sx >= 1 && sy >= 1 && px >= 0 && py >= 0,
+               "%s: bad window fx=%d fy=%d px=%d py=%d sx=%d sy=%d", who, fx, fy, px, py, sx, sy);
+    NB_REQUIRE(H <= 32768 && Wd <= 32768 && Cw <= 32768 && fx <= 1024 && fy <= 1024 && px <= 32768 && py <= 32768,
+               "%s: dimension too large (H=%lld W=%lld Cw=%lld fx=%d fy=%d)", who, (long long)H, (long long)Wd,
+               (long long)Cw, fx, fy);
+    const int64_t h = out_dim(H, fx, px, sx), w = out_dim(Wd, fy, py, sy);
+    NB_REQUIRE(H - fx + 2 * (int64_t)px >= 0 && Wd - fy + 2 * (int64_t)py >= 0,
+               "%s: window %dx%d larger than padded input %lldx%lld", who, fx, fy, (long long)(H + 2 * px),
+               (long long)(Wd + 2 * py));
+    NB_REQUIRE(h * w < (1LL << 30) && (int64_t)fx * fy * Cw < (1LL << 24), "%s: output %lldx%lld too large", who,
+               (long long)h, (long long)w);
+    g->H = (int)H;
+    g->Wd = (int)Wd;
+    g->Cw = (int)Cw;
+    g->fx = fx;
+    g->fy = fy;
+    g->px = px;
+    g->py = py;
+    g->sx = sx;
+    g->sy = sy;
+    g->h = (int)h;
+    g->w = (int)w;
+    return NB_OK;
+}
+
+// ---- conv: row-per-lane kernel with the implicit-im2col loader ----------------------------------
+// POOLMAP: lanes 4q..4q+3 hold the 2x2 window of pooled pixel q (needed by EpiPack<.,true>);
+// otherwise lane p of a member is output pixel p in row-major order.
+template <typename W, class AL, int KC, int NT, bool SINGLE, bool EXACT, bool POOLMAP, class Epi>
+__global__ __launch_bounds__(256) void conv_rowlane_kernel(AL al, const W *__restrict__ filt, Epi epi, int pblocks,
+                                                           int Kw, int N)
+{
+    const ConvGeom &g = al.g;
+    const int64_t z = blockIdx.x / pblocks;
+    const int p = (int)(blockIdx.x - z * pblocks) * 256 + threadIdx.x;
+    int yo, xo;
+    bool valid;
+    int64_t orow;
+    if (POOLMAP) {
+        const int h2 = g.h >> 1, w2 = g.w >> 1;
+        const int q = p >> 2, sub = p & 3;
+        valid = q < h2 * w2;
+        const int qy = q / w2, qx = q - qy * w2;
+        yo = 2 * qy + (sub >> 1);
+        xo = 2 * qx + (sub & 1);
+        orow = z * (int64_t)(h2 * w2) + q;
+    } else {
+        valid = p < g.h * g.w;
+        yo = p / g.w;
+        xo = p - yo * g.w;
+        orow = z * (int64_t)(g.h * g.w) + p;
+    }
+    const typename AL::Lane lane = al.lane_at(z, yo, xo, valid);
+    const W *__restrict__ Fz = filt + z * (int64_t)Kw * N;
+    rowlane_body<W, KC, NT, SINGLE, EXACT>(al, lane, Fz, epi, orow, z, Kw, N);
+}
+
+// Tap-packed conv (narrow channels), defined in nb_conv_tap.hip.  `filt` is the tap-packed filter
+// [D, ceil(fx*fy / (bits/tap_bits)), N]; mode as in conv_impl.
+template <typename W>
+void conv_tap_launch(void *out, const W *in, const W *filt, const int32_t *thresh, const ConvGeom &g, int64_t D,
+                     int64_t lanes, int N, int tap_bits, int mode, hipStream_t s);
+
+inline int taps_per_word(int bits, int tap_bits) { return bits / tap_bits; }
+
+}  // namespace nb

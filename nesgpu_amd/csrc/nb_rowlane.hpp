@@ -88,6 +88,50 @@ struct ConvA {
     }
 };
 
+// Implicit im2col with TAP PACKING for narrow channels (Cw == 1, tap_bits = true channel count <= bits/2):
+// T = bits / tap_bits taps share one word, word w of an output pixel is OR_t tap(w*T + t) << (tap_bits*t).
+// The filter must be packed the same way (tap_pack_filter_kernel).  The popcount sum is unchanged because
+// both operands are zero above tap_bits (extensions/src/pack.cu:17) and an out-of-range tap is the zero word.
+template <typename W>
+struct ConvTapA {
+    const W *__restrict__ in;
+    ConvGeom g;
+    int tap_bits, T;
+    typedef typename ConvA<W>::Lane Lane;
+    __device__ __forceinline__ Lane lane_at(int64_t z, int yo, int xo, bool valid) const
+    {
+        Lane l;
+        l.valid = valid;
+        l.img = in + z * (int64_t)g.H * g.Wd;
+        l.y0 = yo * g.sx - g.px;
+        l.x0 = xo * g.sy - g.py;
+        return l;
+    }
+    template <int KC>
+    __device__ __forceinline__ void load(const Lane &l, int k0, W (&a)[KC]) const
+    {
+        const int taps = g.fx * g.fy;
+        int tap = k0 * T;
+        int ti = tap / g.fy;
+        int tj = tap - ti * g.fy;
+#pragma unroll
+        for (int i = 0; i < KC; i++) {
+            W wv = 0;
+            for (int t = 0; t < T && tap < taps; t++, tap++) {
+                const int y = l.y0 + ti, x = l.x0 + tj;
+                const bool ok = l.valid && y >= 0 && y < g.H && x >= 0 && x < g.Wd;
+                const W v = ok ? l.img[(int64_t)y * g.Wd + x] : (W)0;
+                wv |= v << (tap_bits * t);
+                if (++tj == g.fy) {
+                    tj = 0;
+                    ++ti;
+                }
+            }
+            a[i] = wv;
+        }
+    }
+};
+
 // ---- accumulate one K-chunk into an N-tile ----------------------------------------------------
 // EXACT: the chunk is complete (k0 + KC <= Kw), so the k-steps carry no guards and the scalar loads of
 // later steps can be issued while earlier steps compute.
@@ -217,20 +261,36 @@ struct EpiPack {
     const int32_t *__restrict__ thresh;
     int Ow;
     struct State {
-        W cur = 0;
+        uint32_t cur = 0;   // the 32-bit half being filled
+        uint32_t lo = 0;    // finished low half of a 64-bit word
     };
     template <int NT>
     __device__ __forceinline__ void tile(State &st, int64_t row, bool valid, int64_t z, int n0, int N,
                                          const int (&acc)[NT]) const
     {
         constexpr int bits = WordTraits<W>::bits;
-        static_assert(bits % NT == 0, "an N-tile must not straddle two output words");
+        static_assert(32 % NT == 0, "an N-tile must not straddle two 32-bit halves");
         const int32_t *__restrict__ t = thresh + z * N + n0;
+        const int sh = n0 & 31;
+        // 2*popc > t  <=>  popc > (t >> 1) for every integer t (arithmetic shift)
+        if (n0 + NT <= N) {
 #pragma unroll
-        for (int j = 0; j < NT; j++)
-            if (n0 + j < N) st.cur |= (W)(2 * acc[j] > t[j]) << ((n0 + j) & (bits - 1));
-        if (((n0 + NT) & (bits - 1)) == 0 || n0 + NT >= N) {
-            W v = valid ? st.cur : (W)0;
+            for (int j = 0; j < NT; j++) st.cur |= (uint32_t)(acc[j] > (t[j] >> 1)) << (sh + j);
+        } else {
+#pragma unroll
+            for (int j = 0; j < NT; j++)
+                if (n0 + j < N) st.cur |= (uint32_t)(acc[j] > (t[j] >> 1)) << (sh + j);
+        }
+        const bool last = n0 + NT >= N;
+        if (((n0 + NT) & 31) == 0 || last) {               // a 32-bit half is complete
+            const bool high = bits == 64 && ((n0 >> 5) & 1);
+            if (bits == 64 && !high && !last) {            // low half of a 64-bit word: keep it, go on
+                st.lo = st.cur;
+                st.cur = 0;
+                return;
+            }
+            W v = bits == 64 ? (W)(((uint64_t)(high ? st.cur : 0u) << 32) | (high ? st.lo : st.cur)) : (W)st.cur;
+            v = valid ? v : (W)0;
             bool writer = valid;
             if (POOL) {
                 v = or_reduce_group<4>(v);
@@ -238,6 +298,7 @@ struct EpiPack {
             }
             if (writer) out[row * Ow + n0 / bits] = v;
             st.cur = 0;
+            st.lo = 0;
         }
     }
     __device__ __forceinline__ void finish(State &, int64_t, bool) const {}

@@ -23,7 +23,7 @@ __all__ = [
     "batch_im2col", "bmm", "bmm_act", "conv", "conv_act", "pack", "int8pack", "sample_bits", "weighted_sum",
     "max_pool2d", "next_pow2_clip", "ceil_div", "unpack", "thresholds_from_p", "sample_bits_from_words",
     "flip_from_words", "sample_bits_philox", "flip_philox", "seeded_bmv_from_words", "seeded_bmv_philox",
-    "philox_words", "conv_act_pack",
+    "philox_words", "conv_act_pack", "tap_pack_filter", "tap_packing_applies",
 ]
 
 
@@ -133,7 +133,30 @@ def bmm_act(A, B, threshold):
     return C
 
 
-def _conv_args(input, filter, filterx, filtery):
+def tap_packing_applies(in_bits, Cw, dtype):
+    """True when a conv over inputs with ``in_bits`` true channels in ``Cw`` words per pixel can share one word
+    between several filter taps (Cw == 1 and at least two taps fit a word)."""
+    return in_bits is not None and Cw == 1 and 0 < 2 * int(in_bits) <= torch.iinfo(dtype).bits
+
+
+def tap_pack_filter(filter, taps, in_bits):
+    """[D, taps, O] per-member filters with one word per tap (only the low ``in_bits`` bits used) ->
+    [D, ceil(taps/T), O] with T = bits // in_bits taps per word.  Feed the result to conv / conv_act /
+    conv_act_pack with ``in_bits=...`` and ``filter_tap_packed=True``."""
+    _check(filter, "filter")
+    assert len(filter.shape) == 3 and filter.size(1) == taps
+    suf, bits = _suffix(filter.dtype)
+    assert 0 < 2 * in_bits <= bits
+    T = bits // in_bits
+    out = torch.empty((filter.size(0), ceil_div(taps, T), filter.size(2)), dtype=filter.dtype, device=filter.device)
+    with torch.cuda.device(filter.device):
+        _lib.call("nb_tap_pack_filter" + suf, out.data_ptr(), filter.data_ptr(), filter.size(0), taps, filter.size(2),
+                  int(in_bits), _stream(filter))
+    return out
+
+
+def _conv_args(input, filter, filterx, filtery, in_bits=None, filter_tap_packed=False):
+    """-> (suffix, bits, filter to pass, tap_bits)"""
     _check(input, "input")
     _check(filter, "filter")
     _same_device(input, filter)
@@ -141,26 +164,42 @@ def _conv_args(input, filter, filterx, filtery):
     assert len(filter.shape) == 3
     assert input.size(0) == filter.size(0)                       # "Batch dim doesn't match", booleanOperations.cpp:46
     assert input.dtype == filter.dtype                           # booleanOperations.cpp:48
-    assert filter.size(1) == filterx * filtery * input.size(3)   # the bmm contraction assert (:111)
-    return _suffix(input.dtype)
+    suf, bits = _suffix(input.dtype)
+    taps = filterx * filtery
+    if tap_packing_applies(in_bits, input.size(3), input.dtype):
+        T = bits // int(in_bits)
+        if filter_tap_packed:
+            assert filter.size(1) == ceil_div(taps, T)
+        else:
+            assert filter.size(1) == taps
+            filter = tap_pack_filter(filter, taps, int(in_bits))
+        return suf, bits, filter, int(in_bits)
+    assert not filter_tap_packed, "filter_tap_packed needs in_bits with Cw == 1 and 2*in_bits <= word bits"
+    assert filter.size(1) == taps * input.size(3)                # the bmm contraction assert (:111)
+    return suf, bits, filter, 0
 
 
-def conv(input, filter, filterx, filtery, padx, pady, stridex, stridey):
+def conv(input, filter, filterx, filtery, padx, pady, stridex, stridey, in_bits=None, filter_tap_packed=False):
     """bmm(batch_im2col(input), filter).view(D,h,w,O) without materialising the columns
-    (extensions/booleanOperations.py:162-166).  filter is [D, filterx*filtery*Cw, O]."""
-    suf, _ = _conv_args(input, filter, filterx, filtery)
+    (extensions/booleanOperations.py:162-166).  filter is [D, filterx*filtery*Cw, O].
+
+    ``in_bits`` (optional, not in the reference): the true channel count C of the packed input.  When the
+    input has one word per pixel and 2*C <= word bits, several filter taps share a word (same sums, less
+    work); the filter is re-packed on the fly unless ``filter_tap_packed`` says it already is."""
+    suf, _, filter, tap = _conv_args(input, filter, filterx, filtery, in_bits, filter_tap_packed)
     h, w = _out_hw(input, filterx, filtery, padx, pady, stridex, stridey)
     out = torch.empty((input.size(0), h, w, filter.size(2)), dtype=torch.int32, device=input.device)
     with torch.cuda.device(input.device):
         _lib.call("nb_conv" + suf, out.data_ptr(), input.data_ptr(), filter.data_ptr(), input.size(0), input.size(1),
-                  input.size(2), input.size(3), filter.size(2), filterx, filtery, padx, pady, stridex, stridey,
+                  input.size(2), input.size(3), filter.size(2), filterx, filtery, padx, pady, stridex, stridey, tap,
                   _stream(input))
     return out
 
 
-def conv_act(input, filter, threshold, filterx, filtery, padx, pady, stridex, stridey):
+def conv_act(input, filter, threshold, filterx, filtery, padx, pady, stridex, stridey, in_bits=None,
+             filter_tap_packed=False):
     """bmm_act(batch_im2col(input), filter, threshold).view(D,h,w,O) (extensions/booleanOperations.py:168-172)."""
-    suf, _ = _conv_args(input, filter, filterx, filtery)
+    suf, _, filter, tap = _conv_args(input, filter, filterx, filtery, in_bits, filter_tap_packed)
     _check(threshold, "threshold")
     _same_device(input, threshold)
     assert len(threshold.shape) == 2
@@ -172,7 +211,7 @@ def conv_act(input, filter, threshold, filterx, filtery, padx, pady, stridex, st
     with torch.cuda.device(input.device):
         _lib.call("nb_conv_act" + suf, out.data_ptr(), input.data_ptr(), filter.data_ptr(), threshold.data_ptr(),
                   input.size(0), input.size(1), input.size(2), input.size(3), filter.size(2), filterx, filtery, padx,
-                  pady, stridex, stridey, _stream(input))
+                  pady, stridex, stridey, tap, _stream(input))
     return out
 
 
@@ -394,10 +433,12 @@ def philox_words(count, seed, subsequence=0, first=0, device=None):
     return out
 
 
-def conv_act_pack(input, filter, threshold, filterx, filtery, padx, pady, stridex, stridey, pool=False):
+def conv_act_pack(input, filter, threshold, filterx, filtery, padx, pady, stridex, stridey, pool=False, in_bits=None,
+                  filter_tap_packed=False):
     """pack(conv_act(...)) along the channel axis -> [D,h,w,ceil(O/bits)]; with ``pool`` followed by the
-    2x2/stride-2 OR-pool -> [D,h//2,w//2,ceil(O/bits)].  One kernel; the bool map never reaches memory."""
-    suf, bits = _conv_args(input, filter, filterx, filtery)
+    2x2/stride-2 OR-pool -> [D,h//2,w//2,ceil(O/bits)].  One kernel; the bool map never reaches memory.
+    ``in_bits`` / ``filter_tap_packed`` as in :func:`conv`."""
+    suf, bits, filter, tap = _conv_args(input, filter, filterx, filtery, in_bits, filter_tap_packed)
     _check(threshold, "threshold")
     _same_device(input, threshold)
     assert tuple(threshold.shape) == (input.size(0), filter.size(2))
@@ -409,5 +450,5 @@ def conv_act_pack(input, filter, threshold, filterx, filtery, padx, pady, stride
     with torch.cuda.device(input.device):
         _lib.call("nb_conv_act_pack" + suf, out.data_ptr(), input.data_ptr(), filter.data_ptr(), threshold.data_ptr(),
                   input.size(0), input.size(1), input.size(2), input.size(3), filter.size(2), filterx, filtery, padx,
-                  pady, stridex, stridey, 1 if pool else 0, _stream(input))
+                  pady, stridex, stridey, 1 if pool else 0, tap, _stream(input))
     return out

@@ -164,6 +164,7 @@ class BinarizedConv2d(Binarized):
         if (pack_output or pool_output) and (batch_norm or not threshold):
             raise NotImplementedError("packed output needs threshold=True, batch_norm=False")
         self.weight_noise_reshaped = None
+        self.weight_noise_tap = None
         self.reset_parameters()
 
     def reset_parameters(self):
@@ -175,6 +176,11 @@ class BinarizedConv2d(Binarized):
         r = self.weight_noise.view(self.directions, self.out_channels, *self.kernel_size, -1)
         self.weight_noise_reshaped = r.permute([0, 2, 3, 4, 1]).reshape(self.directions, -1,
                                                                        self.out_channels).contiguous()
+        # narrow inputs (one word per pixel, at most half of it used): several taps share a word
+        self.weight_noise_tap = None
+        if booleanOperations.tap_packing_applies(self.in_channels, self.weight_noise.size(2), self.dtype):
+            self.weight_noise_tap = booleanOperations.tap_pack_filter(
+                self.weight_noise_reshaped, self.kernel_size[0] * self.kernel_size[1], self.in_channels)
 
     def forward(self, input):
         if not self.perturbed_flag:
@@ -186,21 +192,25 @@ class BinarizedConv2d(Binarized):
             packed_input = input
         offset = self.in_channels * self.kernel_size[0] * self.kernel_size[1]
         geom = (*self.kernel_size, self.padding, self.padding, self.stride, self.stride)
+        filt, tapkw = self.weight_noise_reshaped, {}
+        if getattr(self, "weight_noise_tap", None) is not None:
+            filt, tapkw = self.weight_noise_tap, dict(in_bits=self.in_channels, filter_tap_packed=True)
         if self.threshold:
             if self.batch_norm:
-                activation = 2 * booleanOperations.conv(packed_input, self.weight_noise_reshaped, *geom) - offset
+                activation = 2 * booleanOperations.conv(packed_input, filt, *geom, **tapkw) - offset
                 thresh = self.bias + self.bias_noise + activation.type(torch.float16).mean(dim=[1, 2])
                 return activation > thresh.unsqueeze(1).unsqueeze(1)
             thresh = (self.bias + self.bias_noise).type(torch.int32) + offset
             if self.pack_output or self.pool_output:
-                return booleanOperations.conv_act_pack(packed_input, self.weight_noise_reshaped, thresh, *geom,
-                                                       pool=self.pool_output)
-            return booleanOperations.conv_act(packed_input, self.weight_noise_reshaped, thresh, *geom)
-        return 2 * booleanOperations.conv(packed_input, self.weight_noise_reshaped, *geom) - offset
+                return booleanOperations.conv_act_pack(packed_input, filt, thresh, *geom, pool=self.pool_output,
+                                                       **tapkw)
+            return booleanOperations.conv_act(packed_input, filt, thresh, *geom, **tapkw)
+        return 2 * booleanOperations.conv(packed_input, filt, *geom, **tapkw) - offset
 
     def free_memory(self):
         Perturbed.free_memory(self)
         self.weight_noise_reshaped = None
+        self.weight_noise_tap = None
 
 
 class BinarizedMaxPool2d(nn.Module):

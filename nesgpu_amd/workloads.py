@@ -95,6 +95,14 @@ def _conv_filters(base_bits, D, O, k, C, T, seed, subseq, dtype, device):
     return base, Wn, filt
 
 
+def _tap(filt, k, C):
+    """(filter to pass, extra conv kwargs): the tap-packed filter when C is narrow enough, as
+    BinarizedConv2d.set_noise prepares it."""
+    if ops.tap_packing_applies(C, 1, filt.dtype) and filt.size(1) == k * k:
+        return ops.tap_pack_filter(filt, k * k, C), dict(in_bits=C, filter_tap_packed=True)
+    return filt, {}
+
+
 def conv_int32(D=1024, C=64, O=64, S=32, k=3, pad=1, T=T_P02, seed=0, dtype=torch.int64, device="cuda"):
     """Config 3: batched binary conv, int32 popcount maps out."""
     g = _gen(seed)
@@ -122,14 +130,15 @@ def conv_sign_pool(D=1024, C=16, O=16, S=64, k=3, pad=1, T=T_P02, seed=0, dtype=
     base, Wn, filt = _conv_filters(base_bits, D, O, k, C, T, seed, 4, dtype, device)
     K = k * k * C
     thr = torch.full((D, O), K, dtype=torch.int32, device=device)                # 2*popc > K  <=>  2*popc - K > 0
+    ftap, kw = _tap(filt, k, C)
     h = S + 2 * pad - k + 1
     out_words = D * (h // 2) * (h // 2) * ((O + 63) // 64)
     w = Workload(
         name="conv %d->%d %dx%d pad %d on %dx%d D=%d -> sign -> 2x2 OR-pool, packed out" % (C, O, k, k, pad, S, S, D),
         population=D, bit_macs=D * h * h * O * K,
         algo_bytes=x.numel() * x.element_size() + filt.numel() * filt.element_size() + out_words * 8,
-        bound="valu", step=lambda: ops.conv_act_pack(x, filt, thr, k, k, pad, pad, 1, 1, pool=True),
-        tensors=dict(x=x, base=base, Wn=Wn, filt=filt, thr=thr), meta=dict(T=T, seed=seed, subsequence=4, C=C, O=O,
+        bound="valu", step=lambda: ops.conv_act_pack(x, ftap, thr, k, k, pad, pad, 1, 1, pool=True, **kw),
+        tensors=dict(x=x, base=base, Wn=Wn, filt=filt, thr=thr, filt_tap=ftap), meta=dict(T=T, seed=seed, subsequence=4, C=C, O=O,
                                                                              k=k, pad=pad))
     return w
 
@@ -149,7 +158,7 @@ def cifar_net(D=4096, T=T_P01, seed=0, dtype=torch.int64, device="cuda", classes
         base, Wn, filt = _conv_filters(base_bits, D, O, 3, C, T, seed, subseq, dtype, device)
         del Wn
         thr = torch.full((D, O), 9 * C, dtype=torch.int32, device=device)
-        layers.append((filt, thr))
+        layers.append((filt, thr) + _tap(filt, 3, C))
         macs += D * S * S * O * 9 * C
         subseq += 1
     b4 = ops.pack(_bits(g, (1024, 8192)).to(device), dtype)
@@ -159,9 +168,10 @@ def cifar_net(D=4096, T=T_P01, seed=0, dtype=torch.int64, device="cuda", classes
     macs += D * 1024 * 8192 + D * classes * 1024
 
     def step():
-        a = ops.conv_act_pack(x, layers[0][0], layers[0][1], 3, 3, 1, 1, 1, 1)                 # [D,32,32,1]
-        a = ops.conv_act_pack(a, layers[1][0], layers[1][1], 3, 3, 1, 1, 1, 1, pool=True)      # [D,16,16,1]
-        a = ops.conv_act_pack(a, layers[2][0], layers[2][1], 3, 3, 1, 1, 1, 1, pool=True)      # [D,8,8,2]
+        a = x
+        for i, pool in enumerate((False, True, True)):                   # [D,32,32,1] [D,16,16,1] [D,8,8,2]
+            _, thr, f, kw = layers[i]
+            a = ops.conv_act_pack(a, f, thr, 3, 3, 1, 1, 1, 1, pool=pool, **kw)
         a = a.view(D, -1, 1)                                                                    # [D,128,1]
         p4 = ops.bmm(W4, a).squeeze(2)                                                          # [D,1024]
         a = ops.pack(2 * p4 > 8192, dtype).view(D, -1, 1)                                       # [D,16,1]

@@ -53,13 +53,17 @@ def test_bad_arguments_are_rejected_without_a_launch(lib):
     # misaligned words
     assert lib.nb_bmm_i64(one, odd, one, 1, 1, 1, 2, None) == 3
     # conv window larger than the padded input
-    assert lib.nb_conv_i64(one, one, one, 1, 2, 2, 1, 1, 5, 5, 0, 0, 1, 1, None) == 2
+    assert lib.nb_conv_i64(one, one, one, 1, 2, 2, 1, 1, 5, 5, 0, 0, 1, 1, 0, None) == 2
+    # tap packing needs one word per pixel and at most half a word of channels
+    assert lib.nb_conv_i64(one, one, one, 1, 8, 8, 2, 4, 3, 3, 1, 1, 1, 1, 16, None) == 2
+    assert lib.nb_conv_i64(one, one, one, 1, 8, 8, 1, 4, 3, 3, 1, 1, 1, 1, 40, None) == 2
+    assert lib.nb_tap_pack_filter_i64(one, one, 1, 9, 4, 0, None) == 2
     # zero stride
     assert lib.nb_max_pool2d_i64(one, one, 1, 4, 4, 1, 2, 2, 0, 0, 0, 2, None) == 2
     # empty problems succeed without touching the pointers
     assert lib.nb_pack_i64(None, None, 0, 64, None) == 0
     assert lib.nb_bmm_i32(None, None, None, 0, 5, 5, 5, None) == 0
-    assert lib.nb_conv_i64(None, None, None, 0, 8, 8, 1, 4, 3, 3, 1, 1, 1, 1, None) == 0
+    assert lib.nb_conv_i64(None, None, None, 0, 8, 8, 1, 4, 3, 3, 1, 1, 1, 1, 0, None) == 0
     assert lib.nb_sample_from_words_i64(None, None, None, 0, None, 0, 3, 64, None) == 0
     with pytest.raises(RuntimeError, match="negative"):
         _lib.call("nb_unpack_i32", one, one, -2, 1, None)

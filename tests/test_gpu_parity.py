@@ -362,3 +362,48 @@ def test_errors_match_the_reference_conventions(ops):
                  torch.zeros(1, 25, 4, dtype=torch.int64, device="cuda"), 5, 5, 0, 0, 1, 1)
     assert ops.bmm(torch.zeros(0, 3, 4, dtype=torch.int64, device="cuda"),
                    torch.zeros(0, 4, 2, dtype=torch.int64, device="cuda")).shape == (0, 3, 2)
+
+
+@pytest.mark.parametrize("dtype", [torch.int64, torch.int32])
+@pytest.mark.parametrize("C,O,k,pad,stride", [(16, 16, 3, 1, 1), (3, 64, 3, 1, 1), (1, 5, 7, 2, 3), (8, 33, 5, 2, 2),
+                                              (32, 20, 3, 0, 1), (16, 70, 1, 0, 1), (5, 16, 3, 2, 1), (2, 4, 9, 4, 1)])
+def test_conv_tap_packing_gives_the_same_sums(ops, oracle, dtype, C, O, k, pad, stride):
+    """in_bits=C lets several filter taps share a word; every output must equal the one-word-per-tap path."""
+    nd = NDT[dtype]
+    bits = torch.iinfo(dtype).bits
+    D, S = 4, 11
+    g = rng(C * 100 + O + k)
+    xb = g.integers(0, 2, size=(D * S * S, C)).astype(bool)
+    x = oracle.pack(xb, nd).reshape(D, S, S, 1)
+    fb = g.integers(0, 2, size=(D * O * k * k, C)).astype(bool)
+    f = np.ascontiguousarray(oracle.pack(fb, nd).reshape(D, O, k, k, 1).transpose(0, 2, 3, 4, 1).reshape(D, -1, O))
+    K = k * k * C
+    thr = (g.integers(0, K + 1, size=(D, O)) - K // 2 + K).astype(np.int32)
+    geom = (k, k, pad, pad, stride, stride)
+    xd, fd, td = dev(x), dev(f), dev(thr)
+    want = oracle.conv(x, f, *geom)
+    eligible = 2 * C <= bits
+    assert ops.tap_packing_applies(C, 1, dtype) == eligible
+    got = ops.conv(xd, fd, *geom, in_bits=C)
+    np.testing.assert_array_equal(host(got), want)
+    if eligible:
+        fp = ops.tap_pack_filter(fd, k * k, C)
+        T = bits // C
+        assert tuple(fp.shape) == (D, (k * k + T - 1) // T, O)
+        # closed form of the packed filter: OR of tap words shifted by C*t
+        fw = f.astype(np.uint64 if bits == 64 else np.uint32)
+        ref = np.zeros(fp.shape, dtype=fw.dtype)
+        for tap in range(k * k):
+            ref[:, tap // T, :] |= fw[:, tap, :] << fw.dtype.type(C * (tap % T))
+        np.testing.assert_array_equal(host(fp).view(ref.dtype), ref)
+        kw = dict(in_bits=C, filter_tap_packed=True)
+        np.testing.assert_array_equal(host(ops.conv(xd, fp, *geom, **kw)), want)
+        np.testing.assert_array_equal(host(ops.conv_act(xd, fp, td, *geom, **kw)), 2 * want > thr[:, None, None, :])
+        act = oracle.conv_act(x, f, thr, *geom)
+        h, w = act.shape[1:3]
+        packed = oracle.pack(act.reshape(-1, O), nd).reshape(D, h, w, -1)
+        np.testing.assert_array_equal(host(ops.conv_act_pack(xd, fp, td, *geom, **kw)), packed)
+        assert torch.equal(ops.conv_act_pack(xd, fd, td, *geom, in_bits=C), ops.conv_act_pack(xd, fd, td, *geom))
+        if h >= 2 and w >= 2:
+            np.testing.assert_array_equal(host(ops.conv_act_pack(xd, fp, td, *geom, pool=True, **kw)),
+                                          oracle.max_pool2d(packed, 2, 2, 0, 0, 2, 2))
