@@ -108,6 +108,17 @@ int nb_conv_act_pack_i64(int64_t *out, const int64_t *in, const int64_t *filt, c
 int nb_conv_act_pack_i32(int32_t *out, const int32_t *in, const int32_t *filt, const int32_t *thresh, int64_t D,
                          int64_t H, int64_t W, int64_t Cw, int64_t O, int fx, int fy, int px, int py, int sx,
                          int sy, int pool, int tap_bits, nb_stream_t stream);
+/* Conv engine selector (process-wide tunable, not per call).  Two engines compute the same sums bit for bit: the
+ * XOR-popcount kernels (any shape) and an int8 matrix-core kernel (64-bit words, stride 1, O % 16 == 0,
+ * K = taps*channels up to 1152 positions, one member's image fits LDS).  0 = automatic: the matrix-core kernel on
+ * the shapes where it measured faster (output maps from 32x32 on, or from 16x16 when K reaches 1152), else
+ * XOR-popcount; 1 = XOR-popcount only; 2 = matrix cores wherever that kernel covers the shape.  Returns the
+ * previous setting; any other argument only queries.  Initial value from the environment variable
+ * NESBIN_CONV_ENGINE: first letter 'v' -> 1, 'm' -> 2, else 0.  No counterpart in the reference. */
+int nb_conv_engine(int engine);
+/* Engine that served the calling thread's latest conv / conv_act / conv_act_pack launch: 1 = XOR-popcount,
+ * 2 = matrix cores, 0 = none yet.  For tests and tuning.  No counterpart in the reference. */
+int nb_conv_last_engine(void);
 /* tap_pack_filter: filt [D, taps, O] (one word per tap, Cw == 1) -> out [D, ceil(taps/T), O], T = bits/tap_bits,
  * out[d,w,o] = OR_t (filt[d,w*T+t,o] & (2^tap_bits - 1)) << (tap_bits*t).  A layout transform of the
  * per-member filters of modules/binary.py:136-137; no counterpart in the reference. */

@@ -38,6 +38,8 @@ _SUFFIXED = {
 }
 _PLAIN = {
     "nb_philox_words": [_PTR, _U64, _U64, _U64, _I64, _PTR],
+    "nb_conv_engine": [_I32],
+    "nb_conv_last_engine": [],
 }
 
 

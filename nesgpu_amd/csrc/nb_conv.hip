@@ -1,5 +1,7 @@
 // Packed im2col, implicit-im2col binary conv (int32 / bool / packed / packed+pooled outputs) and
 // the packed-bit max-pool.
+#include <cstdlib>
+
 #include "nb_conv_common.hpp"
 
 namespace nb {
@@ -108,6 +110,27 @@ int max_pool_impl(W *out, const W *in, int64_t B, int64_t H, int64_t Wd, int64_t
     return check_launch(who);
 }
 
+// Process-wide choice between the two conv engines (both give identical results): 0 = automatic (matrix cores
+// on the shapes where they measured faster, else XOR-popcount), 1 = XOR-popcount only, 2 = matrix cores wherever
+// a kernel covers the shape.  Initialised from the environment variable NESBIN_CONV_ENGINE ("valu" -> 1,
+// "mfma" -> 2); nb_conv_engine() changes it.
+static int g_conv_engine = -1;
+static int conv_engine()
+{
+    if (g_conv_engine < 0) {
+        const char *v = getenv("NESBIN_CONV_ENGINE");
+        g_conv_engine = (v && v[0] == 'v') ? 1 : (v && v[0] == 'm') ? 2 : 0;
+    }
+    return g_conv_engine;
+}
+static thread_local int t_last_engine = 0;  // engine of this thread's latest conv launch: 1 XOR-popcount, 2 matrix cores
+int set_conv_engine(int e)
+{
+    const int prev = conv_engine();
+    if (e >= 0 && e <= 2) g_conv_engine = e;
+    return prev;
+}
+
 // mode 0: int32 sums, 1: bool bytes, 2: packed words, 3: packed + 2x2 pooled words
 template <typename W>
 int conv_impl(void *out, const W *in, const W *filt, const int32_t *thresh, int64_t D, int64_t H, int64_t Wd,
@@ -139,11 +162,21 @@ int conv_impl(void *out, const W *in, const W *filt, const int32_t *thresh, int6
     hipStream_t s = as_stream(stream);
     const int N = (int)O;
     NB_REQUIRE(tap_bits >= 0, "%s: negative tap_bits", who);
-    if (tap_bits > 0) {
+    if (tap_bits > 0)
         NB_REQUIRE(Cw == 1 && 2 * tap_bits <= bits, "%s: tap packing needs Cw == 1 and tap_bits <= %d (got Cw=%lld, %d)",
                    who, bits / 2, (long long)Cw, tap_bits);
-        if (mode == 0) NB_REQUIRE_ALIGNED(out, 4);
-        if (mode >= 2) NB_REQUIRE_ALIGNED(out, sizeof(W));
+    if (mode == 0) NB_REQUIRE_ALIGNED(out, 4);
+    if (mode >= 2) NB_REQUIRE_ALIGNED(out, sizeof(W));
+    // int8 matrix-core path (64-bit words, stride 1, O % 16 == 0, member fits LDS); same results
+    const int engine = conv_engine();
+    if (bits == 64 && Cw > 0 && engine != 1 &&
+        conv_mfma_try(out, reinterpret_cast<const uint64_t *>(in), reinterpret_cast<const uint64_t *>(filt), thresh, g,
+                      D, N, tap_bits, tap_bits > 0, mode, engine == 2, s)) {
+        t_last_engine = 2;
+        return check_launch(who);
+    }
+    t_last_engine = 1;
+    if (tap_bits > 0) {
         conv_tap_launch<W>(out, in, filt, thresh, g, D, lanes, N, tap_bits, mode, s);
         return check_launch(who);
     }
@@ -172,6 +205,8 @@ int conv_impl(void *out, const W *in, const W *filt, const int32_t *thresh, int6
 #define W32(p) reinterpret_cast<const uint32_t *>(p)
 
 extern "C" {
+int nb_conv_engine(int engine) { return nb::set_conv_engine(engine); }
+int nb_conv_last_engine(void) { return nb::t_last_engine; }
 int nb_im2col_i64(int64_t *out, const int64_t *in, int64_t D, int64_t H, int64_t W, int64_t Cw, int fx, int fy, int px,
                   int py, int sx, int sy, nb_stream_t s)
 {

@@ -23,7 +23,7 @@ __all__ = [
     "batch_im2col", "bmm", "bmm_act", "conv", "conv_act", "pack", "int8pack", "sample_bits", "weighted_sum",
     "max_pool2d", "next_pow2_clip", "ceil_div", "unpack", "thresholds_from_p", "sample_bits_from_words",
     "flip_from_words", "sample_bits_philox", "flip_philox", "seeded_bmv_from_words", "seeded_bmv_philox",
-    "philox_words", "conv_act_pack", "tap_pack_filter", "tap_packing_applies",
+    "philox_words", "conv_act_pack", "tap_pack_filter", "tap_packing_applies", "conv_engine", "conv_last_engine",
 ]
 
 
@@ -131,6 +131,18 @@ def bmm_act(A, B, threshold):
         _lib.call("nb_bmm_act" + suf, C.data_ptr(), A.data_ptr(), B.data_ptr(), threshold.data_ptr(), A.size(0),
                   A.size(1), A.size(2), B.size(2), _stream(A))
     return C
+
+
+def conv_engine(engine=None):
+    """Query / set the process-wide conv engine: 0 = automatic (int8 matrix cores on the shapes where they measured
+    faster, else XOR-popcount), 1 = XOR-popcount kernels only, 2 = matrix cores wherever a kernel covers the shape.
+    Returns the previous setting.  Results are identical either way."""
+    return _lib.load().nb_conv_engine(-1 if engine is None else int(engine))
+
+
+def conv_last_engine():
+    """Engine that served this thread's latest conv launch: 1 = XOR-popcount, 2 = matrix cores, 0 = none yet."""
+    return _lib.load().nb_conv_last_engine()
 
 
 def tap_packing_applies(in_bits, Cw, dtype):

@@ -23,6 +23,15 @@ def ops():
     return booleanOperations
 
 
+@pytest.fixture(params=[1, 2], ids=["popcount", "matrixcore"])
+def engine(request, ops):
+    """Runs a conv test once per engine: 1 = XOR-popcount kernels only, 2 = int8 matrix cores wherever that kernel
+    covers the shape (the XOR-popcount kernels take the rest)."""
+    prev = ops.conv_engine(request.param)
+    yield request.param
+    ops.conv_engine(prev)
+
+
 def dev(a):
     return torch.from_numpy(np.ascontiguousarray(a)).cuda()
 
@@ -63,7 +72,7 @@ def test_golden_bmm(ops, tag, case):
 
 @pytest.mark.parametrize("tag", TAGS)
 @pytest.mark.parametrize("case", CONV_CASES)
-def test_golden_conv(ops, tag, case):
+def test_golden_conv(ops, engine, tag, case):
     x, f = dev(G[f"conv_{tag}_{case}_x"]), dev(G[f"conv_{tag}_{case}_f"])
     thr = dev(G[f"conv_{tag}_{case}_thr"])
     geom = [int(v) for v in G[f"conv_{tag}_{case}_geom"]]
@@ -191,7 +200,7 @@ SWEEP = list(itertools.product([1, 3, 7], [0, 1, 2], [1, 2, 3]))                
 
 @pytest.mark.parametrize("dtype", [torch.int32, torch.int64])
 @pytest.mark.parametrize("C,O", [(1, 64), (16, 16), (64, 5), (70, 33), (130, 8)])
-def test_conv_reference_sweep_vs_oracle(ops, oracle, dtype, C, O):
+def test_conv_reference_sweep_vs_oracle(ops, oracle, engine, dtype, C, O):
     """The reference's check_result sweep (filter x padding x stride on a 10x10 input, booloptests.py:113-124)."""
     D, S = 5, 10
     bits = torch.iinfo(dtype).bits
@@ -221,7 +230,7 @@ def test_conv_reference_sweep_vs_oracle(ops, oracle, dtype, C, O):
             np.testing.assert_array_equal(host(ops.conv_act_pack(xd, fd, td, *geom, pool=True)), pooled)
 
 
-def test_conv_rectangular_window_and_image(ops, oracle):
+def test_conv_rectangular_window_and_image(ops, oracle, engine):
     g = rng(8)
     D, H, W, Cw, O = 3, 9, 13, 2, 20
     x = rand_words(g, (D, H, W, Cw), np.int64)
@@ -367,7 +376,7 @@ def test_errors_match_the_reference_conventions(ops):
 @pytest.mark.parametrize("dtype", [torch.int64, torch.int32])
 @pytest.mark.parametrize("C,O,k,pad,stride", [(16, 16, 3, 1, 1), (3, 64, 3, 1, 1), (1, 5, 7, 2, 3), (8, 33, 5, 2, 2),
                                               (32, 20, 3, 0, 1), (16, 70, 1, 0, 1), (5, 16, 3, 2, 1), (2, 4, 9, 4, 1)])
-def test_conv_tap_packing_gives_the_same_sums(ops, oracle, dtype, C, O, k, pad, stride):
+def test_conv_tap_packing_gives_the_same_sums(ops, oracle, engine, dtype, C, O, k, pad, stride):
     """in_bits=C lets several filter taps share a word; every output must equal the one-word-per-tap path."""
     nd = NDT[dtype]
     bits = torch.iinfo(dtype).bits
@@ -407,3 +416,78 @@ def test_conv_tap_packing_gives_the_same_sums(ops, oracle, dtype, C, O, k, pad, 
         if h >= 2 and w >= 2:
             np.testing.assert_array_equal(host(ops.conv_act_pack(xd, fp, td, *geom, pool=True, **kw)),
                                           oracle.max_pool2d(packed, 2, 2, 0, 0, 2, 2))
+
+
+# (C, O, k, pad, H, W, tap-packed filter, kernel expected): one case per instantiation of the matrix-core kernel
+# (K chunks x channel tiles), ragged widths, channel counts that are not a multiple of 64, and shapes it must decline.
+MATRIX_CORE_CASES = [
+    (3, 64, 3, 1, 9, 20, True, True),      # 1 chunk, 4 channel tiles, 4-byte pixels
+    (3, 16, 3, 1, 12, 12, True, True),     # 1 chunk, 1 tile
+    (4, 16, 3, 0, 7, 33, False, True),     # in_bits known, one word per tap
+    (16, 16, 3, 1, 20, 18, True, True),    # 3 chunks, 1 tile (16 positions per pixel)
+    (16, 64, 3, 1, 10, 16, True, True),    # 3 chunks, 4 tiles
+    (16, 80, 3, 2, 6, 17, False, True),    # O = 80: last channel group ragged
+    (64, 64, 3, 1, 12, 21, False, True),   # 9 chunks, 4 tiles
+    (64, 144, 3, 1, 8, 8, False, True),    # three channel groups, last one 16 wide
+    (64, 16, 3, 1, 9, 31, False, True),    # 9 chunks, 1 tile
+    (50, 64, 3, 0, 9, 9, False, True),     # tail bits of the channel word are zero
+    (128, 32, 3, 1, 10, 12, False, True),  # 18 chunks, 2 tiles
+    (128, 96, 3, 1, 5, 16, False, True),
+    (64, 64, 1, 0, 6, 40, False, True),    # 1x1 filter
+    (8, 16, 5, 2, 9, 9, True, False),      # K = 200 positions: 4 chunks, no kernel -> XOR-popcount
+    (64, 24, 3, 1, 8, 8, False, False),    # O % 16 != 0
+    (192, 64, 3, 1, 8, 8, False, False),   # 27 chunks
+]
+
+
+@pytest.mark.parametrize("C,O,k,pad,H,W,tap,covered", MATRIX_CORE_CASES)
+def test_conv_matrix_core_engine_vs_oracle(ops, oracle, C, O, k, pad, H, W, tap, covered):
+    """Engine 2 on shapes chosen per kernel variant: int32 sums, packed and pooled outputs against the oracle,
+    and the engine that actually served the call."""
+    D = 3
+    g = rng(C * 1000 + O * 10 + k + H + W)
+    Cw = (C + 63) // 64
+    xb = g.integers(0, 2, size=(D * H * W, C)).astype(bool)
+    x = oracle.pack(xb, np.int64).reshape(D, H, W, Cw)
+    fb = g.integers(0, 2, size=(D * O * k * k, C)).astype(bool)
+    f = np.ascontiguousarray(oracle.pack(fb, np.int64).reshape(D, O, k, k, Cw).transpose(0, 2, 3, 4, 1)
+                             .reshape(D, -1, O))
+    K = k * k * C
+    thr = (g.integers(0, K + 1, size=(D, O)) - K // 2 + K).astype(np.int32)
+    thr[0, 0], thr[0, 1] = -5, 2 * K + 3                                   # always / never above the threshold
+    geom = (k, k, pad, pad, 1, 1)
+    xd, fd, td = dev(x), dev(f), dev(thr)
+    kw = {}
+    if C < 64:
+        kw = dict(in_bits=C)
+    if tap:
+        fd = ops.tap_pack_filter(fd, k * k, C)
+        kw["filter_tap_packed"] = True
+    want = oracle.conv(x, f, *geom)
+    act = oracle.conv_act(x, f, thr, *geom)
+    h, w = act.shape[1:3]
+    packed = oracle.pack(act.reshape(-1, O), np.int64).reshape(D, h, w, -1)
+    prev = ops.conv_engine(2)
+    try:
+        got = ops.conv(xd, fd, *geom, **kw)
+        assert ops.conv_last_engine() == (2 if covered else 1)
+        np.testing.assert_array_equal(host(got), want)
+        got = ops.conv_act_pack(xd, fd, td, *geom, **kw)
+        assert ops.conv_last_engine() == (2 if covered else 1)
+        np.testing.assert_array_equal(host(got), packed)
+        got = ops.conv_act_pack(xd, fd, td, *geom, pool=True, **kw)
+        np.testing.assert_array_equal(host(got), oracle.max_pool2d(packed, 2, 2, 0, 0, 2, 2))
+        np.testing.assert_array_equal(host(ops.conv_act(xd, fd, td, *geom, **kw)), act)   # bool output: popcount kernels
+        assert ops.conv_last_engine() == 1
+        ops.conv_engine(1)
+        ops.conv(xd, fd, *geom, **kw)
+        assert ops.conv_last_engine() == 1
+    finally:
+        ops.conv_engine(prev)
+
+
+def test_conv_engine_selector_round_trip(ops):
+    prev = ops.conv_engine()
+    assert prev in (0, 1, 2)
+    assert ops.conv_engine(2) == prev and ops.conv_engine(1) == 2 and ops.conv_engine(7) == 1 and ops.conv_engine() == 1
+    ops.conv_engine(prev)
