@@ -65,6 +65,29 @@ def time_steps(torch, step, steps, warmup):
     return wall / steps, e0.elapsed_time(e1) * 1e-3 / steps
 
 
+def config_entry(cfg, w, per_wall, per_ev):
+    """One line of other_configs.  A compute-shaped configuration is priced against three limits: HBM (algorithmic
+    bytes), the XOR-popcount issue rate of the vector ALUs and the dense int8 rate of the matrix cores (one +-1 byte
+    MAC per bit-MAC); `bound` names the limit that allows the least throughput for the engine that ran, and
+    `roofline_frac` is the fraction of that limit."""
+    from nesgpu_amd import workloads
+    from nesgpu_amd.extensions import booleanOperations as ops
+    entry = {"config": cfg, "workload": w.name, "ms_per_step": round(per_wall * 1e3, 4),
+             "binary_TOPS": round(2 * w.bit_macs / per_wall / 1e12, 3)}
+    hbm = w.algo_bytes / per_ev / workloads.HBM_PEAK
+    if w.bound == "hbm":
+        entry.update(bound="hbm", roofline_frac=round(hbm, 4))
+        return entry
+    valu = w.bit_macs / per_ev / workloads.VALU_POPC_PEAK
+    mfma = w.bit_macs / per_ev / workloads.MFMA_INT8_PEAK
+    engine = "matrixcore" if ops.conv_last_engine() == 2 else "popcount"
+    comp = mfma if engine == "matrixcore" else valu
+    entry.update(conv_engine=engine, bound="hbm" if hbm > comp else ("mfma" if engine == "matrixcore" else "valu"),
+                 roofline_frac=round(max(hbm, comp), 4), frac_of_hbm_peak=round(hbm, 4),
+                 frac_of_valu_popcount_peak=round(valu, 4), frac_of_int8_mfma_peak=round(mfma, 4))
+    return entry
+
+
 def cpu_baseline(wl, members, seconds):
     """Oracle (port) on the first `members` members of the headline workload; words regenerated on the host from
     the same Philox stream the GPU words came from."""
@@ -196,11 +219,9 @@ def main():
     if args.only:
         w = workloads.BUILDERS[args.only]()
         pw, pe = time_steps(torch, w.step, args.steps, args.warmup)
-        peak = workloads.HBM_PEAK if w.bound == "hbm" else workloads.VALU_POPC_PEAK
-        work = w.algo_bytes if w.bound == "hbm" else w.bit_macs
-        print(json.dumps({"config": args.only, "workload": w.name, "ms_per_step": round(pw * 1e3, 4),
-                          "event_ms_per_step": round(pe * 1e3, 4), "binary_TOPS": round(2 * w.bit_macs / pw / 1e12, 3),
-                          "bound": w.bound, "roofline_frac": round(work / pe / peak, 4)}))
+        entry = config_entry(args.only, w, pw, pe)
+        entry["event_ms_per_step"] = round(pe * 1e3, 4)
+        print(json.dumps(entry))
         return 0
 
     wl = workloads.linear_flip_fused()
@@ -233,12 +254,7 @@ def main():
         w = workloads.BUILDERS[cfg]()
         steps = max(3, args.steps // 2) if cfg == 5 else args.steps
         pw, pe = time_steps(torch, w.step, steps, args.warmup)
-        entry = {"config": cfg, "workload": w.name, "ms_per_step": round(pw * 1e3, 4),
-                 "binary_TOPS": round(2 * w.bit_macs / pw / 1e12, 3), "bound": w.bound}
-        if w.bound == "hbm":
-            entry["roofline_frac"] = round(w.algo_bytes / pe / workloads.HBM_PEAK, 4)
-        else:
-            entry["roofline_frac"] = round(w.bit_macs / pe / workloads.VALU_POPC_PEAK, 4)
+        entry = config_entry(cfg, w, pw, pe)
         others.append(entry)
         del w
         torch.cuda.empty_cache()

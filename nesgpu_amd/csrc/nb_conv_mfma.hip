@@ -39,7 +39,7 @@ struct MfmaConv {
     int CB;          // bytes (channel positions) per pixel, multiple of 4
     int PS;          // pixel stride in the LDS image, bytes
     int RW;          // pixels per LDS image row
-    int RIN;         // LDS image rows = h + fx - 1
+    int RIN;         // LDS image rows = hs + fx - 1
     int K;           // taps * CB
     int ntx;         // 16-pixel tiles per output row
     int frows;       // filter rows per member (words per output channel)
@@ -47,6 +47,7 @@ struct MfmaConv {
     int step_q, step_r;  // (waves*MT) / ntx and % ntx: tile advance of one step
     int pix_q, pix_r;    // threads / RW and % RW: image-pixel advance of one fill pass
     int taps, fy, tapT, in_bits;  // tapT > 1: tap-packed filter with in_bits channel bits per tap
+    int S, hs;  // a member's output rows are split over S workgroups, hs rows each (even when pooling)
 };
 
 // Per K position 64*kc + 16*lg + 4*d (index (kc*4 + lg)*4 + d), computed once per workgroup into LDS:
@@ -83,7 +84,9 @@ __global__ __launch_bounds__(kMfmaThreads) void conv_mfma_kernel(const MfmaConv 
 
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
     const int li = lane & 15, lg = lane >> 4;
-    const int64_t z = blockIdx.x;
+    const int64_t z = blockIdx.x / (unsigned)p.S;  // member
+    const int row0 = (int)(blockIdx.x - z * p.S) * p.hs;  // first output row of this workgroup
+    const int hloc = p.h - row0 < p.hs ? p.h - row0 : p.hs;  // its output rows
     const int Ow = (p.O + 63) >> 6;
 
     if (tid < 256)  // expansion table: entry b holds the +-1 bytes of bits 0..7 of b
@@ -142,7 +145,7 @@ __global__ __launch_bounds__(kMfmaThreads) void conv_mfma_kernel(const MfmaConv 
     // one pixel word per item, 8 items per thread loaded before any is expanded; (row, xx) advance incrementally
     {
         const uint64_t *src = p.in + z * (int64_t)p.H * p.Wd * p.Cw;
-        const int npix = p.RIN * p.RW;
+        const int npix = (hloc + p.RIN - p.hs) * p.RW;  // RIN = hs + fx - 1 rows at most
         const int row = tid / p.RW, xx = tid - row * p.RW;
         for (int cw = 0; cw < p.Cw; cw++) {
             const int nbits = p.CB - cw * 64 < 64 ? p.CB - cw * 64 : 64;  // positions held by this word
@@ -152,7 +155,7 @@ __global__ __launch_bounds__(kMfmaThreads) void conv_mfma_kernel(const MfmaConv 
                 uint64_t wd[U];
 #pragma unroll
                 for (int u = 0; u < U; u++) {
-                    const int yy = r0 - p.px, xs = x0 - p.py;
+                    const int yy = row0 + r0 - p.px, xs = x0 - p.py;
                     const bool inb = yy >= 0 && yy < p.H && xs >= 0 && xs < p.Wd;  // false past the last image row too
                     wd[u] = inb ? src[((int64_t)yy * p.Wd + xs) * p.Cw + cw] : 0ull;
                     r0 += p.pix_q;
@@ -190,7 +193,7 @@ __global__ __launch_bounds__(kMfmaThreads) void conv_mfma_kernel(const MfmaConv 
 #pragma unroll
         for (int d = 0; d < (PB16 ? 1 : 4); d++) koff[kc][d] = tab.koff[(kc * 4 + lg) * 4 + d];
 
-    const int mtiles = p.h * p.ntx;
+    const int mtiles = hloc * p.ntx;
     const int ngroups = (p.O + 16 * NT - 1) / (16 * NT);
     for (int cg = 0; cg < ngroups; cg++) {
         const int n0g = cg * 16 * NT;  // first channel of this group
@@ -315,7 +318,7 @@ __global__ __launch_bounds__(kMfmaThreads) void conv_mfma_kernel(const MfmaConv 
                     int32_t *o32 = static_cast<int32_t *>(p.out);
                     constexpr int LPP = 4 * NT;    // lanes per pixel, one int4 each
                     constexpr int PPI = 64 / LPP;  // pixels per store instruction
-                    int32_t *orow = o32 + ((z * p.h + ty[mt]) * (int64_t)p.w + tx[mt]) * p.O + n0g;
+                    int32_t *orow = o32 + ((z * p.h + row0 + ty[mt]) * (int64_t)p.w + tx[mt]) * p.O + n0g;
 #pragma unroll
                     for (int s = 0; s < 16 / PPI; s++) {
                         const int pi = s * PPI + lane / LPP, c4 = (lane % LPP) * 4;
@@ -355,23 +358,25 @@ __global__ __launch_bounds__(kMfmaThreads) void conv_mfma_kernel(const MfmaConv 
         const int lastv = p.O - 64 * (Ow - 1);
         const uint64_t lastmask = lastv >= 64 ? ~0ull : ((1ull << lastv) - 1);
         if (MODE == 2) {
-            const int total = p.h * p.w * Ow;
+            const int total = hloc * p.w * Ow;
+            uint64_t *dst = o64 + (z * p.h + row0) * (int64_t)p.w * Ow;
             int wi = tid % Ow;
             const int dwi = kMfmaThreads % Ow;
             for (int i = tid; i < total; i += kMfmaThreads) {
-                o64[z * (int64_t)total + i] = ob[i] & (wi == Ow - 1 ? lastmask : ~0ull);
+                dst[i] = ob[i] & (wi == Ow - 1 ? lastmask : ~0ull);
                 wi += dwi;
                 wi = wi >= Ow ? wi - Ow : wi;
             }
         } else {
-            const int h2 = p.h >> 1, w2 = p.w >> 1;
+            const int h2 = hloc >> 1, w2 = p.w >> 1;  // row0 is even: hs is
             const int total = h2 * w2 * Ow;
+            uint64_t *dst = o64 + (z * (p.h >> 1) + (row0 >> 1)) * (int64_t)w2 * Ow;
             for (int i = tid; i < total; i += kMfmaThreads) {
                 const int q = i / Ow, wi = i - q * Ow;
                 const int qy = q / w2, qx = q - qy * w2;
                 const int b0 = ((2 * qy) * p.w + 2 * qx) * Ow + wi;
                 const uint64_t v = ob[b0] | ob[b0 + Ow] | ob[b0 + p.w * Ow] | ob[b0 + p.w * Ow + Ow];
-                o64[z * (int64_t)total + i] = v & (wi == Ow - 1 ? lastmask : ~0ull);
+                dst[i] = v & (wi == Ow - 1 ? lastmask : ~0ull);
             }
         }
     }
@@ -393,7 +398,7 @@ static bool launch_one(const MfmaConv &p, int64_t D, size_t lds_bytes, hipStream
         }
         attr_set = true;
     }
-    kfn<<<dim3((unsigned)D), dim3(kMfmaThreads), lds_bytes, s>>>(p);
+    kfn<<<dim3((unsigned)(D * p.S)), dim3(kMfmaThreads), lds_bytes, s>>>(p);
     return true;
 }
 
@@ -447,7 +452,6 @@ bool conv_mfma_try(void *out, const uint64_t *in, const uint64_t *filt, const in
     p.PS = CB > 32 ? CB + 16 : CB;
     p.ntx = (g.w + 15) / 16;
     p.RW = round_up(16 * p.ntx + g.fy - 1, 4);
-    p.RIN = g.h + g.fx - 1;
     p.K = taps * CB;
     p.frows = filter_tap_packed ? (taps + tapT - 1) / tapT : taps * g.Cw;
     if (p.frows > 32767) return false;
@@ -470,14 +474,25 @@ bool conv_mfma_try(void *out, const uint64_t *in, const uint64_t *filt, const in
     p.fy = g.fy;
     p.tapT = tapT;
     p.in_bits = in_bits;
-    p.img_bytes = round_up(p.RIN * p.RW * p.PS + 64, 16);
     p.bfr_bytes = NK * NT * 1024;
     const int Ow = (O + 63) / 64;
     const int stage = waves * 16 * 16 * NT * 4;
     if (mode == 0 && p.bfr_bytes < stage) p.bfr_bytes = stage;
-    const int obuf = mode == 0 ? 0 : round_up(g.h * g.w * Ow * 8, 16);
-    const size_t lds = (size_t)kLutBytes + kTabBytes + p.img_bytes + p.bfr_bytes + obuf;
-    if (lds > 158 * 1024) return false;
+    // Kernels with few filter fragments need few registers, so several workgroups fit a CU and one's set-up
+    // overlaps another's MFMAs -- if their LDS footprints allow it: split a member's rows until a workgroup
+    // needs at most 48 KB (each part re-expands fx - 1 halo rows and rebuilds the small fragment set).
+    const int max_split = NK * NT <= 4 ? 8 : 1;
+    size_t lds = 0;
+    for (p.S = 1;; p.S++) {
+        p.hs = round_up((g.h + p.S - 1) / p.S, 2);
+        p.RIN = p.hs + g.fx - 1;
+        p.img_bytes = round_up(p.RIN * p.RW * p.PS + 64, 16);
+        const int obuf = mode == 0 ? 0 : round_up(p.hs * g.w * Ow * 8, 16);
+        lds = (size_t)kLutBytes + kTabBytes + p.img_bytes + p.bfr_bytes + obuf;
+        if (lds <= 48 * 1024 || p.S >= max_split || p.hs <= 8) break;
+    }
+    p.S = (g.h + p.hs - 1) / p.hs;  // parts that own at least one row
+    if (lds > 158 * 1024 || D * p.S > kMaxBlocks) return false;
     if (mode == 0) return launch_mode<0>(p, D, NK, NT, pb16, lds, s);
     if (mode == 2) return launch_mode<2>(p, D, NK, NT, pb16, lds, s);
     return launch_mode<3>(p, D, NK, NT, pb16, lds, s);
