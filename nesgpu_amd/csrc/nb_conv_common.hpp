@@ -76,6 +76,9 @@ void conv_tap_launch(void *out, const W *in, const W *filt, const int32_t *thres
 bool conv_mfma_try(void *out, const uint64_t *in, const uint64_t *filt, const int32_t *thresh, const ConvGeom &g,
                    int64_t D, int O, int in_bits, bool filter_tap_packed, int mode, bool force, hipStream_t s);
 
+bool conv_rw_try(void *out, const uint64_t *in, const uint64_t *filt, const int32_t *thresh, const ConvGeom &g,
+                 int64_t D, int O, int tap_bits, int mode, hipStream_t s);
+
 inline int taps_per_word(int bits, int tap_bits) { return bits / tap_bits; }
 
 }  // namespace nb
