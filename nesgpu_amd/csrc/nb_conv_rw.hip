@@ -34,7 +34,7 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 
 constexpr int kRwThreads = 256;
 constexpr int kRwWaves = kRwThreads / 64;
-constexpr int kRwLutBytes = 257 * 8 + 8;  // byte -> 8 bytes of +-1, entry 256 -> zeros
+constexpr int kRwLutBytes = 256;  // 4 bits -> 4 bytes of +-1, four interleaved copies
 constexpr int kRwMaxCPR = 6;
 constexpr int kRwTabBytes = 3 * kRwMaxCPR * 4 * 8;  // (chunk, lane group) -> filter word offset, shift, mask
 
@@ -49,6 +49,8 @@ struct RwConv {
     int RW;            // pixels per LDS image row
     int hs, S;         // output rows per band, bands per member
     int hb, nsub;      // output rows per sub-band (even), sub-bands per band
+    int cgl, ngw;      // channel groups per workgroup, workgroups per band
+    int bst_off;       // LDS offset of the filter-fragment staging area (the image area itself when cgl == 1)
     int ntx, ncg;      // 16-column strips, channel groups of 16*NT
     int K;             // expanded positions that count: taps * CB
     int in_bits;       // valid channel bits per pixel
@@ -82,7 +84,6 @@ __global__ __launch_bounds__(kRwThreads, 2) void conv_rw_kernel(const RwConv p)
     constexpr int FX = 3;
     constexpr int NK = FX * CPR;
     extern __shared__ __align__(16) unsigned char lds[];
-    const uint2 *lut = reinterpret_cast<const uint2 *>(lds);
     unsigned char *img = lds + kRwLutBytes + kRwTabBytes;
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -90,16 +91,28 @@ __global__ __launch_bounds__(kRwThreads, 2) void conv_rw_kernel(const RwConv p)
     // MFMA ignores EXEC and a masked-off block that is not jumped over would still accumulate.
     const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int li = lane & 15, lg = lane >> 4;
-    const int64_t z = blockIdx.x / (unsigned)p.S;               // member
-    const int row0 = (int)(blockIdx.x - z * p.S) * p.hs;        // first output row of this band
+    // workgroup = (member, band of rows, set of cgl channel groups), channel groups fastest
+    const unsigned zb = blockIdx.x / (unsigned)p.ngw;
+    const int cg0 = (int)(blockIdx.x - zb * p.ngw) * p.cgl;
+    const int cg1 = cg0 + p.cgl < p.ncg ? cg0 + p.cgl : p.ncg;
+    const int64_t z = zb / (unsigned)p.S;                       // member
+    const int row0 = (int)(zb - (unsigned)z * p.S) * p.hs;      // first output row of this band
     const int hloc = p.h - row0 < p.hs ? p.h - row0 : p.hs;     // its output rows
     const int Ow = (p.O + 63) >> 6;
-    const int upc = p.ntx * p.nsub;                             // units per channel group
-    const int nunits = p.ncg * upc;
+    const int nunits = p.ntx * p.nsub;                          // (strip, sub-band) units for the four waves
 
-    // expansion table: entry b holds the +-1 bytes of bits 0..7 of b; entry 256 is eight zero bytes
-    reinterpret_cast<uint2 *>(lds)[tid] = make_uint2(rw_pm1_bytes(tid & 0xFu), rw_pm1_bytes((unsigned)tid >> 4));
-    if (tid == 0) reinterpret_cast<uint2 *>(lds)[256] = make_uint2(0u, 0u);
+    // Expansion table: dword 4*n + c (c = 0..3) holds the +-1 bytes of the four bits of n.  A lane always reads copy
+    // c = lane % 4, so every address a wave asks for sits in a bank of its own: the look-ups never conflict.
+    if (tid < 64) reinterpret_cast<uint32_t *>(lds)[tid] = rw_pm1_bytes((unsigned)tid >> 2);
+    const unsigned char *lut = lds + (lane & 3) * 4;
+    auto expand16 = [&](uint32_t h16) {  // 16 bits -> 16 bytes of +-1, bit b -> byte b
+        uint4 r;
+        r.x = *reinterpret_cast<const uint32_t *>(lut + ((h16 & 0xFu) << 4));
+        r.y = *reinterpret_cast<const uint32_t *>(lut + (((h16 >> 4) & 0xFu) << 4));
+        r.z = *reinterpret_cast<const uint32_t *>(lut + (((h16 >> 8) & 0xFu) << 4));
+        r.w = *reinterpret_cast<const uint32_t *>(lut + (((h16 >> 12) & 0xFu) << 4));
+        return r;
+    };
 
     // ---- fragment geometry ---------------------------------------------------------------------------------
     // chunk kq = i*CPR + q (filter row i) and lane group g: tap column j, first position c0.  Table entry:
@@ -143,120 +156,140 @@ __global__ __launch_bounds__(kRwThreads, 2) void conv_rw_kernel(const RwConv p)
     }
     __syncthreads();  // tables complete
 
-    // Filter words of one channel group, requested early so that their latency hides behind the image fill.  Every
-    // address is valid (channels past O read channel O-1, dead tap columns word 0); the expansion zeroes them.
-    const unsigned char *fz = reinterpret_cast<const unsigned char *>(
-        p.filt + z * (int64_t)p.fwords);
-    uint64_t fw[NK][NT];
-    auto load_filter = [&](int n0) {
-        uint32_t chb[NT];
+    // The four waves build a channel group's NK*NT filter fragments together: wave w takes fragments w, w+4, ...
+    // (fragment f = chunk f/NT, channel tile f%NT) from global memory, expands them into the staging area, and
+    // after a barrier every wave copies all of them into registers.  Every address is valid (channels past O read
+    // channel O-1, dead tap columns word 0); the expansion zeroes them.
+    constexpr int NF = NK * NT, FPW = (NF + kRwWaves - 1) / kRwWaves;
+    const unsigned char *fz = reinterpret_cast<const unsigned char *>(p.filt + z * (int64_t)p.fwords);
+    unsigned char *bst = lds + p.bst_off;
+    uint64_t fw[FPW];
+    int traw[NT];
+    auto request_filter = [&](int n0) {
 #pragma unroll
-        for (int nt = 0; nt < NT; nt++) {
+        for (int t = 0; t < FPW; t++) {
+            const int f = wv + kRwWaves * t;  // uniform
+            const int kq = f < NF ? f / NT : 0, nt = f < NF ? f - kq * NT : 0;
             const int ch = n0 + nt * 16 + li;
-            chb[nt] = (uint32_t)(ch < p.O ? ch : p.O - 1) * 8u;
+            fw[t] = *reinterpret_cast<const uint64_t *>(fz + (tab[kq * 4 + lg].x + (uint32_t)(ch < p.O ? ch : p.O - 1) * 8u));
         }
-#pragma unroll
-        for (int kq = 0; kq < NK; kq++) {
-            const uint32_t off = tab[kq * 4 + lg].x;
-#pragma unroll
-            for (int nt = 0; nt < NT; nt++) fw[kq][nt] = *reinterpret_cast<const uint64_t *>(fz + (off + chb[nt]));
-        }
-    };
-    int cur_cg = wv < nunits ? wv / upc : -1;  // channel group whose fragments the wave holds
-    if (cur_cg >= 0) load_filter(cur_cg * 16 * NT);
-
-    // ---- phase 1: expand the band's input rows (with border) into LDS ------------------------------------------
-    // one pixel word per item, U items per thread loaded before any is expanded; (row, column, offset) advance
-    // incrementally; an out-of-range pixel reads word 0 of the member and is replaced by the zero word
-    {
-        const unsigned char *src = reinterpret_cast<const unsigned char *>(p.in + z * (int64_t)p.H * p.Wd * p.Cw);
-        const int npix = (hloc + FX - 1) * p.RW;
-        const int row = tid / p.RW, xx = tid - row * p.RW;
-        const int pixb = p.Cw * 8, rowb = p.Wd * pixb;                          // bytes per pixel / image row
-        const int stepb = p.pix_q * rowb + p.pix_r * pixb, wrapb = rowb - p.RW * pixb;
-        for (int cw = 0; cw < p.Cw; cw++) {
-            const int nbytes = p.CB - cw * 64 < 64 ? p.CB - cw * 64 : 64;  // positions held by this word
-            int yy = row0 + row - p.px, xs = xx - p.py;
-            const int xend = p.RW - p.py;
-            int off = yy * rowb + xs * pixb + cw * 8;
-            unsigned char *dst = img + __mul24(tid, p.PS) + cw * 64;
-            const int dstep = kRwThreads * p.PS;
-            constexpr int U = 8;
-            for (int pix0 = tid; pix0 < npix; pix0 += kRwThreads * U) {
-                uint64_t wd[U];
-#pragma unroll
-                for (int u = 0; u < U; u++) {
-                    const bool inb = yy >= 0 && yy < p.H && xs >= 0 && xs < p.Wd;  // false past the last image row too
-                    const uint64_t v = *reinterpret_cast<const uint64_t *>(src + (uint32_t)(inb ? off : 0));
-                    wd[u] = inb ? v : 0ull;
-                    yy += p.pix_q;
-                    xs += p.pix_r;
-                    off += stepb;
-                    if (xs >= xend) {
-                        xs -= p.RW;
-                        yy++;
-                        off += wrapb;
-                    }
-                }
-#pragma unroll
-                for (int u = 0; u < U; u++) {
-                    if (pix0 + u * kRwThreads < npix) {
-                        for (int c = 0; c < nbytes; c += 16) {
-                            const uint2 lo = lut[(uint32_t)(wd[u] >> c) & 0xFFu];
-                            const uint2 hi = lut[(uint32_t)(wd[u] >> (c + 8)) & 0xFFu];
-                            *reinterpret_cast<uint4 *>(dst + c) = make_uint4(lo.x, lo.y, hi.x, hi.y);
-                        }
-                    }
-                    dst += dstep;
-                }
-            }
-        }
-    }
-    __syncthreads();  // image complete
-
-    v4i B[NK][NT];
-    int tdot[NT];
-    // expand the loaded filter words of a channel group into register fragments, fetch its thresholds
-    auto expand_filter = [&](int n0) {
-        bool chlive[NT];
-#pragma unroll
-        for (int nt = 0; nt < NT; nt++) chlive[nt] = n0 + nt * 16 + li < p.O;
-#pragma unroll
-        for (int kq = 0; kq < NK; kq++) {
-            const uint32_t e = tab[kq * 4 + lg].y;
-            const uint32_t sh = e & 63u, vmask = (e >> 8) & 0xFFFFu;
-            const bool inside = (int)e < 0;
-#pragma unroll
-            for (int nt = 0; nt < NT; nt++) {
-                const bool live = inside && chlive[nt];
-                const uint32_t h16 = (uint32_t)(fw[kq][nt] >> sh) & vmask;
-                const uint2 lo = lut[live ? (h16 & 0xFFu) : 256u], hi = lut[live ? (h16 >> 8) : 256u];
-                B[kq][nt] = (v4i){(int)lo.x, (int)lo.y, (int)hi.x, (int)hi.y};
-            }
-        }
-        // thresholds in dot-product terms: 2*popc > t  <=>  popc > (t>>1)  <=>  dot < K - 2*(t>>1)
         if (MODE != 0) {
 #pragma unroll
             for (int nt = 0; nt < NT; nt++) {
                 const int ch = n0 + nt * 16 + li;
-                int64_t td = ch < p.O ? (int64_t)p.K - 2 * (int64_t)(p.thresh[z * p.O + ch] >> 1) : -2147483648LL;
+                traw[nt] = p.thresh[z * p.O + (ch < p.O ? ch : p.O - 1)];
+            }
+        }
+    };
+    auto stage_filter = [&](int n0) {
+#pragma unroll
+        for (int t = 0; t < FPW; t++) {
+            const int f = wv + kRwWaves * t;
+            if (f < NF) {  // uniform
+                const int kq = f / NT, nt = f - kq * NT;
+                const uint32_t e = tab[kq * 4 + lg].y;
+                const uint32_t sh = e & 63u, vmask = (e >> 8) & 0xFFFFu;
+                const bool live = (int)e < 0 && n0 + nt * 16 + li < p.O;
+                const uint32_t h16 = (uint32_t)(fw[t] >> sh) & vmask;
+                const uint4 e16 = expand16(h16);
+                *reinterpret_cast<uint4 *>(bst + (f * 64 + lane) * 16) =
+                    live ? e16 : make_uint4(0u, 0u, 0u, 0u);
+            }
+        }
+    };
+    v4i B[NK][NT];
+    int tdot[NT];
+    auto fetch_fragments = [&](int n0) {
+#pragma unroll
+        for (int kq = 0; kq < NK; kq++)
+#pragma unroll
+            for (int nt = 0; nt < NT; nt++)
+                B[kq][nt] = *reinterpret_cast<const v4i *>(bst + ((kq * NT + nt) * 64 + lane) * 16);
+        // thresholds in dot-product terms: 2*popc > t  <=>  popc > (t>>1)  <=>  dot < K - 2*(t>>1)
+        if (MODE != 0) {
+#pragma unroll
+            for (int nt = 0; nt < NT; nt++) {
+                int64_t td = n0 + nt * 16 + li < p.O ? (int64_t)p.K - 2 * (int64_t)(traw[nt] >> 1) : -2147483648LL;
                 td = td > 2147483647LL ? 2147483647LL : (td < -2147483648LL ? -2147483648LL : td);
                 tdot[nt] = (int)td;
             }
         }
     };
-    if (cur_cg >= 0) expand_filter(cur_cg * 16 * NT);
+    request_filter(cg0 * 16 * NT);
+
+    // ---- phase 1: request the band's input words (with border) --------------------------------------------------
+    // one pixel word per item, up to U items per thread in flight; (row, column, offset) advance incrementally; an
+    // out-of-range pixel reads word 0 of the member and is replaced by the zero word
+    const unsigned char *src = reinterpret_cast<const unsigned char *>(p.in + z * (int64_t)p.H * p.Wd * p.Cw);
+    const int npix = (hloc + FX - 1) * p.RW;
+    const int pixb = p.Cw * 8, rowb = p.Wd * pixb;                          // bytes per pixel / image row
+    const int stepb = p.pix_q * rowb + p.pix_r * pixb, wrapb = rowb - p.RW * pixb;
+    const int xend = p.RW - p.py;
+    constexpr int U = 8;
+    int yy, xs, off;  // running position of the thread's next item
+    {
+        const int row = tid / p.RW, xx = tid - row * p.RW;
+        yy = row0 + row - p.px;
+        xs = xx - p.py;
+        off = yy * rowb + xs * pixb;
+    }
+    uint64_t wd[U];
+    auto load_items = [&](int cw8) {
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const bool inb = yy >= 0 && yy < p.H && xs >= 0 && xs < p.Wd;  // false past the last image row too
+            const uint64_t v = *reinterpret_cast<const uint64_t *>(src + (uint32_t)(inb ? off + cw8 : 0));
+            wd[u] = inb ? v : 0ull;
+            yy += p.pix_q;
+            xs += p.pix_r;
+            off += stepb;
+            if (xs >= xend) {
+                xs -= p.RW;
+                yy++;
+                off += wrapb;
+            }
+        }
+    };
+    load_items(0);
+
+    // ---- phase 2: first channel group's fragments (staged over the still empty image area when cgl == 1) ---------
+    stage_filter(cg0 * 16 * NT);
+    __syncthreads();  // fragments complete
+    fetch_fragments(cg0 * 16 * NT);
+    __syncthreads();  // fragments in registers: the area is free again
+
+    // ---- phase 3: expand the input words into +-1 bytes in LDS -----------------------------------------------------
+    for (int cw = 0; cw < p.Cw; cw++) {
+        const int nbytes = p.CB - cw * 64 < 64 ? p.CB - cw * 64 : 64;  // positions held by this word
+        unsigned char *dst = img + __mul24(tid, p.PS) + cw * 64;
+        const int dstep = kRwThreads * p.PS;
+        for (int pix0 = tid; pix0 < npix; pix0 += kRwThreads * U) {
+            if (pix0 != tid || cw != 0) load_items(cw * 8);
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                if (pix0 + u * kRwThreads < npix) {
+                    for (int c = 0; c < nbytes; c += 16) {
+                        *reinterpret_cast<uint4 *>(dst + c) = expand16((uint32_t)(wd[u] >> c) & 0xFFFFu);
+                    }
+                }
+                dst += dstep;
+            }
+        }
+        if (cw + 1 < p.Cw) {  // rewind to the thread's first item for the next channel word
+            const int row = tid / p.RW, xx = tid - row * p.RW;
+            yy = row0 + row - p.px;
+            xs = xx - p.py;
+            off = yy * rowb + xs * pixb;
+        }
+    }
+    __syncthreads();  // image complete
+
     int *stage = reinterpret_cast<int *>(img + p.img_bytes) + wv * (16 * 16 * NT);  // MODE 0 only
 
+    for (int cg = cg0;;) {
+    const int n0 = cg * 16 * NT;  // first channel of the group
     for (int u = wv; u < nunits; u += kRwWaves) {
-        const int cg = u / upc, rem = u - cg * upc;
-        const int sub = rem / p.ntx, strip = rem - sub * p.ntx;
-        const int n0 = cg * 16 * NT;
-        if (cg != cur_cg) {  // wave-uniform
-            load_filter(n0);
-            expand_filter(n0);
-            cur_cg = cg;
-        }
+        const int sub = u / p.ntx, strip = u - sub * p.ntx;
         const int ys = sub * p.hb;
         const int ye = ys + p.hb < hloc ? ys + p.hb : hloc;
         if (ys >= ye) continue;  // wave-uniform
@@ -446,6 +479,14 @@ __global__ __launch_bounds__(kRwThreads, 2) void conv_rw_kernel(const RwConv p)
         }
         for (; rr < rend; rr++) edge_step(rr);
     }
+    if (++cg >= cg1) break;
+    // next channel group: no wave reads the staging area during a walk, so a wave that is done starts at once
+    request_filter(cg * 16 * NT);
+    stage_filter(cg * 16 * NT);
+    __syncthreads();
+    fetch_fragments(cg * 16 * NT);
+    __syncthreads();  // a fast wave must not restage while a slow one still fetches
+    }
 }
 
 static inline int rw_round_up(int a, int b) { return (a + b - 1) / b * b; }
@@ -463,7 +504,7 @@ static bool rw_launch_one(const RwConv &p, int64_t D, size_t lds_bytes, hipStrea
         }
         attr_set = true;
     }
-    kfn<<<dim3((unsigned)(D * p.S)), dim3(kRwThreads), lds_bytes, s>>>(p);
+    kfn<<<dim3((unsigned)(D * p.S * p.ngw)), dim3(kRwThreads), lds_bytes, s>>>(p);
     return true;
 }
 
@@ -544,21 +585,45 @@ bool conv_rw_try(void *out, const uint64_t *in, const uint64_t *filt, const int3
     p.pix_q = kRwThreads / p.RW;
     p.pix_r = kRwThreads % p.RW;
     // Bands: as few as keep a workgroup's LDS at or below 78 KB (two workgroups per CU), rows per band even.
+    // The NK*NT filter fragments (1 KB each) are staged in LDS on their way to the registers.  With one channel
+    // group they borrow the image area before the image is written.  With several, a workgroup walks all groups
+    // over one expanded image if a separate staging area fits (bands of at least 8 rows); otherwise every channel
+    // group gets workgroups of its own, each expanding the image again.
     const int stage = mode == 0 ? kRwWaves * 16 * 16 * NT * 4 : 0;
     const int rowbytes = p.RW * p.PS;
+    const int frag_bytes = 3 * CPR * NT * 1024;
+    const size_t fixed = (size_t)kRwLutBytes + kRwTabBytes + stage, budget = 78 * 1024;
     size_t lds = 0;
+    p.cgl = 0;
     for (p.S = 1;; p.S++) {
         p.hs = rw_round_up((g.h + p.S - 1) / p.S, 2);
-        p.img_bytes = rw_round_up((p.hs + 2) * rowbytes + 64, 16);
-        lds = (size_t)kRwLutBytes + kRwTabBytes + p.img_bytes + stage;
-        if (lds <= 78 * 1024 || p.hs <= 2) break;
+        const int img = rw_round_up((p.hs + 2) * rowbytes + 64, 16);
+        if (p.ncg > 1 && fixed + img + frag_bytes <= budget && (p.hs >= 8 || p.S == 1)) {
+            p.cgl = p.ncg;
+            p.img_bytes = img;
+            p.bst_off = (int)(fixed + img);
+            lds = fixed + img + frag_bytes;
+            break;
+        }
+        if (p.hs <= 2 || (p.ncg > 1 && p.hs < 8)) break;
+    }
+    if (p.cgl == 0) {
+        for (p.S = 1;; p.S++) {
+            p.hs = rw_round_up((g.h + p.S - 1) / p.S, 2);
+            p.img_bytes = rw_round_up((p.hs + 2) * rowbytes + 64, 16);
+            if (p.img_bytes < frag_bytes) p.img_bytes = frag_bytes;
+            lds = fixed + p.img_bytes;
+            if (lds <= budget || p.hs <= 2) break;
+        }
+        p.cgl = 1;
+        p.bst_off = kRwLutBytes + kRwTabBytes;  // the image area
     }
     if (lds > 158 * 1024) return false;
+    p.ngw = (p.ncg + p.cgl - 1) / p.cgl;
     p.S = (g.h + p.hs - 1) / p.hs;  // bands that own at least one row
-    if (D * p.S > kMaxBlocks) return false;
-    // Sub-bands: enough units (channel group x strip x sub-band) for the four waves of a workgroup.
-    const int base_units = p.ncg * p.ntx;
-    int nsub = base_units >= kRwWaves ? 1 : (kRwWaves + base_units - 1) / base_units;
+    if (D * p.S * p.ngw > kMaxBlocks) return false;
+    // Sub-bands: enough (strip, sub-band) units for the four waves of a workgroup.
+    int nsub = p.ntx >= kRwWaves ? 1 : (kRwWaves + p.ntx - 1) / p.ntx;
     p.hb = rw_round_up((p.hs + nsub - 1) / nsub, 2);
     p.nsub = (p.hs + p.hb - 1) / p.hb;
     if (mode == 0) return rw_launch_mode<0>(p, D, CPR, NT, lds, s);
