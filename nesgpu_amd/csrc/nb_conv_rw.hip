@@ -1,4 +1,4 @@
-// Binary conv on the int8 matrix cores, row-walking variant (3-row filters, stride 1).
+// Binary conv on the int8 matrix cores (3-row filters, stride 1): a persistent producer / consumer kernel.
 //
 // CDNA4 has no 1-bit MFMA, but v_mfma_i32_16x16x64_i8 does 16384 int8 MACs per wave in 16 cycles: 4x the
 // bit-MAC rate of v_xor + v_bcnt.  Bits are expanded to +-1 bytes (bit 1 -> +1, bit 0 -> -1; an out-of-range
@@ -6,16 +6,22 @@
 //     popcount(x ^ w) = (K - dot) / 2
 // gives back the reference's sum bit for bit.
 //
-// Work split.  A workgroup owns a band of output rows of one member; the band's input rows (with the zero-word
-// border, so the implicit im2col needs no bounds checks) are expanded once into LDS.  A wave owns a strip of 16
-// output columns, 16*NT output channels and a sub-band of rows.  It builds its filter fragments straight from
-// global memory into registers (no LDS staging) and then walks DOWN the strip: the A fragment of image row r and
-// tap column j is the same 16 pixels x 64 positions whichever filter row it meets, so it is read from LDS once
-// and multiplied into the three output rows r, r-1, r-2 that are live in a ring of three accumulator sets.  One
-// ds_read_b128 therefore feeds 3*NT MFMAs and the LDS pipe stays far from its limit even for 16 channels.
-// Finished rows leave through the epilogue straight to global memory: int32 sums via a per-wave LDS transpose
-// (full pixel rows, non-temporal), or threshold bits gathered with ballots into packed words, optionally
-// 2x2 OR-pooled (pooling in x is a min over neighbouring accumulator registers, in y over two walked rows).
+// One workgroup of eight waves per CU walks through its share of the population.  A task is a band of output
+// rows of one member for one group of 16*NT output channels.  Waves 4..7 (producers) prepare task k while waves
+// 0..3 (consumers) multiply task k-1, one barrier per step:
+//   producer: the band's input words and, when the (member, channel group) changes, the filter words were
+//     requested one step ahead; it expands the input rows (with the zero-word border, so the implicit im2col
+//     needs no bounds checks) into one of two LDS image buffers and the filter words into MFMA B fragments in an
+//     LDS staging area, then requests the words of task k+1;
+//   consumer: copies new fragments into registers (they stay there for all bands of the member), then every
+//     wave walks DOWN a strip of 16 output columns: the A fragment of image row r and tap column j is the same
+//     16 pixels x 64 positions whichever filter row it meets, so it is read from LDS once and multiplied into
+//     the three output rows r, r-1, r-2.  One ds_read_b128 feeds 3*NT MFMAs.  Finished rows leave straight to
+//     global memory: int32 sums via a per-wave LDS transpose (full pixel rows, non-temporal), or threshold bits
+//     gathered with ballots into packed words, optionally 2x2 OR-pooled (in x a min over neighbouring
+//     accumulator registers, in y over two walked rows).
+// Each SIMD holds one consumer and one producer wave, so the expansion work (VALU, LDS, memory latency) runs in
+// the shadow of the MFMAs instead of in front of them.
 //
 // Fragment layout of v_mfma_i32_16x16x64_i8 (checked on hardware): lane l supplies row l%16 of A and
 // column l%16 of B, its 16 bytes are the K-positions 16*(l/16)..+15 of the 64-chunk (any bijection works as
@@ -32,32 +38,38 @@ namespace nb {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 
-constexpr int kRwThreads = 256;
-constexpr int kRwWaves = kRwThreads / 64;
-constexpr int kRwLutBytes = 256;  // 4 bits -> 4 bytes of +-1, four interleaved copies
+constexpr int kRwCWaves = 8;      // consumer waves: two per SIMD keep the matrix core issuing back to back
+constexpr int kRwPWaves = 4;      // producer waves
+constexpr int kRwThreads = 64 * (kRwCWaves + kRwPWaves);
+constexpr int kRwTeam = 64 * kRwPWaves;  // producer threads
+constexpr int kRwLutBytes = 256 * 8;  // byte -> 8 bytes of +-1
 constexpr int kRwMaxCPR = 6;
 constexpr int kRwTabBytes = 3 * kRwMaxCPR * 4 * 8;  // (chunk, lane group) -> filter word offset, shift, mask
+// dynamic LDS a launch may ask for: the CU's 160 KB minus the kernel's two static tables
+constexpr int kRwMaxDynLds = 160 * 1024 - kRwLutBytes - kRwTabBytes - 512;
+constexpr int kRwItems = 10;      // input words a producer thread holds in flight
 
 struct RwConv {
     const uint64_t *in;
     const uint64_t *filt;
     const int32_t *thresh;
     void *out;
+    int64_t D;
     int H, Wd, Cw, px, py, h, w, O, fy;
     int CB;            // expanded bytes per pixel: 16, 32 or 64*Cw
     int PS;            // pixel stride in the LDS image, bytes (PS/16 odd: conflict-free 16-lane b128 reads)
     int RW;            // pixels per LDS image row
     int hs, S;         // output rows per band, bands per member
     int hb, nsub;      // output rows per sub-band (even), sub-bands per band
-    int cgl, ngw;      // channel groups per workgroup, workgroups per band
-    int bst_off;       // LDS offset of the filter-fragment staging area (the image area itself when cgl == 1)
-    int ntx, ncg;      // 16-column strips, channel groups of 16*NT
+    int ntx, ncg;      // 16-column strips, channel groups (of 16*NT*cgt channels) = tasks per band
+    int cgt;           // consumer channel tiles (of 16*NT channels) per task: 1, 2 or 4
     int K;             // expanded positions that count: taps * CB
     int in_bits;       // valid channel bits per pixel
     int tapT, tapM;    // tap-packed filter: taps per word and ceil(65536 / tapT) + 1 (0: one word per tap and channel word)
-    int img_bytes;
+    int img_bytes;     // one image buffer
+    int nbst;          // fragment staging areas (2 when every task brings new fragments)
     int fwords;        // filter words per member
-    int pix_q, pix_r;  // threads / RW and % RW: image-pixel advance of one fill pass
+    int pix_q, pix_r;  // team threads / RW and % RW: image-pixel advance of one fill pass
     short qj[kRwMaxCPR];  // chunk q of a filter row: first tap column ...
     short qc[kRwMaxCPR];  // ... and first position inside the pixel
     int jsh, cmask;    // lane group g adds (g >> jsh) tap columns and 16 * (g & cmask) positions
@@ -77,41 +89,63 @@ __device__ __forceinline__ uint64_t rw_sel4(int r, uint64_t a, uint64_t b, uint6
     return r == 0 ? a : r == 1 ? b : r == 2 ? c : d;
 }
 
+// Position of a workgroup in its task sequence: members blockIdx.x, blockIdx.x + gridDim.x, ...; per member the
+// channel groups, per channel group the bands.
+struct RwTask {
+    int64_t z;
+    int cg, band;
+};
+__device__ __forceinline__ void rw_next(RwTask &t, const RwConv &p)
+{
+    if (++t.band == p.S) {
+        t.band = 0;
+        if (++t.cg == p.ncg) {
+            t.cg = 0;
+            t.z += gridDim.x;
+        }
+    }
+}
+
 // MODE 0: int32 popcount sums [D,h,w,O]; 2: threshold bits packed along O; 3: the same, 2x2 OR-pooled.
 template <int CPR, int NT, int MODE>
-__global__ __launch_bounds__(kRwThreads, 2) void conv_rw_kernel(const RwConv p)
+__global__ __launch_bounds__(kRwThreads) void conv_rw_kernel(const RwConv p)
 {
     constexpr int FX = 3;
     constexpr int NK = FX * CPR;
+    constexpr int NF = NK * NT;                  // fragments of one consumer channel tile
+    constexpr int CGTMAX = 4 / NT;               // a task covers at most 64 channels
+    constexpr int FPW = (NF * CGTMAX + kRwPWaves - 1) / kRwPWaves;  // fragments per producer wave, at most
+    constexpr int kFragBytes = NF * CGTMAX * 1024 + 64 * 4;         // + the task's thresholds
+    // The two small tables are objects of their own, so that the compiler knows that the stores into the image and
+    // staging buffers never alias the table look-ups and can keep many look-ups in flight.
+    __shared__ __align__(16) uint2 lut_s[kRwLutBytes / 8];
+    __shared__ __align__(16) uint2 tab[kRwTabBytes / 8];
     extern __shared__ __align__(16) unsigned char lds[];
-    unsigned char *img = lds + kRwLutBytes + kRwTabBytes;
+    unsigned char *img0 = lds;
+    unsigned char *bst0 = img0 + 2 * p.img_bytes;
+    int *stage0 = reinterpret_cast<int *>(bst0 + p.nbst * kFragBytes);  // MODE 0 only
 
     const int tid = threadIdx.x, lane = tid & 63;
     // The wave index must be visibly uniform: every branch around MFMAs below has to be a scalar branch, because
     // MFMA ignores EXEC and a masked-off block that is not jumped over would still accumulate.
     const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const bool producer = wv >= kRwCWaves;
+    const int tw = producer ? wv - kRwCWaves : wv;            // wave inside the team
+    const int ttid = tid - (producer ? 64 * kRwCWaves : 0);   // thread inside the team
     const int li = lane & 15, lg = lane >> 4;
-    // workgroup = (member, band of rows, set of cgl channel groups), channel groups fastest
-    const unsigned zb = blockIdx.x / (unsigned)p.ngw;
-    const int cg0 = (int)(blockIdx.x - zb * p.ngw) * p.cgl;
-    const int cg1 = cg0 + p.cgl < p.ncg ? cg0 + p.cgl : p.ncg;
-    const int64_t z = zb / (unsigned)p.S;                       // member
-    const int row0 = (int)(zb - (unsigned)z * p.S) * p.hs;      // first output row of this band
-    const int hloc = p.h - row0 < p.hs ? p.h - row0 : p.hs;     // its output rows
     const int Ow = (p.O + 63) >> 6;
-    const int nunits = p.ntx * p.nsub;                          // (strip, sub-band) units for the four waves
 
-    // Expansion table: dword 4*n + c (c = 0..3) holds the +-1 bytes of the four bits of n.  A lane always reads copy
-    // c = lane % 4, so every address a wave asks for sits in a bank of its own: the look-ups never conflict.
-    if (tid < 64) reinterpret_cast<uint32_t *>(lds)[tid] = rw_pm1_bytes((unsigned)tid >> 2);
-    const unsigned char *lut = lds + (lane & 3) * 4;
-    auto expand16 = [&](uint32_t h16) {  // 16 bits -> 16 bytes of +-1, bit b -> byte b
-        uint4 r;
-        r.x = *reinterpret_cast<const uint32_t *>(lut + ((h16 & 0xFu) << 4));
-        r.y = *reinterpret_cast<const uint32_t *>(lut + (((h16 >> 4) & 0xFu) << 4));
-        r.z = *reinterpret_cast<const uint32_t *>(lut + (((h16 >> 8) & 0xFu) << 4));
-        r.w = *reinterpret_cast<const uint32_t *>(lut + (((h16 >> 12) & 0xFu) << 4));
-        return r;
+    // Expansion table: entry b holds the +-1 bytes of bits 0..7 of b.  The expansion work shares the SIMDs' issue
+    // slots with the MFMAs, so it is written for the fewest instructions: two ALU operations and one 8-byte look-up
+    // per 8 bits (bank conflicts between look-ups cost LDS time, which is plentiful, not issue slots).
+    if (tid < 256) lut_s[tid] = make_uint2(rw_pm1_bytes(tid & 0xFu), rw_pm1_bytes((unsigned)tid >> 4));
+    const unsigned char *lutb = reinterpret_cast<const unsigned char *>(lut_s);
+    // bits 16*hi .. 16*hi+15 of x -> 16 bytes of +-1, bit b -> byte b
+    auto expand_half = [&](uint32_t x, int hi) {
+        const uint32_t i0 = hi ? (x >> 13) & 0x7F8u : (x << 3) & 0x7F8u;
+        const uint32_t i1 = hi ? (x >> 21) & 0x7F8u : (x >> 5) & 0x7F8u;
+        const uint2 a = *reinterpret_cast<const uint2 *>(lutb + i0), b = *reinterpret_cast<const uint2 *>(lutb + i1);
+        return make_uint4(a.x, a.y, b.x, b.y);
     };
 
     // ---- fragment geometry ---------------------------------------------------------------------------------
@@ -120,9 +154,9 @@ __global__ __launch_bounds__(kRwThreads, 2) void conv_rw_kernel(const RwConv p)
     //   y = shift of those bits | mask of the channel bits among them << 8 | (tap column inside the filter) << 31;
     // a tap column past the filter multiplies by zero bytes, channel positions past in_bits by -1 (they equal the
     // pixel's zero tail and are part of K).
-    uint2 *tab = reinterpret_cast<uint2 *>(lds + kRwLutBytes);
-    if (tid < NK * 4) {
-        const int kq = tid >> 2, g = tid & 3;
+    if (tid >= 64 && tid < 64 + NK * 4) {
+        const int e = tid - 64;
+        const int kq = e >> 2, g = e & 3;
         const int i = kq / CPR, q = kq - i * CPR;
         int qj = 0, qc = 0;
         if (p.CB == 32) {
@@ -145,285 +179,373 @@ __global__ __launch_bounds__(kRwThreads, 2) void conv_rw_kernel(const RwConv p)
             sh = c0 & 63;
         }
         const bool inside = j < p.fy;
-        tab[tid] = make_uint2(inside ? (uint32_t)(fr * p.O) * 8u : 0u,
-                              (uint32_t)sh | (((1u << nv) - 1u) << 8) | (inside ? 0x80000000u : 0u));
+        tab[e] = make_uint2(inside ? (uint32_t)(fr * p.O) * 8u : 0u,
+                            (uint32_t)sh | (((1u << nv) - 1u) << 8) | (inside ? 0x80000000u : 0u));
     }
+    __syncthreads();  // tables complete
+
+    // number of tasks of this workgroup
+    const int64_t nmem = (int64_t)blockIdx.x < p.D ? (p.D - blockIdx.x + gridDim.x - 1) / gridDim.x : 0;
+    const int nsteps = (int)(nmem * p.ncg * p.S);
+
+    if (producer) {
+        // =========================================== producer ===================================================
+        // Team thread ttid owns the items (pixel words) ttid, ttid + 256, ... of a band; all of a band's items are
+        // in flight at once (the host sizes bands so that they fit).  An out-of-range pixel reads word 0 of the
+        // member and is replaced by the zero word.
+        const int pixb = p.Cw * 8, rowb = p.Wd * pixb;  // bytes per pixel / image row
+        const int prow = ttid / p.RW, pxx = ttid - prow * p.RW;
+        // input words of this step's and of the next task, and which of them are inside the image (the others are
+        // replaced by the zero word when they are used, so that nothing waits for a load when it is issued)
+        uint64_t wda[kRwItems], wdb[kRwItems];
+        uint32_t ina = 0, inb_ = 0;
+        uint64_t fw[FPW];
+        int traw = 0;
+        // item u of this thread is pixel ttid + 256*u of the band's LDS image: its row, byte offset relative to the
+        // band's first input row, and whether its column is inside the image
+        int irow[kRwItems], ioff[kRwItems];
+        uint32_t xin = 0;
+        {
+            int r = prow, x = pxx;
+#pragma unroll
+            for (int u = 0; u < kRwItems; u++) {
+                irow[u] = r;
+                ioff[u] = r * rowb + (x - p.py) * pixb;
+                xin |= (x - p.py >= 0 && x - p.py < p.Wd) ? 1u << u : 0u;
+                r += p.pix_q;
+                x += p.pix_r;
+                if (x >= p.RW) {
+                    x -= p.RW;
+                    r++;
+                }
+            }
+        }
+        auto request = [&](uint64_t (&wd)[kRwItems], uint32_t &inside, const RwTask &t, int cw) {
+            const unsigned char *src = reinterpret_cast<const unsigned char *>(p.in + t.z * (int64_t)p.H * p.Wd * p.Cw);
+            const int y0 = t.band * p.hs - p.px, off0 = y0 * rowb + cw * 8;
+            inside = 0;
+#pragma unroll
+            for (int u = 0; u < kRwItems; u++) {
+                const bool inb = ((xin >> u) & 1u) && (unsigned)(y0 + irow[u]) < (unsigned)p.H;  // false past the last row too
+                wd[u] = *reinterpret_cast<const uint64_t *>(src + (uint32_t)(inb ? off0 + ioff[u] : 0));
+                inside |= inb ? 1u << u : 0u;
+            }
+        };
+        // Filter words of a channel group: wave tw takes fragments tw, tw+4, ... (fragment f = chunk f/NT, channel
+        // tile f%NT).  Every address is valid (channels past O read channel O-1, dead tap columns word 0); the
+        // expansion zeroes them.
+        auto request_filter = [&](const RwTask &t) {
+            const unsigned char *fz = reinterpret_cast<const unsigned char *>(p.filt + t.z * (int64_t)p.fwords);
+            const int n0 = t.cg * 16 * NT * p.cgt;
+            const int nft = NF * p.cgt;  // fragments of the task: f = (channel tile * NK + chunk) * NT + 16-channel piece
+#pragma unroll
+            for (int i = 0; i < FPW; i++) {
+                const int f = tw + kRwPWaves * i;  // uniform
+                const int fc = f < nft ? f : 0;
+                const int ct = fc / NF, r = fc - ct * NF, kq = r / NT, nt = r - kq * NT;
+                const int ch = n0 + (ct * NT + nt) * 16 + li;
+                fw[i] = *reinterpret_cast<const uint64_t *>(fz + (tab[kq * 4 + lg].x + (uint32_t)(ch < p.O ? ch : p.O - 1) * 8u));
+            }
+            if (MODE != 0) {
+                const int ch = n0 + ttid;
+                traw = p.thresh[t.z * p.O + (ch < p.O ? ch : p.O - 1)];
+            }
+        };
+        RwTask cur{(int64_t)blockIdx.x, 0, 0};
+        if (nsteps > 0) {
+            request_filter(cur);
+            request(wda, ina, cur, 0);
+        }
+        int nb = 0;      // fragment sets staged so far
+        int imgseq = 0;  // images expanded so far; image i sits in buffer i & 1
+        // One step: `wd` holds the input words of task k (requested a step ago); those of task k+1 go to `wn` first
+        // thing, so that their latency hides behind this step's work.
+        auto step = [&](int k, uint64_t (&wd)[kRwItems], uint32_t &wdin, uint64_t (&wn)[kRwItems], uint32_t &wnin) {
+            if (k < nsteps) {
+                RwTask nxt = cur;
+                rw_next(nxt, p);
+                const bool more = k + 1 < nsteps;
+                if (more && (p.S > 1 || nxt.cg == 0)) request(wn, wnin, nxt, 0);
+                const int n0 = cur.cg * 16 * NT * p.cgt;
+                if (cur.band == 0) {
+                    // ---- new (member, channel group): fragments and thresholds -> staging area -------------------
+                    unsigned char *bst = bst0 + (nb % p.nbst) * kFragBytes;
+                    nb++;
+#pragma unroll
+                    for (int i = 0; i < FPW; i++) {
+                        const int f = tw + kRwPWaves * i;
+                        if (f < NF * p.cgt) {  // uniform
+                            const int ct = f / NF, r = f - ct * NF, kq = r / NT, nt = r - kq * NT;
+                            const uint32_t e = tab[kq * 4 + lg].y;
+                            const uint32_t sh = e & 63u, vmask = (e >> 8) & 0xFFFFu;
+                            const bool live = (int)e < 0 && n0 + (ct * NT + nt) * 16 + li < p.O;
+                            const uint4 e16 = expand_half((uint32_t)(fw[i] >> sh) & vmask, 0);
+                            *reinterpret_cast<uint4 *>(bst + (f * 64 + lane) * 16) = live ? e16 : make_uint4(0u, 0u, 0u, 0u);
+                        }
+                    }
+                    // thresholds in dot-product terms: 2*popc > t  <=>  popc > (t>>1)  <=>  dot < K - 2*(t>>1)
+                    if (MODE != 0 && ttid < 64) {
+                        int64_t td = n0 + ttid < p.O ? (int64_t)p.K - 2 * (int64_t)(traw >> 1) : -2147483648LL;
+                        td = td > 2147483647LL ? 2147483647LL : (td < -2147483648LL ? -2147483648LL : td);
+                        reinterpret_cast<int *>(bst + NF * CGTMAX * 1024)[ttid] = (int)td;
+                    }
+                }
+                // the filter words of the next task get the whole image expansion as a head start
+                if (more && nxt.band == 0) request_filter(nxt);
+                // ---- input words -> +-1 bytes in an image buffer (kept when only the channel group changed) ---------
+                if (k == 0 || p.S > 1 || cur.cg == 0) {
+                    unsigned char *img = img0 + (imgseq & 1) * p.img_bytes;
+                    imgseq++;
+                    const int row0 = cur.band * p.hs;
+                    const int hloc = p.h - row0 < p.hs ? p.h - row0 : p.hs;
+                    const int npix = (hloc + FX - 1) * p.RW;
+                    for (int cw = 0; cw < p.Cw; cw++) {
+                        if (cw > 0) request(wd, wdin, cur, cw);
+                        const int nbytes = p.CB - cw * 64 < 64 ? p.CB - cw * 64 : 64;  // positions held by this word
+                        unsigned char *dst = img + __mul24(ttid, p.PS) + cw * 64;
+                        const int dstep = kRwTeam * p.PS;
+#pragma unroll
+                        for (int u = 0; u < kRwItems; u++) {
+                            if (ttid + u * kRwTeam < npix) {
+                                const bool inside = (wdin >> u) & 1u;
+                                const uint32_t lo = inside ? (uint32_t)wd[u] : 0u, hi = inside ? (uint32_t)(wd[u] >> 32) : 0u;
+#pragma unroll
+                                for (int c = 0; c < 4; c++)
+                                    if (16 * c < nbytes)  // uniform
+                                        *reinterpret_cast<uint4 *>(dst + 16 * c) = expand_half(c < 2 ? lo : hi, c & 1);
+                            }
+                            dst += dstep;
+                        }
+                    }
+                }
+                cur = nxt;
+            }
+            __syncthreads();
+        };
+        for (int k = 0; k <= nsteps; k += 2) {
+            step(k, wda, ina, wdb, inb_);
+            if (k + 1 <= nsteps) step(k + 1, wdb, inb_, wda, ina);
+        }
+        return;
+    }
+
+    // ============================================= consumer =====================================================
     int koff[CPR];  // byte offset of the lane's 16 positions relative to the strip's first pixel
 #pragma unroll
     for (int q = 0; q < CPR; q++) {
         const int j = p.qj[q] + (lg >> p.jsh);
         koff[q] = __mul24((j < p.fy ? j : 0) + li, p.PS) + p.qc[q] + 16 * (lg & p.cmask);
     }
-    __syncthreads();  // tables complete
-
-    // The four waves build a channel group's NK*NT filter fragments together: wave w takes fragments w, w+4, ...
-    // (fragment f = chunk f/NT, channel tile f%NT) from global memory, expands them into the staging area, and
-    // after a barrier every wave copies all of them into registers.  Every address is valid (channels past O read
-    // channel O-1, dead tap columns word 0); the expansion zeroes them.
-    constexpr int NF = NK * NT, FPW = (NF + kRwWaves - 1) / kRwWaves;
-    const unsigned char *fz = reinterpret_cast<const unsigned char *>(p.filt + z * (int64_t)p.fwords);
-    unsigned char *bst = lds + p.bst_off;
-    uint64_t fw[FPW];
-    int traw[NT];
-    auto request_filter = [&](int n0) {
-#pragma unroll
-        for (int t = 0; t < FPW; t++) {
-            const int f = wv + kRwWaves * t;  // uniform
-            const int kq = f < NF ? f / NT : 0, nt = f < NF ? f - kq * NT : 0;
-            const int ch = n0 + nt * 16 + li;
-            fw[t] = *reinterpret_cast<const uint64_t *>(fz + (tab[kq * 4 + lg].x + (uint32_t)(ch < p.O ? ch : p.O - 1) * 8u));
-        }
-        if (MODE != 0) {
-#pragma unroll
-            for (int nt = 0; nt < NT; nt++) {
-                const int ch = n0 + nt * 16 + li;
-                traw[nt] = p.thresh[z * p.O + (ch < p.O ? ch : p.O - 1)];
-            }
-        }
-    };
-    auto stage_filter = [&](int n0) {
-#pragma unroll
-        for (int t = 0; t < FPW; t++) {
-            const int f = wv + kRwWaves * t;
-            if (f < NF) {  // uniform
-                const int kq = f / NT, nt = f - kq * NT;
-                const uint32_t e = tab[kq * 4 + lg].y;
-                const uint32_t sh = e & 63u, vmask = (e >> 8) & 0xFFFFu;
-                const bool live = (int)e < 0 && n0 + nt * 16 + li < p.O;
-                const uint32_t h16 = (uint32_t)(fw[t] >> sh) & vmask;
-                const uint4 e16 = expand16(h16);
-                *reinterpret_cast<uint4 *>(bst + (f * 64 + lane) * 16) =
-                    live ? e16 : make_uint4(0u, 0u, 0u, 0u);
-            }
-        }
-    };
     v4i B[NK][NT];
     int tdot[NT];
-    auto fetch_fragments = [&](int n0) {
 #pragma unroll
-        for (int kq = 0; kq < NK; kq++)
+    for (int kq = 0; kq < NK; kq++)
 #pragma unroll
-            for (int nt = 0; nt < NT; nt++)
-                B[kq][nt] = *reinterpret_cast<const v4i *>(bst + ((kq * NT + nt) * 64 + lane) * 16);
-        // thresholds in dot-product terms: 2*popc > t  <=>  popc > (t>>1)  <=>  dot < K - 2*(t>>1)
-        if (MODE != 0) {
+        for (int nt = 0; nt < NT; nt++) B[kq][nt] = (v4i){0, 0, 0, 0};
 #pragma unroll
-            for (int nt = 0; nt < NT; nt++) {
-                int64_t td = n0 + nt * 16 + li < p.O ? (int64_t)p.K - 2 * (int64_t)(traw[nt] >> 1) : -2147483648LL;
-                td = td > 2147483647LL ? 2147483647LL : (td < -2147483648LL ? -2147483648LL : td);
-                tdot[nt] = (int)td;
-            }
-        }
-    };
-    request_filter(cg0 * 16 * NT);
-
-    // ---- phase 1: request the band's input words (with border) --------------------------------------------------
-    // one pixel word per item, up to U items per thread in flight; (row, column, offset) advance incrementally; an
-    // out-of-range pixel reads word 0 of the member and is replaced by the zero word
-    const unsigned char *src = reinterpret_cast<const unsigned char *>(p.in + z * (int64_t)p.H * p.Wd * p.Cw);
-    const int npix = (hloc + FX - 1) * p.RW;
-    const int pixb = p.Cw * 8, rowb = p.Wd * pixb;                          // bytes per pixel / image row
-    const int stepb = p.pix_q * rowb + p.pix_r * pixb, wrapb = rowb - p.RW * pixb;
-    const int xend = p.RW - p.py;
-    constexpr int U = 8;
-    int yy, xs, off;  // running position of the thread's next item
-    {
-        const int row = tid / p.RW, xx = tid - row * p.RW;
-        yy = row0 + row - p.px;
-        xs = xx - p.py;
-        off = yy * rowb + xs * pixb;
-    }
-    uint64_t wd[U];
-    auto load_items = [&](int cw8) {
+    for (int nt = 0; nt < NT; nt++) tdot[nt] = 0;
+    int *stage = stage0 + tw * (16 * 16 * NT);  // MODE 0 only
+    // Wave tw always works on channel tile ct of a task (so its fragments stay valid over a member's bands) and
+    // shares the (strip, sub-band) units of that tile with the other waves of the same tile.
+    const int ct = tw % p.cgt, uw = tw / p.cgt, ustep = kRwCWaves / p.cgt;
+    const int nunits = p.ntx * p.nsub;
+    RwTask cur{(int64_t)blockIdx.x, 0, 0};
+    int nb = 0, imgseq = 0;
+    for (int k = 0; k <= nsteps; k++) {
+        if (k > 0) {
+            // task k-1: image number imgseq, new fragments in staging area nb % nbst
+            const int64_t z = cur.z;
+            const int cg = cur.cg;
+            const int n0 = (cg * p.cgt + ct) * 16 * NT;  // first channel of the wave's tile
+            const int row0 = cur.band * p.hs;
+            const int hloc = p.h - row0 < p.hs ? p.h - row0 : p.hs;
+            if (k == 1 || p.S > 1 || cg == 0) imgseq++;
+            const unsigned char *img = img0 + ((imgseq - 1) & 1) * p.img_bytes;
+            if (cur.band == 0) {
+                const unsigned char *bst = bst0 + (nb % p.nbst) * kFragBytes;
+                nb++;
 #pragma unroll
-        for (int u = 0; u < U; u++) {
-            const bool inb = yy >= 0 && yy < p.H && xs >= 0 && xs < p.Wd;  // false past the last image row too
-            const uint64_t v = *reinterpret_cast<const uint64_t *>(src + (uint32_t)(inb ? off + cw8 : 0));
-            wd[u] = inb ? v : 0ull;
-            yy += p.pix_q;
-            xs += p.pix_r;
-            off += stepb;
-            if (xs >= xend) {
-                xs -= p.RW;
-                yy++;
-                off += wrapb;
-            }
-        }
-    };
-    load_items(0);
-
-    // ---- phase 2: first channel group's fragments (staged over the still empty image area when cgl == 1) ---------
-    stage_filter(cg0 * 16 * NT);
-    __syncthreads();  // fragments complete
-    fetch_fragments(cg0 * 16 * NT);
-    __syncthreads();  // fragments in registers: the area is free again
-
-    // ---- phase 3: expand the input words into +-1 bytes in LDS -----------------------------------------------------
-    for (int cw = 0; cw < p.Cw; cw++) {
-        const int nbytes = p.CB - cw * 64 < 64 ? p.CB - cw * 64 : 64;  // positions held by this word
-        unsigned char *dst = img + __mul24(tid, p.PS) + cw * 64;
-        const int dstep = kRwThreads * p.PS;
-        for (int pix0 = tid; pix0 < npix; pix0 += kRwThreads * U) {
-            if (pix0 != tid || cw != 0) load_items(cw * 8);
+                for (int kq = 0; kq < NK; kq++)
 #pragma unroll
-            for (int u = 0; u < U; u++) {
-                if (pix0 + u * kRwThreads < npix) {
-                    for (int c = 0; c < nbytes; c += 16) {
-                        *reinterpret_cast<uint4 *>(dst + c) = expand16((uint32_t)(wd[u] >> c) & 0xFFFFu);
-                    }
+                    for (int nt = 0; nt < NT; nt++)
+                        B[kq][nt] = *reinterpret_cast<const v4i *>(bst + (((ct * NK + kq) * NT + nt) * 64 + lane) * 16);
+                if (MODE != 0) {
+#pragma unroll
+                    for (int nt = 0; nt < NT; nt++)
+                        tdot[nt] = reinterpret_cast<const int *>(bst + NF * CGTMAX * 1024)[(ct * NT + nt) * 16 + li];
                 }
-                dst += dstep;
             }
-        }
-        if (cw + 1 < p.Cw) {  // rewind to the thread's first item for the next channel word
-            const int row = tid / p.RW, xx = tid - row * p.RW;
-            yy = row0 + row - p.px;
-            xs = xx - p.py;
-            off = yy * rowb + xs * pixb;
-        }
-    }
-    __syncthreads();  // image complete
+            for (int u = uw; u < nunits; u += ustep) {
+                const int sub = u / p.ntx, strip = u - sub * p.ntx;
+                const int ys = sub * p.hb;
+                const int ye = ys + p.hb < hloc ? ys + p.hb : hloc;
+                if (ys >= ye) continue;  // wave-uniform
+                const int x0 = strip * 16;
 
-    int *stage = reinterpret_cast<int *>(img + p.img_bytes) + wv * (16 * 16 * NT);  // MODE 0 only
-
-    for (int cg = cg0;;) {
-    const int n0 = cg * 16 * NT;  // first channel of the group
-    for (int u = wv; u < nunits; u += kRwWaves) {
-        const int sub = u / p.ntx, strip = u - sub * p.ntx;
-        const int ys = sub * p.hb;
-        const int ye = ys + p.hb < hloc ? ys + p.hb : hloc;
-        if (ys >= ye) continue;  // wave-uniform
-        const int x0 = strip * 16;
-
-        int pend[NT][2];  // MODE 3: x-pooled minima of the even row of a pair
+            int pend[NT][2];  // MODE 3: x-pooled minima of the even row of a pair
 #pragma unroll
-        for (int nt = 0; nt < NT; nt++) pend[nt][0] = pend[nt][1] = 0;
+            for (int nt = 0; nt < NT; nt++) pend[nt][0] = pend[nt][1] = 0;
 
-        // ---- epilogue of one finished output row (band-relative y) -------------------------------------------
-        // Output addresses: a uniform row pointer (scalar arithmetic) plus a per-lane 32-bit byte offset.
-        unsigned char *obase;   // first element of the strip's row 0 (band-relative) for this channel group
-        int64_t orowb;          // bytes from one (pooled) output row to the next
-        uint32_t olane[MODE == 0 ? 16 / (64 / (4 * NT)) : 1];
-        bool olive[MODE == 0 ? 16 / (64 / (4 * NT)) : 1];
-        const bool halfword = NT == 2 && p.ncg > 1;  // a 32-channel group is half a word
-        if (MODE == 0) {
-            constexpr int LPP = 4 * NT, PPI = 64 / LPP;  // lanes per pixel (one int4 each), pixels per store
-            obase = static_cast<unsigned char *>(p.out) + ((((z * p.h + row0) * (int64_t)p.w + x0) * p.O + n0) << 2);
-            orowb = ((int64_t)p.w * p.O) << 2;
-#pragma unroll
-            for (int s = 0; s < 16 / PPI; s++) {
-                const int pi = s * PPI + lane / LPP, c4 = (lane % LPP) * 4;
-                olane[s] = (uint32_t)(__mul24(pi, p.O) + c4) << 2;
-                olive[s] = x0 + pi < p.w && n0 + c4 < p.O;
-            }
-        } else {
-            const int hh = MODE == 3 ? p.h >> 1 : p.h, ww = MODE == 3 ? p.w >> 1 : p.w;
-            const int r0 = MODE == 3 ? row0 >> 1 : row0, xx0 = MODE == 3 ? x0 >> 1 : x0;
-            const int64_t e0 = ((z * hh + r0) * (int64_t)ww + xx0) * Ow;  // word index of the strip's first pixel
-            obase = static_cast<unsigned char *>(p.out) + (halfword ? (e0 << 3) + 4 * cg : (e0 + cg) << 3);
-            orowb = ((int64_t)ww * Ow) << 3;
-            olane[0] = (uint32_t)__mul24(lane, Ow) << 3;
-            olive[0] = lane < (MODE == 3 ? 8 : 16) && xx0 + lane < ww;
-        }
-        auto finish_row = [&](v4i (&a)[NT], int y) {
+            // ---- epilogue of one finished output row (band-relative y) -------------------------------------------
+            // Output addresses: a uniform row pointer (scalar arithmetic) plus a per-lane 32-bit byte offset.
+            unsigned char *obase;   // first element of the strip's row 0 (band-relative) for this channel group
+            int64_t orowb;          // bytes from one (pooled) output row to the next
+            uint32_t olane[MODE == 0 ? 16 / (64 / (4 * NT)) : 1];
+            bool olive[MODE == 0 ? 16 / (64 / (4 * NT)) : 1];
+            const bool piece = p.O >= 64;  // the tile's 16*NT bits are one of several pieces of the pixel's word(s)
             if (MODE == 0) {
-                // stage the 16 x (16*NT) tile in LDS, then store whole pixel rows (non-temporal)
-#pragma unroll
-                for (int nt = 0; nt < NT; nt++)
-#pragma unroll
-                    for (int r = 0; r < 4; r++) stage[(4 * lg + r) * (16 * NT) + nt * 16 + li] = (p.K - a[nt][r]) >> 1;
-                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-                __builtin_amdgcn_wave_barrier();
-                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-                constexpr int LPP = 4 * NT, PPI = 64 / LPP;
-                unsigned char *orow = obase + y * orowb;
+                constexpr int LPP = 4 * NT, PPI = 64 / LPP;  // lanes per pixel (one int4 each), pixels per store
+                obase = static_cast<unsigned char *>(p.out) + ((((z * p.h + row0) * (int64_t)p.w + x0) * p.O + n0) << 2);
+                orowb = ((int64_t)p.w * p.O) << 2;
 #pragma unroll
                 for (int s = 0; s < 16 / PPI; s++) {
                     const int pi = s * PPI + lane / LPP, c4 = (lane % LPP) * 4;
-                    if (olive[s]) {
-                        const nb_i32x4 v = *reinterpret_cast<const nb_i32x4 *>(stage + pi * (16 * NT) + c4);
-                        __builtin_nontemporal_store(v, reinterpret_cast<nb_i32x4 *>(orow + olane[s]));
-                    }
-                }
-                __builtin_amdgcn_wave_barrier();
-                return;
-            }
-            uint64_t word = 0;
-            if (MODE == 2) {
-                // ballot r of lane (pixel 4*g+r, channel li): bits 16*g.. are the 16-channel piece of pixel 4*g+r.
-                // Lane j < 16 assembles the pieces of pixel j over the NT channel tiles and writes them.
-#pragma unroll
-                for (int nt = 0; nt < NT; nt++) {
-                    uint64_t m[4];
-#pragma unroll
-                    for (int r = 0; r < 4; r++) m[r] = __ballot(a[nt][r] < tdot[nt]);
-                    const uint64_t mine = rw_sel4(lane & 3, m[0], m[1], m[2], m[3]);
-                    word |= ((mine >> (16 * ((lane >> 2) & 3))) & 0xFFFFull) << (16 * nt);
+                    olane[s] = (uint32_t)(__mul24(pi, p.O) + c4) << 2;
+                    olive[s] = x0 + pi < p.w && n0 + c4 < p.O;
                 }
             } else {
-                // pixels 4g, 4g+1 and 4g+2, 4g+3 pool in x; rows y (even) and y+1 pool in y
-                if ((y & 1) == 0) {
+                const int hh = MODE == 3 ? p.h >> 1 : p.h, ww = MODE == 3 ? p.w >> 1 : p.w;
+                const int r0 = MODE == 3 ? row0 >> 1 : row0, xx0 = MODE == 3 ? x0 >> 1 : x0;
+                const int64_t e0 = ((z * hh + r0) * (int64_t)ww + xx0) * Ow;  // word index of the strip's first pixel
+                obase = static_cast<unsigned char *>(p.out) + (piece ? ((e0 + cg) << 3) + 2 * NT * ct : e0 << 3);
+                orowb = ((int64_t)ww * Ow) << 3;
+                olane[0] = (uint32_t)__mul24(lane, Ow) << 3;
+                olive[0] = lane < (MODE == 3 ? 8 : 16) && xx0 + lane < ww;
+            }
+            auto finish_row = [&](v4i (&a)[NT], int y) {
+                if (MODE == 0) {
+                    // stage the 16 x (16*NT) tile in LDS, then store whole pixel rows (non-temporal)
 #pragma unroll
-                    for (int nt = 0; nt < NT; nt++) {
-                        pend[nt][0] = a[nt][0] < a[nt][1] ? a[nt][0] : a[nt][1];
-                        pend[nt][1] = a[nt][2] < a[nt][3] ? a[nt][2] : a[nt][3];
+                    for (int nt = 0; nt < NT; nt++)
+#pragma unroll
+                        for (int r = 0; r < 4; r++) stage[(4 * lg + r) * (16 * NT) + nt * 16 + li] = (p.K - a[nt][r]) >> 1;
+                    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                    __builtin_amdgcn_wave_barrier();
+                    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+                    constexpr int LPP = 4 * NT, PPI = 64 / LPP;
+                    unsigned char *orow = obase + y * orowb;
+#pragma unroll
+                    for (int s = 0; s < 16 / PPI; s++) {
+                        const int pi = s * PPI + lane / LPP, c4 = (lane % LPP) * 4;
+                        if (olive[s]) {
+                            const nb_i32x4 v = *reinterpret_cast<const nb_i32x4 *>(stage + pi * (16 * NT) + c4);
+                            __builtin_nontemporal_store(v, reinterpret_cast<nb_i32x4 *>(orow + olane[s]));
+                        }
                     }
+                    __builtin_amdgcn_wave_barrier();
                     return;
                 }
+                uint64_t word = 0;
+                if (MODE == 2) {
+                    // ballot r of lane (pixel 4*g+r, channel li): bits 16*g.. are the 16-channel piece of pixel 4*g+r.
+                    // Lane j < 16 assembles the pieces of pixel j over the NT channel tiles and writes them.
 #pragma unroll
-                for (int nt = 0; nt < NT; nt++) {
-                    int v0 = a[nt][0] < a[nt][1] ? a[nt][0] : a[nt][1];
-                    int v1 = a[nt][2] < a[nt][3] ? a[nt][2] : a[nt][3];
-                    v0 = v0 < pend[nt][0] ? v0 : pend[nt][0];
-                    v1 = v1 < pend[nt][1] ? v1 : pend[nt][1];
-                    const uint64_t m0 = __ballot(v0 < tdot[nt]), m1 = __ballot(v1 < tdot[nt]);
-                    const uint64_t mine = (lane & 1) ? m1 : m0;  // pooled pixel 2g + q <-> lane 2g + q
-                    word |= ((mine >> (16 * ((lane >> 1) & 3))) & 0xFFFFull) << (16 * nt);
-                }
-            }
-            unsigned char *orow = obase + (MODE == 3 ? y >> 1 : y) * orowb;
-            if (olive[0]) {
-                if (halfword) {
-                    uint32_t *o = reinterpret_cast<uint32_t *>(orow + olane[0]);
-                    o[0] = (uint32_t)word;
-                    if (cg == p.ncg - 1 && (cg & 1) == 0) o[1] = 0u;
+                    for (int nt = 0; nt < NT; nt++) {
+                        uint64_t m[4];
+#pragma unroll
+                        for (int r = 0; r < 4; r++) m[r] = __ballot(a[nt][r] < tdot[nt]);
+                        const uint64_t mine = rw_sel4(lane & 3, m[0], m[1], m[2], m[3]);
+                        word |= ((mine >> (16 * ((lane >> 2) & 3))) & 0xFFFFull) << (16 * nt);
+                    }
                 } else {
-                    *reinterpret_cast<uint64_t *>(orow + olane[0]) = word;
+                    // pixels 4g, 4g+1 and 4g+2, 4g+3 pool in x; rows y (even) and y+1 pool in y
+                    if ((y & 1) == 0) {
+#pragma unroll
+                        for (int nt = 0; nt < NT; nt++) {
+                            pend[nt][0] = a[nt][0] < a[nt][1] ? a[nt][0] : a[nt][1];
+                            pend[nt][1] = a[nt][2] < a[nt][3] ? a[nt][2] : a[nt][3];
+                        }
+                        return;
+                    }
+#pragma unroll
+                    for (int nt = 0; nt < NT; nt++) {
+                        int v0 = a[nt][0] < a[nt][1] ? a[nt][0] : a[nt][1];
+                        int v1 = a[nt][2] < a[nt][3] ? a[nt][2] : a[nt][3];
+                        v0 = v0 < pend[nt][0] ? v0 : pend[nt][0];
+                        v1 = v1 < pend[nt][1] ? v1 : pend[nt][1];
+                        const uint64_t m0 = __ballot(v0 < tdot[nt]), m1 = __ballot(v1 < tdot[nt]);
+                        const uint64_t mine = (lane & 1) ? m1 : m0;  // pooled pixel 2g + q <-> lane 2g + q
+                        word |= ((mine >> (16 * ((lane >> 1) & 3))) & 0xFFFFull) << (16 * nt);
+                    }
                 }
-            }
-        };
+                unsigned char *orow = obase + (MODE == 3 ? y >> 1 : y) * orowb;
+                if (olive[0]) {
+                    if (piece && NT == 1) {
+                        *reinterpret_cast<uint16_t *>(orow + olane[0]) = (uint16_t)word;
+                    } else if (piece) {
+                        *reinterpret_cast<uint32_t *>(orow + olane[0]) = (uint32_t)word;
+                    } else {
+                        *reinterpret_cast<uint64_t *>(orow + olane[0]) = word;
+                    }
+                }
+            };
 
-        // ---- walk down the strip: image row rr (band-relative) feeds output rows rr, rr-1, rr-2 --------------
-        // a0 holds the partial sums of output row rr-2 (two filter rows done), a1 those of row rr-1 (one done).
-        // Image row rr completes row rr-2 (emitted), continues row rr-1 and opens row rr with a zero C operand,
-        // so nothing is ever cleared or rotated.  Rows rr in [ys+2, ye) take the branch-free loop.
-        const unsigned char *arow = img + (ys * p.RW + x0) * p.PS;
-        const int rowbytes = p.RW * p.PS;
-        const int rend = ye + FX - 1;
-        const int ylast = MODE == 3 ? (p.h & ~1) - row0 : ye;  // pooled maps drop an odd last row
-        v4i F[CPR], a0[NT], a1[NT];
+            // ---- walk down the strip: image row rr (band-relative) feeds output rows rr, rr-1, rr-2 --------------
+            // a0 holds the partial sums of output row rr-2 (two filter rows done), a1 those of row rr-1 (one done).
+            // Image row rr completes row rr-2 (emitted), continues row rr-1 and opens row rr with a zero C operand,
+            // so nothing is ever cleared or rotated.  Rows rr in [ys+2, ye) take the branch-free loop.
+            const unsigned char *arow = img + (ys * p.RW + x0) * p.PS;
+            const int rowbytes = p.RW * p.PS;
+            const int rend = ye + FX - 1;
+            const int ylast = MODE == 3 ? (p.h & ~1) - row0 : ye;  // pooled maps drop an odd last row
+            v4i F[CPR], a0[NT], a1[NT];
 #pragma unroll
-        for (int q = 0; q < CPR; q++) F[q] = *reinterpret_cast<const v4i *>(arow + koff[q]);
+            for (int q = 0; q < CPR; q++) F[q] = *reinterpret_cast<const v4i *>(arow + koff[q]);
 #pragma unroll
-        for (int nt = 0; nt < NT; nt++) a0[nt] = a1[nt] = (v4i){0, 0, 0, 0};
-        auto edge_step = [&](int rr) {  // first two and last two image rows of the sub-band: some parts are missing
-            v4i Fn[CPR];
-            arow += rowbytes;
+            for (int nt = 0; nt < NT; nt++) a0[nt] = a1[nt] = (v4i){0, 0, 0, 0};
+            auto edge_step = [&](int rr) {  // first two and last two image rows of the sub-band: some parts are missing
+                v4i Fn[CPR];
+                arow += rowbytes;
 #pragma unroll
-            for (int q = 0; q < CPR; q++) Fn[q] = F[q];
-            if (rr + 1 < rend) {
+                for (int q = 0; q < CPR; q++) Fn[q] = F[q];
+                if (rr + 1 < rend) {
+#pragma unroll
+                    for (int q = 0; q < CPR; q++) Fn[q] = *reinterpret_cast<const v4i *>(arow + koff[q]);
+                }
+                if (rr - 2 >= ys) {
+#pragma unroll
+                    for (int q = 0; q < CPR; q++)
+#pragma unroll
+                        for (int nt = 0; nt < NT; nt++)
+                            a0[nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(F[q], B[2 * CPR + q][nt], a0[nt], 0, 0, 0);
+                    if (rr - 2 < ylast) finish_row(a0, rr - 2);
+                }
+                if (rr - 1 >= ys && rr - 1 < ye) {
+#pragma unroll
+                    for (int nt = 0; nt < NT; nt++) a0[nt] = a1[nt];
+#pragma unroll
+                    for (int q = 0; q < CPR; q++)
+#pragma unroll
+                        for (int nt = 0; nt < NT; nt++)
+                            a0[nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(F[q], B[CPR + q][nt], a0[nt], 0, 0, 0);
+                }
+                if (rr < ye) {
+#pragma unroll
+                    for (int nt = 0; nt < NT; nt++) a1[nt] = (v4i){0, 0, 0, 0};
+#pragma unroll
+                    for (int q = 0; q < CPR; q++)
+#pragma unroll
+                        for (int nt = 0; nt < NT; nt++)
+                            a1[nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(F[q], B[q][nt], a1[nt], 0, 0, 0);
+                }
+#pragma unroll
+                for (int q = 0; q < CPR; q++) F[q] = Fn[q];
+            };
+            int rr = ys;
+            const int lead = ys + 2 < rend ? ys + 2 : rend;
+            for (; rr < lead; rr++) edge_step(rr);
+            for (; rr < ye; rr++) {
+                v4i Fn[CPR], done[NT];
+                arow += rowbytes;
 #pragma unroll
                 for (int q = 0; q < CPR; q++) Fn[q] = *reinterpret_cast<const v4i *>(arow + koff[q]);
-            }
-            if (rr - 2 >= ys) {
+#pragma unroll
+                for (int nt = 0; nt < NT; nt++) done[nt] = a0[nt];
 #pragma unroll
                 for (int q = 0; q < CPR; q++)
 #pragma unroll
                     for (int nt = 0; nt < NT; nt++)
-                        a0[nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(F[q], B[2 * CPR + q][nt], a0[nt], 0, 0, 0);
-                if (rr - 2 < ylast) finish_row(a0, rr - 2);
-            }
-            if (rr - 1 >= ys && rr - 1 < ye) {
+                        done[nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(F[q], B[2 * CPR + q][nt], done[nt], 0, 0, 0);
 #pragma unroll
                 for (int nt = 0; nt < NT; nt++) a0[nt] = a1[nt];
 #pragma unroll
@@ -431,8 +553,6 @@ __global__ __launch_bounds__(kRwThreads, 2) void conv_rw_kernel(const RwConv p)
 #pragma unroll
                     for (int nt = 0; nt < NT; nt++)
                         a0[nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(F[q], B[CPR + q][nt], a0[nt], 0, 0, 0);
-            }
-            if (rr < ye) {
 #pragma unroll
                 for (int nt = 0; nt < NT; nt++) a1[nt] = (v4i){0, 0, 0, 0};
 #pragma unroll
@@ -440,71 +560,51 @@ __global__ __launch_bounds__(kRwThreads, 2) void conv_rw_kernel(const RwConv p)
 #pragma unroll
                     for (int nt = 0; nt < NT; nt++)
                         a1[nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(F[q], B[q][nt], a1[nt], 0, 0, 0);
+                finish_row(done, rr - 2);  // rr - 2 < ye - 2 <= ylast
+#pragma unroll
+                for (int q = 0; q < CPR; q++) F[q] = Fn[q];
             }
-#pragma unroll
-            for (int q = 0; q < CPR; q++) F[q] = Fn[q];
-        };
-        int rr = ys;
-        const int lead = ys + 2 < rend ? ys + 2 : rend;
-        for (; rr < lead; rr++) edge_step(rr);
-        for (; rr < ye; rr++) {
-            v4i Fn[CPR], done[NT];
-            arow += rowbytes;
-#pragma unroll
-            for (int q = 0; q < CPR; q++) Fn[q] = *reinterpret_cast<const v4i *>(arow + koff[q]);
-#pragma unroll
-            for (int nt = 0; nt < NT; nt++) done[nt] = a0[nt];
-#pragma unroll
-            for (int q = 0; q < CPR; q++)
-#pragma unroll
-                for (int nt = 0; nt < NT; nt++)
-                    done[nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(F[q], B[2 * CPR + q][nt], done[nt], 0, 0, 0);
-#pragma unroll
-            for (int nt = 0; nt < NT; nt++) a0[nt] = a1[nt];
-#pragma unroll
-            for (int q = 0; q < CPR; q++)
-#pragma unroll
-                for (int nt = 0; nt < NT; nt++)
-                    a0[nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(F[q], B[CPR + q][nt], a0[nt], 0, 0, 0);
-#pragma unroll
-            for (int nt = 0; nt < NT; nt++) a1[nt] = (v4i){0, 0, 0, 0};
-#pragma unroll
-            for (int q = 0; q < CPR; q++)
-#pragma unroll
-                for (int nt = 0; nt < NT; nt++)
-                    a1[nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(F[q], B[q][nt], a1[nt], 0, 0, 0);
-            finish_row(done, rr - 2);  // rr - 2 < ye - 2 <= ylast
-#pragma unroll
-            for (int q = 0; q < CPR; q++) F[q] = Fn[q];
+            for (; rr < rend; rr++) edge_step(rr);
+            }
+            rw_next(cur, p);
         }
-        for (; rr < rend; rr++) edge_step(rr);
-    }
-    if (++cg >= cg1) break;
-    // next channel group: no wave reads the staging area during a walk, so a wave that is done starts at once
-    request_filter(cg * 16 * NT);
-    stage_filter(cg * 16 * NT);
-    __syncthreads();
-    fetch_fragments(cg * 16 * NT);
-    __syncthreads();  // a fast wave must not restage while a slow one still fetches
+        __syncthreads();
     }
 }
 
 static inline int rw_round_up(int a, int b) { return (a + b - 1) / b * b; }
 
+// Workgroups per CU that fit by registers (eight waves each) and LDS, and the CU count of the current device.
+struct RwFit {
+    int cus, regs;
+};
 template <int CPR, int NT, int MODE>
 static bool rw_launch_one(const RwConv &p, int64_t D, size_t lds_bytes, hipStream_t s)
 {
-    static bool attr_set = false;  // benign race: setting the same attribute twice is harmless
+    static RwFit fit = {0, 0};  // benign race: every thread computes the same values
     auto *kfn = conv_rw_kernel<CPR, NT, MODE>;
-    if (!attr_set) {
+    if (fit.cus == 0) {
+        hipFuncAttributes fa;
+        int dev = 0, cus = 0;
         if (hipFuncSetAttribute(reinterpret_cast<const void *>(kfn), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                160 * 1024) != hipSuccess) {
+                                kRwMaxDynLds) != hipSuccess ||
+
+            hipFuncGetAttributes(&fa, reinterpret_cast<const void *>(kfn)) != hipSuccess ||
+            hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1) {
             (void)hipGetLastError();
             return false;
         }
-        attr_set = true;
+        fit.regs = fa.numRegs > 0 ? fa.numRegs : 256;
+        fit.cus = cus;
     }
-    kfn<<<dim3((unsigned)(D * p.S * p.ngw)), dim3(kRwThreads), lds_bytes, s>>>(p);
+    // 512 registers per lane and SIMD, three waves of a workgroup per SIMD; 160 KB of LDS per CU
+    int per_cu = 512 / ((fit.regs + 7) / 8 * 8) / 3;
+    const int by_lds = (int)(160 * 1024 / (lds_bytes + kRwLutBytes + kRwTabBytes));
+    per_cu = per_cu < by_lds ? per_cu : by_lds;
+    per_cu = per_cu < 1 ? 1 : (per_cu > 4 ? 4 : per_cu);
+    const int64_t wgs = D < (int64_t)fit.cus * per_cu ? D : (int64_t)fit.cus * per_cu;
+    kfn<<<dim3((unsigned)wgs), dim3(kRwThreads), lds_bytes, s>>>(p);
     return true;
 }
 
@@ -515,14 +615,11 @@ static bool rw_launch_mode(const RwConv &p, int64_t D, int CPR, int NT, size_t l
     if (CPR == cpr && NT == nt) return rw_launch_one<cpr, nt, MODE>(p, D, lds, s)
     NB_RW(1, 1);
     NB_RW(1, 2);
-    NB_RW(1, 4);
     NB_RW(2, 1);
     NB_RW(2, 2);
-    NB_RW(2, 4);
     NB_RW(3, 1);
     NB_RW(3, 2);
-    NB_RW(3, 4);
-    NB_RW(6, 2);
+    NB_RW(6, 1);
 #undef NB_RW
     return false;
 }
@@ -573,57 +670,46 @@ bool conv_rw_try(void *out, const uint64_t *in, const uint64_t *filt, const int3
     }
     for (int q = CPR; q < kRwMaxCPR; q++) p.qj[q] = p.qc[q] = 0;
     if (CPR == 4 || CPR == 5) return false;
-    int NT = O >= 64 ? 4 : O / 16;
-    if (NT == 3) return false;
-    if (CPR == 6) NT = O >= 32 ? 2 : 0;
-    if (CPR == 6 && O == 16) return false;
-    p.ncg = (O + 16 * NT - 1) / (16 * NT);
+    // A consumer wave keeps the fragments of 16*NT channels in registers (at most 72 of its 168); a task covers
+    // cgt such tiles: 64 channels when there are that many, else all of them.
+    int NT, cgt;
+    if (O >= 64) {
+        NT = CPR == 6 ? 1 : 2;
+        cgt = 4 / NT;
+    } else if (O == 16 || (O == 32 && CPR != 6)) {
+        NT = O / 16;
+        cgt = 1;
+    } else {
+        return false;
+    }
+    p.cgt = cgt;
+    p.ncg = (O + 16 * NT * cgt - 1) / (16 * NT * cgt);
     p.PS = ((CB >> 4) & 1) ? CB : CB + 16;
     p.ntx = (g.w + 15) / 16;
     p.RW = 16 * p.ntx + g.fy - 1;
     p.K = 3 * g.fy * CB;
-    p.pix_q = kRwThreads / p.RW;
-    p.pix_r = kRwThreads % p.RW;
-    // Bands: as few as keep a workgroup's LDS at or below 78 KB (two workgroups per CU), rows per band even.
-    // The NK*NT filter fragments (1 KB each) are staged in LDS on their way to the registers.  With one channel
-    // group they borrow the image area before the image is written.  With several, a workgroup walks all groups
-    // over one expanded image if a separate staging area fits (bands of at least 8 rows); otherwise every channel
-    // group gets workgroups of its own, each expanding the image again.
-    const int stage = mode == 0 ? kRwWaves * 16 * 16 * NT * 4 : 0;
+    p.pix_q = kRwTeam / p.RW;
+    p.pix_r = kRwTeam % p.RW;
+    p.D = D;
+    // Bands: as few as possible such that the producers hold a band's input words in flight at once and two image
+    // buffers, the fragment staging areas and the int32 transpose tiles fit the CU's LDS; rows per band even.
+    const int stage = mode == 0 ? kRwCWaves * 16 * 16 * NT * 4 : 0;
     const int rowbytes = p.RW * p.PS;
-    const int frag_bytes = 3 * CPR * NT * 1024;
-    const size_t fixed = (size_t)kRwLutBytes + kRwTabBytes + stage, budget = 78 * 1024;
+    const int frag_bytes = 3 * CPR * 4 * 1024 + 64 * 4;  // NK * NT * (4 / NT) fragments + thresholds
     size_t lds = 0;
-    p.cgl = 0;
     for (p.S = 1;; p.S++) {
         p.hs = rw_round_up((g.h + p.S - 1) / p.S, 2);
-        const int img = rw_round_up((p.hs + 2) * rowbytes + 64, 16);
-        if (p.ncg > 1 && fixed + img + frag_bytes <= budget && (p.hs >= 8 || p.S == 1)) {
-            p.cgl = p.ncg;
-            p.img_bytes = img;
-            p.bst_off = (int)(fixed + img);
-            lds = fixed + img + frag_bytes;
-            break;
-        }
-        if (p.hs <= 2 || (p.ncg > 1 && p.hs < 8)) break;
+        const int bands = (g.h + p.hs - 1) / p.hs;
+        p.nbst = bands == 1 ? 2 : 1;  // every task brings new fragments: stage them alternately
+        p.img_bytes = rw_round_up((p.hs + 2) * rowbytes + 64, 16);
+        lds = 2 * (size_t)p.img_bytes + (size_t)p.nbst * frag_bytes + stage;
+        if ((lds <= (size_t)kRwMaxDynLds && (p.hs + 2) * p.RW <= kRwItems * kRwTeam) || p.hs <= 2) break;
     }
-    if (p.cgl == 0) {
-        for (p.S = 1;; p.S++) {
-            p.hs = rw_round_up((g.h + p.S - 1) / p.S, 2);
-            p.img_bytes = rw_round_up((p.hs + 2) * rowbytes + 64, 16);
-            if (p.img_bytes < frag_bytes) p.img_bytes = frag_bytes;
-            lds = fixed + p.img_bytes;
-            if (lds <= budget || p.hs <= 2) break;
-        }
-        p.cgl = 1;
-        p.bst_off = kRwLutBytes + kRwTabBytes;  // the image area
-    }
-    if (lds > 158 * 1024) return false;
-    p.ngw = (p.ncg + p.cgl - 1) / p.cgl;
+    if (lds > (size_t)kRwMaxDynLds || (p.hs + 2) * p.RW > kRwItems * kRwTeam) return false;
     p.S = (g.h + p.hs - 1) / p.hs;  // bands that own at least one row
-    if (D * p.S * p.ngw > kMaxBlocks) return false;
-    // Sub-bands: enough (strip, sub-band) units for the four waves of a workgroup.
-    int nsub = p.ntx >= kRwWaves ? 1 : (kRwWaves + p.ntx - 1) / p.ntx;
+    // Sub-bands: enough (strip, sub-band) units for the consumer waves of one channel tile.
+    const int wpt = kRwCWaves / cgt;
+    int nsub = p.ntx >= wpt ? 1 : (wpt + p.ntx - 1) / p.ntx;
     p.hb = rw_round_up((p.hs + nsub - 1) / nsub, 2);
     p.nsub = (p.hs + p.hb - 1) / p.hb;
     if (mode == 0) return rw_launch_mode<0>(p, D, CPR, NT, lds, s);
