@@ -169,15 +169,12 @@ int conv_impl(void *out, const W *in, const W *filt, const int32_t *thresh, int6
     if (mode >= 2) NB_REQUIRE_ALIGNED(out, sizeof(W));
     // int8 matrix-core path (64-bit words, stride 1, O % 16 == 0, member fits LDS); same results
     const int engine = conv_engine();
-    if (bits == 64 && Cw > 0 && engine != 1 && !getenv("NESBIN_NO_RW") &&
-        conv_rw_try(out, reinterpret_cast<const uint64_t *>(in), reinterpret_cast<const uint64_t *>(filt), thresh, g, D, N,
-                    tap_bits, mode, s)) {
-        t_last_engine = 2;
-        return check_launch(who);
-    }
-    if (bits == 64 && Cw > 0 && engine != 1 &&
-        conv_mfma_try(out, reinterpret_cast<const uint64_t *>(in), reinterpret_cast<const uint64_t *>(filt), thresh, g,
-                      D, N, tap_bits, tap_bits > 0, mode, engine == 2, s)) {
+    // Automatic choice, measured on MI355X: one workgroup per CU walks whole members, so the matrix-core kernel needs
+    // a population that fills at least half of the CUs; below that the XOR-popcount kernels, which spread one
+    // member's pixels over many workgroups, are faster.
+    if (bits == 64 && Cw > 0 && engine != 1 && (engine == 2 || D >= 128) &&
+        conv_mfma_try(out, reinterpret_cast<const uint64_t *>(in), reinterpret_cast<const uint64_t *>(filt), thresh, g, D,
+                      N, tap_bits, mode, s)) {
         t_last_engine = 2;
         return check_launch(who);
     }

@@ -1,66 +1,82 @@
-// Binary conv on the int8 matrix cores (measured alternative to the VALU popcount path).
+// Binary conv on the int8 matrix cores (3-row filters, stride 1): a persistent producer / consumer kernel.
 //
 // CDNA4 has no 1-bit MFMA, but v_mfma_i32_16x16x64_i8 does 16384 int8 MACs per wave in 16 cycles: 4x the
 // bit-MAC rate of v_xor + v_bcnt.  Bits are expanded to +-1 bytes (bit 1 -> +1, bit 0 -> -1; an out-of-range
-// pixel is the zero word, i.e. all -1), the int32 dot product over K = taps*CB positions is exact, and
+// pixel is the zero word, i.e. all -1), the int32 dot product over the K expanded positions is exact, and
 //     popcount(x ^ w) = (K - dot) / 2
-// gives back the reference's sum bit for bit.  One workgroup owns one member: its image is expanded once
-// into LDS (with the zero-word border, so the implicit im2col needs no bounds checks), the member's filter
-// fragments are expanded once, cooperatively, and then stay in VGPRs, and every wave streams 16-pixel A
-// fragments out of LDS with one ds_read_b128 per fragment.
+// gives back the reference's sum bit for bit.
+//
+// One workgroup of eight waves per CU walks through its share of the population.  A task is a band of output
+// rows of one member for one group of 16*NT output channels.  Waves 4..7 (producers) prepare task k while waves
+// 0..3 (consumers) multiply task k-1, one barrier per step:
+//   producer: the band's input words and, when the (member, channel group) changes, the filter words were
+//     requested one step ahead; it expands the input rows (with the zero-word border, so the implicit im2col
+//     needs no bounds checks) into one of two LDS image buffers and the filter words into MFMA B fragments in an
+//     LDS staging area, then requests the words of task k+1;
+//   consumer: copies new fragments into registers (they stay there for all bands of the member), then every
+//     wave walks DOWN a strip of 16 output columns: the A fragment of image row r and tap column j is the same
+//     16 pixels x 64 positions whichever filter row it meets, so it is read from LDS once and multiplied into
+//     the three output rows r, r-1, r-2.  One ds_read_b128 feeds 3*NT MFMAs.  Finished rows leave straight to
+//     global memory: int32 sums via a per-wave LDS transpose (full pixel rows, non-temporal), or threshold bits
+//     gathered with ballots into packed words, optionally 2x2 OR-pooled (in x a min over neighbouring
+//     accumulator registers, in y over two walked rows).
+// Each SIMD holds one consumer and one producer wave, so the expansion work (VALU, LDS, memory latency) runs in
+// the shadow of the MFMAs instead of in front of them.
 //
 // Fragment layout of v_mfma_i32_16x16x64_i8 (checked on hardware): lane l supplies row l%16 of A and
 // column l%16 of B, its 16 bytes are the K-positions 16*(l/16)..+15 of the 64-chunk (any bijection works as
 // long as A and B use the same one), and acc[r] is D[4*(l/16) + r][l%16].
 //
-// All index arithmetic that needs a division (K position -> tap / channel, tile -> row / column) is done on
-// the host and handed over in the kernel argument block, or advanced incrementally.
+// K chunks of one filter row (the per-pixel byte count CB is 16, 32 or 64*Cw):
+//   CB = 16: one chunk, lane group g holds tap column g (up to 4 columns);
+//   CB = 32: chunk q holds tap columns 2q and 2q+1, 32 positions each;
+//   CB >= 64: one chunk per (tap column, 64-position channel word).
+// Chunks of tap columns past the filter width multiply by zero bytes.
 #include "nb_conv_common.hpp"
 
 namespace nb {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 
-// 512 threads = two waves per SIMD: one wave's LDS reads and epilogue overlap the other's MFMAs.  The filter
-// fragments of up to 36 (chunk, channel tile) pairs stay in registers (144 VGPRs); with more than 18 of them a
-// wave works on two pixel tiles per step instead of four to stay inside 256 VGPRs.
-constexpr int kMfmaThreads = 512;
-constexpr int mfma_mt(int NK, int NT) { return NK * NT > 18 ? 2 : 4; }
-constexpr int kLutBytes = 256 * 8;  // byte -> 8 bytes of +-1
-constexpr int kMaxNK = 18;
-constexpr int kTab = kMaxNK * 16;   // (chunk, lane group, dword) entries
+constexpr int kRwCWaves = 8;      // consumer waves: two per SIMD keep the matrix core issuing back to back
+constexpr int kRwPWaves = 4;      // producer waves
+constexpr int kRwThreads = 64 * (kRwCWaves + kRwPWaves);
+constexpr int kRwTeam = 64 * kRwPWaves;  // producer threads
+constexpr int kRwLutBytes = 256 * 8;  // byte -> 8 bytes of +-1
+constexpr int kRwMaxCPR = 6;
+constexpr int kRwTabBytes = 3 * kRwMaxCPR * 4 * 8;  // (chunk, lane group) -> filter word offset, shift, mask
+// dynamic LDS a launch may ask for: the CU's 160 KB minus the kernel's two static tables
+constexpr int kRwMaxDynLds = 160 * 1024 - kRwLutBytes - kRwTabBytes - 512;
+constexpr int kRwItems = 10;      // input words a producer thread holds in flight
 
-struct MfmaConv {
+struct RwConv {
     const uint64_t *in;
     const uint64_t *filt;
     const int32_t *thresh;
     void *out;
-    int H, Wd, Cw, px, py, h, w, O;
-    int CB;          // bytes (channel positions) per pixel, multiple of 4
-    int PS;          // pixel stride in the LDS image, bytes
-    int RW;          // pixels per LDS image row
-    int RIN;         // LDS image rows = hs + fx - 1
-    int K;           // taps * CB
-    int ntx;         // 16-pixel tiles per output row
-    int frows;       // filter rows per member (words per output channel)
-    int img_bytes, bfr_bytes;
-    int step_q, step_r;  // (waves*MT) / ntx and % ntx: tile advance of one step
-    int pix_q, pix_r;    // threads / RW and % RW: image-pixel advance of one fill pass
-    int taps, fy, tapT, in_bits;  // tapT > 1: tap-packed filter with in_bits channel bits per tap
-    int S, hs;  // a member's output rows are split over S workgroups, hs rows each (even when pooling)
+    int64_t D;
+    int H, Wd, Cw, px, py, h, w, O, fy;
+    int CB;            // expanded bytes per pixel: 16, 32 or 64*Cw
+    int PS;            // pixel stride in the LDS image, bytes (PS/16 odd: conflict-free 16-lane b128 reads)
+    int RW;            // pixels per LDS image row
+    int hs, S;         // output rows per band, bands per member
+    int hb, nsub;      // output rows per sub-band (even), sub-bands per band
+    int ntx, ncg;      // 16-column strips, channel groups (of 16*NT*cgt channels) = tasks per band
+    int cgt;           // consumer channel tiles (of 16*NT channels) per task: 1, 2 or 4
+    int K;             // expanded positions that count: taps * CB
+    int in_bits;       // valid channel bits per pixel
+    int tapT, tapM;    // tap-packed filter: taps per word and ceil(65536 / tapT) + 1 (0: one word per tap and channel word)
+    int img_bytes;     // one image buffer
+    int nbst;          // fragment staging areas (2 when every task brings new fragments)
+    int fwords;        // filter words per member
+    int pix_q, pix_r;  // team threads / RW and % RW: image-pixel advance of one fill pass
+    short qj[kRwMaxCPR];  // chunk q of a filter row: first tap column ...
+    short qc[kRwMaxCPR];  // ... and first position inside the pixel
+    int jsh, cmask;    // lane group g adds (g >> jsh) tap columns and 16 * (g & cmask) positions
 };
-
-// Per K position 64*kc + 16*lg + 4*d (index (kc*4 + lg)*4 + d), computed once per workgroup into LDS:
-struct MfmaTables {
-    int koff[kTab];            // byte offset of that position relative to a tile's pixel in the LDS image
-    short frow[kTab];          // filter row holding the 4 positions
-    unsigned char fsh[kTab];   // bit position inside that filter word
-    unsigned char flf[kTab];   // valid bits from there on (0: multiply by zero)
-};
-constexpr int kTabBytes = (sizeof(MfmaTables) + 15) / 16 * 16;
 
 // 4 bits -> 4 bytes of +-1 (bit j -> byte j): 1 -> 0x01, 0 -> 0xFF
-__device__ __forceinline__ uint32_t pm1_bytes(uint32_t nib)
+__device__ __forceinline__ uint32_t rw_pm1_bytes(uint32_t nib)
 {
     const uint32_t s1 = (nib << 7) | nib;
     const uint32_t s2 = (s1 << 14) | s1;
@@ -68,434 +84,637 @@ __device__ __forceinline__ uint32_t pm1_bytes(uint32_t nib)
     return ((u << 8) - (u << 1)) | 0x01010101u;  // 0xFE where the bit is 0, then | 1
 }
 
-// MODE 0: int32 popcount sums [D,h,w,O]; 2: threshold bits packed along O; 3: the same, 2x2 OR-pooled.
-template <int NK, int NT, int MODE, bool PB16, int MT>
-__global__ __launch_bounds__(kMfmaThreads) void conv_mfma_kernel(const MfmaConv p)
+__device__ __forceinline__ uint64_t rw_sel4(int r, uint64_t a, uint64_t b, uint64_t c, uint64_t d)
 {
-    constexpr int kMfmaWaves = kMfmaThreads / 64;
-    extern __shared__ __align__(16) unsigned char lds[];
-    const uint2 *lut = reinterpret_cast<const uint2 *>(lds);
-    MfmaTables &tab = *reinterpret_cast<MfmaTables *>(lds + kLutBytes);
-    unsigned char *img = lds + kLutBytes + kTabBytes;
-    unsigned char *bfr = img + p.img_bytes;
-    // MODE 0: the per-wave int32 staging tiles reuse the fragment area once the fragments sit in registers;
-    // MODE 2/3: packed words per pixel, behind the fragment area.
-    unsigned char *obuf = MODE == 0 ? bfr : bfr + p.bfr_bytes;
+    return r == 0 ? a : r == 1 ? b : r == 2 ? c : d;
+}
 
-    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+// Position of a workgroup in its task sequence: members blockIdx.x, blockIdx.x + gridDim.x, ...; per member the
+// channel groups, per channel group the bands.
+struct RwTask {
+    int64_t z;
+    int cg, band;
+};
+__device__ __forceinline__ void rw_next(RwTask &t, const RwConv &p)
+{
+    if (++t.band == p.S) {
+        t.band = 0;
+        if (++t.cg == p.ncg) {
+            t.cg = 0;
+            t.z += gridDim.x;
+        }
+    }
+}
+
+// MODE 0: int32 popcount sums [D,h,w,O]; 2: threshold bits packed along O; 3: the same, 2x2 OR-pooled.
+template <int CPR, int NT, int MODE>
+__global__ __launch_bounds__(kRwThreads) void conv_mfma_kernel(const RwConv p)
+{
+    constexpr int FX = 3;
+    constexpr int NK = FX * CPR;
+    constexpr int NF = NK * NT;                  // fragments of one consumer channel tile
+    constexpr int CGTMAX = 4 / NT;               // a task covers at most 64 channels
+    constexpr int FPW = (NF * CGTMAX + kRwPWaves - 1) / kRwPWaves;  // fragments per producer wave, at most
+    constexpr int kFragBytes = NF * CGTMAX * 1024 + 64 * 4;         // + the task's thresholds
+    // The two small tables are objects of their own, so that the compiler knows that the stores into the image and
+    // staging buffers never alias the table look-ups and can keep many look-ups in flight.
+    __shared__ __align__(16) uint2 lut_s[kRwLutBytes / 8];
+    __shared__ __align__(16) uint2 tab[kRwTabBytes / 8];
+    extern __shared__ __align__(16) unsigned char lds[];
+    unsigned char *img0 = lds;
+    unsigned char *bst0 = img0 + 2 * p.img_bytes;
+    int *stage0 = reinterpret_cast<int *>(bst0 + p.nbst * kFragBytes);  // MODE 0 only
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    // The wave index must be visibly uniform: every branch around MFMAs below has to be a scalar branch, because
+    // MFMA ignores EXEC and a masked-off block that is not jumped over would still accumulate.
+    const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const bool producer = wv >= kRwCWaves;
+    const int tw = producer ? wv - kRwCWaves : wv;            // wave inside the team
+    const int ttid = tid - (producer ? 64 * kRwCWaves : 0);   // thread inside the team
     const int li = lane & 15, lg = lane >> 4;
-    const int64_t z = blockIdx.x / (unsigned)p.S;  // member
-    const int row0 = (int)(blockIdx.x - z * p.S) * p.hs;  // first output row of this workgroup
-    const int hloc = p.h - row0 < p.hs ? p.h - row0 : p.hs;  // its output rows
     const int Ow = (p.O + 63) >> 6;
 
-    if (tid < 256)  // expansion table: entry b holds the +-1 bytes of bits 0..7 of b
-        reinterpret_cast<uint2 *>(lds)[tid] = make_uint2(pm1_bytes(tid & 0xFu), pm1_bytes((unsigned)tid >> 4));
-    for (int ti = tid; ti < NK * 16; ti += kMfmaThreads) {  // K-position tables, one entry per thread
-        const int k = 64 * (ti >> 4) + 16 * ((ti >> 2) & 3) + 4 * (ti & 3);
-        int tap = k / p.CB;
-        const int c = k - tap * p.CB;
-        const bool valid = tap < p.taps;
-        tap = valid ? tap : p.taps - 1;  // K padding: the filter side is zero, read any valid pixel
-        const int i = tap / p.fy, j = tap - i * p.fy;
-        tab.koff[ti] = (i * p.RW + j) * p.PS + c;
-        int frow = 0, fsh = 0, flf = 0;
-        if (valid && p.tapT > 1) {
-            // tap t sits at bits in_bits*(t % T) of word t / T; c < in_bits for every position that is asked for
-            // (CB = in_bits rounded up to 4, 8 or a multiple of 16)
-            const int tq = tap / p.tapT;
-            frow = tq;
-            fsh = p.in_bits * (tap - tq * p.tapT) + (c < p.in_bits ? c : 0);
-            flf = c < p.in_bits ? p.in_bits - c : 0;
-        } else if (valid) {
-            frow = tap * p.Cw + (c >> 6);
-            fsh = c & 63;
-            flf = 64;
-        }
-        tab.frow[ti] = (short)frow;
-        tab.fsh[ti] = (unsigned char)fsh;
-        tab.flf[ti] = (unsigned char)flf;
-    }
-    __syncthreads();
-
-    // Filter words of one channel group: wave wv owns fragments wv, wv + waves, ...  The words of group 0 are
-    // requested before the image is touched and those of group cg + 1 before the MFMA loop of group cg, so
-    // their latency never sits on the critical path.
-    constexpr int FPW = (NK * NT + kMfmaWaves - 1) / kMfmaWaves;  // fragments per wave
-    constexpr int LD = PB16 ? 1 : 4;                               // filter words per fragment and lane
-    uint64_t fw[FPW][LD];
-    const uint64_t *fz = p.filt + z * (int64_t)p.frows * p.O;
-    auto load_filter = [&](int n0g) {
-#pragma unroll
-        for (int q = 0; q < FPW; q++) {
-            const int f = wv + kMfmaWaves * q;
-            const int kc = f / NT, nt = f - kc * NT;  // NT is a compile-time constant
-            const int ch = n0g + nt * 16 + li;
-#pragma unroll
-            for (int d = 0; d < LD; d++) {
-                const int ti = f < NK * NT ? (kc * 4 + lg) * 4 + d : 0;
-                const bool need = f < NK * NT && ch < p.O && tab.flf[ti] > 0;
-                fw[q][d] = need ? fz[(int64_t)tab.frow[ti] * p.O + ch] : 0ull;
-            }
-        }
+    // Expansion table: entry b holds the +-1 bytes of bits 0..7 of b.  The expansion work shares the SIMDs' issue
+    // slots with the MFMAs, so it is written for the fewest instructions: two ALU operations and one 8-byte look-up
+    // per 8 bits (bank conflicts between look-ups cost LDS time, which is plentiful, not issue slots).
+    if (tid < 256) lut_s[tid] = make_uint2(rw_pm1_bytes(tid & 0xFu), rw_pm1_bytes((unsigned)tid >> 4));
+    const unsigned char *lutb = reinterpret_cast<const unsigned char *>(lut_s);
+    // bits 16*hi .. 16*hi+15 of x -> 16 bytes of +-1, bit b -> byte b
+    auto expand_half = [&](uint32_t x, int hi) {
+        const uint32_t i0 = hi ? (x >> 13) & 0x7F8u : (x << 3) & 0x7F8u;
+        const uint32_t i1 = hi ? (x >> 21) & 0x7F8u : (x >> 5) & 0x7F8u;
+        const uint2 a = *reinterpret_cast<const uint2 *>(lutb + i0), b = *reinterpret_cast<const uint2 *>(lutb + i1);
+        return make_uint4(a.x, a.y, b.x, b.y);
     };
-    load_filter(0);
 
-    // ---- phase 1: expand the member's image (with border) into LDS -----------------------------------------------
-    // one pixel word per item, 8 items per thread loaded before any is expanded; (row, xx) advance incrementally
-    {
-        const uint64_t *src = p.in + z * (int64_t)p.H * p.Wd * p.Cw;
-        const int npix = (hloc + p.RIN - p.hs) * p.RW;  // RIN = hs + fx - 1 rows at most
-        const int row = tid / p.RW, xx = tid - row * p.RW;
-        for (int cw = 0; cw < p.Cw; cw++) {
-            const int nbits = p.CB - cw * 64 < 64 ? p.CB - cw * 64 : 64;  // positions held by this word
-            int r0 = row, x0 = xx;
-            constexpr int U = 8;
-            for (int pix0 = tid; pix0 < npix; pix0 += kMfmaThreads * U) {
-                uint64_t wd[U];
+    // ---- fragment geometry ---------------------------------------------------------------------------------
+    // chunk kq = i*CPR + q (filter row i) and lane group g: tap column j, first position c0.  Table entry:
+    //   x = byte offset of the filter word holding the group's 16 bits (without the channel),
+    //   y = shift of those bits | mask of the channel bits among them << 8 | (tap column inside the filter) << 31;
+    // a tap column past the filter multiplies by zero bytes, channel positions past in_bits by -1 (they equal the
+    // pixel's zero tail and are part of K).
+    if (tid >= 64 && tid < 64 + NK * 4) {
+        const int e = tid - 64;
+        const int kq = e >> 2, g = e & 3;
+        const int i = kq / CPR, q = kq - i * CPR;
+        int qj = 0, qc = 0;
+        if (p.CB == 32) {
+            qj = 2 * q;
+        } else if (p.CB >= 64) {
+            qj = q / p.Cw;
+            qc = 64 * (q - qj * p.Cw);
+        }
+        const int j = qj + (g >> p.jsh), c0 = qc + 16 * (g & p.cmask);
+        const int tap = i * p.fy + j;
+        const int left = p.in_bits - c0;
+        const int nv = left < 0 ? 0 : (left > 16 ? 16 : left);
+        int fr, sh;
+        if (p.tapT > 0) {
+            fr = (tap * p.tapM) >> 16;  // tap / tapT
+            sh = p.in_bits * (tap - fr * p.tapT) + c0;
+            sh = sh > 63 ? 63 : sh;     // only when nv == 0: the bits are masked off anyway
+        } else {
+            fr = tap * p.Cw + (c0 >> 6);
+            sh = c0 & 63;
+        }
+        const bool inside = j < p.fy;
+        tab[e] = make_uint2(inside ? (uint32_t)(fr * p.O) * 8u : 0u,
+                            (uint32_t)sh | (((1u << nv) - 1u) << 8) | (inside ? 0x80000000u : 0u));
+    }
+    __syncthreads();  // tables complete
+
+    // number of tasks of this workgroup
+    const int64_t nmem = (int64_t)blockIdx.x < p.D ? (p.D - blockIdx.x + gridDim.x - 1) / gridDim.x : 0;
+    const int nsteps = (int)(nmem * p.ncg * p.S);
+
+    if (producer) {
+        // =========================================== producer ===================================================
+        // Team thread ttid owns the items (pixel words) ttid, ttid + 256, ... of a band; all of a band's items are
+        // in flight at once (the host sizes bands so that they fit).  An out-of-range pixel reads word 0 of the
+        // member and is replaced by the zero word.
+        const int pixb = p.Cw * 8, rowb = p.Wd * pixb;  // bytes per pixel / image row
+        const int prow = ttid / p.RW, pxx = ttid - prow * p.RW;
+        // input words of this step's and of the next task, and which of them are inside the image (the others are
+        // replaced by the zero word when they are used, so that nothing waits for a load when it is issued)
+        uint64_t wda[kRwItems], wdb[kRwItems];
+        uint32_t ina = 0, inb_ = 0;
+        uint64_t fw[FPW];
+        int traw = 0;
+        // item u of this thread is pixel ttid + 256*u of the band's LDS image: its row, byte offset relative to the
+        // band's first input row, and whether its column is inside the image
+        int irow[kRwItems], ioff[kRwItems];
+        uint32_t xin = 0;
+        {
+            int r = prow, x = pxx;
 #pragma unroll
-                for (int u = 0; u < U; u++) {
-                    const int yy = row0 + r0 - p.px, xs = x0 - p.py;
-                    const bool inb = yy >= 0 && yy < p.H && xs >= 0 && xs < p.Wd;  // false past the last image row too
-                    wd[u] = inb ? src[((int64_t)yy * p.Wd + xs) * p.Cw + cw] : 0ull;
-                    r0 += p.pix_q;
-                    x0 += p.pix_r;
-                    if (x0 >= p.RW) {
-                        x0 -= p.RW;
-                        r0++;
-                    }
-                }
-#pragma unroll
-                for (int u = 0; u < U; u++) {
-                    const int pix = pix0 + u * kMfmaThreads;
-                    if (pix >= npix) continue;
-                    unsigned char *dst = img + pix * p.PS + cw * 64;
-                    if (nbits >= 16) {
-                        for (int c = 0; c < nbits; c += 16) {
-                            const uint2 lo = lut[(uint32_t)(wd[u] >> c) & 0xFFu];
-                            const uint2 hi = lut[(uint32_t)(wd[u] >> (c + 8)) & 0xFFu];
-                            *reinterpret_cast<uint4 *>(dst + c) = make_uint4(lo.x, lo.y, hi.x, hi.y);
-                        }
-                    } else if (nbits == 8) {
-                        *reinterpret_cast<uint2 *>(dst) = lut[(uint32_t)wd[u] & 0xFFu];
-                    } else {
-                        *reinterpret_cast<uint32_t *>(dst) = lut[(uint32_t)wd[u] & 0xFu].x;
-                    }
+            for (int u = 0; u < kRwItems; u++) {
+                irow[u] = r;
+                ioff[u] = r * rowb + (x - p.py) * pixb;
+                xin |= (x - p.py >= 0 && x - p.py < p.Wd) ? 1u << u : 0u;
+                r += p.pix_q;
+                x += p.pix_r;
+                if (x >= p.RW) {
+                    x -= p.RW;
+                    r++;
                 }
             }
         }
+        auto request = [&](uint64_t (&wd)[kRwItems], uint32_t &inside, const RwTask &t, int cw) {
+            const unsigned char *src = reinterpret_cast<const unsigned char *>(p.in + t.z * (int64_t)p.H * p.Wd * p.Cw);
+            const int y0 = t.band * p.hs - p.px, off0 = y0 * rowb + cw * 8;
+            inside = 0;
+#pragma unroll
+            for (int u = 0; u < kRwItems; u++) {
+                const bool inb = ((xin >> u) & 1u) && (unsigned)(y0 + irow[u]) < (unsigned)p.H;  // false past the last row too
+                wd[u] = *reinterpret_cast<const uint64_t *>(src + (uint32_t)(inb ? off0 + ioff[u] : 0));
+                inside |= inb ? 1u << u : 0u;
+            }
+        };
+        // Filter words of a channel group: wave tw takes fragments tw, tw+4, ... (fragment f = chunk f/NT, channel
+        // tile f%NT).  Every address is valid (channels past O read channel O-1, dead tap columns word 0); the
+        // expansion zeroes them.
+        auto request_filter = [&](const RwTask &t) {
+            const unsigned char *fz = reinterpret_cast<const unsigned char *>(p.filt + t.z * (int64_t)p.fwords);
+            const int n0 = t.cg * 16 * NT * p.cgt;
+            const int nft = NF * p.cgt;  // fragments of the task: f = (channel tile * NK + chunk) * NT + 16-channel piece
+#pragma unroll
+            for (int i = 0; i < FPW; i++) {
+                const int f = tw + kRwPWaves * i;  // uniform
+                const int fc = f < nft ? f : 0;
+                const int ct = fc / NF, r = fc - ct * NF, kq = r / NT, nt = r - kq * NT;
+                const int ch = n0 + (ct * NT + nt) * 16 + li;
+                fw[i] = *reinterpret_cast<const uint64_t *>(fz + (tab[kq * 4 + lg].x + (uint32_t)(ch < p.O ? ch : p.O - 1) * 8u));
+            }
+            if (MODE != 0) {
+                const int ch = n0 + ttid;
+                traw = p.thresh[t.z * p.O + (ch < p.O ? ch : p.O - 1)];
+            }
+        };
+        RwTask cur{(int64_t)blockIdx.x, 0, 0};
+        if (nsteps > 0) {
+            request_filter(cur);
+            request(wda, ina, cur, 0);
+        }
+        int nb = 0;      // fragment sets staged so far
+        int imgseq = 0;  // images expanded so far; image i sits in buffer i & 1
+        // One step: `wd` holds the input words of task k (requested a step ago); those of task k+1 go to `wn` first
+        // thing, so that their latency hides behind this step's work.
+        auto step = [&](int k, uint64_t (&wd)[kRwItems], uint32_t &wdin, uint64_t (&wn)[kRwItems], uint32_t &wnin) {
+            if (k < nsteps) {
+                RwTask nxt = cur;
+                rw_next(nxt, p);
+                const bool more = k + 1 < nsteps;
+                if (more && (p.S > 1 || nxt.cg == 0)) request(wn, wnin, nxt, 0);
+                const int n0 = cur.cg * 16 * NT * p.cgt;
+                if (cur.band == 0) {
+                    // ---- new (member, channel group): fragments and thresholds -> staging area -------------------
+                    unsigned char *bst = bst0 + (nb % p.nbst) * kFragBytes;
+                    nb++;
+#pragma unroll
+                    for (int i = 0; i < FPW; i++) {
+                        const int f = tw + kRwPWaves * i;
+                        if (f < NF * p.cgt) {  // uniform
+                            const int ct = f / NF, r = f - ct * NF, kq = r / NT, nt = r - kq * NT;
+                            const uint32_t e = tab[kq * 4 + lg].y;
+                            const uint32_t sh = e & 63u, vmask = (e >> 8) & 0xFFFFu;
+                            const bool live = (int)e < 0 && n0 + (ct * NT + nt) * 16 + li < p.O;
+                            const uint4 e16 = expand_half((uint32_t)(fw[i] >> sh) & vmask, 0);
+                            *reinterpret_cast<uint4 *>(bst + (f * 64 + lane) * 16) = live ? e16 : make_uint4(0u, 0u, 0u, 0u);
+                        }
+                    }
+                    // thresholds in dot-product terms: 2*popc > t  <=>  popc > (t>>1)  <=>  dot < K - 2*(t>>1)
+                    if (MODE != 0 && ttid < 64) {
+                        int64_t td = n0 + ttid < p.O ? (int64_t)p.K - 2 * (int64_t)(traw >> 1) : -2147483648LL;
+                        td = td > 2147483647LL ? 2147483647LL : (td < -2147483648LL ? -2147483648LL : td);
+                        reinterpret_cast<int *>(bst + NF * CGTMAX * 1024)[ttid] = (int)td;
+                    }
+                }
+                // the filter words of the next task get the whole image expansion as a head start
+                if (more && nxt.band == 0) request_filter(nxt);
+                // ---- input words -> +-1 bytes in an image buffer (kept when only the channel group changed) ---------
+                if (k == 0 || p.S > 1 || cur.cg == 0) {
+                    unsigned char *img = img0 + (imgseq & 1) * p.img_bytes;
+                    imgseq++;
+                    const int row0 = cur.band * p.hs;
+                    const int hloc = p.h - row0 < p.hs ? p.h - row0 : p.hs;
+                    const int npix = (hloc + FX - 1) * p.RW;
+                    for (int cw = 0; cw < p.Cw; cw++) {
+                        if (cw > 0) request(wd, wdin, cur, cw);
+                        const int nbytes = p.CB - cw * 64 < 64 ? p.CB - cw * 64 : 64;  // positions held by this word
+                        unsigned char *dst = img + __mul24(ttid, p.PS) + cw * 64;
+                        const int dstep = kRwTeam * p.PS;
+#pragma unroll
+                        for (int u = 0; u < kRwItems; u++) {
+                            if (ttid + u * kRwTeam < npix) {
+                                const bool inside = (wdin >> u) & 1u;
+                                const uint32_t lo = inside ? (uint32_t)wd[u] : 0u, hi = inside ? (uint32_t)(wd[u] >> 32) : 0u;
+#pragma unroll
+                                for (int c = 0; c < 4; c++)
+                                    if (16 * c < nbytes)  // uniform
+                                        *reinterpret_cast<uint4 *>(dst + 16 * c) = expand_half(c < 2 ? lo : hi, c & 1);
+                            }
+                            dst += dstep;
+                        }
+                    }
+                }
+                cur = nxt;
+            }
+            __syncthreads();
+        };
+        for (int k = 0; k <= nsteps; k += 2) {
+            step(k, wda, ina, wdb, inb_);
+            if (k + 1 <= nsteps) step(k + 1, wdb, inb_, wda, ina);
+        }
+        return;
     }
 
-    // per-lane K offsets into the LDS image
-    int koff[NK][PB16 ? 1 : 4];
+    // ============================================= consumer =====================================================
+    int koff[CPR];  // byte offset of the lane's 16 positions relative to the strip's first pixel
 #pragma unroll
-    for (int kc = 0; kc < NK; kc++)
+    for (int q = 0; q < CPR; q++) {
+        const int j = p.qj[q] + (lg >> p.jsh);
+        koff[q] = __mul24((j < p.fy ? j : 0) + li, p.PS) + p.qc[q] + 16 * (lg & p.cmask);
+    }
+    v4i B[NK][NT];
+    int tdot[NT];
 #pragma unroll
-        for (int d = 0; d < (PB16 ? 1 : 4); d++) koff[kc][d] = tab.koff[(kc * 4 + lg) * 4 + d];
-
-    const int mtiles = hloc * p.ntx;
-    const int ngroups = (p.O + 16 * NT - 1) / (16 * NT);
-    for (int cg = 0; cg < ngroups; cg++) {
-        const int n0g = cg * 16 * NT;  // first channel of this group
-        __syncthreads();               // image complete / previous group's use of the fragment area finished
-        // ---- phase 2: expand the prefetched filter words of this channel group into fragments ------------------
+    for (int kq = 0; kq < NK; kq++)
 #pragma unroll
-        for (int q = 0; q < FPW; q++) {
-            const int f = wv + kMfmaWaves * q;
-            if (f >= NK * NT) continue;  // wave-uniform
-            const int kc = f / NT, nt = f - kc * NT;
-            const bool chv = n0g + nt * 16 + li < p.O;
-            uint32_t e[4];
-            if (PB16) {
-                const int ti = (kc * 4 + lg) * 4;
-                const int left = chv ? tab.flf[ti] : 0;  // valid bits from this position on (0: multiply by zero)
-                uint32_t h16 = (uint32_t)(fw[q][0] >> tab.fsh[ti]) & 0xFFFFu;
-                h16 = left >= 16 ? h16 : h16 & ((1u << left) - 1);
-                const uint2 lo = lut[h16 & 0xFFu], hi = lut[h16 >> 8];
-                e[0] = left > 0 ? lo.x : 0u;
-                e[1] = left > 0 ? lo.y : 0u;
-                e[2] = left > 0 ? hi.x : 0u;
-                e[3] = left > 0 ? hi.y : 0u;
-            } else {
+        for (int nt = 0; nt < NT; nt++) B[kq][nt] = (v4i){0, 0, 0, 0};
 #pragma unroll
-                for (int d = 0; d < 4; d++) {
-                    const int ti = (kc * 4 + lg) * 4 + d;
-                    const int left = chv ? tab.flf[ti] : 0;
-                    uint32_t nib = (uint32_t)(fw[q][d] >> tab.fsh[ti]) & 0xFu;
-                    nib = left >= 4 ? nib : nib & ((1u << left) - 1);
-                    e[d] = left > 0 ? lut[nib].x : 0u;
-                }
-            }
-            *reinterpret_cast<uint4 *>(bfr + (f * 64 + lane) * 16) = make_uint4(e[0], e[1], e[2], e[3]);
-        }
-        __syncthreads();
-        v4i B[NK][NT];
+    for (int nt = 0; nt < NT; nt++) tdot[nt] = 0;
+    int *stage = stage0 + tw * (16 * 16 * NT);  // MODE 0 only
+    // Wave tw always works on channel tile ct of a task (so its fragments stay valid over a member's bands) and
+    // shares the (strip, sub-band) units of that tile with the other waves of the same tile.
+    const int ct = tw % p.cgt, uw = tw / p.cgt, ustep = kRwCWaves / p.cgt;
+    const int nunits = p.ntx * p.nsub;
+    RwTask cur{(int64_t)blockIdx.x, 0, 0};
+    int nb = 0, imgseq = 0;
+    for (int k = 0; k <= nsteps; k++) {
+        if (k > 0) {
+            // task k-1: image number imgseq, new fragments in staging area nb % nbst
+            const int64_t z = cur.z;
+            const int cg = cur.cg;
+            const int n0 = (cg * p.cgt + ct) * 16 * NT;  // first channel of the wave's tile
+            const int row0 = cur.band * p.hs;
+            const int hloc = p.h - row0 < p.hs ? p.h - row0 : p.hs;
+            if (k == 1 || p.S > 1 || cg == 0) imgseq++;
+            const unsigned char *img = img0 + ((imgseq - 1) & 1) * p.img_bytes;
+            if (cur.band == 0) {
+                const unsigned char *bst = bst0 + (nb % p.nbst) * kFragBytes;
+                nb++;
 #pragma unroll
-        for (int kc = 0; kc < NK; kc++)
-#pragma unroll
-            for (int nt = 0; nt < NT; nt++)
-                B[kc][nt] = *reinterpret_cast<const v4i *>(bfr + ((kc * NT + nt) * 64 + lane) * 16);
-        if (MODE == 0) __syncthreads();  // the staging tiles below overwrite the fragment area
-
-        // thresholds in dot-product terms: 2*popc > t  <=>  popc > (t>>1)  <=>  dot < K - 2*(t>>1)
-        int tdot[NT];
-        if (MODE != 0) {
-#pragma unroll
-            for (int nt = 0; nt < NT; nt++) {
-                const int ch = n0g + nt * 16 + li;
-                int64_t td = ch < p.O ? (int64_t)p.K - 2 * (int64_t)(p.thresh[z * p.O + ch] >> 1) : -2147483648LL;
-                td = td > 2147483647LL ? 2147483647LL : (td < -2147483648LL ? -2147483648LL : td);
-                tdot[nt] = (int)td;
-            }
-        }
-
-        if (cg + 1 < ngroups) load_filter(n0g + 16 * NT);
-
-        // ---- phase 3: MT pixel tiles x NT channel tiles per wave and step ---------------------------------------
-        // tile t = ty * ntx + txi; the wave's first tile of a step advances by kMfmaWaves*MT tiles
-        int sty = (wv * MT) / p.ntx, stx = wv * MT - sty * p.ntx;
-        for (int t0 = wv * MT; t0 < mtiles; t0 += kMfmaWaves * MT) {
-            int tbase[MT], ty[MT], tx[MT];
-            {
-                int cy = sty, cx = stx;
-#pragma unroll
-                for (int mt = 0; mt < MT; mt++) {
-                    const bool live = t0 + mt < mtiles;
-                    ty[mt] = live ? cy : 0;  // dead tiles compute on tile 0 and are dropped below
-                    tx[mt] = live ? cx * 16 : 0;
-                    tbase[mt] = (ty[mt] * p.RW + tx[mt] + li) * p.PS;
-                    if (++cx == p.ntx) {
-                        cx = 0;
-                        cy++;
-                    }
-                }
-                sty += p.step_q;
-                stx += p.step_r;
-                if (stx >= p.ntx) {
-                    stx -= p.ntx;
-                    sty++;
-                }
-            }
-            v4i acc[MT][NT];
-#pragma unroll
-            for (int mt = 0; mt < MT; mt++)
-#pragma unroll
-                for (int nt = 0; nt < NT; nt++) acc[mt][nt] = (v4i){0, 0, 0, 0};
-#pragma unroll
-            for (int kc = 0; kc < NK; kc++) {
-                v4i A[MT];
-#pragma unroll
-                for (int mt = 0; mt < MT; mt++) {
-                    if (PB16) {
-                        A[mt] = *reinterpret_cast<const v4i *>(img + tbase[mt] + koff[kc][0]);
-                    } else {
-#pragma unroll
-                        for (int d = 0; d < 4; d++)
-                            A[mt][d] = *reinterpret_cast<const int *>(img + tbase[mt] + koff[kc][PB16 ? 0 : d]);
-                    }
-                }
-#pragma unroll
-                for (int mt = 0; mt < MT; mt++)
+                for (int kq = 0; kq < NK; kq++)
 #pragma unroll
                     for (int nt = 0; nt < NT; nt++)
-                        acc[mt][nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[mt], B[kc][nt], acc[mt][nt], 0, 0, 0);
-            }
-            // ---- epilogue of the step ----------------------------------------------------------------------
+                        B[kq][nt] = *reinterpret_cast<const v4i *>(bst + (((ct * NK + kq) * NT + nt) * 64 + lane) * 16);
+                if (MODE != 0) {
 #pragma unroll
-            for (int mt = 0; mt < MT; mt++) {
-                if (t0 + mt >= mtiles) continue;  // wave-uniform
+                    for (int nt = 0; nt < NT; nt++)
+                        tdot[nt] = reinterpret_cast<const int *>(bst + NF * CGTMAX * 1024)[(ct * NT + nt) * 16 + li];
+                }
+            }
+            for (int u = uw; u < nunits; u += ustep) {
+                const int sub = u / p.ntx, strip = u - sub * p.ntx;
+                const int ys = sub * p.hb;
+                const int ye = ys + p.hb < hloc ? ys + p.hb : hloc;
+                if (ys >= ye) continue;  // wave-uniform
+                const int x0 = strip * 16;
+
+            int pend[NT][2];  // MODE 3: x-pooled minima of the even row of a pair
+#pragma unroll
+            for (int nt = 0; nt < NT; nt++) pend[nt][0] = pend[nt][1] = 0;
+
+            // ---- epilogue of one finished output row (band-relative y) -------------------------------------------
+            // Output addresses: a uniform row pointer (scalar arithmetic) plus a per-lane 32-bit byte offset.
+            unsigned char *obase;   // first element of the strip's row 0 (band-relative) for this channel group
+            int64_t orowb;          // bytes from one (pooled) output row to the next
+            uint32_t olane[MODE == 0 ? 16 / (64 / (4 * NT)) : 1];
+            bool olive[MODE == 0 ? 16 / (64 / (4 * NT)) : 1];
+            const bool piece = p.O >= 64;  // the tile's 16*NT bits are one of several pieces of the pixel's word(s)
+            if (MODE == 0) {
+                constexpr int LPP = 4 * NT, PPI = 64 / LPP;  // lanes per pixel (one int4 each), pixels per store
+                obase = static_cast<unsigned char *>(p.out) + ((((z * p.h + row0) * (int64_t)p.w + x0) * p.O + n0) << 2);
+                orowb = ((int64_t)p.w * p.O) << 2;
+#pragma unroll
+                for (int s = 0; s < 16 / PPI; s++) {
+                    const int pi = s * PPI + lane / LPP, c4 = (lane % LPP) * 4;
+                    olane[s] = (uint32_t)(__mul24(pi, p.O) + c4) << 2;
+                    olive[s] = x0 + pi < p.w && n0 + c4 < p.O;
+                }
+            } else {
+                const int hh = MODE == 3 ? p.h >> 1 : p.h, ww = MODE == 3 ? p.w >> 1 : p.w;
+                const int r0 = MODE == 3 ? row0 >> 1 : row0, xx0 = MODE == 3 ? x0 >> 1 : x0;
+                const int64_t e0 = ((z * hh + r0) * (int64_t)ww + xx0) * Ow;  // word index of the strip's first pixel
+                obase = static_cast<unsigned char *>(p.out) + (piece ? ((e0 + cg) << 3) + 2 * NT * ct : e0 << 3);
+                orowb = ((int64_t)ww * Ow) << 3;
+                olane[0] = (uint32_t)__mul24(lane, Ow) << 3;
+                olive[0] = lane < (MODE == 3 ? 8 : 16) && xx0 + lane < ww;
+            }
+            auto finish_row = [&](v4i (&a)[NT], int y) {
                 if (MODE == 0) {
                     // stage the 16 x (16*NT) tile in LDS, then store whole pixel rows (non-temporal)
-                    int *stage = reinterpret_cast<int *>(obuf) + wv * (16 * 16 * NT);
 #pragma unroll
                     for (int nt = 0; nt < NT; nt++)
 #pragma unroll
-                        for (int r = 0; r < 4; r++)
-                            stage[(4 * lg + r) * (16 * NT) + nt * 16 + li] = (p.K - acc[mt][nt][r]) >> 1;
+                        for (int r = 0; r < 4; r++) stage[(4 * lg + r) * (16 * NT) + nt * 16 + li] = (p.K - a[nt][r]) >> 1;
                     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
                     __builtin_amdgcn_wave_barrier();
                     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-                    int32_t *o32 = static_cast<int32_t *>(p.out);
-                    constexpr int LPP = 4 * NT;    // lanes per pixel, one int4 each
-                    constexpr int PPI = 64 / LPP;  // pixels per store instruction
-                    int32_t *orow = o32 + ((z * p.h + row0 + ty[mt]) * (int64_t)p.w + tx[mt]) * p.O + n0g;
+                    constexpr int LPP = 4 * NT, PPI = 64 / LPP;
+                    unsigned char *orow = obase + y * orowb;
 #pragma unroll
                     for (int s = 0; s < 16 / PPI; s++) {
                         const int pi = s * PPI + lane / LPP, c4 = (lane % LPP) * 4;
-                        if (tx[mt] + pi < p.w && n0g + c4 < p.O) {
+                        if (olive[s]) {
                             const nb_i32x4 v = *reinterpret_cast<const nb_i32x4 *>(stage + pi * (16 * NT) + c4);
-                            __builtin_nontemporal_store(v, reinterpret_cast<nb_i32x4 *>(orow + (int64_t)pi * p.O + c4));
+                            __builtin_nontemporal_store(v, reinterpret_cast<nb_i32x4 *>(orow + olane[s]));
                         }
                     }
                     __builtin_amdgcn_wave_barrier();
-                } else {
-                    // ballot r of lane (pixel 4*lg+r, channel li): bits 16*g.. are the 16-channel piece of pixel
-                    // 4*g+r.  Lane j < 16 extracts the piece of pixel j and writes it.
-                    uint16_t *ob16 = reinterpret_cast<uint16_t *>(obuf);
+                    return;
+                }
+                uint64_t word = 0;
+                if (MODE == 2) {
+                    // ballot r of lane (pixel 4*g+r, channel li): bits 16*g.. are the 16-channel piece of pixel 4*g+r.
+                    // Lane j < 16 assembles the pieces of pixel j over the NT channel tiles and writes them.
 #pragma unroll
                     for (int nt = 0; nt < NT; nt++) {
                         uint64_t m[4];
 #pragma unroll
-                        for (int r = 0; r < 4; r++) m[r] = __ballot(acc[mt][nt][r] < tdot[nt]);
-                        const int r = lane & 3;
-                        const uint64_t mine = r == 0 ? m[0] : r == 1 ? m[1] : r == 2 ? m[2] : m[3];
-                        const uint32_t piece16 = (uint32_t)(mine >> (16 * ((lane >> 2) & 3))) & 0xFFFFu;
-                        const int x = tx[mt] + lane;  // lanes 0..15 <-> the tile's 16 pixels
-                        if (lane < 16 && x < p.w)
-                            ob16[((ty[mt] * p.w + x) * Ow) * 4 + (n0g >> 4) + nt] = (uint16_t)piece16;
+                        for (int r = 0; r < 4; r++) m[r] = __ballot(a[nt][r] < tdot[nt]);
+                        const uint64_t mine = rw_sel4(lane & 3, m[0], m[1], m[2], m[3]);
+                        word |= ((mine >> (16 * ((lane >> 2) & 3))) & 0xFFFFull) << (16 * nt);
+                    }
+                } else {
+                    // pixels 4g, 4g+1 and 4g+2, 4g+3 pool in x; rows y (even) and y+1 pool in y
+                    if ((y & 1) == 0) {
+#pragma unroll
+                        for (int nt = 0; nt < NT; nt++) {
+                            pend[nt][0] = a[nt][0] < a[nt][1] ? a[nt][0] : a[nt][1];
+                            pend[nt][1] = a[nt][2] < a[nt][3] ? a[nt][2] : a[nt][3];
+                        }
+                        return;
+                    }
+#pragma unroll
+                    for (int nt = 0; nt < NT; nt++) {
+                        int v0 = a[nt][0] < a[nt][1] ? a[nt][0] : a[nt][1];
+                        int v1 = a[nt][2] < a[nt][3] ? a[nt][2] : a[nt][3];
+                        v0 = v0 < pend[nt][0] ? v0 : pend[nt][0];
+                        v1 = v1 < pend[nt][1] ? v1 : pend[nt][1];
+                        const uint64_t m0 = __ballot(v0 < tdot[nt]), m1 = __ballot(v1 < tdot[nt]);
+                        const uint64_t mine = (lane & 1) ? m1 : m0;  // pooled pixel 2g + q <-> lane 2g + q
+                        word |= ((mine >> (16 * ((lane >> 1) & 3))) & 0xFFFFull) << (16 * nt);
                     }
                 }
-            }
-        }
-    }
+                unsigned char *orow = obase + (MODE == 3 ? y >> 1 : y) * orowb;
+                if (olive[0]) {
+                    if (piece && NT == 1) {
+                        *reinterpret_cast<uint16_t *>(orow + olane[0]) = (uint16_t)word;
+                    } else if (piece) {
+                        *reinterpret_cast<uint32_t *>(orow + olane[0]) = (uint32_t)word;
+                    } else {
+                        *reinterpret_cast<uint64_t *>(orow + olane[0]) = word;
+                    }
+                }
+            };
 
-    // ---- phase 4 (packed modes): write the member's packed map, optionally 2x2 OR-pooled ----------------------
-    if (MODE != 0) {
-        __syncthreads();
-        const uint64_t *ob = reinterpret_cast<const uint64_t *>(obuf);
-        uint64_t *o64 = static_cast<uint64_t *>(p.out);
-        // 16-bit pieces of channels past O in the last word were never written: mask them off
-        const int lastv = p.O - 64 * (Ow - 1);
-        const uint64_t lastmask = lastv >= 64 ? ~0ull : ((1ull << lastv) - 1);
-        if (MODE == 2) {
-            const int total = hloc * p.w * Ow;
-            uint64_t *dst = o64 + (z * p.h + row0) * (int64_t)p.w * Ow;
-            int wi = tid % Ow;
-            const int dwi = kMfmaThreads % Ow;
-            for (int i = tid; i < total; i += kMfmaThreads) {
-                dst[i] = ob[i] & (wi == Ow - 1 ? lastmask : ~0ull);
-                wi += dwi;
-                wi = wi >= Ow ? wi - Ow : wi;
+            // ---- walk down the strip: image row rr (band-relative) feeds output rows rr, rr-1, rr-2 --------------
+            // a0 holds the partial sums of output row rr-2 (two filter rows done), a1 those of row rr-1 (one done).
+            // Image row rr completes row rr-2 (emitted), continues row rr-1 and opens row rr with a zero C operand,
+            // so nothing is ever cleared or rotated.  Rows rr in [ys+2, ye) take the branch-free loop.
+            const unsigned char *arow = img + (ys * p.RW + x0) * p.PS;
+            const int rowbytes = p.RW * p.PS;
+            const int rend = ye + FX - 1;
+            const int ylast = MODE == 3 ? (p.h & ~1) - row0 : ye;  // pooled maps drop an odd last row
+            v4i F[CPR], a0[NT], a1[NT];
+#pragma unroll
+            for (int q = 0; q < CPR; q++) F[q] = *reinterpret_cast<const v4i *>(arow + koff[q]);
+#pragma unroll
+            for (int nt = 0; nt < NT; nt++) a0[nt] = a1[nt] = (v4i){0, 0, 0, 0};
+            auto edge_step = [&](int rr) {  // first two and last two image rows of the sub-band: some parts are missing
+                v4i Fn[CPR];
+                arow += rowbytes;
+#pragma unroll
+                for (int q = 0; q < CPR; q++) Fn[q] = F[q];
+                if (rr + 1 < rend) {
+#pragma unroll
+                    for (int q = 0; q < CPR; q++) Fn[q] = *reinterpret_cast<const v4i *>(arow + koff[q]);
+                }
+                if (rr - 2 >= ys) {
+#pragma unroll
+                    for (int q = 0; q < CPR; q++)
+#pragma unroll
+                        for (int nt = 0; nt < NT; nt++)
+                            a0[nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(F[q], B[2 * CPR + q][nt], a0[nt], 0, 0, 0);
+                    if (rr - 2 < ylast) finish_row(a0, rr - 2);
+                }
+                if (rr - 1 >= ys && rr - 1 < ye) {
+#pragma unroll
+                    for (int nt = 0; nt < NT; nt++) a0[nt] = a1[nt];
+#pragma unroll
+                    for (int q = 0; q < CPR; q++)
+#pragma unroll
+                        for (int nt = 0; nt < NT; nt++)
+                            a0[nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(F[q], B[CPR + q][nt], a0[nt], 0, 0, 0);
+                }
+                if (rr < ye) {
+#pragma unroll
+                    for (int nt = 0; nt < NT; nt++) a1[nt] = (v4i){0, 0, 0, 0};
+#pragma unroll
+                    for (int q = 0; q < CPR; q++)
+#pragma unroll
+                        for (int nt = 0; nt < NT; nt++)
+                            a1[nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(F[q], B[q][nt], a1[nt], 0, 0, 0);
+                }
+#pragma unroll
+                for (int q = 0; q < CPR; q++) F[q] = Fn[q];
+            };
+            int rr = ys;
+            const int lead = ys + 2 < rend ? ys + 2 : rend;
+            for (; rr < lead; rr++) edge_step(rr);
+            for (; rr < ye; rr++) {
+                v4i Fn[CPR], done[NT];
+                arow += rowbytes;
+#pragma unroll
+                for (int q = 0; q < CPR; q++) Fn[q] = *reinterpret_cast<const v4i *>(arow + koff[q]);
+#pragma unroll
+                for (int nt = 0; nt < NT; nt++) done[nt] = a0[nt];
+#pragma unroll
+                for (int q = 0; q < CPR; q++)
+#pragma unroll
+                    for (int nt = 0; nt < NT; nt++)
+                        done[nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(F[q], B[2 * CPR + q][nt], done[nt], 0, 0, 0);
+#pragma unroll
+                for (int nt = 0; nt < NT; nt++) a0[nt] = a1[nt];
+#pragma unroll
+                for (int q = 0; q < CPR; q++)
+#pragma unroll
+                    for (int nt = 0; nt < NT; nt++)
+                        a0[nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(F[q], B[CPR + q][nt], a0[nt], 0, 0, 0);
+#pragma unroll
+                for (int nt = 0; nt < NT; nt++) a1[nt] = (v4i){0, 0, 0, 0};
+#pragma unroll
+                for (int q = 0; q < CPR; q++)
+#pragma unroll
+                    for (int nt = 0; nt < NT; nt++)
+                        a1[nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(F[q], B[q][nt], a1[nt], 0, 0, 0);
+                finish_row(done, rr - 2);  // rr - 2 < ye - 2 <= ylast
+#pragma unroll
+                for (int q = 0; q < CPR; q++) F[q] = Fn[q];
             }
-        } else {
-            const int h2 = hloc >> 1, w2 = p.w >> 1;  // row0 is even: hs is
-            const int total = h2 * w2 * Ow;
-            uint64_t *dst = o64 + (z * (p.h >> 1) + (row0 >> 1)) * (int64_t)w2 * Ow;
-            for (int i = tid; i < total; i += kMfmaThreads) {
-                const int q = i / Ow, wi = i - q * Ow;
-                const int qy = q / w2, qx = q - qy * w2;
-                const int b0 = ((2 * qy) * p.w + 2 * qx) * Ow + wi;
-                const uint64_t v = ob[b0] | ob[b0 + Ow] | ob[b0 + p.w * Ow] | ob[b0 + p.w * Ow + Ow];
-                dst[i] = v & (wi == Ow - 1 ? lastmask : ~0ull);
+            for (; rr < rend; rr++) edge_step(rr);
             }
+            rw_next(cur, p);
         }
+        __syncthreads();
     }
 }
 
-static inline int round_up(int a, int b) { return (a + b - 1) / b * b; }
+static inline int rw_round_up(int a, int b) { return (a + b - 1) / b * b; }
 
-// Returns false when the launch could not be set up (the caller then uses the XOR-popcount path).
-template <int NK, int NT, int MODE, bool PB16>
-static bool launch_one(const MfmaConv &p, int64_t D, size_t lds_bytes, hipStream_t s)
+// Workgroups per CU that fit by registers (eight waves each) and LDS, and the CU count of the current device.
+struct RwFit {
+    int cus, regs;
+};
+template <int CPR, int NT, int MODE>
+static bool rw_launch_one(const RwConv &p, int64_t D, size_t lds_bytes, hipStream_t s)
 {
-    static bool attr_set = false;  // benign race: setting the same attribute twice is harmless
-    auto *kfn = conv_mfma_kernel<NK, NT, MODE, PB16, mfma_mt(NK, NT)>;
-    if (!attr_set) {
+    static RwFit fit = {0, 0};  // benign race: every thread computes the same values
+    auto *kfn = conv_mfma_kernel<CPR, NT, MODE>;
+    if (fit.cus == 0) {
+        hipFuncAttributes fa;
+        int dev = 0, cus = 0;
         if (hipFuncSetAttribute(reinterpret_cast<const void *>(kfn), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                160 * 1024) != hipSuccess) {
+                                kRwMaxDynLds) != hipSuccess ||
+
+            hipFuncGetAttributes(&fa, reinterpret_cast<const void *>(kfn)) != hipSuccess ||
+            hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1) {
             (void)hipGetLastError();
             return false;
         }
-        attr_set = true;
+        fit.regs = fa.numRegs > 0 ? fa.numRegs : 256;
+        fit.cus = cus;
     }
-    kfn<<<dim3((unsigned)(D * p.S)), dim3(kMfmaThreads), lds_bytes, s>>>(p);
+    // 512 registers per lane and SIMD, three waves of a workgroup per SIMD; 160 KB of LDS per CU
+    int per_cu = 512 / ((fit.regs + 7) / 8 * 8) / 3;
+    const int by_lds = (int)(160 * 1024 / (lds_bytes + kRwLutBytes + kRwTabBytes));
+    per_cu = per_cu < by_lds ? per_cu : by_lds;
+    per_cu = per_cu < 1 ? 1 : (per_cu > 4 ? 4 : per_cu);
+    const int64_t wgs = D < (int64_t)fit.cus * per_cu ? D : (int64_t)fit.cus * per_cu;
+    kfn<<<dim3((unsigned)wgs), dim3(kRwThreads), lds_bytes, s>>>(p);
     return true;
 }
 
 template <int MODE>
-static bool launch_mode(const MfmaConv &p, int64_t D, int NK, int NT, bool pb16, size_t lds, hipStream_t s)
+static bool rw_launch_mode(const RwConv &p, int64_t D, int CPR, int NT, size_t lds, hipStream_t s)
 {
-#define NB_MFMA(nk, nt)                                                           \
-    if (NK == nk && NT == nt)                                                     \
-        return pb16 ? launch_one<nk, nt, MODE, true>(p, D, lds, s) : launch_one<nk, nt, MODE, false>(p, D, lds, s)
-#define NB_MFMA16(nk, nt) \
-    if (NK == nk && NT == nt && pb16) return launch_one<nk, nt, MODE, true>(p, D, lds, s)
-    NB_MFMA(1, 4);
-    NB_MFMA(1, 1);
-    NB_MFMA(3, 1);
-    NB_MFMA(3, 4);
-    NB_MFMA16(9, 4);  // pixels narrower than 16 positions never reach 9 chunks with the usual filter sizes
-    NB_MFMA16(9, 1);
-    NB_MFMA16(18, 2);
-#undef NB_MFMA16
-#undef NB_MFMA
+#define NB_RW(cpr, nt) \
+    if (CPR == cpr && NT == nt) return rw_launch_one<cpr, nt, MODE>(p, D, lds, s)
+    NB_RW(1, 1);
+    NB_RW(1, 2);
+    NB_RW(2, 1);
+    NB_RW(2, 2);
+    NB_RW(3, 1);
+    NB_RW(3, 2);
+    NB_RW(6, 1);
+#undef NB_RW
     return false;
 }
 
-// mode as in conv_impl (0 int32, 2 packed, 3 packed+pooled).  in_bits = true channel count if known, else 0.
-// Returns false when this shape has no matrix-core kernel or, unless force is set, when the XOR-popcount
-// kernels measured faster on shapes of its kind; nothing has been launched then.
+// mode as in conv_impl (0 int32, 2 packed, 3 packed+pooled).  tap_bits > 0: the filter is tap-packed and the
+// input has tap_bits true channels in one word per pixel.  Returns false when this shape has no kernel here;
+// nothing has been launched then.
 bool conv_mfma_try(void *out, const uint64_t *in, const uint64_t *filt, const int32_t *thresh, const ConvGeom &g,
-                   int64_t D, int O, int in_bits, bool filter_tap_packed, int mode, bool force, hipStream_t s)
+                 int64_t D, int O, int tap_bits, int mode, hipStream_t s)
 {
     if (!aligned(out, 16)) return false;
     if (mode != 0 && mode != 2 && mode != 3) return false;
-    if (g.sx != 1 || g.sy != 1 || g.h < 1 || g.w < 1 || D < 1 || D > kMaxBlocks) return false;
-    if (O < 1 || (O & 15) != 0) return false;
+    if (g.sx != 1 || g.sy != 1 || g.h < 1 || g.w < 1 || D < 1) return false;
+    if (g.fx != 3 || g.fy < 1 || g.fy > 3 || g.Cw < 1) return false;
+    if (O < 16 || (O & 15) != 0) return false;
     if (mode == 3 && (g.h < 2 || g.w < 2)) return false;
-    if (filter_tap_packed && (in_bits < 1 || g.Cw != 1)) return false;
-    MfmaConv p;
+    if (tap_bits > 0 && (g.Cw != 1 || tap_bits > 32)) return false;
+    // 32-bit byte offsets inside one member's image and filter block
+    if ((int64_t)g.H * g.Wd * g.Cw * 8 >= (1LL << 31) || (int64_t)9 * g.Cw * O * 8 >= (1LL << 31)) return false;
+    RwConv p;
     p.in = in;
     p.filt = filt;
     p.thresh = thresh;
     p.out = out;
     p.H = g.H; p.Wd = g.Wd; p.Cw = g.Cw; p.px = g.px; p.py = g.py; p.h = g.h; p.w = g.w;
     p.O = O;
-    const int taps = g.fx * g.fy;
-    const int tapT = filter_tap_packed ? 64 / in_bits : 1;
-    int CB = g.Cw * 64;
-    if (in_bits > 0 && g.Cw == 1) CB = round_up(in_bits, 4);
-    if (CB != 4 && CB != 8 && (CB & 15) != 0) CB = round_up(CB, 16);
-    if (CB > g.Cw * 64) return false;
-    p.CB = CB;
-    const bool pb16 = (CB & 15) == 0;
-    p.PS = CB > 32 ? CB + 16 : CB;
-    p.ntx = (g.w + 15) / 16;
-    p.RW = round_up(16 * p.ntx + g.fy - 1, 4);
-    p.K = taps * CB;
-    p.frows = filter_tap_packed ? (taps + tapT - 1) / tapT : taps * g.Cw;
-    if (p.frows > 32767) return false;
-    const int NK = (p.K + 63) / 64;
-    if (NK > kMaxNK) return false;
-    int NT = O >= 64 ? 4 : (O == 16 ? 1 : 0);
-    if (NK == 18) NT = O >= 32 ? 2 : 0;
-    if (NT == 0) return false;
-    // Measured on MI355X (64-bit words, 3x3 filters, 1024-4096 members): the per-member set-up (image and filter
-    // expansion) is paid back from 32x32 output pixels on, or from 16x16 when K = taps*channels reaches 1152;
-    // below that the XOR-popcount kernels win.
-    const int64_t pixels = (int64_t)g.h * g.w;
-    if (!force && !(pixels >= 1024 || (NK >= 18 && pixels >= 256))) return false;
-    const int threads = kMfmaThreads, waves = threads / 64, MT = mfma_mt(NK, NT);
-    p.step_q = (waves * MT) / p.ntx;
-    p.step_r = (waves * MT) % p.ntx;
-    p.pix_q = threads / p.RW;
-    p.pix_r = threads % p.RW;
-    p.taps = taps;
     p.fy = g.fy;
-    p.tapT = tapT;
-    p.in_bits = in_bits;
-    p.bfr_bytes = NK * NT * 1024;
-    const int Ow = (O + 63) / 64;
-    const int stage = waves * 16 * 16 * NT * 4;
-    if (mode == 0 && p.bfr_bytes < stage) p.bfr_bytes = stage;
-    // Kernels with few filter fragments need few registers, so several workgroups fit a CU and one's set-up
-    // overlaps another's MFMAs -- if their LDS footprints allow it: split a member's rows until a workgroup
-    // needs at most 48 KB (each part re-expands fx - 1 halo rows and rebuilds the small fragment set).
-    const int max_split = NK * NT <= 4 ? 8 : 1;
+    const int CB = tap_bits > 0 ? (tap_bits <= 16 ? 16 : 32) : 64 * g.Cw;
+    p.CB = CB;
+    p.in_bits = tap_bits > 0 ? tap_bits : 64 * g.Cw;
+    p.tapT = tap_bits > 0 ? 64 / tap_bits : 0;
+    p.tapM = tap_bits > 0 ? 65536 / p.tapT + 1 : 0;
+    p.fwords = (tap_bits > 0 ? (3 * g.fy + p.tapT - 1) / p.tapT : 3 * g.fy * g.Cw) * O;
+    int CPR;
+    if (CB == 16) {
+        CPR = 1;
+        p.jsh = 0; p.cmask = 0;
+        p.qj[0] = 0; p.qc[0] = 0;
+    } else if (CB == 32) {
+        CPR = (g.fy + 1) / 2;
+        p.jsh = 1; p.cmask = 1;
+        for (int q = 0; q < CPR; q++) { p.qj[q] = (short)(2 * q); p.qc[q] = 0; }
+    } else {
+        CPR = g.fy * g.Cw;
+        if (CPR > kRwMaxCPR) return false;
+        p.jsh = 2; p.cmask = 3;
+        for (int q = 0; q < CPR; q++) { p.qj[q] = (short)(q / g.Cw); p.qc[q] = (short)(64 * (q % g.Cw)); }
+    }
+    for (int q = CPR; q < kRwMaxCPR; q++) p.qj[q] = p.qc[q] = 0;
+    if (CPR == 4 || CPR == 5) return false;
+    // A consumer wave keeps the fragments of 16*NT channels in registers (at most 72 of its 168); a task covers
+    // cgt such tiles: 64 channels when there are that many, else all of them.
+    int NT, cgt;
+    if (O >= 64) {
+        NT = CPR == 6 ? 1 : 2;
+        cgt = 4 / NT;
+    } else if (O == 16 || (O == 32 && CPR != 6)) {
+        NT = O / 16;
+        cgt = 1;
+    } else {
+        return false;
+    }
+    p.cgt = cgt;
+    p.ncg = (O + 16 * NT * cgt - 1) / (16 * NT * cgt);
+    p.PS = ((CB >> 4) & 1) ? CB : CB + 16;
+    p.ntx = (g.w + 15) / 16;
+    p.RW = 16 * p.ntx + g.fy - 1;
+    p.K = 3 * g.fy * CB;
+    p.pix_q = kRwTeam / p.RW;
+    p.pix_r = kRwTeam % p.RW;
+    p.D = D;
+    // Bands: as few as possible such that the producers hold a band's input words in flight at once and two image
+    // buffers, the fragment staging areas and the int32 transpose tiles fit the CU's LDS; rows per band even.
+    const int stage = mode == 0 ? kRwCWaves * 16 * 16 * NT * 4 : 0;
+    const int rowbytes = p.RW * p.PS;
+    const int frag_bytes = 3 * CPR * 4 * 1024 + 64 * 4;  // NK * NT * (4 / NT) fragments + thresholds
     size_t lds = 0;
     for (p.S = 1;; p.S++) {
-        p.hs = round_up((g.h + p.S - 1) / p.S, 2);
-        p.RIN = p.hs + g.fx - 1;
-        p.img_bytes = round_up(p.RIN * p.RW * p.PS + 64, 16);
-        const int obuf = mode == 0 ? 0 : round_up(p.hs * g.w * Ow * 8, 16);
-        lds = (size_t)kLutBytes + kTabBytes + p.img_bytes + p.bfr_bytes + obuf;
-        if (lds <= 48 * 1024 || p.S >= max_split || p.hs <= 8) break;
+        p.hs = rw_round_up((g.h + p.S - 1) / p.S, 2);
+        const int bands = (g.h + p.hs - 1) / p.hs;
+        p.nbst = bands == 1 ? 2 : 1;  // every task brings new fragments: stage them alternately
+        p.img_bytes = rw_round_up((p.hs + 2) * rowbytes + 64, 16);
+        lds = 2 * (size_t)p.img_bytes + (size_t)p.nbst * frag_bytes + stage;
+        if ((lds <= (size_t)kRwMaxDynLds && (p.hs + 2) * p.RW <= kRwItems * kRwTeam) || p.hs <= 2) break;
     }
-    p.S = (g.h + p.hs - 1) / p.hs;  // parts that own at least one row
-    if (lds > 158 * 1024 || D * p.S > kMaxBlocks) return false;
-    if (mode == 0) return launch_mode<0>(p, D, NK, NT, pb16, lds, s);
-    if (mode == 2) return launch_mode<2>(p, D, NK, NT, pb16, lds, s);
-    return launch_mode<3>(p, D, NK, NT, pb16, lds, s);
+    if (lds > (size_t)kRwMaxDynLds || (p.hs + 2) * p.RW > kRwItems * kRwTeam) return false;
+    p.S = (g.h + p.hs - 1) / p.hs;  // bands that own at least one row
+    // Sub-bands: enough (strip, sub-band) units for the consumer waves of one channel tile.
+    const int wpt = kRwCWaves / cgt;
+    int nsub = p.ntx >= wpt ? 1 : (wpt + p.ntx - 1) / p.ntx;
+    p.hb = rw_round_up((p.hs + nsub - 1) / nsub, 2);
+    p.nsub = (p.hs + p.hb - 1) / p.hb;
+    if (mode == 0) return rw_launch_mode<0>(p, D, CPR, NT, lds, s);
+    if (mode == 2) return rw_launch_mode<2>(p, D, CPR, NT, lds, s);
+    return rw_launch_mode<3>(p, D, CPR, NT, lds, s);
 }
 
 }  // namespace nb

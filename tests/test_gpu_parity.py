@@ -419,24 +419,32 @@ def test_conv_tap_packing_gives_the_same_sums(ops, oracle, engine, dtype, C, O, 
 
 
 # (C, O, k, pad, H, W, tap-packed filter, kernel expected): one case per instantiation of the matrix-core kernel
-# (K chunks x channel tiles), ragged widths, channel counts that are not a multiple of 64, and shapes it must decline.
+# (K chunks per filter row x channel tiles per wave), ragged widths, channel counts that are not a multiple of 64,
+# images that need several bands of rows, and shapes it must decline.
 MATRIX_CORE_CASES = [
-    (3, 64, 3, 1, 9, 20, True, True),      # 1 chunk, 4 channel tiles, 4-byte pixels
-    (3, 16, 3, 1, 12, 12, True, True),     # 1 chunk, 1 tile
-    (4, 16, 3, 0, 7, 33, False, True),     # in_bits known, one word per tap
-    (16, 16, 3, 1, 20, 18, True, True),    # 3 chunks, 1 tile (16 positions per pixel)
-    (16, 64, 3, 1, 10, 16, True, True),    # 3 chunks, 4 tiles
-    (16, 80, 3, 2, 6, 17, False, True),    # O = 80: last channel group ragged
-    (64, 64, 3, 1, 12, 21, False, True),   # 9 chunks, 4 tiles
-    (64, 144, 3, 1, 8, 8, False, True),    # three channel groups, last one 16 wide
-    (64, 16, 3, 1, 9, 31, False, True),    # 9 chunks, 1 tile
+    (3, 64, 3, 1, 9, 20, True, True),      # 16-byte pixels, 64 channels = two 32-channel tiles
+    (3, 16, 3, 1, 12, 12, True, True),     # 16-byte pixels, one 16-channel tile
+    (4, 16, 3, 0, 7, 33, False, True),     # in_bits known, filter packed on the fly
+    (16, 16, 3, 1, 20, 18, True, True),
+    (16, 32, 3, 1, 10, 16, True, True),    # one 32-channel tile, full-word stores with a zero upper half
+    (16, 80, 3, 2, 6, 17, False, True),    # O = 80: second task has 16 live channels
+    (24, 64, 3, 1, 9, 17, True, True),     # 32-byte pixels, two tap columns per chunk
+    (32, 16, 3, 1, 11, 8, True, True),
+    (64, 64, 3, 1, 12, 21, False, True),   # 64-byte pixels, one chunk per tap
+    (64, 144, 3, 1, 8, 8, False, True),    # three tasks per image, last one 16 channels wide
+    (64, 16, 3, 1, 9, 31, False, True),
     (50, 64, 3, 0, 9, 9, False, True),     # tail bits of the channel word are zero
-    (128, 32, 3, 1, 10, 12, False, True),  # 18 chunks, 2 tiles
-    (128, 96, 3, 1, 5, 16, False, True),
-    (64, 64, 1, 0, 6, 40, False, True),    # 1x1 filter
-    (8, 16, 5, 2, 9, 9, True, False),      # K = 200 positions: 4 chunks, no kernel -> XOR-popcount
+    (128, 96, 3, 1, 5, 16, False, True),   # two channel words per pixel, 16-channel tiles, four per task
+    (128, 64, 3, 1, 12, 12, False, True),
+    (64, 64, 3, 1, 44, 40, False, True),   # several bands of rows, the last one shorter
+    (64, 64, 3, 0, 43, 21, False, True),   # odd output height and width: the pooled map drops the last row / column
+    (16, 16, 3, 1, 70, 66, True, True),    # bands limited by the words a producer thread holds in flight
+    (64, 64, 1, 0, 6, 40, False, False),   # 1x1 filter: XOR-popcount kernels
+    (128, 32, 3, 1, 10, 12, False, False), # 128 input channels need 64 or more output channels
+    (8, 16, 5, 2, 9, 9, True, False),      # 5x5 filter
     (64, 24, 3, 1, 8, 8, False, False),    # O % 16 != 0
-    (192, 64, 3, 1, 8, 8, False, False),   # 27 chunks
+    (64, 48, 3, 1, 8, 8, False, False),    # three 16-channel tiles
+    (448, 64, 3, 1, 6, 6, False, False),   # more than six chunks per filter row
 ]
 
 
@@ -482,6 +490,38 @@ def test_conv_matrix_core_engine_vs_oracle(ops, oracle, C, O, k, pad, H, W, tap,
         ops.conv_engine(1)
         ops.conv(xd, fd, *geom, **kw)
         assert ops.conv_last_engine() == 1
+    finally:
+        ops.conv_engine(prev)
+
+
+@pytest.mark.parametrize("C,O,S,mode", [(16, 16, 8, "pool"), (64, 64, 8, "pool"), (64, 128, 6, "pack"),
+                                         (64, 64, 8, "sums"), (3, 64, 10, "pack")])
+def test_conv_matrix_core_many_members(ops, oracle, C, O, S, mode):
+    """More members than workgroups: every workgroup of the persistent kernel walks several members (fragments and
+    image buffers change hands many times); every member against the oracle."""
+    D = 1300
+    g = rng(C + O + S)
+    Cw = (C + 63) // 64
+    x = oracle.pack(g.integers(0, 2, size=(D * S * S, C)).astype(bool), np.int64).reshape(D, S, S, Cw)
+    fb = g.integers(0, 2, size=(D * O * 9, C)).astype(bool)
+    f = np.ascontiguousarray(oracle.pack(fb, np.int64).reshape(D, O, 3, 3, Cw).transpose(0, 2, 3, 4, 1).reshape(D, -1, O))
+    K = 9 * C
+    thr = (g.integers(0, K + 1, size=(D, O)) - K // 2 + K).astype(np.int32)
+    geom = (3, 3, 1, 1, 1, 1)
+    xd, fd, td = dev(x), dev(f), dev(thr)
+    kw = dict(in_bits=C) if C < 64 else {}
+    prev = ops.conv_engine(2)
+    try:
+        if mode == "sums":
+            got = ops.conv(xd, fd, *geom, **kw)
+            assert ops.conv_last_engine() == 2
+            np.testing.assert_array_equal(host(got), oracle.conv(x, f, *geom))
+        else:
+            act = oracle.conv_act(x, f, thr, *geom)
+            packed = oracle.pack(act.reshape(-1, O), np.int64).reshape(D, S, S, -1)
+            got = ops.conv_act_pack(xd, fd, td, *geom, pool=(mode == "pool"), **kw)
+            assert ops.conv_last_engine() == 2
+            np.testing.assert_array_equal(host(got), oracle.max_pool2d(packed, 2, 2, 0, 0, 2, 2) if mode == "pool" else packed)
     finally:
         ops.conv_engine(prev)
 
