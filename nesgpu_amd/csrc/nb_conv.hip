@@ -57,6 +57,42 @@ __global__ __launch_bounds__(256) void max_pool_kernel(W *__restrict__ out, cons
     }
 }
 
+// Fast path for the usual pooling geometry (2x2 window, stride 2, no padding, 64-bit words, every window inside
+// the image): 16-byte streaming loads, four in flight per thread.
+// PAIR = true  (Cw == 1, even output width): a thread ORs a 2x4 block of input words into two output words;
+// PAIR = false (Cw even): a thread ORs the same word pair of the window's four pixels into an output word pair.
+template <bool PAIR>
+__global__ __launch_bounds__(256) void max_pool_2x2_kernel(uint64_t *__restrict__ out, const uint64_t *__restrict__ in,
+                                                           int64_t total, ConvGeom g, int units_per_row)
+{
+    NB_FLAT_LOOP(t, total)
+    {
+        if (t >= total) continue;
+        const int64_t rowi = t / units_per_row;  // (b, xo)
+        const int e = (int)(t - rowi * units_per_row);
+        const int64_t b = rowi / g.h;
+        const int xo = (int)(rowi - b * g.h);
+        const int64_t inrow = ((b * g.H + 2 * xo) * (int64_t)g.Wd) * g.Cw, rowstride = (int64_t)g.Wd * g.Cw;
+        int64_t i0, i1;  // word offsets of the two 16-byte pieces inside an input row
+        if (PAIR) {
+            i0 = 4 * (int64_t)e;
+            i1 = i0 + 2;
+        } else {
+            const int half = g.Cw >> 1, yo = e / half, cp = e - yo * half;
+            i0 = (int64_t)(2 * yo) * g.Cw + 2 * cp;
+            i1 = i0 + g.Cw;
+        }
+        const uint4 a0 = load_stream16(in + inrow + i0), a1 = load_stream16(in + inrow + i1);
+        const uint4 b0 = load_stream16(in + inrow + rowstride + i0), b1 = load_stream16(in + inrow + rowstride + i1);
+        const uint4 u = make_uint4(a0.x | b0.x, a0.y | b0.y, a0.z | b0.z, a0.w | b0.w);
+        const uint4 v = make_uint4(a1.x | b1.x, a1.y | b1.y, a1.z | b1.z, a1.w | b1.w);
+        // PAIR: u holds input pixels 4e, 4e+1 -> output pixel 2e; v holds 4e+2, 4e+3 -> output pixel 2e+1
+        const uint4 r = PAIR ? make_uint4(u.x | u.z, u.y | u.w, v.x | v.z, v.y | v.w)
+                             : make_uint4(u.x | v.x, u.y | v.y, u.z | v.z, u.w | v.w);
+        reinterpret_cast<uint4 *>(out)[t] = r;
+    }
+}
+
 template <typename W, bool POOLMAP, class Epi>
 static void dispatch_conv(const ConvA<W> &al, const W *filt, const Epi &epi, int64_t D, int64_t lanes_per_member,
                           int N, hipStream_t s)
@@ -105,6 +141,23 @@ int max_pool_impl(W *out, const W *in, int64_t B, int64_t H, int64_t Wd, int64_t
     NB_REQUIRE_PTR(in);
     NB_REQUIRE_ALIGNED(out, sizeof(W));
     NB_REQUIRE_ALIGNED(in, sizeof(W));
+    if (sizeof(W) == 8 && sx == 2 && sy == 2 && px == 0 && py == 0 && 2 * g.h <= g.H && 2 * g.w <= g.Wd &&
+        aligned(out, 16) && aligned(in, 16) && ((int64_t)g.Wd * Cw) % 2 == 0) {
+        const bool pair = Cw == 1 && g.w % 2 == 0;
+        if (pair || Cw % 2 == 0) {
+            const int units_per_row = pair ? g.w / 2 : g.w * (int)(Cw / 2);
+            const int64_t units = B * g.h * units_per_row;
+            uint64_t *o = reinterpret_cast<uint64_t *>(out);
+            const uint64_t *i = reinterpret_cast<const uint64_t *>(in);
+            if (pair)
+                max_pool_2x2_kernel<true><<<dim3(grid_for(units)), dim3(256), 0, as_stream(stream)>>>(o, i, units, g,
+                                                                                                     units_per_row);
+            else
+                max_pool_2x2_kernel<false><<<dim3(grid_for(units)), dim3(256), 0, as_stream(stream)>>>(o, i, units, g,
+                                                                                                      units_per_row);
+            return check_launch(who);
+        }
+    }
     const unsigned blocks = grid_for(total);
     max_pool_kernel<W><<<dim3(blocks), dim3(256), 0, as_stream(stream)>>>(out, in, total, g);
     return check_launch(who);

@@ -243,7 +243,8 @@ def test_conv_rectangular_window_and_image(ops, oracle, engine):
 @pytest.mark.parametrize("dtype", [torch.int64, torch.int32])
 def test_max_pool_vs_oracle(ops, oracle, dtype):
     g = rng(12)
-    for B, H, W, Cw in [(3, 10, 10, 1), (2, 7, 9, 3), (5, 64, 64, 1), (1, 2, 2, 1), (2, 33, 5, 2)]:
+    for B, H, W, Cw in [(3, 10, 10, 1), (2, 7, 9, 3), (5, 64, 64, 1), (1, 2, 2, 1), (2, 33, 5, 2), (4, 16, 12, 4),
+                        (2, 9, 8, 1), (3, 6, 6, 2), (300, 8, 8, 1), (2, 4, 6, 1)]:
         x = rand_words(g, (B, H, W, Cw), NDT[dtype])
         for geom in [(2, 2, 0, 0, 2, 2), (2, 2, 1, 1, 2, 2), (3, 3, 1, 1, 2, 2), (2, 2, 0, 0, 1, 1), (2, 2, 0, 1, 3, 2)]:
             if H - geom[0] + 2 * geom[2] < 0 or W - geom[1] + 2 * geom[3] < 0:
