@@ -38,9 +38,11 @@ namespace nb {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 
-constexpr int kRwCWaves = 8;      // consumer waves: two per SIMD keep the matrix core issuing back to back
+// Consumer waves: two per SIMD keep the matrix core issuing back to back; kernels whose filter fragments are few
+// (at most 128 registers in all) run three per SIMD, which hides more of the per-row latency chains that dominate
+// when a row step has only a handful of MFMAs.
+constexpr int rw_cwaves(int CPR, int NT) { return CPR * NT <= 4 ? 12 : 8; }
 constexpr int kRwPWaves = 4;      // producer waves
-constexpr int kRwThreads = 64 * (kRwCWaves + kRwPWaves);
 constexpr int kRwTeam = 64 * kRwPWaves;  // producer threads
 constexpr int kRwLutBytes = 256 * 8;  // byte -> 8 bytes of +-1
 constexpr int kRwMaxCPR = 6;
@@ -67,7 +69,7 @@ struct RwConv {
     int in_bits;       // valid channel bits per pixel
     int tapT, tapM;    // tap-packed filter: taps per word and ceil(65536 / tapT) + 1 (0: one word per tap and channel word)
     int img_bytes;     // one image buffer
-    int nbst;          // fragment staging areas (2 when every task brings new fragments)
+    int nbst;          // fragment staging areas: 1, or 2 when every task brings new fragments
     int fwords;        // filter words per member
     int pix_q, pix_r;  // team threads / RW and % RW: image-pixel advance of one fill pass
     short qj[kRwMaxCPR];  // chunk q of a filter row: first tap column ...
@@ -108,8 +110,9 @@ __device__ __forceinline__ void rw_next(RwTask &t, const RwConv &p)
 
 // MODE 0: int32 popcount sums [D,h,w,O]; 2: threshold bits packed along O; 3: the same, 2x2 OR-pooled.
 template <int CPR, int NT, int MODE>
-__global__ __launch_bounds__(kRwThreads) void conv_mfma_kernel(const RwConv p)
+__global__ __launch_bounds__(64 * (rw_cwaves(CPR, NT) + kRwPWaves)) void conv_mfma_kernel(const RwConv p)
 {
+    constexpr int kRwCWaves = rw_cwaves(CPR, NT);
     constexpr int FX = 3;
     constexpr int NK = FX * CPR;
     constexpr int NF = NK * NT;                  // fragments of one consumer channel tile
@@ -269,7 +272,7 @@ __global__ __launch_bounds__(kRwThreads) void conv_mfma_kernel(const RwConv p)
                 const int n0 = cur.cg * 16 * NT * p.cgt;
                 if (cur.band == 0) {
                     // ---- new (member, channel group): fragments and thresholds -> staging area -------------------
-                    unsigned char *bst = bst0 + (nb % p.nbst) * kFragBytes;
+                    unsigned char *bst = bst0 + (nb & (p.nbst - 1)) * kFragBytes;
                     nb++;
 #pragma unroll
                     for (int i = 0; i < FPW; i++) {
@@ -362,7 +365,7 @@ __global__ __launch_bounds__(kRwThreads) void conv_mfma_kernel(const RwConv p)
             if (k == 1 || p.S > 1 || cg == 0) imgseq++;
             const unsigned char *img = img0 + ((imgseq - 1) & 1) * p.img_bytes;
             if (cur.band == 0) {
-                const unsigned char *bst = bst0 + (nb % p.nbst) * kFragBytes;
+                const unsigned char *bst = bst0 + (nb & (p.nbst - 1)) * kFragBytes;
                 nb++;
 #pragma unroll
                 for (int kq = 0; kq < NK; kq++)
@@ -598,13 +601,13 @@ static bool rw_launch_one(const RwConv &p, int64_t D, size_t lds_bytes, hipStrea
         fit.regs = fa.numRegs > 0 ? fa.numRegs : 256;
         fit.cus = cus;
     }
-    // 512 registers per lane and SIMD, three waves of a workgroup per SIMD; 160 KB of LDS per CU
-    int per_cu = 512 / ((fit.regs + 7) / 8 * 8) / 3;
+    // 512 registers per lane and SIMD, three or four waves of a workgroup per SIMD; 160 KB of LDS per CU
+    int per_cu = 512 / ((fit.regs + 7) / 8 * 8) / ((rw_cwaves(CPR, NT) + kRwPWaves) / 4);
     const int by_lds = (int)(160 * 1024 / (lds_bytes + kRwLutBytes + kRwTabBytes));
     per_cu = per_cu < by_lds ? per_cu : by_lds;
     per_cu = per_cu < 1 ? 1 : (per_cu > 4 ? 4 : per_cu);
     const int64_t wgs = D < (int64_t)fit.cus * per_cu ? D : (int64_t)fit.cus * per_cu;
-    kfn<<<dim3((unsigned)wgs), dim3(kRwThreads), lds_bytes, s>>>(p);
+    kfn<<<dim3((unsigned)wgs), dim3(64 * (rw_cwaves(CPR, NT) + kRwPWaves)), lds_bytes, s>>>(p);
     return true;
 }
 
@@ -693,7 +696,8 @@ bool conv_mfma_try(void *out, const uint64_t *in, const uint64_t *filt, const in
     p.D = D;
     // Bands: as few as possible such that the producers hold a band's input words in flight at once and two image
     // buffers, the fragment staging areas and the int32 transpose tiles fit the CU's LDS; rows per band even.
-    const int stage = mode == 0 ? kRwCWaves * 16 * 16 * NT * 4 : 0;
+    const int cwaves = rw_cwaves(CPR, NT);
+    const int stage = mode == 0 ? cwaves * 16 * 16 * NT * 4 : 0;
     const int rowbytes = p.RW * p.PS;
     const int frag_bytes = 3 * CPR * 4 * 1024 + 64 * 4;  // NK * NT * (4 / NT) fragments + thresholds
     size_t lds = 0;
@@ -708,7 +712,7 @@ bool conv_mfma_try(void *out, const uint64_t *in, const uint64_t *filt, const in
     if (lds > (size_t)kRwMaxDynLds || (p.hs + 2) * p.RW > kRwItems * kRwTeam) return false;
     p.S = (g.h + p.hs - 1) / p.hs;  // bands that own at least one row
     // Sub-bands: enough (strip, sub-band) units for the consumer waves of one channel tile.
-    const int wpt = kRwCWaves / cgt;
+    const int wpt = cwaves / cgt;
     int nsub = p.ntx >= wpt ? 1 : (wpt + p.ntx - 1) / p.ntx;
     p.hb = rw_round_up((p.hs + nsub - 1) / nsub, 2);
     p.nsub = (p.hs + p.hb - 1) / p.hb;
