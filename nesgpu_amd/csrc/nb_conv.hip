@@ -60,7 +60,8 @@ __global__ __launch_bounds__(256) void max_pool_kernel(W *__restrict__ out, cons
 // Fast path for the usual pooling geometry (2x2 window, stride 2, no padding, 64-bit words, every window inside
 // the image): 16-byte streaming loads, four in flight per thread.
 // PAIR = true  (Cw == 1, even output width): a thread ORs a 2x4 block of input words into two output words;
-// PAIR = false (Cw even): a thread ORs the same word pair of the window's four pixels into an output word pair.
+// PAIR = false (Cw even; used for Cw == 2): a thread ORs the same word pair of the window's four pixels into an
+// output word pair.
 template <bool PAIR>
 __global__ __launch_bounds__(256) void max_pool_2x2_kernel(uint64_t *__restrict__ out, const uint64_t *__restrict__ in,
                                                            int64_t total, ConvGeom g, int units_per_row)
@@ -144,7 +145,7 @@ int max_pool_impl(W *out, const W *in, int64_t B, int64_t H, int64_t Wd, int64_t
     if (sizeof(W) == 8 && sx == 2 && sy == 2 && px == 0 && py == 0 && 2 * g.h <= g.H && 2 * g.w <= g.Wd &&
         aligned(out, 16) && aligned(in, 16) && ((int64_t)g.Wd * Cw) % 2 == 0) {
         const bool pair = Cw == 1 && g.w % 2 == 0;
-        if (pair || Cw % 2 == 0) {
+        if (pair || Cw == 2) {  // measured: with four or more words per pixel the word-per-thread kernel is faster
             const int units_per_row = pair ? g.w / 2 : g.w * (int)(Cw / 2);
             const int64_t units = B * g.h * units_per_row;
             uint64_t *o = reinterpret_cast<uint64_t *>(out);
