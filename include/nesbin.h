@@ -108,6 +108,17 @@ int nb_conv_act_pack_i64(int64_t *out, const int64_t *in, const int64_t *filt, c
 int nb_conv_act_pack_i32(int32_t *out, const int32_t *in, const int32_t *filt, const int32_t *thresh, int64_t D,
                          int64_t H, int64_t W, int64_t Cw, int64_t O, int fx, int fy, int px, int py, int sx,
                          int sy, int pool, int tap_bits, nb_stream_t stream);
+/* conv_popc_sums: sums[d,o] = sum over the output pixels of conv(...)[d,:,:,o], int32 [D,O] (the library zeroes
+ * it first; rejected when a member's sum could overflow int32).  This is what the per-member mean of
+ * BinarizedConv2d(batch_norm=True) needs (modules/binary.py:147-155: thresh = bias + bias_noise +
+ * activation.mean over h,w with activation = 2*conv - K), without the int32 maps reaching memory.  No single
+ * counterpart in the reference. */
+int nb_conv_popc_sums_i64(int32_t *sums, const int64_t *in, const int64_t *filt, int64_t D, int64_t H, int64_t W,
+                          int64_t Cw, int64_t O, int fx, int fy, int px, int py, int sx, int sy, int tap_bits,
+                          nb_stream_t stream);
+int nb_conv_popc_sums_i32(int32_t *sums, const int32_t *in, const int32_t *filt, int64_t D, int64_t H, int64_t W,
+                          int64_t Cw, int64_t O, int fx, int fy, int px, int py, int sx, int sy, int tap_bits,
+                          nb_stream_t stream);
 /* Conv engine selector (process-wide tunable, not per call).  Two engines compute the same sums bit for bit: the
  * XOR-popcount kernels (any shape) and an int8 matrix-core kernel (64-bit words, stride 1, O % 16 == 0,
  * K = taps*channels up to 1152 positions, one member's image fits LDS).  0 = automatic: the matrix-core kernel on

@@ -185,7 +185,16 @@ int set_conv_engine(int e)
     return prev;
 }
 
-// mode 0: int32 sums, 1: bool bytes, 2: packed words, 3: packed + 2x2 pooled words
+__global__ __launch_bounds__(256) void zero_i32_kernel(int32_t *__restrict__ out, int64_t total)
+{
+    NB_FLAT_LOOP(t, total)
+    {
+        if (t < total) out[t] = 0;
+    }
+}
+
+// mode 0: int32 sums, 1: bool bytes, 2: packed words, 3: packed + 2x2 pooled words, 4: int32 sums added up over
+// the pixels, [D, O]
 template <typename W>
 int conv_impl(void *out, const W *in, const W *filt, const int32_t *thresh, int64_t D, int64_t H, int64_t Wd,
               int64_t Cw, int64_t O, int fx, int fy, int px, int py, int sx, int sy, int mode, int tap_bits,
@@ -198,6 +207,12 @@ int conv_impl(void *out, const W *in, const W *filt, const int32_t *thresh, int6
     const int64_t hw = (int64_t)g.h * g.w;
     const int64_t h2w2 = (int64_t)(g.h >> 1) * (g.w >> 1);
     const int64_t lanes = mode == 3 ? 4 * h2w2 : hw;
+    if (mode == 4 && D * O > 0 && lanes == 0) {  // no output pixels: the sums are zero
+        NB_REQUIRE_PTR(out);
+        NB_REQUIRE_ALIGNED(out, 4);
+        zero_i32_kernel<<<dim3(grid_for(D * O)), dim3(256), 0, as_stream(stream)>>>(static_cast<int32_t *>(out), D * O);
+        return check_launch(who);
+    }
     if (D * lanes * O == 0) return NB_OK;
     NB_REQUIRE_PTR(out);
     if (Cw > 0) {
@@ -206,7 +221,7 @@ int conv_impl(void *out, const W *in, const W *filt, const int32_t *thresh, int6
         NB_REQUIRE_ALIGNED(in, sizeof(W));
         NB_REQUIRE_ALIGNED(filt, sizeof(W));
     }
-    if (mode != 0) {
+    if (mode != 0 && mode != 4) {
         NB_REQUIRE_PTR(thresh);
         NB_REQUIRE_ALIGNED(thresh, 4);
     }
@@ -219,10 +234,14 @@ int conv_impl(void *out, const W *in, const W *filt, const int32_t *thresh, int6
     if (tap_bits > 0)
         NB_REQUIRE(Cw == 1 && 2 * tap_bits <= bits, "%s: tap packing needs Cw == 1 and tap_bits <= %d (got Cw=%lld, %d)",
                    who, bits / 2, (long long)Cw, tap_bits);
-    if (mode == 0) NB_REQUIRE_ALIGNED(out, 4);
-    if (mode >= 2) NB_REQUIRE_ALIGNED(out, sizeof(W));
+    if (mode == 0 || mode == 4) NB_REQUIRE_ALIGNED(out, 4);
+    if (mode == 2 || mode == 3) NB_REQUIRE_ALIGNED(out, sizeof(W));
     // int8 matrix-core path (64-bit words, stride 1, O % 16 == 0, member fits LDS); same results
     const int engine = conv_engine();
+    if (mode == 4) {
+        NB_REQUIRE(hw * (int64_t)fx * fy * Cw * bits < (1LL << 31), "%s: a member's pixel sum may overflow int32", who);
+        zero_i32_kernel<<<dim3(grid_for(D * O)), dim3(256), 0, s>>>(static_cast<int32_t *>(out), D * O);
+    }
     // Automatic choice, measured on MI355X: one workgroup per CU walks whole members, so the matrix-core kernel needs
     // a population that fills at least half of the CUs; below that the XOR-popcount kernels, which spread one
     // member's pixels over many workgroups, are faster.
@@ -241,6 +260,9 @@ int conv_impl(void *out, const W *in, const W *filt, const int32_t *thresh, int6
         NB_REQUIRE_ALIGNED(out, 4);
         EpiI32 epi{static_cast<int32_t *>(out), (N & 3) == 0 && aligned(out, 16)};
         dispatch_conv<W, false, EpiI32>(al, filt, epi, D, lanes, N, s);
+    } else if (mode == 4) {
+        EpiSum epi{static_cast<int32_t *>(out)};
+        dispatch_conv<W, false, EpiSum>(al, filt, epi, D, lanes, N, s);
     } else if (mode == 1) {
         EpiBool epi{static_cast<uint8_t *>(out), thresh, (N & 3) == 0 && aligned(out, 4)};
         dispatch_conv<W, false, EpiBool>(al, filt, epi, D, lanes, N, s);
@@ -299,6 +321,20 @@ int nb_conv_i32(int32_t *out, const int32_t *in, const int32_t *filt, int64_t D,
 {
     return nb::conv_impl<uint32_t>(out, W32(in), W32(filt), nullptr, D, H, W, Cw, O, fx, fy, px, py, sx, sy, 0,
                                    tap_bits, s, "nb_conv_i32");
+}
+int nb_conv_popc_sums_i64(int32_t *sums, const int64_t *in, const int64_t *filt, int64_t D, int64_t H, int64_t W,
+                          int64_t Cw, int64_t O, int fx, int fy, int px, int py, int sx, int sy, int tap_bits,
+                          nb_stream_t s)
+{
+    return nb::conv_impl<uint64_t>(sums, W64(in), W64(filt), nullptr, D, H, W, Cw, O, fx, fy, px, py, sx, sy, 4,
+                                   tap_bits, s, "nb_conv_popc_sums_i64");
+}
+int nb_conv_popc_sums_i32(int32_t *sums, const int32_t *in, const int32_t *filt, int64_t D, int64_t H, int64_t W,
+                          int64_t Cw, int64_t O, int fx, int fy, int px, int py, int sx, int sy, int tap_bits,
+                          nb_stream_t s)
+{
+    return nb::conv_impl<uint32_t>(sums, W32(in), W32(filt), nullptr, D, H, W, Cw, O, fx, fy, px, py, sx, sy, 4,
+                                   tap_bits, s, "nb_conv_popc_sums_i32");
 }
 int nb_conv_act_i64(uint8_t *out, const int64_t *in, const int64_t *filt, const int32_t *thresh, int64_t D, int64_t H,
                     int64_t W, int64_t Cw, int64_t O, int fx, int fy, int px, int py, int sx, int sy, int tap_bits,

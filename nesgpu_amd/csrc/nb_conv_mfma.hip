@@ -108,7 +108,8 @@ __device__ __forceinline__ void rw_next(RwTask &t, const RwConv &p)
     }
 }
 
-// MODE 0: int32 popcount sums [D,h,w,O]; 2: threshold bits packed along O; 3: the same, 2x2 OR-pooled.
+// MODE 0: int32 popcount sums [D,h,w,O]; 2: threshold bits packed along O; 3: the same, 2x2 OR-pooled;
+// 4: the popcount sums added up over the pixels, int32 [D,O] (atomic adds into a zeroed array).
 template <int CPR, int NT, int MODE>
 __global__ __launch_bounds__(64 * (rw_cwaves(CPR, NT) + kRwPWaves)) void conv_mfma_kernel(const RwConv p)
 {
@@ -249,7 +250,7 @@ __global__ __launch_bounds__(64 * (rw_cwaves(CPR, NT) + kRwPWaves)) void conv_mf
                 const int ch = n0 + (ct * NT + nt) * 16 + li;
                 fw[i] = *reinterpret_cast<const uint64_t *>(fz + (tab[kq * 4 + lg].x + (uint32_t)(ch < p.O ? ch : p.O - 1) * 8u));
             }
-            if (MODE != 0) {
+            if (MODE == 2 || MODE == 3) {
                 const int ch = n0 + ttid;
                 traw = p.thresh[t.z * p.O + (ch < p.O ? ch : p.O - 1)];
             }
@@ -287,7 +288,7 @@ __global__ __launch_bounds__(64 * (rw_cwaves(CPR, NT) + kRwPWaves)) void conv_mf
                         }
                     }
                     // thresholds in dot-product terms: 2*popc > t  <=>  popc > (t>>1)  <=>  dot < K - 2*(t>>1)
-                    if (MODE != 0 && ttid < 64) {
+                    if ((MODE == 2 || MODE == 3) && ttid < 64) {
                         int64_t td = n0 + ttid < p.O ? (int64_t)p.K - 2 * (int64_t)(traw >> 1) : -2147483648LL;
                         td = td > 2147483647LL ? 2147483647LL : (td < -2147483648LL ? -2147483648LL : td);
                         reinterpret_cast<int *>(bst + NF * CGTMAX * 1024)[ttid] = (int)td;
@@ -372,7 +373,7 @@ __global__ __launch_bounds__(64 * (rw_cwaves(CPR, NT) + kRwPWaves)) void conv_mf
 #pragma unroll
                     for (int nt = 0; nt < NT; nt++)
                         B[kq][nt] = *reinterpret_cast<const v4i *>(bst + (((ct * NK + kq) * NT + nt) * 64 + lane) * 16);
-                if (MODE != 0) {
+                if (MODE == 2 || MODE == 3) {
 #pragma unroll
                     for (int nt = 0; nt < NT; nt++)
                         tdot[nt] = reinterpret_cast<const int *>(bst + NF * CGTMAX * 1024)[(ct * NT + nt) * 16 + li];
@@ -388,6 +389,13 @@ __global__ __launch_bounds__(64 * (rw_cwaves(CPR, NT) + kRwPWaves)) void conv_mf
             int pend[NT][2];  // MODE 3: x-pooled minima of the even row of a pair
 #pragma unroll
             for (int nt = 0; nt < NT; nt++) pend[nt][0] = pend[nt][1] = 0;
+            // MODE 4: the lane's running sum of dot products over its four pixel columns (columns past the image
+            // masked off) and all rows of the unit
+            int csum[NT], cmask[4];
+#pragma unroll
+            for (int nt = 0; nt < NT; nt++) csum[nt] = 0;
+#pragma unroll
+            for (int r = 0; r < 4; r++) cmask[r] = x0 + 4 * lg + r < p.w ? -1 : 0;
 
             // ---- epilogue of one finished output row (band-relative y) -------------------------------------------
             // Output addresses: a uniform row pointer (scalar arithmetic) plus a per-lane 32-bit byte offset.
@@ -416,6 +424,12 @@ __global__ __launch_bounds__(64 * (rw_cwaves(CPR, NT) + kRwPWaves)) void conv_mf
                 olive[0] = lane < (MODE == 3 ? 8 : 16) && xx0 + lane < ww;
             }
             auto finish_row = [&](v4i (&a)[NT], int y) {
+                if (MODE == 4) {
+#pragma unroll
+                    for (int nt = 0; nt < NT; nt++)
+                        csum[nt] += (a[nt][0] & cmask[0]) + (a[nt][1] & cmask[1]) + (a[nt][2] & cmask[2]) + (a[nt][3] & cmask[3]);
+                    return;
+                }
                 if (MODE == 0) {
                     // stage the 16 x (16*NT) tile in LDS, then store whole pixel rows (non-temporal)
 #pragma unroll
@@ -568,6 +582,19 @@ __global__ __launch_bounds__(64 * (rw_cwaves(CPR, NT) + kRwPWaves)) void conv_mf
                 for (int q = 0; q < CPR; q++) F[q] = Fn[q];
             }
             for (; rr < rend; rr++) edge_step(rr);
+            if (MODE == 4) {
+                // popcount = (K - dot) / 2 per pixel: add the four lane groups, then one atomic per channel
+                const int cols = p.w - x0 < 16 ? p.w - x0 : 16;
+                const int kn = p.K * (ye - ys) * cols;
+#pragma unroll
+                for (int nt = 0; nt < NT; nt++) {
+                    int v = csum[nt];
+                    v += __shfl_xor(v, 16);
+                    v += __shfl_xor(v, 32);
+                    const int ch = n0 + nt * 16 + li;
+                    if (lg == 0 && ch < p.O) atomicAdd(static_cast<int *>(p.out) + z * p.O + ch, (kn - v) >> 1);
+                }
+            }
             }
             rw_next(cur, p);
         }
@@ -634,7 +661,7 @@ bool conv_mfma_try(void *out, const uint64_t *in, const uint64_t *filt, const in
                  int64_t D, int O, int tap_bits, int mode, hipStream_t s)
 {
     if (!aligned(out, 16)) return false;
-    if (mode != 0 && mode != 2 && mode != 3) return false;
+    if (mode != 0 && mode != 2 && mode != 3 && mode != 4) return false;
     if (g.sx != 1 || g.sy != 1 || g.h < 1 || g.w < 1 || D < 1) return false;
     if (g.fx != 3 || g.fy < 1 || g.fy > 3 || g.Cw < 1) return false;
     if (O < 16 || (O & 15) != 0) return false;
@@ -718,6 +745,7 @@ bool conv_mfma_try(void *out, const uint64_t *in, const uint64_t *filt, const in
     p.nsub = (p.hs + p.hb - 1) / p.hb;
     if (mode == 0) return rw_launch_mode<0>(p, D, CPR, NT, lds, s);
     if (mode == 2) return rw_launch_mode<2>(p, D, CPR, NT, lds, s);
+    if (mode == 4) return rw_launch_mode<4>(p, D, CPR, NT, lds, s);
     return rw_launch_mode<3>(p, D, CPR, NT, lds, s);
 }
 

@@ -60,6 +60,9 @@ void conv_tap_launch(void *out, const W *in, const W *filt, const int32_t *thres
     } else if (mode == 1) {
         EpiBool epi{static_cast<uint8_t *>(out), thresh, (N & 3) == 0 && aligned(out, 4)};
         dispatch_tap<W, false, EpiBool>(al, filt, epi, D, lanes, Kp, N, s);
+    } else if (mode == 4) {
+        EpiSum epi{static_cast<int32_t *>(out)};
+        dispatch_tap<W, false, EpiSum>(al, filt, epi, D, lanes, Kp, N, s);
     } else if (mode == 2) {
         EpiPack<W, false> epi{static_cast<W *>(out), thresh, (int)ceil_div(N, bits)};
         dispatch_tap<W, false, EpiPack<W, false>>(al, filt, epi, D, lanes, Kp, N, s);

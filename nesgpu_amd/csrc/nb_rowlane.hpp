@@ -223,6 +223,26 @@ struct EpiI32 {
     __device__ __forceinline__ void finish(State &, int64_t, bool) const {}
 };
 
+// popcount sums added up over the rows of a member: S [Z, N] (zeroed beforehand), one atomic add per wave and
+// column.  Every lane of a wave works on the same member z.
+struct EpiSum {
+    int32_t *__restrict__ S;
+    struct State {};
+    template <int NT>
+    __device__ __forceinline__ void tile(State &, int64_t, bool valid, int64_t z, int n0, int N,
+                                         const int (&acc)[NT]) const
+    {
+#pragma unroll
+        for (int j = 0; j < NT; j++) {
+            int v = valid ? acc[j] : 0;
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
+            if ((threadIdx.x & 63) == 0 && n0 + j < N) atomicAdd(S + z * N + n0 + j, v);
+        }
+    }
+    __device__ __forceinline__ void finish(State &, int64_t, bool) const {}
+};
+
 // bool bytes (2*popc > thresh[z,y]), C [Z, M, N]   (extensions/src/bmm_act.cu:56)
 struct EpiBool {
     uint8_t *__restrict__ C;

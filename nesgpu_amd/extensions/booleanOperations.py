@@ -23,7 +23,7 @@ __all__ = [
     "batch_im2col", "bmm", "bmm_act", "conv", "conv_act", "pack", "int8pack", "sample_bits", "weighted_sum",
     "max_pool2d", "next_pow2_clip", "ceil_div", "unpack", "thresholds_from_p", "sample_bits_from_words",
     "flip_from_words", "sample_bits_philox", "flip_philox", "seeded_bmv_from_words", "seeded_bmv_philox",
-    "philox_words", "conv_act_pack", "tap_pack_filter", "tap_packing_applies", "conv_engine", "conv_last_engine",
+    "philox_words", "conv_act_pack", "conv_popc_sums", "tap_pack_filter", "tap_packing_applies", "conv_engine", "conv_last_engine",
 ]
 
 
@@ -205,6 +205,20 @@ def conv(input, filter, filterx, filtery, padx, pady, stridex, stridey, in_bits=
         _lib.call("nb_conv" + suf, out.data_ptr(), input.data_ptr(), filter.data_ptr(), input.size(0), input.size(1),
                   input.size(2), input.size(3), filter.size(2), filterx, filtery, padx, pady, stridex, stridey, tap,
                   _stream(input))
+    return out
+
+
+def conv_popc_sums(input, filter, filterx, filtery, padx, pady, stridex, stridey, in_bits=None,
+                   filter_tap_packed=False):
+    """conv(...).sum over the output pixels -> int32 [D, O], without the [D,h,w,O] maps reaching memory (not in the
+    reference; it is the statistic behind the per-member mean of BinarizedConv2d(batch_norm=True),
+    modules/binary.py:147-155)."""
+    suf, _, filter, tap = _conv_args(input, filter, filterx, filtery, in_bits, filter_tap_packed)
+    out = torch.empty((input.size(0), filter.size(2)), dtype=torch.int32, device=input.device)
+    with torch.cuda.device(input.device):
+        _lib.call("nb_conv_popc_sums" + suf, out.data_ptr(), input.data_ptr(), filter.data_ptr(), input.size(0),
+                  input.size(1), input.size(2), input.size(3), filter.size(2), filterx, filtery, padx, pady, stridex,
+                  stridey, tap, _stream(input))
     return out
 
 

@@ -161,8 +161,8 @@ class BinarizedConv2d(Binarized):
         self.batch_norm = batch_norm
         self.pack_output = pack_output
         self.pool_output = pool_output
-        if (pack_output or pool_output) and (batch_norm or not threshold):
-            raise NotImplementedError("packed output needs threshold=True, batch_norm=False")
+        if (pack_output or pool_output) and not threshold:
+            raise NotImplementedError("packed output needs threshold=True")
         self.weight_noise_reshaped = None
         self.weight_noise_tap = None
         self.reset_parameters()
@@ -196,11 +196,21 @@ class BinarizedConv2d(Binarized):
         if getattr(self, "weight_noise_tap", None) is not None:
             filt, tapkw = self.weight_noise_tap, dict(in_bits=self.in_channels, filter_tap_packed=True)
         if self.threshold:
-            if self.batch_norm:
+            if self.batch_norm and offset > 2048:
+                # activations beyond fp16's exact integers: keep the reference's composition, roundings included
                 activation = 2 * booleanOperations.conv(packed_input, filt, *geom, **tapkw) - offset
                 thresh = self.bias + self.bias_noise + activation.type(torch.float16).mean(dim=[1, 2])
                 return activation > thresh.unsqueeze(1).unsqueeze(1)
-            thresh = (self.bias + self.bias_noise).type(torch.int32) + offset
+            if self.batch_norm:
+                # modules/binary.py:147-155 without the int32 maps: the per-member mean over h,w needs only the sum of
+                # the popcounts (exact integers), mean = fp16(float(sum of activations) / (h*w)); activations are
+                # integers that fp16 holds exactly, so activation > thresh  <=>  2*popc > floor(thresh) + offset.
+                sums = booleanOperations.conv_popc_sums(packed_input, filt, *geom, **tapkw).to(torch.int64)
+                h, w = booleanOperations._out_hw(packed_input, *geom)
+                mean = ((2 * sums - offset * h * w).to(torch.float32) / float(h * w)).to(torch.float16)
+                thresh = torch.floor((self.bias + self.bias_noise + mean).to(torch.float32)).to(torch.int32) + offset
+            else:
+                thresh = (self.bias + self.bias_noise).type(torch.int32) + offset
             if self.pack_output or self.pool_output:
                 return booleanOperations.conv_act_pack(packed_input, filt, thresh, *geom, pool=self.pool_output,
                                                        **tapkw)

@@ -106,9 +106,20 @@ def test_conv_forward(binary, oracle, dtype, C, O, k, pad, stride):
             continue
         assert out.dtype == torch.bool and tuple(out.shape) == act.shape
         if batch_norm:
+            # :147-155 with the mean taken from exact integer sums: fp16(float32(sum) / float32(h*w))
+            npix = act.shape[1] * act.shape[2]
+            mean = (act.sum(axis=(1, 2), dtype=np.int64).astype(np.float32) / np.float32(npix)).astype(np.float16)
+            bn = (layer.bias + layer.bias_noise).detach().cpu().numpy()                           # fp16 [D, O]
+            thresh = (bn + mean).astype(np.float16)
+            np.testing.assert_array_equal(out.cpu().numpy(), act.astype(np.float16) > thresh[:, None, None, :])
+            # ... which is what torch's own fp16 mean gives as well (the reference's expression)
             act_t = torch.from_numpy(act.astype(np.int32)).cuda()
-            thresh = layer.bias + layer.bias_noise + act_t.type(torch.float16).mean(dim=[1, 2])   # :151
-            assert torch.equal(out, act_t > thresh.unsqueeze(1).unsqueeze(1))
+            tref = layer.bias + layer.bias_noise + act_t.type(torch.float16).mean(dim=[1, 2])   # :151
+            assert torch.equal(out, act_t > tref.unsqueeze(1).unsqueeze(1))
+            layer.pack_output = True                                                               # fused packed form
+            np.testing.assert_array_equal(layer(dev(xp)).cpu().numpy(),
+                                          oracle.pack(out.cpu().numpy().reshape(-1, O), nd).reshape(*out.shape[:3], -1))
+            layer.pack_output = False
         else:
             thr = (layer.bias + layer.bias_noise).type(torch.int32).cpu().numpy() + K          # :156
             np.testing.assert_array_equal(out.cpu().numpy(), oracle.conv_act(xp, filt, thr, *geom))

@@ -527,6 +527,32 @@ def test_conv_matrix_core_many_members(ops, oracle, C, O, S, mode):
         ops.conv_engine(prev)
 
 
+@pytest.mark.parametrize("dtype", [torch.int64, torch.int32])
+@pytest.mark.parametrize("C,O,k,pad,stride,H,W,D", [(16, 16, 3, 1, 1, 9, 20, 5), (64, 64, 3, 1, 1, 12, 21, 3),
+                                                     (3, 64, 3, 1, 1, 10, 10, 4), (64, 144, 3, 0, 1, 8, 8, 3),
+                                                     (128, 64, 3, 1, 1, 6, 18, 2), (20, 7, 5, 2, 2, 11, 9, 3),
+                                                     (70, 33, 1, 0, 1, 4, 40, 2), (64, 64, 3, 1, 1, 36, 34, 2),
+                                                     (16, 16, 3, 1, 1, 8, 8, 300)])
+def test_conv_popc_sums_vs_oracle(ops, oracle, engine, dtype, C, O, k, pad, stride, H, W, D):
+    """Sums of the popcount maps over the pixels, per member and channel, against the oracle's conv summed in numpy;
+    both engines, shapes the matrix-core kernel covers (several strips, bands, ragged widths) and shapes it does not."""
+    nd = NDT[dtype]
+    bits = torch.iinfo(dtype).bits
+    g = rng(C + O + k + H + W)
+    Cw = (C + bits - 1) // bits
+    x = oracle.pack(g.integers(0, 2, size=(D * H * W, C)).astype(bool), nd).reshape(D, H, W, Cw)
+    fb = g.integers(0, 2, size=(D * O * k * k, C)).astype(bool)
+    f = np.ascontiguousarray(oracle.pack(fb, nd).reshape(D, O, k, k, Cw).transpose(0, 2, 3, 4, 1).reshape(D, -1, O))
+    geom = (k, k, pad, pad, stride, stride)
+    want = oracle.conv(x, f, *geom).sum(axis=(1, 2), dtype=np.int64).astype(np.int32)
+    got = ops.conv_popc_sums(dev(x), dev(f), *geom)
+    assert got.dtype == torch.int32 and tuple(got.shape) == (D, O)
+    np.testing.assert_array_equal(host(got), want)
+    if ops.tap_packing_applies(C, Cw, dtype):
+        np.testing.assert_array_equal(host(ops.conv_popc_sums(dev(x), dev(f), *geom, in_bits=C)), want)
+    np.testing.assert_array_equal(host(ops.conv_popc_sums(dev(x), dev(f), *geom)), want)   # zeroed again on every call
+
+
 def test_conv_engine_selector_round_trip(ops):
     prev = ops.conv_engine()
     assert prev in (0, 1, 2)
