@@ -63,6 +63,73 @@ __global__ __launch_bounds__(BS) void bmv_kernel(int32_t *__restrict__ C, const 
     }
 }
 
+// Matrix-vector form for long rows: L lanes (16, 32 or 64) walk FOUR rows of one member with 16-byte streaming
+// loads, so the input vector is loaded once per step for all four, and the four per-lane sums are reduced by a
+// transposing butterfly: two quad steps halve the rows a lane carries (4 -> 2 -> 1) while they add, then two
+// rotations inside the row of 16 and at most two cross-row exchanges finish the one remaining value.  That is 9
+// cross-lane operations instead of 24, which matters because at HBM speed the vector ALUs, not the memory
+// system, are what this kernel runs out of.  Popcounts do not care about the word width: rows are handled as
+// 16-byte vectors.  Needs M % 4 == 0 (the four rows share the member's input) and rows of whole 16-byte vectors.
+// U = 2: two steps of the row walk are requested together (8 loads of 16 bytes in flight per lane); needs
+// rowvecs % (2*L) == 0.
+template <int L, int U, int BS>
+__global__ __launch_bounds__(BS) void bmv_quad_kernel(int32_t *__restrict__ C, const uint4 *__restrict__ A,
+                                                      const uint4 *__restrict__ X, int64_t quads, int64_t M,
+                                                      int rowvecs)
+{
+    const int64_t gid = ((int64_t)blockIdx.x * BS + threadIdx.x) / L;
+    const int sub = threadIdx.x % L;
+    const bool live = gid < quads;
+    const int64_t r0 = (live ? gid : quads - 1) * 4;  // dead groups recompute the last quad and store nothing
+    const int64_t z = r0 / M;
+    const uint4 *a = A + r0 * rowvecs, *x = X + z * rowvecs;
+    int acc[4] = {0, 0, 0, 0};
+    for (int k = sub; k < rowvecs; k += L * U) {
+        uint4 xv[U], av[U][4];
+#pragma unroll
+        for (int u = 0; u < U; u++) xv[u] = x[k + u * L];
+#pragma unroll
+        for (int u = 0; u < U; u++)
+#pragma unroll
+            for (int q = 0; q < 4; q++) av[u][q] = load_stream16(a + (int64_t)q * rowvecs + k + u * L);  // read once
+        __builtin_amdgcn_sched_barrier(0);  // all loads of the step in flight before the first use
+#pragma unroll
+        for (int u = 0; u < U; u++)
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                acc[q] = bcnt_acc(av[u][q].x ^ xv[u].x, acc[q]);
+                acc[q] = bcnt_acc(av[u][q].y ^ xv[u].y, acc[q]);
+                acc[q] = bcnt_acc(av[u][q].z ^ xv[u].z, acc[q]);
+                acc[q] = bcnt_acc(av[u][q].w ^ xv[u].w, acc[q]);
+            }
+    }
+    const bool b0 = threadIdx.x & 1, b1 = threadIdx.x & 2;
+    // lanes with bit 0 clear keep rows 0,1 and hand rows 2,3 to their neighbour, the others the reverse
+    int k0 = b0 ? acc[2] : acc[0], k1 = b0 ? acc[3] : acc[1];
+    const int s0 = b0 ? acc[0] : acc[2], s1 = b0 ? acc[1] : acc[3];
+    k0 += (int)dpp_mov<0xB1>((uint32_t)s0);  // quad_perm [1,0,3,2]
+    k1 += (int)dpp_mov<0xB1>((uint32_t)s1);
+    // bit 1 clear: keep the first of the two rows
+    int v = b1 ? k1 : k0;
+    v += (int)dpp_mov<0x4E>((uint32_t)(b1 ? k0 : k1));  // quad_perm [2,3,0,1]
+    v += (int)dpp_mov<0x124>((uint32_t)v);               // row_ror:4
+    v += (int)dpp_mov<0x128>((uint32_t)v);               // row_ror:8
+    if (L >= 32) v += __shfl_xor(v, 16);
+    if (L >= 64) v += __shfl_xor(v, 32);
+    // lane q < 4 of the group now holds row 2*(q&1) + (q>>1)
+    if (live && sub < 4) C[r0 + 2 * (sub & 1) + (sub >> 1)] = v;
+}
+
+template <int L, int U>
+static void launch_bmv_quad(int32_t *C, const void *A, const void *X, int64_t rows, int64_t M, int rowvecs, hipStream_t s)
+{
+    constexpr int BS = 1024;
+    const int64_t quads = rows / 4;
+    const int64_t blocks = ceil_div(quads * L, BS);
+    bmv_quad_kernel<L, U, BS><<<dim3((unsigned)blocks), dim3(BS), 0, s>>>(C, static_cast<const uint4 *>(A),
+                                                                        static_cast<const uint4 *>(X), quads, M, rowvecs);
+}
+
 template <typename W, int KC, int NT, bool SINGLE, bool EXACT, class Epi>
 __global__ __launch_bounds__(256) void bmm_rowlane_kernel(RowsA<W> al, const W *__restrict__ Bm, Epi epi, int mblocks,
                                                           int N)
@@ -145,7 +212,16 @@ int bmm_impl(int32_t *C, const W *A, const W *B, int64_t Z, int64_t M, int64_t K
         const int64_t rows = Z * M;
         NB_REQUIRE(ceil_div(ceil_div(rows, 4) * 64, 256) <= kMaxGridX, "%s: %lld rows exceed one launch", who,
                    (long long)rows);
-        if ((Kw & 1) == 0 && aligned(A, 2 * sizeof(W)) && aligned(B, 2 * sizeof(W)))
+        const int64_t rowbytes = Kw * (int64_t)sizeof(W);
+        if (rowbytes % 16 == 0 && rowbytes >= 256 && M % 4 == 0 && aligned(A, 16) && aligned(B, 16)) {
+            const int rowvecs = (int)(rowbytes / 16);
+            if (rowvecs % 128 == 0) launch_bmv_quad<64, 2>(C, A, B, rows, M, rowvecs, s);
+            else if (rowvecs % 64 == 0) launch_bmv_quad<32, 2>(C, A, B, rows, M, rowvecs, s);
+            else if (rowvecs >= 64) launch_bmv_quad<64, 1>(C, A, B, rows, M, rowvecs, s);
+            else if (rowvecs == 32) launch_bmv_quad<16, 2>(C, A, B, rows, M, rowvecs, s);
+            else if (rowvecs >= 32) launch_bmv_quad<32, 1>(C, A, B, rows, M, rowvecs, s);
+            else launch_bmv_quad<16, 1>(C, A, B, rows, M, rowvecs, s);
+        } else if ((Kw & 1) == 0 && aligned(A, 2 * sizeof(W)) && aligned(B, 2 * sizeof(W)))
             dispatch_bmv<W, 2>(C, A, B, rows, M, (int)Kw, s);
         else
             dispatch_bmv<W, 1>(C, A, B, rows, M, (int)Kw, s);

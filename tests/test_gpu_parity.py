@@ -145,7 +145,9 @@ def test_int8pack_vs_oracle(ops, oracle, dtype):
 
 
 LINEAR_SHAPES = [(8, 256, 4), (5, 10, 16), (3, 1000, 128), (7, 33, 9), (4, 64, 1), (2, 3, 200), (9, 1, 2), (1, 5, 31),
-                 (6, 130, 6)]
+                 (6, 130, 6),
+                 # four-rows-per-group kernel: 16, 32 and 64 lanes per row, rows that are not a multiple of the lane count
+                 (5, 12, 32), (2, 8, 200), (3, 4, 66), (2, 20, 34), (1, 4, 512), (300, 8, 64)]
 
 
 @pytest.mark.parametrize("dtype", [torch.int64, torch.int32])
