@@ -6,22 +6,22 @@
 //     popcount(x ^ w) = (K - dot) / 2
 // gives back the reference's sum bit for bit.
 //
-// One workgroup of eight waves per CU walks through its share of the population.  A task is a band of output
-// rows of one member for one group of 16*NT output channels.  Waves 4..7 (producers) prepare task k while waves
-// 0..3 (consumers) multiply task k-1, one barrier per step:
+// One workgroup per CU (8 or 12 consumer waves + 4 producer waves) walks through its share of the population.  A
+// task is a band of output rows of one member for one group of up to 64 output channels.  The producer waves
+// prepare task k while the consumer waves multiply task k-1, one barrier per step:
 //   producer: the band's input words and, when the (member, channel group) changes, the filter words were
 //     requested one step ahead; it expands the input rows (with the zero-word border, so the implicit im2col
 //     needs no bounds checks) into one of two LDS image buffers and the filter words into MFMA B fragments in an
 //     LDS staging area, then requests the words of task k+1;
-//   consumer: copies new fragments into registers (they stay there for all bands of the member), then every
-//     wave walks DOWN a strip of 16 output columns: the A fragment of image row r and tap column j is the same
+//   consumer: a wave owns 16*NT of the task's channels; it copies new fragments into registers (they stay there
+//     for all bands of the member), then walks DOWN a strip of 16 output columns: the A fragment of image row r and tap column j is the same
 //     16 pixels x 64 positions whichever filter row it meets, so it is read from LDS once and multiplied into
 //     the three output rows r, r-1, r-2.  One ds_read_b128 feeds 3*NT MFMAs.  Finished rows leave straight to
 //     global memory: int32 sums via a per-wave LDS transpose (full pixel rows, non-temporal), or threshold bits
 //     gathered with ballots into packed words, optionally 2x2 OR-pooled (in x a min over neighbouring
-//     accumulator registers, in y over two walked rows).
-// Each SIMD holds one consumer and one producer wave, so the expansion work (VALU, LDS, memory latency) runs in
-// the shadow of the MFMAs instead of in front of them.
+//     accumulator registers, in y over two walked rows), or sums over the pixels (atomic adds).
+// Each SIMD holds two or three consumer waves and one producer wave: one wave alone cannot issue MFMAs back to
+// back, and the expansion work (VALU, LDS, memory latency) runs beside the MFMAs instead of in front of them.
 //
 // Fragment layout of v_mfma_i32_16x16x64_i8 (checked on hardware): lane l supplies row l%16 of A and
 // column l%16 of B, its 16 bytes are the K-positions 16*(l/16)..+15 of the 64-chunk (any bijection works as
@@ -604,7 +604,7 @@ __global__ __launch_bounds__(64 * (rw_cwaves(CPR, NT) + kRwPWaves)) void conv_mf
 
 static inline int rw_round_up(int a, int b) { return (a + b - 1) / b * b; }
 
-// Workgroups per CU that fit by registers (eight waves each) and LDS, and the CU count of the current device.
+// Registers of a kernel instantiation and the CU count of the current device (for the workgroups-per-CU estimate).
 struct RwFit {
     int cus, regs;
 };
