@@ -70,6 +70,25 @@ def _stream(t):
     return torch.cuda.current_stream(t.device).cuda_stream
 
 
+class _Here:
+    """No-op context: the tensor already lives on the current device (the usual case; saves the two device
+    switches of torch.cuda.device on every op)."""
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        return False
+
+
+_HERE = _Here()
+
+
+def _on(t):
+    """Context that makes ``t``'s device current for the launch."""
+    return _HERE if t.device.index == torch.cuda.current_device() else torch.cuda.device(t.device)
+
+
 def _out_hw(inp, filterx, filtery, padx, pady, stridex, stridey):
     h = (inp.size(1) - filterx + 2 * padx) // stridex + 1
     w = (inp.size(2) - filtery + 2 * pady) // stridey + 1
@@ -86,7 +105,7 @@ def batch_im2col(input, filterx, filtery, padx, pady, stridex, stridey, REPEAT=1
     h, w = _out_hw(input, filterx, filtery, padx, pady, stridex, stridey)
     out = torch.empty((input.size(0), h * w, filterx * filtery * input.size(3)), dtype=input.dtype,
                       device=input.device)
-    with torch.cuda.device(input.device):
+    with _on(input):
         _lib.call("nb_im2col" + suf, out.data_ptr(), input.data_ptr(), input.size(0), input.size(1), input.size(2),
                   input.size(3), filterx, filtery, padx, pady, stridex, stridey, _stream(input))
     return out
@@ -104,7 +123,7 @@ def bmm(A, B):
     assert A.dtype == B.dtype
     suf, _ = _suffix(A.dtype)
     C = torch.empty((A.size(0), A.size(1), B.size(2)), dtype=torch.int32, device=A.device)
-    with torch.cuda.device(A.device):
+    with _on(A):
         _lib.call("nb_bmm" + suf, C.data_ptr(), A.data_ptr(), B.data_ptr(), A.size(0), A.size(1), A.size(2), B.size(2),
                   _stream(A))
     return C
@@ -127,7 +146,7 @@ def bmm_act(A, B, threshold):
     assert A.dtype == B.dtype
     suf, _ = _suffix(A.dtype)
     C = torch.empty((A.size(0), A.size(1), B.size(2)), dtype=torch.bool, device=A.device)
-    with torch.cuda.device(A.device):
+    with _on(A):
         _lib.call("nb_bmm_act" + suf, C.data_ptr(), A.data_ptr(), B.data_ptr(), threshold.data_ptr(), A.size(0),
                   A.size(1), A.size(2), B.size(2), _stream(A))
     return C
@@ -161,7 +180,7 @@ def tap_pack_filter(filter, taps, in_bits):
     assert 0 < 2 * in_bits <= bits
     T = bits // in_bits
     out = torch.empty((filter.size(0), ceil_div(taps, T), filter.size(2)), dtype=filter.dtype, device=filter.device)
-    with torch.cuda.device(filter.device):
+    with _on(filter):
         _lib.call("nb_tap_pack_filter" + suf, out.data_ptr(), filter.data_ptr(), filter.size(0), taps, filter.size(2),
                   int(in_bits), _stream(filter))
     return out
@@ -201,7 +220,7 @@ def conv(input, filter, filterx, filtery, padx, pady, stridex, stridey, in_bits=
     suf, _, filter, tap = _conv_args(input, filter, filterx, filtery, in_bits, filter_tap_packed)
     h, w = _out_hw(input, filterx, filtery, padx, pady, stridex, stridey)
     out = torch.empty((input.size(0), h, w, filter.size(2)), dtype=torch.int32, device=input.device)
-    with torch.cuda.device(input.device):
+    with _on(input):
         _lib.call("nb_conv" + suf, out.data_ptr(), input.data_ptr(), filter.data_ptr(), input.size(0), input.size(1),
                   input.size(2), input.size(3), filter.size(2), filterx, filtery, padx, pady, stridex, stridey, tap,
                   _stream(input))
@@ -215,7 +234,7 @@ def conv_popc_sums(input, filter, filterx, filtery, padx, pady, stridex, stridey
     modules/binary.py:147-155)."""
     suf, _, filter, tap = _conv_args(input, filter, filterx, filtery, in_bits, filter_tap_packed)
     out = torch.empty((input.size(0), filter.size(2)), dtype=torch.int32, device=input.device)
-    with torch.cuda.device(input.device):
+    with _on(input):
         _lib.call("nb_conv_popc_sums" + suf, out.data_ptr(), input.data_ptr(), filter.data_ptr(), input.size(0),
                   input.size(1), input.size(2), input.size(3), filter.size(2), filterx, filtery, padx, pady, stridex,
                   stridey, tap, _stream(input))
@@ -234,7 +253,7 @@ def conv_act(input, filter, threshold, filterx, filtery, padx, pady, stridex, st
     assert threshold.dtype == torch.int32
     h, w = _out_hw(input, filterx, filtery, padx, pady, stridex, stridey)
     out = torch.empty((input.size(0), h, w, filter.size(2)), dtype=torch.bool, device=input.device)
-    with torch.cuda.device(input.device):
+    with _on(input):
         _lib.call("nb_conv_act" + suf, out.data_ptr(), input.data_ptr(), filter.data_ptr(), threshold.data_ptr(),
                   input.size(0), input.size(1), input.size(2), input.size(3), filter.size(2), filterx, filtery, padx,
                   pady, stridex, stridey, tap, _stream(input))
@@ -250,7 +269,7 @@ def pack(input, dtype=torch.int32):
         raise TypeError("pack expects a torch.bool tensor, got %r" % (input.dtype,))
     suf, bits = _suffix(dtype)
     ret = torch.empty((input.size(0), ceil_div(input.shape[1], bits)), dtype=dtype, device=input.device)
-    with torch.cuda.device(input.device):
+    with _on(input):
         _lib.call("nb_pack" + suf, ret.data_ptr(), input.data_ptr(), input.size(0), input.size(1), _stream(input))
     return ret
 
@@ -263,7 +282,7 @@ def int8pack(input, dtype=torch.int32):
         raise TypeError("int8pack expects a uint8 tensor, got %r" % (input.dtype,))
     suf, bits = _suffix(dtype)
     ret = torch.empty((input.size(0), ceil_div(input.shape[1], bits // 8)), dtype=dtype, device=input.device)
-    with torch.cuda.device(input.device):
+    with _on(input):
         _lib.call("nb_int8pack" + suf, ret.data_ptr(), input.data_ptr(), input.size(0), input.size(1), _stream(input))
     return ret
 
@@ -290,7 +309,7 @@ def weighted_sum(input, weights, zbits):
     suf, bits = _suffix(input.dtype)
     assert zbits <= input.size(2) * bits
     ret = torch.empty((input.size(1), zbits), dtype=torch.float16, device=input.device)
-    with torch.cuda.device(input.device):
+    with _on(input):
         _lib.call("nb_weighted_sum" + suf, ret.data_ptr(), input.data_ptr(), weights.data_ptr(), input.size(0),
                   input.size(1), input.size(2), zbits, _stream(input))
     return ret
@@ -305,7 +324,7 @@ def max_pool2d(input, filterx, filtery, padx, pady, stridex, stridey, REPEAT=128
     suf, _ = _suffix(input.dtype)
     h, w = _out_hw(input, filterx, filtery, padx, pady, stridex, stridey)
     out = torch.empty((input.size(0), h, w, input.size(3)), dtype=input.dtype, device=input.device)
-    with torch.cuda.device(input.device):
+    with _on(input):
         _lib.call("nb_max_pool2d" + suf, out.data_ptr(), input.data_ptr(), input.size(0), input.size(1), input.size(2),
                   input.size(3), filterx, filtery, padx, pady, stridex, stridey, _stream(input))
     return out
@@ -318,7 +337,7 @@ def unpack(input):
     _check(input, "input")
     suf, bits = _suffix(input.dtype)
     ret = torch.empty((input.size(0), input.size(1) * bits), dtype=torch.bool, device=input.device)
-    with torch.cuda.device(input.device):
+    with _on(input):
         _lib.call("nb_unpack" + suf, ret.data_ptr(), input.data_ptr(), input.size(0), input.size(1), _stream(input))
     return ret
 
@@ -375,7 +394,7 @@ def sample_bits_from_words(threshold, words, dtype, base=None):
     Rw = ceil_div(C, bits)
     bptr = _base_check(base, R, Rw, dtype, words.device)
     ret = torch.empty((n, R, Rw), dtype=dtype, device=words.device)
-    with torch.cuda.device(words.device):
+    with _on(words):
         _lib.call("nb_sample_from_words" + suf, ret.data_ptr(), bptr, tptr, ts, words.data_ptr(), n, R, C,
                   _stream(words))
     return ret
@@ -426,7 +445,7 @@ def seeded_bmv_from_words(threshold, x_packed, words, base=None):
     keep, tptr, ts = _thr_args(threshold, R, C, words.device)
     bptr = _base_check(base, R, Rw, x_packed.dtype, words.device)
     out = torch.empty((n, R), dtype=torch.int32, device=words.device)
-    with torch.cuda.device(words.device):
+    with _on(words):
         _lib.call("nb_seeded_bmv_from_words" + suf, out.data_ptr(), bptr, tptr, ts, x_packed.data_ptr(),
                   words.data_ptr(), n, R, C, _stream(words))
     return out
@@ -443,7 +462,7 @@ def seeded_bmv_philox(threshold, x_packed, rows, in_bits, seed, subsequence=0, f
     keep, tptr, ts = _thr_args(threshold, R, C, x_packed.device)
     bptr = _base_check(base, R, Rw, x_packed.dtype, x_packed.device)
     out = torch.empty((n, R), dtype=torch.int32, device=x_packed.device)
-    with torch.cuda.device(x_packed.device):
+    with _on(x_packed):
         _lib.call("nb_seeded_bmv_philox" + suf, out.data_ptr(), bptr, tptr, ts, x_packed.data_ptr(),
                   int(seed) & (2 ** 64 - 1), int(subsequence), int(first), n, R, C, _stream(x_packed))
     return out
@@ -473,7 +492,7 @@ def conv_act_pack(input, filter, threshold, filterx, filtery, padx, pady, stride
     Ow = ceil_div(filter.size(2), bits)
     shape = (input.size(0), h // 2, w // 2, Ow) if pool else (input.size(0), h, w, Ow)
     out = torch.empty(shape, dtype=input.dtype, device=input.device)
-    with torch.cuda.device(input.device):
+    with _on(input):
         _lib.call("nb_conv_act_pack" + suf, out.data_ptr(), input.data_ptr(), filter.data_ptr(), threshold.data_ptr(),
                   input.size(0), input.size(1), input.size(2), input.size(3), filter.size(2), filterx, filtery, padx,
                   pady, stridex, stridey, 1 if pool else 0, tap, _stream(input))
