@@ -64,33 +64,42 @@ __global__ __launch_bounds__(256) void max_pool_kernel(W *__restrict__ out, cons
 // output word pair.
 template <bool PAIR>
 __global__ __launch_bounds__(256) void max_pool_2x2_kernel(uint64_t *__restrict__ out, const uint64_t *__restrict__ in,
-                                                           int64_t total, ConvGeom g, int units_per_row)
+                                                           uint32_t total, ConvGeom g, uint32_t units_per_row)
 {
-    NB_FLAT_LOOP(t, total)
-    {
-        if (t >= total) continue;
-        const int64_t rowi = t / units_per_row;  // (b, xo)
-        const int e = (int)(t - rowi * units_per_row);
-        const int64_t b = rowi / g.h;
-        const int xo = (int)(rowi - b * g.h);
-        const int64_t inrow = ((b * g.H + 2 * xo) * (int64_t)g.Wd) * g.Cw, rowstride = (int64_t)g.Wd * g.Cw;
+    // 32-bit unit indices (the host checks that they fit); a thread handles units t and t + half with all eight
+    // loads requested before the first OR
+    const uint32_t half = (total + 1) >> 1;
+    const uint32_t t0 = blockIdx.x * 256u + threadIdx.x;
+    if (t0 >= half) return;
+    const uint32_t tt[2] = {t0, t0 + half < total ? t0 + half : t0};
+    uint4 a0[2], a1[2], b0[2], b1[2];
+#pragma unroll
+    for (int k = 0; k < 2; k++) {
+        const uint32_t rowi = tt[k] / units_per_row, e = tt[k] - rowi * units_per_row;  // (b, xo), unit in the row
+        const uint32_t b = rowi / (uint32_t)g.h, xo = rowi - b * (uint32_t)g.h;
+        const int64_t rowstride = (int64_t)g.Wd * g.Cw, inrow = ((int64_t)b * g.H + 2 * xo) * rowstride;
         int64_t i0, i1;  // word offsets of the two 16-byte pieces inside an input row
         if (PAIR) {
             i0 = 4 * (int64_t)e;
             i1 = i0 + 2;
         } else {
-            const int half = g.Cw >> 1, yo = e / half, cp = e - yo * half;
+            const uint32_t hw = (uint32_t)g.Cw >> 1, yo = e / hw, cp = e - yo * hw;
             i0 = (int64_t)(2 * yo) * g.Cw + 2 * cp;
             i1 = i0 + g.Cw;
         }
-        const uint4 a0 = load_stream16(in + inrow + i0), a1 = load_stream16(in + inrow + i1);
-        const uint4 b0 = load_stream16(in + inrow + rowstride + i0), b1 = load_stream16(in + inrow + rowstride + i1);
-        const uint4 u = make_uint4(a0.x | b0.x, a0.y | b0.y, a0.z | b0.z, a0.w | b0.w);
-        const uint4 v = make_uint4(a1.x | b1.x, a1.y | b1.y, a1.z | b1.z, a1.w | b1.w);
+        a0[k] = load_stream16(in + inrow + i0);
+        a1[k] = load_stream16(in + inrow + i1);
+        b0[k] = load_stream16(in + inrow + rowstride + i0);
+        b1[k] = load_stream16(in + inrow + rowstride + i1);
+    }
+#pragma unroll
+    for (int k = 0; k < 2; k++) {
+        const uint4 u = make_uint4(a0[k].x | b0[k].x, a0[k].y | b0[k].y, a0[k].z | b0[k].z, a0[k].w | b0[k].w);
+        const uint4 v = make_uint4(a1[k].x | b1[k].x, a1[k].y | b1[k].y, a1[k].z | b1[k].z, a1[k].w | b1[k].w);
         // PAIR: u holds input pixels 4e, 4e+1 -> output pixel 2e; v holds 4e+2, 4e+3 -> output pixel 2e+1
         const uint4 r = PAIR ? make_uint4(u.x | u.z, u.y | u.w, v.x | v.z, v.y | v.w)
                              : make_uint4(u.x | v.x, u.y | v.y, u.z | v.z, u.w | v.w);
-        reinterpret_cast<uint4 *>(out)[t] = r;
+        if (k == 0 || t0 + half < total) reinterpret_cast<uint4 *>(out)[tt[k]] = r;
     }
 }
 
@@ -148,15 +157,18 @@ int max_pool_impl(W *out, const W *in, int64_t B, int64_t H, int64_t Wd, int64_t
         if (pair || Cw == 2) {  // measured: with four or more words per pixel the word-per-thread kernel is faster
             const int units_per_row = pair ? g.w / 2 : g.w * (int)(Cw / 2);
             const int64_t units = B * g.h * units_per_row;
-            uint64_t *o = reinterpret_cast<uint64_t *>(out);
-            const uint64_t *i = reinterpret_cast<const uint64_t *>(in);
-            if (pair)
-                max_pool_2x2_kernel<true><<<dim3(grid_for(units)), dim3(256), 0, as_stream(stream)>>>(o, i, units, g,
-                                                                                                     units_per_row);
-            else
-                max_pool_2x2_kernel<false><<<dim3(grid_for(units)), dim3(256), 0, as_stream(stream)>>>(o, i, units, g,
-                                                                                                      units_per_row);
-            return check_launch(who);
+            if (units < (1LL << 31)) {
+                uint64_t *o = reinterpret_cast<uint64_t *>(out);
+                const uint64_t *i = reinterpret_cast<const uint64_t *>(in);
+                const unsigned blocks = (unsigned)ceil_div((units + 1) / 2, 256);
+                if (pair)
+                    max_pool_2x2_kernel<true><<<dim3(blocks), dim3(256), 0, as_stream(stream)>>>(
+                        o, i, (uint32_t)units, g, (uint32_t)units_per_row);
+                else
+                    max_pool_2x2_kernel<false><<<dim3(blocks), dim3(256), 0, as_stream(stream)>>>(
+                        o, i, (uint32_t)units, g, (uint32_t)units_per_row);
+                return check_launch(who);
+            }
         }
     }
     const unsigned blocks = grid_for(total);
