@@ -70,8 +70,8 @@ __global__ __launch_bounds__(BS) void bmv_kernel(int32_t *__restrict__ C, const 
 // cross-lane operations instead of 24, which matters because at HBM speed the vector ALUs, not the memory
 // system, are what this kernel runs out of.  Popcounts do not care about the word width: rows are handled as
 // 16-byte vectors.  Needs M % 4 == 0 (the four rows share the member's input) and rows of whole 16-byte vectors.
-// U = 2: two steps of the row walk are requested together (8 loads of 16 bytes in flight per lane); needs
-// rowvecs % (2*L) == 0.
+// U steps of the row walk are requested together (4*U loads of 16 bytes in flight per lane); needs
+// rowvecs % (U*L) == 0.
 template <int L, int U, int BS>
 __global__ __launch_bounds__(BS) void bmv_quad_kernel(int32_t *__restrict__ C, const uint4 *__restrict__ A,
                                                       const uint4 *__restrict__ X, int64_t quads, int64_t M,
@@ -215,10 +215,12 @@ int bmm_impl(int32_t *C, const W *A, const W *B, int64_t Z, int64_t M, int64_t K
         const int64_t rowbytes = Kw * (int64_t)sizeof(W);
         if (rowbytes % 16 == 0 && rowbytes >= 256 && M % 4 == 0 && aligned(A, 16) && aligned(B, 16)) {
             const int rowvecs = (int)(rowbytes / 16);
-            if (rowvecs % 128 == 0) launch_bmv_quad<64, 2>(C, A, B, rows, M, rowvecs, s);
-            else if (rowvecs % 64 == 0) launch_bmv_quad<32, 2>(C, A, B, rows, M, rowvecs, s);
+            // as many row steps in flight as divide the row (up to 16 loads of 16 bytes per lane), fewest lanes per row
+            if (rowvecs % 256 == 0) launch_bmv_quad<64, 4>(C, A, B, rows, M, rowvecs, s);
+            else if (rowvecs % 128 == 0) launch_bmv_quad<32, 4>(C, A, B, rows, M, rowvecs, s);
+            else if (rowvecs % 64 == 0) launch_bmv_quad<16, 4>(C, A, B, rows, M, rowvecs, s);
+            else if (rowvecs % 32 == 0) launch_bmv_quad<16, 2>(C, A, B, rows, M, rowvecs, s);
             else if (rowvecs >= 64) launch_bmv_quad<64, 1>(C, A, B, rows, M, rowvecs, s);
-            else if (rowvecs == 32) launch_bmv_quad<16, 2>(C, A, B, rows, M, rowvecs, s);
             else if (rowvecs >= 32) launch_bmv_quad<32, 1>(C, A, B, rows, M, rowvecs, s);
             else launch_bmv_quad<16, 1>(C, A, B, rows, M, rowvecs, s);
         } else if ((Kw & 1) == 0 && aligned(A, 2 * sizeof(W)) && aligned(B, 2 * sizeof(W)))
