@@ -87,6 +87,23 @@ def linear_flip_fused(D=1024, out_f=1024, in_f=1024, T=T_P05, seed=0, dtype=torc
     return w
 
 
+def linear_flip_generated(D=1024, out_f=1024, in_f=1024, T=T_P05, seed=0, dtype=torch.int64, device="cuda"):
+    """Config 2 in generator mode: the same product with the random words produced inside the kernel by
+    Philox4x32-10 (seed, subsequence 2) instead of being read: no 4 GiB operand, the generator's arithmetic is the
+    limit.  Bit for bit the same output as :func:`linear_flip_fused` (same stream)."""
+    g = _gen(seed)
+    base_bits = _bits(g, (out_f, in_f))
+    x_bits = _bits(g, (D, in_f))
+    base = ops.pack(base_bits.to(device), dtype)
+    x = ops.pack(x_bits.to(device), dtype)
+    return Workload(
+        name="linear %dx%d D=%d N=1 p=0.05 flips from in-kernel Philox words, fused" % (out_f, in_f, D),
+        population=D, bit_macs=D * out_f * in_f,
+        algo_bytes=base.numel() * base.element_size() + x.numel() * x.element_size() + D * out_f * 4,
+        bound="generator", step=lambda: ops.seeded_bmv_philox(T, x, out_f, in_f, seed, subsequence=2, base=base),
+        tensors=dict(base=base, x=x), meta=dict(T=T, seed=seed, subsequence=2, in_f=in_f, out_f=out_f))
+
+
 def _conv_filters(base_bits, D, O, k, C, T, seed, subseq, dtype, device):
     """base_bits [O*k*k, C] (rows ordered (out, kx, ky), modules/binary.py:125) -> per-member filters
     [D, k*k*Cw, O] (modules/binary.py:136-137)."""
