@@ -338,7 +338,7 @@ def test_sample_bits_law_and_layout(ops):
 @pytest.mark.parametrize("dtype", [torch.int64, torch.int32])
 def test_weighted_sum_vs_oracle(ops, oracle, dtype):
     g = rng(21)
-    for n, R, C in [(37, 5, 100), (128, 16, 64), (64, 3, 256)]:
+    for n, R, C in [(37, 5, 100), (128, 16, 64), (64, 3, 256), (200, 7, 90), (130, 3, 330), (1, 1, 1)]:
         nd = NDT[dtype]
         wb = np.dtype(nd).itemsize * 8
         words = rand_words(g, (n, R, (C + wb - 1) // wb), nd)
