@@ -32,6 +32,8 @@
 //   CB = 32: chunk q holds tap columns 2q and 2q+1, 32 positions each;
 //   CB >= 64: one chunk per (tap column, 64-position channel word).
 // Chunks of tap columns past the filter width multiply by zero bytes.
+#include <type_traits>
+
 #include "nb_conv_common.hpp"
 
 namespace nb {
@@ -268,8 +270,12 @@ __global__ __launch_bounds__(64 * (rw_cwaves(CPR, NT) + kRwPWaves)) void conv_mf
             if (k < nsteps) {
                 RwTask nxt = cur;
                 rw_next(nxt, p);
-                const bool more = k + 1 < nsteps;
-                if (more && (p.S > 1 || nxt.cg == 0)) request(wn, wnin, nxt, 0);
+                // Every step issues the same loads (the last one asks for its own task again, a step that keeps the
+                // image for another channel group asks for it anyway): the number of loads in flight behind the
+                // words used below is then known when the kernel is compiled, and waiting for this task's words
+                // does not wait for the next task's as well.
+                const RwTask ahead = k + 1 < nsteps ? nxt : cur;
+                request(wn, wnin, ahead, 0);
                 const int n0 = cur.cg * 16 * NT * p.cgt;
                 if (cur.band == 0) {
                     // ---- new (member, channel group): fragments and thresholds -> staging area -------------------
@@ -295,7 +301,7 @@ __global__ __launch_bounds__(64 * (rw_cwaves(CPR, NT) + kRwPWaves)) void conv_mf
                     }
                 }
                 // the filter words of the next task get the whole image expansion as a head start
-                if (more && nxt.band == 0) request_filter(nxt);
+                request_filter(ahead);
                 // ---- input words -> +-1 bytes in an image buffer (kept when only the channel group changed) ---------
                 if (k == 0 || p.S > 1 || cur.cg == 0) {
                     unsigned char *img = img0 + (imgseq & 1) * p.img_bytes;
@@ -303,6 +309,37 @@ __global__ __launch_bounds__(64 * (rw_cwaves(CPR, NT) + kRwPWaves)) void conv_mf
                     const int row0 = cur.band * p.hs;
                     const int hloc = p.h - row0 < p.hs ? p.h - row0 : p.hs;
                     const int npix = (hloc + FX - 1) * p.RW;
+                    // Narrow pixels (at most 32 positions, one input word): the look-ups of several items are issued
+                    // before the first store, so that no item waits for the LDS round trip of the one before.
+                    auto fill_narrow = [&](auto pieces) {
+                        constexpr int P = decltype(pieces)::value;
+                        constexpr int G = P == 1 ? 5 : 2;  // items per batch: kRwItems is a multiple of both
+                        unsigned char *dst = img + __mul24(ttid, p.PS);
+                        const int dstep = kRwTeam * p.PS;
+#pragma unroll
+                        for (int u0 = 0; u0 < kRwItems; u0 += G) {
+                            uint4 e[G][P];
+#pragma unroll
+                            for (int v = 0; v < G; v++) {
+                                const uint32_t lo = (wdin >> (u0 + v)) & 1u ? (uint32_t)wd[u0 + v] : 0u;
+#pragma unroll
+                                for (int c = 0; c < P; c++) e[v][c] = expand_half(lo, c);
+                            }
+#pragma unroll
+                            for (int v = 0; v < G; v++) {
+                                if (ttid + (u0 + v) * kRwTeam < npix) {
+#pragma unroll
+                                    for (int c = 0; c < P; c++) *reinterpret_cast<uint4 *>(dst + 16 * c) = e[v][c];
+                                }
+                                dst += dstep;
+                            }
+                        }
+                    };
+                    if (CPR == 1 && p.CB == 16) {
+                        fill_narrow(std::integral_constant<int, 1>{});
+                    } else if (CPR <= 2 && p.CB == 32) {
+                        fill_narrow(std::integral_constant<int, 2>{});
+                    } else
                     for (int cw = 0; cw < p.Cw; cw++) {
                         if (cw > 0) request(wd, wdin, cur, cw);
                         const int nbytes = p.CB - cw * 64 < 64 ? p.CB - cw * 64 : 64;  // positions held by this word
@@ -423,7 +460,7 @@ __global__ __launch_bounds__(64 * (rw_cwaves(CPR, NT) + kRwPWaves)) void conv_mf
                 olane[0] = (uint32_t)__mul24(lane, Ow) << 3;
                 olive[0] = lane < (MODE == 3 ? 8 : 16) && xx0 + lane < ww;
             }
-            auto finish_row = [&](v4i (&a)[NT], int y) {
+            auto finish_row = [&](v4i (&a)[NT], int y, int par = -1) {  // par: y & 1 when the caller knows it
                 if (MODE == 4) {
 #pragma unroll
                     for (int nt = 0; nt < NT; nt++)
@@ -466,7 +503,7 @@ __global__ __launch_bounds__(64 * (rw_cwaves(CPR, NT) + kRwPWaves)) void conv_mf
                     }
                 } else {
                     // pixels 4g, 4g+1 and 4g+2, 4g+3 pool in x; rows y (even) and y+1 pool in y
-                    if ((y & 1) == 0) {
+                    if ((par < 0 ? y & 1 : par) == 0) {
 #pragma unroll
                         for (int nt = 0; nt < NT; nt++) {
                             pend[nt][0] = a[nt][0] < a[nt][1] ? a[nt][0] : a[nt][1];
@@ -551,35 +588,47 @@ __global__ __launch_bounds__(64 * (rw_cwaves(CPR, NT) + kRwPWaves)) void conv_mf
             int rr = ys;
             const int lead = ys + 2 < rend ? ys + 2 : rend;
             for (; rr < lead; rr++) edge_step(rr);
-            for (; rr < ye; rr++) {
-                v4i Fn[CPR], done[NT];
+            // Steady rows two at a time: the fragments alternate between F and G (no register copies), and the first
+            // row of a pair is an even output row (sub-bands start on even rows), which the pooled epilogue needs to
+            // know at compile time to be free of branches.
+            v4i G[CPR];
+            auto row_step = [&](v4i (&Fu)[CPR], v4i (&Fl)[CPR], int r, int par) {
+                v4i done[NT];
                 arow += rowbytes;
 #pragma unroll
-                for (int q = 0; q < CPR; q++) Fn[q] = *reinterpret_cast<const v4i *>(arow + koff[q]);
+                for (int q = 0; q < CPR; q++) Fl[q] = *reinterpret_cast<const v4i *>(arow + koff[q]);
 #pragma unroll
                 for (int nt = 0; nt < NT; nt++) done[nt] = a0[nt];
 #pragma unroll
                 for (int q = 0; q < CPR; q++)
 #pragma unroll
                     for (int nt = 0; nt < NT; nt++)
-                        done[nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(F[q], B[2 * CPR + q][nt], done[nt], 0, 0, 0);
+                        done[nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(Fu[q], B[2 * CPR + q][nt], done[nt], 0, 0, 0);
 #pragma unroll
                 for (int nt = 0; nt < NT; nt++) a0[nt] = a1[nt];
 #pragma unroll
                 for (int q = 0; q < CPR; q++)
 #pragma unroll
                     for (int nt = 0; nt < NT; nt++)
-                        a0[nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(F[q], B[CPR + q][nt], a0[nt], 0, 0, 0);
+                        a0[nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(Fu[q], B[CPR + q][nt], a0[nt], 0, 0, 0);
 #pragma unroll
                 for (int nt = 0; nt < NT; nt++) a1[nt] = (v4i){0, 0, 0, 0};
 #pragma unroll
                 for (int q = 0; q < CPR; q++)
 #pragma unroll
                     for (int nt = 0; nt < NT; nt++)
-                        a1[nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(F[q], B[q][nt], a1[nt], 0, 0, 0);
-                finish_row(done, rr - 2);  // rr - 2 < ye - 2 <= ylast
+                        a1[nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(Fu[q], B[q][nt], a1[nt], 0, 0, 0);
+                finish_row(done, r - 2, par);  // r - 2 < ye - 2 <= ylast
+            };
+            for (; rr + 1 < ye; rr += 2) {
+                row_step(F, G, rr, 0);
+                row_step(G, F, rr + 1, 1);
+            }
+            if (rr < ye) {
+                row_step(F, G, rr, 0);
 #pragma unroll
-                for (int q = 0; q < CPR; q++) F[q] = Fn[q];
+                for (int q = 0; q < CPR; q++) F[q] = G[q];
+                rr++;
             }
             for (; rr < rend; rr++) edge_step(rr);
             if (MODE == 4) {
