@@ -199,6 +199,10 @@ __global__ __launch_bounds__(64 * (rw_cwaves(CPR, NT) + kRwPWaves)) void conv_mf
         // Team thread ttid owns the items (pixel words) ttid, ttid + 256, ... of a band; all of a band's items are
         // in flight at once (the host sizes bands so that they fit).  An out-of-range pixel reads word 0 of the
         // member and is replaced by the zero word.
+        // The producers' few instructions per step go first: they are the last waves of the workgroup, which the
+        // SIMD's oldest-first issue would otherwise serve only when its three consumer waves stall, and the
+        // consumers then wait for them at the step's barrier.
+        __builtin_amdgcn_s_setprio(3);
         const int pixb = p.Cw * 8, rowb = p.Wd * pixb;  // bytes per pixel / image row
         const int prow = ttid / p.RW, pxx = ttid - prow * p.RW;
         // input words of this step's and of the next task, and which of them are inside the image (the others are
