@@ -230,6 +230,13 @@ def hbm_kernels(torch, steps, warmup):
     W = torch.randint(-2 ** 62, 2 ** 62, (1024, 1024, 128), device=dev, generator=g, dtype=torch.int64)
     xv = torch.randint(-2 ** 62, 2 ** 62, (1024, 128, 1), device=dev, generator=g, dtype=torch.int64)
     run("bmm N=1 [1024,1024,128]", lambda: ops.bmm(W, xv), W.numel() * 8 + xv.numel() * 8 + 1024 * 1024 * 4)
+    del W, xv
+    # update step: weighted sum of the population's masks of a 1024x1024 layer (one fp32 add per member and weight
+    # bit in member order: the vector ALUs, not HBM, bound it; the fraction is reported for comparison)
+    m = torch.randint(-2 ** 62, 2 ** 62, (1024, 1024, 16), device=dev, generator=g, dtype=torch.int64)
+    wts = torch.randn(1024, device=dev, generator=g).half()
+    run("weighted_sum [1024,1024,16] -> fp16 [1024,1024]", lambda: ops.weighted_sum(m, wts, 1024),
+        m.numel() * 8 + 1024 * 1024 * 2)
     return res
 
 
