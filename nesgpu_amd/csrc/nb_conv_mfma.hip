@@ -14,14 +14,16 @@
 //     needs no bounds checks) into one of two LDS image buffers and the filter words into MFMA B fragments in an
 //     LDS staging area, then requests the words of task k+1;
 //   consumer: a wave owns 16*NT of the task's channels; it copies new fragments into registers (they stay there
-//     for all bands of the member), then walks DOWN a strip of 16 output columns: the A fragment of image row r and tap column j is the same
-//     16 pixels x 64 positions whichever filter row it meets, so it is read from LDS once and multiplied into
-//     the three output rows r, r-1, r-2.  One ds_read_b128 feeds 3*NT MFMAs.  Finished rows leave straight to
+//     for all bands of the member), then walks DOWN a strip of 16 output columns: the A fragment of image row r
+//     and tap column j is the same 16 pixels x 64 positions whichever filter row it meets, so it is read from LDS
+//     once and multiplied into the three output rows r, r-1, r-2.  One ds_read_b128 feeds 3*NT MFMAs.  Finished rows leave straight to
 //     global memory: int32 sums via a per-wave LDS transpose (full pixel rows, non-temporal), or threshold bits
 //     gathered with ballots into packed words, optionally 2x2 OR-pooled (in x a min over neighbouring
 //     accumulator registers, in y over two walked rows), or sums over the pixels (atomic adds).
 // Each SIMD holds two or three consumer waves and one producer wave: one wave alone cannot issue MFMAs back to
 // back, and the expansion work (VALU, LDS, memory latency) runs beside the MFMAs instead of in front of them.
+// The producer waves run at raised issue priority and issue the same loads on every step (which keeps the
+// compiler's wait counts exact), so that they are done early in the step and the consumers set its length.
 //
 // Fragment layout of v_mfma_i32_16x16x64_i8 (checked on hardware): lane l supplies row l%16 of A and
 // column l%16 of B, its 16 bytes are the K-positions 16*(l/16)..+15 of the 64-chunk (any bijection works as
