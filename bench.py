@@ -12,6 +12,7 @@ roofline   the dominant kernel against MI355X's published HBM bandwidth: algorit
            (4 B per weight bit of random words + base + inputs + int32 outputs) / average launch duration
 cpu_baseline  the C oracle (a port of the same arithmetic) timed on this box's host cores on a subset of
            the members of the same workload
+cpu_float_formulation  the reference's own ground truth (torch.bmm on +-1 fp32) on the host cores, for information
 """
 import argparse
 import json
@@ -153,6 +154,44 @@ def cpu_baseline(wl, members, seconds):
                                                                                   total, med)}
 
 
+def cpu_float_formulation(wl, members, seconds):
+    """The reference's own ground truth for a binary product, moved to the CPU: torch.bmm on +-1 fp32 operands
+    (booloptests.py:54-55, 150-160); fp32 is exact for K <= 2**24.  The float formulation has no fused sampler, so the
+    members' +-1 weight matrices are built outside the timed region; only the batched product is timed."""
+    import numpy as np
+    import torch
+    from oracle import oracle as O
+    m = wl.meta
+    out_f, in_f = m["out_f"], m["in_f"]
+    members = min(members, wl.population)
+    words = O.philox_words(m["seed"], m["subsequence"], 0, members * out_f * in_f).reshape(members, out_f, in_f)
+
+    def bits(t, n):                                    # packed int64 [..., Kw] -> 0/1 bytes [..., n], LSB first
+        return np.unpackbits(np.ascontiguousarray(t.cpu().numpy()).view(np.uint8), axis=-1, bitorder="little")[..., :n]
+
+    wbits = bits(wl.tensors["base"], in_f)[None] ^ (words < np.uint32(m["T"])).astype(np.uint8)
+    del words
+    Wf = torch.from_numpy(wbits.astype(np.float32) * 2 - 1)
+    del wbits
+    xf = torch.from_numpy(bits(wl.tensors["x"][:members], in_f).astype(np.float32) * 2 - 1).unsqueeze(2)
+    times, total, dot = [], 0.0, None
+    while total < seconds or len(times) < 3:
+        t0 = time.perf_counter()
+        dot = torch.bmm(Wf, xf)
+        dt = time.perf_counter() - t0
+        times.append(dt)
+        total += dt
+    popc = ((in_f - dot.squeeze(2)) / 2).to(torch.int32).numpy()
+    if not np.array_equal(wl.step()[:members].cpu().numpy(), popc):
+        raise SystemExit("bench: GPU result differs from the float formulation on the baseline sample")
+    med = sorted(times)[len(times) // 2]
+    return {"value": round(2 * members * out_f * in_f / med / 1e12, 6), "unit": "binary TOPS",
+            "cores": torch.get_num_threads(), "kind": "reference formulation (torch.bmm on +-1 fp32, CPU)",
+            "sample": "first %d of %d members, weights prepared outside the timed region, %d passes over %.1f s, "
+                      "median %.4f s per pass; popcounts recovered as (K - dot) / 2 equal the GPU's"
+                      % (members, wl.population, len(times), total, med)}
+
+
 def calibrate(torch):
     """Measured ceilings reported beside the datasheet peaks: streaming copy, streaming read, xor+bcnt loop."""
     import ctypes
@@ -287,6 +326,7 @@ def main():
     }
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(wl, args.cpu_members, args.cpu_seconds)
+        line["cpu_float_formulation"] = cpu_float_formulation(wl, 64, 4.0)
     del wl
     torch.cuda.empty_cache()
 
