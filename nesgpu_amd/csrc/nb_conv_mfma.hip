@@ -666,16 +666,23 @@ struct RwFit {
 template <int CPR, int NT, int MODE>
 static bool rw_launch_one(const RwConv &p, int64_t D, size_t lds_bytes, hipStream_t s)
 {
-    static RwFit fit = {0, 0};  // benign race: every thread computes the same values
+    // Per device (the attribute belongs to the device's copy of the kernel).  Benign race: every thread computes
+    // the same values.
+    constexpr int kMaxDevices = 16;
+    static RwFit fits[kMaxDevices] = {};
     auto *kfn = conv_mfma_kernel<CPR, NT, MODE>;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        (void)hipGetLastError();
+        return false;
+    }
+    RwFit &fit = fits[dev];
     if (fit.cus == 0) {
         hipFuncAttributes fa;
-        int dev = 0, cus = 0;
+        int cus = 0;
         if (hipFuncSetAttribute(reinterpret_cast<const void *>(kfn), hipFuncAttributeMaxDynamicSharedMemorySize,
                                 kRwMaxDynLds) != hipSuccess ||
-
             hipFuncGetAttributes(&fa, reinterpret_cast<const void *>(kfn)) != hipSuccess ||
-            hipGetDevice(&dev) != hipSuccess ||
             hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1) {
             (void)hipGetLastError();
             return false;

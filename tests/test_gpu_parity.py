@@ -497,6 +497,65 @@ def test_conv_matrix_core_engine_vs_oracle(ops, oracle, C, O, k, pad, H, W, tap,
         ops.conv_engine(prev)
 
 
+def _random_matrix_core_cases(n, seed):
+    g = np.random.default_rng(seed)
+    cases = []
+    while len(cases) < n:
+        C = int(g.choice([1, 3, 5, 8, 13, 16, 17, 24, 31, 32, 33, 50, 64, 65, 100, 128]))
+        O = int(g.choice([16, 32, 64, 80, 96, 128, 144]))
+        fy = int(g.integers(1, 4))
+        px, py = int(g.integers(0, 3)), int(g.integers(0, 3))
+        H, W = int(g.integers(3, 41)), int(g.integers(3, 71))
+        if W + 2 * py < fy:
+            continue
+        cases.append((C, O, fy, px, py, H, W, int(g.integers(1, 6)), bool(g.integers(0, 2))))
+    return cases
+
+
+def test_conv_matrix_core_random_shapes(ops, oracle):
+    """Forty-eight seeded random shapes (channels, output channels, 3 x fy windows, unequal paddings, ragged image
+    sizes, 1-5 members, filters tap-packed or not) with engine 2 asked for: all four outputs against the oracle, and
+    the matrix-core kernel serves exactly the shapes it is built for."""
+    prev = ops.conv_engine(2)
+    try:
+        for ci, (C, O, fy, px, py, H, W, D, tap) in enumerate(_random_matrix_core_cases(48, 20240607)):
+            print("case", ci, (C, O, fy, px, py, H, W, D, tap), flush=True)
+            g = rng(7000 + ci)
+            Cw = (C + 63) // 64
+            x = oracle.pack(g.integers(0, 2, size=(D * H * W, C)).astype(bool), np.int64).reshape(D, H, W, Cw)
+            fb = g.integers(0, 2, size=(D * O * 3 * fy, C)).astype(bool)
+            f = np.ascontiguousarray(oracle.pack(fb, np.int64).reshape(D, O, 3, fy, Cw).transpose(0, 2, 3, 4, 1)
+                                     .reshape(D, -1, O))
+            K = 3 * fy * C
+            thr = (g.integers(0, K + 1, size=(D, O)) - K // 2 + K).astype(np.int32)
+            geom = (3, fy, px, py, 1, 1)
+            xd, fd, td = dev(x), dev(f), dev(thr)
+            kw = {}
+            if C < 64:
+                kw = dict(in_bits=C)
+                if tap and C <= 32:
+                    fd = ops.tap_pack_filter(fd, 3 * fy, C)
+                    kw["filter_tap_packed"] = True
+            want = oracle.conv(x, f, *geom)
+            act = oracle.conv_act(x, f, thr, *geom)
+            h, w = act.shape[1:3]
+            packed = oracle.pack(act.reshape(-1, O), np.int64).reshape(D, h, w, -1)
+            # chunks per filter row: the kernel exists for 1, 2, 3 and 6; 6 needs 16 or at least 64 output channels
+            cpr = (1 if C <= 16 else (fy + 1) // 2) if C <= 32 else fy * Cw
+            covered = cpr in (1, 2, 3, 6) and (O >= 64 or O == 16 or (O == 32 and cpr != 6))
+            np.testing.assert_array_equal(host(ops.conv(xd, fd, *geom, **kw)), want)
+            if cpr != 6:                                 # with 6 chunks it also depends on the band fitting the LDS
+                assert ops.conv_last_engine() == (2 if covered else 1)
+            np.testing.assert_array_equal(host(ops.conv_act_pack(xd, fd, td, *geom, **kw)), packed)
+            if h >= 2 and w >= 2:
+                got = ops.conv_act_pack(xd, fd, td, *geom, pool=True, **kw)
+                np.testing.assert_array_equal(host(got), oracle.max_pool2d(packed, 2, 2, 0, 0, 2, 2))
+            np.testing.assert_array_equal(host(ops.conv_popc_sums(xd, fd, *geom, **kw)),
+                                          want.reshape(D, -1, O).sum(axis=1))
+    finally:
+        ops.conv_engine(prev)
+
+
 @pytest.mark.parametrize("C,O,S,mode", [(16, 16, 8, "pool"), (64, 64, 8, "pool"), (64, 128, 6, "pack"),
                                          (64, 64, 8, "sums"), (3, 64, 10, "pack")])
 def test_conv_matrix_core_many_members(ops, oracle, C, O, S, mode):
