@@ -167,6 +167,23 @@ def test_bmm_matrix_vector_unaligned_operands(ops, oracle):
     np.testing.assert_array_equal(host(ops.bmm(bigA, dev(x))), oracle.bmm(A, x))
 
 
+@pytest.mark.parametrize("dtype", [torch.int64, torch.int32])
+def test_bmm_random_shapes_vs_oracle(ops, oracle, dtype):
+    """Sixty seeded random (Z, M, Kw, N): matrix-vector forms of every row length class (the row-group kernel and the
+    16/32/64-lane four-row kernel with one to four row steps in flight) and general products."""
+    g = rng(4242)
+    for ci in range(60):
+        Z, M = int(g.integers(1, 7)), int(g.integers(1, 70))
+        Kw = int(g.choice([1, 2, 3, 4, 7, 16, 31, 32, 33, 64, 96, 128, 130, 256, 512]))
+        N = 1 if ci % 3 else int(g.integers(2, 40))
+        if ci % 6 == 1:
+            M = 4 * int(g.integers(1, 30))                # the four-row kernel needs M % 4 == 0
+        print("case", ci, (Z, M, Kw, N), flush=True)
+        A = rand_words(g, (Z, M, Kw), NDT[dtype])
+        B = rand_words(g, (Z, Kw, N), NDT[dtype])
+        np.testing.assert_array_equal(host(ops.bmm(dev(A), dev(B))), oracle.bmm(A, B))
+
+
 GENERAL_SHAPES = [(2, 300, 9, 64), (3, 65, 4, 16), (2, 257, 18, 5), (2, 40, 40, 33), (1, 1, 1, 2), (2, 513, 3, 128),
                   (3, 7, 17, 17), (2, 100, 0, 4)]
 
