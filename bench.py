@@ -220,6 +220,18 @@ def calibrate(torch):
     lane_ops = blocks * 256 * iters * 8 * 16 * 2
     res["xor_bcnt_lane_ops_per_s"] = float("%.4g" % (lane_ops / ev))
     res["xor_bcnt_binary_TOPS"] = round(2 * (lane_ops / 4 * 64) / ev / 1e12, 1)
+    # how int8 MFMAs and ordinary vector instructions share a SIMD's issue (four waves per SIMD): ns per MFMA and SIMD
+    if hasattr(lib, "nb_calib_mfma_valu"):
+        lib.nb_calib_mfma_valu.argtypes = [vp, i32, i32, i32, vp]
+        names = ["mfma_alone", "plus_2_valu_same_wave", "plus_4_valu_same_wave", "mfma_waves_and_valu_waves_4_per_mfma",
+                 "same_mfma_waves_at_priority", "same_valu_waves_at_priority"]
+        mblocks, miters = 1024, 4000
+        issue = {}
+        for v, name in enumerate(names):
+            per, ev = time_steps(torch, lambda: lib.nb_calib_mfma_valu(out.data_ptr(), mblocks, miters, v, st), 3, 1)
+            mfmas_per_simd = mblocks * 4 / 1024 * miters * 8 * (1.0 if v < 3 else 0.5)
+            issue[name] = round(ev * 1e9 / mfmas_per_simd, 2)
+        res["ns_per_int8_mfma_per_simd"] = issue
     return res
 
 

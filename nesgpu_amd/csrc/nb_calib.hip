@@ -54,6 +54,49 @@ __global__ __launch_bounds__(256) void calib_popc_kernel(int32_t *__restrict__ o
     out[(int64_t)blockIdx.x * 256 + threadIdx.x] = t;
 }
 
+typedef int calib_v4i __attribute__((ext_vector_type(4)));
+
+// How int8 MFMAs and ordinary vector instructions share a SIMD's issue.  Every iteration has eight
+// v_mfma_i32_16x16x64_i8 on independent accumulators, each followed by V independent v_add_u32.
+// SPLIT = false: every wave runs that mixed stream.  SPLIT = true: even waves of a workgroup issue only the MFMAs,
+// odd waves only the adds (16*V per iteration... the same totals per SIMD pair), at wave priorities PM and PV.
+template <int V, bool SPLIT, int PM, int PV>
+__global__ __launch_bounds__(256) void calib_mfma_valu_kernel(int32_t *__restrict__ out, int iters)
+{
+    calib_v4i a = {(int)threadIdx.x, 1, 2, 3}, b = {5, 6, 7, (int)blockIdx.x};
+    calib_v4i acc[8];
+    int x[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        acc[i] = (calib_v4i){0, 0, 0, 0};
+        x[i] = threadIdx.x + i;
+    }
+    const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // scalar branches only: MFMA ignores EXEC
+    const bool do_m = !SPLIT || (wv & 1) == 0, do_v = !SPLIT || (wv & 1) == 1;
+    if (SPLIT) {
+        if (do_m) {
+            __builtin_amdgcn_s_setprio(PM);
+        } else {
+            __builtin_amdgcn_s_setprio(PV);
+        }
+    }
+    for (int it = 0; it < iters; it++) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            if (do_m) asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+v"(acc[i]) : "v"(a), "v"(b));
+            if (do_v) {
+#pragma unroll
+                for (int j = 0; j < V; j++) asm volatile("v_add_u32 %0, %0, %1" : "+v"(x[(i + j) & 7]) : "v"(it));
+            }
+        }
+    }
+    asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15");  // the accumulators are read below without the compiler's hazard padding
+    int t = 0;
+#pragma unroll
+    for (int i = 0; i < 8; i++) t += acc[i][0] + acc[i][3] + x[i];
+    out[(int64_t)blockIdx.x * 256 + threadIdx.x] = t;
+}
+
 }  // namespace nb
 
 extern "C" {
@@ -78,5 +121,24 @@ int nb_calib_popc(void *out, const void *s1024, int blocks, int iters, nb_stream
     nb::calib_popc_kernel<<<dim3((unsigned)blocks), dim3(256), 0, nb::as_stream(s)>>>(
         static_cast<int32_t *>(out), static_cast<const uint32_t *>(s1024), iters);
     return nb::check_launch("nb_calib_popc");
+}
+// variant 0: MFMAs alone; 1: + 2 adds per MFMA in the same wave; 2: + 4 adds in the same wave; 3: MFMA waves and
+// add waves (4 adds per MFMA) at equal priority; 4: the same with the MFMA waves at priority 3; 5: with the add waves
+// at priority 3.  MFMAs executed per SIMD = blocks * 4 / 1024 * iters * 8 (half of that for variants 3-5).
+int nb_calib_mfma_valu(void *out, int blocks, int iters, int variant, nb_stream_t s)
+{
+    int32_t *o = static_cast<int32_t *>(out);
+    const dim3 g((unsigned)blocks), b(256);
+    hipStream_t st = nb::as_stream(s);
+    switch (variant) {
+    case 0: nb::calib_mfma_valu_kernel<0, false, 0, 0><<<g, b, 0, st>>>(o, iters); break;
+    case 1: nb::calib_mfma_valu_kernel<2, false, 0, 0><<<g, b, 0, st>>>(o, iters); break;
+    case 2: nb::calib_mfma_valu_kernel<4, false, 0, 0><<<g, b, 0, st>>>(o, iters); break;
+    case 3: nb::calib_mfma_valu_kernel<4, true, 0, 0><<<g, b, 0, st>>>(o, iters); break;
+    case 4: nb::calib_mfma_valu_kernel<4, true, 3, 0><<<g, b, 0, st>>>(o, iters); break;
+    case 5: nb::calib_mfma_valu_kernel<4, true, 0, 3><<<g, b, 0, st>>>(o, iters); break;
+    default: return NB_ERR_SHAPE;
+    }
+    return nb::check_launch("nb_calib_mfma_valu");
 }
 }
