@@ -41,6 +41,7 @@
 namespace nb {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v2i __attribute__((ext_vector_type(2)));
 
 // Consumer waves: two per SIMD keep the matrix core issuing back to back; kernels whose filter fragments are few
 // (at most 128 registers in all) run three per SIMD, which hides more of the per-row latency chains that dominate
@@ -199,31 +200,29 @@ __global__ __launch_bounds__(64 * (rw_cwaves(CPR, NT) + kRwPWaves)) void conv_mf
     if (producer) {
         // =========================================== producer ===================================================
         // Team thread ttid owns the items (pixel words) ttid, ttid + 256, ... of a band; all of a band's items are
-        // in flight at once (the host sizes bands so that they fit).  An out-of-range pixel reads word 0 of the
-        // member and is replaced by the zero word.
+        // in flight at once (the host sizes bands so that they fit).  The words are fetched with buffer loads whose
+        // range is the member's image: a row above or below the image gives a byte offset outside the range and the
+        // hardware returns the zero word, which is what an out-of-range pixel is; a column outside the image is
+        // given an offset that is out of range for every row.  No bounds arithmetic per item, no select afterwards.
         // The producers' few instructions per step go first: they are the last waves of the workgroup, which the
         // SIMD's oldest-first issue would otherwise serve only when its three consumer waves stall, and the
         // consumers then wait for them at the step's barrier.
         __builtin_amdgcn_s_setprio(3);
         const int pixb = p.Cw * 8, rowb = p.Wd * pixb;  // bytes per pixel / image row
         const int prow = ttid / p.RW, pxx = ttid - prow * p.RW;
-        // input words of this step's and of the next task, and which of them are inside the image (the others are
-        // replaced by the zero word when they are used, so that nothing waits for a load when it is issued)
+        // input words of this step's and of the next task
         uint64_t wda[kRwItems], wdb[kRwItems];
-        uint32_t ina = 0, inb_ = 0;
         uint64_t fw[FPW];
         int traw = 0;
-        // item u of this thread is pixel ttid + 256*u of the band's LDS image: its row, byte offset relative to the
-        // band's first input row, and whether its column is inside the image
-        int irow[kRwItems], ioff[kRwItems];
-        uint32_t xin = 0;
+        // item u of this thread is pixel ttid + 256*u of the band's LDS image: its byte offset relative to the band's
+        // first input row (kOutside for a column outside the image)
+        constexpr uint32_t kOutside = 0xC0000000u;  // +- any band offset (below 2^30 in size) stays past every image
+        uint32_t ioff[kRwItems];
         {
             int r = prow, x = pxx;
 #pragma unroll
             for (int u = 0; u < kRwItems; u++) {
-                irow[u] = r;
-                ioff[u] = r * rowb + (x - p.py) * pixb;
-                xin |= (x - p.py >= 0 && x - p.py < p.Wd) ? 1u << u : 0u;
+                ioff[u] = (x - p.py >= 0 && x - p.py < p.Wd) ? (uint32_t)(r * rowb + (x - p.py) * pixb) : kOutside;
                 r += p.pix_q;
                 x += p.pix_r;
                 if (x >= p.RW) {
@@ -232,15 +231,16 @@ __global__ __launch_bounds__(64 * (rw_cwaves(CPR, NT) + kRwPWaves)) void conv_mf
                 }
             }
         }
-        auto request = [&](uint64_t (&wd)[kRwItems], uint32_t &inside, const RwTask &t, int cw) {
-            const unsigned char *src = reinterpret_cast<const unsigned char *>(p.in + t.z * (int64_t)p.H * p.Wd * p.Cw);
-            const int y0 = t.band * p.hs - p.px, off0 = y0 * rowb + cw * 8;
-            inside = 0;
+        const int img_range = p.H * rowb;  // bytes of one member's image
+        auto request = [&](uint64_t (&wd)[kRwItems], const RwTask &t, int cw) {
+            const uint64_t *src = p.in + t.z * (int64_t)p.H * p.Wd * p.Cw;
+            const __amdgpu_buffer_rsrc_t rsrc =
+                __builtin_amdgcn_make_buffer_rsrc(const_cast<uint64_t *>(src), (short)0, img_range, 0x00020000);
+            const uint32_t off0 = (uint32_t)((t.band * p.hs - p.px) * rowb + cw * 8);
 #pragma unroll
             for (int u = 0; u < kRwItems; u++) {
-                const bool inb = ((xin >> u) & 1u) && (unsigned)(y0 + irow[u]) < (unsigned)p.H;  // false past the last row too
-                wd[u] = *reinterpret_cast<const uint64_t *>(src + (uint32_t)(inb ? off0 + ioff[u] : 0));
-                inside |= inb ? 1u << u : 0u;
+                const v2i v = __builtin_amdgcn_raw_buffer_load_b64(rsrc, (int)(off0 + ioff[u]), 0, 0);
+                wd[u] = ((uint64_t)(uint32_t)v[1] << 32) | (uint32_t)v[0];
             }
         };
         // Filter words of a channel group: wave tw takes fragments tw, tw+4, ... (fragment f = chunk f/NT, channel
@@ -266,13 +266,13 @@ __global__ __launch_bounds__(64 * (rw_cwaves(CPR, NT) + kRwPWaves)) void conv_mf
         RwTask cur{(int64_t)blockIdx.x, 0, 0};
         if (nsteps > 0) {
             request_filter(cur);
-            request(wda, ina, cur, 0);
+            request(wda, cur, 0);
         }
         int nb = 0;      // fragment sets staged so far
         int imgseq = 0;  // images expanded so far; image i sits in buffer i & 1
         // One step: `wd` holds the input words of task k (requested a step ago); those of task k+1 go to `wn` first
         // thing, so that their latency hides behind this step's work.
-        auto step = [&](int k, uint64_t (&wd)[kRwItems], uint32_t &wdin, uint64_t (&wn)[kRwItems], uint32_t &wnin) {
+        auto step = [&](int k, uint64_t (&wd)[kRwItems], uint64_t (&wn)[kRwItems]) {
             if (k < nsteps) {
                 RwTask nxt = cur;
                 rw_next(nxt, p);
@@ -281,7 +281,7 @@ __global__ __launch_bounds__(64 * (rw_cwaves(CPR, NT) + kRwPWaves)) void conv_mf
                 // words used below is then known when the kernel is compiled, and waiting for this task's words
                 // does not wait for the next task's as well.
                 const RwTask ahead = k + 1 < nsteps ? nxt : cur;
-                request(wn, wnin, ahead, 0);
+                request(wn, ahead, 0);
                 const int n0 = cur.cg * 16 * NT * p.cgt;
                 if (cur.band == 0) {
                     // ---- new (member, channel group): fragments and thresholds -> staging area -------------------
@@ -327,7 +327,7 @@ __global__ __launch_bounds__(64 * (rw_cwaves(CPR, NT) + kRwPWaves)) void conv_mf
                             uint4 e[G][P];
 #pragma unroll
                             for (int v = 0; v < G; v++) {
-                                const uint32_t lo = (wdin >> (u0 + v)) & 1u ? (uint32_t)wd[u0 + v] : 0u;
+                                const uint32_t lo = (uint32_t)wd[u0 + v];
 #pragma unroll
                                 for (int c = 0; c < P; c++) e[v][c] = expand_half(lo, c);
                             }
@@ -347,15 +347,14 @@ __global__ __launch_bounds__(64 * (rw_cwaves(CPR, NT) + kRwPWaves)) void conv_mf
                         fill_narrow(std::integral_constant<int, 2>{});
                     } else
                     for (int cw = 0; cw < p.Cw; cw++) {
-                        if (cw > 0) request(wd, wdin, cur, cw);
+                        if (cw > 0) request(wd, cur, cw);
                         const int nbytes = p.CB - cw * 64 < 64 ? p.CB - cw * 64 : 64;  // positions held by this word
                         unsigned char *dst = img + __mul24(ttid, p.PS) + cw * 64;
                         const int dstep = kRwTeam * p.PS;
 #pragma unroll
                         for (int u = 0; u < kRwItems; u++) {
                             if (ttid + u * kRwTeam < npix) {
-                                const bool inside = (wdin >> u) & 1u;
-                                const uint32_t lo = inside ? (uint32_t)wd[u] : 0u, hi = inside ? (uint32_t)(wd[u] >> 32) : 0u;
+                                const uint32_t lo = (uint32_t)wd[u], hi = (uint32_t)(wd[u] >> 32);
 #pragma unroll
                                 for (int c = 0; c < 4; c++)
                                     if (16 * c < nbytes)  // uniform
@@ -370,8 +369,8 @@ __global__ __launch_bounds__(64 * (rw_cwaves(CPR, NT) + kRwPWaves)) void conv_mf
             __syncthreads();
         };
         for (int k = 0; k <= nsteps; k += 2) {
-            step(k, wda, ina, wdb, inb_);
-            if (k + 1 <= nsteps) step(k + 1, wdb, inb_, wda, ina);
+            step(k, wda, wdb);
+            if (k + 1 <= nsteps) step(k + 1, wdb, wda);
         }
         return;
     }
@@ -729,8 +728,9 @@ bool conv_mfma_try(void *out, const uint64_t *in, const uint64_t *filt, const in
     if (O < 16 || (O & 15) != 0) return false;
     if (mode == 3 && (g.h < 2 || g.w < 2)) return false;
     if (tap_bits > 0 && (g.Cw != 1 || tap_bits > 32)) return false;
-    // 32-bit byte offsets inside one member's image and filter block
-    if ((int64_t)g.H * g.Wd * g.Cw * 8 >= (1LL << 31) || (int64_t)9 * g.Cw * O * 8 >= (1LL << 31)) return false;
+    // 32-bit byte offsets inside one member's image (below 2^30, so that the out-of-range marker of the producers'
+    // buffer loads stays out of range for every band offset) and filter block
+    if ((int64_t)g.H * g.Wd * g.Cw * 8 >= (1LL << 30) || (int64_t)9 * g.Cw * O * 8 >= (1LL << 31)) return false;
     RwConv p;
     p.in = in;
     p.filt = filt;
