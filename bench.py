@@ -115,11 +115,14 @@ def config_entry(cfg, w, per_wall, per_ev, per_graph=None):
         return entry
     valu = w.bit_macs / per_ev / workloads.VALU_POPC_PEAK
     mfma = w.bit_macs / per_ev / workloads.MFMA_INT8_PEAK
-    engine = "matrixcore" if ops.conv_last_engine() == 2 else "popcount"
-    comp = mfma if engine == "matrixcore" else valu
-    entry.update(conv_engine=engine, bound="hbm" if hbm > comp else ("mfma" if engine == "matrixcore" else "valu"),
+    fp4 = w.bit_macs / per_ev / workloads.MFMA_FP4_PEAK
+    last = ops.conv_last_engine()                    # of the step's last conv launch
+    engine = {2: "matrixcore-int8", 4: "matrixcore-fp4"}.get(last, "popcount")
+    comp = {2: mfma, 4: fp4}.get(last, valu)
+    entry.update(conv_engine=engine, bound="hbm" if hbm > comp else ("valu" if engine == "popcount" else "mfma"),
                  roofline_frac=round(max(hbm, comp), 4), frac_of_hbm_peak=round(hbm, 4),
-                 frac_of_valu_popcount_peak=round(valu, 4), frac_of_int8_mfma_peak=round(mfma, 4))
+                 frac_of_valu_popcount_peak=round(valu, 4), frac_of_int8_mfma_peak=round(mfma, 4),
+                 frac_of_fp4_mfma_peak=round(fp4, 4))
     return entry
 
 

@@ -119,16 +119,18 @@ int nb_conv_popc_sums_i64(int32_t *sums, const int64_t *in, const int64_t *filt,
 int nb_conv_popc_sums_i32(int32_t *sums, const int32_t *in, const int32_t *filt, int64_t D, int64_t H, int64_t W,
                           int64_t Cw, int64_t O, int fx, int fy, int px, int py, int sx, int sy, int tap_bits,
                           nb_stream_t stream);
-/* Conv engine selector (process-wide tunable, not per call).  Two engines compute the same sums bit for bit: the
- * XOR-popcount kernels (any shape) and an int8 matrix-core kernel (64-bit words, stride 1, O % 16 == 0,
- * K = taps*channels up to 1152 positions, one member's image fits LDS).  0 = automatic: the matrix-core kernel on
- * the shapes where it measured faster (output maps from 32x32 on, or from 16x16 when K reaches 1152), else
- * XOR-popcount; 1 = XOR-popcount only; 2 = matrix cores wherever that kernel covers the shape.  Returns the
- * previous setting; any other argument only queries.  Initial value from the environment variable
- * NESBIN_CONV_ENGINE: first letter 'v' -> 1, 'm' -> 2, else 0.  No counterpart in the reference. */
+/* Conv engine selector (process-wide tunable, not per call).  The engines compute the same sums bit for bit: the
+ * XOR-popcount kernels (any shape) and a matrix-core kernel (64-bit words, 3-row windows, stride 1, O % 16 == 0,
+ * one band of a member's image fits LDS) that feeds the bits to the matrix cores as +-1 bytes (int8 MFMA) or, for
+ * full channel words of 64, 128 or 256 channels, as FP4 codes (FP4 MFMA, twice the rate, exact for +-1).
+ * 0 = automatic: the matrix-core kernel for populations of 128 members or more, else XOR-popcount;
+ * 1 = XOR-popcount only; 2 = matrix cores wherever a kernel covers the shape; 3 = as 2, +-1 bytes only.  Returns
+ * the previous setting; any other argument only queries.  Initial value from the environment variable
+ * NESBIN_CONV_ENGINE: first letter 'v' -> 1, 'm' -> 2, 'i' -> 3, else 0.  No counterpart in the reference. */
 int nb_conv_engine(int engine);
 /* Engine that served the calling thread's latest conv / conv_act / conv_act_pack launch: 1 = XOR-popcount,
- * 2 = matrix cores, 0 = none yet.  For tests and tuning.  No counterpart in the reference. */
+ * 2 = matrix cores on +-1 bytes, 4 = matrix cores on FP4 codes, 0 = none yet.  For tests and tuning.  No
+ * counterpart in the reference. */
 int nb_conv_last_engine(void);
 /* tap_pack_filter: filt [D, taps, O] (one word per tap, Cw == 1) -> out [D, ceil(taps/T), O], T = bits/tap_bits,
  * out[d,w,o] = OR_t (filt[d,w*T+t,o] & (2^tap_bits - 1)) << (tap_bits*t).  A layout transform of the

@@ -176,24 +176,26 @@ int max_pool_impl(W *out, const W *in, int64_t B, int64_t H, int64_t Wd, int64_t
     return check_launch(who);
 }
 
-// Process-wide choice between the two conv engines (both give identical results): 0 = automatic (matrix cores
+// Process-wide choice between the conv engines (all give identical results): 0 = automatic (matrix cores
 // on the shapes where they measured faster, else XOR-popcount), 1 = XOR-popcount only, 2 = matrix cores wherever
-// a kernel covers the shape.  Initialised from the environment variable NESBIN_CONV_ENGINE ("valu" -> 1,
-// "mfma" -> 2); nb_conv_engine() changes it.
+// a kernel covers the shape (FP4 codes where that flavour exists, else +-1 bytes), 3 = as 2 but +-1 bytes only.
+// Initialised from the environment variable NESBIN_CONV_ENGINE ("valu" -> 1, "mfma" -> 2, "int8" -> 3);
+// nb_conv_engine() changes it.
 static int g_conv_engine = -1;
 static int conv_engine()
 {
     if (g_conv_engine < 0) {
         const char *v = getenv("NESBIN_CONV_ENGINE");
-        g_conv_engine = (v && v[0] == 'v') ? 1 : (v && v[0] == 'm') ? 2 : 0;
+        g_conv_engine = (v && v[0] == 'v') ? 1 : (v && v[0] == 'm') ? 2 : (v && v[0] == 'i') ? 3 : 0;
     }
     return g_conv_engine;
 }
-static thread_local int t_last_engine = 0;  // engine of this thread's latest conv launch: 1 XOR-popcount, 2 matrix cores
+// engine of this thread's latest conv launch: 1 XOR-popcount, 2 matrix cores on +-1 bytes, 4 matrix cores on FP4 codes
+static thread_local int t_last_engine = 0;
 int set_conv_engine(int e)
 {
     const int prev = conv_engine();
-    if (e >= 0 && e <= 2) g_conv_engine = e;
+    if (e >= 0 && e <= 3) g_conv_engine = e;
     return prev;
 }
 
@@ -257,11 +259,13 @@ int conv_impl(void *out, const W *in, const W *filt, const int32_t *thresh, int6
     // Automatic choice, measured on MI355X: one workgroup per CU walks whole members, so the matrix-core kernel needs
     // a population that fills at least half of the CUs; below that the XOR-popcount kernels, which spread one
     // member's pixels over many workgroups, are faster.
-    if (bits == 64 && Cw > 0 && engine != 1 && (engine == 2 || D >= 128) &&
-        conv_mfma_try(out, reinterpret_cast<const uint64_t *>(in), reinterpret_cast<const uint64_t *>(filt), thresh, g, D,
-                      N, tap_bits, mode, s)) {
-        t_last_engine = 2;
-        return check_launch(who);
+    if (bits == 64 && Cw > 0 && engine != 1 && (engine >= 2 || D >= 128)) {
+        const int ran = conv_mfma_try(out, reinterpret_cast<const uint64_t *>(in), reinterpret_cast<const uint64_t *>(filt),
+                                      thresh, g, D, N, tap_bits, mode, engine != 3, s);
+        if (ran) {
+            t_last_engine = ran;
+            return check_launch(who);
+        }
     }
     t_last_engine = 1;
     if (tap_bits > 0) {

@@ -72,10 +72,10 @@ template <typename W>
 void conv_tap_launch(void *out, const W *in, const W *filt, const int32_t *thresh, const ConvGeom &g, int64_t D,
                      int64_t lanes, int N, int tap_bits, int mode, hipStream_t s);
 
-// int8 matrix-core conv (nb_conv_mfma.hip): 3-row filters, stride 1, O % 16 == 0; mode as in conv_impl (0, 2, 3).
-// false = no kernel for this shape, nothing launched.
-bool conv_mfma_try(void *out, const uint64_t *in, const uint64_t *filt, const int32_t *thresh, const ConvGeom &g,
-                   int64_t D, int O, int tap_bits, int mode, hipStream_t s);
+// Matrix-core conv (nb_conv_mfma.hip): 3-row filters, stride 1, O % 16 == 0; mode as in conv_impl (0, 2, 3, 4).
+// 0 = no kernel for this shape, nothing launched; 2 = the int8 kernel ran; 4 = the FP4 kernel ran (allow_fp4 only).
+int conv_mfma_try(void *out, const uint64_t *in, const uint64_t *filt, const int32_t *thresh, const ConvGeom &g,
+                  int64_t D, int O, int tap_bits, int mode, bool allow_fp4, hipStream_t s);
 
 inline int taps_per_word(int bits, int tap_bits) { return bits / tap_bits; }
 

@@ -1,10 +1,15 @@
-// Binary conv on the int8 matrix cores (3-row filters, stride 1): a persistent producer / consumer kernel.
+// Binary conv on the matrix cores (3-row filters, stride 1): a persistent producer / consumer kernel.
 //
 // CDNA4 has no 1-bit MFMA, but v_mfma_i32_16x16x64_i8 does 16384 int8 MACs per wave in 16 cycles: 4x the
 // bit-MAC rate of v_xor + v_bcnt.  Bits are expanded to +-1 bytes (bit 1 -> +1, bit 0 -> -1; an out-of-range
 // pixel is the zero word, i.e. all -1), the int32 dot product over the K expanded positions is exact, and
 //     popcount(x ^ w) = (K - dot) / 2
 // gives back the reference's sum bit for bit.
+// A second flavour (template parameter Q = 1) expands to FP4 (E2M1) codes instead, two positions per byte, and
+// multiplies with v_mfma_scale_f32_16x16x128_f8f6f4 at unit scales: 128 positions per instruction in the same 16
+// cycles.  +1, -1 and 0 are exact in E2M1, the fp32 sums are integers far below 2^24, so the result is the same
+// integer.  It exists for full channel words (64, 128 or 256 channels), where a filter row then takes 2, 3 or 6
+// instructions instead of 3, 6 or 12; its byte geometry is that of the +-1 flavour with half the bytes per pixel.
 //
 // One workgroup per CU (8 or 12 consumer waves + 4 producer waves) walks through its share of the population.  A
 // task is a band of output rows of one member for one group of up to 64 output channels.  The producer waves
@@ -29,7 +34,7 @@
 // column l%16 of B, its 16 bytes are the K-positions 16*(l/16)..+15 of the 64-chunk (any bijection works as
 // long as A and B use the same one), and acc[r] is D[4*(l/16) + r][l%16].
 //
-// K chunks of one filter row (the per-pixel byte count CB is 16, 32 or 64*Cw):
+// K chunks of one filter row (the per-pixel byte count CB is 16, 32 or 64*Cw as +-1 bytes, 32*Cw as FP4 codes):
 //   CB = 16: one chunk, lane group g holds tap column g (up to 4 columns);
 //   CB = 32: chunk q holds tap columns 2q and 2q+1, 32 positions each;
 //   CB >= 64: one chunk per (tap column, 64-position channel word).
@@ -42,6 +47,8 @@ namespace nb {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v2i __attribute__((ext_vector_type(2)));
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef float v4f __attribute__((ext_vector_type(4)));
 
 // Consumer waves: two per SIMD keep the matrix core issuing back to back; kernels whose filter fragments are few
 // (at most 128 registers in all) run three per SIMD, which hides more of the per-row latency chains that dominate
@@ -63,7 +70,7 @@ struct RwConv {
     void *out;
     int64_t D;
     int H, Wd, Cw, px, py, h, w, O, fy;
-    int CB;            // expanded bytes per pixel: 16, 32 or 64*Cw
+    int CB;            // expanded bytes per pixel: 16, 32 or 64*Cw as +-1 bytes; 32*Cw as FP4 codes
     int PS;            // pixel stride in the LDS image, bytes (PS/16 odd: conflict-free 16-lane b128 reads)
     int RW;            // pixels per LDS image row
     int hs, S;         // output rows per band, bands per member
@@ -91,6 +98,36 @@ __device__ __forceinline__ uint32_t rw_pm1_bytes(uint32_t nib)
     return ((u << 8) - (u << 1)) | 0x01010101u;  // 0xFE where the bit is 0, then | 1
 }
 
+// 8 bits -> 8 FP4 (E2M1) codes, bit j -> nibble j: 1 -> 0x2 (+1.0), 0 -> 0xA (-1.0)
+__device__ __forceinline__ uint32_t rw_pm1_fp4(uint32_t b)
+{
+    uint32_t w = 0;
+#pragma unroll
+    for (int j = 0; j < 8; j++) w |= (((b >> j) & 1u) ? 0x2u : 0xAu) << (4 * j);
+    return w;
+}
+
+// One matrix-core step on 16-byte fragments.  Q = 0: v_mfma_i32_16x16x64_i8 on +-1 bytes (64 positions).  Q = 1:
+// v_mfma_scale_f32_16x16x128_f8f6f4 on FP4 codes with unit scales (128 positions, the same issue time: twice the
+// rate); +-1 and 0 are exact in E2M1 and the fp32 sums are integers far below 2^24, so the result is exact too.
+template <int Q>
+struct RwAcc {
+    typedef v4i type;
+    typedef int scalar;
+};
+template <>
+struct RwAcc<1> {
+    typedef v4f type;
+    typedef float scalar;
+};
+__device__ __forceinline__ v4i rw_mfma(v4i a, v4i b, v4i c) { return __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, c, 0, 0, 0); }
+__device__ __forceinline__ v4f rw_mfma(v4i a, v4i b, v4f c)
+{
+    const v8i a8 = __builtin_shufflevector(a, a, 0, 1, 2, 3, -1, -1, -1, -1);
+    const v8i b8 = __builtin_shufflevector(b, b, 0, 1, 2, 3, -1, -1, -1, -1);
+    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a8, b8, c, 4, 4, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
+}
+
 __device__ __forceinline__ uint64_t rw_sel4(int r, uint64_t a, uint64_t b, uint64_t c, uint64_t d)
 {
     return r == 0 ? a : r == 1 ? b : r == 2 ? c : d;
@@ -115,9 +152,13 @@ __device__ __forceinline__ void rw_next(RwTask &t, const RwConv &p)
 
 // MODE 0: int32 popcount sums [D,h,w,O]; 2: threshold bits packed along O; 3: the same, 2x2 OR-pooled;
 // 4: the popcount sums added up over the pixels, int32 [D,O] (atomic adds into a zeroed array).
-template <int CPR, int NT, int MODE>
+// Q: 0 = +-1 bytes and the int8 MFMA, 1 = FP4 codes and the FP4 MFMA (full channel words only).
+template <int CPR, int NT, int MODE, int Q>
 __global__ __launch_bounds__(64 * (rw_cwaves(CPR, NT) + kRwPWaves)) void conv_mfma_kernel(const RwConv p)
 {
+    typedef typename RwAcc<Q>::type acc_t;    // accumulator fragment
+    typedef typename RwAcc<Q>::scalar acc_s;  // one dot product
+    constexpr int PPL = Q ? 32 : 16;          // positions in a lane's 16 bytes
     constexpr int kRwCWaves = rw_cwaves(CPR, NT);
     constexpr int FX = 3;
     constexpr int NK = FX * CPR;
@@ -147,8 +188,23 @@ __global__ __launch_bounds__(64 * (rw_cwaves(CPR, NT) + kRwPWaves)) void conv_mf
     // Expansion table: entry b holds the +-1 bytes of bits 0..7 of b.  The expansion work shares the SIMDs' issue
     // slots with the MFMAs, so it is written for the fewest instructions: two ALU operations and one 8-byte look-up
     // per 8 bits (bank conflicts between look-ups cost LDS time, which is plentiful, not issue slots).
-    if (tid < 256) lut_s[tid] = make_uint2(rw_pm1_bytes(tid & 0xFu), rw_pm1_bytes((unsigned)tid >> 4));
+    // (FP4: entry b holds the 8 codes of b in 4 bytes.)
+    if (tid < 256) {
+        if (Q) {
+            reinterpret_cast<uint32_t *>(lut_s)[tid] = rw_pm1_fp4(tid);
+        } else {
+            lut_s[tid] = make_uint2(rw_pm1_bytes(tid & 0xFu), rw_pm1_bytes((unsigned)tid >> 4));
+        }
+    }
     const unsigned char *lutb = reinterpret_cast<const unsigned char *>(lut_s);
+    // FP4: 32 bits -> 16 bytes of codes, four 4-byte look-ups
+    auto expand32_fp4 = [&](uint32_t x) {
+        const uint32_t a = *reinterpret_cast<const uint32_t *>(lutb + ((x << 2) & 0x3FCu));
+        const uint32_t b = *reinterpret_cast<const uint32_t *>(lutb + ((x >> 6) & 0x3FCu));
+        const uint32_t c = *reinterpret_cast<const uint32_t *>(lutb + ((x >> 14) & 0x3FCu));
+        const uint32_t d = *reinterpret_cast<const uint32_t *>(lutb + ((x >> 22) & 0x3FCu));
+        return make_uint4(a, b, c, d);
+    };
     // bits 16*hi .. 16*hi+15 of x -> 16 bytes of +-1, bit b -> byte b
     auto expand_half = [&](uint32_t x, int hi) {
         const uint32_t i0 = hi ? (x >> 13) & 0x7F8u : (x << 3) & 0x7F8u;
@@ -159,8 +215,8 @@ __global__ __launch_bounds__(64 * (rw_cwaves(CPR, NT) + kRwPWaves)) void conv_mf
 
     // ---- fragment geometry ---------------------------------------------------------------------------------
     // chunk kq = i*CPR + q (filter row i) and lane group g: tap column j, first position c0.  Table entry:
-    //   x = byte offset of the filter word holding the group's 16 bits (without the channel),
-    //   y = shift of those bits | mask of the channel bits among them << 8 | (tap column inside the filter) << 31;
+    //   x = byte offset of the filter word holding the group's 16 (FP4: 32) bits (without the channel),
+    //   y = shift of those bits | number of channel bits among them << 8 | (tap column inside the filter) << 31;
     // a tap column past the filter multiplies by zero bytes, channel positions past in_bits by -1 (they equal the
     // pixel's zero tail and are part of K).
     if (tid >= 64 && tid < 64 + NK * 4) {
@@ -171,13 +227,15 @@ __global__ __launch_bounds__(64 * (rw_cwaves(CPR, NT) + kRwPWaves)) void conv_mf
         if (p.CB == 32) {
             qj = 2 * q;
         } else if (p.CB >= 64) {
-            qj = q / p.Cw;
-            qc = 64 * (q - qj * p.Cw);
+            const int nch = p.CB >> 6;  // 64-byte pieces of a pixel
+            qj = q / nch;
+            qc = 64 * (q - qj * nch);
         }
-        const int j = qj + (g >> p.jsh), c0 = qc + 16 * (g & p.cmask);
+        const int j = qj + (g >> p.jsh);
+        const int c0 = (qc + 16 * (g & p.cmask)) * (PPL / 16);  // first position of the lane group inside the pixel
         const int tap = i * p.fy + j;
         const int left = p.in_bits - c0;
-        const int nv = left < 0 ? 0 : (left > 16 ? 16 : left);
+        const int nv = left < 0 ? 0 : (left > PPL ? PPL : left);
         int fr, sh;
         if (p.tapT > 0) {
             fr = (tap * p.tapM) >> 16;  // tap / tapT
@@ -189,7 +247,7 @@ __global__ __launch_bounds__(64 * (rw_cwaves(CPR, NT) + kRwPWaves)) void conv_mf
         }
         const bool inside = j < p.fy;
         tab[e] = make_uint2(inside ? (uint32_t)(fr * p.O) * 8u : 0u,
-                            (uint32_t)sh | (((1u << nv) - 1u) << 8) | (inside ? 0x80000000u : 0u));
+                            (uint32_t)sh | ((uint32_t)nv << 8) | (inside ? 0x80000000u : 0u));
     }
     __syncthreads();  // tables complete
 
@@ -293,17 +351,26 @@ __global__ __launch_bounds__(64 * (rw_cwaves(CPR, NT) + kRwPWaves)) void conv_mf
                         if (f < NF * p.cgt) {  // uniform
                             const int ct = f / NF, r = f - ct * NF, kq = r / NT, nt = r - kq * NT;
                             const uint32_t e = tab[kq * 4 + lg].y;
-                            const uint32_t sh = e & 63u, vmask = (e >> 8) & 0xFFFFu;
+                            const uint32_t sh = e & 63u, nv = (e >> 8) & 63u;
+                            const uint32_t vmask = nv >= 32u ? 0xFFFFFFFFu : (1u << nv) - 1u;
                             const bool live = (int)e < 0 && n0 + (ct * NT + nt) * 16 + li < p.O;
-                            const uint4 e16 = expand_half((uint32_t)(fw[i] >> sh) & vmask, 0);
+                            const uint32_t fbits = (uint32_t)(fw[i] >> sh) & vmask;
+                            const uint4 e16 = Q ? expand32_fp4(fbits) : expand_half(fbits, 0);
                             *reinterpret_cast<uint4 *>(bst + (f * 64 + lane) * 16) = live ? e16 : make_uint4(0u, 0u, 0u, 0u);
                         }
                     }
                     // thresholds in dot-product terms: 2*popc > t  <=>  popc > (t>>1)  <=>  dot < K - 2*(t>>1)
                     if ((MODE == 2 || MODE == 3) && ttid < 64) {
                         int64_t td = n0 + ttid < p.O ? (int64_t)p.K - 2 * (int64_t)(traw >> 1) : -2147483648LL;
-                        td = td > 2147483647LL ? 2147483647LL : (td < -2147483648LL ? -2147483648LL : td);
-                        reinterpret_cast<int *>(bst + NF * CGTMAX * 1024)[ttid] = (int)td;
+                        if (Q) {
+                            // every dot product lies in [-K, K]: thresholds outside mean always / never and are
+                            // pulled in to K + 1 / -K - 1, which fp32 holds exactly
+                            td = td > p.K + 1 ? p.K + 1 : (td < -p.K - 1 ? -p.K - 1 : td);
+                            reinterpret_cast<float *>(bst + NF * CGTMAX * 1024)[ttid] = (float)td;
+                        } else {
+                            td = td > 2147483647LL ? 2147483647LL : (td < -2147483648LL ? -2147483648LL : td);
+                            reinterpret_cast<int *>(bst + NF * CGTMAX * 1024)[ttid] = (int)td;
+                        }
                     }
                 }
                 // the filter words of the next task get the whole image expansion as a head start
@@ -341,24 +408,29 @@ __global__ __launch_bounds__(64 * (rw_cwaves(CPR, NT) + kRwPWaves)) void conv_mf
                             }
                         }
                     };
-                    if (CPR == 1 && p.CB == 16) {
+                    if (Q == 0 && CPR == 1 && p.CB == 16) {
                         fill_narrow(std::integral_constant<int, 1>{});
-                    } else if (CPR <= 2 && p.CB == 32) {
+                    } else if (Q == 0 && CPR <= 2 && p.CB == 32) {
                         fill_narrow(std::integral_constant<int, 2>{});
                     } else
                     for (int cw = 0; cw < p.Cw; cw++) {
                         if (cw > 0) request(wd, cur, cw);
-                        const int nbytes = p.CB - cw * 64 < 64 ? p.CB - cw * 64 : 64;  // positions held by this word
-                        unsigned char *dst = img + __mul24(ttid, p.PS) + cw * 64;
+                        const int nbytes = Q ? 32 : (p.CB - cw * 64 < 64 ? p.CB - cw * 64 : 64);  // bytes this word expands to
+                        unsigned char *dst = img + __mul24(ttid, p.PS) + cw * (Q ? 32 : 64);
                         const int dstep = kRwTeam * p.PS;
 #pragma unroll
                         for (int u = 0; u < kRwItems; u++) {
                             if (ttid + u * kRwTeam < npix) {
                                 const uint32_t lo = (uint32_t)wd[u], hi = (uint32_t)(wd[u] >> 32);
+                                if (Q) {
+                                    *reinterpret_cast<uint4 *>(dst) = expand32_fp4(lo);
+                                    *reinterpret_cast<uint4 *>(dst + 16) = expand32_fp4(hi);
+                                } else {
 #pragma unroll
-                                for (int c = 0; c < 4; c++)
-                                    if (16 * c < nbytes)  // uniform
-                                        *reinterpret_cast<uint4 *>(dst + 16 * c) = expand_half(c < 2 ? lo : hi, c & 1);
+                                    for (int c = 0; c < 4; c++)
+                                        if (16 * c < nbytes)  // uniform
+                                            *reinterpret_cast<uint4 *>(dst + 16 * c) = expand_half(c < 2 ? lo : hi, c & 1);
+                                }
                             }
                             dst += dstep;
                         }
@@ -383,7 +455,7 @@ __global__ __launch_bounds__(64 * (rw_cwaves(CPR, NT) + kRwPWaves)) void conv_mf
         koff[q] = __mul24((j < p.fy ? j : 0) + li, p.PS) + p.qc[q] + 16 * (lg & p.cmask);
     }
     v4i B[NK][NT];
-    int tdot[NT];
+    acc_s tdot[NT];
 #pragma unroll
     for (int kq = 0; kq < NK; kq++)
 #pragma unroll
@@ -418,7 +490,7 @@ __global__ __launch_bounds__(64 * (rw_cwaves(CPR, NT) + kRwPWaves)) void conv_mf
                 if (MODE == 2 || MODE == 3) {
 #pragma unroll
                     for (int nt = 0; nt < NT; nt++)
-                        tdot[nt] = reinterpret_cast<const int *>(bst + NF * CGTMAX * 1024)[(ct * NT + nt) * 16 + li];
+                        tdot[nt] = reinterpret_cast<const acc_s *>(bst + NF * CGTMAX * 1024)[(ct * NT + nt) * 16 + li];
                 }
             }
             for (int u = uw; u < nunits; u += ustep) {
@@ -428,12 +500,13 @@ __global__ __launch_bounds__(64 * (rw_cwaves(CPR, NT) + kRwPWaves)) void conv_mf
                 if (ys >= ye) continue;  // wave-uniform
                 const int x0 = strip * 16;
 
-            int pend[NT][2];  // MODE 3: x-pooled minima of the even row of a pair
+            acc_s pend[NT][2];  // MODE 3: x-pooled minima of the even row of a pair
 #pragma unroll
             for (int nt = 0; nt < NT; nt++) pend[nt][0] = pend[nt][1] = 0;
             // MODE 4: the lane's running sum of dot products over its four pixel columns (columns past the image
             // masked off) and all rows of the unit
-            int csum[NT], cmask[4];
+            acc_s csum[NT];
+            int cmask[4];
 #pragma unroll
             for (int nt = 0; nt < NT; nt++) csum[nt] = 0;
 #pragma unroll
@@ -465,11 +538,12 @@ __global__ __launch_bounds__(64 * (rw_cwaves(CPR, NT) + kRwPWaves)) void conv_mf
                 olane[0] = (uint32_t)__mul24(lane, Ow) << 3;
                 olive[0] = lane < (MODE == 3 ? 8 : 16) && xx0 + lane < ww;
             }
-            auto finish_row = [&](v4i (&a)[NT], int y, int par = -1) {  // par: y & 1 when the caller knows it
+            auto finish_row = [&](acc_t (&a)[NT], int y, int par = -1) {  // par: y & 1 when the caller knows it
                 if (MODE == 4) {
 #pragma unroll
                     for (int nt = 0; nt < NT; nt++)
-                        csum[nt] += (a[nt][0] & cmask[0]) + (a[nt][1] & cmask[1]) + (a[nt][2] & cmask[2]) + (a[nt][3] & cmask[3]);
+                        csum[nt] += (cmask[0] ? a[nt][0] : 0) + (cmask[1] ? a[nt][1] : 0) + (cmask[2] ? a[nt][2] : 0) +
+                                    (cmask[3] ? a[nt][3] : 0);
                     return;
                 }
                 if (MODE == 0) {
@@ -477,7 +551,9 @@ __global__ __launch_bounds__(64 * (rw_cwaves(CPR, NT) + kRwPWaves)) void conv_mf
 #pragma unroll
                     for (int nt = 0; nt < NT; nt++)
 #pragma unroll
-                        for (int r = 0; r < 4; r++) stage[(4 * lg + r) * (16 * NT) + nt * 16 + li] = (p.K - a[nt][r]) >> 1;
+                        for (int r = 0; r < 4; r++)
+                            stage[(4 * lg + r) * (16 * NT) + nt * 16 + li] =
+                                Q ? (int)__builtin_fmaf((float)a[nt][r], -0.5f, 0.5f * (float)p.K) : (p.K - (int)a[nt][r]) >> 1;
                     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
                     __builtin_amdgcn_wave_barrier();
                     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
@@ -518,8 +594,8 @@ __global__ __launch_bounds__(64 * (rw_cwaves(CPR, NT) + kRwPWaves)) void conv_mf
                     }
 #pragma unroll
                     for (int nt = 0; nt < NT; nt++) {
-                        int v0 = a[nt][0] < a[nt][1] ? a[nt][0] : a[nt][1];
-                        int v1 = a[nt][2] < a[nt][3] ? a[nt][2] : a[nt][3];
+                        acc_s v0 = a[nt][0] < a[nt][1] ? a[nt][0] : a[nt][1];
+                        acc_s v1 = a[nt][2] < a[nt][3] ? a[nt][2] : a[nt][3];
                         v0 = v0 < pend[nt][0] ? v0 : pend[nt][0];
                         v1 = v1 < pend[nt][1] ? v1 : pend[nt][1];
                         const uint64_t m0 = __ballot(v0 < tdot[nt]), m1 = __ballot(v1 < tdot[nt]);
@@ -547,11 +623,12 @@ __global__ __launch_bounds__(64 * (rw_cwaves(CPR, NT) + kRwPWaves)) void conv_mf
             const int rowbytes = p.RW * p.PS;
             const int rend = ye + FX - 1;
             const int ylast = MODE == 3 ? (p.h & ~1) - row0 : ye;  // pooled maps drop an odd last row
-            v4i F[CPR], a0[NT], a1[NT];
+            v4i F[CPR];
+            acc_t a0[NT], a1[NT];
 #pragma unroll
             for (int q = 0; q < CPR; q++) F[q] = *reinterpret_cast<const v4i *>(arow + koff[q]);
 #pragma unroll
-            for (int nt = 0; nt < NT; nt++) a0[nt] = a1[nt] = (v4i){0, 0, 0, 0};
+            for (int nt = 0; nt < NT; nt++) a0[nt] = a1[nt] = (acc_t){0, 0, 0, 0};
             auto edge_step = [&](int rr) {  // first two and last two image rows of the sub-band: some parts are missing
                 v4i Fn[CPR];
                 arow += rowbytes;
@@ -566,7 +643,7 @@ __global__ __launch_bounds__(64 * (rw_cwaves(CPR, NT) + kRwPWaves)) void conv_mf
                     for (int q = 0; q < CPR; q++)
 #pragma unroll
                         for (int nt = 0; nt < NT; nt++)
-                            a0[nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(F[q], B[2 * CPR + q][nt], a0[nt], 0, 0, 0);
+                            a0[nt] = rw_mfma(F[q], B[2 * CPR + q][nt], a0[nt]);
                     if (rr - 2 < ylast) finish_row(a0, rr - 2);
                 }
                 if (rr - 1 >= ys && rr - 1 < ye) {
@@ -576,16 +653,16 @@ __global__ __launch_bounds__(64 * (rw_cwaves(CPR, NT) + kRwPWaves)) void conv_mf
                     for (int q = 0; q < CPR; q++)
 #pragma unroll
                         for (int nt = 0; nt < NT; nt++)
-                            a0[nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(F[q], B[CPR + q][nt], a0[nt], 0, 0, 0);
+                            a0[nt] = rw_mfma(F[q], B[CPR + q][nt], a0[nt]);
                 }
                 if (rr < ye) {
 #pragma unroll
-                    for (int nt = 0; nt < NT; nt++) a1[nt] = (v4i){0, 0, 0, 0};
+                    for (int nt = 0; nt < NT; nt++) a1[nt] = (acc_t){0, 0, 0, 0};
 #pragma unroll
                     for (int q = 0; q < CPR; q++)
 #pragma unroll
                         for (int nt = 0; nt < NT; nt++)
-                            a1[nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(F[q], B[q][nt], a1[nt], 0, 0, 0);
+                            a1[nt] = rw_mfma(F[q], B[q][nt], a1[nt]);
                 }
 #pragma unroll
                 for (int q = 0; q < CPR; q++) F[q] = Fn[q];
@@ -598,7 +675,7 @@ __global__ __launch_bounds__(64 * (rw_cwaves(CPR, NT) + kRwPWaves)) void conv_mf
             // know at compile time to be free of branches.
             v4i G[CPR];
             auto row_step = [&](v4i (&Fu)[CPR], v4i (&Fl)[CPR], int r, int par) {
-                v4i done[NT];
+                acc_t done[NT];
                 arow += rowbytes;
 #pragma unroll
                 for (int q = 0; q < CPR; q++) Fl[q] = *reinterpret_cast<const v4i *>(arow + koff[q]);
@@ -608,21 +685,21 @@ __global__ __launch_bounds__(64 * (rw_cwaves(CPR, NT) + kRwPWaves)) void conv_mf
                 for (int q = 0; q < CPR; q++)
 #pragma unroll
                     for (int nt = 0; nt < NT; nt++)
-                        done[nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(Fu[q], B[2 * CPR + q][nt], done[nt], 0, 0, 0);
+                        done[nt] = rw_mfma(Fu[q], B[2 * CPR + q][nt], done[nt]);
 #pragma unroll
                 for (int nt = 0; nt < NT; nt++) a0[nt] = a1[nt];
 #pragma unroll
                 for (int q = 0; q < CPR; q++)
 #pragma unroll
                     for (int nt = 0; nt < NT; nt++)
-                        a0[nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(Fu[q], B[CPR + q][nt], a0[nt], 0, 0, 0);
+                        a0[nt] = rw_mfma(Fu[q], B[CPR + q][nt], a0[nt]);
 #pragma unroll
-                for (int nt = 0; nt < NT; nt++) a1[nt] = (v4i){0, 0, 0, 0};
+                for (int nt = 0; nt < NT; nt++) a1[nt] = (acc_t){0, 0, 0, 0};
 #pragma unroll
                 for (int q = 0; q < CPR; q++)
 #pragma unroll
                     for (int nt = 0; nt < NT; nt++)
-                        a1[nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(Fu[q], B[q][nt], a1[nt], 0, 0, 0);
+                        a1[nt] = rw_mfma(Fu[q], B[q][nt], a1[nt]);
                 finish_row(done, r - 2, par);  // r - 2 < ye - 2 <= ylast
             };
             for (; rr + 1 < ye; rr += 2) {
@@ -642,7 +719,7 @@ __global__ __launch_bounds__(64 * (rw_cwaves(CPR, NT) + kRwPWaves)) void conv_mf
                 const int kn = p.K * (ye - ys) * cols;
 #pragma unroll
                 for (int nt = 0; nt < NT; nt++) {
-                    int v = csum[nt];
+                    int v = (int)csum[nt];
                     v += __shfl_xor(v, 16);
                     v += __shfl_xor(v, 32);
                     const int ch = n0 + nt * 16 + li;
@@ -662,14 +739,14 @@ static inline int rw_round_up(int a, int b) { return (a + b - 1) / b * b; }
 struct RwFit {
     int cus, regs;
 };
-template <int CPR, int NT, int MODE>
+template <int CPR, int NT, int MODE, int Q>
 static bool rw_launch_one(const RwConv &p, int64_t D, size_t lds_bytes, hipStream_t s)
 {
     // Per device (the attribute belongs to the device's copy of the kernel).  Benign race: every thread computes
     // the same values.
     constexpr int kMaxDevices = 16;
     static RwFit fits[kMaxDevices] = {};
-    auto *kfn = conv_mfma_kernel<CPR, NT, MODE>;
+    auto *kfn = conv_mfma_kernel<CPR, NT, MODE, Q>;
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
         (void)hipGetLastError();
@@ -700,26 +777,30 @@ static bool rw_launch_one(const RwConv &p, int64_t D, size_t lds_bytes, hipStrea
 }
 
 template <int MODE>
-static bool rw_launch_mode(const RwConv &p, int64_t D, int CPR, int NT, size_t lds, hipStream_t s)
+static bool rw_launch_mode(const RwConv &p, int64_t D, int CPR, int NT, int q, size_t lds, hipStream_t s)
 {
-#define NB_RW(cpr, nt) \
-    if (CPR == cpr && NT == nt) return rw_launch_one<cpr, nt, MODE>(p, D, lds, s)
-    NB_RW(1, 1);
-    NB_RW(1, 2);
-    NB_RW(2, 1);
-    NB_RW(2, 2);
-    NB_RW(3, 1);
-    NB_RW(3, 2);
-    NB_RW(6, 1);
+#define NB_RW(cpr, nt, qq) \
+    if (CPR == cpr && NT == nt && q == qq) return rw_launch_one<cpr, nt, MODE, qq>(p, D, lds, s)
+    NB_RW(1, 1, 0);
+    NB_RW(1, 2, 0);
+    NB_RW(2, 1, 0);
+    NB_RW(2, 2, 0);
+    NB_RW(3, 1, 0);
+    NB_RW(3, 2, 0);
+    NB_RW(6, 1, 0);
+    NB_RW(2, 1, 1);  // FP4: 64 channels (one word per pixel, two tap columns per 128-position chunk)
+    NB_RW(2, 2, 1);
+    NB_RW(3, 1, 1);  // FP4: 128 channels (one chunk per tap column)
+    NB_RW(3, 2, 1);
+    NB_RW(6, 1, 1);  // FP4: 256 channels
 #undef NB_RW
     return false;
 }
 
-// mode as in conv_impl (0 int32, 2 packed, 3 packed+pooled).  tap_bits > 0: the filter is tap-packed and the
-// input has tap_bits true channels in one word per pixel.  Returns false when this shape has no kernel here;
-// nothing has been launched then.
-bool conv_mfma_try(void *out, const uint64_t *in, const uint64_t *filt, const int32_t *thresh, const ConvGeom &g,
-                 int64_t D, int O, int tap_bits, int mode, hipStream_t s)
+// One attempt with +-1 bytes (q = 0) or FP4 codes (q = 1).  Returns false when this shape has no kernel in that
+// flavour; nothing has been launched then.
+static bool rw_try(void *out, const uint64_t *in, const uint64_t *filt, const int32_t *thresh, const ConvGeom &g,
+                   int64_t D, int O, int tap_bits, int mode, int q, hipStream_t s)
 {
     if (!aligned(out, 16)) return false;
     if (mode != 0 && mode != 2 && mode != 3 && mode != 4) return false;
@@ -739,7 +820,9 @@ bool conv_mfma_try(void *out, const uint64_t *in, const uint64_t *filt, const in
     p.H = g.H; p.Wd = g.Wd; p.Cw = g.Cw; p.px = g.px; p.py = g.py; p.h = g.h; p.w = g.w;
     p.O = O;
     p.fy = g.fy;
-    const int CB = tap_bits > 0 ? (tap_bits <= 16 ? 16 : 32) : 64 * g.Cw;
+    if (q && (tap_bits > 0 || (g.Cw != 1 && g.Cw != 2 && g.Cw != 4))) return false;
+    const int CB = q ? 32 * g.Cw : tap_bits > 0 ? (tap_bits <= 16 ? 16 : 32) : 64 * g.Cw;  // bytes per pixel
+    const int nch = CB >> 6;                                                              // 64-byte pieces of a pixel
     p.CB = CB;
     p.in_bits = tap_bits > 0 ? tap_bits : 64 * g.Cw;
     p.tapT = tap_bits > 0 ? 64 / tap_bits : 0;
@@ -753,14 +836,14 @@ bool conv_mfma_try(void *out, const uint64_t *in, const uint64_t *filt, const in
     } else if (CB == 32) {
         CPR = (g.fy + 1) / 2;
         p.jsh = 1; p.cmask = 1;
-        for (int q = 0; q < CPR; q++) { p.qj[q] = (short)(2 * q); p.qc[q] = 0; }
+        for (int c = 0; c < CPR; c++) { p.qj[c] = (short)(2 * c); p.qc[c] = 0; }
     } else {
-        CPR = g.fy * g.Cw;
+        CPR = g.fy * nch;
         if (CPR > kRwMaxCPR) return false;
         p.jsh = 2; p.cmask = 3;
-        for (int q = 0; q < CPR; q++) { p.qj[q] = (short)(q / g.Cw); p.qc[q] = (short)(64 * (q % g.Cw)); }
+        for (int c = 0; c < CPR; c++) { p.qj[c] = (short)(c / nch); p.qc[c] = (short)(64 * (c % nch)); }
     }
-    for (int q = CPR; q < kRwMaxCPR; q++) p.qj[q] = p.qc[q] = 0;
+    for (int c = CPR; c < kRwMaxCPR; c++) p.qj[c] = p.qc[c] = 0;
     if (CPR == 4 || CPR == 5) return false;
     // A consumer wave keeps the fragments of 16*NT channels in registers (at most 72 of its 168); a task covers
     // cgt such tiles: 64 channels when there are that many, else all of them.
@@ -779,7 +862,7 @@ bool conv_mfma_try(void *out, const uint64_t *in, const uint64_t *filt, const in
     p.PS = ((CB >> 4) & 1) ? CB : CB + 16;
     p.ntx = (g.w + 15) / 16;
     p.RW = 16 * p.ntx + g.fy - 1;
-    p.K = 3 * g.fy * CB;
+    p.K = 3 * g.fy * (q ? 64 * g.Cw : CB);  // positions
     p.pix_q = kRwTeam / p.RW;
     p.pix_r = kRwTeam % p.RW;
     p.D = D;
@@ -805,10 +888,21 @@ bool conv_mfma_try(void *out, const uint64_t *in, const uint64_t *filt, const in
     int nsub = p.ntx >= wpt ? 1 : (wpt + p.ntx - 1) / p.ntx;
     p.hb = rw_round_up((p.hs + nsub - 1) / nsub, 2);
     p.nsub = (p.hs + p.hb - 1) / p.hb;
-    if (mode == 0) return rw_launch_mode<0>(p, D, CPR, NT, lds, s);
-    if (mode == 2) return rw_launch_mode<2>(p, D, CPR, NT, lds, s);
-    if (mode == 4) return rw_launch_mode<4>(p, D, CPR, NT, lds, s);
-    return rw_launch_mode<3>(p, D, CPR, NT, lds, s);
+    if (mode == 0) return rw_launch_mode<0>(p, D, CPR, NT, q, lds, s);
+    if (mode == 2) return rw_launch_mode<2>(p, D, CPR, NT, q, lds, s);
+    if (mode == 4) return rw_launch_mode<4>(p, D, CPR, NT, q, lds, s);
+    return rw_launch_mode<3>(p, D, CPR, NT, q, lds, s);
+}
+
+// mode as in conv_impl (0 int32, 2 packed, 3 packed+pooled, 4 pixel sums).  tap_bits > 0: the filter is tap-packed
+// and the input has tap_bits true channels in one word per pixel.  Returns 0 when this shape has no kernel here
+// (nothing has been launched then), 2 when the int8 kernel ran, 4 when the FP4 kernel ran (full channel words of 64,
+// 128 or 256 channels; results are identical).
+int conv_mfma_try(void *out, const uint64_t *in, const uint64_t *filt, const int32_t *thresh, const ConvGeom &g,
+                  int64_t D, int O, int tap_bits, int mode, bool allow_fp4, hipStream_t s)
+{
+    if (allow_fp4 && rw_try(out, in, filt, thresh, g, D, O, tap_bits, mode, 1, s)) return 4;
+    return rw_try(out, in, filt, thresh, g, D, O, tap_bits, mode, 0, s) ? 2 : 0;
 }
 
 }  // namespace nb

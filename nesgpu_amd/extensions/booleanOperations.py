@@ -153,14 +153,16 @@ def bmm_act(A, B, threshold):
 
 
 def conv_engine(engine=None):
-    """Query / set the process-wide conv engine: 0 = automatic (int8 matrix cores on the shapes where they measured
-    faster, else XOR-popcount), 1 = XOR-popcount kernels only, 2 = matrix cores wherever a kernel covers the shape.
+    """Query / set the process-wide conv engine: 0 = automatic (matrix cores for populations of 128 or more, else
+    XOR-popcount), 1 = XOR-popcount kernels only, 2 = matrix cores wherever a kernel covers the shape (FP4 codes for
+    full channel words of 64, 128 or 256 channels, +-1 bytes otherwise), 3 = as 2 with +-1 bytes only.
     Returns the previous setting.  Results are identical either way."""
     return _lib.load().nb_conv_engine(-1 if engine is None else int(engine))
 
 
 def conv_last_engine():
-    """Engine that served this thread's latest conv launch: 1 = XOR-popcount, 2 = matrix cores, 0 = none yet."""
+    """Engine that served this thread's latest conv launch: 1 = XOR-popcount, 2 = matrix cores on +-1 bytes (int8
+    MFMA), 4 = matrix cores on FP4 codes, 0 = none yet."""
     return _lib.load().nb_conv_last_engine()
 
 

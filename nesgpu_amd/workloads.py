@@ -24,6 +24,7 @@ T_P05 = 214748364
 HBM_PEAK = 8.0e12                     # B/s, MI355X datasheet
 VALU_POPC_PEAK = 6.29e14              # bit-MAC/s: 256 CU x 64 lanes x 2.4 GHz / (4 lane-ops per 64 bits) x 64
 MFMA_INT8_PEAK = 2.5e15               # byte-MAC/s: dense int8 5.0 POP/s, one +-1 byte MAC per bit-MAC
+MFMA_FP4_PEAK = 5.05e15               # MAC/s: dense FP4 10.1 PFLOP/s, one +-1 FP4 MAC per bit-MAC
 
 
 @dataclass

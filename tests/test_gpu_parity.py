@@ -23,10 +23,28 @@ def ops():
     return booleanOperations
 
 
-@pytest.fixture(params=[1, 2], ids=["popcount", "matrixcore"])
+@pytest.fixture(params=[2, 3], ids=["fp4-where-it-exists", "int8-only"])
+def mc_engine(request):
+    """The two matrix-core settings: 2 = FP4 kernel where it exists, 3 = int8 kernel only."""
+    return request.param
+
+
+def _fp4_shape(C, O, fy):
+    """Shapes the FP4 flavour of the matrix-core kernel takes: 3 x fy windows on full channel words (1, 2 or 4 words
+    per pixel, no tap packing: more than 32 channels), more than one 128-position chunk per filter row, and the
+    output-channel counts the kernel tiles (16, 32, or 64 and more; not 32 with four words per pixel)."""
+    Cw = (C + 63) // 64
+    if C <= 32 or Cw not in (1, 2, 4) or O % 16:
+        return False
+    cpr = (fy + 1) // 2 if Cw == 1 else fy * (Cw // 2)           # 128-position chunks per filter row
+    return cpr in (2, 3, 6) and (O >= 64 or O == 16 or (O == 32 and cpr != 6))
+
+
+@pytest.fixture(params=[1, 2, 3], ids=["popcount", "matrixcore", "matrixcore-int8"])
 def engine(request, ops):
-    """Runs a conv test once per engine: 1 = XOR-popcount kernels only, 2 = int8 matrix cores wherever that kernel
-    covers the shape (the XOR-popcount kernels take the rest)."""
+    """Runs a conv test once per engine: 1 = XOR-popcount kernels only, 2 = matrix cores wherever a kernel covers the
+    shape (FP4 codes for full channel words of 64, 128 or 256 channels, +-1 bytes otherwise; the XOR-popcount kernels
+    take the rest), 3 = the same with +-1 bytes only."""
     prev = ops.conv_engine(request.param)
     yield request.param
     ops.conv_engine(prev)
@@ -469,9 +487,9 @@ MATRIX_CORE_CASES = [
 
 
 @pytest.mark.parametrize("C,O,k,pad,H,W,tap,covered", MATRIX_CORE_CASES)
-def test_conv_matrix_core_engine_vs_oracle(ops, oracle, C, O, k, pad, H, W, tap, covered):
-    """Engine 2 on shapes chosen per kernel variant: int32 sums, packed and pooled outputs against the oracle,
-    and the engine that actually served the call."""
+def test_conv_matrix_core_engine_vs_oracle(ops, oracle, mc_engine, C, O, k, pad, H, W, tap, covered):
+    """The matrix-core engines on shapes chosen per kernel variant: int32 sums, packed and pooled outputs against the
+    oracle, and the engine that actually served the call (1 popcount, 2 int8, 4 FP4)."""
     D = 3
     g = rng(C * 1000 + O * 10 + k + H + W)
     Cw = (C + 63) // 64
@@ -495,13 +513,14 @@ def test_conv_matrix_core_engine_vs_oracle(ops, oracle, C, O, k, pad, H, W, tap,
     act = oracle.conv_act(x, f, thr, *geom)
     h, w = act.shape[1:3]
     packed = oracle.pack(act.reshape(-1, O), np.int64).reshape(D, h, w, -1)
-    prev = ops.conv_engine(2)
+    served = 4 if mc_engine == 2 and k == 3 and _fp4_shape(C, O, k) else (2 if covered else 1)
+    prev = ops.conv_engine(mc_engine)
     try:
         got = ops.conv(xd, fd, *geom, **kw)
-        assert ops.conv_last_engine() == (2 if covered else 1)
+        assert ops.conv_last_engine() == served
         np.testing.assert_array_equal(host(got), want)
         got = ops.conv_act_pack(xd, fd, td, *geom, **kw)
-        assert ops.conv_last_engine() == (2 if covered else 1)
+        assert ops.conv_last_engine() == served
         np.testing.assert_array_equal(host(got), packed)
         got = ops.conv_act_pack(xd, fd, td, *geom, pool=True, **kw)
         np.testing.assert_array_equal(host(got), oracle.max_pool2d(packed, 2, 2, 0, 0, 2, 2))
@@ -529,11 +548,11 @@ def _random_matrix_core_cases(n, seed):
     return cases
 
 
-def test_conv_matrix_core_random_shapes(ops, oracle):
+def test_conv_matrix_core_random_shapes(ops, oracle, mc_engine):
     """Forty-eight seeded random shapes (channels, output channels, 3 x fy windows, unequal paddings, ragged image
     sizes, 1-5 members, filters tap-packed or not) with engine 2 asked for: all four outputs against the oracle, and
     the matrix-core kernel serves exactly the shapes it is built for."""
-    prev = ops.conv_engine(2)
+    prev = ops.conv_engine(mc_engine)
     try:
         for ci, (C, O, fy, px, py, H, W, D, tap) in enumerate(_random_matrix_core_cases(48, 20240607)):
             print("case", ci, (C, O, fy, px, py, H, W, D, tap), flush=True)
@@ -561,8 +580,13 @@ def test_conv_matrix_core_random_shapes(ops, oracle):
             cpr = (1 if C <= 16 else (fy + 1) // 2) if C <= 32 else fy * Cw
             covered = cpr in (1, 2, 3, 6) and (O >= 64 or O == 16 or (O == 32 and cpr != 6))
             np.testing.assert_array_equal(host(ops.conv(xd, fd, *geom, **kw)), want)
-            if cpr != 6:                                 # with 6 chunks it also depends on the band fitting the LDS
+            fp4 = mc_engine == 2 and _fp4_shape(C, O, fy)
+            if fp4 and not (Cw == 4 and fy == 3):        # six chunks: also depends on the band fitting the LDS
+                assert ops.conv_last_engine() == 4
+            elif not fp4 and cpr != 6:                   # likewise with 6 chunks of +-1 bytes
                 assert ops.conv_last_engine() == (2 if covered else 1)
+            if mc_engine == 3:
+                assert ops.conv_last_engine() != 4
             np.testing.assert_array_equal(host(ops.conv_act_pack(xd, fd, td, *geom, **kw)), packed)
             if h >= 2 and w >= 2:
                 got = ops.conv_act_pack(xd, fd, td, *geom, pool=True, **kw)
@@ -575,7 +599,7 @@ def test_conv_matrix_core_random_shapes(ops, oracle):
 
 @pytest.mark.parametrize("C,O,S,mode", [(16, 16, 8, "pool"), (64, 64, 8, "pool"), (64, 128, 6, "pack"),
                                          (64, 64, 8, "sums"), (3, 64, 10, "pack")])
-def test_conv_matrix_core_many_members(ops, oracle, C, O, S, mode):
+def test_conv_matrix_core_many_members(ops, oracle, mc_engine, C, O, S, mode):
     """More members than workgroups: every workgroup of the persistent kernel walks several members (fragments and
     image buffers change hands many times); every member against the oracle."""
     D = 1300
@@ -589,17 +613,18 @@ def test_conv_matrix_core_many_members(ops, oracle, C, O, S, mode):
     geom = (3, 3, 1, 1, 1, 1)
     xd, fd, td = dev(x), dev(f), dev(thr)
     kw = dict(in_bits=C) if C < 64 else {}
-    prev = ops.conv_engine(2)
+    served = 4 if mc_engine == 2 and _fp4_shape(C, O, 3) else 2
+    prev = ops.conv_engine(mc_engine)
     try:
         if mode == "sums":
             got = ops.conv(xd, fd, *geom, **kw)
-            assert ops.conv_last_engine() == 2
+            assert ops.conv_last_engine() == served
             np.testing.assert_array_equal(host(got), oracle.conv(x, f, *geom))
         else:
             act = oracle.conv_act(x, f, thr, *geom)
             packed = oracle.pack(act.reshape(-1, O), np.int64).reshape(D, S, S, -1)
             got = ops.conv_act_pack(xd, fd, td, *geom, pool=(mode == "pool"), **kw)
-            assert ops.conv_last_engine() == 2
+            assert ops.conv_last_engine() == served
             np.testing.assert_array_equal(host(got), oracle.max_pool2d(packed, 2, 2, 0, 0, 2, 2) if mode == "pool" else packed)
     finally:
         ops.conv_engine(prev)
@@ -633,6 +658,7 @@ def test_conv_popc_sums_vs_oracle(ops, oracle, engine, dtype, C, O, k, pad, stri
 
 def test_conv_engine_selector_round_trip(ops):
     prev = ops.conv_engine()
-    assert prev in (0, 1, 2)
-    assert ops.conv_engine(2) == prev and ops.conv_engine(1) == 2 and ops.conv_engine(7) == 1 and ops.conv_engine() == 1
+    assert prev in (0, 1, 2, 3)
+    assert ops.conv_engine(2) == prev and ops.conv_engine(3) == 2 and ops.conv_engine(1) == 3
+    assert ops.conv_engine(7) == 1 and ops.conv_engine() == 1                 # values out of range change nothing
     ops.conv_engine(prev)
