@@ -901,6 +901,9 @@ static bool rw_try(void *out, const uint64_t *in, const uint64_t *filt, const in
 int conv_mfma_try(void *out, const uint64_t *in, const uint64_t *filt, const int32_t *thresh, const ConvGeom &g,
                   int64_t D, int O, int tap_bits, int mode, bool allow_fp4, hipStream_t s)
 {
+    // int32 maps of a 64-channel layer with up to 64 output channels are bound by writing the maps; there the FP4
+    // flavour measured no faster (52.9 against 49.6 us at 32x32, population 1024) and the +-1 bytes stay.
+    if (mode == 0 && g.Cw == 1 && O <= 64) allow_fp4 = false;
     if (allow_fp4 && rw_try(out, in, filt, thresh, g, D, O, tap_bits, mode, 1, s)) return 4;
     return rw_try(out, in, filt, thresh, g, D, O, tap_bits, mode, 0, s) ? 2 : 0;
 }
