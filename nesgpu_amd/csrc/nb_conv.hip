@@ -259,6 +259,12 @@ int conv_impl(void *out, const W *in, const W *filt, const int32_t *thresh, int6
     // Automatic choice, measured on MI355X: one workgroup per CU walks whole members, so the matrix-core kernel needs
     // a population that fills at least half of the CUs; below that the XOR-popcount kernels, which spread one
     // member's pixels over many workgroups, are faster.
+    // A window of at most 32 bits (3x3 on up to 3 channels) with packed output: one register per pixel, four vector
+    // instructions per output channel; faster than either engine on that shape.
+    if (engine <= 1 && Cw > 0 && conv_window_try<W>(out, in, filt, thresh, g, D, N, tap_bits, mode, s)) {
+        t_last_engine = 1;
+        return check_launch(who);
+    }
     if (bits == 64 && Cw > 0 && engine != 1 && (engine >= 2 || D >= 128)) {
         const int ran = conv_mfma_try(out, reinterpret_cast<const uint64_t *>(in), reinterpret_cast<const uint64_t *>(filt),
                                       thresh, g, D, N, tap_bits, mode, engine != 3, s);

@@ -72,6 +72,12 @@ template <typename W>
 void conv_tap_launch(void *out, const W *in, const W *filt, const int32_t *thresh, const ConvGeom &g, int64_t D,
                      int64_t lanes, int N, int tap_bits, int mode, hipStream_t s);
 
+// Window-in-a-register kernel (nb_conv_tap.hip): mode 2 on tap-packed filters whose whole window fits 32 bits.
+// false = not this shape, nothing launched.
+template <typename W>
+bool conv_window_try(void *out, const W *in, const W *filt, const int32_t *thresh, const ConvGeom &g, int64_t D, int O,
+                     int tap_bits, int mode, hipStream_t s);
+
 // Matrix-core conv (nb_conv_mfma.hip): 3-row filters, stride 1, O % 16 == 0; mode as in conv_impl (0, 2, 3, 4).
 // 0 = no kernel for this shape, nothing launched; 2 = the int8 kernel ran; 4 = the FP4 kernel ran (allow_fp4 only).
 int conv_mfma_try(void *out, const uint64_t *in, const uint64_t *filt, const int32_t *thresh, const ConvGeom &g,

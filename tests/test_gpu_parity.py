@@ -633,6 +633,56 @@ def test_conv_matrix_core_many_members(ops, oracle, mc_engine, C, O, S, mode):
 
 
 @pytest.mark.parametrize("dtype", [torch.int64, torch.int32])
+@pytest.mark.parametrize("C,O,fx,fy,px,py,sx,sy,H,W,D", [
+    (3, 64, 3, 3, 1, 1, 1, 1, 32, 32, 5),      # the first layer of an RGB network
+    (3, 128, 3, 3, 1, 1, 1, 1, 9, 21, 3),      # two output words per pixel
+    (3, 40, 3, 3, 0, 2, 1, 1, 7, 300, 2),      # O not a multiple of 32, more pixels than one workgroup per row
+    (2, 100, 3, 3, 2, 0, 2, 1, 11, 13, 4),     # strides, 18-bit window
+    (1, 16, 5, 5, 2, 2, 1, 2, 12, 12, 3),      # 25-bit window
+    (1, 33, 3, 1, 1, 0, 1, 1, 6, 6, 2),
+    (3, 64, 3, 3, 1, 1, 1, 1, 5, 5, 300),      # many members
+    (1, 32, 5, 5, 2, 2, 1, 1, 10, 11, 2),      # stride 1 with one to five window rows / columns: the row gather
+    (2, 48, 2, 4, 0, 3, 1, 1, 9, 10, 2),
+    (4, 32, 1, 5, 0, 1, 1, 1, 4, 7, 3),
+    (1, 64, 4, 2, 3, 1, 1, 1, 5, 6, 2),
+    (5, 24, 2, 3, 1, 2, 1, 1, 3, 3, 7),        # output wider than the input
+])
+def test_conv_window_in_a_register_vs_oracle(ops, oracle, dtype, C, O, fx, fy, px, py, sx, sy, H, W, D):
+    """Windows of at most 32 bits with packed output take the window-in-a-register kernel (engines 0 and 1):
+    against the oracle, with the filter tap-packed by the caller or on the fly, and identical to the matrix-core
+    answer where that engine has a kernel."""
+    nd = NDT[dtype]
+    bits = np.dtype(nd).itemsize * 8
+    g = rng(C * 100 + O + fx + H)
+    x = oracle.pack(g.integers(0, 2, size=(D * H * W, C)).astype(bool), nd).reshape(D, H, W, 1)
+    fb = g.integers(0, 2, size=(D * O * fx * fy, C)).astype(bool)
+    f = np.ascontiguousarray(oracle.pack(fb, nd).reshape(D, O, fx, fy, 1).transpose(0, 2, 3, 4, 1).reshape(D, -1, O))
+    K = fx * fy * C
+    thr = (g.integers(0, K + 3, size=(D, O)) - K // 2 + K - 1).astype(np.int32)
+    thr[0, 0], thr[0, 1] = -7, 2 * K + 5                                     # always / never above the threshold
+    geom = (fx, fy, px, py, sx, sy)
+    act = oracle.conv_act(x, f, thr, *geom)
+    h, w = act.shape[1:3]
+    want = oracle.pack(act.reshape(-1, O), nd).reshape(D, h, w, -1)
+    xd, fd, td = dev(x), dev(f), dev(thr)
+    prev = ops.conv_engine(0)
+    try:
+        for eng in (0, 1):
+            ops.conv_engine(eng)
+            np.testing.assert_array_equal(host(ops.conv_act_pack(xd, fd, td, *geom, in_bits=C)), want)
+            assert ops.conv_last_engine() == 1
+            ft = ops.tap_pack_filter(fd, fx * fy, C)
+            got = ops.conv_act_pack(xd, ft, td, *geom, in_bits=C, filter_tap_packed=True)
+            np.testing.assert_array_equal(host(got), want)
+        if bits == 64 and fx == 3 and sx == 1 and sy == 1 and O % 16 == 0:
+            ops.conv_engine(2)
+            np.testing.assert_array_equal(host(ops.conv_act_pack(xd, fd, td, *geom, in_bits=C)), want)
+            assert ops.conv_last_engine() == 2
+    finally:
+        ops.conv_engine(prev)
+
+
+@pytest.mark.parametrize("dtype", [torch.int64, torch.int32])
 @pytest.mark.parametrize("C,O,k,pad,stride,H,W,D", [(16, 16, 3, 1, 1, 9, 20, 5), (64, 64, 3, 1, 1, 12, 21, 3),
                                                      (3, 64, 3, 1, 1, 10, 10, 4), (64, 144, 3, 0, 1, 8, 8, 3),
                                                      (128, 64, 3, 1, 1, 6, 18, 2), (20, 7, 5, 2, 2, 11, 9, 3),
