@@ -243,6 +243,20 @@ def conv_popc_sums(input, filter, filterx, filtery, padx, pady, stridex, stridey
     return out
 
 
+def _bool_map_via_packed(input, filter, filterx, filtery, stridex, stridey, tap):
+    """True where conv_act's bool map is better made by a packed-output kernel and unpack: whole output words, and
+    either a shape the matrix-core kernels take (64-bit words, 3-row windows, stride 1, a population of 128 or
+    more; not with the engine pinned to XOR-popcount) or a window of at most 32 bits."""
+    bits = torch.iinfo(input.dtype).bits
+    O = filter.size(2)
+    if O == 0 or O % bits != 0 or input.size(0) * input.size(1) * input.size(2) == 0:
+        return False
+    if tap and filterx * filtery * tap <= 32:
+        return True
+    return (bits == 64 and filterx == 3 and stridex == 1 and stridey == 1 and input.size(0) >= 128
+            and input.size(3) > 0 and conv_engine() != 1)
+
+
 def conv_act(input, filter, threshold, filterx, filtery, padx, pady, stridex, stridey, in_bits=None,
              filter_tap_packed=False):
     """bmm_act(batch_im2col(input), filter, threshold).view(D,h,w,O) (extensions/booleanOperations.py:168-172)."""
@@ -254,6 +268,12 @@ def conv_act(input, filter, threshold, filterx, filtery, padx, pady, stridex, st
     assert threshold.size(1) == filter.size(2)
     assert threshold.dtype == torch.int32
     h, w = _out_hw(input, filterx, filtery, padx, pady, stridex, stridey)
+    if _bool_map_via_packed(input, filter, filterx, filtery, stridex, stridey, tap):
+        # the packed-output kernels (matrix cores, window-in-a-register) followed by unpack: same bools, and faster
+        # than the XOR-popcount kernel that writes bool bytes itself, although the bits make one more trip
+        packed = conv_act_pack(input, filter, threshold, filterx, filtery, padx, pady, stridex, stridey,
+                               in_bits=tap if tap else None, filter_tap_packed=bool(tap))
+        return unpack(packed.view(-1, packed.size(3))).view(input.size(0), h, w, filter.size(2))
     out = torch.empty((input.size(0), h, w, filter.size(2)), dtype=torch.bool, device=input.device)
     with _on(input):
         _lib.call("nb_conv_act" + suf, out.data_ptr(), input.data_ptr(), filter.data_ptr(), threshold.data_ptr(),

@@ -526,8 +526,10 @@ def test_conv_matrix_core_engine_vs_oracle(ops, oracle, mc_engine, C, O, k, pad,
         np.testing.assert_array_equal(host(got), packed)
         got = ops.conv_act_pack(xd, fd, td, *geom, pool=True, **kw)
         np.testing.assert_array_equal(host(got), oracle.max_pool2d(packed, 2, 2, 0, 0, 2, 2))
-        np.testing.assert_array_equal(host(ops.conv_act(xd, fd, td, *geom, **kw)), act)   # bool output: popcount kernels
-        assert ops.conv_last_engine() == 1
+        np.testing.assert_array_equal(host(ops.conv_act(xd, fd, td, *geom, **kw)), act)
+        # bool output: the popcount kernels for three members, except a window of at most 32 bits with whole output
+        # words, which goes through the packed-output kernel and unpack
+        assert ops.conv_last_engine() == (served if tap and k * k * C <= 32 and O % 64 == 0 else 1)
         ops.conv_engine(1)
         ops.conv(xd, fd, *geom, **kw)
         assert ops.conv_last_engine() == 1
@@ -628,6 +630,41 @@ def test_conv_matrix_core_many_members(ops, oracle, mc_engine, C, O, S, mode):
             got = ops.conv_act_pack(xd, fd, td, *geom, pool=(mode == "pool"), **kw)
             assert ops.conv_last_engine() == served
             np.testing.assert_array_equal(host(got), oracle.max_pool2d(packed, 2, 2, 0, 0, 2, 2) if mode == "pool" else packed)
+    finally:
+        ops.conv_engine(prev)
+
+
+@pytest.mark.parametrize("C,O,D,H,W,engine_served", [
+    (64, 64, 130, 6, 7, 4),      # full channel word, a population the matrix cores take: FP4 pack kernel + unpack
+    (100, 128, 128, 5, 5, 4),    # two channel words with zero tail bits
+    (64, 64, 128, 4, 5, 4),
+    (3, 64, 5, 9, 9, 1),         # 27-bit window: window-in-a-register kernel + unpack, any population
+    (64, 64, 5, 6, 6, 1),        # small population: the XOR-popcount kernel writes the bools itself
+    (64, 48, 130, 6, 6, 1),      # O is not a whole number of words: likewise
+])
+def test_conv_act_bool_map_via_packed_kernels(ops, oracle, C, O, D, H, W, engine_served):
+    """conv_act's bool map comes from a packed-output kernel plus unpack where that is the faster way; same bools
+    as the oracle either way, and the same as with the engine pinned to the XOR-popcount kernels."""
+    g = rng(C + O + D)
+    Cw = (C + 63) // 64
+    x = oracle.pack(g.integers(0, 2, size=(D * H * W, C)).astype(bool), np.int64).reshape(D, H, W, Cw)
+    fb = g.integers(0, 2, size=(D * O * 9, C)).astype(bool)
+    f = np.ascontiguousarray(oracle.pack(fb, np.int64).reshape(D, O, 3, 3, Cw).transpose(0, 2, 3, 4, 1).reshape(D, -1, O))
+    K = 9 * C
+    thr = (g.integers(0, K + 1, size=(D, O)) - K // 2 + K).astype(np.int32)
+    geom = (3, 3, 1, 1, 1, 1)
+    want = oracle.conv_act(x, f, thr, *geom)
+    xd, fd, td = dev(x), dev(f), dev(thr)
+    kw = dict(in_bits=C) if C < 32 else {}
+    prev = ops.conv_engine(0)
+    try:
+        got = ops.conv_act(xd, fd, td, *geom, **kw)
+        assert got.dtype == torch.bool and got.is_contiguous() and tuple(got.shape) == want.shape
+        assert ops.conv_last_engine() == engine_served
+        np.testing.assert_array_equal(host(got), want)
+        ops.conv_engine(1)
+        np.testing.assert_array_equal(host(ops.conv_act(xd, fd, td, *geom, **kw)), want)
+        assert ops.conv_last_engine() == 1
     finally:
         ops.conv_engine(prev)
 
