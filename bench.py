@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--extra 1,3,4,5] [--no-cpu]
 
-Headline workload (BASELINE configs[1]): binary linear 1024x1024, population 1024, one input row per member,
+Headline workload (configuration 2 of the five): binary linear 1024x1024, population 1024, one input row per member,
 p = 0.05 flip masks sampled by threshold compare from SUPPLIED uint32 words, fused into the XOR-popcount
 product.  A step is one such population forward with every operand resident in HBM.  Prints one JSON line.
 
