@@ -89,7 +89,9 @@ template void conv_tap_launch<uint32_t>(void *, const uint32_t *, const uint32_t
 // Output: threshold bits packed along O (mode 2).
 constexpr uint32_t kWinOutside = 0xC0000000u;  // a buffer offset no image reaches: the load returns zero
 constexpr int kWinPix = 4;  // pixels per lane: one batch of scalar loads serves four windows
-template <typename W, bool ROWQUAD>
+// GATHER: 0 = any geometry, one pixel's window at a time; 1 = rows of four neighbouring pixels straight from memory;
+// 2 = the same rows out of an LDS copy of the image rows the workgroup's pixels touch.
+template <typename W, int GATHER>
 __global__ __launch_bounds__(256) void conv_window_pack_kernel(W *__restrict__ out, const W *__restrict__ in,
                                                                const W *__restrict__ ftap,
                                                                const int32_t *__restrict__ thresh, ConvGeom g, int O,
@@ -103,7 +105,7 @@ __global__ __launch_bounds__(256) void conv_window_pack_kernel(W *__restrict__ o
     uint32_t win[kWinPix];
     bool live[kWinPix];
     int pcs[kWinPix];
-    if (ROWQUAD) {
+    if (GATHER != 0) {
         // stride 1, windows at most 5 wide: a lane takes four neighbouring pixels of one output row, whose windows
         // share their columns: fx * (fy + 3) words are fetched instead of 4 * fx * fy, with one row / column test each
         const int wq = (g.w + kWinPix - 1) / kWinPix;  // quads per output row
@@ -120,20 +122,79 @@ __global__ __launch_bounds__(256) void conv_window_pack_kernel(W *__restrict__ o
         // (an offset outside the member's image reads as zero, the padding word) need no branch around them
         const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
             const_cast<W *>(img), (short)0, g.H * g.Wd * (int)sizeof(W), 0x00020000);
+        // GATHER == 2: the input rows that the workgroup's 256 quads touch are copied to LDS first, every word
+        // fetched once with coalesced loads (low 32 bits, masked to the channel bits; rows outside the image as
+        // zeros).  A row is stored as four runs, columns 0,4,8.. then 1,5,9.. and so on, so that the lanes of a
+        // wave, which stand four columns apart, read neighbouring LDS words.
+        extern __shared__ uint32_t wl[];
+        const int qs = (g.Wd + 3) / 4 + 1;  // words per run, one spare
+        const int qfirst = (int)(blockIdx.x - z * pixblocks) * 256;
+        const int ya = qfirst / wq - g.px;  // first input row staged
+        if (GATHER == 2) {
+            const int qlast = qfirst + 255 < g.h * wq ? qfirst + 255 : g.h * wq - 1;
+            const int total = (qlast / wq - qfirst / wq + g.fx) * g.Wd;  // staged rows x words per row
+            // word idx = base + 256 * u + thread sits in staged row r at column xx; one division per thread, then
+            // steps of 256 words = rstep rows and xstep columns (wave-uniform)
+            const int rstep = 256 / g.Wd, xstep = 256 - rstep * g.Wd;
+            int r = (int)threadIdx.x / g.Wd, xx = (int)threadIdx.x - r * g.Wd;
+            for (int base = 0; base < total; base += 1024) {
+                uint32_t val[4];
+                int at[4];
+#pragma unroll
+                for (int u = 0; u < 4; u++) {
+                    const int idx = base + u * 256 + (int)threadIdx.x;
+                    const int yy = ya + r;
+                    const bool ok = (idx < total) & ((unsigned)yy < (unsigned)g.H);
+                    const uint32_t off = ok ? (uint32_t)(yy * g.Wd + xx) * (uint32_t)sizeof(W) : kWinOutside;
+                    val[u] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)off, 0, 0) & cm;
+                    at[u] = idx < total ? r * 4 * qs + (xx & 3) * qs + (xx >> 2) : -1;
+                    r += rstep;
+                    xx += xstep;
+                    if (xx >= g.Wd) {
+                        xx -= g.Wd;
+                        r++;
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < 4; u++)
+                    if (at[u] >= 0) wl[at[u]] = val[u];
+            }
+            __syncthreads();
+        }
         auto gather = [&](auto fxc, auto fyc) {
             constexpr int FX = decltype(fxc)::value, FY = decltype(fyc)::value;  // FY: upper bound of g.fy
             constexpr int NC = FY + kWinPix - 1;
             uint32_t v[FX][NC];
+            bool cv[NC];  // column x0 - py + jc lies inside the image (and inside the window's span)
 #pragma unroll
-            for (int i = 0; i < FX; i++) {
-                const int yy = yo - g.px + i;
-                const bool rv = (unsigned)yy < (unsigned)g.H;
+            for (int jc = 0; jc < NC; jc++)
+                cv[jc] = ((unsigned)(x0 - g.py + jc) < (unsigned)g.Wd) & (jc < g.fy + kWinPix - 1);
+            if (GATHER == 2) {
+                int ci[NC];  // place of column x0 - py + jc inside a staged row
 #pragma unroll
-                for (int jc = 0; jc < NC; jc++) {  // column x0 - py + jc serves pixel q as tap column jc - q
+                for (int jc = 0; jc < NC; jc++) {
                     const int xx = x0 - g.py + jc;
-                    const bool inside = rv && (unsigned)xx < (unsigned)g.Wd && jc < g.fy + kWinPix - 1;
-                    const uint32_t off = inside ? (uint32_t)(yy * g.Wd + xx) * (uint32_t)sizeof(W) : kWinOutside;
-                    v[i][jc] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)off, 0, 0) & cm;
+                    ci[jc] = cv[jc] ? (xx & 3) * qs + (xx >> 2) : 0;
+                }
+                const int rbase = (yo - g.px - ya) * 4 * qs;
+#pragma unroll
+                for (int i = 0; i < FX; i++)
+#pragma unroll
+                    for (int jc = 0; jc < NC; jc++) {
+                        const uint32_t t = wl[rbase + i * 4 * qs + ci[jc]];
+                        v[i][jc] = cv[jc] ? t : 0u;  // rows outside the image were staged as zeros
+                    }
+            } else {
+#pragma unroll
+                for (int i = 0; i < FX; i++) {
+                    const int yy = yo - g.px + i;
+                    const bool rv = (unsigned)yy < (unsigned)g.H;
+                    const int rb = yy * g.Wd + x0 - g.py;  // word index of the row's first column
+#pragma unroll
+                    for (int jc = 0; jc < NC; jc++) {  // column x0 - py + jc serves pixel q as tap column jc - q
+                        const uint32_t off = (rv & cv[jc]) ? (uint32_t)(rb + jc) * (uint32_t)sizeof(W) : kWinOutside;
+                        v[i][jc] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)off, 0, 0) & cm;
+                    }
                 }
             }
 #pragma unroll
@@ -248,14 +309,23 @@ bool conv_window_try(void *out, const W *in, const W *filt, const int32_t *thres
     const int64_t hw = (int64_t)g.h * g.w;
     if (hw < 1 || hw >= (1LL << 30) || (int64_t)g.H * g.Wd >= (1LL << 31)) return false;
     if (g.sx == 1 && g.sy == 1 && g.fy <= 5 && g.fx <= 5 && (int64_t)g.H * g.Wd * (int64_t)sizeof(W) < (1 << 30)) {
-        const int64_t pixblocks = ceil_div((int64_t)g.h * ceil_div(g.w, kWinPix), 256);
+        const int wq = (int)ceil_div(g.w, kWinPix);
+        const int64_t pixblocks = ceil_div((int64_t)g.h * wq, 256);
         if (D * pixblocks > kMaxGridX) return false;
-        conv_window_pack_kernel<W, true><<<dim3((unsigned)(D * pixblocks)), dim3(256), 0, s>>>(
-            static_cast<W *>(out), in, filt, thresh, g, O, tap_bits, (int)pixblocks);
+        // LDS copy of the rows a workgroup touches: (rows of 256 quads + fx - 1) x four runs of Wd/4 + 1 words, and
+        // a few words of slack for the reads of columns just past a row (dropped by the column test)
+        const int64_t rows = (255 + wq - 1) / wq + 1 + g.fx - 1;
+        const int64_t lds = (rows * 4 * ((g.Wd + 3) / 4 + 1) + 8) * 4;
+        if (lds <= 48 * 1024)
+            conv_window_pack_kernel<W, 2><<<dim3((unsigned)(D * pixblocks)), dim3(256), (size_t)lds, s>>>(
+                static_cast<W *>(out), in, filt, thresh, g, O, tap_bits, (int)pixblocks);
+        else
+            conv_window_pack_kernel<W, 1><<<dim3((unsigned)(D * pixblocks)), dim3(256), 0, s>>>(
+                static_cast<W *>(out), in, filt, thresh, g, O, tap_bits, (int)pixblocks);
     } else {
         const int64_t pixblocks = ceil_div(hw, 256 * kWinPix);
         if (D * pixblocks > kMaxGridX) return false;
-        conv_window_pack_kernel<W, false><<<dim3((unsigned)(D * pixblocks)), dim3(256), 0, s>>>(
+        conv_window_pack_kernel<W, 0><<<dim3((unsigned)(D * pixblocks)), dim3(256), 0, s>>>(
             static_cast<W *>(out), in, filt, thresh, g, O, tap_bits, (int)pixblocks);
     }
     return true;
