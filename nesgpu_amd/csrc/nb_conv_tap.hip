@@ -308,6 +308,7 @@ bool conv_window_try(void *out, const W *in, const W *filt, const int32_t *thres
     if (mode != 2 || tap_bits <= 0 || g.Cw != 1 || taps * tap_bits > 32 || taps > taps_per_word(bits, tap_bits)) return false;
     const int64_t hw = (int64_t)g.h * g.w;
     if (hw < 1 || hw >= (1LL << 30) || (int64_t)g.H * g.Wd >= (1LL << 31)) return false;
+    if (g.H < 1 || g.Wd < 1) return false;  // an empty image under padding: the general kernels take it
     if (g.sx == 1 && g.sy == 1 && g.fy <= 5 && g.fx <= 5 && (int64_t)g.H * g.Wd * (int64_t)sizeof(W) < (1 << 30)) {
         const int wq = (int)ceil_div(g.w, kWinPix);
         const int64_t pixblocks = ceil_div((int64_t)g.h * wq, 256);
