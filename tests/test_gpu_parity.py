@@ -634,6 +634,42 @@ def test_conv_matrix_core_many_members(ops, oracle, mc_engine, C, O, S, mode):
         ops.conv_engine(prev)
 
 
+def test_conv_window_random_shapes(ops, oracle):
+    """Randomly drawn small-window geometries (1-5 channels, windows up to 5x5 with at most 32 window bits, strides,
+    paddings, ragged channel counts, both word widths): packed and bool outputs against the oracle."""
+    g0 = rng(4242)
+    done = 0
+    for ci in range(260):
+        nd = np.int64 if g0.integers(0, 2) else np.int32
+        bits = np.dtype(nd).itemsize * 8
+        C, fx, fy = int(g0.integers(1, 6)), int(g0.integers(1, 6)), int(g0.integers(1, 6))
+        sx, sy = int(g0.choice([1, 1, 1, 2])), int(g0.choice([1, 1, 1, 2]))
+        px, py = int(g0.integers(0, 4)), int(g0.integers(0, 4))
+        H, W, D = int(g0.integers(1, 40)), int(g0.integers(1, 90)), int(g0.integers(1, 6))
+        O = int(g0.choice([1, 7, 16, 31, 32, 33, 64, 64, 64, 100, 128]))
+        if fx * fy * C > 32 or fx * fy > bits // C or H + 2 * px < fx or W + 2 * py < fy:
+            continue
+        g = rng(100 + ci)
+        x = oracle.pack(g.integers(0, 2, size=(D * H * W, C)).astype(bool), nd).reshape(D, H, W, 1)
+        fb = g.integers(0, 2, size=(D * O * fx * fy, C)).astype(bool)
+        f = np.ascontiguousarray(oracle.pack(fb, nd).reshape(D, O, fx, fy, 1).transpose(0, 2, 3, 4, 1)
+                                 .reshape(D, -1, O))
+        K = fx * fy * C
+        thr = (g.integers(0, K + 3, size=(D, O)) - K // 2 + K - 1).astype(np.int32)
+        geom = (fx, fy, px, py, sx, sy)
+        act = oracle.conv_act(x, f, thr, *geom)
+        h, w = act.shape[1:3]
+        want = oracle.pack(act.reshape(-1, O), nd).reshape(D, h, w, -1)
+        xd, fd, td = dev(x), dev(f), dev(thr)
+        case = "case %d: %s C=%d O=%d window %dx%d pad %d,%d stride %d,%d image %dx%d D=%d" % (
+            ci, np.dtype(nd).name, C, O, fx, fy, px, py, sx, sy, H, W, D)
+        np.testing.assert_array_equal(host(ops.conv_act_pack(xd, fd, td, *geom, in_bits=C)), want, err_msg=case)
+        assert ops.conv_last_engine() == 1, case
+        np.testing.assert_array_equal(host(ops.conv_act(xd, fd, td, *geom, in_bits=C)), act, err_msg=case)
+        done += 1
+    assert done > 100
+
+
 @pytest.mark.parametrize("C,O,D,H,W,engine_served", [
     (64, 64, 130, 6, 7, 4),      # full channel word, a population the matrix cores take: FP4 pack kernel + unpack
     (100, 128, 128, 5, 5, 4),    # two channel words with zero tail bits
