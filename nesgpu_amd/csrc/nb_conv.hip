@@ -99,7 +99,10 @@ __global__ __launch_bounds__(256) void max_pool_2x2_kernel(uint64_t *__restrict_
         // PAIR: u holds input pixels 4e, 4e+1 -> output pixel 2e; v holds 4e+2, 4e+3 -> output pixel 2e+1
         const uint4 r = PAIR ? make_uint4(u.x | u.z, u.y | u.w, v.x | v.z, v.y | v.w)
                              : make_uint4(u.x | v.x, u.y | v.y, u.z | v.z, u.w | v.w);
-        if (k == 0 || t0 + half < total) reinterpret_cast<uint4 *>(out)[tt[k]] = r;
+        if (k == 0 || t0 + half < total) {
+            u32x4_t rv = {r.x, r.y, r.z, r.w};
+            __builtin_nontemporal_store(rv, reinterpret_cast<u32x4_t *>(out) + tt[k]);
+        }
     }
 }
 

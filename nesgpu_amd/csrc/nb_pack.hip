@@ -36,12 +36,17 @@ __global__ __launch_bounds__(256) void pack_vec16_kernel(W *__restrict__ out, co
         const uint4 *src = reinterpret_cast<const uint4 *>(in + row * C + col0);
         int64_t left = C - col0;
         const int chunks = (int)((left < bits ? left : bits) >> 4);
+        // all loads first and none behind a branch (a chunk past the row re-reads the first one and is dropped):
+        // a load behind a branch waits for the one before it
+        const int cmax = (int)((C < bits ? C : bits) >> 4);  // the same for every thread
+        uint4 v[bits / 16];
+#pragma unroll
+        for (int c = 0; c < bits / 16; c++)
+            v[c] = c < cmax ? load_stream16(reinterpret_cast<const uint8_t *>(src + (c < chunks ? c : 0))) : make_uint4(0, 0, 0, 0);
         W w = 0;
 #pragma unroll
-        for (int c = 0; c < bits / 16; c++) {
-            if (c < chunks) w |= (W)bits16_of_bools(src[c]) << (16 * c);
-        }
-        out[t] = w;
+        for (int c = 0; c < bits / 16; c++) w |= (W)(c < chunks ? bits16_of_bools(v[c]) : 0u) << (16 * c);
+        __builtin_nontemporal_store(w, out + t);
     }
 }
 
@@ -73,7 +78,7 @@ __global__ __launch_bounds__(256) void pack_quad_kernel(uint64_t *__restrict__ o
             if ((lane & 3) == i) mine = q;
         }
         const int64_t word = (lane & 3) * 16 + (lane >> 2);
-        if (word < left) out[w0 + word] = mine;
+        if (word < left) __builtin_nontemporal_store(mine, out + w0 + word);
     }
 }
 
@@ -116,7 +121,8 @@ __global__ __launch_bounds__(256) void unpack_kernel(uint8_t *__restrict__ out, 
             const uint32_t nib = (h >> (4 * q)) & 0xFu;
             d[q] = (nib * 0x00204081u) & 0x01010101u;   // bit j -> byte j
         }
-        reinterpret_cast<uint4 *>(out)[t] = make_uint4(d[0], d[1], d[2], d[3]);
+        u32x4_t dv = {d[0], d[1], d[2], d[3]};
+        __builtin_nontemporal_store(dv, reinterpret_cast<u32x4_t *>(out) + t);  // written once, read by another kernel
     }
 }
 
