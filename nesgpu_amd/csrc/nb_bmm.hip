@@ -116,8 +116,9 @@ __global__ __launch_bounds__(BS) void bmv_quad_kernel(int32_t *__restrict__ C, c
     v += (int)dpp_mov<0x128>((uint32_t)v);               // row_ror:8
     if (L >= 32) v += __shfl_xor(v, 16);
     if (L >= 64) v += __shfl_xor(v, 32);
-    // lane q < 4 of the group now holds row 2*(q&1) + (q>>1)
-    if (live && sub < 4) C[r0 + 2 * (sub & 1) + (sub >> 1)] = v;
+    // lane q < 4 of the group now holds row 2*(q&1) + (q>>1); streaming stores: the results are read by another
+    // kernel, and ordinary stores between the row loads cost this kernel 2 % of its bandwidth (measured)
+    if (live && sub < 4) __builtin_nontemporal_store(v, C + r0 + 2 * (sub & 1) + (sub >> 1));
 }
 
 template <int L, int U>

@@ -606,11 +606,11 @@ __global__ __launch_bounds__(64 * (rw_cwaves(CPR, NT) + kRwPWaves)) void conv_mf
                 unsigned char *orow = obase + (MODE == 3 ? y >> 1 : y) * orowb;
                 if (olive[0]) {
                     if (piece && NT == 1) {
-                        *reinterpret_cast<uint16_t *>(orow + olane[0]) = (uint16_t)word;
+                        __builtin_nontemporal_store((uint16_t)(uint16_t)word, reinterpret_cast<uint16_t *>(orow + olane[0]));
                     } else if (piece) {
-                        *reinterpret_cast<uint32_t *>(orow + olane[0]) = (uint32_t)word;
+                        __builtin_nontemporal_store((uint32_t)(uint32_t)word, reinterpret_cast<uint32_t *>(orow + olane[0]));
                     } else {
-                        *reinterpret_cast<uint64_t *>(orow + olane[0]) = word;
+                        __builtin_nontemporal_store((uint64_t)word, reinterpret_cast<uint64_t *>(orow + olane[0]));
                     }
                 }
             };
