@@ -66,6 +66,15 @@ int nb_bmm_act_i64(uint8_t *C, const int64_t *A, const int64_t *B, const int32_t
                    int64_t Kw, int64_t N, nb_stream_t stream);
 int nb_bmm_act_i32(uint8_t *C, const int32_t *A, const int32_t *B, const int32_t *thresh, int64_t Z, int64_t M,
                    int64_t Kw, int64_t N, nb_stream_t stream);
+/* Matrix-vector form of a linear layer with the threshold and the pack fused: bit m of member z's output row is
+ * (2 * sum_k popcount(A[z,m,k] ^ x[z,k]) > thresh[z,m]); A [Z,M,Kw], x [Z,Kw], thresh [Z,M] int32,
+ * out [Z, ceil(M/bits)] words, LSB-first, tail bits zero.
+ *   no single counterpart in the reference: it is BinarizedLinear.forward's bmm -> compare (modules/binary.py:97-106)
+ *   followed by the next layer's pack (extensions/src/pack.cu:5-30), without the int32 and bool maps in between. */
+int nb_bmv_act_pack_i64(int64_t *out, const int64_t *A, const int64_t *x, const int32_t *thresh, int64_t Z, int64_t M,
+                        int64_t Kw, nb_stream_t stream);
+int nb_bmv_act_pack_i32(int32_t *out, const int32_t *A, const int32_t *x, const int32_t *thresh, int64_t Z, int64_t M,
+                        int64_t Kw, nb_stream_t stream);
 
 /* ---- packed im2col / conv -----------------------------------------------------------------
  * Geometry: input [D,H,W,Cw] (channels-last packed), fx taps along H, fy taps along W,

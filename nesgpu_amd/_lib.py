@@ -24,6 +24,7 @@ _SUFFIXED = {
     "nb_int8pack": [_PTR, _PTR, _I64, _I64, _PTR],
     "nb_bmm": [_PTR, _PTR, _PTR, _I64, _I64, _I64, _I64, _PTR],
     "nb_bmm_act": [_PTR, _PTR, _PTR, _PTR, _I64, _I64, _I64, _I64, _PTR],
+    "nb_bmv_act_pack": [_PTR, _PTR, _PTR, _PTR, _I64, _I64, _I64, _PTR],
     "nb_im2col": [_PTR, _PTR, _I64, _I64, _I64, _I64] + _GEOM + [_PTR],
     "nb_conv": [_PTR, _PTR, _PTR, _I64, _I64, _I64, _I64, _I64] + _GEOM + [_I32, _PTR],
     "nb_conv_popc_sums": [_PTR, _PTR, _PTR, _I64, _I64, _I64, _I64, _I64] + _GEOM + [_I32, _PTR],

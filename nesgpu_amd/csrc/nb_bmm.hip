@@ -72,11 +72,20 @@ __global__ __launch_bounds__(BS) void bmv_kernel(int32_t *__restrict__ C, const 
 // 16-byte vectors.  Needs M % 4 == 0 (the four rows share the member's input) and rows of whole 16-byte vectors.
 // U steps of the row walk are requested together (4*U loads of 16 bytes in flight per lane); needs
 // rowvecs % (U*L) == 0.
-template <int L, int U, int BS>
+// PACK: instead of the int32 sums, the bits (2*sum > thresh[row]) of the workgroup's 4*BS/L consecutive rows, packed
+// LSB-first (C is then the output bit array in 32-bit pieces; the host makes sure that a member's rows fill whole
+// words, so the flat row number is the flat bit number).
+template <int L, int U, int BS, bool PACK = false>
 __global__ __launch_bounds__(BS) void bmv_quad_kernel(int32_t *__restrict__ C, const uint4 *__restrict__ A,
                                                       const uint4 *__restrict__ X, int64_t quads, int64_t M,
-                                                      int rowvecs)
+                                                      int rowvecs, const int32_t *__restrict__ thresh = nullptr)
 {
+    constexpr int RPB = 4 * BS / L;  // rows of a workgroup
+    __shared__ uint32_t pieces[PACK ? RPB / 32 : 1];
+    if (PACK) {
+        if (threadIdx.x < RPB / 32) pieces[threadIdx.x] = 0u;
+        __syncthreads();
+    }
     const int64_t gid = ((int64_t)blockIdx.x * BS + threadIdx.x) / L;
     const int sub = threadIdx.x % L;
     const bool live = gid < quads;
@@ -118,17 +127,58 @@ __global__ __launch_bounds__(BS) void bmv_quad_kernel(int32_t *__restrict__ C, c
     if (L >= 64) v += __shfl_xor(v, 32);
     // lane q < 4 of the group now holds row 2*(q&1) + (q>>1); streaming stores: the results are read by another
     // kernel, and ordinary stores between the row loads cost this kernel 2 % of its bandwidth (measured)
-    if (live && sub < 4) __builtin_nontemporal_store(v, C + r0 + 2 * (sub & 1) + (sub >> 1));
+    if (!PACK) {
+        if (live && sub < 4) __builtin_nontemporal_store(v, C + r0 + 2 * (sub & 1) + (sub >> 1));
+    } else {
+        if (live && sub < 4) {
+            const int64_t row = r0 + 2 * (sub & 1) + (sub >> 1);
+            const int local = (int)(row - (int64_t)blockIdx.x * RPB);
+            if (2 * v > thresh[row]) atomicOr(&pieces[local >> 5], 1u << (local & 31));
+        }
+        __syncthreads();
+        const int64_t piece = (int64_t)blockIdx.x * (RPB / 32) + threadIdx.x;
+        if (threadIdx.x < RPB / 32 && piece * 32 < quads * 4) reinterpret_cast<uint32_t *>(C)[piece] = pieces[threadIdx.x];
+    }
 }
 
 template <int L, int U>
-static void launch_bmv_quad(int32_t *C, const void *A, const void *X, int64_t rows, int64_t M, int rowvecs, hipStream_t s)
+static void launch_bmv_quad(int32_t *C, const void *A, const void *X, int64_t rows, int64_t M, int rowvecs, hipStream_t s,
+                            const int32_t *thresh = nullptr)
 {
     constexpr int BS = 1024;
     const int64_t quads = rows / 4;
     const int64_t blocks = ceil_div(quads * L, BS);
-    bmv_quad_kernel<L, U, BS><<<dim3((unsigned)blocks), dim3(BS), 0, s>>>(C, static_cast<const uint4 *>(A),
-                                                                        static_cast<const uint4 *>(X), quads, M, rowvecs);
+    if (thresh)
+        bmv_quad_kernel<L, U, BS, true><<<dim3((unsigned)blocks), dim3(BS), 0, s>>>(
+            C, static_cast<const uint4 *>(A), static_cast<const uint4 *>(X), quads, M, rowvecs, thresh);
+    else
+        bmv_quad_kernel<L, U, BS><<<dim3((unsigned)blocks), dim3(BS), 0, s>>>(C, static_cast<const uint4 *>(A),
+                                                                            static_cast<const uint4 *>(X), quads, M, rowvecs);
+}
+
+// Any shape: one wave per output word, its rows one after the other (lanes stride over the row's words).
+template <typename W>
+__global__ __launch_bounds__(256) void bmv_act_pack_generic_kernel(W *__restrict__ out, const W *__restrict__ A,
+                                                                   const W *__restrict__ X,
+                                                                   const int32_t *__restrict__ thresh, int64_t words,
+                                                                   int64_t M, int Mw, int Kw)
+{
+    constexpr int bits = WordTraits<W>::bits;
+    const int lane = threadIdx.x & 63;
+    const int64_t wd = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (wd >= words) return;  // wave-uniform, no barrier below
+    const int64_t z = wd / Mw;
+    const int64_t m0 = (wd - z * Mw) * bits;
+    W word = 0;
+    for (int i = 0; i < bits && m0 + i < M; i++) {
+        const W *a = A + (z * M + m0 + i) * Kw, *x = X + z * Kw;
+        int acc = 0;
+        for (int k = lane; k < Kw; k += 64) acc += popc_xor(a[k], x[k]);
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off);
+        if (2 * acc > thresh[z * M + m0 + i]) word |= (W)1 << i;
+    }
+    if (lane == 0) out[wd] = word;
 }
 
 template <typename W, int KC, int NT, bool SINGLE, bool EXACT, class Epi>
@@ -251,9 +301,66 @@ int bmm_act_impl(uint8_t *C, const W *A, const W *B, const int32_t *thresh, int6
     return check_launch(who);
 }
 
+template <typename W>
+int bmv_act_pack_impl(W *out, const W *A, const W *X, const int32_t *thresh, int64_t Z, int64_t M, int64_t Kw,
+                      nb_stream_t stream, const char *who)
+{
+    constexpr int bits = WordTraits<W>::bits;
+    NB_REQUIRE(Z >= 0 && M >= 0 && Kw >= 0, "%s: negative shape Z=%lld M=%lld Kw=%lld", who, (long long)Z, (long long)M,
+               (long long)Kw);
+    if (Z * M == 0) return NB_OK;
+    NB_REQUIRE_PTR(out);
+    NB_REQUIRE_PTR(thresh);
+    NB_REQUIRE_ALIGNED(out, sizeof(W));
+    NB_REQUIRE_ALIGNED(thresh, 4);
+    if (Kw > 0) {
+        NB_REQUIRE_PTR(A);
+        NB_REQUIRE_PTR(X);
+        NB_REQUIRE_ALIGNED(A, sizeof(W));
+        NB_REQUIRE_ALIGNED(X, sizeof(W));
+    }
+    NB_REQUIRE(Kw <= (1 << 24) && Z * M < (1LL << 40), "%s: Kw=%lld or Z*M=%lld too large", who, (long long)Kw,
+               (long long)(Z * M));
+    hipStream_t s = as_stream(stream);
+    const int64_t rows = Z * M;
+    const int64_t rowbytes = Kw * (int64_t)sizeof(W);
+    const int64_t Mw = ceil_div(M, bits);
+    NB_REQUIRE(ceil_div(Z * Mw, 4) <= kMaxGridX && ceil_div(ceil_div(rows, 4) * 64, 256) <= kMaxGridX,
+               "%s: %lld rows exceed one launch", who, (long long)rows);
+    if (rowbytes % 16 == 0 && rowbytes >= 256 && M % bits == 0 && aligned(A, 16) && aligned(X, 16)) {
+        const int rowvecs = (int)(rowbytes / 16);
+        int32_t *C = reinterpret_cast<int32_t *>(out);
+        if (rowvecs % 256 == 0) launch_bmv_quad<64, 4>(C, A, X, rows, M, rowvecs, s, thresh);
+        else if (rowvecs % 128 == 0) launch_bmv_quad<32, 4>(C, A, X, rows, M, rowvecs, s, thresh);
+        else if (rowvecs % 64 == 0) launch_bmv_quad<16, 4>(C, A, X, rows, M, rowvecs, s, thresh);
+        else if (rowvecs % 32 == 0) launch_bmv_quad<16, 2>(C, A, X, rows, M, rowvecs, s, thresh);
+        else if (rowvecs >= 64) launch_bmv_quad<64, 1>(C, A, X, rows, M, rowvecs, s, thresh);
+        else if (rowvecs >= 32) launch_bmv_quad<32, 1>(C, A, X, rows, M, rowvecs, s, thresh);
+        else launch_bmv_quad<16, 1>(C, A, X, rows, M, rowvecs, s, thresh);
+    } else {
+        bmv_act_pack_generic_kernel<W><<<dim3((unsigned)ceil_div(Z * Mw, 4)), dim3(256), 0, s>>>(
+            out, A, X, thresh, Z * Mw, M, (int)Mw, (int)Kw);
+    }
+    return check_launch(who);
+}
+
 }  // namespace nb
 
 extern "C" {
+int nb_bmv_act_pack_i64(int64_t *out, const int64_t *A, const int64_t *x, const int32_t *thresh, int64_t Z, int64_t M,
+                        int64_t Kw, nb_stream_t s)
+{
+    return nb::bmv_act_pack_impl<uint64_t>(reinterpret_cast<uint64_t *>(out), reinterpret_cast<const uint64_t *>(A),
+                                           reinterpret_cast<const uint64_t *>(x), thresh, Z, M, Kw, s,
+                                           "nb_bmv_act_pack_i64");
+}
+int nb_bmv_act_pack_i32(int32_t *out, const int32_t *A, const int32_t *x, const int32_t *thresh, int64_t Z, int64_t M,
+                        int64_t Kw, nb_stream_t s)
+{
+    return nb::bmv_act_pack_impl<uint32_t>(reinterpret_cast<uint32_t *>(out), reinterpret_cast<const uint32_t *>(A),
+                                           reinterpret_cast<const uint32_t *>(x), thresh, Z, M, Kw, s,
+                                           "nb_bmv_act_pack_i32");
+}
 int nb_bmm_i64(int32_t *C, const int64_t *A, const int64_t *B, int64_t Z, int64_t M, int64_t Kw, int64_t N,
                nb_stream_t s)
 {

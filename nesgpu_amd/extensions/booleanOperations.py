@@ -152,6 +152,29 @@ def bmm_act(A, B, threshold):
     return C
 
 
+def bmv_act_pack(A, x, threshold):
+    """One input row per member, as the linear layers have it: A [Z,M,Kw] packed weights, x [Z,Kw] (or [Z,Kw,1])
+    packed inputs, threshold [Z,M] int32 -> packed bits (2*popc(A[z,m] ^ x[z]) > threshold[z,m]) as [Z, ceil(M/bits)]
+    words.  Not in the reference: it is ``pack(2 * bmm(A, x) > threshold)`` (the compare of
+    modules/binary.py:97-106 and the next layer's pack) in one kernel, without the int32 and bool maps."""
+    _check(A, "A")
+    _check(x, "x")
+    _check(threshold, "threshold")
+    _same_device(A, x)
+    _same_device(A, threshold)
+    assert len(A.shape) == 3
+    assert A.dtype == x.dtype
+    Z, M, Kw = A.shape
+    assert x.numel() == Z * Kw and x.size(0) == Z                # "Batch dim doesn't match", booleanOperations.cpp:46
+    assert tuple(threshold.shape) == (Z, M) and threshold.dtype == torch.int32
+    suf, bits = _suffix(A.dtype)
+    out = torch.empty((Z, ceil_div(M, bits)), dtype=A.dtype, device=A.device)
+    with _on(A):
+        _lib.call("nb_bmv_act_pack" + suf, out.data_ptr(), A.data_ptr(), x.data_ptr(), threshold.data_ptr(), Z, M, Kw,
+                  _stream(A))
+    return out
+
+
 def conv_engine(engine=None):
     """Query / set the process-wide conv engine: 0 = automatic (matrix cores for populations of 128 or more, else
     XOR-popcount), 1 = XOR-popcount kernels only, 2 = matrix cores wherever a kernel covers the shape (FP4 codes for

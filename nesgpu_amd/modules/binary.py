@@ -115,10 +115,13 @@ class BinarizedLinear(Binarized):
     row per member (a batched matrix-VECTOR product, modules/binary.py:97)."""
 
     def __init__(self, in_features, out_features, directions, threshold=True, batch_norm=False, dtype=torch.int64,
-                 device="cuda"):
+                 device="cuda", pack_output=False):
         Binarized.__init__(self, in_features, out_features, directions, threshold, dtype, device)
         self.in_features = in_features
         self.out_features = out_features
+        if pack_output and (not threshold or batch_norm):
+            raise NotImplementedError("packed output needs threshold=True and batch_norm=False")
+        self.pack_output = pack_output    # not in the reference: return the thresholded row packed, from one kernel
         self.weight = Parameter(torch.zeros(out_features, in_features, dtype=torch.float16, device=device))
         if threshold:
             self.bias = Parameter(torch.zeros(out_features, dtype=torch.float16, device=device))
@@ -129,6 +132,10 @@ class BinarizedLinear(Binarized):
         if not self.perturbed_flag:
             raise NotImplementedError                     # modules/binary.py:108-109: no inference path
         packed_input = booleanOperations.pack(input, self.dtype) if input.dtype == torch.bool else input
+        if self.pack_output:
+            # activation > t  <=>  2*popc - K > floor(t)  <=>  2*popc > floor(t) + K  (activation is an integer)
+            thresh = torch.floor((self.bias + self.bias_noise).to(torch.float32)).to(torch.int32) + self.in_features
+            return booleanOperations.bmv_act_pack(self.weight_noise, packed_input.view(self.directions, -1), thresh)
         popc = booleanOperations.bmm(self.weight_noise, packed_input.view(self.directions, -1, 1))
         activation = 2 * popc.squeeze(dim=2) - self.in_features
         if self.threshold:

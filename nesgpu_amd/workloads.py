@@ -185,6 +185,7 @@ def cifar_net(D=4096, T=T_P01, seed=0, dtype=torch.int64, device="cuda", classes
     b5 = ops.pack(_bits(g, (classes, 1024)).to(device), dtype)
     W5 = ops.flip_philox(b5, 1024, D, T, seed, subsequence=subseq + 1)
     macs += D * 1024 * 8192 + D * classes * 1024
+    thr4 = torch.full((D, 1024), 8192, dtype=torch.int32, device=device)
 
     def step():
         a = x
@@ -192,8 +193,7 @@ def cifar_net(D=4096, T=T_P01, seed=0, dtype=torch.int64, device="cuda", classes
             _, thr, f, kw = layers[i]
             a = ops.conv_act_pack(a, f, thr, 3, 3, 1, 1, 1, 1, pool=pool, **kw)
         a = a.view(D, -1, 1)                                                                    # [D,128,1]
-        p4 = ops.bmm(W4, a).squeeze(2)                                                          # [D,1024]
-        a = ops.pack(2 * p4 > 8192, dtype).view(D, -1, 1)                                       # [D,16,1]
+        a = ops.bmv_act_pack(W4, a, thr4).view(D, -1, 1)                  # pack(2 * bmm(W4, a) > 8192): [D,16,1]
         return ops.bmm(W5, a).squeeze(2)                                                        # [D,classes] popc
 
     w = Workload(

@@ -75,6 +75,13 @@ def test_linear_forward(binary, oracle, dtype, in_f, out_f):
         assert torch.equal(out, act_t > thresh)
         # packed input is accepted as is (modules/binary.py:95)
         assert torch.equal(layer(dev(oracle.pack(xb, nd))), out)
+        if not batch_norm:
+            # pack_output=True: the same bits, packed, from the fused kernel
+            layer.pack_output = True
+            packed = layer(dev(xb))
+            layer.pack_output = False
+            assert packed.dtype == dtype
+            np.testing.assert_array_equal(packed.cpu().numpy(), oracle.pack(out.cpu().numpy(), nd))
 
 
 @pytest.mark.parametrize("dtype", [torch.int64, torch.int32])

@@ -202,6 +202,38 @@ def test_bmm_random_shapes_vs_oracle(ops, oracle, dtype):
         np.testing.assert_array_equal(host(ops.bmm(dev(A), dev(B))), oracle.bmm(A, B))
 
 
+@pytest.mark.parametrize("dtype", [torch.int64, torch.int32])
+def test_bmv_act_pack_random_shapes_vs_oracle(ops, oracle, dtype):
+    """The fused matrix-vector -> threshold -> pack op against pack(2 * bmm > threshold) of the oracle: rows of every
+    length class of the four-row kernel (members of whole words, several workgroups, ragged last workgroup) and the
+    general kernel (ragged members, short rows), thresholds around the sums plus always / never."""
+    nd = NDT[dtype]
+    bits = np.dtype(nd).itemsize * 8
+    g = rng(777)
+    vec = 16 // np.dtype(nd).itemsize                      # words per 16 bytes
+    for ci in range(48):
+        Z = int(g.integers(1, 6))
+        if ci % 2 == 0:                                    # shapes the four-row kernel takes
+            M = bits * int(g.integers(1, 9))
+            Kw = vec * int(g.choice([16, 17, 32, 48, 64, 96, 128, 256, 272]))
+        else:
+            M = int(g.integers(1, 200))
+            Kw = int(g.choice([0, 1, 3, 16, 31, 64, 130]))
+        print("case", ci, (Z, M, Kw), flush=True)
+        A = rand_words(g, (Z, M, Kw), nd)
+        x = rand_words(g, (Z, Kw, 1), nd)
+        sums = oracle.bmm(A, x)[:, :, 0]
+        K = Kw * bits
+        thr = (2 * sums + g.integers(-3, 4, size=sums.shape)).astype(np.int32)
+        thr[0, 0] = -1
+        thr[-1, -1] = 2 * K + 1
+        want = oracle.pack(2 * sums.astype(np.int64) > thr, nd)
+        got = ops.bmv_act_pack(dev(A), dev(x), dev(thr))
+        assert tuple(got.shape) == want.shape
+        np.testing.assert_array_equal(host(got), want, err_msg="case %d: Z=%d M=%d Kw=%d" % (ci, Z, M, Kw))
+        np.testing.assert_array_equal(host(ops.bmv_act_pack(dev(A), dev(x[:, :, 0]), dev(thr))), want)
+
+
 GENERAL_SHAPES = [(2, 300, 9, 64), (3, 65, 4, 16), (2, 257, 18, 5), (2, 40, 40, 33), (1, 1, 1, 2), (2, 513, 3, 128),
                   (3, 7, 17, 17), (2, 100, 0, 4)]
 
