@@ -365,8 +365,9 @@ def main():
     line["generator_mode"] = {"workload": wg.name, "ms_per_step": round(pw * 1e3, 4),
                               "binary_TOPS": round(2 * wg.bit_macs / pw / 1e12, 3),
                               "random_words_per_s": float("%.4g" % (wg.bit_macs / pe)),
-                              "note": "same output as the headline workload; about 25 vector ALU operations per "
-                                      "generated word, so the vector ALUs are the limit, not HBM"}
+                              "note": "same output as the headline workload; about 18 vector ALU operations per "
+                                      "generated word (each 32x32->64 product of a Philox round is one v_mad_u64_u32), "
+                                      "so the vector ALUs are the limit, not HBM"}
     del wg
     if others:
         line["other_configs"] = others
