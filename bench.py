@@ -365,8 +365,8 @@ def main():
     line["generator_mode"] = {"workload": wg.name, "ms_per_step": round(pw * 1e3, 4),
                               "binary_TOPS": round(2 * wg.bit_macs / pw / 1e12, 3),
                               "random_words_per_s": float("%.4g" % (wg.bit_macs / pe)),
-                              "note": "same output as the headline workload; about 18 vector ALU operations per "
-                                      "generated word (each 32x32->64 product of a Philox round is one v_mad_u64_u32), "
+                              "note": "same output as the headline workload; about 14 vector ALU operations per "
+                                      "generated word (a Philox round is two v_mad_u64_u32 and two v_bitop3_b32), "
                                       "so the vector ALUs are the limit, not HBM"}
     del wg
     if others:

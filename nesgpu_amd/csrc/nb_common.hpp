@@ -84,12 +84,13 @@ __device__ __forceinline__ uint4 philox4x32_10(uint4 c, uint2 k)
 {
 #pragma unroll
     for (int r = 0; r < 10; r++) {
-        // full 64-bit products: one v_mad_u64_u32 each instead of a v_mul_lo / v_mul_hi pair (a fifth fewer
-        // vector instructions per generated word, and the generator is bound by their number)
+        // full 64-bit products: one v_mad_u64_u32 each instead of a v_mul_lo / v_mul_hi pair (the generator is bound
+        // by the number of vector instructions per word)
         const uint64_t p0 = (uint64_t)0xD2511F53u * c.x, p1 = (uint64_t)0xCD9E8D57u * c.z;
         const uint32_t lo0 = (uint32_t)p0, hi0 = (uint32_t)(p0 >> 32);
         const uint32_t lo1 = (uint32_t)p1, hi1 = (uint32_t)(p1 >> 32);
-        c = make_uint4(hi1 ^ c.y ^ k.x, lo1, hi0 ^ c.w ^ k.y, lo0);
+        // three-input XOR in one instruction (v_bitop3_b32, truth table 0x96)
+        c = make_uint4(__builtin_amdgcn_bitop3_b32(hi1, c.y, k.x, 0x96), lo1, __builtin_amdgcn_bitop3_b32(hi0, c.w, k.y, 0x96), lo0);
         k.x += 0x9E3779B9u;
         k.y += 0xBB67AE85u;
     }
