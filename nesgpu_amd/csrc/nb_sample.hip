@@ -33,10 +33,19 @@ __device__ __forceinline__ uint4 thr4(const uint32_t *__restrict__ thresh, uint3
     return thresh ? *reinterpret_cast<const uint4 *>(thresh + idx) : make_uint4(ts, ts, ts, ts);
 }
 
+// bit j of the result = (word j < threshold j).  Each compare's carry is shifted in by an add-with-carry of the
+// running value to itself: two vector instructions per word instead of compare, select and shift-or.
 __device__ __forceinline__ uint32_t nibble_lt(uint4 w, uint4 t)
 {
-    return (uint32_t)(w.x < t.x) | ((uint32_t)(w.y < t.y) << 1) | ((uint32_t)(w.z < t.z) << 2) |
-           ((uint32_t)(w.w < t.w) << 3);
+    uint32_t r;
+    asm("v_cmp_lt_u32 vcc, %1, %5\n\tv_addc_co_u32 %0, vcc, 0, 0, vcc\n\t"
+        "v_cmp_lt_u32 vcc, %2, %6\n\tv_addc_co_u32 %0, vcc, %0, %0, vcc\n\t"
+        "v_cmp_lt_u32 vcc, %3, %7\n\tv_addc_co_u32 %0, vcc, %0, %0, vcc\n\t"
+        "v_cmp_lt_u32 vcc, %4, %8\n\tv_addc_co_u32 %0, vcc, %0, %0, vcc"
+        : "=&v"(r)
+        : "v"(w.w), "v"(w.z), "v"(w.y), "v"(w.x), "v"(t.w), "v"(t.z), "v"(t.y), "v"(t.x)
+        : "vcc");
+    return r;
 }
 
 // ---- materialised sampler, wide path: C % bits == 0 and 16-byte aligned streams ------------------
