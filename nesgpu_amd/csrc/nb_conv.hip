@@ -7,26 +7,26 @@
 namespace nb {
 
 // ---- im2col (kept for API parity; conv itself never materialises the columns) ----------------
-// One thread per output word; consecutive threads write consecutive words.
+// One thread per output word; consecutive threads write consecutive words.  Members are walked by blockIdx.y so
+// that the index arithmetic inside a member stays in 32 bits (the host checks that a member's columns fit).
 template <typename W>
-__global__ __launch_bounds__(256) void im2col_kernel(W *__restrict__ out, const W *__restrict__ in, int64_t total,
-                                                     ConvGeom g)
+__global__ __launch_bounds__(256) void im2col_kernel(W *__restrict__ out, const W *__restrict__ in, int64_t D,
+                                                     uint32_t per_member, ConvGeom g)
 {
-    NB_FLAT_LOOP(t, total)
-    {
-        if (t >= total) continue;
-        const int K = g.fx * g.fy * g.Cw;
-        const int64_t rowi = t / K;  // (b, loc)
-        const int e = (int)(t - rowi * K);
-        const int hw = g.h * g.w;
-        const int64_t b = rowi / hw;
-        const int loc = (int)(rowi - b * hw);
-        const int xo = loc / g.w, yo = loc - xo * g.w;
-        const int tap = e / g.Cw, c = e - tap * g.Cw;
-        const int i = tap / g.fy, j = tap - i * g.fy;
-        const int xi = i + xo * g.sx - g.px, yi = j + yo * g.sy - g.py;
-        const bool ok = xi >= 0 && xi < g.H && yi >= 0 && yi < g.Wd;
-        out[t] = ok ? in[((b * g.H + xi) * g.Wd + yi) * g.Cw + c] : (W)0;
+    const uint32_t idx = blockIdx.x * 256u + threadIdx.x;
+    if (idx >= per_member) return;
+    const uint32_t K = (uint32_t)(g.fx * g.fy * g.Cw);
+    const uint32_t loc = idx / K, e = idx - loc * K;
+    const uint32_t xo = loc / (uint32_t)g.w, yo = loc - xo * (uint32_t)g.w;
+    const uint32_t tap = e / (uint32_t)g.Cw, c = e - tap * (uint32_t)g.Cw;
+    const uint32_t i = tap / (uint32_t)g.fy, j = tap - i * (uint32_t)g.fy;
+    const int xi = (int)(i + xo * g.sx) - g.px, yi = (int)(j + yo * g.sy) - g.py;
+    const bool ok = xi >= 0 && xi < g.H && yi >= 0 && yi < g.Wd;
+    const int64_t img = (int64_t)g.H * g.Wd * g.Cw;
+    const int64_t off = ok ? ((int64_t)xi * g.Wd + yi) * g.Cw + c : 0;
+    for (int64_t b = blockIdx.y; b < D; b += gridDim.y) {
+        const W v = in[b * img + off];  // an element outside re-reads the member's first word and is dropped
+        __builtin_nontemporal_store(ok ? v : (W)0, out + b * (int64_t)per_member + idx);
     }
 }
 
@@ -137,8 +137,11 @@ int im2col_impl(W *out, const W *in, int64_t D, int64_t H, int64_t Wd, int64_t C
     NB_REQUIRE_PTR(in);
     NB_REQUIRE_ALIGNED(out, sizeof(W));
     NB_REQUIRE_ALIGNED(in, sizeof(W));
-    const unsigned blocks = grid_for(total);
-    im2col_kernel<W><<<dim3(blocks), dim3(256), 0, as_stream(stream)>>>(out, in, total, g);
+    const int64_t per_member = total / D;
+    NB_REQUIRE(per_member < (1LL << 31) && H * Wd * Cw > 0, "%s: a member's columns exceed 2^31 words or its image is empty",
+               who);
+    const dim3 grid((unsigned)ceil_div(per_member, 256), (unsigned)(D < 65535 ? D : 65535));
+    im2col_kernel<W><<<grid, dim3(256), 0, as_stream(stream)>>>(out, in, D, (uint32_t)per_member, g);
     return check_launch(who);
 }
 
