@@ -126,6 +126,12 @@ def test_config5_cifar_net(wk, ops, oracle):
     assert tuple(out.shape) == (D, 10) and out.dtype == torch.int32
     assert torch.equal(w.step(), out)                                      # deterministic
     t = w.tensors
+    # the fused linear-layer kernel against the unfused composition, every member, thresholds around the sums
+    a4 = torch.randint(-2 ** 62, 2 ** 62, (D, 128, 1), dtype=torch.int64, device="cuda")
+    sums = ops.bmm(t["W4"], a4).squeeze(2)
+    thr4 = (2 * sums + torch.randint(-2, 3, sums.shape, device="cuda")).to(torch.int32)
+    assert torch.equal(ops.bmv_act_pack(t["W4"], a4, thr4), ops.pack(2 * sums > thr4, torch.int64))
+    del a4, sums, thr4
     for m in (0, 2047, 4095):
         a = t["x"][m:m + 1].cpu().numpy()                                  # [1,32,32,1]
         for name, C, O, pool in (("f1", 3, 64, False), ("f2", 64, 64, True), ("f3", 64, 128, True)):
