@@ -132,6 +132,18 @@ def test_config5_cifar_net(wk, ops, oracle):
     thr4 = (2 * sums + torch.randint(-2, 3, sums.shape, device="cuda")).to(torch.int32)
     assert torch.equal(ops.bmv_act_pack(t["W4"], a4, thr4), ops.pack(2 * sums > thr4, torch.int64))
     del a4, sums, thr4
+    # the first layer on all members: window-per-register kernel (automatic choice) == int8 matrix-core kernel
+    thr1 = torch.full((D, 64), 27, dtype=torch.int32, device="cuda")
+    prev = ops.conv_engine(0)
+    try:
+        l1 = ops.conv_act_pack(t["x"], t["f1"], thr1, 3, 3, 1, 1, 1, 1, in_bits=3)
+        assert ops.conv_last_engine() == 1
+        ops.conv_engine(3)
+        assert torch.equal(ops.conv_act_pack(t["x"], t["f1"], thr1, 3, 3, 1, 1, 1, 1, in_bits=3), l1)
+        assert ops.conv_last_engine() == 2
+    finally:
+        ops.conv_engine(prev)
+    del l1, thr1
     for m in (0, 2047, 4095):
         a = t["x"][m:m + 1].cpu().numpy()                                  # [1,32,32,1]
         for name, C, O, pool in (("f1", 3, 64, False), ("f2", 64, 64, True), ("f3", 64, 128, True)):
