@@ -5,7 +5,10 @@
  *
  * Conventions (all entry points)
  *   - every pointer is a DEVICE pointer into dense row-major memory owned by the caller; the
- *     library allocates nothing and keeps no state between calls (re-entrant);
+ *     library allocates nothing and keeps no per-call state, so calls from several threads do not
+ *     interfere.  The only process-wide state is the conv engine selector (nb_conv_engine, an atomic
+ *     that every conv call reads once; all engines give identical results) and a per-device cache of
+ *     kernel attributes;
  *   - `stream` is a hipStream_t passed as void* (NULL = the null stream); launches are
  *     asynchronous on it and the call never synchronises;
  *   - packed words are LSB-first: bit i of word y of a row is element y*bits+i

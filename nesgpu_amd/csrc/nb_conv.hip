@@ -1,5 +1,6 @@
 // Packed im2col, implicit-im2col binary conv (int32 / bool / packed / packed+pooled outputs) and
 // the packed-bit max-pool.
+#include <atomic>
 #include <cstdlib>
 
 #include "nb_conv_common.hpp"
@@ -187,22 +188,24 @@ int max_pool_impl(W *out, const W *in, int64_t B, int64_t H, int64_t Wd, int64_t
 // a kernel covers the shape (FP4 codes where that flavour exists, else +-1 bytes), 3 = as 2 but +-1 bytes only.
 // Initialised from the environment variable NESBIN_CONV_ENGINE ("valu" -> 1, "mfma" -> 2, "int8" -> 3);
 // nb_conv_engine() changes it.
-static int g_conv_engine = -1;
-static int conv_engine()
+// The one piece of process-wide state of the library: an atomic, read once per conv call.
+static int conv_engine_from_env()
 {
-    if (g_conv_engine < 0) {
-        const char *v = getenv("NESBIN_CONV_ENGINE");
-        g_conv_engine = (v && v[0] == 'v') ? 1 : (v && v[0] == 'm') ? 2 : (v && v[0] == 'i') ? 3 : 0;
-    }
-    return g_conv_engine;
+    const char *v = getenv("NESBIN_CONV_ENGINE");
+    return (v && v[0] == 'v') ? 1 : (v && v[0] == 'm') ? 2 : (v && v[0] == 'i') ? 3 : 0;
 }
+static std::atomic<int> &conv_engine_cell()
+{
+    static std::atomic<int> cell{conv_engine_from_env()};  // initialised once, thread-safe (function-local static)
+    return cell;
+}
+static int conv_engine() { return conv_engine_cell().load(std::memory_order_relaxed); }
 // engine of this thread's latest conv launch: 1 XOR-popcount, 2 matrix cores on +-1 bytes, 4 matrix cores on FP4 codes
 static thread_local int t_last_engine = 0;
 int set_conv_engine(int e)
 {
-    const int prev = conv_engine();
-    if (e >= 0 && e <= 3) g_conv_engine = e;
-    return prev;
+    if (e >= 0 && e <= 3) return conv_engine_cell().exchange(e, std::memory_order_relaxed);
+    return conv_engine();
 }
 
 __global__ __launch_bounds__(256) void zero_i32_kernel(int32_t *__restrict__ out, int64_t total)

@@ -39,6 +39,7 @@
 //   CB = 32: chunk q holds tap columns 2q and 2q+1, 32 positions each;
 //   CB >= 64: one chunk per (tap column, 64-position channel word).
 // Chunks of tap columns past the filter width multiply by zero bytes.
+#include <atomic>
 #include <type_traits>
 
 #include "nb_conv_common.hpp"
@@ -736,16 +737,17 @@ __global__ __launch_bounds__(64 * (rw_cwaves(CPR, NT) + kRwPWaves)) void conv_mf
 static inline int rw_round_up(int a, int b) { return (a + b - 1) / b * b; }
 
 // Registers of a kernel instantiation and the CU count of the current device (for the workgroups-per-CU estimate).
+// Written once per device: regs first, then cus with release order; a reader that sees cus != 0 sees regs too.
 struct RwFit {
-    int cus, regs;
+    std::atomic<int> cus{0}, regs{0};
 };
 template <int CPR, int NT, int MODE, int Q>
 static bool rw_launch_one(const RwConv &p, int64_t D, size_t lds_bytes, hipStream_t s)
 {
-    // Per device (the attribute belongs to the device's copy of the kernel).  Benign race: every thread computes
-    // the same values.
+    // Per device (the attribute belongs to the device's copy of the kernel).  Threads that arrive together all
+    // compute the same values and publish them through the atomics.
     constexpr int kMaxDevices = 16;
-    static RwFit fits[kMaxDevices] = {};
+    static RwFit fits[kMaxDevices];
     auto *kfn = conv_mfma_kernel<CPR, NT, MODE, Q>;
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
@@ -753,7 +755,8 @@ static bool rw_launch_one(const RwConv &p, int64_t D, size_t lds_bytes, hipStrea
         return false;
     }
     RwFit &fit = fits[dev];
-    if (fit.cus == 0) {
+    int fit_cus = fit.cus.load(std::memory_order_acquire);
+    if (fit_cus == 0) {
         hipFuncAttributes fa;
         int cus = 0;
         if (hipFuncSetAttribute(reinterpret_cast<const void *>(kfn), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -763,15 +766,17 @@ static bool rw_launch_one(const RwConv &p, int64_t D, size_t lds_bytes, hipStrea
             (void)hipGetLastError();
             return false;
         }
-        fit.regs = fa.numRegs > 0 ? fa.numRegs : 256;
-        fit.cus = cus;
+        fit.regs.store(fa.numRegs > 0 ? fa.numRegs : 256, std::memory_order_relaxed);
+        fit.cus.store(cus, std::memory_order_release);
+        fit_cus = cus;
     }
+    const int fit_regs = fit.regs.load(std::memory_order_relaxed);
     // 512 registers per lane and SIMD, three or four waves of a workgroup per SIMD; 160 KB of LDS per CU
-    int per_cu = 512 / ((fit.regs + 7) / 8 * 8) / ((rw_cwaves(CPR, NT) + kRwPWaves) / 4);
+    int per_cu = 512 / ((fit_regs + 7) / 8 * 8) / ((rw_cwaves(CPR, NT) + kRwPWaves) / 4);
     const int by_lds = (int)(160 * 1024 / (lds_bytes + kRwLutBytes + kRwTabBytes));
     per_cu = per_cu < by_lds ? per_cu : by_lds;
     per_cu = per_cu < 1 ? 1 : (per_cu > 4 ? 4 : per_cu);
-    const int64_t wgs = D < (int64_t)fit.cus * per_cu ? D : (int64_t)fit.cus * per_cu;
+    const int64_t wgs = D < (int64_t)fit_cus * per_cu ? D : (int64_t)fit_cus * per_cu;
     kfn<<<dim3((unsigned)wgs), dim3(64 * (rw_cwaves(CPR, NT) + kRwPWaves)), lds_bytes, s>>>(p);
     return true;
 }

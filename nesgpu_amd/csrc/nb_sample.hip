@@ -346,7 +346,8 @@ int sample_impl(W *out, const W *base, const uint32_t *thresh, uint32_t ts, Src 
     NB_REQUIRE_ALIGNED(out, sizeof(W));
     hipStream_t s = as_stream(stream);
     const int64_t Rw = ceil_div(C, bits);
-    if (C % bits == 0 && src_vec_ok && (!thresh || aligned(thresh, 16)) && R * (C / 4) < (1LL << 31)) {
+    if (C % bits == 0 && src_vec_ok && (!thresh || aligned(thresh, 16)) &&
+        R * (C / 4) < (1LL << 30)) {  // the kernel forms 32-bit word offsets 4 * (R * C / 4) inside a member's plane
         constexpr int U = 8, BS = 1024;
         const uint32_t rc4 = (uint32_t)(R * (C / 4));
         const uint32_t plane_tiles = (uint32_t)ceil_div(rc4, BS);

@@ -73,6 +73,7 @@ int weighted_sum_impl(uint16_t *ret, const W *in, const uint16_t *w, int64_t n, 
         NB_REQUIRE_ALIGNED(w, 2);
     }
     NB_REQUIRE(zbits <= (1 << 30) && Rw <= (1 << 30), "%s: row too long", who);
+    NB_REQUIRE(zbits <= Rw * (int64_t)WordTraits<W>::bits, "%s: zbits exceeds the Rw words of a row", who);
     const int64_t ncol = ceil_div(zbits, 64);
     const int64_t blocks = ceil_div(R * ncol, 4);
     NB_REQUIRE(blocks <= kMaxGridX, "%s: output exceeds one launch", who);

@@ -9,7 +9,8 @@ defects of the reference snapshot are not reproduced: construction order (``Pert
 (modules/binary.py:36 vs modules/base.py:47).
 
 Additions, all opt-in: ``set_noise(words=...)`` samples from caller-supplied uint32 words (bit-exact
-parity mode), and ``BinarizedConv2d(pack_output=True[, pool_output=True])`` returns the thresholded map
+parity mode), ``set_noise(bias_generator=...)`` draws the bias noise from a given torch.Generator instead of the
+global one, and ``BinarizedConv2d(pack_output=True[, pool_output=True])`` returns the thresholded map
 already packed along channels (and 2x2 OR-pooled) from one fused kernel instead of a bool map.
 """
 import torch
@@ -76,9 +77,11 @@ class Binarized(Perturbed, nn.Module):
             norm_weight = self.weight / (self.weight.abs().mean() + 1e-5) * 5
             return torch.sigmoid(norm_weight.float()).half()
 
-    def set_noise(self, noise_scale=None, words=None):
+    def set_noise(self, noise_scale=None, words=None, bias_generator=None):
         """modules/binary.py:54-64.  ``words`` (uint32 [directions, rows, in_degree]) replaces the
-        generator: bit = words < floor(P * 2**32)."""
+        generator: bit = words < floor(P * 2**32).  The bias noise comes from torch's global generator of the
+        weight's device, as in the reference (:63-64): every call draws fresh values and no two layers share them;
+        ``bias_generator`` (a torch.Generator on that device, not in the reference) makes it reproducible."""
         if self.seed is None:
             self.set_seed()
         if noise_scale is not None:
@@ -89,13 +92,8 @@ class Binarized(Perturbed, nn.Module):
         else:
             self.weight_noise = booleanOperations.sample_bits_from_words(
                 booleanOperations.thresholds_from_p(P), words, self.dtype)
-        if self.threshold:
-            gen = torch.Generator(device=self.weight.device)
-            gen.manual_seed(int(self.seed))
-            self.bias_noise = (torch.rand(size=(self.directions, self.out_degree), dtype=torch.float16,
-                                          device=self.weight.device, generator=gen) - .5) * 6
-        else:
-            self.bias_noise = None
+        self.bias_noise = (torch.rand(size=(self.directions, self.out_degree), dtype=torch.float16,
+                                      device=self.weight.device, generator=bias_generator) - .5) * 6
 
     def update(self, weights, l1=0, l2=1e-3):
         """modules/binary.py:67-77."""
@@ -177,9 +175,9 @@ class BinarizedConv2d(Binarized):
     def reset_parameters(self):
         Binarized.reset_parameters(self)
 
-    def set_noise(self, noise_scale=None, words=None):
+    def set_noise(self, noise_scale=None, words=None, bias_generator=None):
         """modules/binary.py:134-137: [D, out*kx*ky, Cw] -> [D, kx*ky*Cw, out], out contiguous."""
-        Binarized.set_noise(self, noise_scale, words)
+        Binarized.set_noise(self, noise_scale, words, bias_generator)
         r = self.weight_noise.view(self.directions, self.out_channels, *self.kernel_size, -1)
         self.weight_noise_reshaped = r.permute([0, 2, 3, 4, 1]).reshape(self.directions, -1,
                                                                        self.out_channels).contiguous()

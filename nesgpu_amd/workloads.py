@@ -170,12 +170,14 @@ def cifar_net(D=4096, T=T_P01, seed=0, dtype=torch.int64, device="cuda", classes
     x_bits = (z > z.mean(dim=(0, 2, 3), keepdim=True)).permute(0, 2, 3, 1).contiguous()      # [D,32,32,3]
     x = ops.pack(x_bits.view(-1, 3).to(device), dtype).view(D, 32, 32, 1)
     layers = []
+    bases = []
     macs = 0
     subseq = 10
     for (C, O, S) in ((3, 64, 32), (64, 64, 32), (64, 128, 16)):
         base_bits = _bits(g, (O * 9, C))
         base, Wn, filt = _conv_filters(base_bits, D, O, 3, C, T, seed, subseq, dtype, device)
         del Wn
+        bases.append(base)
         thr = torch.full((D, O), 9 * C, dtype=torch.int32, device=device)
         layers.append((filt, thr) + _tap(filt, 3, C))
         macs += D * S * S * O * 9 * C
@@ -200,8 +202,9 @@ def cifar_net(D=4096, T=T_P01, seed=0, dtype=torch.int64, device="cuda", classes
         name="CIFAR-shaped binary net D=%d (conv3-64, conv64-64, pool, conv64-128, pool, fc8192-1024, fc1024-%d)"
              % (D, classes),
         population=D, bit_macs=macs, algo_bytes=W4.numel() * 8, bound="valu", step=step,
-        tensors=dict(x=x, f1=layers[0][0], f2=layers[1][0], f3=layers[2][0], W4=W4, W5=W5),
-        meta=dict(T=T, seed=seed))
+        tensors=dict(x=x, f1=layers[0][0], f2=layers[1][0], f3=layers[2][0], W4=W4, W5=W5, b1=bases[0], b2=bases[1],
+                     b3=bases[2], b4=b4, b5=b5),
+        meta=dict(T=T, seed=seed, first_subsequence=10))
     return w
 
 

@@ -60,6 +60,10 @@ def test_bad_arguments_are_rejected_without_a_launch(lib):
     assert lib.nb_tap_pack_filter_i64(one, one, 1, 9, 4, 0, None) == 2
     # zero stride
     assert lib.nb_max_pool2d_i64(one, one, 1, 4, 4, 1, 2, 2, 0, 0, 0, 2, None) == 2
+    # weighted_sum: more output bits than a row's words hold
+    assert lib.nb_weighted_sum_i64(one, one, one, 4, 2, 1, 65, None) == 2
+    assert b"zbits" in lib.nb_last_error_string()
+    assert lib.nb_weighted_sum_i32(one, one, one, 4, 2, 2, 65, None) == 2
     # empty problems succeed without touching the pointers
     assert lib.nb_pack_i64(None, None, 0, 64, None) == 0
     assert lib.nb_bmm_i32(None, None, None, 0, 5, 5, 5, None) == 0

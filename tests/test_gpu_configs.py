@@ -144,6 +144,21 @@ def test_config5_cifar_net(wk, ops, oracle):
     finally:
         ops.conv_engine(prev)
     del l1, thr1
+    # the members' weights regenerated on the host from the Philox stream (subsequences 10..14 in layer order) must
+    # be what the GPU sampler wrote: all filters, eight rows of the 8192 -> 1024 layer, all of the last layer
+    T, seed = w.meta["T"], w.meta["seed"]
+    b4h, b5h = t["b4"].cpu().numpy(), t["b5"].cpu().numpy()
+    for m in (0, 2047, 4095):
+        for li, (name, C, O) in enumerate((("f1", 3, 64), ("f2", 64, 64), ("f3", 64, 128))):
+            Wn = host_member_weights(oracle, t["b%d" % (li + 1)].cpu().numpy(), C, O * 9, T, seed, 10 + li, m)
+            f = np.ascontiguousarray(Wn.reshape(1, O, 3, 3, 1).transpose(0, 2, 3, 4, 1).reshape(9, O))
+            np.testing.assert_array_equal(t[name][m].cpu().numpy(), f, err_msg="%s member %d" % (name, m))
+        W4m = t["W4"][m].cpu().numpy()
+        for r in (0, 1, 255, 256, 511, 777, 1022, 1023):
+            words = oracle.philox_words(seed, 13, (m * 1024 + r) * 8192, 8192).reshape(1, 1, 8192)
+            want = oracle.sample_from_words(T, words, np.int64, base=b4h[r:r + 1])
+            np.testing.assert_array_equal(W4m[r], want[0, 0], err_msg="W4 member %d row %d" % (m, r))
+        np.testing.assert_array_equal(t["W5"][m].cpu().numpy(), host_member_weights(oracle, b5h, 1024, 10, T, seed, 14, m))
     for m in (0, 2047, 4095):
         a = t["x"][m:m + 1].cpu().numpy()                                  # [1,32,32,1]
         for name, C, O, pool in (("f1", 3, 64, False), ("f2", 64, 64, True), ("f3", 64, 128, True)):

@@ -171,17 +171,34 @@ def test_perturbed_model_step(binary):
     for layer in pm.perturbed_layers:
         randomise(layer, g)
     pm.set_seed(123)
-    pm.set_noise()
+    bg = torch.Generator(device="cuda")
+    bg.manual_seed(9)
+    pm.set_noise(bias_generator=bg)
     x = dev(g.integers(0, 2, size=(D, 8, 8, 16)).astype(bool))
     out = pm.forward(x)
     assert tuple(out.shape) == (D, 10) and out.dtype == torch.int32
     assert all(not l.perturbed_flag for l in pm.perturbed_layers)
     assert int(out.abs().max()) <= 256 and (out % 2 == 0).all()               # 2*popc - K with K even
-    # same seed -> same noise -> same output; another seed -> different weights
+    # same seed (and the same state of the bias generator) -> same noise -> same output; another seed -> different
+    # weights
     w0 = [l.weight_noise.clone() for l in pm.perturbed_layers]
+    b0 = [l.bias_noise.clone() for l in pm.perturbed_layers]
+    bg.manual_seed(9)
+    pm.set_noise(bias_generator=bg)
+    assert all(torch.equal(a, l.weight_noise) for a, l in zip(w0, pm.perturbed_layers))
+    assert all(torch.equal(a, l.bias_noise) for a, l in zip(b0, pm.perturbed_layers))
+    assert torch.equal(pm.forward(x), out)
+    # without a generator the bias noise comes from torch's global one, as in the reference (modules/binary.py:63-64):
+    # a second set_noise() under the same seed keeps the weights but draws fresh bias noise, and two layers of the
+    # same shape under one shared seed do not share it
     pm.set_noise()
     assert all(torch.equal(a, l.weight_noise) for a, l in zip(w0, pm.perturbed_layers))
-    assert torch.equal(pm.forward(x), out)
+    b1 = [l.bias_noise.clone() for l in pm.perturbed_layers]
+    pm.set_noise()
+    assert all(not torch.equal(a, l.bias_noise) for a, l in zip(b1, pm.perturbed_layers))
+    c0, c1 = pm.perturbed_layers[0], pm.perturbed_layers[1]
+    assert c0.bias_noise.shape == c1.bias_noise.shape and not torch.equal(c0.bias_noise, c1.bias_noise)
+    assert all(float(l.bias_noise.abs().max()) <= 3.0 for l in pm.perturbed_layers)
     pm.set_seed(124)
     pm.set_noise()
     assert not torch.equal(w0[0], pm.perturbed_layers[0].weight_noise)

@@ -323,7 +323,9 @@ def test_max_pool_vs_oracle(ops, oracle, dtype):
 
 
 SAMPLE_SHAPES = [(3, 4, 64), (2, 3, 1), (5, 2, 63), (2, 5, 65), (3, 2, 200), (4, 7, 256), (2, 576, 64), (3, 10, 1024),
-                 (2, 9, 16), (3, 5, 128), (2, 3, 100), (2, 5, 256), (2, 7, 512), (2, 3, 768), (2, 3, 2048), (3, 33, 1024)]
+                 (2, 9, 16), (3, 5, 128), (2, 3, 100), (2, 5, 256), (2, 7, 512), (2, 3, 768), (2, 3, 2048), (3, 33, 1024),
+                 # more members than one member group of the wide kernel; a long row; a 3-column row (first conv layer)
+                 (17, 4, 8192), (2, 27, 3), (19, 6, 256), (9, 1024, 8)]
 
 
 @pytest.mark.parametrize("dtype", [torch.int64, torch.int32])
@@ -751,6 +753,11 @@ def test_conv_act_bool_map_via_packed_kernels(ops, oracle, C, O, D, H, W, engine
     (4, 32, 1, 5, 0, 1, 1, 1, 4, 7, 3),
     (1, 64, 4, 2, 3, 1, 1, 1, 5, 6, 2),
     (5, 24, 2, 3, 1, 2, 1, 1, 3, 3, 7),        # output wider than the input
+    # rows so wide that the LDS copy of a workgroup's input rows would pass 48 KB: the stride-1 gather straight from
+    # memory (a workgroup's 256 pixel quads lie inside one output row, or straddle two)
+    (1, 33, 3, 3, 1, 1, 1, 1, 3, 3300, 1),
+    (3, 40, 3, 3, 1, 0, 1, 1, 4, 3100, 2),
+    (2, 64, 2, 5, 0, 2, 1, 1, 2, 4099, 1),
 ])
 def test_conv_window_in_a_register_vs_oracle(ops, oracle, dtype, C, O, fx, fy, px, py, sx, sy, H, W, D):
     """Windows of at most 32 bits with packed output take the window-in-a-register kernel (engines 0 and 1):
