@@ -79,6 +79,26 @@ int nb_bmv_act_pack_i64(int64_t *out, const int64_t *A, const int64_t *x, const 
 int nb_bmv_act_pack_i32(int32_t *out, const int32_t *A, const int32_t *x, const int32_t *thresh, int64_t Z, int64_t M,
                         int64_t Kw, nb_stream_t stream);
 
+/* ---- linear layer with the population-mean threshold --------------------------------------------------
+ * BinarizedLinear(batch_norm=True) in one call: with popc[z,m] = sum_k popcount(A[z,m,k] ^ x[z,k]) and
+ * act = 2*popc - K,
+ *     mean[m]  = fp16( float(sum_z act[z,m]) / float(Z) )       (the sum is exact integer arithmetic)
+ *     thr[z,m] = fp16( fp16(bias[m] + bias_noise[z,m]) + mean[m] )
+ *     bit[z,m] = act[z,m] > thr[z,m]                            (compared exactly; false for a NaN threshold)
+ * A [Z,M,Kw], x [Z,Kw], bias [M] fp16, bias_noise [Z,M] fp16 (raw 16-bit patterns), K = true bit count of a row.
+ * pack == 0: out = bool bytes [Z,M]; pack != 0: out = words [Z, ceil(M/bits)], LSB-first, tail bits zero.
+ * workspace: device memory, 256-byte aligned, at least nb_bmv_bn_workspace_bytes(Z, M) bytes (the members' int32
+ * sums and the per-output totals pass through it; contents undefined afterwards).  The weights are read once.
+ *   replaces the composition of modules/binary.py:97-102 (bmm -> 2*popc - in_features -> .type(float16).mean(dim=0)
+ *   -> thresh -> compare); equal to it wherever act is exact in fp16 (K <= 2048) and torch's fp16 mean is exact. */
+int64_t nb_bmv_bn_workspace_bytes(int64_t Z, int64_t M);
+int nb_bmv_bn_act_i64(void *out, const int64_t *A, const int64_t *x, const uint16_t *bias, const uint16_t *bias_noise,
+                      int64_t Z, int64_t M, int64_t Kw, int64_t K, int pack, void *workspace, int64_t workspace_bytes,
+                      nb_stream_t stream);
+int nb_bmv_bn_act_i32(void *out, const int32_t *A, const int32_t *x, const uint16_t *bias, const uint16_t *bias_noise,
+                      int64_t Z, int64_t M, int64_t Kw, int64_t K, int pack, void *workspace, int64_t workspace_bytes,
+                      nb_stream_t stream);
+
 /* ---- packed im2col / conv -----------------------------------------------------------------
  * Geometry: input [D,H,W,Cw] (channels-last packed), fx taps along H, fy taps along W,
  * h=(H-fx+2px)/sx+1, w=(W-fy+2py)/sy+1, out-of-range taps read the zero word.

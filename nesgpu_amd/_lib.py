@@ -37,17 +37,22 @@ _SUFFIXED = {
     "nb_seeded_bmv_from_words": [_PTR, _PTR, _PTR, _U32, _PTR, _PTR, _I64, _I64, _I64, _PTR],
     "nb_seeded_bmv_philox": [_PTR, _PTR, _PTR, _U32, _PTR, _U64, _U64, _U64, _I64, _I64, _I64, _PTR],
     "nb_weighted_sum": [_PTR, _PTR, _PTR, _I64, _I64, _I64, _I64, _PTR],
+    "nb_bmv_bn_act": [_PTR, _PTR, _PTR, _PTR, _PTR, _I64, _I64, _I64, _I64, _I32, _PTR, _I64, _PTR],
 }
 _PLAIN = {
     "nb_philox_words": [_PTR, _U64, _U64, _U64, _I64, _PTR],
     "nb_conv_engine": [_I32],
     "nb_conv_last_engine": [],
 }
+# entry points that return a size (int64) instead of a status
+_SIZES = {
+    "nb_bmv_bn_workspace_bytes": [_I64, _I64],
+}
 
 
 def exported_symbols():
     """Every symbol include/nesbin.h declares."""
-    names = ["nb_version", "nb_last_error_string"] + list(_PLAIN)
+    names = ["nb_version", "nb_last_error_string"] + list(_PLAIN) + list(_SIZES)
     for base in _SUFFIXED:
         names += [base + "_i64", base + "_i32"]
     return names
@@ -75,6 +80,10 @@ def load():
     for name, args in _PLAIN.items():
         fn = getattr(lib, name)
         fn.restype = ctypes.c_int
+        fn.argtypes = args
+    for name, args in _SIZES.items():
+        fn = getattr(lib, name)
+        fn.restype = ctypes.c_int64
         fn.argtypes = args
     _lib = lib
     return lib

@@ -1,0 +1,166 @@
+// Linear layer with the population-mean threshold (BinarizedLinear(batch_norm=True), modules/binary.py:97-102) as one
+// call: XOR-popcount matrix-vector products of all members -> per-output sum over the population -> threshold
+// bias + bias_noise + mean in fp16 -> compare (-> pack).  The weights are streamed once; what the steps hand to each
+// other (the int32 sums of every member and the per-output totals) lives in a caller-supplied workspace.
+#include "nb_common.hpp"
+
+namespace nb {
+
+// Workspace layout: per-output totals first, then the members' sums.
+static int64_t bn_colsum_bytes(int64_t M) { return ceil_div(M * 8, 256) * 256; }
+static int64_t bn_workspace_bytes(int64_t Z, int64_t M) { return bn_colsum_bytes(M) + ceil_div(Z * M * 4, 256) * 256; }
+
+// Clears by a kernel, not a memset node, so that the call can be captured into a HIP graph.
+__global__ __launch_bounds__(256) void bn_zero_kernel(uint32_t *__restrict__ p, int64_t n)
+{
+    NB_FLAT_LOOP(t, n)
+    {
+        if (t < n) p[t] = 0u;
+    }
+}
+
+// colsum[m] += sum of popc[z, m] over one chunk of members; consecutive threads take consecutive m.
+constexpr int kBnChunk = 64;
+__global__ __launch_bounds__(256) void bn_colsum_kernel(unsigned long long *__restrict__ colsum,
+                                                        const int32_t *__restrict__ popc, int64_t Z, int64_t M)
+{
+    const int64_t m = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (m >= M) return;
+    const int64_t z0 = (int64_t)blockIdx.y * kBnChunk;
+    const int64_t z1 = z0 + kBnChunk < Z ? z0 + kBnChunk : Z;
+    unsigned long long s = 0;
+    for (int64_t z = z0; z < z1; z++) s += (unsigned long long)(uint32_t)popc[z * M + m];
+    atomicAdd(colsum + m, s);
+}
+
+// act = 2*popc - K against thr = fp16(fp16(bias + bias_noise) + mean), mean = fp16(float(sum of act) / float(Z)).
+// act is an integer and thr an fp16 number, so act > thr <=> act > floor(thr) (never for NaN).
+__device__ __forceinline__ bool bn_bit(int32_t popc, unsigned long long total, _Float16 bias, _Float16 noise, int64_t Z,
+                                       int64_t K)
+{
+    const long long sum_act = 2ll * (long long)total - (long long)K * (long long)Z;
+    const _Float16 mean = (_Float16)((float)sum_act / (float)Z);
+    const _Float16 tb = bias + noise;
+    const float t = (float)(_Float16)(tb + mean);
+    if (t != t) return false;
+    const float tc = fminf(fmaxf(t, -1.0e9f), 1.0e9f);
+    const long long act = 2ll * popc - (long long)K;
+    return act > (long long)floorf(tc);
+}
+
+__global__ __launch_bounds__(256) void bn_bool_kernel(uint8_t *__restrict__ out, const int32_t *__restrict__ popc,
+                                                      const unsigned long long *__restrict__ colsum,
+                                                      const _Float16 *__restrict__ bias,
+                                                      const _Float16 *__restrict__ noise, int64_t Z, int64_t M,
+                                                      int64_t K)
+{
+    NB_FLAT_LOOP(t, Z * M)
+    {
+        if (t < Z * M) {
+            const int64_t m = t % M;
+            out[t] = bn_bit(popc[t], colsum[m], bias[m], noise[t], Z, K) ? 1 : 0;
+        }
+    }
+}
+
+// One wave per output word: lane i < bits decides bit i, the ballot is the word.
+template <typename W>
+__global__ __launch_bounds__(256) void bn_pack_kernel(W *__restrict__ out, const int32_t *__restrict__ popc,
+                                                      const unsigned long long *__restrict__ colsum,
+                                                      const _Float16 *__restrict__ bias,
+                                                      const _Float16 *__restrict__ noise, int64_t Z, int64_t M,
+                                                      int64_t Mw, int64_t K)
+{
+    constexpr int bits = WordTraits<W>::bits;
+    const int lane = threadIdx.x & 63;
+    const int64_t wd = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (wd >= Z * Mw) return;  // wave-uniform
+    const int64_t z = wd / Mw;
+    const int64_t m = (wd - z * Mw) * bits + lane;
+    bool bit = false;
+    if (lane < bits && m < M) bit = bn_bit(popc[z * M + m], colsum[m], bias[m], noise[z * M + m], Z, K);
+    const unsigned long long word = __ballot(bit);
+    if (lane == 0) out[wd] = (W)word;
+}
+
+template <typename W>
+static int bn_impl(void *out, const W *A, const W *x, const uint16_t *bias, const uint16_t *noise, int64_t Z, int64_t M,
+                   int64_t Kw, int64_t K, int pack, void *workspace, int64_t workspace_bytes, nb_stream_t stream,
+                   const char *who)
+{
+    constexpr int bits = WordTraits<W>::bits;
+    NB_REQUIRE(Z >= 0 && M >= 0 && Kw >= 0 && K >= 0, "%s: negative shape Z=%lld M=%lld Kw=%lld K=%lld", who,
+               (long long)Z, (long long)M, (long long)Kw, (long long)K);
+    NB_REQUIRE(K <= Kw * (int64_t)bits, "%s: K=%lld exceeds the %lld bits of a row", who, (long long)K,
+               (long long)(Kw * bits));
+    if (Z * M == 0) return NB_OK;
+    NB_REQUIRE_PTR(out);
+    NB_REQUIRE_PTR(bias);
+    NB_REQUIRE_PTR(noise);
+    NB_REQUIRE_ALIGNED(bias, 2);
+    NB_REQUIRE_ALIGNED(noise, 2);
+    if (pack) NB_REQUIRE_ALIGNED(out, sizeof(W));
+    NB_REQUIRE(Z < (1LL << 31) && M < (1LL << 31) && Z * M < (1LL << 40), "%s: Z=%lld or M=%lld too large", who,
+               (long long)Z, (long long)M);
+    NB_REQUIRE(Z <= 65535 * (int64_t)kBnChunk, "%s: more than %lld members", who, (long long)(65535 * (int64_t)kBnChunk));
+    const int64_t Mw = ceil_div(M, bits);
+    NB_REQUIRE(!pack || ceil_div(Z * Mw, 4) <= kMaxGridX, "%s: output exceeds one launch", who);
+    NB_REQUIRE_PTR(workspace);
+    NB_REQUIRE_ALIGNED(workspace, 256);
+    NB_REQUIRE(workspace_bytes >= bn_workspace_bytes(Z, M), "%s: workspace of %lld bytes, %lld needed", who,
+               (long long)workspace_bytes, (long long)bn_workspace_bytes(Z, M));
+    hipStream_t s = as_stream(stream);
+    auto *colsum = static_cast<unsigned long long *>(workspace);
+    auto *popc = reinterpret_cast<int32_t *>(static_cast<unsigned char *>(workspace) + bn_colsum_bytes(M));
+    const unsigned mblocks = (unsigned)ceil_div(M, 256);
+    bn_zero_kernel<<<dim3(grid_for(2 * M)), dim3(256), 0, s>>>(reinterpret_cast<uint32_t *>(colsum), 2 * M);
+    if (int rc = check_launch(who)) return rc;
+    // the members' sums: the matrix-vector form of the XOR-popcount product (Kw == 0: all zero)
+    int rc;
+    if (Kw == 0) {
+        bn_zero_kernel<<<dim3(grid_for(Z * M)), dim3(256), 0, s>>>(reinterpret_cast<uint32_t *>(popc), Z * M);
+        rc = check_launch(who);
+    } else if (sizeof(W) == 8) {
+        rc = nb_bmm_i64(popc, reinterpret_cast<const int64_t *>(A), reinterpret_cast<const int64_t *>(x), Z, M, Kw, 1,
+                        stream);
+    } else {
+        rc = nb_bmm_i32(popc, reinterpret_cast<const int32_t *>(A), reinterpret_cast<const int32_t *>(x), Z, M, Kw, 1,
+                        stream);
+    }
+    if (rc) return rc;
+    bn_colsum_kernel<<<dim3(mblocks, (unsigned)ceil_div(Z, kBnChunk)), dim3(256), 0, s>>>(colsum, popc, Z, M);
+    if (int rc2 = check_launch(who)) return rc2;
+    const auto *b16 = reinterpret_cast<const _Float16 *>(bias), *n16 = reinterpret_cast<const _Float16 *>(noise);
+    if (pack) {
+        bn_pack_kernel<W><<<dim3((unsigned)ceil_div(Z * Mw, 4)), dim3(256), 0, s>>>(static_cast<W *>(out), popc, colsum,
+                                                                                    b16, n16, Z, M, Mw, K);
+    } else {
+        bn_bool_kernel<<<dim3(grid_for(Z * M)), dim3(256), 0, s>>>(static_cast<uint8_t *>(out), popc, colsum, b16, n16, Z,
+                                                                   M, K);
+    }
+    return check_launch(who);
+}
+
+}  // namespace nb
+
+extern "C" {
+int64_t nb_bmv_bn_workspace_bytes(int64_t Z, int64_t M)
+{
+    if (Z < 0 || M < 0 || Z >= (1LL << 31) || M >= (1LL << 31)) return -1;
+    return nb::bn_workspace_bytes(Z, M);
+}
+int nb_bmv_bn_act_i64(void *out, const int64_t *A, const int64_t *x, const uint16_t *bias, const uint16_t *bias_noise,
+                      int64_t Z, int64_t M, int64_t Kw, int64_t K, int pack, void *workspace, int64_t workspace_bytes,
+                      nb_stream_t s)
+{
+    return nb::bn_impl<uint64_t>(out, reinterpret_cast<const uint64_t *>(A), reinterpret_cast<const uint64_t *>(x), bias,
+                                 bias_noise, Z, M, Kw, K, pack, workspace, workspace_bytes, s, "nb_bmv_bn_act_i64");
+}
+int nb_bmv_bn_act_i32(void *out, const int32_t *A, const int32_t *x, const uint16_t *bias, const uint16_t *bias_noise,
+                      int64_t Z, int64_t M, int64_t Kw, int64_t K, int pack, void *workspace, int64_t workspace_bytes,
+                      nb_stream_t s)
+{
+    return nb::bn_impl<uint32_t>(out, reinterpret_cast<const uint32_t *>(A), reinterpret_cast<const uint32_t *>(x), bias,
+                                 bias_noise, Z, M, Kw, K, pack, workspace, workspace_bytes, s, "nb_bmv_bn_act_i32");
+}
+}

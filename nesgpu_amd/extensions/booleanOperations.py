@@ -24,6 +24,7 @@ __all__ = [
     "max_pool2d", "next_pow2_clip", "ceil_div", "unpack", "thresholds_from_p", "sample_bits_from_words",
     "flip_from_words", "sample_bits_philox", "flip_philox", "seeded_bmv_from_words", "seeded_bmv_philox",
     "philox_words", "conv_act_pack", "conv_popc_sums", "tap_pack_filter", "tap_packing_applies", "conv_engine", "conv_last_engine",
+    "bmv_act_pack", "bmv_bn_act",
 ]
 
 
@@ -172,6 +173,45 @@ def bmv_act_pack(A, x, threshold):
     with _on(A):
         _lib.call("nb_bmv_act_pack" + suf, out.data_ptr(), A.data_ptr(), x.data_ptr(), threshold.data_ptr(), Z, M, Kw,
                   _stream(A))
+    return out
+
+
+def bmv_bn_act(A, x, bias, bias_noise, in_bits, pack=False, workspace=None):
+    """Linear layer with the population-mean threshold in one call (not in the reference as an op: it is the
+    composition of modules/binary.py:97-102).  A [Z,M,Kw] packed weights, x [Z,Kw] (or [Z,Kw,1]) packed inputs, bias [M]
+    and bias_noise [Z,M] fp16, ``in_bits`` the true bit count K of a row.  With act = 2*popc - K:
+    thr[z,m] = fp16(fp16(bias + bias_noise) + fp16(float(sum_z act[z,m]) / Z)), result = act > thr as bool [Z,M], or with
+    ``pack`` packed along M into [Z, ceil(M/bits)] words.  ``workspace`` (uint8 CUDA tensor) is allocated when absent."""
+    _check(A, "A")
+    _check(x, "x")
+    _check(bias, "bias")
+    _check(bias_noise, "bias_noise")
+    _same_device(A, x)
+    _same_device(A, bias)
+    _same_device(A, bias_noise)
+    assert len(A.shape) == 3
+    assert A.dtype == x.dtype
+    Z, M, Kw = A.shape
+    assert x.numel() == Z * Kw and x.size(0) == Z
+    assert bias.dtype == torch.float16 and tuple(bias.shape) == (M,)
+    assert bias_noise.dtype == torch.float16 and tuple(bias_noise.shape) == (Z, M)
+    suf, bits = _suffix(A.dtype)
+    assert 0 <= in_bits <= Kw * bits
+    need = _lib.load().nb_bmv_bn_workspace_bytes(Z, M)
+    if workspace is None:
+        workspace = torch.empty((max(need, 1),), dtype=torch.uint8, device=A.device)
+    else:
+        _check(workspace, "workspace")
+        _same_device(A, workspace)
+        assert workspace.dtype == torch.uint8 and workspace.numel() >= need
+    if pack:
+        out = torch.empty((Z, ceil_div(M, bits)), dtype=A.dtype, device=A.device)
+    else:
+        out = torch.empty((Z, M), dtype=torch.bool, device=A.device)
+    with _on(A):
+        _lib.call("nb_bmv_bn_act" + suf, out.data_ptr(), A.data_ptr(), x.data_ptr(), bias.data_ptr(),
+                  bias_noise.data_ptr(), Z, M, Kw, int(in_bits), 1 if pack else 0, workspace.data_ptr(),
+                  workspace.numel(), _stream(A))
     return out
 
 

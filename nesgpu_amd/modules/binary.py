@@ -117,8 +117,8 @@ class BinarizedLinear(Binarized):
         Binarized.__init__(self, in_features, out_features, directions, threshold, dtype, device)
         self.in_features = in_features
         self.out_features = out_features
-        if pack_output and (not threshold or batch_norm):
-            raise NotImplementedError("packed output needs threshold=True and batch_norm=False")
+        if pack_output and not threshold:
+            raise NotImplementedError("packed output needs threshold=True")
         self.pack_output = pack_output    # not in the reference: return the thresholded row packed, from one kernel
         self.weight = Parameter(torch.zeros(out_features, in_features, dtype=torch.float16, device=device))
         if threshold:
@@ -130,6 +130,13 @@ class BinarizedLinear(Binarized):
         if not self.perturbed_flag:
             raise NotImplementedError                     # modules/binary.py:108-109: no inference path
         packed_input = booleanOperations.pack(input, self.dtype) if input.dtype == torch.bool else input
+        if self.threshold and self.batch_norm and (self.in_features <= 2048 or self.pack_output):
+            # modules/binary.py:97-102 in one call: the weights are streamed once, the population mean of every output
+            # comes from exact integer sums, mean = fp16(float(sum of activations) / directions), and the compare is
+            # exact (activations up to 2048 are exact in fp16, which is what the reference compares in)
+            return booleanOperations.bmv_bn_act(self.weight_noise, packed_input.view(self.directions, -1),
+                                                self.bias.detach(), self.bias_noise, self.in_features,
+                                                pack=self.pack_output)
         if self.pack_output:
             # activation > t  <=>  2*popc - K > floor(t)  <=>  2*popc > floor(t) + K  (activation is an integer)
             thresh = torch.floor((self.bias + self.bias_noise).to(torch.float32)).to(torch.int32) + self.in_features

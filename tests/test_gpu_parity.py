@@ -826,3 +826,67 @@ def test_conv_engine_selector_round_trip(ops):
     assert ops.conv_engine(2) == prev and ops.conv_engine(3) == 2 and ops.conv_engine(1) == 3
     assert ops.conv_engine(7) == 1 and ops.conv_engine() == 1                 # values out of range change nothing
     ops.conv_engine(prev)
+
+
+def _bn_expected(popc, bias, noise, K):
+    """numpy restatement of the population-mean threshold: exact integer sums, one rounding to float32, one division,
+    one rounding to fp16; fp16 additions in the reference's order (modules/binary.py:99-101); exact comparison."""
+    Z = popc.shape[0]
+    act = 2 * popc.astype(np.int64) - K
+    mean = (act.sum(axis=0).astype(np.float32) / np.float32(Z)).astype(np.float16)
+    with np.errstate(invalid="ignore", over="ignore"):
+        thr = (bias[None, :] + noise).astype(np.float16)
+        thr = (thr + mean[None, :]).astype(np.float16)
+    return act.astype(np.float64) > thr.astype(np.float64)
+
+
+@pytest.mark.parametrize("dtype", [torch.int64, torch.int32])
+def test_bmv_bn_act_vs_oracle(ops, oracle, dtype):
+    """Linear layer with the population-mean threshold in one call: the oracle's bmm for the sums, numpy for the
+    fp16 threshold arithmetic; bool and packed output, ragged member / output counts, rows of every kernel class,
+    thresholds that sit on the sums, infinities and NaNs in the noise."""
+    nd = NDT[dtype]
+    bits = np.dtype(nd).itemsize * 8
+    g = rng(31337)
+    vec = 16 // np.dtype(nd).itemsize
+    for ci, (Z, M, Kw) in enumerate([(16, 64, 4), (7, 10, 2), (33, 130, 16), (5, 64, vec * 16), (12, 256, vec * 32),
+                                     (3, 1, 1), (100, 33, 3), (9, 128, 0), (64, 1000, 8)]):
+        K = Kw * bits - (ci % 3) * (Kw > 0)                       # the true bit count may stop inside the last word
+        A = rand_words(g, (Z, M, Kw), nd)
+        x = rand_words(g, (Z, Kw), nd)
+        if Kw and K < Kw * bits:                                   # tail bits are zero on both operands (pack.cu:17)
+            keep = nd(-1) if bits - (Kw * bits - K) == bits else nd((1 << (bits - (Kw * bits - K))) - 1)
+            A[:, :, -1] &= keep
+            x[:, -1] &= keep
+        popc = oracle.bmm(A, x.reshape(Z, Kw, 1))[:, :, 0] if Kw else np.zeros((Z, M), np.int32)
+        bias = (g.standard_normal(M) * 4).astype(np.float16)
+        noise = ((g.random((Z, M)) - 0.5) * 6).astype(np.float16)
+        # make some thresholds land exactly on an activation: noise = act - mean - bias, then the compare is a tie
+        act = 2 * popc.astype(np.int64) - K
+        mean = (act.sum(axis=0).astype(np.float32) / np.float32(Z)).astype(np.float16)
+        tie = g.random((Z, M)) < 0.2
+        noise[tie] = (act - mean[None, :].astype(np.float64) - bias[None, :].astype(np.float64)).astype(np.float16)[tie]
+        noise[0, 0] = np.float16(np.inf)
+        if Z > 1:
+            noise[1, 0] = np.float16(-np.inf)
+        if M > 1:
+            noise[0, 1] = np.float16(np.nan)
+        want = _bn_expected(popc, bias, noise, K)
+        Ad, xd, bd, nz = dev(A), dev(x), dev(bias), dev(noise)
+        got = ops.bmv_bn_act(Ad, xd, bd, nz, K)
+        assert got.dtype == torch.bool and tuple(got.shape) == (Z, M)
+        np.testing.assert_array_equal(host(got), want, err_msg="case %d" % ci)
+        ws = torch.empty(int(ops._lib.load().nb_bmv_bn_workspace_bytes(Z, M)) + 256, dtype=torch.uint8, device="cuda")
+        ws.fill_(0xA5)                                             # stale contents must not matter
+        gotp = ops.bmv_bn_act(Ad, xd.view(Z, Kw, 1), bd, nz, K, pack=True, workspace=ws)
+        assert gotp.dtype == dtype and tuple(gotp.shape) == (Z, (M + bits - 1) // bits)
+        np.testing.assert_array_equal(host(gotp), oracle.pack(want, nd), err_msg="case %d packed" % ci)
+        # against torch's own expression of the reference wherever that is exact (activations within fp16's integers,
+        # a population whose reciprocal is exact)
+        if K <= 2048 and Z & (Z - 1) == 0:
+            act_t = dev(act.astype(np.int32))
+            thresh = bd + nz
+            thresh += act_t.type(torch.float16).mean(dim=0, keepdim=True)
+            assert torch.equal(got, act_t > thresh)
+    with pytest.raises(RuntimeError, match="workspace"):
+        ops._lib.call("nb_bmv_bn_act_i64", 256, 256, 256, 256, 256, 4, 64, 1, 64, 0, 256, 16, None)
