@@ -98,6 +98,17 @@ int nb_bmv_bn_act_i64(void *out, const int64_t *A, const int64_t *x, const uint1
 int nb_bmv_bn_act_i32(void *out, const int32_t *A, const int32_t *x, const uint16_t *bias, const uint16_t *bias_noise,
                       int64_t Z, int64_t M, int64_t Kw, int64_t K, int pack, void *workspace, int64_t workspace_bytes,
                       nb_stream_t stream);
+/* nb_bmv_bn_act_i64 for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc): the same computation with the workspace in a fixed device array of
+ * nb_bmv_bn_static_bytes() bytes (4 MiB + 64 KiB) that the library holds on every GPU it runs on until the process
+ * ends.  Calls no hipMalloc / hipFree / allocating routine.  Shapes that need more
+ * (nb_bmv_bn_workspace_bytes(Z, M) > nb_bmv_bn_static_bytes(), i.e. beyond about a million outputs) are rejected with
+ * NB_ERR_SHAPE.  All calls on one GPU share that array: calls that overlap in time on one GPU (different streams or
+ * threads) race; calls on one stream do not.  No counterpart in the reference. */
+int64_t nb_bmv_bn_static_bytes(void);
+int nb_bmv_bn_act_static_i64(void *out, const int64_t *A, const int64_t *x, const uint16_t *bias,
+                             const uint16_t *bias_noise, int64_t Z, int64_t M, int64_t Kw, int64_t K, int pack,
+                             nb_stream_t stream);
 
 /* ---- packed im2col / conv -----------------------------------------------------------------
  * Geometry: input [D,H,W,Cw] (channels-last packed), fx taps along H, fy taps along W,

@@ -43,10 +43,12 @@ _PLAIN = {
     "nb_philox_words": [_PTR, _U64, _U64, _U64, _I64, _PTR],
     "nb_conv_engine": [_I32],
     "nb_conv_last_engine": [],
+    "nb_bmv_bn_act_static_i64": [_PTR, _PTR, _PTR, _PTR, _PTR, _I64, _I64, _I64, _I64, _I32, _PTR],
 }
 # entry points that return a size (int64) instead of a status
 _SIZES = {
     "nb_bmv_bn_workspace_bytes": [_I64, _I64],
+    "nb_bmv_bn_static_bytes": [],
 }
 
 

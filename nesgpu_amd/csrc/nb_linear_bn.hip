@@ -1,12 +1,18 @@
 // Linear layer with the population-mean threshold (BinarizedLinear(batch_norm=True), modules/binary.py:97-102) as one
 // call: XOR-popcount matrix-vector products of all members -> per-output sum over the population -> threshold
 // bias + bias_noise + mean in fp16 -> compare (-> pack).  The weights are streamed once; what the steps hand to each
-// other (the int32 sums of every member and the per-output totals) lives in a caller-supplied workspace.
+// other (the int32 sums of every member and the per-output totals) lives in a workspace: caller-supplied, or the
+// library's own fixed device array for callers that cannot allocate.
+#include <mutex>
+
 #include "nb_common.hpp"
 
 namespace nb {
 
-// Workspace layout: per-output totals first, then the members' sums.
+// Fixed device array behind nb_bmv_bn_act_static_i64: per-output totals first, then the members' sums.
+constexpr int64_t kBnStaticBytes = (4 << 20) + (64 << 10);
+static __device__ __align__(256) unsigned char scratch[kBnStaticBytes];
+
 static int64_t bn_colsum_bytes(int64_t M) { return ceil_div(M * 8, 256) * 256; }
 static int64_t bn_workspace_bytes(int64_t Z, int64_t M) { return bn_colsum_bytes(M) + ceil_div(Z * M * 4, 256) * 256; }
 
@@ -141,6 +147,33 @@ static int bn_impl(void *out, const W *A, const W *x, const uint16_t *bias, cons
     return check_launch(who);
 }
 
+// Device address of `scratch` on the current device, looked up once per device (each GPU holds its own copy of the
+// array at its own address).
+static int bn_static_ptr(void **ptr, const char *who)
+{
+    constexpr int kMaxDevices = 64;
+    static std::mutex mu;
+    static void *ptrs[kMaxDevices] = {};
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        (void)hipGetLastError();
+        return fail(NB_ERR_UNSUPPORTED, "%s: no current device", who);
+    }
+    std::lock_guard<std::mutex> lock(mu);
+    if (!ptrs[dev]) {
+        void *p = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) {
+            (void)hipGetLastError();
+            set_error("%s: hipGetSymbolAddress failed: %s", who, hipGetErrorString(e));
+            return NB_ERR_HIP_BASE + (int)e;
+        }
+        ptrs[dev] = p;
+    }
+    *ptr = ptrs[dev];
+    return NB_OK;
+}
+
 }  // namespace nb
 
 extern "C" {
@@ -149,6 +182,7 @@ int64_t nb_bmv_bn_workspace_bytes(int64_t Z, int64_t M)
     if (Z < 0 || M < 0 || Z >= (1LL << 31) || M >= (1LL << 31)) return -1;
     return nb::bn_workspace_bytes(Z, M);
 }
+int64_t nb_bmv_bn_static_bytes(void) { return nb::kBnStaticBytes; }
 int nb_bmv_bn_act_i64(void *out, const int64_t *A, const int64_t *x, const uint16_t *bias, const uint16_t *bias_noise,
                       int64_t Z, int64_t M, int64_t Kw, int64_t K, int pack, void *workspace, int64_t workspace_bytes,
                       nb_stream_t s)
@@ -162,5 +196,20 @@ int nb_bmv_bn_act_i32(void *out, const int32_t *A, const int32_t *x, const uint1
 {
     return nb::bn_impl<uint32_t>(out, reinterpret_cast<const uint32_t *>(A), reinterpret_cast<const uint32_t *>(x), bias,
                                  bias_noise, Z, M, Kw, K, pack, workspace, workspace_bytes, s, "nb_bmv_bn_act_i32");
+}
+int nb_bmv_bn_act_static_i64(void *out, const int64_t *A, const int64_t *x, const uint16_t *bias,
+                             const uint16_t *bias_noise, int64_t Z, int64_t M, int64_t Kw, int64_t K, int pack,
+                             nb_stream_t s)
+{
+    const char *who = "nb_bmv_bn_act_static_i64";
+    if (Z >= 0 && M >= 0 && Z < (1LL << 31) && M < (1LL << 31) && nb::bn_workspace_bytes(Z, M) > nb::kBnStaticBytes)
+        return nb::fail(NB_ERR_SHAPE, "%s: Z=%lld, M=%lld need %lld bytes of workspace, the fixed array holds %lld", who,
+                        (long long)Z, (long long)M, (long long)nb::bn_workspace_bytes(Z, M),
+                        (long long)nb::kBnStaticBytes);
+    void *ptr = nullptr;
+    if (Z * M != 0)
+        if (int rc = nb::bn_static_ptr(&ptr, who)) return rc;
+    return nb::bn_impl<uint64_t>(out, reinterpret_cast<const uint64_t *>(A), reinterpret_cast<const uint64_t *>(x), bias,
+                                 bias_noise, Z, M, Kw, K, pack, ptr, nb::kBnStaticBytes, s, who);
 }
 }
