@@ -110,6 +110,48 @@ int nb_bmv_bn_act_static_i64(void *out, const int64_t *A, const int64_t *x, cons
                              const uint16_t *bias_noise, int64_t Z, int64_t M, int64_t Kw, int64_t K, int pack,
                              nb_stream_t stream);
 
+/* ---- sparse form of a population's linear layer: shared base + per-member flip lists ------------------------
+ * For per-member weights W[d] = base ^ flips[d] with few flips per row (BASELINE's "base XOR Bernoulli(p) flip mask"),
+ *     popcount(x ^ W[d,r]) = popcount(x ^ base[r]) + |flips[d,r]| - 2 * popcount(flips[d,r] & (x ^ base[r])):
+ * one shared product for the whole population plus a correction that reads 2 bytes per flip instead of 1 bit per
+ * weight bit.  Same integers as nb_bmm_i64 / nb_bmv_act_pack_i64 on the materialised W.  64-bit words only (a row of
+ * 32-bit words with an even count has the same bytes).  No counterpart in the reference, whose linear layer always
+ * streams materialised weights (modules/binary.py:97).
+ *
+ * Flip lists ("sorted slices"): perm[d, :] lists member d's rows so that every run of 64 (a slice) lies inside one
+ * block of 1024 rows (the builder orders each block by flip count); slice (d, s) owns slice_len[d, s] dwords per lane
+ * at entries[slice_off[d, s] + j * 64 + l]: the flips 2j (low half) and 2j+1 (high half) of row perm[d, 64 s + l] in
+ * column order, 16 bits each: [4:0] = column % 32, [15:5] = b * 2Kw + column / 32 with b the base bit at that column;
+ * past a row's end the sentinel (4Kw) << 5.  Kw <= 511, R <= 65536.
+ *
+ * nb_flip_count: cnt[d, r] = popcount(W[d, r, :] ^ base[r, :]) (uint16); W [D, R, Kw], base [R, Kw].
+ * nb_flip_fill:  writes the entries of every slice from W ^ base, given perm, slice_off (in dwords) and slice_len
+ *                (dwords per lane, at least ceil(max count in the slice / 2)); never writes past a slice.
+ * nb_expand_fp4: packed rows [rows, Kw] -> FP4 (E2M1) codes [rows_padded, 32 * Kw_padded] bytes, bit 1 -> +1.0,
+ *                bit 0 -> -1.0, padding -> 0.0: the operand form of nb_bmm_nt_fp4.
+ * nb_bmm_nt_fp4: C[m, n] = popcount(A_m ^ B_n), int32 [M, N], for two expanded operands (rows padded to multiples of
+ *                128, Kw_padded even); the shared-base form of the product of extensions/src/bmm.cu:5-58 on the matrix
+ *                cores (FP4 MFMA, exact for +-1).
+ * nb_bmv_flip:   out[d, r] = G[d, r] + cnt[d, r] - 2 * (number of member d's flips in row r whose looked-up bit is
+ *                set), int32 [D, R], with G = nb_bmm_nt_fp4(x, base): equal to nb_bmm_i64(W, x) with N = 1.
+ * nb_bmv_flip_act_pack: the same sums thresholded (2 * sum > thresh[d, r]) and packed along r into
+ *                [D, ceil(R/64)] words: equal to nb_bmv_act_pack_i64(W, x, thresh). */
+int nb_flip_count_i64(uint16_t *cnt, const int64_t *W, const int64_t *base, int64_t D, int64_t R, int64_t Kw,
+                      nb_stream_t stream);
+int nb_flip_fill_i64(uint32_t *entries, const int64_t *W, const int64_t *base, const uint16_t *perm,
+                     const int64_t *slice_off, const int32_t *slice_len, int64_t D, int64_t R, int64_t Kw,
+                     nb_stream_t stream);
+int nb_expand_fp4_i64(uint8_t *out, const int64_t *in, int64_t rows, int64_t Kw, int64_t rows_padded, int64_t Kw_padded,
+                      nb_stream_t stream);
+int nb_bmm_nt_fp4(int32_t *C, const uint8_t *A, const uint8_t *B, int64_t M, int64_t N, int64_t Kw, int64_t M_padded,
+                  int64_t N_padded, int64_t Kw_padded, nb_stream_t stream);
+int nb_bmv_flip_i64(int32_t *out, const int32_t *G, const uint32_t *entries, const int64_t *slice_off,
+                    const int32_t *slice_len, const uint16_t *perm, const uint16_t *cnt, const int64_t *x, int64_t D,
+                    int64_t R, int64_t Kw, nb_stream_t stream);
+int nb_bmv_flip_act_pack_i64(int64_t *out, const int32_t *G, const uint32_t *entries, const int64_t *slice_off,
+                             const int32_t *slice_len, const uint16_t *perm, const uint16_t *cnt, const int64_t *x,
+                             const int32_t *thresh, int64_t D, int64_t R, int64_t Kw, nb_stream_t stream);
+
 /* ---- packed im2col / conv -----------------------------------------------------------------
  * Geometry: input [D,H,W,Cw] (channels-last packed), fx taps along H, fy taps along W,
  * h=(H-fx+2px)/sx+1, w=(W-fy+2py)/sy+1, out-of-range taps read the zero word.

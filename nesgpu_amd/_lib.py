@@ -43,6 +43,12 @@ _PLAIN = {
     "nb_philox_words": [_PTR, _U64, _U64, _U64, _I64, _PTR],
     "nb_conv_engine": [_I32],
     "nb_conv_last_engine": [],
+    "nb_flip_count_i64": [_PTR, _PTR, _PTR, _I64, _I64, _I64, _PTR],
+    "nb_flip_fill_i64": [_PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _I64, _I64, _I64, _PTR],
+    "nb_expand_fp4_i64": [_PTR, _PTR, _I64, _I64, _I64, _I64, _PTR],
+    "nb_bmm_nt_fp4": [_PTR, _PTR, _PTR, _I64, _I64, _I64, _I64, _I64, _I64, _PTR],
+    "nb_bmv_flip_i64": [_PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _I64, _I64, _I64, _PTR],
+    "nb_bmv_flip_act_pack_i64": [_PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _I64, _I64, _I64, _PTR],
     "nb_bmv_bn_act_static_i64": [_PTR, _PTR, _PTR, _PTR, _PTR, _I64, _I64, _I64, _I64, _I32, _PTR],
 }
 # entry points that return a size (int64) instead of a status

@@ -1,0 +1,460 @@
+// Sparse form of a population's linear layer: per-member weights = base ^ flips with few flips per row.
+//
+//   popcount(x ^ (b ^ f)) = popcount(x ^ b) + |f| - 2 * popcount(f & (x ^ b))
+//
+// so a member's row sum is the SHARED product popcount(x_d ^ b_r) (one base matrix for the whole population: a real
+// matrix product with reuse, done on the matrix cores) plus a correction that only touches the member's flipped
+// columns.  With flip probability p the correction reads 2 bytes per flip (16 p bits per weight bit) instead of the
+// 1 bit per weight bit of the materialised weights: 12 % of the bytes at p = 0.01.  The result is the same integer.
+//
+// Flip lists ("sorted slices"): the rows of a member are ordered by flip count inside blocks of 1024 rows and cut into
+// slices of 64 rows; a slice stores its rows' flips interleaved, dword j of lane l = flips 2j and 2j+1 of the
+// slice's l-th row, padded with a sentinel to the slice's longest row.  A wave takes one slice: every load is one
+// 256-byte run, no per-row offsets, no cross-lane reduction.  A flip is 16 bits:
+//     [4:0]  bit inside a 32-bit piece of the input row        [15:5]  b * 2Kw + (column / 32)
+// where b is the BASE bit at that column: the kernel keeps the member's input row and its complement in LDS (2Kw
+// dwords each, then one zero dword for the sentinel 4Kw), so that the looked-up bit already is x ^ b.
+#include "nb_common.hpp"
+
+namespace nb {
+
+typedef int fl_v4i __attribute__((ext_vector_type(4)));
+typedef int fl_v8i __attribute__((ext_vector_type(8)));
+typedef float fl_v4f __attribute__((ext_vector_type(4)));
+
+constexpr int kFlipMaxKw = 511;       // 4 * Kw must fit the 11-bit piece index
+constexpr int kFlipBlockRows = 1024;  // rows are ordered inside blocks of this many (16 slices, one workgroup)
+
+// ---- bits -> FP4 (E2M1) codes: bit 1 -> 0x2 (+1.0), bit 0 -> 0xA (-1.0); bit j of the byte -> nibble j ------------
+__device__ __forceinline__ uint32_t fl_codes8(uint32_t b)
+{
+    uint32_t x = (b | (b << 12)) & 0x000F000Fu;
+    x = (x | (x << 6)) & 0x03030303u;
+    x = (x | (x << 3)) & 0x11111111u;
+    return 0xAAAAAAAAu ^ (x << 3);
+}
+
+// in [rows, Kw] 64-bit words -> out [rows_p, 32 * Kw_p] bytes: 32 bits become 16 bytes; rows past `rows` and words
+// past Kw become zero codes (0.0), which add nothing to a dot product.
+__global__ __launch_bounds__(256) void fl_expand_kernel(uint4 *__restrict__ out, const uint32_t *__restrict__ in,
+                                                        int64_t rows, int pieces, int64_t rows_p, int pieces_p)
+{
+    NB_FLAT_LOOP(t, rows_p * pieces_p)
+    {
+        if (t < rows_p * pieces_p) {
+            const int64_t r = t / pieces_p;
+            const int p = (int)(t - r * pieces_p);
+            uint4 v = make_uint4(0u, 0u, 0u, 0u);
+            if (r < rows && p < pieces) {
+                const uint32_t b = in[r * pieces + p];
+                v = make_uint4(fl_codes8(b & 255u), fl_codes8((b >> 8) & 255u), fl_codes8((b >> 16) & 255u),
+                               fl_codes8(b >> 24));
+            }
+            out[t] = v;
+        }
+    }
+}
+
+// ---- shared product on the matrix cores ---------------------------------------------------------------------------
+// C[m, n] = popcount(A_m ^ B_n) = (K - dot(+-1 codes)) / 2 with v_mfma_scale_f32_16x16x128_f8f6f4 on FP4 codes at
+// unit scales (exact: +-1 and 0 are E2M1 values, the fp32 sums are integers below 2^24).  A workgroup of four waves
+// owns a 128 x 128 tile (a wave 64 x 64 = 4 x 4 MFMA tiles); a step stages 128 positions (64 bytes) of the tile's
+// 128 + 128 rows in LDS (rows 80 bytes apart: the 16 rows of a fragment read land in different banks) while the
+// previous step's fragments are multiplied; one barrier per step.  Fragment layout: lane l supplies row l % 16 and
+// the 32 positions of 16-byte piece l / 16 (any assignment works as long as both operands use the same one);
+// acc[r] is C[4 * (l / 16) + r][l % 16].
+constexpr int kGemmTile = 128, kGemmStepBytes = 64, kGemmLd = kGemmStepBytes + 16;
+constexpr int kGemmBufBytes = 2 * kGemmTile * kGemmLd;  // both operands of one step
+
+__global__ __launch_bounds__(256) void fl_gemm_fp4_kernel(int32_t *__restrict__ C, const uint8_t *__restrict__ A,
+                                                          const uint8_t *__restrict__ B, int64_t M, int64_t N,
+                                                          int rowbytes, int kbits, int mtiles, int ntiles)
+{
+    __shared__ __align__(16) uint8_t lds[2 * kGemmBufBytes];
+    // workgroup b runs on XCD b % 8: give each XCD a contiguous run of tiles (neighbours share their A rows in L2)
+    const int T = mtiles * ntiles, per = (T + 7) / 8;
+    const int L = (int)(blockIdx.x % 8) * per + (int)(blockIdx.x / 8);
+    if (L >= T) return;  // whole workgroup, before any barrier
+    const int mt = L / ntiles, nt = L - mt * ntiles;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int lrow = tid >> 1, lhalf = tid & 1;  // staging: two threads per row, 32 bytes each
+    const uint8_t *ga = A + ((int64_t)mt * kGemmTile + lrow) * rowbytes + lhalf * 32;
+    const uint8_t *gb = B + ((int64_t)nt * kGemmTile + lrow) * rowbytes + lhalf * 32;
+    const int st_off = lrow * kGemmLd + lhalf * 32;
+    const int fa_off = (wm * 64 + (lane & 15)) * kGemmLd + (lane >> 4) * 16;
+    const int fb_off = kGemmTile * kGemmLd + (wn * 64 + (lane & 15)) * kGemmLd + (lane >> 4) * 16;
+    fl_v4f acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) acc[i][j] = fl_v4f{0.f, 0.f, 0.f, 0.f};
+    const int steps = rowbytes / kGemmStepBytes;
+    uint4 ra[2], rb[2];
+    ra[0] = *reinterpret_cast<const uint4 *>(ga);
+    ra[1] = *reinterpret_cast<const uint4 *>(ga + 16);
+    rb[0] = *reinterpret_cast<const uint4 *>(gb);
+    rb[1] = *reinterpret_cast<const uint4 *>(gb + 16);
+    {
+        uint8_t *w = lds + st_off;
+        *reinterpret_cast<uint4 *>(w) = ra[0];
+        *reinterpret_cast<uint4 *>(w + 16) = ra[1];
+        *reinterpret_cast<uint4 *>(w + kGemmTile * kGemmLd) = rb[0];
+        *reinterpret_cast<uint4 *>(w + kGemmTile * kGemmLd + 16) = rb[1];
+    }
+    __syncthreads();
+    for (int s = 0; s < steps; s++) {
+        // the next step's bytes are requested before this step's products (the last step asks for its own again, so
+        // that every step issues the same loads)
+        const int nx = (s + 1 < steps ? s + 1 : s) * kGemmStepBytes;
+        ra[0] = *reinterpret_cast<const uint4 *>(ga + nx);
+        ra[1] = *reinterpret_cast<const uint4 *>(ga + nx + 16);
+        rb[0] = *reinterpret_cast<const uint4 *>(gb + nx);
+        rb[1] = *reinterpret_cast<const uint4 *>(gb + nx + 16);
+        const uint8_t *buf = lds + (s & 1) * kGemmBufBytes;
+        fl_v4i fa[4], fb[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) fa[i] = *reinterpret_cast<const fl_v4i *>(buf + fa_off + i * 16 * kGemmLd);
+#pragma unroll
+        for (int j = 0; j < 4; j++) fb[j] = *reinterpret_cast<const fl_v4i *>(buf + fb_off + j * 16 * kGemmLd);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const fl_v8i a8 = __builtin_shufflevector(fa[i], fa[i], 0, 1, 2, 3, -1, -1, -1, -1);
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const fl_v8i b8 = __builtin_shufflevector(fb[j], fb[j], 0, 1, 2, 3, -1, -1, -1, -1);
+                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a8, b8, acc[i][j], 4, 4, 0, 0x7F7F7F7F, 0,
+                                                                             0x7F7F7F7F);
+            }
+        }
+        uint8_t *w = lds + ((s + 1) & 1) * kGemmBufBytes + st_off;
+        *reinterpret_cast<uint4 *>(w) = ra[0];
+        *reinterpret_cast<uint4 *>(w + 16) = ra[1];
+        *reinterpret_cast<uint4 *>(w + kGemmTile * kGemmLd) = rb[0];
+        *reinterpret_cast<uint4 *>(w + kGemmTile * kGemmLd + 16) = rb[1];
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const int64_t m = (int64_t)mt * kGemmTile + wm * 64 + i * 16 + 4 * (lane >> 4) + r;
+                const int64_t n = (int64_t)nt * kGemmTile + wn * 64 + j * 16 + (lane & 15);
+                if (m < M && n < N) C[m * N + n] = (kbits - (int)acc[i][j][r]) >> 1;
+            }
+}
+
+// ---- flip counts: cnt[d, r] = popcount(W[d, r, :] ^ base[r, :]), sixteen lanes per row ---------------------------
+__global__ __launch_bounds__(256) void fl_count_kernel(uint16_t *__restrict__ cnt, const uint64_t *__restrict__ W,
+                                                       const uint64_t *__restrict__ base, int64_t rows, int64_t R,
+                                                       int Kw)
+{
+    const int64_t gid = ((int64_t)blockIdx.x * 256 + threadIdx.x) >> 4;
+    const int sub = threadIdx.x & 15;
+    const bool live = gid < rows;
+    const int64_t row = live ? gid : rows - 1;
+    const int64_t r = row % R;
+    const uint64_t *w = W + row * Kw, *b = base + r * Kw;
+    int acc = 0;
+    for (int k = sub; k < Kw; k += 16) acc += __popcll(__builtin_nontemporal_load(w + k) ^ b[k]);
+    acc += __shfl_xor(acc, 8);
+    acc += __shfl_xor(acc, 4);
+    acc += __shfl_xor(acc, 2);
+    acc += __shfl_xor(acc, 1);
+    if (live && sub == 0) cnt[row] = (uint16_t)acc;
+}
+
+// ---- flip lists: one wave per slice, lane l walks the row perm[d, 64 s + l] ---------------------------------------
+__global__ __launch_bounds__(256) void fl_fill_kernel(uint32_t *__restrict__ entries, const uint64_t *__restrict__ W,
+                                                      const uint64_t *__restrict__ base,
+                                                      const uint16_t *__restrict__ perm,
+                                                      const int64_t *__restrict__ slice_off,
+                                                      const int32_t *__restrict__ slice_len, int64_t nslices, int S,
+                                                      int64_t R, int Kw)
+{
+    const int lane = threadIdx.x & 63;
+    const int64_t sl = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (sl >= nslices) return;
+    const int64_t d = sl / S;
+    const int s = (int)(sl - d * S);
+    const int64_t p = (int64_t)s * 64 + lane;
+    const bool valid = p < R;
+    int64_t r = valid ? perm[d * R + p] : 0;
+    r = r < R ? r : R - 1;
+    const int L = slice_len[sl];
+    uint32_t *dst = entries + slice_off[sl] + lane;
+    const uint32_t sentinel = (uint32_t)(4 * Kw) << 5;
+    int j = 0;
+    uint32_t pend = 0;
+    bool half = false;
+    if (valid) {
+        const uint64_t *w = W + (d * R + r) * Kw, *b = base + r * Kw;
+        for (int k = 0; k < Kw; k++) {
+            const uint64_t bw = b[k];
+            uint64_t m = w[k] ^ bw;
+            while (m) {
+                const int bit = __builtin_ctzll(m);
+                m &= m - 1;
+                const uint32_t col = (uint32_t)k * 64u + (uint32_t)bit;
+                const uint32_t bb = (uint32_t)(bw >> bit) & 1u;
+                const uint32_t e = ((bb * 2u * (uint32_t)Kw + (col >> 5)) << 5) | (col & 31u);
+                if (!half) {
+                    pend = e;
+                    half = true;
+                } else {
+                    if (j < L) dst[(int64_t)j * 64] = pend | (e << 16);  // never past the slice, whatever the inputs
+                    j++;
+                    half = false;
+                }
+            }
+        }
+    }
+    if (half) {
+        if (j < L) dst[(int64_t)j * 64] = pend | (sentinel << 16);
+        j++;
+    }
+    for (; j < L; j++) dst[(int64_t)j * 64] = sentinel | (sentinel << 16);
+}
+
+// ---- the members' corrections, threshold and pack --------------------------------------------------------------------
+// One workgroup per (member, block of 1024 rows), one wave per slice.  PACK: out = bits (2 * sum > thresh) of the
+// block's rows, OR-ed into an LDS bit array (the rows of a slice are scattered over the block) and written as 32-bit
+// pieces; else out = the int32 sums.
+template <bool PACK>
+__global__ __launch_bounds__(1024) void fl_bmv_kernel(void *__restrict__ out, const int32_t *__restrict__ G,
+                                                      const uint32_t *__restrict__ entries,
+                                                      const int64_t *__restrict__ slice_off,
+                                                      const int32_t *__restrict__ slice_len,
+                                                      const uint16_t *__restrict__ perm,
+                                                      const uint16_t *__restrict__ cnt, const uint32_t *__restrict__ x32,
+                                                      const int32_t *__restrict__ thresh, int64_t R, int S, int Kw,
+                                                      int blocks_per_member)
+{
+    extern __shared__ uint32_t fl_tab[];  // x, ~x, one zero dword, then the block's bit array
+    const int64_t d = blockIdx.x / blocks_per_member;
+    const int blk = (int)(blockIdx.x - d * blocks_per_member);
+    const int nd = 2 * Kw;
+    for (int i = threadIdx.x; i < nd; i += blockDim.x) {
+        const uint32_t v = x32[d * nd + i];
+        fl_tab[i] = v;
+        fl_tab[nd + i] = ~v;
+    }
+    uint32_t *bitmap = fl_tab + 2 * nd + 1;
+    if (threadIdx.x == 0) fl_tab[2 * nd] = 0u;
+    if (threadIdx.x < 32) bitmap[threadIdx.x] = 0u;
+    __syncthreads();
+    const int lane = threadIdx.x & 63;
+    const int s = blk * (kFlipBlockRows / 64) + (int)(threadIdx.x >> 6);  // wave-uniform
+    if (s < S) {
+        const int64_t p = (int64_t)s * 64 + lane;
+        const bool valid = p < R;
+        int64_t r = perm[d * R + (valid ? p : R - 1)];
+        r = r < R ? r : R - 1;
+        const int64_t sl = d * S + s;
+        const int L = slice_len[sl];
+        const uint32_t *src = entries + slice_off[sl] + lane;
+        const int n = cnt[d * R + r];
+        const int g = G[d * R + r];
+        const int t = PACK ? thresh[d * R + r] : 0;
+        int sy = 0;
+        auto take = [&](uint32_t e) {
+            const uint32_t w0 = fl_tab[(e >> 5) & 0x7FFu];
+            const uint32_t w1 = fl_tab[e >> 21];
+            sy += (int)((w0 >> (e & 31u)) & 1u) + (int)((w1 >> ((e >> 16) & 31u)) & 1u);
+        };
+        constexpr int U = 8;
+        int j = 0;
+        for (; j + U <= L; j += U) {
+            uint32_t e[U];
+#pragma unroll
+            for (int u = 0; u < U; u++) e[u] = load_stream4(src + (int64_t)(j + u) * 64);
+            __builtin_amdgcn_sched_barrier(0);  // all loads of the step in flight before the first look-up
+#pragma unroll
+            for (int u = 0; u < U; u++) take(e[u]);
+        }
+        for (; j < L; j++) take(load_stream4(src + (int64_t)j * 64));
+        const int sum = g + n - 2 * sy;
+        if (PACK) {
+            const int local = (int)(r - (int64_t)blk * kFlipBlockRows);
+            if (valid && 2 * sum > t) atomicOr(&bitmap[(local >> 5) & 31], 1u << (local & 31));
+        } else if (valid) {
+            static_cast<int32_t *>(out)[d * R + r] = sum;
+        }
+    }
+    if (PACK) {
+        __syncthreads();
+        const int pieces = 2 * (int)((R + 63) / 64);  // 32-bit pieces of a member's output row
+        const int q = blk * 32 + (int)threadIdx.x;
+        if (threadIdx.x < 32 && q < pieces) static_cast<uint32_t *>(out)[d * pieces + q] = bitmap[threadIdx.x];
+    }
+}
+
+static int flip_shape_check(int64_t D, int64_t R, int64_t Kw, const char *who)
+{
+    NB_REQUIRE(D >= 0 && R >= 0 && Kw >= 0, "%s: negative shape D=%lld R=%lld Kw=%lld", who, (long long)D, (long long)R,
+               (long long)Kw);
+    NB_REQUIRE(Kw <= kFlipMaxKw, "%s: rows of %lld words, at most %d", who, (long long)Kw, kFlipMaxKw);
+    NB_REQUIRE(R <= 65536, "%s: %lld rows per member, at most 65536", who, (long long)R);
+    NB_REQUIRE(D * ((R + 63) / 64) <= (1LL << 31) && D * R < (1LL << 40), "%s: too many rows", who);
+    return NB_OK;
+}
+
+}  // namespace nb
+
+extern "C" {
+int nb_expand_fp4_i64(uint8_t *out, const int64_t *in, int64_t rows, int64_t Kw, int64_t rows_padded, int64_t Kw_padded,
+                      nb_stream_t stream)
+{
+    const char *who = "nb_expand_fp4_i64";
+    NB_REQUIRE(rows >= 0 && Kw >= 0 && rows_padded >= rows && Kw_padded >= Kw, "%s: bad shape", who);
+    NB_REQUIRE(Kw_padded < (1 << 20) && rows_padded < (1LL << 40), "%s: too large", who);
+    if (rows_padded * Kw_padded == 0) return NB_OK;
+    NB_REQUIRE_PTR(out);
+    NB_REQUIRE_ALIGNED(out, 16);
+    if (rows * Kw > 0) {
+        NB_REQUIRE_PTR(in);
+        NB_REQUIRE_ALIGNED(in, 8);
+    }
+    nb::fl_expand_kernel<<<dim3(nb::grid_for(rows_padded * Kw_padded * 2)), dim3(256), 0, nb::as_stream(stream)>>>(
+        reinterpret_cast<uint4 *>(out), reinterpret_cast<const uint32_t *>(in), rows, (int)(2 * Kw), rows_padded,
+        (int)(2 * Kw_padded));
+    return nb::check_launch(who);
+}
+
+int nb_bmm_nt_fp4(int32_t *C, const uint8_t *A, const uint8_t *B, int64_t M, int64_t N, int64_t Kw, int64_t M_padded,
+                  int64_t N_padded, int64_t Kw_padded, nb_stream_t stream)
+{
+    const char *who = "nb_bmm_nt_fp4";
+    NB_REQUIRE(M >= 0 && N >= 0 && Kw >= 0 && Kw_padded >= Kw, "%s: bad shape", who);
+    if (M * N == 0) return NB_OK;
+    NB_REQUIRE(M_padded >= nb::ceil_div(M, nb::kGemmTile) * nb::kGemmTile &&
+                   N_padded >= nb::ceil_div(N, nb::kGemmTile) * nb::kGemmTile,
+               "%s: operands must be padded to whole tiles of %d rows (M_padded=%lld, N_padded=%lld)", who,
+               nb::kGemmTile, (long long)M_padded, (long long)N_padded);
+    NB_REQUIRE(Kw_padded >= 2 && Kw_padded % 2 == 0, "%s: padded row of %lld words, a positive even count needed", who,
+               (long long)Kw_padded);
+    NB_REQUIRE(Kw_padded * 64 < (1 << 24), "%s: rows too long for exact fp32 sums", who);
+    NB_REQUIRE_PTR(C);
+    NB_REQUIRE_PTR(A);
+    NB_REQUIRE_PTR(B);
+    NB_REQUIRE_ALIGNED(C, 4);
+    NB_REQUIRE_ALIGNED(A, 16);
+    NB_REQUIRE_ALIGNED(B, 16);
+    const int64_t mt = nb::ceil_div(M, nb::kGemmTile), nt = nb::ceil_div(N, nb::kGemmTile);
+    NB_REQUIRE(mt * nt < (1 << 24), "%s: too many tiles", who);
+    const int64_t grid = nb::ceil_div(mt * nt, 8) * 8;
+    nb::fl_gemm_fp4_kernel<<<dim3((unsigned)grid), dim3(256), 0, nb::as_stream(stream)>>>(
+        C, A, B, M, N, (int)(Kw_padded * 32), (int)(Kw * 64), (int)mt, (int)nt);
+    return nb::check_launch(who);
+}
+
+int nb_flip_count_i64(uint16_t *cnt, const int64_t *W, const int64_t *base, int64_t D, int64_t R, int64_t Kw,
+                      nb_stream_t stream)
+{
+    const char *who = "nb_flip_count_i64";
+    if (int rc = nb::flip_shape_check(D, R, Kw, who)) return rc;
+    if (D * R == 0) return NB_OK;
+    NB_REQUIRE_PTR(cnt);
+    NB_REQUIRE_ALIGNED(cnt, 2);
+    if (Kw > 0) {
+        NB_REQUIRE_PTR(W);
+        NB_REQUIRE_PTR(base);
+        NB_REQUIRE_ALIGNED(W, 8);
+        NB_REQUIRE_ALIGNED(base, 8);
+    }
+    const int64_t blocks = nb::ceil_div(D * R * 16, 256);
+    NB_REQUIRE(blocks <= nb::kMaxGridX, "%s: too many rows for one launch", who);
+    nb::fl_count_kernel<<<dim3((unsigned)blocks), dim3(256), 0, nb::as_stream(stream)>>>(
+        cnt, reinterpret_cast<const uint64_t *>(W), reinterpret_cast<const uint64_t *>(base), D * R, R, (int)Kw);
+    return nb::check_launch(who);
+}
+
+int nb_flip_fill_i64(uint32_t *entries, const int64_t *W, const int64_t *base, const uint16_t *perm,
+                     const int64_t *slice_off, const int32_t *slice_len, int64_t D, int64_t R, int64_t Kw,
+                     nb_stream_t stream)
+{
+    const char *who = "nb_flip_fill_i64";
+    if (int rc = nb::flip_shape_check(D, R, Kw, who)) return rc;
+    if (D * R == 0) return NB_OK;
+    NB_REQUIRE_PTR(entries);
+    NB_REQUIRE_PTR(perm);
+    NB_REQUIRE_PTR(slice_off);
+    NB_REQUIRE_PTR(slice_len);
+    NB_REQUIRE_ALIGNED(entries, 4);
+    NB_REQUIRE_ALIGNED(perm, 2);
+    NB_REQUIRE_ALIGNED(slice_off, 8);
+    NB_REQUIRE_ALIGNED(slice_len, 4);
+    if (Kw > 0) {
+        NB_REQUIRE_PTR(W);
+        NB_REQUIRE_PTR(base);
+        NB_REQUIRE_ALIGNED(W, 8);
+        NB_REQUIRE_ALIGNED(base, 8);
+    }
+    const int64_t S = (R + 63) / 64;
+    nb::fl_fill_kernel<<<dim3((unsigned)nb::ceil_div(D * S, 4)), dim3(256), 0, nb::as_stream(stream)>>>(
+        entries, reinterpret_cast<const uint64_t *>(W), reinterpret_cast<const uint64_t *>(base), perm, slice_off,
+        slice_len, D * S, (int)S, R, (int)Kw);
+    return nb::check_launch(who);
+}
+
+static int flip_bmv(void *out, const int32_t *G, const uint32_t *entries, const int64_t *slice_off,
+                    const int32_t *slice_len, const uint16_t *perm, const uint16_t *cnt, const int64_t *x,
+                    const int32_t *thresh, int64_t D, int64_t R, int64_t Kw, bool pack, nb_stream_t stream,
+                    const char *who)
+{
+    if (int rc = nb::flip_shape_check(D, R, Kw, who)) return rc;
+    if (D * R == 0) return NB_OK;
+    NB_REQUIRE_PTR(out);
+    NB_REQUIRE_PTR(G);
+    NB_REQUIRE_PTR(entries);
+    NB_REQUIRE_PTR(slice_off);
+    NB_REQUIRE_PTR(slice_len);
+    NB_REQUIRE_PTR(perm);
+    NB_REQUIRE_PTR(cnt);
+    if (pack) NB_REQUIRE_PTR(thresh);
+    if (Kw > 0) NB_REQUIRE_PTR(x);
+    NB_REQUIRE_ALIGNED(out, pack ? 8 : 4);
+    NB_REQUIRE_ALIGNED(G, 4);
+    NB_REQUIRE_ALIGNED(entries, 4);
+    NB_REQUIRE_ALIGNED(slice_off, 8);
+    NB_REQUIRE_ALIGNED(slice_len, 4);
+    NB_REQUIRE_ALIGNED(perm, 2);
+    NB_REQUIRE_ALIGNED(cnt, 2);
+    NB_REQUIRE_ALIGNED(x, 8);
+    NB_REQUIRE_ALIGNED(thresh, 4);
+    const int64_t S = (R + 63) / 64;
+    const int per_block = nb::kFlipBlockRows / 64;
+    const int64_t bpm = nb::ceil_div(S, per_block);
+    NB_REQUIRE(D * bpm <= nb::kMaxGridX, "%s: too many rows for one launch", who);
+    const unsigned threads = 64u * (unsigned)(S < per_block ? S : per_block);
+    const size_t lds = (size_t)(4 * Kw + 1 + 32) * 4;
+    const dim3 grid((unsigned)(D * bpm));
+    if (pack)
+        nb::fl_bmv_kernel<true><<<grid, dim3(threads), lds, nb::as_stream(stream)>>>(
+            out, G, entries, slice_off, slice_len, perm, cnt, reinterpret_cast<const uint32_t *>(x), thresh, R, (int)S,
+            (int)Kw, (int)bpm);
+    else
+        nb::fl_bmv_kernel<false><<<grid, dim3(threads), lds, nb::as_stream(stream)>>>(
+            out, G, entries, slice_off, slice_len, perm, cnt, reinterpret_cast<const uint32_t *>(x), thresh, R, (int)S,
+            (int)Kw, (int)bpm);
+    return nb::check_launch(who);
+}
+
+int nb_bmv_flip_i64(int32_t *out, const int32_t *G, const uint32_t *entries, const int64_t *slice_off,
+                    const int32_t *slice_len, const uint16_t *perm, const uint16_t *cnt, const int64_t *x, int64_t D,
+                    int64_t R, int64_t Kw, nb_stream_t stream)
+{
+    return flip_bmv(out, G, entries, slice_off, slice_len, perm, cnt, x, nullptr, D, R, Kw, false, stream,
+                    "nb_bmv_flip_i64");
+}
+
+int nb_bmv_flip_act_pack_i64(int64_t *out, const int32_t *G, const uint32_t *entries, const int64_t *slice_off,
+                             const int32_t *slice_len, const uint16_t *perm, const uint16_t *cnt, const int64_t *x,
+                             const int32_t *thresh, int64_t D, int64_t R, int64_t Kw, nb_stream_t stream)
+{
+    return flip_bmv(out, G, entries, slice_off, slice_len, perm, cnt, x, thresh, D, R, Kw, true, stream,
+                    "nb_bmv_flip_act_pack_i64");
+}
+}

@@ -24,7 +24,8 @@ __all__ = [
     "max_pool2d", "next_pow2_clip", "ceil_div", "unpack", "thresholds_from_p", "sample_bits_from_words",
     "flip_from_words", "sample_bits_philox", "flip_philox", "seeded_bmv_from_words", "seeded_bmv_philox",
     "philox_words", "conv_act_pack", "conv_popc_sums", "tap_pack_filter", "tap_packing_applies", "conv_engine", "conv_last_engine",
-    "bmv_act_pack", "bmv_bn_act",
+    "bmv_act_pack", "bmv_bn_act", "ExpandedRows", "expand_rows", "bmm_nt", "FlipRows", "flip_rows_from_weights",
+    "bmv_flip", "bmv_flip_act_pack",
 ]
 
 
@@ -581,4 +582,139 @@ def conv_act_pack(input, filter, threshold, filterx, filtery, padx, pady, stride
         _lib.call("nb_conv_act_pack" + suf, out.data_ptr(), input.data_ptr(), filter.data_ptr(), threshold.data_ptr(),
                   input.size(0), input.size(1), input.size(2), input.size(3), filter.size(2), filterx, filtery, padx,
                   pady, stridex, stridey, 1 if pool else 0, tap, _stream(input))
+    return out
+
+
+# ---- sparse form of a population's linear layer: shared base + per-member flip lists ----------------------------
+_GEMM_TILE = 128                     # row padding of the expanded operands of bmm_nt (the matrix-core tile)
+
+
+class ExpandedRows:
+    """Packed rows [rows, Kw] expanded to FP4 codes (+1.0 / -1.0, zero padding) for :func:`bmm_nt`:
+    ``codes`` is uint8 [rows_padded, 32 * Kw_padded]."""
+
+    def __init__(self, codes, rows, Kw, rows_padded, Kw_padded):
+        self.codes, self.rows, self.Kw, self.rows_padded, self.Kw_padded = codes, rows, Kw, rows_padded, Kw_padded
+
+
+def expand_rows(x):
+    """int64 [rows, Kw] packed bits -> :class:`ExpandedRows` (one pass, 16 bytes out per 32 bits in)."""
+    _check(x, "x")
+    assert len(x.shape) == 2
+    if x.dtype != torch.int64:
+        raise TypeError("expand_rows takes 64-bit words")
+    rows, Kw = x.shape
+    rp = ceil_div(rows, _GEMM_TILE) * _GEMM_TILE
+    kp = max(2, ceil_div(Kw, 2) * 2)
+    codes = torch.empty((rp, 32 * kp), dtype=torch.uint8, device=x.device)
+    with _on(x):
+        _lib.call("nb_expand_fp4_i64", codes.data_ptr(), x.data_ptr(), rows, Kw, rp, kp, _stream(x))
+    return ExpandedRows(codes, rows, Kw, rp, kp)
+
+
+def bmm_nt(A, B):
+    """C[m, n] = popcount(A[m, :] ^ B[n, :]), int32 [M, N]: the XOR-popcount product of two row sets that share K
+    (both K-contiguous), on the matrix cores.  A, B: int64 [M, Kw] / [N, Kw] or :class:`ExpandedRows`.  Equals
+    ``bmm(A[None], B.t()[None])[0]`` of the reference op (extensions/booleanOperations.py:107-129)."""
+    ea = A if isinstance(A, ExpandedRows) else expand_rows(A)
+    eb = B if isinstance(B, ExpandedRows) else expand_rows(B)
+    assert ea.Kw == eb.Kw and ea.Kw_padded == eb.Kw_padded
+    if ea.codes.device != eb.codes.device:
+        raise RuntimeError("Tensors are on different devices")
+    C = torch.empty((ea.rows, eb.rows), dtype=torch.int32, device=ea.codes.device)
+    with _on(ea.codes):
+        _lib.call("nb_bmm_nt_fp4", C.data_ptr(), ea.codes.data_ptr(), eb.codes.data_ptr(), ea.rows, eb.rows, ea.Kw,
+                  ea.rows_padded, eb.rows_padded, ea.Kw_padded, _stream(ea.codes))
+    return C
+
+
+class FlipRows:
+    """Per-member weights of a linear layer, W[d] = base ^ flips[d], kept as the shared base and per-member flip
+    lists (layout in include/nesbin.h).  Built by :func:`flip_rows_from_weights`; consumed by :func:`bmv_flip` and
+    :func:`bmv_flip_act_pack`, which return what ``bmm`` / ``bmv_act_pack`` return on the materialised weights."""
+
+    def __init__(self, base, D, R, Kw, cnt, perm, slice_off, slice_len, entries):
+        self.base, self.D, self.R, self.Kw = base, D, R, Kw
+        self.cnt, self.perm, self.slice_off, self.slice_len, self.entries = cnt, perm, slice_off, slice_len, entries
+        self.base_expanded = expand_rows(base)
+
+    def nbytes(self):
+        """Bytes one forward reads of the member-specific data (flip lists, counts, row order, slice tables)."""
+        return sum(t.numel() * t.element_size() for t in (self.entries, self.cnt, self.perm, self.slice_off,
+                                                           self.slice_len))
+
+
+def flip_rows_from_weights(W, base):
+    """W int64 [D, R, Kw] (a population's materialised weights), base int64 [R, Kw] -> :class:`FlipRows` holding
+    exactly the bits W ^ base.  Rows are ordered by flip count inside blocks of 1024 rows so that the 64 rows of a
+    slice are about equally long."""
+    _check(W, "W")
+    _check(base, "base")
+    _same_device(W, base)
+    assert len(W.shape) == 3 and len(base.shape) == 2
+    if W.dtype != torch.int64 or base.dtype != torch.int64:
+        raise TypeError("flip lists take 64-bit words")
+    D, R, Kw = W.shape
+    assert tuple(base.shape) == (R, Kw)
+    dev = W.device
+    cnt = torch.empty((D, R), dtype=torch.uint16, device=dev)
+    with _on(W):
+        _lib.call("nb_flip_count_i64", cnt.data_ptr(), W.data_ptr(), base.data_ptr(), D, R, Kw, _stream(W))
+    S = ceil_div(R, 64)
+    nblk = ceil_div(R, 1024)
+    c = cnt.view(torch.int16).to(torch.int32) & 0xFFFF
+    cp = torch.nn.functional.pad(c, (0, nblk * 1024 - R), value=1 << 20).view(D, nblk, 1024)
+    order = torch.sort(cp, dim=2, stable=True).indices + (torch.arange(nblk, device=dev) * 1024).view(1, nblk, 1)
+    order = order.view(D, nblk * 1024)[:, :R].contiguous()                       # padding sorts last in its block
+    cs = torch.nn.functional.pad(c.gather(1, order), (0, S * 64 - R)).view(D, S, 64)
+    slice_len = ((cs.max(dim=2).values + 1) // 2).to(torch.int32).contiguous()  # dwords (two flips) per lane
+    lens = slice_len.view(-1).to(torch.int64) * 64
+    slice_off = (torch.cumsum(lens, 0) - lens).view(D, S).contiguous()
+    total = int(lens.sum().item()) if D * S else 0
+    perm = order.to(torch.uint16).contiguous()
+    entries = torch.empty((max(total, 1),), dtype=torch.uint32, device=dev)
+    with _on(W):
+        _lib.call("nb_flip_fill_i64", entries.data_ptr(), W.data_ptr(), base.data_ptr(), perm.data_ptr(),
+                  slice_off.data_ptr(), slice_len.data_ptr(), D, R, Kw, _stream(W))
+    return FlipRows(base, D, R, Kw, cnt, perm, slice_off, slice_len, entries)
+
+
+def _flip_args(rows, x, G):
+    _check(x, "x")
+    if x.dtype != torch.int64:
+        raise TypeError("flip lists take 64-bit words")
+    assert x.numel() == rows.D * rows.Kw and x.size(0) == rows.D
+    if x.device != rows.entries.device:
+        raise RuntimeError("Tensors are on different devices")
+    if G is None:
+        G = bmm_nt(x.view(rows.D, rows.Kw), rows.base_expanded)       # the shared product popcount(x_d ^ base_r)
+    else:
+        _check(G, "G")
+        assert tuple(G.shape) == (rows.D, rows.R) and G.dtype == torch.int32
+    return G
+
+
+def bmv_flip(rows, x, G=None):
+    """int32 [D, R]: sum_k popcount(W[d, r, k] ^ x[d, k]) for the weights held by ``rows`` (:class:`FlipRows`); what
+    ``bmm(W, x.view(D, Kw, 1)).squeeze(2)`` gives on the materialised weights."""
+    G = _flip_args(rows, x, G)
+    out = torch.empty((rows.D, rows.R), dtype=torch.int32, device=x.device)
+    with _on(x):
+        _lib.call("nb_bmv_flip_i64", out.data_ptr(), G.data_ptr(), rows.entries.data_ptr(), rows.slice_off.data_ptr(),
+                  rows.slice_len.data_ptr(), rows.perm.data_ptr(), rows.cnt.data_ptr(), x.data_ptr(), rows.D, rows.R,
+                  rows.Kw, _stream(x))
+    return out
+
+
+def bmv_flip_act_pack(rows, x, threshold, G=None):
+    """Packed bits (2 * sum > threshold[d, r]) as int64 [D, ceil(R/64)]: what ``bmv_act_pack(W, x, threshold)`` gives
+    on the materialised weights."""
+    G = _flip_args(rows, x, G)
+    _check(threshold, "threshold")
+    assert tuple(threshold.shape) == (rows.D, rows.R) and threshold.dtype == torch.int32
+    out = torch.empty((rows.D, ceil_div(rows.R, 64)), dtype=torch.int64, device=x.device)
+    with _on(x):
+        _lib.call("nb_bmv_flip_act_pack_i64", out.data_ptr(), G.data_ptr(), rows.entries.data_ptr(),
+                  rows.slice_off.data_ptr(), rows.slice_len.data_ptr(), rows.perm.data_ptr(), rows.cnt.data_ptr(),
+                  x.data_ptr(), threshold.data_ptr(), rows.D, rows.R, rows.Kw, _stream(x))
     return out
