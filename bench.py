@@ -106,6 +106,8 @@ def config_entry(cfg, w, per_wall, per_ev, per_graph=None):
     from nesgpu_amd.extensions import booleanOperations as ops
     entry = {"config": cfg, "workload": w.name, "ms_per_step": round(per_wall * 1e3, 4),
              "binary_TOPS": round(2 * w.bit_macs / per_wall / 1e12, 3)}
+    if "fc" in w.meta:
+        entry["fc_8192_1024"] = w.meta["fc"]
     if per_graph:
         # device time per step from a graph replay; the roofline fractions below use it when it is available
         entry.update(ms_per_step_graph=round(per_graph * 1e3, 4),

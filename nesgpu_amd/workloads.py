@@ -162,9 +162,13 @@ def conv_sign_pool(D=1024, C=16, O=16, S=64, k=3, pad=1, T=T_P02, seed=0, dtype=
     return w
 
 
-def cifar_net(D=4096, T=T_P01, seed=0, dtype=torch.int64, device="cuda", classes=10):
+def cifar_net(D=4096, T=T_P01, seed=0, dtype=torch.int64, device="cuda", classes=10, sparse_fc=True):
     """Config 5: conv3->64, conv64->64, pool, conv64->128, pool, linear 8192->1024, linear 1024->10 on 3x32x32
-    inputs binarised at their per-channel mean; sign threshold 0 between layers; int32 logits (raw popc)."""
+    inputs binarised at their per-channel mean; sign threshold 0 between layers; int32 logits (raw popc).
+
+    ``sparse_fc``: the 8192->1024 layer runs from the shared base and the members' flip lists (one product for the
+    whole population on the matrix cores + 2 bytes per flipped weight) instead of streaming the 4 GiB of
+    materialised per-member weights; the same bits either way (``step_dense`` in ``meta`` is the other form)."""
     g = _gen(seed)
     z = torch.randn((D, 3, 32, 32), generator=g)
     x_bits = (z > z.mean(dim=(0, 2, 3), keepdim=True)).permute(0, 2, 3, 1).contiguous()      # [D,32,32,3]
@@ -188,23 +192,34 @@ def cifar_net(D=4096, T=T_P01, seed=0, dtype=torch.int64, device="cuda", classes
     W5 = ops.flip_philox(b5, 1024, D, T, seed, subsequence=subseq + 1)
     macs += D * 1024 * 8192 + D * classes * 1024
     thr4 = torch.full((D, 1024), 8192, dtype=torch.int32, device=device)
+    rows4 = ops.flip_rows_from_weights(W4, b4) if (sparse_fc and dtype == torch.int64) else None
 
-    def step():
+    def features():
         a = x
         for i, pool in enumerate((False, True, True)):                   # [D,32,32,1] [D,16,16,1] [D,8,8,2]
             _, thr, f, kw = layers[i]
             a = ops.conv_act_pack(a, f, thr, 3, 3, 1, 1, 1, 1, pool=pool, **kw)
-        a = a.view(D, -1, 1)                                                                    # [D,128,1]
-        a = ops.bmv_act_pack(W4, a, thr4).view(D, -1, 1)                  # pack(2 * bmm(W4, a) > 8192): [D,16,1]
+        return a.view(D, -1, 1)                                                                 # [D,128,1]
+
+    def step_dense():
+        a = ops.bmv_act_pack(W4, features(), thr4).view(D, -1, 1)         # pack(2 * bmm(W4, a) > 8192): [D,16,1]
         return ops.bmm(W5, a).squeeze(2)                                                        # [D,classes] popc
+
+    def step_sparse():
+        a = ops.bmv_flip_act_pack(rows4, features(), thr4).view(D, -1, 1)  # the same bits from base + flip lists
+        return ops.bmm(W5, a).squeeze(2)
+
+    step = step_sparse if rows4 is not None else step_dense
 
     w = Workload(
         name="CIFAR-shaped binary net D=%d (conv3-64, conv64-64, pool, conv64-128, pool, fc8192-1024, fc1024-%d)"
              % (D, classes),
-        population=D, bit_macs=macs, algo_bytes=W4.numel() * 8, bound="valu", step=step,
+        population=D, bit_macs=macs, algo_bytes=rows4.nbytes() if rows4 is not None else W4.numel() * 8, bound="valu",
+        step=step,
         tensors=dict(x=x, f1=layers[0][0], f2=layers[1][0], f3=layers[2][0], W4=W4, W5=W5, b1=bases[0], b2=bases[1],
                      b3=bases[2], b4=b4, b5=b5),
-        meta=dict(T=T, seed=seed, first_subsequence=10))
+        meta=dict(T=T, seed=seed, first_subsequence=10, step_dense=step_dense, features=features, rows4=rows4,
+                  thr4=thr4, fc="base + flip lists" if rows4 is not None else "materialised weights"))
     return w
 
 

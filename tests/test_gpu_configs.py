@@ -126,11 +126,22 @@ def test_config5_cifar_net(wk, ops, oracle):
     assert tuple(out.shape) == (D, 10) and out.dtype == torch.int32
     assert torch.equal(w.step(), out)                                      # deterministic
     t = w.tensors
+    # the 8192 -> 1024 layer runs from the shared base + flip lists: the logits must be those of the materialised
+    # weights, every member; and so must the layer itself on the net's real features and on random inputs with
+    # thresholds around the sums
+    assert w.meta["fc"] == "base + flip lists"
+    assert torch.equal(w.meta["step_dense"](), out)
+    rows4, feats = w.meta["rows4"], w.meta["features"]()
+    assert torch.equal(ops.bmv_flip_act_pack(rows4, feats, w.meta["thr4"]), ops.bmv_act_pack(t["W4"], feats, w.meta["thr4"]))
+    assert torch.equal(ops.bmv_flip(rows4, feats), ops.bmm(t["W4"], feats).squeeze(2))
+    del feats
     # the fused linear-layer kernel against the unfused composition, every member, thresholds around the sums
     a4 = torch.randint(-2 ** 62, 2 ** 62, (D, 128, 1), dtype=torch.int64, device="cuda")
     sums = ops.bmm(t["W4"], a4).squeeze(2)
     thr4 = (2 * sums + torch.randint(-2, 3, sums.shape, device="cuda")).to(torch.int32)
     assert torch.equal(ops.bmv_act_pack(t["W4"], a4, thr4), ops.pack(2 * sums > thr4, torch.int64))
+    assert torch.equal(ops.bmv_flip_act_pack(rows4, a4, thr4), ops.pack(2 * sums > thr4, torch.int64))
+    assert torch.equal(ops.bmv_flip(rows4, a4), sums)
     del a4, sums, thr4
     # the first layer on all members: window-per-register kernel (automatic choice) == int8 matrix-core kernel
     thr1 = torch.full((D, 64), 27, dtype=torch.int32, device="cuda")
