@@ -119,14 +119,15 @@ int nb_bmv_bn_act_static_i64(void *out, const int64_t *A, const int64_t *x, cons
  * streams materialised weights (modules/binary.py:97).
  *
  * Flip lists ("sorted slices"): perm[d, :] lists member d's rows so that every run of 64 (a slice) lies inside one
- * block of 1024 rows (the builder orders each block by flip count); slice (d, s) owns slice_len[d, s] dwords per lane
- * at entries[slice_off[d, s] + j * 64 + l]: the flips 2j (low half) and 2j+1 (high half) of row perm[d, 64 s + l] in
- * column order, 16 bits each: [4:0] = column % 32, [15:5] = b * 2Kw + column / 32 with b the base bit at that column;
+ * block of 1024 rows (the builder orders each block by flip count); slice (d, s) owns slice_len[d, s] 16-byte pieces
+ * per lane, piece j of lane l at dword offset slice_off[d, s] + (j * 64 + l) * 4 of entries (slice_off a multiple of
+ * 4, entries 16-byte aligned): the flips 8j .. 8j+7 of row perm[d, 64 s + l] in column order (low half of a dword
+ * first), 16 bits each: [4:0] = column % 32, [15:5] = 2 * (column / 32) + b with b the base bit at that column;
  * past a row's end the sentinel (4Kw) << 5.  Kw <= 511, R <= 65536.
  *
  * nb_flip_count: cnt[d, r] = popcount(W[d, r, :] ^ base[r, :]) (uint16); W [D, R, Kw], base [R, Kw].
  * nb_flip_fill:  writes the entries of every slice from W ^ base, given perm, slice_off (in dwords) and slice_len
- *                (dwords per lane, at least ceil(max count in the slice / 2)); never writes past a slice.
+ *                (pieces per lane, at least ceil(max count in the slice / 8)); never writes past a slice.
  * nb_expand_fp4: packed rows [rows, Kw] -> FP4 (E2M1) codes [rows_padded, 32 * Kw_padded] bytes, bit 1 -> +1.0,
  *                bit 0 -> -1.0, padding -> 0.0: the operand form of nb_bmm_nt_fp4.
  * nb_bmm_nt_fp4: C[m, n] = popcount(A_m ^ B_n), int32 [M, N], for two expanded operands (rows padded to multiples of

@@ -8,12 +8,16 @@
 // 1 bit per weight bit of the materialised weights: 12 % of the bytes at p = 0.01.  The result is the same integer.
 //
 // Flip lists ("sorted slices"): the rows of a member are ordered by flip count inside blocks of 1024 rows and cut into
-// slices of 64 rows; a slice stores its rows' flips interleaved, dword j of lane l = flips 2j and 2j+1 of the
-// slice's l-th row, padded with a sentinel to the slice's longest row.  A wave takes one slice: every load is one
-// 256-byte run, no per-row offsets, no cross-lane reduction.  A flip is 16 bits:
-//     [4:0]  bit inside a 32-bit piece of the input row        [15:5]  b * 2Kw + (column / 32)
-// where b is the BASE bit at that column: the kernel keeps the member's input row and its complement in LDS (2Kw
-// dwords each, then one zero dword for the sentinel 4Kw), so that the looked-up bit already is x ^ b.
+// slices of 64 rows; a slice stores its rows' flips interleaved in 16-byte pieces: piece j of lane l = flips 8j ..
+// 8j+7 of the slice's l-th row, padded with a sentinel to the slice's longest row.  A wave takes one slice: every
+// load is one 1 KB run of 16 bytes per lane, no per-row offsets, no cross-lane reduction.  A flip is 16 bits:
+//     [4:0]  bit inside a 32-bit piece of the input row        [15:5]  2 * (column / 32) + b
+// where b is the BASE bit at that column: the kernel keeps the pieces of the member's input row interleaved with
+// their complements in LDS (piece, ~piece, piece, ~piece ...: 4Kw dwords, then one zero dword for the sentinel 4Kw),
+// so that the looked-up bit already is x ^ b.  The rows of a slice move through the columns at about the same pace,
+// so at any moment the 64 lanes look into a narrow window of the table: neighbouring dwords, different banks.
+#include <type_traits>
+
 #include "nb_common.hpp"
 
 namespace nb {
@@ -58,18 +62,21 @@ __global__ __launch_bounds__(256) void fl_expand_kernel(uint4 *__restrict__ out,
 // ---- shared product on the matrix cores ---------------------------------------------------------------------------
 // C[m, n] = popcount(A_m ^ B_n) = (K - dot(+-1 codes)) / 2 with v_mfma_scale_f32_16x16x128_f8f6f4 on FP4 codes at
 // unit scales (exact: +-1 and 0 are E2M1 values, the fp32 sums are integers below 2^24).  A workgroup of four waves
-// owns a 128 x 128 tile (a wave 64 x 64 = 4 x 4 MFMA tiles); a step stages 128 positions (64 bytes) of the tile's
-// 128 + 128 rows in LDS (rows 80 bytes apart: the 16 rows of a fragment read land in different banks) while the
-// previous step's fragments are multiplied; one barrier per step.  Fragment layout: lane l supplies row l % 16 and
+// owns a 128 x 128 tile (a wave 64 x 64 = 4 x 4 MFMA tiles: 8 KB of fragment reads per 16 products; eight waves of
+// 64 x 32 measured slower, 37.6 against 31.4 us at 4096 x 1024 x 8192, the LDS traffic per product grows); a step
+// stages 128 positions (64 bytes) of the tile's 128 + 128 rows in LDS (rows 80 bytes apart: the 16 rows of a fragment
+// read land in different banks) while the previous step's fragments are multiplied; one barrier per step.  Fragment layout: lane l supplies row l % 16 and
 // the 32 positions of 16-byte piece l / 16 (any assignment works as long as both operands use the same one);
 // acc[r] is C[4 * (l / 16) + r][l % 16].
 constexpr int kGemmTile = 128, kGemmStepBytes = 64, kGemmLd = kGemmStepBytes + 16;
 constexpr int kGemmBufBytes = 2 * kGemmTile * kGemmLd;  // both operands of one step
+constexpr int kGemmAhead = 4;                           // steps whose bytes are in flight, held in registers
 
 __global__ __launch_bounds__(256) void fl_gemm_fp4_kernel(int32_t *__restrict__ C, const uint8_t *__restrict__ A,
                                                           const uint8_t *__restrict__ B, int64_t M, int64_t N,
                                                           int rowbytes, int kbits, int mtiles, int ntiles)
 {
+    constexpr int P = kGemmAhead;
     __shared__ __align__(16) uint8_t lds[2 * kGemmBufBytes];
     // workgroup b runs on XCD b % 8: give each XCD a contiguous run of tiles (neighbours share their A rows in L2)
     const int T = mtiles * ntiles, per = (T + 7) / 8;
@@ -90,28 +97,30 @@ __global__ __launch_bounds__(256) void fl_gemm_fp4_kernel(int32_t *__restrict__ 
 #pragma unroll
         for (int j = 0; j < 4; j++) acc[i][j] = fl_v4f{0.f, 0.f, 0.f, 0.f};
     const int steps = rowbytes / kGemmStepBytes;
-    uint4 ra[2], rb[2];
-    ra[0] = *reinterpret_cast<const uint4 *>(ga);
-    ra[1] = *reinterpret_cast<const uint4 *>(ga + 16);
-    rb[0] = *reinterpret_cast<const uint4 *>(gb);
-    rb[1] = *reinterpret_cast<const uint4 *>(gb + 16);
-    {
-        uint8_t *w = lds + st_off;
-        *reinterpret_cast<uint4 *>(w) = ra[0];
-        *reinterpret_cast<uint4 *>(w + 16) = ra[1];
-        *reinterpret_cast<uint4 *>(w + kGemmTile * kGemmLd) = rb[0];
-        *reinterpret_cast<uint4 *>(w + kGemmTile * kGemmLd + 16) = rb[1];
-    }
-    __syncthreads();
-    for (int s = 0; s < steps; s++) {
-        // the next step's bytes are requested before this step's products (the last step asks for its own again, so
-        // that every step issues the same loads)
-        const int nx = (s + 1 < steps ? s + 1 : s) * kGemmStepBytes;
-        ra[0] = *reinterpret_cast<const uint4 *>(ga + nx);
-        ra[1] = *reinterpret_cast<const uint4 *>(ga + nx + 16);
-        rb[0] = *reinterpret_cast<const uint4 *>(gb + nx);
-        rb[1] = *reinterpret_cast<const uint4 *>(gb + nx + 16);
-        const uint8_t *buf = lds + (s & 1) * kGemmBufBytes;
+    // Register sets: a set holds the bytes of a step that is still to come.  Memory latency is several steps long and
+    // a CU runs one workgroup, so four steps are kept in flight; a step past the end asks for the last one again (every
+    // step issues the same loads, which keeps the wait counts exact).  The sets are separate named variables: indexing
+    // an array of sets, even by a constant that only appears after inlining, sends them to scratch memory.
+    static_assert(kGemmAhead == 4, "the step sequence below is written for four register sets");
+    uint4 a0x, a0y, b0x, b0y, a1x, a1y, b1x, b1y, a2x, a2y, b2x, b2y, a3x, a3y, b3x, b3y;
+#define NB_GEMM_REQUEST(ax, ay, bx, by, step)                                        \
+    do {                                                                             \
+        const int nx_ = ((step) < steps ? (step) : steps - 1) * kGemmStepBytes;      \
+        ax = *reinterpret_cast<const uint4 *>(ga + nx_);                             \
+        ay = *reinterpret_cast<const uint4 *>(ga + nx_ + 16);                        \
+        bx = *reinterpret_cast<const uint4 *>(gb + nx_);                             \
+        by = *reinterpret_cast<const uint4 *>(gb + nx_ + 16);                        \
+    } while (0)
+#define NB_GEMM_STAGE(ax, ay, bx, by, bufno)                                         \
+    do {                                                                             \
+        uint8_t *w_ = lds + (bufno) * kGemmBufBytes + st_off;                        \
+        *reinterpret_cast<uint4 *>(w_) = ax;                                         \
+        *reinterpret_cast<uint4 *>(w_ + 16) = ay;                                    \
+        *reinterpret_cast<uint4 *>(w_ + kGemmTile * kGemmLd) = bx;                   \
+        *reinterpret_cast<uint4 *>(w_ + kGemmTile * kGemmLd + 16) = by;              \
+    } while (0)
+    auto multiply = [&](int cur) {
+        const uint8_t *buf = lds + (cur & 1) * kGemmBufBytes;
         fl_v4i fa[4], fb[4];
 #pragma unroll
         for (int i = 0; i < 4; i++) fa[i] = *reinterpret_cast<const fl_v4i *>(buf + fa_off + i * 16 * kGemmLd);
@@ -127,13 +136,37 @@ __global__ __launch_bounds__(256) void fl_gemm_fp4_kernel(int32_t *__restrict__ 
                                                                              0x7F7F7F7F);
             }
         }
-        uint8_t *w = lds + ((s + 1) & 1) * kGemmBufBytes + st_off;
-        *reinterpret_cast<uint4 *>(w) = ra[0];
-        *reinterpret_cast<uint4 *>(w + 16) = ra[1];
-        *reinterpret_cast<uint4 *>(w + kGemmTile * kGemmLd) = rb[0];
-        *reinterpret_cast<uint4 *>(w + kGemmTile * kGemmLd + 16) = rb[1];
-        __syncthreads();
+    };
+    // One step: the set that holds step cur + 1 goes to the buffer that step cur - 1 has left (every wave passed the
+    // barrier that ended it) and is asked for step cur + 5; then the products of step cur; then the barrier.
+#define NB_GEMM_STEP(ax, ay, bx, by, cur)                        \
+    do {                                                         \
+        NB_GEMM_STAGE(ax, ay, bx, by, ((cur) + 1) & 1);          \
+        NB_GEMM_REQUEST(ax, ay, bx, by, (cur) + 1 + kGemmAhead); \
+        __builtin_amdgcn_sched_barrier(0);                       \
+        multiply(cur);                                           \
+        __syncthreads();                                         \
+    } while (0)
+    NB_GEMM_REQUEST(a0x, a0y, b0x, b0y, 0);
+    NB_GEMM_REQUEST(a1x, a1y, b1x, b1y, 1);
+    NB_GEMM_REQUEST(a2x, a2y, b2x, b2y, 2);
+    NB_GEMM_REQUEST(a3x, a3y, b3x, b3y, 3);
+    NB_GEMM_STAGE(a0x, a0y, b0x, b0y, 0);
+    NB_GEMM_REQUEST(a0x, a0y, b0x, b0y, 4);
+    __syncthreads();
+    int s = 0;
+    for (; s + 4 <= steps; s += 4) {
+        NB_GEMM_STEP(a1x, a1y, b1x, b1y, s);
+        NB_GEMM_STEP(a2x, a2y, b2x, b2y, s + 1);
+        NB_GEMM_STEP(a3x, a3y, b3x, b3y, s + 2);
+        NB_GEMM_STEP(a0x, a0y, b0x, b0y, s + 3);
     }
+    if (s < steps) NB_GEMM_STEP(a1x, a1y, b1x, b1y, s);  // uniform tails
+    if (s + 1 < steps) NB_GEMM_STEP(a2x, a2y, b2x, b2y, s + 1);
+    if (s + 2 < steps) NB_GEMM_STEP(a3x, a3y, b3x, b3y, s + 2);
+#undef NB_GEMM_STEP
+#undef NB_GEMM_STAGE
+#undef NB_GEMM_REQUEST
 #pragma unroll
     for (int i = 0; i < 4; i++)
 #pragma unroll
@@ -183,8 +216,9 @@ __global__ __launch_bounds__(256) void fl_fill_kernel(uint32_t *__restrict__ ent
     const bool valid = p < R;
     int64_t r = valid ? perm[d * R + p] : 0;
     r = r < R ? r : R - 1;
-    const int L = slice_len[sl];
-    uint32_t *dst = entries + slice_off[sl] + lane;
+    const int L = 4 * slice_len[sl];  // dwords per lane; dword j of lane l sits at piece j / 4, component j % 4
+    uint32_t *dst = entries + slice_off[sl] + lane * 4;
+    auto at = [](int j) { return (int64_t)(j >> 2) * 256 + (j & 3); };
     const uint32_t sentinel = (uint32_t)(4 * Kw) << 5;
     int j = 0;
     uint32_t pend = 0;
@@ -199,12 +233,12 @@ __global__ __launch_bounds__(256) void fl_fill_kernel(uint32_t *__restrict__ ent
                 m &= m - 1;
                 const uint32_t col = (uint32_t)k * 64u + (uint32_t)bit;
                 const uint32_t bb = (uint32_t)(bw >> bit) & 1u;
-                const uint32_t e = ((bb * 2u * (uint32_t)Kw + (col >> 5)) << 5) | (col & 31u);
+                const uint32_t e = ((2u * (col >> 5) + bb) << 5) | (col & 31u);
                 if (!half) {
                     pend = e;
                     half = true;
                 } else {
-                    if (j < L) dst[(int64_t)j * 64] = pend | (e << 16);  // never past the slice, whatever the inputs
+                    if (j < L) dst[at(j)] = pend | (e << 16);  // never past the slice, whatever the inputs
                     j++;
                     half = false;
                 }
@@ -212,10 +246,10 @@ __global__ __launch_bounds__(256) void fl_fill_kernel(uint32_t *__restrict__ ent
         }
     }
     if (half) {
-        if (j < L) dst[(int64_t)j * 64] = pend | (sentinel << 16);
+        if (j < L) dst[at(j)] = pend | (sentinel << 16);
         j++;
     }
-    for (; j < L; j++) dst[(int64_t)j * 64] = sentinel | (sentinel << 16);
+    for (; j < L; j++) dst[at(j)] = sentinel | (sentinel << 16);
 }
 
 // ---- the members' corrections, threshold and pack --------------------------------------------------------------------
@@ -232,49 +266,67 @@ __global__ __launch_bounds__(1024) void fl_bmv_kernel(void *__restrict__ out, co
                                                       const int32_t *__restrict__ thresh, int64_t R, int S, int Kw,
                                                       int blocks_per_member)
 {
-    extern __shared__ uint32_t fl_tab[];  // x, ~x, one zero dword, then the block's bit array
+    extern __shared__ uint32_t fl_tab[];  // x and ~x interleaved, one zero dword, then the block's bit array
+    constexpr int U = 4;                  // 16-byte pieces of a lane's list requested together
     const int64_t d = blockIdx.x / blocks_per_member;
     const int blk = (int)(blockIdx.x - d * blocks_per_member);
     const int nd = 2 * Kw;
+    const int lane = threadIdx.x & 63;
+    const int s = blk * (kFlipBlockRows / 64) + (int)(threadIdx.x >> 6);  // wave-uniform
+    const bool active = s < S;
+    const int64_t sl = d * S + (active ? s : S - 1);
+    const int L = active ? __builtin_amdgcn_readfirstlane(slice_len[sl]) : 0;
+    const uint4 *src = reinterpret_cast<const uint4 *>(entries + slice_off[sl]) + lane;
+    // Two register sets take turns: while one batch is looked up, the batch after it is in flight.  Only pieces
+    // that exist are requested (L is wave-uniform, so every such test is a scalar branch).  The first two batches
+    // are requested before anything else: they do not depend on the table.
+    uint4 e0[U], e1[U];
+    auto request = [&](uint4(&e)[U], int j) {
+#pragma unroll
+        for (int u = 0; u < U; u++)
+            if (j + u < L) e[u] = load_stream16(src + (int64_t)(j + u) * 64);
+    };
+    request(e0, 0);
+    request(e1, U);
     for (int i = threadIdx.x; i < nd; i += blockDim.x) {
         const uint32_t v = x32[d * nd + i];
-        fl_tab[i] = v;
-        fl_tab[nd + i] = ~v;
+        fl_tab[2 * i] = v;
+        fl_tab[2 * i + 1] = ~v;
     }
     uint32_t *bitmap = fl_tab + 2 * nd + 1;
     if (threadIdx.x == 0) fl_tab[2 * nd] = 0u;
     if (threadIdx.x < 32) bitmap[threadIdx.x] = 0u;
+    const int64_t p = (int64_t)s * 64 + lane;
+    const bool valid = active && p < R;
+    int64_t r = perm[d * R + (valid ? p : R - 1)];
+    r = r < R ? r : R - 1;
+    const int n = cnt[d * R + r];
+    const int g = G[d * R + r];
+    const int t = PACK ? thresh[d * R + r] : 0;
     __syncthreads();
-    const int lane = threadIdx.x & 63;
-    const int s = blk * (kFlipBlockRows / 64) + (int)(threadIdx.x >> 6);  // wave-uniform
-    if (s < S) {
-        const int64_t p = (int64_t)s * 64 + lane;
-        const bool valid = p < R;
-        int64_t r = perm[d * R + (valid ? p : R - 1)];
-        r = r < R ? r : R - 1;
-        const int64_t sl = d * S + s;
-        const int L = slice_len[sl];
-        const uint32_t *src = entries + slice_off[sl] + lane;
-        const int n = cnt[d * R + r];
-        const int g = G[d * R + r];
-        const int t = PACK ? thresh[d * R + r] : 0;
-        int sy = 0;
-        auto take = [&](uint32_t e) {
-            const uint32_t w0 = fl_tab[(e >> 5) & 0x7FFu];
-            const uint32_t w1 = fl_tab[e >> 21];
-            sy += (int)((w0 >> (e & 31u)) & 1u) + (int)((w1 >> ((e >> 16) & 31u)) & 1u);
-        };
-        constexpr int U = 8;
-        int j = 0;
-        for (; j + U <= L; j += U) {
-            uint32_t e[U];
+    int sy = 0;
+    auto take = [&](uint32_t e) {
+        const uint32_t w0 = fl_tab[(e >> 5) & 0x7FFu];
+        const uint32_t w1 = fl_tab[e >> 21];
+        sy += (int)((w0 >> (e & 31u)) & 1u) + (int)((w1 >> ((e >> 16) & 31u)) & 1u);
+    };
+    auto look_up = [&](const uint4(&e)[U], int j) {
 #pragma unroll
-            for (int u = 0; u < U; u++) e[u] = load_stream4(src + (int64_t)(j + u) * 64);
-            __builtin_amdgcn_sched_barrier(0);  // all loads of the step in flight before the first look-up
-#pragma unroll
-            for (int u = 0; u < U; u++) take(e[u]);
-        }
-        for (; j < L; j++) take(load_stream4(src + (int64_t)j * 64));
+        for (int u = 0; u < U; u++)
+            if (j + u < L) {
+                take(e[u].x);
+                take(e[u].y);
+                take(e[u].z);
+                take(e[u].w);
+            }
+    };
+    for (int j = 0; j < L; j += 2 * U) {
+        look_up(e0, j);
+        request(e0, j + 2 * U);
+        look_up(e1, j + U);
+        request(e1, j + 3 * U);
+    }
+    if (active) {
         const int sum = g + n - 2 * sy;
         if (PACK) {
             const int local = (int)(r - (int64_t)blk * kFlipBlockRows);
@@ -382,7 +434,7 @@ int nb_flip_fill_i64(uint32_t *entries, const int64_t *W, const int64_t *base, c
     NB_REQUIRE_PTR(perm);
     NB_REQUIRE_PTR(slice_off);
     NB_REQUIRE_PTR(slice_len);
-    NB_REQUIRE_ALIGNED(entries, 4);
+    NB_REQUIRE_ALIGNED(entries, 16);
     NB_REQUIRE_ALIGNED(perm, 2);
     NB_REQUIRE_ALIGNED(slice_off, 8);
     NB_REQUIRE_ALIGNED(slice_len, 4);
@@ -417,7 +469,7 @@ static int flip_bmv(void *out, const int32_t *G, const uint32_t *entries, const 
     if (Kw > 0) NB_REQUIRE_PTR(x);
     NB_REQUIRE_ALIGNED(out, pack ? 8 : 4);
     NB_REQUIRE_ALIGNED(G, 4);
-    NB_REQUIRE_ALIGNED(entries, 4);
+    NB_REQUIRE_ALIGNED(entries, 16);
     NB_REQUIRE_ALIGNED(slice_off, 8);
     NB_REQUIRE_ALIGNED(slice_len, 4);
     NB_REQUIRE_ALIGNED(perm, 2);

@@ -667,12 +667,12 @@ def flip_rows_from_weights(W, base):
     order = torch.sort(cp, dim=2, stable=True).indices + (torch.arange(nblk, device=dev) * 1024).view(1, nblk, 1)
     order = order.view(D, nblk * 1024)[:, :R].contiguous()                       # padding sorts last in its block
     cs = torch.nn.functional.pad(c.gather(1, order), (0, S * 64 - R)).view(D, S, 64)
-    slice_len = ((cs.max(dim=2).values + 1) // 2).to(torch.int32).contiguous()  # dwords (two flips) per lane
-    lens = slice_len.view(-1).to(torch.int64) * 64
+    slice_len = ((cs.max(dim=2).values + 7) // 8).to(torch.int32).contiguous()  # 16-byte pieces (8 flips) per lane
+    lens = slice_len.view(-1).to(torch.int64) * 256                              # dwords of a slice
     slice_off = (torch.cumsum(lens, 0) - lens).view(D, S).contiguous()
     total = int(lens.sum().item()) if D * S else 0
     perm = order.to(torch.uint16).contiguous()
-    entries = torch.empty((max(total, 1),), dtype=torch.uint32, device=dev)
+    entries = torch.empty((max(total, 4),), dtype=torch.uint32, device=dev)
     with _on(W):
         _lib.call("nb_flip_fill_i64", entries.data_ptr(), W.data_ptr(), base.data_ptr(), perm.data_ptr(),
                   slice_off.data_ptr(), slice_len.data_ptr(), D, R, Kw, _stream(W))

@@ -79,9 +79,10 @@ def decode_flip_rows(rows):
     sentinel = (4 * Kw) << 5
     for d in range(D):
         for s in range(S):
-            L = int(ln[d, s])
-            blk = ent[off[d, s]: off[d, s] + L * 64].reshape(L, 64)
-            halves = np.stack([blk & 0xFFFF, blk >> 16], axis=1).reshape(2 * L, 64)     # flips in order, per lane
+            L = int(ln[d, s])                                                            # 16-byte pieces per lane
+            assert off[d, s] % 4 == 0
+            blk = ent[off[d, s]: off[d, s] + L * 256].reshape(L, 64, 4).transpose(0, 2, 1).reshape(4 * L, 64)
+            halves = np.stack([blk & 0xFFFF, blk >> 16], axis=1).reshape(8 * L, 64)     # flips in order, per lane
             for lane in range(64):
                 p = s * 64 + lane
                 col_prev, ended = -1, False
@@ -92,8 +93,9 @@ def decode_flip_rows(rows):
                         continue
                     assert not ended and p < R, "a flip after the sentinel / in a lane without a row"
                     piece, bit = e >> 5, e & 31
-                    b = piece >= 2 * Kw
-                    col = (piece - 2 * Kw * b) * 32 + bit
+                    assert piece < 4 * Kw
+                    b = bool(piece & 1)
+                    col = (piece >> 1) * 32 + bit
                     assert col > col_prev                                                # column order
                     col_prev = col
                     mask[d, perm[d, p], col] = True
@@ -121,7 +123,7 @@ def test_flip_rows_hold_exactly_the_flipped_bits(ops, D, R, C, p):
             assert (np.diff(cnt[d, perm[d, b0:b0 + 1024]]) >= 0).all()                         # ordered by flip count
     S = (R + 63) // 64
     cs = np.pad(np.take_along_axis(cnt, perm, axis=1), ((0, 0), (0, S * 64 - R))).reshape(D, S, 64)
-    np.testing.assert_array_equal(host(rows.slice_len), (cs.max(axis=2) + 1) // 2)
+    np.testing.assert_array_equal(host(rows.slice_len), (cs.max(axis=2) + 7) // 8)
     mask, bflag = decode_flip_rows(rows)
     np.testing.assert_array_equal(mask, want_bits)
     base_bits = np.unpackbits(base.view(np.uint8), axis=1, bitorder="little").astype(bool)
