@@ -97,10 +97,15 @@ def load():
     return lib
 
 
+_fns = {}
+
+
 def call(name, *args):
     """Call an entry point and turn a non-zero status into RuntimeError."""
-    lib = load()
-    rc = getattr(lib, name)(*args)
+    fn = _fns.get(name)
+    if fn is None:
+        fn = _fns[name] = getattr(load(), name)
+    rc = fn(*args)
     if rc != NB_OK:
-        msg = lib.nb_last_error_string().decode("utf-8", "replace")
+        msg = load().nb_last_error_string().decode("utf-8", "replace")
         raise RuntimeError("%s failed with status %d: %s" % (name, rc, msg))

@@ -63,6 +63,51 @@ __global__ __launch_bounds__(BS) void bmv_kernel(int32_t *__restrict__ C, const 
     }
 }
 
+// Matrix-vector form for short rows (16, 32 or 64 bytes: VPR 16-byte vectors): a lane owns whole rows, so there is no
+// cross-lane reduction at all.  A wave takes Q runs of 64 consecutive rows (every load instruction reads one
+// contiguous run of 64 rows), all Q * VPR streaming loads of a lane are requested before the first use, and the
+// member's input vector (the same few bytes for all lanes of a run, or two neighbouring ones) comes through the cache.
+template <int VPR, int Q>
+__global__ __launch_bounds__(256) void bmv_short_kernel(int32_t *__restrict__ C, const uint4 *__restrict__ A,
+                                                        const uint4 *__restrict__ X, uint32_t rows, uint32_t M)
+{
+    const uint32_t wave_first = (blockIdx.x * 256u + (threadIdx.x & ~63u)) * Q;
+    const uint32_t lane = threadIdx.x & 63u;
+    uint32_t row[Q];
+    uint4 a[Q][VPR], x[Q][VPR];
+#pragma unroll
+    for (int q = 0; q < Q; q++) {
+        row[q] = wave_first + q * 64u + lane;
+        const uint32_t rc = row[q] < rows ? row[q] : rows - 1;  // rows past the end are recomputed, never stored
+#pragma unroll
+        for (int v = 0; v < VPR; v++) a[q][v] = load_stream16(A + (int64_t)rc * VPR + v);
+        const uint32_t z = rc / M;
+#pragma unroll
+        for (int v = 0; v < VPR; v++) x[q][v] = X[(int64_t)z * VPR + v];
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int q = 0; q < Q; q++) {
+        int acc = 0;
+#pragma unroll
+        for (int v = 0; v < VPR; v++) {
+            acc = bcnt_acc(a[q][v].x ^ x[q][v].x, acc);
+            acc = bcnt_acc(a[q][v].y ^ x[q][v].y, acc);
+            acc = bcnt_acc(a[q][v].z ^ x[q][v].z, acc);
+            acc = bcnt_acc(a[q][v].w ^ x[q][v].w, acc);
+        }
+        if (row[q] < rows) C[row[q]] = acc;
+    }
+}
+
+template <int VPR>
+static void launch_bmv_short(int32_t *C, const void *A, const void *X, int64_t rows, int64_t M, hipStream_t s)
+{
+    constexpr int Q = 4;
+    bmv_short_kernel<VPR, Q><<<dim3((unsigned)ceil_div(rows, 256 * Q)), dim3(256), 0, s>>>(
+        C, static_cast<const uint4 *>(A), static_cast<const uint4 *>(X), (uint32_t)rows, (uint32_t)M);
+}
+
 // Matrix-vector form for long rows: L lanes (16, 32 or 64) walk FOUR rows of one member with 16-byte streaming
 // loads, so the input vector is loaded once per step for all four, and the four per-lane sums are reduced by a
 // transposing butterfly: two quad steps halve the rows a lane carries (4 -> 2 -> 1) while they add, then two
@@ -264,7 +309,12 @@ int bmm_impl(int32_t *C, const W *A, const W *B, int64_t Z, int64_t M, int64_t K
         NB_REQUIRE(ceil_div(ceil_div(rows, 4) * 64, 256) <= kMaxGridX, "%s: %lld rows exceed one launch", who,
                    (long long)rows);
         const int64_t rowbytes = Kw * (int64_t)sizeof(W);
-        if (rowbytes % 16 == 0 && rowbytes >= 256 && M % 4 == 0 && aligned(A, 16) && aligned(B, 16)) {
+        if ((rowbytes == 16 || rowbytes == 32 || rowbytes == 64) && rows < (1LL << 31) && aligned(A, 16) &&
+            aligned(B, 16)) {
+            if (rowbytes == 16) launch_bmv_short<1>(C, A, B, rows, M, s);
+            else if (rowbytes == 32) launch_bmv_short<2>(C, A, B, rows, M, s);
+            else launch_bmv_short<4>(C, A, B, rows, M, s);
+        } else if (rowbytes % 16 == 0 && rowbytes >= 256 && M % 4 == 0 && aligned(A, 16) && aligned(B, 16)) {
             const int rowvecs = (int)(rowbytes / 16);
             // as many row steps in flight as divide the row (up to 16 loads of 16 bytes per lane), fewest lanes per row
             if (rowvecs % 256 == 0) launch_bmv_quad<64, 4>(C, A, B, rows, M, rowvecs, s);

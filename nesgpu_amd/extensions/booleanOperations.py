@@ -68,7 +68,15 @@ def _same_device(a, b):
         raise RuntimeError("Tensors are on different devices")       # booleanOperations.cpp:39
 
 
+# The current stream's handle and the current device index straight from torch's C layer: the public wrappers build a
+# Stream object / re-check initialisation on every call, which costs more than the rest of an op's host work together.
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_raw_device = getattr(torch._C, "_cuda_getDevice", None)
+
+
 def _stream(t):
+    if _raw_stream is not None:
+        return _raw_stream(t.device.index)
     return torch.cuda.current_stream(t.device).cuda_stream
 
 
@@ -88,7 +96,8 @@ _HERE = _Here()
 
 def _on(t):
     """Context that makes ``t``'s device current for the launch."""
-    return _HERE if t.device.index == torch.cuda.current_device() else torch.cuda.device(t.device)
+    cur = _raw_device() if _raw_device is not None else torch.cuda.current_device()
+    return _HERE if t.device.index == cur else torch.cuda.device(t.device)
 
 
 def _out_hw(inp, filterx, filtery, padx, pady, stridex, stridey):
@@ -115,19 +124,19 @@ def batch_im2col(input, filterx, filtery, padx, pady, stridex, stridey, REPEAT=1
 
 def bmm(A, B):
     """C[z,x,y] = sum_k popcount(A[z,x,k] ^ B[z,k,y]), int32 (extensions/booleanOperations.py:107-129)."""
-    assert len(A.shape) == 3
-    assert len(B.shape) == 3
-    assert A.size(0) == B.size(0)
-    assert A.size(2) == B.size(1)
+    sa, sb = A.shape, B.shape
+    assert len(sa) == 3
+    assert len(sb) == 3
+    assert sa[0] == sb[0]
+    assert sa[2] == sb[1]
     _check(A, "A")
     _check(B, "B")
     _same_device(A, B)
     assert A.dtype == B.dtype
     suf, _ = _suffix(A.dtype)
-    C = torch.empty((A.size(0), A.size(1), B.size(2)), dtype=torch.int32, device=A.device)
+    C = torch.empty((sa[0], sa[1], sb[2]), dtype=torch.int32, device=A.device)
     with _on(A):
-        _lib.call("nb_bmm" + suf, C.data_ptr(), A.data_ptr(), B.data_ptr(), A.size(0), A.size(1), A.size(2), B.size(2),
-                  _stream(A))
+        _lib.call("nb_bmm" + suf, C.data_ptr(), A.data_ptr(), B.data_ptr(), sa[0], sa[1], sa[2], sb[2], _stream(A))
     return C
 
 

@@ -165,7 +165,10 @@ def test_int8pack_vs_oracle(ops, oracle, dtype):
 LINEAR_SHAPES = [(8, 256, 4), (5, 10, 16), (3, 1000, 128), (7, 33, 9), (4, 64, 1), (2, 3, 200), (9, 1, 2), (1, 5, 31),
                  (6, 130, 6),
                  # four-rows-per-group kernel: 16, 32 and 64 lanes per row, rows that are not a multiple of the lane count
-                 (5, 12, 32), (2, 8, 200), (3, 4, 66), (2, 20, 34), (1, 4, 512), (300, 8, 64)]
+                 (5, 12, 32), (2, 8, 200), (3, 4, 66), (2, 20, 34), (1, 4, 512), (300, 8, 64),
+                 # row-per-lane kernel for rows of 16, 32 or 64 bytes: members that do not fill a run of 64 rows, a ragged
+                 # last workgroup, one row
+                 (1000, 3, 8), (7, 300, 2), (3, 1025, 4), (1, 1, 8), (600, 5, 4), (2, 2048, 16)]
 
 
 @pytest.mark.parametrize("dtype", [torch.int64, torch.int32])
