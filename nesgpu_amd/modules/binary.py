@@ -33,18 +33,24 @@ class AsType(nn.Module):
 
 
 class ExtractBits(nn.Module):
-    """Expands every integer into its bits, LSB first, along the last axis (modules/binary.py:20-29)."""
+    """Expands every integer into its bits, LSB first, along the last axis (modules/binary.py:20-29).
 
-    def __init__(self, dtype):
+    As in the reference, a bit counts as set when ``(value & mask) > 0``; for a SIGNED dtype the top mask is the
+    (negative) sign bit, so that position is always False there (for torch.uint8, what image bytes come as, all eight
+    bits are extracted).  ``sign_bit=True`` (not in the reference) extracts the sign bit of signed types as well."""
+
+    def __init__(self, dtype, sign_bit=False):
         nn.Module.__init__(self)
         self.dtype = dtype
         self.bitlength = torch.iinfo(dtype).bits
+        self.sign_bit = sign_bit
         # 1 << i; the top bit of a signed type is the sign bit, built by shifting rather than 2 ** i
         self.mask = torch.ones(self.bitlength, dtype=dtype) << torch.arange(self.bitlength, dtype=dtype)
 
     def forward(self, input):
         mask = self.mask.to(input.device)
-        return ((input.unsqueeze(-1) & mask) != 0).view(*input.shape[:-1], -1)
+        hit = input.unsqueeze(-1) & mask
+        return ((hit != 0) if self.sign_bit else (hit > 0)).view(*input.shape[:-1], -1)
 
 
 class Binarized(Perturbed, nn.Module):

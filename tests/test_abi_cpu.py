@@ -112,4 +112,9 @@ def test_layer_construction_and_lifecycle_on_cpu():
     eb = binary.ExtractBits(torch.int64)
     v = torch.tensor([[5, -1]], dtype=torch.int64)
     bits = eb(v)
-    assert bits.shape == (1, 128) and bits[0, :3].tolist() == [True, False, True] and bits[0, 64:].all()
+    assert bits.shape == (1, 128) and bits[0, :3].tolist() == [True, False, True]
+    # (value & mask) > 0 as in the reference (modules/binary.py:29): the sign bit of a signed type never counts
+    assert bits[0, 64:127].all() and not bits[0, 127]
+    assert binary.ExtractBits(torch.int64, sign_bit=True)(v)[0, 64:].all()
+    u8 = binary.ExtractBits(torch.uint8)(torch.tensor([[0x81, 0xFF]], dtype=torch.uint8))
+    assert u8.shape == (1, 16) and u8[0].tolist() == [True] + [False] * 6 + [True] + [True] * 8
