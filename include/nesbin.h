@@ -260,6 +260,23 @@ int nb_sample_philox_i32(int32_t *out, const int32_t *base, const uint32_t *thre
                          nb_stream_t stream);
 int nb_philox_words(uint32_t *out, uint64_t seed, uint64_t subseq, uint64_t first, int64_t count,
                     nb_stream_t stream);
+/* The same samplers for a conv layer's filters: the R = O * KK rows are (out channel o, tap t) pairs, r = o * KK + t
+ * (the layer's weight is [O*kx*ky, C], modules/binary.py:125), and the kernel writes every sampled word ALSO (or
+ * only, when out_rows is NULL) where the conv multiplies it: out_conv [n, KK * Rw, O] with word wi of row (o, t) at
+ * [m][t * Rw + wi][o], Rw = ceil(C/bits).  One pass instead of sample -> view -> permute(0,2,3,4,1) -> contiguous
+ * (modules/binary.py:134-137); out_rows keeps the [n, R, Rw] layout that the update step sums over. */
+int nb_sample_conv_from_words_i64(int64_t *out_conv, int64_t *out_rows, const int64_t *base, const uint32_t *thresh,
+                                  uint32_t thr_scalar, const uint32_t *words, int64_t n, int64_t O, int64_t KK,
+                                  int64_t C, nb_stream_t stream);
+int nb_sample_conv_from_words_i32(int32_t *out_conv, int32_t *out_rows, const int32_t *base, const uint32_t *thresh,
+                                  uint32_t thr_scalar, const uint32_t *words, int64_t n, int64_t O, int64_t KK,
+                                  int64_t C, nb_stream_t stream);
+int nb_sample_conv_philox_i64(int64_t *out_conv, int64_t *out_rows, const int64_t *base, const uint32_t *thresh,
+                              uint32_t thr_scalar, uint64_t seed, uint64_t subseq, uint64_t first, int64_t n, int64_t O,
+                              int64_t KK, int64_t C, nb_stream_t stream);
+int nb_sample_conv_philox_i32(int32_t *out_conv, int32_t *out_rows, const int32_t *base, const uint32_t *thresh,
+                              uint32_t thr_scalar, uint64_t seed, uint64_t subseq, uint64_t first, int64_t n, int64_t O,
+                              int64_t KK, int64_t C, nb_stream_t stream);
 
 /* ---- fused sample + XOR-popcount matrix-vector product -------------------------------------------
  * C[m,r] = sum_k popcount(w(m,r,k) ^ x[m,k]) where w is what nb_sample_* would have written;

@@ -55,11 +55,24 @@ __device__ __forceinline__ uint32_t nibble_lt(uint4 w, uint4 t)
 // the base word of a quad are fetched once and reused for the U members, whose stream loads (U independent
 // 16-byte non-temporal loads per lane, 16 KiB contiguous per member and workgroup) are all issued before
 // the first use.
+// Second, optional output in the layout a conv layer multiplies with (modules/binary.py:134-137): the rows are
+// (out channel o, tap t) pairs, r = o * KK + t, and word wi of row r goes to out2[m][(t * Rw + wi) * O + o].
+template <typename W>
+struct ConvOut {
+    W *__restrict__ out2;
+    uint32_t KK, O;
+    __device__ __forceinline__ int64_t at(uint32_t r, uint32_t wi, uint32_t Rw) const
+    {
+        const uint32_t o = r / KK, t = r - o * KK;
+        return (int64_t)(t * Rw + wi) * O + o;
+    }
+};
+
 template <typename W, class Src, int U, int BS, bool HAS_THR, bool HAS_BASE>
 __global__ __launch_bounds__(BS) void sample_wide_kernel(W *__restrict__ out, const W *__restrict__ base,
                                                          const uint32_t *__restrict__ thresh, uint32_t ts, Src src,
                                                          int64_t n, uint32_t RC4, uint32_t plane_tiles,
-                                                         int64_t total_blocks)
+                                                         int64_t total_blocks, ConvOut<W> conv, uint32_t Rw)
 {
     constexpr int bits = WordTraits<W>::bits;
     constexpr int G = bits / 4;      // lanes per output word
@@ -96,7 +109,13 @@ __global__ __launch_bounds__(BS) void sample_wide_kernel(W *__restrict__ out, co
             const int u = i / WPB, wi = i - u * WPB;
             const int64_t m = mg * U + u;
             const uint32_t pw = pt * WPB + wi;  // word inside the plane; C % bits == 0: words never straddle rows
-            if (m < n && pw < RC4 / G) __builtin_nontemporal_store(stage[i], out + m * (RC4 / G) + pw);
+            if (m < n && pw < RC4 / G) {
+                if (out) __builtin_nontemporal_store(stage[i], out + m * (RC4 / G) + pw);
+                if (conv.out2) {
+                    const uint32_t r = pw / Rw;
+                    conv.out2[m * (RC4 / G) + conv.at(r, pw - r * Rw, Rw)] = stage[i];
+                }
+            }
         }
     }
 }
@@ -105,7 +124,7 @@ __global__ __launch_bounds__(BS) void sample_wide_kernel(W *__restrict__ out, co
 template <typename W, class Src>
 __global__ __launch_bounds__(256) void sample_ballot_kernel(W *__restrict__ out, const W *__restrict__ base,
                                                             const uint32_t *__restrict__ thresh, uint32_t ts, Src src,
-                                                            int64_t nrows, int64_t R, int C, int Rw)
+                                                            int64_t nrows, int64_t R, int C, int Rw, ConvOut<W> conv)
 {
     constexpr int bits = WordTraits<W>::bits;
     const int lane = threadIdx.x & 63;
@@ -121,13 +140,17 @@ __global__ __launch_bounds__(256) void sample_ballot_kernel(W *__restrict__ out,
             }
             const uint64_t m = __ballot(bit);
             if (lane == 0) {
+                auto put = [&](int wi, W v) {
+                    v ^= base ? base[r * Rw + wi] : (W)0;
+                    if (out) out[row * Rw + wi] = v;
+                    if (conv.out2) conv.out2[(row / R) * (R * Rw) + conv.at((uint32_t)r, (uint32_t)wi, (uint32_t)Rw)] = v;
+                };
                 if (bits == 64) {
-                    const int wi = c0 >> 6;
-                    out[row * Rw + wi] = (W)m ^ (base ? base[r * Rw + wi] : (W)0);
+                    put(c0 >> 6, (W)m);
                 } else {
                     const int wi = c0 >> 5;
-                    out[row * Rw + wi] = (W)m ^ (base ? base[r * Rw + wi] : (W)0);
-                    if (wi + 1 < Rw) out[row * Rw + wi + 1] = (W)(m >> 32) ^ (base ? base[r * Rw + wi + 1] : (W)0);
+                    put(wi, (W)m);
+                    if (wi + 1 < Rw) put(wi + 1, (W)(m >> 32));
                 }
             }
         }
@@ -337,13 +360,17 @@ static int sample_check(const void *out, const W *base, const uint32_t *thresh, 
 
 template <typename W, class Src>
 int sample_impl(W *out, const W *base, const uint32_t *thresh, uint32_t ts, Src src, bool src_vec_ok, int64_t n,
-                int64_t R, int64_t C, nb_stream_t stream, const char *who)
+                int64_t R, int64_t C, nb_stream_t stream, const char *who, W *out_conv = nullptr, int64_t KK = 1)
 {
     constexpr int bits = WordTraits<W>::bits;
     bool empty;
-    if (int rc = sample_check<W>(out, base, thresh, n, R, C, who, &empty)) return rc;
+    if (int rc = sample_check<W>(out ? out : out_conv, base, thresh, n, R, C, who, &empty)) return rc;
     if (empty) return NB_OK;
     NB_REQUIRE_ALIGNED(out, sizeof(W));
+    NB_REQUIRE_ALIGNED(out_conv, sizeof(W));
+    NB_REQUIRE(KK >= 1 && R % KK == 0 && R < (1LL << 31), "%s: %lld rows are not whole groups of %lld taps", who,
+               (long long)R, (long long)KK);
+    const ConvOut<W> conv{out_conv, (uint32_t)KK, (uint32_t)(R / KK)};
     hipStream_t s = as_stream(stream);
     const int64_t Rw = ceil_div(C, bits);
     if (C % bits == 0 && src_vec_ok && (!thresh || aligned(thresh, 16)) &&
@@ -355,7 +382,7 @@ int sample_impl(W *out, const W *base, const uint32_t *thresh, uint32_t ts, Src 
         const dim3 grid((unsigned)(total_blocks < kMaxBlocks ? total_blocks : kMaxBlocks)), block(BS);
 #define NB_LAUNCH_WIDE(T, B)                                                                                   \
     sample_wide_kernel<W, Src, U, BS, T, B><<<grid, block, 0, s>>>(out, base, thresh, ts, src, n, rc4, plane_tiles, \
-                                                                   total_blocks)
+                                                                   total_blocks, conv, (uint32_t)Rw)
         if (thresh && base) NB_LAUNCH_WIDE(true, true);
         else if (thresh) NB_LAUNCH_WIDE(true, false);
         else if (base) NB_LAUNCH_WIDE(false, true);
@@ -363,7 +390,7 @@ int sample_impl(W *out, const W *base, const uint32_t *thresh, uint32_t ts, Src 
 #undef NB_LAUNCH_WIDE
     } else {
         sample_ballot_kernel<W, Src><<<dim3(grid_for(n * R * 64)), dim3(256), 0, s>>>(
-            out, base, thresh, ts, src, n * R, R, (int)C, (int)Rw);
+            out, base, thresh, ts, src, n * R, R, (int)C, (int)Rw, conv);
     }
     return check_launch(who);
 }
@@ -446,6 +473,52 @@ int nb_sample_philox_i32(int32_t *out, const int32_t *base, const uint32_t *thre
 {
     return nb::sample_impl<uint32_t, PhiloxSrc>(U32(out), CU32(base), thresh, ts, PhiloxSrc{{seed, subseq, first}},
                                                 (first & 3) == 0 && (C & 3) == 0, n, R, C, s, "nb_sample_philox_i32");
+}
+int nb_sample_conv_from_words_i64(int64_t *out_conv, int64_t *out_rows, const int64_t *base, const uint32_t *thresh,
+                                  uint32_t ts, const uint32_t *words, int64_t n, int64_t O, int64_t KK, int64_t C,
+                                  nb_stream_t s)
+{
+    const char *who = "nb_sample_conv_from_words_i64";
+    if (O < 0 || KK < 1) return nb::fail(NB_ERR_SHAPE, "%s: bad shape O=%lld KK=%lld", who, (long long)O, (long long)KK);
+    if (n * O * KK * C > 0 && !words) return nb::fail(NB_ERR_NULL, "%s: words is NULL", who);
+    if (n * O * KK * C > 0 && !out_conv) return nb::fail(NB_ERR_NULL, "%s: out_conv is NULL", who);
+    return nb::sample_impl<uint64_t, WordsSrc>(U64(out_rows), CU64(base), thresh, ts, WordsSrc{words},
+                                               nb::aligned(words, 16) && (C & 3) == 0, n, O * KK, C, s, who,
+                                               U64(out_conv), KK);
+}
+int nb_sample_conv_from_words_i32(int32_t *out_conv, int32_t *out_rows, const int32_t *base, const uint32_t *thresh,
+                                  uint32_t ts, const uint32_t *words, int64_t n, int64_t O, int64_t KK, int64_t C,
+                                  nb_stream_t s)
+{
+    const char *who = "nb_sample_conv_from_words_i32";
+    if (O < 0 || KK < 1) return nb::fail(NB_ERR_SHAPE, "%s: bad shape O=%lld KK=%lld", who, (long long)O, (long long)KK);
+    if (n * O * KK * C > 0 && !words) return nb::fail(NB_ERR_NULL, "%s: words is NULL", who);
+    if (n * O * KK * C > 0 && !out_conv) return nb::fail(NB_ERR_NULL, "%s: out_conv is NULL", who);
+    return nb::sample_impl<uint32_t, WordsSrc>(U32(out_rows), CU32(base), thresh, ts, WordsSrc{words},
+                                               nb::aligned(words, 16) && (C & 3) == 0, n, O * KK, C, s, who,
+                                               U32(out_conv), KK);
+}
+int nb_sample_conv_philox_i64(int64_t *out_conv, int64_t *out_rows, const int64_t *base, const uint32_t *thresh,
+                              uint32_t ts, uint64_t seed, uint64_t subseq, uint64_t first, int64_t n, int64_t O,
+                              int64_t KK, int64_t C, nb_stream_t s)
+{
+    const char *who = "nb_sample_conv_philox_i64";
+    if (O < 0 || KK < 1) return nb::fail(NB_ERR_SHAPE, "%s: bad shape O=%lld KK=%lld", who, (long long)O, (long long)KK);
+    if (n * O * KK * C > 0 && !out_conv) return nb::fail(NB_ERR_NULL, "%s: out_conv is NULL", who);
+    return nb::sample_impl<uint64_t, PhiloxSrc>(U64(out_rows), CU64(base), thresh, ts, PhiloxSrc{{seed, subseq, first}},
+                                                (first & 3) == 0 && (C & 3) == 0, n, O * KK, C, s, who, U64(out_conv),
+                                                KK);
+}
+int nb_sample_conv_philox_i32(int32_t *out_conv, int32_t *out_rows, const int32_t *base, const uint32_t *thresh,
+                              uint32_t ts, uint64_t seed, uint64_t subseq, uint64_t first, int64_t n, int64_t O,
+                              int64_t KK, int64_t C, nb_stream_t s)
+{
+    const char *who = "nb_sample_conv_philox_i32";
+    if (O < 0 || KK < 1) return nb::fail(NB_ERR_SHAPE, "%s: bad shape O=%lld KK=%lld", who, (long long)O, (long long)KK);
+    if (n * O * KK * C > 0 && !out_conv) return nb::fail(NB_ERR_NULL, "%s: out_conv is NULL", who);
+    return nb::sample_impl<uint32_t, PhiloxSrc>(U32(out_rows), CU32(base), thresh, ts, PhiloxSrc{{seed, subseq, first}},
+                                                (first & 3) == 0 && (C & 3) == 0, n, O * KK, C, s, who, U32(out_conv),
+                                                KK);
 }
 int nb_philox_words(uint32_t *out, uint64_t seed, uint64_t subseq, uint64_t first, int64_t count, nb_stream_t s)
 {

@@ -382,14 +382,15 @@ def int8pack(input, dtype=torch.int32):
     return ret
 
 
-def sample_bits(p, n, dtype, seed):
+def sample_bits(p, n, dtype, seed, conv_taps=None):
     """ret[m,r,z] bit i = Bernoulli(p[r, z*bits+i]), n independent members
     (extensions/booleanOperations.py:203-215, extensions/src/sample_bits.cu:47-57).
 
     Same law, layout and tail rule as the reference; the random stream is Philox4x32-10 keyed by
-    ``seed`` instead of cuRAND XORWOW (whose exact bitstream no reference test pins)."""
+    ``seed`` instead of cuRAND XORWOW (whose exact bitstream no reference test pins).  ``conv_taps`` (not in the
+    reference): see :func:`sample_bits_from_words`; returns ``(rows_layout, conv_layout)``."""
     assert len(p.shape) == 2
-    return sample_bits_philox(thresholds_from_p(p), n, dtype, seed)
+    return sample_bits_philox(thresholds_from_p(p), n, dtype, seed, conv_taps=conv_taps)
 
 
 def weighted_sum(input, weights, zbits):
@@ -479,15 +480,35 @@ def _base_check(base, R, Rw, dtype, device):
     return base.data_ptr()
 
 
-def sample_bits_from_words(threshold, words, dtype, base=None):
+def _conv_outputs(conv_taps, rows_too, n, R, Rw, dtype, device):
+    """-> (conv-layout tensor [n, KK*Rw, O], row-layout tensor [n, R, Rw] or None, O)"""
+    KK = int(conv_taps)
+    assert KK >= 1 and R % KK == 0, "the rows must be (out channel, tap) pairs: R = O * taps"
+    O = R // KK
+    conv = torch.empty((n, KK * Rw, O), dtype=dtype, device=device)
+    rows = torch.empty((n, R, Rw), dtype=dtype, device=device) if rows_too else None
+    return conv, rows, O
+
+
+def sample_bits_from_words(threshold, words, dtype, base=None, conv_taps=None, rows_too=True):
     """ret[m,r,z] bit i = words[m,r,z*bits+i] < threshold[r,z*bits+i]  (threshold: uint32 [R,C] tensor or a
-    Python int); with ``base`` ([R,Rw] packed) the result is ``base ^ mask``."""
+    Python int); with ``base`` ([R,Rw] packed) the result is ``base ^ mask``.
+
+    ``conv_taps`` = kx*ky (not in the reference): the rows are a conv layer's (out channel, tap) pairs and the same
+    kernel also writes the filters where the conv multiplies them, [n, kx*ky*Rw, O] (modules/binary.py:134-137 in
+    the same pass); returns ``(rows_layout, conv_layout)``, the first ``None`` when ``rows_too`` is False."""
     _words_check(words)
     suf, bits = _suffix(dtype)
     n, R, C = words.shape
     keep, tptr, ts = _thr_args(threshold, R, C, words.device)
     Rw = ceil_div(C, bits)
     bptr = _base_check(base, R, Rw, dtype, words.device)
+    if conv_taps is not None:
+        conv, rows, O = _conv_outputs(conv_taps, rows_too, n, R, Rw, dtype, words.device)
+        with _on(words):
+            _lib.call("nb_sample_conv_from_words" + suf, conv.data_ptr(), None if rows is None else rows.data_ptr(), bptr,
+                      tptr, ts, words.data_ptr(), n, O, int(conv_taps), C, _stream(words))
+        return rows, conv
     ret = torch.empty((n, R, Rw), dtype=dtype, device=words.device)
     with _on(words):
         _lib.call("nb_sample_from_words" + suf, ret.data_ptr(), bptr, tptr, ts, words.data_ptr(), n, R, C,
@@ -500,7 +521,8 @@ def flip_from_words(base_packed, words, threshold):
     return sample_bits_from_words(threshold, words, base_packed.dtype, base=base_packed)
 
 
-def sample_bits_philox(threshold, n, dtype, seed, subsequence=0, first=0, base=None, shape=None):
+def sample_bits_philox(threshold, n, dtype, seed, subsequence=0, first=0, base=None, shape=None, conv_taps=None,
+                       rows_too=True):
     """Like :func:`sample_bits_from_words` with the words generated in-kernel: word (m,r,c) is element
     ``first + (m*R+r)*C + c`` of the Philox4x32-10 stream (seed, subsequence) -- exactly what
     :func:`philox_words` returns, so both forms agree bit for bit."""
@@ -514,6 +536,13 @@ def sample_bits_philox(threshold, n, dtype, seed, subsequence=0, first=0, base=N
     keep, tptr, ts = _thr_args(threshold, R, C, device)
     Rw = ceil_div(C, bits)
     bptr = _base_check(base, R, Rw, dtype, device)
+    if conv_taps is not None:
+        conv, rows, O = _conv_outputs(conv_taps, rows_too, n, R, Rw, dtype, device)
+        with torch.cuda.device(device):
+            _lib.call("nb_sample_conv_philox" + suf, conv.data_ptr(), None if rows is None else rows.data_ptr(), bptr,
+                      tptr, ts, int(seed) & (2 ** 64 - 1), int(subsequence), int(first), n, O, int(conv_taps), C,
+                      torch.cuda.current_stream(device).cuda_stream)
+        return rows, conv
     ret = torch.empty((n, R, Rw), dtype=dtype, device=device)
     with torch.cuda.device(device):
         _lib.call("nb_sample_philox" + suf, ret.data_ptr(), bptr, tptr, ts, int(seed) & (2 ** 64 - 1),

@@ -83,6 +83,8 @@ class Binarized(Perturbed, nn.Module):
             norm_weight = self.weight / (self.weight.abs().mean() + 1e-5) * 5
             return torch.sigmoid(norm_weight.float()).half()
 
+    conv_taps = None     # conv layers: kx*ky, and the sampler also writes weight_noise_reshaped
+
     def set_noise(self, noise_scale=None, words=None, bias_generator=None):
         """modules/binary.py:54-64.  ``words`` (uint32 [directions, rows, in_degree]) replaces the
         generator: bit = words < floor(P * 2**32).  The bias noise comes from torch's global generator of the
@@ -94,10 +96,15 @@ class Binarized(Perturbed, nn.Module):
             self.set_noise_scale(noise_scale)
         P = self.probabilities()
         if words is None:
-            self.weight_noise = booleanOperations.sample_bits(P, self.directions, self.dtype, self.seed)
+            sampled = booleanOperations.sample_bits(P, self.directions, self.dtype, self.seed, conv_taps=self.conv_taps)
         else:
-            self.weight_noise = booleanOperations.sample_bits_from_words(
-                booleanOperations.thresholds_from_p(P), words, self.dtype)
+            sampled = booleanOperations.sample_bits_from_words(
+                booleanOperations.thresholds_from_p(P), words, self.dtype, conv_taps=self.conv_taps)
+        if self.conv_taps is None:
+            self.weight_noise = sampled
+        else:
+            # one kernel wrote both layouts: rows (what update sums over) and [D, kx*ky*Cw, out] (what conv multiplies)
+            self.weight_noise, self.weight_noise_reshaped = sampled
         self.bias_noise = (torch.rand(size=(self.directions, self.out_degree), dtype=torch.float16,
                                       device=self.weight.device, generator=bias_generator) - .5) * 6
 
@@ -172,6 +179,7 @@ class BinarizedConv2d(Binarized):
         self.stride = stride
         self.padding = padding
         self.kernel_size = (kernel_size, kernel_size) if isinstance(kernel_size, int) else kernel_size
+        self.conv_taps = self.kernel_size[0] * self.kernel_size[1]
         self.weight = Parameter(torch.zeros(out_channels * self.kernel_size[0] * self.kernel_size[1], in_channels,
                                             dtype=torch.float16, device=device))
         if threshold:
@@ -190,10 +198,7 @@ class BinarizedConv2d(Binarized):
 
     def set_noise(self, noise_scale=None, words=None, bias_generator=None):
         """modules/binary.py:134-137: [D, out*kx*ky, Cw] -> [D, kx*ky*Cw, out], out contiguous."""
-        Binarized.set_noise(self, noise_scale, words, bias_generator)
-        r = self.weight_noise.view(self.directions, self.out_channels, *self.kernel_size, -1)
-        self.weight_noise_reshaped = r.permute([0, 2, 3, 4, 1]).reshape(self.directions, -1,
-                                                                       self.out_channels).contiguous()
+        Binarized.set_noise(self, noise_scale, words, bias_generator)     # fills weight_noise_reshaped as well
         # narrow inputs (one word per pixel, at most half of it used): several taps share a word
         self.weight_noise_tap = None
         if booleanOperations.tap_packing_applies(self.in_channels, self.weight_noise.size(2), self.dtype):

@@ -109,8 +109,8 @@ def _conv_filters(base_bits, D, O, k, C, T, seed, subseq, dtype, device):
     """base_bits [O*k*k, C] (rows ordered (out, kx, ky), modules/binary.py:125) -> per-member filters
     [D, k*k*Cw, O] (modules/binary.py:136-137)."""
     base = ops.pack(base_bits.to(device), dtype)                                  # [O*k*k, Cw]
-    Wn = ops.flip_philox(base, C, D, T, seed, subsequence=subseq)                # [D, O*k*k, Cw]
-    filt = Wn.view(D, O, k, k, -1).permute(0, 2, 3, 4, 1).reshape(D, -1, O).contiguous()
+    # one sampler pass writes the rows layout [D, O*k*k, Cw] and the conv layout [D, k*k*Cw, O]
+    Wn, filt = ops.sample_bits_philox(T, D, dtype, seed, subseq, base=base, shape=(O * k * k, C), conv_taps=k * k)
     return base, Wn, filt
 
 

@@ -893,3 +893,40 @@ def test_bmv_bn_act_vs_oracle(ops, oracle, dtype):
             assert torch.equal(got, act_t > thresh)
     with pytest.raises(RuntimeError, match="workspace"):
         ops._lib.call("nb_bmv_bn_act_i64", 256, 256, 256, 256, 256, 4, 64, 1, 64, 0, 256, 16, None)
+
+
+@pytest.mark.parametrize("dtype", [torch.int64, torch.int32])
+@pytest.mark.parametrize("n,O,k,C", [(3, 16, 3, 16), (2, 64, 3, 64), (5, 8, 3, 3), (2, 33, 5, 70), (17, 64, 3, 128),
+                                     (2, 4, 1, 256), (9, 128, 3, 64)])
+def test_sampler_writes_the_conv_layout_in_the_same_pass(ops, oracle, dtype, n, O, k, C):
+    """sample_bits*(conv_taps=k*k): the rows layout [n, O*k*k, Cw] equals the plain sampler's (and the oracle's), and
+    the conv layout equals its view -> permute(0,2,3,4,1) -> reshape(n, k*k*Cw, O) (modules/binary.py:134-137);
+    supplied words and generator mode, thresholds per element and a scalar flip probability with a base."""
+    nd = NDT[dtype]
+    wb = np.dtype(nd).itemsize * 8
+    KK, R, Cw = k * k, O * k * k, (C + wb - 1) // wb
+    g = rng(n + O + k + C)
+    words = g.integers(0, 2 ** 32, size=(n, R, C), dtype=np.uint64).astype(np.uint32)
+    thr = g.integers(0, 2 ** 32, size=(R, C), dtype=np.uint64).astype(np.uint32)
+    base = rand_words(g, (R, Cw), nd)
+    if C % wb:
+        base[:, -1] &= nd((1 << (C % wb)) - 1)
+    T = int(0.02 * 2 ** 32)
+
+    def permuted(rows):                                                   # numpy restatement of the layer's permute
+        return np.ascontiguousarray(rows.reshape(n, O, k, k, Cw).transpose(0, 2, 3, 4, 1).reshape(n, KK * Cw, O))
+
+    want = oracle.sample_from_words(thr, words, nd)
+    rows, conv = ops.sample_bits_from_words(dev(thr), dev(words), dtype, conv_taps=KK)
+    np.testing.assert_array_equal(host(rows), want)
+    assert tuple(conv.shape) == (n, KK * Cw, O) and conv.is_contiguous()
+    np.testing.assert_array_equal(host(conv), permuted(want))
+    want = oracle.sample_from_words(T, words, nd, base=base)
+    rows, conv = ops.sample_bits_from_words(T, dev(words), dtype, base=dev(base), conv_taps=KK, rows_too=False)
+    assert rows is None
+    np.testing.assert_array_equal(host(conv), permuted(want))
+    # generator mode: the same stream as the plain sampler
+    plain = ops.sample_bits_philox(dev(thr), n, dtype, 99, 5)
+    rows, conv = ops.sample_bits_philox(dev(thr), n, dtype, 99, 5, conv_taps=KK)
+    assert torch.equal(rows, plain)
+    np.testing.assert_array_equal(host(conv), permuted(host(plain)))
