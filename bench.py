@@ -97,6 +97,20 @@ def time_graph(torch, step, steps, replays=5):
         return None
 
 
+def time_resample(torch, w, reps=3):
+    """ms to draw every member's weights of every layer again (a training step's set_noise), when the workload can."""
+    fn = w.meta.get("resample")
+    if fn is None:
+        return
+    fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        fn()
+    torch.cuda.synchronize()
+    w.meta["set_noise_ms"] = round((time.perf_counter() - t0) / reps * 1e3, 3)
+
+
 def config_entry(cfg, w, per_wall, per_ev, per_graph=None):
     """One line of other_configs.  A compute-shaped configuration is priced against three limits: HBM (algorithmic
     bytes), the XOR-popcount issue rate of the vector ALUs and the dense int8 rate of the matrix cores (one +-1 byte
@@ -108,6 +122,8 @@ def config_entry(cfg, w, per_wall, per_ev, per_graph=None):
              "binary_TOPS": round(2 * w.bit_macs / per_wall / 1e12, 3)}
     if "fc" in w.meta:
         entry["fc_8192_1024"] = w.meta["fc"]
+    if "set_noise_ms" in w.meta:
+        entry["set_noise_ms"] = w.meta["set_noise_ms"]
     if per_graph:
         # device time per step from a graph replay; the roofline fractions below use it when it is available
         entry.update(ms_per_step_graph=round(per_graph * 1e3, 4),
@@ -320,6 +336,7 @@ def main():
         return 0
     if args.only:
         w = workloads.BUILDERS[args.only]()
+        time_resample(torch, w)
         pw, pe = time_steps(torch, w.step, args.steps, args.warmup)
         entry = config_entry(args.only, w, pw, pe, None if args.no_graph else time_graph(torch, w.step, args.steps))
         entry["event_ms_per_step"] = round(pe * 1e3, 4)
@@ -355,6 +372,7 @@ def main():
         if cfg == 2:
             continue
         w = workloads.BUILDERS[cfg]()
+        time_resample(torch, w)
         steps = max(3, args.steps // 2) if cfg == 5 else args.steps
         pw, pe = time_steps(torch, w.step, steps, args.warmup)
         entry = config_entry(cfg, w, pw, pe, None if args.no_graph else time_graph(torch, w.step, steps))

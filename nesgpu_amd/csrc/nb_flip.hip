@@ -252,6 +252,164 @@ __global__ __launch_bounds__(256) void fl_fill_kernel(uint32_t *__restrict__ ent
     for (; j < L; j++) dst[at(j)] = sentinel | (sentinel << 16);
 }
 
+// ---- skip sampler: flip lists straight from the generator, without ever drawing the bits that do not flip -----------
+// For a uniform flip probability p the columns that flip in a row form a renewal process with geometric gaps.  Row q
+// (flat over members and rows) reads the Philox words first + q*C + i, i = 0, 1, ...; word i has the rank
+// #{k < Kt : cdf[k] <= word} (cdf[k-1] = floor(2^32 * (1 - (1-p)^k)), supplied by the caller; Kt == 0 means no
+// flips): a rank below Kt moves the position on by rank + 1 columns and flips the column reached, rank Kt (a word
+// beyond the table) moves it on by Kt columns without a flip; the row ends when the position passes C.  About
+// C*p + 1 words per row instead of C: 100 times fewer at p = 0.01.  The same law as the per-bit compare (i.i.d. Bernoulli(p), quantised to
+// 2^-32), not the same stream.
+constexpr int kSkipMaxTable = 4096;
+
+struct SkipChain {
+    PhiloxKey key;
+    uint64_t g;   // index of the next word
+    uint4 blk;
+    bool fresh;
+    __device__ __forceinline__ SkipChain(const PhiloxKey &k, uint64_t start) : key(k), g(start), fresh(true) {}
+    __device__ __forceinline__ uint32_t next()
+    {
+        if (fresh || (g & 3u) == 0) blk = philox_block(key, g >> 2);
+        fresh = false;
+        const uint32_t e = (uint32_t)g & 3u;
+        g++;
+        return e == 0 ? blk.x : e == 1 ? blk.y : e == 2 ? blk.z : blk.w;
+    }
+};
+
+// number of table entries <= u (the table is sorted): thirteen fixed probes, no divergence
+__device__ __forceinline__ int skip_rank(const uint32_t *tab, int Kt, uint32_t u)
+{
+    int lo = 0;
+#pragma unroll
+    for (int step = kSkipMaxTable; step > 0; step >>= 1) {
+        const int idx = lo + step;
+        if (idx <= Kt && tab[idx - 1] <= u) lo = idx;
+    }
+    return lo;
+}
+
+__global__ __launch_bounds__(256) void fl_skip_count_kernel(uint16_t *__restrict__ cnt, const uint32_t *__restrict__ cdf,
+                                                            int Kt, PhiloxKey key, int64_t rows, int C)
+{
+    __shared__ uint32_t tab[kSkipMaxTable];
+    for (int i = threadIdx.x; i < Kt; i += 256) tab[i] = cdf[i];
+    __syncthreads();
+    const int64_t q = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (q >= rows) return;
+    int n = 0;
+    if (Kt > 0) {
+        SkipChain chain(key, key.first + (uint64_t)q * (uint64_t)C);
+        int pos = -1;
+        for (;;) {
+            const int rank = skip_rank(tab, Kt, chain.next());
+            pos += rank < Kt ? rank + 1 : Kt;
+            if (pos >= C) break;
+            n += rank < Kt ? 1 : 0;
+        }
+    }
+    cnt[q] = (uint16_t)n;
+}
+
+__global__ __launch_bounds__(256) void fl_skip_fill_kernel(uint32_t *__restrict__ entries,
+                                                           const uint64_t *__restrict__ base,
+                                                           const uint16_t *__restrict__ perm,
+                                                           const int64_t *__restrict__ slice_off,
+                                                           const int32_t *__restrict__ slice_len,
+                                                           const uint32_t *__restrict__ cdf, int Kt, PhiloxKey key,
+                                                           int64_t nslices, int S, int64_t R, int Kw, int C)
+{
+    __shared__ uint32_t tab[kSkipMaxTable];
+    for (int i = threadIdx.x; i < Kt; i += 256) tab[i] = cdf[i];
+    __syncthreads();
+    const int lane = threadIdx.x & 63;
+    const int64_t sl = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (sl >= nslices) return;
+    const int64_t d = sl / S;
+    const int s = (int)(sl - d * S);
+    const int64_t p = (int64_t)s * 64 + lane;
+    const bool valid = p < R;
+    int64_t r = valid ? perm[d * R + p] : 0;
+    r = r < R ? r : R - 1;
+    const int L = 4 * slice_len[sl];
+    uint32_t *dst = entries + slice_off[sl] + lane * 4;
+    auto at = [](int j) { return (int64_t)(j >> 2) * 256 + (j & 3); };
+    const uint32_t sentinel = (uint32_t)(4 * Kw) << 5;
+    int j = 0;
+    uint32_t pend = 0;
+    bool half = false;
+    if (valid && Kt > 0) {
+        const uint64_t *b = base + r * Kw;
+        SkipChain chain(key, key.first + (uint64_t)(d * R + r) * (uint64_t)C);
+        int pos = -1;
+        for (;;) {
+            const int rank = skip_rank(tab, Kt, chain.next());
+            pos += rank < Kt ? rank + 1 : Kt;
+            if (pos >= C) break;
+            if (rank >= Kt) continue;  // a word beyond the table: moved on, no flip
+            const uint32_t col = (uint32_t)pos;
+            const uint32_t bb = (uint32_t)(b[col >> 6] >> (col & 63u)) & 1u;
+            const uint32_t e = ((2u * (col >> 5) + bb) << 5) | (col & 31u);
+            if (!half) {
+                pend = e;
+                half = true;
+            } else {
+                if (j < L) dst[at(j)] = pend | (e << 16);
+                j++;
+                half = false;
+            }
+        }
+    }
+    if (half) {
+        if (j < L) dst[at(j)] = pend | (sentinel << 16);
+        j++;
+    }
+    for (; j < L; j++) dst[at(j)] = sentinel | (sentinel << 16);
+}
+
+// Flip lists -> materialised weights: W must hold the base in every member on entry; every flip is XOR-ed in.  A
+// lane owns its row, so plain read-modify-writes suffice (flips come in column order: one write per touched word).
+__global__ __launch_bounds__(256) void fl_to_dense_kernel(uint64_t *__restrict__ W, const uint32_t *__restrict__ entries,
+                                                          const int64_t *__restrict__ slice_off,
+                                                          const int32_t *__restrict__ slice_len,
+                                                          const uint16_t *__restrict__ perm, int64_t nslices, int S,
+                                                          int64_t R, int Kw)
+{
+    const int lane = threadIdx.x & 63;
+    const int64_t sl = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (sl >= nslices) return;
+    const int64_t d = sl / S;
+    const int s = (int)(sl - d * S);
+    const int64_t p = (int64_t)s * 64 + lane;
+    if (p >= R) return;
+    int64_t r = perm[d * R + p];
+    r = r < R ? r : R - 1;
+    uint64_t *row = W + (d * R + r) * Kw;
+    const uint32_t *src = entries + slice_off[sl] + lane * 4;
+    const int L = 4 * slice_len[sl];
+    int curw = -1;
+    uint64_t mask = 0;
+    for (int j = 0; j < L; j++) {
+        const uint32_t pair = src[(int64_t)(j >> 2) * 256 + (j & 3)];
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const uint32_t e = h ? pair >> 16 : pair & 0xFFFFu;
+            const uint32_t piece = e >> 5;
+            if (piece >= (uint32_t)(4 * Kw)) continue;  // sentinel
+            const uint32_t col = (piece >> 1) * 32u + (e & 31u);
+            const int w = (int)(col >> 6);
+            if (w != curw) {
+                if (curw >= 0) row[curw] ^= mask;
+                curw = w;
+                mask = 0;
+            }
+            mask |= (uint64_t)1 << (col & 63u);
+        }
+    }
+    if (curw >= 0) row[curw] ^= mask;
+}
+
 // ---- the members' corrections, threshold and pack --------------------------------------------------------------------
 // One workgroup per (member, block of 1024 rows), one wave per slice.  PACK: out = bits (2 * sum > thresh) of the
 // block's rows, OR-ed into an LDS bit array (the rows of a slice are scattered over the block) and written as 32-bit
@@ -448,6 +606,76 @@ int nb_flip_fill_i64(uint32_t *entries, const int64_t *W, const int64_t *base, c
     nb::fl_fill_kernel<<<dim3((unsigned)nb::ceil_div(D * S, 4)), dim3(256), 0, nb::as_stream(stream)>>>(
         entries, reinterpret_cast<const uint64_t *>(W), reinterpret_cast<const uint64_t *>(base), perm, slice_off,
         slice_len, D * S, (int)S, R, (int)Kw);
+    return nb::check_launch(who);
+}
+
+int nb_flip_skip_count_i64(uint16_t *cnt, const uint32_t *cdf, int64_t Kt, uint64_t seed, uint64_t subseq, uint64_t first,
+                           int64_t D, int64_t R, int64_t C, nb_stream_t stream)
+{
+    const char *who = "nb_flip_skip_count_i64";
+    NB_REQUIRE(C >= 0 && Kt >= 0 && Kt <= nb::kSkipMaxTable, "%s: bad C=%lld or table of %lld entries (at most %d)", who,
+               (long long)C, (long long)Kt, nb::kSkipMaxTable);
+    if (int rc = nb::flip_shape_check(D, R, (C + 63) / 64, who)) return rc;
+    if (D * R == 0) return NB_OK;
+    NB_REQUIRE_PTR(cnt);
+    NB_REQUIRE_ALIGNED(cnt, 2);
+    if (Kt > 0) NB_REQUIRE_PTR(cdf);
+    NB_REQUIRE_ALIGNED(cdf, 4);
+    const int64_t blocks = nb::ceil_div(D * R, 256);
+    NB_REQUIRE(blocks <= nb::kMaxGridX, "%s: too many rows for one launch", who);
+    nb::fl_skip_count_kernel<<<dim3((unsigned)blocks), dim3(256), 0, nb::as_stream(stream)>>>(
+        cnt, cdf, (int)Kt, nb::PhiloxKey{seed, subseq, first}, D * R, (int)C);
+    return nb::check_launch(who);
+}
+
+int nb_flip_skip_fill_i64(uint32_t *entries, const int64_t *base, const uint16_t *perm, const int64_t *slice_off,
+                          const int32_t *slice_len, const uint32_t *cdf, int64_t Kt, uint64_t seed, uint64_t subseq,
+                          uint64_t first, int64_t D, int64_t R, int64_t C, nb_stream_t stream)
+{
+    const char *who = "nb_flip_skip_fill_i64";
+    NB_REQUIRE(C >= 0 && Kt >= 0 && Kt <= nb::kSkipMaxTable, "%s: bad C=%lld or table of %lld entries (at most %d)", who,
+               (long long)C, (long long)Kt, nb::kSkipMaxTable);
+    const int64_t Kw = (C + 63) / 64;
+    if (int rc = nb::flip_shape_check(D, R, Kw, who)) return rc;
+    if (D * R == 0) return NB_OK;
+    NB_REQUIRE_PTR(entries);
+    NB_REQUIRE_PTR(perm);
+    NB_REQUIRE_PTR(slice_off);
+    NB_REQUIRE_PTR(slice_len);
+    NB_REQUIRE_ALIGNED(entries, 16);
+    NB_REQUIRE_ALIGNED(perm, 2);
+    NB_REQUIRE_ALIGNED(slice_off, 8);
+    NB_REQUIRE_ALIGNED(slice_len, 4);
+    if (Kt > 0) NB_REQUIRE_PTR(cdf);
+    NB_REQUIRE_ALIGNED(cdf, 4);
+    if (Kw > 0) NB_REQUIRE_PTR(base);
+    NB_REQUIRE_ALIGNED(base, 8);
+    const int64_t S = (R + 63) / 64;
+    nb::fl_skip_fill_kernel<<<dim3((unsigned)nb::ceil_div(D * S, 4)), dim3(256), 0, nb::as_stream(stream)>>>(
+        entries, reinterpret_cast<const uint64_t *>(base), perm, slice_off, slice_len, cdf, (int)Kt,
+        nb::PhiloxKey{seed, subseq, first}, D * S, (int)S, R, (int)Kw, (int)C);
+    return nb::check_launch(who);
+}
+
+int nb_flip_to_dense_i64(int64_t *W, const uint32_t *entries, const int64_t *slice_off, const int32_t *slice_len,
+                         const uint16_t *perm, int64_t D, int64_t R, int64_t Kw, nb_stream_t stream)
+{
+    const char *who = "nb_flip_to_dense_i64";
+    if (int rc = nb::flip_shape_check(D, R, Kw, who)) return rc;
+    if (D * R * Kw == 0) return NB_OK;
+    NB_REQUIRE_PTR(W);
+    NB_REQUIRE_PTR(entries);
+    NB_REQUIRE_PTR(perm);
+    NB_REQUIRE_PTR(slice_off);
+    NB_REQUIRE_PTR(slice_len);
+    NB_REQUIRE_ALIGNED(W, 8);
+    NB_REQUIRE_ALIGNED(entries, 16);
+    NB_REQUIRE_ALIGNED(perm, 2);
+    NB_REQUIRE_ALIGNED(slice_off, 8);
+    NB_REQUIRE_ALIGNED(slice_len, 4);
+    const int64_t S = (R + 63) / 64;
+    nb::fl_to_dense_kernel<<<dim3((unsigned)nb::ceil_div(D * S, 4)), dim3(256), 0, nb::as_stream(stream)>>>(
+        reinterpret_cast<uint64_t *>(W), entries, slice_off, slice_len, perm, D * S, (int)S, R, (int)Kw);
     return nb::check_launch(who);
 }
 

@@ -25,7 +25,7 @@ __all__ = [
     "flip_from_words", "sample_bits_philox", "flip_philox", "seeded_bmv_from_words", "seeded_bmv_philox",
     "philox_words", "conv_act_pack", "conv_popc_sums", "tap_pack_filter", "tap_packing_applies", "conv_engine", "conv_last_engine",
     "bmv_act_pack", "bmv_bn_act", "ExpandedRows", "expand_rows", "bmm_nt", "FlipRows", "flip_rows_from_weights",
-    "bmv_flip", "bmv_flip_act_pack",
+    "bmv_flip", "bmv_flip_act_pack", "skip_table", "flip_rows_skip", "flip_rows_to_weights",
 ]
 
 
@@ -682,6 +682,24 @@ class FlipRows:
                                                            self.slice_len))
 
 
+def _flip_rows_layout(cnt, D, R):
+    """Flip counts [D, R] (uint16) -> (perm, slice_len, slice_off, total dwords): rows ordered by count inside blocks
+    of 1024 rows, slices of 64 rows padded to their longest row in 16-byte pieces of 8 flips."""
+    dev = cnt.device
+    S = ceil_div(R, 64)
+    nblk = ceil_div(R, 1024)
+    c = cnt.view(torch.int16).to(torch.int32) & 0xFFFF
+    cp = torch.nn.functional.pad(c, (0, nblk * 1024 - R), value=1 << 20).view(D, nblk, 1024)
+    order = torch.sort(cp, dim=2, stable=True).indices + (torch.arange(nblk, device=dev) * 1024).view(1, nblk, 1)
+    order = order.view(D, nblk * 1024)[:, :R].contiguous()                       # padding sorts last in its block
+    cs = torch.nn.functional.pad(c.gather(1, order), (0, S * 64 - R)).view(D, S, 64)
+    slice_len = ((cs.max(dim=2).values + 7) // 8).to(torch.int32).contiguous()  # 16-byte pieces (8 flips) per lane
+    lens = slice_len.view(-1).to(torch.int64) * 256                              # dwords of a slice
+    slice_off = (torch.cumsum(lens, 0) - lens).view(D, S).contiguous()
+    total = int(lens.sum().item()) if D * S else 0
+    return order.to(torch.uint16).contiguous(), slice_len, slice_off, total
+
+
 def flip_rows_from_weights(W, base):
     """W int64 [D, R, Kw] (a population's materialised weights), base int64 [R, Kw] -> :class:`FlipRows` holding
     exactly the bits W ^ base.  Rows are ordered by flip count inside blocks of 1024 rows so that the 64 rows of a
@@ -698,23 +716,72 @@ def flip_rows_from_weights(W, base):
     cnt = torch.empty((D, R), dtype=torch.uint16, device=dev)
     with _on(W):
         _lib.call("nb_flip_count_i64", cnt.data_ptr(), W.data_ptr(), base.data_ptr(), D, R, Kw, _stream(W))
-    S = ceil_div(R, 64)
-    nblk = ceil_div(R, 1024)
-    c = cnt.view(torch.int16).to(torch.int32) & 0xFFFF
-    cp = torch.nn.functional.pad(c, (0, nblk * 1024 - R), value=1 << 20).view(D, nblk, 1024)
-    order = torch.sort(cp, dim=2, stable=True).indices + (torch.arange(nblk, device=dev) * 1024).view(1, nblk, 1)
-    order = order.view(D, nblk * 1024)[:, :R].contiguous()                       # padding sorts last in its block
-    cs = torch.nn.functional.pad(c.gather(1, order), (0, S * 64 - R)).view(D, S, 64)
-    slice_len = ((cs.max(dim=2).values + 7) // 8).to(torch.int32).contiguous()  # 16-byte pieces (8 flips) per lane
-    lens = slice_len.view(-1).to(torch.int64) * 256                              # dwords of a slice
-    slice_off = (torch.cumsum(lens, 0) - lens).view(D, S).contiguous()
-    total = int(lens.sum().item()) if D * S else 0
-    perm = order.to(torch.uint16).contiguous()
+    perm, slice_len, slice_off, total = _flip_rows_layout(cnt, D, R)
     entries = torch.empty((max(total, 4),), dtype=torch.uint32, device=dev)
     with _on(W):
         _lib.call("nb_flip_fill_i64", entries.data_ptr(), W.data_ptr(), base.data_ptr(), perm.data_ptr(),
                   slice_off.data_ptr(), slice_len.data_ptr(), D, R, Kw, _stream(W))
     return FlipRows(base, D, R, Kw, cnt, perm, slice_off, slice_len, entries)
+
+
+def skip_table(threshold, cap=4096):
+    """Gap table of the skip sampler for flip probability p = threshold / 2**32 (uint32 numpy array): entry k-1 =
+    floor(2**32 * (1 - (1-p)**k)) for k = 1, 2, ... until it saturates at 2**32 - 1 (at most ``cap`` entries); entry
+    0 is ``threshold`` itself; empty for p = 0 (no flips).  A random word with ``rank`` entries <= it moves a row's
+    walk on by rank + 1 columns to the next flip, or, beyond the table, by its length without a flip."""
+    import numpy as np
+    t = int(threshold)
+    if not 0 <= t <= 0xFFFFFFFF:
+        raise ValueError("threshold must fit in uint32")
+    p = t / 4294967296.0
+    if p <= 0.0:
+        return np.zeros(0, dtype=np.uint32)
+    k = np.arange(1, cap + 1, dtype=np.float64)
+    v = np.minimum(np.floor(-np.expm1(k * np.log1p(-p)) * 4294967296.0), 4294967295.0)
+    v[0] = float(t)
+    v = np.maximum.accumulate(v)
+    full = v >= 4294967295.0
+    n = int(np.argmax(full)) + 1 if full.any() else cap
+    return v[:n].astype(np.uint32)
+
+
+def flip_rows_skip(base, in_bits, n, threshold, seed, subsequence=0, first=0):
+    """:class:`FlipRows` for ``n`` members drawn by the skip sampler: every bit of a member's [R, in_bits] weights
+    differs from ``base`` with probability threshold / 2**32, independently, as with :func:`flip_philox`, but the
+    generator only draws the gaps between flips (about in_bits * p + 1 words per row instead of in_bits), and the
+    materialised weights never exist.  Row q = m*R + r consumes the Philox words first + q*in_bits + i of the stream
+    (seed, subsequence).  The stream differs from :func:`flip_philox`'s: the law is the same, the bits are not."""
+    _check(base, "base")
+    assert len(base.shape) == 2
+    if base.dtype != torch.int64:
+        raise TypeError("flip lists take 64-bit words")
+    R, Kw = base.shape
+    C = int(in_bits)
+    assert ceil_div(C, 64) == Kw
+    dev = base.device
+    table = skip_table(threshold)
+    cdf = torch.from_numpy(table.view("int32").copy()).to(dev).view(torch.uint32) if table.size else None
+    cptr, Kt = (cdf.data_ptr(), int(table.size)) if cdf is not None else (None, 0)
+    cnt = torch.empty((n, R), dtype=torch.uint16, device=dev)
+    key = (int(seed) & (2 ** 64 - 1), int(subsequence), int(first))
+    with _on(base):
+        _lib.call("nb_flip_skip_count_i64", cnt.data_ptr(), cptr, Kt, *key, n, R, C, _stream(base))
+    perm, slice_len, slice_off, total = _flip_rows_layout(cnt, n, R)
+    entries = torch.empty((max(total, 4),), dtype=torch.uint32, device=dev)
+    with _on(base):
+        _lib.call("nb_flip_skip_fill_i64", entries.data_ptr(), base.data_ptr(), perm.data_ptr(), slice_off.data_ptr(),
+                  slice_len.data_ptr(), cptr, Kt, *key, n, R, C, _stream(base))
+    return FlipRows(base, n, R, Kw, cnt, perm, slice_off, slice_len, entries)
+
+
+def flip_rows_to_weights(rows):
+    """:class:`FlipRows` -> the materialised weights int64 [D, R, Kw] = base ^ flips (for the dense kernels, and for
+    checking the two forms against each other)."""
+    W = rows.base.unsqueeze(0).expand(rows.D, rows.R, rows.Kw).contiguous()
+    with _on(W):
+        _lib.call("nb_flip_to_dense_i64", W.data_ptr(), rows.entries.data_ptr(), rows.slice_off.data_ptr(),
+                  rows.slice_len.data_ptr(), rows.perm.data_ptr(), rows.D, rows.R, rows.Kw, _stream(W))
+    return W
 
 
 def _flip_args(rows, x, G):

@@ -166,60 +166,73 @@ def cifar_net(D=4096, T=T_P01, seed=0, dtype=torch.int64, device="cuda", classes
     """Config 5: conv3->64, conv64->64, pool, conv64->128, pool, linear 8192->1024, linear 1024->10 on 3x32x32
     inputs binarised at their per-channel mean; sign threshold 0 between layers; int32 logits (raw popc).
 
-    ``sparse_fc``: the 8192->1024 layer runs from the shared base and the members' flip lists (one product for the
-    whole population on the matrix cores + 2 bytes per flipped weight) instead of streaming the 4 GiB of
-    materialised per-member weights; the same bits either way (``step_dense`` in ``meta`` is the other form)."""
+    ``sparse_fc`` (64-bit words): the 8192->1024 layer keeps its per-member weights as the shared base plus flip
+    lists drawn by the skip sampler (Philox stream (seed, subsequence 13); only the gaps between flips are drawn, the
+    4 GiB of materialised weights never exist) and runs as one product for the whole population on the matrix cores
+    plus 2 bytes per flipped weight.  ``meta["W4"]()`` materialises the same weights for the dense kernels
+    (``meta["step_dense"]``), which give the same bits.  With ``sparse_fc=False`` the layer's weights come from the
+    per-bit compare sampler (same law, another stream) and are streamed."""
     g = _gen(seed)
     z = torch.randn((D, 3, 32, 32), generator=g)
     x_bits = (z > z.mean(dim=(0, 2, 3), keepdim=True)).permute(0, 2, 3, 1).contiguous()      # [D,32,32,3]
     x = ops.pack(x_bits.view(-1, 3).to(device), dtype).view(D, 32, 32, 1)
-    layers = []
-    bases = []
-    macs = 0
-    subseq = 10
-    for (C, O, S) in ((3, 64, 32), (64, 64, 32), (64, 128, 16)):
-        base_bits = _bits(g, (O * 9, C))
-        base, Wn, filt = _conv_filters(base_bits, D, O, 3, C, T, seed, subseq, dtype, device)
-        del Wn
-        bases.append(base)
-        thr = torch.full((D, O), 9 * C, dtype=torch.int32, device=device)
-        layers.append((filt, thr) + _tap(filt, 3, C))
-        macs += D * S * S * O * 9 * C
-        subseq += 1
+    shapes = ((3, 64, 32), (64, 64, 32), (64, 128, 16))
+    conv_bases = [ops.pack(_bits(g, (O * 9, C)).to(device), dtype) for (C, O, S) in shapes]
     b4 = ops.pack(_bits(g, (1024, 8192)).to(device), dtype)
-    W4 = ops.flip_philox(b4, 8192, D, T, seed, subsequence=subseq)              # [D,1024,128]: 4 GiB at D=4096
     b5 = ops.pack(_bits(g, (classes, 1024)).to(device), dtype)
-    W5 = ops.flip_philox(b5, 1024, D, T, seed, subsequence=subseq + 1)
-    macs += D * 1024 * 8192 + D * classes * 1024
+    sparse = bool(sparse_fc) and dtype == torch.int64
+    macs = sum(D * S * S * O * 9 * C for (C, O, S) in shapes) + D * 1024 * 8192 + D * classes * 1024
     thr4 = torch.full((D, 1024), 8192, dtype=torch.int32, device=device)
-    rows4 = ops.flip_rows_from_weights(W4, b4) if (sparse_fc and dtype == torch.int64) else None
+    state = {}
+
+    def resample():
+        """Draw every member's weights of every layer again (what a training step's set_noise does)."""
+        layers = []
+        for i, (C, O, S) in enumerate(shapes):
+            _, filt = ops.sample_bits_philox(T, D, dtype, seed, 10 + i, base=conv_bases[i], shape=(O * 9, C),
+                                             conv_taps=9, rows_too=False)
+            thr = torch.full((D, O), 9 * C, dtype=torch.int32, device=device)
+            layers.append((filt, thr) + _tap(filt, 3, C))
+        state["layers"] = layers
+        if sparse:
+            state["rows4"], state["W4"] = ops.flip_rows_skip(b4, 8192, D, T, seed, subsequence=13), None
+        else:
+            state["rows4"], state["W4"] = None, ops.flip_philox(b4, 8192, D, T, seed, subsequence=13)  # 4 GiB at 4096
+        state["W5"] = ops.flip_philox(b5, 1024, D, T, seed, subsequence=14)
+
+    resample()
+
+    def W4():
+        if state["W4"] is None:
+            state["W4"] = ops.flip_rows_to_weights(state["rows4"])
+        return state["W4"]
 
     def features():
         a = x
         for i, pool in enumerate((False, True, True)):                   # [D,32,32,1] [D,16,16,1] [D,8,8,2]
-            _, thr, f, kw = layers[i]
+            _, thr, f, kw = state["layers"][i]
             a = ops.conv_act_pack(a, f, thr, 3, 3, 1, 1, 1, 1, pool=pool, **kw)
         return a.view(D, -1, 1)                                                                 # [D,128,1]
 
     def step_dense():
-        a = ops.bmv_act_pack(W4, features(), thr4).view(D, -1, 1)         # pack(2 * bmm(W4, a) > 8192): [D,16,1]
-        return ops.bmm(W5, a).squeeze(2)                                                        # [D,classes] popc
+        a = ops.bmv_act_pack(W4(), features(), thr4).view(D, -1, 1)       # pack(2 * bmm(W4, a) > 8192): [D,16,1]
+        return ops.bmm(state["W5"], a).squeeze(2)                                               # [D,classes] popc
 
     def step_sparse():
-        a = ops.bmv_flip_act_pack(rows4, features(), thr4).view(D, -1, 1)  # the same bits from base + flip lists
-        return ops.bmm(W5, a).squeeze(2)
-
-    step = step_sparse if rows4 is not None else step_dense
+        a = ops.bmv_flip_act_pack(state["rows4"], features(), thr4).view(D, -1, 1)   # the same bits from the lists
+        return ops.bmm(state["W5"], a).squeeze(2)
 
     w = Workload(
         name="CIFAR-shaped binary net D=%d (conv3-64, conv64-64, pool, conv64-128, pool, fc8192-1024, fc1024-%d)"
              % (D, classes),
-        population=D, bit_macs=macs, algo_bytes=rows4.nbytes() if rows4 is not None else W4.numel() * 8, bound="valu",
-        step=step,
-        tensors=dict(x=x, f1=layers[0][0], f2=layers[1][0], f3=layers[2][0], W4=W4, W5=W5, b1=bases[0], b2=bases[1],
-                     b3=bases[2], b4=b4, b5=b5),
-        meta=dict(T=T, seed=seed, first_subsequence=10, step_dense=step_dense, features=features, rows4=rows4,
-                  thr4=thr4, fc="base + flip lists" if rows4 is not None else "materialised weights"))
+        population=D, bit_macs=macs,
+        algo_bytes=state["rows4"].nbytes() if sparse else D * 1024 * 128 * 8, bound="valu",
+        step=step_sparse if sparse else step_dense,
+        tensors=dict(x=x, f1=state["layers"][0][0], f2=state["layers"][1][0], f3=state["layers"][2][0],
+                     W5=state["W5"], b1=conv_bases[0], b2=conv_bases[1], b3=conv_bases[2], b4=b4, b5=b5),
+        meta=dict(T=T, seed=seed, first_subsequence=10, step_dense=step_dense, features=features,
+                  rows4=state["rows4"], W4=W4, thr4=thr4, resample=resample,
+                  fc="base + flip lists (skip sampler)" if sparse else "materialised weights"))
     return w
 
 

@@ -18,6 +18,8 @@
  *   seeded_bmv           must equal bmm(sample_from_words(...), x)
  *   philox4x32_10        Random123 known-answer vectors and rocRAND's host engine
  *   weighted_sum         float64 numpy einsum over unpacked bits (tolerance)
+ *   skip_flips           numpy searchsorted + cumsum over the (pinned) Philox words; flip rate,
+ *                        gap histogram against the geometric law, neighbouring columns uncorrelated
  * The cuRAND XORWOW stream of the reference samplers (sample_bits.cu:23-25,54) is NOT
  * reproduced anywhere: parity unpinned for that stream; supplied-word parity replaces it.
  *
@@ -131,6 +133,45 @@ void nbo_philox_words(uint32_t *out, uint64_t seed, uint64_t subseq, uint64_t fi
         uint32_t o[4];
         nbo_philox4x32_10(o, ctr, key);
         out[i] = o[g & 3];
+    }
+}
+
+/* Flip masks by gap sampling: the contract of the library's skip sampler (nb_flip_skip_*; no counterpart in the
+ * reference, whose sampler draws every bit, extensions/src/sample_bits.cu:47-57).  Row q (flat over members and rows)
+ * reads the Philox words first + q*C + i, i = 0, 1, ...; word i has rank #{k < Kt : cdf[k] <= word}: a rank below Kt
+ * moves the position on by rank + 1 columns and flips the column reached; rank Kt (the word lies beyond the table)
+ * moves it on by Kt columns without a flip (the geometric law has no memory, so the walk just continues); the row
+ * ends when the position passes C.  With cdf[k-1] = floor(2^32 * (1 - (1-p)^k)) the gaps are geometric and the
+ * columns i.i.d. Bernoulli(p), quantised to 2^-32.  An empty table (Kt == 0) stands for p = 0: no flips.  mask is
+ * [rows, ceil(C/64)] 64-bit words, LSB first. */
+void nbo_skip_flips_i64(uint64_t *mask, const uint32_t *cdf, int64_t Kt, uint64_t seed, uint64_t subseq, uint64_t first,
+                        int64_t rows, int64_t C)
+{
+    const uint32_t key[2] = {(uint32_t)seed, (uint32_t)(seed >> 32)};
+    const int64_t Kw = (C + 63) / 64;
+#pragma omp parallel for schedule(static)
+    for (int64_t q = 0; q < rows; q++) {
+        uint64_t *row = mask + q * Kw;
+        memset(row, 0, (size_t)Kw * 8);
+        if (Kt == 0) continue;
+        int64_t pos = -1;
+        for (int64_t i = 0;; i++) {
+            const uint64_t g = first + (uint64_t)q * (uint64_t)C + (uint64_t)i;
+            const uint64_t blk = g >> 2;
+            const uint32_t ctr[4] = {(uint32_t)blk, (uint32_t)(blk >> 32), (uint32_t)subseq, (uint32_t)(subseq >> 32)};
+            uint32_t o[4];
+            nbo_philox4x32_10(o, ctr, key);
+            const uint32_t u = o[g & 3];
+            int64_t lo = 0, hi = Kt; /* first index whose entry exceeds u */
+            while (lo < hi) {
+                const int64_t mid = (lo + hi) / 2;
+                if (cdf[mid] <= u) lo = mid + 1;
+                else hi = mid;
+            }
+            pos += lo < Kt ? 1 + lo : Kt;
+            if (pos >= C) break;
+            if (lo < Kt) row[pos >> 6] |= (uint64_t)1 << (pos & 63);
+        }
     }
 }
 

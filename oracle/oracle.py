@@ -219,6 +219,32 @@ def philox_words(seed, subseq, first, count):
     return out
 
 
+def skip_cdf(T, cap=4096):
+    """Gap table of the skip sampler for flip probability p = T / 2**32: entry k-1 = floor(2**32 * (1 - (1-p)**k)),
+    k = 1, 2, ... until the table saturates at 2**32 - 1 (at most ``cap`` entries; a word beyond a table cut short
+    moves the walk on without a flip); entry 0 is T itself.  The same
+    formula as the product's ``skip_table`` (the table is INPUT DATA of the contract, not part of it)."""
+    p = int(T) / 4294967296.0
+    if p <= 0.0:
+        return np.zeros(0, dtype=np.uint32)                 # the empty table stands for "no flips"
+    k = np.arange(1, cap + 1, dtype=np.float64)
+    v = np.floor(-np.expm1(k * np.log1p(-p)) * 4294967296.0) if p < 1.0 else np.full(cap, 4294967295.0)
+    v = np.minimum(v, 4294967295.0)
+    v[0] = float(min(int(T), 4294967295))
+    v = np.maximum.accumulate(v)
+    n = int(np.argmax(v >= 4294967295.0)) + 1 if (v >= 4294967295.0).any() else cap
+    return v[:n].astype(np.uint32)
+
+
+def skip_flips(cdf, seed, subseq, first, rows, C):
+    """Flip masks [rows, ceil(C/64)] int64 by gap sampling (see nbo_skip_flips_i64)."""
+    cdf = _c(cdf, np.uint32)
+    out = np.empty((int(rows), (int(C) + 63) // 64), dtype=np.int64)
+    lib().nbo_skip_flips_i64(_p(out), _p(cdf), _i64(cdf.shape[0]), ctypes.c_uint64(int(seed)),
+                             ctypes.c_uint64(int(subseq)), ctypes.c_uint64(int(first)), _i64(rows), _i64(C))
+    return out
+
+
 def max_threads():
     return int(lib().nbo_max_threads())
 

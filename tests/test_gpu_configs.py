@@ -125,13 +125,20 @@ def test_config5_cifar_net(wk, ops, oracle):
     out = w.step()
     assert tuple(out.shape) == (D, 10) and out.dtype == torch.int32
     assert torch.equal(w.step(), out)                                      # deterministic
-    t = w.tensors
-    # the 8192 -> 1024 layer runs from the shared base + flip lists: the logits must be those of the materialised
+    t = dict(w.tensors)
+    # the 8192 -> 1024 layer runs from the shared base + flip lists (drawn by the skip sampler; the 4 GiB of weights
+    # are materialised here only to check): the logits must be those of the dense kernels on the materialised
     # weights, every member; and so must the layer itself on the net's real features and on random inputs with
     # thresholds around the sums
-    assert w.meta["fc"] == "base + flip lists"
+    assert w.meta["fc"].startswith("base + flip lists")
+    t["W4"] = w.meta["W4"]()
+    assert tuple(t["W4"].shape) == (D, 1024, 128)
+    rows4 = w.meta["rows4"]
+    rate = float(rows4.cnt.view(torch.int16).double().sum()) / (D * 1024 * 8192)
+    assert abs(rate - 0.01) < 2e-5                                          # Bernoulli(p = 0.01) per weight bit
+    assert torch.equal(ops.flip_rows_from_weights(t["W4"], t["b4"]).cnt, rows4.cnt)      # counted on the dense form
     assert torch.equal(w.meta["step_dense"](), out)
-    rows4, feats = w.meta["rows4"], w.meta["features"]()
+    feats = w.meta["features"]()
     assert torch.equal(ops.bmv_flip_act_pack(rows4, feats, w.meta["thr4"]), ops.bmv_act_pack(t["W4"], feats, w.meta["thr4"]))
     assert torch.equal(ops.bmv_flip(rows4, feats), ops.bmm(t["W4"], feats).squeeze(2))
     del feats
@@ -165,10 +172,10 @@ def test_config5_cifar_net(wk, ops, oracle):
             f = np.ascontiguousarray(Wn.reshape(1, O, 3, 3, 1).transpose(0, 2, 3, 4, 1).reshape(9, O))
             np.testing.assert_array_equal(t[name][m].cpu().numpy(), f, err_msg="%s member %d" % (name, m))
         W4m = t["W4"][m].cpu().numpy()
-        for r in (0, 1, 255, 256, 511, 777, 1022, 1023):
-            words = oracle.philox_words(seed, 13, (m * 1024 + r) * 8192, 8192).reshape(1, 1, 8192)
-            want = oracle.sample_from_words(T, words, np.int64, base=b4h[r:r + 1])
-            np.testing.assert_array_equal(W4m[r], want[0, 0], err_msg="W4 member %d row %d" % (m, r))
+        table = oracle.skip_cdf(T)
+        for r in (0, 1, 255, 256, 511, 777, 1022, 1023):                   # the skip sampler's walk, row by row
+            want = b4h[r] ^ oracle.skip_flips(table, seed, 13, (m * 1024 + r) * 8192, 1, 8192)[0]
+            np.testing.assert_array_equal(W4m[r], want, err_msg="W4 member %d row %d" % (m, r))
         np.testing.assert_array_equal(t["W5"][m].cpu().numpy(), host_member_weights(oracle, b5h, 1024, 10, T, seed, 14, m))
     for m in (0, 2047, 4095):
         a = t["x"][m:m + 1].cpu().numpy()                                  # [1,32,32,1]

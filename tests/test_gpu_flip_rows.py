@@ -164,3 +164,51 @@ def test_flip_shapes_are_checked(ops):
         ops._lib.call("nb_flip_count_i64", 256, 256, 256, 1, 4, 512, None)
     with pytest.raises(RuntimeError, match="whole tiles"):
         ops._lib.call("nb_bmm_nt_fp4", 256, 256, 256, 130, 4, 2, 128, 128, 2, None)
+
+
+@pytest.mark.parametrize("D,R,C,p,first", [(3, 64, 64, 0.1, 0), (2, 100, 200, 0.05, 8), (4, 1024, 8192, 0.01, 0),
+                                           (2, 1100, 128, 0.3, 3), (300, 128, 256, 0.02, 0), (2, 70, 3000, 0.0002, 5),
+                                           (2, 10, 64, 0.0, 0), (2, 130, 70, 1.0, 0), (3, 1, 1, 0.5, 1)])
+def test_skip_sampler_vs_oracle(ops, oracle, D, R, C, p, first):
+    """Flip lists drawn by the skip sampler == the oracle's restatement of the same walk (materialised through
+    flip_rows_to_weights), and the products from those lists == the oracle's bmm on the oracle's weights."""
+    g = np.random.default_rng(D + R + C)
+    Kw = (C + 63) // 64
+    T = min(int(p * 2 ** 32), 2 ** 32 - 1)
+    seed, sub = 0x5EED0000 + C, 21
+    base = sparse_mask(g, (R, C), 0.5)
+    table = ops.skip_table(T)
+    np.testing.assert_array_equal(table, oracle.skip_cdf(T))
+    want_W = base[None] ^ oracle.skip_flips(table, seed, sub, first, D * R, C).reshape(D, R, Kw)
+    rows = ops.flip_rows_skip(dev(base), C, D, T, seed, subsequence=sub, first=first)
+    flips = np.unpackbits((want_W ^ base[None]).view(np.uint8), axis=2, bitorder="little")
+    np.testing.assert_array_equal(host(rows.cnt).astype(np.int64), flips.sum(axis=2))
+    W = ops.flip_rows_to_weights(rows)
+    np.testing.assert_array_equal(host(W), want_W)
+    x = sparse_mask(g, (D, C), 0.5)
+    want = oracle.bmm(want_W, x.reshape(D, Kw, 1))[:, :, 0]
+    np.testing.assert_array_equal(host(ops.bmv_flip(rows, dev(x))), want)
+    assert torch.equal(ops.bmm(W, dev(x).view(D, Kw, 1)).squeeze(2), ops.bmv_flip(rows, dev(x)))
+    if D * R * C <= 500000:                                     # the lists themselves, entry by entry
+        mask, bflag = decode_flip_rows(rows)
+        np.testing.assert_array_equal(mask[:, :, :C], flips[:, :, :C].astype(bool))
+        base_bits = np.unpackbits(base.view(np.uint8), axis=1, bitorder="little").astype(bool)
+        np.testing.assert_array_equal(bflag, mask & base_bits[None])
+    # lists built from the materialised weights hold the same flips
+    again = ops.flip_rows_from_weights(W, dev(base))
+    assert torch.equal(again.cnt, rows.cnt) and torch.equal(ops.flip_rows_to_weights(again), W)
+
+
+def test_skip_sampler_rate_at_the_size_of_a_wide_layer(ops):
+    """8192 columns, p = 0.01, 64 members x 1024 rows: flip rate, row-count spread and column uniformity."""
+    T = 42949672
+    base = torch.zeros((1024, 128), dtype=torch.int64, device="cuda")
+    rows = ops.flip_rows_skip(base, 8192, 64, T, 7)
+    cnt = rows.cnt.view(torch.int16).to(torch.float64)
+    n = cnt.numel() * 8192
+    p = T / 2 ** 32
+    assert abs(float(cnt.sum()) / n - p) < 4 * (p / n) ** 0.5
+    assert abs(float(cnt.std()) - (8192 * p * (1 - p)) ** 0.5) < 0.1
+    W = ops.flip_rows_to_weights(rows)
+    per_col = ops.unpack(W.view(-1, 128)).view(64 * 1024, 8192).float().mean(dim=0)
+    assert float((per_col - p).abs().max()) < 6 * (p / (64 * 1024)) ** 0.5

@@ -247,3 +247,54 @@ def test_weighted_sum_matches_einsum(oracle, dtype):
     got = oracle.weighted_sum(words, w, C)
     want = np.einsum("n,nrc->rc", w.astype(np.float64), bits.astype(np.float64))
     np.testing.assert_allclose(got, want, rtol=1e-4, atol=1e-4)
+
+
+def test_skip_flips_against_searchsorted_and_the_geometric_law(oracle):
+    """Gap sampling of flip masks (the skip sampler's contract): the C restatement against an independent numpy
+    evaluation (searchsorted + cumsum over the Philox words, which the known-answer vectors pin), then what the law
+    fixes: flip rate p, geometric gap frequencies, no correlation between neighbouring columns."""
+    T = int(0.03 * 2 ** 32)
+    cdf = oracle.skip_cdf(T)
+    assert cdf[0] == T and cdf[-1] == 2 ** 32 - 1 and (np.diff(cdf.astype(np.int64)) >= 0).all()
+    p = T / 2.0 ** 32
+    np.testing.assert_allclose(cdf[:50] / 2.0 ** 32, 1 - (1 - p) ** np.arange(1, 51), atol=2 ** -31)
+    for rows, C, first in [(7, 200, 0), (3, 64, 5), (5, 1, 2), (4, 1000, 4 * 0xFFFFFFFF)]:
+        seed, sub = 0xABCDEF0123, 9
+        got = oracle.skip_flips(cdf, seed, sub, first, rows, C)
+        bits = np.unpackbits(got.view(np.uint8), axis=1, bitorder="little")[:, :((C + 63) // 64) * 64]
+        assert not bits[:, C:].any()
+        for q in range(rows):
+            words = oracle.philox_words(seed, sub, first + q * C, C)
+            rank = np.searchsorted(cdf, words, side="right").astype(np.int64)
+            pos = np.cumsum(np.where(rank < len(cdf), rank + 1, len(cdf))) - 1
+            want = np.zeros(bits.shape[1], np.uint8)
+            want[pos[(pos < C) & (rank < len(cdf))]] = 1
+            np.testing.assert_array_equal(bits[q], want, err_msg="rows=%d C=%d row %d" % (rows, C, q))
+    rows, C = 400, 4096
+    bits = np.unpackbits(oracle.skip_flips(cdf, 1, 2, 0, rows, C).view(np.uint8), axis=1, bitorder="little")
+    assert abs(bits.mean() - p) < 4 * np.sqrt(p * (1 - p) / bits.size)
+    assert abs(bits[:, 0].mean() - p) < 5 * np.sqrt(p / rows)                    # the first gap starts before column 0
+    cols = [np.flatnonzero(r) for r in bits]
+    gaps = np.concatenate([np.diff(c) for c in cols])
+    for k in range(1, 6):
+        expect = (1 - p) ** (k - 1) * p
+        assert abs((gaps == k).mean() - expect) < 5 * np.sqrt(expect / gaps.size), k
+    a, b = bits[:, :-1].astype(np.float64), bits[:, 1:].astype(np.float64)
+    assert abs((a * b).mean() - p * p) < 5 * p / np.sqrt(a.size)                 # neighbours independent
+    # a table cut short of saturation (tiny p): words beyond it move on without a flip, the rate stays p
+    T2 = 2 ** 32 // 5000
+    short = oracle.skip_cdf(T2, cap=64)
+    assert len(short) == 64 and short[-1] < 2 ** 32 - 1
+    got = oracle.skip_flips(short, 5, 1, 0, 300, 3000)
+    b2 = np.unpackbits(got.view(np.uint8), axis=1, bitorder="little")[:, :3000]
+    assert abs(b2.mean() - 1 / 5000) < 5 * np.sqrt(1 / 5000 / b2.size)
+    words = oracle.philox_words(5, 1, 7 * 3000, 3000)
+    rank = np.searchsorted(short, words, side="right").astype(np.int64)
+    pos = np.cumsum(np.where(rank < 64, rank + 1, 64)) - 1
+    want = np.zeros(3000, np.uint8)
+    want[pos[(pos < 3000) & (rank < 64)]] = 1
+    np.testing.assert_array_equal(b2[7], want)
+    # p = 1: every column flips (one word in 2**32 would skip one); p = 0: none
+    ones = oracle.skip_flips(oracle.skip_cdf(2 ** 32 - 1), 3, 0, 0, 4, 130)
+    assert np.unpackbits(ones.view(np.uint8), axis=1, bitorder="little")[:, :130].all()
+    assert not oracle.skip_flips(oracle.skip_cdf(0), 3, 0, 0, 4, 130).any()
