@@ -144,16 +144,17 @@ int nb_bmv_bn_act_static_i64(void *out, const int64_t *A, const int64_t *x, cons
  * (stream (seed, subseq), as nb_philox_words numbers them); word i has the rank #{k < Kt : cdf[k] <= word}: a rank
  * below Kt moves the position (start: -1) on by rank + 1 columns and flips the column reached, rank Kt moves it on by
  * Kt columns without a flip; the row ends when the position passes C.  cdf [Kt] uint32, sorted, Kt <= 4096, is
- * supplied by the caller: cdf[k-1] = floor(2^32 * (1 - (1-p)^k)); Kt == 0 means no flips.  Same law as
+ * supplied by the caller: cdf[k-1] = floor(2^32 * (1 - (1-p)^k)); Kt == 0 means no flips.  cdf0 = the table's first
+ * entry (p * 2^32) as a host value: a hint for where a look-up starts probing; it does not change any result.  Same law as
  * nb_sample_philox with a base and thr_scalar = p * 2^32 (i.i.d. Bernoulli(p), quantised to 2^-32), another stream.
  * nb_flip_skip_count: cnt[d, r] = number of flips of the row.   nb_flip_skip_fill: the entries, as nb_flip_fill.
  * nb_flip_to_dense: materialises flip lists: W [D, R, Kw] must hold base in every member on entry, every listed
  *                flip is XOR-ed in (interop with the dense kernels, and what the tests compare through). */
-int nb_flip_skip_count_i64(uint16_t *cnt, const uint32_t *cdf, int64_t Kt, uint64_t seed, uint64_t subseq, uint64_t first,
-                           int64_t D, int64_t R, int64_t C, nb_stream_t stream);
+int nb_flip_skip_count_i64(uint16_t *cnt, const uint32_t *cdf, uint32_t cdf0, int64_t Kt, uint64_t seed, uint64_t subseq,
+                           uint64_t first, int64_t D, int64_t R, int64_t C, nb_stream_t stream);
 int nb_flip_skip_fill_i64(uint32_t *entries, const int64_t *base, const uint16_t *perm, const int64_t *slice_off,
-                          const int32_t *slice_len, const uint32_t *cdf, int64_t Kt, uint64_t seed, uint64_t subseq,
-                          uint64_t first, int64_t D, int64_t R, int64_t C, nb_stream_t stream);
+                          const int32_t *slice_len, const uint32_t *cdf, uint32_t cdf0, int64_t Kt, uint64_t seed,
+                          uint64_t subseq, uint64_t first, int64_t D, int64_t R, int64_t C, nb_stream_t stream);
 int nb_flip_to_dense_i64(int64_t *W, const uint32_t *entries, const int64_t *slice_off, const int32_t *slice_len,
                          const uint16_t *perm, int64_t D, int64_t R, int64_t Kw, nb_stream_t stream);
 int nb_flip_count_i64(uint16_t *cnt, const int64_t *W, const int64_t *base, int64_t D, int64_t R, int64_t Kw,

@@ -16,6 +16,7 @@
 // their complements in LDS (piece, ~piece, piece, ~piece ...: 4Kw dwords, then one zero dword for the sentinel 4Kw),
 // so that the looked-up bit already is x ^ b.  The rows of a slice move through the columns at about the same pace,
 // so at any moment the 64 lanes look into a narrow window of the table: neighbouring dwords, different banks.
+#include <cmath>
 #include <type_traits>
 
 #include "nb_common.hpp"
@@ -278,20 +279,21 @@ struct SkipChain {
     }
 };
 
-// number of table entries <= u (the table is sorted): thirteen fixed probes, no divergence
-__device__ __forceinline__ int skip_rank(const uint32_t *tab, int Kt, uint32_t u)
+// Number of table entries <= u (the table is sorted).  The entries follow 2^32 * (1 - q^k), so
+// log2(1 - u / 2^32) / log2(q) lands within a step or two of the answer; the walk from there is against the table
+// itself, which keeps the result exact whatever the float arithmetic does (a wrong estimate only costs probes).
+__device__ __forceinline__ int skip_rank(const uint32_t *tab, int Kt, uint32_t u, float inv_log2q)
 {
-    int lo = 0;
-#pragma unroll
-    for (int step = kSkipMaxTable; step > 0; step >>= 1) {
-        const int idx = lo + step;
-        if (idx <= Kt && tab[idx - 1] <= u) lo = idx;
-    }
-    return lo;
+    const float s = ((float)(~u) + 1.0f) * 2.3283064365386963e-10f;  // 1 - u / 2^32, from the complement: no cancellation
+    int est = (int)(__log2f(s) * inv_log2q);
+    est = est < 0 ? 0 : (est > Kt ? Kt : est);
+    while (est < Kt && tab[est] <= u) est++;
+    while (est > 0 && tab[est - 1] > u) est--;
+    return est;
 }
 
 __global__ __launch_bounds__(256) void fl_skip_count_kernel(uint16_t *__restrict__ cnt, const uint32_t *__restrict__ cdf,
-                                                            int Kt, PhiloxKey key, int64_t rows, int C)
+                                                            int Kt, float inv_log2q, PhiloxKey key, int64_t rows, int C)
 {
     __shared__ uint32_t tab[kSkipMaxTable];
     for (int i = threadIdx.x; i < Kt; i += 256) tab[i] = cdf[i];
@@ -303,7 +305,7 @@ __global__ __launch_bounds__(256) void fl_skip_count_kernel(uint16_t *__restrict
         SkipChain chain(key, key.first + (uint64_t)q * (uint64_t)C);
         int pos = -1;
         for (;;) {
-            const int rank = skip_rank(tab, Kt, chain.next());
+            const int rank = skip_rank(tab, Kt, chain.next(), inv_log2q);
             pos += rank < Kt ? rank + 1 : Kt;
             if (pos >= C) break;
             n += rank < Kt ? 1 : 0;
@@ -317,8 +319,9 @@ __global__ __launch_bounds__(256) void fl_skip_fill_kernel(uint32_t *__restrict_
                                                            const uint16_t *__restrict__ perm,
                                                            const int64_t *__restrict__ slice_off,
                                                            const int32_t *__restrict__ slice_len,
-                                                           const uint32_t *__restrict__ cdf, int Kt, PhiloxKey key,
-                                                           int64_t nslices, int S, int64_t R, int Kw, int C)
+                                                           const uint32_t *__restrict__ cdf, int Kt, float inv_log2q,
+                                                           PhiloxKey key, int64_t nslices, int S, int64_t R, int Kw,
+                                                           int C)
 {
     __shared__ uint32_t tab[kSkipMaxTable];
     for (int i = threadIdx.x; i < Kt; i += 256) tab[i] = cdf[i];
@@ -344,7 +347,7 @@ __global__ __launch_bounds__(256) void fl_skip_fill_kernel(uint32_t *__restrict_
         SkipChain chain(key, key.first + (uint64_t)(d * R + r) * (uint64_t)C);
         int pos = -1;
         for (;;) {
-            const int rank = skip_rank(tab, Kt, chain.next());
+            const int rank = skip_rank(tab, Kt, chain.next(), inv_log2q);
             pos += rank < Kt ? rank + 1 : Kt;
             if (pos >= C) break;
             if (rank >= Kt) continue;  // a word beyond the table: moved on, no flip
@@ -609,10 +612,19 @@ int nb_flip_fill_i64(uint32_t *entries, const int64_t *W, const int64_t *base, c
     return nb::check_launch(who);
 }
 
-int nb_flip_skip_count_i64(uint16_t *cnt, const uint32_t *cdf, int64_t Kt, uint64_t seed, uint64_t subseq, uint64_t first,
-                           int64_t D, int64_t R, int64_t C, nb_stream_t stream)
+// 1 / log2(1 - p) for the table's first entry p * 2^32: only a hint for where a look-up starts probing
+static float skip_hint(uint32_t cdf0)
+{
+    const double p = (double)cdf0 / 4294967296.0;
+    if (p <= 0.0 || p >= 1.0) return 0.0f;
+    return (float)(1.0 / std::log2(1.0 - p));
+}
+
+int nb_flip_skip_count_i64(uint16_t *cnt, const uint32_t *cdf, uint32_t cdf0, int64_t Kt, uint64_t seed, uint64_t subseq,
+                           uint64_t first, int64_t D, int64_t R, int64_t C, nb_stream_t stream)
 {
     const char *who = "nb_flip_skip_count_i64";
+    const float inv_log2q = skip_hint(cdf0);
     NB_REQUIRE(C >= 0 && Kt >= 0 && Kt <= nb::kSkipMaxTable, "%s: bad C=%lld or table of %lld entries (at most %d)", who,
                (long long)C, (long long)Kt, nb::kSkipMaxTable);
     if (int rc = nb::flip_shape_check(D, R, (C + 63) / 64, who)) return rc;
@@ -624,15 +636,16 @@ int nb_flip_skip_count_i64(uint16_t *cnt, const uint32_t *cdf, int64_t Kt, uint6
     const int64_t blocks = nb::ceil_div(D * R, 256);
     NB_REQUIRE(blocks <= nb::kMaxGridX, "%s: too many rows for one launch", who);
     nb::fl_skip_count_kernel<<<dim3((unsigned)blocks), dim3(256), 0, nb::as_stream(stream)>>>(
-        cnt, cdf, (int)Kt, nb::PhiloxKey{seed, subseq, first}, D * R, (int)C);
+        cnt, cdf, (int)Kt, inv_log2q, nb::PhiloxKey{seed, subseq, first}, D * R, (int)C);
     return nb::check_launch(who);
 }
 
 int nb_flip_skip_fill_i64(uint32_t *entries, const int64_t *base, const uint16_t *perm, const int64_t *slice_off,
-                          const int32_t *slice_len, const uint32_t *cdf, int64_t Kt, uint64_t seed, uint64_t subseq,
-                          uint64_t first, int64_t D, int64_t R, int64_t C, nb_stream_t stream)
+                          const int32_t *slice_len, const uint32_t *cdf, uint32_t cdf0, int64_t Kt, uint64_t seed,
+                          uint64_t subseq, uint64_t first, int64_t D, int64_t R, int64_t C, nb_stream_t stream)
 {
     const char *who = "nb_flip_skip_fill_i64";
+    const float inv_log2q = skip_hint(cdf0);
     NB_REQUIRE(C >= 0 && Kt >= 0 && Kt <= nb::kSkipMaxTable, "%s: bad C=%lld or table of %lld entries (at most %d)", who,
                (long long)C, (long long)Kt, nb::kSkipMaxTable);
     const int64_t Kw = (C + 63) / 64;
@@ -652,7 +665,7 @@ int nb_flip_skip_fill_i64(uint32_t *entries, const int64_t *base, const uint16_t
     NB_REQUIRE_ALIGNED(base, 8);
     const int64_t S = (R + 63) / 64;
     nb::fl_skip_fill_kernel<<<dim3((unsigned)nb::ceil_div(D * S, 4)), dim3(256), 0, nb::as_stream(stream)>>>(
-        entries, reinterpret_cast<const uint64_t *>(base), perm, slice_off, slice_len, cdf, (int)Kt,
+        entries, reinterpret_cast<const uint64_t *>(base), perm, slice_off, slice_len, cdf, (int)Kt, inv_log2q,
         nb::PhiloxKey{seed, subseq, first}, D * S, (int)S, R, (int)Kw, (int)C);
     return nb::check_launch(who);
 }

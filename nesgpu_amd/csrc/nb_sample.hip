@@ -5,6 +5,8 @@
 // (supplied) or word first+(m*R+r)*C+c of a Philox4x32-10 stream.  The supplied stream is
 // 4 bytes per weight bit, so these kernels are HBM-bound on it: lanes read it with 16-byte
 // loads at consecutive addresses and every word is touched exactly once.
+#include <type_traits>
+
 #include "nb_common.hpp"
 
 namespace nb {
@@ -153,6 +155,41 @@ __global__ __launch_bounds__(256) void sample_ballot_kernel(W *__restrict__ out,
                     if (wi + 1 < Rw) put(wi + 1, (W)(m >> 32));
                 }
             }
+        }
+    }
+}
+
+// ---- materialised sampler, rows shorter than a word: one lane per (member,row) -----------------------------------------
+// (the first conv layer of an RGB network has 3 columns per row, a 16-channel layer 16: a wave per row would leave
+// most lanes idle).  The generator is asked block by block: a block's four words are consecutive columns.
+template <typename W, class Src>
+__global__ __launch_bounds__(256) void sample_narrow_kernel(W *__restrict__ out, const W *__restrict__ base,
+                                                            const uint32_t *__restrict__ thresh, uint32_t ts, Src src,
+                                                            int64_t nrows, int64_t R, int C, ConvOut<W> conv)
+{
+    NB_FLAT_LOOP(row, nrows)
+    {
+        if (row < nrows) {
+            const int64_t r = row % R;
+            const uint32_t *__restrict__ tr = thresh ? thresh + r * C : nullptr;
+            W v = 0;
+            if constexpr (std::is_same<Src, PhiloxSrc>::value) {
+                const uint64_t g0 = src.key.first + (uint64_t)row * (uint64_t)C;
+                for (uint64_t blk = g0 >> 2; blk <= (g0 + (uint64_t)C - 1) >> 2; blk++) {
+                    const uint4 b = philox_block(src.key, blk);
+                    const uint32_t w4[4] = {b.x, b.y, b.z, b.w};
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const int64_t c = (int64_t)(blk * 4 + e - g0);  // column of this word, if it is one of the row's
+                        if (c >= 0 && c < C) v |= (W)(w4[e] < (tr ? tr[c] : ts)) << c;
+                    }
+                }
+            } else {
+                for (int c = 0; c < C; c++) v |= (W)(src.load1(row * C + c) < (tr ? tr[c] : ts)) << c;
+            }
+            v ^= base ? base[r] : (W)0;
+            if (out) out[row] = v;
+            if (conv.out2) conv.out2[(row / R) * R + conv.at((uint32_t)r, 0u, 1u)] = v;
         }
     }
 }
@@ -388,6 +425,9 @@ int sample_impl(W *out, const W *base, const uint32_t *thresh, uint32_t ts, Src 
         else if (base) NB_LAUNCH_WIDE(false, true);
         else NB_LAUNCH_WIDE(false, false);
 #undef NB_LAUNCH_WIDE
+    } else if (C < bits) {
+        sample_narrow_kernel<W, Src><<<dim3(grid_for(n * R)), dim3(256), 0, s>>>(out, base, thresh, ts, src, n * R, R,
+                                                                               (int)C, conv);
     } else {
         sample_ballot_kernel<W, Src><<<dim3(grid_for(n * R * 64)), dim3(256), 0, s>>>(
             out, base, thresh, ts, src, n * R, R, (int)C, (int)Rw, conv);

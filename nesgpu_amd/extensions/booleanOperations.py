@@ -762,15 +762,16 @@ def flip_rows_skip(base, in_bits, n, threshold, seed, subsequence=0, first=0):
     table = skip_table(threshold)
     cdf = torch.from_numpy(table.view("int32").copy()).to(dev).view(torch.uint32) if table.size else None
     cptr, Kt = (cdf.data_ptr(), int(table.size)) if cdf is not None else (None, 0)
+    cdf0 = int(table[0]) if table.size else 0
     cnt = torch.empty((n, R), dtype=torch.uint16, device=dev)
     key = (int(seed) & (2 ** 64 - 1), int(subsequence), int(first))
     with _on(base):
-        _lib.call("nb_flip_skip_count_i64", cnt.data_ptr(), cptr, Kt, *key, n, R, C, _stream(base))
+        _lib.call("nb_flip_skip_count_i64", cnt.data_ptr(), cptr, cdf0, Kt, *key, n, R, C, _stream(base))
     perm, slice_len, slice_off, total = _flip_rows_layout(cnt, n, R)
     entries = torch.empty((max(total, 4),), dtype=torch.uint32, device=dev)
     with _on(base):
         _lib.call("nb_flip_skip_fill_i64", entries.data_ptr(), base.data_ptr(), perm.data_ptr(), slice_off.data_ptr(),
-                  slice_len.data_ptr(), cptr, Kt, *key, n, R, C, _stream(base))
+                  slice_len.data_ptr(), cptr, cdf0, Kt, *key, n, R, C, _stream(base))
     return FlipRows(base, n, R, Kw, cnt, perm, slice_off, slice_len, entries)
 
 
