@@ -25,10 +25,17 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 
-# HBM bytes per launch of the headline kernel from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE in KiB per
-# dispatch, each scaled by what the same counter reads for the 2 GiB calibration copy kernel: x2.0 and x1.0);
-# the summary with the commands is kept under profiles/.
-MEASURED_TRAFFIC_BYTES = 4300908544
+def measured_traffic():
+    """HBM bytes per launch of the headline kernel from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE in KiB per
+    dispatch, each scaled by what the same counter reads for the 2 GiB calibration copy kernel).  The counter
+    readings live in profiles/headline_traffic.json, next to the summary that quotes them; None if that file is gone."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "headline_traffic.json")) as f:
+            t = json.load(f)
+        return int(round((t["fetch_kib_per_dispatch"] * t["fetch_scale"]
+                          + t["write_kib_per_dispatch"] * t["write_scale"]) * 1024))
+    except (OSError, KeyError, ValueError):
+        return None
 
 
 def parse_args():
@@ -258,7 +265,7 @@ def calibrate(torch):
     return res
 
 
-def hbm_kernels(torch, steps, warmup):
+def hbm_kernels(torch, steps, warmup, graph=True):
     """Each HBM-bound kernel of the path alone, at a configuration-sized shape: algorithmic bytes / event time."""
     from nesgpu_amd import workloads
     from nesgpu_amd.extensions import booleanOperations as ops
@@ -267,7 +274,7 @@ def hbm_kernels(torch, steps, warmup):
 
     def run(name, fn, nbytes):
         pw, pe = time_steps(torch, fn, steps, warmup)
-        pg = time_graph(torch, fn, steps)                  # device time without the host's launch pacing
+        pg = time_graph(torch, fn, steps) if graph else None   # device time without the host's launch pacing
         t = pg if pg else pe
         res.append({"kernel": name, "us": round(t * 1e6, 2), "GBps": round(nbytes / t / 1e9, 1),
                     "hbm_frac": round(nbytes / t / workloads.HBM_PEAK, 4), "algorithmic_bytes": nbytes,
@@ -305,6 +312,30 @@ def hbm_kernels(torch, steps, warmup):
     xv = torch.randint(-2 ** 62, 2 ** 62, (1024, 128, 1), device=dev, generator=g, dtype=torch.int64)
     run("bmm N=1 [1024,1024,128]", lambda: ops.bmm(W, xv), W.numel() * 8 + xv.numel() * 8 + 1024 * 1024 * 4)
     del W, xv
+    # config 1's kernel: rows of 32 bytes, one row per lane
+    W1 = torch.randint(-2 ** 62, 2 ** 62, (1024, 256, 4), device=dev, generator=g, dtype=torch.int64)
+    x1 = torch.randint(-2 ** 62, 2 ** 62, (1024, 4, 1), device=dev, generator=g, dtype=torch.int64)
+    run("bmm N=1 [1024,256,4] (config 1)", lambda: ops.bmm(W1, x1), W1.numel() * 8 + x1.numel() * 8 + 1024 * 256 * 4)
+    del W1, x1
+    # sparse form of config 5's 8192 -> 1024 layer at D = 4096: flip lists drawn by the skip sampler
+    b4 = torch.randint(-2 ** 62, 2 ** 62, (1024, 128), device=dev, generator=g, dtype=torch.int64)
+    rows = ops.flip_rows_skip(b4, 8192, 4096, workloads.T_P01, 0, subsequence=13)
+    x4 = torch.randint(-2 ** 62, 2 ** 62, (4096, 128), device=dev, generator=g, dtype=torch.int64)
+    thr4 = torch.full((4096, 1024), 8192, dtype=torch.int32, device=dev)
+    ex = ops.expand_rows(x4)
+    G = ops.bmm_nt(ex, rows.base_expanded)
+    run("expand_rows [4096,128] -> FP4 codes", lambda: ops.expand_rows(x4), x4.numel() * 8 + ex.codes.numel())
+    run("bmm_nt 4096 x 1024 x 8192 bits (FP4 matrix cores; bytes: operands once + int32 out)",
+        lambda: ops.bmm_nt(ex, rows.base_expanded), ex.codes.numel() + rows.base_expanded.codes.numel() + G.numel() * 4)
+    run("bmv_flip_act_pack D=4096 [1024 x 8192], p=0.01 (lists + counts + order + G + thresholds)",
+        lambda: ops.bmv_flip_act_pack(rows, x4, thr4, G=G), rows.nbytes() + G.numel() * 4 + thr4.numel() * 4 + x4.numel() * 8)
+    run("flip_rows_skip D=4096 [1024 x 8192], p=0.01 (bytes written)",
+        lambda: ops.flip_rows_skip(b4, 8192, 4096, workloads.T_P01, 0, subsequence=13), rows.nbytes())
+    del rows, x4, thr4, ex, G
+    # first-layer filters of an RGB network: rows of 3 columns, one lane per row
+    b1 = torch.randint(0, 8, (576, 1), device=dev, generator=g, dtype=torch.int64)
+    run("sample (3-column rows) D=4096 x 576 rows, generator mode",
+        lambda: ops.sample_bits_philox(workloads.T_P01, 4096, torch.int64, 0, 10, base=b1, shape=(576, 3)), 4096 * 576 * 8)
     # update step: weighted sum of the population's masks of a 1024x1024 layer (one fp32 add per member and weight
     # bit in member order: the vector ALUs, not HBM, bound it; the fraction is reported for comparison)
     m = torch.randint(-2 ** 62, 2 ** 62, (1024, 1024, 16), device=dev, generator=g, dtype=torch.int64)
@@ -332,7 +363,7 @@ def main():
         return 0
 
     if args.kernels:
-        print(json.dumps({"hbm_kernels": hbm_kernels(torch, args.steps, args.warmup)}))
+        print(json.dumps({"hbm_kernels": hbm_kernels(torch, args.steps, args.warmup, not args.no_graph)}))
         return 0
     if args.only:
         w = workloads.BUILDERS[args.only]()
@@ -356,7 +387,7 @@ def main():
         "config": {"workload": wl.name, "population": wl.population, "word_bits": 64,
                    "bit_macs_per_step": wl.bit_macs},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": workloads.HBM_PEAK / 1e9, "unit": "GB/s",
-                     "frac": round(achieved * 1e9 / workloads.HBM_PEAK, 4), "traffic": MEASURED_TRAFFIC_BYTES,
+                     "frac": round(achieved * 1e9 / workloads.HBM_PEAK, 4), "traffic": measured_traffic(),
                      "kernel": "seeded_bmv_stream_kernel", "algorithmic_bytes_per_launch": wl.algo_bytes,
                      "avg_launch_ms": round(per_ev * 1e3, 4)},
     }

@@ -218,12 +218,22 @@ __global__ __launch_bounds__(256) void fl_fill_kernel(uint32_t *__restrict__ ent
     int64_t r = valid ? perm[d * R + p] : 0;
     r = r < R ? r : R - 1;
     const int L = 4 * slice_len[sl];  // dwords per lane; dword j of lane l sits at piece j / 4, component j % 4
-    uint32_t *dst = entries + slice_off[sl] + lane * 4;
-    auto at = [](int j) { return (int64_t)(j >> 2) * 256 + (j & 3); };
+    uint4 *dst = reinterpret_cast<uint4 *>(entries + slice_off[sl]) + lane;
     const uint32_t sentinel = (uint32_t)(4 * Kw) << 5;
     int j = 0;
     uint32_t pend = 0;
     bool half = false;
+    // a lane's dwords leave four at a time, as whole 16-byte pieces (L is a multiple of 4); never past the slice,
+    // whatever the inputs
+    uint32_t q0 = 0, q1 = 0, q2 = 0;
+    auto put = [&](uint32_t v) {
+        const int c = j & 3;
+        if (c == 0) q0 = v;
+        else if (c == 1) q1 = v;
+        else if (c == 2) q2 = v;
+        else if (j < L) dst[(int64_t)(j >> 2) * 64] = make_uint4(q0, q1, q2, v);
+        j++;
+    };
     if (valid) {
         const uint64_t *w = W + (d * R + r) * Kw, *b = base + r * Kw;
         for (int k = 0; k < Kw; k++) {
@@ -239,18 +249,14 @@ __global__ __launch_bounds__(256) void fl_fill_kernel(uint32_t *__restrict__ ent
                     pend = e;
                     half = true;
                 } else {
-                    if (j < L) dst[at(j)] = pend | (e << 16);  // never past the slice, whatever the inputs
-                    j++;
+                    put(pend | (e << 16));
                     half = false;
                 }
             }
         }
     }
-    if (half) {
-        if (j < L) dst[at(j)] = pend | (sentinel << 16);
-        j++;
-    }
-    for (; j < L; j++) dst[at(j)] = sentinel | (sentinel << 16);
+    if (half) put(pend | (sentinel << 16));
+    while (j < L) put(sentinel | (sentinel << 16));
 }
 
 // ---- skip sampler: flip lists straight from the generator, without ever drawing the bits that do not flip -----------
@@ -336,12 +342,22 @@ __global__ __launch_bounds__(256) void fl_skip_fill_kernel(uint32_t *__restrict_
     int64_t r = valid ? perm[d * R + p] : 0;
     r = r < R ? r : R - 1;
     const int L = 4 * slice_len[sl];
-    uint32_t *dst = entries + slice_off[sl] + lane * 4;
-    auto at = [](int j) { return (int64_t)(j >> 2) * 256 + (j & 3); };
+    uint4 *dst = reinterpret_cast<uint4 *>(entries + slice_off[sl]) + lane;
     const uint32_t sentinel = (uint32_t)(4 * Kw) << 5;
     int j = 0;
     uint32_t pend = 0;
     bool half = false;
+    // a lane's dwords leave four at a time, as whole 16-byte pieces (L is a multiple of 4); never past the slice,
+    // whatever the inputs
+    uint32_t q0 = 0, q1 = 0, q2 = 0;
+    auto put = [&](uint32_t v) {
+        const int c = j & 3;
+        if (c == 0) q0 = v;
+        else if (c == 1) q1 = v;
+        else if (c == 2) q2 = v;
+        else if (j < L) dst[(int64_t)(j >> 2) * 64] = make_uint4(q0, q1, q2, v);
+        j++;
+    };
     if (valid && Kt > 0) {
         const uint64_t *b = base + r * Kw;
         SkipChain chain(key, key.first + (uint64_t)(d * R + r) * (uint64_t)C);
@@ -358,17 +374,13 @@ __global__ __launch_bounds__(256) void fl_skip_fill_kernel(uint32_t *__restrict_
                 pend = e;
                 half = true;
             } else {
-                if (j < L) dst[at(j)] = pend | (e << 16);
-                j++;
+                put(pend | (e << 16));
                 half = false;
             }
         }
     }
-    if (half) {
-        if (j < L) dst[at(j)] = pend | (sentinel << 16);
-        j++;
-    }
-    for (; j < L; j++) dst[at(j)] = sentinel | (sentinel << 16);
+    if (half) put(pend | (sentinel << 16));
+    while (j < L) put(sentinel | (sentinel << 16));
 }
 
 // Flip lists -> materialised weights: W must hold the base in every member on entry; every flip is XOR-ed in.  A
