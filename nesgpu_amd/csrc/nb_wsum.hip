@@ -5,7 +5,7 @@
 
 namespace nb {
 
-// One wave per (row, 64-bit column): lane z owns output bit z of the column and adds the members' weights in member
+// Rows of any length.  One wave per (row, 64-bit column): lane z owns output bit z of the column and adds the members' weights in member
 // order (the reference's order, so the fp32 sums are the same).  Members are taken 64 at a time: lane j fetches the
 // column word of member m0 + j (64 strided loads in flight at once instead of one load per loop step), the
 // workgroup's four waves share the chunk's weights as fp32 in LDS, and then for each member its word, read out of
@@ -58,6 +58,79 @@ __global__ __launch_bounds__(256) void weighted_sum_kernel(_Float16 *__restrict_
     if (live && z < zbits) ret[r * zbits + z] = (_Float16)acc;
 }
 
+// Rows whose length is a multiple of 32 bytes: one wave per (row, 32-byte piece), a workgroup's four waves on four
+// consecutive pieces, so that every 128-byte line of every member's row is fetched by one workgroup, once, in one
+// 32-byte access per lane (lane j holds the piece of member m0 + j in 8 registers; the next 64 members' pieces are
+// requested before the current ones are used).  The piece holds four 64-bit columns; lane z owns output bit z of
+// each and keeps four running sums, all in member order.  The members' words reach the lanes through LDS instead
+// of v_readlane: the wave stores its 64 pieces split into the low and the high halves of the four columns, and lane
+// z reads, per member, the 16 bytes that hold its half of all four columns (one broadcast read).  Per member and
+// column that leaves v_bfe_i32 (bit z as 0 / -1), v_and with the member's weight and v_add: three vector
+// instructions and no scalar operand, against two lane reads, an LDS read, a select and an add above.  (A wave per
+// 64-byte piece with eight sums measured the same or slower: half as many waves to hide the LDS reads behind.)
+#define NB_WS_COL(ACC, D) ACC += __builtin_bit_cast(float, __builtin_amdgcn_sbfe((int)(D), zz, 1u) & wbits);
+
+__global__ __launch_bounds__(256) void weighted_sum_line_kernel(_Float16 *__restrict__ ret,
+                                                                const uint4 *__restrict__ in,
+                                                                const _Float16 *__restrict__ w, int64_t n, int64_t R,
+                                                                int row16, int zbits, int npiece)
+{
+    __shared__ uint4 msk[2][4][2][64];  // [buffer][wave][low halves, high halves][member]
+    __shared__ float wsh[2][64];
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const int64_t pid = (int64_t)blockIdx.x * 4 + wv;  // (row, piece); past the end: idle but in step
+    const bool live = pid < R * npiece;
+    const int64_t r = live ? pid / npiece : 0;
+    const int g = live ? (int)(pid - r * npiece) : 0;
+    const int64_t stride16 = R * (int64_t)row16;
+    const uint4 *p = in + r * row16 + (int64_t)g * 2;
+    const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
+    const uint32_t zz = lane & 31;
+    const int half = lane >> 5;
+    float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+    uint4 a0 = zero, a1 = zero;  // members past n contribute zero words: nothing is added for them
+    float wa = 0.f;
+    if (live && lane < n) {
+        const uint4 *q = p + lane * stride16;
+        a0 = load_stream16(q), a1 = load_stream16(q + 1);
+    }
+    if (wv == 0 && lane < n) wa = (float)w[lane];
+    int buf = 0;
+    for (int64_t m0 = 0; m0 < n; m0 += 64, buf ^= 1) {
+        msk[buf][wv][0][lane] = make_uint4(a0.x, a0.z, a1.x, a1.z);
+        msk[buf][wv][1][lane] = make_uint4(a0.y, a0.w, a1.y, a1.w);
+        if (wv == 0) wsh[buf][lane] = wa;
+        // one barrier per chunk: a buffer is written again two chunks later, after every wave has passed the barrier
+        // of the chunk in between and so has finished reading it
+        __syncthreads();
+        a0 = a1 = zero;
+        wa = 0.f;
+        if (live && m0 + 64 + lane < n) {
+            const uint4 *q = p + (m0 + 64 + lane) * stride16;
+            a0 = load_stream16(q), a1 = load_stream16(q + 1);
+        }
+        if (wv == 0 && m0 + 64 + lane < n) wa = (float)w[m0 + 64 + lane];
+        const uint4 *mine = &msk[buf][wv][half][0];
+#pragma unroll 8
+        for (int j = 0; j < 64; j++) {
+            const int wbits = __builtin_bit_cast(int, wsh[buf][j]);
+            const uint4 d = mine[j];
+            NB_WS_COL(s0, d.x)
+            NB_WS_COL(s1, d.y)
+            NB_WS_COL(s2, d.z)
+            NB_WS_COL(s3, d.w)
+        }
+    }
+    if (!live) return;
+    _Float16 *o = ret + r * zbits;
+    const int z = g * 256 + lane;
+    if (z < zbits) o[z] = (_Float16)s0;
+    if (z + 64 < zbits) o[z + 64] = (_Float16)s1;
+    if (z + 128 < zbits) o[z + 128] = (_Float16)s2;
+    if (z + 192 < zbits) o[z + 192] = (_Float16)s3;
+}
+#undef NB_WS_COL
+
 template <typename W>
 int weighted_sum_impl(uint16_t *ret, const W *in, const uint16_t *w, int64_t n, int64_t R, int64_t Rw, int64_t zbits,
                       nb_stream_t stream, const char *who)
@@ -74,6 +147,16 @@ int weighted_sum_impl(uint16_t *ret, const W *in, const uint16_t *w, int64_t n, 
     }
     NB_REQUIRE(zbits <= (1 << 30) && Rw <= (1 << 30), "%s: row too long", who);
     NB_REQUIRE(zbits <= Rw * (int64_t)WordTraits<W>::bits, "%s: zbits exceeds the Rw words of a row", who);
+    const int64_t rowbytes = Rw * (int64_t)sizeof(W);
+    if (n > 0 && rowbytes % 32 == 0 && (reinterpret_cast<uintptr_t>(in) & 15) == 0) {
+        const int64_t npiece = ceil_div(zbits, 256);  // 32-byte pieces of a row that hold output bits
+        const int64_t blocks = ceil_div(R * npiece, 4);
+        NB_REQUIRE(blocks <= kMaxGridX, "%s: output exceeds one launch", who);
+        weighted_sum_line_kernel<<<dim3((unsigned)blocks), dim3(256), 0, as_stream(stream)>>>(
+            reinterpret_cast<_Float16 *>(ret), reinterpret_cast<const uint4 *>(in),
+            reinterpret_cast<const _Float16 *>(w), n, R, (int)(rowbytes / 16), (int)zbits, (int)npiece);
+        return check_launch(who);
+    }
     const int64_t ncol = ceil_div(zbits, 64);
     const int64_t blocks = ceil_div(R * ncol, 4);
     NB_REQUIRE(blocks <= kMaxGridX, "%s: output exceeds one launch", who);
