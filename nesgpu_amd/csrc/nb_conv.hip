@@ -274,6 +274,14 @@ int conv_impl(void *out, const W *in, const W *filt, const int32_t *thresh, int6
         t_last_engine = 1;
         return check_launch(who);
     }
+    // Narrow layers (at most 16 channels in and out, threshold bits out): a wave per strip of 16 output columns on
+    // the int8 matrix cores, no staged image; any population size.
+    if (bits == 64 && Cw > 0 && engine != 1 &&
+        conv_direct_try(out, reinterpret_cast<const uint64_t *>(in), reinterpret_cast<const uint64_t *>(filt), thresh, g,
+                        D, N, tap_bits, mode, s)) {
+        t_last_engine = 2;
+        return check_launch(who);
+    }
     if (bits == 64 && Cw > 0 && engine != 1 && (engine >= 2 || D >= 128)) {
         const int ran = conv_mfma_try(out, reinterpret_cast<const uint64_t *>(in), reinterpret_cast<const uint64_t *>(filt),
                                       thresh, g, D, N, tap_bits, mode, engine != 3, s);

@@ -577,6 +577,65 @@ def test_conv_matrix_core_engine_vs_oracle(ops, oracle, mc_engine, C, O, k, pad,
         ops.conv_engine(prev)
 
 
+# (C, O, fy, px, py, H, W, D): the wave-per-strip matrix-core kernel for narrow layers (at most 16 channels in and
+# out, packed output).  Output channel counts below 16, channel counts that leave zero positions in a pixel's 16,
+# one to three filter columns, paddings 0-2, images of one to three rows (the short sub-band path), odd heights (the
+# pooled map drops the last row), several sub-bands with 13 to 20 rows (every remainder of the four-row loop),
+# several strips with a ragged last one, and a population large enough for whole-image sub-bands.
+NARROW_CASES = [
+    (16, 16, 3, 1, 1, 20, 18, 3),
+    (16, 5, 3, 1, 1, 19, 33, 2),
+    (7, 16, 3, 1, 1, 67, 20, 2),
+    (13, 9, 2, 0, 1, 73, 17, 1),
+    (1, 1, 3, 2, 2, 9, 9, 4),
+    (16, 16, 1, 1, 0, 35, 70, 2),
+    (12, 3, 3, 0, 0, 3, 40, 3),
+    (16, 16, 3, 1, 1, 1, 16, 5),
+    (16, 16, 3, 1, 1, 2, 5, 5),
+    (5, 16, 3, 2, 1, 3, 3, 2),
+    (16, 11, 3, 1, 1, 50, 48, 1),
+    (9, 16, 3, 1, 2, 38, 31, 3),
+    (16, 16, 3, 1, 1, 21, 16, 300),
+]
+
+
+@pytest.mark.parametrize("C,O,fy,px,py,H,W,D", NARROW_CASES)
+def test_conv_narrow_matrix_core_kernel_vs_oracle(ops, oracle, C, O, fy, px, py, H, W, D):
+    """Packed and pooled outputs of narrow layers against the oracle, thresholds spread around the sums (and one
+    always / one never above), filter tap-packed by the caller and on the fly, and identical to the XOR-popcount
+    kernels' answer."""
+    g = rng(C * 1000 + O * 10 + fy + H + W)
+    x = oracle.pack(g.integers(0, 2, size=(D * H * W, C)).astype(bool), np.int64).reshape(D, H, W, 1)
+    fb = g.integers(0, 2, size=(D * O * 3 * fy, C)).astype(bool)
+    f = np.ascontiguousarray(oracle.pack(fb, np.int64).reshape(D, O, 3, fy, 1).transpose(0, 2, 3, 4, 1).reshape(D, -1, O))
+    K = 3 * fy * C
+    thr = (g.integers(0, K + 3, size=(D, O)) - K // 2 + K - 1).astype(np.int32)
+    thr[0, 0] = -7
+    if O > 1:
+        thr[0, 1] = 2 * K + 5
+    geom = (3, fy, px, py, 1, 1)
+    act = oracle.conv_act(x, f, thr, *geom)
+    h, w = act.shape[1:3]
+    packed = oracle.pack(act.reshape(-1, O), np.int64).reshape(D, h, w, -1)
+    xd, fd, td = dev(x), dev(f), dev(thr)
+    ft = ops.tap_pack_filter(fd, 3 * fy, C)
+    prev = ops.conv_engine(3)
+    try:
+        got = ops.conv_act_pack(xd, ft, td, *geom, in_bits=C, filter_tap_packed=True)
+        assert ops.conv_last_engine() == 2
+        np.testing.assert_array_equal(host(got), packed)
+        assert torch.equal(ops.conv_act_pack(xd, fd, td, *geom, in_bits=C), got)
+        if h >= 2 and w >= 2:
+            pooled = ops.conv_act_pack(xd, ft, td, *geom, pool=True, in_bits=C, filter_tap_packed=True)
+            assert ops.conv_last_engine() == 2
+            np.testing.assert_array_equal(host(pooled), oracle.max_pool2d(packed, 2, 2, 0, 0, 2, 2))
+        ops.conv_engine(1)
+        assert torch.equal(ops.conv_act_pack(xd, ft, td, *geom, in_bits=C, filter_tap_packed=True), got)
+        assert ops.conv_last_engine() == 1
+    finally:
+        ops.conv_engine(prev)
+
+
 def _random_matrix_core_cases(n, seed):
     g = np.random.default_rng(seed)
     cases = []
