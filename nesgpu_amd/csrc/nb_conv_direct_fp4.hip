@@ -1,0 +1,365 @@
+// Binary conv on the FP4 matrix cores for layers with one full channel word per pixel (33 to 64 channels), 3x3
+// windows, stride 1, threshold bits out (optionally 2x2 OR-pooled): the wave-per-strip scheme of
+// nb_conv_direct.hip with v_mfma_scale_f32_16x16x128_f8f6f4 at unit scales.
+//
+// Bits become FP4 (E2M1) codes, 1 -> +1.0 (0x2), 0 -> -1.0 (0xA), two positions per byte; +-1 and 0 are exact, the
+// fp32 sums are integers far below 2^24, so popcount(x ^ w) = (K - dot) / 2 is the reference's sum bit for bit.  An
+// out-of-range pixel is the zero word, i.e. all -1; the zero tail of a channel word multiplies -1 by -1 and is part
+// of K.
+//
+// A wave owns 16 output columns of a sub-band of one member's rows for 16*NT output channels (one output word when
+// NT = 4) and walks down.  One MFMA takes 128 positions = two (pixel column, 64 channels) pairs: lane (pixel li,
+// group g) supplies the 32 channels of half g&1 of pixel column g>>1, which it fetches itself (a 4-byte buffer load
+// whose range check returns zero outside the image) and takes through a 256-entry LDS table, 8 bits -> 4 bytes.
+// Per image row r two fragments:
+//   A0(r) = [row r, tap column 0 | row r, tap column 1]            x filter rows 0, 1, 2  -> output rows r, r-1, r-2
+//   A1(r) = [row r, tap column 2 | row r+1, tap column 2]          x [f(0,2) | f(1,2)]    -> output row r
+//                                                                  x [f(2,2) |   0   ]    -> output row r-2
+// so the third tap column costs two MFMAs per row instead of three: five per row and 16 channels, not six.
+// Finished rows are compared with the thresholds (as dot products), gathered with ballots, pooled (in x a min over
+// neighbouring accumulator registers, in y over two walked rows) and stored as whole words.
+#include "nb_conv_common.hpp"
+
+namespace nb {
+
+typedef int dw_v4i __attribute__((ext_vector_type(4)));
+typedef int dw_v8i __attribute__((ext_vector_type(8)));
+typedef float dw_v4f __attribute__((ext_vector_type(4)));
+
+struct DwConv {
+    const uint64_t *in, *filt;
+    const int32_t *thresh;
+    uint64_t *out;
+    int H, Wd, px, py, h, w, O, Ow, K;
+    int ntx, ncg, nsb, hb;  // strips of 16 columns, channel groups of 16*NT, sub-bands per member, rows per sub-band
+    uint32_t units;         // D * nsb * ncg * ntx
+    uint32_t mntx, mncg, mnsb;
+};
+
+__device__ __forceinline__ uint32_t dw_div(uint32_t n, uint32_t d, uint32_t m)  // n / d, m = floor(2^32 / d)
+{
+    uint32_t q = d == 1 ? n : __umulhi(n, m);
+    q += n - q * d >= d;
+    q += n - q * d >= d;
+    return q;
+}
+
+// entry b: the FP4 codes of bits 0..7 of b, bit j -> nibble j
+struct DwLut {
+    uint32_t e[256];
+};
+constexpr DwLut dw_make_lut()
+{
+    DwLut t{};
+    for (uint32_t b = 0; b < 256; b++) {
+        uint32_t w = 0;
+        for (int j = 0; j < 8; j++) w |= (((b >> j) & 1u) ? 0x2u : 0xAu) << (4 * j);
+        t.e[b] = w;
+    }
+    return t;
+}
+__device__ const DwLut dw_lut_src = dw_make_lut();
+
+__device__ __forceinline__ dw_v4f dw_mfma(dw_v4i a, dw_v4i b, dw_v4f c)
+{
+    const dw_v8i a8 = __builtin_shufflevector(a, a, 0, 1, 2, 3, -1, -1, -1, -1);
+    const dw_v8i b8 = __builtin_shufflevector(b, b, 0, 1, 2, 3, -1, -1, -1, -1);
+    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a8, b8, c, 4, 4, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
+}
+
+// MODE 2: threshold bits packed along the channels; 3: the same, 2x2 OR-pooled
+template <int NT, int MODE>
+__global__ __launch_bounds__(256) void conv_direct_fp4_kernel(const DwConv p)
+{
+    __shared__ uint32_t lut[256];
+    lut[threadIdx.x] = dw_lut_src.e[threadIdx.x];
+    __syncthreads();
+    const unsigned char *lutb = reinterpret_cast<const unsigned char *>(lut);
+    auto expand32 = [&](uint32_t x) {  // 32 bits -> 32 codes in 16 bytes
+        const uint32_t a = *reinterpret_cast<const uint32_t *>(lutb + ((x & 0xFFu) << 2));
+        const uint32_t b = *reinterpret_cast<const uint32_t *>(lutb + (((x >> 8) & 0xFFu) << 2));
+        const uint32_t c = *reinterpret_cast<const uint32_t *>(lutb + (((x >> 16) & 0xFFu) << 2));
+        const uint32_t d = *reinterpret_cast<const uint32_t *>(lutb + ((x >> 24) << 2));
+        return (dw_v4i){(int)a, (int)b, (int)c, (int)d};
+    };
+    const int lane = threadIdx.x & 63;
+    // the unit is uniform over the wave, and visibly so: every branch around an MFMA must be a scalar branch,
+    // because MFMA ignores EXEC
+    const uint32_t u = blockIdx.x * 4u + (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    if (u >= p.units) return;
+    const uint32_t t1 = dw_div(u, (uint32_t)p.ntx, p.mntx);
+    const int st = (int)(u - t1 * (uint32_t)p.ntx);
+    const uint32_t t2 = dw_div(t1, (uint32_t)p.ncg, p.mncg);
+    const int cg = (int)(t1 - t2 * (uint32_t)p.ncg);
+    const int64_t z = dw_div(t2, (uint32_t)p.nsb, p.mnsb);
+    const int sb = (int)(t2 - (uint32_t)z * (uint32_t)p.nsb);
+    const int li = lane & 15, lg = lane >> 4;
+    const int tc = lg >> 1, hf = lg & 1;  // pixel column inside the 128-position chunk, half of the channel word
+
+    // ---- filter fragments: lane (channel li of tile nt, group lg) ---------------------------------------------------
+    const dw_v4i zero_i = {0, 0, 0, 0};
+    dw_v4i B0[3][NT], B1a[NT], B1b[NT];
+    int tdot[NT];
+    {
+        const uint64_t *fz = p.filt + z * (int64_t)(9 * p.O);
+        auto half = [&](int tap, int ch) {
+            const uint64_t wd = fz[(int64_t)tap * p.O + ch];
+            return hf ? (uint32_t)(wd >> 32) : (uint32_t)wd;
+        };
+#pragma unroll
+        for (int nt = 0; nt < NT; nt++) {
+            const int ch = (cg * NT + nt) * 16 + li;
+            const bool live = ch < p.O;
+            const int chc = live ? ch : p.O - 1;
+#pragma unroll
+            for (int i = 0; i < 3; i++) {
+                const dw_v4i e = expand32(half(i * 3 + tc, chc));
+                B0[i][nt] = live ? e : zero_i;
+            }
+            const dw_v4i ea = expand32(half(tc * 3 + 2, chc));  // f(0,2) | f(1,2)
+            B1a[nt] = live ? ea : zero_i;
+            const dw_v4i eb = expand32(half(8, chc));           // f(2,2) | 0
+            B1b[nt] = live && tc == 0 ? eb : zero_i;
+            // thresholds in dot-product terms: 2*popc > t  <=>  popc > (t>>1)  <=>  dot < K - 2*(t>>1); every dot
+            // product lies in [-K, K], so thresholds outside mean always / never and are pulled in to K + 1 / -K - 1
+            int64_t td = live ? (int64_t)p.K - 2 * (int64_t)(p.thresh[z * p.O + chc] >> 1) : -2147483648LL;
+            td = td > p.K + 1 ? p.K + 1 : (td < -p.K - 1 ? -p.K - 1 : td);
+            // The accumulators start at K + 1 instead of 0, so every sum is a positive float and its bit pattern
+            // orders like the value: minima and comparisons are integer instructions (one each; the float forms
+            // cost a compare and a select).
+            tdot[nt] = __builtin_bit_cast(int, (float)(td + p.K + 1));
+        }
+    }
+
+    // ---- input addressing ------------------------------------------------------------------------------------------
+    const int x0 = st * 16;
+    const int ys = sb * p.hb;
+    const int hout = MODE == 3 ? (p.h & ~1) : p.h;  // pooled maps drop an odd last row
+    const int ye = ys + p.hb < hout ? ys + p.hb : hout;
+    if (ys >= ye) return;
+    const int rowb = p.Wd * 8;
+    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint64_t *>(p.in + z * (int64_t)p.H * p.Wd), (short)0, p.H * rowb, 0x00020000);
+    // A column outside the image gets an offset that is out of range whatever row offset (below 2^29 either way) is
+    // added; a row outside gives a negative or too large offset by itself.
+    constexpr uint32_t kOutside = 0xC0000000u;
+    const int xa = x0 + li + tc - p.py, xb = x0 + li + 2 - p.py;
+    const uint32_t offa = (xa >= 0 && xa < p.Wd) ? (uint32_t)(xa * 8 + 4 * hf) : kOutside;
+    const uint32_t offb = (xb >= 0 && xb < p.Wd) ? (uint32_t)(xb * 8 + 4 * hf + tc * rowb) : kOutside;
+    auto load_a = [&](int rr) {  // band row rr is image row rr - px
+        return (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)(offa + (uint32_t)((rr - p.px) * rowb)), 0, 0);
+    };
+    auto load_b = [&](int rr) {
+        return (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)(offb + (uint32_t)((rr - p.px) * rowb)), 0, 0);
+    };
+
+    // ---- output ----------------------------------------------------------------------------------------------------
+    const int hh = MODE == 3 ? p.h >> 1 : p.h, ww = MODE == 3 ? p.w >> 1 : p.w;
+    const int xx0 = MODE == 3 ? x0 >> 1 : x0;
+    uint64_t *obase = p.out + ((z * hh * (int64_t)ww + xx0 + lane) * p.Ow + cg);  // NT < 4: one group, one word
+    const int64_t orow = (int64_t)ww * p.Ow;
+    const bool olive = lane < (MODE == 3 ? 8 : 16) && xx0 + lane < ww;
+    int pend[NT][2];  // MODE 3: x-pooled minima of the even row of a pair
+#pragma unroll
+    for (int nt = 0; nt < NT; nt++) pend[nt][0] = pend[nt][1] = 0;
+    auto finish_row = [&](dw_v4f (&af)[NT], int y, int par) {
+        uint64_t word = 0;
+        int a[NT][4];
+#pragma unroll
+        for (int nt = 0; nt < NT; nt++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const float f = af[nt][r];  // a copy first: the cast below wants an object, not a vector element
+                a[nt][r] = __builtin_bit_cast(int, f);
+            }
+        if (MODE == 2) {
+            // ballot r of lane (pixel 4*g+r, channel li): bits 16*g.. are the 16-channel piece of pixel 4*g+r; lane
+            // j < 16 assembles the pieces of pixel j over the NT channel tiles
+#pragma unroll
+            for (int nt = 0; nt < NT; nt++) {
+                const uint64_t m0 = __ballot(a[nt][0] < tdot[nt]), m1 = __ballot(a[nt][1] < tdot[nt]),
+                               m2 = __ballot(a[nt][2] < tdot[nt]), m3 = __ballot(a[nt][3] < tdot[nt]);
+                const int r = lane & 3;
+                const uint64_t mine = r == 0 ? m0 : r == 1 ? m1 : r == 2 ? m2 : m3;
+                word |= ((mine >> (16 * ((lane >> 2) & 3))) & 0xFFFFull) << (16 * nt);
+            }
+        } else {
+            // pixels 4g, 4g+1 and 4g+2, 4g+3 pool in x; rows y (even) and y+1 pool in y
+            if (par == 0) {
+#pragma unroll
+                for (int nt = 0; nt < NT; nt++) {
+                    pend[nt][0] = a[nt][0] < a[nt][1] ? a[nt][0] : a[nt][1];
+                    pend[nt][1] = a[nt][2] < a[nt][3] ? a[nt][2] : a[nt][3];
+                }
+                return;
+            }
+#pragma unroll
+            for (int nt = 0; nt < NT; nt++) {
+                int v0 = a[nt][0] < a[nt][1] ? a[nt][0] : a[nt][1];
+                int v1 = a[nt][2] < a[nt][3] ? a[nt][2] : a[nt][3];
+                v0 = v0 < pend[nt][0] ? v0 : pend[nt][0];
+                v1 = v1 < pend[nt][1] ? v1 : pend[nt][1];
+                const uint64_t m0 = __ballot(v0 < tdot[nt]), m1 = __ballot(v1 < tdot[nt]);
+                const uint64_t mine = (lane & 1) ? m1 : m0;  // pooled pixel 2g + q <-> lane 2g + q
+                word |= ((mine >> (16 * ((lane >> 1) & 3))) & 0xFFFFull) << (16 * nt);
+            }
+        }
+        if (olive) __builtin_nontemporal_store(word, obase + (int64_t)(MODE == 3 ? y >> 1 : y) * orow);
+    };
+
+    // ---- walk down the strip: band row rr feeds output rows rr (filter row 0), rr-1 (1) and rr-2 (2) ---------------
+    // a0 holds the partial sums of output row rr-2, a1 those of row rr-1; band row rr completes row rr-2 (emitted),
+    // continues row rr-1 and opens row rr with a zero C operand.
+    dw_v4f a0[NT], a1[NT];
+    const float kb = (float)(p.K + 1);
+    const dw_v4f zero = {kb, kb, kb, kb};  // the C operand that opens an output row: the bias described above
+#pragma unroll
+    for (int nt = 0; nt < NT; nt++) a0[nt] = a1[nt] = zero;
+    uint32_t ra0 = load_a(ys), rb0 = load_b(ys), ra1 = load_a(ys + 1), rb1 = load_b(ys + 1);
+    uint32_t ra2 = load_a(ys + 2), rb2 = load_b(ys + 2), ra3 = load_a(ys + 3), rb3 = load_b(ys + 3);
+    // the parts of a step: C = last (third) row of output row rr-2, M = middle row of rr-1, F = first row of rr
+#define NB_DW_PART_C(done)                                                                   \
+    _Pragma("unroll") for (int nt = 0; nt < NT; nt++) done[nt] = dw_mfma(A0, B0[2][nt], a0[nt]); \
+    _Pragma("unroll") for (int nt = 0; nt < NT; nt++) done[nt] = dw_mfma(A1, B1b[nt], done[nt]);
+#define NB_DW_PART_M _Pragma("unroll") for (int nt = 0; nt < NT; nt++) a0[nt] = dw_mfma(A0, B0[1][nt], a1[nt]);
+#define NB_DW_PART_F                                                                         \
+    _Pragma("unroll") for (int nt = 0; nt < NT; nt++) a1[nt] = dw_mfma(A0, B0[0][nt], zero); \
+    _Pragma("unroll") for (int nt = 0; nt < NT; nt++) a1[nt] = dw_mfma(A1, B1a[nt], a1[nt]);
+    if (ye - ys < 4) {
+        // short sub-band (a few last rows of an image): every part of a step under its own (uniform) condition
+#define NB_DW_ANY(RR, XA, XB, PAR)                                      \
+    {                                                                   \
+        const int rr_ = (RR);                                           \
+        const dw_v4i A0 = expand32(XA), A1 = expand32(XB);              \
+        XA = load_a(rr_ + 4);                                           \
+        XB = load_b(rr_ + 4);                                           \
+        dw_v4f done[NT];                                                \
+        if (rr_ - 2 >= ys) { NB_DW_PART_C(done) }                       \
+        if (rr_ - 1 >= ys && rr_ - 1 < ye) { NB_DW_PART_M }             \
+        if (rr_ < ye) { NB_DW_PART_F }                                  \
+        if (rr_ - 2 >= ys) finish_row(done, rr_ - 2, PAR);              \
+    }
+        for (int rr = ys; rr < ye + 2; rr += 4) {
+            NB_DW_ANY(rr, ra0, rb0, 0)
+            if (rr + 1 < ye + 2) NB_DW_ANY(rr + 1, ra1, rb1, 1)
+            if (rr + 2 < ye + 2) NB_DW_ANY(rr + 2, ra2, rb2, 0)
+            if (rr + 3 < ye + 2) NB_DW_ANY(rr + 3, ra3, rb3, 1)
+        }
+#undef NB_DW_ANY
+        return;
+    }
+    // The steady rows carry no conditions and always issue the same loads, so that the wait for a row's words is a
+    // wait for exactly the loads issued before them (four rows ahead).
+    int rr = ys + 2;
+    {
+        dw_v4i A0 = expand32(ra0), A1 = expand32(rb0);
+        ra0 = load_a(ys + 4);
+        rb0 = load_b(ys + 4);
+        NB_DW_PART_F
+        A0 = expand32(ra1), A1 = expand32(rb1);
+        ra1 = load_a(ys + 5);
+        rb1 = load_b(ys + 5);
+        NB_DW_PART_M
+        NB_DW_PART_F
+    }
+#define NB_DW_ROW(XA, XB, PAR)                                 \
+    {                                                          \
+        const dw_v4i A0 = expand32(XA), A1 = expand32(XB);     \
+        XA = load_a(rr + 4);                                   \
+        XB = load_b(rr + 4);                                   \
+        dw_v4f done[NT];                                       \
+        NB_DW_PART_C(done)                                     \
+        NB_DW_PART_M                                           \
+        NB_DW_PART_F                                           \
+        finish_row(done, rr - 2, PAR);                         \
+        rr++;                                                  \
+    }
+    // sub-bands start on even rows, so the parity of a finished row is known where the loop is unrolled
+    const int nsteady = ye - ys - 2, rem = nsteady & 3;
+    for (int q = nsteady >> 2; q > 0; q--) {
+        NB_DW_ROW(ra2, rb2, 0)
+        NB_DW_ROW(ra3, rb3, 1)
+        NB_DW_ROW(ra0, rb0, 0)
+        NB_DW_ROW(ra1, rb1, 1)
+    }
+    if (rem >= 1) NB_DW_ROW(ra2, rb2, 0)
+    if (rem >= 2) NB_DW_ROW(ra3, rb3, 1)
+    if (rem >= 3) NB_DW_ROW(ra0, rb0, 0)
+#undef NB_DW_ROW
+    // band rows ye and ye + 1 finish the last two output rows; their words sit in the ring behind the steady rows
+    {
+        const uint32_t ta = rem == 0 ? ra2 : rem == 1 ? ra3 : rem == 2 ? ra0 : ra1;
+        const uint32_t tb = rem == 0 ? rb2 : rem == 1 ? rb3 : rem == 2 ? rb0 : rb1;
+        const uint32_t ua = rem == 0 ? ra3 : rem == 1 ? ra0 : rem == 2 ? ra1 : ra2;
+        const uint32_t ub = rem == 0 ? rb3 : rem == 1 ? rb0 : rem == 2 ? rb1 : rb2;
+        dw_v4i A0 = expand32(ta), A1 = expand32(tb);
+        dw_v4f done[NT];
+        NB_DW_PART_C(done)
+        NB_DW_PART_M
+        finish_row(done, ye - 2, (ye - ys) & 1);
+        A0 = expand32(ua), A1 = expand32(ub);
+        NB_DW_PART_C(done)
+        finish_row(done, ye - 1, (ye - 1 - ys) & 1);
+    }
+#undef NB_DW_PART_C
+#undef NB_DW_PART_M
+#undef NB_DW_PART_F
+}
+
+// mode 2 (packed threshold bits) or 3 (2x2 OR-pooled), one channel word per pixel, filter [D, 9, O].  false = not
+// this shape, nothing launched.
+bool conv_direct_fp4_try(void *out, const uint64_t *in, const uint64_t *filt, const int32_t *thresh, const ConvGeom &g,
+                         int64_t D, int O, int tap_bits, int mode, hipStream_t s)
+{
+    if (mode != 2 && mode != 3) return false;
+    if (tap_bits != 0 || g.Cw != 1) return false;
+    if (g.sx != 1 || g.sy != 1 || g.fx != 3 || g.fy != 3) return false;
+    if (D < 1 || g.h < 1 || g.w < 1) return false;
+    if (!(O == 16 || O == 32 || (O >= 64 && O % 16 == 0))) return false;
+    if (mode == 3 && (g.h < 2 || g.w < 2)) return false;
+    // 32-bit byte offsets inside one member's image, far enough below 2^30 for the out-of-range marker
+    if ((int64_t)(g.H + g.px + 8) * g.Wd * 8 >= (1LL << 29) || (int64_t)9 * O * 8 >= (1LL << 31)) return false;
+    const int NT = O >= 64 ? 4 : O / 16;
+    DwConv p;
+    p.in = in;
+    p.filt = filt;
+    p.thresh = thresh;
+    p.out = static_cast<uint64_t *>(out);
+    p.H = g.H; p.Wd = g.Wd; p.px = g.px; p.py = g.py; p.h = g.h; p.w = g.w;
+    p.O = O;
+    p.Ow = (O + 63) / 64;
+    p.K = 9 * 64;
+    p.ntx = (g.w + 15) / 16;
+    p.ncg = (O + 16 * NT - 1) / (16 * NT);
+    // Sub-bands as tall as the population allows: whole images once that gives every SIMD a few waves, else down
+    // to 16 rows (a wave's start, the filter fragments, costs about as much as six rows).
+    {
+        const int64_t per = D * p.ntx * p.ncg;
+        int64_t want = per >= 2048 ? 1 : (2048 + per - 1) / per;
+        const int64_t most = g.h / 16 > 1 ? g.h / 16 : 1;
+        want = want > most ? most : want;
+        p.hb = (int)((g.h + want - 1) / want + 1) & ~1;
+    }
+    p.nsb = (g.h + p.hb - 1) / p.hb;
+    const int64_t units = D * p.nsb * p.ncg * p.ntx;
+    if (units >= (1LL << 31)) return false;
+    p.units = (uint32_t)units;
+    p.mntx = (uint32_t)((1ULL << 32) / (uint32_t)p.ntx);  // unused for a divisor of 1
+    p.mncg = (uint32_t)((1ULL << 32) / (uint32_t)p.ncg);
+    p.mnsb = (uint32_t)((1ULL << 32) / (uint32_t)p.nsb);
+    const dim3 grid((unsigned)ceil_div(units, 4)), block(256);
+#define NB_DW_LAUNCH(nt)                                                       \
+    if (NT == nt) {                                                            \
+        if (mode == 2)                                                         \
+            conv_direct_fp4_kernel<nt, 2><<<grid, block, 0, s>>>(p);           \
+        else                                                                   \
+            conv_direct_fp4_kernel<nt, 3><<<grid, block, 0, s>>>(p);           \
+    }
+    NB_DW_LAUNCH(1)
+    NB_DW_LAUNCH(2)
+    NB_DW_LAUNCH(4)
+#undef NB_DW_LAUNCH
+    return true;
+}
+
+}  // namespace nb
