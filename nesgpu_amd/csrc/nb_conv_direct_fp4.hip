@@ -60,6 +60,9 @@ constexpr DwLut dw_make_lut()
 }
 __device__ const DwLut dw_lut_src = dw_make_lut();
 
+// lane `LANE` (a constant) of w = the scalar value v; the other lanes keep theirs
+#define NB_DW_WRITELANE(w, v, LANE) asm("v_writelane_b32 %0, %1, %2" : "+v"(w) : "s"(v), "n"(LANE))
+
 __device__ __forceinline__ dw_v4f dw_mfma(dw_v4i a, dw_v4i b, dw_v4f c)
 {
     const dw_v8i a8 = __builtin_shufflevector(a, a, 0, 1, 2, 3, -1, -1, -1, -1);
@@ -113,16 +116,16 @@ __global__ __launch_bounds__(256) void conv_direct_fp4_kernel(const DwConv p)
             const int chc = live ? ch : p.O - 1;
 #pragma unroll
             for (int i = 0; i < 3; i++) {
-                const dw_v4i e = expand32(half(i * 3 + tc, chc));
-                B0[i][nt] = live ? e : zero_i;
+                B0[i][nt] = expand32(half(i * 3 + tc, chc));  // a channel past O multiplies whatever: it never fires
             }
-            const dw_v4i ea = expand32(half(tc * 3 + 2, chc));  // f(0,2) | f(1,2)
-            B1a[nt] = live ? ea : zero_i;
-            const dw_v4i eb = expand32(half(8, chc));           // f(2,2) | 0
-            B1b[nt] = live && tc == 0 ? eb : zero_i;
+            B1a[nt] = expand32(half(tc * 3 + 2, chc));    // f(0,2) | f(1,2)
+            const dw_v4i eb = expand32(half(8, chc));     // f(2,2) | 0
+            B1b[nt] = tc == 0 ? eb : zero_i;
             // thresholds in dot-product terms: 2*popc > t  <=>  popc > (t>>1)  <=>  dot < K - 2*(t>>1); every dot
             // product lies in [-K, K], so thresholds outside mean always / never and are pulled in to K + 1 / -K - 1
-            int64_t td = live ? (int64_t)p.K - 2 * (int64_t)(p.thresh[z * p.O + chc] >> 1) : -2147483648LL;
+            int t = p.thresh[z * p.O + chc];
+            t = t > 2 * p.K + 4 ? 2 * p.K + 4 : (t < -2 * p.K - 4 ? -2 * p.K - 4 : t);  // beyond: always / never, too
+            int td = live ? p.K - 2 * (t >> 1) : -p.K - 1;
             td = td > p.K + 1 ? p.K + 1 : (td < -p.K - 1 ? -p.K - 1 : td);
             // The accumulators start at K + 1 instead of 0, so every sum is a positive float and its bit pattern
             // orders like the value: minima and comparisons are integer instructions (one each; the float forms
@@ -156,14 +159,24 @@ __global__ __launch_bounds__(256) void conv_direct_fp4_kernel(const DwConv p)
     // ---- output ----------------------------------------------------------------------------------------------------
     const int hh = MODE == 3 ? p.h >> 1 : p.h, ww = MODE == 3 ? p.w >> 1 : p.w;
     const int xx0 = MODE == 3 ? x0 >> 1 : x0;
-    uint64_t *obase = p.out + ((z * hh * (int64_t)ww + xx0 + lane) * p.Ow + cg);  // NT < 4: one group, one word
+    // a channel group is a whole output word (NT = 4), or the layer has one group and one word (O = 16 or 32; the
+    // upper part of the word is written as zero)
+    uint64_t *obase = p.out + ((z * hh * (int64_t)ww + xx0 + lane) * p.Ow + cg);
     const int64_t orow = (int64_t)ww * p.Ow;
     const bool olive = lane < (MODE == 3 ? 8 : 16) && xx0 + lane < ww;
     int pend[NT][2];  // MODE 3: x-pooled minima of the even row of a pair
 #pragma unroll
     for (int nt = 0; nt < NT; nt++) pend[nt][0] = pend[nt][1] = 0;
+    // 16-bit field gq (0..3) of ballot a in the low half, that of ballot b in the high half: scalar pack instructions
+    auto fields = [](uint64_t a, uint64_t b, int gq) {
+        const uint32_t x = gq < 2 ? (uint32_t)a : (uint32_t)(a >> 32), y = gq < 2 ? (uint32_t)b : (uint32_t)(b >> 32);
+        return (gq & 1) ? (x >> 16) | (y & 0xFFFF0000u) : (x & 0xFFFFu) | (y << 16);
+    };
+    // A finished row's comparison results are ballots (scalar registers): bit 16*g + li of the ballot of accumulator
+    // register r is (pixel 4*g + r, channel li of the tile).  The output word of a pixel is put together from 16-bit
+    // fields of the NT tiles' ballots with scalar pack instructions and written into the storing lane's registers
+    // with v_writelane: two vector instructions per stored word, whatever NT is.
     auto finish_row = [&](dw_v4f (&af)[NT], int y, int par) {
-        uint64_t word = 0;
         int a[NT][4];
 #pragma unroll
         for (int nt = 0; nt < NT; nt++)
@@ -172,17 +185,21 @@ __global__ __launch_bounds__(256) void conv_direct_fp4_kernel(const DwConv p)
                 const float f = af[nt][r];  // a copy first: the cast below wants an object, not a vector element
                 a[nt][r] = __builtin_bit_cast(int, f);
             }
+        int wlo = 0, whi = 0;
         if (MODE == 2) {
-            // ballot r of lane (pixel 4*g+r, channel li): bits 16*g.. are the 16-channel piece of pixel 4*g+r; lane
-            // j < 16 assembles the pieces of pixel j over the NT channel tiles
+            // lane j < 16 stores pixel j = 4*g + r: field g of ballot r
+            uint64_t m[4][4];
 #pragma unroll
-            for (int nt = 0; nt < NT; nt++) {
-                const uint64_t m0 = __ballot(a[nt][0] < tdot[nt]), m1 = __ballot(a[nt][1] < tdot[nt]),
-                               m2 = __ballot(a[nt][2] < tdot[nt]), m3 = __ballot(a[nt][3] < tdot[nt]);
-                const int r = lane & 3;
-                const uint64_t mine = r == 0 ? m0 : r == 1 ? m1 : r == 2 ? m2 : m3;
-                word |= ((mine >> (16 * ((lane >> 2) & 3))) & 0xFFFFull) << (16 * nt);
-            }
+            for (int nt = 0; nt < 4; nt++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) m[nt][r] = nt < NT ? __ballot(a[nt < NT ? nt : 0][r] < tdot[nt < NT ? nt : 0]) : 0;
+#pragma unroll
+            for (int g = 0; g < 4; g++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    NB_DW_WRITELANE(wlo, fields(m[0][r], m[1][r], g), 4 * g + r);
+                    if (NT > 2) NB_DW_WRITELANE(whi, fields(m[2][r], m[3][r], g), 4 * g + r);
+                }
         } else {
             // pixels 4g, 4g+1 and 4g+2, 4g+3 pool in x; rows y (even) and y+1 pool in y
             if (par == 0) {
@@ -193,17 +210,30 @@ __global__ __launch_bounds__(256) void conv_direct_fp4_kernel(const DwConv p)
                 }
                 return;
             }
+            // lane P < 8 stores pooled pixel P = 2*g + q: field g of ballot q
+            uint64_t m[4][2];
 #pragma unroll
-            for (int nt = 0; nt < NT; nt++) {
-                int v0 = a[nt][0] < a[nt][1] ? a[nt][0] : a[nt][1];
-                int v1 = a[nt][2] < a[nt][3] ? a[nt][2] : a[nt][3];
-                v0 = v0 < pend[nt][0] ? v0 : pend[nt][0];
-                v1 = v1 < pend[nt][1] ? v1 : pend[nt][1];
-                const uint64_t m0 = __ballot(v0 < tdot[nt]), m1 = __ballot(v1 < tdot[nt]);
-                const uint64_t mine = (lane & 1) ? m1 : m0;  // pooled pixel 2g + q <-> lane 2g + q
-                word |= ((mine >> (16 * ((lane >> 1) & 3))) & 0xFFFFull) << (16 * nt);
+            for (int nt = 0; nt < 4; nt++) {
+                m[nt][0] = m[nt][1] = 0;
+                if (nt < NT) {
+                    const int n = nt < NT ? nt : 0;
+                    int v0 = a[n][0] < a[n][1] ? a[n][0] : a[n][1];
+                    int v1 = a[n][2] < a[n][3] ? a[n][2] : a[n][3];
+                    v0 = v0 < pend[n][0] ? v0 : pend[n][0];
+                    v1 = v1 < pend[n][1] ? v1 : pend[n][1];
+                    m[nt][0] = __ballot(v0 < tdot[n]);
+                    m[nt][1] = __ballot(v1 < tdot[n]);
+                }
             }
+#pragma unroll
+            for (int g = 0; g < 4; g++)
+#pragma unroll
+                for (int q = 0; q < 2; q++) {
+                    NB_DW_WRITELANE(wlo, fields(m[0][q], m[1][q], g), 2 * g + q);
+                    if (NT > 2) NB_DW_WRITELANE(whi, fields(m[2][q], m[3][q], g), 2 * g + q);
+                }
         }
+        const uint64_t word = ((uint64_t)(uint32_t)whi << 32) | (uint32_t)wlo;
         if (olive) __builtin_nontemporal_store(word, obase + (int64_t)(MODE == 3 ? y >> 1 : y) * orow);
     };
 
@@ -218,11 +248,11 @@ __global__ __launch_bounds__(256) void conv_direct_fp4_kernel(const DwConv p)
     uint32_t ra0 = load_a(ys), rb0 = load_b(ys), ra1 = load_a(ys + 1), rb1 = load_b(ys + 1);
     uint32_t ra2 = load_a(ys + 2), rb2 = load_b(ys + 2), ra3 = load_a(ys + 3), rb3 = load_b(ys + 3);
     // the parts of a step: C = last (third) row of output row rr-2, M = middle row of rr-1, F = first row of rr
-#define NB_DW_PART_C(done)                                                                   \
+#define NB_DW_PART_C(done, A0, A1)                                                           \
     _Pragma("unroll") for (int nt = 0; nt < NT; nt++) done[nt] = dw_mfma(A0, B0[2][nt], a0[nt]); \
     _Pragma("unroll") for (int nt = 0; nt < NT; nt++) done[nt] = dw_mfma(A1, B1b[nt], done[nt]);
-#define NB_DW_PART_M _Pragma("unroll") for (int nt = 0; nt < NT; nt++) a0[nt] = dw_mfma(A0, B0[1][nt], a1[nt]);
-#define NB_DW_PART_F                                                                         \
+#define NB_DW_PART_M(A0) _Pragma("unroll") for (int nt = 0; nt < NT; nt++) a0[nt] = dw_mfma(A0, B0[1][nt], a1[nt]);
+#define NB_DW_PART_F(A0, A1)                                                                 \
     _Pragma("unroll") for (int nt = 0; nt < NT; nt++) a1[nt] = dw_mfma(A0, B0[0][nt], zero); \
     _Pragma("unroll") for (int nt = 0; nt < NT; nt++) a1[nt] = dw_mfma(A1, B1a[nt], a1[nt]);
     if (ye - ys < 4) {
@@ -234,9 +264,9 @@ __global__ __launch_bounds__(256) void conv_direct_fp4_kernel(const DwConv p)
         XA = load_a(rr_ + 4);                                           \
         XB = load_b(rr_ + 4);                                           \
         dw_v4f done[NT];                                                \
-        if (rr_ - 2 >= ys) { NB_DW_PART_C(done) }                       \
-        if (rr_ - 1 >= ys && rr_ - 1 < ye) { NB_DW_PART_M }             \
-        if (rr_ < ye) { NB_DW_PART_F }                                  \
+        if (rr_ - 2 >= ys) { NB_DW_PART_C(done, A0, A1) }               \
+        if (rr_ - 1 >= ys && rr_ - 1 < ye) { NB_DW_PART_M(A0) }         \
+        if (rr_ < ye) { NB_DW_PART_F(A0, A1) }                          \
         if (rr_ - 2 >= ys) finish_row(done, rr_ - 2, PAR);              \
     }
         for (int rr = ys; rr < ye + 2; rr += 4) {
@@ -249,56 +279,59 @@ __global__ __launch_bounds__(256) void conv_direct_fp4_kernel(const DwConv p)
         return;
     }
     // The steady rows carry no conditions and always issue the same loads, so that the wait for a row's words is a
-    // wait for exactly the loads issued before them (four rows ahead).
+    // wait for exactly the loads issued before them (four rows ahead).  The fragments of the next row are looked up
+    // while the current row is multiplied: two fragment sets, P and Q, used in turn.
     int rr = ys + 2;
+    dw_v4i P0 = expand32(ra0), P1 = expand32(rb0), Q0, Q1;
     {
-        dw_v4i A0 = expand32(ra0), A1 = expand32(rb0);
+        Q0 = expand32(ra1), Q1 = expand32(rb1);
         ra0 = load_a(ys + 4);
         rb0 = load_b(ys + 4);
-        NB_DW_PART_F
-        A0 = expand32(ra1), A1 = expand32(rb1);
+        NB_DW_PART_F(P0, P1)
+        P0 = expand32(ra2), P1 = expand32(rb2);
         ra1 = load_a(ys + 5);
         rb1 = load_b(ys + 5);
-        NB_DW_PART_M
-        NB_DW_PART_F
+        NB_DW_PART_M(Q0)
+        NB_DW_PART_F(Q0, Q1)
     }
-#define NB_DW_ROW(XA, XB, PAR)                                 \
+    // C0, C1: the current row's fragments; N0, N1: set for the next row, whose words are XNA, XNB; XCA, XCB: the ring
+    // slot of the current row, free since its words were looked up a step ago
+#define NB_DW_ROW(C0, C1, N0, N1, XNA, XNB, XCA, XCB, PAR)     \
     {                                                          \
-        const dw_v4i A0 = expand32(XA), A1 = expand32(XB);     \
-        XA = load_a(rr + 4);                                   \
-        XB = load_b(rr + 4);                                   \
+        N0 = expand32(XNA), N1 = expand32(XNB);                \
+        XCA = load_a(rr + 4);                                  \
+        XCB = load_b(rr + 4);                                  \
         dw_v4f done[NT];                                       \
-        NB_DW_PART_C(done)                                     \
-        NB_DW_PART_M                                           \
-        NB_DW_PART_F                                           \
+        NB_DW_PART_C(done, C0, C1)                             \
+        NB_DW_PART_M(C0)                                       \
+        NB_DW_PART_F(C0, C1)                                   \
         finish_row(done, rr - 2, PAR);                         \
         rr++;                                                  \
     }
     // sub-bands start on even rows, so the parity of a finished row is known where the loop is unrolled
     const int nsteady = ye - ys - 2, rem = nsteady & 3;
     for (int q = nsteady >> 2; q > 0; q--) {
-        NB_DW_ROW(ra2, rb2, 0)
-        NB_DW_ROW(ra3, rb3, 1)
-        NB_DW_ROW(ra0, rb0, 0)
-        NB_DW_ROW(ra1, rb1, 1)
+        NB_DW_ROW(P0, P1, Q0, Q1, ra3, rb3, ra2, rb2, 0)
+        NB_DW_ROW(Q0, Q1, P0, P1, ra0, rb0, ra3, rb3, 1)
+        NB_DW_ROW(P0, P1, Q0, Q1, ra1, rb1, ra0, rb0, 0)
+        NB_DW_ROW(Q0, Q1, P0, P1, ra2, rb2, ra1, rb1, 1)
     }
-    if (rem >= 1) NB_DW_ROW(ra2, rb2, 0)
-    if (rem >= 2) NB_DW_ROW(ra3, rb3, 1)
-    if (rem >= 3) NB_DW_ROW(ra0, rb0, 0)
+    if (rem >= 1) NB_DW_ROW(P0, P1, Q0, Q1, ra3, rb3, ra2, rb2, 0)
+    if (rem >= 2) NB_DW_ROW(Q0, Q1, P0, P1, ra0, rb0, ra3, rb3, 1)
+    if (rem >= 3) NB_DW_ROW(P0, P1, Q0, Q1, ra1, rb1, ra0, rb0, 0)
 #undef NB_DW_ROW
-    // band rows ye and ye + 1 finish the last two output rows; their words sit in the ring behind the steady rows
+    // band rows ye and ye + 1 finish the last two output rows: row ye's fragments are in the current set, row
+    // ye + 1's words in the ring slot behind it
     {
-        const uint32_t ta = rem == 0 ? ra2 : rem == 1 ? ra3 : rem == 2 ? ra0 : ra1;
-        const uint32_t tb = rem == 0 ? rb2 : rem == 1 ? rb3 : rem == 2 ? rb0 : rb1;
+        if (rem & 1) P0 = Q0, P1 = Q1;
         const uint32_t ua = rem == 0 ? ra3 : rem == 1 ? ra0 : rem == 2 ? ra1 : ra2;
         const uint32_t ub = rem == 0 ? rb3 : rem == 1 ? rb0 : rem == 2 ? rb1 : rb2;
-        dw_v4i A0 = expand32(ta), A1 = expand32(tb);
+        Q0 = expand32(ua), Q1 = expand32(ub);
         dw_v4f done[NT];
-        NB_DW_PART_C(done)
-        NB_DW_PART_M
+        NB_DW_PART_C(done, P0, P1)
+        NB_DW_PART_M(P0)
         finish_row(done, ye - 2, (ye - ys) & 1);
-        A0 = expand32(ua), A1 = expand32(ub);
-        NB_DW_PART_C(done)
+        NB_DW_PART_C(done, Q0, Q1)
         finish_row(done, ye - 1, (ye - 1 - ys) & 1);
     }
 #undef NB_DW_PART_C
@@ -319,6 +352,7 @@ bool conv_direct_fp4_try(void *out, const uint64_t *in, const uint64_t *filt, co
     if (mode == 3 && (g.h < 2 || g.w < 2)) return false;
     // 32-bit byte offsets inside one member's image, far enough below 2^30 for the out-of-range marker
     if ((int64_t)(g.H + g.px + 8) * g.Wd * 8 >= (1LL << 29) || (int64_t)9 * O * 8 >= (1LL << 31)) return false;
+    // 64 channels per wave from 64 channels on (32 per wave, with twice the waves per SIMD, measured 5-8 % slower)
     const int NT = O >= 64 ? 4 : O / 16;
     DwConv p;
     p.in = in;
@@ -330,7 +364,7 @@ bool conv_direct_fp4_try(void *out, const uint64_t *in, const uint64_t *filt, co
     p.Ow = (O + 63) / 64;
     p.K = 9 * 64;
     p.ntx = (g.w + 15) / 16;
-    p.ncg = (O + 16 * NT - 1) / (16 * NT);
+    p.ncg = p.Ow;  // groups cover whole output words (dead channels give zero bits)
     // Sub-bands as tall as the population allows: whole images once that gives every SIMD a few waves, else down
     // to 16 rows (a wave's start, the filter fragments, costs about as much as six rows).
     {
