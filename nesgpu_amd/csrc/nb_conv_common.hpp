@@ -89,7 +89,7 @@ bool conv_direct_try(void *out, const uint64_t *in, const uint64_t *filt, const 
                      int64_t D, int O, int tap_bits, int mode, hipStream_t s);
 
 // The same scheme on the FP4 matrix cores for one full channel word per pixel (nb_conv_direct_fp4.hip): filter
-// [D, 9, O], 3x3 windows, stride 1, O = 16, 32 or a multiple of 16 from 64 on, mode 2 or 3.
+// [D, 9, O], 3x3 windows, stride 1, O = 16, 32 or a multiple of 16 from 64 on, mode 2, 3 or 4.
 bool conv_direct_fp4_try(void *out, const uint64_t *in, const uint64_t *filt, const int32_t *thresh, const ConvGeom &g,
                          int64_t D, int O, int tap_bits, int mode, hipStream_t s);
 

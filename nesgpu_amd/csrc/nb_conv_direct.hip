@@ -142,8 +142,15 @@ __global__ __launch_bounds__(256) void conv_direct_kernel(const DcConv p)
     // ---- output ----------------------------------------------------------------------------------------------------
     const int hh = MODE == 3 ? p.h >> 1 : p.h, ww = MODE == 3 ? p.w >> 1 : p.w;
     const int xx0 = MODE == 3 ? x0 >> 1 : x0;
-    uint64_t *obase = p.out + (z * hh * (int64_t)ww + xx0 + lane);  // row 0; one word per pixel (O <= 16)
+    // The words leave through buffer stores whose range is the member's map: a lane with nothing to store is given an
+    // offset beyond the range and the hardware drops its store.  No branch on the lane then, which matters here: an
+    // MFMA that the compiler sinks into a branch taken by some lanes only (its results being used only there) runs
+    // with the other lanes' operands and results masked off and gives wrong sums, so the walk has no divergent
+    // branch at all.
     const bool olive = lane < (MODE == 3 ? 8 : 16) && xx0 + lane < ww;
+    const __amdgpu_buffer_rsrc_t orsrc =
+        __builtin_amdgcn_make_buffer_rsrc(p.out + z * hh * (int64_t)ww, (short)0, hh * ww * 8, 0x00020000);
+    const uint32_t ooff = olive ? (uint32_t)((xx0 + lane) * 8) : 0xC0000000u;  // one word per pixel (O <= 16)
     int pend0 = 0, pend1 = 0;  // MODE 3: x-pooled minima of the even row of a pair
     auto finish_row = [&](const dc_v4i &a, int y, int par) {
         uint64_t word;
@@ -167,7 +174,9 @@ __global__ __launch_bounds__(256) void conv_direct_kernel(const DcConv p)
             const uint64_t mine = (lane & 1) ? m1 : m0;  // pooled pixel 2g + q <-> lane 2g + q
             word = (mine >> (16 * ((lane >> 1) & 3))) & 0xFFFFull;
         }
-        if (olive) __builtin_nontemporal_store(word, obase + (int64_t)(MODE == 3 ? y >> 1 : y) * ww);
+        typedef int dc_v2i __attribute__((ext_vector_type(2)));
+        __builtin_amdgcn_raw_buffer_store_b64((dc_v2i){(int)(uint32_t)word, 0}, orsrc,
+                                              (int)(ooff + (uint32_t)((MODE == 3 ? y >> 1 : y) * ww * 8)), 0, 2);
     };
 
     // ---- walk down the strip: band row rr feeds output rows rr (filter row 0), rr-1 (1) and rr-2 (2) ---------------
@@ -259,7 +268,7 @@ bool conv_direct_try(void *out, const uint64_t *in, const uint64_t *filt, const 
     if (O < 1 || O > 16 || D < 1 || g.h < 1 || g.w < 1) return false;
     if (mode == 3 && (g.h < 2 || g.w < 2)) return false;
     // 32-bit byte offsets inside one member's image, far enough below 2^30 for the out-of-range marker
-    if ((int64_t)(g.H + g.px + 8) * g.Wd * 8 >= (1LL << 29)) return false;
+    if ((int64_t)(g.H + g.px + 8) * g.Wd * 8 >= (1LL << 29) || (int64_t)g.h * g.w * 8 >= (1LL << 30)) return false;
     DcConv p;
     p.in = in;
     p.filt = filt;

@@ -1,6 +1,8 @@
 // Binary conv on the FP4 matrix cores for layers with one full channel word per pixel (33 to 64 channels), 3x3
-// windows, stride 1, threshold bits out (optionally 2x2 OR-pooled): the wave-per-strip scheme of
-// nb_conv_direct.hip with v_mfma_scale_f32_16x16x128_f8f6f4 at unit scales.
+// windows, stride 1: threshold bits out (optionally 2x2 OR-pooled), or the popcount maps' sums over the pixels.  The
+// wave-per-strip scheme of nb_conv_direct.hip with v_mfma_scale_f32_16x16x128_f8f6f4 at unit scales.  (The int32
+// maps themselves stay with the staged-image kernel, whose LDS transpose writes whole pixel rows: from this kernel's
+// register layout they left as 64-byte pieces and took 78-90 us where that kernel takes 50.)
 //
 // Bits become FP4 (E2M1) codes, 1 -> +1.0 (0x2), 0 -> -1.0 (0xA), two positions per byte; +-1 and 0 are exact, the
 // fp32 sums are integers far below 2^24, so popcount(x ^ w) = (K - dot) / 2 is the reference's sum bit for bit.  An
@@ -29,7 +31,7 @@ typedef float dw_v4f __attribute__((ext_vector_type(4)));
 struct DwConv {
     const uint64_t *in, *filt;
     const int32_t *thresh;
-    uint64_t *out;
+    void *out;
     int H, Wd, px, py, h, w, O, Ow, K;
     int ntx, ncg, nsb, hb;  // strips of 16 columns, channel groups of 16*NT, sub-bands per member, rows per sub-band
     uint32_t units;         // D * nsb * ncg * ntx
@@ -70,7 +72,8 @@ __device__ __forceinline__ dw_v4f dw_mfma(dw_v4i a, dw_v4i b, dw_v4f c)
     return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a8, b8, c, 4, 4, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
 }
 
-// MODE 2: threshold bits packed along the channels; 3: the same, 2x2 OR-pooled
+// MODE 2: threshold bits packed along the channels; 3: the same, 2x2 OR-pooled; 4: the popcount sums added up over
+// the pixels, int32 [D,O] (atomic adds into a zeroed array)
 template <int NT, int MODE>
 __global__ __launch_bounds__(256) void conv_direct_fp4_kernel(const DwConv p)
 {
@@ -123,7 +126,7 @@ __global__ __launch_bounds__(256) void conv_direct_fp4_kernel(const DwConv p)
             B1b[nt] = tc == 0 ? eb : zero_i;
             // thresholds in dot-product terms: 2*popc > t  <=>  popc > (t>>1)  <=>  dot < K - 2*(t>>1); every dot
             // product lies in [-K, K], so thresholds outside mean always / never and are pulled in to K + 1 / -K - 1
-            int t = p.thresh[z * p.O + chc];
+            int t = MODE == 2 || MODE == 3 ? p.thresh[z * p.O + chc] : 0;
             t = t > 2 * p.K + 4 ? 2 * p.K + 4 : (t < -2 * p.K - 4 ? -2 * p.K - 4 : t);  // beyond: always / never, too
             int td = live ? p.K - 2 * (t >> 1) : -p.K - 1;
             td = td > p.K + 1 ? p.K + 1 : (td < -p.K - 1 ? -p.K - 1 : td);
@@ -161,8 +164,6 @@ __global__ __launch_bounds__(256) void conv_direct_fp4_kernel(const DwConv p)
     const int xx0 = MODE == 3 ? x0 >> 1 : x0;
     // a channel group is a whole output word (NT = 4), or the layer has one group and one word (O = 16 or 32; the
     // upper part of the word is written as zero)
-    uint64_t *obase = p.out + ((z * hh * (int64_t)ww + xx0 + lane) * p.Ow + cg);
-    const int64_t orow = (int64_t)ww * p.Ow;
     const bool olive = lane < (MODE == 3 ? 8 : 16) && xx0 + lane < ww;
     int pend[NT][2];  // MODE 3: x-pooled minima of the even row of a pair
 #pragma unroll
@@ -176,7 +177,33 @@ __global__ __launch_bounds__(256) void conv_direct_fp4_kernel(const DwConv p)
     // register r is (pixel 4*g + r, channel li of the tile).  The output word of a pixel is put together from 16-bit
     // fields of the NT tiles' ballots with scalar pack instructions and written into the storing lane's registers
     // with v_writelane: two vector instructions per stored word, whatever NT is.
+    // MODE 4: the lane's running sum over its four pixel columns (columns past the image masked off) and all rows
+    int csum[NT];
+    int cmask[4];
+#pragma unroll
+    for (int nt = 0; nt < NT; nt++) csum[nt] = 0;
+#pragma unroll
+    for (int r = 0; r < 4; r++) cmask[r] = x0 + 4 * lg + r < p.w ? -1 : 0;
+    // The words leave through buffer stores whose range is the member's map: a lane with nothing to store is given an
+    // offset beyond the range and the hardware drops its store.  No branch on the lane then, which matters here: an
+    // MFMA that the compiler sinks into a branch taken by some lanes only (its results being used only there) runs
+    // with the other lanes' operands and results masked off and gives wrong sums, so the walk has no divergent
+    // branch at all.
+    __amdgpu_buffer_rsrc_t orsrc = rsrc;
+    uint32_t ooff = 0;
+    if (MODE == 2 || MODE == 3) {  // lane P < 8 (16) stores the word of (pooled) pixel xx0 + P for channel group cg
+        orsrc = __builtin_amdgcn_make_buffer_rsrc(static_cast<uint64_t *>(p.out) + z * hh * (int64_t)ww * p.Ow, (short)0,
+                                                  hh * ww * p.Ow * 8, 0x00020000);
+        ooff = olive ? (uint32_t)(((xx0 + lane) * p.Ow + cg) * 8) : 0xC0000000u;
+    }
     auto finish_row = [&](dw_v4f (&af)[NT], int y, int par) {
+        if (MODE == 4) {
+#pragma unroll
+            for (int nt = 0; nt < NT; nt++)
+                csum[nt] += (int)((cmask[0] ? af[nt][0] : 0.f) + (cmask[1] ? af[nt][1] : 0.f) +
+                                  (cmask[2] ? af[nt][2] : 0.f) + (cmask[3] ? af[nt][3] : 0.f));  // exact: below 2^13
+            return;
+        }
         int a[NT][4];
 #pragma unroll
         for (int nt = 0; nt < NT; nt++)
@@ -233,8 +260,9 @@ __global__ __launch_bounds__(256) void conv_direct_fp4_kernel(const DwConv p)
                     if (NT > 2) NB_DW_WRITELANE(whi, fields(m[2][q], m[3][q], g), 2 * g + q);
                 }
         }
-        const uint64_t word = ((uint64_t)(uint32_t)whi << 32) | (uint32_t)wlo;
-        if (olive) __builtin_nontemporal_store(word, obase + (int64_t)(MODE == 3 ? y >> 1 : y) * orow);
+        typedef int dw_v2i __attribute__((ext_vector_type(2)));
+        __builtin_amdgcn_raw_buffer_store_b64((dw_v2i){wlo, whi}, orsrc,
+                                              (int)(ooff + (uint32_t)((MODE == 3 ? y >> 1 : y) * ww * p.Ow * 8)), 0, 2);
     };
 
     // ---- walk down the strip: band row rr feeds output rows rr (filter row 0), rr-1 (1) and rr-2 (2) ---------------
@@ -248,13 +276,15 @@ __global__ __launch_bounds__(256) void conv_direct_fp4_kernel(const DwConv p)
     uint32_t ra0 = load_a(ys), rb0 = load_b(ys), ra1 = load_a(ys + 1), rb1 = load_b(ys + 1);
     uint32_t ra2 = load_a(ys + 2), rb2 = load_b(ys + 2), ra3 = load_a(ys + 3), rb3 = load_b(ys + 3);
     // the parts of a step: C = last (third) row of output row rr-2, M = middle row of rr-1, F = first row of rr
+    // image fragment x filter fragment: register r of a lane is (pixel 4g + r, channel li)
+#define NB_DW_MM(A, B, C) dw_mfma(A, B, C)
 #define NB_DW_PART_C(done, A0, A1)                                                           \
-    _Pragma("unroll") for (int nt = 0; nt < NT; nt++) done[nt] = dw_mfma(A0, B0[2][nt], a0[nt]); \
-    _Pragma("unroll") for (int nt = 0; nt < NT; nt++) done[nt] = dw_mfma(A1, B1b[nt], done[nt]);
-#define NB_DW_PART_M(A0) _Pragma("unroll") for (int nt = 0; nt < NT; nt++) a0[nt] = dw_mfma(A0, B0[1][nt], a1[nt]);
+    _Pragma("unroll") for (int nt = 0; nt < NT; nt++) done[nt] = NB_DW_MM(A0, B0[2][nt], a0[nt]); \
+    _Pragma("unroll") for (int nt = 0; nt < NT; nt++) done[nt] = NB_DW_MM(A1, B1b[nt], done[nt]);
+#define NB_DW_PART_M(A0) _Pragma("unroll") for (int nt = 0; nt < NT; nt++) a0[nt] = NB_DW_MM(A0, B0[1][nt], a1[nt]);
 #define NB_DW_PART_F(A0, A1)                                                                 \
-    _Pragma("unroll") for (int nt = 0; nt < NT; nt++) a1[nt] = dw_mfma(A0, B0[0][nt], zero); \
-    _Pragma("unroll") for (int nt = 0; nt < NT; nt++) a1[nt] = dw_mfma(A1, B1a[nt], a1[nt]);
+    _Pragma("unroll") for (int nt = 0; nt < NT; nt++) a1[nt] = NB_DW_MM(A0, B0[0][nt], zero); \
+    _Pragma("unroll") for (int nt = 0; nt < NT; nt++) a1[nt] = NB_DW_MM(A1, B1a[nt], a1[nt]);
     if (ye - ys < 4) {
         // short sub-band (a few last rows of an image): every part of a step under its own (uniform) condition
 #define NB_DW_ANY(RR, XA, XB, PAR)                                      \
@@ -337,14 +367,30 @@ __global__ __launch_bounds__(256) void conv_direct_fp4_kernel(const DwConv p)
 #undef NB_DW_PART_C
 #undef NB_DW_PART_M
 #undef NB_DW_PART_F
+#undef NB_DW_MM
+    if (MODE == 4) {
+        // popcount = (2K + 1 - biased dot) / 2 per pixel: add the four lane groups, then one atomic per channel
+        const int cols = p.w - x0 < 16 ? p.w - x0 : 16;
+        const int kn = (2 * p.K + 1) * (ye - ys) * cols;
+#pragma unroll
+        for (int nt = 0; nt < NT; nt++) {
+            int v = csum[nt];
+            v += __shfl_xor(v, 16);
+            v += __shfl_xor(v, 32);
+            const int ch = (cg * NT + nt) * 16 + li;
+            if (lg == 0 && ch < p.O) atomicAdd(reinterpret_cast<int *>(p.out) + z * p.O + ch, (kn - v) >> 1);
+        }
+    }
 }
 
-// mode 2 (packed threshold bits) or 3 (2x2 OR-pooled), one channel word per pixel, filter [D, 9, O].  false = not
-// this shape, nothing launched.
+// mode 2 (packed threshold bits), 3 (2x2 OR-pooled) or 4 (pixel sums into a zeroed array), one channel word per
+// pixel, filter [D, 9, O].  false = not this shape, nothing launched.
 bool conv_direct_fp4_try(void *out, const uint64_t *in, const uint64_t *filt, const int32_t *thresh, const ConvGeom &g,
                          int64_t D, int O, int tap_bits, int mode, hipStream_t s)
 {
-    if (mode != 2 && mode != 3) return false;
+    if (mode != 2 && mode != 3 && mode != 4) return false;
+    // 32-bit byte offsets inside one member's output, below 2^30 for the out-of-range marker of the stores
+    if ((mode == 2 || mode == 3) && (int64_t)g.h * g.w * ((O + 63) / 64) * 8 >= (1LL << 30)) return false;
     if (tap_bits != 0 || g.Cw != 1) return false;
     if (g.sx != 1 || g.sy != 1 || g.fx != 3 || g.fy != 3) return false;
     if (D < 1 || g.h < 1 || g.w < 1) return false;
@@ -358,7 +404,7 @@ bool conv_direct_fp4_try(void *out, const uint64_t *in, const uint64_t *filt, co
     p.in = in;
     p.filt = filt;
     p.thresh = thresh;
-    p.out = static_cast<uint64_t *>(out);
+    p.out = out;
     p.H = g.H; p.Wd = g.Wd; p.px = g.px; p.py = g.py; p.h = g.h; p.w = g.w;
     p.O = O;
     p.Ow = (O + 63) / 64;
@@ -386,8 +432,10 @@ bool conv_direct_fp4_try(void *out, const uint64_t *in, const uint64_t *filt, co
     if (NT == nt) {                                                            \
         if (mode == 2)                                                         \
             conv_direct_fp4_kernel<nt, 2><<<grid, block, 0, s>>>(p);           \
-        else                                                                   \
+        else if (mode == 3)                                                    \
             conv_direct_fp4_kernel<nt, 3><<<grid, block, 0, s>>>(p);           \
+        else                                                                   \
+            conv_direct_fp4_kernel<nt, 4><<<grid, block, 0, s>>>(p);           \
     }
     NB_DW_LAUNCH(1)
     NB_DW_LAUNCH(2)

@@ -703,8 +703,9 @@ def test_conv_matrix_core_random_shapes(ops, oracle, mc_engine):
 @pytest.mark.parametrize("C,O,S,mode", [(16, 16, 8, "pool"), (64, 64, 8, "pool"), (64, 128, 6, "pack"),
                                          (64, 64, 8, "sums"), (3, 64, 10, "pack")])
 def test_conv_matrix_core_many_members(ops, oracle, mc_engine, C, O, S, mode):
-    """More members than workgroups: every workgroup of the persistent kernel walks several members (fragments and
-    image buffers change hands many times); every member against the oracle."""
+    """More members than workgroups or wave slots: every workgroup of the persistent kernel walks several members
+    (fragments and image buffers change hands many times), the strip kernels run in several rounds; every member
+    against the oracle."""
     D = 1300
     g = rng(C + O + S)
     Cw = (C + 63) // 64
