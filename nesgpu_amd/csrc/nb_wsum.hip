@@ -5,7 +5,7 @@
 
 namespace nb {
 
-// Rows of any length.  One wave per (row, 64-bit column): lane z owns output bit z of the column and adds the members' weights in member
+// Rows shorter than 32 bytes.  One wave per (row, 64-bit column): lane z owns output bit z of the column and adds the members' weights in member
 // order (the reference's order, so the fp32 sums are the same).  Members are taken 64 at a time: lane j fetches the
 // column word of member m0 + j (64 strided loads in flight at once instead of one load per loop step), the
 // workgroup's four waves share the chunk's weights as fp32 in LDS, and then for each member its word, read out of
@@ -58,7 +58,7 @@ __global__ __launch_bounds__(256) void weighted_sum_kernel(_Float16 *__restrict_
     if (live && z < zbits) ret[r * zbits + z] = (_Float16)acc;
 }
 
-// Rows whose length is a multiple of 32 bytes: one wave per (row, 32-byte piece), a workgroup's four waves on four
+// Rows of 32 bytes or more: one wave per (row, 32-byte piece), a workgroup's four waves on four
 // consecutive pieces, so that every 128-byte line of every member's row is fetched by one workgroup, once, in one
 // 32-byte access per lane (lane j holds the piece of member m0 + j in 8 registers; the next 64 members' pieces are
 // requested before the current ones are used).  The piece holds four 64-bit columns; lane z owns output bit z of
@@ -70,10 +70,13 @@ __global__ __launch_bounds__(256) void weighted_sum_kernel(_Float16 *__restrict_
 // 64-byte piece with eight sums measured the same or slower: half as many waves to hide the LDS reads behind.)
 #define NB_WS_COL(ACC, D) ACC += __builtin_bit_cast(float, __builtin_amdgcn_sbfe((int)(D), zz, 1u) & wbits);
 
+// VEC: rows are whole 32-byte pieces and 16-byte aligned (two 16-byte loads per lane); otherwise the piece is fetched
+// as eight 4-byte loads, those past the end of the row left out (rows of 9 words, say: a conv layer's filters).
+template <bool VEC>
 __global__ __launch_bounds__(256) void weighted_sum_line_kernel(_Float16 *__restrict__ ret,
-                                                                const uint4 *__restrict__ in,
+                                                                const uint32_t *__restrict__ in,
                                                                 const _Float16 *__restrict__ w, int64_t n, int64_t R,
-                                                                int row16, int zbits, int npiece)
+                                                                int rowdw, int zbits, int npiece)
 {
     __shared__ uint4 msk[2][4][2][64];  // [buffer][wave][low halves, high halves][member]
     __shared__ float wsh[2][64];
@@ -82,18 +85,32 @@ __global__ __launch_bounds__(256) void weighted_sum_line_kernel(_Float16 *__rest
     const bool live = pid < R * npiece;
     const int64_t r = live ? pid / npiece : 0;
     const int g = live ? (int)(pid - r * npiece) : 0;
-    const int64_t stride16 = R * (int64_t)row16;
-    const uint4 *p = in + r * row16 + (int64_t)g * 2;
+    const int64_t stride = R * (int64_t)rowdw;  // dwords from one member's row to the next member's
+    const uint32_t *p = in + r * rowdw + (int64_t)g * 8;
+    const int left = rowdw - g * 8;             // dwords of the row from this piece on
     const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
+    auto fetch = [&](uint4 &x, uint4 &y, int64_t m) {
+        const uint32_t *q = p + m * stride;
+        if (VEC) {
+            x = load_stream16(q), y = load_stream16(q + 4);
+        } else {
+            // plain loads: the eight of a lane share a cache line, which streaming loads would fetch eight times
+            x.x = q[0];
+            x.y = left > 1 ? q[1] : 0u;
+            x.z = left > 2 ? q[2] : 0u;
+            x.w = left > 3 ? q[3] : 0u;
+            y.x = left > 4 ? q[4] : 0u;
+            y.y = left > 5 ? q[5] : 0u;
+            y.z = left > 6 ? q[6] : 0u;
+            y.w = left > 7 ? q[7] : 0u;
+        }
+    };
     const uint32_t zz = lane & 31;
     const int half = lane >> 5;
     float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
     uint4 a0 = zero, a1 = zero;  // members past n contribute zero words: nothing is added for them
     float wa = 0.f;
-    if (live && lane < n) {
-        const uint4 *q = p + lane * stride16;
-        a0 = load_stream16(q), a1 = load_stream16(q + 1);
-    }
+    if (live && lane < n) fetch(a0, a1, lane);
     if (wv == 0 && lane < n) wa = (float)w[lane];
     int buf = 0;
     for (int64_t m0 = 0; m0 < n; m0 += 64, buf ^= 1) {
@@ -105,10 +122,7 @@ __global__ __launch_bounds__(256) void weighted_sum_line_kernel(_Float16 *__rest
         __syncthreads();
         a0 = a1 = zero;
         wa = 0.f;
-        if (live && m0 + 64 + lane < n) {
-            const uint4 *q = p + (m0 + 64 + lane) * stride16;
-            a0 = load_stream16(q), a1 = load_stream16(q + 1);
-        }
+        if (live && m0 + 64 + lane < n) fetch(a0, a1, m0 + 64 + lane);
         if (wv == 0 && m0 + 64 + lane < n) wa = (float)w[m0 + 64 + lane];
         const uint4 *mine = &msk[buf][wv][half][0];
 #pragma unroll 8
@@ -148,13 +162,16 @@ int weighted_sum_impl(uint16_t *ret, const W *in, const uint16_t *w, int64_t n, 
     NB_REQUIRE(zbits <= (1 << 30) && Rw <= (1 << 30), "%s: row too long", who);
     NB_REQUIRE(zbits <= Rw * (int64_t)WordTraits<W>::bits, "%s: zbits exceeds the Rw words of a row", who);
     const int64_t rowbytes = Rw * (int64_t)sizeof(W);
-    if (n > 0 && rowbytes % 32 == 0 && (reinterpret_cast<uintptr_t>(in) & 15) == 0) {
+    // a wave per 32-byte piece once that gives every SIMD a wave; smaller outputs spread better with a wave per column
+    if (n > 0 && rowbytes >= 32 && R * ceil_div(zbits, 256) >= 1024) {
         const int64_t npiece = ceil_div(zbits, 256);  // 32-byte pieces of a row that hold output bits
         const int64_t blocks = ceil_div(R * npiece, 4);
         NB_REQUIRE(blocks <= kMaxGridX, "%s: output exceeds one launch", who);
-        weighted_sum_line_kernel<<<dim3((unsigned)blocks), dim3(256), 0, as_stream(stream)>>>(
-            reinterpret_cast<_Float16 *>(ret), reinterpret_cast<const uint4 *>(in),
-            reinterpret_cast<const _Float16 *>(w), n, R, (int)(rowbytes / 16), (int)zbits, (int)npiece);
+        const bool vec = rowbytes % 32 == 0 && (reinterpret_cast<uintptr_t>(in) & 15) == 0;
+        auto *kern = vec ? weighted_sum_line_kernel<true> : weighted_sum_line_kernel<false>;
+        kern<<<dim3((unsigned)blocks), dim3(256), 0, as_stream(stream)>>>(
+            reinterpret_cast<_Float16 *>(ret), reinterpret_cast<const uint32_t *>(in),
+            reinterpret_cast<const _Float16 *>(w), n, R, (int)(rowbytes / 4), (int)zbits, (int)npiece);
         return check_launch(who);
     }
     const int64_t ncol = ceil_div(zbits, 64);

@@ -410,10 +410,14 @@ def test_sample_bits_law_and_layout(ops):
 @pytest.mark.parametrize("dtype", [torch.int64, torch.int32])
 def test_weighted_sum_vs_oracle(ops, oracle, dtype):
     g = rng(21)
-    # the second line: rows that are whole 64-byte pieces (a wave per piece), also with fewer output bits than the
-    # row holds, fewer members than a wave has lanes, and a member count that is not a multiple of 64
+    # the second line: rows that are whole 32-byte pieces (a wave per piece), also with fewer output bits than the
+    # row holds, fewer members than a wave has lanes, and a member count that is not a multiple of 64; the third:
+    # rows of 32 bytes or more that are not whole pieces (a conv layer's nine words); the fourth: outputs large enough for
+    # the wave-per-piece kernel (1024 pieces or more), whole pieces and ragged
     for n, R, C in [(37, 5, 100), (128, 16, 64), (64, 3, 256), (200, 7, 90), (130, 3, 330), (1, 1, 1),
-                    (64, 5, 512), (70, 3, 1000), (130, 2, 1536), (100, 9, 2048), (3, 6, 1024), (257, 1, 520 + 504)]:
+                    (64, 5, 512), (70, 3, 1000), (130, 2, 1536), (100, 9, 2048), (3, 6, 1024), (257, 1, 520 + 504),
+                    (70, 4, 576), (65, 2, 2600), (9, 3, 300),
+                    (66, 400, 576), (10, 1100, 256), (5, 130, 2300)]:
         nd = NDT[dtype]
         wb = np.dtype(nd).itemsize * 8
         words = rand_words(g, (n, R, (C + wb - 1) // wb), nd)
