@@ -347,19 +347,33 @@ __global__ __launch_bounds__(256) void fl_skip_fill_kernel(uint32_t *__restrict_
     int j = 0;
     uint32_t pend = 0;
     bool half = false;
-    // a lane's dwords leave four at a time, as whole 16-byte pieces (L is a multiple of 4); never past the slice,
-    // whatever the inputs
+    // A lane's dwords leave four at a time, as whole 16-byte pieces (L is a multiple of 4); never past the slice,
+    // whatever the inputs.  The walk writes its entries without the base bit; when a piece is complete, the base
+    // words of its (up to eight) columns are asked for together and the bits put in before the piece is stored: one
+    // wait for memory per piece instead of one per flip (a wait for a load also waits for the stores before it).
+    const uint64_t *b = base + r * Kw;
+    const uint32_t npieces = (uint32_t)(4 * Kw);
     uint32_t q0 = 0, q1 = 0, q2 = 0;
+    auto base_bit = [&](uint32_t e) -> uint32_t {  // e: one 16-bit entry; 0 for a sentinel
+        const uint32_t piece = e >> 5;
+        const uint32_t col = (piece >> 1) * 32u + (e & 31u);
+        const uint32_t live = piece < npieces;
+        const uint64_t word = live ? b[col >> 6] : 0ull;  // nothing is read for a sentinel
+        return (uint32_t)(word >> (col & 63u)) & 1u;
+    };
+    auto patched = [&](uint32_t v) { return v | (base_bit(v & 0xFFFFu) << 5) | (base_bit(v >> 16) << 21); };
     auto put = [&](uint32_t v) {
         const int c = j & 3;
         if (c == 0) q0 = v;
         else if (c == 1) q1 = v;
         else if (c == 2) q2 = v;
-        else if (j < L) dst[(int64_t)(j >> 2) * 64] = make_uint4(q0, q1, q2, v);
+        else if (j < L) {
+            const uint32_t p0 = patched(q0), p1 = patched(q1), p2 = patched(q2), p3 = patched(v);
+            dst[(int64_t)(j >> 2) * 64] = make_uint4(p0, p1, p2, p3);
+        }
         j++;
     };
     if (valid && Kt > 0) {
-        const uint64_t *b = base + r * Kw;
         SkipChain chain(key, key.first + (uint64_t)(d * R + r) * (uint64_t)C);
         int pos = -1;
         for (;;) {
@@ -368,8 +382,7 @@ __global__ __launch_bounds__(256) void fl_skip_fill_kernel(uint32_t *__restrict_
             if (pos >= C) break;
             if (rank >= Kt) continue;  // a word beyond the table: moved on, no flip
             const uint32_t col = (uint32_t)pos;
-            const uint32_t bb = (uint32_t)(b[col >> 6] >> (col & 63u)) & 1u;
-            const uint32_t e = ((2u * (col >> 5) + bb) << 5) | (col & 31u);
+            const uint32_t e = ((2u * (col >> 5)) << 5) | (col & 31u);  // base bit still to come
             if (!half) {
                 pend = e;
                 half = true;
