@@ -161,6 +161,26 @@ def test_config5_cifar_net(wk, ops, oracle):
         assert ops.conv_last_engine() == 2
     finally:
         ops.conv_engine(prev)
+    # the two 64-channel layers on all members, pooled packed output with thresholds spread around the sums and the
+    # maps' pixel sums: the wave-per-strip FP4 kernel (automatic choice) == the staged-image int8 kernel == the
+    # XOR-popcount kernels
+    g5 = torch.Generator(device="cuda")
+    g5.manual_seed(5)
+    for name, S, O in (("f2", 32, 64), ("f3", 16, 128)):
+        xin = torch.randint(-2 ** 62, 2 ** 62, (D, S, S, 1), dtype=torch.int64, device="cuda", generator=g5)
+        thr = (576 + torch.randint(-40, 41, (D, O), device="cuda", generator=g5)).to(torch.int32)
+        got, sums = {}, {}
+        for eng, served in ((0, 4), (3, 2), (1, 1)):
+            ops.conv_engine(eng)
+            got[eng] = ops.conv_act_pack(xin, t[name], thr, 3, 3, 1, 1, 1, 1, pool=True)
+            assert ops.conv_last_engine() == served
+            sums[eng] = ops.conv_popc_sums(xin, t[name], 3, 3, 1, 1, 1, 1)
+            assert ops.conv_last_engine() == served
+        ops.conv_engine(prev)
+        assert torch.equal(got[0], got[3]) and torch.equal(got[0], got[1]), name
+        assert torch.equal(sums[0], sums[3]) and torch.equal(sums[0], sums[1]), name
+        assert 0.2 < float(ops.unpack(got[0].view(-1, got[0].shape[-1])).float().mean()) < 0.8      # not degenerate
+        del xin, thr, got, sums
     del l1, thr1
     # the members' weights regenerated on the host from the Philox stream (subsequences 10..14 in layer order) must
     # be what the GPU sampler wrote: all filters, eight rows of the 8192 -> 1024 layer, all of the last layer
