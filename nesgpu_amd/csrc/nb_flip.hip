@@ -452,13 +452,16 @@ __global__ __launch_bounds__(1024) void fl_bmv_kernel(void *__restrict__ out, co
                                                       const int32_t *__restrict__ thresh, int64_t R, int S, int Kw,
                                                       int blocks_per_member)
 {
-    extern __shared__ uint32_t fl_tab[];  // x and ~x interleaved, one zero dword, then the block's bit array
+    // x and ~x interleaved, one zero dword (the sentinel's entry: 4 * Kw), then the block's bit array.  A static
+    // array: its address is then known when the look-ups are compiled and needs no add per look-up.
+    __shared__ uint32_t fl_tab[4 * kFlipMaxKw + 1 + 32];
     constexpr int U = 4;                  // 16-byte pieces of a lane's list requested together
     const int64_t d = blockIdx.x / blocks_per_member;
     const int blk = (int)(blockIdx.x - d * blocks_per_member);
     const int nd = 2 * Kw;
     const int lane = threadIdx.x & 63;
-    const int s = blk * (kFlipBlockRows / 64) + (int)(threadIdx.x >> 6);  // wave-uniform
+    // the slice is uniform over the wave, and visibly so: the tests on the slice's length below are scalar branches
+    const int s = blk * (kFlipBlockRows / 64) + __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const bool active = s < S;
     const int64_t sl = d * S + (active ? s : S - 1);
     const int L = active ? __builtin_amdgcn_readfirstlane(slice_len[sl]) : 0;
@@ -747,14 +750,13 @@ static int flip_bmv(void *out, const int32_t *G, const uint32_t *entries, const 
     const int64_t bpm = nb::ceil_div(S, per_block);
     NB_REQUIRE(D * bpm <= nb::kMaxGridX, "%s: too many rows for one launch", who);
     const unsigned threads = 64u * (unsigned)(S < per_block ? S : per_block);
-    const size_t lds = (size_t)(4 * Kw + 1 + 32) * 4;
     const dim3 grid((unsigned)(D * bpm));
     if (pack)
-        nb::fl_bmv_kernel<true><<<grid, dim3(threads), lds, nb::as_stream(stream)>>>(
+        nb::fl_bmv_kernel<true><<<grid, dim3(threads), 0, nb::as_stream(stream)>>>(
             out, G, entries, slice_off, slice_len, perm, cnt, reinterpret_cast<const uint32_t *>(x), thresh, R, (int)S,
             (int)Kw, (int)bpm);
     else
-        nb::fl_bmv_kernel<false><<<grid, dim3(threads), lds, nb::as_stream(stream)>>>(
+        nb::fl_bmv_kernel<false><<<grid, dim3(threads), 0, nb::as_stream(stream)>>>(
             out, G, entries, slice_off, slice_len, perm, cnt, reinterpret_cast<const uint32_t *>(x), thresh, R, (int)S,
             (int)Kw, (int)bpm);
     return nb::check_launch(who);
