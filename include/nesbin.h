@@ -229,7 +229,7 @@ int nb_conv_popc_sums_i32(int32_t *sums, const int32_t *in, const int32_t *filt,
  * XOR-popcount kernels (any shape) and a matrix-core kernel (64-bit words, 3-row windows, stride 1, O % 16 == 0,
  * one band of a member's image fits LDS) that feeds the bits to the matrix cores as +-1 bytes (int8 MFMA) or, for
  * full channel words of 64, 128 or 256 channels, as FP4 codes (FP4 MFMA, twice the rate, exact for +-1).
- * Narrow layers (tap-packed filters of at most 16 channels, at most 16 output channels, 3-row windows of up to 3
+ * Narrow layers (tap-packed filters of at most 16 channels, at most 64 output channels, 3-row windows of up to 3
  * columns, stride 1, packed output) have a matrix-core kernel of their own that serves any population; so have
  * packed outputs of 3x3 windows over one full channel word per pixel (FP4; engines 0 and 2).
  * 0 = automatic: the matrix-core kernels for populations of 128 members or more (the narrow one always), else

@@ -83,7 +83,7 @@ bool conv_window_try(void *out, const W *in, const W *filt, const int32_t *thres
 int conv_mfma_try(void *out, const uint64_t *in, const uint64_t *filt, const int32_t *thresh, const ConvGeom &g,
                   int64_t D, int O, int tap_bits, int mode, bool allow_fp4, hipStream_t s);
 
-// Matrix-core conv for narrow layers (nb_conv_direct.hip): tap-packed filters of at most 16 channels, O <= 16, 3-row
+// Matrix-core conv for narrow layers (nb_conv_direct.hip): tap-packed filters of at most 16 channels, O <= 64, 3-row
 // filters of up to 3 columns, stride 1, mode 2 or 3.  false = not this shape, nothing launched.
 bool conv_direct_try(void *out, const uint64_t *in, const uint64_t *filt, const int32_t *thresh, const ConvGeom &g,
                      int64_t D, int O, int tap_bits, int mode, hipStream_t s);

@@ -1,9 +1,10 @@
-// Binary conv on the matrix cores for narrow layers: at most 16 input channels (tap-packed filters), at most 16
-// output channels, 3-row filters of up to 3 columns, stride 1, threshold bits out (optionally 2x2 OR-pooled).
+// Binary conv on the matrix cores for narrow layers: at most 16 input channels (tap-packed filters), at most 64
+// output channels (one output word), 3-row filters of up to 3 columns, stride 1, threshold bits out (optionally 2x2
+// OR-pooled).
 //
 // Such a layer has too little arithmetic per pixel to pay for a staged image: one v_mfma_i32_16x16x64_i8 covers 16
 // pixels x 16 channels x one filter row (3 tap columns x 16 channel positions + 16 idle positions), three of them
-// finish a row of 16 output pixels.  So there is no producer / consumer split and no image in LDS here.  Every wave
+// finish a row of 16 output pixels for 16 channels (a wave takes NT = 1, 2 or 4 such channel tiles).  So there is no producer / consumer split and no image in LDS here.  Every wave
 // is on its own: it owns a strip of 16 output columns of one sub-band of one member's rows and walks down the strip.
 // Lane (pixel li, tap column g) fetches the word of input pixel (row, x0 + li + g - py) itself (a buffer load whose
 // range check returns the zero word for every pixel outside the image: the implicit im2col needs no bounds
@@ -43,6 +44,9 @@ __device__ __forceinline__ uint32_t dc_div(uint32_t n, uint32_t d, uint32_t m)
     return q;
 }
 
+// lane `LANE` (a constant) of w = the scalar value v; the other lanes keep theirs
+#define NB_DC_WRITELANE(w, v, LANE) asm("v_writelane_b32 %0, %1, %2" : "+v"(w) : "s"(v), "n"(LANE))
+
 // entry b: the +-1 bytes of bits 0..7 of b
 struct DcLut {
     uint2 e[256];
@@ -65,7 +69,7 @@ constexpr DcLut dc_make_lut()
 __device__ const DcLut dc_lut_src = dc_make_lut();
 
 // MODE 2: threshold bits packed along the channels; 3: the same, 2x2 OR-pooled
-template <int MODE>
+template <int NT, int MODE>
 __global__ __launch_bounds__(256) void conv_direct_kernel(const DcConv p)
 {
     __shared__ __align__(16) uint2 lut[256];
@@ -89,36 +93,40 @@ __global__ __launch_bounds__(256) void conv_direct_kernel(const DcConv p)
     const int li = lane & 15, lg = lane >> 4;
 
     // ---- filter fragments: filter row i, lane (channel li, tap column lg) -----------------------------------------
-    dc_v4i B0, B1, B2;
-    int tdot;
+    dc_v4i B0[NT], B1[NT], B2[NT];
+    int tdot[NT];
     {
         const uint64_t *fz = p.filt + z * (int64_t)p.fwords;
-        const int ch = li < p.O ? li : p.O - 1;
-        const bool live = lg < p.fy && li < p.O;
         const uint32_t vbits = (1u << p.in_bits) - 1u;  // in_bits <= 16
-        uint32_t pmask[4];                               // bytes of the true channel positions
 #pragma unroll
-        for (int d = 0; d < 4; d++) {
-            const int nv = p.in_bits - 4 * d;
-            pmask[d] = !live || nv <= 0 ? 0u : (nv >= 4 ? 0xFFFFFFFFu : (1u << (8 * nv)) - 1u);
-        }
-        dc_v4i e[3];
+        for (int nt = 0; nt < NT; nt++) {
+            const int chn = nt * 16 + li;
+            const int ch = chn < p.O ? chn : p.O - 1;
+            const bool live = lg < p.fy && chn < p.O;
+            uint32_t pmask[4];  // bytes of the true channel positions
 #pragma unroll
-        for (int i = 0; i < 3; i++) {
-            const int tap = i * p.fy + (lg < p.fy ? lg : 0);
-            const int fr = (tap * p.tapM) >> 16, sh = p.in_bits * (tap - fr * p.tapT);  // fr = tap / tapT
-            const uint32_t fbits = (uint32_t)(fz[(int64_t)fr * p.O + ch] >> sh) & vbits;
-            e[i] = expand16(fbits);
-            e[i][0] &= (int)pmask[0];
-            e[i][1] &= (int)pmask[1];
-            e[i][2] &= (int)pmask[2];
-            e[i][3] &= (int)pmask[3];
+            for (int d = 0; d < 4; d++) {
+                const int nv = p.in_bits - 4 * d;
+                pmask[d] = !live || nv <= 0 ? 0u : (nv >= 4 ? 0xFFFFFFFFu : (1u << (8 * nv)) - 1u);
+            }
+            dc_v4i e[3];
+#pragma unroll
+            for (int i = 0; i < 3; i++) {
+                const int tap = i * p.fy + (lg < p.fy ? lg : 0);
+                const int fr = (tap * p.tapM) >> 16, sh = p.in_bits * (tap - fr * p.tapT);  // fr = tap / tapT
+                const uint32_t fbits = (uint32_t)(fz[(int64_t)fr * p.O + ch] >> sh) & vbits;
+                e[i] = expand16(fbits);
+                e[i][0] &= (int)pmask[0];
+                e[i][1] &= (int)pmask[1];
+                e[i][2] &= (int)pmask[2];
+                e[i][3] &= (int)pmask[3];
+            }
+            B0[nt] = e[0], B1[nt] = e[1], B2[nt] = e[2];
+            // thresholds in dot-product terms: 2*popc > t  <=>  popc > (t>>1)  <=>  dot < K - 2*(t>>1)
+            int64_t td = (int64_t)p.K - 2 * (int64_t)(p.thresh[z * p.O + ch] >> 1);
+            td = td > 2147483647LL ? 2147483647LL : td;
+            tdot[nt] = chn < p.O ? (int)td : -2147483647 - 1;  // channels past O never fire
         }
-        B0 = e[0], B1 = e[1], B2 = e[2];
-        // thresholds in dot-product terms: 2*popc > t  <=>  popc > (t>>1)  <=>  dot < K - 2*(t>>1)
-        int64_t td = (int64_t)p.K - 2 * (int64_t)(p.thresh[z * p.O + ch] >> 1);
-        td = td > 2147483647LL ? 2147483647LL : td;
-        tdot = li < p.O ? (int)td : -2147483647 - 1;  // channels past O never fire
     }
 
     // ---- input addressing ------------------------------------------------------------------------------------------
@@ -150,54 +158,118 @@ __global__ __launch_bounds__(256) void conv_direct_kernel(const DcConv p)
     const bool olive = lane < (MODE == 3 ? 8 : 16) && xx0 + lane < ww;
     const __amdgpu_buffer_rsrc_t orsrc =
         __builtin_amdgcn_make_buffer_rsrc(p.out + z * hh * (int64_t)ww, (short)0, hh * ww * 8, 0x00020000);
-    const uint32_t ooff = olive ? (uint32_t)((xx0 + lane) * 8) : 0xC0000000u;  // one word per pixel (O <= 16)
-    int pend0 = 0, pend1 = 0;  // MODE 3: x-pooled minima of the even row of a pair
-    auto finish_row = [&](const dc_v4i &a, int y, int par) {
-        uint64_t word;
-        if (MODE == 2) {
-            // ballot r of lane (pixel 4*g+r, channel li): bits 16*g.. are the channels of pixel 4*g+r; lane j < 16
-            // takes the piece of pixel j
-            const uint64_t m0 = __ballot(a[0] < tdot), m1 = __ballot(a[1] < tdot), m2 = __ballot(a[2] < tdot),
-                           m3 = __ballot(a[3] < tdot);
-            const int r = lane & 3;
-            const uint64_t mine = r == 0 ? m0 : r == 1 ? m1 : r == 2 ? m2 : m3;
-            word = (mine >> (16 * ((lane >> 2) & 3))) & 0xFFFFull;
+    const uint32_t ooff = olive ? (uint32_t)((xx0 + lane) * 8) : 0xC0000000u;  // one word per pixel (O <= 64)
+    int pend[NT][2];  // MODE 3: x-pooled minima of the even row of a pair
+#pragma unroll
+    for (int nt = 0; nt < NT; nt++) pend[nt][0] = pend[nt][1] = 0;
+    // 16-bit field gq (0..3) of ballot a in the low half, that of ballot b in the high half: scalar instructions
+    auto fields = [](uint64_t a, uint64_t b, int gq) {
+        const uint32_t x = gq < 2 ? (uint32_t)a : (uint32_t)(a >> 32), y = gq < 2 ? (uint32_t)b : (uint32_t)(b >> 32);
+        return (gq & 1) ? (x >> 16) | (y & 0xFFFF0000u) : (x & 0xFFFFu) | (y << 16);
+    };
+    typedef int dc_v2i __attribute__((ext_vector_type(2)));
+    auto finish_row = [&](dc_v4i (&a)[NT], int y, int par) {
+        int wlo = 0, whi = 0;
+        if (NT == 1) {
+            // one channel tile: the storing lane picks its ballot and shifts its 16 bits down itself
+            uint64_t word;
+            if (MODE == 2) {
+                // ballot r of lane (pixel 4*g+r, channel li): bits 16*g.. are the channels of pixel 4*g+r; lane
+                // j < 16 takes the piece of pixel j
+                const uint64_t m0 = __ballot(a[0][0] < tdot[0]), m1 = __ballot(a[0][1] < tdot[0]),
+                               m2 = __ballot(a[0][2] < tdot[0]), m3 = __ballot(a[0][3] < tdot[0]);
+                const int r = lane & 3;
+                const uint64_t mine = r == 0 ? m0 : r == 1 ? m1 : r == 2 ? m2 : m3;
+                word = (mine >> (16 * ((lane >> 2) & 3))) & 0xFFFFull;
+            } else {
+                // pixels 4g, 4g+1 and 4g+2, 4g+3 pool in x; rows y (even) and y+1 pool in y
+                const int v0 = a[0][0] < a[0][1] ? a[0][0] : a[0][1], v1 = a[0][2] < a[0][3] ? a[0][2] : a[0][3];
+                if (par == 0) {
+                    pend[0][0] = v0, pend[0][1] = v1;
+                    return;
+                }
+                const int w0 = v0 < pend[0][0] ? v0 : pend[0][0], w1 = v1 < pend[0][1] ? v1 : pend[0][1];
+                const uint64_t m0 = __ballot(w0 < tdot[0]), m1 = __ballot(w1 < tdot[0]);
+                const uint64_t mine = (lane & 1) ? m1 : m0;  // pooled pixel 2g + q <-> lane 2g + q
+                word = (mine >> (16 * ((lane >> 1) & 3))) & 0xFFFFull;
+            }
+            wlo = (int)(uint32_t)word;
+        } else if (MODE == 2) {
+            // several tiles: the word of pixel j = 4*g + r is put together from field g of the tiles' ballots r with
+            // scalar instructions and written into lane j's registers with v_writelane
+            uint64_t m[4][4];
+#pragma unroll
+            for (int nt = 0; nt < 4; nt++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) m[nt][r] = nt < NT ? __ballot(a[nt < NT ? nt : 0][r] < tdot[nt < NT ? nt : 0]) : 0;
+#pragma unroll
+            for (int g = 0; g < 4; g++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    NB_DC_WRITELANE(wlo, fields(m[0][r], m[1][r], g), 4 * g + r);
+                    if (NT > 2) NB_DC_WRITELANE(whi, fields(m[2][r], m[3][r], g), 4 * g + r);
+                }
         } else {
-            // pixels 4g, 4g+1 and 4g+2, 4g+3 pool in x; rows y (even) and y+1 pool in y
-            const int v0 = a[0] < a[1] ? a[0] : a[1], v1 = a[2] < a[3] ? a[2] : a[3];
             if (par == 0) {
-                pend0 = v0, pend1 = v1;
+#pragma unroll
+                for (int nt = 0; nt < NT; nt++) {
+                    pend[nt][0] = a[nt][0] < a[nt][1] ? a[nt][0] : a[nt][1];
+                    pend[nt][1] = a[nt][2] < a[nt][3] ? a[nt][2] : a[nt][3];
+                }
                 return;
             }
-            const int w0 = v0 < pend0 ? v0 : pend0, w1 = v1 < pend1 ? v1 : pend1;
-            const uint64_t m0 = __ballot(w0 < tdot), m1 = __ballot(w1 < tdot);
-            const uint64_t mine = (lane & 1) ? m1 : m0;  // pooled pixel 2g + q <-> lane 2g + q
-            word = (mine >> (16 * ((lane >> 1) & 3))) & 0xFFFFull;
+            // lane P < 8 stores pooled pixel P = 2*g + q: field g of ballot q
+            uint64_t m[4][2];
+#pragma unroll
+            for (int nt = 0; nt < 4; nt++) {
+                m[nt][0] = m[nt][1] = 0;
+                if (nt < NT) {
+                    const int n = nt < NT ? nt : 0;
+                    int v0 = a[n][0] < a[n][1] ? a[n][0] : a[n][1];
+                    int v1 = a[n][2] < a[n][3] ? a[n][2] : a[n][3];
+                    v0 = v0 < pend[n][0] ? v0 : pend[n][0];
+                    v1 = v1 < pend[n][1] ? v1 : pend[n][1];
+                    m[nt][0] = __ballot(v0 < tdot[n]);
+                    m[nt][1] = __ballot(v1 < tdot[n]);
+                }
+            }
+#pragma unroll
+            for (int g = 0; g < 4; g++)
+#pragma unroll
+                for (int q = 0; q < 2; q++) {
+                    NB_DC_WRITELANE(wlo, fields(m[0][q], m[1][q], g), 2 * g + q);
+                    if (NT > 2) NB_DC_WRITELANE(whi, fields(m[2][q], m[3][q], g), 2 * g + q);
+                }
         }
-        typedef int dc_v2i __attribute__((ext_vector_type(2)));
-        __builtin_amdgcn_raw_buffer_store_b64((dc_v2i){(int)(uint32_t)word, 0}, orsrc,
+        __builtin_amdgcn_raw_buffer_store_b64((dc_v2i){wlo, whi}, orsrc,
                                               (int)(ooff + (uint32_t)((MODE == 3 ? y >> 1 : y) * ww * 8)), 0, 2);
     };
 
     // ---- walk down the strip: band row rr feeds output rows rr (filter row 0), rr-1 (1) and rr-2 (2) ---------------
     // a0 holds the partial sums of output row rr-2 (two filter rows done), a1 those of row rr-1 (one done).  Band row
     // rr completes row rr-2 (emitted), continues row rr-1 and opens row rr with a zero C operand.
-    dc_v4i a0 = {0, 0, 0, 0}, a1 = {0, 0, 0, 0};
+    dc_v4i a0[NT], a1[NT];
     const dc_v4i zero = {0, 0, 0, 0};
+#pragma unroll
+    for (int nt = 0; nt < NT; nt++) a0[nt] = a1[nt] = zero;
     uint32_t r0 = load_row(ys), r1 = load_row(ys + 1), r2 = load_row(ys + 2), r3 = load_row(ys + 3);
 #define NB_DC_MFMA(A, B, C) __builtin_amdgcn_mfma_i32_16x16x64_i8(A, B, C, 0, 0, 0)
+    // the parts of a step: C = last (third) row of output row rr-2, M = middle row of rr-1, F = first row of rr
+#define NB_DC_PART_C(done) _Pragma("unroll") for (int nt = 0; nt < NT; nt++) done[nt] = NB_DC_MFMA(A, B2[nt], a0[nt]);
+#define NB_DC_PART_M _Pragma("unroll") for (int nt = 0; nt < NT; nt++) a0[nt] = NB_DC_MFMA(A, B1[nt], a1[nt]);
+#define NB_DC_PART_F _Pragma("unroll") for (int nt = 0; nt < NT; nt++) a1[nt] = NB_DC_MFMA(A, B0[nt], zero);
     if (ye - ys < 4) {
         // short sub-band (a few last rows of an image): every part of a step under its own (uniform) condition
-#define NB_DC_ANY(RR, X, PAR)                                                      \
-    {                                                                              \
-        const int rr_ = (RR);                                                      \
-        const dc_v4i A = expand16(X);                                              \
-        X = load_row(rr_ + 4);                                                     \
-        dc_v4i done = zero;                                                        \
-        if (rr_ - 2 >= ys) done = NB_DC_MFMA(A, B2, a0);                           \
-        if (rr_ - 1 >= ys && rr_ - 1 < ye) a0 = NB_DC_MFMA(A, B1, a1);             \
-        if (rr_ < ye) a1 = NB_DC_MFMA(A, B0, zero);                                \
-        if (rr_ - 2 >= ys) finish_row(done, rr_ - 2, PAR);                         \
+#define NB_DC_ANY(RR, X, PAR)                                          \
+    {                                                                  \
+        const int rr_ = (RR);                                          \
+        const dc_v4i A = expand16(X);                                  \
+        X = load_row(rr_ + 4);                                         \
+        dc_v4i done[NT];                                               \
+        if (rr_ - 2 >= ys) { NB_DC_PART_C(done) }                      \
+        if (rr_ - 1 >= ys && rr_ - 1 < ye) { NB_DC_PART_M }            \
+        if (rr_ < ye) { NB_DC_PART_F }                                 \
+        if (rr_ - 2 >= ys) finish_row(done, rr_ - 2, PAR);             \
     }
         for (int rr = ys; rr < ye + 2; rr += 4) {
             NB_DC_ANY(rr, r0, 0)
@@ -214,19 +286,20 @@ __global__ __launch_bounds__(256) void conv_direct_kernel(const DcConv p)
     {
         dc_v4i A = expand16(r0);
         r0 = load_row(ys + 4);
-        a1 = NB_DC_MFMA(A, B0, zero);
+        NB_DC_PART_F
         A = expand16(r1);
         r1 = load_row(ys + 5);
-        a0 = NB_DC_MFMA(A, B1, a1);
-        a1 = NB_DC_MFMA(A, B0, zero);
+        NB_DC_PART_M
+        NB_DC_PART_F
     }
 #define NB_DC_ROW(X, PAR)                                \
     {                                                    \
         const dc_v4i A = expand16(X);                    \
         X = load_row(rr + 4);                            \
-        const dc_v4i done = NB_DC_MFMA(A, B2, a0);       \
-        a0 = NB_DC_MFMA(A, B1, a1);                      \
-        a1 = NB_DC_MFMA(A, B0, zero);                    \
+        dc_v4i done[NT];                                 \
+        NB_DC_PART_C(done)                               \
+        NB_DC_PART_M                                     \
+        NB_DC_PART_F                                     \
         finish_row(done, rr - 2, PAR);                   \
         rr++;                                            \
     }
@@ -247,13 +320,17 @@ __global__ __launch_bounds__(256) void conv_direct_kernel(const DcConv p)
         const uint32_t ta = rem == 0 ? r2 : rem == 1 ? r3 : rem == 2 ? r0 : r1;
         const uint32_t tb = rem == 0 ? r3 : rem == 1 ? r0 : rem == 2 ? r1 : r2;
         dc_v4i A = expand16(ta);
-        dc_v4i done = NB_DC_MFMA(A, B2, a0);
-        a0 = NB_DC_MFMA(A, B1, a1);
+        dc_v4i done[NT];
+        NB_DC_PART_C(done)
+        NB_DC_PART_M
         finish_row(done, ye - 2, (ye - ys) & 1);
         A = expand16(tb);
-        done = NB_DC_MFMA(A, B2, a0);
+        NB_DC_PART_C(done)
         finish_row(done, ye - 1, (ye - 1 - ys) & 1);
     }
+#undef NB_DC_PART_C
+#undef NB_DC_PART_M
+#undef NB_DC_PART_F
 #undef NB_DC_MFMA
 }
 
@@ -265,7 +342,7 @@ bool conv_direct_try(void *out, const uint64_t *in, const uint64_t *filt, const 
     if (mode != 2 && mode != 3) return false;
     if (tap_bits < 1 || tap_bits > 16 || g.Cw != 1) return false;
     if (g.sx != 1 || g.sy != 1 || g.fx != 3 || g.fy < 1 || g.fy > 3) return false;
-    if (O < 1 || O > 16 || D < 1 || g.h < 1 || g.w < 1) return false;
+    if (O < 1 || O > 64 || D < 1 || g.h < 1 || g.w < 1) return false;
     if (mode == 3 && (g.h < 2 || g.w < 2)) return false;
     // 32-bit byte offsets inside one member's image, far enough below 2^30 for the out-of-range marker
     if ((int64_t)(g.H + g.px + 8) * g.Wd * 8 >= (1LL << 29) || (int64_t)g.h * g.w * 8 >= (1LL << 30)) return false;
@@ -300,10 +377,18 @@ bool conv_direct_try(void *out, const uint64_t *in, const uint64_t *filt, const 
     p.mntx = (uint32_t)((1ULL << 32) / (uint32_t)p.ntx);  // unused for a divisor of 1
     p.mnsb = (uint32_t)((1ULL << 32) / (uint32_t)p.nsb);
     const int64_t blocks = ceil_div(units, 4);
-    if (mode == 2)
-        conv_direct_kernel<2><<<dim3((unsigned)blocks), dim3(256), 0, s>>>(p);
-    else
-        conv_direct_kernel<3><<<dim3((unsigned)blocks), dim3(256), 0, s>>>(p);
+    const int NT = O <= 16 ? 1 : O <= 32 ? 2 : 4;
+#define NB_DC_LAUNCH(nt)                                                   \
+    if (NT == nt) {                                                        \
+        if (mode == 2)                                                     \
+            conv_direct_kernel<nt, 2><<<dim3((unsigned)blocks), dim3(256), 0, s>>>(p); \
+        else                                                               \
+            conv_direct_kernel<nt, 3><<<dim3((unsigned)blocks), dim3(256), 0, s>>>(p); \
+    }
+    NB_DC_LAUNCH(1)
+    NB_DC_LAUNCH(2)
+    NB_DC_LAUNCH(4)
+#undef NB_DC_LAUNCH
     return true;
 }
 

@@ -581,8 +581,8 @@ def test_conv_matrix_core_engine_vs_oracle(ops, oracle, mc_engine, C, O, k, pad,
         ops.conv_engine(prev)
 
 
-# (C, O, fy, px, py, H, W, D): the wave-per-strip matrix-core kernel for narrow layers (at most 16 channels in and
-# out, packed output).  Output channel counts below 16, channel counts that leave zero positions in a pixel's 16,
+# (C, O, fy, px, py, H, W, D): the wave-per-strip matrix-core kernel for narrow layers (at most 16 channels in, at
+# most 64 out, packed output).  Output channel counts below 16, channel counts that leave zero positions in a pixel's 16,
 # one to three filter columns, paddings 0-2, images of one to three rows (the short sub-band path), odd heights (the
 # pooled map drops the last row), several sub-bands with 13 to 20 rows (every remainder of the four-row loop),
 # several strips with a ragged last one, and a population large enough for whole-image sub-bands.
@@ -600,6 +600,12 @@ NARROW_CASES = [
     (16, 11, 3, 1, 1, 50, 48, 1),
     (9, 16, 3, 1, 2, 38, 31, 3),
     (16, 16, 3, 1, 1, 21, 16, 300),
+    (16, 32, 3, 1, 1, 20, 18, 3),              # two channel tiles per wave
+    (12, 17, 3, 1, 1, 19, 33, 2),
+    (16, 64, 3, 1, 1, 35, 40, 2),              # four tiles: a whole output word
+    (9, 33, 2, 0, 1, 67, 20, 2),
+    (16, 48, 3, 1, 1, 3, 40, 3),               # four tiles, one of them dead; the short sub-band path
+    (8, 64, 3, 1, 1, 38, 31, 130),
 ]
 
 
