@@ -110,6 +110,16 @@ int nb_bmv_bn_act_static_i64(void *out, const int64_t *A, const int64_t *x, cons
                              const uint16_t *bias_noise, int64_t Z, int64_t M, int64_t Kw, int64_t K, int pack,
                              nb_stream_t stream);
 
+/* Thresholds of BinarizedConv2d(batch_norm=True) (modules/binary.py:147-155) from the pixel sums that
+ * nb_conv_popc_sums_* returns: with act = 2*popc - K over the HW output pixels,
+ *     mean[d,o] = fp16(float(sum_pixels act) / float(HW)),  thr = fp16(fp16(bias[o] + bias_noise[d,o]) + mean),
+ *     thresh[d,o] = floor(thr) + K  (int32, clamped; INT32_MAX for NaN),
+ * so that nb_conv_act*(..., thresh, ...) (2*popc > thresh) decides act > thr exactly as long as the activations are
+ * integers that fp16 holds exactly (K <= 2048).  sums, thresh int32 [D,O]; bias fp16 [O]; bias_noise fp16 [D,O].
+ * Replaces a dozen elementwise tensor operations of the layer; no single counterpart in the reference. */
+int nb_conv_bn_thresholds(int32_t *thresh, const int32_t *sums, const uint16_t *bias, const uint16_t *bias_noise,
+                          int64_t D, int64_t O, int64_t K, int64_t HW, nb_stream_t stream);
+
 /* ---- sparse form of a population's linear layer: shared base + per-member flip lists ------------------------
  * For per-member weights W[d] = base ^ flips[d] with few flips per row (BASELINE's "base XOR Bernoulli(p) flip mask"),
  *     popcount(x ^ W[d,r]) = popcount(x ^ base[r]) + |flips[d,r]| - 2 * popcount(flips[d,r] & (x ^ base[r])):

@@ -55,6 +55,7 @@ _PLAIN = {
     "nb_bmv_flip_i64": [_PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _I64, _I64, _I64, _PTR],
     "nb_bmv_flip_act_pack_i64": [_PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _I64, _I64, _I64, _PTR],
     "nb_bmv_bn_act_static_i64": [_PTR, _PTR, _PTR, _PTR, _PTR, _I64, _I64, _I64, _I64, _I32, _PTR],
+    "nb_conv_bn_thresholds": [_PTR, _PTR, _PTR, _PTR, _I64, _I64, _I64, _I64, _PTR],
 }
 # entry points that return a size (int64) instead of a status
 _SIZES = {

@@ -174,9 +174,59 @@ static int bn_static_ptr(void **ptr, const char *who)
     return NB_OK;
 }
 
+// Thresholds of BinarizedConv2d(batch_norm=True) from the pixel sums of the popcount maps (modules/binary.py:147-155):
+// act = 2*popc - K, mean[d,o] = fp16(float(sum over the HW pixels of act) / float(HW)),
+// thr = fp16(fp16(bias[o] + noise[d,o]) + mean); act > thr  <=>  2*popc > floor(thr) + K, which is what is written
+// (clamped to int32; never for NaN).  One thread per (member, channel).
+__global__ __launch_bounds__(256) void bn_conv_thresh_kernel(int32_t *__restrict__ thresh, const int32_t *__restrict__ sums,
+                                                             const _Float16 *__restrict__ bias,
+                                                             const _Float16 *__restrict__ noise, int64_t D, int64_t O,
+                                                             int64_t K, int64_t HW)
+{
+    NB_FLAT_LOOP(t, D * O)
+    {
+        if (t < D * O) {
+            const int64_t o = t % O;
+            const long long sum_act = 2ll * (long long)sums[t] - (long long)K * (long long)HW;
+            const _Float16 mean = (_Float16)((float)sum_act / (float)HW);
+            const _Float16 tb = bias[o] + noise[t];
+            const float v = (float)(_Float16)(tb + mean);
+            long long th;
+            if (v != v) {
+                th = 2147483647ll;  // NaN: never above it
+            } else {
+                th = (long long)floorf(fminf(fmaxf(v, -3.0e9f), 3.0e9f)) + (long long)K;
+                th = th > 2147483647ll ? 2147483647ll : (th < -2147483648ll ? -2147483648ll : th);
+            }
+            thresh[t] = (int32_t)th;
+        }
+    }
+}
+
 }  // namespace nb
 
 extern "C" {
+int nb_conv_bn_thresholds(int32_t *thresh, const int32_t *sums, const uint16_t *bias, const uint16_t *bias_noise,
+                           int64_t D, int64_t O, int64_t K, int64_t HW, nb_stream_t stream)
+{
+    const char *who = "nb_conv_bn_thresholds";
+    NB_REQUIRE(D >= 0 && O >= 0 && K >= 0 && HW >= 1, "%s: bad shape D=%lld O=%lld K=%lld HW=%lld", who, (long long)D,
+               (long long)O, (long long)K, (long long)HW);
+    NB_REQUIRE(K < (1LL << 31) && HW < (1LL << 31) && D * O < (1LL << 40), "%s: too large", who);
+    if (D * O == 0) return NB_OK;
+    NB_REQUIRE_PTR(thresh);
+    NB_REQUIRE_PTR(sums);
+    NB_REQUIRE_PTR(bias);
+    NB_REQUIRE_PTR(bias_noise);
+    NB_REQUIRE_ALIGNED(thresh, 4);
+    NB_REQUIRE_ALIGNED(sums, 4);
+    NB_REQUIRE_ALIGNED(bias, 2);
+    NB_REQUIRE_ALIGNED(bias_noise, 2);
+    nb::bn_conv_thresh_kernel<<<dim3(nb::grid_for(D * O)), dim3(256), 0, nb::as_stream(stream)>>>(
+        thresh, sums, reinterpret_cast<const _Float16 *>(bias), reinterpret_cast<const _Float16 *>(bias_noise), D, O, K,
+        HW);
+    return nb::check_launch(who);
+}
 int64_t nb_bmv_bn_workspace_bytes(int64_t Z, int64_t M)
 {
     if (Z < 0 || M < 0 || Z >= (1LL << 31) || M >= (1LL << 31)) return -1;

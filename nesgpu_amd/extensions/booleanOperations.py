@@ -225,6 +225,29 @@ def bmv_bn_act(A, x, bias, bias_noise, in_bits, pack=False, workspace=None):
     return out
 
 
+def conv_bn_thresholds(sums, bias, bias_noise, in_bits, pixels):
+    """Thresholds of ``BinarizedConv2d(batch_norm=True)`` (modules/binary.py:147-155) from ``conv_popc_sums``: with
+    act = 2*popc - in_bits, mean = fp16(float(sum over the pixels of act) / pixels),
+    thr = fp16(fp16(bias + bias_noise) + mean); returns int32 [D,O] = floor(thr) + in_bits (INT32_MAX for NaN), the
+    threshold of ``conv_act`` / ``conv_act_pack`` (2*popc > threshold).  sums int32 [D,O], bias fp16 [O], bias_noise
+    fp16 [D,O].  One kernel instead of a dozen elementwise tensor operations."""
+    _check(sums, "sums")
+    _check(bias, "bias")
+    _check(bias_noise, "bias_noise")
+    _same_device(sums, bias)
+    _same_device(sums, bias_noise)
+    assert sums.dtype == torch.int32 and len(sums.shape) == 2
+    D, O = sums.shape
+    assert bias.dtype == torch.float16 and tuple(bias.shape) == (O,)
+    assert bias_noise.dtype == torch.float16 and tuple(bias_noise.shape) == (D, O)
+    assert in_bits >= 0 and pixels >= 1
+    out = torch.empty((D, O), dtype=torch.int32, device=sums.device)
+    with _on(sums):
+        _lib.call("nb_conv_bn_thresholds", out.data_ptr(), sums.data_ptr(), bias.data_ptr(), bias_noise.data_ptr(), D, O,
+                  int(in_bits), int(pixels), _stream(sums))
+    return out
+
+
 def conv_engine(engine=None):
     """Query / set the process-wide conv engine: 0 = automatic (matrix cores for populations of 128 or more, else
     XOR-popcount), 1 = XOR-popcount kernels only, 2 = matrix cores wherever a kernel covers the shape (FP4 codes for

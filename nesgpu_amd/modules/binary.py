@@ -228,10 +228,9 @@ class BinarizedConv2d(Binarized):
                 # modules/binary.py:147-155 without the int32 maps: the per-member mean over h,w needs only the sum of
                 # the popcounts (exact integers), mean = fp16(float(sum of activations) / (h*w)); activations are
                 # integers that fp16 holds exactly, so activation > thresh  <=>  2*popc > floor(thresh) + offset.
-                sums = booleanOperations.conv_popc_sums(packed_input, filt, *geom, **tapkw).to(torch.int64)
+                sums = booleanOperations.conv_popc_sums(packed_input, filt, *geom, **tapkw)
                 h, w = booleanOperations._out_hw(packed_input, *geom)
-                mean = ((2 * sums - offset * h * w).to(torch.float32) / float(h * w)).to(torch.float16)
-                thresh = torch.floor((self.bias + self.bias_noise + mean).to(torch.float32)).to(torch.int32) + offset
+                thresh = booleanOperations.conv_bn_thresholds(sums, self.bias.detach(), self.bias_noise, offset, h * w)
             else:
                 thresh = (self.bias + self.bias_noise).type(torch.int32) + offset
             if self.pack_output or self.pool_output:

@@ -240,3 +240,28 @@ def test_reference_import_names_resolve(binary):
                 sys.modules.pop(k, None)
             else:
                 sys.modules[k] = v
+
+
+def test_conv_bn_thresholds_equal_the_layer_arithmetic():
+    from nesgpu_amd.extensions import booleanOperations as ops
+    """conv_bn_thresholds against the tensor expression it replaces (modules/binary.py:147-155 on exact pixel sums):
+    mean = fp16(float32(sum of activations) / float32(pixels)), thr = fp16(fp16(bias + noise) + mean),
+    threshold = floor(thr) + K; random sums over the whole range, biases that round in fp16, and the non-finite cases
+    decided like `activation > thr` (never for NaN and +inf, always for -inf)."""
+    g = torch.Generator(device="cuda")
+    g.manual_seed(11)
+    for D, O, K, pixels in [(64, 64, 576, 1024), (7, 5, 144, 4096), (300, 16, 27, 49), (3, 130, 2048, 1)]:
+        sums = torch.randint(0, K * pixels + 1, (D, O), dtype=torch.int32, device="cuda", generator=g)
+        bias = (torch.randn(O, device="cuda", generator=g) * 30).to(torch.float16)
+        noise = (torch.rand(D, O, device="cuda", generator=g) - 0.5).to(torch.float16)
+        got = ops.conv_bn_thresholds(sums, bias, noise, K, pixels)
+        s64 = sums.to(torch.int64)
+        mean = ((2 * s64 - K * pixels).to(torch.float32) / float(pixels)).to(torch.float16)
+        want = torch.floor((bias + noise + mean).to(torch.float32)).to(torch.int32) + K
+        assert got.dtype == torch.int32 and torch.equal(got, want)
+    sums = torch.full((1, 4), 100, dtype=torch.int32, device="cuda")
+    bias = torch.tensor([float("nan"), float("inf"), float("-inf"), 60000.0], dtype=torch.float16, device="cuda")
+    noise = torch.tensor([[0.0, 0.0, 0.0, 60000.0]], dtype=torch.float16, device="cuda")       # 60000 + 60000 = inf
+    got = ops.conv_bn_thresholds(sums, bias, noise, 144, 64).cpu().tolist()[0]
+    assert got[0] == 2 ** 31 - 1 and got[1] == 2 ** 31 - 1 and got[3] == 2 ** 31 - 1             # never above
+    assert got[2] < -2 ** 30                                                                      # always above
