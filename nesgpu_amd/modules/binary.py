@@ -11,7 +11,8 @@ defects of the reference snapshot are not reproduced: construction order (``Pert
 Additions, all opt-in: ``set_noise(words=...)`` samples from caller-supplied uint32 words (bit-exact
 parity mode), ``set_noise(bias_generator=...)`` draws the bias noise from a given torch.Generator instead of the
 global one, and ``BinarizedConv2d(pack_output=True[, pool_output=True])`` returns the thresholded map
-already packed along channels (and 2x2 OR-pooled) from one fused kernel instead of a bool map.
+already packed along channels (and 2x2 OR-pooled) from one fused kernel instead of a bool map;
+``fuse_packed_outputs(model)`` switches those on wherever a reference-style ``nn.Sequential`` allows it.
 """
 import torch
 from torch import nn
@@ -262,3 +263,57 @@ class BinarizedMaxPool2d(nn.Module):
         else:
             packed_input = input
         return booleanOperations.max_pool2d(packed_input, *self.kernel_size, *self.padding, *self.stride)
+
+
+def fuse_packed_outputs(model):
+    """Switches the fused outputs on in a reference-style stack of layers (not in the reference; results unchanged).
+
+    Walks every ``nn.Sequential`` inside ``model``: a thresholding ``BinarizedConv2d`` followed by a 2x2 / stride 2 /
+    no-padding ``BinarizedMaxPool2d`` gets ``pool_output=True`` and the pool becomes ``nn.Identity``; a thresholding
+    conv or linear layer whose output goes (through ``nn.Flatten`` at most) into another binary layer, which accepts
+    packed words, gets ``pack_output=True``.  A conv in front of ``nn.Flatten`` is only switched when its channel
+    count fills whole words, so that the flattened packed words are the flattened bits, and layers with more than
+    2048 inputs per output are left alone (their activations are beyond fp16's exact integers, where the reference's
+    fp16 comparison and the fused integer comparison can differ).  Returns the number of layers changed."""
+    changed = 0
+    for seq in [m for m in model.modules() if isinstance(m, nn.Sequential)]:
+        layers = list(seq)
+        for i, layer in enumerate(layers):
+            if not isinstance(layer, (BinarizedConv2d, BinarizedLinear)) or not layer.threshold:
+                continue
+            # the fused kernels compare integers; the reference compares in fp16, which is the same thing as long as
+            # the activations are integers that fp16 holds exactly
+            if isinstance(layer, BinarizedConv2d):
+                fan_in = layer.in_channels * layer.kernel_size[0] * layer.kernel_size[1]
+            else:
+                fan_in = layer.in_features
+            if fan_in > 2048:
+                continue
+            j = i + 1
+            if isinstance(layer, BinarizedConv2d) and j < len(layers) and isinstance(layers[j], BinarizedMaxPool2d):
+                pool = layers[j]
+                if (tuple(pool.kernel_size), tuple(pool.padding), tuple(pool.stride)) == ((2, 2), (0, 0), (2, 2)) \
+                        and pool.dtype == layer.dtype and not layer.pool_output:
+                    layer.pool_output = True
+                    seq[j] = nn.Identity()
+                    layers[j] = seq[j]
+                    changed += 1
+                continue                      # a pool's output is packed either way
+            if getattr(layer, "pool_output", False):
+                continue                      # already packed (and pooled)
+            through_flatten = False
+            while j < len(layers) and isinstance(layers[j], (nn.Flatten, nn.Identity)):
+                through_flatten = through_flatten or isinstance(layers[j], nn.Flatten)
+                j += 1
+            if j >= len(layers) or not isinstance(layers[j], (BinarizedConv2d, BinarizedLinear, BinarizedMaxPool2d)):
+                continue
+            if layers[j].dtype != layer.dtype or layer.pack_output:
+                continue
+            bits = torch.iinfo(layer.dtype).bits
+            if isinstance(layer, BinarizedConv2d) and through_flatten and layer.out_channels % bits:
+                continue
+            if isinstance(layer, BinarizedLinear) and isinstance(layers[j], (BinarizedConv2d, BinarizedMaxPool2d)):
+                continue                      # a linear layer's row is not an image
+            layer.pack_output = True
+            changed += 1
+    return changed

@@ -179,3 +179,46 @@ def test_extract_bits_on_the_gpu(binary, oracle, dtype, np_dtype):
     np.testing.assert_array_equal(packed.view(np.uint8).reshape(5, -1), raw)
     if dtype == torch.uint8:                                     # the same words int8pack makes from the bytes
         np.testing.assert_array_equal(ops.int8pack(dev(v), torch.int64).cpu().numpy(), packed)
+
+
+def test_fuse_packed_outputs_changes_nothing_but_the_kernels(binary):
+    """fuse_packed_outputs on the SmallNet-shaped stack: the two convs take their pools in (pool_output), nothing else
+    is eligible (the last layer has 16384 inputs per output); same predictions as the unfused stack from the same
+    seeds.  On a stack of small layers every boundary is fused: conv -> pool, conv -> Flatten -> linear (64 channels =
+    whole words), linear -> linear; same outputs again."""
+    D = 8
+    g = np.random.default_rng(9)
+    planes = binary.ExtractBits(torch.uint8)(dev(g.integers(0, 256, size=(D, 32, 32, 3)).astype(np.uint8)))
+    bg = torch.Generator(device="cuda")
+
+    def run(model):
+        pm = binary.PerturbedModel(model, D)
+        with torch.no_grad():
+            pm.set_seed(31)
+            pm.set_noise_scale(0.1)
+            bg.manual_seed(5)
+            pm.set_noise(bias_generator=bg)
+            return pm.forward(planes)
+
+    model = small_net(binary, D, 10)
+    randomise(model, 3)
+    want = run(model)
+    assert binary.fuse_packed_outputs(model) == 2
+    assert [type(l).__name__ for l in model] == ["BinarizedConv2d", "Identity", "BinarizedConv2d", "Identity", "Flatten",
+                                                 "BinarizedLinear"]
+    assert model[0].pool_output and model[2].pool_output and not model[5].pack_output
+    assert torch.equal(run(model), want)
+    assert binary.fuse_packed_outputs(model) == 0                               # idempotent
+
+    small = torch.nn.Sequential(
+        binary.BinarizedConv2d(24, 16, D, 3, batch_norm=True, padding=1), binary.BinarizedMaxPool2d(),
+        binary.BinarizedConv2d(16, 64, D, 3, batch_norm=False, padding=1), torch.nn.Flatten(),
+        binary.BinarizedLinear(16 * 16 * 64, 96, D),
+        binary.BinarizedLinear(96, 10, D, batch_norm=True))
+    randomise(small, 4)
+    want = run(small)
+    n = binary.fuse_packed_outputs(small)
+    assert small[0].pool_output and small[2].pack_output and small[5].threshold
+    assert not small[4].pack_output                                            # 16384 inputs per output: left alone
+    assert n == 2
+    assert torch.equal(run(small), want)
