@@ -240,8 +240,9 @@ int nb_conv_popc_sums_i32(int32_t *sums, const int32_t *in, const int32_t *filt,
  * one band of a member's image fits LDS) that feeds the bits to the matrix cores as +-1 bytes (int8 MFMA) or, for
  * full channel words of 64, 128 or 256 channels, as FP4 codes (FP4 MFMA, twice the rate, exact for +-1).
  * Narrow layers (tap-packed filters of at most 16 channels, at most 64 output channels, 3-row windows of up to 3
- * columns, stride 1, packed output) have a matrix-core kernel of their own that serves any population; so have
- * packed outputs of 3x3 windows over one full channel word per pixel (FP4; engines 0 and 2).
+ * columns, stride 1, packed output) have a matrix-core kernel of their own that serves any population; packed
+ * outputs and pixel sums of 3x3 windows over one word per pixel have another (tap-packed filters of 17 to 32
+ * channels as +-1 bytes; full channel words as FP4 codes, engines 0 and 2).
  * 0 = automatic: the matrix-core kernels for populations of 128 members or more (the narrow one always), else
  * XOR-popcount;
  * 1 = XOR-popcount only; 2 = matrix cores wherever a kernel covers the shape; 3 = as 2, +-1 bytes only.  Returns

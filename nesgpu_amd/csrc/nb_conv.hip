@@ -282,12 +282,16 @@ int conv_impl(void *out, const W *in, const W *filt, const int32_t *thresh, int6
         t_last_engine = 2;
         return check_launch(who);
     }
-    // One full channel word per pixel, 3x3, packed output: the same wave-per-strip scheme on the FP4 matrix cores.
-    if (bits == 64 && Cw == 1 && (engine == 2 || (engine == 0 && D >= 128)) &&
-        conv_direct_fp4_try(out, reinterpret_cast<const uint64_t *>(in), reinterpret_cast<const uint64_t *>(filt), thresh,
-                            g, D, N, tap_bits, mode, s)) {
-        t_last_engine = 4;
-        return check_launch(who);
+    // One word per pixel, 3x3, packed output or pixel sums: the same wave-per-strip scheme for full channel words
+    // (FP4 matrix cores) and for tap-packed layers of 17 to 32 channels (int8).
+    if (bits == 64 && Cw == 1 && engine != 1 && (engine >= 2 || D >= 128)) {
+        const int ran = conv_direct_fp4_try(out, reinterpret_cast<const uint64_t *>(in),
+                                            reinterpret_cast<const uint64_t *>(filt), thresh, g, D, N, tap_bits, mode,
+                                            engine != 3, s);
+        if (ran) {
+            t_last_engine = ran;
+            return check_launch(who);
+        }
     }
     if (bits == 64 && Cw > 0 && engine != 1 && (engine >= 2 || D >= 128)) {
         const int ran = conv_mfma_try(out, reinterpret_cast<const uint64_t *>(in), reinterpret_cast<const uint64_t *>(filt),

@@ -20,6 +20,11 @@
 // so the third tap column costs two MFMAs per row instead of three: five per row and 16 channels, not six.
 // Finished rows are compared with the thresholds (as dot products), gathered with ballots, pooled (in x a min over
 // neighbouring accumulator registers, in y over two walked rows) and stored as whole words.
+//
+// The same kernel has an int8 flavour (Q = 0) for tap-packed layers of 17 to 32 channels (the first layer of a
+// network fed with 3 x 8 bit planes): a pixel is 32 positions of +-1 bytes, a lane supplies 16 of them, one
+// v_mfma_i32_16x16x64_i8 takes two (pixel column, 32 channels) pairs, and everything else is as above with integer
+// sums (no bias needed).  Positions past the channel count are zero bytes in the filter fragments.
 #include "nb_conv_common.hpp"
 
 namespace nb {
@@ -33,6 +38,7 @@ struct DwConv {
     const int32_t *thresh;
     void *out;
     int H, Wd, px, py, h, w, O, Ow, K;
+    int in_bits, tapT, tapM, fwords;  // Q = 0: channels, taps per filter word, (tap * tapM) >> 16 = tap / tapT, words
     int ntx, ncg, nsb, hb;  // strips of 16 columns, channel groups of 16*NT, sub-bands per member, rows per sub-band
     uint32_t units;         // D * nsb * ncg * ntx
     uint32_t mntx, mncg, mnsb;
@@ -62,6 +68,27 @@ constexpr DwLut dw_make_lut()
 }
 __device__ const DwLut dw_lut_src = dw_make_lut();
 
+// entry b: the +-1 bytes of bits 0..7 of b (1 -> 0x01, 0 -> 0xFF)
+struct DwLut8 {
+    uint2 e[256];
+};
+constexpr uint32_t dw_pm1_const(uint32_t nib)
+{
+    uint32_t w = 0;
+    for (int j = 0; j < 4; j++) w |= (((nib >> j) & 1u) ? 0x01u : 0xFFu) << (8 * j);
+    return w;
+}
+constexpr DwLut8 dw_make_lut8()
+{
+    DwLut8 t{};
+    for (uint32_t b = 0; b < 256; b++) {
+        t.e[b].x = dw_pm1_const(b & 15u);
+        t.e[b].y = dw_pm1_const(b >> 4);
+    }
+    return t;
+}
+__device__ const DwLut8 dw_lut8_src = dw_make_lut8();
+
 // lane `LANE` (a constant) of w = the scalar value v; the other lanes keep theirs
 #define NB_DW_WRITELANE(w, v, LANE) asm("v_writelane_b32 %0, %1, %2" : "+v"(w) : "s"(v), "n"(LANE))
 
@@ -71,22 +98,46 @@ __device__ __forceinline__ dw_v4f dw_mfma(dw_v4i a, dw_v4i b, dw_v4f c)
     const dw_v8i b8 = __builtin_shufflevector(b, b, 0, 1, 2, 3, -1, -1, -1, -1);
     return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a8, b8, c, 4, 4, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
 }
+__device__ __forceinline__ dw_v4i dw_mfma(dw_v4i a, dw_v4i b, dw_v4i c)
+{
+    return __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, c, 0, 0, 0);
+}
+template <int Q>
+struct DwAcc {
+    typedef dw_v4f type;
+};
+template <>
+struct DwAcc<0> {
+    typedef dw_v4i type;
+};
 
 // MODE 2: threshold bits packed along the channels; 3: the same, 2x2 OR-pooled; 4: the popcount sums added up over
 // the pixels, int32 [D,O] (atomic adds into a zeroed array)
-template <int NT, int MODE>
+// Q: 1 = FP4 codes, one full channel word per pixel; 0 = +-1 bytes, 17 to 32 channels (tap-packed filter)
+template <int NT, int MODE, int Q>
 __global__ __launch_bounds__(256) void conv_direct_fp4_kernel(const DwConv p)
 {
-    __shared__ uint32_t lut[256];
-    lut[threadIdx.x] = dw_lut_src.e[threadIdx.x];
+    typedef typename DwAcc<Q>::type acc_t;
+    __shared__ __align__(16) uint2 lut_s[Q ? 128 : 256];  // Q = 1: 256 four-byte entries; Q = 0: 256 eight-byte entries
+    if (Q)
+        reinterpret_cast<uint32_t *>(lut_s)[threadIdx.x] = dw_lut_src.e[threadIdx.x];
+    else
+        lut_s[threadIdx.x] = dw_lut8_src.e[threadIdx.x];
     __syncthreads();
-    const unsigned char *lutb = reinterpret_cast<const unsigned char *>(lut);
-    auto expand32 = [&](uint32_t x) {  // 32 bits -> 32 codes in 16 bytes
-        const uint32_t a = *reinterpret_cast<const uint32_t *>(lutb + ((x & 0xFFu) << 2));
-        const uint32_t b = *reinterpret_cast<const uint32_t *>(lutb + (((x >> 8) & 0xFFu) << 2));
-        const uint32_t c = *reinterpret_cast<const uint32_t *>(lutb + (((x >> 16) & 0xFFu) << 2));
-        const uint32_t d = *reinterpret_cast<const uint32_t *>(lutb + ((x >> 24) << 2));
-        return (dw_v4i){(int)a, (int)b, (int)c, (int)d};
+    const unsigned char *lutb = reinterpret_cast<const unsigned char *>(lut_s);
+    // the lane's 16 bytes of a pixel: Q = 1: the 32 bits x -> 32 codes; Q = 0: bits 0..15 of x -> 16 bytes of +-1
+    auto expand32 = [&](uint32_t x) {
+        if (Q) {
+            const uint32_t a = *reinterpret_cast<const uint32_t *>(lutb + ((x & 0xFFu) << 2));
+            const uint32_t b = *reinterpret_cast<const uint32_t *>(lutb + (((x >> 8) & 0xFFu) << 2));
+            const uint32_t c = *reinterpret_cast<const uint32_t *>(lutb + (((x >> 16) & 0xFFu) << 2));
+            const uint32_t d = *reinterpret_cast<const uint32_t *>(lutb + ((x >> 24) << 2));
+            return (dw_v4i){(int)a, (int)b, (int)c, (int)d};
+        } else {
+            const uint2 a = *reinterpret_cast<const uint2 *>(lutb + ((x & 0xFFu) << 3));
+            const uint2 b = *reinterpret_cast<const uint2 *>(lutb + (((x >> 8) & 0xFFu) << 3));
+            return (dw_v4i){(int)a.x, (int)a.y, (int)b.x, (int)b.y};
+        }
     };
     const int lane = threadIdx.x & 63;
     // the unit is uniform over the wave, and visibly so: every branch around an MFMA must be a scalar branch,
@@ -107,11 +158,28 @@ __global__ __launch_bounds__(256) void conv_direct_fp4_kernel(const DwConv p)
     dw_v4i B0[3][NT], B1a[NT], B1b[NT];
     int tdot[NT];
     {
-        const uint64_t *fz = p.filt + z * (int64_t)(9 * p.O);
+        const uint64_t *fz = p.filt + z * (int64_t)(Q ? 9 * p.O : p.fwords);
+        // the lane's half of the filter word of (tap, channel): Q = 1: 32 of its 64 bits; Q = 0: bits 16*hf.. of the
+        // tap's in_bits bits inside a tap-packed word
         auto half = [&](int tap, int ch) {
-            const uint64_t wd = fz[(int64_t)tap * p.O + ch];
-            return hf ? (uint32_t)(wd >> 32) : (uint32_t)wd;
+            if (Q) {
+                const uint64_t wd = fz[(int64_t)tap * p.O + ch];
+                return hf ? (uint32_t)(wd >> 32) : (uint32_t)wd;
+            } else {
+                const int fr = (tap * p.tapM) >> 16, sh = p.in_bits * (tap - fr * p.tapT);  // fr = tap / tapT
+                const uint32_t bits = (uint32_t)(fz[(int64_t)fr * p.O + ch] >> sh) & (uint32_t)((1ull << p.in_bits) - 1ull);
+                return (bits >> (16 * hf)) & 0xFFFFu;
+            }
         };
+        // Q = 0: the bytes of positions past the channel count are cleared (the upper half holds positions 16..31)
+        dw_v4i pmask = {-1, -1, -1, -1};
+        if (!Q && hf) {
+#pragma unroll
+            for (int d = 0; d < 4; d++) {
+                const int nv = p.in_bits - 16 - 4 * d;
+                pmask[d] = nv <= 0 ? 0 : (nv >= 4 ? -1 : (int)((1u << (8 * nv)) - 1u));
+            }
+        }
 #pragma unroll
         for (int nt = 0; nt < NT; nt++) {
             const int ch = (cg * NT + nt) * 16 + li;
@@ -119,10 +187,10 @@ __global__ __launch_bounds__(256) void conv_direct_fp4_kernel(const DwConv p)
             const int chc = live ? ch : p.O - 1;
 #pragma unroll
             for (int i = 0; i < 3; i++) {
-                B0[i][nt] = expand32(half(i * 3 + tc, chc));  // a channel past O multiplies whatever: it never fires
+                B0[i][nt] = expand32(half(i * 3 + tc, chc)) & pmask;  // a channel past O multiplies whatever: it never fires
             }
-            B1a[nt] = expand32(half(tc * 3 + 2, chc));    // f(0,2) | f(1,2)
-            const dw_v4i eb = expand32(half(8, chc));     // f(2,2) | 0
+            B1a[nt] = expand32(half(tc * 3 + 2, chc)) & pmask;    // f(0,2) | f(1,2)
+            const dw_v4i eb = expand32(half(8, chc)) & pmask;     // f(2,2) | 0
             B1b[nt] = tc == 0 ? eb : zero_i;
             // thresholds in dot-product terms: 2*popc > t  <=>  popc > (t>>1)  <=>  dot < K - 2*(t>>1); every dot
             // product lies in [-K, K], so thresholds outside mean always / never and are pulled in to K + 1 / -K - 1
@@ -130,10 +198,10 @@ __global__ __launch_bounds__(256) void conv_direct_fp4_kernel(const DwConv p)
             t = t > 2 * p.K + 4 ? 2 * p.K + 4 : (t < -2 * p.K - 4 ? -2 * p.K - 4 : t);  // beyond: always / never, too
             int td = live ? p.K - 2 * (t >> 1) : -p.K - 1;
             td = td > p.K + 1 ? p.K + 1 : (td < -p.K - 1 ? -p.K - 1 : td);
-            // The accumulators start at K + 1 instead of 0, so every sum is a positive float and its bit pattern
-            // orders like the value: minima and comparisons are integer instructions (one each; the float forms
-            // cost a compare and a select).
-            tdot[nt] = __builtin_bit_cast(int, (float)(td + p.K + 1));
+            // Q = 1: the accumulators start at K + 1 instead of 0, so every sum is a positive float and its bit
+            // pattern orders like the value: minima and comparisons are integer instructions (one each; the float
+            // forms cost a compare and a select).
+            tdot[nt] = Q ? __builtin_bit_cast(int, (float)(td + p.K + 1)) : td;
         }
     }
 
@@ -150,13 +218,15 @@ __global__ __launch_bounds__(256) void conv_direct_fp4_kernel(const DwConv p)
     // added; a row outside gives a negative or too large offset by itself.
     constexpr uint32_t kOutside = 0xC0000000u;
     const int xa = x0 + li + tc - p.py, xb = x0 + li + 2 - p.py;
-    const uint32_t offa = (xa >= 0 && xa < p.Wd) ? (uint32_t)(xa * 8 + 4 * hf) : kOutside;
-    const uint32_t offb = (xb >= 0 && xb < p.Wd) ? (uint32_t)(xb * 8 + 4 * hf + tc * rowb) : kOutside;
+    const int hoff = Q ? 4 * hf : 0;  // Q = 0: both halves of a pixel come from the low dword of its word
+    const uint32_t offa = (xa >= 0 && xa < p.Wd) ? (uint32_t)(xa * 8 + hoff) : kOutside;
+    const uint32_t offb = (xb >= 0 && xb < p.Wd) ? (uint32_t)(xb * 8 + hoff + tc * rowb) : kOutside;
+    const int hsh = Q ? 0 : 16 * hf;  // Q = 0: the lane's 16 channel bits inside the loaded dword
     auto load_a = [&](int rr) {  // band row rr is image row rr - px
-        return (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)(offa + (uint32_t)((rr - p.px) * rowb)), 0, 0);
+        return (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)(offa + (uint32_t)((rr - p.px) * rowb)), 0, 0) >> hsh;
     };
     auto load_b = [&](int rr) {
-        return (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)(offb + (uint32_t)((rr - p.px) * rowb)), 0, 0);
+        return (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)(offb + (uint32_t)((rr - p.px) * rowb)), 0, 0) >> hsh;
     };
 
     // ---- output ----------------------------------------------------------------------------------------------------
@@ -196,12 +266,12 @@ __global__ __launch_bounds__(256) void conv_direct_fp4_kernel(const DwConv p)
                                                   hh * ww * p.Ow * 8, 0x00020000);
         ooff = olive ? (uint32_t)(((xx0 + lane) * p.Ow + cg) * 8) : 0xC0000000u;
     }
-    auto finish_row = [&](dw_v4f (&af)[NT], int y, int par) {
+    auto finish_row = [&](acc_t (&af)[NT], int y, int par) {
         if (MODE == 4) {
 #pragma unroll
             for (int nt = 0; nt < NT; nt++)
-                csum[nt] += (int)((cmask[0] ? af[nt][0] : 0.f) + (cmask[1] ? af[nt][1] : 0.f) +
-                                  (cmask[2] ? af[nt][2] : 0.f) + (cmask[3] ? af[nt][3] : 0.f));  // exact: below 2^13
+                csum[nt] += (int)((cmask[0] ? af[nt][0] : 0) + (cmask[1] ? af[nt][1] : 0) + (cmask[2] ? af[nt][2] : 0) +
+                                  (cmask[3] ? af[nt][3] : 0));  // Q = 1: float sums, exact: below 2^13
             return;
         }
         int a[NT][4];
@@ -209,7 +279,7 @@ __global__ __launch_bounds__(256) void conv_direct_fp4_kernel(const DwConv p)
         for (int nt = 0; nt < NT; nt++)
 #pragma unroll
             for (int r = 0; r < 4; r++) {
-                const float f = af[nt][r];  // a copy first: the cast below wants an object, not a vector element
+                const auto f = af[nt][r];  // a copy first: the cast below wants an object, not a vector element
                 a[nt][r] = __builtin_bit_cast(int, f);
             }
         int wlo = 0, whi = 0;
@@ -268,9 +338,10 @@ __global__ __launch_bounds__(256) void conv_direct_fp4_kernel(const DwConv p)
     // ---- walk down the strip: band row rr feeds output rows rr (filter row 0), rr-1 (1) and rr-2 (2) ---------------
     // a0 holds the partial sums of output row rr-2, a1 those of row rr-1; band row rr completes row rr-2 (emitted),
     // continues row rr-1 and opens row rr with a zero C operand.
-    dw_v4f a0[NT], a1[NT];
-    const float kb = (float)(p.K + 1);
-    const dw_v4f zero = {kb, kb, kb, kb};  // the C operand that opens an output row: the bias described above
+    acc_t a0[NT], a1[NT];
+    typedef decltype(a0[0][0] + a0[0][0]) acc_s;
+    const acc_s kb = Q ? (acc_s)(p.K + 1) : (acc_s)0;
+    const acc_t zero = {kb, kb, kb, kb};  // the C operand that opens an output row: Q = 1: the bias described above
 #pragma unroll
     for (int nt = 0; nt < NT; nt++) a0[nt] = a1[nt] = zero;
     uint32_t ra0 = load_a(ys), rb0 = load_b(ys), ra1 = load_a(ys + 1), rb1 = load_b(ys + 1);
@@ -293,7 +364,7 @@ __global__ __launch_bounds__(256) void conv_direct_fp4_kernel(const DwConv p)
         const dw_v4i A0 = expand32(XA), A1 = expand32(XB);              \
         XA = load_a(rr_ + 4);                                           \
         XB = load_b(rr_ + 4);                                           \
-        dw_v4f done[NT];                                                \
+        acc_t done[NT];                                                 \
         if (rr_ - 2 >= ys) { NB_DW_PART_C(done, A0, A1) }               \
         if (rr_ - 1 >= ys && rr_ - 1 < ye) { NB_DW_PART_M(A0) }         \
         if (rr_ < ye) { NB_DW_PART_F(A0, A1) }                          \
@@ -306,72 +377,73 @@ __global__ __launch_bounds__(256) void conv_direct_fp4_kernel(const DwConv p)
             if (rr + 3 < ye + 2) NB_DW_ANY(rr + 3, ra3, rb3, 1)
         }
 #undef NB_DW_ANY
-        return;
-    }
-    // The steady rows carry no conditions and always issue the same loads, so that the wait for a row's words is a
-    // wait for exactly the loads issued before them (four rows ahead).  The fragments of the next row are looked up
-    // while the current row is multiplied: two fragment sets, P and Q, used in turn.
-    int rr = ys + 2;
-    dw_v4i P0 = expand32(ra0), P1 = expand32(rb0), Q0, Q1;
-    {
-        Q0 = expand32(ra1), Q1 = expand32(rb1);
-        ra0 = load_a(ys + 4);
-        rb0 = load_b(ys + 4);
-        NB_DW_PART_F(P0, P1)
-        P0 = expand32(ra2), P1 = expand32(rb2);
-        ra1 = load_a(ys + 5);
-        rb1 = load_b(ys + 5);
-        NB_DW_PART_M(Q0)
-        NB_DW_PART_F(Q0, Q1)
-    }
-    // C0, C1: the current row's fragments; N0, N1: set for the next row, whose words are XNA, XNB; XCA, XCB: the ring
-    // slot of the current row, free since its words were looked up a step ago
+    } else {
+        // The steady rows carry no conditions and always issue the same loads, so that the wait for a row's words is a
+        // wait for exactly the loads issued before them (four rows ahead).  The fragments of the next row are looked up
+        // while the current row is multiplied: two fragment sets, P and Q, used in turn.
+        int rr = ys + 2;
+        dw_v4i P0 = expand32(ra0), P1 = expand32(rb0), Q0, Q1;
+        {
+            Q0 = expand32(ra1), Q1 = expand32(rb1);
+            ra0 = load_a(ys + 4);
+            rb0 = load_b(ys + 4);
+            NB_DW_PART_F(P0, P1)
+            P0 = expand32(ra2), P1 = expand32(rb2);
+            ra1 = load_a(ys + 5);
+            rb1 = load_b(ys + 5);
+            NB_DW_PART_M(Q0)
+            NB_DW_PART_F(Q0, Q1)
+        }
+        // C0, C1: the current row's fragments; N0, N1: set for the next row, whose words are XNA, XNB; XCA, XCB: the ring
+        // slot of the current row, free since its words were looked up a step ago
 #define NB_DW_ROW(C0, C1, N0, N1, XNA, XNB, XCA, XCB, PAR)     \
     {                                                          \
         N0 = expand32(XNA), N1 = expand32(XNB);                \
         XCA = load_a(rr + 4);                                  \
         XCB = load_b(rr + 4);                                  \
-        dw_v4f done[NT];                                       \
+        acc_t done[NT];                                        \
         NB_DW_PART_C(done, C0, C1)                             \
         NB_DW_PART_M(C0)                                       \
         NB_DW_PART_F(C0, C1)                                   \
         finish_row(done, rr - 2, PAR);                         \
         rr++;                                                  \
     }
-    // sub-bands start on even rows, so the parity of a finished row is known where the loop is unrolled
-    const int nsteady = ye - ys - 2, rem = nsteady & 3;
-    for (int q = nsteady >> 2; q > 0; q--) {
-        NB_DW_ROW(P0, P1, Q0, Q1, ra3, rb3, ra2, rb2, 0)
-        NB_DW_ROW(Q0, Q1, P0, P1, ra0, rb0, ra3, rb3, 1)
-        NB_DW_ROW(P0, P1, Q0, Q1, ra1, rb1, ra0, rb0, 0)
-        NB_DW_ROW(Q0, Q1, P0, P1, ra2, rb2, ra1, rb1, 1)
-    }
-    if (rem >= 1) NB_DW_ROW(P0, P1, Q0, Q1, ra3, rb3, ra2, rb2, 0)
-    if (rem >= 2) NB_DW_ROW(Q0, Q1, P0, P1, ra0, rb0, ra3, rb3, 1)
-    if (rem >= 3) NB_DW_ROW(P0, P1, Q0, Q1, ra1, rb1, ra0, rb0, 0)
+        // sub-bands start on even rows, so the parity of a finished row is known where the loop is unrolled
+        const int nsteady = ye - ys - 2, rem = nsteady & 3;
+        for (int q = nsteady >> 2; q > 0; q--) {
+            NB_DW_ROW(P0, P1, Q0, Q1, ra3, rb3, ra2, rb2, 0)
+            NB_DW_ROW(Q0, Q1, P0, P1, ra0, rb0, ra3, rb3, 1)
+            NB_DW_ROW(P0, P1, Q0, Q1, ra1, rb1, ra0, rb0, 0)
+            NB_DW_ROW(Q0, Q1, P0, P1, ra2, rb2, ra1, rb1, 1)
+        }
+        if (rem >= 1) NB_DW_ROW(P0, P1, Q0, Q1, ra3, rb3, ra2, rb2, 0)
+        if (rem >= 2) NB_DW_ROW(Q0, Q1, P0, P1, ra0, rb0, ra3, rb3, 1)
+        if (rem >= 3) NB_DW_ROW(P0, P1, Q0, Q1, ra1, rb1, ra0, rb0, 0)
 #undef NB_DW_ROW
-    // band rows ye and ye + 1 finish the last two output rows: row ye's fragments are in the current set, row
-    // ye + 1's words in the ring slot behind it
-    {
-        if (rem & 1) P0 = Q0, P1 = Q1;
-        const uint32_t ua = rem == 0 ? ra3 : rem == 1 ? ra0 : rem == 2 ? ra1 : ra2;
-        const uint32_t ub = rem == 0 ? rb3 : rem == 1 ? rb0 : rem == 2 ? rb1 : rb2;
-        Q0 = expand32(ua), Q1 = expand32(ub);
-        dw_v4f done[NT];
-        NB_DW_PART_C(done, P0, P1)
-        NB_DW_PART_M(P0)
-        finish_row(done, ye - 2, (ye - ys) & 1);
-        NB_DW_PART_C(done, Q0, Q1)
-        finish_row(done, ye - 1, (ye - 1 - ys) & 1);
+        // band rows ye and ye + 1 finish the last two output rows: row ye's fragments are in the current set, row
+        // ye + 1's words in the ring slot behind it
+        {
+            if (rem & 1) P0 = Q0, P1 = Q1;
+            const uint32_t ua = rem == 0 ? ra3 : rem == 1 ? ra0 : rem == 2 ? ra1 : ra2;
+            const uint32_t ub = rem == 0 ? rb3 : rem == 1 ? rb0 : rem == 2 ? rb1 : rb2;
+            Q0 = expand32(ua), Q1 = expand32(ub);
+            acc_t done[NT];
+            NB_DW_PART_C(done, P0, P1)
+            NB_DW_PART_M(P0)
+            finish_row(done, ye - 2, (ye - ys) & 1);
+            NB_DW_PART_C(done, Q0, Q1)
+            finish_row(done, ye - 1, (ye - 1 - ys) & 1);
+        }
     }
 #undef NB_DW_PART_C
 #undef NB_DW_PART_M
 #undef NB_DW_PART_F
 #undef NB_DW_MM
     if (MODE == 4) {
-        // popcount = (2K + 1 - biased dot) / 2 per pixel: add the four lane groups, then one atomic per channel
+        // popcount = (K - dot) / 2 per pixel (Q = 1: the sums carry the bias K + 1): add the four lane groups, then
+        // one atomic per channel
         const int cols = p.w - x0 < 16 ? p.w - x0 : 16;
-        const int kn = (2 * p.K + 1) * (ye - ys) * cols;
+        const int kn = (Q ? 2 * p.K + 1 : p.K) * (ye - ys) * cols;
 #pragma unroll
         for (int nt = 0; nt < NT; nt++) {
             int v = csum[nt];
@@ -383,21 +455,24 @@ __global__ __launch_bounds__(256) void conv_direct_fp4_kernel(const DwConv p)
     }
 }
 
-// mode 2 (packed threshold bits), 3 (2x2 OR-pooled) or 4 (pixel sums into a zeroed array), one channel word per
-// pixel, filter [D, 9, O].  false = not this shape, nothing launched.
-bool conv_direct_fp4_try(void *out, const uint64_t *in, const uint64_t *filt, const int32_t *thresh, const ConvGeom &g,
-                         int64_t D, int O, int tap_bits, int mode, hipStream_t s)
+// mode 2 (packed threshold bits), 3 (2x2 OR-pooled) or 4 (pixel sums into a zeroed array).  tap_bits == 0: one full
+// channel word per pixel, filter [D, 9, O], FP4 (returns 4; only with allow_fp4); tap_bits in 17..32: tap-packed filter,
+// +-1 bytes (returns 2).  0 = not this shape, nothing launched.
+int conv_direct_fp4_try(void *out, const uint64_t *in, const uint64_t *filt, const int32_t *thresh, const ConvGeom &g,
+                        int64_t D, int O, int tap_bits, int mode, bool allow_fp4, hipStream_t s)
 {
-    if (mode != 2 && mode != 3 && mode != 4) return false;
+    if (mode != 2 && mode != 3 && mode != 4) return 0;
+    const int q = tap_bits == 0 ? 1 : 0;
+    if (q ? !allow_fp4 : (tap_bits < 17 || tap_bits > 32)) return 0;
     // 32-bit byte offsets inside one member's output, below 2^30 for the out-of-range marker of the stores
-    if ((mode == 2 || mode == 3) && (int64_t)g.h * g.w * ((O + 63) / 64) * 8 >= (1LL << 30)) return false;
-    if (tap_bits != 0 || g.Cw != 1) return false;
-    if (g.sx != 1 || g.sy != 1 || g.fx != 3 || g.fy != 3) return false;
-    if (D < 1 || g.h < 1 || g.w < 1) return false;
-    if (!(O == 16 || O == 32 || (O >= 64 && O % 16 == 0))) return false;
-    if (mode == 3 && (g.h < 2 || g.w < 2)) return false;
+    if ((mode == 2 || mode == 3) && (int64_t)g.h * g.w * ((O + 63) / 64) * 8 >= (1LL << 30)) return 0;
+    if (g.Cw != 1) return 0;
+    if (g.sx != 1 || g.sy != 1 || g.fx != 3 || g.fy != 3) return 0;
+    if (D < 1 || g.h < 1 || g.w < 1) return 0;
+    if (!(O == 16 || O == 32 || (O >= 64 && O % 16 == 0))) return 0;
+    if (mode == 3 && (g.h < 2 || g.w < 2)) return 0;
     // 32-bit byte offsets inside one member's image, far enough below 2^30 for the out-of-range marker
-    if ((int64_t)(g.H + g.px + 8) * g.Wd * 8 >= (1LL << 29) || (int64_t)9 * O * 8 >= (1LL << 31)) return false;
+    if ((int64_t)(g.H + g.px + 8) * g.Wd * 8 >= (1LL << 29) || (int64_t)9 * O * 8 >= (1LL << 31)) return 0;
     // 64 channels per wave from 64 channels on (32 per wave, with twice the waves per SIMD, measured 5-8 % slower)
     const int NT = O >= 64 ? 4 : O / 16;
     DwConv p;
@@ -408,7 +483,11 @@ bool conv_direct_fp4_try(void *out, const uint64_t *in, const uint64_t *filt, co
     p.H = g.H; p.Wd = g.Wd; p.px = g.px; p.py = g.py; p.h = g.h; p.w = g.w;
     p.O = O;
     p.Ow = (O + 63) / 64;
-    p.K = 9 * 64;
+    p.K = q ? 9 * 64 : 9 * tap_bits;
+    p.in_bits = q ? 64 : tap_bits;
+    p.tapT = q ? 1 : 64 / tap_bits;
+    p.tapM = 65536 / p.tapT + 1;  // (tap * tapM) >> 16 = tap / tapT for the nine taps
+    p.fwords = (9 + p.tapT - 1) / p.tapT * O;
     p.ntx = (g.w + 15) / 16;
     p.ncg = p.Ow;  // groups cover whole output words (dead channels give zero bits)
     // Sub-bands as tall as the population allows: whole images once that gives every SIMD a few waves, else down
@@ -422,26 +501,29 @@ bool conv_direct_fp4_try(void *out, const uint64_t *in, const uint64_t *filt, co
     }
     p.nsb = (g.h + p.hb - 1) / p.hb;
     const int64_t units = D * p.nsb * p.ncg * p.ntx;
-    if (units >= (1LL << 31)) return false;
+    if (units >= (1LL << 31)) return 0;
     p.units = (uint32_t)units;
     p.mntx = (uint32_t)((1ULL << 32) / (uint32_t)p.ntx);  // unused for a divisor of 1
     p.mncg = (uint32_t)((1ULL << 32) / (uint32_t)p.ncg);
     p.mnsb = (uint32_t)((1ULL << 32) / (uint32_t)p.nsb);
     const dim3 grid((unsigned)ceil_div(units, 4)), block(256);
-#define NB_DW_LAUNCH(nt)                                                       \
-    if (NT == nt) {                                                            \
+#define NB_DW_LAUNCH(nt, qq)                                                   \
+    if (NT == nt && q == qq) {                                                 \
         if (mode == 2)                                                         \
-            conv_direct_fp4_kernel<nt, 2><<<grid, block, 0, s>>>(p);           \
+            conv_direct_fp4_kernel<nt, 2, qq><<<grid, block, 0, s>>>(p);       \
         else if (mode == 3)                                                    \
-            conv_direct_fp4_kernel<nt, 3><<<grid, block, 0, s>>>(p);           \
+            conv_direct_fp4_kernel<nt, 3, qq><<<grid, block, 0, s>>>(p);       \
         else                                                                   \
-            conv_direct_fp4_kernel<nt, 4><<<grid, block, 0, s>>>(p);           \
+            conv_direct_fp4_kernel<nt, 4, qq><<<grid, block, 0, s>>>(p);       \
     }
-    NB_DW_LAUNCH(1)
-    NB_DW_LAUNCH(2)
-    NB_DW_LAUNCH(4)
+    NB_DW_LAUNCH(1, 1)
+    NB_DW_LAUNCH(2, 1)
+    NB_DW_LAUNCH(4, 1)
+    NB_DW_LAUNCH(1, 0)
+    NB_DW_LAUNCH(2, 0)
+    NB_DW_LAUNCH(4, 0)
 #undef NB_DW_LAUNCH
-    return true;
+    return q ? 4 : 2;
 }
 
 }  // namespace nb

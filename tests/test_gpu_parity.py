@@ -646,6 +646,74 @@ def test_conv_narrow_matrix_core_kernel_vs_oracle(ops, oracle, C, O, fy, px, py,
         ops.conv_engine(prev)
 
 
+# The strip kernels for one word per pixel: tap-packed layers of 17 to 32 channels (+-1 bytes; every taps-per-word
+# count and channel counts that leave dead byte positions in the upper half) and full channel words (FP4), with 16,
+# 32, 64 and more output channels, images of one to three rows (the short sub-band path), every remainder of the
+# four-row loop, ragged strips, unequal paddings, and a population large enough for whole-image sub-bands.
+WIDE_STRIP_CASES = [
+    (17, 16, 1, 1, 19, 18, 3),
+    (21, 32, 1, 1, 20, 33, 2),
+    (22, 64, 1, 1, 21, 20, 2),
+    (24, 64, 1, 1, 32, 32, 3),
+    (31, 128, 0, 1, 22, 17, 2),
+    (32, 80, 1, 0, 35, 40, 2),
+    (29, 64, 2, 2, 9, 9, 4),
+    (24, 64, 1, 1, 1, 16, 5),
+    (32, 16, 1, 1, 2, 5, 5),
+    (20, 32, 1, 1, 3, 40, 3),
+    (27, 64, 1, 1, 67, 31, 1),
+    (24, 64, 1, 1, 12, 12, 300),
+    (33, 64, 1, 1, 21, 20, 2),
+    (64, 32, 1, 2, 38, 31, 2),
+    (50, 16, 2, 1, 3, 40, 3),
+    (64, 64, 1, 1, 2, 20, 3),                  # the short path of the FP4 flavour
+    (64, 16, 1, 1, 129, 5, 1),                 # eight sub-bands of 18 rows, the last one 3 rows: short path after others
+    (24, 16, 1, 1, 129, 7, 1),
+]
+
+
+@pytest.mark.parametrize("C,O,px,py,H,W,D", WIDE_STRIP_CASES)
+def test_conv_wide_strip_kernels_vs_oracle(ops, oracle, C, O, px, py, H, W, D):
+    """Packed and pooled outputs and pixel sums of 3x3 layers with one word per pixel against the oracle, thresholds
+    spread around the sums (one always, one never above), on the engine that the shape should get, and identical to
+    the XOR-popcount kernels' answer."""
+    g = rng(C * 1000 + O * 10 + H + W)
+    x = oracle.pack(g.integers(0, 2, size=(D * H * W, C)).astype(bool), np.int64).reshape(D, H, W, 1)
+    fb = g.integers(0, 2, size=(D * O * 9, C)).astype(bool)
+    f = np.ascontiguousarray(oracle.pack(fb, np.int64).reshape(D, O, 3, 3, 1).transpose(0, 2, 3, 4, 1).reshape(D, -1, O))
+    K = 9 * C
+    thr = (g.integers(0, K + 3, size=(D, O)) - K // 2 + K - 1).astype(np.int32)
+    thr[0, 0], thr[0, 1] = -7, 2 * K + 5
+    geom = (3, 3, px, py, 1, 1)
+    want = oracle.conv(x, f, *geom)
+    act = oracle.conv_act(x, f, thr, *geom)
+    h, w = act.shape[1:3]
+    packed = oracle.pack(act.reshape(-1, O), np.int64).reshape(D, h, w, -1)
+    xd, fd, td = dev(x), dev(f), dev(thr)
+    kw = dict(in_bits=C) if C < 64 else {}
+    served = 2 if C <= 32 else 4
+    if C <= 32:
+        fd = ops.tap_pack_filter(fd, 9, C)
+        kw["filter_tap_packed"] = True
+    prev = ops.conv_engine(2)
+    try:
+        got = ops.conv_act_pack(xd, fd, td, *geom, **kw)
+        assert ops.conv_last_engine() == served
+        np.testing.assert_array_equal(host(got), packed)
+        if h >= 2 and w >= 2:
+            pooled = ops.conv_act_pack(xd, fd, td, *geom, pool=True, **kw)
+            assert ops.conv_last_engine() == served
+            np.testing.assert_array_equal(host(pooled), oracle.max_pool2d(packed, 2, 2, 0, 0, 2, 2))
+        sums = ops.conv_popc_sums(xd, fd, *geom, **kw)
+        assert ops.conv_last_engine() == served
+        np.testing.assert_array_equal(host(sums), want.reshape(D, -1, O).sum(axis=1))
+        ops.conv_engine(1)
+        assert torch.equal(ops.conv_act_pack(xd, fd, td, *geom, **kw), got)
+        assert ops.conv_last_engine() == 1
+    finally:
+        ops.conv_engine(prev)
+
+
 def _random_matrix_core_cases(n, seed):
     g = np.random.default_rng(seed)
     cases = []
