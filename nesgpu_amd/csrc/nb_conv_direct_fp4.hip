@@ -239,9 +239,15 @@ __global__ __launch_bounds__(256) void conv_direct_fp4_kernel(const DwConv p)
 #pragma unroll
     for (int nt = 0; nt < NT; nt++) pend[nt][0] = pend[nt][1] = 0;
     // 16-bit field gq (0..3) of ballot a in the low half, that of ballot b in the high half: scalar pack instructions
-    auto fields = [](uint64_t a, uint64_t b, int gq) {
+    auto fields = [](uint64_t a, uint64_t b, int gq, bool both) {
         const uint32_t x = gq < 2 ? (uint32_t)a : (uint32_t)(a >> 32), y = gq < 2 ? (uint32_t)b : (uint32_t)(b >> 32);
-        return (gq & 1) ? (x >> 16) | (y & 0xFFFF0000u) : (x & 0xFFFFu) | (y << 16);
+        if (!both) return (gq & 1) ? x >> 16 : x & 0xFFFFu;  // b is a constant zero
+        uint32_t r;  // one instruction; the compiler spells the same thing out as a shift, an and and an or
+        if (gq & 1)
+            asm("s_pack_hh_b32_b16 %0, %1, %2" : "=s"(r) : "s"(x), "s"(y));
+        else
+            asm("s_pack_ll_b32_b16 %0, %1, %2" : "=s"(r) : "s"(x), "s"(y));
+        return r;
     };
     // A finished row's comparison results are ballots (scalar registers): bit 16*g + li of the ballot of accumulator
     // register r is (pixel 4*g + r, channel li of the tile).  The output word of a pixel is put together from 16-bit
@@ -294,8 +300,8 @@ __global__ __launch_bounds__(256) void conv_direct_fp4_kernel(const DwConv p)
             for (int g = 0; g < 4; g++)
 #pragma unroll
                 for (int r = 0; r < 4; r++) {
-                    NB_DW_WRITELANE(wlo, fields(m[0][r], m[1][r], g), 4 * g + r);
-                    if (NT > 2) NB_DW_WRITELANE(whi, fields(m[2][r], m[3][r], g), 4 * g + r);
+                    NB_DW_WRITELANE(wlo, fields(m[0][r], m[1][r], g, NT > 1), 4 * g + r);
+                    if (NT > 2) NB_DW_WRITELANE(whi, fields(m[2][r], m[3][r], g, NT > 3), 4 * g + r);
                 }
         } else {
             // pixels 4g, 4g+1 and 4g+2, 4g+3 pool in x; rows y (even) and y+1 pool in y
@@ -326,8 +332,8 @@ __global__ __launch_bounds__(256) void conv_direct_fp4_kernel(const DwConv p)
             for (int g = 0; g < 4; g++)
 #pragma unroll
                 for (int q = 0; q < 2; q++) {
-                    NB_DW_WRITELANE(wlo, fields(m[0][q], m[1][q], g), 2 * g + q);
-                    if (NT > 2) NB_DW_WRITELANE(whi, fields(m[2][q], m[3][q], g), 2 * g + q);
+                    NB_DW_WRITELANE(wlo, fields(m[0][q], m[1][q], g, NT > 1), 2 * g + q);
+                    if (NT > 2) NB_DW_WRITELANE(whi, fields(m[2][q], m[3][q], g, NT > 3), 2 * g + q);
                 }
         }
         typedef int dw_v2i __attribute__((ext_vector_type(2)));
