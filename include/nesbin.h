@@ -244,13 +244,14 @@ int nb_conv_popc_sums_i32(int32_t *sums, const int32_t *in, const int32_t *filt,
  * outputs and pixel sums of 3x3 windows over one word per pixel have another (tap-packed filters of 17 to 32
  * channels as +-1 bytes; full channel words as FP4 codes, engines 0 and 2).
  * 0 = automatic: the matrix-core kernels for populations of 128 members or more (the narrow one always), else
- * XOR-popcount;
+ * XOR-popcount; nb_conv_popc_sums_i64 of a stride-1 layer with filters of at most 5 x 5 runs no conv at all then: it
+ * counts the image's bits per tap and finishes with one small dot product per output channel (same integers);
  * 1 = XOR-popcount only; 2 = matrix cores wherever a kernel covers the shape; 3 = as 2, +-1 bytes only.  Returns
  * the previous setting; any other argument only queries.  Initial value from the environment variable
  * NESBIN_CONV_ENGINE: first letter 'v' -> 1, 'm' -> 2, 'i' -> 3, else 0.  No counterpart in the reference. */
 int nb_conv_engine(int engine);
 /* Engine that served the calling thread's latest conv / conv_act / conv_act_pack launch: 1 = XOR-popcount,
- * 2 = matrix cores on +-1 bytes, 4 = matrix cores on FP4 codes, 0 = none yet.  For tests and tuning.  No
+ * 2 = matrix cores on +-1 bytes, 4 = matrix cores on FP4 codes, 5 = pixel sums from bit counts, 0 = none yet.  For tests and tuning.  No
  * counterpart in the reference. */
 int nb_conv_last_engine(void);
 /* tap_pack_filter: filt [D, taps, O] (one word per tap, Cw == 1) -> out [D, ceil(taps/T), O], T = bits/tap_bits,

@@ -200,7 +200,8 @@ static std::atomic<int> &conv_engine_cell()
     return cell;
 }
 static int conv_engine() { return conv_engine_cell().load(std::memory_order_relaxed); }
-// engine of this thread's latest conv launch: 1 XOR-popcount, 2 matrix cores on +-1 bytes, 4 matrix cores on FP4 codes
+// engine of this thread's latest conv launch: 1 XOR-popcount, 2 matrix cores on +-1 bytes, 4 matrix cores on FP4 codes,
+// 5 pixel sums from bit counts (no conv)
 static thread_local int t_last_engine = 0;
 int set_conv_engine(int e)
 {
@@ -263,6 +264,14 @@ int conv_impl(void *out, const W *in, const W *filt, const int32_t *thresh, int6
     const int engine = conv_engine();
     if (mode == 4) {
         NB_REQUIRE(hw * (int64_t)fx * fy * Cw * bits < (1LL << 31), "%s: a member's pixel sum may overflow int32", who);
+        // Automatic choice: the sums over the pixels need no conv at all (counts of the image's bits per tap, then one
+        // small dot product per output channel); a pinned engine still runs its conv kernels.
+        if (bits == 64 && engine == 0 && Cw > 0 &&
+            conv_sums_count_try(static_cast<int32_t *>(out), reinterpret_cast<const uint64_t *>(in),
+                                reinterpret_cast<const uint64_t *>(filt), g, D, N, tap_bits, s)) {
+            t_last_engine = 5;
+            return check_launch(who);
+        }
         zero_i32_kernel<<<dim3(grid_for(D * O)), dim3(256), 0, s>>>(static_cast<int32_t *>(out), D * O);
     }
     // Automatic choice, measured on MI355X: one workgroup per CU walks whole members, so the matrix-core kernel needs

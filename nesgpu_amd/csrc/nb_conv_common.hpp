@@ -94,6 +94,11 @@ bool conv_direct_try(void *out, const uint64_t *in, const uint64_t *filt, const 
 int conv_direct_fp4_try(void *out, const uint64_t *in, const uint64_t *filt, const int32_t *thresh, const ConvGeom &g,
                         int64_t D, int O, int tap_bits, int mode, bool allow_fp4, hipStream_t s);
 
+// Pixel sums (mode 4) from counts of the image's bits per tap, without a conv (nb_conv_sums.hip): 64-bit words, stride
+// 1, filters of at most 5 x 5; tap_bits > 0: tap-packed filter.  false = not this shape, nothing launched.
+bool conv_sums_count_try(int32_t *out, const uint64_t *in, const uint64_t *filt, const ConvGeom &g, int64_t D, int O,
+                         int tap_bits, hipStream_t s);
+
 inline int taps_per_word(int bits, int tap_bits) { return bits / tap_bits; }
 
 }  // namespace nb

@@ -258,7 +258,7 @@ def conv_engine(engine=None):
 
 def conv_last_engine():
     """Engine that served this thread's latest conv launch: 1 = XOR-popcount, 2 = matrix cores on +-1 bytes (int8
-    MFMA), 4 = matrix cores on FP4 codes, 0 = none yet."""
+    MFMA), 4 = matrix cores on FP4 codes, 5 = pixel sums from counts of the image's bits (no conv), 0 = none yet."""
     return _lib.load().nb_conv_last_engine()
 
 
@@ -329,7 +329,9 @@ def conv_popc_sums(input, filter, filterx, filtery, padx, pady, stridex, stridey
                    filter_tap_packed=False):
     """conv(...).sum over the output pixels -> int32 [D, O], without the [D,h,w,O] maps reaching memory (not in the
     reference; it is the statistic behind the per-member mean of BinarizedConv2d(batch_norm=True),
-    modules/binary.py:147-155)."""
+    modules/binary.py:147-155).  With the automatic engine, 64-bit words, stride 1 and filters of at most 5 x 5 no
+    conv runs at all: the sum over the pixels is taken first (counts of the image's bits per tap), then one small dot
+    product per output channel; the same integers."""
     suf, _, filter, tap = _conv_args(input, filter, filterx, filtery, in_bits, filter_tap_packed)
     out = torch.empty((input.size(0), filter.size(2)), dtype=torch.int32, device=input.device)
     with _on(input):

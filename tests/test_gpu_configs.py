@@ -170,15 +170,17 @@ def test_config5_cifar_net(wk, ops, oracle):
         xin = torch.randint(-2 ** 62, 2 ** 62, (D, S, S, 1), dtype=torch.int64, device="cuda", generator=g5)
         thr = (576 + torch.randint(-40, 41, (D, O), device="cuda", generator=g5)).to(torch.int32)
         got, sums = {}, {}
-        for eng, served in ((0, 4), (3, 2), (1, 1)):
+        # (engine asked for, engine that serves the packed map, engine that serves the pixel sums: the automatic choice
+        # takes those from bit counts, without a conv)
+        for eng, served, served_sums in ((0, 4, 5), (2, 4, 4), (3, 2, 2), (1, 1, 1)):
             ops.conv_engine(eng)
             got[eng] = ops.conv_act_pack(xin, t[name], thr, 3, 3, 1, 1, 1, 1, pool=True)
             assert ops.conv_last_engine() == served
             sums[eng] = ops.conv_popc_sums(xin, t[name], 3, 3, 1, 1, 1, 1)
-            assert ops.conv_last_engine() == served
+            assert ops.conv_last_engine() == served_sums
         ops.conv_engine(prev)
-        assert torch.equal(got[0], got[3]) and torch.equal(got[0], got[1]), name
-        assert torch.equal(sums[0], sums[3]) and torch.equal(sums[0], sums[1]), name
+        assert torch.equal(got[0], got[3]) and torch.equal(got[0], got[1]) and torch.equal(got[0], got[2]), name
+        assert torch.equal(sums[0], sums[3]) and torch.equal(sums[0], sums[1]) and torch.equal(sums[0], sums[2]), name
         assert 0.2 < float(ops.unpack(got[0].view(-1, got[0].shape[-1])).float().mean()) < 0.8      # not degenerate
         del xin, thr, got, sums
     del l1, thr1

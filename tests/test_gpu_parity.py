@@ -964,6 +964,57 @@ def test_conv_popc_sums_vs_oracle(ops, oracle, engine, dtype, C, O, k, pad, stri
     np.testing.assert_array_equal(host(ops.conv_popc_sums(dev(x), dev(f), *geom)), want)   # zeroed again on every call
 
 
+COUNT_SUM_CASES = [
+    # C, O, fx, fy, px, py, H, W, D, tap-packed filter
+    (64, 64, 3, 3, 1, 1, 32, 32, 5, False),
+    (24, 64, 3, 3, 1, 1, 20, 33, 3, True),
+    (3, 16, 3, 3, 1, 1, 9, 9, 4, True),
+    (200, 48, 5, 5, 2, 2, 19, 20, 2, False),       # four channel words, the 5 x 5 instance
+    (64, 64, 3, 3, 0, 0, 9, 10, 5, False),         # no padding: two border rows / columns at either end
+    (70, 33, 1, 1, 0, 0, 4, 40, 2, False),         # 1 x 1: no borders at all
+    (16, 16, 3, 2, 2, 0, 7, 5, 3, True),           # unequal paddings, two filter columns
+    (64, 16, 3, 3, 1, 1, 70, 66, 2, False),        # more pixels than one LDS chunk holds
+    (128, 256, 3, 3, 1, 1, 8, 8, 3, False),
+    (64, 2100, 3, 3, 1, 1, 6, 6, 2, False),        # more channels than one LDS sum array holds
+    (8, 16, 5, 3, 2, 1, 3, 3, 2, True),            # no row that every tap sees
+    (64, 32, 3, 3, 2, 2, 5, 6, 3, False),          # padding of 2 with a 3 x 3 filter: output larger than the image
+    (33, 16, 2, 4, 0, 1, 12, 9, 2, False),
+]
+
+
+@pytest.mark.parametrize("C,O,fx,fy,px,py,H,W,D,tap", COUNT_SUM_CASES)
+def test_conv_popc_sums_from_bit_counts(ops, oracle, C, O, fx, fy, px, py, H, W, D, tap):
+    """The automatic engine takes the pixel sums of stride-1 layers from counts of the image's bits per tap (no conv):
+    against the oracle's conv summed in numpy, and identical to the conv kernels' sums."""
+    g = rng(C * 100 + O + fx + fy + H + W)
+    Cw = (C + 63) // 64
+    x = oracle.pack(g.integers(0, 2, size=(D * H * W, C)).astype(bool), np.int64).reshape(D, H, W, Cw)
+    fb = g.integers(0, 2, size=(D * O * fx * fy, C)).astype(bool)
+    f = np.ascontiguousarray(oracle.pack(fb, np.int64).reshape(D, O, fx, fy, Cw).transpose(0, 2, 3, 4, 1)
+                             .reshape(D, -1, O))
+    geom = (fx, fy, px, py, 1, 1)
+    want = oracle.conv(x, f, *geom).sum(axis=(1, 2), dtype=np.int64).astype(np.int32)
+    xd, fd = dev(x), dev(f)
+    kw = {}
+    if tap:
+        fd = ops.tap_pack_filter(fd, fx * fy, C)
+        kw = dict(in_bits=C, filter_tap_packed=True)
+    prev = ops.conv_engine(0)
+    try:
+        got = ops.conv_popc_sums(xd, fd, *geom, **kw)
+        assert ops.conv_last_engine() == 5
+        np.testing.assert_array_equal(host(got), want)
+        ops.conv_engine(1)
+        assert torch.equal(ops.conv_popc_sums(xd, fd, *geom, **kw), got)
+        assert ops.conv_last_engine() == 1
+        ops.conv_engine(0)
+        strided = ops.conv_popc_sums(xd, fd, fx, fy, px, py, 2, 1, **kw)       # a stride: the conv kernels' business
+        assert ops.conv_last_engine() != 5
+        np.testing.assert_array_equal(host(strided), oracle.conv(x, f, fx, fy, px, py, 2, 1).sum(axis=(1, 2)))
+    finally:
+        ops.conv_engine(prev)
+
+
 def test_conv_engine_selector_round_trip(ops):
     prev = ops.conv_engine()
     assert prev in (0, 1, 2, 3)
