@@ -119,6 +119,18 @@ int nb_bmv_bn_act_static_i64(void *out, const int64_t *A, const int64_t *x, cons
  * Replaces a dozen elementwise tensor operations of the layer; no single counterpart in the reference. */
 int nb_conv_bn_thresholds(int32_t *thresh, const int32_t *sums, const uint16_t *bias, const uint16_t *bias_noise,
                           int64_t D, int64_t O, int64_t K, int64_t HW, nb_stream_t stream);
+/* The same thresholds straight from the layer's input: nb_conv_popc_sums_* and nb_conv_bn_thresholds in one call, without
+ * a sums array (arguments as nb_conv_popc_sums_*, K = channels x taps, at least one output pixel).  Where the sums
+ * come from bit counts (see the engine selector below) it is a single kernel; else the sums are written into thresh
+ * and turned into thresholds in place. */
+int nb_conv_bn_thresholds_from_input_i64(int32_t *thresh, const int64_t *in, const int64_t *filt, const uint16_t *bias,
+                                         const uint16_t *bias_noise, int64_t D, int64_t H, int64_t W, int64_t Cw,
+                                         int64_t O, int fx, int fy, int px, int py, int sx, int sy, int tap_bits,
+                                         int64_t K, nb_stream_t stream);
+int nb_conv_bn_thresholds_from_input_i32(int32_t *thresh, const int32_t *in, const int32_t *filt, const uint16_t *bias,
+                                         const uint16_t *bias_noise, int64_t D, int64_t H, int64_t W, int64_t Cw,
+                                         int64_t O, int fx, int fy, int px, int py, int sx, int sy, int tap_bits,
+                                         int64_t K, nb_stream_t stream);
 
 /* ---- sparse form of a population's linear layer: shared base + per-member flip lists ------------------------
  * For per-member weights W[d] = base ^ flips[d] with few flips per row (BASELINE's "base XOR Bernoulli(p) flip mask"),

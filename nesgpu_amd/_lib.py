@@ -28,6 +28,8 @@ _SUFFIXED = {
     "nb_im2col": [_PTR, _PTR, _I64, _I64, _I64, _I64] + _GEOM + [_PTR],
     "nb_conv": [_PTR, _PTR, _PTR, _I64, _I64, _I64, _I64, _I64] + _GEOM + [_I32, _PTR],
     "nb_conv_popc_sums": [_PTR, _PTR, _PTR, _I64, _I64, _I64, _I64, _I64] + _GEOM + [_I32, _PTR],
+    "nb_conv_bn_thresholds_from_input": [_PTR, _PTR, _PTR, _PTR, _PTR, _I64, _I64, _I64, _I64, _I64] + _GEOM
+                                        + [_I32, _I64, _PTR],
     "nb_conv_act": [_PTR, _PTR, _PTR, _PTR, _I64, _I64, _I64, _I64, _I64] + _GEOM + [_I32, _PTR],
     "nb_conv_act_pack": [_PTR, _PTR, _PTR, _PTR, _I64, _I64, _I64, _I64, _I64] + _GEOM + [_I32, _I32, _PTR],
     "nb_tap_pack_filter": [_PTR, _PTR, _I64, _I64, _I64, _I32, _PTR],

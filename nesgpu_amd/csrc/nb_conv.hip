@@ -222,7 +222,8 @@ __global__ __launch_bounds__(256) void zero_i32_kernel(int32_t *__restrict__ out
 template <typename W>
 int conv_impl(void *out, const W *in, const W *filt, const int32_t *thresh, int64_t D, int64_t H, int64_t Wd,
               int64_t Cw, int64_t O, int fx, int fy, int px, int py, int sx, int sy, int mode, int tap_bits,
-              nb_stream_t stream, const char *who)
+              nb_stream_t stream, const char *who, const _Float16 *bn_bias = nullptr, const _Float16 *bn_noise = nullptr,
+              int64_t bn_K = 0)
 {
     constexpr int bits = WordTraits<W>::bits;
     ConvGeom g;
@@ -268,7 +269,7 @@ int conv_impl(void *out, const W *in, const W *filt, const int32_t *thresh, int6
         // small dot product per output channel); a pinned engine still runs its conv kernels.
         if (bits == 64 && engine == 0 && Cw > 0 &&
             conv_sums_count_try(static_cast<int32_t *>(out), reinterpret_cast<const uint64_t *>(in),
-                                reinterpret_cast<const uint64_t *>(filt), g, D, N, tap_bits, s)) {
+                                reinterpret_cast<const uint64_t *>(filt), g, D, N, tap_bits, s, bn_bias, bn_noise, bn_K)) {
             t_last_engine = 5;
             return check_launch(who);
         }
@@ -342,6 +343,37 @@ int conv_impl(void *out, const W *in, const W *filt, const int32_t *thresh, int6
 #define W64(p) reinterpret_cast<const uint64_t *>(p)
 #define W32(p) reinterpret_cast<const uint32_t *>(p)
 
+// Thresholds of the batch-norm conv layer straight from the image: the pixel sums (mode 4, whatever kernel serves them)
+// and the threshold arithmetic; one kernel where the sums come from bit counts, else the sums land in `thresh` and
+// are turned into thresholds in place.
+template <typename W>
+static int conv_bn_thresholds_impl(int32_t *thresh, const W *in, const W *filt, const uint16_t *bias,
+                                   const uint16_t *bias_noise, int64_t D, int64_t H, int64_t Wd, int64_t Cw, int64_t O,
+                                   int fx, int fy, int px, int py, int sx, int sy, int tap_bits, int64_t K,
+                                   nb_stream_t stream, const char *who)
+{
+    nb::ConvGeom g;
+    if (int rc = nb::geom_check(&g, D, H, Wd, Cw, fx, fy, px, py, sx, sy, who)) return rc;
+    NB_REQUIRE(O >= 0 && O <= (1 << 24), "%s: bad output channel count %lld", who, (long long)O);
+    NB_REQUIRE(K >= 0 && K < (1LL << 31), "%s: bad K=%lld", who, (long long)K);
+    if (D * O == 0) return NB_OK;
+    const int64_t hw = (int64_t)g.h * g.w;
+    NB_REQUIRE(hw >= 1, "%s: no output pixels to take a mean over", who);
+    NB_REQUIRE_PTR(thresh);
+    NB_REQUIRE_PTR(bias);
+    NB_REQUIRE_PTR(bias_noise);
+    NB_REQUIRE_ALIGNED(bias, 2);
+    NB_REQUIRE_ALIGNED(bias_noise, 2);
+    const _Float16 *b = reinterpret_cast<const _Float16 *>(bias), *n = reinterpret_cast<const _Float16 *>(bias_noise);
+    nb::t_last_engine = 0;
+    if (int rc = nb::conv_impl<W>(thresh, in, filt, nullptr, D, H, Wd, Cw, O, fx, fy, px, py, sx, sy, 4, tap_bits, stream,
+                                  who, b, n, K))
+        return rc;
+    if (nb::t_last_engine == 5) return NB_OK;  // the counting kernel wrote thresholds
+    nb::bn_conv_thresh_launch(thresh, thresh, b, n, D, O, K, hw, nb::as_stream(stream));
+    return nb::check_launch(who);
+}
+
 extern "C" {
 int nb_conv_engine(int engine) { return nb::set_conv_engine(engine); }
 int nb_conv_last_engine(void) { return nb::t_last_engine; }
@@ -380,6 +412,22 @@ int nb_conv_i32(int32_t *out, const int32_t *in, const int32_t *filt, int64_t D,
 {
     return nb::conv_impl<uint32_t>(out, W32(in), W32(filt), nullptr, D, H, W, Cw, O, fx, fy, px, py, sx, sy, 0,
                                    tap_bits, s, "nb_conv_i32");
+}
+int nb_conv_bn_thresholds_from_input_i64(int32_t *thresh, const int64_t *in, const int64_t *filt, const uint16_t *bias,
+                                         const uint16_t *bias_noise, int64_t D, int64_t H, int64_t W, int64_t Cw,
+                                         int64_t O, int fx, int fy, int px, int py, int sx, int sy, int tap_bits,
+                                         int64_t K, nb_stream_t s)
+{
+    return conv_bn_thresholds_impl<uint64_t>(thresh, W64(in), W64(filt), bias, bias_noise, D, H, W, Cw, O, fx, fy, px, py,
+                                             sx, sy, tap_bits, K, s, "nb_conv_bn_thresholds_from_input_i64");
+}
+int nb_conv_bn_thresholds_from_input_i32(int32_t *thresh, const int32_t *in, const int32_t *filt, const uint16_t *bias,
+                                         const uint16_t *bias_noise, int64_t D, int64_t H, int64_t W, int64_t Cw,
+                                         int64_t O, int fx, int fy, int px, int py, int sx, int sy, int tap_bits,
+                                         int64_t K, nb_stream_t s)
+{
+    return conv_bn_thresholds_impl<uint32_t>(thresh, W32(in), W32(filt), bias, bias_noise, D, H, W, Cw, O, fx, fy, px, py,
+                                             sx, sy, tap_bits, K, s, "nb_conv_bn_thresholds_from_input_i32");
 }
 int nb_conv_popc_sums_i64(int32_t *sums, const int64_t *in, const int64_t *filt, int64_t D, int64_t H, int64_t W,
                           int64_t Cw, int64_t O, int fx, int fy, int px, int py, int sx, int sy, int tap_bits,

@@ -96,8 +96,32 @@ int conv_direct_fp4_try(void *out, const uint64_t *in, const uint64_t *filt, con
 
 // Pixel sums (mode 4) from counts of the image's bits per tap, without a conv (nb_conv_sums.hip): 64-bit words, stride
 // 1, filters of at most 5 x 5; tap_bits > 0: tap-packed filter.  false = not this shape, nothing launched.
+// With bias != nullptr the kernel writes the batch-norm layer's thresholds (bn_conv_threshold below, K channels x taps)
+// instead of the sums.
 bool conv_sums_count_try(int32_t *out, const uint64_t *in, const uint64_t *filt, const ConvGeom &g, int64_t D, int O,
-                         int tap_bits, hipStream_t s);
+                         int tap_bits, hipStream_t s, const _Float16 *bias = nullptr, const _Float16 *noise = nullptr,
+                         int64_t K = 0);
+
+// Threshold of BinarizedConv2d(batch_norm=True) for one (member, channel) from the sum of its popcount map over the HW
+// output pixels (modules/binary.py:147-155): act = 2*popc - K, mean = fp16(float(sum of act) / float(HW)),
+// thr = fp16(fp16(bias + noise) + mean); act > thr  <=>  2*popc > floor(thr) + K, which is what is returned (clamped to
+// int32; INT32_MAX, never exceeded, for NaN).
+__device__ __forceinline__ int32_t bn_conv_threshold(long long popc_sum, _Float16 bias, _Float16 noise, long long K,
+                                                     long long HW)
+{
+    const long long sum_act = 2ll * popc_sum - K * HW;
+    const _Float16 mean = (_Float16)((float)sum_act / (float)HW);
+    const _Float16 tb = bias + noise;
+    const float v = (float)(_Float16)(tb + mean);
+    if (v != v) return 2147483647;
+    long long th = (long long)floorf(fminf(fmaxf(v, -3.0e9f), 3.0e9f)) + K;
+    th = th > 2147483647ll ? 2147483647ll : (th < -2147483648ll ? -2147483648ll : th);
+    return (int32_t)th;
+}
+
+// thresh[d,o] = bn_conv_threshold(sums[d,o], ...), in place if thresh == sums (nb_linear_bn.hip)
+void bn_conv_thresh_launch(int32_t *thresh, const int32_t *sums, const _Float16 *bias, const _Float16 *noise, int64_t D,
+                           int64_t O, int64_t K, int64_t HW, hipStream_t s);
 
 inline int taps_per_word(int bits, int tap_bits) { return bits / tap_bits; }
 

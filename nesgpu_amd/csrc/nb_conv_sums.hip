@@ -38,6 +38,8 @@ struct CsConv {
     int H, Wd, Cw, h, w, fx, fy, px, py, O;
     int taps, nplanes, hw, rows_chunk, chunk_words, n1_ints, chan_chunk;
     int tap_bits, tapT, fwords;  // tap-packed filters: bits per tap, taps per word, filter words per channel
+    const _Float16 *bias, *noise;  // not null: write the batch-norm layer's thresholds instead of the sums
+    long long K;
 };
 
 // F: the largest filter extent the instance is built for (3 or kCsMaxF); the per-tap code is spelled out F x F times
@@ -249,14 +251,18 @@ __global__ __launch_bounds__(256) void conv_sums_count_kernel(const CsConv p)
             atomicAdd(&osum[oq], part - 2 * dot);
         }
         __syncthreads();
-        for (int i = threadIdx.x; i < oc; i += 256) p.out[d * p.O + o0 + i] = osum[i];
+        for (int i = threadIdx.x; i < oc; i += 256) {
+            const int64_t at = d * p.O + o0 + i;
+            p.out[at] = p.bias ? bn_conv_threshold(osum[i], p.bias[o0 + i], p.noise[at], p.K, p.hw) : osum[i];
+        }
         __syncthreads();
     }
 }
 
-// Pixel sums (mode 4 of the conv) for 64-bit words, stride 1, filters of at most 5 x 5: true = launched.
+// Pixel sums (mode 4 of the conv) for 64-bit words, stride 1, filters of at most 5 x 5: true = launched.  With bias /
+// noise the batch-norm layer's thresholds are written instead (K = channels x taps).
 bool conv_sums_count_try(int32_t *out, const uint64_t *in, const uint64_t *filt, const ConvGeom &g, int64_t D, int O,
-                         int tap_bits, hipStream_t s)
+                         int tap_bits, hipStream_t s, const _Float16 *bias, const _Float16 *noise, int64_t K)
 {
     if (g.sx != 1 || g.sy != 1 || g.fx > kCsMaxF || g.fy > kCsMaxF || g.fx < 1 || g.fy < 1) return false;
     if (g.Cw < 1 || D < 1 || O < 1 || g.h < 1 || g.w < 1 || D > kMaxGridX) return false;
@@ -267,6 +273,7 @@ bool conv_sums_count_try(int32_t *out, const uint64_t *in, const uint64_t *filt,
     if (g.Wd > kCsChunkWords) return false;  // a row of the image must fit the LDS chunk
     CsConv p;
     p.in = in; p.filt = filt; p.out = out;
+    p.bias = bias; p.noise = noise; p.K = K;
     p.H = g.H; p.Wd = g.Wd; p.Cw = g.Cw; p.h = g.h; p.w = g.w; p.fx = g.fx; p.fy = g.fy; p.px = g.px; p.py = g.py;
     p.O = O;
     p.taps = taps;

@@ -6,6 +6,7 @@
 #include <mutex>
 
 #include "nb_common.hpp"
+#include "nb_conv_common.hpp"
 
 namespace nb {
 
@@ -174,33 +175,23 @@ static int bn_static_ptr(void **ptr, const char *who)
     return NB_OK;
 }
 
-// Thresholds of BinarizedConv2d(batch_norm=True) from the pixel sums of the popcount maps (modules/binary.py:147-155):
-// act = 2*popc - K, mean[d,o] = fp16(float(sum over the HW pixels of act) / float(HW)),
-// thr = fp16(fp16(bias[o] + noise[d,o]) + mean); act > thr  <=>  2*popc > floor(thr) + K, which is what is written
-// (clamped to int32; never for NaN).  One thread per (member, channel).
-__global__ __launch_bounds__(256) void bn_conv_thresh_kernel(int32_t *__restrict__ thresh, const int32_t *__restrict__ sums,
+// Thresholds of BinarizedConv2d(batch_norm=True) from the pixel sums of the popcount maps (bn_conv_threshold in
+// nb_conv_common.hpp holds the arithmetic).  One thread per (member, channel); thresh may be sums.
+__global__ __launch_bounds__(256) void bn_conv_thresh_kernel(int32_t *thresh, const int32_t *sums,
                                                              const _Float16 *__restrict__ bias,
                                                              const _Float16 *__restrict__ noise, int64_t D, int64_t O,
                                                              int64_t K, int64_t HW)
 {
     NB_FLAT_LOOP(t, D * O)
     {
-        if (t < D * O) {
-            const int64_t o = t % O;
-            const long long sum_act = 2ll * (long long)sums[t] - (long long)K * (long long)HW;
-            const _Float16 mean = (_Float16)((float)sum_act / (float)HW);
-            const _Float16 tb = bias[o] + noise[t];
-            const float v = (float)(_Float16)(tb + mean);
-            long long th;
-            if (v != v) {
-                th = 2147483647ll;  // NaN: never above it
-            } else {
-                th = (long long)floorf(fminf(fmaxf(v, -3.0e9f), 3.0e9f)) + (long long)K;
-                th = th > 2147483647ll ? 2147483647ll : (th < -2147483648ll ? -2147483648ll : th);
-            }
-            thresh[t] = (int32_t)th;
-        }
+        if (t < D * O) thresh[t] = bn_conv_threshold(sums[t], bias[t % O], noise[t], K, HW);
     }
+}
+
+void bn_conv_thresh_launch(int32_t *thresh, const int32_t *sums, const _Float16 *bias, const _Float16 *noise, int64_t D,
+                           int64_t O, int64_t K, int64_t HW, hipStream_t s)
+{
+    bn_conv_thresh_kernel<<<dim3(grid_for(D * O)), dim3(256), 0, s>>>(thresh, sums, bias, noise, D, O, K, HW);
 }
 
 }  // namespace nb
@@ -222,9 +213,8 @@ int nb_conv_bn_thresholds(int32_t *thresh, const int32_t *sums, const uint16_t *
     NB_REQUIRE_ALIGNED(sums, 4);
     NB_REQUIRE_ALIGNED(bias, 2);
     NB_REQUIRE_ALIGNED(bias_noise, 2);
-    nb::bn_conv_thresh_kernel<<<dim3(nb::grid_for(D * O)), dim3(256), 0, nb::as_stream(stream)>>>(
-        thresh, sums, reinterpret_cast<const _Float16 *>(bias), reinterpret_cast<const _Float16 *>(bias_noise), D, O, K,
-        HW);
+    nb::bn_conv_thresh_launch(thresh, sums, reinterpret_cast<const _Float16 *>(bias),
+                              reinterpret_cast<const _Float16 *>(bias_noise), D, O, K, HW, nb::as_stream(stream));
     return nb::check_launch(who);
 }
 int64_t nb_bmv_bn_workspace_bytes(int64_t Z, int64_t M)

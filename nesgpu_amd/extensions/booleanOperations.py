@@ -23,7 +23,7 @@ __all__ = [
     "batch_im2col", "bmm", "bmm_act", "conv", "conv_act", "pack", "int8pack", "sample_bits", "weighted_sum",
     "max_pool2d", "next_pow2_clip", "ceil_div", "unpack", "thresholds_from_p", "sample_bits_from_words",
     "flip_from_words", "sample_bits_philox", "flip_philox", "seeded_bmv_from_words", "seeded_bmv_philox",
-    "philox_words", "conv_act_pack", "conv_popc_sums", "tap_pack_filter", "tap_packing_applies", "conv_engine", "conv_last_engine",
+    "philox_words", "conv_act_pack", "conv_popc_sums", "conv_bn_thresholds_from_input", "tap_pack_filter", "tap_packing_applies", "conv_engine", "conv_last_engine",
     "bmv_act_pack", "bmv_bn_act", "ExpandedRows", "expand_rows", "bmm_nt", "FlipRows", "flip_rows_from_weights",
     "bmv_flip", "bmv_flip_act_pack", "skip_table", "flip_rows_skip", "flip_rows_to_weights",
 ]
@@ -245,6 +245,31 @@ def conv_bn_thresholds(sums, bias, bias_noise, in_bits, pixels):
     with _on(sums):
         _lib.call("nb_conv_bn_thresholds", out.data_ptr(), sums.data_ptr(), bias.data_ptr(), bias_noise.data_ptr(), D, O,
                   int(in_bits), int(pixels), _stream(sums))
+    return out
+
+
+def conv_bn_thresholds_from_input(input, filter, bias, bias_noise, filterx, filtery, padx, pady, stridex, stridey,
+                                  in_bits=None, filter_tap_packed=False, channels=None):
+    """``conv_bn_thresholds(conv_popc_sums(input, filter, ...), bias, bias_noise, channels * taps, h * w)`` in one call
+    (one kernel where the pixel sums come from bit counts).  ``channels``: the layer's true input channels (default
+    ``in_bits``, else every bit of the channel words)."""
+    suf, _, filter, tap = _conv_args(input, filter, filterx, filtery, in_bits, filter_tap_packed)
+    _check(bias, "bias")
+    _check(bias_noise, "bias_noise")
+    _same_device(input, bias)
+    _same_device(input, bias_noise)
+    D, O = input.size(0), filter.size(2)
+    assert bias.dtype == torch.float16 and tuple(bias.shape) == (O,)
+    assert bias_noise.dtype == torch.float16 and tuple(bias_noise.shape) == (D, O)
+    if channels is None:
+        channels = in_bits if in_bits is not None else input.size(3) * torch.iinfo(input.dtype).bits
+    h, w = _out_hw(input, filterx, filtery, padx, pady, stridex, stridey)
+    assert h * w >= 1
+    out = torch.empty((D, O), dtype=torch.int32, device=input.device)
+    with _on(input):
+        _lib.call("nb_conv_bn_thresholds_from_input" + suf, out.data_ptr(), input.data_ptr(), filter.data_ptr(),
+                  bias.data_ptr(), bias_noise.data_ptr(), D, input.size(1), input.size(2), input.size(3), O, filterx,
+                  filtery, padx, pady, stridex, stridey, tap, int(channels) * filterx * filtery, _stream(input))
     return out
 
 

@@ -229,9 +229,8 @@ class BinarizedConv2d(Binarized):
                 # modules/binary.py:147-155 without the int32 maps: the per-member mean over h,w needs only the sum of
                 # the popcounts (exact integers), mean = fp16(float(sum of activations) / (h*w)); activations are
                 # integers that fp16 holds exactly, so activation > thresh  <=>  2*popc > floor(thresh) + offset.
-                sums = booleanOperations.conv_popc_sums(packed_input, filt, *geom, **tapkw)
-                h, w = booleanOperations._out_hw(packed_input, *geom)
-                thresh = booleanOperations.conv_bn_thresholds(sums, self.bias.detach(), self.bias_noise, offset, h * w)
+                thresh = booleanOperations.conv_bn_thresholds_from_input(
+                    packed_input, filt, self.bias.detach(), self.bias_noise, *geom, channels=self.in_channels, **tapkw)
             else:
                 thresh = (self.bias + self.bias_noise).type(torch.int32) + offset
             if self.pack_output or self.pool_output:

@@ -68,6 +68,15 @@ def test_bad_arguments_are_rejected_without_a_launch(lib):
     assert lib.nb_conv_bn_thresholds(one, one, one, one, 2, 3, 144, 0, None) == 2
     assert lib.nb_conv_bn_thresholds(one, one, ctypes.c_void_p(9), one, 2, 3, 144, 64, None) == 3
     assert lib.nb_conv_bn_thresholds(None, None, None, None, 0, 3, 144, 64, None) == 0
+    # the same thresholds from the layer's input: a window larger than the padded image (no output pixel), a missing
+    # bias, a misaligned noise pointer, an empty population
+    args = (1, 2, 2, 1, 4, 5, 5, 0, 0, 1, 1, 0, 100, None)
+    assert lib.nb_conv_bn_thresholds_from_input_i64(one, one, one, one, one, *args) == 2
+    args = (1, 8, 8, 1, 4, 3, 3, 1, 1, 1, 1, 0, 576, None)
+    assert lib.nb_conv_bn_thresholds_from_input_i64(one, one, one, None, one, *args) == 1
+    assert lib.nb_conv_bn_thresholds_from_input_i32(one, one, one, one, ctypes.c_void_p(9), *args) == 3
+    assert lib.nb_conv_bn_thresholds_from_input_i64(None, None, None, None, None, 0, 8, 8, 1, 4, 3, 3, 1, 1, 1, 1, 0, 576,
+                                                    None) == 0
     # empty problems succeed without touching the pointers
     assert lib.nb_pack_i64(None, None, 0, 64, None) == 0
     assert lib.nb_bmm_i32(None, None, None, 0, 5, 5, 5, None) == 0
