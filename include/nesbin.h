@@ -308,6 +308,10 @@ int nb_sample_philox_i32(int32_t *out, const int32_t *base, const uint32_t *thre
                          nb_stream_t stream);
 int nb_philox_words(uint32_t *out, uint64_t seed, uint64_t subseq, uint64_t first, int64_t count,
                     nb_stream_t stream);
+/* Sampler thresholds from fp16 probabilities (what the layers' set_noise feeds the samplers, modules/binary.py:59-62):
+ * T[i] = min(floor(P[i] * 2^32), 2^32 - 1), 0 for P <= 0 and NaN; exact (fp16 has 11 significant bits).  P = 1.0 fails
+ * only for the word 0xFFFFFFFF, like `p > u` with u in (0, 1] (extensions/src/sample_bits.cu:54). */
+int nb_thresholds_from_p(uint32_t *T, const uint16_t *P, int64_t n, nb_stream_t stream);
 /* The same samplers for a conv layer's filters: the R = O * KK rows are (out channel o, tap t) pairs, r = o * KK + t
  * (the layer's weight is [O*kx*ky, C], modules/binary.py:125), and the kernel writes every sampled word ALSO (or
  * only, when out_rows is NULL) where the conv multiplies it: out_conv [n, KK * Rw, O] with word wi of row (o, t) at

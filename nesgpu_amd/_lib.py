@@ -45,6 +45,7 @@ _SUFFIXED = {
 }
 _PLAIN = {
     "nb_philox_words": [_PTR, _U64, _U64, _U64, _I64, _PTR],
+    "nb_thresholds_from_p": [_PTR, _PTR, _I64, _PTR],
     "nb_conv_engine": [_I32],
     "nb_conv_last_engine": [],
     "nb_flip_count_i64": [_PTR, _PTR, _PTR, _I64, _I64, _I64, _PTR],

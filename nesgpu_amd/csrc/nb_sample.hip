@@ -165,7 +165,7 @@ __global__ __launch_bounds__(256) void sample_ballot_kernel(W *__restrict__ out,
 template <typename W, class Src>
 __global__ __launch_bounds__(256) void sample_narrow_kernel(W *__restrict__ out, const W *__restrict__ base,
                                                             const uint32_t *__restrict__ thresh, uint32_t ts, Src src,
-                                                            int64_t nrows, int64_t R, int C, ConvOut<W> conv)
+                                                            int64_t nrows, int64_t R, int C, ConvOut<W> conv, bool quads)
 {
     NB_FLAT_LOOP(row, nrows)
     {
@@ -175,6 +175,18 @@ __global__ __launch_bounds__(256) void sample_narrow_kernel(W *__restrict__ out,
             W v = 0;
             if constexpr (std::is_same<Src, PhiloxSrc>::value) {
                 const uint64_t g0 = src.key.first + (uint64_t)row * (uint64_t)C;
+                if (quads) {
+                    // whole generator blocks: four columns per block, their thresholds in one 16-byte load (the rows
+                    // of neighbouring lanes lie C words apart: single loads would touch a cache line per lane and word)
+                    const uint4 *__restrict__ tq = reinterpret_cast<const uint4 *>(tr);
+                    for (int k = 0; k < (C >> 2); k++) {
+                        const uint4 b = philox_block(src.key, (g0 >> 2) + (uint64_t)k);
+                        const uint4 t = tr ? tq[k] : make_uint4(ts, ts, ts, ts);
+                        const uint32_t nib = (uint32_t)(b.x < t.x) | ((uint32_t)(b.y < t.y) << 1) |
+                                             ((uint32_t)(b.z < t.z) << 2) | ((uint32_t)(b.w < t.w) << 3);
+                        v |= (W)nib << (4 * k);
+                    }
+                } else
                 for (uint64_t blk = g0 >> 2; blk <= (g0 + (uint64_t)C - 1) >> 2; blk++) {
                     const uint4 b = philox_block(src.key, blk);
                     const uint32_t w4[4] = {b.x, b.y, b.z, b.w};
@@ -426,8 +438,10 @@ int sample_impl(W *out, const W *base, const uint32_t *thresh, uint32_t ts, Src 
         else NB_LAUNCH_WIDE(false, false);
 #undef NB_LAUNCH_WIDE
     } else if (C < bits) {
+        // rows that are whole generator blocks with 16-byte aligned thresholds (src_vec_ok: the stream starts on a block)
+        const bool quads = C % 4 == 0 && src_vec_ok && (!thresh || aligned(thresh, 16));
         sample_narrow_kernel<W, Src><<<dim3(grid_for(n * R)), dim3(256), 0, s>>>(out, base, thresh, ts, src, n * R, R,
-                                                                               (int)C, conv);
+                                                                               (int)C, conv, quads);
     } else {
         sample_ballot_kernel<W, Src><<<dim3(grid_for(n * R * 64)), dim3(256), 0, s>>>(
             out, base, thresh, ts, src, n * R, R, (int)C, (int)Rw, conv);
@@ -474,6 +488,20 @@ int seeded_bmv_impl(int32_t *Cout, const W *base, const uint32_t *thresh, uint32
             Cout, base, thresh, ts, x, src, n * R, R, (int)C, (int)Rw);
     }
     return check_launch(who);
+}
+
+// Probabilities -> sampler thresholds: T = min(floor(p * 2^32), 2^32 - 1), 0 for p <= 0 and for NaN.  p is fp16 (11
+// significant bits), so p * 2^32 is exact in fp32.
+__global__ __launch_bounds__(256) void thresholds_from_p_kernel(uint32_t *__restrict__ T, const _Float16 *__restrict__ P,
+                                                                int64_t n)
+{
+    NB_FLAT_LOOP(i, n)
+    {
+        if (i < n) {
+            const float v = (float)P[i] * 4294967296.0f;
+            T[i] = v >= 4294967295.0f ? 0xFFFFFFFFu : (v > 0.0f ? (uint32_t)floorf(v) : 0u);
+        }
+    }
 }
 
 }  // namespace nb
@@ -602,5 +630,18 @@ int nb_seeded_bmv_philox_i32(int32_t *C, const int32_t *base, const uint32_t *th
     return nb::seeded_bmv_impl<uint32_t, PhiloxSrc>(C, CU32(base), thresh, ts, CU32(x),
                                                     PhiloxSrc{{seed, subseq, first}}, (first & 3) == 0, n, R, Cbits, s,
                                                     "nb_seeded_bmv_philox_i32");
+}
+int nb_thresholds_from_p(uint32_t *T, const uint16_t *P, int64_t n, nb_stream_t stream)
+{
+    const char *who = "nb_thresholds_from_p";
+    NB_REQUIRE(n >= 0 && n < (1LL << 40), "%s: bad count %lld", who, (long long)n);
+    if (n == 0) return NB_OK;
+    NB_REQUIRE_PTR(T);
+    NB_REQUIRE_PTR(P);
+    NB_REQUIRE_ALIGNED(T, 4);
+    NB_REQUIRE_ALIGNED(P, 2);
+    nb::thresholds_from_p_kernel<<<dim3(nb::grid_for(n)), dim3(256), 0, nb::as_stream(stream)>>>(
+        T, reinterpret_cast<const _Float16 *>(P), n);
+    return nb::check_launch(who);
 }
 }

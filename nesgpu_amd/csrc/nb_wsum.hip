@@ -161,6 +161,14 @@ int weighted_sum_impl(uint16_t *ret, const W *in, const uint16_t *w, int64_t n, 
     }
     NB_REQUIRE(zbits <= (1 << 30) && Rw <= (1 << 30), "%s: row too long", who);
     NB_REQUIRE(zbits <= Rw * (int64_t)WordTraits<W>::bits, "%s: zbits exceeds the Rw words of a row", who);
+    // Rows without a tail (every bit of every word is an output bit) are one long row: the output [R, zbits] and the
+    // members' [R, Rw] words are the same memory as [1, R * zbits] and [1, R * Rw].  One-word rows (a conv layer's
+    // 64-channel taps) get the wide kernel that way.
+    if (R > 1 && zbits == Rw * (int64_t)WordTraits<W>::bits && R * zbits <= (1 << 30)) {
+        Rw *= R;
+        zbits *= R;
+        R = 1;
+    }
     const int64_t rowbytes = Rw * (int64_t)sizeof(W);
     // a wave per 32-byte piece once that gives every SIMD a wave; smaller outputs spread better with a wave per column
     if (n > 0 && rowbytes >= 32 && R * ceil_div(zbits, 256) >= 1024) {

@@ -493,7 +493,13 @@ def thresholds_from_p(p):
     T = min(floor(p * 2**32), 2**32 - 1), computed exactly in float64.  p = 1.0 therefore fails only
     for the single word 0xFFFFFFFF, like ``p > u`` with u in (0, 1] in the reference
     (extensions/src/sample_bits.cu:54)."""
-    t = torch.floor(p.detach().to(torch.float64) * 4294967296.0).clamp_(0.0, 4294967295.0)
+    p = p.detach()
+    if p.dtype == torch.float16 and p.is_cuda and p.is_contiguous():     # the layers' case: one kernel
+        out = torch.empty(p.shape, dtype=torch.uint32, device=p.device)
+        with _on(p):
+            _lib.call("nb_thresholds_from_p", out.data_ptr(), p.data_ptr(), p.numel(), _stream(p))
+        return out
+    t = torch.floor(p.to(torch.float64) * 4294967296.0).clamp_(0.0, 4294967295.0)
     return t.to(torch.int64).to(torch.uint32)
 
 

@@ -77,6 +77,10 @@ def test_bad_arguments_are_rejected_without_a_launch(lib):
     assert lib.nb_conv_bn_thresholds_from_input_i32(one, one, one, one, ctypes.c_void_p(9), *args) == 3
     assert lib.nb_conv_bn_thresholds_from_input_i64(None, None, None, None, None, 0, 8, 8, 1, 4, 3, 3, 1, 1, 1, 1, 0, 576,
                                                     None) == 0
+    # sampler thresholds: a NULL probability array, an odd fp16 address, an empty array
+    assert lib.nb_thresholds_from_p(one, None, 4, None) == 1
+    assert lib.nb_thresholds_from_p(one, ctypes.c_void_p(9), 4, None) == 3
+    assert lib.nb_thresholds_from_p(None, None, 0, None) == 0
     # empty problems succeed without touching the pointers
     assert lib.nb_pack_i64(None, None, 0, 64, None) == 0
     assert lib.nb_bmm_i32(None, None, None, 0, 5, 5, 5, None) == 0

@@ -328,7 +328,7 @@ def test_max_pool_vs_oracle(ops, oracle, dtype):
 SAMPLE_SHAPES = [(3, 4, 64), (2, 3, 1), (5, 2, 63), (2, 5, 65), (3, 2, 200), (4, 7, 256), (2, 576, 64), (3, 10, 1024),
                  (2, 9, 16), (3, 5, 128), (2, 3, 100), (2, 5, 256), (2, 7, 512), (2, 3, 768), (2, 3, 2048), (3, 33, 1024),
                  # more members than one member group of the wide kernel; a long row; a 3-column row (first conv layer)
-                 (17, 4, 8192), (2, 27, 3), (19, 6, 256), (9, 1024, 8)]
+                 (17, 4, 8192), (2, 27, 3), (19, 6, 256), (9, 1024, 8), (6, 576, 24), (3, 40, 12)]
 
 
 @pytest.mark.parametrize("dtype", [torch.int64, torch.int32])
@@ -363,7 +363,11 @@ def test_sampling_from_words_vs_oracle(ops, oracle, dtype, n, R, C):
 
 @pytest.mark.parametrize("dtype", [torch.int64, torch.int32])
 @pytest.mark.parametrize("n,R,C,first", [(3, 4, 64, 0), (2, 5, 100, 0), (2, 3, 256, 8), (2, 3, 64, 5), (3, 2, 63, 2),
-                                         (2, 7, 1024, 4 * 0xFFFFFFFE)])
+                                         (2, 7, 1024, 4 * 0xFFFFFFFE),
+                                         # rows shorter than a word: whole generator blocks (24, 16, 4 columns), blocks
+                                         # that straddle rows (a stream that starts inside a block; 3 and 30 columns)
+                                         (5, 70, 24, 0), (3, 9, 16, 12), (2, 5, 24, 6), (4, 27, 3, 0), (130, 3, 4, 0),
+                                         (3, 11, 30, 0)])
 def test_philox_mode_equals_supplied_words_mode(ops, oracle, dtype, n, R, C, first):
     """Generator mode is defined as: the words nb_philox_words writes, fed to the supplied-words kernels."""
     seed, sub = 0x1234ABCD5678EF01, 3
@@ -394,6 +398,19 @@ def test_philox_mode_equals_supplied_words_mode(ops, oracle, dtype, n, R, C, fir
     assert torch.equal(a, ops.seeded_bmv_from_words(thr, x, words))
 
 
+def test_thresholds_from_p_kernel_equals_the_float64_expression(ops):
+    """Every fp16 bit pattern (finite, subnormal, negative, above one, infinities, NaNs) through the one-kernel
+    thresholds against floor(p * 2**32) clamped in float64 on the host."""
+    bits = np.arange(65536, dtype=np.uint16)
+    p = bits.view(np.float16)
+    got = host(ops.thresholds_from_p(dev(p).view(torch.float16))).astype(np.int64) & 0xFFFFFFFF
+    with np.errstate(invalid="ignore", over="ignore"):
+        want = np.floor(p.astype(np.float64) * 4294967296.0)
+    want = np.where(np.isnan(want), 0.0, np.clip(want, 0.0, 4294967295.0)).astype(np.int64)
+    np.testing.assert_array_equal(got, want)
+    assert int(got[np.float16(0.5).view(np.uint16)]) == 2 ** 31 and int(got[np.float16(1.0).view(np.uint16)]) == 2 ** 32 - 1
+
+
 def test_sample_bits_law_and_layout(ops):
     """sample_bits(p, n, dtype, seed): shape [n,R,ceil(C/bits)], zero tail bits, rate ~= p, seed-reproducible."""
     p = torch.tensor([[0.0] * 100, [1.0] * 100, [0.25] * 100, [0.5] * 100], dtype=torch.float16, device="cuda")
@@ -417,7 +434,9 @@ def test_weighted_sum_vs_oracle(ops, oracle, dtype):
     for n, R, C in [(37, 5, 100), (128, 16, 64), (64, 3, 256), (200, 7, 90), (130, 3, 330), (1, 1, 1),
                     (64, 5, 512), (70, 3, 1000), (130, 2, 1536), (100, 9, 2048), (3, 6, 1024), (257, 1, 520 + 504),
                     (70, 4, 576), (65, 2, 2600), (9, 3, 300),
-                    (66, 400, 576), (10, 1100, 256), (5, 130, 2300)]:
+                    (66, 400, 576), (10, 1100, 256), (5, 130, 2300),
+                    # rows without a tail bit (a conv layer's one- and two-word taps): summed as one long row
+                    (130, 5000, 64), (40, 4500, 128), (33, 4099, 64), (70, 600, 64)]:
         nd = NDT[dtype]
         wb = np.dtype(nd).itemsize * 8
         words = rand_words(g, (n, R, (C + wb - 1) // wb), nd)
