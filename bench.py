@@ -345,6 +345,17 @@ def hbm_kernels(torch, steps, warmup, graph=True):
     wts = torch.randn(1024, device=dev, generator=g).half()
     run("weighted_sum [1024,1024,16] -> fp16 [1024,1024]", lambda: ops.weighted_sum(m, wts, 1024),
         m.numel() * 8 + 1024 * 1024 * 2)
+    del m
+    # batch-norm conv layer: thresholds straight from the layer's input (pixel sums from counts of the image's bits, no
+    # conv; bound by the latency of a workgroup's chain and by vector instructions, the fraction is for comparison)
+    for (D, C, O, S) in ((1024, 64, 64, 32), (4096, 64, 128, 16)):
+        x = torch.randint(-2 ** 62, 2 ** 62, (D, S, S, 1), device=dev, generator=g, dtype=torch.int64)
+        f = torch.randint(-2 ** 62, 2 ** 62, (D, 9, O), device=dev, generator=g, dtype=torch.int64)
+        bias = torch.randn(O, device=dev, generator=g).half()
+        noise = torch.randn(D, O, device=dev, generator=g).half()
+        run("conv_bn_thresholds_from_input conv %d->%d 3x3 on %dx%d, D=%d" % (C, O, S, S, D),
+            lambda: ops.conv_bn_thresholds_from_input(x, f, bias, noise, 3, 3, 1, 1, 1, 1),
+            x.numel() * 8 + f.numel() * 8 + D * O * 6)
     return res
 
 
