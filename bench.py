@@ -261,10 +261,29 @@ def calibrate(torch):
         res["ns_per_int8_mfma_per_simd"] = issue
     # the two memory-bound calibrations come last: what follows a calibration in this program is the timed region of
     # an HBM-bound kernel, and the memory clocks should not have come down behind compute-only kernels by then
-    per, ev = time_steps(torch, lambda: lib.nb_calib_copy(dst.data_ptr(), src.data_ptr(), nbytes, 256 * 32, st), 10, 2)
+    # one 16-byte chunk per thread: the workgroups in flight then cover one compact window that moves through the
+    # buffer (a few thousand workgroups that each stride through all of it measured 4.3-4.6 TB/s for the same bytes)
+    per, ev = time_steps(torch, lambda: lib.nb_calib_copy(dst.data_ptr(), src.data_ptr(), nbytes, nbytes // 16 // 256, st),
+                         10, 2)
     res["copy_GBps"] = round(2 * nbytes / ev / 1e9, 1)
     per, ev = time_steps(torch, lambda: lib.nb_calib_read(sink.data_ptr(), src.data_ptr(), nbytes, st), 10, 2)
     res["read_GBps"] = round(nbytes / ev / 1e9, 1)
+    if hasattr(lib, "nb_calib_fill"):
+        # writes alone: a plain fill, and the store pattern of the conv kernels' int32 maps (configuration 3: 1024
+        # members x 256 KB, a wave per 16 pixel columns of a member, 4 KB per row) alternating between two buffers
+        # as successive steps do
+        lib.nb_calib_fill.argtypes = [vp, i64, i32, vp]
+        lib.nb_calib_store_rows.argtypes = [vp, i32, vp]
+        per, ev = time_steps(torch, lambda: lib.nb_calib_fill(dst.data_ptr(), nbytes, nbytes // 16 // 256, st), 10, 2)
+        res["fill_GBps"] = round(nbytes / ev / 1e9, 1)
+        half = 1024 * 262144
+        flip = [0]
+
+        def rows():
+            flip[0] ^= 1
+            lib.nb_calib_store_rows(dst.data_ptr() + flip[0] * half, 1024, st)
+        per, ev = time_steps(torch, rows, 20, 4)
+        res["conv_map_store_GBps"] = round(half / ev / 1e9, 1)
     return res
 
 

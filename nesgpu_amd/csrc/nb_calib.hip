@@ -12,6 +12,30 @@ __global__ __launch_bounds__(256) void calib_copy_kernel(uint4 *__restrict__ dst
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += stride) dst[i] = src[i];
 }
 
+// Streaming writes alone: every thread stores 16-byte chunks at wave-contiguous addresses.
+__global__ __launch_bounds__(256) void calib_fill_kernel(uint4 *__restrict__ dst, int64_t n16, uint32_t v)
+{
+    const int64_t stride = (int64_t)gridDim.x * 256;
+    const uint4 w = make_uint4(v, v + 1u, v + 2u, v + 3u);
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += stride) dst[i] = w;
+}
+
+// The store pattern of the conv kernels' int32 maps without any arithmetic: members of [32 rows][32 pixels][64
+// channels] int32 (256 KB each); a wave owns 16 pixel columns of a member and writes, row after row, its 4 KB of the
+// row (four 16-byte stores per lane), 8 KB apart from row to row.
+__global__ __launch_bounds__(256) void calib_store_rows_kernel(int *__restrict__ out, int units)
+{
+    const int u = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+    if (u >= units) return;
+    const int st = u & 1, z = u >> 1;
+    uint4 *base = reinterpret_cast<uint4 *>(out + (int64_t)z * 65536);
+    const uint4 v = make_uint4(1u, 2u, 3u, (uint32_t)lane);
+    for (int y = 0; y < 32; y++) {
+#pragma unroll
+        for (int s = 0; s < 4; s++) base[((y * 32 + st * 16 + 4 * s + lane / 16) * 64 + 4 * (lane % 16)) / 4] = v;
+    }
+}
+
 // Each thread owns UNR consecutive 16-byte chunks at wave-contiguous addresses.
 template <int UNR>
 __global__ __launch_bounds__(256) void calib_read_kernel(uint32_t *__restrict__ sink, const uint4 *__restrict__ src,
@@ -105,6 +129,20 @@ int nb_calib_copy(void *dst, const void *src, int64_t bytes, int blocks, nb_stre
     nb::calib_copy_kernel<<<dim3((unsigned)blocks), dim3(256), 0, nb::as_stream(s)>>>(
         static_cast<uint4 *>(dst), static_cast<const uint4 *>(src), bytes / 16);
     return nb::check_launch("nb_calib_copy");
+}
+int nb_calib_fill(void *dst, int64_t bytes, int blocks, nb_stream_t s)
+{
+    nb::calib_fill_kernel<<<dim3((unsigned)blocks), dim3(256), 0, nb::as_stream(s)>>>(static_cast<uint4 *>(dst),
+                                                                                     bytes / 16, 7u);
+    return nb::check_launch("nb_calib_fill");
+}
+// members x 256 KB written
+int nb_calib_store_rows(void *dst, int members, nb_stream_t s)
+{
+    const int units = members * 2;
+    nb::calib_store_rows_kernel<<<dim3((unsigned)((units + 3) / 4)), dim3(256), 0, nb::as_stream(s)>>>(
+        static_cast<int *>(dst), units);
+    return nb::check_launch("nb_calib_store_rows");
 }
 int nb_calib_read(void *sink, const void *src, int64_t bytes, nb_stream_t s)
 {

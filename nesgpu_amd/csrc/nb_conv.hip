@@ -292,9 +292,12 @@ int conv_impl(void *out, const W *in, const W *filt, const int32_t *thresh, int6
         t_last_engine = 2;
         return check_launch(who);
     }
-    // One word per pixel, 3x3, packed output or pixel sums: the same wave-per-strip scheme for full channel words
-    // (FP4 matrix cores) and for tap-packed layers of 17 to 32 channels (int8).
-    if (bits == 64 && Cw == 1 && engine != 1 && (engine >= 2 || D >= 128)) {
+    // One word per pixel, 3x3: the same wave-per-strip scheme for full channel words (FP4 matrix cores) and for
+    // tap-packed layers of 17 to 32 channels (int8).  Packed outputs and pixel sums always; the int32 maps unless they
+    // are large (images of 1024 pixels or more and 256 MiB or more to write: there the staged-image kernel below
+    // measured 5-10 % faster, on smaller maps the strip kernel 10-50 %).
+    const bool big_maps = mode == 0 && hw >= 1024 && D * hw * O * 4 >= (1LL << 28);
+    if (bits == 64 && Cw == 1 && engine != 1 && (engine >= 2 || D >= 128) && !big_maps) {
         const int ran = conv_direct_fp4_try(out, reinterpret_cast<const uint64_t *>(in),
                                             reinterpret_cast<const uint64_t *>(filt), thresh, g, D, N, tap_bits, mode,
                                             engine != 3, s);

@@ -89,7 +89,7 @@ bool conv_direct_try(void *out, const uint64_t *in, const uint64_t *filt, const 
                      int64_t D, int O, int tap_bits, int mode, hipStream_t s);
 
 // The same scheme for wider pixels (nb_conv_direct_fp4.hip), 3x3 windows, stride 1, O = 16, 32 or a multiple of 16 from
-// 64 on, mode 2, 3 or 4: one full channel word per pixel with filter [D, 9, O] on the FP4 matrix cores (returns 4; only
+// 64 on, mode 0, 2, 3 or 4: one full channel word per pixel with filter [D, 9, O] on the FP4 matrix cores (returns 4; only
 // with allow_fp4), tap-packed filters of 17 to 32 channels on the int8 matrix cores (returns 2).  0 = not this shape.
 int conv_direct_fp4_try(void *out, const uint64_t *in, const uint64_t *filt, const int32_t *thresh, const ConvGeom &g,
                         int64_t D, int O, int tap_bits, int mode, bool allow_fp4, hipStream_t s);

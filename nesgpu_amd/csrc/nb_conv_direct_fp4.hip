@@ -1,8 +1,8 @@
 // Binary conv on the FP4 matrix cores for layers with one full channel word per pixel (33 to 64 channels), 3x3
-// windows, stride 1: threshold bits out (optionally 2x2 OR-pooled), or the popcount maps' sums over the pixels.  The
-// wave-per-strip scheme of nb_conv_direct.hip with v_mfma_scale_f32_16x16x128_f8f6f4 at unit scales.  (The int32
-// maps themselves stay with the staged-image kernel, whose LDS transpose writes whole pixel rows: from this kernel's
-// register layout they left as 64-byte pieces and took 78-90 us where that kernel takes 50.)
+// windows, stride 1: threshold bits out (optionally 2x2 OR-pooled), the popcount maps' sums over the pixels, or the
+// int32 maps themselves (a finished row goes through an LDS tile, so that whole pixels leave in 16-byte stores; written
+// straight from the accumulators' layout, as 64-byte pieces, they took 78-90 us where 50 are possible).  The
+// wave-per-strip scheme of nb_conv_direct.hip with v_mfma_scale_f32_16x16x128_f8f6f4 at unit scales.
 //
 // Bits become FP4 (E2M1) codes, 1 -> +1.0 (0x2), 0 -> -1.0 (0xA), two positions per byte; +-1 and 0 are exact, the
 // fp32 sums are integers far below 2^24, so popcount(x ^ w) = (K - dot) / 2 is the reference's sum bit for bit.  An
@@ -111,14 +111,19 @@ struct DwAcc<0> {
     typedef dw_v4i type;
 };
 
-// MODE 2: threshold bits packed along the channels; 3: the same, 2x2 OR-pooled; 4: the popcount sums added up over
-// the pixels, int32 [D,O] (atomic adds into a zeroed array)
+// MODE 0: the popcount maps themselves, int32 [D,h,w,O]; 2: threshold bits packed along the channels; 3: the same, 2x2
+// OR-pooled; 4: the popcount sums added up over the pixels, int32 [D,O] (atomic adds into a zeroed array)
 // Q: 1 = FP4 codes, one full channel word per pixel; 0 = +-1 bytes, 17 to 32 channels (tap-packed filter)
 template <int NT, int MODE, int Q>
 __global__ __launch_bounds__(256) void conv_direct_fp4_kernel(const DwConv p)
 {
     typedef typename DwAcc<Q>::type acc_t;
     __shared__ __align__(16) uint2 lut_s[Q ? 128 : 256];  // Q = 1: 256 four-byte entries; Q = 0: 256 eight-byte entries
+    // MODE 0: a wave's finished row, 16 pixels x 16*NT channels of int32, on its way from the accumulators' layout
+    // (a lane holds 4 pixels of one channel) to whole pixels (a lane stores 4 channels of one pixel); pixel rows
+    // 16*NT + 4 dwords apart, so that the four lane groups' writes fall into different banks
+    constexpr int kTileRow = 16 * NT + 4;
+    __shared__ __align__(16) int tile_s[MODE == 0 ? 4 * 16 * kTileRow : 4];
     if (Q)
         reinterpret_cast<uint32_t *>(lut_s)[threadIdx.x] = dw_lut_src.e[threadIdx.x];
     else
@@ -272,12 +277,49 @@ __global__ __launch_bounds__(256) void conv_direct_fp4_kernel(const DwConv p)
                                                   hh * ww * p.Ow * 8, 0x00020000);
         ooff = olive ? (uint32_t)(((xx0 + lane) * p.Ow + cg) * 8) : 0xC0000000u;
     }
+    // MODE 0: int32 [h, w, O]; step s of a row stores pixels 4s .. 4s+3: lane l the channels 4*(l % (4*NT)) .. +3 of the
+    // group of pixel 4s + l / (4*NT) (NT = 4: one pixel per 16 lanes = 256 bytes, a whole run of lines)
+    constexpr int kLpp = 4 * NT, kPps = 64 / kLpp;  // lanes per pixel, pixels per store step
+    int *tile = tile_s + (threadIdx.x >> 6) * 16 * kTileRow;
+    uint32_t ooff0[16 / kPps];
+    if (MODE == 0) {
+        orsrc = __builtin_amdgcn_make_buffer_rsrc(static_cast<int32_t *>(p.out) + z * p.h * (int64_t)p.w * p.O, (short)0,
+                                                  p.h * p.w * p.O * 4, 0x00020000);
+#pragma unroll
+        for (int s2 = 0; s2 < 16 / kPps; s2++) {
+            const int px = s2 * kPps + lane / kLpp, ch = cg * 16 * NT + 4 * (lane % kLpp);
+            ooff0[s2] = (x0 + px < p.w && ch < p.O) ? (uint32_t)(((x0 + px) * p.O + ch) * 4) : 0xC0000000u;
+        }
+    }
     auto finish_row = [&](acc_t (&af)[NT], int y, int par) {
         if (MODE == 4) {
 #pragma unroll
             for (int nt = 0; nt < NT; nt++)
                 csum[nt] += (int)((cmask[0] ? af[nt][0] : 0) + (cmask[1] ? af[nt][1] : 0) + (cmask[2] ? af[nt][2] : 0) +
                                   (cmask[3] ? af[nt][3] : 0));  // Q = 1: float sums, exact: below 2^13
+            return;
+        }
+        if (MODE == 0) {
+            // popcount = (K - dot) / 2; Q = 1: the sums carry the bias K + 1
+#pragma unroll
+            for (int nt = 0; nt < NT; nt++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const auto f = af[nt][r];
+                    tile[(4 * lg + r) * kTileRow + 16 * nt + li] =
+                        Q ? (int)(((float)(2 * p.K + 1) - (float)f) * 0.5f) : (p.K - (int)f) >> 1;
+                }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            typedef int dw_v4s __attribute__((ext_vector_type(4)));
+#pragma unroll
+            for (int s2 = 0; s2 < 16 / kPps; s2++) {
+                const dw_v4s v = *reinterpret_cast<const dw_v4s *>(tile + (s2 * kPps + lane / kLpp) * kTileRow +
+                                                                    4 * (lane % kLpp));
+                __builtin_amdgcn_raw_buffer_store_b128(v, orsrc, (int)(ooff0[s2] + (uint32_t)(y * p.w * p.O * 4)), 0, 0);
+            }
+            __builtin_amdgcn_wave_barrier();
             return;
         }
         int a[NT][4];
@@ -461,13 +503,13 @@ __global__ __launch_bounds__(256) void conv_direct_fp4_kernel(const DwConv p)
     }
 }
 
-// mode 2 (packed threshold bits), 3 (2x2 OR-pooled) or 4 (pixel sums into a zeroed array).  tap_bits == 0: one full
+// mode 0 (int32 maps), 2 (packed threshold bits), 3 (2x2 OR-pooled) or 4 (pixel sums into a zeroed array).  tap_bits == 0: one full
 // channel word per pixel, filter [D, 9, O], FP4 (returns 4; only with allow_fp4); tap_bits in 17..32: tap-packed filter,
 // +-1 bytes (returns 2).  0 = not this shape, nothing launched.
 int conv_direct_fp4_try(void *out, const uint64_t *in, const uint64_t *filt, const int32_t *thresh, const ConvGeom &g,
                         int64_t D, int O, int tap_bits, int mode, bool allow_fp4, hipStream_t s)
 {
-    if (mode != 2 && mode != 3 && mode != 4) return 0;
+    if (mode != 0 && mode != 2 && mode != 3 && mode != 4) return 0;
     const int q = tap_bits == 0 ? 1 : 0;
     if (q ? !allow_fp4 : (tap_bits < 17 || tap_bits > 32)) return 0;
     // 32-bit byte offsets inside one member's output, below 2^30 for the out-of-range marker of the stores
@@ -477,6 +519,7 @@ int conv_direct_fp4_try(void *out, const uint64_t *in, const uint64_t *filt, con
     if (D < 1 || g.h < 1 || g.w < 1) return 0;
     if (!(O == 16 || O == 32 || (O >= 64 && O % 16 == 0))) return 0;
     if (mode == 3 && (g.h < 2 || g.w < 2)) return 0;
+    if (mode == 0 && (int64_t)g.h * g.w * O * 4 >= (1LL << 30)) return 0;  // 32-bit byte offsets inside a member's maps
     // 32-bit byte offsets inside one member's image, far enough below 2^30 for the out-of-range marker
     if ((int64_t)(g.H + g.px + 8) * g.Wd * 8 >= (1LL << 29) || (int64_t)9 * O * 8 >= (1LL << 31)) return 0;
     // 64 channels per wave from 64 channels on (32 per wave, with twice the waves per SIMD, measured 5-8 % slower)
@@ -515,7 +558,9 @@ int conv_direct_fp4_try(void *out, const uint64_t *in, const uint64_t *filt, con
     const dim3 grid((unsigned)ceil_div(units, 4)), block(256);
 #define NB_DW_LAUNCH(nt, qq)                                                   \
     if (NT == nt && q == qq) {                                                 \
-        if (mode == 2)                                                         \
+        if (mode == 0)                                                         \
+            conv_direct_fp4_kernel<nt, 0, qq><<<grid, block, 0, s>>>(p);       \
+        else if (mode == 2)                                                    \
             conv_direct_fp4_kernel<nt, 2, qq><<<grid, block, 0, s>>>(p);       \
         else if (mode == 3)                                                    \
             conv_direct_fp4_kernel<nt, 3, qq><<<grid, block, 0, s>>>(p);       \

@@ -577,8 +577,9 @@ def test_conv_matrix_core_engine_vs_oracle(ops, oracle, mc_engine, C, O, k, pad,
     h, w = act.shape[1:3]
     packed = oracle.pack(act.reshape(-1, O), np.int64).reshape(D, h, w, -1)
     served = 4 if mc_engine == 2 and k == 3 and _fp4_shape(C, O, k) else (2 if covered else 1)
-    # int32 maps of one-word pixels with up to 64 output channels stay on the int8 flavour (write bound)
-    served_i32 = (2 if covered else 1) if Cw == 1 and O <= 64 else served
+    # int32 maps of one-word pixels with up to 64 output channels stay on the int8 flavour of the staged-image kernel
+    # (write bound) unless the wave-per-strip kernel takes them (3x3 windows)
+    served_i32 = (2 if covered else 1) if Cw == 1 and O <= 64 and k != 3 else served
     prev = ops.conv_engine(mc_engine)
     try:
         got = ops.conv(xd, fd, *geom, **kw)
@@ -693,8 +694,8 @@ WIDE_STRIP_CASES = [
 
 @pytest.mark.parametrize("C,O,px,py,H,W,D", WIDE_STRIP_CASES)
 def test_conv_wide_strip_kernels_vs_oracle(ops, oracle, C, O, px, py, H, W, D):
-    """Packed and pooled outputs and pixel sums of 3x3 layers with one word per pixel against the oracle, thresholds
-    spread around the sums (one always, one never above), on the engine that the shape should get, and identical to
+    """Packed and pooled outputs, pixel sums and int32 maps of 3x3 layers with one word per pixel against the oracle,
+    thresholds spread around the sums (one always, one never above), on the engine that the shape should get, and identical to
     the XOR-popcount kernels' answer."""
     g = rng(C * 1000 + O * 10 + H + W)
     x = oracle.pack(g.integers(0, 2, size=(D * H * W, C)).astype(bool), np.int64).reshape(D, H, W, 1)
@@ -726,6 +727,9 @@ def test_conv_wide_strip_kernels_vs_oracle(ops, oracle, C, O, px, py, H, W, D):
         sums = ops.conv_popc_sums(xd, fd, *geom, **kw)
         assert ops.conv_last_engine() == served
         np.testing.assert_array_equal(host(sums), want.reshape(D, -1, O).sum(axis=1))
+        maps = ops.conv(xd, fd, *geom, **kw)                                  # int32 maps: whole pixels through an LDS tile
+        assert ops.conv_last_engine() == served
+        np.testing.assert_array_equal(host(maps), want)
         ops.conv_engine(1)
         assert torch.equal(ops.conv_act_pack(xd, fd, td, *geom, **kw), got)
         assert ops.conv_last_engine() == 1
@@ -819,7 +823,7 @@ def test_conv_matrix_core_many_members(ops, oracle, mc_engine, C, O, S, mode):
     try:
         if mode == "sums":
             got = ops.conv(xd, fd, *geom, **kw)
-            assert ops.conv_last_engine() == (2 if Cw == 1 and O <= 64 else served)
+            assert ops.conv_last_engine() == served
             np.testing.assert_array_equal(host(got), oracle.conv(x, f, *geom))
         else:
             act = oracle.conv_act(x, f, thr, *geom)
