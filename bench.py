@@ -54,6 +54,7 @@ def parse_args():
     ap.add_argument("--only-calib", action="store_true", help="run only the calibration kernels (for counter runs)")
     ap.add_argument("--only", type=int, default=0, help="time just this configuration (for profiler runs)")
     ap.add_argument("--no-graph", action="store_true", help="skip the graph-replay timings of the other configurations")
+    ap.add_argument("--no-step", action="store_true", help="skip the NES step of the SmallNet-shaped network")
     ap.add_argument("--kernels", action="store_true",
                     help="time the HBM-bound helper kernels (pack, unpack, samplers, max-pool, im2col) on their own")
     return ap.parse_args()
@@ -457,6 +458,17 @@ def main():
                                       "generated word (a Philox round is two v_mad_u64_u32 and two v_bitop3_b32), "
                                       "so the vector ALUs are the limit, not HBM"}
     del wg
+    if not args.no_step:
+        # the layer API end to end: one NES step of a SmallNet-shaped network (population 1024), phase by phase
+        sn, fw, up = workloads.small_net_step()
+        reps = max(3, args.steps // 2)
+        line["nes_step_smallnet"] = {
+            "workload": "conv 24->64, pool, conv 64->256, pool, linear 16384->10, batch_norm everywhere, population "
+                        "1024, 32x32 images of 3 x 8 bit planes, through modules.binary (eager launches)",
+            "set_noise_ms": round(time_steps(torch, sn, reps, 2)[0] * 1e3, 4),
+            "forward_ms": round(time_steps(torch, fw, reps, 2)[0] * 1e3, 4),
+            "update_ms": round(time_steps(torch, up, reps, 2)[0] * 1e3, 4)}
+        del sn, fw, up
     if others:
         line["other_configs"] = others
     if cal:

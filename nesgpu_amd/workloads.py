@@ -236,4 +236,50 @@ def cifar_net(D=4096, T=T_P01, seed=0, dtype=torch.int64, device="cuda", classes
     return w
 
 
+def small_net_step(D=1024, classes=10, in_channels=24, seed=0, device="cuda", fuse=True):
+    """One NES step of a SmallNet-shaped binary network through the layer API (the reference's
+    models/cifar10models.py:76-104 driven as in cifar10test.py:150-179): conv 24->64, pool, conv 64->256, pool,
+    flatten, linear 16384->classes, batch_norm everywhere, on 32x32 images of 3 x 8 bit planes.  Returns
+    (set_noise, forward, update): the three phases of a step as callables, for timing.  ``fuse``: packed and pooled
+    outputs between the layers (:func:`nesgpu_amd.modules.binary.fuse_packed_outputs`; same results)."""
+    from .modules import binary
+    layers, cin = [], in_channels
+    for oc in (64, "M", 256, "M"):
+        if oc == "M":
+            layers.append(binary.BinarizedMaxPool2d())
+        else:
+            layers.append(binary.BinarizedConv2d(cin, oc, D, 3, batch_norm=True, padding=1, device=device))
+            cin = oc
+    layers += [torch.nn.Flatten(), binary.BinarizedLinear(cin * 64, classes, D, batch_norm=True, device=device)]
+    net = torch.nn.Sequential(*layers)
+    if fuse:
+        binary.fuse_packed_outputs(net)
+    g = _gen(seed)
+    with torch.no_grad():
+        for p in net.parameters():
+            p.copy_(torch.randn(p.shape, generator=g).to(torch.float16).to(p.device))
+    mods = [m for m in net.modules() if isinstance(m, binary.Binarized)]
+    for i, m in enumerate(mods):
+        m.set_seed(seed + 1 + i)
+        m.perturbed_flag = True
+    img = torch.randint(0, 256, (D, 32, 32, in_channels // 8), generator=g, dtype=torch.uint8).to(device)
+    bits = binary.ExtractBits(torch.uint8)(img)                                       # [D,32,32,in_channels] bool
+    fitness = torch.randn(D, generator=g).to(device)
+
+    def set_noise():
+        for m in mods:
+            m.set_noise()
+
+    def forward():
+        with torch.no_grad():
+            return net(bits)
+
+    def update():
+        for m in mods:
+            m.update(fitness)
+
+    set_noise()
+    return set_noise, forward, update
+
+
 BUILDERS = {1: linear_flip_materialised, 2: linear_flip_fused, 3: conv_int32, 4: conv_sign_pool, 5: cifar_net}
