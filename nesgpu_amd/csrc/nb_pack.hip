@@ -50,6 +50,35 @@ __global__ __launch_bounds__(256) void pack_vec16_kernel(W *__restrict__ out, co
     }
 }
 
+// One thread per output word, 8-byte loads.  Requires C % 8 == 0 and an 8-byte aligned input, so every 8-byte chunk
+// lies inside one row (rows of 24 or 40 bools: 3 x 8 bit planes of an image, say).
+template <typename W>
+__global__ __launch_bounds__(256) void pack_vec8_kernel(W *__restrict__ out, const uint8_t *__restrict__ in,
+                                                        int64_t total_words, int Rw, int64_t C)
+{
+    constexpr int bits = WordTraits<W>::bits;
+    NB_FLAT_LOOP(t, total_words)
+    {
+        if (t >= total_words) continue;
+        const int64_t row = t / Rw;
+        const int y = (int)(t - row * Rw);
+        const int64_t col0 = (int64_t)y * bits;
+        const uint2 *src = reinterpret_cast<const uint2 *>(in + row * C + col0);
+        const int64_t left = C - col0;
+        const int chunks = (int)((left < bits ? left : bits) >> 3);
+        // all loads first and none behind a branch (a chunk past the row re-reads the first one and is dropped)
+        const int cmax = (int)((C < bits ? C : bits) >> 3);  // the same for every thread
+        uint2 v[bits / 8];
+#pragma unroll
+        for (int c = 0; c < bits / 8; c++) v[c] = c < cmax ? src[c < chunks ? c : 0] : make_uint2(0u, 0u);
+        W w = 0;
+#pragma unroll
+        for (int c = 0; c < bits / 8; c++)
+            w |= (W)(c < chunks ? nibble_of_bools(v[c].x) | (nibble_of_bools(v[c].y) << 4) : 0u) << (8 * c);
+        __builtin_nontemporal_store(w, out + t);
+    }
+}
+
 // 64-bit words, C % 64 == 0, 16-byte aligned input: a wave converts 4 KiB of bools (64 words) per step.
 // Load i (0..3) takes the 1 KiB slice i with lanes at consecutive 16-byte chunks (fully coalesced); the four
 // lanes of a quad then hold the four 16-bit quarters of word i*16 + lane/4 and OR them together, and lane
@@ -164,6 +193,8 @@ int pack_impl(W *out, const uint8_t *in, int64_t R, int64_t C, nb_stream_t strea
         pack_quad_kernel<<<dim3(qb), dim3(256), 0, as_stream(stream)>>>(reinterpret_cast<uint64_t *>(out), in, total);
     } else if ((C & 15) == 0 && aligned(in, 16))
         pack_vec16_kernel<W><<<dim3(blocks), dim3(256), 0, as_stream(stream)>>>(out, in, total, (int)Rw, C);
+    else if ((C & 7) == 0 && aligned(in, 8))
+        pack_vec8_kernel<W><<<dim3(blocks), dim3(256), 0, as_stream(stream)>>>(out, in, total, (int)Rw, C);
     else
         pack_generic_kernel<W><<<dim3(blocks), dim3(256), 0, as_stream(stream)>>>(out, in, total, (int)Rw, C);
     return check_launch(who);

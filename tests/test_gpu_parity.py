@@ -131,7 +131,9 @@ def test_golden_philox(ops):
 # ---------------------------------------------------------------------------------------------- vs oracle
 @pytest.mark.parametrize("dtype", [torch.int64, torch.int32])
 @pytest.mark.parametrize("R,C", [(1, 16), (5, 64), (300, 128), (1000, 16), (77, 48), (33, 256), (9, 8192), (4097, 3),
-                                 (64, 80), (2, 1), (513, 576)])
+                                 (64, 80), (2, 1), (513, 576),
+                                 # rows of whole 8-byte chunks that are not whole 16-byte chunks
+                                 (1000, 24), (333, 8), (77, 40), (65, 72), (9, 200), (3, 1048)])
 def test_pack_unpack_vs_oracle(ops, oracle, dtype, R, C):
     bits = rng(R + C).integers(0, 2, size=(R, C)).astype(bool)
     want = oracle.pack(bits, NDT[dtype])
@@ -145,6 +147,11 @@ def test_pack_counts_any_nonzero_byte_as_one(ops):
     t = dev(raw).view(torch.bool)
     got = host(ops.pack(t, torch.int64))
     want = np.packbits(raw != 0, axis=1, bitorder="little").view("<i8")
+    np.testing.assert_array_equal(got, want)
+    raw = rng(2).integers(0, 256, size=(9, 24)).astype(np.uint8)          # rows of three 8-byte chunks
+    raw[raw > 200] = 0
+    got = host(ops.pack(dev(raw).view(torch.bool), torch.int64))
+    want = np.packbits(np.pad(raw != 0, ((0, 0), (0, 40))), axis=1, bitorder="little").view("<i8")
     np.testing.assert_array_equal(got, want)
 
 
