@@ -86,11 +86,14 @@ int nb_bmv_act_pack_i32(int32_t *out, const int32_t *A, const int32_t *x, const 
  *     thr[z,m] = fp16( fp16(bias[m] + bias_noise[z,m]) + mean[m] )
  *     bit[z,m] = act[z,m] > thr[z,m]                            (compared exactly; false for a NaN threshold)
  * A [Z,M,Kw], x [Z,Kw], bias [M] fp16, bias_noise [Z,M] fp16 (raw 16-bit patterns), K = true bit count of a row.
- * pack == 0: out = bool bytes [Z,M]; pack != 0: out = words [Z, ceil(M/bits)], LSB-first, tail bits zero.
+ * pack bit 0 clear: out = bool bytes [Z,M]; set: out = words [Z, ceil(M/bits)], LSB-first, tail bits zero.
+ * pack bit 1 set (values 2, 3): act is rounded to fp16 before it is summed and before it is compared, which is what the
+ * reference's tensor expression does; it matters for K > 2048 only (K <= 65504 then).
  * workspace: device memory, 256-byte aligned, at least nb_bmv_bn_workspace_bytes(Z, M) bytes (the members' int32
  * sums and the per-output totals pass through it; contents undefined afterwards).  The weights are read once.
  *   replaces the composition of modules/binary.py:97-102 (bmm -> 2*popc - in_features -> .type(float16).mean(dim=0)
- *   -> thresh -> compare); equal to it wherever act is exact in fp16 (K <= 2048) and torch's fp16 mean is exact. */
+ *   -> thresh -> compare); equal to it wherever act is exact in fp16 (K <= 2048), or with pack bit 1 set, and torch's
+ *   fp32 sum over the population is exact (Z * K <= 2^24) and Z is a power of two (torch multiplies by 1 / Z). */
 int64_t nb_bmv_bn_workspace_bytes(int64_t Z, int64_t M);
 int nb_bmv_bn_act_i64(void *out, const int64_t *A, const int64_t *x, const uint16_t *bias, const uint16_t *bias_noise,
                       int64_t Z, int64_t M, int64_t Kw, int64_t K, int pack, void *workspace, int64_t workspace_bytes,

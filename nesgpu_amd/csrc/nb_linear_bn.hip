@@ -28,33 +28,48 @@ __global__ __launch_bounds__(256) void bn_zero_kernel(uint32_t *__restrict__ p, 
 
 // colsum[m] += sum of popc[z, m] over one chunk of members; consecutive threads take consecutive m.
 constexpr int kBnChunk = 64;
+// ROUND: the activations 2*popc - K are rounded to fp16 first, as `activation.type(torch.float16)` does, and their
+// (signed) sum is what is added up, in two's complement.
+template <bool ROUND>
 __global__ __launch_bounds__(256) void bn_colsum_kernel(unsigned long long *__restrict__ colsum,
-                                                        const int32_t *__restrict__ popc, int64_t Z, int64_t M)
+                                                        const int32_t *__restrict__ popc, int64_t Z, int64_t M, int64_t K)
 {
     const int64_t m = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (m >= M) return;
     const int64_t z0 = (int64_t)blockIdx.y * kBnChunk;
     const int64_t z1 = z0 + kBnChunk < Z ? z0 + kBnChunk : Z;
     unsigned long long s = 0;
-    for (int64_t z = z0; z < z1; z++) s += (unsigned long long)(uint32_t)popc[z * M + m];
+    for (int64_t z = z0; z < z1; z++) {
+        const int32_t pc = popc[z * M + m];
+        if (ROUND)
+            s += (unsigned long long)(long long)(float)(_Float16)(float)(2ll * pc - K);  // an integer again: |.| <= 65504
+        else
+            s += (unsigned long long)(uint32_t)pc;
+    }
     atomicAdd(colsum + m, s);
 }
 
 // act = 2*popc - K against thr = fp16(fp16(bias + bias_noise) + mean), mean = fp16(float(sum of act) / float(Z)).
 // act is an integer and thr an fp16 number, so act > thr <=> act > floor(thr) (never for NaN).
+// ROUND: total is the sum of the fp16-rounded activations, and the activation is rounded to fp16 for the compare as
+// well (torch compares an int32 tensor with an fp16 one in fp16): the reference's arithmetic for rows of more than
+// 2048 bits, where 2*popc - K is no longer exact in fp16.
+template <bool ROUND>
 __device__ __forceinline__ bool bn_bit(int32_t popc, unsigned long long total, _Float16 bias, _Float16 noise, int64_t Z,
                                        int64_t K)
 {
-    const long long sum_act = 2ll * (long long)total - (long long)K * (long long)Z;
+    const long long sum_act = ROUND ? (long long)total : 2ll * (long long)total - (long long)K * (long long)Z;
     const _Float16 mean = (_Float16)((float)sum_act / (float)Z);
     const _Float16 tb = bias + noise;
     const float t = (float)(_Float16)(tb + mean);
     if (t != t) return false;
-    const float tc = fminf(fmaxf(t, -1.0e9f), 1.0e9f);
     const long long act = 2ll * popc - (long long)K;
+    if (ROUND) return (float)(_Float16)(float)act > t;
+    const float tc = fminf(fmaxf(t, -1.0e9f), 1.0e9f);
     return act > (long long)floorf(tc);
 }
 
+template <bool ROUND>
 __global__ __launch_bounds__(256) void bn_bool_kernel(uint8_t *__restrict__ out, const int32_t *__restrict__ popc,
                                                       const unsigned long long *__restrict__ colsum,
                                                       const _Float16 *__restrict__ bias,
@@ -65,13 +80,13 @@ __global__ __launch_bounds__(256) void bn_bool_kernel(uint8_t *__restrict__ out,
     {
         if (t < Z * M) {
             const int64_t m = t % M;
-            out[t] = bn_bit(popc[t], colsum[m], bias[m], noise[t], Z, K) ? 1 : 0;
+            out[t] = bn_bit<ROUND>(popc[t], colsum[m], bias[m], noise[t], Z, K) ? 1 : 0;
         }
     }
 }
 
 // One wave per output word: lane i < bits decides bit i, the ballot is the word.
-template <typename W>
+template <typename W, bool ROUND>
 __global__ __launch_bounds__(256) void bn_pack_kernel(W *__restrict__ out, const int32_t *__restrict__ popc,
                                                       const unsigned long long *__restrict__ colsum,
                                                       const _Float16 *__restrict__ bias,
@@ -85,7 +100,7 @@ __global__ __launch_bounds__(256) void bn_pack_kernel(W *__restrict__ out, const
     const int64_t z = wd / Mw;
     const int64_t m = (wd - z * Mw) * bits + lane;
     bool bit = false;
-    if (lane < bits && m < M) bit = bn_bit(popc[z * M + m], colsum[m], bias[m], noise[z * M + m], Z, K);
+    if (lane < bits && m < M) bit = bn_bit<ROUND>(popc[z * M + m], colsum[m], bias[m], noise[z * M + m], Z, K);
     const unsigned long long word = __ballot(bit);
     if (lane == 0) out[wd] = (W)word;
 }
@@ -96,6 +111,10 @@ static int bn_impl(void *out, const W *A, const W *x, const uint16_t *bias, cons
                    const char *who)
 {
     constexpr int bits = WordTraits<W>::bits;
+    NB_REQUIRE(pack >= 0 && pack <= 3, "%s: pack must be 0..3 (bit 0: packed output, bit 1: fp16-rounded activations)", who);
+    const bool round16 = (pack & 2) != 0;
+    pack &= 1;
+    NB_REQUIRE(!round16 || K <= 65504, "%s: K=%lld is beyond fp16", who, (long long)K);
     NB_REQUIRE(Z >= 0 && M >= 0 && Kw >= 0 && K >= 0, "%s: negative shape Z=%lld M=%lld Kw=%lld K=%lld", who,
                (long long)Z, (long long)M, (long long)Kw, (long long)K);
     NB_REQUIRE(K <= Kw * (int64_t)bits, "%s: K=%lld exceeds the %lld bits of a row", who, (long long)K,
@@ -135,15 +154,25 @@ static int bn_impl(void *out, const W *A, const W *x, const uint16_t *bias, cons
                         stream);
     }
     if (rc) return rc;
-    bn_colsum_kernel<<<dim3(mblocks, (unsigned)ceil_div(Z, kBnChunk)), dim3(256), 0, s>>>(colsum, popc, Z, M);
+    const dim3 cgrid(mblocks, (unsigned)ceil_div(Z, kBnChunk));
+    if (round16)
+        bn_colsum_kernel<true><<<cgrid, dim3(256), 0, s>>>(colsum, popc, Z, M, K);
+    else
+        bn_colsum_kernel<false><<<cgrid, dim3(256), 0, s>>>(colsum, popc, Z, M, K);
     if (int rc2 = check_launch(who)) return rc2;
     const auto *b16 = reinterpret_cast<const _Float16 *>(bias), *n16 = reinterpret_cast<const _Float16 *>(noise);
     if (pack) {
-        bn_pack_kernel<W><<<dim3((unsigned)ceil_div(Z * Mw, 4)), dim3(256), 0, s>>>(static_cast<W *>(out), popc, colsum,
-                                                                                    b16, n16, Z, M, Mw, K);
+        const dim3 pgrid((unsigned)ceil_div(Z * Mw, 4));
+        if (round16)
+            bn_pack_kernel<W, true><<<pgrid, dim3(256), 0, s>>>(static_cast<W *>(out), popc, colsum, b16, n16, Z, M, Mw, K);
+        else
+            bn_pack_kernel<W, false><<<pgrid, dim3(256), 0, s>>>(static_cast<W *>(out), popc, colsum, b16, n16, Z, M, Mw, K);
     } else {
-        bn_bool_kernel<<<dim3(grid_for(Z * M)), dim3(256), 0, s>>>(static_cast<uint8_t *>(out), popc, colsum, b16, n16, Z,
-                                                                   M, K);
+        const dim3 bgrid(grid_for(Z * M));
+        if (round16)
+            bn_bool_kernel<true><<<bgrid, dim3(256), 0, s>>>(static_cast<uint8_t *>(out), popc, colsum, b16, n16, Z, M, K);
+        else
+            bn_bool_kernel<false><<<bgrid, dim3(256), 0, s>>>(static_cast<uint8_t *>(out), popc, colsum, b16, n16, Z, M, K);
     }
     return check_launch(who);
 }

@@ -186,12 +186,15 @@ def bmv_act_pack(A, x, threshold):
     return out
 
 
-def bmv_bn_act(A, x, bias, bias_noise, in_bits, pack=False, workspace=None):
+def bmv_bn_act(A, x, bias, bias_noise, in_bits, pack=False, workspace=None, round_fp16=False):
     """Linear layer with the population-mean threshold in one call (not in the reference as an op: it is the
     composition of modules/binary.py:97-102).  A [Z,M,Kw] packed weights, x [Z,Kw] (or [Z,Kw,1]) packed inputs, bias [M]
     and bias_noise [Z,M] fp16, ``in_bits`` the true bit count K of a row.  With act = 2*popc - K:
     thr[z,m] = fp16(fp16(bias + bias_noise) + fp16(float(sum_z act[z,m]) / Z)), result = act > thr as bool [Z,M], or with
-    ``pack`` packed along M into [Z, ceil(M/bits)] words.  ``workspace`` (uint8 CUDA tensor) is allocated when absent."""
+    ``pack`` packed along M into [Z, ceil(M/bits)] words.  ``workspace`` (uint8 CUDA tensor) is allocated when absent.
+    ``round_fp16``: act is rounded to fp16 before the mean and the compare, as the reference's tensor expression does
+    (``activation.type(torch.float16).mean(dim=0)``, then an int32 tensor compared with an fp16 one); it only matters
+    for rows of more than 2048 bits, whose activations fp16 no longer holds exactly."""
     _check(A, "A")
     _check(x, "x")
     _check(bias, "bias")
@@ -220,7 +223,8 @@ def bmv_bn_act(A, x, bias, bias_noise, in_bits, pack=False, workspace=None):
         out = torch.empty((Z, M), dtype=torch.bool, device=A.device)
     with _on(A):
         _lib.call("nb_bmv_bn_act" + suf, out.data_ptr(), A.data_ptr(), x.data_ptr(), bias.data_ptr(),
-                  bias_noise.data_ptr(), Z, M, Kw, int(in_bits), 1 if pack else 0, workspace.data_ptr(),
+                  bias_noise.data_ptr(), Z, M, Kw, int(in_bits), (1 if pack else 0) | (2 if round_fp16 else 0),
+                  workspace.data_ptr(),
                   workspace.numel(), _stream(A))
     return out
 

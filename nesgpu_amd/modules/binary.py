@@ -151,6 +151,15 @@ class BinarizedLinear(Binarized):
             return booleanOperations.bmv_bn_act(self.weight_noise, packed_input.view(self.directions, -1),
                                                 self.bias.detach(), self.bias_noise, self.in_features,
                                                 pack=self.pack_output)
+        Z = self.directions
+        if (self.threshold and self.batch_norm and self.in_features <= 65504 and Z & (Z - 1) == 0
+                and Z * self.in_features <= 2 ** 24):
+            # Longer rows: the reference's expression rounds the activations to fp16 (for the mean and for the
+            # compare).  The same call does that too, and gives the very bits of the tensor expression below as long
+            # as torch's fp32 sum over the population is exact (integers below 2**24) and its multiplication by
+            # 1 / directions is a division (a power of two).
+            return booleanOperations.bmv_bn_act(self.weight_noise, packed_input.view(Z, -1), self.bias.detach(),
+                                                self.bias_noise, self.in_features, round_fp16=True)
         if self.pack_output:
             # activation > t  <=>  2*popc - K > floor(t)  <=>  2*popc > floor(t) + K  (activation is an integer)
             thresh = torch.floor((self.bias + self.bias_noise).to(torch.float32)).to(torch.int32) + self.in_features

@@ -301,3 +301,37 @@ def test_conv_bn_thresholds_from_input_equal_the_two_steps(C, O, k, pad, stride,
             assert got.dtype == torch.int32 and torch.equal(got, want), eng
     finally:
         ops.conv_engine(prev)
+
+
+
+@pytest.mark.parametrize("K,M,Z", [(16384, 10, 1024), (4096, 33, 256), (8192, 7, 64), (3000, 5, 128), (65504, 3, 256)])
+def test_linear_bn_beyond_2048_inputs_equals_the_tensor_expression(K, M, Z):
+    """BinarizedLinear(batch_norm=True) with rows longer than fp16's exact integers: the one-call kernel with
+    fp16-rounded activations against the reference's tensor expression (modules/binary.py:97-102) evaluated by torch,
+    bit for bit; weights with few ones / many ones so that the activations spread over the whole range."""
+    from nesgpu_amd.modules import binary
+    from nesgpu_amd.extensions import booleanOperations as ops
+    g = torch.Generator(device="cuda")
+    g.manual_seed(K + M)
+    lin = binary.BinarizedLinear(K, M, Z, batch_norm=True)
+    with torch.no_grad():
+        lin.weight.copy_((torch.randn(M, K, device="cuda", generator=g) * 2).to(torch.float16))
+        lin.bias.copy_((torch.randn(M, device="cuda", generator=g) * 40).to(torch.float16))
+    lin.set_seed(5)
+    lin.set_noise()
+    lin.perturbed_flag = True
+    Kw = (K + 63) // 64
+    x = torch.randint(-2 ** 62, 2 ** 62, (Z, Kw), dtype=torch.int64, device="cuda", generator=g)
+    if K % 64:
+        x[:, -1] &= (1 << (K % 64)) - 1
+    # half of the members see the complement of their weights' majority: large positive and negative activations
+    x[::2] = ~x[::2] if K % 64 == 0 else x[::2]
+    with torch.no_grad():
+        got = lin(x)
+        popc = ops.bmm(lin.weight_noise, x.view(Z, -1, 1))
+        activation = 2 * popc.squeeze(dim=2) - K
+        thresh = (lin.bias + lin.bias_noise)
+        thresh = thresh + activation.type(torch.float16).mean(dim=0, keepdim=True)
+        want = activation > thresh
+    assert got.dtype == torch.bool and torch.equal(got, want)
+    assert 0.02 < float(want.float().mean()) < 0.98
