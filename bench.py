@@ -468,6 +468,10 @@ def main():
             "set_noise_ms": round(time_steps(torch, sn, reps, 2)[0] * 1e3, 4),
             "forward_ms": round(time_steps(torch, fw, reps, 2)[0] * 1e3, 4),
             "update_ms": round(time_steps(torch, up, reps, 2)[0] * 1e3, 4)}
+        if not args.no_graph:
+            fg = time_graph(torch, fw, reps)                 # the same forward without the host's launch pacing
+            if fg:
+                line["nes_step_smallnet"]["forward_graph_ms"] = round(fg * 1e3, 4)
         del sn, fw, up
     if others:
         line["other_configs"] = others
