@@ -1,6 +1,8 @@
 // weighted_sum: ret[r,z] = fp16( sum_m float(w[m]) * bit(in[m,r,z/bits], z%bits) ), the reduction over
 // the population that the update step applies to the sampled masks
 // (extensions/src/weighted_sum.cu:28-46).  fp32 accumulation in member order, like the reference.
+#include <type_traits>
+
 #include "nb_common.hpp"
 
 namespace nb {
@@ -70,15 +72,18 @@ __global__ __launch_bounds__(256) void weighted_sum_kernel(_Float16 *__restrict_
 // 64-byte piece with eight sums measured the same or slower: half as many waves to hide the LDS reads behind.)
 #define NB_WS_COL(ACC, D) ACC += __builtin_bit_cast(float, __builtin_amdgcn_sbfe((int)(D), zz, 1u) & wbits);
 
-// VEC: rows are whole 32-byte pieces and 16-byte aligned (two 16-byte loads per lane); otherwise the piece is fetched
-// as eight 4-byte loads, those past the end of the row left out (rows of 9 words, say: a conv layer's filters).
-template <bool VEC>
+// VEC: rows are whole pieces and 16-byte aligned (16-byte loads); otherwise the piece is fetched as 4-byte loads, those
+// past the end of the row left out (rows of 9 words, say: a conv layer's filters).
+// COLS: 64-bit columns per wave, 4 (a 32-byte piece) or 2 (16 bytes: twice the waves, for outputs too small to give
+// every SIMD a wave otherwise).
+template <bool VEC, int COLS>
 __global__ __launch_bounds__(256) void weighted_sum_line_kernel(_Float16 *__restrict__ ret,
                                                                 const uint32_t *__restrict__ in,
                                                                 const _Float16 *__restrict__ w, int64_t n, int64_t R,
                                                                 int rowdw, int zbits, int npiece)
 {
-    __shared__ uint4 msk[2][4][2][64];  // [buffer][wave][low halves, high halves][member]
+    typedef typename std::conditional<COLS == 4, uint4, uint2>::type half_t;  // one half (low or high) of the columns
+    __shared__ half_t msk[2][4][2][64];  // [buffer][wave][low halves, high halves][member]
     __shared__ float wsh[2][64];
     const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
     const int64_t pid = (int64_t)blockIdx.x * 4 + wv;  // (row, piece); past the end: idle but in step
@@ -86,23 +91,26 @@ __global__ __launch_bounds__(256) void weighted_sum_line_kernel(_Float16 *__rest
     const int64_t r = live ? pid / npiece : 0;
     const int g = live ? (int)(pid - r * npiece) : 0;
     const int64_t stride = R * (int64_t)rowdw;  // dwords from one member's row to the next member's
-    const uint32_t *p = in + r * rowdw + (int64_t)g * 8;
-    const int left = rowdw - g * 8;             // dwords of the row from this piece on
+    const uint32_t *p = in + r * rowdw + (int64_t)g * (2 * COLS);
+    const int left = rowdw - g * (2 * COLS);    // dwords of the row from this piece on
     const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
     auto fetch = [&](uint4 &x, uint4 &y, int64_t m) {
         const uint32_t *q = p + m * stride;
         if (VEC) {
-            x = load_stream16(q), y = load_stream16(q + 4);
+            x = load_stream16(q);
+            if (COLS == 4) y = load_stream16(q + 4);
         } else {
-            // plain loads: the eight of a lane share a cache line, which streaming loads would fetch eight times
+            // plain loads: those of a lane share a cache line, which streaming loads would fetch once per load
             x.x = q[0];
             x.y = left > 1 ? q[1] : 0u;
             x.z = left > 2 ? q[2] : 0u;
             x.w = left > 3 ? q[3] : 0u;
-            y.x = left > 4 ? q[4] : 0u;
-            y.y = left > 5 ? q[5] : 0u;
-            y.z = left > 6 ? q[6] : 0u;
-            y.w = left > 7 ? q[7] : 0u;
+            if (COLS == 4) {
+                y.x = left > 4 ? q[4] : 0u;
+                y.y = left > 5 ? q[5] : 0u;
+                y.z = left > 6 ? q[6] : 0u;
+                y.w = left > 7 ? q[7] : 0u;
+            }
         }
     };
     const uint32_t zz = lane & 31;
@@ -114,8 +122,13 @@ __global__ __launch_bounds__(256) void weighted_sum_line_kernel(_Float16 *__rest
     if (wv == 0 && lane < n) wa = (float)w[lane];
     int buf = 0;
     for (int64_t m0 = 0; m0 < n; m0 += 64, buf ^= 1) {
-        msk[buf][wv][0][lane] = make_uint4(a0.x, a0.z, a1.x, a1.z);
-        msk[buf][wv][1][lane] = make_uint4(a0.y, a0.w, a1.y, a1.w);
+        if constexpr (COLS == 4) {
+            msk[buf][wv][0][lane] = make_uint4(a0.x, a0.z, a1.x, a1.z);
+            msk[buf][wv][1][lane] = make_uint4(a0.y, a0.w, a1.y, a1.w);
+        } else {
+            msk[buf][wv][0][lane] = make_uint2(a0.x, a0.z);
+            msk[buf][wv][1][lane] = make_uint2(a0.y, a0.w);
+        }
         if (wv == 0) wsh[buf][lane] = wa;
         // one barrier per chunk: a buffer is written again two chunks later, after every wave has passed the barrier
         // of the chunk in between and so has finished reading it
@@ -124,24 +137,28 @@ __global__ __launch_bounds__(256) void weighted_sum_line_kernel(_Float16 *__rest
         wa = 0.f;
         if (live && m0 + 64 + lane < n) fetch(a0, a1, m0 + 64 + lane);
         if (wv == 0 && m0 + 64 + lane < n) wa = (float)w[m0 + 64 + lane];
-        const uint4 *mine = &msk[buf][wv][half][0];
+        const half_t *mine = &msk[buf][wv][half][0];
 #pragma unroll 8
         for (int j = 0; j < 64; j++) {
             const int wbits = __builtin_bit_cast(int, wsh[buf][j]);
-            const uint4 d = mine[j];
+            const half_t d = mine[j];
             NB_WS_COL(s0, d.x)
             NB_WS_COL(s1, d.y)
-            NB_WS_COL(s2, d.z)
-            NB_WS_COL(s3, d.w)
+            if constexpr (COLS == 4) {
+                NB_WS_COL(s2, d.z)
+                NB_WS_COL(s3, d.w)
+            }
         }
     }
     if (!live) return;
     _Float16 *o = ret + r * zbits;
-    const int z = g * 256 + lane;
+    const int z = g * (64 * COLS) + lane;
     if (z < zbits) o[z] = (_Float16)s0;
     if (z + 64 < zbits) o[z + 64] = (_Float16)s1;
-    if (z + 128 < zbits) o[z + 128] = (_Float16)s2;
-    if (z + 192 < zbits) o[z + 192] = (_Float16)s3;
+    if (COLS == 4) {
+        if (z + 128 < zbits) o[z + 128] = (_Float16)s2;
+        if (z + 192 < zbits) o[z + 192] = (_Float16)s3;
+    }
 }
 #undef NB_WS_COL
 
@@ -170,13 +187,17 @@ int weighted_sum_impl(uint16_t *ret, const W *in, const uint16_t *w, int64_t n, 
         R = 1;
     }
     const int64_t rowbytes = Rw * (int64_t)sizeof(W);
-    // a wave per 32-byte piece once that gives every SIMD a wave; smaller outputs spread better with a wave per column
-    if (n > 0 && rowbytes >= 32 && R * ceil_div(zbits, 256) >= 1024) {
-        const int64_t npiece = ceil_div(zbits, 256);  // 32-byte pieces of a row that hold output bits
+    // a wave per 32-byte piece once that gives every SIMD a wave, a wave per 16-byte piece for outputs half that size;
+    // smaller outputs spread better with a wave per column
+    if (n > 0 && rowbytes >= 32 && R * ceil_div(zbits, 128) >= 1024) {
+        const bool wide = R * ceil_div(zbits, 256) >= 1024;
+        const int pbits = wide ? 256 : 128;
+        const int64_t npiece = ceil_div(zbits, pbits);  // pieces of a row that hold output bits
         const int64_t blocks = ceil_div(R * npiece, 4);
         NB_REQUIRE(blocks <= kMaxGridX, "%s: output exceeds one launch", who);
-        const bool vec = rowbytes % 32 == 0 && (reinterpret_cast<uintptr_t>(in) & 15) == 0;
-        auto *kern = vec ? weighted_sum_line_kernel<true> : weighted_sum_line_kernel<false>;
+        const bool vec = rowbytes % (pbits / 8) == 0 && (reinterpret_cast<uintptr_t>(in) & 15) == 0;
+        auto *kern = wide ? (vec ? weighted_sum_line_kernel<true, 4> : weighted_sum_line_kernel<false, 4>)
+                          : (vec ? weighted_sum_line_kernel<true, 2> : weighted_sum_line_kernel<false, 2>);
         kern<<<dim3((unsigned)blocks), dim3(256), 0, as_stream(stream)>>>(
             reinterpret_cast<_Float16 *>(ret), reinterpret_cast<const uint32_t *>(in),
             reinterpret_cast<const _Float16 *>(w), n, R, (int)(rowbytes / 4), (int)zbits, (int)npiece);
