@@ -153,6 +153,11 @@ int nb_conv_bn_thresholds_from_input_i32(int32_t *thresh, const int32_t *in, con
  * nb_flip_count: cnt[d, r] = popcount(W[d, r, :] ^ base[r, :]) (uint16); W [D, R, Kw], base [R, Kw].
  * nb_flip_fill:  writes the entries of every slice from W ^ base, given perm, slice_off (in dwords) and slice_len
  *                (pieces per lane, at least ceil(max count in the slice / 8)); never writes past a slice.
+ * nb_flip_layout: perm [D, R] (uint16) and slice_len [D, ceil(R/64)] from cnt [D, R]: inside every block of 1024
+ *                rows the rows in the order of their counts (equal counts in row order), slice_len = ceil(count of
+ *                the slice's last row / 8); slice_off [D, ceil(R/64)] (int64) = the running sum of slice_len * 256
+ *                dwords before each slice, total[0] (int64, device memory) = the dwords of all slices: what the
+ *                caller reads back to size entries.  slice_len 16-byte aligned.
  * nb_expand_fp4: packed rows [rows, Kw] -> FP4 (E2M1) codes [rows_padded, 32 * Kw_padded] bytes, bit 1 -> +1.0,
  *                bit 0 -> -1.0, padding -> 0.0: the operand form of nb_bmm_nt_fp4.
  * nb_bmm_nt_fp4: C[m, n] = popcount(A_m ^ B_n), int32 [M, N], for two expanded operands (rows padded to multiples of
@@ -175,6 +180,8 @@ int nb_conv_bn_thresholds_from_input_i32(int32_t *thresh, const int32_t *in, con
  * nb_flip_skip_count: cnt[d, r] = number of flips of the row.   nb_flip_skip_fill: the entries, as nb_flip_fill.
  * nb_flip_to_dense: materialises flip lists: W [D, R, Kw] must hold base in every member on entry, every listed
  *                flip is XOR-ed in (interop with the dense kernels, and what the tests compare through). */
+int nb_flip_layout(uint16_t *perm, int32_t *slice_len, int64_t *slice_off, int64_t *total, const uint16_t *cnt, int64_t D,
+                   int64_t R, nb_stream_t stream);
 int nb_flip_skip_count_i64(uint16_t *cnt, const uint32_t *cdf, uint32_t cdf0, int64_t Kt, uint64_t seed, uint64_t subseq,
                            uint64_t first, int64_t D, int64_t R, int64_t C, nb_stream_t stream);
 int nb_flip_skip_fill_i64(uint32_t *entries, const int64_t *base, const uint16_t *perm, const int64_t *slice_off,

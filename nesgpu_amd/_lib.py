@@ -50,6 +50,7 @@ _PLAIN = {
     "nb_conv_last_engine": [],
     "nb_flip_count_i64": [_PTR, _PTR, _PTR, _I64, _I64, _I64, _PTR],
     "nb_flip_fill_i64": [_PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _I64, _I64, _I64, _PTR],
+    "nb_flip_layout": [_PTR, _PTR, _PTR, _PTR, _PTR, _I64, _I64, _PTR],
     "nb_flip_skip_count_i64": [_PTR, _PTR, _U32, _I64, _U64, _U64, _U64, _I64, _I64, _I64, _PTR],
     "nb_flip_skip_fill_i64": [_PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _U32, _I64, _U64, _U64, _U64, _I64, _I64, _I64, _PTR],
     "nb_flip_to_dense_i64": [_PTR, _PTR, _PTR, _PTR, _PTR, _I64, _I64, _I64, _PTR],

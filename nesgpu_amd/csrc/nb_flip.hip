@@ -320,39 +320,97 @@ __global__ __launch_bounds__(256) void fl_skip_count_kernel(uint16_t *__restrict
     cnt[q] = (uint16_t)n;
 }
 
-__global__ __launch_bounds__(256) void fl_skip_fill_kernel(uint32_t *__restrict__ entries,
-                                                           const uint64_t *__restrict__ base,
-                                                           const uint16_t *__restrict__ perm,
-                                                           const int64_t *__restrict__ slice_off,
-                                                           const int32_t *__restrict__ slice_len,
-                                                           const uint32_t *__restrict__ cdf, int Kt, float inv_log2q,
-                                                           PhiloxKey key, int64_t nslices, int S, int64_t R, int Kw,
-                                                           int C)
+// ---- the same walk when every row starts on a block boundary of the stream (C and first multiples of 4) ------------
+// All lanes then take word e of their current block at the same time, so a block's four words are four straight-line
+// steps without a per-lane word select.  The table sits in LDS with one entry of padding on either side
+// (tab1[k] = cdf[k - 1], tab1[0] = 0, tab1[Kt + 1] = 2^32 - 1): the float estimate is almost always the rank itself,
+// and one two-entry read confirms it (tab1[est] <= u < tab1[est + 1]); a wave in which any lane fails that test walks
+// the table as skip_rank does.  Same ranks, same words, same results as the kernels above.
+__device__ __forceinline__ void skip_table_load(uint32_t *tab1, const uint32_t *cdf, int Kt)
 {
-    __shared__ uint32_t tab[kSkipMaxTable];
-    for (int i = threadIdx.x; i < Kt; i += 256) tab[i] = cdf[i];
+    for (int i = threadIdx.x; i < Kt + 2; i += 256) tab1[i] = i == 0 ? 0u : (i <= Kt ? cdf[i - 1] : 0xFFFFFFFFu);
     __syncthreads();
-    const int lane = threadIdx.x & 63;
-    const int64_t sl = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (sl >= nslices) return;
-    const int64_t d = sl / S;
-    const int s = (int)(sl - d * S);
-    const int64_t p = (int64_t)s * 64 + lane;
-    const bool valid = p < R;
-    int64_t r = valid ? perm[d * R + p] : 0;
-    r = r < R ? r : R - 1;
-    const int L = 4 * slice_len[sl];
-    uint4 *dst = reinterpret_cast<uint4 *>(entries + slice_off[sl]) + lane;
+}
+
+// ranks of a block's four words: estimates and table reads first, one test for all four
+__device__ __forceinline__ void skip_rank4(int (&rank)[4], const uint32_t *tab1, int Kt, const uint4 &w, float inv_log2q,
+                                           float c0)
+{
+    const uint32_t u[4] = {w.x, w.y, w.z, w.w};
+    uint32_t lo[4], hi[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const float t = (float)(~u[e]) + 1.0f;                    // 2^32 - u, rounded
+        int est = (int)fmaf(__log2f(t), inv_log2q, c0);           // log2(t / 2^32) / log2(q)
+        est = est < 0 ? 0 : (est > Kt ? Kt : est);
+        rank[e] = est;
+        lo[e] = tab1[est];
+        hi[e] = tab1[est + 1];
+    }
+    uint32_t bad = 0;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) bad |= (uint32_t)(lo[e] > u[e]) | (uint32_t)(hi[e] <= u[e]);
+    if (__any(bad != 0)) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            int est = rank[e];
+            while (est < Kt && tab1[est + 1] <= u[e]) est++;
+            while (est > 0 && tab1[est] > u[e]) est--;
+            rank[e] = est;
+        }
+    }
+}
+
+// A lane counts rows q, q + T, q + 2T, ... (T = threads of the grid): lanes whose rows end early start their next
+// one at the following block instead of idling until the longest row of the wave has ended.
+__global__ __launch_bounds__(256) void fl_skip_count_aligned_kernel(uint16_t *__restrict__ cnt,
+                                                                    const uint32_t *__restrict__ cdf, int Kt,
+                                                                    float inv_log2q, PhiloxKey key, int64_t rows, int C)
+{
+    __shared__ uint32_t tab1[kSkipMaxTable + 2];
+    skip_table_load(tab1, cdf, Kt);
+    const int64_t T = (int64_t)gridDim.x * 256;
+    int64_t q = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const uint64_t row_blocks = (uint64_t)C >> 2;
+    uint64_t row_blk = (key.first >> 2) + (uint64_t)q * row_blocks, blk = row_blk;
+    const uint64_t blk_step = (uint64_t)T * row_blocks;
+    const float c0 = -32.0f * inv_log2q;
+    int pos = -1, n = 0;
+    bool live = q < rows;
+    while (__any(live)) {
+        int rank[4];
+        skip_rank4(rank, tab1, Kt, philox_block(key, blk++), inv_log2q, c0);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {   // past the row's end pos stays >= C and nothing more is counted
+            pos += rank[e] < Kt ? rank[e] + 1 : Kt;
+            n += (rank[e] < Kt && pos < C) ? 1 : 0;
+        }
+        if (pos >= C) {
+            if (live) cnt[q] = (uint16_t)n;
+            q += T;
+            row_blk += blk_step;
+            blk = row_blk;
+            pos = -1;
+            n = 0;
+            live = q < rows;
+        }
+    }
+}
+
+// One lane's row, walked word by word (any C, any first): its entries into dwords lane, lane + 64, ... of the slice.
+// A lane's dwords leave four at a time, as whole 16-byte pieces (L is a multiple of 4); never past the slice,
+// whatever the inputs.  The walk writes its entries without the base bit; when a piece is complete, the base
+// words of its (up to eight) columns are asked for together and the bits put in before the piece is stored: one
+// wait for memory per piece instead of one per flip (a wait for a load also waits for the stores before it).
+__device__ __forceinline__ void skip_fill_row(uint4 *__restrict__ dst, int L, const uint64_t *__restrict__ b, int Kw,
+                                              const uint32_t *tab, int Kt, float inv_log2q, const PhiloxKey &key,
+                                              uint64_t start, bool valid, int C)
+{
     const uint32_t sentinel = (uint32_t)(4 * Kw) << 5;
+    const uint32_t npieces = (uint32_t)(4 * Kw);
     int j = 0;
     uint32_t pend = 0;
     bool half = false;
-    // A lane's dwords leave four at a time, as whole 16-byte pieces (L is a multiple of 4); never past the slice,
-    // whatever the inputs.  The walk writes its entries without the base bit; when a piece is complete, the base
-    // words of its (up to eight) columns are asked for together and the bits put in before the piece is stored: one
-    // wait for memory per piece instead of one per flip (a wait for a load also waits for the stores before it).
-    const uint64_t *b = base + r * Kw;
-    const uint32_t npieces = (uint32_t)(4 * Kw);
     uint32_t q0 = 0, q1 = 0, q2 = 0;
     auto base_bit = [&](uint32_t e) -> uint32_t {  // e: one 16-bit entry; 0 for a sentinel
         const uint32_t piece = e >> 5;
@@ -374,7 +432,7 @@ __global__ __launch_bounds__(256) void fl_skip_fill_kernel(uint32_t *__restrict_
         j++;
     };
     if (valid && Kt > 0) {
-        SkipChain chain(key, key.first + (uint64_t)(d * R + r) * (uint64_t)C);
+        SkipChain chain(key, start);
         int pos = -1;
         for (;;) {
             const int rank = skip_rank(tab, Kt, chain.next(), inv_log2q);
@@ -395,6 +453,236 @@ __global__ __launch_bounds__(256) void fl_skip_fill_kernel(uint32_t *__restrict_
     if (half) put(pend | (sentinel << 16));
     while (j < L) put(sentinel | (sentinel << 16));
 }
+
+__global__ __launch_bounds__(256) void fl_skip_fill_kernel(uint32_t *__restrict__ entries,
+                                                           const uint64_t *__restrict__ base,
+                                                           const uint16_t *__restrict__ perm,
+                                                           const int64_t *__restrict__ slice_off,
+                                                           const int32_t *__restrict__ slice_len,
+                                                           const uint32_t *__restrict__ cdf, int Kt, float inv_log2q,
+                                                           PhiloxKey key, int64_t nslices, int S, int64_t R, int Kw,
+                                                           int C)
+{
+    __shared__ uint32_t tab[kSkipMaxTable];
+    for (int i = threadIdx.x; i < Kt; i += 256) tab[i] = cdf[i];
+    __syncthreads();
+    const int lane = threadIdx.x & 63;
+    const int64_t sl = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (sl >= nslices) return;
+    const int64_t d = sl / S;
+    const int s = (int)(sl - d * S);
+    const int64_t p = (int64_t)s * 64 + lane;
+    const bool valid = p < R;
+    int64_t r = valid ? perm[d * R + p] : 0;
+    r = r < R ? r : R - 1;
+    uint4 *dst = reinterpret_cast<uint4 *>(entries + slice_off[sl]) + lane;
+    skip_fill_row(dst, 4 * slice_len[sl], base + r * Kw, Kw, tab, Kt, inv_log2q, key,
+                  key.first + (uint64_t)(d * R + r) * (uint64_t)C, valid, C);
+}
+
+// Rows on block boundaries of the stream (C and first multiples of 4, a table with entries): the lanes of a slice
+// walk in step, eight words (two blocks) to a 16-byte piece.  As long as every word of a live row yields a flip, word
+// i of a row is its flip i, so the piece a wave is on is the same for all its lanes and nothing about the entry's
+// place is per lane; a row that has ended gives sentinels.  A word beyond the table (no flip) in any live row breaks
+// that: the wave then starts its slice again, row by row as above (with a table that runs to saturation this takes a
+// word of 2^32 - 1).
+__global__ __launch_bounds__(256) void fl_skip_fill_aligned_kernel(uint32_t *__restrict__ entries,
+                                                                   const uint64_t *__restrict__ base,
+                                                                   const uint16_t *__restrict__ perm,
+                                                                   const int64_t *__restrict__ slice_off,
+                                                                   const int32_t *__restrict__ slice_len,
+                                                                   const uint32_t *__restrict__ cdf, int Kt,
+                                                                   float inv_log2q, PhiloxKey key, int64_t nslices,
+                                                                   int S, int64_t R, int Kw, int C)
+{
+    __shared__ uint32_t tab1[kSkipMaxTable + 2];
+    skip_table_load(tab1, cdf, Kt);
+    const int lane = threadIdx.x & 63;
+    const int64_t sl = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (sl >= nslices) return;
+    const int64_t d = sl / S;
+    const int s = (int)(sl - d * S);
+    const int64_t p = (int64_t)s * 64 + lane;
+    const bool valid = p < R;
+    int64_t r = valid ? perm[d * R + p] : 0;
+    r = r < R ? r : R - 1;
+    const int P = slice_len[sl];
+    uint4 *dst = reinterpret_cast<uint4 *>(entries + slice_off[sl]) + lane;
+    const uint32_t *b32 = reinterpret_cast<const uint32_t *>(base + r * Kw);
+    const uint32_t sentinel = (uint32_t)(4 * Kw) << 5;
+    const float c0 = -32.0f * inv_log2q;
+    uint64_t blk = (key.first >> 2) + (uint64_t)(d * R + r) * ((uint64_t)C >> 2);
+    int pos = valid ? -1 : C;
+    bool irregular = false;
+    uint4 cur = make_uint4(0u, 0u, 0u, 0u);   // the row's window that the last entry lay in, and its first dword
+    uint32_t curwin = 0xFFFFFFFFu;
+    const uint32_t last_start = (uint32_t)(2 * Kw - 4);
+    int piece = 0;
+    for (; piece < P; ++piece) {
+        uint32_t e[8];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            int rank4[4];
+            skip_rank4(rank4, tab1, Kt, philox_block(key, blk++), inv_log2q, c0);
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const int rank = rank4[k];
+                irregular |= rank >= Kt && pos < C;
+                pos += rank < Kt ? rank + 1 : Kt;
+                const uint32_t col = (uint32_t)pos;
+                e[4 * h + k] = pos < C ? (((col >> 5) << 6) | (col & 31u)) : sentinel;
+            }
+        }
+        if (__any(irregular)) break;
+        // Base bits from 16-byte windows of the row (128 columns; the last one ends with the row): a window is asked
+        // for only where an entry leaves the one before it, since what the look-ups cost is the number of lanes that
+        // ask, not the bytes.  Four entries' windows are asked for together; nothing is read for a sentinel.
+#pragma unroll
+        for (int h = 0; h < 8; h += 4) {
+            uint32_t st[4];
+            bool need[4];
+            uint4 w[4];
+            uint32_t prev = curwin;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const uint32_t dw = e[h + k] >> 6, a = dw & ~3u;
+                st[k] = a < last_start ? a : last_start;
+                const bool live = e[h + k] != sentinel;
+                need[k] = live && st[k] != prev;
+                prev = live ? st[k] : prev;
+            }
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+                if (need[k]) __builtin_memcpy(&w[k], b32 + st[k], 16);
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                if (need[k]) {
+                    cur = w[k];
+                    curwin = st[k];
+                }
+                const uint32_t d = (e[h + k] >> 6) - curwin;
+                const uint32_t word = d == 0 ? cur.x : d == 1 ? cur.y : d == 2 ? cur.z : cur.w;
+                const uint32_t bit = e[h + k] != sentinel ? (word >> (e[h + k] & 31u)) & 1u : 0u;
+                e[h + k] |= bit << 5;
+            }
+        }
+        dst[(int64_t)piece * 64] = make_uint4(e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16),
+                                              e[6] | (e[7] << 16));
+    }
+    if (piece < P)
+        skip_fill_row(dst, 4 * P, base + r * Kw, Kw, tab1 + 1, Kt, inv_log2q, key,
+                      key.first + (uint64_t)(d * R + r) * (uint64_t)C, valid, C);
+}
+
+// v of lane (lane ^ j), j a power of two below 64: quad permutes, swizzles inside 32 lanes, a general exchange for 32
+__device__ __forceinline__ uint32_t xor_lane(uint32_t v, int j)
+{
+    switch (j) {
+    case 1: return (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0xB1, 0xF, 0xF, true);   // quad_perm [1, 0, 3, 2]
+    case 2: return (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0x4E, 0xF, 0xF, true);   // quad_perm [2, 3, 0, 1]
+    case 4: return (uint32_t)__builtin_amdgcn_ds_swizzle((int)v, (4 << 10) | 0x1F);    // bit mode: and 31, xor j
+    case 8: return (uint32_t)__builtin_amdgcn_ds_swizzle((int)v, (8 << 10) | 0x1F);
+    case 16: return (uint32_t)__builtin_amdgcn_ds_swizzle((int)v, (16 << 10) | 0x1F);
+    default: return (uint32_t)__shfl_xor((int)v, j);
+    }
+}
+
+// Row order and slice lengths from the counts: workgroup (d, block of 1024 rows) sorts its rows by (count, row) with a
+// bitonic network, a key per thread, partners inside a wave by lane exchange and others through LDS (keys
+// count << 10 | row-in-block are distinct, so the order is the stable one; rows past R
+// sort last) and writes perm and, from the last row of every run of 64, the slice's pieces per lane.
+__global__ __launch_bounds__(1024) void fl_layout_kernel(uint16_t *__restrict__ perm, int32_t *__restrict__ slice_len,
+                                                         const uint16_t *__restrict__ cnt, int64_t R, int nblk, int S)
+{
+    __shared__ uint32_t key[1024];
+    const int t = threadIdx.x;
+    const int64_t d = blockIdx.x / nblk;
+    const int blk = (int)(blockIdx.x - d * nblk);
+    const int64_t r0 = (int64_t)blk * 1024;
+    const int valid = (int)(R - r0 < 1024 ? R - r0 : 1024);
+    uint32_t v = t < valid ? ((uint32_t)cnt[d * R + r0 + t] << 10) | (uint32_t)t : 0xFFFFFC00u | (uint32_t)t;
+#pragma unroll
+    for (int k = 2; k <= 1024; k <<= 1) {
+#pragma unroll
+        for (int j = k >> 1; j > 0; j >>= 1) {
+            uint32_t o;
+            if (j >= 64) {  // the partner sits in another wave: through LDS
+                __syncthreads();
+                key[t] = v;
+                __syncthreads();
+                o = key[t ^ j];
+            } else {
+                o = xor_lane(v, j);
+            }
+            const bool keep_min = ((t & j) == 0) == ((t & k) == 0);
+            v = keep_min ? (v < o ? v : o) : (v > o ? v : o);
+        }
+    }
+    if (t < valid) {
+        perm[d * R + r0 + t] = (uint16_t)(r0 + (v & 1023u));
+        if ((t & 63) == 63 || t == valid - 1) slice_len[d * S + (r0 + t) / 64] = (int32_t)(((v >> 10) + 7) >> 3);
+    }
+}
+
+// slice_off = running sum of slice_len * 256 dwords (exclusive), total[0] = the sum.  Workgroup b owns slices
+// 8192 b .. 8192 b + 8191, eight per thread, and first adds up everything before them itself.
+__device__ __forceinline__ int64_t block_sum_1024(int64_t v, int64_t *wave_sum, int64_t *incl_out)
+{
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    int64_t incl = v;  // inclusive sum over the wave's lanes
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const int64_t up = __shfl_up(incl, o);
+        if (lane >= o) incl += up;
+    }
+    __syncthreads();
+    if (lane == 63) wave_sum[wv] = incl;
+    __syncthreads();
+    int64_t before = 0, all = 0;
+#pragma unroll
+    for (int w = 0; w < 16; ++w) {
+        before += w < wv ? wave_sum[w] : 0;
+        all += wave_sum[w];
+    }
+    *incl_out = before + incl;
+    return all;
+}
+
+__global__ __launch_bounds__(1024) void fl_offsets_kernel(int64_t *__restrict__ slice_off, int64_t *__restrict__ total,
+                                                          const int32_t *__restrict__ slice_len, int64_t n)
+{
+    __shared__ int64_t wave_sum[16];
+    const int t = threadIdx.x;
+    const int64_t tile = (int64_t)blockIdx.x * 8192;
+    int64_t head = 0, unused;
+    const int4 *len4 = reinterpret_cast<const int4 *>(slice_len);  // a tile is 2048 of these
+#pragma unroll 4
+    for (int64_t i = t; i < tile / 4; i += 1024) {
+        const int4 q = len4[i];
+        head += (int64_t)q.x + q.y + q.z + q.w;
+    }
+    const int64_t carry = block_sum_1024(head, wave_sum, &unused) * 256;
+    const int64_t i0 = tile + (int64_t)t * 8;
+    int64_t v[8], mine = 0, incl;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        v[k] = i0 + k < n ? (int64_t)slice_len[i0 + k] * 256 : 0;
+        mine += v[k];
+    }
+    const int64_t all = block_sum_1024(mine, wave_sum, &incl);
+    int64_t run = carry + incl - mine;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        if (i0 + k < n) slice_off[i0 + k] = run;
+        run += v[k];
+    }
+    if (t == 0 && blockIdx.x == gridDim.x - 1) total[0] = carry + all;
+}
+
+// whether every row of the walk starts on a block boundary of the stream (and there is a table to look up)
+static inline bool skip_rows_aligned(int64_t C, uint64_t first, int64_t Kt) { return Kt > 0 && C % 4 == 0 && first % 4 == 0; }
+// the aligned fill reads the base in 16-byte windows: rows of at least two words
+static inline bool skip_fill_aligned(int64_t C, uint64_t first, int64_t Kt) { return skip_rows_aligned(C, first, Kt) && C > 64; }
 
 // Flip lists -> materialised weights: W must hold the base in every member on entry; every flip is XOR-ed in.  A
 // lane owns its row, so plain read-modify-writes suffice (flips come in column order: one write per touched word).
@@ -663,8 +951,15 @@ int nb_flip_skip_count_i64(uint16_t *cnt, const uint32_t *cdf, uint32_t cdf0, in
     NB_REQUIRE_ALIGNED(cdf, 4);
     const int64_t blocks = nb::ceil_div(D * R, 256);
     NB_REQUIRE(blocks <= nb::kMaxGridX, "%s: too many rows for one launch", who);
-    nb::fl_skip_count_kernel<<<dim3((unsigned)blocks), dim3(256), 0, nb::as_stream(stream)>>>(
-        cnt, cdf, (int)Kt, inv_log2q, nb::PhiloxKey{seed, subseq, first}, D * R, (int)C);
+    if (nb::skip_rows_aligned(C, first, Kt)) {
+        // beyond 2048 workgroups (eight per compute unit) a lane takes several rows, up to eight
+        const int64_t grid = blocks <= 2048 ? blocks : std::max<int64_t>(2048, nb::ceil_div(blocks, 8));
+        nb::fl_skip_count_aligned_kernel<<<dim3((unsigned)grid), dim3(256), 0, nb::as_stream(stream)>>>(
+            cnt, cdf, (int)Kt, inv_log2q, nb::PhiloxKey{seed, subseq, first}, D * R, (int)C);
+    } else {
+        nb::fl_skip_count_kernel<<<dim3((unsigned)blocks), dim3(256), 0, nb::as_stream(stream)>>>(
+            cnt, cdf, (int)Kt, inv_log2q, nb::PhiloxKey{seed, subseq, first}, D * R, (int)C);
+    }
     return nb::check_launch(who);
 }
 
@@ -692,9 +987,44 @@ int nb_flip_skip_fill_i64(uint32_t *entries, const int64_t *base, const uint16_t
     if (Kw > 0) NB_REQUIRE_PTR(base);
     NB_REQUIRE_ALIGNED(base, 8);
     const int64_t S = (R + 63) / 64;
-    nb::fl_skip_fill_kernel<<<dim3((unsigned)nb::ceil_div(D * S, 4)), dim3(256), 0, nb::as_stream(stream)>>>(
-        entries, reinterpret_cast<const uint64_t *>(base), perm, slice_off, slice_len, cdf, (int)Kt, inv_log2q,
-        nb::PhiloxKey{seed, subseq, first}, D * S, (int)S, R, (int)Kw, (int)C);
+    const dim3 grid((unsigned)nb::ceil_div(D * S, 4));
+    if (nb::skip_fill_aligned(C, first, Kt))
+        nb::fl_skip_fill_aligned_kernel<<<grid, dim3(256), 0, nb::as_stream(stream)>>>(
+            entries, reinterpret_cast<const uint64_t *>(base), perm, slice_off, slice_len, cdf, (int)Kt, inv_log2q,
+            nb::PhiloxKey{seed, subseq, first}, D * S, (int)S, R, (int)Kw, (int)C);
+    else
+        nb::fl_skip_fill_kernel<<<grid, dim3(256), 0, nb::as_stream(stream)>>>(
+            entries, reinterpret_cast<const uint64_t *>(base), perm, slice_off, slice_len, cdf, (int)Kt, inv_log2q,
+            nb::PhiloxKey{seed, subseq, first}, D * S, (int)S, R, (int)Kw, (int)C);
+    return nb::check_launch(who);
+}
+
+int nb_flip_layout(uint16_t *perm, int32_t *slice_len, int64_t *slice_off, int64_t *total, const uint16_t *cnt, int64_t D,
+                   int64_t R, nb_stream_t stream)
+{
+    const char *who = "nb_flip_layout";
+    if (int rc = nb::flip_shape_check(D, R, 0, who)) return rc;
+    NB_REQUIRE_PTR(total);
+    NB_REQUIRE_ALIGNED(total, 8);
+    const int64_t S = (R + 63) / 64;
+    if (D * R > 0) {
+        NB_REQUIRE_PTR(perm);
+        NB_REQUIRE_PTR(slice_len);
+        NB_REQUIRE_PTR(slice_off);
+        NB_REQUIRE_PTR(cnt);
+        NB_REQUIRE_ALIGNED(perm, 2);
+        NB_REQUIRE_ALIGNED(slice_len, 16);
+        NB_REQUIRE_ALIGNED(slice_off, 8);
+        NB_REQUIRE_ALIGNED(cnt, 2);
+        const int64_t nblk = nb::ceil_div(R, 1024);
+        NB_REQUIRE(D * nblk <= nb::kMaxGridX / 4, "%s: too many rows for one launch", who);
+        nb::fl_layout_kernel<<<dim3((unsigned)(D * nblk)), dim3(1024), 0, nb::as_stream(stream)>>>(
+            perm, slice_len, cnt, R, (int)nblk, (int)S);
+        if (int rc = nb::check_launch(who)) return rc;
+    }
+    const int64_t n = D * R > 0 ? D * S : 0;
+    nb::fl_offsets_kernel<<<dim3((unsigned)std::max<int64_t>(1, nb::ceil_div(n, 8192))), dim3(1024), 0,
+                            nb::as_stream(stream)>>>(slice_off, total, slice_len, n);
     return nb::check_launch(who);
 }
 

@@ -747,17 +747,14 @@ def _flip_rows_layout(cnt, D, R):
     of 1024 rows, slices of 64 rows padded to their longest row in 16-byte pieces of 8 flips."""
     dev = cnt.device
     S = ceil_div(R, 64)
-    nblk = ceil_div(R, 1024)
-    c = cnt.view(torch.int16).to(torch.int32) & 0xFFFF
-    cp = torch.nn.functional.pad(c, (0, nblk * 1024 - R), value=1 << 20).view(D, nblk, 1024)
-    order = torch.sort(cp, dim=2, stable=True).indices + (torch.arange(nblk, device=dev) * 1024).view(1, nblk, 1)
-    order = order.view(D, nblk * 1024)[:, :R].contiguous()                       # padding sorts last in its block
-    cs = torch.nn.functional.pad(c.gather(1, order), (0, S * 64 - R)).view(D, S, 64)
-    slice_len = ((cs.max(dim=2).values + 7) // 8).to(torch.int32).contiguous()  # 16-byte pieces (8 flips) per lane
-    lens = slice_len.view(-1).to(torch.int64) * 256                              # dwords of a slice
-    slice_off = (torch.cumsum(lens, 0) - lens).view(D, S).contiguous()
-    total = int(lens.sum().item()) if D * S else 0
-    return order.to(torch.uint16).contiguous(), slice_len, slice_off, total
+    perm = torch.empty((D, R), dtype=torch.uint16, device=dev)
+    slice_len = torch.empty((D, S), dtype=torch.int32, device=dev)
+    slice_off = torch.empty((D, S), dtype=torch.int64, device=dev)
+    total = torch.empty((1,), dtype=torch.int64, device=dev)
+    with _on(cnt):
+        _lib.call("nb_flip_layout", perm.data_ptr(), slice_len.data_ptr(), slice_off.data_ptr(), total.data_ptr(),
+                  cnt.data_ptr(), D, R, _stream(cnt))
+    return perm, slice_len, slice_off, int(total.item())     # the one read-back: entries is sized by it
 
 
 def flip_rows_from_weights(W, base):

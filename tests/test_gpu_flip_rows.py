@@ -159,6 +159,29 @@ def test_bmv_flip_vs_oracle(ops, oracle, D, R, C, p):
     assert torch.equal(ops.bmv_flip(rows, xd, G=G), got)
 
 
+@pytest.mark.parametrize("D,R,hi", [(1, 1, 5), (3, 63, 3), (2, 64, 100), (5, 100, 2), (3, 1024, 40), (2, 1100, 7),
+                                    (2, 2053, 65535), (70, 130, 9)])
+def test_flip_layout_orders_blocks_of_rows_by_count(ops, D, R, hi):
+    """Row order and slice lengths against numpy: a stable sort by count inside every block of 1024 rows, pieces per
+    lane from the longest row of each run of 64; running offsets in dwords."""
+    g = np.random.default_rng(D * 1000 + R)
+    cnt = g.integers(0, hi + 1, size=(D, R)).astype(np.uint16)
+    perm, slice_len, slice_off, total = ops._flip_rows_layout(dev(cnt.view(np.int16)).view(torch.uint16), D, R)
+    S = (R + 63) // 64
+    want_perm = np.concatenate([b0 + np.argsort(cnt[:, b0:b0 + 1024].astype(np.int64), axis=1, kind="stable")
+                                for b0 in range(0, R, 1024)], axis=1)
+    np.testing.assert_array_equal(host(perm.view(torch.int16)).view(np.uint16), want_perm.astype(np.uint16))
+    sorted_cnt = np.take_along_axis(cnt.astype(np.int64), want_perm, axis=1)
+    padded = np.zeros((D, S * 64), dtype=np.int64)
+    padded[:, :R] = sorted_cnt
+    want_len = (padded.reshape(D, S, 64).max(axis=2) + 7) // 8
+    np.testing.assert_array_equal(host(slice_len), want_len.astype(np.int32))
+    lens = want_len.reshape(-1) * 256
+    np.testing.assert_array_equal(host(slice_off).reshape(-1), np.cumsum(lens) - lens)
+    assert total == int(lens.sum())
+    assert slice_off.dtype == torch.int64 and slice_len.dtype == torch.int32 and perm.dtype == torch.uint16
+
+
 def test_flip_shapes_are_checked(ops):
     with pytest.raises(RuntimeError, match="at most 511"):
         ops._lib.call("nb_flip_count_i64", 256, 256, 256, 1, 4, 512, None)
@@ -168,7 +191,11 @@ def test_flip_shapes_are_checked(ops):
 
 @pytest.mark.parametrize("D,R,C,p,first", [(3, 64, 64, 0.1, 0), (2, 100, 200, 0.05, 8), (4, 1024, 8192, 0.01, 0),
                                            (2, 1100, 128, 0.3, 3), (300, 128, 256, 0.02, 0), (2, 70, 3000, 0.0002, 5),
-                                           (2, 10, 64, 0.0, 0), (2, 130, 70, 1.0, 0), (3, 1, 1, 0.5, 1)])
+                                           (2, 10, 64, 0.0, 0), (2, 130, 70, 1.0, 0), (3, 1, 1, 0.5, 1),
+                                           # rows on block boundaries of the stream with a table cut short (words
+                                           # beyond it: no flip), p = 1 there, and more rows than one pass of lanes
+                                           (2, 70, 3000, 0.0002, 4), (3, 130, 72, 1.0, 0), (2, 64, 4, 0.5, 12),
+                                           (600, 1024, 64, 0.1, 0)])
 def test_skip_sampler_vs_oracle(ops, oracle, D, R, C, p, first):
     """Flip lists drawn by the skip sampler == the oracle's restatement of the same walk (materialised through
     flip_rows_to_weights), and the products from those lists == the oracle's bmm on the oracle's weights."""
