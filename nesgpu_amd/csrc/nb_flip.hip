@@ -338,11 +338,12 @@ __device__ __forceinline__ void skip_rank4(int (&rank)[4], const uint32_t *tab1,
 {
     const uint32_t u[4] = {w.x, w.y, w.z, w.w};
     uint32_t lo[4], hi[4];
+    const float kt_f = (float)Kt;
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-        const float t = (float)(~u[e]) + 1.0f;                    // 2^32 - u, rounded
-        int est = (int)fmaf(__log2f(t), inv_log2q, c0);           // log2(t / 2^32) / log2(q)
-        est = est < 0 ? 0 : (est > Kt ? Kt : est);
+        // log2((2^32 - 1 - u) / 2^32) / log2(q): never negative, +inf for u = 2^32 - 1; the missing 1 moves the
+        // estimate for about two words in a million
+        const int est = (int)fminf(fmaf(__log2f((float)(~u[e])), inv_log2q, c0), kt_f);
         rank[e] = est;
         lo[e] = tab1[est];
         hi[e] = tab1[est + 1];
