@@ -81,6 +81,10 @@ def test_bad_arguments_are_rejected_without_a_launch(lib):
     assert lib.nb_thresholds_from_p(one, None, 4, None) == 1
     assert lib.nb_thresholds_from_p(one, ctypes.c_void_p(9), 4, None) == 3
     assert lib.nb_thresholds_from_p(None, None, 0, None) == 0
+    # flip-list layout: the list length has to go somewhere, slice lengths are read 16 bytes at a time, R <= 65536
+    assert lib.nb_flip_layout(one, one, one, None, one, 2, 64, None) == 1
+    assert lib.nb_flip_layout(one, ctypes.c_void_p(8), one, one, one, 2, 64, None) == 3
+    assert lib.nb_flip_layout(one, one, one, one, one, 2, 65537, None) == 2
     # empty problems succeed without touching the pointers
     assert lib.nb_pack_i64(None, None, 0, 64, None) == 0
     assert lib.nb_bmm_i32(None, None, None, 0, 5, 5, 5, None) == 0
