@@ -371,6 +371,7 @@ def test_sampling_from_words_vs_oracle(ops, oracle, dtype, n, R, C):
 @pytest.mark.parametrize("dtype", [torch.int64, torch.int32])
 @pytest.mark.parametrize("n,R,C,first", [(3, 4, 64, 0), (2, 5, 100, 0), (2, 3, 256, 8), (2, 3, 64, 5), (3, 2, 63, 2),
                                          (2, 7, 1024, 4 * 0xFFFFFFFE),
+                                         (20, 700, 4096, 0),   # enough words for eight members per lane
                                          # rows shorter than a word: whole generator blocks (24, 16, 4 columns), blocks
                                          # that straddle rows (a stream that starts inside a block; 3 and 30 columns)
                                          (5, 70, 24, 0), (3, 9, 16, 12), (2, 5, 24, 6), (4, 27, 3, 0), (130, 3, 4, 0),
