@@ -20,7 +20,7 @@ __global__ __launch_bounds__(256) void weighted_sum_kernel(_Float16 *__restrict_
 {
     constexpr int bits = WordTraits<W>::bits;
     constexpr int wpc = 64 / bits;  // words per 64-bit column
-    __shared__ float wsh[64];
+    __shared__ float wsh[2][64];
     const int lane = threadIdx.x & 63;
     const int64_t cid = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);  // (row, column); past the end: idle but in step
     const bool live = cid < R * ncol;
@@ -29,28 +29,45 @@ __global__ __launch_bounds__(256) void weighted_sum_kernel(_Float16 *__restrict_
     const int64_t stride = R * (int64_t)Rw;
     const W *p = in + r * Rw + (int64_t)c * wpc;
     const bool has_hi = wpc == 1 || c * wpc + 1 < Rw;
-    float acc = 0.f;
-    for (int64_t m0 = 0; m0 < n; m0 += 64) {
-        __syncthreads();
-        if (threadIdx.x < 64) wsh[threadIdx.x] = m0 + threadIdx.x < n ? (float)w[m0 + threadIdx.x] : 0.f;
-        __syncthreads();
-        uint32_t vlo = 0, vhi = 0;  // members past n contribute the zero word: nothing is added for them
-        if (live && m0 + lane < n) {
-            if (wpc == 1) {
-                const uint64_t v = (uint64_t)p[(m0 + lane) * stride];
-                vlo = (uint32_t)v;
-                vhi = (uint32_t)(v >> 32);
-            } else {
-                vlo = (uint32_t)p[(m0 + lane) * stride];
-                vhi = has_hi ? (uint32_t)p[(m0 + lane) * stride + 1] : 0u;
-            }
+    const uint16_t *wr = reinterpret_cast<const uint16_t *>(w);
+    // The next chunk's words and weights are fetched before the current chunk is summed, always and from a valid place
+    // (members past n: the last member again; idle waves: row 0), and masked where they are used: a load whose result
+    // joins a zero from another path would be waited for right where it is issued.
+    uint32_t vlo, vhi, wa;
+    auto fetch = [&](int64_t m) {
+        const W *q = p + (m < n ? m : n - 1) * stride;
+        if (wpc == 1) {
+            const uint64_t v = (uint64_t)q[0];
+            vlo = (uint32_t)v;
+            vhi = (uint32_t)(v >> 32);
+        } else {
+            vlo = (uint32_t)q[0];
+            vhi = (uint32_t)q[has_hi ? 1 : 0];
         }
+        wa = wr[m < n ? m : n - 1];
+    };
+    if (n <= 0) {  // no members: zeros, and nothing to fetch
+        if (live && c * 64 + lane < zbits) ret[r * zbits + c * 64 + lane] = (_Float16)0.f;
+        return;
+    }
+    fetch(lane);
+    float acc = 0.f;
+    int buf = 0;
+    for (int64_t m0 = 0; m0 < n; m0 += 64, buf ^= 1) {
+        const int64_t m = m0 + lane;
+        const uint32_t keep = live && m < n ? 0xFFFFFFFFu : 0u;  // members past n: the zero word, nothing is added
+        const uint32_t clo = vlo & keep, chi = has_hi ? vhi & keep : 0u;
+        if (threadIdx.x < 64) wsh[buf][lane] = m < n ? (float)__builtin_bit_cast(_Float16, (uint16_t)wa) : 0.f;
+        // one barrier per chunk: a buffer is written again two chunks later, after every wave has passed the barrier
+        // of the chunk in between
+        __syncthreads();
+        fetch(m + 64);
 #pragma unroll 8
         for (int j = 0; j < 64; j++) {
-            const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)vlo, j);
-            const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)vhi, j);
+            const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)clo, j);
+            const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)chi, j);
             const uint64_t mask = ((uint64_t)hi << 32) | lo;
-            const float wm = wsh[j];
+            const float wm = wsh[buf][j];
             float t;
             asm("v_cndmask_b32_e64 %0, 0, %1, %2" : "=v"(t) : "v"(wm), "s"(mask));  // t = bit z of the word ? wm : 0
             acc += t;  // adding zero for a clear bit leaves the running sum unchanged
@@ -93,50 +110,58 @@ __global__ __launch_bounds__(256) void weighted_sum_line_kernel(_Float16 *__rest
     const int64_t stride = R * (int64_t)rowdw;  // dwords from one member's row to the next member's
     const uint32_t *p = in + r * rowdw + (int64_t)g * (2 * COLS);
     const int left = rowdw - g * (2 * COLS);    // dwords of the row from this piece on
-    const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
+    // The fetch is unconditional and what it brings is masked where it is used, a chunk later: a load whose result
+    // joins a zero from another path (a member past n, a dword past the row's end) gets moved out of the registers it
+    // arrives in, and the wait for it would then sit right behind the load instead of behind the chunk's arithmetic.
+    // Members past n read the last member's piece, dwords past the row's end the row's last dword; idle waves read
+    // row 0.  The weight stays fp16 until then for the same reason.  (Fetching two or four chunks ahead measured slower.)
     auto fetch = [&](uint4 &x, uint4 &y, int64_t m) {
-        const uint32_t *q = p + m * stride;
+        const uint32_t *q = p + (m < n ? m : n - 1) * stride;
         if (VEC) {
             x = load_stream16(q);
             if (COLS == 4) y = load_stream16(q + 4);
         } else {
             // plain loads: those of a lane share a cache line, which streaming loads would fetch once per load
+            const int last = left - 1;  // >= 0: a piece holds output bits
             x.x = q[0];
-            x.y = left > 1 ? q[1] : 0u;
-            x.z = left > 2 ? q[2] : 0u;
-            x.w = left > 3 ? q[3] : 0u;
+            x.y = q[last < 1 ? last : 1];
+            x.z = q[last < 2 ? last : 2];
+            x.w = q[last < 3 ? last : 3];
             if (COLS == 4) {
-                y.x = left > 4 ? q[4] : 0u;
-                y.y = left > 5 ? q[5] : 0u;
-                y.z = left > 6 ? q[6] : 0u;
-                y.w = left > 7 ? q[7] : 0u;
+                y.x = q[last < 4 ? last : 4];
+                y.y = q[last < 5 ? last : 5];
+                y.z = q[last < 6 ? last : 6];
+                y.w = q[last < 7 ? last : 7];
             }
         }
     };
+    // keep(k): the mask that dword k of the piece fetched for member m has to pass
+    auto keep = [&](int k, int64_t m) -> uint32_t { return (live && m < n && (VEC || k < left)) ? 0xFFFFFFFFu : 0u; };
     const uint32_t zz = lane & 31;
     const int half = lane >> 5;
     float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
-    uint4 a0 = zero, a1 = zero;  // members past n contribute zero words: nothing is added for them
-    float wa = 0.f;
-    if (live && lane < n) fetch(a0, a1, lane);
-    if (wv == 0 && lane < n) wa = (float)w[lane];
+    uint4 a0, a1 = make_uint4(0u, 0u, 0u, 0u);
+    const uint16_t *wr = reinterpret_cast<const uint16_t *>(w);
+    uint32_t wa;  // the weight's fp16 bits, as loaded
+    fetch(a0, a1, lane);
+    wa = wr[lane < n ? lane : n - 1];
     int buf = 0;
     for (int64_t m0 = 0; m0 < n; m0 += 64, buf ^= 1) {
+        const int64_t m = m0 + lane;
         if constexpr (COLS == 4) {
-            msk[buf][wv][0][lane] = make_uint4(a0.x, a0.z, a1.x, a1.z);
-            msk[buf][wv][1][lane] = make_uint4(a0.y, a0.w, a1.y, a1.w);
+            msk[buf][wv][0][lane] = make_uint4(a0.x & keep(0, m), a0.z & keep(2, m), a1.x & keep(4, m), a1.z & keep(6, m));
+            msk[buf][wv][1][lane] = make_uint4(a0.y & keep(1, m), a0.w & keep(3, m), a1.y & keep(5, m), a1.w & keep(7, m));
         } else {
-            msk[buf][wv][0][lane] = make_uint2(a0.x, a0.z);
-            msk[buf][wv][1][lane] = make_uint2(a0.y, a0.w);
+            msk[buf][wv][0][lane] = make_uint2(a0.x & keep(0, m), a0.z & keep(2, m));
+            msk[buf][wv][1][lane] = make_uint2(a0.y & keep(1, m), a0.w & keep(3, m));
         }
-        if (wv == 0) wsh[buf][lane] = wa;
+        if (wv == 0) wsh[buf][lane] = m < n ? (float)__builtin_bit_cast(_Float16, (uint16_t)wa) : 0.f;
         // one barrier per chunk: a buffer is written again two chunks later, after every wave has passed the barrier
         // of the chunk in between and so has finished reading it
         __syncthreads();
-        a0 = a1 = zero;
-        wa = 0.f;
-        if (live && m0 + 64 + lane < n) fetch(a0, a1, m0 + 64 + lane);
-        if (wv == 0 && m0 + 64 + lane < n) wa = (float)w[m0 + 64 + lane];
+        // the next chunk, always (past n: the last member's piece again, masked when used)
+        fetch(a0, a1, m + 64);
+        wa = wr[m + 64 < n ? m + 64 : n - 1];
         const half_t *mine = &msk[buf][wv][half][0];
 #pragma unroll 8
         for (int j = 0; j < 64; j++) {

@@ -446,7 +446,9 @@ def test_weighted_sum_vs_oracle(ops, oracle, dtype):
                     # rows without a tail bit (a conv layer's one- and two-word taps): summed as one long row
                     (130, 5000, 64), (40, 4500, 128), (33, 4099, 64), (70, 600, 64),
                     # outputs of 1024 to 2047 16-byte pieces: a wave per two columns (whole pieces, rows of 9 words, ragged)
-                    (70, 2304, 64), (50, 300, 576), (37, 260, 520)]:
+                    (70, 2304, 64), (50, 300, 576), (37, 260, 520),
+                    # no members: zeros
+                    (0, 3, 100), (0, 2, 4096)]:
         nd = NDT[dtype]
         wb = np.dtype(nd).itemsize * 8
         words = rand_words(g, (n, R, (C + wb - 1) // wb), nd)
