@@ -39,6 +39,9 @@ __global__ __launch_bounds__(256) void bn_colsum_kernel(unsigned long long *__re
     const int64_t z0 = (int64_t)blockIdx.y * kBnChunk;
     const int64_t z1 = z0 + kBnChunk < Z ? z0 + kBnChunk : Z;
     unsigned long long s = 0;
+    // unrolled: the loads of sixteen members are in flight together (with few columns a workgroup has few lanes at
+    // work and nothing else hides their round trips)
+#pragma unroll 16
     for (int64_t z = z0; z < z1; z++) {
         const int32_t pc = popc[z * M + m];
         if (ROUND)
