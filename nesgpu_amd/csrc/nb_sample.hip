@@ -226,6 +226,7 @@ __global__ __launch_bounds__(256) void sample_narrow_kernel(W *__restrict__ out,
                     // whole generator blocks: four columns per block, their thresholds in one 16-byte load (the rows
                     // of neighbouring lanes lie C words apart: single loads would touch a cache line per lane and word)
                     const uint4 *__restrict__ tq = reinterpret_cast<const uint4 *>(tr);
+#pragma unroll 4  // four blocks' thresholds asked for together
                     for (int k = 0; k < (C >> 2); k++) {
                         const uint4 b = philox_block(src.key, (g0 >> 2) + (uint64_t)k);
                         const uint4 t = tr ? tq[k] : make_uint4(ts, ts, ts, ts);
