@@ -82,7 +82,9 @@ int nb_bmv_act_pack_i32(int32_t *out, const int32_t *A, const int32_t *x, const 
 /* ---- linear layer with the population-mean threshold --------------------------------------------------
  * BinarizedLinear(batch_norm=True) in one call: with popc[z,m] = sum_k popcount(A[z,m,k] ^ x[z,k]) and
  * act = 2*popc - K,
- *     mean[m]  = fp16( float(sum_z act[z,m]) / float(Z) )       (the sum is exact integer arithmetic)
+ *     mean[m]  = fp16( float(sum_z act[z,m]) * (float(M) / float(Z*M)) )   (the sum is exact integer arithmetic; the
+ *                factor is what torch's fp16 mean multiplies its fp32 sum by: the quotient of the element counts;
+ *                the exact product is rounded once, to fp16, as torch's kernel does)
  *     thr[z,m] = fp16( fp16(bias[m] + bias_noise[z,m]) + mean[m] )
  *     bit[z,m] = act[z,m] > thr[z,m]                            (compared exactly; false for a NaN threshold)
  * A [Z,M,Kw], x [Z,Kw], bias [M] fp16, bias_noise [Z,M] fp16 (raw 16-bit patterns), K = true bit count of a row.
@@ -93,7 +95,7 @@ int nb_bmv_act_pack_i32(int32_t *out, const int32_t *A, const int32_t *x, const 
  * sums and the per-output totals pass through it; contents undefined afterwards).  The weights are read once.
  *   replaces the composition of modules/binary.py:97-102 (bmm -> 2*popc - in_features -> .type(float16).mean(dim=0)
  *   -> thresh -> compare); equal to it wherever act is exact in fp16 (K <= 2048), or with pack bit 1 set, and torch's
- *   fp32 sum over the population is exact (Z * K <= 2^24) and Z is a power of two (torch multiplies by 1 / Z). */
+ *   fp32 sum over the population is exact (Z * K < 2^24); beyond that torch's sum depends on its summation order. */
 int64_t nb_bmv_bn_workspace_bytes(int64_t Z, int64_t M);
 int nb_bmv_bn_act_i64(void *out, const int64_t *A, const int64_t *x, const uint16_t *bias, const uint16_t *bias_noise,
                       int64_t Z, int64_t M, int64_t Kw, int64_t K, int pack, void *workspace, int64_t workspace_bytes,
@@ -115,7 +117,9 @@ int nb_bmv_bn_act_static_i64(void *out, const int64_t *A, const int64_t *x, cons
 
 /* Thresholds of BinarizedConv2d(batch_norm=True) (modules/binary.py:147-155) from the pixel sums that
  * nb_conv_popc_sums_* returns: with act = 2*popc - K over the HW output pixels,
- *     mean[d,o] = fp16(float(sum_pixels act) / float(HW)),  thr = fp16(fp16(bias[o] + bias_noise[d,o]) + mean),
+ *     mean[d,o] = fp16(float(sum_pixels act) * (float(D*O) / float(D*O*HW)))   (the exact product rounded once: torch's
+ *                 fp16 mean of a [D,h,w,O] map over its pixels wherever the fp32 sum is exact, K * HW <= 2^24),
+ *     thr = fp16(fp16(bias[o] + bias_noise[d,o]) + mean),
  *     thresh[d,o] = floor(thr) + K  (int32, clamped; INT32_MAX for NaN),
  * so that nb_conv_act*(..., thresh, ...) (2*popc > thresh) decides act > thr exactly as long as the activations are
  * integers that fp16 holds exactly (K <= 2048).  sums, thresh int32 [D,O]; bias fp16 [O]; bias_noise fp16 [D,O].
@@ -143,67 +147,90 @@ int nb_conv_bn_thresholds_from_input_i32(int32_t *thresh, const int32_t *in, con
  * 32-bit words with an even count has the same bytes).  No counterpart in the reference, whose linear layer always
  * streams materialised weights (modules/binary.py:97).
  *
- * Flip lists ("sorted slices"): perm[d, :] lists member d's rows so that every run of 64 (a slice) lies inside one
- * block of 1024 rows (the builder orders each block by flip count); slice (d, s) owns slice_len[d, s] 16-byte pieces
- * per lane, piece j of lane l at dword offset slice_off[d, s] + (j * 64 + l) * 4 of entries (slice_off a multiple of
- * 4, entries 16-byte aligned): the flips 8j .. 8j+7 of row perm[d, 64 s + l] in column order (low half of a dword
- * first), 16 bits each: [4:0] = column % 32, [15:5] = 2 * (column / 32) + b with b the base bit at that column;
- * past a row's end the sentinel (4Kw) << 5.  Kw <= 511, R <= 65536.
+ * Flip lists ("fixed slices"): with S = ceil(R / 64) and a capacity of `cap` 16-byte pieces per row, piece j of row
+ * r of member d sits at dword offset (((d * S + r / 64) * cap + j) * 64 + r % 64) * 4 of entries (16-byte aligned,
+ * D * S * cap * 256 dwords): the row's flips 8j .. 8j+7 in column order (low half of a dword first), 16 bits each:
+ * [4:0] = column % 32, [15:5] = 2 * (column / 32) + b with b the base bit at that column; the last piece is padded
+ * with the sentinel (4Kw) << 5, which may also stand between flips.  info[d, r] (uint32) = flips | pieces << 16: only the
+ * first `pieces` pieces of a row are ever written or read.  Every row has a fixed place, so lists are written in one
+ * pass, in any order, without a count first.  A row that needs more than cap pieces keeps its first 8 * cap flips and
+ * adds one to overflow[0] (uint32, device memory, cleared by the caller): check it when convenient, choose a larger
+ * cap and draw again.  Kw <= 511, R <= 65536, cap <= 8191.
  *
- * nb_flip_count: cnt[d, r] = popcount(W[d, r, :] ^ base[r, :]) (uint16); W [D, R, Kw], base [R, Kw].
- * nb_flip_fill:  writes the entries of every slice from W ^ base, given perm, slice_off (in dwords) and slice_len
- *                (pieces per lane, at least ceil(max count in the slice / 8)); never writes past a slice.
- * nb_flip_layout: perm [D, R] (uint16) and slice_len [D, ceil(R/64)] from cnt [D, R]: inside every block of 1024
- *                rows the rows in the order of their counts (equal counts in row order), slice_len = ceil(count of
- *                the slice's last row / 8); slice_off [D, ceil(R/64)] (int64) = the running sum of slice_len * 256
- *                dwords before each slice, total[0] (int64, device memory) = the dwords of all slices: what the
- *                caller reads back to size entries.  slice_len 16-byte aligned.
+ * nb_flip_count: info[d, r] = popcount(W[d, r, :] ^ base[r, :]) | ceil(that / 8) << 16; W [D, R, Kw], base [R, Kw].
+ * nb_flip_fill:  the entries and info of every row from W ^ base.
  * nb_expand_fp4: packed rows [rows, Kw] -> FP4 (E2M1) codes [rows_padded, 32 * Kw_padded] bytes, bit 1 -> +1.0,
  *                bit 0 -> -1.0, padding -> 0.0: the operand form of nb_bmm_nt_fp4.
  * nb_bmm_nt_fp4: C[m, n] = popcount(A_m ^ B_n), int32 [M, N], for two expanded operands (rows padded to multiples of
  *                128, Kw_padded even); the shared-base form of the product of extensions/src/bmm.cu:5-58 on the matrix
  *                cores (FP4 MFMA, exact for +-1).
- * nb_bmv_flip:   out[d, r] = G[d, r] + cnt[d, r] - 2 * (number of member d's flips in row r whose looked-up bit is
+ * nb_bmv_flip:   out[d, r] = G[d, r] + flips(d, r) - 2 * (number of member d's flips in row r whose looked-up bit is
  *                set), int32 [D, R], with G = nb_bmm_nt_fp4(x, base): equal to nb_bmm_i64(W, x) with N = 1.
  * nb_bmv_flip_act_pack: the same sums thresholded (2 * sum > thresh[d, r]) and packed along r into
  *                [D, ceil(R/64)] words: equal to nb_bmv_act_pack_i64(W, x, thresh).
- *
- * Skip sampler (generator mode of the flip form): for a uniform flip probability the flipped columns of a row are a
- * renewal process with geometric gaps, so the lists can be drawn directly, about C*p + 1 random words per row instead
- * of the C words of the per-bit compare.  Row q = d*R + r reads the Philox4x32-10 words first + q*C + i, i = 0, 1, ...
- * (stream (seed, subseq), as nb_philox_words numbers them); word i has the rank #{k < Kt : cdf[k] <= word}: a rank
- * below Kt moves the position (start: -1) on by rank + 1 columns and flips the column reached, rank Kt moves it on by
- * Kt columns without a flip; the row ends when the position passes C.  cdf [Kt] uint32, sorted, Kt <= 4096, is
- * supplied by the caller: cdf[k-1] = floor(2^32 * (1 - (1-p)^k)); Kt == 0 means no flips.  cdf0 = the table's first
- * entry (p * 2^32) as a host value: a hint for where a look-up starts probing; it does not change any result.  Same law as
- * nb_sample_philox with a base and thr_scalar = p * 2^32 (i.i.d. Bernoulli(p), quantised to 2^-32), another stream.
- * nb_flip_skip_count: cnt[d, r] = number of flips of the row.   nb_flip_skip_fill: the entries, as nb_flip_fill.
  * nb_flip_to_dense: materialises flip lists: W [D, R, Kw] must hold base in every member on entry, every listed
- *                flip is XOR-ed in (interop with the dense kernels, and what the tests compare through). */
-int nb_flip_layout(uint16_t *perm, int32_t *slice_len, int64_t *slice_off, int64_t *total, const uint16_t *cnt, int64_t D,
-                   int64_t R, nb_stream_t stream);
-int nb_flip_skip_count_i64(uint16_t *cnt, const uint32_t *cdf, uint32_t cdf0, int64_t Kt, uint64_t seed, uint64_t subseq,
-                           uint64_t first, int64_t D, int64_t R, int64_t C, nb_stream_t stream);
-int nb_flip_skip_fill_i64(uint32_t *entries, const int64_t *base, const uint16_t *perm, const int64_t *slice_off,
-                          const int32_t *slice_len, const uint32_t *cdf, uint32_t cdf0, int64_t Kt, uint64_t seed,
-                          uint64_t subseq, uint64_t first, int64_t D, int64_t R, int64_t C, nb_stream_t stream);
-int nb_flip_to_dense_i64(int64_t *W, const uint32_t *entries, const int64_t *slice_off, const int32_t *slice_len,
-                         const uint16_t *perm, int64_t D, int64_t R, int64_t Kw, nb_stream_t stream);
-int nb_flip_count_i64(uint16_t *cnt, const int64_t *W, const int64_t *base, int64_t D, int64_t R, int64_t Kw,
-                      nb_stream_t stream);
-int nb_flip_fill_i64(uint32_t *entries, const int64_t *W, const int64_t *base, const uint16_t *perm,
-                     const int64_t *slice_off, const int32_t *slice_len, int64_t D, int64_t R, int64_t Kw,
+ *                flip is XOR-ed in (interop with the dense kernels, and what the tests compare through).
+ * nb_flip_weighted_sum: out[r, c] (fp16 [R, C]) = sum_d weights[d] * bit_d[r, c] with bit = base ^ flip, i.e.
+ *                base[r, c] * sum_d weights[d] +- the weights of the members that flip (r, c): what
+ *                nb_weighted_sum_i64 gives on the materialised weights (extensions/src/weighted_sum.cu:28-46, the
+ *                update step of modules/binary.py:70), up to the order of the additions: the weights are scaled by a
+ *                power of two to 32-bit integers (sum |w| * scale < 2^29) and added exactly, in any order.
+ *
+ * Skip sampler (generator mode of the flip form): the flipped columns of a row are a renewal process with geometric
+ * gaps, so the lists can be drawn directly, about C*p + 1 random words per row instead of the C words of the per-bit
+ * compare.  Row q = d*R + r reads the Philox4x32-10 words first + q*C + i, i = 0, 1, ... (stream (seed, subseq), as
+ * nb_philox_words numbers them); a word has the rank #{k < Kt : cdf[k] <= word}: a rank below Kt moves the position
+ * (start: -1) on by rank + 1 columns and flips the column reached, rank Kt moves it on by Kt columns without a flip;
+ * the row ends when the position passes C.  The table is device memory of nb_skip_table_words() uint32: [0] = Kt
+ * (<= 4096), [1] = the bits of the float 1 / log2(1 - p) (a hint for where a look-up starts probing; it changes no
+ * result), [2] = the threshold p * 2^32, [3] = 0, [4 + k] = cdf[k] = floor(2^32 * (1 - (1-p)^(k+1))), sorted; Kt == 0
+ * means no flips.  Written by the caller, or by nb_skip_table from a threshold in device memory (which may be
+ * table + 2).  Same law as nb_sample_philox with a base and thr_scalar = p * 2^32 (i.i.d. Bernoulli(p), quantised to
+ * 2^-32), another stream.  One kernel, nothing read back: the call can be captured into a HIP graph.
+ * nb_flip_skip: lists with a uniform flip probability against base [R, Kw].
+ * nb_flip_skip_thin: per-element probabilities by thinning.  law [R, C] uint16: bit 15 = the base bit of the column,
+ *                bits 14:0 = the fp16 pattern of its flip probability y <= 1/2, Tf = floor(y * 2^32); table: made for
+ *                the largest Tf of the layer (T_max = table[2]).  The words of a row come in pairs: word 2i is a gap as
+ *                above, and the column it reaches flips only if word 2i+1 times T_max is below Tf * 2^32 (64-bit
+ *                integers): each column flips with probability Tf / 2^32, independently.
+ * The layers' law (modules/binary.py:59-60), P = sigmoid(5 w / (mean|w| + 1e-5)), rounded to fp16 wherever the tensor
+ * expression rounds; mean|w| = the exact sum over the count, rounded once to fp16.  workspace: nb_law_workspace_bytes()
+ * bytes of device memory, 8-byte aligned.
+ * nb_thresholds_from_weights: thresholds[i] = min(floor(P_i * 2^32), 2^32 - 1), what nb_sample_philox takes.
+ * nb_probabilities_from_weights: the fp16 probabilities themselves.
+ * nb_flip_law_from_weights: the sparse form of the same law: law [R, C] as nb_flip_skip_thin takes it (base bit =
+ *                P >= 1/2, y = min(P, 1 - P)), base [R, Kw] packed, and table made for the layer's largest Tf. */
+int64_t nb_skip_table_words(void);
+int nb_skip_table(uint32_t *table, const uint32_t *threshold, nb_stream_t stream);
+int nb_flip_skip_i64(uint32_t *entries, uint32_t *info, uint32_t *overflow, const int64_t *base, const uint32_t *table,
+                     uint64_t seed, uint64_t subseq, uint64_t first, int64_t D, int64_t R, int64_t C, int64_t cap,
                      nb_stream_t stream);
+int nb_flip_skip_thin_i64(uint32_t *entries, uint32_t *info, uint32_t *overflow, const uint16_t *law,
+                          const uint32_t *table, uint64_t seed, uint64_t subseq, uint64_t first, int64_t D, int64_t R,
+                          int64_t C, int64_t cap, nb_stream_t stream);
+int64_t nb_law_workspace_bytes(void);
+int nb_thresholds_from_weights(uint32_t *thresholds, const uint16_t *weights, int64_t n, void *workspace,
+                               nb_stream_t stream);
+int nb_probabilities_from_weights(uint16_t *p, const uint16_t *weights, int64_t n, void *workspace, nb_stream_t stream);
+int nb_flip_law_from_weights(uint16_t *law, int64_t *base, uint32_t *table, const uint16_t *weights, int64_t R, int64_t C,
+                             void *workspace, nb_stream_t stream);
+int nb_flip_to_dense_i64(int64_t *W, const uint32_t *entries, const uint32_t *info, int64_t D, int64_t R, int64_t Kw,
+                         int64_t cap, nb_stream_t stream);
+int nb_flip_count_i64(uint32_t *info, const int64_t *W, const int64_t *base, int64_t D, int64_t R, int64_t Kw,
+                      nb_stream_t stream);
+int nb_flip_fill_i64(uint32_t *entries, uint32_t *info, uint32_t *overflow, const int64_t *W, const int64_t *base,
+                     int64_t D, int64_t R, int64_t Kw, int64_t cap, nb_stream_t stream);
 int nb_expand_fp4_i64(uint8_t *out, const int64_t *in, int64_t rows, int64_t Kw, int64_t rows_padded, int64_t Kw_padded,
                       nb_stream_t stream);
 int nb_bmm_nt_fp4(int32_t *C, const uint8_t *A, const uint8_t *B, int64_t M, int64_t N, int64_t Kw, int64_t M_padded,
                   int64_t N_padded, int64_t Kw_padded, nb_stream_t stream);
-int nb_bmv_flip_i64(int32_t *out, const int32_t *G, const uint32_t *entries, const int64_t *slice_off,
-                    const int32_t *slice_len, const uint16_t *perm, const uint16_t *cnt, const int64_t *x, int64_t D,
-                    int64_t R, int64_t Kw, nb_stream_t stream);
-int nb_bmv_flip_act_pack_i64(int64_t *out, const int32_t *G, const uint32_t *entries, const int64_t *slice_off,
-                             const int32_t *slice_len, const uint16_t *perm, const uint16_t *cnt, const int64_t *x,
-                             const int32_t *thresh, int64_t D, int64_t R, int64_t Kw, nb_stream_t stream);
+int nb_bmv_flip_i64(int32_t *out, const int32_t *G, const uint32_t *entries, const uint32_t *info, const int64_t *x,
+                    int64_t D, int64_t R, int64_t Kw, int64_t cap, nb_stream_t stream);
+int nb_bmv_flip_act_pack_i64(int64_t *out, const int32_t *G, const uint32_t *entries, const uint32_t *info,
+                             const int64_t *x, const int32_t *thresh, int64_t D, int64_t R, int64_t Kw, int64_t cap,
+                             nb_stream_t stream);
+int nb_flip_weighted_sum_i64(uint16_t *out, const uint32_t *entries, const uint32_t *info, const int64_t *base,
+                             const uint16_t *weights, int64_t D, int64_t R, int64_t C, int64_t cap, nb_stream_t stream);
 
 /* ---- packed im2col / conv -----------------------------------------------------------------
  * Geometry: input [D,H,W,Cw] (channels-last packed), fx taps along H, fy taps along W,

@@ -49,15 +49,19 @@ _PLAIN = {
     "nb_conv_engine": [_I32],
     "nb_conv_last_engine": [],
     "nb_flip_count_i64": [_PTR, _PTR, _PTR, _I64, _I64, _I64, _PTR],
-    "nb_flip_fill_i64": [_PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _I64, _I64, _I64, _PTR],
-    "nb_flip_layout": [_PTR, _PTR, _PTR, _PTR, _PTR, _I64, _I64, _PTR],
-    "nb_flip_skip_count_i64": [_PTR, _PTR, _U32, _I64, _U64, _U64, _U64, _I64, _I64, _I64, _PTR],
-    "nb_flip_skip_fill_i64": [_PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _U32, _I64, _U64, _U64, _U64, _I64, _I64, _I64, _PTR],
-    "nb_flip_to_dense_i64": [_PTR, _PTR, _PTR, _PTR, _PTR, _I64, _I64, _I64, _PTR],
+    "nb_flip_fill_i64": [_PTR, _PTR, _PTR, _PTR, _PTR, _I64, _I64, _I64, _I64, _PTR],
+    "nb_flip_to_dense_i64": [_PTR, _PTR, _PTR, _I64, _I64, _I64, _I64, _PTR],
+    "nb_skip_table": [_PTR, _PTR, _PTR],
+    "nb_flip_skip_i64": [_PTR, _PTR, _PTR, _PTR, _PTR, _U64, _U64, _U64, _I64, _I64, _I64, _I64, _PTR],
+    "nb_flip_skip_thin_i64": [_PTR, _PTR, _PTR, _PTR, _PTR, _U64, _U64, _U64, _I64, _I64, _I64, _I64, _PTR],
+    "nb_thresholds_from_weights": [_PTR, _PTR, _I64, _PTR, _PTR],
+    "nb_probabilities_from_weights": [_PTR, _PTR, _I64, _PTR, _PTR],
+    "nb_flip_law_from_weights": [_PTR, _PTR, _PTR, _PTR, _I64, _I64, _PTR, _PTR],
     "nb_expand_fp4_i64": [_PTR, _PTR, _I64, _I64, _I64, _I64, _PTR],
     "nb_bmm_nt_fp4": [_PTR, _PTR, _PTR, _I64, _I64, _I64, _I64, _I64, _I64, _PTR],
-    "nb_bmv_flip_i64": [_PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _I64, _I64, _I64, _PTR],
-    "nb_bmv_flip_act_pack_i64": [_PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _I64, _I64, _I64, _PTR],
+    "nb_bmv_flip_i64": [_PTR, _PTR, _PTR, _PTR, _PTR, _I64, _I64, _I64, _I64, _PTR],
+    "nb_bmv_flip_act_pack_i64": [_PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _I64, _I64, _I64, _I64, _PTR],
+    "nb_flip_weighted_sum_i64": [_PTR, _PTR, _PTR, _PTR, _PTR, _I64, _I64, _I64, _I64, _PTR],
     "nb_bmv_bn_act_static_i64": [_PTR, _PTR, _PTR, _PTR, _PTR, _I64, _I64, _I64, _I64, _I32, _PTR],
     "nb_conv_bn_thresholds": [_PTR, _PTR, _PTR, _PTR, _I64, _I64, _I64, _I64, _PTR],
 }
@@ -65,6 +69,8 @@ _PLAIN = {
 _SIZES = {
     "nb_bmv_bn_workspace_bytes": [_I64, _I64],
     "nb_bmv_bn_static_bytes": [],
+    "nb_skip_table_words": [],
+    "nb_law_workspace_bytes": [],
 }
 
 

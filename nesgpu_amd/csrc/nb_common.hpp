@@ -116,6 +116,9 @@ __device__ __forceinline__ uint32_t philox_word(const PhiloxKey &key, uint64_t g
     return e == 0 ? b.x : e == 1 ? b.y : e == 2 ? b.z : b.w;
 }
 
+// Flip lists of the sparse linear form: what info[d, r] holds for a row with `flips` entries in `pieces` 16-byte pieces
+__host__ __device__ __forceinline__ uint32_t flip_info(uint32_t flips, uint32_t pieces) { return flips | (pieces << 16); }
+
 // Block-uniform stride loop over a flat index space: every thread of a workgroup runs the same number of
 // iterations (so wave-level collectives inside the body are safe); `T` may be >= TOTAL on the last one.
 #define NB_FLAT_LOOP(T, TOTAL)                                                                            \

@@ -102,15 +102,42 @@ bool conv_sums_count_try(int32_t *out, const uint64_t *in, const uint64_t *filt,
                          int tap_bits, hipStream_t s, const _Float16 *bias = nullptr, const _Float16 *noise = nullptr,
                          int64_t K = 0);
 
+// What torch's mean over `in_elems` elements reduced to `out_elems` results multiplies its fp32 sums by: the quotient of
+// the two counts, each converted to fp32 first.
+inline float mean_factor(int64_t out_elems, int64_t in_elems) { return (float)out_elems / (float)in_elems; }
+
+// A double rounded ONCE to fp16: brought to fp32 with round-to-odd (an inexact result keeps a set last bit), after
+// which the rounding to fp16 is the one of the exact value.
+__device__ __forceinline__ _Float16 double_round_once_fp16(double p)
+{
+    float r = (float)p;
+    if ((double)r != p) {
+        uint32_t u = __float_as_uint(r);
+        if (fabs((double)r) > fabs(p)) u -= 1u;  // towards zero (r is not zero here: |r| > |p| > 0)
+        r = __uint_as_float(u | 1u);
+    }
+    return (_Float16)r;
+}
+
+// fp16(a * b) with one rounding, which is what torch's fp16 mean does with its fp32 sum and that factor (its kernel
+// converts the product straight to fp16); the product of two floats is exact in a double.  Written out so that the
+// result does not depend on which instructions the compiler picks for `(_Float16)(a * b)`.
+__device__ __forceinline__ _Float16 mul_round_once_fp16(float a, float b)
+{
+    return double_round_once_fp16((double)a * (double)b);
+}
+
 // Threshold of BinarizedConv2d(batch_norm=True) for one (member, channel) from the sum of its popcount map over the HW
-// output pixels (modules/binary.py:147-155): act = 2*popc - K, mean = fp16(float(sum of act) / float(HW)),
-// thr = fp16(fp16(bias + noise) + mean); act > thr  <=>  2*popc > floor(thr) + K, which is what is returned (clamped to
-// int32; INT32_MAX, never exceeded, for NaN).
+// output pixels (modules/binary.py:147-155): act = 2*popc - K, mean = fp16(float(sum of act) * factor), rounded once,
+// with factor = mean_factor(D * O, D * O * HW) (torch's fp16 mean: fp32 sum times that quotient; the same number
+// whenever the fp32 sum is exact, i.e. up to 2^24 in magnitude), thr = fp16(fp16(bias + noise) + mean);
+// act > thr  <=>  2*popc > floor(thr) + K, which is what is returned (clamped to int32; INT32_MAX, never exceeded,
+// for NaN).
 __device__ __forceinline__ int32_t bn_conv_threshold(long long popc_sum, _Float16 bias, _Float16 noise, long long K,
-                                                     long long HW)
+                                                     long long HW, float factor)
 {
     const long long sum_act = 2ll * popc_sum - K * HW;
-    const _Float16 mean = (_Float16)((float)sum_act / (float)HW);
+    const _Float16 mean = mul_round_once_fp16((float)sum_act, factor);
     const _Float16 tb = bias + noise;
     const float v = (float)(_Float16)(tb + mean);
     if (v != v) return 2147483647;

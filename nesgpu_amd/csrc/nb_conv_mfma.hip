@@ -390,12 +390,15 @@ __global__ __launch_bounds__(64 * (rw_cwaves(CPR, NT) + kRwPWaves)) void conv_mf
                         constexpr int G = P == 1 ? 5 : 2;  // items per batch: kRwItems is a multiple of both
                         unsigned char *dst = img + __mul24(ttid, p.PS);
                         const int dstep = kRwTeam * p.PS;
+                        // input bits above the channel count count for nothing (the positions they would take stand
+                        // for the zero tail)
+                        const uint32_t inmask = p.in_bits >= 32 ? 0xFFFFFFFFu : (1u << p.in_bits) - 1u;
 #pragma unroll
                         for (int u0 = 0; u0 < kRwItems; u0 += G) {
                             uint4 e[G][P];
 #pragma unroll
                             for (int v = 0; v < G; v++) {
-                                const uint32_t lo = (uint32_t)wd[u0 + v];
+                                const uint32_t lo = (uint32_t)wd[u0 + v] & inmask;
 #pragma unroll
                                 for (int c = 0; c < P; c++) e[v][c] = expand_half(lo, c);
                             }

@@ -40,6 +40,7 @@ struct CsConv {
     int tap_bits, tapT, fwords;  // tap-packed filters: bits per tap, taps per word, filter words per channel
     const _Float16 *bias, *noise;  // not null: write the batch-norm layer's thresholds instead of the sums
     long long K;
+    float mean_factor;  // what the fp32 sum of a (member, channel)'s activations is multiplied by for its mean
 };
 
 // F: the largest filter extent the instance is built for (3 or kCsMaxF); the per-tap code is spelled out F x F times
@@ -192,7 +193,8 @@ __global__ __launch_bounds__(256) void conv_sums_count_kernel(const CsConv p)
         // bit planes of the counts: plane k of (tap, cw) is the ballot of bit k over the 64 channel bits; the ballots
         // of a tap are handed to lanes 0 .. nplanes-1 and stored together
         for (int t = wv; t < p.taps; t += 4) {
-            const int v = n1[t * 64 + lane];
+            // tap-packed filters only see the channel bits: input bits above them count for nothing, as in the conv kernels
+            const int v = (p.tap_bits && lane >= p.tap_bits) ? 0 : n1[t * 64 + lane];
             int a = 0;
             uint32_t lo = 0, hi = 0;
 #define NB_CS_PLANE(K)                                    \
@@ -253,7 +255,7 @@ __global__ __launch_bounds__(256) void conv_sums_count_kernel(const CsConv p)
         __syncthreads();
         for (int i = threadIdx.x; i < oc; i += 256) {
             const int64_t at = d * p.O + o0 + i;
-            p.out[at] = p.bias ? bn_conv_threshold(osum[i], p.bias[o0 + i], p.noise[at], p.K, p.hw) : osum[i];
+            p.out[at] = p.bias ? bn_conv_threshold(osum[i], p.bias[o0 + i], p.noise[at], p.K, p.hw, p.mean_factor) : osum[i];
         }
         __syncthreads();
     }
@@ -283,6 +285,7 @@ bool conv_sums_count_try(int32_t *out, const uint64_t *in, const uint64_t *filt,
     p.chan_chunk = O < kCsChanChunk ? O : kCsChanChunk;
     p.n1_ints = taps * 64 > p.chan_chunk ? taps * 64 : p.chan_chunk;
     p.hw = (int)hw;
+    p.mean_factor = mean_factor(D * O, D * O * hw);
     p.nplanes = 1;
     while ((1LL << p.nplanes) <= hw) p.nplanes++;
     p.tap_bits = tap_bits;

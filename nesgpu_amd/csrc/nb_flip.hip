@@ -16,7 +16,9 @@
 // their complements in LDS (piece, ~piece, piece, ~piece ...: 4Kw dwords, then one zero dword for the sentinel 4Kw),
 // so that the looked-up bit already is x ^ b.  The rows of a slice move through the columns at about the same pace,
 // so at any moment the 64 lanes look into a narrow window of the table: neighbouring dwords, different banks.
+#include <algorithm>
 #include <cmath>
+#include <mutex>
 #include <type_traits>
 
 #include "nb_common.hpp"
@@ -180,8 +182,14 @@ __global__ __launch_bounds__(256) void fl_gemm_fp4_kernel(int32_t *__restrict__ 
             }
 }
 
-// ---- flip counts: cnt[d, r] = popcount(W[d, r, :] ^ base[r, :]), sixteen lanes per row ---------------------------
-__global__ __launch_bounds__(256) void fl_count_kernel(uint16_t *__restrict__ cnt, const uint64_t *__restrict__ W,
+// ---- flip lists ("fixed slices") -----------------------------------------------------------------------------------
+// Slice (d, s) = rows 64 s .. 64 s + 63 of member d owns `cap` 16-byte pieces per lane at entries + ((d * S + s) * cap
+// + j) * 256 + 4 * l dwords (piece j of lane l = row 64 s + l): the row's flips 8j .. 8j+7 in column order, the last
+// piece padded with sentinels.  info[d, r] = flips | pieces << 16: only the first `pieces` pieces of a row's lane were
+// written, and nothing else of the lane is ever read.  Every slice sits at a fixed place, so lists can be written in
+// one pass, by rows in any order, without knowing the other rows' lengths.
+// info[d, r] from materialised weights: popcount(W[d, r, :] ^ base[r, :]), sixteen lanes per row
+__global__ __launch_bounds__(256) void fl_count_kernel(uint32_t *__restrict__ info, const uint64_t *__restrict__ W,
                                                        const uint64_t *__restrict__ base, int64_t rows, int64_t R,
                                                        int Kw)
 {
@@ -197,251 +205,49 @@ __global__ __launch_bounds__(256) void fl_count_kernel(uint16_t *__restrict__ cn
     acc += __shfl_xor(acc, 4);
     acc += __shfl_xor(acc, 2);
     acc += __shfl_xor(acc, 1);
-    if (live && sub == 0) cnt[row] = (uint16_t)acc;
+    if (live && sub == 0) info[row] = flip_info((uint32_t)acc, (uint32_t)(acc + 7) >> 3);
 }
 
-// ---- flip lists: one wave per slice, lane l walks the row perm[d, 64 s + l] ---------------------------------------
-__global__ __launch_bounds__(256) void fl_fill_kernel(uint32_t *__restrict__ entries, const uint64_t *__restrict__ W,
-                                                      const uint64_t *__restrict__ base,
-                                                      const uint16_t *__restrict__ perm,
-                                                      const int64_t *__restrict__ slice_off,
-                                                      const int32_t *__restrict__ slice_len, int64_t nslices, int S,
-                                                      int64_t R, int Kw)
+// the lists from materialised weights: one wave per slice, lane l walks row 64 s + l.  A row with more flips than
+// cap * 8 keeps its first cap * 8 and is counted in overflow[0].
+__global__ __launch_bounds__(256) void fl_fill_kernel(uint32_t *__restrict__ entries, uint32_t *__restrict__ info,
+                                                      uint32_t *__restrict__ overflow, const uint64_t *__restrict__ W,
+                                                      const uint64_t *__restrict__ base, int64_t nslices, int S,
+                                                      int64_t R, int Kw, int cap)
 {
     const int lane = threadIdx.x & 63;
     const int64_t sl = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (sl >= nslices) return;
     const int64_t d = sl / S;
     const int s = (int)(sl - d * S);
-    const int64_t p = (int64_t)s * 64 + lane;
-    const bool valid = p < R;
-    int64_t r = valid ? perm[d * R + p] : 0;
-    r = r < R ? r : R - 1;
-    const int L = 4 * slice_len[sl];  // dwords per lane; dword j of lane l sits at piece j / 4, component j % 4
-    uint4 *dst = reinterpret_cast<uint4 *>(entries + slice_off[sl]) + lane;
+    const int64_t r = (int64_t)s * 64 + lane;
+    if (r >= R) return;
+    uint4 *dst = reinterpret_cast<uint4 *>(entries) + sl * (int64_t)cap * 64 + lane;
     const uint32_t sentinel = (uint32_t)(4 * Kw) << 5;
-    int j = 0;
+    const int limit = 4 * cap;  // dwords of a lane
+    int j = 0, n = 0;
     uint32_t pend = 0;
     bool half = false;
-    // a lane's dwords leave four at a time, as whole 16-byte pieces (L is a multiple of 4); never past the slice,
-    // whatever the inputs
     uint32_t q0 = 0, q1 = 0, q2 = 0;
-    auto put = [&](uint32_t v) {
+    auto put = [&](uint32_t v) {  // a lane's dwords leave four at a time, as whole pieces; never past the lane's share
         const int c = j & 3;
         if (c == 0) q0 = v;
         else if (c == 1) q1 = v;
         else if (c == 2) q2 = v;
-        else if (j < L) dst[(int64_t)(j >> 2) * 64] = make_uint4(q0, q1, q2, v);
+        else if (j < limit) dst[(int64_t)(j >> 2) * 64] = make_uint4(q0, q1, q2, v);
         j++;
     };
-    if (valid) {
-        const uint64_t *w = W + (d * R + r) * Kw, *b = base + r * Kw;
-        for (int k = 0; k < Kw; k++) {
-            const uint64_t bw = b[k];
-            uint64_t m = w[k] ^ bw;
-            while (m) {
-                const int bit = __builtin_ctzll(m);
-                m &= m - 1;
-                const uint32_t col = (uint32_t)k * 64u + (uint32_t)bit;
-                const uint32_t bb = (uint32_t)(bw >> bit) & 1u;
-                const uint32_t e = ((2u * (col >> 5) + bb) << 5) | (col & 31u);
-                if (!half) {
-                    pend = e;
-                    half = true;
-                } else {
-                    put(pend | (e << 16));
-                    half = false;
-                }
-            }
-        }
-    }
-    if (half) put(pend | (sentinel << 16));
-    while (j < L) put(sentinel | (sentinel << 16));
-}
-
-// ---- skip sampler: flip lists straight from the generator, without ever drawing the bits that do not flip -----------
-// For a uniform flip probability p the columns that flip in a row form a renewal process with geometric gaps.  Row q
-// (flat over members and rows) reads the Philox words first + q*C + i, i = 0, 1, ...; word i has the rank
-// #{k < Kt : cdf[k] <= word} (cdf[k-1] = floor(2^32 * (1 - (1-p)^k)), supplied by the caller; Kt == 0 means no
-// flips): a rank below Kt moves the position on by rank + 1 columns and flips the column reached, rank Kt (a word
-// beyond the table) moves it on by Kt columns without a flip; the row ends when the position passes C.  About
-// C*p + 1 words per row instead of C: 100 times fewer at p = 0.01.  The same law as the per-bit compare (i.i.d. Bernoulli(p), quantised to
-// 2^-32), not the same stream.
-constexpr int kSkipMaxTable = 4096;
-
-struct SkipChain {
-    PhiloxKey key;
-    uint64_t g;   // index of the next word
-    uint4 blk;
-    bool fresh;
-    __device__ __forceinline__ SkipChain(const PhiloxKey &k, uint64_t start) : key(k), g(start), fresh(true) {}
-    __device__ __forceinline__ uint32_t next()
-    {
-        if (fresh || (g & 3u) == 0) blk = philox_block(key, g >> 2);
-        fresh = false;
-        const uint32_t e = (uint32_t)g & 3u;
-        g++;
-        return e == 0 ? blk.x : e == 1 ? blk.y : e == 2 ? blk.z : blk.w;
-    }
-};
-
-// Number of table entries <= u (the table is sorted).  The entries follow 2^32 * (1 - q^k), so
-// log2(1 - u / 2^32) / log2(q) lands within a step or two of the answer; the walk from there is against the table
-// itself, which keeps the result exact whatever the float arithmetic does (a wrong estimate only costs probes).
-__device__ __forceinline__ int skip_rank(const uint32_t *tab, int Kt, uint32_t u, float inv_log2q)
-{
-    const float s = ((float)(~u) + 1.0f) * 2.3283064365386963e-10f;  // 1 - u / 2^32, from the complement: no cancellation
-    int est = (int)(__log2f(s) * inv_log2q);
-    est = est < 0 ? 0 : (est > Kt ? Kt : est);
-    while (est < Kt && tab[est] <= u) est++;
-    while (est > 0 && tab[est - 1] > u) est--;
-    return est;
-}
-
-__global__ __launch_bounds__(256) void fl_skip_count_kernel(uint16_t *__restrict__ cnt, const uint32_t *__restrict__ cdf,
-                                                            int Kt, float inv_log2q, PhiloxKey key, int64_t rows, int C)
-{
-    __shared__ uint32_t tab[kSkipMaxTable];
-    for (int i = threadIdx.x; i < Kt; i += 256) tab[i] = cdf[i];
-    __syncthreads();
-    const int64_t q = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (q >= rows) return;
-    int n = 0;
-    if (Kt > 0) {
-        SkipChain chain(key, key.first + (uint64_t)q * (uint64_t)C);
-        int pos = -1;
-        for (;;) {
-            const int rank = skip_rank(tab, Kt, chain.next(), inv_log2q);
-            pos += rank < Kt ? rank + 1 : Kt;
-            if (pos >= C) break;
-            n += rank < Kt ? 1 : 0;
-        }
-    }
-    cnt[q] = (uint16_t)n;
-}
-
-// ---- the same walk when every row starts on a block boundary of the stream (C and first multiples of 4) ------------
-// All lanes then take word e of their current block at the same time, so a block's four words are four straight-line
-// steps without a per-lane word select.  The table sits in LDS with one entry of padding on either side
-// (tab1[k] = cdf[k - 1], tab1[0] = 0, tab1[Kt + 1] = 2^32 - 1): the float estimate is almost always the rank itself,
-// and one two-entry read confirms it (tab1[est] <= u < tab1[est + 1]); a wave in which any lane fails that test walks
-// the table as skip_rank does.  Same ranks, same words, same results as the kernels above.
-__device__ __forceinline__ void skip_table_load(uint32_t *tab1, const uint32_t *cdf, int Kt)
-{
-    for (int i = threadIdx.x; i < Kt + 2; i += 256) tab1[i] = i == 0 ? 0u : (i <= Kt ? cdf[i - 1] : 0xFFFFFFFFu);
-    __syncthreads();
-}
-
-// ranks of a block's four words: estimates and table reads first, one test for all four
-__device__ __forceinline__ void skip_rank4(int (&rank)[4], const uint32_t *tab1, int Kt, const uint4 &w, float inv_log2q,
-                                           float c0)
-{
-    const uint32_t u[4] = {w.x, w.y, w.z, w.w};
-    uint32_t lo[4], hi[4];
-    const float kt_f = (float)Kt;
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-        // log2((2^32 - 1 - u) / 2^32) / log2(q): never negative, +inf for u = 2^32 - 1; the missing 1 moves the
-        // estimate for about two words in a million
-        const int est = (int)fminf(fmaf(__log2f((float)(~u[e])), inv_log2q, c0), kt_f);
-        rank[e] = est;
-        lo[e] = tab1[est];
-        hi[e] = tab1[est + 1];
-    }
-    uint32_t bad = 0;
-#pragma unroll
-    for (int e = 0; e < 4; ++e) bad |= (uint32_t)(lo[e] > u[e]) | (uint32_t)(hi[e] <= u[e]);
-    if (__any(bad != 0)) {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            int est = rank[e];
-            while (est < Kt && tab1[est + 1] <= u[e]) est++;
-            while (est > 0 && tab1[est] > u[e]) est--;
-            rank[e] = est;
-        }
-    }
-}
-
-// A lane counts rows q, q + T, q + 2T, ... (T = threads of the grid): lanes whose rows end early start their next
-// one at the following block instead of idling until the longest row of the wave has ended.
-__global__ __launch_bounds__(256) void fl_skip_count_aligned_kernel(uint16_t *__restrict__ cnt,
-                                                                    const uint32_t *__restrict__ cdf, int Kt,
-                                                                    float inv_log2q, PhiloxKey key, int64_t rows, int C)
-{
-    __shared__ uint32_t tab1[kSkipMaxTable + 2];
-    skip_table_load(tab1, cdf, Kt);
-    const int64_t T = (int64_t)gridDim.x * 256;
-    int64_t q = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    const uint64_t row_blocks = (uint64_t)C >> 2;
-    uint64_t row_blk = (key.first >> 2) + (uint64_t)q * row_blocks, blk = row_blk;
-    const uint64_t blk_step = (uint64_t)T * row_blocks;
-    const float c0 = -32.0f * inv_log2q;
-    int pos = -1, n = 0;
-    bool live = q < rows;
-    while (__any(live)) {
-        int rank[4];
-        skip_rank4(rank, tab1, Kt, philox_block(key, blk++), inv_log2q, c0);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {   // past the row's end pos stays >= C and nothing more is counted
-            pos += rank[e] < Kt ? rank[e] + 1 : Kt;
-            n += (rank[e] < Kt && pos < C) ? 1 : 0;
-        }
-        if (pos >= C) {
-            if (live) cnt[q] = (uint16_t)n;
-            q += T;
-            row_blk += blk_step;
-            blk = row_blk;
-            pos = -1;
-            n = 0;
-            live = q < rows;
-        }
-    }
-}
-
-// One lane's row, walked word by word (any C, any first): its entries into dwords lane, lane + 64, ... of the slice.
-// A lane's dwords leave four at a time, as whole 16-byte pieces (L is a multiple of 4); never past the slice,
-// whatever the inputs.  The walk writes its entries without the base bit; when a piece is complete, the base
-// words of its (up to eight) columns are asked for together and the bits put in before the piece is stored: one
-// wait for memory per piece instead of one per flip (a wait for a load also waits for the stores before it).
-__device__ __forceinline__ void skip_fill_row(uint4 *__restrict__ dst, int L, const uint64_t *__restrict__ b, int Kw,
-                                              const uint32_t *tab, int Kt, float inv_log2q, const PhiloxKey &key,
-                                              uint64_t start, bool valid, int C)
-{
-    const uint32_t sentinel = (uint32_t)(4 * Kw) << 5;
-    const uint32_t npieces = (uint32_t)(4 * Kw);
-    int j = 0;
-    uint32_t pend = 0;
-    bool half = false;
-    uint32_t q0 = 0, q1 = 0, q2 = 0;
-    auto base_bit = [&](uint32_t e) -> uint32_t {  // e: one 16-bit entry; 0 for a sentinel
-        const uint32_t piece = e >> 5;
-        const uint32_t col = (piece >> 1) * 32u + (e & 31u);
-        const uint32_t live = piece < npieces;
-        const uint64_t word = live ? b[col >> 6] : 0ull;  // nothing is read for a sentinel
-        return (uint32_t)(word >> (col & 63u)) & 1u;
-    };
-    auto patched = [&](uint32_t v) { return v | (base_bit(v & 0xFFFFu) << 5) | (base_bit(v >> 16) << 21); };
-    auto put = [&](uint32_t v) {
-        const int c = j & 3;
-        if (c == 0) q0 = v;
-        else if (c == 1) q1 = v;
-        else if (c == 2) q2 = v;
-        else if (j < L) {
-            const uint32_t p0 = patched(q0), p1 = patched(q1), p2 = patched(q2), p3 = patched(v);
-            dst[(int64_t)(j >> 2) * 64] = make_uint4(p0, p1, p2, p3);
-        }
-        j++;
-    };
-    if (valid && Kt > 0) {
-        SkipChain chain(key, start);
-        int pos = -1;
-        for (;;) {
-            const int rank = skip_rank(tab, Kt, chain.next(), inv_log2q);
-            pos += rank < Kt ? rank + 1 : Kt;
-            if (pos >= C) break;
-            if (rank >= Kt) continue;  // a word beyond the table: moved on, no flip
-            const uint32_t col = (uint32_t)pos;
-            const uint32_t e = ((2u * (col >> 5)) << 5) | (col & 31u);  // base bit still to come
+    const uint64_t *w = W + (d * R + r) * Kw, *b = base + r * Kw;
+    for (int k = 0; k < Kw; k++) {
+        const uint64_t bw = b[k];
+        uint64_t m = w[k] ^ bw;
+        while (m) {
+            const int bit = __builtin_ctzll(m);
+            m &= m - 1;
+            const uint32_t col = (uint32_t)k * 64u + (uint32_t)bit;
+            const uint32_t bb = (uint32_t)(bw >> bit) & 1u;
+            const uint32_t e = ((2u * (col >> 5) + bb) << 5) | (col & 31u);
+            n++;
             if (!half) {
                 pend = e;
                 half = true;
@@ -452,262 +258,36 @@ __device__ __forceinline__ void skip_fill_row(uint4 *__restrict__ dst, int L, co
         }
     }
     if (half) put(pend | (sentinel << 16));
-    while (j < L) put(sentinel | (sentinel << 16));
-}
-
-__global__ __launch_bounds__(256) void fl_skip_fill_kernel(uint32_t *__restrict__ entries,
-                                                           const uint64_t *__restrict__ base,
-                                                           const uint16_t *__restrict__ perm,
-                                                           const int64_t *__restrict__ slice_off,
-                                                           const int32_t *__restrict__ slice_len,
-                                                           const uint32_t *__restrict__ cdf, int Kt, float inv_log2q,
-                                                           PhiloxKey key, int64_t nslices, int S, int64_t R, int Kw,
-                                                           int C)
-{
-    __shared__ uint32_t tab[kSkipMaxTable];
-    for (int i = threadIdx.x; i < Kt; i += 256) tab[i] = cdf[i];
-    __syncthreads();
-    const int lane = threadIdx.x & 63;
-    const int64_t sl = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (sl >= nslices) return;
-    const int64_t d = sl / S;
-    const int s = (int)(sl - d * S);
-    const int64_t p = (int64_t)s * 64 + lane;
-    const bool valid = p < R;
-    int64_t r = valid ? perm[d * R + p] : 0;
-    r = r < R ? r : R - 1;
-    uint4 *dst = reinterpret_cast<uint4 *>(entries + slice_off[sl]) + lane;
-    skip_fill_row(dst, 4 * slice_len[sl], base + r * Kw, Kw, tab, Kt, inv_log2q, key,
-                  key.first + (uint64_t)(d * R + r) * (uint64_t)C, valid, C);
-}
-
-// Rows on block boundaries of the stream (C and first multiples of 4, a table with entries): the lanes of a slice
-// walk in step, eight words (two blocks) to a 16-byte piece.  As long as every word of a live row yields a flip, word
-// i of a row is its flip i, so the piece a wave is on is the same for all its lanes and nothing about the entry's
-// place is per lane; a row that has ended gives sentinels.  A word beyond the table (no flip) in any live row breaks
-// that: the wave then starts its slice again, row by row as above (with a table that runs to saturation this takes a
-// word of 2^32 - 1).
-__global__ __launch_bounds__(256) void fl_skip_fill_aligned_kernel(uint32_t *__restrict__ entries,
-                                                                   const uint64_t *__restrict__ base,
-                                                                   const uint16_t *__restrict__ perm,
-                                                                   const int64_t *__restrict__ slice_off,
-                                                                   const int32_t *__restrict__ slice_len,
-                                                                   const uint32_t *__restrict__ cdf, int Kt,
-                                                                   float inv_log2q, PhiloxKey key, int64_t nslices,
-                                                                   int S, int64_t R, int Kw, int C)
-{
-    __shared__ uint32_t tab1[kSkipMaxTable + 2];
-    skip_table_load(tab1, cdf, Kt);
-    const int lane = threadIdx.x & 63;
-    const int64_t sl = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (sl >= nslices) return;
-    const int64_t d = sl / S;
-    const int s = (int)(sl - d * S);
-    const int64_t p = (int64_t)s * 64 + lane;
-    const bool valid = p < R;
-    int64_t r = valid ? perm[d * R + p] : 0;
-    r = r < R ? r : R - 1;
-    const int P = slice_len[sl];
-    uint4 *dst = reinterpret_cast<uint4 *>(entries + slice_off[sl]) + lane;
-    const uint32_t *b32 = reinterpret_cast<const uint32_t *>(base + r * Kw);
-    const uint32_t sentinel = (uint32_t)(4 * Kw) << 5;
-    const float c0 = -32.0f * inv_log2q;
-    uint64_t blk = (key.first >> 2) + (uint64_t)(d * R + r) * ((uint64_t)C >> 2);
-    int pos = valid ? -1 : C;
-    bool irregular = false;
-    uint4 cur = make_uint4(0u, 0u, 0u, 0u);   // the row's window that the last entry lay in, and its first dword
-    uint32_t curwin = 0xFFFFFFFFu;
-    const uint32_t last_start = (uint32_t)(2 * Kw - 4);
-    int piece = 0;
-    for (; piece < P; ++piece) {
-        uint32_t e[8];
-#pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            int rank4[4];
-            skip_rank4(rank4, tab1, Kt, philox_block(key, blk++), inv_log2q, c0);
-#pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                const int rank = rank4[k];
-                irregular |= rank >= Kt && pos < C;
-                pos += rank < Kt ? rank + 1 : Kt;
-                const uint32_t col = (uint32_t)pos;
-                e[4 * h + k] = pos < C ? (((col >> 5) << 6) | (col & 31u)) : sentinel;
-            }
-        }
-        if (__any(irregular)) break;
-        // Base bits from 16-byte windows of the row (128 columns; the last one ends with the row): a window is asked
-        // for only where an entry leaves the one before it, since what the look-ups cost is the number of lanes that
-        // ask, not the bytes.  Four entries' windows are asked for together; nothing is read for a sentinel.
-#pragma unroll
-        for (int h = 0; h < 8; h += 4) {
-            uint32_t st[4];
-            bool need[4];
-            uint4 w[4];
-            uint32_t prev = curwin;
-#pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                const uint32_t dw = e[h + k] >> 6, a = dw & ~3u;
-                st[k] = a < last_start ? a : last_start;
-                const bool live = e[h + k] != sentinel;
-                need[k] = live && st[k] != prev;
-                prev = live ? st[k] : prev;
-            }
-#pragma unroll
-            for (int k = 0; k < 4; ++k)
-                if (need[k]) __builtin_memcpy(&w[k], b32 + st[k], 16);
-#pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                if (need[k]) {
-                    cur = w[k];
-                    curwin = st[k];
-                }
-                const uint32_t d = (e[h + k] >> 6) - curwin;
-                const uint32_t word = d == 0 ? cur.x : d == 1 ? cur.y : d == 2 ? cur.z : cur.w;
-                const uint32_t bit = e[h + k] != sentinel ? (word >> (e[h + k] & 31u)) & 1u : 0u;
-                e[h + k] |= bit << 5;
-            }
-        }
-        dst[(int64_t)piece * 64] = make_uint4(e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16),
-                                              e[6] | (e[7] << 16));
-    }
-    if (piece < P)
-        skip_fill_row(dst, 4 * P, base + r * Kw, Kw, tab1 + 1, Kt, inv_log2q, key,
-                      key.first + (uint64_t)(d * R + r) * (uint64_t)C, valid, C);
-}
-
-// v of lane (lane ^ j), j a power of two below 64: quad permutes, swizzles inside 32 lanes, a general exchange for 32
-__device__ __forceinline__ uint32_t xor_lane(uint32_t v, int j)
-{
-    switch (j) {
-    case 1: return (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0xB1, 0xF, 0xF, true);   // quad_perm [1, 0, 3, 2]
-    case 2: return (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0x4E, 0xF, 0xF, true);   // quad_perm [2, 3, 0, 1]
-    case 4: return (uint32_t)__builtin_amdgcn_ds_swizzle((int)v, (4 << 10) | 0x1F);    // bit mode: and 31, xor j
-    case 8: return (uint32_t)__builtin_amdgcn_ds_swizzle((int)v, (8 << 10) | 0x1F);
-    case 16: return (uint32_t)__builtin_amdgcn_ds_swizzle((int)v, (16 << 10) | 0x1F);
-    default: return (uint32_t)__shfl_xor((int)v, j);
+    while (j & 3) put(sentinel | (sentinel << 16));
+    const int pieces = j >> 2;
+    if (pieces > cap) {
+        atomicAdd(overflow, 1u);
+        info[d * R + r] = flip_info((uint32_t)(8 * cap), (uint32_t)cap);
+    } else {
+        info[d * R + r] = flip_info((uint32_t)n, (uint32_t)pieces);
     }
 }
-
-// Row order and slice lengths from the counts: workgroup (d, block of 1024 rows) sorts its rows by (count, row) with a
-// bitonic network, a key per thread, partners inside a wave by lane exchange and others through LDS (keys
-// count << 10 | row-in-block are distinct, so the order is the stable one; rows past R
-// sort last) and writes perm and, from the last row of every run of 64, the slice's pieces per lane.
-__global__ __launch_bounds__(1024) void fl_layout_kernel(uint16_t *__restrict__ perm, int32_t *__restrict__ slice_len,
-                                                         const uint16_t *__restrict__ cnt, int64_t R, int nblk, int S)
-{
-    __shared__ uint32_t key[1024];
-    const int t = threadIdx.x;
-    const int64_t d = blockIdx.x / nblk;
-    const int blk = (int)(blockIdx.x - d * nblk);
-    const int64_t r0 = (int64_t)blk * 1024;
-    const int valid = (int)(R - r0 < 1024 ? R - r0 : 1024);
-    uint32_t v = t < valid ? ((uint32_t)cnt[d * R + r0 + t] << 10) | (uint32_t)t : 0xFFFFFC00u | (uint32_t)t;
-#pragma unroll
-    for (int k = 2; k <= 1024; k <<= 1) {
-#pragma unroll
-        for (int j = k >> 1; j > 0; j >>= 1) {
-            uint32_t o;
-            if (j >= 64) {  // the partner sits in another wave: through LDS
-                __syncthreads();
-                key[t] = v;
-                __syncthreads();
-                o = key[t ^ j];
-            } else {
-                o = xor_lane(v, j);
-            }
-            const bool keep_min = ((t & j) == 0) == ((t & k) == 0);
-            v = keep_min ? (v < o ? v : o) : (v > o ? v : o);
-        }
-    }
-    if (t < valid) {
-        perm[d * R + r0 + t] = (uint16_t)(r0 + (v & 1023u));
-        if ((t & 63) == 63 || t == valid - 1) slice_len[d * S + (r0 + t) / 64] = (int32_t)(((v >> 10) + 7) >> 3);
-    }
-}
-
-// slice_off = running sum of slice_len * 256 dwords (exclusive), total[0] = the sum.  Workgroup b owns slices
-// 8192 b .. 8192 b + 8191, eight per thread, and first adds up everything before them itself.
-__device__ __forceinline__ int64_t block_sum_1024(int64_t v, int64_t *wave_sum, int64_t *incl_out)
-{
-    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
-    int64_t incl = v;  // inclusive sum over the wave's lanes
-#pragma unroll
-    for (int o = 1; o < 64; o <<= 1) {
-        const int64_t up = __shfl_up(incl, o);
-        if (lane >= o) incl += up;
-    }
-    __syncthreads();
-    if (lane == 63) wave_sum[wv] = incl;
-    __syncthreads();
-    int64_t before = 0, all = 0;
-#pragma unroll
-    for (int w = 0; w < 16; ++w) {
-        before += w < wv ? wave_sum[w] : 0;
-        all += wave_sum[w];
-    }
-    *incl_out = before + incl;
-    return all;
-}
-
-__global__ __launch_bounds__(1024) void fl_offsets_kernel(int64_t *__restrict__ slice_off, int64_t *__restrict__ total,
-                                                          const int32_t *__restrict__ slice_len, int64_t n)
-{
-    __shared__ int64_t wave_sum[16];
-    const int t = threadIdx.x;
-    const int64_t tile = (int64_t)blockIdx.x * 8192;
-    int64_t head = 0, unused;
-    const int4 *len4 = reinterpret_cast<const int4 *>(slice_len);  // a tile is 2048 of these
-#pragma unroll 4
-    for (int64_t i = t; i < tile / 4; i += 1024) {
-        const int4 q = len4[i];
-        head += (int64_t)q.x + q.y + q.z + q.w;
-    }
-    const int64_t carry = block_sum_1024(head, wave_sum, &unused) * 256;
-    const int64_t i0 = tile + (int64_t)t * 8;
-    int64_t v[8], mine = 0, incl;
-#pragma unroll
-    for (int k = 0; k < 8; ++k) {
-        v[k] = i0 + k < n ? (int64_t)slice_len[i0 + k] * 256 : 0;
-        mine += v[k];
-    }
-    const int64_t all = block_sum_1024(mine, wave_sum, &incl);
-    int64_t run = carry + incl - mine;
-#pragma unroll
-    for (int k = 0; k < 8; ++k) {
-        if (i0 + k < n) slice_off[i0 + k] = run;
-        run += v[k];
-    }
-    if (t == 0 && blockIdx.x == gridDim.x - 1) total[0] = carry + all;
-}
-
-// whether every row of the walk starts on a block boundary of the stream (and there is a table to look up)
-static inline bool skip_rows_aligned(int64_t C, uint64_t first, int64_t Kt) { return Kt > 0 && C % 4 == 0 && first % 4 == 0; }
-// the aligned fill reads the base in 16-byte windows: rows of at least two words
-static inline bool skip_fill_aligned(int64_t C, uint64_t first, int64_t Kt) { return skip_rows_aligned(C, first, Kt) && C > 64; }
 
 // Flip lists -> materialised weights: W must hold the base in every member on entry; every flip is XOR-ed in.  A
 // lane owns its row, so plain read-modify-writes suffice (flips come in column order: one write per touched word).
 __global__ __launch_bounds__(256) void fl_to_dense_kernel(uint64_t *__restrict__ W, const uint32_t *__restrict__ entries,
-                                                          const int64_t *__restrict__ slice_off,
-                                                          const int32_t *__restrict__ slice_len,
-                                                          const uint16_t *__restrict__ perm, int64_t nslices, int S,
-                                                          int64_t R, int Kw)
+                                                          const uint32_t *__restrict__ info, int64_t nslices, int S,
+                                                          int64_t R, int Kw, int cap)
 {
     const int lane = threadIdx.x & 63;
     const int64_t sl = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (sl >= nslices) return;
     const int64_t d = sl / S;
     const int s = (int)(sl - d * S);
-    const int64_t p = (int64_t)s * 64 + lane;
-    if (p >= R) return;
-    int64_t r = perm[d * R + p];
-    r = r < R ? r : R - 1;
+    const int64_t r = (int64_t)s * 64 + lane;
+    if (r >= R) return;
     uint64_t *row = W + (d * R + r) * Kw;
-    const uint32_t *src = entries + slice_off[sl] + lane * 4;
-    const int L = 4 * slice_len[sl];
+    const uint32_t *src = entries + sl * (int64_t)cap * 256 + lane * 4;
+    int pieces = (int)(info[d * R + r] >> 16);
+    pieces = pieces < cap ? pieces : cap;
     int curw = -1;
     uint64_t mask = 0;
-    for (int j = 0; j < L; j++) {
+    for (int j = 0; j < 4 * pieces; j++) {
         const uint32_t pair = src[(int64_t)(j >> 2) * 256 + (j & 3)];
 #pragma unroll
         for (int h = 0; h < 2; h++) {
@@ -728,18 +308,16 @@ __global__ __launch_bounds__(256) void fl_to_dense_kernel(uint64_t *__restrict__
 }
 
 // ---- the members' corrections, threshold and pack --------------------------------------------------------------------
-// One workgroup per (member, block of 1024 rows), one wave per slice.  PACK: out = bits (2 * sum > thresh) of the
-// block's rows, OR-ed into an LDS bit array (the rows of a slice are scattered over the block) and written as 32-bit
-// pieces; else out = the int32 sums.
+// One workgroup per (member, block of 1024 rows), one wave per slice, lane l on row 64 s + l.  A lane asks only for
+// the pieces its own row has (a lane that is done requests nothing: the bytes a slice costs follow its rows' lengths
+// in 64-byte sectors, not its longest row); the wave walks to its longest row.  PACK: out = bits (2 * sum > thresh)
+// of the block's rows, collected in an LDS bit array and written as 32-bit pieces; else out = the int32 sums.
 template <bool PACK>
 __global__ __launch_bounds__(1024) void fl_bmv_kernel(void *__restrict__ out, const int32_t *__restrict__ G,
                                                       const uint32_t *__restrict__ entries,
-                                                      const int64_t *__restrict__ slice_off,
-                                                      const int32_t *__restrict__ slice_len,
-                                                      const uint16_t *__restrict__ perm,
-                                                      const uint16_t *__restrict__ cnt, const uint32_t *__restrict__ x32,
+                                                      const uint32_t *__restrict__ info, const uint32_t *__restrict__ x32,
                                                       const int32_t *__restrict__ thresh, int64_t R, int S, int Kw,
-                                                      int blocks_per_member)
+                                                      int blocks_per_member, int cap)
 {
     // x and ~x interleaved, one zero dword (the sentinel's entry: 4 * Kw), then the block's bit array.  A static
     // array: its address is then known when the look-ups are compiled and needs no add per look-up.
@@ -753,16 +331,31 @@ __global__ __launch_bounds__(1024) void fl_bmv_kernel(void *__restrict__ out, co
     const int s = blk * (kFlipBlockRows / 64) + __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const bool active = s < S;
     const int64_t sl = d * S + (active ? s : S - 1);
-    const int L = active ? __builtin_amdgcn_readfirstlane(slice_len[sl]) : 0;
-    const uint4 *src = reinterpret_cast<const uint4 *>(entries + slice_off[sl]) + lane;
-    // Two register sets take turns: while one batch is looked up, the batch after it is in flight.  Only pieces
-    // that exist are requested (L is wave-uniform, so every such test is a scalar branch).  The first two batches
-    // are requested before anything else: they do not depend on the table.
+    const int64_t r = (int64_t)s * 64 + lane;
+    const bool valid = active && r < R;
+    const uint32_t inf = valid ? info[d * R + r] : 0u;
+    const int n = (int)(inf & 0xFFFFu);
+    int mine = (int)(inf >> 16);          // pieces of this lane's row
+    mine = mine < cap ? mine : cap;
+    int longest = mine;                   // of the slice
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const int other = __shfl_xor(longest, o);
+        longest = longest > other ? longest : other;
+    }
+    const int L = __builtin_amdgcn_readfirstlane(longest);
+    const uint4 *src = reinterpret_cast<const uint4 *>(entries) + sl * (int64_t)cap * 64 + lane;
+    const uint32_t sent2 = ((uint32_t)(4 * Kw) << 5) * 0x00010001u;
+    // Two register sets take turns: while one batch is looked up, the batch after it is in flight.  The first two
+    // batches are requested before anything else: they do not depend on the table.
     uint4 e0[U], e1[U];
     auto request = [&](uint4(&e)[U], int j) {
 #pragma unroll
         for (int u = 0; u < U; u++)
-            if (j + u < L) e[u] = load_stream16(src + (int64_t)(j + u) * 64);
+            if (j + u < L) {
+                e[u] = make_uint4(sent2, sent2, sent2, sent2);
+                if (j + u < mine) e[u] = load_stream16(src + (int64_t)(j + u) * 64);
+            }
     };
     request(e0, 0);
     request(e1, U);
@@ -774,13 +367,8 @@ __global__ __launch_bounds__(1024) void fl_bmv_kernel(void *__restrict__ out, co
     uint32_t *bitmap = fl_tab + 2 * nd + 1;
     if (threadIdx.x == 0) fl_tab[2 * nd] = 0u;
     if (threadIdx.x < 32) bitmap[threadIdx.x] = 0u;
-    const int64_t p = (int64_t)s * 64 + lane;
-    const bool valid = active && p < R;
-    int64_t r = perm[d * R + (valid ? p : R - 1)];
-    r = r < R ? r : R - 1;
-    const int n = cnt[d * R + r];
-    const int g = G[d * R + r];
-    const int t = PACK ? thresh[d * R + r] : 0;
+    const int g = valid ? G[d * R + r] : 0;
+    const int t = (PACK && valid) ? thresh[d * R + r] : 0;
     __syncthreads();
     int sy = 0;
     auto take = [&](uint32_t e) {
@@ -804,12 +392,14 @@ __global__ __launch_bounds__(1024) void fl_bmv_kernel(void *__restrict__ out, co
         look_up(e1, j + U);
         request(e1, j + 3 * U);
     }
-    if (active) {
+    if (valid) {
         const int sum = g + n - 2 * sy;
         if (PACK) {
             const int local = (int)(r - (int64_t)blk * kFlipBlockRows);
-            if (valid && 2 * sum > t) atomicOr(&bitmap[(local >> 5) & 31], 1u << (local & 31));
-        } else if (valid) {
+            // the 32 rows of a bitmap word are 32 consecutive lanes of this wave: one ballot half per word
+            const unsigned long long m = __ballot(2 * sum > t);
+            if ((lane & 31) == 0) bitmap[(local >> 5) & 31] = (uint32_t)(m >> (lane & 32));
+        } else {
             static_cast<int32_t *>(out)[d * R + r] = sum;
         }
     }
@@ -818,6 +408,88 @@ __global__ __launch_bounds__(1024) void fl_bmv_kernel(void *__restrict__ out, co
         const int pieces = 2 * (int)((R + 63) / 64);  // 32-bit pieces of a member's output row
         const int q = blk * 32 + (int)threadIdx.x;
         if (threadIdx.x < 32 && q < pieces) static_cast<uint32_t *>(out)[d * pieces + q] = bitmap[threadIdx.x];
+    }
+}
+
+// ---- weighted sum over the lists: out[r, c] = fp16( sum_d w[d] * bit_d[r, c] ), bit = base ^ flip -------------------
+//   = base[r, c] * (sum_d w[d])  +  (1 - 2 base[r, c]) * sum over the members d that flip (r, c) of w[d]
+// The entry carries the base bit, so a flip adds +-w[d] to its column.  A workgroup owns RB rows (four where LDS has
+// room: 64 bytes of every piece, whole sectors) and keeps their columns' sums in LDS as 32-bit fixed-point integers
+// (weights scaled by a power of two chosen from sum |w[d]|, so that no sum can overflow, populations below 2^30
+// members: integer adds commute, the result does not depend on the order in which the members arrive);
+// lane = (row, member), 64 / RB members per wave and step; a lane asks for its next piece before it adds the current.
+__global__ __launch_bounds__(1024) void fl_wsum_kernel(_Float16 *__restrict__ out, const uint32_t *__restrict__ entries,
+                                                       const uint32_t *__restrict__ info,
+                                                       const uint64_t *__restrict__ base,
+                                                       const _Float16 *__restrict__ wts, int64_t D, int64_t R, int C,
+                                                       int Kw, int S, int cap, int RB)
+{
+    extern __shared__ int32_t fl_ws_acc[];  // [RB][64 * Kw] column sums, then 16 x 8 bytes of scratch
+    float *red = reinterpret_cast<float *>(fl_ws_acc + RB * 64 * Kw);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int cols = 64 * Kw;
+    for (int i = tid; i < RB * cols; i += 1024) fl_ws_acc[i] = 0;
+    // A = sum |w[d]| (every workgroup adds in the same order, so all agree on the scale)
+    float part = 0.f;
+    for (int64_t i = tid; i < D; i += 1024) part += fabsf((float)wts[i]);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) part += __shfl_xor(part, o);
+    if (lane == 0) red[wave] = part;
+    __syncthreads();
+    float A = 0.f;
+#pragma unroll
+    for (int w = 0; w < 16; w++) A += red[w];
+    // scale = 2^k with A * 2^k < 2^30 (and the rounding of each term, at most D / 2 in all, stays below 2^30 as well)
+    int ex;
+    (void)frexpf(A + 1.0f, &ex);  // A + 1 < 2^ex
+    const int k = 29 - ex;
+    const float scale = ldexpf(1.0f, k), inv_scale = ldexpf(1.0f, -k);
+    const int row = lane & (RB - 1);
+    const int64_t r = (int64_t)blockIdx.x * RB + row;
+    const bool rvalid = r < R;
+    const int s = (int)(r >> 6), l = (int)(r & 63);
+    int32_t *acc = fl_ws_acc + row * cols;
+    const uint32_t npieces = (uint32_t)(4 * Kw);
+    long long total = 0;  // sum of the scaled weights (this lane's members)
+    const int per_wave = 64 / RB, shift = RB == 4 ? 2 : (RB == 2 ? 1 : 0);
+    for (int64_t d = (int64_t)wave * per_wave + (lane >> shift); d < D; d += 16 * per_wave) {
+        const int wq = (int)rintf((float)wts[d] * scale);
+        if (row == 0) total += wq;
+        if (!rvalid) continue;
+        int pieces = (int)(info[d * R + r] >> 16);
+        pieces = pieces < cap ? pieces : cap;
+        const uint4 *src = reinterpret_cast<const uint4 *>(entries) + (d * S + s) * (int64_t)cap * 64 + l;
+        uint4 nxt = make_uint4(0u, 0u, 0u, 0u);
+        if (pieces > 0) nxt = load_stream16(src);
+        for (int j = 0; j < pieces; j++) {
+            const uint4 q = nxt;
+            if (j + 1 < pieces) nxt = load_stream16(src + (int64_t)(j + 1) * 64);
+            const uint32_t e[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+            for (int h = 0; h < 8; h++) {
+                const uint32_t v = (h & 1) ? e[h >> 1] >> 16 : e[h >> 1] & 0xFFFFu;
+                const uint32_t piece = v >> 5;
+                if (piece < npieces) atomicAdd(acc + (piece >> 1) * 32 + (v & 31u), (piece & 1u) ? -wq : wq);
+            }
+        }
+    }
+    // total of the scaled weights over all members
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) total += __shfl_xor(total, o);
+    __syncthreads();
+    long long *tred = reinterpret_cast<long long *>(red);
+    if (lane == 0) tred[wave] = total;
+    __syncthreads();
+    long long F = 0;
+#pragma unroll
+    for (int w = 0; w < 16; w++) F += tred[w];
+    for (int i = tid; i < RB * C; i += 1024) {
+        const int rr = i / C, c = i - rr * C;
+        const int64_t ro = (int64_t)blockIdx.x * RB + rr;
+        if (ro < R) {
+            const long long b = (long long)((base[ro * Kw + (c >> 6)] >> (c & 63)) & 1ull);
+            out[ro * C + c] = (_Float16)((float)(b * F + (long long)fl_ws_acc[rr * cols + c]) * inv_scale);
+        }
     }
 }
 
@@ -880,14 +552,28 @@ int nb_bmm_nt_fp4(int32_t *C, const uint8_t *A, const uint8_t *B, int64_t M, int
     return nb::check_launch(who);
 }
 
-int nb_flip_count_i64(uint16_t *cnt, const int64_t *W, const int64_t *base, int64_t D, int64_t R, int64_t Kw,
+static int flip_list_check(const uint32_t *entries, const uint32_t *info, int64_t D, int64_t R, int64_t Kw, int64_t cap,
+                           const char *who)
+{
+    if (int rc = nb::flip_shape_check(D, R, Kw, who)) return rc;
+    NB_REQUIRE(cap >= 0 && cap <= 8191, "%s: %lld pieces per row, at most 8191", who, (long long)cap);
+    NB_REQUIRE(D * ((R + 63) / 64) * std::max<int64_t>(cap, 1) < (1LL << 36), "%s: lists too large", who);
+    if (D * R == 0) return NB_OK;
+    NB_REQUIRE_PTR(info);
+    NB_REQUIRE_ALIGNED(info, 4);
+    if (cap > 0) NB_REQUIRE_PTR(entries);
+    NB_REQUIRE_ALIGNED(entries, 16);
+    return NB_OK;
+}
+
+int nb_flip_count_i64(uint32_t *info, const int64_t *W, const int64_t *base, int64_t D, int64_t R, int64_t Kw,
                       nb_stream_t stream)
 {
     const char *who = "nb_flip_count_i64";
     if (int rc = nb::flip_shape_check(D, R, Kw, who)) return rc;
     if (D * R == 0) return NB_OK;
-    NB_REQUIRE_PTR(cnt);
-    NB_REQUIRE_ALIGNED(cnt, 2);
+    NB_REQUIRE_PTR(info);
+    NB_REQUIRE_ALIGNED(info, 4);
     if (Kw > 0) {
         NB_REQUIRE_PTR(W);
         NB_REQUIRE_PTR(base);
@@ -897,25 +583,18 @@ int nb_flip_count_i64(uint16_t *cnt, const int64_t *W, const int64_t *base, int6
     const int64_t blocks = nb::ceil_div(D * R * 16, 256);
     NB_REQUIRE(blocks <= nb::kMaxGridX, "%s: too many rows for one launch", who);
     nb::fl_count_kernel<<<dim3((unsigned)blocks), dim3(256), 0, nb::as_stream(stream)>>>(
-        cnt, reinterpret_cast<const uint64_t *>(W), reinterpret_cast<const uint64_t *>(base), D * R, R, (int)Kw);
+        info, reinterpret_cast<const uint64_t *>(W), reinterpret_cast<const uint64_t *>(base), D * R, R, (int)Kw);
     return nb::check_launch(who);
 }
 
-int nb_flip_fill_i64(uint32_t *entries, const int64_t *W, const int64_t *base, const uint16_t *perm,
-                     const int64_t *slice_off, const int32_t *slice_len, int64_t D, int64_t R, int64_t Kw,
-                     nb_stream_t stream)
+int nb_flip_fill_i64(uint32_t *entries, uint32_t *info, uint32_t *overflow, const int64_t *W, const int64_t *base,
+                     int64_t D, int64_t R, int64_t Kw, int64_t cap, nb_stream_t stream)
 {
     const char *who = "nb_flip_fill_i64";
-    if (int rc = nb::flip_shape_check(D, R, Kw, who)) return rc;
+    if (int rc = flip_list_check(entries, info, D, R, Kw, cap, who)) return rc;
     if (D * R == 0) return NB_OK;
-    NB_REQUIRE_PTR(entries);
-    NB_REQUIRE_PTR(perm);
-    NB_REQUIRE_PTR(slice_off);
-    NB_REQUIRE_PTR(slice_len);
-    NB_REQUIRE_ALIGNED(entries, 16);
-    NB_REQUIRE_ALIGNED(perm, 2);
-    NB_REQUIRE_ALIGNED(slice_off, 8);
-    NB_REQUIRE_ALIGNED(slice_len, 4);
+    NB_REQUIRE_PTR(overflow);
+    NB_REQUIRE_ALIGNED(overflow, 4);
     if (Kw > 0) {
         NB_REQUIRE_PTR(W);
         NB_REQUIRE_PTR(base);
@@ -924,156 +603,37 @@ int nb_flip_fill_i64(uint32_t *entries, const int64_t *W, const int64_t *base, c
     }
     const int64_t S = (R + 63) / 64;
     nb::fl_fill_kernel<<<dim3((unsigned)nb::ceil_div(D * S, 4)), dim3(256), 0, nb::as_stream(stream)>>>(
-        entries, reinterpret_cast<const uint64_t *>(W), reinterpret_cast<const uint64_t *>(base), perm, slice_off,
-        slice_len, D * S, (int)S, R, (int)Kw);
+        entries, info, overflow, reinterpret_cast<const uint64_t *>(W), reinterpret_cast<const uint64_t *>(base), D * S,
+        (int)S, R, (int)Kw, (int)cap);
     return nb::check_launch(who);
 }
 
-// 1 / log2(1 - p) for the table's first entry p * 2^32: only a hint for where a look-up starts probing
-static float skip_hint(uint32_t cdf0)
-{
-    const double p = (double)cdf0 / 4294967296.0;
-    if (p <= 0.0 || p >= 1.0) return 0.0f;
-    return (float)(1.0 / std::log2(1.0 - p));
-}
-
-int nb_flip_skip_count_i64(uint16_t *cnt, const uint32_t *cdf, uint32_t cdf0, int64_t Kt, uint64_t seed, uint64_t subseq,
-                           uint64_t first, int64_t D, int64_t R, int64_t C, nb_stream_t stream)
-{
-    const char *who = "nb_flip_skip_count_i64";
-    const float inv_log2q = skip_hint(cdf0);
-    NB_REQUIRE(C >= 0 && Kt >= 0 && Kt <= nb::kSkipMaxTable, "%s: bad C=%lld or table of %lld entries (at most %d)", who,
-               (long long)C, (long long)Kt, nb::kSkipMaxTable);
-    if (int rc = nb::flip_shape_check(D, R, (C + 63) / 64, who)) return rc;
-    if (D * R == 0) return NB_OK;
-    NB_REQUIRE_PTR(cnt);
-    NB_REQUIRE_ALIGNED(cnt, 2);
-    if (Kt > 0) NB_REQUIRE_PTR(cdf);
-    NB_REQUIRE_ALIGNED(cdf, 4);
-    const int64_t blocks = nb::ceil_div(D * R, 256);
-    NB_REQUIRE(blocks <= nb::kMaxGridX, "%s: too many rows for one launch", who);
-    if (nb::skip_rows_aligned(C, first, Kt)) {
-        // beyond 2048 workgroups (eight per compute unit) a lane takes several rows, up to eight
-        const int64_t grid = blocks <= 2048 ? blocks : std::max<int64_t>(2048, nb::ceil_div(blocks, 8));
-        nb::fl_skip_count_aligned_kernel<<<dim3((unsigned)grid), dim3(256), 0, nb::as_stream(stream)>>>(
-            cnt, cdf, (int)Kt, inv_log2q, nb::PhiloxKey{seed, subseq, first}, D * R, (int)C);
-    } else {
-        nb::fl_skip_count_kernel<<<dim3((unsigned)blocks), dim3(256), 0, nb::as_stream(stream)>>>(
-            cnt, cdf, (int)Kt, inv_log2q, nb::PhiloxKey{seed, subseq, first}, D * R, (int)C);
-    }
-    return nb::check_launch(who);
-}
-
-int nb_flip_skip_fill_i64(uint32_t *entries, const int64_t *base, const uint16_t *perm, const int64_t *slice_off,
-                          const int32_t *slice_len, const uint32_t *cdf, uint32_t cdf0, int64_t Kt, uint64_t seed,
-                          uint64_t subseq, uint64_t first, int64_t D, int64_t R, int64_t C, nb_stream_t stream)
-{
-    const char *who = "nb_flip_skip_fill_i64";
-    const float inv_log2q = skip_hint(cdf0);
-    NB_REQUIRE(C >= 0 && Kt >= 0 && Kt <= nb::kSkipMaxTable, "%s: bad C=%lld or table of %lld entries (at most %d)", who,
-               (long long)C, (long long)Kt, nb::kSkipMaxTable);
-    const int64_t Kw = (C + 63) / 64;
-    if (int rc = nb::flip_shape_check(D, R, Kw, who)) return rc;
-    if (D * R == 0) return NB_OK;
-    NB_REQUIRE_PTR(entries);
-    NB_REQUIRE_PTR(perm);
-    NB_REQUIRE_PTR(slice_off);
-    NB_REQUIRE_PTR(slice_len);
-    NB_REQUIRE_ALIGNED(entries, 16);
-    NB_REQUIRE_ALIGNED(perm, 2);
-    NB_REQUIRE_ALIGNED(slice_off, 8);
-    NB_REQUIRE_ALIGNED(slice_len, 4);
-    if (Kt > 0) NB_REQUIRE_PTR(cdf);
-    NB_REQUIRE_ALIGNED(cdf, 4);
-    if (Kw > 0) NB_REQUIRE_PTR(base);
-    NB_REQUIRE_ALIGNED(base, 8);
-    const int64_t S = (R + 63) / 64;
-    const dim3 grid((unsigned)nb::ceil_div(D * S, 4));
-    if (nb::skip_fill_aligned(C, first, Kt))
-        nb::fl_skip_fill_aligned_kernel<<<grid, dim3(256), 0, nb::as_stream(stream)>>>(
-            entries, reinterpret_cast<const uint64_t *>(base), perm, slice_off, slice_len, cdf, (int)Kt, inv_log2q,
-            nb::PhiloxKey{seed, subseq, first}, D * S, (int)S, R, (int)Kw, (int)C);
-    else
-        nb::fl_skip_fill_kernel<<<grid, dim3(256), 0, nb::as_stream(stream)>>>(
-            entries, reinterpret_cast<const uint64_t *>(base), perm, slice_off, slice_len, cdf, (int)Kt, inv_log2q,
-            nb::PhiloxKey{seed, subseq, first}, D * S, (int)S, R, (int)Kw, (int)C);
-    return nb::check_launch(who);
-}
-
-int nb_flip_layout(uint16_t *perm, int32_t *slice_len, int64_t *slice_off, int64_t *total, const uint16_t *cnt, int64_t D,
-                   int64_t R, nb_stream_t stream)
-{
-    const char *who = "nb_flip_layout";
-    if (int rc = nb::flip_shape_check(D, R, 0, who)) return rc;
-    NB_REQUIRE_PTR(total);
-    NB_REQUIRE_ALIGNED(total, 8);
-    const int64_t S = (R + 63) / 64;
-    if (D * R > 0) {
-        NB_REQUIRE_PTR(perm);
-        NB_REQUIRE_PTR(slice_len);
-        NB_REQUIRE_PTR(slice_off);
-        NB_REQUIRE_PTR(cnt);
-        NB_REQUIRE_ALIGNED(perm, 2);
-        NB_REQUIRE_ALIGNED(slice_len, 16);
-        NB_REQUIRE_ALIGNED(slice_off, 8);
-        NB_REQUIRE_ALIGNED(cnt, 2);
-        const int64_t nblk = nb::ceil_div(R, 1024);
-        NB_REQUIRE(D * nblk <= nb::kMaxGridX / 4, "%s: too many rows for one launch", who);
-        nb::fl_layout_kernel<<<dim3((unsigned)(D * nblk)), dim3(1024), 0, nb::as_stream(stream)>>>(
-            perm, slice_len, cnt, R, (int)nblk, (int)S);
-        if (int rc = nb::check_launch(who)) return rc;
-    }
-    const int64_t n = D * R > 0 ? D * S : 0;
-    nb::fl_offsets_kernel<<<dim3((unsigned)std::max<int64_t>(1, nb::ceil_div(n, 8192))), dim3(1024), 0,
-                            nb::as_stream(stream)>>>(slice_off, total, slice_len, n);
-    return nb::check_launch(who);
-}
-
-int nb_flip_to_dense_i64(int64_t *W, const uint32_t *entries, const int64_t *slice_off, const int32_t *slice_len,
-                         const uint16_t *perm, int64_t D, int64_t R, int64_t Kw, nb_stream_t stream)
+int nb_flip_to_dense_i64(int64_t *W, const uint32_t *entries, const uint32_t *info, int64_t D, int64_t R, int64_t Kw,
+                         int64_t cap, nb_stream_t stream)
 {
     const char *who = "nb_flip_to_dense_i64";
-    if (int rc = nb::flip_shape_check(D, R, Kw, who)) return rc;
+    if (int rc = flip_list_check(entries, info, D, R, Kw, cap, who)) return rc;
     if (D * R * Kw == 0) return NB_OK;
     NB_REQUIRE_PTR(W);
-    NB_REQUIRE_PTR(entries);
-    NB_REQUIRE_PTR(perm);
-    NB_REQUIRE_PTR(slice_off);
-    NB_REQUIRE_PTR(slice_len);
     NB_REQUIRE_ALIGNED(W, 8);
-    NB_REQUIRE_ALIGNED(entries, 16);
-    NB_REQUIRE_ALIGNED(perm, 2);
-    NB_REQUIRE_ALIGNED(slice_off, 8);
-    NB_REQUIRE_ALIGNED(slice_len, 4);
     const int64_t S = (R + 63) / 64;
     nb::fl_to_dense_kernel<<<dim3((unsigned)nb::ceil_div(D * S, 4)), dim3(256), 0, nb::as_stream(stream)>>>(
-        reinterpret_cast<uint64_t *>(W), entries, slice_off, slice_len, perm, D * S, (int)S, R, (int)Kw);
+        reinterpret_cast<uint64_t *>(W), entries, info, D * S, (int)S, R, (int)Kw, (int)cap);
     return nb::check_launch(who);
 }
 
-static int flip_bmv(void *out, const int32_t *G, const uint32_t *entries, const int64_t *slice_off,
-                    const int32_t *slice_len, const uint16_t *perm, const uint16_t *cnt, const int64_t *x,
-                    const int32_t *thresh, int64_t D, int64_t R, int64_t Kw, bool pack, nb_stream_t stream,
+static int flip_bmv(void *out, const int32_t *G, const uint32_t *entries, const uint32_t *info, const int64_t *x,
+                    const int32_t *thresh, int64_t D, int64_t R, int64_t Kw, int64_t cap, bool pack, nb_stream_t stream,
                     const char *who)
 {
-    if (int rc = nb::flip_shape_check(D, R, Kw, who)) return rc;
+    if (int rc = flip_list_check(entries, info, D, R, Kw, cap, who)) return rc;
     if (D * R == 0) return NB_OK;
     NB_REQUIRE_PTR(out);
     NB_REQUIRE_PTR(G);
-    NB_REQUIRE_PTR(entries);
-    NB_REQUIRE_PTR(slice_off);
-    NB_REQUIRE_PTR(slice_len);
-    NB_REQUIRE_PTR(perm);
-    NB_REQUIRE_PTR(cnt);
     if (pack) NB_REQUIRE_PTR(thresh);
     if (Kw > 0) NB_REQUIRE_PTR(x);
     NB_REQUIRE_ALIGNED(out, pack ? 8 : 4);
     NB_REQUIRE_ALIGNED(G, 4);
-    NB_REQUIRE_ALIGNED(entries, 16);
-    NB_REQUIRE_ALIGNED(slice_off, 8);
-    NB_REQUIRE_ALIGNED(slice_len, 4);
-    NB_REQUIRE_ALIGNED(perm, 2);
-    NB_REQUIRE_ALIGNED(cnt, 2);
     NB_REQUIRE_ALIGNED(x, 8);
     NB_REQUIRE_ALIGNED(thresh, 4);
     const int64_t S = (R + 63) / 64;
@@ -1084,28 +644,59 @@ static int flip_bmv(void *out, const int32_t *G, const uint32_t *entries, const 
     const dim3 grid((unsigned)(D * bpm));
     if (pack)
         nb::fl_bmv_kernel<true><<<grid, dim3(threads), 0, nb::as_stream(stream)>>>(
-            out, G, entries, slice_off, slice_len, perm, cnt, reinterpret_cast<const uint32_t *>(x), thresh, R, (int)S,
-            (int)Kw, (int)bpm);
+            out, G, entries, info, reinterpret_cast<const uint32_t *>(x), thresh, R, (int)S, (int)Kw, (int)bpm, (int)cap);
     else
         nb::fl_bmv_kernel<false><<<grid, dim3(threads), 0, nb::as_stream(stream)>>>(
-            out, G, entries, slice_off, slice_len, perm, cnt, reinterpret_cast<const uint32_t *>(x), thresh, R, (int)S,
-            (int)Kw, (int)bpm);
+            out, G, entries, info, reinterpret_cast<const uint32_t *>(x), thresh, R, (int)S, (int)Kw, (int)bpm, (int)cap);
     return nb::check_launch(who);
 }
 
-int nb_bmv_flip_i64(int32_t *out, const int32_t *G, const uint32_t *entries, const int64_t *slice_off,
-                    const int32_t *slice_len, const uint16_t *perm, const uint16_t *cnt, const int64_t *x, int64_t D,
-                    int64_t R, int64_t Kw, nb_stream_t stream)
+int nb_bmv_flip_i64(int32_t *out, const int32_t *G, const uint32_t *entries, const uint32_t *info, const int64_t *x,
+                    int64_t D, int64_t R, int64_t Kw, int64_t cap, nb_stream_t stream)
 {
-    return flip_bmv(out, G, entries, slice_off, slice_len, perm, cnt, x, nullptr, D, R, Kw, false, stream,
-                    "nb_bmv_flip_i64");
+    return flip_bmv(out, G, entries, info, x, nullptr, D, R, Kw, cap, false, stream, "nb_bmv_flip_i64");
 }
 
-int nb_bmv_flip_act_pack_i64(int64_t *out, const int32_t *G, const uint32_t *entries, const int64_t *slice_off,
-                             const int32_t *slice_len, const uint16_t *perm, const uint16_t *cnt, const int64_t *x,
-                             const int32_t *thresh, int64_t D, int64_t R, int64_t Kw, nb_stream_t stream)
+int nb_bmv_flip_act_pack_i64(int64_t *out, const int32_t *G, const uint32_t *entries, const uint32_t *info,
+                             const int64_t *x, const int32_t *thresh, int64_t D, int64_t R, int64_t Kw, int64_t cap,
+                             nb_stream_t stream)
 {
-    return flip_bmv(out, G, entries, slice_off, slice_len, perm, cnt, x, thresh, D, R, Kw, true, stream,
-                    "nb_bmv_flip_act_pack_i64");
+    return flip_bmv(out, G, entries, info, x, thresh, D, R, Kw, cap, true, stream, "nb_bmv_flip_act_pack_i64");
+}
+
+int nb_flip_weighted_sum_i64(uint16_t *out, const uint32_t *entries, const uint32_t *info, const int64_t *base,
+                             const uint16_t *weights, int64_t D, int64_t R, int64_t C, int64_t cap, nb_stream_t stream)
+{
+    const char *who = "nb_flip_weighted_sum_i64";
+    NB_REQUIRE(C >= 0, "%s: negative C", who);
+    const int64_t Kw = (C + 63) / 64;
+    if (int rc = flip_list_check(entries, info, D, R, Kw, cap, who)) return rc;
+    NB_REQUIRE(D < (1LL << 30), "%s: at most 2^30 - 1 members", who);
+    if (R * C == 0) return NB_OK;
+    NB_REQUIRE_PTR(out);
+    NB_REQUIRE_ALIGNED(out, 2);
+    NB_REQUIRE_PTR(base);
+    NB_REQUIRE_ALIGNED(base, 8);
+    if (D > 0) NB_REQUIRE_PTR(weights);
+    NB_REQUIRE_ALIGNED(weights, 2);
+    // rows per workgroup: as many of 4, 2, 1 as LDS (160 KB per workgroup on this part) holds
+    int RB = 4;
+    while (RB > 1 && (size_t)RB * 64 * Kw * 4 + 128 > 150 * 1024) RB >>= 1;
+    const size_t lds = (size_t)RB * 64 * Kw * 4 + 128;
+    static std::once_flag once;
+    static hipError_t attr = hipSuccess;
+    std::call_once(once, [] {
+        attr = hipFuncSetAttribute(reinterpret_cast<const void *>(nb::fl_wsum_kernel),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024 + 128);
+    });
+    if (attr != hipSuccess) {
+        (void)hipGetLastError();
+        return nb::fail(NB_ERR_UNSUPPORTED, "%s: cannot raise the kernel's LDS limit: %s", who, hipGetErrorString(attr));
+    }
+    const int64_t S = (R + 63) / 64;
+    nb::fl_wsum_kernel<<<dim3((unsigned)nb::ceil_div(R, RB)), dim3(1024), lds, nb::as_stream(stream)>>>(
+        reinterpret_cast<_Float16 *>(out), entries, info, reinterpret_cast<const uint64_t *>(base),
+        reinterpret_cast<const _Float16 *>(weights), D, R, (int)C, (int)Kw, (int)S, (int)cap, RB);
+    return nb::check_launch(who);
 }
 }

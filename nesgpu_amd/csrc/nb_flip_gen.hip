@@ -1,0 +1,595 @@
+// Drawing the flip lists of the sparse linear form straight from the generator, in one pass and without a read-back.
+//
+// Skip sampler: with flip probability p the flipped columns of a row are a renewal process with geometric gaps, so
+// only the gaps are drawn (about C*p + 1 random words per row instead of C).  Row q = d*R + r reads the Philox words
+// first + q*C + i, i = 0, 1, ...; a word's rank in the table cdf[k-1] = floor(2^32 (1 - (1-p)^k)) (how many entries
+// are <= the word) moves the position on by rank + 1 columns to a flip, or, beyond the table, by the table's length
+// without one; the row ends when the position passes C.
+//
+// Thinning (per-element probabilities): the walk runs at the LARGEST flip probability p_max of the layer; words come
+// in pairs (gap, accept), and a column c reached by the walk flips only if accept * T_max < Tf[r, c] * 2^32, i.e.
+// with probability Tf / T_max: every column then flips with its own probability Tf[r, c] / 2^32, independently.
+//
+// Work is laid out by ROWS, not by members: a workgroup owns a few rows and keeps what a look-up needs of them in LDS
+// (their base bits, or their probabilities), its lanes walk those rows for member after member (a lane that has
+// finished a row starts its next member at once), and every row's entries go to the fixed place the list layout
+// gives them (nb_flip.hip), so nothing has to be counted first.
+#include <cmath>
+#include <mutex>
+
+#include "nb_common.hpp"
+#include "nb_conv_common.hpp"
+
+namespace nb {
+
+constexpr int kSkipMaxTable = 4096;
+// The table as the kernels take it, in device memory: [0] entries Kt, [1] the bits of the float 1 / log2(1 - p) (a hint
+// for where a look-up starts probing; it changes no result), [2] the threshold p * 2^32 the table was made for, [3] 0,
+// [4 + k] = cdf[k].
+constexpr int kSkipHeader = 4;
+constexpr int kSkipTableWords = kSkipHeader + kSkipMaxTable;
+
+struct SkipChain {
+    PhiloxKey key;
+    uint64_t g;   // index of the next word
+    uint4 blk;
+    bool fresh;
+    __device__ __forceinline__ SkipChain(const PhiloxKey &k, uint64_t start) : key(k), g(start), fresh(true) {}
+    __device__ __forceinline__ void restart(uint64_t start)
+    {
+        g = start;
+        fresh = true;
+    }
+    __device__ __forceinline__ uint32_t next()
+    {
+        if (fresh || (g & 3u) == 0) blk = philox_block(key, g >> 2);
+        fresh = false;
+        const uint32_t e = (uint32_t)g & 3u;
+        g++;
+        return e == 0 ? blk.x : e == 1 ? blk.y : e == 2 ? blk.z : blk.w;
+    }
+};
+
+// Ranks of N words in the padded table tab1 (tab1[0] = 0, tab1[k] = cdf[k - 1], tab1[Kt + 1] = 2^32 - 1): the number of
+// cdf entries <= the word.  The entries follow 2^32 (1 - q^k), so log2((2^32 - 1 - u) / 2^32) / log2(q) is almost always
+// the rank itself; one two-entry read confirms it (tab1[est] <= u < tab1[est + 1]), and a wave in which any lane fails
+// that test walks the table from its estimate.  The result never depends on the float arithmetic.
+template <int N>
+__device__ __forceinline__ void skip_ranks(int (&rank)[N], const uint32_t *tab1, int Kt, const uint32_t (&u)[N],
+                                           float inv_log2q, float c0)
+{
+    uint32_t lo[N], hi[N];
+    const float kt_f = (float)Kt;
+#pragma unroll
+    for (int e = 0; e < N; ++e) {
+        const int est = (int)fminf(fmaf(__log2f((float)(~u[e])), inv_log2q, c0), kt_f);
+        rank[e] = est;
+        lo[e] = tab1[est];
+        hi[e] = tab1[est + 1];
+    }
+    uint32_t bad = 0;
+#pragma unroll
+    for (int e = 0; e < N; ++e) bad |= (uint32_t)(lo[e] > u[e]) | (uint32_t)(hi[e] <= u[e]);
+    if (__any(bad != 0)) {
+#pragma unroll
+        for (int e = 0; e < N; ++e) {
+            int est = rank[e];
+            while (est < Kt && tab1[est + 1] <= u[e]) est++;
+            while (est > 0 && tab1[est] > u[e]) est--;
+            rank[e] = est;
+        }
+    }
+}
+
+struct GenArgs {
+    uint4 *entries;
+    uint32_t *info, *overflow;
+    const void *rows;        // uniform: base bits [R, 2 Kw] dwords; thinning: [R, C] 16-bit flip laws
+    const uint32_t *table;   // kSkipTableWords
+    PhiloxKey key;
+    int64_t D, R;
+    int C, Kw, S, cap, MC, rb_shift;  // MC members per workgroup; 1 << rb_shift rows per workgroup
+};
+
+// ALIGNED: every row starts on a block boundary of the stream (C and first multiples of 4): a block's four words are
+// four straight-line steps.  THIN: words in (gap, accept) pairs against the 16-bit laws of the columns:
+// bit 15 = base bit, bits 14:0 = the fp16 flip probability y <= 1/2, Tf = floor(y * 2^32).
+template <bool ALIGNED, bool THIN>
+__global__ __launch_bounds__(1024) void fl_gen_kernel(const GenArgs a)
+{
+    extern __shared__ uint32_t gen_lds[];
+    uint32_t *tab1 = gen_lds;                              // kSkipMaxTable + 2
+    uint32_t *rowdata = gen_lds + kSkipMaxTable + 2;       // the workgroup's rows
+    const int Kt = (int)a.table[0];
+    const float inv_log2q = __uint_as_float(a.table[1]);
+    const uint32_t Tmax = a.table[2];
+    const int RB = 1 << a.rb_shift;
+    const int nrg = (int)((a.R + RB - 1) >> a.rb_shift);
+    const int rg = (int)(blockIdx.x % (unsigned)nrg), mc = (int)(blockIdx.x / (unsigned)nrg);
+    const int64_t r0 = (int64_t)rg << a.rb_shift;
+    for (int i = threadIdx.x; i < Kt + 2; i += blockDim.x)
+        tab1[i] = i == 0 ? 0u : (i <= Kt ? a.table[kSkipHeader + i - 1] : 0xFFFFFFFFu);
+    const int row_dwords = THIN ? (a.C + 1) / 2 : 2 * a.Kw;   // LDS dwords of a row
+    if (THIN) {
+        const uint16_t *src = static_cast<const uint16_t *>(a.rows);
+        uint16_t *dst16 = reinterpret_cast<uint16_t *>(rowdata);
+        for (int rr = 0; rr < RB && r0 + rr < a.R; rr++)
+            for (int i = threadIdx.x; i < a.C; i += blockDim.x) dst16[rr * 2 * row_dwords + i] = src[(r0 + rr) * a.C + i];
+    } else {
+        const uint32_t *src = static_cast<const uint32_t *>(a.rows);
+        for (int rr = 0; rr < RB && r0 + rr < a.R; rr++)
+            for (int i = threadIdx.x; i < row_dwords; i += blockDim.x)
+                rowdata[rr * row_dwords + i] = src[(r0 + rr) * row_dwords + i];
+    }
+    __syncthreads();
+    const int rr = (int)threadIdx.x & (RB - 1);
+    const int64_t r = r0 + rr;
+    const int slots = (int)blockDim.x >> a.rb_shift;         // members a workgroup walks at a time
+    const int64_t dend = (int64_t)(mc + 1) * a.MC < a.D ? (int64_t)(mc + 1) * a.MC : a.D;
+    int64_t d = (int64_t)mc * a.MC + ((int)threadIdx.x >> a.rb_shift);
+    const uint32_t *myrow = rowdata + rr * row_dwords;
+    const uint16_t *myrow16 = reinterpret_cast<const uint16_t *>(myrow);
+    const uint32_t sentinel = (uint32_t)(4 * a.Kw) << 5;
+    const float c0 = -32.0f * inv_log2q;
+    const int C = a.C;
+    if (r >= a.R) d = dend;                                   // a lane without a row
+    if (Kt == 0) {                                            // p = 0: no flips anywhere
+        for (; d < dend; d += slots) a.info[d * a.R + r] = 0u;
+        return;
+    }
+    // per-lane walk state
+    bool live = d < dend;
+    int64_t q = 0;
+    uint64_t blk = 0;
+    SkipChain chain(a.key, 0);
+    uint4 *dst = a.entries;
+    int pos = -1, n = 0, k = 0, piece = 0;
+    uint32_t q0 = 0, q1 = 0, q2 = 0, q3 = 0;
+    auto start_row = [&]() {
+        live = d < dend;
+        if (live) {
+            q = d * a.R + r;
+            const uint64_t g0 = a.key.first + (uint64_t)q * (uint64_t)C;
+            if (ALIGNED) blk = g0 >> 2;
+            else chain.restart(g0);
+            dst = a.entries + ((d * a.S + (r >> 6)) * (int64_t)a.cap) * 64 + (r & 63);
+        }
+        pos = live ? -1 : C;
+        n = 0;
+        k = 0;
+        piece = 0;
+    };
+    auto insert = [&](uint32_t e) {                          // the piece as a 128-bit shift register: oldest entry lowest
+        q0 = __builtin_amdgcn_alignbit(q1, q0, 16);
+        q1 = __builtin_amdgcn_alignbit(q2, q1, 16);
+        q2 = __builtin_amdgcn_alignbit(q3, q2, 16);
+        q3 = (q3 >> 16) | (e << 16);
+    };
+    auto flush = [&]() {
+        if (piece < a.cap) dst[(int64_t)piece * 64] = make_uint4(q0, q1, q2, q3);
+        piece++;
+        k = 0;
+    };
+    // one step of the walk: `rank` of the gap word; `acc` the pair's second word (THIN)
+    auto step = [&](int rank, uint32_t acc) {
+        pos += rank < Kt ? rank + 1 : Kt;
+        bool flip = rank < Kt && pos < C;
+        const int pc = pos < C ? pos : 0;
+        uint32_t b;
+        if (THIN) {
+            const uint32_t h = myrow16[pc];
+            b = h >> 15;
+            const float y = (float)__builtin_bit_cast(_Float16, (uint16_t)(h & 0x7FFFu));
+            const uint32_t Tf = (uint32_t)fminf(y * 4294967296.0f, 4294967040.0f);
+            flip = flip && ((uint64_t)acc * (uint64_t)Tmax < ((uint64_t)Tf << 32));
+        } else {
+            b = (myrow[pc >> 5] >> (pc & 31)) & 1u;
+        }
+        if (flip) {
+            insert((((2u * ((uint32_t)pc >> 5)) + b) << 5) | ((uint32_t)pc & 31u));
+            n++;
+            if (++k == 8) flush();
+        }
+    };
+    auto finish_row = [&]() {
+        if (k) {
+            for (; k < 8; k++) insert(sentinel);
+            flush();
+        }
+        const bool over = piece > a.cap;
+        a.info[q] = over ? flip_info((uint32_t)(8 * a.cap), (uint32_t)a.cap) : flip_info((uint32_t)n, (uint32_t)piece);
+        if (over) atomicAdd(a.overflow, 1u);
+        d += slots;
+        start_row();
+    };
+    start_row();
+    while (__any(live)) {
+        if (ALIGNED) {
+            const uint4 w = philox_block(a.key, blk++);
+            if (THIN) {
+                const uint32_t u[2] = {w.x, w.z};
+                int rank[2];
+                skip_ranks<2>(rank, tab1, Kt, u, inv_log2q, c0);
+                step(rank[0], w.y);
+                step(rank[1], w.w);
+            } else {
+                const uint32_t u[4] = {w.x, w.y, w.z, w.w};
+                int rank[4];
+                skip_ranks<4>(rank, tab1, Kt, u, inv_log2q, c0);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) step(rank[e], 0u);
+            }
+        } else {
+            const uint32_t u[1] = {chain.next()};
+            const uint32_t acc = THIN ? chain.next() : 0u;
+            int rank[1];
+            skip_ranks<1>(rank, tab1, Kt, u, inv_log2q, c0);
+            step(rank[0], acc);
+        }
+        if (live && pos >= C) finish_row();
+    }
+}
+
+// ---- the table, made on the device from a threshold that lives there ---------------------------------------------------
+// cdf[k - 1] = floor(2^32 (1 - (1 - p)^k)), p = T / 2^32, cdf[0] = T itself, made non-decreasing, cut where it
+// saturates at 2^32 - 1 (at most kSkipMaxTable entries); T == 0: an empty table.  One workgroup of 1024 threads, four
+// entries each.
+__device__ __forceinline__ void skip_table_build(uint32_t *table, const uint32_t *thr)
+{
+    __shared__ uint32_t wave_max[16];
+    __shared__ int first_full;
+    const int t = threadIdx.x, lane = t & 63, wv = t >> 6;
+    const uint32_t T = thr[0];
+    const double p = (double)T / 4294967296.0;
+    if (t == 0) first_full = kSkipMaxTable;   // index of the first saturated entry
+    uint32_t v[4];
+    const double l1p = p < 1.0 ? log1p(-p) : -INFINITY;
+    uint32_t run = 0;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int k = 4 * t + i + 1;
+        double x = floor(-expm1((double)k * l1p) * 4294967296.0);
+        x = x < 4294967295.0 ? x : 4294967295.0;
+        uint32_t e = T == 0 ? 0u : (uint32_t)x;
+        if (k == 1) e = T;
+        run = run > e ? run : e;
+        v[i] = run;
+    }
+    // running maximum across threads: inside the wave, then over the waves before
+    uint32_t incl = run;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const uint32_t up = (uint32_t)__shfl_up((int)incl, o);
+        if (lane >= o) incl = incl > up ? incl : up;
+    }
+    if (lane == 63) wave_max[wv] = incl;
+    __syncthreads();
+    uint32_t before = 0;
+    for (int w = 0; w < wv; w++) before = before > wave_max[w] ? before : wave_max[w];
+    uint32_t prev = (uint32_t)__shfl_up((int)incl, 1);
+    prev = lane == 0 ? 0u : prev;
+    prev = prev > before ? prev : before;   // maximum of everything before this thread's entries
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        v[i] = v[i] > prev ? v[i] : prev;
+        if (v[i] == 0xFFFFFFFFu) atomicMin(&first_full, 4 * t + i);
+        table[kSkipHeader + 4 * t + i] = v[i];
+    }
+    __syncthreads();
+    if (t == 0) {
+        const int Kt = T == 0 ? 0 : (first_full < kSkipMaxTable ? first_full + 1 : kSkipMaxTable);
+        table[0] = (uint32_t)Kt;
+        const float hint = (p > 0.0 && p < 1.0) ? (float)(1.0 / log2(1.0 - p)) : 0.0f;
+        table[1] = __float_as_uint(hint);
+        table[2] = T;
+        table[3] = 0u;
+    }
+}
+
+// ---- the layers' law: weights -> probabilities --------------------------------------------------------------------------
+// P = fp16(sigmoid(float(fp16(fp16(w / m) * 5)))) with m = fp16(mean|w| + 1e-5), every step rounded to fp16 where the
+// tensor expression of modules/binary.py:59-60 rounds it.  mean|w| is the exact sum (fp16 values add exactly in a
+// double) divided by the count and rounded once to fp16.
+constexpr int kLawBlocks = 256;   // partial sums
+
+__global__ __launch_bounds__(256) void law_abs_sum_kernel(double *__restrict__ partial, uint32_t *__restrict__ table,
+                                                          const _Float16 *__restrict__ w, int64_t n)
+{
+    __shared__ double red[4];
+    double s = 0.0;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256)
+        s += (double)fabsf((float)w[i]);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = s;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        partial[blockIdx.x] = red[0] + red[1] + red[2] + red[3];
+        if (blockIdx.x == 0 && table) table[2] = 0u;   // the largest flip threshold is collected there next
+    }
+}
+
+__device__ __forceinline__ _Float16 law_denominator(const double *partial, int nparts, int64_t n)
+{
+    double s = 0.0;
+    for (int i = 0; i < nparts; i++) s += partial[i];   // the same order in every thread: all agree
+    const _Float16 mean = double_round_once_fp16(s / (double)n);
+    return (_Float16)((float)mean + 1e-5f);
+}
+
+__device__ __forceinline__ _Float16 law_probability(_Float16 w, _Float16 denom)
+{
+    const _Float16 qn = (_Float16)((float)w / (float)denom);
+    const _Float16 nw = (_Float16)((float)qn * 5.0f);
+    return (_Float16)(1.0f / (1.0f + expf(-(float)nw)));
+}
+
+__device__ __forceinline__ uint32_t law_threshold(_Float16 p)   // min(floor(p * 2^32), 2^32 - 1); 0 for NaN
+{
+    const float v = (float)p * 4294967296.0f;
+    return v >= 4294967296.0f ? 0xFFFFFFFFu : (v > 0.0f ? (uint32_t)v : 0u);
+}
+
+// MODE 0: out32 = thresholds; 1: out16 = probabilities (fp16)
+template <int MODE>
+__global__ __launch_bounds__(256) void law_dense_kernel(uint32_t *__restrict__ out32, _Float16 *__restrict__ out16,
+                                                        const _Float16 *__restrict__ w, const double *__restrict__ partial,
+                                                        int nparts, int64_t n)
+{
+    const _Float16 denom = law_denominator(partial, nparts, n);
+    NB_FLAT_LOOP(t, n)
+    {
+        if (t < n) {
+            const _Float16 p = law_probability(w[t], denom);
+            if (MODE == 0) out32[t] = law_threshold(p);
+            else out16[t] = p;
+        }
+    }
+}
+
+// Sparse form: law[r, c] = base bit << 15 | fp16 bits of the flip probability y = min(P, 1 - P) (exact in fp16),
+// base[r, :] packed, and the largest flip threshold floor(y * 2^32) of the layer into table[2] (cleared by the sum
+// kernel).  One wave per 64 columns of a row: the ballot of the base bits is the packed word.
+__global__ __launch_bounds__(256) void law_sparse_kernel(uint16_t *__restrict__ law, uint64_t *__restrict__ base,
+                                                         uint32_t *__restrict__ table, const _Float16 *__restrict__ w,
+                                                         const double *__restrict__ partial, int nparts, int64_t R,
+                                                         int C, int Kw)
+{
+    const _Float16 denom = law_denominator(partial, nparts, R * (int64_t)C);
+    const int lane = threadIdx.x & 63;
+    uint32_t tmax = 0;
+    for (int64_t wd = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6); wd < R * Kw; wd += (int64_t)gridDim.x * 4) {
+        const int64_t r = wd / Kw;
+        const int c = (int)(wd - r * Kw) * 64 + lane;
+        bool one = false;
+        if (c < C) {
+            const float p = (float)law_probability(w[r * C + c], denom);
+            one = p >= 0.5f;
+            const _Float16 y = (_Float16)(one ? 1.0f - p : p);   // exact: p is a multiple of 2^-11 from 1/2 on
+            const uint16_t ybits = __builtin_bit_cast(uint16_t, y) & 0x7FFFu;   // NaN weights: some probability, no fault
+            law[r * C + c] = (uint16_t)(ybits | (one ? 0x8000u : 0u));
+            const uint32_t tf = (uint32_t)fminf((float)__builtin_bit_cast(_Float16, ybits) * 4294967296.0f, 4294967040.0f);
+            tmax = tmax > tf ? tmax : tf;
+        }
+        const unsigned long long word = __ballot(one);
+        if (lane == 0) base[wd] = word;
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const uint32_t other = (uint32_t)__shfl_xor((int)tmax, o);
+        tmax = tmax > other ? tmax : other;
+    }
+    if (lane == 0 && tmax) atomicMax(table + 2, tmax);
+}
+
+// thr may be table + 2 (the threshold read before anything is written, and written back unchanged)
+__global__ __launch_bounds__(1024) void fl_skip_table_kernel(uint32_t *table, const uint32_t *thr)
+{
+    skip_table_build(table, thr);
+}
+
+static int gen_launch(GenArgs a, bool thin, hipStream_t s, const char *who)
+{
+    const bool aligned = a.C % 4 == 0 && a.key.first % 4 == 0;
+    // rows per workgroup: eight (a 128-byte line of every piece) where LDS holds them
+    const size_t tab_bytes = (size_t)(kSkipMaxTable + 2) * 4;
+    const size_t row_bytes = thin ? (size_t)((a.C + 1) / 2) * 4 : (size_t)a.Kw * 8;
+    int shift = 3;
+    while (shift > 0 && tab_bytes + (row_bytes << shift) > 150 * 1024) shift--;
+    NB_REQUIRE(tab_bytes + (row_bytes << shift) <= 150 * 1024, "%s: a row of %d columns does not fit LDS", who, a.C);
+    a.rb_shift = shift;
+    const size_t lds = tab_bytes + (row_bytes << shift);
+    // large workgroups when the rows fill LDS (one workgroup per compute unit then), else four waves each
+    const int threads = lds > 40 * 1024 ? 1024 : 256;
+    const int slots = threads >> shift;
+    // about eight members per lane, so that a wave does not wait long for its slowest lane at the end
+    int64_t MC = (int64_t)slots * 8;
+    if (MC > a.D) MC = ceil_div(a.D, slots) * slots;
+    a.MC = (int)MC;
+    const int64_t nrg = ceil_div(a.R, (int64_t)1 << shift), nmc = ceil_div(a.D, MC);
+    NB_REQUIRE(nrg * nmc <= kMaxGridX, "%s: too many rows for one launch", who);
+    static std::once_flag once;
+    static hipError_t attr = hipSuccess;
+    std::call_once(once, [] {
+        const void *fns[4] = {reinterpret_cast<const void *>(fl_gen_kernel<false, false>),
+                              reinterpret_cast<const void *>(fl_gen_kernel<false, true>),
+                              reinterpret_cast<const void *>(fl_gen_kernel<true, false>),
+                              reinterpret_cast<const void *>(fl_gen_kernel<true, true>)};
+        for (const void *f : fns) {
+            const hipError_t e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
+            if (e != hipSuccess) attr = e;
+        }
+    });
+    if (attr != hipSuccess) {
+        (void)hipGetLastError();
+        return fail(NB_ERR_UNSUPPORTED, "%s: cannot raise the kernel's LDS limit: %s", who, hipGetErrorString(attr));
+    }
+    const dim3 grid((unsigned)(nrg * nmc)), block((unsigned)threads);
+    if (aligned && thin) fl_gen_kernel<true, true><<<grid, block, lds, s>>>(a);
+    else if (aligned) fl_gen_kernel<true, false><<<grid, block, lds, s>>>(a);
+    else if (thin) fl_gen_kernel<false, true><<<grid, block, lds, s>>>(a);
+    else fl_gen_kernel<false, false><<<grid, block, lds, s>>>(a);
+    return check_launch(who);
+}
+
+static int gen_check(const uint32_t *entries, const uint32_t *info, const uint32_t *overflow, const void *rows,
+                     const uint32_t *table, int64_t D, int64_t R, int64_t C, int64_t cap, const char *who)
+{
+    NB_REQUIRE(D >= 0 && R >= 0 && C >= 0, "%s: negative shape D=%lld R=%lld C=%lld", who, (long long)D, (long long)R,
+               (long long)C);
+    const int64_t Kw = (C + 63) / 64;
+    NB_REQUIRE(Kw <= 511, "%s: rows of %lld words, at most 511", who, (long long)Kw);
+    NB_REQUIRE(R <= 65536, "%s: %lld rows per member, at most 65536", who, (long long)R);
+    NB_REQUIRE(D * ((R + 63) / 64) <= (1LL << 31) && D * R < (1LL << 40), "%s: too many rows", who);
+    NB_REQUIRE(cap >= 0 && cap <= 8191, "%s: %lld pieces per row, at most 8191", who, (long long)cap);
+    NB_REQUIRE(D * ((R + 63) / 64) * std::max<int64_t>(cap, 1) < (1LL << 36), "%s: lists too large", who);
+    if (D * R == 0) return NB_OK;
+    NB_REQUIRE_PTR(info);
+    NB_REQUIRE_PTR(overflow);
+    NB_REQUIRE_PTR(table);
+    NB_REQUIRE_ALIGNED(info, 4);
+    NB_REQUIRE_ALIGNED(overflow, 4);
+    NB_REQUIRE_ALIGNED(table, 4);
+    if (cap > 0) NB_REQUIRE_PTR(entries);
+    NB_REQUIRE_ALIGNED(entries, 16);
+    if (C > 0) NB_REQUIRE_PTR(rows);
+    return NB_OK;
+}
+
+}  // namespace nb
+
+extern "C" {
+int64_t nb_skip_table_words(void) { return nb::kSkipTableWords; }
+
+int nb_skip_table(uint32_t *table, const uint32_t *threshold, nb_stream_t stream)
+{
+    const char *who = "nb_skip_table";
+    NB_REQUIRE_PTR(table);
+    NB_REQUIRE_PTR(threshold);
+    NB_REQUIRE_ALIGNED(table, 4);
+    NB_REQUIRE_ALIGNED(threshold, 4);
+    nb::fl_skip_table_kernel<<<dim3(1), dim3(1024), 0, nb::as_stream(stream)>>>(table, threshold);
+    return nb::check_launch(who);
+}
+
+int nb_flip_skip_i64(uint32_t *entries, uint32_t *info, uint32_t *overflow, const int64_t *base, const uint32_t *table,
+                     uint64_t seed, uint64_t subseq, uint64_t first, int64_t D, int64_t R, int64_t C, int64_t cap,
+                     nb_stream_t stream)
+{
+    const char *who = "nb_flip_skip_i64";
+    if (int rc = nb::gen_check(entries, info, overflow, base, table, D, R, C, cap, who)) return rc;
+    if (D * R == 0) return NB_OK;
+    NB_REQUIRE_ALIGNED(base, 8);
+    nb::GenArgs a{};
+    a.entries = reinterpret_cast<uint4 *>(entries);
+    a.info = info;
+    a.overflow = overflow;
+    a.rows = base;
+    a.table = table;
+    a.key = nb::PhiloxKey{seed, subseq, first};
+    a.D = D;
+    a.R = R;
+    a.C = (int)C;
+    a.Kw = (int)((C + 63) / 64);
+    a.S = (int)((R + 63) / 64);
+    a.cap = (int)cap;
+    return nb::gen_launch(a, false, nb::as_stream(stream), who);
+}
+
+int nb_flip_skip_thin_i64(uint32_t *entries, uint32_t *info, uint32_t *overflow, const uint16_t *law,
+                          const uint32_t *table, uint64_t seed, uint64_t subseq, uint64_t first, int64_t D, int64_t R,
+                          int64_t C, int64_t cap, nb_stream_t stream)
+{
+    const char *who = "nb_flip_skip_thin_i64";
+    if (int rc = nb::gen_check(entries, info, overflow, law, table, D, R, C, cap, who)) return rc;
+    if (D * R == 0) return NB_OK;
+    NB_REQUIRE_ALIGNED(law, 2);
+    nb::GenArgs a{};
+    a.entries = reinterpret_cast<uint4 *>(entries);
+    a.info = info;
+    a.overflow = overflow;
+    a.rows = law;
+    a.table = table;
+    a.key = nb::PhiloxKey{seed, subseq, first};
+    a.D = D;
+    a.R = R;
+    a.C = (int)C;
+    a.Kw = (int)((C + 63) / 64);
+    a.S = (int)((R + 63) / 64);
+    a.cap = (int)cap;
+    return nb::gen_launch(a, true, nb::as_stream(stream), who);
+}
+
+int64_t nb_law_workspace_bytes(void) { return nb::kLawBlocks * 8; }
+
+static int law_sum(double *ws, uint32_t *table, const uint16_t *w, int64_t n, hipStream_t s, int *nparts,
+                   const char *who)
+{
+    NB_REQUIRE_PTR(ws);
+    NB_REQUIRE_ALIGNED(ws, 8);
+    NB_REQUIRE_PTR(w);
+    NB_REQUIRE_ALIGNED(w, 2);
+    const int64_t blocks = std::min<int64_t>(nb::kLawBlocks, nb::ceil_div(n, 2048));
+    *nparts = (int)blocks;
+    nb::law_abs_sum_kernel<<<dim3((unsigned)blocks), dim3(256), 0, s>>>(ws, table, reinterpret_cast<const _Float16 *>(w), n);
+    return nb::check_launch(who);
+}
+
+int nb_thresholds_from_weights(uint32_t *thresholds, const uint16_t *weights, int64_t n, void *workspace,
+                               nb_stream_t stream)
+{
+    const char *who = "nb_thresholds_from_weights";
+    NB_REQUIRE(n >= 0 && n < (1LL << 40), "%s: bad element count %lld", who, (long long)n);
+    if (n == 0) return NB_OK;
+    NB_REQUIRE_PTR(thresholds);
+    NB_REQUIRE_ALIGNED(thresholds, 4);
+    int nparts = 0;
+    if (int rc = law_sum(static_cast<double *>(workspace), nullptr, weights, n, nb::as_stream(stream), &nparts, who))
+        return rc;
+    nb::law_dense_kernel<0><<<dim3(nb::grid_for(n)), dim3(256), 0, nb::as_stream(stream)>>>(
+        thresholds, nullptr, reinterpret_cast<const _Float16 *>(weights), static_cast<const double *>(workspace), nparts, n);
+    return nb::check_launch(who);
+}
+
+int nb_probabilities_from_weights(uint16_t *p, const uint16_t *weights, int64_t n, void *workspace, nb_stream_t stream)
+{
+    const char *who = "nb_probabilities_from_weights";
+    NB_REQUIRE(n >= 0 && n < (1LL << 40), "%s: bad element count %lld", who, (long long)n);
+    if (n == 0) return NB_OK;
+    NB_REQUIRE_PTR(p);
+    NB_REQUIRE_ALIGNED(p, 2);
+    int nparts = 0;
+    if (int rc = law_sum(static_cast<double *>(workspace), nullptr, weights, n, nb::as_stream(stream), &nparts, who))
+        return rc;
+    nb::law_dense_kernel<1><<<dim3(nb::grid_for(n)), dim3(256), 0, nb::as_stream(stream)>>>(
+        nullptr, reinterpret_cast<_Float16 *>(p), reinterpret_cast<const _Float16 *>(weights),
+        static_cast<const double *>(workspace), nparts, n);
+    return nb::check_launch(who);
+}
+
+int nb_flip_law_from_weights(uint16_t *law, int64_t *base, uint32_t *table, const uint16_t *weights, int64_t R, int64_t C,
+                             void *workspace, nb_stream_t stream)
+{
+    const char *who = "nb_flip_law_from_weights";
+    NB_REQUIRE(R >= 0 && C >= 0 && R * C < (1LL << 40) && C <= 511 * 64, "%s: bad shape R=%lld C=%lld", who, (long long)R,
+               (long long)C);
+    NB_REQUIRE_PTR(table);
+    NB_REQUIRE_ALIGNED(table, 4);
+    NB_REQUIRE(R * C > 0, "%s: empty layer", who);
+    NB_REQUIRE_PTR(law);
+    NB_REQUIRE_PTR(base);
+    NB_REQUIRE_ALIGNED(law, 2);
+    NB_REQUIRE_ALIGNED(base, 8);
+    const int64_t Kw = (C + 63) / 64;
+    int nparts = 0;
+    if (int rc = law_sum(static_cast<double *>(workspace), table, weights, R * C, nb::as_stream(stream), &nparts, who))
+        return rc;
+    const int64_t blocks = std::min<int64_t>(nb::ceil_div(R * Kw, 4), 65536);
+    nb::law_sparse_kernel<<<dim3((unsigned)blocks), dim3(256), 0, nb::as_stream(stream)>>>(
+        law, reinterpret_cast<uint64_t *>(base), table, reinterpret_cast<const _Float16 *>(weights),
+        static_cast<const double *>(workspace), nparts, R, (int)C, (int)Kw);
+    if (int rc = nb::check_launch(who)) return rc;
+    nb::fl_skip_table_kernel<<<dim3(1), dim3(1024), 0, nb::as_stream(stream)>>>(table, table + 2);
+    return nb::check_launch(who);
+}
+}

@@ -52,17 +52,20 @@ __global__ __launch_bounds__(256) void bn_colsum_kernel(unsigned long long *__re
     atomicAdd(colsum + m, s);
 }
 
-// act = 2*popc - K against thr = fp16(fp16(bias + bias_noise) + mean), mean = fp16(float(sum of act) / float(Z)).
+// act = 2*popc - K against thr = fp16(fp16(bias + bias_noise) + mean), mean = fp16(float(sum of act) * factor), the
+// exact product rounded once, with factor = float(M) / float(Z * M): torch's fp16 mean accumulates in fp32 and
+// multiplies by that quotient of the output and input element counts, so this is its result whenever the fp32 sum
+// is exact (up to 2^24 in magnitude).
 // act is an integer and thr an fp16 number, so act > thr <=> act > floor(thr) (never for NaN).
 // ROUND: total is the sum of the fp16-rounded activations, and the activation is rounded to fp16 for the compare as
 // well (torch compares an int32 tensor with an fp16 one in fp16): the reference's arithmetic for rows of more than
 // 2048 bits, where 2*popc - K is no longer exact in fp16.
 template <bool ROUND>
 __device__ __forceinline__ bool bn_bit(int32_t popc, unsigned long long total, _Float16 bias, _Float16 noise, int64_t Z,
-                                       int64_t K)
+                                       int64_t K, float factor)
 {
     const long long sum_act = ROUND ? (long long)total : 2ll * (long long)total - (long long)K * (long long)Z;
-    const _Float16 mean = (_Float16)((float)sum_act / (float)Z);
+    const _Float16 mean = mul_round_once_fp16((float)sum_act, factor);
     const _Float16 tb = bias + noise;
     const float t = (float)(_Float16)(tb + mean);
     if (t != t) return false;
@@ -77,13 +80,13 @@ __global__ __launch_bounds__(256) void bn_bool_kernel(uint8_t *__restrict__ out,
                                                       const unsigned long long *__restrict__ colsum,
                                                       const _Float16 *__restrict__ bias,
                                                       const _Float16 *__restrict__ noise, int64_t Z, int64_t M,
-                                                      int64_t K)
+                                                      int64_t K, float factor)
 {
     NB_FLAT_LOOP(t, Z * M)
     {
         if (t < Z * M) {
             const int64_t m = t % M;
-            out[t] = bn_bit<ROUND>(popc[t], colsum[m], bias[m], noise[t], Z, K) ? 1 : 0;
+            out[t] = bn_bit<ROUND>(popc[t], colsum[m], bias[m], noise[t], Z, K, factor) ? 1 : 0;
         }
     }
 }
@@ -94,7 +97,7 @@ __global__ __launch_bounds__(256) void bn_pack_kernel(W *__restrict__ out, const
                                                       const unsigned long long *__restrict__ colsum,
                                                       const _Float16 *__restrict__ bias,
                                                       const _Float16 *__restrict__ noise, int64_t Z, int64_t M,
-                                                      int64_t Mw, int64_t K)
+                                                      int64_t Mw, int64_t K, float factor)
 {
     constexpr int bits = WordTraits<W>::bits;
     const int lane = threadIdx.x & 63;
@@ -103,7 +106,7 @@ __global__ __launch_bounds__(256) void bn_pack_kernel(W *__restrict__ out, const
     const int64_t z = wd / Mw;
     const int64_t m = (wd - z * Mw) * bits + lane;
     bool bit = false;
-    if (lane < bits && m < M) bit = bn_bit<ROUND>(popc[z * M + m], colsum[m], bias[m], noise[z * M + m], Z, K);
+    if (lane < bits && m < M) bit = bn_bit<ROUND>(popc[z * M + m], colsum[m], bias[m], noise[z * M + m], Z, K, factor);
     const unsigned long long word = __ballot(bit);
     if (lane == 0) out[wd] = (W)word;
 }
@@ -164,18 +167,19 @@ static int bn_impl(void *out, const W *A, const W *x, const uint16_t *bias, cons
         bn_colsum_kernel<false><<<cgrid, dim3(256), 0, s>>>(colsum, popc, Z, M, K);
     if (int rc2 = check_launch(who)) return rc2;
     const auto *b16 = reinterpret_cast<const _Float16 *>(bias), *n16 = reinterpret_cast<const _Float16 *>(noise);
+    const float factor = mean_factor(M, Z * M);
     if (pack) {
         const dim3 pgrid((unsigned)ceil_div(Z * Mw, 4));
         if (round16)
-            bn_pack_kernel<W, true><<<pgrid, dim3(256), 0, s>>>(static_cast<W *>(out), popc, colsum, b16, n16, Z, M, Mw, K);
+            bn_pack_kernel<W, true><<<pgrid, dim3(256), 0, s>>>(static_cast<W *>(out), popc, colsum, b16, n16, Z, M, Mw, K, factor);
         else
-            bn_pack_kernel<W, false><<<pgrid, dim3(256), 0, s>>>(static_cast<W *>(out), popc, colsum, b16, n16, Z, M, Mw, K);
+            bn_pack_kernel<W, false><<<pgrid, dim3(256), 0, s>>>(static_cast<W *>(out), popc, colsum, b16, n16, Z, M, Mw, K, factor);
     } else {
         const dim3 bgrid(grid_for(Z * M));
         if (round16)
-            bn_bool_kernel<true><<<bgrid, dim3(256), 0, s>>>(static_cast<uint8_t *>(out), popc, colsum, b16, n16, Z, M, K);
+            bn_bool_kernel<true><<<bgrid, dim3(256), 0, s>>>(static_cast<uint8_t *>(out), popc, colsum, b16, n16, Z, M, K, factor);
         else
-            bn_bool_kernel<false><<<bgrid, dim3(256), 0, s>>>(static_cast<uint8_t *>(out), popc, colsum, b16, n16, Z, M, K);
+            bn_bool_kernel<false><<<bgrid, dim3(256), 0, s>>>(static_cast<uint8_t *>(out), popc, colsum, b16, n16, Z, M, K, factor);
     }
     return check_launch(who);
 }
@@ -212,18 +216,19 @@ static int bn_static_ptr(void **ptr, const char *who)
 __global__ __launch_bounds__(256) void bn_conv_thresh_kernel(int32_t *thresh, const int32_t *sums,
                                                              const _Float16 *__restrict__ bias,
                                                              const _Float16 *__restrict__ noise, int64_t D, int64_t O,
-                                                             int64_t K, int64_t HW)
+                                                             int64_t K, int64_t HW, float factor)
 {
     NB_FLAT_LOOP(t, D * O)
     {
-        if (t < D * O) thresh[t] = bn_conv_threshold(sums[t], bias[t % O], noise[t], K, HW);
+        if (t < D * O) thresh[t] = bn_conv_threshold(sums[t], bias[t % O], noise[t], K, HW, factor);
     }
 }
 
 void bn_conv_thresh_launch(int32_t *thresh, const int32_t *sums, const _Float16 *bias, const _Float16 *noise, int64_t D,
                            int64_t O, int64_t K, int64_t HW, hipStream_t s)
 {
-    bn_conv_thresh_kernel<<<dim3(grid_for(D * O)), dim3(256), 0, s>>>(thresh, sums, bias, noise, D, O, K, HW);
+    bn_conv_thresh_kernel<<<dim3(grid_for(D * O)), dim3(256), 0, s>>>(thresh, sums, bias, noise, D, O, K, HW,
+                                                                      mean_factor(D * O, D * O * HW));
 }
 
 }  // namespace nb

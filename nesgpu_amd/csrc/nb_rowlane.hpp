@@ -91,7 +91,8 @@ struct ConvA {
 // Implicit im2col with TAP PACKING for narrow channels (Cw == 1, tap_bits = true channel count <= bits/2):
 // T = bits / tap_bits taps share one word, word w of an output pixel is OR_t tap(w*T + t) << (tap_bits*t).
 // The filter must be packed the same way (tap_pack_filter_kernel).  The popcount sum is unchanged because
-// both operands are zero above tap_bits (extensions/src/pack.cu:17) and an out-of-range tap is the zero word.
+// both operands are zero above tap_bits (extensions/src/pack.cu:17; input bits above them are masked off here, so a
+// stray bit counts for nothing, as in the matrix-core kernels) and an out-of-range tap is the zero word.
 template <typename W>
 struct ConvTapA {
     const W *__restrict__ in;
@@ -111,6 +112,7 @@ struct ConvTapA {
     __device__ __forceinline__ void load(const Lane &l, int k0, W (&a)[KC]) const
     {
         const int taps = g.fx * g.fy;
+        const W cmask = (W)(((W)1 << tap_bits) - 1);
         int tap = k0 * T;
         int ti = tap / g.fy;
         int tj = tap - ti * g.fy;
@@ -120,7 +122,7 @@ struct ConvTapA {
             for (int t = 0; t < T && tap < taps; t++, tap++) {
                 const int y = l.y0 + ti, x = l.x0 + tj;
                 const bool ok = l.valid && y >= 0 && y < g.H && x >= 0 && x < g.Wd;
-                const W v = ok ? l.img[(int64_t)y * g.Wd + x] : (W)0;
+                const W v = ok ? (l.img[(int64_t)y * g.Wd + x] & cmask) : (W)0;
                 wv |= v << (tap_bits * t);
                 if (++tj == g.fy) {
                     tj = 0;

@@ -15,6 +15,8 @@ half of the reference (extensions/booleanOperations.cpp:13-15) -- non-CUDA or no
 Additions that the reference lacks are grouped at the end (supplied-word / Philox sampling, the fused
 sample+popcount product with a flip base, the fused conv->threshold->pack(->pool) op).
 """
+import math
+
 import torch
 
 from .. import _lib
@@ -123,7 +125,12 @@ def batch_im2col(input, filterx, filtery, padx, pady, stridex, stridey, REPEAT=1
 
 
 def bmm(A, B):
-    """C[z,x,y] = sum_k popcount(A[z,x,k] ^ B[z,k,y]), int32 (extensions/booleanOperations.py:107-129)."""
+    """C[z,x,y] = sum_k popcount(A[z,x,k] ^ B[z,k,y]), int32 (extensions/booleanOperations.py:107-129).
+    ``A`` may be a :class:`FlipRows` (a population's weights as base + flip lists) with ``B`` [Z, Kw, 1]: the same
+    sums from the sparse form."""
+    if isinstance(A, FlipRows):
+        assert len(B.shape) == 3 and B.size(0) == A.D and B.size(1) == A.Kw and B.size(2) == 1
+        return bmv_flip(A, B.view(A.D, A.Kw)).unsqueeze(2)
     sa, sb = A.shape, B.shape
     assert len(sa) == 3
     assert len(sb) == 3
@@ -167,7 +174,10 @@ def bmv_act_pack(A, x, threshold):
     """One input row per member, as the linear layers have it: A [Z,M,Kw] packed weights, x [Z,Kw] (or [Z,Kw,1])
     packed inputs, threshold [Z,M] int32 -> packed bits (2*popc(A[z,m] ^ x[z]) > threshold[z,m]) as [Z, ceil(M/bits)]
     words.  Not in the reference: it is ``pack(2 * bmm(A, x) > threshold)`` (the compare of
-    modules/binary.py:97-106 and the next layer's pack) in one kernel, without the int32 and bool maps."""
+    modules/binary.py:97-106 and the next layer's pack) in one kernel, without the int32 and bool maps.  ``A`` may be
+    a :class:`FlipRows`."""
+    if isinstance(A, FlipRows):
+        return bmv_flip_act_pack(A, x, threshold)
     _check(A, "A")
     _check(x, "x")
     _check(threshold, "threshold")
@@ -190,7 +200,8 @@ def bmv_bn_act(A, x, bias, bias_noise, in_bits, pack=False, workspace=None, roun
     """Linear layer with the population-mean threshold in one call (not in the reference as an op: it is the
     composition of modules/binary.py:97-102).  A [Z,M,Kw] packed weights, x [Z,Kw] (or [Z,Kw,1]) packed inputs, bias [M]
     and bias_noise [Z,M] fp16, ``in_bits`` the true bit count K of a row.  With act = 2*popc - K:
-    thr[z,m] = fp16(fp16(bias + bias_noise) + fp16(float(sum_z act[z,m]) / Z)), result = act > thr as bool [Z,M], or with
+    thr[z,m] = fp16(fp16(bias + bias_noise) + fp16(float(sum_z act[z,m]) * (float(M) / float(Z*M)))) (torch's fp16
+    mean: fp32 sum times the fp32 quotient of the element counts, the exact product rounded once), result = act > thr as bool [Z,M], or with
     ``pack`` packed along M into [Z, ceil(M/bits)] words.  ``workspace`` (uint8 CUDA tensor) is allocated when absent.
     ``round_fp16``: act is rounded to fp16 before the mean and the compare, as the reference's tensor expression does
     (``activation.type(torch.float16).mean(dim=0)``, then an int32 tensor compared with an fp16 one); it only matters
@@ -231,7 +242,8 @@ def bmv_bn_act(A, x, bias, bias_noise, in_bits, pack=False, workspace=None, roun
 
 def conv_bn_thresholds(sums, bias, bias_noise, in_bits, pixels):
     """Thresholds of ``BinarizedConv2d(batch_norm=True)`` (modules/binary.py:147-155) from ``conv_popc_sums``: with
-    act = 2*popc - in_bits, mean = fp16(float(sum over the pixels of act) / pixels),
+    act = 2*popc - in_bits, mean = fp16(float(sum over the pixels of act) * (float(D*O) / float(D*O*pixels))) (torch's
+    fp16 mean over the pixels of a [D,h,w,O] map),
     thr = fp16(fp16(bias + bias_noise) + mean); returns int32 [D,O] = floor(thr) + in_bits (INT32_MAX for NaN), the
     threshold of ``conv_act`` / ``conv_act_pack`` (2*popc > threshold).  sums int32 [D,O], bias fp16 [O], bias_noise
     fp16 [D,O].  One kernel instead of a dozen elementwise tensor operations."""
@@ -449,7 +461,10 @@ def sample_bits(p, n, dtype, seed, conv_taps=None):
 
 def weighted_sum(input, weights, zbits):
     """ret[r,z] = fp16(sum_m weights[m] * bit(input[m,r,z/bits], z%bits)), fp32 accumulation
-    (extensions/booleanOperations.py:218-229, extensions/src/weighted_sum.cu:28-46)."""
+    (extensions/booleanOperations.py:218-229, extensions/src/weighted_sum.cu:28-46).  ``input`` may be a
+    :class:`FlipRows` (see :func:`weighted_sum_flip`)."""
+    if isinstance(input, FlipRows):
+        return weighted_sum_flip(input, weights, zbits)
     assert len(input.shape) == 3
     assert input.size(0) == weights.size(0)
     _check(input, "input")
@@ -728,39 +743,67 @@ def bmm_nt(A, B):
 
 class FlipRows:
     """Per-member weights of a linear layer, W[d] = base ^ flips[d], kept as the shared base and per-member flip
-    lists (layout in include/nesbin.h).  Built by :func:`flip_rows_from_weights`; consumed by :func:`bmv_flip` and
-    :func:`bmv_flip_act_pack`, which return what ``bmm`` / ``bmv_act_pack`` return on the materialised weights."""
+    lists (layout in include/nesbin.h: every row owns ``cap`` 16-byte pieces at a fixed place, ``info[d, r]`` says how
+    many flips and pieces it has).  Built by :func:`flip_rows_from_weights`, :func:`flip_rows_skip` or
+    :func:`flip_rows_thin`; ``bmm`` / ``bmv_act_pack`` / ``weighted_sum`` accept it where they take materialised
+    weights, and return what they return on those."""
 
-    def __init__(self, base, D, R, Kw, cnt, perm, slice_off, slice_len, entries):
-        self.base, self.D, self.R, self.Kw = base, D, R, Kw
-        self.cnt, self.perm, self.slice_off, self.slice_len, self.entries = cnt, perm, slice_off, slice_len, entries
+    def __init__(self, base, D, R, Kw, in_bits, info, entries, cap, overflow):
+        self.base, self.D, self.R, self.Kw, self.in_bits = base, D, R, Kw, in_bits
+        self.info, self.entries, self.cap, self.overflow = info, entries, cap, overflow
         self.base_expanded = expand_rows(base)
 
+    @property
+    def cnt(self):
+        """Flips per row, int32 [D, R]."""
+        return (self.info.view(torch.int32) & 0xFFFF)
+
+    def overflowed(self):
+        """Rows whose lists did not fit ``cap`` pieces (a device read-back; such rows were cut short)."""
+        return int(self.overflow.item())
+
+    # what the reference's layer code asks of weight_noise (modules/binary.py:97)
+    def size(self, dim=None):
+        shape = (self.D, self.R, self.Kw)
+        return shape if dim is None else shape[dim]
+
+    @property
+    def shape(self):
+        return (self.D, self.R, self.Kw)
+
+    @property
+    def dtype(self):
+        return torch.int64
+
+    @property
+    def device(self):
+        return self.base.device
+
     def nbytes(self):
-        """Bytes one forward reads of the member-specific data (flip lists, counts, row order, slice tables)."""
-        return sum(t.numel() * t.element_size() for t in (self.entries, self.cnt, self.perm, self.slice_off,
-                                                           self.slice_len))
+        """Bytes one forward reads of the member-specific data (the pieces the rows have, and info)."""
+        pieces = int((self.info.view(torch.int32) >> 16).sum().item())
+        return pieces * 16 + self.info.numel() * 4
 
 
-def _flip_rows_layout(cnt, D, R):
-    """Flip counts [D, R] (uint16) -> (perm, slice_len, slice_off, total dwords): rows ordered by count inside blocks
-    of 1024 rows, slices of 64 rows padded to their longest row in 16-byte pieces of 8 flips."""
-    dev = cnt.device
+def _flip_alloc(D, R, cap, dev):
     S = ceil_div(R, 64)
-    perm = torch.empty((D, R), dtype=torch.uint16, device=dev)
-    slice_len = torch.empty((D, S), dtype=torch.int32, device=dev)
-    slice_off = torch.empty((D, S), dtype=torch.int64, device=dev)
-    total = torch.empty((1,), dtype=torch.int64, device=dev)
-    with _on(cnt):
-        _lib.call("nb_flip_layout", perm.data_ptr(), slice_len.data_ptr(), slice_off.data_ptr(), total.data_ptr(),
-                  cnt.data_ptr(), D, R, _stream(cnt))
-    return perm, slice_len, slice_off, int(total.item())     # the one read-back: entries is sized by it
+    entries = torch.empty((max(D * S * cap * 256, 4),), dtype=torch.uint32, device=dev)
+    info = torch.empty((D, R), dtype=torch.uint32, device=dev)
+    overflow = torch.zeros((1,), dtype=torch.int32, device=dev).view(torch.uint32)
+    return entries, info, overflow
 
 
-def flip_rows_from_weights(W, base):
+def flip_capacity(in_bits, p, sigmas=8.0):
+    """16-byte pieces per row that hold the flips of a row of ``in_bits`` columns at flip probability ``p`` with
+    ``sigmas`` standard deviations to spare (a row beyond it is cut short and counted in ``FlipRows.overflow``)."""
+    mean = in_bits * p
+    need = mean + sigmas * math.sqrt(max(mean * (1.0 - p), 1.0)) + 8
+    return int(min(ceil_div(int(math.ceil(min(need, in_bits))), 8), 8191))
+
+
+def flip_rows_from_weights(W, base, cap=None):
     """W int64 [D, R, Kw] (a population's materialised weights), base int64 [R, Kw] -> :class:`FlipRows` holding
-    exactly the bits W ^ base.  Rows are ordered by flip count inside blocks of 1024 rows so that the 64 rows of a
-    slice are about equally long."""
+    exactly the bits W ^ base.  ``cap`` (pieces per row) defaults to what the longest row needs (one read-back)."""
     _check(W, "W")
     _check(base, "base")
     _same_device(W, base)
@@ -770,15 +813,16 @@ def flip_rows_from_weights(W, base):
     D, R, Kw = W.shape
     assert tuple(base.shape) == (R, Kw)
     dev = W.device
-    cnt = torch.empty((D, R), dtype=torch.uint16, device=dev)
+    if cap is None:
+        info = torch.empty((D, R), dtype=torch.uint32, device=dev)
+        with _on(W):
+            _lib.call("nb_flip_count_i64", info.data_ptr(), W.data_ptr(), base.data_ptr(), D, R, Kw, _stream(W))
+        cap = int((info.view(torch.int32) >> 16).max().item()) if D * R else 0
+    entries, info, overflow = _flip_alloc(D, R, int(cap), dev)
     with _on(W):
-        _lib.call("nb_flip_count_i64", cnt.data_ptr(), W.data_ptr(), base.data_ptr(), D, R, Kw, _stream(W))
-    perm, slice_len, slice_off, total = _flip_rows_layout(cnt, D, R)
-    entries = torch.empty((max(total, 4),), dtype=torch.uint32, device=dev)
-    with _on(W):
-        _lib.call("nb_flip_fill_i64", entries.data_ptr(), W.data_ptr(), base.data_ptr(), perm.data_ptr(),
-                  slice_off.data_ptr(), slice_len.data_ptr(), D, R, Kw, _stream(W))
-    return FlipRows(base, D, R, Kw, cnt, perm, slice_off, slice_len, entries)
+        _lib.call("nb_flip_fill_i64", entries.data_ptr(), info.data_ptr(), overflow.data_ptr(), W.data_ptr(),
+                  base.data_ptr(), D, R, Kw, int(cap), _stream(W))
+    return FlipRows(base, D, R, Kw, 64 * Kw, info, entries, int(cap), overflow)
 
 
 def skip_table(threshold, cap=4096):
@@ -802,12 +846,45 @@ def skip_table(threshold, cap=4096):
     return v[:n].astype(np.uint32)
 
 
-def flip_rows_skip(base, in_bits, n, threshold, seed, subsequence=0, first=0):
+_skip_tables = {}
+
+
+def skip_table_buffer(table, device):
+    """A gap table (uint32 numpy array, see :func:`skip_table`) as the kernels take it, in device memory:
+    [entries, bits of the float 1 / log2(1 - p), p * 2**32, 0, table...]."""
+    import numpy as np
+    words = int(_lib.load().nb_skip_table_words())
+    buf = np.zeros(words, dtype=np.uint32)
+    n = int(table.size)
+    assert n <= words - 4
+    buf[0] = n
+    p = (float(table[0]) / 4294967296.0) if n else 0.0
+    hint = np.float32(1.0 / math.log2(1.0 - p)) if 0.0 < p < 1.0 else np.float32(0.0)
+    buf[1] = np.frombuffer(hint.tobytes(), dtype=np.uint32)[0]
+    buf[2] = table[0] if n else 0
+    buf[4:4 + n] = table
+    return torch.from_numpy(buf.view(np.int32)).to(device).view(torch.uint32)
+
+
+def _skip_table_for(threshold, device):
+    """The device table for a host threshold, made once per (threshold, device)."""
+    key = (int(threshold), str(device))
+    buf = _skip_tables.get(key)
+    if buf is None:
+        if len(_skip_tables) > 64:
+            _skip_tables.clear()
+        buf = _skip_tables[key] = skip_table_buffer(skip_table(threshold), device)
+    return buf
+
+
+def flip_rows_skip(base, in_bits, n, threshold, seed, subsequence=0, first=0, cap=None, table=None):
     """:class:`FlipRows` for ``n`` members drawn by the skip sampler: every bit of a member's [R, in_bits] weights
     differs from ``base`` with probability threshold / 2**32, independently, as with :func:`flip_philox`, but the
     generator only draws the gaps between flips (about in_bits * p + 1 words per row instead of in_bits), and the
     materialised weights never exist.  Row q = m*R + r consumes the Philox words first + q*in_bits + i of the stream
-    (seed, subsequence).  The stream differs from :func:`flip_philox`'s: the law is the same, the bits are not."""
+    (seed, subsequence).  The stream differs from :func:`flip_philox`'s: the law is the same, the bits are not.
+    One kernel and nothing read back; ``cap``: pieces per row (default :func:`flip_capacity` of the probability);
+    ``table``: a device table from :func:`skip_table_buffer` (default: made from ``threshold`` and kept)."""
     _check(base, "base")
     assert len(base.shape) == 2
     if base.dtype != torch.int64:
@@ -816,20 +893,96 @@ def flip_rows_skip(base, in_bits, n, threshold, seed, subsequence=0, first=0):
     C = int(in_bits)
     assert ceil_div(C, 64) == Kw
     dev = base.device
-    table = skip_table(threshold)
-    cdf = torch.from_numpy(table.view("int32").copy()).to(dev).view(torch.uint32) if table.size else None
-    cptr, Kt = (cdf.data_ptr(), int(table.size)) if cdf is not None else (None, 0)
-    cdf0 = int(table[0]) if table.size else 0
-    cnt = torch.empty((n, R), dtype=torch.uint16, device=dev)
-    key = (int(seed) & (2 ** 64 - 1), int(subsequence), int(first))
+    t = int(threshold)
+    if table is None:
+        table = _skip_table_for(t, dev)
+    if cap is None:
+        cap = flip_capacity(C, t / 4294967296.0)
+    entries, info, overflow = _flip_alloc(n, R, int(cap), dev)
     with _on(base):
-        _lib.call("nb_flip_skip_count_i64", cnt.data_ptr(), cptr, cdf0, Kt, *key, n, R, C, _stream(base))
-    perm, slice_len, slice_off, total = _flip_rows_layout(cnt, n, R)
-    entries = torch.empty((max(total, 4),), dtype=torch.uint32, device=dev)
-    with _on(base):
-        _lib.call("nb_flip_skip_fill_i64", entries.data_ptr(), base.data_ptr(), perm.data_ptr(), slice_off.data_ptr(),
-                  slice_len.data_ptr(), cptr, cdf0, Kt, *key, n, R, C, _stream(base))
-    return FlipRows(base, n, R, Kw, cnt, perm, slice_off, slice_len, entries)
+        _lib.call("nb_flip_skip_i64", entries.data_ptr(), info.data_ptr(), overflow.data_ptr(), base.data_ptr(),
+                  table.data_ptr(), int(seed) & (2 ** 64 - 1), int(subsequence), int(first), n, R, C, int(cap),
+                  _stream(base))
+    return FlipRows(base, n, R, Kw, C, info, entries, int(cap), overflow)
+
+
+class FlipLaw:
+    """The sparse form of a layer's per-element law: ``law`` uint16 [R, C] (bit 15 = base bit, bits 14:0 = the fp16
+    pattern of the flip probability min(P, 1 - P)), ``base`` int64 [R, Kw] packed base bits, ``table`` the skip
+    sampler's device table for the largest flip probability of the layer (``table[2]`` = that threshold)."""
+
+    def __init__(self, law, base, table, in_bits):
+        self.law, self.base, self.table, self.in_bits = law, base, table, in_bits
+
+    def max_flip_probability(self):
+        """The largest flip probability of the layer (a device read-back)."""
+        return float(self.table[2:3].view(torch.int32).to(torch.int64).item() & 0xFFFFFFFF) / 4294967296.0
+
+    def mean_flip_probability(self):
+        """The mean flip probability of the layer (a device read-back)."""
+        return float((self.law.view(torch.int16) & 0x7FFF).view(torch.float16).float().mean().item())
+
+
+def _law_workspace(device):
+    return torch.empty((int(_lib.load().nb_law_workspace_bytes()),), dtype=torch.uint8, device=device)
+
+
+def thresholds_from_weights(weight):
+    """Latent fp16 weights -> uint32 sampler thresholds of P = sigmoid(5 w / (mean|w| + 1e-5)) (modules/binary.py:59-60):
+    the tensor expression's roundings, in two kernels instead of nine."""
+    w = weight.detach()
+    _check(w, "weight")
+    assert w.dtype == torch.float16
+    out = torch.empty(w.shape, dtype=torch.uint32, device=w.device)
+    ws = _law_workspace(w.device)
+    with _on(w):
+        _lib.call("nb_thresholds_from_weights", out.data_ptr(), w.data_ptr(), w.numel(), ws.data_ptr(), _stream(w))
+    return out
+
+
+def probabilities_from_weights(weight):
+    """Latent fp16 weights -> fp16 probabilities P = sigmoid(5 w / (mean|w| + 1e-5)) (modules/binary.py:59-60)."""
+    w = weight.detach()
+    _check(w, "weight")
+    assert w.dtype == torch.float16
+    out = torch.empty(w.shape, dtype=torch.float16, device=w.device)
+    ws = _law_workspace(w.device)
+    with _on(w):
+        _lib.call("nb_probabilities_from_weights", out.data_ptr(), w.data_ptr(), w.numel(), ws.data_ptr(), _stream(w))
+    return out
+
+
+def flip_law_from_weights(weight):
+    """Latent fp16 weights [R, C] -> :class:`FlipLaw` of P = sigmoid(5 w / (mean|w| + 1e-5)): base bit = P >= 1/2,
+    flip probability min(P, 1 - P), and the skip sampler's table for the layer's largest flip probability, all made
+    on the device (three kernels, nothing read back)."""
+    w = weight.detach()
+    _check(w, "weight")
+    assert w.dtype == torch.float16 and len(w.shape) == 2
+    R, C = w.shape
+    law = torch.empty((R, C), dtype=torch.uint16, device=w.device)
+    base = torch.empty((R, ceil_div(C, 64)), dtype=torch.int64, device=w.device)
+    table = torch.empty((int(_lib.load().nb_skip_table_words()),), dtype=torch.uint32, device=w.device)
+    ws = _law_workspace(w.device)
+    with _on(w):
+        _lib.call("nb_flip_law_from_weights", law.data_ptr(), base.data_ptr(), table.data_ptr(), w.data_ptr(), R, C,
+                  ws.data_ptr(), _stream(w))
+    return FlipLaw(law, base, table, C)
+
+
+def flip_rows_thin(law, n, seed, cap, subsequence=0, first=0):
+    """:class:`FlipRows` for ``n`` members under a per-element law (:class:`FlipLaw`): the skip sampler walks at the
+    layer's largest flip probability and a column it reaches flips with probability (its own) / (the largest), decided
+    by the second word of a pair, so that every bit differs from the base with its own probability, independently.
+    ``cap``: pieces per row (see :func:`flip_capacity`; rows beyond it are counted in ``overflow``)."""
+    R, C = law.law.shape
+    dev = law.law.device
+    entries, info, overflow = _flip_alloc(n, R, int(cap), dev)
+    with _on(law.law):
+        _lib.call("nb_flip_skip_thin_i64", entries.data_ptr(), info.data_ptr(), overflow.data_ptr(), law.law.data_ptr(),
+                  law.table.data_ptr(), int(seed) & (2 ** 64 - 1), int(subsequence), int(first), n, R, C, int(cap),
+                  _stream(law.law))
+    return FlipRows(law.base, n, R, law.base.size(1), C, info, entries, int(cap), overflow)
 
 
 def flip_rows_to_weights(rows):
@@ -837,8 +990,8 @@ def flip_rows_to_weights(rows):
     checking the two forms against each other)."""
     W = rows.base.unsqueeze(0).expand(rows.D, rows.R, rows.Kw).contiguous()
     with _on(W):
-        _lib.call("nb_flip_to_dense_i64", W.data_ptr(), rows.entries.data_ptr(), rows.slice_off.data_ptr(),
-                  rows.slice_len.data_ptr(), rows.perm.data_ptr(), rows.D, rows.R, rows.Kw, _stream(W))
+        _lib.call("nb_flip_to_dense_i64", W.data_ptr(), rows.entries.data_ptr(), rows.info.data_ptr(), rows.D, rows.R,
+                  rows.Kw, rows.cap, _stream(W))
     return W
 
 
@@ -863,9 +1016,8 @@ def bmv_flip(rows, x, G=None):
     G = _flip_args(rows, x, G)
     out = torch.empty((rows.D, rows.R), dtype=torch.int32, device=x.device)
     with _on(x):
-        _lib.call("nb_bmv_flip_i64", out.data_ptr(), G.data_ptr(), rows.entries.data_ptr(), rows.slice_off.data_ptr(),
-                  rows.slice_len.data_ptr(), rows.perm.data_ptr(), rows.cnt.data_ptr(), x.data_ptr(), rows.D, rows.R,
-                  rows.Kw, _stream(x))
+        _lib.call("nb_bmv_flip_i64", out.data_ptr(), G.data_ptr(), rows.entries.data_ptr(), rows.info.data_ptr(),
+                  x.data_ptr(), rows.D, rows.R, rows.Kw, rows.cap, _stream(x))
     return out
 
 
@@ -878,6 +1030,23 @@ def bmv_flip_act_pack(rows, x, threshold, G=None):
     out = torch.empty((rows.D, ceil_div(rows.R, 64)), dtype=torch.int64, device=x.device)
     with _on(x):
         _lib.call("nb_bmv_flip_act_pack_i64", out.data_ptr(), G.data_ptr(), rows.entries.data_ptr(),
-                  rows.slice_off.data_ptr(), rows.slice_len.data_ptr(), rows.perm.data_ptr(), rows.cnt.data_ptr(),
-                  x.data_ptr(), threshold.data_ptr(), rows.D, rows.R, rows.Kw, _stream(x))
+                  rows.info.data_ptr(), x.data_ptr(), threshold.data_ptr(), rows.D, rows.R, rows.Kw, rows.cap,
+                  _stream(x))
+    return out
+
+
+def weighted_sum_flip(rows, weights, zbits):
+    """``weighted_sum`` over flip lists: fp16 [R, zbits] = sum_d weights[d] * bit_d with bit = base ^ flip; reads two
+    bytes per flip instead of a bit per weight.  The additions are exact (integers after scaling by a power of two), so
+    the result is the correctly rounded sum up to that scaling, whatever the order; ``weighted_sum`` on the
+    materialised weights adds in fp32 in member order, and the two agree to fp32 rounding of the partial sums."""
+    _check(weights, "weights")
+    assert weights.dtype == torch.float16 and tuple(weights.shape) == (rows.D,)
+    if weights.device != rows.entries.device:
+        raise RuntimeError("Tensors are on different devices")
+    assert zbits <= rows.Kw * 64
+    out = torch.empty((rows.R, zbits), dtype=torch.float16, device=weights.device)
+    with _on(weights):
+        _lib.call("nb_flip_weighted_sum_i64", out.data_ptr(), rows.entries.data_ptr(), rows.info.data_ptr(),
+                  rows.base.data_ptr(), weights.data_ptr(), rows.D, rows.R, int(zbits), rows.cap, _stream(weights))
     return out

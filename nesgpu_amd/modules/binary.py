@@ -13,6 +13,10 @@ parity mode), ``set_noise(bias_generator=...)`` draws the bias noise from a give
 global one, and ``BinarizedConv2d(pack_output=True[, pool_output=True])`` returns the thresholded map
 already packed along channels (and 2x2 OR-pooled) from one fused kernel instead of a bool map;
 ``fuse_packed_outputs(model)`` switches those on wherever a reference-style ``nn.Sequential`` allows it.
+``flip_probability=p`` (any layer) replaces the law sigmoid(5 w / mean|w|) by "sign of the latent weight, flipped with
+probability p" (base XOR Bernoulli(p) flip mask).  ``BinarizedLinear(sparse=...)`` keeps ``weight_noise`` as the
+shared base plus per-member flip lists (:class:`booleanOperations.FlipRows`) instead of materialised weights: the ops
+the layer calls (``bmm``, ``bmv_act_pack``, ``weighted_sum``) take either form and give the same results.
 """
 import torch
 from torch import nn
@@ -61,7 +65,8 @@ class Binarized(Perturbed, nn.Module):
     probability sigmoid(5 * w / (mean|w| + 1e-5)) (modules/binary.py:59-62) and stored packed as
     ``weight_noise`` [directions, rows, ceil(in_degree/bits)]."""
 
-    def __init__(self, in_degree, out_degree, directions, threshold=False, dtype=torch.int64, device="cuda"):
+    def __init__(self, in_degree, out_degree, directions, threshold=False, dtype=torch.int64, device="cuda",
+                 flip_probability=None):
         nn.Module.__init__(self)
         Perturbed.__init__(self, directions)
         self.in_degree = in_degree
@@ -71,6 +76,11 @@ class Binarized(Perturbed, nn.Module):
         self.device = device
         self.directions = directions
         self.bias = None
+        if flip_probability is not None and not 0.0 <= flip_probability <= 1.0:
+            raise ValueError("flip_probability must lie in [0, 1]")
+        self.flip_probability = flip_probability      # not in the reference: weights = sign(w) XOR Bernoulli(p)
+        self.sparse = False                           # BinarizedLinear only: flip lists instead of weights
+        self._cache = {}
 
     def reset_parameters(self):
         with torch.no_grad():
@@ -79,10 +89,31 @@ class Binarized(Perturbed, nn.Module):
                 self.bias.fill_(0)
 
     def probabilities(self):
-        """fp16 [rows, in_degree] per-bit probabilities of a 1 (modules/binary.py:59-60)."""
+        """fp16 [rows, in_degree] per-bit probabilities of a 1 (modules/binary.py:59-60): the tensor expression
+        ``sigmoid((w / (w.abs().mean() + 1e-5) * 5).float()).half()`` with its roundings, in two kernels (the mean of
+        |w| is the exact one rounded once to fp16, where torch's adds in fp32 in its own order).  With
+        ``flip_probability`` p: 1 - p where the latent weight is >= 0, p elsewhere."""
         with torch.no_grad():
+            if self.flip_probability is not None:
+                p = torch.tensor(self.flip_probability, dtype=torch.float32, device=self.weight.device)
+                return torch.where(self.weight >= 0, 1.0 - p, p).half()
+            if self.weight.is_cuda:
+                return booleanOperations.probabilities_from_weights(self.weight)
             norm_weight = self.weight / (self.weight.abs().mean() + 1e-5) * 5
             return torch.sigmoid(norm_weight.float()).half()
+
+    def _cached(self, key, tensor, make):
+        """``make()`` once per version of ``tensor`` (a parameter): what depends only on the latent values."""
+        tag = (tensor._version, tensor.data_ptr())
+        hit = self._cache.get(key)
+        if hit is None or hit[0] != tag:
+            with torch.no_grad():
+                hit = self._cache[key] = (tag, make())
+        return hit[1]
+
+    def sign_base(self):
+        """Packed sign bits of the latent weights, [rows, ceil(in_degree/bits)] (bit = w >= 0)."""
+        return self._cached("base", self.weight, lambda: booleanOperations.pack(self.weight.detach() >= 0, self.dtype))
 
     conv_taps = None     # conv layers: kx*ky, and the sampler also writes weight_noise_reshaped
 
@@ -95,12 +126,25 @@ class Binarized(Perturbed, nn.Module):
             self.set_seed()
         if noise_scale is not None:
             self.set_noise_scale(noise_scale)
-        P = self.probabilities()
-        if words is None:
-            sampled = booleanOperations.sample_bits(P, self.directions, self.dtype, self.seed, conv_taps=self.conv_taps)
-        else:
+        sampled = None
+        if words is not None:
             sampled = booleanOperations.sample_bits_from_words(
-                booleanOperations.thresholds_from_p(P), words, self.dtype, conv_taps=self.conv_taps)
+                booleanOperations.thresholds_from_p(self.probabilities()), words, self.dtype, conv_taps=self.conv_taps)
+        elif self.conv_taps is None and self._sparse_now():
+            sampled = self._sample_sparse()
+        elif self.flip_probability is not None:
+            T = min(int(self.flip_probability * 4294967296.0), 0xFFFFFFFF)
+            sampled = booleanOperations.sample_bits_philox(T, self.directions, self.dtype, self.seed, base=self.sign_base(),
+                                                           shape=tuple(self.weight.shape), conv_taps=self.conv_taps)
+        elif self.weight.is_cuda:
+            # sample_bits(P, directions, dtype, seed) of modules/binary.py:62 with the thresholds taken straight from
+            # the latent weights
+            sampled = booleanOperations.sample_bits_philox(booleanOperations.thresholds_from_weights(self.weight),
+                                                           self.directions, self.dtype, self.seed,
+                                                           conv_taps=self.conv_taps)
+        else:
+            sampled = booleanOperations.sample_bits(self.probabilities(), self.directions, self.dtype, self.seed,
+                                                    conv_taps=self.conv_taps)
         if self.conv_taps is None:
             self.weight_noise = sampled
         else:
@@ -108,6 +152,27 @@ class Binarized(Perturbed, nn.Module):
             self.weight_noise, self.weight_noise_reshaped = sampled
         self.bias_noise = (torch.rand(size=(self.directions, self.out_degree), dtype=torch.float16,
                                       device=self.weight.device, generator=bias_generator) - .5) * 6
+
+    def _sparse_now(self):
+        return False
+
+    def int_thresholds(self, offset, floor=False):
+        """int32 [directions, out] thresholds ``(bias + bias_noise) -> int + offset`` of the integer compare
+        2*popc > threshold (modules/binary.py:157), made once per (bias, bias_noise) pair instead of on every
+        forward."""
+        noise = self.bias_noise
+        tag = (self.bias._version, self.bias.data_ptr(), noise._version, offset, floor)
+        hit = self._cache.get("thresh")
+        if hit is None or hit[0] != tag or hit[2] is not noise:
+            with torch.no_grad():
+                t = self.bias + noise
+                t = torch.floor(t.to(torch.float32)).to(torch.int32) if floor else t.type(torch.int32)
+                hit = self._cache["thresh"] = (tag, t + offset, noise)   # holds the noise: its identity stays its own
+        return hit[1]
+
+    def free_memory(self):
+        Perturbed.free_memory(self)
+        self._cache = {}
 
     def update(self, weights, l1=0, l2=1e-3):
         """modules/binary.py:67-77."""
@@ -127,10 +192,15 @@ class BinarizedLinear(Binarized):
     row per member (a batched matrix-VECTOR product, modules/binary.py:97)."""
 
     def __init__(self, in_features, out_features, directions, threshold=True, batch_norm=False, dtype=torch.int64,
-                 device="cuda", pack_output=False):
-        Binarized.__init__(self, in_features, out_features, directions, threshold, dtype, device)
+                 device="cuda", pack_output=False, flip_probability=None, sparse="auto"):
+        Binarized.__init__(self, in_features, out_features, directions, threshold, dtype, device, flip_probability)
         self.in_features = in_features
         self.out_features = out_features
+        # True / False / "auto": base + flip lists when the layer is wide and its flip probabilities are small
+        # (64-bit words, at least 2048 inputs, at most 65536 outputs)
+        if sparse not in (True, False, "auto"):
+            raise ValueError("sparse must be True, False or 'auto'")
+        self.sparse = sparse
         if pack_output and not threshold:
             raise NotImplementedError("packed output needs threshold=True")
         self.pack_output = pack_output    # not in the reference: return the thresholded row packed, from one kernel
@@ -140,29 +210,73 @@ class BinarizedLinear(Binarized):
         self.batch_norm = batch_norm
         self.reset_parameters()
 
+    # ---- sparse form: shared base + per-member flip lists ------------------------------------------------------------
+    def _sparse_possible(self):
+        return (self.dtype == torch.int64 and self.weight.is_cuda and self.in_features <= 511 * 64
+                and self.out_features <= 65536)
+
+    def _sparse_plan(self):
+        """What the sparse sampler needs of the latent weights, made once per version of them: with
+        ``flip_probability`` the packed sign bits; else the per-element law (base bits, flip probabilities, the skip
+        sampler's table) and, read back once, its mean / largest / largest row-mean flip probability, from which the
+        decision (``sparse="auto"``) and the lists' capacity follow."""
+        def make():
+            if self.flip_probability is not None:
+                p = min(self.flip_probability, 1.0 - self.flip_probability)
+                return dict(law=None, mean=p, peak=p, row=p)
+            law = booleanOperations.flip_law_from_weights(self.weight)
+            y = (law.law.view(torch.int16) & 0x7FFF).view(torch.float16).float()
+            stats = torch.stack([y.mean(), y.mean(dim=1).max()]).tolist()          # the one read-back
+            return dict(law=law, mean=stats[0], peak=law.max_flip_probability(), row=stats[1])
+        return self._cached("sparse_plan", self.weight, make)
+
+    def _sparse_now(self):
+        if self.sparse is False or not self._sparse_possible():
+            if self.sparse is True:
+                raise NotImplementedError("the sparse form needs 64-bit words on a GPU, at most 32704 inputs and 65536 "
+                                          "outputs")
+            return False
+        if self.sparse is True:
+            return True
+        if self.in_features < 2048:
+            return False
+        plan = self._sparse_plan()
+        # two bytes per flip against a bit per weight: worth it below one flip in sixteen bits; the thinned walk draws
+        # two words per candidate, at the largest probability of the layer
+        return plan["mean"] <= 0.04 and plan["peak"] <= 0.25
+
+    def _sample_sparse(self):
+        plan = self._sparse_plan()
+        cap = booleanOperations.flip_capacity(self.in_features, plan["row"])
+        if plan["law"] is None:
+            p = self.flip_probability
+            base = self.sign_base() if p <= 0.5 else self._cached(
+                "antibase", self.weight, lambda: booleanOperations.pack(self.weight.detach() < 0, self.dtype))
+            T = min(int(min(p, 1.0 - p) * 4294967296.0), 0xFFFFFFFF)
+            return booleanOperations.flip_rows_skip(base, self.in_features, self.directions, T, self.seed, cap=cap)
+        return booleanOperations.flip_rows_thin(plan["law"], self.directions, self.seed, cap)
+
     def forward(self, input):
         if not self.perturbed_flag:
             raise NotImplementedError                     # modules/binary.py:108-109: no inference path
         packed_input = booleanOperations.pack(input, self.dtype) if input.dtype == torch.bool else input
-        if self.threshold and self.batch_norm and (self.in_features <= 2048 or self.pack_output):
-            # modules/binary.py:97-102 in one call: the weights are streamed once, the population mean of every output
-            # comes from exact integer sums, mean = fp16(float(sum of activations) / directions), and the compare is
-            # exact (activations up to 2048 are exact in fp16, which is what the reference compares in)
-            return booleanOperations.bmv_bn_act(self.weight_noise, packed_input.view(self.directions, -1),
-                                                self.bias.detach(), self.bias_noise, self.in_features,
-                                                pack=self.pack_output)
         Z = self.directions
-        if (self.threshold and self.batch_norm and self.in_features <= 65504 and Z & (Z - 1) == 0
-                and Z * self.in_features <= 2 ** 24):
-            # Longer rows: the reference's expression rounds the activations to fp16 (for the mean and for the
-            # compare).  The same call does that too, and gives the very bits of the tensor expression below as long
-            # as torch's fp32 sum over the population is exact (integers below 2**24) and its multiplication by
-            # 1 / directions is a division (a power of two).
+        dense = not isinstance(self.weight_noise, booleanOperations.FlipRows)
+        if dense and self.threshold and self.batch_norm and self.in_features <= 65504 and (
+                self.in_features <= 2048 or self.pack_output or Z * self.in_features <= 2 ** 24):
+            # modules/binary.py:97-102 in one call: the weights are streamed once, the population mean of every output
+            # comes from exact integer sums the way torch's fp16 mean forms it (the fp32 sum times the fp32 quotient of
+            # the element counts), and the compare is exact.  Rows of more than 2048 bits: the reference's expression
+            # rounds the activations to fp16 (for the mean and for the compare), and so does the call.  Its bits are
+            # those of the tensor expression below as long as torch's fp32 sum over the population is exact (integers
+            # up to 2**24); beyond that torch's sum depends on its summation order, the call's is the exact one rounded
+            # once, and only short rows and packed outputs (which have no tensor expression) take it.
             return booleanOperations.bmv_bn_act(self.weight_noise, packed_input.view(Z, -1), self.bias.detach(),
-                                                self.bias_noise, self.in_features, round_fp16=True)
-        if self.pack_output:
+                                                self.bias_noise, self.in_features, pack=self.pack_output,
+                                                round_fp16=self.in_features > 2048)
+        if self.pack_output and not self.batch_norm:
             # activation > t  <=>  2*popc - K > floor(t)  <=>  2*popc > floor(t) + K  (activation is an integer)
-            thresh = torch.floor((self.bias + self.bias_noise).to(torch.float32)).to(torch.int32) + self.in_features
+            thresh = self.int_thresholds(self.in_features, floor=True)
             return booleanOperations.bmv_act_pack(self.weight_noise, packed_input.view(self.directions, -1), thresh)
         popc = booleanOperations.bmm(self.weight_noise, packed_input.view(self.directions, -1, 1))
         activation = 2 * popc.squeeze(dim=2) - self.in_features
@@ -170,7 +284,8 @@ class BinarizedLinear(Binarized):
             thresh = (self.bias + self.bias_noise)
             if self.batch_norm:
                 thresh = thresh + activation.type(torch.float16).mean(dim=0, keepdim=True)
-            return activation > thresh
+            bits = activation > thresh
+            return booleanOperations.pack(bits, self.dtype) if self.pack_output else bits
         return activation
 
 
@@ -180,8 +295,8 @@ class BinarizedConv2d(Binarized):
 
     def __init__(self, in_channels, out_channels, directions, kernel_size, stride=1, padding=0, dilation=1, groups=1,
                  threshold=True, batch_norm=True, padding_mode='zeros', dtype=torch.int64, device="cuda",
-                 pack_output=False, pool_output=False):
-        Binarized.__init__(self, in_channels, out_channels, directions, threshold, dtype, device)
+                 pack_output=False, pool_output=False, flip_probability=None):
+        Binarized.__init__(self, in_channels, out_channels, directions, threshold, dtype, device, flip_probability)
         if dilation != 1 or groups != 1 or padding_mode != "zeros":
             raise NotImplementedError
         self.in_channels = in_channels
@@ -241,7 +356,7 @@ class BinarizedConv2d(Binarized):
                 thresh = booleanOperations.conv_bn_thresholds_from_input(
                     packed_input, filt, self.bias.detach(), self.bias_noise, *geom, channels=self.in_channels, **tapkw)
             else:
-                thresh = (self.bias + self.bias_noise).type(torch.int32) + offset
+                thresh = self.int_thresholds(offset)
             if self.pack_output or self.pool_output:
                 return booleanOperations.conv_act_pack(packed_input, filt, thresh, *geom, pool=self.pool_output,
                                                        **tapkw)
@@ -249,7 +364,7 @@ class BinarizedConv2d(Binarized):
         return 2 * booleanOperations.conv(packed_input, filt, *geom, **tapkw) - offset
 
     def free_memory(self):
-        Perturbed.free_memory(self)
+        Binarized.free_memory(self)
         self.weight_noise_reshaped = None
         self.weight_noise_tap = None
 
@@ -273,7 +388,7 @@ class BinarizedMaxPool2d(nn.Module):
         return booleanOperations.max_pool2d(packed_input, *self.kernel_size, *self.padding, *self.stride)
 
 
-def fuse_packed_outputs(model):
+def fuse_packed_outputs(model, max_fan_in=2048):
     """Switches the fused outputs on in a reference-style stack of layers (not in the reference; results unchanged).
 
     Walks every ``nn.Sequential`` inside ``model``: a thresholding ``BinarizedConv2d`` followed by a 2x2 / stride 2 /
@@ -281,8 +396,11 @@ def fuse_packed_outputs(model):
     conv or linear layer whose output goes (through ``nn.Flatten`` at most) into another binary layer, which accepts
     packed words, gets ``pack_output=True``.  A conv in front of ``nn.Flatten`` is only switched when its channel
     count fills whole words, so that the flattened packed words are the flattened bits, and layers with more than
-    2048 inputs per output are left alone (their activations are beyond fp16's exact integers, where the reference's
-    fp16 comparison and the fused integer comparison can differ).  Returns the number of layers changed."""
+    ``max_fan_in`` = 2048 inputs per output are left alone (their activations are beyond fp16's exact integers, where
+    the reference's fp16 comparison and the fused integer comparison can differ: without batch norm they differ only
+    for thresholds ``bias + bias_noise`` beyond +-2048, since rounding an activation to fp16 never moves it across a
+    smaller threshold; ``max_fan_in=None`` fuses such layers too, for models whose biases stay below that).
+    Returns the number of layers changed."""
     changed = 0
     for seq in [m for m in model.modules() if isinstance(m, nn.Sequential)]:
         layers = list(seq)
@@ -295,7 +413,9 @@ def fuse_packed_outputs(model):
                 fan_in = layer.in_channels * layer.kernel_size[0] * layer.kernel_size[1]
             else:
                 fan_in = layer.in_features
-            if fan_in > 2048:
+            if max_fan_in is not None and fan_in > max_fan_in:
+                continue
+            if fan_in > 2048 and layer.batch_norm:
                 continue
             j = i + 1
             if isinstance(layer, BinarizedConv2d) and j < len(layers) and isinstance(layers[j], BinarizedMaxPool2d):

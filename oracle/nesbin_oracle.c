@@ -20,6 +20,10 @@
  *   weighted_sum         float64 numpy einsum over unpacked bits (tolerance)
  *   skip_flips           numpy searchsorted + cumsum over the (pinned) Philox words; flip rate,
  *                        gap histogram against the geometric law, neighbouring columns uncorrelated
+ *   skip_flips_thin      the same numpy walk with the pair's second word deciding each column
+ *                        (Python integers); per-column flip rates against their own probabilities,
+ *                        neighbouring columns uncorrelated, reduction to skip_flips' law when all
+ *                        probabilities equal the largest one
  * The cuRAND XORWOW stream of the reference samplers (sample_bits.cu:23-25,54) is NOT
  * reproduced anywhere: parity unpinned for that stream; supplied-word parity replaces it.
  *
@@ -171,6 +175,65 @@ void nbo_skip_flips_i64(uint64_t *mask, const uint32_t *cdf, int64_t Kt, uint64_
             pos += lo < Kt ? 1 + lo : Kt;
             if (pos >= C) break;
             if (lo < Kt) row[pos >> 6] |= (uint64_t)1 << (pos & 63);
+        }
+    }
+}
+
+/* fp16 bit pattern (sign ignored by the caller) -> float, exactly */
+static float nbo_half_bits_to_float(uint16_t h)
+{
+    const uint32_t e = (h >> 10) & 31u, m = h & 1023u;
+    if (e == 0) return (float)m * 5.9604644775390625e-08f;              /* m * 2^-24 */
+    if (e == 31) return m ? __builtin_nanf("") : __builtin_inff();
+    float v = (float)(1024u + m) * 0.0009765625f;                       /* 1.m */
+    int sh = (int)e - 15;
+    while (sh > 0) { v *= 2.0f; sh--; }
+    while (sh < 0) { v *= 0.5f; sh++; }
+    return v;
+}
+
+/* Flip masks under a per-element law, by thinning: the contract of nb_flip_skip_thin_i64 (no counterpart in the
+ * reference, whose sampler compares every bit's probability with its own draw, extensions/src/sample_bits.cu:47-57).
+ * law [R, C]: bit 15 = base bit of the column (not used here), bits 14:0 = fp16 pattern of its flip probability
+ * y <= 1/2, Tf = floor(y * 2^32).  Row q = d*R + r reads the Philox words first + q*C + 2i (a gap, ranked in cdf as
+ * in nbo_skip_flips_i64; cdf belongs to the largest Tf of the layer, tmax) and first + q*C + 2i + 1: the column the
+ * gap reaches flips iff that second word times tmax is below Tf * 2^32, i.e. with probability Tf / tmax.  mask is
+ * [D*R, ceil(C/64)] 64-bit words, LSB first. */
+void nbo_skip_flips_thin_i64(uint64_t *mask, const uint16_t *law, const uint32_t *cdf, int64_t Kt, uint32_t tmax,
+                             uint64_t seed, uint64_t subseq, uint64_t first, int64_t D, int64_t R, int64_t C)
+{
+    const uint32_t key[2] = {(uint32_t)seed, (uint32_t)(seed >> 32)};
+    const int64_t Kw = (C + 63) / 64;
+#pragma omp parallel for schedule(static)
+    for (int64_t q = 0; q < D * R; q++) {
+        uint64_t *row = mask + q * Kw;
+        const uint16_t *lr = law + (q % R) * C;
+        memset(row, 0, (size_t)Kw * 8);
+        if (Kt == 0) continue;
+        int64_t pos = -1;
+        for (int64_t i = 0;; i++) {
+            uint32_t pair[2];
+            for (int h = 0; h < 2; h++) {
+                const uint64_t g = first + (uint64_t)q * (uint64_t)C + (uint64_t)(2 * i + h);
+                const uint64_t blk = g >> 2;
+                const uint32_t ctr[4] = {(uint32_t)blk, (uint32_t)(blk >> 32), (uint32_t)subseq, (uint32_t)(subseq >> 32)};
+                uint32_t o[4];
+                nbo_philox4x32_10(o, ctr, key);
+                pair[h] = o[g & 3];
+            }
+            int64_t lo = 0, hi = Kt; /* first index whose entry exceeds the gap word */
+            while (lo < hi) {
+                const int64_t mid = (lo + hi) / 2;
+                if (cdf[mid] <= pair[0]) lo = mid + 1;
+                else hi = mid;
+            }
+            pos += lo < Kt ? 1 + lo : Kt;
+            if (pos >= C) break;
+            if (lo >= Kt) continue;
+            float t = nbo_half_bits_to_float((uint16_t)(lr[pos] & 0x7FFFu)) * 4294967296.0f;
+            if (!(t <= 4294967040.0f)) t = 4294967040.0f;
+            const uint64_t tf = (uint64_t)(uint32_t)t;
+            if ((uint64_t)pair[1] * (uint64_t)tmax < (tf << 32)) row[pos >> 6] |= (uint64_t)1 << (pos & 63);
         }
     }
 }

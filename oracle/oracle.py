@@ -245,6 +245,32 @@ def skip_flips(cdf, seed, subseq, first, rows, C):
     return out
 
 
+def skip_flips_thin(law, cdf, tmax, seed, subseq, first, D):
+    """Flip masks [D*R, ceil(C/64)] int64 under the per-element law ``law`` uint16 [R, C], by thinning (see
+    nbo_skip_flips_thin_i64)."""
+    law = _c(law, np.uint16)
+    cdf = _c(cdf, np.uint32)
+    R, C = law.shape
+    out = np.empty((int(D) * R, (C + 63) // 64), dtype=np.int64)
+    lib().nbo_skip_flips_thin_i64(_p(out), _p(law), _p(cdf), _i64(cdf.shape[0]), ctypes.c_uint32(int(tmax)),
+                                  ctypes.c_uint64(int(seed)), ctypes.c_uint64(int(subseq)), ctypes.c_uint64(int(first)),
+                                  _i64(D), _i64(R), _i64(C))
+    return out
+
+
+def flip_law(P):
+    """fp16 probabilities [R, C] -> (law uint16 [R, C], base bool [R, C], tmax): base = P >= 1/2, flip probability
+    y = min(P, 1 - P) (exact in fp16), law = base << 15 | fp16 bits of y, tmax = the largest floor(y * 2**32)."""
+    P = np.asarray(P, dtype=np.float16)
+    p32 = P.astype(np.float32)
+    base = p32 >= 0.5
+    y = np.where(base, np.float32(1.0) - p32, p32).astype(np.float16)
+    assert (y.astype(np.float32) == np.where(base, np.float32(1.0) - p32, p32)).all()
+    law = (y.view(np.uint16) & 0x7FFF) | (base.astype(np.uint16) << 15)
+    tf = np.minimum(y.astype(np.float64) * 4294967296.0, 4294967040.0).astype(np.uint64)
+    return law.astype(np.uint16), base, int(tf.max()) if tf.size else 0
+
+
 def max_threads():
     return int(lib().nbo_max_threads())
 

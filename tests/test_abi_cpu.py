@@ -81,10 +81,19 @@ def test_bad_arguments_are_rejected_without_a_launch(lib):
     assert lib.nb_thresholds_from_p(one, None, 4, None) == 1
     assert lib.nb_thresholds_from_p(one, ctypes.c_void_p(9), 4, None) == 3
     assert lib.nb_thresholds_from_p(None, None, 0, None) == 0
-    # flip-list layout: the list length has to go somewhere, slice lengths are read 16 bytes at a time, R <= 65536
-    assert lib.nb_flip_layout(one, one, one, None, one, 2, 64, None) == 1
-    assert lib.nb_flip_layout(one, ctypes.c_void_p(8), one, one, one, 2, 64, None) == 3
-    assert lib.nb_flip_layout(one, one, one, one, one, 2, 65537, None) == 2
+    # flip lists: the overflow count has to go somewhere, entries are read 16 bytes at a time, R <= 65536, a
+    # capacity of at most 8191 pieces per row; the skip sampler needs its table
+    big = ctypes.c_void_p(256)
+    assert lib.nb_flip_fill_i64(big, one, None, one, one, 2, 64, 1, 4, None) == 1
+    assert lib.nb_flip_fill_i64(one, one, one, one, one, 2, 64, 1, 4, None) == 3
+    assert lib.nb_flip_fill_i64(big, one, one, one, one, 2, 65537, 1, 4, None) == 2
+    assert lib.nb_bmv_flip_i64(one, one, big, one, one, 2, 64, 1, 8192, None) == 2
+    assert lib.nb_flip_skip_i64(big, one, one, one, None, 1, 0, 0, 2, 64, 64, 4, None) == 1
+    assert lib.nb_flip_skip_thin_i64(big, one, one, ctypes.c_void_p(9), one, 1, 0, 0, 2, 64, 64, 4, None) == 3
+    assert lib.nb_flip_weighted_sum_i64(one, big, one, one, ctypes.c_void_p(9), 2, 64, 64, 4, None) == 3
+    assert lib.nb_flip_law_from_weights(one, one, None, one, 4, 64, one, None) == 1
+    assert lib.nb_thresholds_from_weights(one, one, 4, ctypes.c_void_p(4), None) == 3
+    assert lib.nb_skip_table_words() == 4100 and lib.nb_law_workspace_bytes() == 2048
     # empty problems succeed without touching the pointers
     assert lib.nb_pack_i64(None, None, 0, 64, None) == 0
     assert lib.nb_bmm_i32(None, None, None, 0, 5, 5, 5, None) == 0

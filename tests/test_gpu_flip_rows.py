@@ -70,36 +70,33 @@ def test_expand_rows_codes(ops):
 
 def decode_flip_rows(rows):
     """FlipRows -> boolean flip mask [D, R, 64 * Kw] and the base bit every entry claims, read back entry by entry."""
-    D, R, Kw = rows.D, rows.R, rows.Kw
+    D, R, Kw, cap = rows.D, rows.R, rows.Kw, rows.cap
     S = (R + 63) // 64
     ent = host(rows.entries).astype(np.uint32)
-    off, ln, perm = host(rows.slice_off), host(rows.slice_len), host(rows.perm).astype(np.int64)
+    info = host(rows.info.view(torch.int32)).astype(np.int64)
     mask = np.zeros((D, R, 64 * Kw), dtype=bool)
     bflag = np.zeros((D, R, 64 * Kw), dtype=bool)
     sentinel = (4 * Kw) << 5
     for d in range(D):
-        for s in range(S):
-            L = int(ln[d, s])                                                            # 16-byte pieces per lane
-            assert off[d, s] % 4 == 0
-            blk = ent[off[d, s]: off[d, s] + L * 256].reshape(L, 64, 4).transpose(0, 2, 1).reshape(4 * L, 64)
-            halves = np.stack([blk & 0xFFFF, blk >> 16], axis=1).reshape(8 * L, 64)     # flips in order, per lane
-            for lane in range(64):
-                p = s * 64 + lane
-                col_prev, ended = -1, False
-                for e in halves[:, lane]:
-                    e = int(e)
-                    if e == sentinel:
-                        ended = True
-                        continue
-                    assert not ended and p < R, "a flip after the sentinel / in a lane without a row"
-                    piece, bit = e >> 5, e & 31
-                    assert piece < 4 * Kw
-                    b = bool(piece & 1)
-                    col = (piece >> 1) * 32 + bit
-                    assert col > col_prev                                                # column order
-                    col_prev = col
-                    mask[d, perm[d, p], col] = True
-                    bflag[d, perm[d, p], col] = b
+        for r in range(R):
+            n, pieces = int(info[d, r] & 0xFFFF), int(info[d, r] >> 16)
+            assert pieces <= cap and (n + 7) // 8 <= pieces
+            col_prev, seen = -1, 0
+            for j in range(pieces):
+                at = (((d * S + r // 64) * cap + j) * 64 + r % 64) * 4
+                for dw in ent[at: at + 4]:
+                    for e in (int(dw) & 0xFFFF, int(dw) >> 16):
+                        if e == sentinel:
+                            continue
+                        piece, bit = e >> 5, e & 31
+                        assert piece < 4 * Kw
+                        col = (piece >> 1) * 32 + bit
+                        assert col > col_prev                                            # column order
+                        col_prev = col
+                        seen += 1
+                        mask[d, r, col] = True
+                        bflag[d, r, col] = bool(piece & 1)
+            assert seen == n
     return mask, bflag
 
 
@@ -107,27 +104,23 @@ def decode_flip_rows(rows):
                                      (1, 2100, 64, 0.01), (4, 7, 960, 0.0), (2, 130, 70, 1.0)])
 def test_flip_rows_hold_exactly_the_flipped_bits(ops, D, R, C, p):
     g = np.random.default_rng(D + R + C)
-    Kw = (C + 63) // 64
     base = sparse_mask(g, (R, C), 0.5)
     flips = sparse_mask(g, (D, R, C), p)
     W = base[None] ^ flips
     rows = ops.flip_rows_from_weights(dev(W), dev(base))
-    cnt = host(rows.cnt).astype(np.int64)
     want_bits = np.unpackbits(flips.view(np.uint8), axis=2, bitorder="little").astype(bool)   # [D, R, 64 Kw]
-    np.testing.assert_array_equal(cnt, want_bits.sum(axis=2))
-    perm = host(rows.perm).astype(np.int64)
-    for d in range(D):
-        assert sorted(perm[d].tolist()) == list(range(R))                                      # a permutation ...
-        assert (perm[d] // 1024 == np.arange(R) // 1024).all()                                 # ... inside blocks of 1024
-        for b0 in range(0, R, 1024):
-            assert (np.diff(cnt[d, perm[d, b0:b0 + 1024]]) >= 0).all()                         # ordered by flip count
-    S = (R + 63) // 64
-    cs = np.pad(np.take_along_axis(cnt, perm, axis=1), ((0, 0), (0, S * 64 - R))).reshape(D, S, 64)
-    np.testing.assert_array_equal(host(rows.slice_len), (cs.max(axis=2) + 7) // 8)
+    np.testing.assert_array_equal(host(rows.cnt).astype(np.int64), want_bits.sum(axis=2))
+    assert rows.cap == (int(want_bits.sum(axis=2).max()) + 7) // 8 and rows.overflowed() == 0
     mask, bflag = decode_flip_rows(rows)
     np.testing.assert_array_equal(mask, want_bits)
     base_bits = np.unpackbits(base.view(np.uint8), axis=1, bitorder="little").astype(bool)
     np.testing.assert_array_equal(bflag, mask & base_bits[None])
+    # a capacity with room to spare holds the same lists; one that is too small is reported
+    roomy = ops.flip_rows_from_weights(dev(W), dev(base), cap=rows.cap + 3)
+    assert torch.equal(ops.flip_rows_to_weights(roomy), dev(W)) and roomy.overflowed() == 0
+    if rows.cap > 1:
+        tight = ops.flip_rows_from_weights(dev(W), dev(base), cap=rows.cap - 1)
+        assert tight.overflowed() == int(((want_bits.sum(axis=2) + 7) // 8 > rows.cap - 1).sum())
 
 
 @pytest.mark.parametrize("D,R,C,p", [(5, 64, 64, 0.1), (3, 100, 200, 0.05), (4, 1024, 8192, 0.01), (2, 1100, 128, 0.3),
@@ -159,32 +152,11 @@ def test_bmv_flip_vs_oracle(ops, oracle, D, R, C, p):
     assert torch.equal(ops.bmv_flip(rows, xd, G=G), got)
 
 
-@pytest.mark.parametrize("D,R,hi", [(1, 1, 5), (3, 63, 3), (2, 64, 100), (5, 100, 2), (3, 1024, 40), (2, 1100, 7),
-                                    (2, 2053, 65535), (70, 130, 9)])
-def test_flip_layout_orders_blocks_of_rows_by_count(ops, D, R, hi):
-    """Row order and slice lengths against numpy: a stable sort by count inside every block of 1024 rows, pieces per
-    lane from the longest row of each run of 64; running offsets in dwords."""
-    g = np.random.default_rng(D * 1000 + R)
-    cnt = g.integers(0, hi + 1, size=(D, R)).astype(np.uint16)
-    perm, slice_len, slice_off, total = ops._flip_rows_layout(dev(cnt.view(np.int16)).view(torch.uint16), D, R)
-    S = (R + 63) // 64
-    want_perm = np.concatenate([b0 + np.argsort(cnt[:, b0:b0 + 1024].astype(np.int64), axis=1, kind="stable")
-                                for b0 in range(0, R, 1024)], axis=1)
-    np.testing.assert_array_equal(host(perm.view(torch.int16)).view(np.uint16), want_perm.astype(np.uint16))
-    sorted_cnt = np.take_along_axis(cnt.astype(np.int64), want_perm, axis=1)
-    padded = np.zeros((D, S * 64), dtype=np.int64)
-    padded[:, :R] = sorted_cnt
-    want_len = (padded.reshape(D, S, 64).max(axis=2) + 7) // 8
-    np.testing.assert_array_equal(host(slice_len), want_len.astype(np.int32))
-    lens = want_len.reshape(-1) * 256
-    np.testing.assert_array_equal(host(slice_off).reshape(-1), np.cumsum(lens) - lens)
-    assert total == int(lens.sum())
-    assert slice_off.dtype == torch.int64 and slice_len.dtype == torch.int32 and perm.dtype == torch.uint16
-
-
 def test_flip_shapes_are_checked(ops):
     with pytest.raises(RuntimeError, match="at most 511"):
         ops._lib.call("nb_flip_count_i64", 256, 256, 256, 1, 4, 512, None)
+    with pytest.raises(RuntimeError, match="at most 8191"):
+        ops._lib.call("nb_bmv_flip_i64", 256, 256, 256, 256, 256, 1, 4, 2, 9000, None)
     with pytest.raises(RuntimeError, match="whole tiles"):
         ops._lib.call("nb_bmm_nt_fp4", 256, 256, 256, 130, 4, 2, 128, 128, 2, None)
 
@@ -208,6 +180,7 @@ def test_skip_sampler_vs_oracle(ops, oracle, D, R, C, p, first):
     np.testing.assert_array_equal(table, oracle.skip_cdf(T))
     want_W = base[None] ^ oracle.skip_flips(table, seed, sub, first, D * R, C).reshape(D, R, Kw)
     rows = ops.flip_rows_skip(dev(base), C, D, T, seed, subsequence=sub, first=first)
+    assert rows.overflowed() == 0
     flips = np.unpackbits((want_W ^ base[None]).view(np.uint8), axis=2, bitorder="little")
     np.testing.assert_array_equal(host(rows.cnt).astype(np.int64), flips.sum(axis=2))
     W = ops.flip_rows_to_weights(rows)
@@ -231,7 +204,7 @@ def test_skip_sampler_rate_at_the_size_of_a_wide_layer(ops):
     T = 42949672
     base = torch.zeros((1024, 128), dtype=torch.int64, device="cuda")
     rows = ops.flip_rows_skip(base, 8192, 64, T, 7)
-    cnt = rows.cnt.view(torch.int16).to(torch.float64)
+    cnt = rows.cnt.to(torch.float64)
     n = cnt.numel() * 8192
     p = T / 2 ** 32
     assert abs(float(cnt.sum()) / n - p) < 4 * (p / n) ** 0.5
@@ -239,3 +212,124 @@ def test_skip_sampler_rate_at_the_size_of_a_wide_layer(ops):
     W = ops.flip_rows_to_weights(rows)
     per_col = ops.unpack(W.view(-1, 128)).view(64 * 1024, 8192).float().mean(dim=0)
     assert float((per_col - p).abs().max()) < 6 * (p / (64 * 1024)) ** 0.5
+
+
+def test_skip_sampler_reports_rows_beyond_the_capacity(ops, oracle):
+    """A capacity below what some rows need: those rows are cut to capacity * 8 flips and counted, the others are
+    what they are with room to spare."""
+    g = np.random.default_rng(4)
+    R, C, D, T = 70, 512, 9, int(0.05 * 2 ** 32)
+    base = dev(sparse_mask(g, (R, C), 0.5))
+    full = ops.flip_rows_skip(base, C, D, T, 11)
+    need = (full.cnt + 7) // 8
+    cap = int(need.max().item()) - 1
+    cut = ops.flip_rows_skip(base, C, D, T, 11, cap=cap)
+    assert cut.overflowed() == int((need > cap).sum().item()) > 0
+    fine = (need <= cap)
+    assert torch.equal(cut.cnt[fine], full.cnt[fine]) and bool((cut.cnt[~fine] == 8 * cap).all())
+    Wc, Wf = ops.flip_rows_to_weights(cut), ops.flip_rows_to_weights(full)
+    assert torch.equal(Wc[fine], Wf[fine])
+
+
+@pytest.mark.parametrize("D,R,C,first,spread", [(3, 64, 64, 0, 0.2), (2, 100, 200, 8, 0.05), (3, 1024, 2048, 0, 0.02),
+                                                (2, 70, 300, 3, 0.1), (40, 130, 72, 0, 0.3), (2, 9, 8192, 4, 0.01),
+                                                (3, 5, 77, 1, 0.05), (2, 16, 16384, 0, 0.004)])
+def test_thinning_sampler_vs_oracle(ops, oracle, D, R, C, first, spread):
+    """Flip lists under a per-element law == the oracle's restatement of the thinned walk, given the same law and the
+    same table (the one the library made on the device); sums from the lists == the oracle's bmm."""
+    g = np.random.default_rng(D + R + C)
+    Kw = (C + 63) // 64
+    P = np.where(g.random((R, C)) < 0.5, g.random((R, C)) * spread, 1.0 - g.random((R, C)) * spread).astype(np.float16)
+    law_np, base_bits, tmax = oracle.flip_law(P)
+    base = oracle.pack(base_bits, np.int64)
+    # the table: made on the device from the largest threshold
+    tbl = torch.zeros((int(ops._lib.load().nb_skip_table_words()),), dtype=torch.int32, device="cuda")
+    thr = torch.tensor([tmax - 2 ** 32 if tmax >= 2 ** 31 else tmax], dtype=torch.int32, device="cuda")
+    ops._lib.call("nb_skip_table", tbl.data_ptr(), thr.data_ptr(), None)
+    th = host(tbl).view(np.uint32)
+    Kt = int(th[0])
+    cdf = th[4:4 + Kt].copy()
+    assert int(th[2]) == tmax and (np.diff(cdf.astype(np.int64)) >= 0).all()
+    ref = ops.skip_table(tmax)
+    assert Kt == len(ref) and np.abs(cdf.astype(np.int64) - ref.astype(np.int64)).max() <= 1   # another libm: +-1
+    law = ops.FlipLaw(dev(law_np.view(np.int16)).view(torch.uint16), dev(base), tbl.view(torch.uint32), C)
+    seed, sub = 0xFEED + C, 5
+    want_flips = oracle.skip_flips_thin(law_np, cdf, tmax, seed, sub, first, D).reshape(D, R, Kw)
+    cap = ops.flip_capacity(C, min(2 * spread, 0.5))
+    rows = ops.flip_rows_thin(law, D, seed, cap, subsequence=sub, first=first)
+    assert rows.overflowed() == 0
+    W = ops.flip_rows_to_weights(rows)
+    np.testing.assert_array_equal(host(W), base[None] ^ want_flips)
+    np.testing.assert_array_equal(host(rows.cnt).astype(np.int64),
+                                  np.unpackbits(want_flips.view(np.uint8), axis=2, bitorder="little").sum(axis=2))
+    x = sparse_mask(g, (D, C), 0.5)
+    want = oracle.bmm(base[None] ^ want_flips, x.reshape(D, Kw, 1))[:, :, 0]
+    np.testing.assert_array_equal(host(ops.bmm(rows, dev(x).view(D, Kw, 1)))[:, :, 0], want)
+    if D * R * C <= 500000:
+        mask, bflag = decode_flip_rows(rows)
+        fb = np.unpackbits(want_flips.view(np.uint8), axis=2, bitorder="little").astype(bool)
+        np.testing.assert_array_equal(mask, fb)
+        bb = np.unpackbits(base.view(np.uint8), axis=1, bitorder="little").astype(bool)
+        np.testing.assert_array_equal(bflag, mask & bb[None])
+
+
+@pytest.mark.parametrize("D,R,C,p", [(64, 8, 64, 0.1), (300, 70, 200, 0.05), (1024, 16, 8192, 0.01), (5, 1, 1, 0.5),
+                                     (33, 130, 960, 0.0), (17, 9, 32704, 0.001)])
+def test_weighted_sum_over_flip_lists(ops, oracle, D, R, C, p):
+    """weighted_sum on the lists against the float64 sum over the unpacked bits (exact up to the scaling of the
+    weights to integers and the final rounding to fp16), and against the dense kernel on the materialised weights."""
+    g = np.random.default_rng(D + R + C)
+    Kw = (C + 63) // 64
+    base = sparse_mask(g, (R, C), 0.5)
+    W = base[None] ^ sparse_mask(g, (D, R, C), p)
+    rows = ops.flip_rows_from_weights(dev(W), dev(base))
+    w = (g.standard_normal(D) * (1 + 10 * (D % 3))).astype(np.float16)
+    got = ops.weighted_sum(rows, dev(w), C)
+    assert got.dtype == torch.float16 and tuple(got.shape) == (R, C)
+    bits = np.unpackbits(W.view(np.uint8), axis=2, bitorder="little")[:, :, :C].astype(np.float64)
+    want = np.einsum("d,drc->rc", w.astype(np.float64), bits)
+    scale = np.abs(w.astype(np.float64)).sum() + 1.0
+    err = np.abs(host(got).astype(np.float64) - want)
+    # half an fp16 ulp of the result + the integer scaling (2**-29 of sum |w| per term, at most D terms)
+    tol = np.maximum(np.abs(want), 2.0 ** -14) * 2.0 ** -11 + D * scale * 2.0 ** -28
+    assert (err <= tol).all(), float((err / tol).max())
+    dense = ops.weighted_sum(dev(W), dev(w), C)
+    np.testing.assert_allclose(host(got).astype(np.float64), host(dense).astype(np.float64), rtol=2e-3,
+                               atol=2e-3 * float(np.abs(w.astype(np.float64)).sum()) / max(D, 1) ** 0.5 + 1e-6)
+    # the same call twice: integer additions commute, so the result does not depend on the order of arrival
+    assert torch.equal(got, ops.weighted_sum(rows, dev(w), C))
+
+
+@pytest.mark.parametrize("R,C,scale", [(64, 64, 1.0), (10, 1000, 0.01), (1024, 1024, 3.0), (7, 3, 100.0), (33, 130, 0.0)])
+def test_law_kernels_against_the_tensor_expression(ops, R, C, scale):
+    """probabilities / thresholds / sparse law of a layer against modules/binary.py:59-60 evaluated by torch:
+    P = sigmoid((w / (mean|w| + 1e-5) * 5).float()).half().  The elementwise steps round where the tensor expression
+    rounds; torch's fp16 mean adds in fp32 in its own order, the kernel's mean is the exact one rounded once, so the
+    denominators may differ by an fp16 ulp when the mean falls next to a rounding boundary: the test asks for equal
+    denominators and, given those, bit-equal probabilities."""
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(R * 1000 + C)
+    w = (torch.randn(R, C, device="cuda", generator=gen) * scale).to(torch.float16)
+    denom = w.abs().mean() + 1e-5
+    P_t = torch.sigmoid((w / denom * 5).float()).half()
+    P = ops.probabilities_from_weights(w)
+    exact = (w.abs().double().sum() / w.numel()).item()
+    assert float(w.abs().mean()) == float(torch.tensor(exact, dtype=torch.float64).to(torch.float16)), \
+        "the test's weights put torch's mean on the other side of a rounding boundary: pick another seed"
+    assert torch.equal(P, P_t)
+    T = ops.thresholds_from_weights(w)
+    assert torch.equal(T.view(torch.int32), ops.thresholds_from_p(P_t).view(torch.int32))
+    law = ops.flip_law_from_weights(w)
+    Pf = P_t.float()
+    one = Pf >= 0.5
+    y = torch.where(one, 1.0 - Pf, Pf).half()
+    want_law = (y.view(torch.int16) & 0x7FFF) | torch.where(one, torch.tensor(-32768, dtype=torch.int16, device="cuda"),
+                                                            torch.tensor(0, dtype=torch.int16, device="cuda"))
+    assert torch.equal(law.law.view(torch.int16), want_law)
+    assert torch.equal(law.base, ops.pack(one, torch.int64))
+    tmax = int(torch.floor(y.double() * 2.0 ** 32).max().item())
+    th = host(law.table.view(torch.int32)).view(np.uint32)
+    assert int(th[2]) == tmax
+    ref = ops.skip_table(tmax)
+    assert int(th[0]) == len(ref) and (len(ref) == 0 or np.abs(th[4:4 + len(ref)].astype(np.int64) - ref.astype(np.int64)).max() <= 1)
+    assert abs(law.max_flip_probability() - tmax / 2.0 ** 32) < 1e-12

@@ -4,6 +4,8 @@ import numpy as np
 import pytest
 import torch
 
+from golden_util import torch_mean_fp16
+
 pytestmark = pytest.mark.gpu
 
 
@@ -113,9 +115,8 @@ def test_conv_forward(binary, oracle, dtype, C, O, k, pad, stride):
             continue
         assert out.dtype == torch.bool and tuple(out.shape) == act.shape
         if batch_norm:
-            # :147-155 with the mean taken from exact integer sums: fp16(float32(sum) / float32(h*w))
-            npix = act.shape[1] * act.shape[2]
-            mean = (act.sum(axis=(1, 2), dtype=np.int64).astype(np.float32) / np.float32(npix)).astype(np.float16)
+            # :147-155 with the mean taken from exact integer sums, as torch's fp16 mean forms it
+            mean = torch_mean_fp16(act.sum(axis=(1, 2), dtype=np.int64), D * O, act.size)
             bn = (layer.bias + layer.bias_noise).detach().cpu().numpy()                           # fp16 [D, O]
             thresh = (bn + mean).astype(np.float16)
             np.testing.assert_array_equal(out.cpu().numpy(), act.astype(np.float16) > thresh[:, None, None, :])
@@ -245,20 +246,29 @@ def test_reference_import_names_resolve(binary):
 def test_conv_bn_thresholds_equal_the_layer_arithmetic():
     from nesgpu_amd.extensions import booleanOperations as ops
     """conv_bn_thresholds against the tensor expression it replaces (modules/binary.py:147-155 on exact pixel sums):
-    mean = fp16(float32(sum of activations) / float32(pixels)), thr = fp16(fp16(bias + noise) + mean),
+    mean = the exact product float32(sum of activations) * (float32(D * O) / float32(D * O * pixels)) rounded once to
+    fp16, as torch's fp16 mean over the pixels of a [D, h, w, O] map; thr = fp16(fp16(bias + noise) + mean),
     threshold = floor(thr) + K; random sums over the whole range, biases that round in fp16, and the non-finite cases
     decided like `activation > thr` (never for NaN and +inf, always for -inf)."""
     g = torch.Generator(device="cuda")
     g.manual_seed(11)
-    for D, O, K, pixels in [(64, 64, 576, 1024), (7, 5, 144, 4096), (300, 16, 27, 49), (3, 130, 2048, 1)]:
+    for D, O, K, pixels in [(64, 64, 576, 1024), (7, 5, 144, 4096), (300, 16, 27, 49), (3, 130, 2048, 1),
+                            (50, 24, 216, 112), (9, 64, 576, 56)]:
         sums = torch.randint(0, K * pixels + 1, (D, O), dtype=torch.int32, device="cuda", generator=g)
         bias = (torch.randn(O, device="cuda", generator=g) * 30).to(torch.float16)
         noise = (torch.rand(D, O, device="cuda", generator=g) - 0.5).to(torch.float16)
         got = ops.conv_bn_thresholds(sums, bias, noise, K, pixels)
         s64 = sums.to(torch.int64)
-        mean = ((2 * s64 - K * pixels).to(torch.float32) / float(pixels)).to(torch.float16)
+        tot = 2 * s64 - K * pixels
+        mean = torch.from_numpy(torch_mean_fp16(tot.cpu().numpy(), D * O, D * O * pixels)).cuda()
         want = torch.floor((bias + noise + mean).to(torch.float32)).to(torch.int32) + K
         assert got.dtype == torch.int32 and torch.equal(got, want)
+        # torch's own fp16 mean of a map with these pixel sums (an activation per pixel: the sum spread evenly, the
+        # remainder on the first pixels), wherever its fp32 sums are exact
+        if K <= 2048 and K * pixels < 2 ** 24:
+            q, r = torch.div(tot, pixels, rounding_mode="floor"), torch.remainder(tot, pixels)
+            amap = q[:, None, :] + (torch.arange(pixels, device="cuda")[None, :, None] < r[:, None, :]).to(torch.int64)
+            assert torch.equal(amap.to(torch.float16).view(D, pixels, 1, O).mean(dim=[1, 2]), mean)
     sums = torch.full((1, 4), 100, dtype=torch.int32, device="cuda")
     bias = torch.tensor([float("nan"), float("inf"), float("-inf"), 60000.0], dtype=torch.float16, device="cuda")
     noise = torch.tensor([[0.0, 0.0, 0.0, 60000.0]], dtype=torch.float16, device="cuda")       # 60000 + 60000 = inf
@@ -303,8 +313,32 @@ def test_conv_bn_thresholds_from_input_equal_the_two_steps(C, O, k, pad, stride,
         ops.conv_engine(prev)
 
 
+@pytest.mark.parametrize("C,O,k", [(16, 16, 3), (8, 32, 3), (3, 8, 5), (24, 64, 3)])
+def test_pixel_sums_ignore_input_bits_above_the_channels(C, O, k):
+    """Tap-packed layers: an input word with bits set above the layer's channel count gives the same pixel sums (and
+    so the same batch-norm thresholds) under every engine, namely those of the input with these bits cleared."""
+    from nesgpu_amd.extensions import booleanOperations as ops
+    g = torch.Generator(device="cuda")
+    g.manual_seed(C * 7 + O)
+    D, H, W = 130, 9, 11
+    x = torch.randint(-2 ** 62, 2 ** 62, (D, H, W, 1), dtype=torch.int64, device="cuda", generator=g)   # stray bits
+    clean = x & ((1 << C) - 1)
+    f = torch.randint(0, 2 ** C, (D, k * k, O), dtype=torch.int64, device="cuda", generator=g)
+    assert ops.tap_packing_applies(C, 1, torch.int64)
+    geom = (k, k, k // 2, k // 2, 1, 1)
+    prev = ops.conv_engine(0)
+    try:
+        ops.conv_engine(1)
+        want = ops.conv_popc_sums(clean, f, *geom, in_bits=C)
+        for eng in (0, 1, 2):
+            ops.conv_engine(eng)
+            assert torch.equal(ops.conv_popc_sums(x, f, *geom, in_bits=C), want), eng
+    finally:
+        ops.conv_engine(prev)
 
-@pytest.mark.parametrize("K,M,Z", [(16384, 10, 1024), (4096, 33, 256), (8192, 7, 64), (3000, 5, 128), (65504, 3, 256)])
+
+@pytest.mark.parametrize("K,M,Z", [(16384, 10, 1024), (4096, 33, 256), (8192, 7, 64), (3000, 5, 128), (65504, 3, 256),
+                                   (4096, 33, 1000), (3000, 5, 100), (2100, 9, 7)])
 def test_linear_bn_beyond_2048_inputs_equals_the_tensor_expression(K, M, Z):
     """BinarizedLinear(batch_norm=True) with rows longer than fp16's exact integers: the one-call kernel with
     fp16-rounded activations against the reference's tensor expression (modules/binary.py:97-102) evaluated by torch,
@@ -335,3 +369,107 @@ def test_linear_bn_beyond_2048_inputs_equals_the_tensor_expression(K, M, Z):
         want = activation > thresh
     assert got.dtype == torch.bool and torch.equal(got, want)
     assert 0.02 < float(want.float().mean()) < 0.98
+
+
+def _saturated(shape, g, lo=0.9, hi=1.6):
+    """Latent weights of one magnitude scale and random signs: flip probabilities sigmoid(-5 |w| / mean|w|) of about
+    a percent, the regime in which a wide layer keeps its members as base + flip lists."""
+    w = (lo + (hi - lo) * torch.rand(shape, device="cuda", generator=g)) * (torch.randint(0, 2, shape, device="cuda", generator=g) * 2 - 1)
+    return w.to(torch.float16)
+
+
+@pytest.mark.parametrize("mode", ["law", "flip_probability"])
+@pytest.mark.parametrize("threshold,batch_norm,pack_output", [(True, False, True), (True, False, False),
+                                                              (False, False, False), (True, True, False)])
+def test_wide_linear_layer_in_sparse_form(binary, oracle, mode, threshold, batch_norm, pack_output):
+    """BinarizedLinear keeps a wide layer's members as base + flip lists when their flip probabilities are small
+    (sparse="auto"): the lists are the oracle's restatement of the sampler's walk on the layer's own law, forward
+    equals the oracle's bmm on those weights, and update equals weighted_sum on them."""
+    from nesgpu_amd.extensions import booleanOperations as ops
+    K, M, D = 4096, 70, 24
+    g = torch.Generator(device="cuda")
+    g.manual_seed(5 + len(mode))
+    kw = dict(flip_probability=0.01) if mode == "flip_probability" else {}
+    lin = binary.BinarizedLinear(K, M, D, threshold=threshold, batch_norm=batch_norm, pack_output=pack_output, **kw)
+    with torch.no_grad():
+        lin.weight.copy_(_saturated((M, K), g))
+        if threshold:
+            lin.bias.copy_((torch.randn(M, device="cuda", generator=g) * 20).to(torch.float16))
+    lin.set_seed(77)
+    lin.set_noise()
+    rows = lin.weight_noise
+    assert isinstance(rows, ops.FlipRows) and rows.overflowed() == 0
+    # the members' weights, regenerated on the host
+    if mode == "law":
+        P = lin.probabilities().cpu().numpy()
+        law_np, base_bits, tmax = oracle.flip_law(P)
+        plan = lin._sparse_plan()
+        np.testing.assert_array_equal(plan["law"].law.view(torch.int16).cpu().numpy().view(np.uint16), law_np)
+        th = plan["law"].table.view(torch.int32).cpu().numpy().view(np.uint32)
+        assert int(th[2]) == tmax
+        flips = oracle.skip_flips_thin(law_np, th[4:4 + int(th[0])].copy(), tmax, 77, 0, 0, D)
+        base = oracle.pack(base_bits, np.int64)
+    else:
+        base = oracle.pack(lin.weight.detach().cpu().numpy() >= 0, np.int64)
+        flips = oracle.skip_flips(ops.skip_table(int(0.01 * 2 ** 32)), 77, 0, 0, D * M, K)
+    W = base[None] ^ flips.reshape(D, M, K // 64)
+    np.testing.assert_array_equal(ops.flip_rows_to_weights(rows).cpu().numpy(), W)
+    rate = np.unpackbits(flips.view(np.uint8), axis=1, bitorder="little").mean()
+    assert 0.002 < rate < 0.03
+    x = torch.randint(-2 ** 62, 2 ** 62, (D, K // 64), dtype=torch.int64, device="cuda", generator=g)
+    lin.perturbed_flag = True
+    with torch.no_grad():
+        out = lin(x)
+    act = 2 * oracle.bmm(W, x.cpu().numpy().reshape(D, -1, 1))[:, :, 0].astype(np.int64) - K
+    if not threshold:
+        np.testing.assert_array_equal(out.cpu().numpy(), act)
+    else:
+        thr = (lin.bias + lin.bias_noise).detach()
+        act_t = torch.from_numpy(act.astype(np.int32)).cuda()
+        if batch_norm:
+            thr = thr + act_t.type(torch.float16).mean(dim=0, keepdim=True)
+        want = act_t > thr                                                      # modules/binary.py:97-103
+        if pack_output:
+            assert torch.equal(out, ops.pack(want, torch.int64))
+        else:
+            assert torch.equal(out, want)
+    # update: the gradient estimate from the lists against the dense op on the materialised weights
+    fit = torch.randn(D, device="cuda", generator=g)
+    lin.update(fit)
+    wts = (fit.half() - fit.half().mean())
+    dense = ops.weighted_sum(torch.from_numpy(W).cuda(), wts.contiguous(), K).float() + 1e-3 * lin.weight.float()
+    torch.testing.assert_close(lin.weight.grad.float(), dense, rtol=2e-3, atol=2e-2)
+    lin.free_memory()
+    assert lin.weight_noise is None and not lin._cache
+
+
+def test_sparse_form_is_chosen_by_the_flip_probabilities(binary):
+    from nesgpu_amd.extensions import booleanOperations as ops
+    g = torch.Generator(device="cuda")
+    g.manual_seed(3)
+    lin = binary.BinarizedLinear(2048, 16, 8)
+    lin.set_seed(1)
+    lin.set_noise()                                          # zero latent weights: every probability 1/2
+    assert isinstance(lin.weight_noise, torch.Tensor) and tuple(lin.weight_noise.shape) == (8, 16, 32)
+    with torch.no_grad():
+        lin.weight.copy_(_saturated((16, 2048), g))
+    lin.set_noise()
+    assert isinstance(lin.weight_noise, ops.FlipRows)
+    with torch.no_grad():
+        lin.weight[3, 5] = 0.0                               # one undecided weight: walking at 1/2 would not pay
+    lin.set_noise()
+    assert isinstance(lin.weight_noise, torch.Tensor)
+    narrow = binary.BinarizedLinear(1024, 16, 8)
+    with torch.no_grad():
+        narrow.weight.copy_(_saturated((16, 1024), g))
+    narrow.set_seed(1)
+    narrow.set_noise()
+    assert isinstance(narrow.weight_noise, torch.Tensor)     # short rows stay dense
+    with pytest.raises(NotImplementedError):
+        binary.BinarizedLinear(1024, 16, 8, dtype=torch.int32, sparse=True).set_noise()
+    off = binary.BinarizedLinear(2048, 16, 8, sparse=False, flip_probability=0.01)
+    off.set_seed(2)
+    off.set_noise()
+    assert isinstance(off.weight_noise, torch.Tensor)
+    flips = ops.unpack((off.weight_noise ^ off.sign_base()[None]).view(-1, 32)).float().mean().item()
+    assert abs(flips - 0.01) < 0.002

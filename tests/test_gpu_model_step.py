@@ -7,6 +7,8 @@ import numpy as np
 import pytest
 import torch
 
+from golden_util import torch_mean_fp16
+
 pytestmark = pytest.mark.gpu
 
 
@@ -70,7 +72,7 @@ def host_forward(oracle, layers, images_bits, D):
         H = a.shape[1]
         x = oracle.pack(a.reshape(-1, C), np.int64).reshape(D, H, H, Cw) if a.dtype == np.bool_ else a
         act = 2 * oracle.conv(x, filt, 3, 3, 1, 1, 1, 1).astype(np.int64) - K        # modules/binary.py:145
-        mean = (act.sum(axis=(1, 2)).astype(np.float32) / np.float32(H * H)).astype(np.float16)   # :151, exact sums
+        mean = torch_mean_fp16(act.sum(axis=(1, 2)), D * O, act.size)                   # :151, exact sums
         thr = (f16(conv.bias)[None] + f16(conv.bias_noise)).astype(np.float16)
         thr = (thr + mean).astype(np.float16)
         bits = act > thr[:, None, None, :].astype(np.float64)                         # :155

@@ -7,7 +7,8 @@ import numpy as np
 import pytest
 import torch
 
-from golden_util import (BMM_CASES, CONV_CASES, PACK_WIDTHS, POOL_CASES, SMP_CASES, TAGS, load_ops, load_philox)
+from golden_util import (BMM_CASES, CONV_CASES, PACK_WIDTHS, POOL_CASES, SMP_CASES, TAGS, load_ops, load_philox,
+                         torch_mean_fp16)
 
 pytestmark = pytest.mark.gpu
 
@@ -1059,11 +1060,12 @@ def test_conv_engine_selector_round_trip(ops):
 
 
 def _bn_expected(popc, bias, noise, K):
-    """numpy restatement of the population-mean threshold: exact integer sums, one rounding to float32, one division,
-    one rounding to fp16; fp16 additions in the reference's order (modules/binary.py:99-101); exact comparison."""
-    Z = popc.shape[0]
+    """numpy restatement of the population-mean threshold: exact integer sums, one rounding to float32, torch's
+    multiplication by float32(M) / float32(Z * M), one rounding to fp16; fp16 additions in the reference's order
+    (modules/binary.py:99-101); exact comparison."""
+    Z, M = popc.shape
     act = 2 * popc.astype(np.int64) - K
-    mean = (act.sum(axis=0).astype(np.float32) / np.float32(Z)).astype(np.float16)
+    mean = torch_mean_fp16(act.sum(axis=0), M, Z * M)
     with np.errstate(invalid="ignore", over="ignore"):
         thr = (bias[None, :] + noise).astype(np.float16)
         thr = (thr + mean[None, :]).astype(np.float16)
@@ -1080,7 +1082,8 @@ def test_bmv_bn_act_vs_oracle(ops, oracle, dtype):
     g = rng(31337)
     vec = 16 // np.dtype(nd).itemsize
     for ci, (Z, M, Kw) in enumerate([(16, 64, 4), (7, 10, 2), (33, 130, 16), (5, 64, vec * 16), (12, 256, vec * 32),
-                                     (3, 1, 1), (100, 33, 3), (9, 128, 0), (64, 1000, 8)]):
+                                     (3, 1, 1), (100, 33, 3), (9, 128, 0), (64, 1000, 8), (1000, 24, 5),
+                                     (112, 56, 9)]):
         K = Kw * bits - (ci % 3) * (Kw > 0)                       # the true bit count may stop inside the last word
         A = rand_words(g, (Z, M, Kw), nd)
         x = rand_words(g, (Z, Kw), nd)
@@ -1093,7 +1096,7 @@ def test_bmv_bn_act_vs_oracle(ops, oracle, dtype):
         noise = ((g.random((Z, M)) - 0.5) * 6).astype(np.float16)
         # make some thresholds land exactly on an activation: noise = act - mean - bias, then the compare is a tie
         act = 2 * popc.astype(np.int64) - K
-        mean = (act.sum(axis=0).astype(np.float32) / np.float32(Z)).astype(np.float16)
+        mean = torch_mean_fp16(act.sum(axis=0), M, Z * M)
         tie = g.random((Z, M)) < 0.2
         noise[tie] = (act - mean[None, :].astype(np.float64) - bias[None, :].astype(np.float64)).astype(np.float16)[tie]
         noise[0, 0] = np.float16(np.inf)
@@ -1111,9 +1114,9 @@ def test_bmv_bn_act_vs_oracle(ops, oracle, dtype):
         gotp = ops.bmv_bn_act(Ad, xd.view(Z, Kw, 1), bd, nz, K, pack=True, workspace=ws)
         assert gotp.dtype == dtype and tuple(gotp.shape) == (Z, (M + bits - 1) // bits)
         np.testing.assert_array_equal(host(gotp), oracle.pack(want, nd), err_msg="case %d packed" % ci)
-        # against torch's own expression of the reference wherever that is exact (activations within fp16's integers,
-        # a population whose reciprocal is exact)
-        if K <= 2048 and Z & (Z - 1) == 0:
+        # against torch's own expression of the reference wherever its fp32 sums are exact (activations within
+        # fp16's integers, totals below 2**24): any population size, also those whose reciprocal is not exact
+        if K <= 2048 and Z * K < 2 ** 24:
             act_t = dev(act.astype(np.int32))
             thresh = bd + nz
             thresh += act_t.type(torch.float16).mean(dim=0, keepdim=True)

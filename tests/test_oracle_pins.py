@@ -298,3 +298,61 @@ def test_skip_flips_against_searchsorted_and_the_geometric_law(oracle):
     ones = oracle.skip_flips(oracle.skip_cdf(2 ** 32 - 1), 3, 0, 0, 4, 130)
     assert np.unpackbits(ones.view(np.uint8), axis=1, bitorder="little")[:, :130].all()
     assert not oracle.skip_flips(oracle.skip_cdf(0), 3, 0, 0, 4, 130).any()
+
+
+def test_skip_flips_thin_against_a_numpy_walk_and_the_per_column_law(oracle):
+    """Thinned gap sampling (per-element flip probabilities): the C restatement against an independent evaluation
+    (searchsorted + cumsum over the pinned Philox words, the acceptance in Python integers), then what the law fixes:
+    every column flips at its own rate, neighbouring columns are uncorrelated, and a law whose probabilities all equal
+    the largest one accepts everything, i.e. reduces to the plain walk over the pairs' first words."""
+    g = np.random.default_rng(77)
+    R, C, D = 3, 500, 4
+    # probabilities on both sides of 1/2, most of them near 0 or 1: flip probabilities of a few percent
+    P = np.where(g.random((R, C)) < 0.5, g.random((R, C)) * 0.06, 1.0 - g.random((R, C)) * 0.06).astype(np.float16)
+    law, base, tmax = oracle.flip_law(P)
+    assert ((law >> 15).astype(bool) == (P.astype(np.float32) >= 0.5)).all()
+    y = (law & 0x7FFF).view(np.float16).astype(np.float64)
+    np.testing.assert_array_equal(y, np.minimum(P.astype(np.float64), 1.0 - P.astype(np.float64)))
+    tf = np.floor(y * 2.0 ** 32).astype(np.uint64)
+    assert tmax == int(tf.max())
+    cdf = oracle.skip_cdf(tmax)
+    seed, sub = 0x1234567, 3
+    for first in (0, 6, 1):
+        got = oracle.skip_flips_thin(law, cdf, tmax, seed, sub, first, D)
+        bits = np.unpackbits(got.view(np.uint8), axis=1, bitorder="little")
+        assert not bits[:, C:].any()
+        for q in range(D * R):
+            words = oracle.philox_words(seed, sub, first + q * C, 2 * C + 2)
+            gap, acc = words[0::2], words[1::2]
+            rank = np.searchsorted(cdf, gap, side="right").astype(np.int64)
+            pos = np.cumsum(np.where(rank < len(cdf), rank + 1, len(cdf))) - 1
+            want = np.zeros(bits.shape[1], np.uint8)
+            for i in np.flatnonzero((pos < C) & (rank < len(cdf))):
+                if int(acc[i]) * tmax < (int(tf[q % R, pos[i]]) << 32):
+                    want[pos[i]] = 1
+            np.testing.assert_array_equal(bits[q], want, err_msg="first=%d row %d" % (first, q))
+    # rates: many members of one row whose probabilities come in two levels
+    R2, C2, D2 = 1, 256, 6000
+    y2 = np.where(np.arange(C2) % 2 == 0, 0.05, 0.0125).astype(np.float16)
+    law2, _, tmax2 = oracle.flip_law(y2[None, :])
+    bits = np.unpackbits(oracle.skip_flips_thin(law2, oracle.skip_cdf(tmax2), tmax2, 9, 0, 0, D2).view(np.uint8),
+                         axis=1, bitorder="little")[:, :C2].astype(np.float64)
+    p2 = y2.astype(np.float64)
+    rate = bits.mean(axis=0)
+    assert (np.abs(rate - p2) < 5 * np.sqrt(p2 * (1 - p2) / D2)).all()
+    assert abs(rate[0::2].mean() - p2[0]) < 4 * np.sqrt(p2[0] / (D2 * C2 / 2))
+    assert abs(rate[1::2].mean() - p2[1]) < 4 * np.sqrt(p2[1] / (D2 * C2 / 2))
+    a, b = bits[:, :-1], bits[:, 1:]
+    assert abs((a * b).mean() - p2[0] * p2[1]) < 5 * np.sqrt(p2[0] * p2[1] / a.size)      # neighbours independent
+    # all probabilities equal to the largest: every column the walk reaches flips
+    y3 = np.full((2, 300), 0.03, dtype=np.float16)
+    law3, _, tmax3 = oracle.flip_law(y3)
+    cdf3 = oracle.skip_cdf(tmax3)
+    got = np.unpackbits(oracle.skip_flips_thin(law3, cdf3, tmax3, 5, 2, 0, 3).view(np.uint8), axis=1, bitorder="little")
+    for q in range(6):
+        gap = oracle.philox_words(5, 2, q * 300, 600)[0::2]
+        rank = np.searchsorted(cdf3, gap, side="right").astype(np.int64)
+        pos = np.cumsum(np.where(rank < len(cdf3), rank + 1, len(cdf3))) - 1
+        want = np.zeros(got.shape[1], np.uint8)
+        want[pos[(pos < 300) & (rank < len(cdf3))]] = 1
+        np.testing.assert_array_equal(got[q], want)
