@@ -15,6 +15,7 @@
 // finished a row starts its next member at once), and every row's entries go to the fixed place the list layout
 // gives them (nb_flip.hip), so nothing has to be counted first.
 #include <cmath>
+#include <cstdlib>
 #include <mutex>
 
 #include "nb_common.hpp"
@@ -89,6 +90,7 @@ struct GenArgs {
     PhiloxKey key;
     int64_t D, R;
     int C, Kw, S, cap, MC, rb_shift;  // MC members per workgroup; 1 << rb_shift rows per workgroup
+    int group;                        // lanes (rows of one member) that start their members together
 };
 
 // ALIGNED: every row starts on a block boundary of the stream (C and first multiples of 4): a block's four words are
@@ -227,6 +229,117 @@ __global__ __launch_bounds__(1024) void fl_gen_kernel(const GenArgs a)
             step(rank[0], acc);
         }
         if (live && pos >= C) finish_row();
+    }
+}
+
+// Uniform probability, rows on block boundaries of the stream: the lanes of a wave walk in step, eight words (two
+// blocks) to a 16-byte piece.  Every word of a live row is a flip unless it lies beyond the table (rank Kt: the slot
+// gets a sentinel, which the list layout allows anywhere) or the row has ended (sentinels to the end of the piece),
+// so word i of an iteration is slot i of the piece for every lane: nothing about an entry's place is per lane, and a
+// lane that has finished its row starts its next member with the next piece.  Same words, same ranks, same flips as
+// fl_gen_kernel<true, false>; the lists differ only in where sentinels stand.
+__global__ __launch_bounds__(1024) void fl_gen_static_kernel(const GenArgs a)
+{
+    extern __shared__ uint32_t gen_lds[];
+    uint32_t *tab1 = gen_lds;
+    uint32_t *rowdata = gen_lds + kSkipMaxTable + 2;
+    const int Kt = (int)a.table[0];
+    const float inv_log2q = __uint_as_float(a.table[1]);
+    const int RB = 1 << a.rb_shift;
+    const int nrg = (int)((a.R + RB - 1) >> a.rb_shift);
+    const int rg = (int)(blockIdx.x % (unsigned)nrg), mc = (int)(blockIdx.x / (unsigned)nrg);
+    const int64_t r0 = (int64_t)rg << a.rb_shift;
+    for (int i = threadIdx.x; i < Kt + 2; i += blockDim.x)
+        tab1[i] = i == 0 ? 0u : (i <= Kt ? a.table[kSkipHeader + i - 1] : 0xFFFFFFFFu);
+    const int row_dwords = 2 * a.Kw;
+    {
+        const uint32_t *src = static_cast<const uint32_t *>(a.rows);
+        for (int rr = 0; rr < RB && r0 + rr < a.R; rr++)
+            for (int i = threadIdx.x; i < row_dwords; i += blockDim.x)
+                rowdata[rr * row_dwords + i] = src[(r0 + rr) * row_dwords + i];
+    }
+    __syncthreads();
+    const int rr = (int)threadIdx.x & (RB - 1);
+    const int64_t r = r0 + rr;
+    const int slots = (int)blockDim.x >> a.rb_shift;
+    const int64_t dend = (int64_t)(mc + 1) * a.MC < a.D ? (int64_t)(mc + 1) * a.MC : a.D;
+    int64_t d = (int64_t)mc * a.MC + ((int)threadIdx.x >> a.rb_shift);
+    const uint32_t *myrow = rowdata + rr * row_dwords;
+    const uint32_t sentinel = (uint32_t)(4 * a.Kw) << 5;
+    const float c0 = -32.0f * inv_log2q;
+    const int C = a.C;
+    if (r >= a.R) d = dend;
+    if (Kt == 0) {
+        for (; d < dend; d += slots) a.info[d * a.R + r] = 0u;
+        return;
+    }
+    bool live = d < dend;
+    int64_t q = 0;
+    uint64_t blk = 0;
+    uint4 *dst = a.entries;
+    int pos = C, n = 0, piece = 0;
+    auto start_row = [&]() {
+        live = d < dend;
+        if (live) {
+            q = d * a.R + r;
+            blk = (a.key.first + (uint64_t)q * (uint64_t)C) >> 2;
+            dst = a.entries + ((d * a.S + (r >> 6)) * (int64_t)a.cap) * 64 + (r & 63);
+        }
+        pos = live ? -1 : C;
+        n = 0;
+        piece = 0;
+    };
+    start_row();
+    // The RB lanes that hold the rows of one 16 RB-byte run of a member's pieces (a whole 128-byte line for eight
+    // rows) start every member together: they are then on the same piece in every iteration and one store
+    // instruction writes the run in one piece (single 16-byte stores to scattered lines reach a third of the
+    // memory's write rate).  A lane whose row has ended waits for the longest of the group's rows.
+    bool rowlive = live;
+    const int G = RB < a.group ? RB : a.group;
+    const int gshift = (int)(threadIdx.x & 63u) & ~(G - 1);
+    const unsigned long long gmask = (1ull << G) - 1ull;
+    while (__any(live)) {
+        uint32_t e[8];
+        const int n_before = n;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const uint4 w = philox_block(a.key, blk++);
+            const uint32_t u[4] = {w.x, w.y, w.z, w.w};
+            int rank[4];
+            skip_ranks<4>(rank, tab1, Kt, u, inv_log2q, c0);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const bool beyond = rank[i] >= Kt;               // the word lies past the table: Kt columns on, no flip
+                pos = pos + rank[i] + (beyond ? 0 : 1);
+                const bool flip = !beyond && pos < C;
+                const uint32_t pc = (uint32_t)(pos < C ? pos : 0);
+                const uint32_t b = __builtin_amdgcn_ubfe(myrow[pc >> 5], pc, 1);
+                const uint32_t ent = pc + (pc & ~31u) + (b << 5);   // ((2 * (pc >> 5) + b) << 5) | (pc & 31)
+                e[4 * h + i] = flip ? ent : sentinel;
+                n += flip ? 1 : 0;
+            }
+        }
+        if (rowlive) {
+            if (!(pos >= C && n == n_before)) {   // a last piece without a flip is not part of the list
+                if (piece < a.cap)
+                    dst[(int64_t)piece * 64] = make_uint4(e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16),
+                                                          e[6] | (e[7] << 16));
+                piece++;
+            }
+            if (pos >= C) {
+                const bool over = piece > a.cap;
+                a.info[q] = over ? flip_info((uint32_t)(8 * a.cap), (uint32_t)a.cap) : flip_info((uint32_t)n, (uint32_t)piece);
+                if (over) atomicAdd(a.overflow, 1u);
+                rowlive = false;
+            }
+        }
+        pos = rowlive ? pos : C;                  // a finished lane draws on, and nothing comes of it
+        const unsigned long long busy = __ballot(rowlive);
+        if (live && ((busy >> gshift) & gmask) == 0ull) {
+            d += slots;
+            start_row();
+            rowlive = live;
+        }
     }
 }
 
@@ -388,7 +501,7 @@ __global__ __launch_bounds__(1024) void fl_skip_table_kernel(uint32_t *table, co
     skip_table_build(table, thr);
 }
 
-static int gen_launch(GenArgs a, bool thin, hipStream_t s, const char *who)
+static int gen_launch(GenArgs a, bool thin, bool force_walk, hipStream_t s, const char *who)
 {
     const bool aligned = a.C % 4 == 0 && a.key.first % 4 == 0;
     // rows per workgroup: eight (a 128-byte line of every piece) where LDS holds them
@@ -398,6 +511,7 @@ static int gen_launch(GenArgs a, bool thin, hipStream_t s, const char *who)
     while (shift > 0 && tab_bytes + (row_bytes << shift) > 150 * 1024) shift--;
     NB_REQUIRE(tab_bytes + (row_bytes << shift) <= 150 * 1024, "%s: a row of %d columns does not fit LDS", who, a.C);
     a.rb_shift = shift;
+    a.group = getenv("NESBIN_FLIP_GROUP") ? atoi(getenv("NESBIN_FLIP_GROUP")) : 8;
     const size_t lds = tab_bytes + (row_bytes << shift);
     // large workgroups when the rows fill LDS (one workgroup per compute unit then), else four waves each
     const int threads = lds > 40 * 1024 ? 1024 : 256;
@@ -411,10 +525,11 @@ static int gen_launch(GenArgs a, bool thin, hipStream_t s, const char *who)
     static std::once_flag once;
     static hipError_t attr = hipSuccess;
     std::call_once(once, [] {
-        const void *fns[4] = {reinterpret_cast<const void *>(fl_gen_kernel<false, false>),
+        const void *fns[5] = {reinterpret_cast<const void *>(fl_gen_kernel<false, false>),
                               reinterpret_cast<const void *>(fl_gen_kernel<false, true>),
                               reinterpret_cast<const void *>(fl_gen_kernel<true, false>),
-                              reinterpret_cast<const void *>(fl_gen_kernel<true, true>)};
+                              reinterpret_cast<const void *>(fl_gen_kernel<true, true>),
+                              reinterpret_cast<const void *>(fl_gen_static_kernel)};
         for (const void *f : fns) {
             const hipError_t e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
             if (e != hipSuccess) attr = e;
@@ -426,6 +541,7 @@ static int gen_launch(GenArgs a, bool thin, hipStream_t s, const char *who)
     }
     const dim3 grid((unsigned)(nrg * nmc)), block((unsigned)threads);
     if (aligned && thin) fl_gen_kernel<true, true><<<grid, block, lds, s>>>(a);
+    else if (aligned && !force_walk) fl_gen_static_kernel<<<grid, block, lds, s>>>(a);
     else if (aligned) fl_gen_kernel<true, false><<<grid, block, lds, s>>>(a);
     else if (thin) fl_gen_kernel<false, true><<<grid, block, lds, s>>>(a);
     else fl_gen_kernel<false, false><<<grid, block, lds, s>>>(a);
@@ -493,7 +609,7 @@ int nb_flip_skip_i64(uint32_t *entries, uint32_t *info, uint32_t *overflow, cons
     a.Kw = (int)((C + 63) / 64);
     a.S = (int)((R + 63) / 64);
     a.cap = (int)cap;
-    return nb::gen_launch(a, false, nb::as_stream(stream), who);
+    return nb::gen_launch(a, false, getenv("NESBIN_FLIP_WALK") != nullptr, nb::as_stream(stream), who);
 }
 
 int nb_flip_skip_thin_i64(uint32_t *entries, uint32_t *info, uint32_t *overflow, const uint16_t *law,
@@ -517,7 +633,7 @@ int nb_flip_skip_thin_i64(uint32_t *entries, uint32_t *info, uint32_t *overflow,
     a.Kw = (int)((C + 63) / 64);
     a.S = (int)((R + 63) / 64);
     a.cap = (int)cap;
-    return nb::gen_launch(a, true, nb::as_stream(stream), who);
+    return nb::gen_launch(a, true, false, nb::as_stream(stream), who);
 }
 
 int64_t nb_law_workspace_bytes(void) { return nb::kLawBlocks * 8; }
