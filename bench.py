@@ -27,15 +27,25 @@ if ROOT not in sys.path:
 
 def measured_traffic():
     """HBM bytes per launch of the headline kernel from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE in KiB per
-    dispatch, each scaled by what the same counter reads for the 2 GiB calibration copy kernel).  The counter
-    readings live in profiles/headline_traffic.json, next to the summary that quotes them; None if that file is gone."""
+    dispatch, each scaled by what the same counter reads for the 2 GiB calibration copy kernel).  Counters cannot be
+    read from inside this program; the readings live in profiles/headline_traffic.json, next to the summary that
+    quotes them, together with the commit they were taken at and the hash of the kernel's source file then.
+    -> (bytes or None, note): None when the file is gone or the kernel's source has changed since (a stale figure
+    is not reported)."""
+    import hashlib
     try:
         with open(os.path.join(ROOT, "profiles", "headline_traffic.json")) as f:
             t = json.load(f)
+        with open(os.path.join(ROOT, t["kernel_source"]), "rb") as f:
+            same = hashlib.sha256(f.read()).hexdigest() == t["kernel_source_sha256"]
+        note = "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE at commit %s; %s unchanged since: %s" % (
+            t["measured_at_commit"], t["kernel_source"], same)
+        if not same:
+            return None, note
         return int(round((t["fetch_kib_per_dispatch"] * t["fetch_scale"]
-                          + t["write_kib_per_dispatch"] * t["write_scale"]) * 1024))
+                          + t["write_kib_per_dispatch"] * t["write_scale"]) * 1024)), note
     except (OSError, KeyError, ValueError):
-        return None
+        return None, "profiles/headline_traffic.json not readable"
 
 
 def parse_args():
@@ -141,6 +151,13 @@ def config_entry(cfg, w, per_wall, per_ev, per_graph=None):
     if w.bound == "hbm":
         entry.update(bound="hbm", roofline_frac=round(hbm, 4))
         return entry
+    if "stages" in w.meta:
+        # a network has no single roofline: one line per kernel instead (kernel_table), and the whole step against the
+        # two compute limits
+        entry.update(conv_engine="matrixcore-fp4 / window kernel",
+                     frac_of_valu_popcount_peak=round(w.bit_macs / per_ev / workloads.VALU_POPC_PEAK, 4),
+                     frac_of_fp4_mfma_peak=round(w.bit_macs / per_ev / workloads.MFMA_FP4_PEAK, 4))
+        return entry
     valu = w.bit_macs / per_ev / workloads.VALU_POPC_PEAK
     mfma = w.bit_macs / per_ev / workloads.MFMA_INT8_PEAK
     fp4 = w.bit_macs / per_ev / workloads.MFMA_FP4_PEAK
@@ -152,6 +169,56 @@ def config_entry(cfg, w, per_wall, per_ev, per_graph=None):
                  frac_of_valu_popcount_peak=round(valu, 4), frac_of_int8_mfma_peak=round(mfma, 4),
                  frac_of_fp4_mfma_peak=round(fp4, 4))
     return entry
+
+
+def extend_entry(torch, args, cfg, w, entry, steps):
+    """What the conv-shaped configurations report beside their step: the same step on the XOR-popcount kernels
+    (engine 1: the engine the vector-ALU roofline is about), configuration 5's launches one by one, and configuration
+    5 built through the layer API."""
+    from nesgpu_amd import workloads
+    from nesgpu_amd.extensions import booleanOperations as ops
+    if cfg in (3, 4, 5):
+        prev = ops.conv_engine(1)
+        try:
+            n = max(3, steps // 4)
+            pw, pe = time_steps(torch, w.step, n, 2)
+            pg = None if args.no_graph else time_graph(torch, w.step, n)
+            t = min(pe, pg) if pg else pe
+            entry["engine_popcount"] = {"ms_per_step": round(t * 1e3, 4),
+                                        "frac_of_valu_popcount_peak": round(w.bit_macs / t / workloads.VALU_POPC_PEAK, 4),
+                                        "timing": "graph replay" if pg and pg <= pe else "eager launches",
+                                        "note": "conv kernels forced to XOR + popcount (nb_conv_engine(1)); other "
+                                                "kernels of the step unchanged"}
+        finally:
+            ops.conv_engine(prev)
+    if "stages" in w.meta:
+        table = []
+        peaks = {"valu": workloads.VALU_POPC_PEAK, "fp4": workloads.MFMA_FP4_PEAK, "hbm": workloads.HBM_PEAK}
+        for name, fn, bound, work in w.meta["stages"]():
+            pw, pe = time_steps(torch, fn, max(3, steps // 2), 3)
+            pg = None if args.no_graph else time_graph(torch, fn, max(3, steps // 2))
+            t = min(pe, pg) if pg else pe
+            table.append({"kernel": name, "us": round(t * 1e6, 2), "bound": bound,
+                          "frac": round(work / t / peaks[bound], 4)})
+        entry["kernel_table"] = table
+        entry["kernel_table_note"] = ("each launch of the step timed alone (graph replay); frac = bit-MACs or "
+                                      "algorithmic bytes per second over the peak its bound names (valu: 6.29e14 "
+                                      "bit-MAC/s, fp4: 5.05e15 MAC/s, hbm: 8e12 B/s)")
+    if cfg == 5:
+        model, step, set_noise = workloads.cifar_net_layers()
+        n = max(3, steps // 2)
+        pw, pe = time_steps(torch, step, n, 3)
+        pg = None if args.no_graph else time_graph(torch, step, n)
+        sw, se = time_steps(torch, set_noise, 5, 2)
+        fc = model.perturbed_layers[3].weight_noise
+        entry["layer_api"] = {
+            "workload": "the same network from BinarizedConv2d / BinarizedMaxPool2d / BinarizedLinear "
+                        "(flip_probability=0.01) through PerturbedModel, fuse_packed_outputs",
+            "ms_per_step": round(pw * 1e3, 4), "ms_per_step_graph": round(pg * 1e3, 4) if pg else None,
+            "set_noise_ms": round(sw * 1e3, 4),
+            "fc_8192_1024": type(fc).__name__,
+            "ratio_to_ops_level": round(pw * 1e3 / entry["ms_per_step"], 3)}
+        del model, step, set_noise
 
 
 def cpu_baseline(wl, members, seconds):
@@ -245,7 +312,7 @@ def calibrate(torch):
     out = torch.empty(blocks * 256, dtype=torch.int32, device="cuda")
     per, ev = time_steps(torch, lambda: lib.nb_calib_popc(out.data_ptr(), s.data_ptr(), blocks, iters, st), 5, 1)
     lane_ops = blocks * 256 * iters * 8 * 16 * 2
-    res["copy_GBps"] = res["read_GBps"] = None   # keeps the keys' order in the printed line
+    res["copy_GBps"] = res["read_GBps"] = res["read_stream_GBps"] = None   # keeps the keys' order in the printed line
     res["xor_bcnt_lane_ops_per_s"] = float("%.4g" % (lane_ops / ev))
     res["xor_bcnt_binary_TOPS"] = round(2 * (lane_ops / 4 * 64) / ev / 1e12, 1)
     # how int8 MFMAs and ordinary vector instructions share a SIMD's issue (four waves per SIMD): ns per MFMA and SIMD
@@ -269,6 +336,12 @@ def calibrate(torch):
     res["copy_GBps"] = round(2 * nbytes / ev / 1e9, 1)
     per, ev = time_steps(torch, lambda: lib.nb_calib_read(sink.data_ptr(), src.data_ptr(), nbytes, st), 10, 2)
     res["read_GBps"] = round(nbytes / ev / 1e9, 1)
+    if hasattr(lib, "nb_calib_read_stream"):
+        # the loads the library's streaming kernels use (non-temporal, eight 16-byte requests per thread before the
+        # first use): what a read-once stream reaches, and the figure to hold the headline kernel against
+        lib.nb_calib_read_stream.argtypes = [vp, vp, i64, vp]
+        per, ev = time_steps(torch, lambda: lib.nb_calib_read_stream(sink.data_ptr(), src.data_ptr(), nbytes, st), 10, 2)
+        res["read_stream_GBps"] = round(nbytes / ev / 1e9, 1)
     if hasattr(lib, "nb_calib_fill"):
         # writes alone: a plain fill, and the store pattern of the conv kernels' int32 maps (configuration 3: 1024
         # members x 256 KB, a wave per 16 pixel columns of a member, 4 KB per row) alternating between two buffers
@@ -288,14 +361,17 @@ def calibrate(torch):
     return res
 
 
-def hbm_kernels(torch, steps, warmup, graph=True):
-    """Each HBM-bound kernel of the path alone, at a configuration-sized shape: algorithmic bytes / event time."""
+def hbm_kernels(torch, steps, warmup, graph=True, core=False):
+    """Each HBM-bound kernel of the path alone, at a configuration-sized shape: algorithmic bytes / event time.
+    ``core``: only pack, unpack, the samplers from supplied words and max-pool (the kernels the 70 % target names)."""
     from nesgpu_amd import workloads
     from nesgpu_amd.extensions import booleanOperations as ops
     dev = "cuda"
     res = []
 
     def run(name, fn, nbytes):
+        if core and not name.startswith(("pack", "unpack", "flip_from_words", "max_pool2d")):
+            return
         pw, pe = time_steps(torch, fn, steps, warmup)
         pg = time_graph(torch, fn, steps) if graph else None   # device time without the host's launch pacing
         t = pg if pg else pe
@@ -321,13 +397,17 @@ def hbm_kernels(torch, steps, warmup, graph=True):
         base = ops.pack(torch.randint(0, 2, (R, C), device=dev, generator=g, dtype=torch.uint8).bool(), torch.int64)
         nb = words.numel() * 4 + n * R * ((C + 63) // 64) * 8
         run("flip_from_words [%d,%d,%d]" % (n, R, C), lambda: ops.flip_from_words(base, words, T), nb)
-        thr = ops.thresholds_from_p(torch.rand(R, C, device=dev, generator=g).half())
-        run("sample_bits_from_words [%d,%d,%d]" % (n, R, C), lambda: ops.sample_bits_from_words(thr, words, torch.int64), nb)
+        if not core:
+            thr = ops.thresholds_from_p(torch.rand(R, C, device=dev, generator=g).half())
+            run("sample_bits_from_words [%d,%d,%d]" % (n, R, C),
+                lambda: ops.sample_bits_from_words(thr, words, torch.int64), nb)
         del words
     # max-pool 2x2/s2 on config 4's thresholded map [1024,64,64,1] and on a 2-word map
     for shape in ((1024, 64, 64, 1), (4096, 16, 16, 2), (1024, 64, 64, 4)):
         x = torch.randint(-2 ** 62, 2 ** 62, shape, device=dev, generator=g, dtype=torch.int64)
         run("max_pool2d %s" % (list(shape),), lambda: ops.max_pool2d(x, 2, 2, 0, 0, 2, 2), x.numel() * 8 * 5 // 4)
+    if core:
+        return res
     x = torch.randint(-2 ** 62, 2 ** 62, (1024, 32, 32, 1), device=dev, generator=g, dtype=torch.int64)
     run("batch_im2col [1024,32,32,1] 3x3 p1", lambda: ops.batch_im2col(x, 3, 3, 1, 1, 1, 1), x.numel() * 8 * 10)
     # linear matrix-vector product streaming materialised weights (config 5's 8192 -> 1024 layer at D=1024)
@@ -410,6 +490,8 @@ def main():
         pw, pe = time_steps(torch, w.step, args.steps, args.warmup)
         entry = config_entry(args.only, w, pw, pe, None if args.no_graph else time_graph(torch, w.step, args.steps))
         entry["event_ms_per_step"] = round(pe * 1e3, 4)
+        if not args.no_graph:
+            extend_entry(torch, args, args.only, w, entry, args.steps)
         print(json.dumps(entry))
         return 0
 
@@ -421,6 +503,7 @@ def main():
     per_wall, per_ev = time_steps(torch, wl.step, args.steps, args.warmup)
     tops = 2 * wl.bit_macs / per_wall / 1e12
     achieved = wl.algo_bytes / per_ev / 1e9
+    traffic, traffic_note = measured_traffic()
     line = {
         "metric": "packed binary TOPS (2 x valid bit-MACs / s) per population forward",
         "value": round(tops, 4), "unit": "binary TOPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -430,7 +513,8 @@ def main():
         "config": {"workload": wl.name, "population": wl.population, "word_bits": 64,
                    "bit_macs_per_step": wl.bit_macs},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": workloads.HBM_PEAK / 1e9, "unit": "GB/s",
-                     "frac": round(achieved * 1e9 / workloads.HBM_PEAK, 4), "traffic": measured_traffic(),
+                     "frac": round(achieved * 1e9 / workloads.HBM_PEAK, 4), "traffic": traffic,
+                     "traffic_source": traffic_note,
                      "kernel": "seeded_bmv_stream_kernel", "algorithmic_bytes_per_launch": wl.algo_bytes,
                      "avg_launch_ms": round(per_ev * 1e3, 4)},
     }
@@ -450,6 +534,7 @@ def main():
         steps = max(3, args.steps // 2) if cfg == 5 else args.steps
         pw, pe = time_steps(torch, w.step, steps, args.warmup)
         entry = config_entry(cfg, w, pw, pe, None if args.no_graph else time_graph(torch, w.step, steps))
+        extend_entry(torch, args, cfg, w, entry, steps)
         others.append(entry)
         del w
         torch.cuda.empty_cache()
@@ -478,6 +563,9 @@ def main():
             if fg:
                 line["nes_step_smallnet"]["forward_graph_ms"] = round(fg * 1e3, 4)
         del sn, fw, up
+    # the helper kernels the 70 %-of-HBM target names, each alone, after everything above has warmed the clocks
+    line["hbm_kernels"] = [{"kernel": k["kernel"], "us": k["us"], "hbm_frac": k["hbm_frac"], "timing": k["timing"]}
+                           for k in hbm_kernels(torch, max(10, args.steps // 4), 5, not args.no_graph, core=True)]
     if others:
         line["other_configs"] = others
     if cal:

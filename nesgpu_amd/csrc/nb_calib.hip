@@ -54,6 +54,26 @@ __global__ __launch_bounds__(256) void calib_read_kernel(uint32_t *__restrict__ 
     if (acc == 0x9E3779B9u) sink[0] = acc;  // practically never; keeps the loads alive
 }
 
+// The same read with the load the streaming kernels of the library use: non-temporal 16-byte loads, all of a
+// thread's UNR requests issued before the first use, 1024-thread workgroups.
+template <int UNR>
+__global__ __launch_bounds__(1024) void calib_read_stream_kernel(uint32_t *__restrict__ sink, const uint4 *__restrict__ src,
+                                                                 int64_t n16)
+{
+    const int64_t base = ((int64_t)blockIdx.x * 1024 * UNR) + threadIdx.x;
+    uint4 v[UNR];
+#pragma unroll
+    for (int u = 0; u < UNR; u++) {
+        const int64_t i = base + (int64_t)u * 1024;
+        v[u] = load_stream16(src + (i < n16 ? i : n16 - 1));
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    uint32_t acc = 0;
+#pragma unroll
+    for (int u = 0; u < UNR; u++) acc ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+    if (acc == 0x9E3779B9u) sink[0] = acc;
+}
+
 // iters x 16 independent (v_xor_b32 with an SGPR operand, accumulating v_bcnt_u32_b32) pairs per lane.
 __global__ __launch_bounds__(256) void calib_popc_kernel(int32_t *__restrict__ out, const uint32_t *__restrict__ s,
                                                          int iters)
@@ -152,6 +172,15 @@ int nb_calib_read(void *sink, const void *src, int64_t bytes, nb_stream_t s)
     nb::calib_read_kernel<UNR><<<dim3((unsigned)blocks), dim3(256), 0, nb::as_stream(s)>>>(
         static_cast<uint32_t *>(sink), static_cast<const uint4 *>(src), n16);
     return nb::check_launch("nb_calib_read");
+}
+int nb_calib_read_stream(void *sink, const void *src, int64_t bytes, nb_stream_t s)
+{
+    const int64_t n16 = bytes / 16;
+    constexpr int UNR = 8;
+    const int64_t blocks = nb::ceil_div(n16, 1024 * UNR);
+    nb::calib_read_stream_kernel<UNR><<<dim3((unsigned)blocks), dim3(1024), 0, nb::as_stream(s)>>>(
+        static_cast<uint32_t *>(sink), static_cast<const uint4 *>(src), n16);
+    return nb::check_launch("nb_calib_read_stream");
 }
 // lane-ops executed = blocks*256 * iters * 8*16 * 2 (one xor + one bcnt per pair)
 int nb_calib_popc(void *out, const void *s1024, int blocks, int iters, nb_stream_t s)

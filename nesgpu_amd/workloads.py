@@ -222,6 +222,44 @@ def cifar_net(D=4096, T=T_P01, seed=0, dtype=torch.int64, device="cuda", classes
         a = ops.bmv_flip_act_pack(state["rows4"], features(), thr4).view(D, -1, 1)   # the same bits from the lists
         return ops.bmm(state["W5"], a).squeeze(2)
 
+    def stages():
+        """The step's launches one by one, for timing each alone: (name, callable, bound, bit-MACs or bytes).
+        bound: "valu" (XOR-popcount issue), "fp4" (FP4 matrix cores) or "hbm"."""
+        acts = [x]
+        for i, pool in enumerate((False, True, True)):
+            _, thr, f, kw = state["layers"][i]
+            acts.append(ops.conv_act_pack(acts[-1], f, thr, 3, 3, 1, 1, 1, 1, pool=pool, **kw))
+        feats = acts[3].view(D, -1)
+        out = []
+        for i, pool in enumerate((False, True, True)):
+            C, O, S = shapes[i]
+            _, thr, f, kw = state["layers"][i]
+            a_in = acts[i]
+            out.append(("conv %d->%d on %dx%d%s" % (C, O, S, S, ", pooled" if pool else ""),
+                        (lambda a_in=a_in, f=f, thr=thr, pool=pool, kw=kw:
+                         ops.conv_act_pack(a_in, f, thr, 3, 3, 1, 1, 1, 1, pool=pool, **kw)),
+                        "valu" if C == 3 else "fp4", D * S * S * O * 9 * C))
+        if sparse:
+            rows = state["rows4"]
+            ex = ops.expand_rows(feats)
+            G = ops.bmm_nt(ex, rows.base_expanded)
+            out.append(("input bits -> FP4 codes", lambda: ops.expand_rows(feats), "hbm",
+                        feats.numel() * 8 + ex.codes.numel()))
+            out.append(("shared product 4096 x 1024 x 8192", lambda: ops.bmm_nt(ex, rows.base_expanded), "fp4",
+                        D * 1024 * 8192))
+            out.append(("corrections from the flip lists, threshold, pack",
+                        lambda: ops.bmv_flip_act_pack(rows, feats, thr4, G=G), "hbm",
+                        rows.nbytes() + G.numel() * 4 + thr4.numel() * 4 + feats.numel() * 8))
+        else:
+            W = W4()
+            out.append(("linear 8192->1024 on materialised weights", lambda: ops.bmv_act_pack(W, feats, thr4), "hbm",
+                        W.numel() * 8))
+        a5 = ops.bmv_act_pack(W4(), feats, thr4).view(D, -1, 1) if not sparse else \
+            ops.bmv_flip_act_pack(state["rows4"], feats, thr4).view(D, -1, 1)
+        out.append(("linear 1024->%d" % classes, lambda: ops.bmm(state["W5"], a5), "hbm",
+                    state["W5"].numel() * 8 + D * classes * 4))
+        return out
+
     w = Workload(
         name="CIFAR-shaped binary net D=%d (conv3-64, conv64-64, pool, conv64-128, pool, fc8192-1024, fc1024-%d)"
              % (D, classes),
@@ -231,9 +269,49 @@ def cifar_net(D=4096, T=T_P01, seed=0, dtype=torch.int64, device="cuda", classes
         tensors=dict(x=x, f1=state["layers"][0][0], f2=state["layers"][1][0], f3=state["layers"][2][0],
                      W5=state["W5"], b1=conv_bases[0], b2=conv_bases[1], b3=conv_bases[2], b4=b4, b5=b5),
         meta=dict(T=T, seed=seed, first_subsequence=10, step_dense=step_dense, features=features,
-                  rows4=state["rows4"], W4=W4, thr4=thr4, resample=resample,
+                  rows4=state["rows4"], W4=W4, thr4=thr4, resample=resample, stages=stages,
                   fc="base + flip lists (skip sampler)" if sparse else "materialised weights"))
     return w
+
+
+def cifar_net_layers(D=4096, p=0.01, seed=0, device="cuda", classes=10):
+    """Config 5 through the layer API: the same network as :func:`cifar_net` built from BinarizedConv2d /
+    BinarizedMaxPool2d / BinarizedLinear with ``flip_probability=p`` (weights = sign of the latent weight XOR a
+    Bernoulli(p) flip mask), wrapped in a PerturbedModel; packed and pooled outputs between the layers
+    (``fuse_packed_outputs``); the wide layer picks the base + flip list form itself.  Thresholds are the layers' own
+    ``bias + bias_noise`` (zero bias, noise in [-3, 3)) instead of the fixed 0 of the ops-level workload: the same
+    kernels and the same work.  Returns (model, step, set_noise): ``step()`` is one population forward giving int32
+    logits ``2 * popc - 1024``."""
+    from .modules import binary
+    from .modules.base import PerturbedModel
+    kw = dict(batch_norm=False, padding=1, device=device, flip_probability=p)
+    net = torch.nn.Sequential(
+        binary.BinarizedConv2d(3, 64, D, 3, **kw), binary.BinarizedConv2d(64, 64, D, 3, **kw),
+        binary.BinarizedMaxPool2d(), binary.BinarizedConv2d(64, 128, D, 3, **kw), binary.BinarizedMaxPool2d(),
+        torch.nn.Flatten(), binary.BinarizedLinear(8192, 1024, D, device=device, flip_probability=p),
+        binary.BinarizedLinear(1024, classes, D, threshold=False, device=device, flip_probability=p))
+    binary.fuse_packed_outputs(net, max_fan_in=None)
+    g = _gen(seed)
+    with torch.no_grad():
+        for m in net.modules():
+            if isinstance(m, binary.Binarized):
+                m.weight.copy_((torch.randint(0, 2, m.weight.shape, generator=g) * 2 - 1).to(torch.float16))
+    model = PerturbedModel(net, D)
+    for i, m in enumerate(model.perturbed_layers):
+        m.set_seed(seed + 100 + i)
+    z = torch.randn((D, 3, 32, 32), generator=g)
+    x_bits = (z > z.mean(dim=(0, 2, 3), keepdim=True)).permute(0, 2, 3, 1).contiguous()
+    x = ops.pack(x_bits.view(-1, 3).to(device), torch.int64).view(D, 32, 32, 1)
+
+    def set_noise():
+        model.set_noise()
+
+    def step():
+        with torch.no_grad():
+            return model.forward(x)
+
+    set_noise()
+    return model, step, set_noise
 
 
 def small_net_step(D=1024, classes=10, in_channels=24, seed=0, device="cuda", fuse=True):
