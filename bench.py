@@ -562,6 +562,26 @@ def main():
             fg = time_graph(torch, fw, reps)                 # the same forward without the host's launch pacing
             if fg:
                 line["nes_step_smallnet"]["forward_graph_ms"] = round(fg * 1e3, 4)
+            # the same step with the forward replayed from a HIP graph (binary.capture): new noise is drawn eagerly and
+            # copied to where the graph reads it
+            from nesgpu_amd.modules import binary
+            cap = binary.capture(fw.model, fw.input)
+            line["nes_step_smallnet"]["captured"] = {
+                "set_noise_ms": round(time_steps(torch, cap.set_noise, reps, 2)[0] * 1e3, 4),
+                "forward_ms": round(time_steps(torch, cap, reps, 2)[0] * 1e3, 4),
+                "update_ms": round(time_steps(torch, up, reps, 2)[0] * 1e3, 4),
+                "note": "binary.capture: one graph replay per forward; set_noise draws eagerly and copies into the "
+                        "graph's tensors"}
+            pm1, x1 = workloads.linear_layer_config1()
+            eager1 = time_steps(torch, lambda: pm1.forward(x1), args.steps, 5)
+            cap1 = binary.capture(pm1, x1)
+            rep1 = time_steps(torch, cap1, args.steps, 5)
+            line["config1_layer"] = {
+                "workload": "configuration 1 as BinarizedLinear(256, 256, 1024, threshold=False) through "
+                            "PerturbedModel: bmm + 2*popc - K",
+                "eager_us_per_step": round(eager1[0] * 1e6, 2), "captured_us_per_step": round(rep1[0] * 1e6, 2),
+                "note": "captured: one graph replay per step, launched from Python"}
+            del cap, cap1, pm1
         del sn, fw, up
     # the helper kernels the 70 %-of-HBM target names, each alone, after everything above has warmed the clocks
     line["hbm_kernels"] = [{"kernel": k["kernel"], "us": k["us"], "hbm_frac": k["hbm_frac"], "timing": k["timing"]}

@@ -445,3 +445,94 @@ def fuse_packed_outputs(model, max_fan_in=2048):
             layer.pack_output = True
             changed += 1
     return changed
+
+
+def _noise_state(layer):
+    """The tensors a layer's forward reads besides its input and its parameters, in a fixed order:
+    [(name, tensor), ...].  A flip-list layer contributes its lists, their info words and the shared base."""
+    out = []
+    wn = layer.weight_noise
+    if isinstance(wn, booleanOperations.FlipRows):
+        out += [("entries", wn.entries), ("info", wn.info), ("overflow", wn.overflow), ("base", wn.base),
+                ("base_codes", wn.base_expanded.codes)]
+    elif wn is not None:
+        out.append(("weight_noise", wn))
+    for name in ("weight_noise_reshaped", "weight_noise_tap", "bias_noise"):
+        t = getattr(layer, name, None)
+        if t is not None:
+            out.append((name, t))
+    hit = layer._cache.get("thresh")
+    if hit is not None:
+        out.append(("thresh", hit[1]))
+    return out
+
+
+class CapturedForward:
+    """A population forward recorded once as a HIP graph and replayed (not in the reference): a step of a small
+    network is a handful of kernels of a few microseconds each, which eager launches from Python cannot keep fed.
+
+    ``capture(model, example_input)`` runs the forward of ``model`` (an ``nn.Module`` of binary layers or a
+    :class:`PerturbedModel`; ``set_noise`` must have been called) under graph capture.  The graph reads the layers'
+    noise tensors at the addresses they had then, so new noise has to arrive there: :meth:`set_noise` draws it with
+    the layers' own ``set_noise`` and copies it into those tensors (and makes them the layers' noise again), and
+    brings the integer thresholds that depend on ``bias`` up to date.  Shapes must not change between draws (a
+    flip-list layer keeps its capacity as long as its latent weights give the same one; otherwise capture again).
+    ``forward(input)`` copies ``input`` into the graph's input tensor, replays, and returns the graph's output tensor
+    (overwritten by the next replay)."""
+
+    def __init__(self, model, example_input, warmup=2):
+        self.model = model if isinstance(model, PerturbedModel) else PerturbedModel(model, None)
+        self.layers = [m for m in self.model.perturbed_layers if isinstance(m, Binarized)]
+        self.input = example_input.clone()
+        with torch.no_grad():
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                for _ in range(max(1, warmup)):          # also fills the layers' threshold caches
+                    self.model.forward(self.input)
+            torch.cuda.current_stream().wait_stream(side)
+            self._static = [_noise_state(m) for m in self.layers]
+            self._thresh_args = [m._cache["thresh"][0][3:5] if "thresh" in m._cache else None for m in self.layers]
+            self._objects = [(m.weight_noise, getattr(m, "weight_noise_reshaped", None),
+                              getattr(m, "weight_noise_tap", None), m.bias_noise) for m in self.layers]
+            self.graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(self.graph):
+                self.output = self.model.forward(self.input)
+
+    def forward(self, input=None):
+        if input is not None:
+            self.input.copy_(input)
+        self.graph.replay()
+        return self.output
+
+    __call__ = forward
+
+    def set_noise(self, *args, **kwargs):
+        """``set_noise`` of every layer, with the new noise copied to where the graph reads it."""
+        with torch.no_grad():
+            for m, static, targs, objs in zip(self.layers, self._static, self._thresh_args, self._objects):
+                m._cache.pop("thresh", None)
+                m.set_noise(*args, **kwargs)
+                if targs is not None:
+                    m.int_thresholds(*targs)
+                fresh = _noise_state(m)
+                if [(n, tuple(t.shape), t.dtype) for n, t in fresh] != [(n, tuple(t.shape), t.dtype) for n, t in static]:
+                    raise RuntimeError("the layer's noise changed shape since the capture; capture again")
+                for (_, dst), (_, src) in zip(static, fresh):
+                    if dst.data_ptr() != src.data_ptr():
+                        dst.copy_(src)
+                # the graph's tensors are the layer's noise again (eager calls and update() see what the graph sees)
+                m.weight_noise, reshaped, tap, m.bias_noise = objs
+                if reshaped is not None:
+                    m.weight_noise_reshaped = reshaped
+                if tap is not None:
+                    m.weight_noise_tap = tap
+                if targs is not None:
+                    thr = dict(static)["thresh"]
+                    tag = (m.bias._version, m.bias.data_ptr(), m.bias_noise._version) + tuple(targs)
+                    m._cache["thresh"] = (tag, thr, m.bias_noise)
+
+
+def capture(model, example_input, warmup=2):
+    """See :class:`CapturedForward`."""
+    return CapturedForward(model, example_input, warmup)

@@ -357,7 +357,24 @@ def small_net_step(D=1024, classes=10, in_channels=24, seed=0, device="cuda", fu
             m.update(fitness)
 
     set_noise()
+    forward.model, forward.input = net, bits          # for callers that capture the forward (binary.capture)
     return set_noise, forward, update
+
+
+def linear_layer_config1(D=1024, device="cuda", seed=0):
+    """Config 1 as a layer: BinarizedLinear(256, 256) without threshold, weights = sign XOR Bernoulli(0.01) flips,
+    one packed input row per member; returns (layer wrapped in a PerturbedModel, packed input)."""
+    from .modules import binary
+    from .modules.base import PerturbedModel
+    lin = binary.BinarizedLinear(256, 256, D, threshold=False, device=device, flip_probability=0.01)
+    g = _gen(seed)
+    with torch.no_grad():
+        lin.weight.copy_((torch.randint(0, 2, lin.weight.shape, generator=g) * 2 - 1).to(torch.float16))
+    x = ops.pack(_bits(g, (D, 256)).to(device), torch.int64)
+    pm = PerturbedModel(torch.nn.Sequential(lin), D)
+    pm.set_seed(seed + 1)
+    pm.set_noise()
+    return pm, x
 
 
 BUILDERS = {1: linear_flip_materialised, 2: linear_flip_fused, 3: conv_int32, 4: conv_sign_pool, 5: cifar_net}

@@ -224,3 +224,58 @@ def test_fuse_packed_outputs_changes_nothing_but_the_kernels(binary):
     assert not small[4].pack_output                                            # 16384 inputs per output: left alone
     assert n == 2
     assert torch.equal(run(small), want)
+
+
+@pytest.mark.parametrize("kind", ["smallnet", "plain"])
+def test_captured_forward_follows_the_eager_one(binary, kind):
+    """binary.capture: the forward replayed from a HIP graph gives what the eager forward gives, for new inputs, for
+    new noise drawn through the helper (several draws: replays after the first must see the new values, with eager
+    work and synchronisations in between), and after the parameters have moved (thresholds that depend on the bias)."""
+    D = 16
+    g = torch.Generator(device="cuda")
+    g.manual_seed(9)
+    if kind == "smallnet":
+        model = small_net(binary, D, 10)
+        binary.fuse_packed_outputs(model)
+        x = torch.randint(0, 2, (D, 32, 32, 24), device="cuda", generator=g).bool()
+    else:
+        # thresholds from bias + bias_noise (no batch norm), a flip-list layer, an int32 output
+        model = torch.nn.Sequential(
+            binary.BinarizedConv2d(16, 64, D, 3, padding=1, batch_norm=False, flip_probability=0.02),
+            binary.BinarizedMaxPool2d(), torch.nn.Flatten(),
+            binary.BinarizedLinear(64 * 8 * 8, 64, D, flip_probability=0.01, sparse=True),
+            binary.BinarizedLinear(64, 10, D, threshold=False))
+        binary.fuse_packed_outputs(model, max_fan_in=None)
+        x = torch.randint(0, 2, (D, 16, 16, 16), device="cuda", generator=g).bool()
+    randomise(model, 3)
+    pm = binary.PerturbedModel(model, D)
+    pm.set_seed(11)
+    pm.set_noise()
+    cap = binary.capture(pm, x)
+    with torch.no_grad():
+        assert torch.equal(cap(), pm.forward(x))
+        for it in range(3):
+            x2 = torch.randint(0, 2, tuple(x.shape), device="cuda", generator=g).bool()
+            pm.set_seed(100 + it)
+            if it == 2:
+                for p in model.parameters():                       # an optimiser step between two draws
+                    p.add_(torch.randn(p.shape, device="cuda", generator=g).to(p.dtype))
+            cap.set_noise()
+            got = cap(x2).clone()
+            torch.cuda.synchronize()
+            want = pm.forward(x2)                                    # eager, on the same (static) noise tensors
+            assert torch.equal(got, want), it
+            assert torch.equal(cap(x2), want)
+            # the noise the graph used is the noise a fresh eager draw with the same seeds gives
+            ref_model = pm.model
+            before = [l.weight_noise for l in pm.perturbed_layers]
+            gen_state = torch.cuda.get_rng_state()
+            pm.set_noise()
+            torch.cuda.set_rng_state(gen_state)
+            for l, b in zip(pm.perturbed_layers, before):
+                if isinstance(b, torch.Tensor):
+                    assert torch.equal(l.weight_noise, b)
+                else:
+                    assert torch.equal(l.weight_noise.entries[:8], b.entries[:8]) and torch.equal(l.weight_noise.info, b.info)
+            cap.set_noise()                                         # back onto the graph's tensors
+            assert ref_model is pm.model
