@@ -286,9 +286,9 @@ int conv_impl(void *out, const W *in, const W *filt, const int32_t *thresh, int6
     }
     // Narrow layers (at most 16 channels in, at most 64 out, threshold bits out): a wave per strip of 16 output columns on
     // the int8 matrix cores, no staged image; any population size.
-    if (bits == 64 && Cw > 0 && engine != 1 &&
+    if (Cw > 0 && engine != 1 &&
         conv_direct_try(out, reinterpret_cast<const uint64_t *>(in), reinterpret_cast<const uint64_t *>(filt), thresh, g,
-                        D, N, tap_bits, mode, s)) {
+                        D, N, tap_bits, mode, s, bits / 8)) {
         t_last_engine = 2;
         return check_launch(who);
     }

@@ -86,7 +86,7 @@ int conv_mfma_try(void *out, const uint64_t *in, const uint64_t *filt, const int
 // Matrix-core conv for narrow layers (nb_conv_direct.hip): tap-packed filters of at most 16 channels, O <= 64, 3-row
 // filters of up to 3 columns, stride 1, mode 2 or 3.  false = not this shape, nothing launched.
 bool conv_direct_try(void *out, const uint64_t *in, const uint64_t *filt, const int32_t *thresh, const ConvGeom &g,
-                     int64_t D, int O, int tap_bits, int mode, hipStream_t s);
+                     int64_t D, int O, int tap_bits, int mode, hipStream_t s, int word_bytes = 8);
 
 // The same scheme for wider pixels (nb_conv_direct_fp4.hip), 3x3 windows, stride 1, O = 16, 32 or a multiple of 16 from
 // 64 on, mode 0, 2, 3 or 4: one full channel word per pixel with filter [D, 9, O] on the FP4 matrix cores (returns 4; only

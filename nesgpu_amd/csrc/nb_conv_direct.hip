@@ -31,6 +31,8 @@ struct DcConv {
     int H, Wd, px, py, h, w, O, fy;
     int in_bits, tapT, tapM, fwords, K;
     int ntx, nsb, hb;       // strips of 16 columns, sub-bands per member, rows per sub-band (even)
+    int wbytes;             // 8: 64-bit words; 4: 32-bit words (pixels 4 bytes apart, 32-bit filter words, and
+                            // 4-byte output words when O <= 32)
     uint32_t units;         // D * nsb * ntx
     uint32_t mntx, mnsb;    // floor(2^32 / ntx), floor(2^32 / nsb): quotients by multiplication
 };
@@ -97,6 +99,7 @@ __global__ __launch_bounds__(256) void conv_direct_kernel(const DcConv p)
     int tdot[NT];
     {
         const uint64_t *fz = p.filt + z * (int64_t)p.fwords;
+        const uint32_t *fz32 = reinterpret_cast<const uint32_t *>(p.filt) + z * (int64_t)p.fwords;
         const uint32_t vbits = (1u << p.in_bits) - 1u;  // in_bits <= 16
 #pragma unroll
         for (int nt = 0; nt < NT; nt++) {
@@ -114,7 +117,8 @@ __global__ __launch_bounds__(256) void conv_direct_kernel(const DcConv p)
             for (int i = 0; i < 3; i++) {
                 const int tap = i * p.fy + (lg < p.fy ? lg : 0);
                 const int fr = (tap * p.tapM) >> 16, sh = p.in_bits * (tap - fr * p.tapT);  // fr = tap / tapT
-                const uint32_t fbits = (uint32_t)(fz[(int64_t)fr * p.O + ch] >> sh) & vbits;
+                const uint64_t fword = p.wbytes == 8 ? fz[(int64_t)fr * p.O + ch] : (uint64_t)fz32[(int64_t)fr * p.O + ch];
+                const uint32_t fbits = (uint32_t)(fword >> sh) & vbits;
                 e[i] = expand16(fbits);
                 e[i][0] &= (int)pmask[0];
                 e[i][1] &= (int)pmask[1];
@@ -135,14 +139,15 @@ __global__ __launch_bounds__(256) void conv_direct_kernel(const DcConv p)
     const int hout = MODE == 3 ? (p.h & ~1) : p.h;  // pooled maps drop an odd last row
     const int ye = ys + p.hb < hout ? ys + p.hb : hout;
     if (ys >= ye) return;
-    const int rowb = p.Wd * 8;
+    const int rowb = p.Wd * p.wbytes;
     const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint64_t *>(p.in + z * (int64_t)p.H * p.Wd), (short)0, p.H * rowb, 0x00020000);
+        const_cast<char *>(reinterpret_cast<const char *>(p.in) + z * (int64_t)p.H * rowb), (short)0, p.H * rowb,
+        0x00020000);
     // A column outside the image (or the idle fourth lane group) gets an offset that is out of range whatever row
     // offset (below 2^30 either way) is added; a row outside gives a negative or too large offset by itself.
     constexpr uint32_t kOutside = 0xC0000000u;
     const int xc = x0 + li + lg - p.py;
-    const uint32_t coloff = (lg < p.fy && xc >= 0 && xc < p.Wd) ? (uint32_t)xc * 8u : kOutside;
+    const uint32_t coloff = (lg < p.fy && xc >= 0 && xc < p.Wd) ? (uint32_t)(xc * p.wbytes) : kOutside;
     auto load_row = [&](int rr) {  // band row rr is image row rr - px
         return (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)(coloff + (uint32_t)((rr - p.px) * rowb)), 0, 0);
     };
@@ -156,9 +161,11 @@ __global__ __launch_bounds__(256) void conv_direct_kernel(const DcConv p)
     // with the other lanes' operands and results masked off and gives wrong sums, so the walk has no divergent
     // branch at all.
     const bool olive = lane < (MODE == 3 ? 8 : 16) && xx0 + lane < ww;
-    const __amdgpu_buffer_rsrc_t orsrc =
-        __builtin_amdgcn_make_buffer_rsrc(p.out + z * hh * (int64_t)ww, (short)0, hh * ww * 8, 0x00020000);
-    const uint32_t ooff = olive ? (uint32_t)((xx0 + lane) * 8) : 0xC0000000u;  // one word per pixel (O <= 64)
+    // one 64-bit word per pixel (O <= 64), or, with 32-bit words and O <= 32, one 32-bit word
+    const int obytes = (p.wbytes == 4 && p.O <= 32) ? 4 : 8;
+    const __amdgpu_buffer_rsrc_t orsrc = __builtin_amdgcn_make_buffer_rsrc(
+        reinterpret_cast<char *>(p.out) + z * hh * (int64_t)ww * obytes, (short)0, hh * ww * obytes, 0x00020000);
+    const uint32_t ooff = olive ? (uint32_t)((xx0 + lane) * obytes) : 0xC0000000u;
     int pend[NT][2];  // MODE 3: x-pooled minima of the even row of a pair
 #pragma unroll
     for (int nt = 0; nt < NT; nt++) pend[nt][0] = pend[nt][1] = 0;
@@ -247,8 +254,12 @@ __global__ __launch_bounds__(256) void conv_direct_kernel(const DcConv p)
                     if (NT > 2) NB_DC_WRITELANE(whi, fields(m[2][q], m[3][q], g, NT > 3), 2 * g + q);
                 }
         }
-        __builtin_amdgcn_raw_buffer_store_b64((dc_v2i){wlo, whi}, orsrc,
-                                              (int)(ooff + (uint32_t)((MODE == 3 ? y >> 1 : y) * ww * 8)), 0, 2);
+        if (obytes == 8)   // uniform
+            __builtin_amdgcn_raw_buffer_store_b64((dc_v2i){wlo, whi}, orsrc,
+                                                  (int)(ooff + (uint32_t)((MODE == 3 ? y >> 1 : y) * ww * 8)), 0, 2);
+        else
+            __builtin_amdgcn_raw_buffer_store_b32(wlo, orsrc, (int)(ooff + (uint32_t)((MODE == 3 ? y >> 1 : y) * ww * 4)),
+                                                  0, 2);
     };
 
     // ---- walk down the strip: band row rr feeds output rows rr (filter row 0), rr-1 (1) and rr-2 (2) ---------------
@@ -343,7 +354,7 @@ __global__ __launch_bounds__(256) void conv_direct_kernel(const DcConv p)
 // mode 2 (packed threshold bits) or 3 (2x2 OR-pooled) on a tap-packed filter.  false = not this shape, nothing
 // launched.
 bool conv_direct_try(void *out, const uint64_t *in, const uint64_t *filt, const int32_t *thresh, const ConvGeom &g,
-                     int64_t D, int O, int tap_bits, int mode, hipStream_t s)
+                     int64_t D, int O, int tap_bits, int mode, hipStream_t s, int word_bytes)
 {
     if (mode != 2 && mode != 3) return false;
     if (tap_bits < 1 || tap_bits > 16 || g.Cw != 1) return false;
@@ -361,7 +372,8 @@ bool conv_direct_try(void *out, const uint64_t *in, const uint64_t *filt, const 
     p.O = O;
     p.fy = g.fy;
     p.in_bits = tap_bits;
-    p.tapT = 64 / tap_bits;
+    p.wbytes = word_bytes;
+    p.tapT = 8 * word_bytes / tap_bits;
     p.tapM = 65536 / p.tapT + 1;  // (tap * tapM) >> 16 = tap / tapT for the nine taps
     p.fwords = (3 * g.fy + p.tapT - 1) / p.tapT * O;
     p.K = 3 * g.fy * tap_bits;

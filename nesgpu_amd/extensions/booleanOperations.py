@@ -269,7 +269,7 @@ def conv_bn_thresholds_from_input(input, filter, bias, bias_noise, filterx, filt
     """``conv_bn_thresholds(conv_popc_sums(input, filter, ...), bias, bias_noise, channels * taps, h * w)`` in one call
     (one kernel where the pixel sums come from bit counts).  ``channels``: the layer's true input channels (default
     ``in_bits``, else every bit of the channel words)."""
-    suf, _, filter, tap = _conv_args(input, filter, filterx, filtery, in_bits, filter_tap_packed)
+    suf, _, input, filter, tap = _conv_args(input, filter, filterx, filtery, in_bits, filter_tap_packed)
     _check(bias, "bias")
     _check(bias_noise, "bias_noise")
     _same_device(input, bias)
@@ -325,8 +325,23 @@ def tap_pack_filter(filter, taps, in_bits):
     return out
 
 
-def _conv_args(input, filter, filterx, filtery, in_bits=None, filter_tap_packed=False):
-    """-> (suffix, bits, filter to pass, tap_bits)"""
+def _pair_words(input, filter, taps):
+    """32-bit words, an even number per pixel: the same bytes as 64-bit words.  The image is viewed as int64
+    [D,H,W,Cw/2]; the filter [D, taps*Cw, O] has the two halves of a 64-bit word O words apart and is re-packed to
+    int64 [D, taps*Cw/2, O] (one copy of the filters).  The kernels for 64-bit words then serve 32-bit tensors:
+    half the instructions on the XOR-popcount path, and the matrix-core engines.  None if the tensors do not allow it."""
+    Cw = input.size(3)
+    if Cw == 0 or Cw % 2 or input.data_ptr() % 8 or filter.size(1) != taps * Cw:
+        return None
+    D, K, O = filter.shape
+    f64 = filter.view(D, K // 2, 2, O).transpose(2, 3).contiguous().view(torch.int64).view(D, K // 2, O)
+    return input.view(torch.int64), f64
+
+
+def _conv_args(input, filter, filterx, filtery, in_bits=None, filter_tap_packed=False, out_words=None):
+    """-> (suffix, bits, input to pass, filter to pass, tap_bits).  ``out_words``: for packed outputs, the words per
+    pixel of the result in the input's word type (32-bit tensors are only handed to the 64-bit kernels when those
+    write the same bytes)."""
     _check(input, "input")
     _check(filter, "filter")
     _same_device(input, filter)
@@ -343,10 +358,14 @@ def _conv_args(input, filter, filterx, filtery, in_bits=None, filter_tap_packed=
         else:
             assert filter.size(1) == taps
             filter = tap_pack_filter(filter, taps, int(in_bits))
-        return suf, bits, filter, int(in_bits)
+        return suf, bits, input, filter, int(in_bits)
     assert not filter_tap_packed, "filter_tap_packed needs in_bits with Cw == 1 and 2*in_bits <= word bits"
     assert filter.size(1) == taps * input.size(3)                # the bmm contraction assert (:111)
-    return suf, bits, filter, 0
+    if bits == 32 and (out_words is None or out_words % 2 == 0):
+        paired = _pair_words(input, filter, taps)
+        if paired is not None:
+            return "_i64", 64, paired[0], paired[1], 0
+    return suf, bits, input, filter, 0
 
 
 def conv(input, filter, filterx, filtery, padx, pady, stridex, stridey, in_bits=None, filter_tap_packed=False):
@@ -356,7 +375,7 @@ def conv(input, filter, filterx, filtery, padx, pady, stridex, stridey, in_bits=
     ``in_bits`` (optional, not in the reference): the true channel count C of the packed input.  When the
     input has one word per pixel and 2*C <= word bits, several filter taps share a word (same sums, less
     work); the filter is re-packed on the fly unless ``filter_tap_packed`` says it already is."""
-    suf, _, filter, tap = _conv_args(input, filter, filterx, filtery, in_bits, filter_tap_packed)
+    suf, _, input, filter, tap = _conv_args(input, filter, filterx, filtery, in_bits, filter_tap_packed)
     h, w = _out_hw(input, filterx, filtery, padx, pady, stridex, stridey)
     out = torch.empty((input.size(0), h, w, filter.size(2)), dtype=torch.int32, device=input.device)
     with _on(input):
@@ -373,7 +392,7 @@ def conv_popc_sums(input, filter, filterx, filtery, padx, pady, stridex, stridey
     modules/binary.py:147-155).  With the automatic engine, 64-bit words, stride 1 and filters of at most 5 x 5 no
     conv runs at all: the sum over the pixels is taken first (counts of the image's bits per tap), then one small dot
     product per output channel; the same integers."""
-    suf, _, filter, tap = _conv_args(input, filter, filterx, filtery, in_bits, filter_tap_packed)
+    suf, _, input, filter, tap = _conv_args(input, filter, filterx, filtery, in_bits, filter_tap_packed)
     out = torch.empty((input.size(0), filter.size(2)), dtype=torch.int32, device=input.device)
     with _on(input):
         _lib.call("nb_conv_popc_sums" + suf, out.data_ptr(), input.data_ptr(), filter.data_ptr(), input.size(0),
@@ -399,7 +418,8 @@ def _bool_map_via_packed(input, filter, filterx, filtery, stridex, stridey, tap)
 def conv_act(input, filter, threshold, filterx, filtery, padx, pady, stridex, stridey, in_bits=None,
              filter_tap_packed=False):
     """bmm_act(batch_im2col(input), filter, threshold).view(D,h,w,O) (extensions/booleanOperations.py:168-172)."""
-    suf, _, filter, tap = _conv_args(input, filter, filterx, filtery, in_bits, filter_tap_packed)
+    given, given_filter = input, filter
+    suf, _, input, filter, tap = _conv_args(input, filter, filterx, filtery, in_bits, filter_tap_packed)
     _check(threshold, "threshold")
     _same_device(input, threshold)
     assert len(threshold.shape) == 2
@@ -410,8 +430,11 @@ def conv_act(input, filter, threshold, filterx, filtery, padx, pady, stridex, st
     if _bool_map_via_packed(input, filter, filterx, filtery, stridex, stridey, tap):
         # the packed-output kernels (matrix cores, window-in-a-register) followed by unpack: same bools, and faster
         # than the XOR-popcount kernel that writes bool bytes itself, although the bits make one more trip
-        packed = conv_act_pack(input, filter, threshold, filterx, filtery, padx, pady, stridex, stridey,
-                               in_bits=tap if tap else None, filter_tap_packed=bool(tap))
+        if input.dtype != given.dtype:          # 32-bit words handed on as 64-bit ones: whole 64-bit output words
+            packed = conv_act_pack(input, filter, threshold, filterx, filtery, padx, pady, stridex, stridey)
+        else:
+            packed = conv_act_pack(given, filter if tap else given_filter, threshold, filterx, filtery, padx, pady,
+                                   stridex, stridey, in_bits=tap if tap else None, filter_tap_packed=bool(tap))
         return unpack(packed.view(-1, packed.size(3))).view(input.size(0), h, w, filter.size(2))
     out = torch.empty((input.size(0), h, w, filter.size(2)), dtype=torch.bool, device=input.device)
     with _on(input):
@@ -682,15 +705,17 @@ def conv_act_pack(input, filter, threshold, filterx, filtery, padx, pady, stride
     """pack(conv_act(...)) along the channel axis -> [D,h,w,ceil(O/bits)]; with ``pool`` followed by the
     2x2/stride-2 OR-pool -> [D,h//2,w//2,ceil(O/bits)].  One kernel; the bool map never reaches memory.
     ``in_bits`` / ``filter_tap_packed`` as in :func:`conv`."""
-    suf, bits, filter, tap = _conv_args(input, filter, filterx, filtery, in_bits, filter_tap_packed)
+    _, word_bits = _suffix(input.dtype)
+    Ow = ceil_div(filter.size(2), word_bits)
+    out_dtype = input.dtype
+    suf, bits, input, filter, tap = _conv_args(input, filter, filterx, filtery, in_bits, filter_tap_packed, out_words=Ow)
     _check(threshold, "threshold")
     _same_device(input, threshold)
     assert tuple(threshold.shape) == (input.size(0), filter.size(2))
     assert threshold.dtype == torch.int32
     h, w = _out_hw(input, filterx, filtery, padx, pady, stridex, stridey)
-    Ow = ceil_div(filter.size(2), bits)
     shape = (input.size(0), h // 2, w // 2, Ow) if pool else (input.size(0), h, w, Ow)
-    out = torch.empty(shape, dtype=input.dtype, device=input.device)
+    out = torch.empty(shape, dtype=out_dtype, device=input.device)
     with _on(input):
         _lib.call("nb_conv_act_pack" + suf, out.data_ptr(), input.data_ptr(), filter.data_ptr(), threshold.data_ptr(),
                   input.size(0), input.size(1), input.size(2), input.size(3), filter.size(2), filterx, filtery, padx,

@@ -562,6 +562,51 @@ MATRIX_CORE_CASES = [
 ]
 
 
+@pytest.mark.parametrize("C,O,H,W,served", [(64, 64, 12, 20, "wide"), (128, 64, 9, 9, "wide"), (16, 16, 20, 18, "narrow"),
+                                            (16, 64, 11, 17, "narrow"), (8, 32, 16, 16, "narrow"), (64, 16, 8, 8, "odd"),
+                                            (96, 64, 8, 8, "odd")])
+def test_conv_matrix_core_engines_take_32_bit_words(ops, oracle, mc_engine, C, O, H, W, served):
+    """int32 tensors (the word type of the reference's own check, booloptests.py:121) on the matrix-core engines:
+    an even number of 32-bit words per pixel is handed on as 64-bit words (filters re-packed), narrow tap-packed layers
+    are read as they are by the wave-per-strip kernel; odd word counts and packed outputs of an odd number of 32-bit
+    words stay on the XOR-popcount kernels.  All against the oracle run on the int32 tensors."""
+    D, k = 3, 3
+    g = rng(C * 100 + O + H)
+    Cw = (C + 31) // 32
+    x = oracle.pack(g.integers(0, 2, size=(D * H * W, C)).astype(bool), np.int32).reshape(D, H, W, Cw)
+    f = np.ascontiguousarray(oracle.pack(g.integers(0, 2, size=(D * O * 9, C)).astype(bool), np.int32)
+                             .reshape(D, O, 3, 3, Cw).transpose(0, 2, 3, 4, 1).reshape(D, -1, O))
+    K = 9 * C
+    thr = (g.integers(0, K + 1, size=(D, O)) - K // 2 + K).astype(np.int32)
+    thr[0, 0], thr[0, 1] = -5, 2 * K + 3
+    geom = (3, 3, 1, 1, 1, 1)
+    xd, fd, td = dev(x), dev(f), dev(thr)
+    kw = dict(in_bits=C) if 2 * C <= 32 else {}
+    want = oracle.conv(x, f, *geom)
+    act = oracle.conv_act(x, f, thr, *geom)
+    packed = oracle.pack(act.reshape(-1, O), np.int32).reshape(D, H, W, -1)
+    prev = ops.conv_engine(mc_engine)
+    try:
+        got = ops.conv(xd, fd, *geom, **kw)
+        assert got.dtype == torch.int32
+        np.testing.assert_array_equal(host(got), want)
+        if served == "wide":
+            assert ops.conv_last_engine() in (2, 4)
+        gotp = ops.conv_act_pack(xd, fd, td, *geom, **kw)
+        assert gotp.dtype == torch.int32 and tuple(gotp.shape) == packed.shape
+        np.testing.assert_array_equal(host(gotp), packed)
+        if served in ("wide", "narrow"):
+            assert ops.conv_last_engine() in (2, 4), ops.conv_last_engine()
+        elif C == 64:
+            assert ops.conv_last_engine() == 1            # one 32-bit output word per pixel: not what the 64-bit kernels write
+        gotq = ops.conv_act_pack(xd, fd, td, *geom, pool=True, **kw)
+        np.testing.assert_array_equal(host(gotq), oracle.max_pool2d(packed, 2, 2, 0, 0, 2, 2))
+        np.testing.assert_array_equal(host(ops.conv_act(xd, fd, td, *geom, **kw)), act)
+        np.testing.assert_array_equal(host(ops.conv_popc_sums(xd, fd, *geom, **kw)), want.sum(axis=(1, 2)))
+    finally:
+        ops.conv_engine(prev)
+
+
 @pytest.mark.parametrize("C,O,k,pad,H,W,tap,covered", MATRIX_CORE_CASES)
 def test_conv_matrix_core_engine_vs_oracle(ops, oracle, mc_engine, C, O, k, pad, H, W, tap, covered):
     """The matrix-core engines on shapes chosen per kernel variant: int32 sums, packed and pooled outputs against the
