@@ -50,6 +50,27 @@ __global__ __launch_bounds__(256) void pack_vec16_kernel(W *__restrict__ out, co
     }
 }
 
+// Rows of exactly 16 bools (one 16-byte chunk per row, one word per row): a workgroup takes 1024 consecutive rows,
+// thread i the rows i, i + 256, i + 512, i + 768: every load instruction of a wave reads 1 KiB in one piece, all four
+// of a thread are in flight before the first is used, and the words leave as runs of 64.
+template <typename W>
+__global__ __launch_bounds__(256) void pack_rows16_kernel(W *__restrict__ out, const uint8_t *__restrict__ in, int64_t rows)
+{
+    const int64_t base = (int64_t)blockIdx.x * 1024 + threadIdx.x;
+    uint4 v[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const int64_t r = base + 256 * j;
+        v[j] = load_stream16(in + (r < rows ? r : rows - 1) * 16);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const int64_t r = base + 256 * j;
+        if (r < rows) __builtin_nontemporal_store((W)bits16_of_bools(v[j]), out + r);
+    }
+}
+
 // One thread per output word, 8-byte loads.  Requires C % 8 == 0 and an 8-byte aligned input, so every 8-byte chunk
 // lies inside one row (rows of 24 or 40 bools: 3 x 8 bit planes of an image, say).
 template <typename W>
@@ -191,7 +212,9 @@ int pack_impl(W *out, const uint8_t *in, int64_t R, int64_t C, nb_stream_t strea
     if (bits == 64 && (C & 63) == 0 && aligned(in, 16)) {
         const unsigned qb = grid_for(ceil_div(total, 64) * 64);  // one wave per 64 words
         pack_quad_kernel<<<dim3(qb), dim3(256), 0, as_stream(stream)>>>(reinterpret_cast<uint64_t *>(out), in, total);
-    } else if ((C & 15) == 0 && aligned(in, 16))
+    } else if (C == 16 && aligned(in, 16) && ceil_div(R, 1024) <= kMaxGridX)
+        pack_rows16_kernel<W><<<dim3((unsigned)ceil_div(R, 1024)), dim3(256), 0, as_stream(stream)>>>(out, in, R);
+    else if ((C & 15) == 0 && aligned(in, 16))
         pack_vec16_kernel<W><<<dim3(blocks), dim3(256), 0, as_stream(stream)>>>(out, in, total, (int)Rw, C);
     else if ((C & 7) == 0 && aligned(in, 8))
         pack_vec8_kernel<W><<<dim3(blocks), dim3(256), 0, as_stream(stream)>>>(out, in, total, (int)Rw, C);
