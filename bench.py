@@ -445,11 +445,16 @@ def hbm_kernels(torch, steps, warmup, graph=True, core=False):
     wts = torch.randn(1024, device=dev, generator=g).half()
     run("weighted_sum [1024,1024,16] -> fp16 [1024,1024]", lambda: ops.weighted_sum(m, wts, 1024),
         m.numel() * 8 + 1024 * 1024 * 2)
+    # the blocked sum the layers' update uses (tables of partial sums over 8 members)
+    run("weighted_sum fast [1024,1024,16] -> fp16 [1024,1024]", lambda: ops.weighted_sum(m, wts, 1024, fast=True),
+        m.numel() * 8 + 1024 * 1024 * 2)
     del m
     # the same for a conv layer's masks (256 filters of 3x3 taps x 64 channels): an output of 147 456 weights, a wave or
     # two per SIMD
     m = torch.randint(-2 ** 62, 2 ** 62, (1024, 2304, 1), device=dev, generator=g, dtype=torch.int64)
     run("weighted_sum [1024,2304,1] -> fp16 [2304,64]", lambda: ops.weighted_sum(m, wts, 64), m.numel() * 8 + 2304 * 64 * 2)
+    run("weighted_sum fast [1024,2304,1] -> fp16 [2304,64]", lambda: ops.weighted_sum(m, wts, 64, fast=True),
+        m.numel() * 8 + 2304 * 64 * 2)
     del m
     # batch-norm conv layer: thresholds straight from the layer's input (pixel sums from counts of the image's bits, no
     # conv; bound by the latency of a workgroup's chain and by vector instructions, the fraction is for comparison)

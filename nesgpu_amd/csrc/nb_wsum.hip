@@ -1,6 +1,9 @@
 // weighted_sum: ret[r,z] = fp16( sum_m float(w[m]) * bit(in[m,r,z/bits], z%bits) ), the reduction over
 // the population that the update step applies to the sampled masks
 // (extensions/src/weighted_sum.cu:28-46).  fp32 accumulation in member order, like the reference.
+#include <stdlib.h>
+
+#include <mutex>
 #include <type_traits>
 
 #include "nb_common.hpp"
@@ -237,6 +240,265 @@ int weighted_sum_impl(uint16_t *ret, const W *in, const uint16_t *w, int64_t n, 
     return check_launch(who);
 }
 
+
+// ---- fast mode: blocked sums through tables of partial sums -----------------------------------------------------
+// The member-order kernels above spend three vector instructions per member and output bit (one bit test, one mask,
+// one add).  Here a lane owns a 32-bit column of the members' words (lanes side by side: every load of a wave is one
+// 256-byte run), takes the members 32 at a time, transposes the 32 x 32 bit block in its registers (word k then
+// holds output bit k of the 32 members), and adds, per output bit and group of 8 members, one entry of a table
+// T[group][byte] = sum of the weights of the members whose bit is set in `byte`: a quarter of an instruction per
+// transposed bit plus 3 instructions and one LDS read per 8 members.  Sums are fp32; their order is by groups of 8,
+// chunks of 64 and the waves that share a column set, not by member: results differ from the member-order kernel by
+// fp32 rounding only (about 1e-7 of the sum of |weights|), far inside the fp16 spacing of any result that is not
+// dominated by cancellation.
+//
+// A workgroup has 16 waves = (16 >> SPLIT) column sets of 64 columns x (1 << SPLIT) member shares; wave (cs, ms)
+// takes the chunks of 64 members ms, ms + shares, ... of its column set and builds the 8 tables of each chunk
+// itself (8 KB of LDS per wave, no workgroup barrier in the loop).  At the end the shares of a column set are
+// added in a fixed order through LDS (so the result does not change from run to run).
+constexpr int kLutRedStride = 33;                                      // floats per lane in the reduction buffer
+constexpr int kLutLdsBytes = 16 * 64 * kLutRedStride * 4;              // >= 16 waves x 8 KB of tables
+
+template <int J>
+__device__ __forceinline__ void transpose_stage(uint32_t (&a)[32])
+{
+    constexpr uint32_t m = J == 4 ? 0x0F0F0F0Fu : J == 2 ? 0x33333333u : 0x55555555u;
+#pragma unroll
+    for (int k = 0; k < 32; k++) {
+        if (k & J) continue;
+        // v_bitop3_b32 with table 0xE4: third operand set ? first : second, bit by bit
+        const uint32_t lo = a[k], hi = a[k + J];
+        a[k] = __builtin_amdgcn_bitop3_b32(lo, hi << J, m, 0xE4);
+        a[k + J] = __builtin_amdgcn_bitop3_b32(lo >> J, hi, m, 0xE4);
+    }
+}
+
+__device__ __forceinline__ void transpose_bits_32x32(uint32_t (&a)[32])
+{
+    // stage j swaps, for every k with bit j clear, the bits of a[k] at positions with bit j set with the bits of
+    // a[k + j] at positions with bit j clear; after the five stages bit p of a[k] is what bit k of a[p] was
+#pragma unroll
+    for (int k = 0; k < 16; k++) {
+        const uint32_t lo = a[k], hi = a[k + 16];
+        a[k] = __builtin_amdgcn_perm(hi, lo, 0x05040100u);       // low halves: lo.b0 lo.b1 hi.b0 hi.b1
+        a[k + 16] = __builtin_amdgcn_perm(hi, lo, 0x07060302u);  // high halves
+    }
+#pragma unroll
+    for (int k0 = 0; k0 < 32; k0 += 16)
+#pragma unroll
+        for (int k = k0; k < k0 + 8; k++) {
+            const uint32_t lo = a[k], hi = a[k + 8];
+            a[k] = __builtin_amdgcn_perm(hi, lo, 0x06020400u);      // lo.b0 hi.b0 lo.b2 hi.b2
+            a[k + 8] = __builtin_amdgcn_perm(hi, lo, 0x07030501u);  // lo.b1 hi.b1 lo.b3 hi.b3
+        }
+    transpose_stage<4>(a);
+    transpose_stage<2>(a);
+    transpose_stage<1>(a);
+}
+
+template <int SPLIT>
+__global__ __launch_bounds__(1024) void weighted_sum_lut_kernel(_Float16 *__restrict__ ret,
+                                                                 const uint32_t *__restrict__ in,
+                                                                 const _Float16 *__restrict__ w, int64_t n, int64_t Q,
+                                                                 int rowdw, int zbits, int whole_rows)
+{
+    extern __shared__ __align__(16) float lds[];
+    constexpr int SHARES = 1 << SPLIT, SETS = 16 >> SPLIT;
+    const int lane = threadIdx.x & 63;
+    const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int ms = wv & (SHARES - 1), cs = wv >> SPLIT;
+    const int64_t q = ((int64_t)blockIdx.x * SETS + cs) * 64 + lane;  // this lane's column of 32-bit words
+    // byte offset of the lane's column (past the end: the last column, never stored): 32 bits, so that a load is a
+    // wave-uniform base plus a lane offset
+    const uint32_t qoff = (uint32_t)(q < Q ? q : Q - 1) * 4u;
+    float *tbl = lds + wv * 2048;
+    const uint16_t *wr = reinterpret_cast<const uint16_t *>(w);
+    float acc[32];
+#pragma unroll
+    for (int k = 0; k < 32; k++) acc[k] = 0.f;
+    const int64_t nchunks = (n + 63) >> 6;
+    for (int64_t c = ms; c < nchunks; c += SHARES) {
+        const int64_t m0 = c * 64;
+        uint32_t a[32];
+        // the block's 32 loads: one buffer per block that ends with the last member, so that members past n read as
+        // zero words (their weights are zero too); per load a wave-uniform offset and the lane's column offset
+        auto fetch = [&](int64_t mb) {
+            const int64_t left = n - mb;
+            const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
+                const_cast<uint32_t *>(in + mb * Q), (short)0, (int)((left < 32 ? left : 32) * Q * 4), 0x00020000);
+#pragma unroll
+            for (int j = 0; j < 32; j++)
+                a[j] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)qoff, (int)(j * (uint32_t)Q * 4u), 2);
+        };
+        fetch(m0);
+        {
+            // lane (g, s): group g of the chunk, the entries whose bits 2..4 are s; bits 0, 1, 5, 6 by doubling
+            const int g = lane >> 3, s = lane & 7;
+            float wj[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const int64_t m = m0 + 8 * g + j;
+                wj[j] = m < n ? (float)__builtin_bit_cast(_Float16, wr[m]) : 0.f;
+            }
+            // 16 entries at a time (bit 7 clear, then set) to keep the registers for the members' words
+            float e[16];
+            e[0] = ((s & 1) ? wj[2] : 0.f) + ((s & 2) ? wj[3] : 0.f) + ((s & 4) ? wj[4] : 0.f);
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const float wk = wj[k < 2 ? k : k + 3];
+#pragma unroll
+                for (int t = 0; t < (1 << k); t++) e[t + (1 << k)] = e[t] + wk;
+            }
+            // register index = (bits 5, 6) << 2 | bits 0..1: the eight lanes of a group write 128 contiguous bytes
+            float4 *dst = reinterpret_cast<float4 *>(tbl + g * 256 + 4 * s);
+#pragma unroll
+            for (int i = 0; i < 4; i++) dst[8 * i] = make_float4(e[4 * i], e[4 * i + 1], e[4 * i + 2], e[4 * i + 3]);
+#pragma unroll
+            for (int t = 0; t < 16; t++) e[t] += wj[7];
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                dst[8 * (i + 4)] = make_float4(e[4 * i], e[4 * i + 1], e[4 * i + 2], e[4 * i + 3]);
+        }
+        // the tables are read by other lanes of this wave only: LDS accesses of a wave are served in order
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        auto block = [&](auto blk) {
+            transpose_bits_32x32(a);
+#pragma unroll
+            for (int k = 0; k < 32; k++) {
+                const float t0 = tbl[(blk * 4 + 0) * 256 + (a[k] & 255u)];
+                const float t1 = tbl[(blk * 4 + 1) * 256 + ((a[k] >> 8) & 255u)];
+                const float t2 = tbl[(blk * 4 + 2) * 256 + ((a[k] >> 16) & 255u)];
+                const float t3 = tbl[(blk * 4 + 3) * 256 + (a[k] >> 24)];
+                acc[k] += (t0 + t1) + (t2 + t3);
+                if ((k & 3) == 3) __builtin_amdgcn_sched_barrier(0);  // 16 lookups in flight, not all 128
+            }
+        };
+        block(std::integral_constant<int, 0>());
+        if (m0 + 32 < n) {
+            fetch(m0 + 32);
+            block(std::integral_constant<int, 1>());
+        }
+        // the next chunk's tables overwrite these: same wave, in order
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+    }
+    if (SPLIT == 0) {
+        if (q >= Q) return;
+        const int64_t r = q / rowdw;
+        const int z0 = (int)(q - r * rowdw) * 32;
+        if (whole_rows) {
+            uint4 *o = reinterpret_cast<uint4 *>(ret + q * 32);
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                uint32_t h[4];
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    h[e] = (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)acc[8 * i + 2 * e]) |
+                           ((uint32_t)__builtin_bit_cast(uint16_t, (_Float16)acc[8 * i + 2 * e + 1]) << 16);
+                o[i] = make_uint4(h[0], h[1], h[2], h[3]);
+            }
+        } else {
+#pragma unroll
+            for (int k = 0; k < 32; k++)
+                if (z0 + k < zbits) ret[r * zbits + z0 + k] = (_Float16)acc[k];
+        }
+        return;
+    }
+    __syncthreads();  // every wave is done with its tables
+#pragma unroll
+    for (int k = 0; k < 32; k++) lds[(wv * 64 + lane) * kLutRedStride + k] = acc[k];
+    __syncthreads();
+    // thread t adds the shares of 32 / SHARES consecutive output bits of one column
+    constexpr int KP = 32 >> SPLIT;
+    const int col = threadIdx.x >> SPLIT, part = threadIdx.x & (SHARES - 1);
+    const int cs2 = col >> 6, l2 = col & 63;
+    const int64_t q2 = ((int64_t)blockIdx.x * SETS + cs2) * 64 + l2;
+    if (q2 >= Q) return;
+    float sum[KP];
+#pragma unroll
+    for (int i = 0; i < KP; i++) sum[i] = 0.f;
+#pragma unroll
+    for (int m = 0; m < SHARES; m++)
+#pragma unroll
+        for (int i = 0; i < KP; i++) sum[i] += lds[(((cs2 << SPLIT) + m) * 64 + l2) * kLutRedStride + part * KP + i];
+    const int64_t r = q2 / rowdw;
+    const int z0 = (int)(q2 - r * rowdw) * 32 + part * KP;
+    if (whole_rows) {
+        uint32_t *o = reinterpret_cast<uint32_t *>(ret + q2 * 32 + part * KP);
+#pragma unroll
+        for (int i = 0; i < KP; i += 2)
+            o[i >> 1] = (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)sum[i]) |
+                        ((uint32_t)__builtin_bit_cast(uint16_t, (_Float16)sum[i + 1]) << 16);
+    } else {
+#pragma unroll
+        for (int i = 0; i < KP; i++)
+            if (z0 + i < zbits) ret[r * zbits + z0 + i] = (_Float16)sum[i];
+    }
+}
+
+template <typename W>
+int weighted_sum_fast_impl(uint16_t *ret, const W *in, const uint16_t *w, int64_t n, int64_t R, int64_t Rw,
+                           int64_t zbits, nb_stream_t stream, const char *who)
+{
+    NB_REQUIRE(n >= 0 && R >= 0 && Rw >= 0 && zbits >= 0, "%s: negative shape", who);
+    if (R * zbits == 0) return NB_OK;
+    NB_REQUIRE_PTR(ret);
+    NB_REQUIRE_ALIGNED(ret, 2);
+    if (n > 0) {
+        NB_REQUIRE_PTR(in);
+        NB_REQUIRE_PTR(w);
+        NB_REQUIRE_ALIGNED(in, sizeof(W));
+        NB_REQUIRE_ALIGNED(w, 2);
+    }
+    NB_REQUIRE(zbits <= (1 << 30) && Rw <= (1 << 30), "%s: row too long", who);
+    NB_REQUIRE(zbits <= Rw * (int64_t)WordTraits<W>::bits, "%s: zbits exceeds the Rw words of a row", who);
+    const int64_t rowdw = Rw * (int64_t)(sizeof(W) / 4), Q = R * rowdw;
+    NB_REQUIRE(Q < (1LL << 25), "%s: more than 2^25 32-bit columns", who);
+    const int64_t sets = ceil_div(Q, 64), nchunks = ceil_div(n, 64);
+    // member shares per column set: as many as it takes to give the chip about 4096 waves, while every share has a chunk
+    int split = 0;
+    while (split < 4 && (sets << split) < 4096 && (2LL << split) <= nchunks) split++;
+    if (const char *v = getenv("NESBIN_WSUM_SPLIT")) {
+        const int f = atoi(v);
+        if (f >= 0 && f <= 4) split = f;
+    }
+    const int whole = zbits == rowdw * 32 && aligned(ret, 16);
+    const int64_t blocks = ceil_div(sets, 16 >> split);
+    NB_REQUIRE(blocks <= kMaxGridX, "%s: output exceeds one launch", who);
+    static std::once_flag once;
+    static hipError_t attr = hipSuccess;
+    std::call_once(once, [] {
+        const void *fns[5] = {reinterpret_cast<const void *>(weighted_sum_lut_kernel<0>),
+                              reinterpret_cast<const void *>(weighted_sum_lut_kernel<1>),
+                              reinterpret_cast<const void *>(weighted_sum_lut_kernel<2>),
+                              reinterpret_cast<const void *>(weighted_sum_lut_kernel<3>),
+                              reinterpret_cast<const void *>(weighted_sum_lut_kernel<4>)};
+        for (const void *f : fns) {
+            const hipError_t e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, kLutLdsBytes);
+            if (e != hipSuccess) attr = e;
+        }
+    });
+    if (attr != hipSuccess) {
+        (void)hipGetLastError();
+        return fail(NB_ERR_UNSUPPORTED, "%s: cannot raise the kernel's LDS limit: %s", who, hipGetErrorString(attr));
+    }
+    auto launch = [&](auto kern) {
+        kern<<<dim3((unsigned)blocks), dim3(1024), kLutLdsBytes, as_stream(stream)>>>(
+            reinterpret_cast<_Float16 *>(ret), reinterpret_cast<const uint32_t *>(in),
+            reinterpret_cast<const _Float16 *>(w), n, Q, (int)rowdw, (int)zbits, whole);
+    };
+    switch (split) {
+        case 0: launch(weighted_sum_lut_kernel<0>); break;
+        case 1: launch(weighted_sum_lut_kernel<1>); break;
+        case 2: launch(weighted_sum_lut_kernel<2>); break;
+        case 3: launch(weighted_sum_lut_kernel<3>); break;
+        default: launch(weighted_sum_lut_kernel<4>); break;
+    }
+    return check_launch(who);
+}
+
 }  // namespace nb
 
 extern "C" {
@@ -251,5 +513,17 @@ int nb_weighted_sum_i32(uint16_t *ret, const int32_t *in, const uint16_t *w, int
 {
     return nb::weighted_sum_impl<uint32_t>(ret, reinterpret_cast<const uint32_t *>(in), w, n, R, Rw, zbits, s,
                                            "nb_weighted_sum_i32");
+}
+int nb_weighted_sum_fast_i64(uint16_t *ret, const int64_t *in, const uint16_t *w, int64_t n, int64_t R, int64_t Rw,
+                             int64_t zbits, nb_stream_t s)
+{
+    return nb::weighted_sum_fast_impl<uint64_t>(ret, reinterpret_cast<const uint64_t *>(in), w, n, R, Rw, zbits, s,
+                                                "nb_weighted_sum_fast_i64");
+}
+int nb_weighted_sum_fast_i32(uint16_t *ret, const int32_t *in, const uint16_t *w, int64_t n, int64_t R, int64_t Rw,
+                             int64_t zbits, nb_stream_t s)
+{
+    return nb::weighted_sum_fast_impl<uint32_t>(ret, reinterpret_cast<const uint32_t *>(in), w, n, R, Rw, zbits, s,
+                                                "nb_weighted_sum_fast_i32");
 }
 }

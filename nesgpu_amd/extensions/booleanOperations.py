@@ -482,10 +482,15 @@ def sample_bits(p, n, dtype, seed, conv_taps=None):
     return sample_bits_philox(thresholds_from_p(p), n, dtype, seed, conv_taps=conv_taps)
 
 
-def weighted_sum(input, weights, zbits):
+def weighted_sum(input, weights, zbits, fast=False):
     """ret[r,z] = fp16(sum_m weights[m] * bit(input[m,r,z/bits], z%bits)), fp32 accumulation
     (extensions/booleanOperations.py:218-229, extensions/src/weighted_sum.cu:28-46).  ``input`` may be a
-    :class:`FlipRows` (see :func:`weighted_sum_flip`)."""
+    :class:`FlipRows` (see :func:`weighted_sum_flip`).
+
+    ``fast=False`` adds in member order, as the reference's kernel does.  ``fast=True`` adds the members in blocks
+    (tables of partial sums over 8 members): the fp32 roundings fall elsewhere, a few 1e-7 of sum|weights| away from
+    the member-order result and far inside the reference's own tolerance for this op (booloptests.py:284-285), about
+    three times as fast."""
     if isinstance(input, FlipRows):
         return weighted_sum_flip(input, weights, zbits)
     assert len(input.shape) == 3
@@ -498,7 +503,8 @@ def weighted_sum(input, weights, zbits):
     assert zbits <= input.size(2) * bits
     ret = torch.empty((input.size(1), zbits), dtype=torch.float16, device=input.device)
     with _on(input):
-        _lib.call("nb_weighted_sum" + suf, ret.data_ptr(), input.data_ptr(), weights.data_ptr(), input.size(0),
+        _lib.call("nb_weighted_sum" + ("_fast" if fast else "") + suf, ret.data_ptr(), input.data_ptr(),
+                  weights.data_ptr(), input.size(0),
                   input.size(1), input.size(2), zbits, _stream(input))
     return ret
 

@@ -174,11 +174,14 @@ class Binarized(Perturbed, nn.Module):
         Perturbed.free_memory(self)
         self._cache = {}
 
-    def update(self, weights, l1=0, l2=1e-3):
-        """modules/binary.py:67-77."""
+    def update(self, weights, l1=0, l2=1e-3, exact=False):
+        """modules/binary.py:67-77.  The sum over the population adds the members in blocks (``weighted_sum`` with
+        ``fast=True``: fp32 roundings placed differently, far inside the reference's tolerance for the op,
+        booloptests.py:284-285); ``exact=True`` adds them one by one in member order like the reference's kernel."""
         weights = weights.type(torch.float16)
         weights = (weights - weights.mean())
-        self.weight.grad = booleanOperations.weighted_sum(self.weight_noise, weights.contiguous(), self.in_degree)
+        self.weight.grad = booleanOperations.weighted_sum(self.weight_noise, weights.contiguous(), self.in_degree,
+                                                          fast=not exact)
         if l1:
             self.weight.grad += l1 * torch.sign(self.weight)
         if l2:

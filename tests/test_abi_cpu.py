@@ -64,6 +64,8 @@ def test_bad_arguments_are_rejected_without_a_launch(lib):
     assert lib.nb_weighted_sum_i64(one, one, one, 4, 2, 1, 65, None) == 2
     assert b"zbits" in lib.nb_last_error_string()
     assert lib.nb_weighted_sum_i32(one, one, one, 4, 2, 2, 65, None) == 2
+    assert lib.nb_weighted_sum_fast_i64(one, one, one, 4, 2, 1, 65, None) == 2
+    assert lib.nb_weighted_sum_fast_i32(one, one, one, -1, 2, 2, 64, None) == 2
     # conv batch-norm thresholds: a pixel count below one, a misaligned fp16 pointer
     assert lib.nb_conv_bn_thresholds(one, one, one, one, 2, 3, 144, 0, None) == 2
     assert lib.nb_conv_bn_thresholds(one, one, ctypes.c_void_p(9), one, 2, 3, 144, 64, None) == 3

@@ -219,6 +219,12 @@ def test_perturbed_model_step(binary):
     f16 = f16 - f16.mean()
     want = torch.einsum("d,doi->oi", f16.float(), bits.float()) + 1e-3 * lin.weight.float()
     assert torch.allclose(lin.weight.grad.float(), want, rtol=1e-2, atol=2e-2)     # tolerance of booloptests.py:284
+    # the default adds the members in blocks; exact=True is the member-order op, bit for bit
+    fast = lin.weight.grad.clone()
+    pm.update(fitness, exact=True)
+    member_order = ops.weighted_sum(lin.weight_noise, f16.contiguous(), lin.in_degree) + 1e-3 * lin.weight
+    assert torch.equal(lin.weight.grad, member_order)
+    assert (fast.float() - lin.weight.grad.float()).abs().max().item() <= 2.0 ** -6
     pm.free_memory()
     assert all(l.weight_noise is None for l in pm.perturbed_layers)
 

@@ -460,6 +460,44 @@ def test_weighted_sum_vs_oracle(ops, oracle, dtype):
         np.testing.assert_array_equal(got, want.astype(np.float16).astype(np.float32))
 
 
+def _fp16_interval(exact, slack):
+    """The fp16 values a correctly rounded result may take when `exact` is known to within `slack`."""
+    with np.errstate(over="ignore"):
+        return (exact - slack).astype(np.float16).astype(np.float64), (exact + slack).astype(np.float16).astype(np.float64)
+
+
+@pytest.mark.parametrize("dtype", [torch.int64, torch.int32])
+def test_weighted_sum_fast_mode_within_fp16_rounding_of_the_exact_sum(ops, dtype):
+    """fast=True adds the members in blocks through tables of partial sums; the check is the float64 sum over the
+    unpacked bits: the result must be the fp16 rounding of a value within 1e-6 * sum|w| of it (fp32 roundings of
+    the partial sums), whatever the order.  Shapes: every member split (few / many columns), member counts around
+    the chunk of 64 and the block of 32, ragged rows, rows with unused words, one member, no members."""
+    g = rng(77)
+    nd = NDT[dtype]
+    wb = np.dtype(nd).itemsize * 8
+    for n, R, C in [(1024, 64, 1024), (1000, 7, 200), (64, 3, 256), (65, 2, 330), (33, 5, 100), (32, 4, 64),
+                    (31, 1, 31), (1, 1, 1), (200, 9, 576), (130, 700, 64), (257, 1, 1024), (2100, 3, 96),
+                    (96, 1300, 128), (70, 16, 2048), (40, 4200, 64), (512, 300, 1152), (0, 3, 100), (5, 2, 40)]:
+        for extra in (0, 1):  # rows with a word that holds no output bit
+            words = rand_words(g, (n, R, (C + wb - 1) // wb + extra), nd)
+            w = (g.standard_normal(n) * (3.0 if n % 2 else 0.05)).astype(np.float16)
+            got = host(ops.weighted_sum(dev(words), dev(w), C, fast=True)).astype(np.float64)
+            bits = np.unpackbits(np.ascontiguousarray(words).view(np.uint8), axis=-1, bitorder="little")[:, :, :C]
+            exact = np.einsum("m,mrc->rc", w.astype(np.float64), bits.astype(np.float64))
+            lo, hi = _fp16_interval(exact, 1e-6 * float(np.abs(w.astype(np.float64)).sum()) + 1e-30)
+            assert got.shape == (R, C)
+            bad = (got < lo) | (got > hi)
+            assert not bad.any(), (n, R, C, extra, int(bad.sum()), got[bad][:4], exact[bad][:4])
+    # the same call twice: the same bits (the order of the additions is fixed)
+    words = dev(rand_words(g, (1024, 256, 1024 // wb), nd))
+    w = dev(g.standard_normal(1024).astype(np.float16))
+    a = ops.weighted_sum(words, w, 1024, fast=True)
+    assert torch.equal(a, ops.weighted_sum(words, w, 1024, fast=True))
+    # and against the member-order kernel: equal up to the last fp16 digit
+    b = ops.weighted_sum(words, w, 1024)
+    assert (a.float() - b.float()).abs().max().item() <= 2.0 ** -5
+
+
 def test_ops_run_on_the_current_stream(ops, oracle):
     g = rng(2)
     A = rand_words(g, (4, 100, 9), np.int64)
