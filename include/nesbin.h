@@ -405,6 +405,26 @@ int nb_weighted_sum_fast_i64(uint16_t *ret, const int64_t *in, const uint16_t *w
 int nb_weighted_sum_fast_i32(uint16_t *ret, const int32_t *in, const uint16_t *w, int64_t n, int64_t R, int64_t Rw,
                              int64_t zbits, nb_stream_t stream);
 
+/* ---- the steps around weighted_sum in a layer's update ---------------------------------------------
+ * The tensor expressions of modules/binary.py:67-77 other than the weighted sum, one launch each.
+ *
+ * nb_center_fitness: out[i] (fp16) = fp16(x[i] - mean), x = fp16(in[i]) (round to nearest even), mean = the mean of the
+ *   x[i] rounded once to fp16 (the sum taken in double precision); replaces modules/binary.py:68-69
+ *   (weights.type(torch.float16); weights - weights.mean()).  torch's fp16 mean adds in fp32 in an order of its own
+ *   and multiplies by a rounded 1/n, so the two means can differ by one fp16 step when the exact mean lies within a
+ *   few 1e-7 (relative) of the middle between two fp16 numbers.  in: fp16 (_f16) or fp32 (_f32), n values.
+ * nb_grad_regularize: grad[i] = fp16(fp16(grad[i] + fp16(l1 * sign(weight[i]))) + fp16(l2 * weight[i])), in place, a
+ *   zero coefficient skipping its step; replaces modules/binary.py:73-76 with the same roundings (products in fp32
+ *   with the coefficient as a float, every tensor fp16).  sign(NaN) = 0.
+ * nb_bias_grad: out[o] (fp16 [O]) = fp16(sum_d centered[d] * bias_noise[d, o]), fp32 accumulation in a fixed order;
+ *   replaces modules/binary.py:77 (weights @ self.bias_noise; a library product there, whose order is its own).
+ *   centered fp16 [n], bias_noise fp16 [n, O]. */
+int nb_center_fitness_f16(uint16_t *out, const uint16_t *in, int64_t n, nb_stream_t stream);
+int nb_center_fitness_f32(uint16_t *out, const float *in, int64_t n, nb_stream_t stream);
+int nb_grad_regularize(uint16_t *grad, const uint16_t *weight, float l1, float l2, int64_t n, nb_stream_t stream);
+int nb_bias_grad(uint16_t *out, const uint16_t *centered, const uint16_t *bias_noise, int64_t n, int64_t O,
+                 nb_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

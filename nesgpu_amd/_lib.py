@@ -65,6 +65,10 @@ _PLAIN = {
     "nb_flip_weighted_sum_i64": [_PTR, _PTR, _PTR, _PTR, _PTR, _I64, _I64, _I64, _I64, _PTR],
     "nb_bmv_bn_act_static_i64": [_PTR, _PTR, _PTR, _PTR, _PTR, _I64, _I64, _I64, _I64, _I32, _PTR],
     "nb_conv_bn_thresholds": [_PTR, _PTR, _PTR, _PTR, _I64, _I64, _I64, _I64, _PTR],
+    "nb_center_fitness_f16": [_PTR, _PTR, _I64, _PTR],
+    "nb_center_fitness_f32": [_PTR, _PTR, _I64, _PTR],
+    "nb_grad_regularize": [_PTR, _PTR, ctypes.c_float, ctypes.c_float, _I64, _PTR],
+    "nb_bias_grad": [_PTR, _PTR, _PTR, _I64, _I64, _PTR],
 }
 # entry points that return a size (int64) instead of a status
 _SIZES = {

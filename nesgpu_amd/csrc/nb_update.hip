@@ -1,0 +1,138 @@
+// The small steps around weighted_sum in a layer's update (modules/binary.py:67-77), one kernel each instead of
+// three to four tensor expressions: the fitness vector centred in fp16, the l1 / l2 terms added to the gradient
+// estimate, and the bias gradient fitness @ bias_noise.
+#include "nb_common.hpp"
+#include "nb_conv_common.hpp"
+
+namespace nb {
+
+// out[i] = fp16(x[i] - mean) with x = fp16(in) and mean = the mean of the x[i] rounded once to fp16
+// (modules/binary.py:68-69: weights.type(float16), then weights - weights.mean()).  The sum of the x[i] is taken in
+// double precision (exact for any fitness vector whose values span less than 53 bits), where torch's fp16 mean adds
+// in fp32 in an order of its own and multiplies by a rounded 1/n: the two means agree unless the exact one lies
+// within a few 1e-7 (relative) of the middle between two fp16 numbers.  One workgroup.
+template <typename T>
+__global__ __launch_bounds__(1024) void center_fitness_kernel(_Float16 *__restrict__ out, const T *__restrict__ in,
+                                                              int64_t n)
+{
+    __shared__ double part[16];
+    __shared__ float mean_sh;
+    double s = 0.0;
+    for (int64_t i = threadIdx.x; i < n; i += 1024) s += (double)(float)(_Float16)in[i];
+#pragma unroll
+    for (int o = 32; o; o >>= 1) s += __shfl_xor(s, o);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = s;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        double t = 0.0;
+        for (int k = 0; k < 16; k++) t += part[k];
+        mean_sh = (float)double_round_once_fp16(t / (double)n);
+    }
+    __syncthreads();
+    const float m = mean_sh;
+    for (int64_t i = threadIdx.x; i < n; i += 1024) out[i] = (_Float16)((float)(_Float16)in[i] - m);
+}
+
+// grad += l1 * sign(w), then grad += l2 * w, each with the roundings of the fp16 tensor expressions of
+// modules/binary.py:73-76: the product with the coefficient (a float) rounded to fp16, then the sum rounded to fp16;
+// a coefficient of zero skips its step, as the `if` there does.  sign(NaN) = 0, like torch.sign.
+__global__ __launch_bounds__(256) void grad_regularize_kernel(_Float16 *__restrict__ grad, const _Float16 *__restrict__ w,
+                                                              float l1, float l2, int64_t n)
+{
+    NB_FLAT_LOOP(i, n)
+    {
+        if (i >= n) continue;
+        const float x = (float)w[i];
+        _Float16 g = grad[i];
+        if (l1 != 0.f) {
+            const float sg = (float)((0.f < x) - (x < 0.f));
+            g = (_Float16)((float)g + (float)(_Float16)(l1 * sg));
+        }
+        if (l2 != 0.f) g = (_Float16)((float)g + (float)(_Float16)(l2 * x));
+        grad[i] = g;
+    }
+}
+
+// out[o] = fp16(sum_d c[d] * noise[d, o]), fp32 accumulation (modules/binary.py:77: weights @ bias_noise).  A workgroup
+// takes 64 outputs (a lane each, so a wave reads 128 contiguous bytes per member); its 16 waves take the members
+// d = wave, wave + 16, ... with a fused multiply-add each, and the 16 partial sums are added in wave order: a fixed
+// order (the same bits on every run), not that of a library GEMV.
+__global__ __launch_bounds__(1024) void bias_grad_kernel(_Float16 *__restrict__ out, const _Float16 *__restrict__ c,
+                                                         const _Float16 *__restrict__ noise, int64_t n, int64_t O)
+{
+    __shared__ float part[16][64];
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const int64_t o = (int64_t)blockIdx.x * 64 + lane;
+    const int64_t oc = o < O ? o : O - 1;
+    float acc = 0.f;
+#pragma unroll 8
+    for (int64_t d = wv; d < n; d += 16) acc = fmaf((float)c[d], (float)noise[d * O + oc], acc);
+    part[wv][lane] = acc;
+    __syncthreads();
+    if (wv == 0 && o < O) {
+        float t = 0.f;
+#pragma unroll
+        for (int k = 0; k < 16; k++) t += part[k][lane];
+        out[o] = (_Float16)t;
+    }
+}
+
+template <typename T>
+static int center_fitness_impl(uint16_t *out, const T *in, int64_t n, nb_stream_t stream, const char *who)
+{
+    NB_REQUIRE(n >= 0, "%s: negative length", who);
+    if (n == 0) return NB_OK;
+    NB_REQUIRE_PTR(out);
+    NB_REQUIRE_PTR(in);
+    NB_REQUIRE_ALIGNED(out, 2);
+    NB_REQUIRE_ALIGNED(in, sizeof(T));
+    center_fitness_kernel<<<dim3(1), dim3(1024), 0, as_stream(stream)>>>(reinterpret_cast<_Float16 *>(out), in, n);
+    return check_launch(who);
+}
+
+}  // namespace nb
+
+extern "C" {
+int nb_center_fitness_f16(uint16_t *out, const uint16_t *in, int64_t n, nb_stream_t stream)
+{
+    return nb::center_fitness_impl(out, reinterpret_cast<const _Float16 *>(in), n, stream, "nb_center_fitness_f16");
+}
+int nb_center_fitness_f32(uint16_t *out, const float *in, int64_t n, nb_stream_t stream)
+{
+    return nb::center_fitness_impl(out, in, n, stream, "nb_center_fitness_f32");
+}
+
+int nb_grad_regularize(uint16_t *grad, const uint16_t *weight, float l1, float l2, int64_t n, nb_stream_t stream)
+{
+    NB_REQUIRE(n >= 0, "nb_grad_regularize: negative length");
+    if (n == 0 || (l1 == 0.f && l2 == 0.f)) return NB_OK;
+    NB_REQUIRE_PTR(grad);
+    NB_REQUIRE_PTR(weight);
+    NB_REQUIRE_ALIGNED(grad, 2);
+    NB_REQUIRE_ALIGNED(weight, 2);
+    nb::grad_regularize_kernel<<<dim3(nb::grid_for(n)), dim3(256), 0, nb::as_stream(stream)>>>(
+        reinterpret_cast<_Float16 *>(grad), reinterpret_cast<const _Float16 *>(weight), l1, l2, n);
+    return nb::check_launch("nb_grad_regularize");
+}
+
+int nb_bias_grad(uint16_t *out, const uint16_t *centered, const uint16_t *bias_noise, int64_t n, int64_t O,
+                 nb_stream_t stream)
+{
+    NB_REQUIRE(n >= 0 && O >= 0, "nb_bias_grad: negative shape");
+    if (O == 0) return NB_OK;
+    NB_REQUIRE_PTR(out);
+    NB_REQUIRE_ALIGNED(out, 2);
+    if (n > 0) {
+        NB_REQUIRE_PTR(centered);
+        NB_REQUIRE_PTR(bias_noise);
+        NB_REQUIRE_ALIGNED(centered, 2);
+        NB_REQUIRE_ALIGNED(bias_noise, 2);
+    }
+    const int64_t blocks = nb::ceil_div(O, 64);
+    NB_REQUIRE(blocks <= nb::kMaxGridX, "nb_bias_grad: too many outputs for one launch");
+    nb::bias_grad_kernel<<<dim3((unsigned)blocks), dim3(1024), 0, nb::as_stream(stream)>>>(
+        reinterpret_cast<_Float16 *>(out), reinterpret_cast<const _Float16 *>(centered),
+        reinterpret_cast<const _Float16 *>(bias_noise), n, O);
+    return nb::check_launch("nb_bias_grad");
+}
+}

@@ -28,6 +28,7 @@ __all__ = [
     "philox_words", "conv_act_pack", "conv_popc_sums", "conv_bn_thresholds_from_input", "tap_pack_filter", "tap_packing_applies", "conv_engine", "conv_last_engine",
     "bmv_act_pack", "bmv_bn_act", "ExpandedRows", "expand_rows", "bmm_nt", "FlipRows", "flip_rows_from_weights",
     "bmv_flip", "bmv_flip_act_pack", "skip_table", "flip_rows_skip", "flip_rows_to_weights",
+    "center_fitness", "grad_regularize_", "bias_grad",
 ]
 
 
@@ -507,6 +508,52 @@ def weighted_sum(input, weights, zbits, fast=False):
                   weights.data_ptr(), input.size(0),
                   input.size(1), input.size(2), zbits, _stream(input))
     return ret
+
+
+def center_fitness(weights):
+    """fp16 [n]: ``w = weights.type(torch.float16); w - w.mean()`` (modules/binary.py:68-69) in one kernel.  The mean
+    is the exact one of the fp16 values rounded once to fp16 (torch's own adds in fp32 and can land one fp16 step
+    away when the exact mean sits next to the middle between two fp16 numbers)."""
+    assert len(weights.shape) == 1
+    _check(weights, "weights")
+    if weights.dtype not in (torch.float16, torch.float32):
+        weights = weights.type(torch.float16)
+    weights = weights.contiguous()
+    out = torch.empty(weights.shape, dtype=torch.float16, device=weights.device)
+    with _on(weights):
+        _lib.call("nb_center_fitness_f16" if weights.dtype == torch.float16 else "nb_center_fitness_f32",
+                  out.data_ptr(), weights.data_ptr(), weights.numel(), _stream(weights))
+    return out
+
+
+def grad_regularize_(grad, weight, l1=0.0, l2=0.0):
+    """In place ``grad += l1 * sign(weight)`` (if l1), then ``grad += l2 * weight`` (if l2), with the roundings of
+    those fp16 tensor expressions (modules/binary.py:73-76), in one kernel.  Returns ``grad``."""
+    assert grad.dtype == torch.float16 and weight.dtype == torch.float16 and grad.shape == weight.shape
+    _check(grad, "grad")
+    _check(weight, "weight")
+    _same_device(grad, weight)
+    assert grad.is_contiguous() and weight.is_contiguous()
+    with _on(grad):
+        _lib.call("nb_grad_regularize", grad.data_ptr(), weight.data_ptr(), float(l1), float(l2), grad.numel(),
+                  _stream(grad))
+    return grad
+
+
+def bias_grad(centered, bias_noise):
+    """fp16 [out] = ``centered @ bias_noise`` (modules/binary.py:77) with fp32 accumulation in a fixed order; centered
+    fp16 [n], bias_noise fp16 [n, out]."""
+    assert centered.dtype == torch.float16 and bias_noise.dtype == torch.float16
+    assert len(centered.shape) == 1 and len(bias_noise.shape) == 2 and bias_noise.size(0) == centered.size(0)
+    _check(centered, "centered")
+    _check(bias_noise, "bias_noise")
+    _same_device(centered, bias_noise)
+    centered, bias_noise = centered.contiguous(), bias_noise.contiguous()
+    out = torch.empty((bias_noise.size(1),), dtype=torch.float16, device=centered.device)
+    with _on(centered):
+        _lib.call("nb_bias_grad", out.data_ptr(), centered.data_ptr(), bias_noise.data_ptr(), centered.size(0),
+                  bias_noise.size(1), _stream(centered))
+    return out
 
 
 def max_pool2d(input, filterx, filtery, padx, pady, stridex, stridey, REPEAT=128):

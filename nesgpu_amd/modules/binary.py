@@ -177,17 +177,18 @@ class Binarized(Perturbed, nn.Module):
     def update(self, weights, l1=0, l2=1e-3, exact=False):
         """modules/binary.py:67-77.  The sum over the population adds the members in blocks (``weighted_sum`` with
         ``fast=True``: fp32 roundings placed differently, far inside the reference's tolerance for the op,
-        booloptests.py:284-285); ``exact=True`` adds them one by one in member order like the reference's kernel."""
-        weights = weights.type(torch.float16)
-        weights = (weights - weights.mean())
-        self.weight.grad = booleanOperations.weighted_sum(self.weight_noise, weights.contiguous(), self.in_degree,
-                                                          fast=not exact)
-        if l1:
-            self.weight.grad += l1 * torch.sign(self.weight)
-        if l2:
-            self.weight.grad += l2 * self.weight
-        if self.threshold:
-            self.bias.grad = weights @ self.bias_noise
+        booloptests.py:284-285); ``exact=True`` adds them one by one in member order like the reference's kernel.
+        The tensor expressions around it are one kernel each with the same roundings (``center_fitness``,
+        ``grad_regularize_``, ``bias_grad`` of booleanOperations; the fitness mean is the exact one rounded once and
+        the bias gradient is added in a fixed order, where torch's reductions have orders of their own)."""
+        with torch.no_grad():
+            weights = booleanOperations.center_fitness(weights)
+            grad = booleanOperations.weighted_sum(self.weight_noise, weights, self.in_degree, fast=not exact)
+            if l1 or l2:
+                booleanOperations.grad_regularize_(grad, self.weight.detach(), l1, l2)
+            self.weight.grad = grad
+            if self.threshold:
+                self.bias.grad = booleanOperations.bias_grad(weights, self.bias_noise)
 
 
 class BinarizedLinear(Binarized):
@@ -487,6 +488,7 @@ class CapturedForward:
         self.model = model if isinstance(model, PerturbedModel) else PerturbedModel(model, None)
         self.layers = [m for m in self.model.perturbed_layers if isinstance(m, Binarized)]
         self.input = example_input.clone()
+        self._updates = {}
         with torch.no_grad():
             side = torch.cuda.Stream()
             side.wait_stream(torch.cuda.current_stream())
@@ -534,6 +536,37 @@ class CapturedForward:
                     thr = dict(static)["thresh"]
                     tag = (m.bias._version, m.bias.data_ptr(), m.bias_noise._version) + tuple(targs)
                     m._cache["thresh"] = (tag, thr, m.bias_noise)
+
+
+    def update(self, weights, l1=0, l2=1e-3, exact=False):
+        """``update`` of every layer (modules/binary.py:67-77) as one graph replay: recorded on the first call for a
+        given (l1, l2, exact) and shape of ``weights``, replayed afterwards with ``weights`` copied into the graph's
+        tensor.  The layers' ``.grad`` tensors are the graph's: the next replay overwrites them.  The graph reads the
+        noise where this object's :meth:`set_noise` puts it."""
+        key = (l1, l2, exact, weights.dtype, tuple(weights.shape))
+        rec = self._updates.get(key)
+        with torch.no_grad():
+            if rec is None:
+                static = weights.clone()
+                side = torch.cuda.Stream()
+                side.wait_stream(torch.cuda.current_stream())
+                with torch.cuda.stream(side):
+                    for m in self.layers:
+                        m.update(static, l1, l2, exact)
+                torch.cuda.current_stream().wait_stream(side)
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph):
+                    for m in self.layers:
+                        m.update(static, l1, l2, exact)
+                grads = [(m.weight.grad, m.bias.grad if m.threshold else None) for m in self.layers]
+                rec = self._updates[key] = (graph, static, grads)
+            graph, static, grads = rec
+            static.copy_(weights)
+            graph.replay()
+            for m, (gw, gb) in zip(self.layers, grads):
+                m.weight.grad = gw
+                if gb is not None:
+                    m.bias.grad = gb
 
 
 def capture(model, example_input, warmup=2):

@@ -358,6 +358,7 @@ def small_net_step(D=1024, classes=10, in_channels=24, seed=0, device="cuda", fu
 
     set_noise()
     forward.model, forward.input = net, bits          # for callers that capture the forward (binary.capture)
+    update.fitness = fitness
     return set_noise, forward, update
 
 

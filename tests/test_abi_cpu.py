@@ -66,6 +66,11 @@ def test_bad_arguments_are_rejected_without_a_launch(lib):
     assert lib.nb_weighted_sum_i32(one, one, one, 4, 2, 2, 65, None) == 2
     assert lib.nb_weighted_sum_fast_i64(one, one, one, 4, 2, 1, 65, None) == 2
     assert lib.nb_weighted_sum_fast_i32(one, one, one, -1, 2, 2, 64, None) == 2
+    # the update helpers: negative lengths, a misaligned fp32 pointer
+    assert lib.nb_center_fitness_f16(one, one, -1, None) == 2
+    assert lib.nb_center_fitness_f32(one, ctypes.c_void_p(10), 4, None) == 3
+    assert lib.nb_grad_regularize(one, one, 0.1, 0.1, -1, None) == 2
+    assert lib.nb_bias_grad(one, one, one, -1, 4, None) == 2
     # conv batch-norm thresholds: a pixel count below one, a misaligned fp16 pointer
     assert lib.nb_conv_bn_thresholds(one, one, one, one, 2, 3, 144, 0, None) == 2
     assert lib.nb_conv_bn_thresholds(one, one, ctypes.c_void_p(9), one, 2, 3, 144, 64, None) == 3

@@ -479,3 +479,45 @@ def test_sparse_form_is_chosen_by_the_flip_probabilities(binary):
     assert isinstance(off.weight_noise, torch.Tensor)
     flips = ops.unpack((off.weight_noise ^ off.sign_base()[None]).view(-1, 32)).float().mean().item()
     assert abs(flips - 0.01) < 0.002
+
+
+def test_update_helper_kernels_against_the_tensor_expressions(binary):
+    """center_fitness, grad_regularize_ and bias_grad against the lines of modules/binary.py:67-77 they replace:
+    the elementwise ones bit for bit (given the same mean), the two reductions against float64."""
+    from nesgpu_amd.extensions import booleanOperations as ops
+    g = torch.Generator(device="cuda")
+    g.manual_seed(5)
+    for n, dtype in [(1024, torch.float32), (1000, torch.float16), (1, torch.float32), (4096, torch.float64), (70, torch.float32)]:
+        fit = (torch.randn(n, device="cuda", generator=g, dtype=torch.float32) * 3 + 0.7).to(dtype)
+        got = ops.center_fitness(fit)
+        w16 = fit.type(torch.float16)
+        # the definition: exact mean of the fp16 values, rounded once
+        mean = torch.tensor(float(w16.double().sum().item() / n), dtype=torch.float64).to(torch.float16).cuda()
+        assert torch.equal(got, w16 - mean), (n, dtype)
+        # torch's own mean: the same, or one fp16 step of the mean away
+        theirs = w16 - w16.mean()
+        step = float(torch.finfo(torch.float16).eps) * max(abs(float(mean)), 2.0 ** -14)
+        # (one step of the mean, plus one of the difference where the two roundings fall apart)
+        assert (got.float() - theirs.float()).abs().max().item() <= step + 2.0 ** -10 * float((w16.abs().max() + mean.abs()))
+    for shape in [(10, 300), (64, 576), (1, 1), (257, 33)]:
+        w = torch.randn(shape, device="cuda", generator=g).half()
+        w[0, 0] = 0.0
+        grad0 = torch.randn(shape, device="cuda", generator=g).half()
+        for l1, l2 in [(0, 1e-3), (0.01, 0), (0.02, 0.3), (0, 0)]:
+            want = grad0.clone()
+            if l1:
+                want += l1 * torch.sign(w)
+            if l2:
+                want += l2 * w
+            got = ops.grad_regularize_(grad0.clone(), w, l1, l2)
+            assert torch.equal(got, want), (shape, l1, l2)
+    for n, O in [(1024, 64), (1000, 10), (16, 256), (3, 1), (2048, 130)]:
+        c = torch.randn(n, device="cuda", generator=g).half()
+        noise = ((torch.rand((n, O), device="cuda", generator=g) - 0.5) * 6).half()
+        got = ops.bias_grad(c, noise).double()
+        exact = c.double() @ noise.double()
+        slack = 1e-6 * float((c.double().abs().unsqueeze(1) * noise.double().abs()).sum(0).max())
+        lo, hi = (exact - slack).half().double(), (exact + slack).half().double()
+        assert ((got >= lo) & (got <= hi)).all(), (n, O)
+        assert torch.allclose(got.float(), (c @ noise).float(), rtol=2e-3, atol=2e-2)
+        assert torch.equal(ops.bias_grad(c, noise).double(), got)

@@ -279,3 +279,14 @@ def test_captured_forward_follows_the_eager_one(binary, kind):
                     assert torch.equal(l.weight_noise.entries[:8], b.entries[:8]) and torch.equal(l.weight_noise.info, b.info)
             cap.set_noise()                                         # back onto the graph's tensors
             assert ref_model is pm.model
+            # update replayed from its own graph against the eager update on the same noise and fitness
+            fit = torch.randn(D, device="cuda", generator=g)
+            cap.update(fit)
+            got_grads = [(l.weight.grad.clone(), l.bias.grad.clone() if l.threshold else None)
+                         for l in pm.perturbed_layers]
+            torch.cuda.synchronize()
+            pm.update(fit)
+            for l, (gw, gb) in zip(pm.perturbed_layers, got_grads):
+                assert torch.equal(l.weight.grad, gw), (it, type(l).__name__)
+                if gb is not None:
+                    assert torch.equal(l.bias.grad, gb), (it, type(l).__name__)
