@@ -208,6 +208,23 @@ int nb_flip_skip_i64(uint32_t *entries, uint32_t *info, uint32_t *overflow, cons
 int nb_flip_skip_thin_i64(uint32_t *entries, uint32_t *info, uint32_t *overflow, const uint16_t *law,
                           const uint32_t *table, uint64_t seed, uint64_t subseq, uint64_t first, int64_t D, int64_t R,
                           int64_t C, int64_t cap, nb_stream_t stream);
+/* The skip sampler's masks as packed words, for short rows (at most 8 words): out = base ^ mask (base NULL: the mask
+ * alone), the mask of row q = m*R + r being exactly the flips nb_flip_skip_i64 lists for it (same table, same words
+ * first + q*C + i of the stream), i.e. what nb_flip_to_dense_i64 makes of those lists.  Same layouts as the per-bit
+ * samplers: nb_sample_skip writes [n, R, ceil(C/bits)]; nb_sample_conv_skip takes the rows as (out channel, tap) pairs,
+ * R = O * KK, and writes out_rows [n, R, Rw] and / or out_conv [n, KK * Rw, O] like nb_sample_conv_philox (either may
+ * be NULL, not both).  About C*p + 1 random words per row instead of C: the conv layers' filters at small flip
+ * probabilities.  No counterpart in the reference (extensions/src/sample_bits.cu:47-57 draws every bit). */
+int nb_sample_skip_i64(int64_t *out, const int64_t *base, const uint32_t *table, uint64_t seed, uint64_t subseq,
+                       uint64_t first, int64_t n, int64_t R, int64_t C, nb_stream_t stream);
+int nb_sample_skip_i32(int32_t *out, const int32_t *base, const uint32_t *table, uint64_t seed, uint64_t subseq,
+                       uint64_t first, int64_t n, int64_t R, int64_t C, nb_stream_t stream);
+int nb_sample_conv_skip_i64(int64_t *out_conv, int64_t *out_rows, const int64_t *base, const uint32_t *table,
+                            uint64_t seed, uint64_t subseq, uint64_t first, int64_t n, int64_t O, int64_t KK, int64_t C,
+                            nb_stream_t stream);
+int nb_sample_conv_skip_i32(int32_t *out_conv, int32_t *out_rows, const int32_t *base, const uint32_t *table,
+                            uint64_t seed, uint64_t subseq, uint64_t first, int64_t n, int64_t O, int64_t KK, int64_t C,
+                            nb_stream_t stream);
 int64_t nb_law_workspace_bytes(void);
 int nb_thresholds_from_weights(uint32_t *thresholds, const uint16_t *weights, int64_t n, void *workspace,
                                nb_stream_t stream);

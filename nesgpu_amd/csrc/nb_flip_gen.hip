@@ -14,6 +14,7 @@
 // (their base bits, or their probabilities), its lanes walk those rows for member after member (a lane that has
 // finished a row starts its next member at once), and every row's entries go to the fixed place the list layout
 // gives them (nb_flip.hip), so nothing has to be counted first.
+#include <algorithm>
 #include <cmath>
 #include <cstdlib>
 #include <mutex>
@@ -572,6 +573,196 @@ static int gen_check(const uint32_t *entries, const uint32_t *info, const uint32
     return NB_OK;
 }
 
+
+// ---- the skip sampler's masks as packed words (short rows) ---------------------------------------------------------
+// out = base ^ mask for rows of at most KW words, the mask being the one the lists above describe: row q = m*R + r
+// walks the Philox words first + q*C + i exactly as fl_gen_kernel does, so the result is what expanding
+// nb_flip_skip's lists gives.  For the filters of a conv layer (64 to 512 channels per tap, a few flips per row at
+// most) that is one or two random words per row instead of one per bit.
+// A workgroup takes a chunk of `rc` rows (conv: whole output channels, rc = oc * KK) of `mc` members: a lane walks
+// row after row and leaves their words in LDS, then the workgroup writes the chunks where the update
+// step reads it ([n, R, Rw]) and, for a conv layer, where the conv multiplies it ([n, KK * Rw, O], word k of row
+// (o, t) at [m][t * Rw + k][o]), both in runs of whole lines.
+template <typename W>
+struct SkipDenseArgs {
+    W *out_rows, *out_conv;   // either may be null
+    const W *base;            // may be null: the mask alone
+    const uint32_t *table;
+    PhiloxKey key;
+    int64_t n, R;
+    int C, Rw, O, KK, oc, mc, nchunk;   // a chunk: oc output channels = oc * KK rows; nchunk chunks; mc members per workgroup
+    int tabw;                 // LDS words kept for the table: min(C, kSkipMaxTable) + 2, rounded up to even
+};
+
+template <typename W, int KW>
+__global__ __launch_bounds__(256) void sample_skip_kernel(const SkipDenseArgs<W> a)
+{
+    constexpr int bits = WordTraits<W>::bits, lb = WordTraits<W>::log2bits;
+    extern __shared__ uint32_t gen_lds[];
+    uint32_t *tab1 = gen_lds;                                            // a.tabw words
+    W *basebuf = reinterpret_cast<W *>(gen_lds + a.tabw);                // rc * Rw words: the chunk's base rows
+    W *stage = basebuf + a.oc * a.KK * a.Rw;                             // mc * rc * Rw words
+    // a rank of C or more ends the row whatever it is: only the first C entries of the table are ever looked at
+    const int Kfull = (int)a.table[0];
+    const int Kt = Kfull < a.C ? Kfull : a.C;
+    const float inv_log2q = __uint_as_float(a.table[1]);
+    const float c0 = -32.0f * inv_log2q;
+    for (int i = threadIdx.x; i < Kt + 2; i += 256)
+        tab1[i] = i == 0 ? 0u : (i <= Kt ? a.table[kSkipHeader + i - 1] : 0xFFFFFFFFu);
+    // 32-bit arithmetic throughout (the host checks the ranges): a 64-bit division costs as much as a row's walk
+    const unsigned ch = blockIdx.x % (unsigned)a.nchunk, mg = blockIdx.x / (unsigned)a.nchunk;
+    const int o0 = (int)ch * a.oc;                                      // first output channel of the chunk
+    const int ocl = a.O - o0 < a.oc ? a.O - o0 : a.oc;                  // its channels
+    const int r0 = o0 * a.KK, rows = ocl * a.KK;
+    const int64_t m0 = (int64_t)mg * a.mc;
+    const int members = (int)(a.n - m0 < a.mc ? a.n - m0 : a.mc);      // members of this workgroup
+    const int C = a.C, Rw = a.Rw;
+    const int words = rows * Rw;                                        // of one member's chunk
+    const int items = members * rows;                                   // rows to walk: item = ml * rows + rl
+    // the chunk's base rows, four loads in flight per lane
+    for (int j0 = 0; j0 < words; j0 += 1024) {
+        W v[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const int j = j0 + e * 256 + (int)threadIdx.x;
+            v[e] = (a.base && j < words) ? a.base[(int64_t)r0 * Rw + j] : (W)0;
+        }
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const int j = j0 + e * 256 + (int)threadIdx.x;
+            if (j < words) basebuf[j] = v[e];
+        }
+    }
+    __syncthreads();
+    // A lane walks item after item (lane, lane + 256, ...) without waiting for the others: a row takes one word or
+    // many, and lanes in step row by row would idle through the longest row of every pass.  One step of the walk is
+    // the same straight code for every lane (a lane out of items computes on and is ignored); only handing a finished
+    // row over is a branch.
+    const int qd = 256 / rows, qr = 256 - qd * rows;                    // the next item: 256 further
+    int it = (int)threadIdx.x;
+    int ml = it / rows, rl = it - ml * rows;
+    bool live = it < items;
+    auto first_word = [&]() { return a.key.first + (uint64_t)((m0 + ml) * a.R + r0 + rl) * (uint64_t)C; };
+    uint64_t g = live ? first_word() : 0;
+    W mask[KW];
+#pragma unroll
+    for (int k = 0; k < KW; k++) mask[k] = 0;
+    int pos = -1;
+    while (__any(live)) {
+        int rank[1] = {0};
+        if (Kt > 0) {                                                   // p = 0: no word is drawn, every row ends at once
+            const uint4 b = philox_block(a.key, g >> 2);
+            const uint32_t e = (uint32_t)g & 3u;
+            const uint32_t u[1] = {e == 0 ? b.x : e == 1 ? b.y : e == 2 ? b.z : b.w};
+            skip_ranks<1>(rank, tab1, Kt, u, inv_log2q, c0);
+        }
+        g++;
+        pos += rank[0] < Kt ? rank[0] + 1 : (Kt == Kfull && Kt > 0 ? Kt : C);
+        const bool done = pos >= C;
+        const W bit = (!done && rank[0] < Kt) ? (W)1 << (pos & (bits - 1)) : (W)0;
+#pragma unroll
+        for (int k = 0; k < KW; k++) mask[k] |= (pos >> lb) == k ? bit : (W)0;
+        if (live && done) {
+#pragma unroll
+            for (int k = 0; k < KW; k++) {
+                if (k < Rw) stage[ml * words + rl * Rw + k] = mask[k] ^ basebuf[rl * Rw + k];
+                mask[k] = 0;
+            }
+            it += 256;
+            ml += qd;
+            rl += qr;
+            if (rl >= rows) {
+                rl -= rows;
+                ml++;
+            }
+            live = it < items;
+            g = first_word();
+            pos = -1;
+        }
+    }
+    __syncthreads();
+    for (int mm = 0; mm < members; mm++) {
+        const int64_t m = m0 + mm;
+        const W *src = stage + mm * words;
+        if (a.out_rows) {
+            W *dst = a.out_rows + (m * a.R + r0) * Rw;
+            for (int j = threadIdx.x; j < words; j += 256) __builtin_nontemporal_store(src[j], dst + j);
+        }
+        if (a.out_conv) {
+            // the chunk's output channels o0 .. o0 + oc - 1; j = (t * Rw + k) * oc + ol.  No division per word where
+            // oc is a power of two (it almost always is) and a row is one word
+            const int oc = ocl;
+            const int sh = (oc & (oc - 1)) == 0 ? 31 - __builtin_clz((unsigned)oc) : -1;
+            W *dst = a.out_conv + m * (int64_t)a.KK * Rw * a.O + o0;
+            for (int j = threadIdx.x; j < words; j += 256) {
+                const int tk = sh >= 0 ? j >> sh : j / oc, ol = j - tk * oc;
+                int t = tk, k = 0;
+                if (KW > 1) {
+                    t = tk / Rw;
+                    k = tk - t * Rw;
+                }
+                __builtin_nontemporal_store(src[(ol * a.KK + t) * Rw + k], dst + (int64_t)tk * a.O + ol);
+            }
+        }
+    }
+}
+
+template <typename W>
+static int sample_skip_launch(W *out_conv, W *out_rows, const W *base, const uint32_t *table, uint64_t seed,
+                              uint64_t subseq, uint64_t first, int64_t n, int64_t O, int64_t KK, int64_t C,
+                              hipStream_t s, const char *who)
+{
+    constexpr int bits = WordTraits<W>::bits;
+    NB_REQUIRE(n >= 0 && O >= 0 && KK >= 1 && C >= 0, "%s: negative shape", who);
+    const int64_t R = O * KK, Rw = ceil_div(C, bits);
+    if (n * R * Rw == 0) return NB_OK;
+    NB_REQUIRE(out_conv || out_rows, "%s: no output", who);
+    NB_REQUIRE_PTR(table);
+    NB_REQUIRE_ALIGNED(table, 4);
+    NB_REQUIRE_ALIGNED(out_conv, sizeof(W));
+    NB_REQUIRE_ALIGNED(out_rows, sizeof(W));
+    NB_REQUIRE_ALIGNED(base, sizeof(W));
+    if (Rw > 8)
+        return fail(NB_ERR_UNSUPPORTED, "%s: rows of more than 8 words (%lld): use the flip lists or the per-bit sampler",
+                    who, (long long)Rw);
+    NB_REQUIRE(KK * Rw <= 4096 && R * Rw < (1LL << 31) && n < (1LL << 40), "%s: shape too large", who);
+    // rows per chunk: whole output channels, about 2048 words of staging at most; members per workgroup: enough rows
+    // to spread the table's load over, while the launch keeps a few thousand workgroups
+    int64_t oc = std::max<int64_t>(1, 2048 / (KK * Rw));
+    if (oc > O) oc = O;
+    if (oc >= 16) oc &= ~15LL;  // runs of whole 128-byte lines in the conv layout
+    const int64_t rc = oc * KK, nchunk = ceil_div(R, rc);
+    // members per workgroup: as many as 4096 words of staging hold (long queues of rows per lane even out the lanes),
+    // while the launch keeps a thousand workgroups
+    int64_t mc = std::max<int64_t>(1, 4096 / (rc * Rw));
+    while (mc > 1 && nchunk * ceil_div(n, mc) < 2048) mc >>= 1;
+    const int64_t blocks = nchunk * ceil_div(n, mc);
+    NB_REQUIRE(blocks <= kMaxGridX, "%s: too many workgroups for one launch", who);
+    SkipDenseArgs<W> a{};
+    a.out_rows = out_rows;
+    a.out_conv = out_conv;
+    a.base = base;
+    a.table = table;
+    a.key = PhiloxKey{seed, subseq, first};
+    a.n = n;
+    a.R = R;
+    a.C = (int)C;
+    a.Rw = (int)Rw;
+    a.O = (int)O;
+    a.KK = (int)KK;
+    a.oc = (int)oc;
+    a.mc = (int)mc;
+    a.nchunk = (int)nchunk;
+    a.tabw = (int)((std::min<int64_t>(C, kSkipMaxTable) + 3) & ~1LL);
+    const size_t lds = (size_t)a.tabw * 4 + (size_t)((mc + 1) * rc * Rw) * sizeof(W);
+    const dim3 grid((unsigned)blocks), block(256);
+    if (Rw == 1) sample_skip_kernel<W, 1><<<grid, block, lds, s>>>(a);
+    else if (Rw == 2) sample_skip_kernel<W, 2><<<grid, block, lds, s>>>(a);
+    else if (Rw <= 4) sample_skip_kernel<W, 4><<<grid, block, lds, s>>>(a);
+    else sample_skip_kernel<W, 8><<<grid, block, lds, s>>>(a);
+    return check_launch(who);
+}
+
 }  // namespace nb
 
 extern "C" {
@@ -634,6 +825,39 @@ int nb_flip_skip_thin_i64(uint32_t *entries, uint32_t *info, uint32_t *overflow,
     a.S = (int)((R + 63) / 64);
     a.cap = (int)cap;
     return nb::gen_launch(a, true, false, nb::as_stream(stream), who);
+}
+
+int nb_sample_skip_i64(int64_t *out, const int64_t *base, const uint32_t *table, uint64_t seed, uint64_t subseq,
+                       uint64_t first, int64_t n, int64_t R, int64_t C, nb_stream_t stream)
+{
+    NB_REQUIRE_PTR(out);
+    return nb::sample_skip_launch<uint64_t>(nullptr, reinterpret_cast<uint64_t *>(out),
+                                            reinterpret_cast<const uint64_t *>(base), table, seed, subseq, first, n, R, 1,
+                                            C, nb::as_stream(stream), "nb_sample_skip_i64");
+}
+int nb_sample_skip_i32(int32_t *out, const int32_t *base, const uint32_t *table, uint64_t seed, uint64_t subseq,
+                       uint64_t first, int64_t n, int64_t R, int64_t C, nb_stream_t stream)
+{
+    NB_REQUIRE_PTR(out);
+    return nb::sample_skip_launch<uint32_t>(nullptr, reinterpret_cast<uint32_t *>(out),
+                                            reinterpret_cast<const uint32_t *>(base), table, seed, subseq, first, n, R, 1,
+                                            C, nb::as_stream(stream), "nb_sample_skip_i32");
+}
+int nb_sample_conv_skip_i64(int64_t *out_conv, int64_t *out_rows, const int64_t *base, const uint32_t *table,
+                            uint64_t seed, uint64_t subseq, uint64_t first, int64_t n, int64_t O, int64_t KK, int64_t C,
+                            nb_stream_t stream)
+{
+    return nb::sample_skip_launch<uint64_t>(reinterpret_cast<uint64_t *>(out_conv), reinterpret_cast<uint64_t *>(out_rows),
+                                            reinterpret_cast<const uint64_t *>(base), table, seed, subseq, first, n, O, KK,
+                                            C, nb::as_stream(stream), "nb_sample_conv_skip_i64");
+}
+int nb_sample_conv_skip_i32(int32_t *out_conv, int32_t *out_rows, const int32_t *base, const uint32_t *table,
+                            uint64_t seed, uint64_t subseq, uint64_t first, int64_t n, int64_t O, int64_t KK, int64_t C,
+                            nb_stream_t stream)
+{
+    return nb::sample_skip_launch<uint32_t>(reinterpret_cast<uint32_t *>(out_conv), reinterpret_cast<uint32_t *>(out_rows),
+                                            reinterpret_cast<const uint32_t *>(base), table, seed, subseq, first, n, O, KK,
+                                            C, nb::as_stream(stream), "nb_sample_conv_skip_i32");
 }
 
 int64_t nb_law_workspace_bytes(void) { return nb::kLawBlocks * 8; }

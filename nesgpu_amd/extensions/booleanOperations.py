@@ -28,7 +28,7 @@ __all__ = [
     "philox_words", "conv_act_pack", "conv_popc_sums", "conv_bn_thresholds_from_input", "tap_pack_filter", "tap_packing_applies", "conv_engine", "conv_last_engine",
     "bmv_act_pack", "bmv_bn_act", "ExpandedRows", "expand_rows", "bmm_nt", "FlipRows", "flip_rows_from_weights",
     "bmv_flip", "bmv_flip_act_pack", "skip_table", "flip_rows_skip", "flip_rows_to_weights",
-    "center_fitness", "grad_regularize_", "bias_grad",
+    "center_fitness", "grad_regularize_", "bias_grad", "sample_bits_skip",
 ]
 
 
@@ -982,6 +982,44 @@ def flip_rows_skip(base, in_bits, n, threshold, seed, subsequence=0, first=0, ca
                   table.data_ptr(), int(seed) & (2 ** 64 - 1), int(subsequence), int(first), n, R, C, int(cap),
                   _stream(base))
     return FlipRows(base, n, R, Kw, C, info, entries, int(cap), overflow)
+
+
+SKIP_DENSE_MAX_WORDS = 8      # rows the dense form of the skip sampler takes (words per row)
+
+
+def sample_bits_skip(threshold, n, dtype, seed, subsequence=0, first=0, base=None, shape=None, conv_taps=None,
+                     rows_too=True, table=None):
+    """The skip sampler's draw as packed words, for rows of at most ``SKIP_DENSE_MAX_WORDS`` words: every bit of a
+    member's [R, C] tensor is set (or, with ``base`` [R, Rw], differs from it) with probability threshold / 2**32,
+    independently, like :func:`sample_bits_philox` with a scalar threshold; the generator draws only the gaps between
+    the set bits (about C*p + 1 words per row).  The bits are those of :func:`flip_rows_skip` with the same seed
+    (``flip_rows_to_weights`` of its lists), not those of the per-bit samplers.  ``conv_taps`` as in
+    :func:`sample_bits_from_words`: returns ``(rows_layout, conv_layout)``."""
+    suf, bits = _suffix(dtype)
+    if base is not None:
+        device = base.device
+        R = base.size(0)
+        C = int(shape[1]) if shape is not None else base.size(1) * bits
+    else:
+        R, C = shape
+        device = torch.device("cuda", torch.cuda.current_device())
+    Rw = ceil_div(C, bits)
+    if Rw > SKIP_DENSE_MAX_WORDS:
+        raise ValueError("sample_bits_skip takes rows of at most %d words; use flip_rows_skip" % SKIP_DENSE_MAX_WORDS)
+    bptr = _base_check(base, R, Rw, dtype, device)
+    if table is None:
+        table = _skip_table_for(int(threshold), device)
+    key = (int(seed) & (2 ** 64 - 1), int(subsequence), int(first))
+    with torch.cuda.device(device):
+        stream = torch.cuda.current_stream(device).cuda_stream
+        if conv_taps is not None:
+            conv, rows, O = _conv_outputs(conv_taps, rows_too, n, R, Rw, dtype, device)
+            _lib.call("nb_sample_conv_skip" + suf, conv.data_ptr(), None if rows is None else rows.data_ptr(), bptr,
+                      table.data_ptr(), *key, n, O, int(conv_taps), C, stream)
+            return rows, conv
+        ret = torch.empty((n, R, Rw), dtype=dtype, device=device)
+        _lib.call("nb_sample_skip" + suf, ret.data_ptr(), bptr, table.data_ptr(), *key, n, R, C, stream)
+    return ret
 
 
 class FlipLaw:

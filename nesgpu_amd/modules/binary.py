@@ -134,8 +134,15 @@ class Binarized(Perturbed, nn.Module):
             sampled = self._sample_sparse()
         elif self.flip_probability is not None:
             T = min(int(self.flip_probability * 4294967296.0), 0xFFFFFFFF)
-            sampled = booleanOperations.sample_bits_philox(T, self.directions, self.dtype, self.seed, base=self.sign_base(),
-                                                           shape=tuple(self.weight.shape), conv_taps=self.conv_taps)
+            words = booleanOperations.ceil_div(self.weight.size(1), torch.iinfo(self.dtype).bits)
+            # short rows and few flips (a conv layer's filters): only the gaps between flips are drawn.  Measured on
+            # 3x3 filters of 64 channels, population 4096: 2.3x the per-bit sampler's speed at p = 0.01, level with it
+            # near p = 0.07; rows of a few bits gain nothing
+            skip = (self.flip_probability <= 0.05 and self.weight.size(1) >= 32
+                    and words <= booleanOperations.SKIP_DENSE_MAX_WORDS)
+            sampler = booleanOperations.sample_bits_skip if skip else booleanOperations.sample_bits_philox
+            sampled = sampler(T, self.directions, self.dtype, self.seed, base=self.sign_base(),
+                              shape=tuple(self.weight.shape), conv_taps=self.conv_taps)
         elif self.weight.is_cuda:
             # sample_bits(P, directions, dtype, seed) of modules/binary.py:62 with the thresholds taken straight from
             # the latent weights

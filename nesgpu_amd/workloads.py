@@ -189,8 +189,9 @@ def cifar_net(D=4096, T=T_P01, seed=0, dtype=torch.int64, device="cuda", classes
         """Draw every member's weights of every layer again (what a training step's set_noise does)."""
         layers = []
         for i, (C, O, S) in enumerate(shapes):
-            _, filt = ops.sample_bits_philox(T, D, dtype, seed, 10 + i, base=conv_bases[i], shape=(O * 9, C),
-                                             conv_taps=9, rows_too=False)
+            # 64-channel taps: only the gaps between flips are drawn; the 3-channel first layer keeps the per-bit sampler
+            draw = ops.sample_bits_skip if C >= 32 else ops.sample_bits_philox
+            _, filt = draw(T, D, dtype, seed, 10 + i, base=conv_bases[i], shape=(O * 9, C), conv_taps=9, rows_too=False)
             thr = torch.full((D, O), 9 * C, dtype=torch.int32, device=device)
             layers.append((filt, thr) + _tap(filt, 3, C))
         state["layers"] = layers

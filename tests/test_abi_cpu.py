@@ -66,6 +66,10 @@ def test_bad_arguments_are_rejected_without_a_launch(lib):
     assert lib.nb_weighted_sum_i32(one, one, one, 4, 2, 2, 65, None) == 2
     assert lib.nb_weighted_sum_fast_i64(one, one, one, 4, 2, 1, 65, None) == 2
     assert lib.nb_weighted_sum_fast_i32(one, one, one, -1, 2, 2, 64, None) == 2
+    # the skip sampler as packed words: no output, rows of more than 8 words
+    assert lib.nb_sample_conv_skip_i64(None, None, one, one, 1, 0, 0, 2, 4, 9, 64, None) == 2
+    assert lib.nb_sample_skip_i64(one, one, one, 1, 0, 0, 2, 4, 576, None) == 4
+    assert lib.nb_sample_skip_i32(one, one, one, 1, 0, 0, 2, 4, 288, None) == 4
     # the update helpers: negative lengths, a misaligned fp32 pointer
     assert lib.nb_center_fitness_f16(one, one, -1, None) == 2
     assert lib.nb_center_fitness_f32(one, ctypes.c_void_p(10), 4, None) == 3

@@ -199,6 +199,58 @@ def test_skip_sampler_vs_oracle(ops, oracle, D, R, C, p, first):
     assert torch.equal(again.cnt, rows.cnt) and torch.equal(ops.flip_rows_to_weights(again), W)
 
 
+@pytest.mark.parametrize("dtype", [torch.int64, torch.int32])
+@pytest.mark.parametrize("n,O,KK,C,p,first", [(5, 64, 9, 64, 0.01, 0), (3, 128, 9, 64, 0.05, 4), (4, 16, 9, 16, 0.1, 3),
+                                              (2, 64, 9, 3, 0.02, 0), (3, 24, 1, 512, 0.01, 0), (2, 300, 1, 200, 0.3, 8),
+                                              (2, 7, 25, 130, 0.002, 1), (3, 70, 9, 256, 0.0, 0), (2, 33, 4, 100, 1.0, 0),
+                                              (9, 512, 9, 64, 0.01, 0), (1, 1, 1, 1, 0.5, 0)])
+def test_skip_sampler_as_packed_words_vs_oracle(ops, oracle, dtype, n, O, KK, C, p, first):
+    """sample_bits_skip (short rows, packed words) == base ^ the oracle's skip walk, in the row layout and in the conv
+    layout; for 64-bit words also == the lists of flip_rows_skip with the same seed, expanded."""
+    bits = 64 if dtype == torch.int64 else 32
+    R = O * KK
+    Rw = (C + bits - 1) // bits
+    if Rw > 8:
+        pytest.skip("rows of more than 8 words take the lists")
+    g = np.random.default_rng(n + O + C)
+    T = min(int(p * 2 ** 32), 2 ** 32 - 1)
+    seed, sub = 0xABCD + C, 5
+    base64 = sparse_mask(g, (R, C), 0.5)                                       # int64 [R, ceil(C/64)], tail bits zero
+    mask64 = oracle.skip_flips(ops.skip_table(T), seed, sub, first, n * R, C).reshape(n, R, -1)
+    want64 = base64[None] ^ mask64
+    if bits == 64:
+        base, want = base64, want64
+    else:                                                                       # the same bits as 32-bit words
+        base = np.ascontiguousarray(base64.view(np.int32)[:, :Rw])
+        want = np.ascontiguousarray(want64.view(np.int32).reshape(n, R, -1)[:, :, :Rw])
+    got = ops.sample_bits_skip(T, n, dtype, seed, subsequence=sub, first=first, base=dev(base), shape=(R, C))
+    np.testing.assert_array_equal(host(got), want)
+    rows, conv = ops.sample_bits_skip(T, n, dtype, seed, subsequence=sub, first=first, base=dev(base), shape=(R, C),
+                                      conv_taps=KK)
+    np.testing.assert_array_equal(host(rows), want)
+    # [n, KK*Rw, O]: word k of row (o, t) at [m][t*Rw + k][o]
+    want_conv = want.reshape(n, O, KK, Rw).transpose(0, 2, 3, 1).reshape(n, KK * Rw, O)
+    np.testing.assert_array_equal(host(conv), want_conv)
+    only_conv = ops.sample_bits_skip(T, n, dtype, seed, subsequence=sub, first=first, base=dev(base), shape=(R, C),
+                                     conv_taps=KK, rows_too=False)
+    assert only_conv[0] is None and torch.equal(only_conv[1], conv)
+    nobase = ops.sample_bits_skip(T, n, dtype, seed, subsequence=sub, first=first, shape=(R, C))
+    np.testing.assert_array_equal(host(nobase) ^ base[None], want)
+    if bits == 64:
+        lists = ops.flip_rows_skip(dev(base), C, n, T, seed, subsequence=sub, first=first)
+        if lists.overflowed() == 0:
+            assert torch.equal(ops.flip_rows_to_weights(lists), got)
+
+
+def test_skip_sampler_as_packed_words_rejects_long_rows(ops):
+    base = torch.zeros((4, 9), dtype=torch.int64, device="cuda")
+    with pytest.raises(ValueError, match="at most 8 words"):
+        ops.sample_bits_skip(1 << 24, 2, torch.int64, 1, base=base, shape=(4, 576))
+    with pytest.raises(RuntimeError, match="more than 8 words"):
+        ops._lib.call("nb_sample_skip_i64", base.data_ptr(), base.data_ptr(), ops.skip_table_buffer(ops.skip_table(1 << 24), "cuda").data_ptr(),
+                      1, 0, 0, 1, 4, 576, None)
+
+
 def test_skip_sampler_rate_at_the_size_of_a_wide_layer(ops):
     """8192 columns, p = 0.01, 64 members x 1024 rows: flip rate, row-count spread and column uniformity."""
     T = 42949672
