@@ -430,11 +430,21 @@ def hbm_kernels(torch, steps, warmup, graph=True, core=False):
     run("expand_rows [4096,128] -> FP4 codes", lambda: ops.expand_rows(x4), x4.numel() * 8 + ex.codes.numel())
     run("bmm_nt 4096 x 1024 x 8192 bits (FP4 matrix cores; bytes: operands once + int32 out)",
         lambda: ops.bmm_nt(ex, rows.base_expanded), ex.codes.numel() + rows.base_expanded.codes.numel() + G.numel() * 4)
-    run("bmv_flip_act_pack D=4096 [1024 x 8192], p=0.01 (lists + counts + order + G + thresholds)",
+    run("bmv_flip_act_pack D=4096 [1024 x 8192], p=0.01 (lists + row info + G + thresholds)",
         lambda: ops.bmv_flip_act_pack(rows, x4, thr4, G=G), rows.nbytes() + G.numel() * 4 + thr4.numel() * 4 + x4.numel() * 8)
     run("flip_rows_skip D=4096 [1024 x 8192], p=0.01 (bytes written)",
         lambda: ops.flip_rows_skip(b4, 8192, 4096, workloads.T_P01, 0, subsequence=13), rows.nbytes())
     del rows, x4, thr4, ex, G
+    # a conv layer's filters (128 x 3x3 taps of 64 channels) at p = 0.01 for 4096 members, both layouts: the skip
+    # sampler as packed words against one draw per bit
+    bc = torch.randint(-2 ** 62, 2 ** 62, (1152, 1), device=dev, generator=g, dtype=torch.int64)
+    run("sample_bits_skip D=4096 x [1152 rows x 64], p=0.01, rows + conv layout (bytes written)",
+        lambda: ops.sample_bits_skip(workloads.T_P01, 4096, torch.int64, 0, 11, base=bc, shape=(1152, 64), conv_taps=9),
+        2 * 4096 * 1152 * 8)
+    run("sample_bits_philox D=4096 x [1152 rows x 64], p=0.01, rows + conv layout (bytes written)",
+        lambda: ops.sample_bits_philox(workloads.T_P01, 4096, torch.int64, 0, 11, base=bc, shape=(1152, 64), conv_taps=9),
+        2 * 4096 * 1152 * 8)
+    del bc
     # first-layer filters of an RGB network: rows of 3 columns, one lane per row
     b1 = torch.randint(0, 8, (576, 1), device=dev, generator=g, dtype=torch.int64)
     run("sample (3-column rows) D=4096 x 576 rows, generator mode",
