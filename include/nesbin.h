@@ -362,6 +362,26 @@ int nb_sample_philox_i32(int32_t *out, const int32_t *base, const uint32_t *thre
                          nb_stream_t stream);
 int nb_philox_words(uint32_t *out, uint64_t seed, uint64_t subseq, uint64_t first, int64_t count,
                     nb_stream_t stream);
+/* philox16: the same law from 16-bit draws, two columns per generated word (the generator's vector instructions,
+ * not memory, bound the per-bit samplers above).  Column g = first + (m*R+r)*C + c takes half-word g % 2 (low half
+ * first) of element g / 2 of the stream (seed, subseq): h; the bit is set iff h < T >> 16, or h == T >> 16 and
+ * l < (T & 0xFFFF) with l the low 16 bits of element g of the stream (seed, subseq ^ 2^63): probability exactly
+ * T / 2^32, independent columns; the second stream is read on ties only (2^-16 of the columns).  Other bits than
+ * nb_sample_philox draws from the same seed.  Needs rows of whole words (C % bits == 0), first % 8 == 0 and 16-byte
+ * aligned thresholds; NB_ERR_UNSUPPORTED otherwise.  The conv forms write the second layout like
+ * nb_sample_conv_philox.  No counterpart in the reference (one 32-bit uniform per bit, extensions/src/sample_bits.cu:54). */
+int nb_sample_philox16_i64(int64_t *out, const int64_t *base, const uint32_t *thresh, uint32_t thr_scalar,
+                           uint64_t seed, uint64_t subseq, uint64_t first, int64_t n, int64_t R, int64_t C,
+                           nb_stream_t stream);
+int nb_sample_philox16_i32(int32_t *out, const int32_t *base, const uint32_t *thresh, uint32_t thr_scalar,
+                           uint64_t seed, uint64_t subseq, uint64_t first, int64_t n, int64_t R, int64_t C,
+                           nb_stream_t stream);
+int nb_sample_conv_philox16_i64(int64_t *out_conv, int64_t *out_rows, const int64_t *base, const uint32_t *thresh,
+                                uint32_t thr_scalar, uint64_t seed, uint64_t subseq, uint64_t first, int64_t n,
+                                int64_t O, int64_t KK, int64_t C, nb_stream_t stream);
+int nb_sample_conv_philox16_i32(int32_t *out_conv, int32_t *out_rows, const int32_t *base, const uint32_t *thresh,
+                                uint32_t thr_scalar, uint64_t seed, uint64_t subseq, uint64_t first, int64_t n,
+                                int64_t O, int64_t KK, int64_t C, nb_stream_t stream);
 /* Sampler thresholds from fp16 probabilities (what the layers' set_noise feeds the samplers, modules/binary.py:59-62):
  * T[i] = min(floor(P[i] * 2^32), 2^32 - 1), 0 for P <= 0 and NaN; exact (fp16 has 11 significant bits).  P = 1.0 fails
  * only for the word 0xFFFFFFFF, like `p > u` with u in (0, 1] (extensions/src/sample_bits.cu:54). */
@@ -441,6 +461,9 @@ int nb_center_fitness_f32(uint16_t *out, const float *in, int64_t n, nb_stream_t
 int nb_grad_regularize(uint16_t *grad, const uint16_t *weight, float l1, float l2, int64_t n, nb_stream_t stream);
 int nb_bias_grad(uint16_t *out, const uint16_t *centered, const uint16_t *bias_noise, int64_t n, int64_t O,
                  nb_stream_t stream);
+/* nb_bias_noise_scale: x[i] (fp16, in place) = fp16(fp16(x[i] - 0.5) * 6): the arithmetic of the bias noise of
+ *   modules/binary.py:63-64 on the uniform draw (which stays torch.rand), with the tensor expression's roundings. */
+int nb_bias_noise_scale(uint16_t *x, int64_t n, nb_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -36,6 +36,8 @@ _SUFFIXED = {
     "nb_max_pool2d": [_PTR, _PTR, _I64, _I64, _I64, _I64] + _GEOM + [_PTR],
     "nb_sample_from_words": [_PTR, _PTR, _PTR, _U32, _PTR, _I64, _I64, _I64, _PTR],
     "nb_sample_philox": [_PTR, _PTR, _PTR, _U32, _U64, _U64, _U64, _I64, _I64, _I64, _PTR],
+    "nb_sample_philox16": [_PTR, _PTR, _PTR, _U32, _U64, _U64, _U64, _I64, _I64, _I64, _PTR],
+    "nb_sample_conv_philox16": [_PTR, _PTR, _PTR, _PTR, _U32, _U64, _U64, _U64, _I64, _I64, _I64, _I64, _PTR],
     "nb_sample_conv_from_words": [_PTR, _PTR, _PTR, _PTR, _U32, _PTR, _I64, _I64, _I64, _I64, _PTR],
     "nb_sample_conv_philox": [_PTR, _PTR, _PTR, _PTR, _U32, _U64, _U64, _U64, _I64, _I64, _I64, _I64, _PTR],
     "nb_seeded_bmv_from_words": [_PTR, _PTR, _PTR, _U32, _PTR, _PTR, _I64, _I64, _I64, _PTR],
@@ -71,6 +73,7 @@ _PLAIN = {
     "nb_center_fitness_f32": [_PTR, _PTR, _I64, _PTR],
     "nb_grad_regularize": [_PTR, _PTR, ctypes.c_float, ctypes.c_float, _I64, _PTR],
     "nb_bias_grad": [_PTR, _PTR, _PTR, _I64, _I64, _PTR],
+    "nb_bias_noise_scale": [_PTR, _I64, _PTR],
 }
 # entry points that return a size (int64) instead of a status
 _SIZES = {

@@ -169,6 +169,124 @@ __global__ __launch_bounds__(256) void sample_word_philox_kernel(W *__restrict__
     }
 }
 
+// ---- the same with 16-bit draws: two weight bits per generated word -----------------------------------------------
+// Column g (flat index first + (m*R + r)*C + c) takes the half-word h = half g % 2 (low half first) of element g / 2 of
+// the stream (seed, subsequence) and is set iff h < T >> 16, or h == T >> 16 and l < (T & 0xFFFF) with l the low 16
+// bits of element g of the stream (seed, subsequence ^ 2^63): every bit is set with probability exactly T / 2^32,
+// independently, like the 32-bit compare, at half the generator work; the second stream is only read on a tie
+// (2^-16 of the columns).  A generator block serves 8 columns.
+//
+// One column: the subtraction's borrow IS h < T >> 16 when the half-word sits in the upper 16 bits and the threshold's
+// lower 16 bits are cleared, and is shifted in by an add-with-carry as in nibble_lt; the difference is below 65536
+// exactly on a tie, and the smallest difference of a block says whether any of its columns had one.
+__device__ __forceinline__ void col_lt16(uint32_t &r, uint32_t &zmin, uint32_t w_hi, uint32_t t_hi)
+{
+    uint32_t d;
+    asm("v_sub_co_u32 %1, vcc, %2, %3\n\tv_addc_co_u32 %0, vcc, %0, %0, vcc" : "+v"(r), "=&v"(d) : "v"(w_hi), "v"(t_hi) : "vcc");
+    zmin = d < zmin ? d : zmin;
+}
+
+// the 8 columns of a block, column 0 in bit 0; ta / tb: thresholds of columns 0..3 / 4..7 with their low halves cleared
+__device__ __forceinline__ uint32_t byte_lt16(uint4 w, uint4 ta, uint4 tb, uint32_t &zmin)
+{
+    uint32_t r = 0;
+    col_lt16(r, zmin, w.w, tb.w);
+    col_lt16(r, zmin, w.w << 16, tb.z);
+    col_lt16(r, zmin, w.z, tb.y);
+    col_lt16(r, zmin, w.z << 16, tb.x);
+    col_lt16(r, zmin, w.y, ta.w);
+    col_lt16(r, zmin, w.y << 16, ta.z);
+    col_lt16(r, zmin, w.x, ta.y);
+    col_lt16(r, zmin, w.x << 16, ta.x);
+    return r;
+}
+
+// the columns of a block that tied, decided by the second stream; g0: flat index of the block's column 0
+__device__ __forceinline__ uint32_t byte_ties16(uint32_t byte, uint4 w, uint4 ta, uint4 tb, const PhiloxKey &key, uint64_t g0)
+{
+    const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
+    const uint32_t tt[8] = {ta.x, ta.y, ta.z, ta.w, tb.x, tb.y, tb.z, tb.w};
+    const PhiloxKey tie{key.seed, key.subseq ^ 0x8000000000000000ull, 0};
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        const uint32_t h = (j & 1) ? ww[j >> 1] >> 16 : ww[j >> 1] & 0xFFFFu;
+        if (h == tt[j] >> 16) {
+            const uint32_t l = philox_word(tie, g0 + (uint64_t)j) & 0xFFFFu;
+            byte = (byte & ~(1u << j)) | ((uint32_t)(l < (tt[j] & 0xFFFFu)) << j);
+        }
+    }
+    return byte;
+}
+
+template <typename W, int U, bool HAS_THR, bool HAS_BASE>
+__global__ __launch_bounds__(256) void sample_word_philox16_kernel(W *__restrict__ out, const W *__restrict__ base,
+                                                                   const uint32_t *__restrict__ thresh, uint32_t ts,
+                                                                   PhiloxKey key, int64_t n, uint32_t PW, int64_t total,
+                                                                   ConvOut<W> conv, uint32_t Rw)
+{
+    constexpr int bits = WordTraits<W>::bits;
+    constexpr int NB = bits / 8;  // generator blocks per word
+    NB_FLAT_LOOP(i, total)
+    {
+        if (i < total) {
+            const int64_t mg = i / PW;
+            const uint32_t pw = (uint32_t)(i - mg * PW);
+            const uint4 *__restrict__ tq = reinterpret_cast<const uint4 *>(thresh) + (int64_t)pw * (2 * NB);
+            uint64_t blk[U];
+            W v[U];
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                blk[u] = (key.first >> 3) + (uint64_t)((mg * U + u) * PW + pw) * NB;  // first % 8 == 0 (host)
+                v[u] = 0;
+            }
+            uint64_t tied = 0;  // bit 8 * u + k: member u's block k had a tie (U <= 8, NB <= 8)
+            for (int k = 0; k < NB; k++) {
+                const uint4 ta = HAS_THR ? tq[2 * k] : make_uint4(ts, ts, ts, ts);
+                const uint4 tb = HAS_THR ? tq[2 * k + 1] : ta;
+                const uint4 ha = make_uint4(ta.x & 0xFFFF0000u, ta.y & 0xFFFF0000u, ta.z & 0xFFFF0000u, ta.w & 0xFFFF0000u);
+                const uint4 hb = make_uint4(tb.x & 0xFFFF0000u, tb.y & 0xFFFF0000u, tb.z & 0xFFFF0000u, tb.w & 0xFFFF0000u);
+#pragma unroll
+                for (int u = 0; u < U; u++) {
+                    uint32_t zmin = 0xFFFFFFFFu;
+                    const uint32_t byte = byte_lt16(philox_block(key, blk[u] + (uint64_t)k), ha, hb, zmin);
+                    tied |= (uint64_t)(zmin < 65536u) << (8 * u + k);
+                    v[u] |= (W)byte << (8 * k);
+                }
+            }
+            // ties (2^-16 of the columns): the blocks that had one are drawn again and decided by the second stream
+            if (__any(tied != 0)) {
+                while (tied) {
+                    const int bit = __builtin_ctzll(tied);
+                    tied &= tied - 1;
+                    const int uu = bit >> 3, k = bit & 7;
+                    const uint64_t b = (key.first >> 3) + (uint64_t)((mg * U + uu) * PW + pw) * NB + (uint64_t)k;
+                    const uint4 ta = HAS_THR ? tq[2 * k] : make_uint4(ts, ts, ts, ts);
+                    const uint4 tb = HAS_THR ? tq[2 * k + 1] : ta;
+                    const uint4 w = philox_block(key, b);
+                    uint32_t zmin = 0xFFFFFFFFu;
+                    const uint4 ha = make_uint4(ta.x & 0xFFFF0000u, ta.y & 0xFFFF0000u, ta.z & 0xFFFF0000u, ta.w & 0xFFFF0000u);
+                    const uint4 hb = make_uint4(tb.x & 0xFFFF0000u, tb.y & 0xFFFF0000u, tb.z & 0xFFFF0000u, tb.w & 0xFFFF0000u);
+                    const uint32_t byte = byte_ties16(byte_lt16(w, ha, hb, zmin), w, ta, tb, key, b << 3);
+                    const W clear = ~((W)0xFF << (8 * k)), put = (W)byte << (8 * k);
+#pragma unroll
+                    for (int u = 0; u < U; u++) v[u] = u == uu ? (v[u] & clear) | put : v[u];
+                }
+            }
+            const W bw = HAS_BASE ? base[pw] : (W)0;
+            const uint32_t r = pw / Rw;
+            const int64_t at2 = conv.out2 ? conv.at(r, pw - r * Rw, Rw) : 0;
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const int64_t m = mg * U + u;
+                if (m < n) {
+                    if (out) __builtin_nontemporal_store((W)(v[u] ^ bw), out + m * PW + pw);
+                    if (conv.out2) conv.out2[m * PW + at2] = v[u] ^ bw;
+                }
+            }
+        }
+    }
+}
+
 // ---- materialised sampler, generic path: one wave per (member,row), ballot builds the words ------
 template <typename W, class Src>
 __global__ __launch_bounds__(256) void sample_ballot_kernel(W *__restrict__ out, const W *__restrict__ base,
@@ -522,6 +640,46 @@ int sample_impl(W *out, const W *base, const uint32_t *thresh, uint32_t ts, Src 
     return check_launch(who);
 }
 
+// 16-bit draws: rows of whole words, a stream that starts on a block of 8 columns, thresholds (if any) 16-byte aligned
+template <typename W>
+int sample16_impl(W *out, const W *base, const uint32_t *thresh, uint32_t ts, PhiloxKey key, int64_t n, int64_t R,
+                  int64_t C, nb_stream_t stream, const char *who, W *out_conv = nullptr, int64_t KK = 1)
+{
+    constexpr int bits = WordTraits<W>::bits;
+    bool empty;
+    if (int rc = sample_check<W>(out ? out : out_conv, base, thresh, n, R, C, who, &empty)) return rc;
+    if (empty) return NB_OK;
+    NB_REQUIRE_ALIGNED(out, sizeof(W));
+    NB_REQUIRE_ALIGNED(out_conv, sizeof(W));
+    NB_REQUIRE(KK >= 1 && R % KK == 0 && R < (1LL << 31), "%s: %lld rows are not whole groups of %lld taps", who,
+               (long long)R, (long long)KK);
+    if (C % bits != 0 || (key.first & 7) != 0 || (thresh && !aligned(thresh, 16)) || R * (C / 4) >= (1LL << 30))
+        return fail(NB_ERR_UNSUPPORTED,
+                    "%s: 16-bit draws take rows of whole words, first %% 8 == 0 and 16-byte aligned thresholds", who);
+    const ConvOut<W> conv{out_conv, (uint32_t)KK, (uint32_t)(R / KK)};
+    hipStream_t s = as_stream(stream);
+    const int64_t Rw = C / bits;
+    const uint32_t PW = (uint32_t)(R * Rw);
+    const bool many = ceil_div(n, 8) * PW >= 131072;
+    const int64_t total = ceil_div(n, many ? 8 : 2) * PW;
+    const dim3 grid(grid_for(total)), block(256);
+#define NB_LAUNCH_WORD(UU, T, B)                                                                                       \
+    sample_word_philox16_kernel<W, UU, T, B><<<grid, block, 0, s>>>(out, base, thresh, ts, key, n, PW, total, conv, \
+                                                                   (uint32_t)Rw)
+#define NB_LAUNCH_WORD_U(T, B)            \
+    do {                                  \
+        if (many) NB_LAUNCH_WORD(8, T, B); \
+        else NB_LAUNCH_WORD(2, T, B);      \
+    } while (0)
+    if (thresh && base) NB_LAUNCH_WORD_U(true, true);
+    else if (thresh) NB_LAUNCH_WORD_U(true, false);
+    else if (base) NB_LAUNCH_WORD_U(false, true);
+    else NB_LAUNCH_WORD_U(false, false);
+#undef NB_LAUNCH_WORD_U
+#undef NB_LAUNCH_WORD
+    return check_launch(who);
+}
+
 template <typename W, class Src>
 int seeded_bmv_impl(int32_t *Cout, const W *base, const uint32_t *thresh, uint32_t ts, const W *x, Src src,
                     bool src_vec_ok, int64_t n, int64_t R, int64_t C, nb_stream_t stream, const char *who)
@@ -614,6 +772,38 @@ int nb_sample_philox_i32(int32_t *out, const int32_t *base, const uint32_t *thre
 {
     return nb::sample_impl<uint32_t, PhiloxSrc>(U32(out), CU32(base), thresh, ts, PhiloxSrc{{seed, subseq, first}},
                                                 (first & 3) == 0 && (C & 3) == 0, n, R, C, s, "nb_sample_philox_i32");
+}
+int nb_sample_philox16_i64(int64_t *out, const int64_t *base, const uint32_t *thresh, uint32_t ts, uint64_t seed,
+                           uint64_t subseq, uint64_t first, int64_t n, int64_t R, int64_t C, nb_stream_t s)
+{
+    return nb::sample16_impl<uint64_t>(U64(out), CU64(base), thresh, ts, nb::PhiloxKey{seed, subseq, first}, n, R, C, s,
+                                       "nb_sample_philox16_i64");
+}
+int nb_sample_philox16_i32(int32_t *out, const int32_t *base, const uint32_t *thresh, uint32_t ts, uint64_t seed,
+                           uint64_t subseq, uint64_t first, int64_t n, int64_t R, int64_t C, nb_stream_t s)
+{
+    return nb::sample16_impl<uint32_t>(U32(out), CU32(base), thresh, ts, nb::PhiloxKey{seed, subseq, first}, n, R, C, s,
+                                       "nb_sample_philox16_i32");
+}
+int nb_sample_conv_philox16_i64(int64_t *out_conv, int64_t *out_rows, const int64_t *base, const uint32_t *thresh,
+                                uint32_t ts, uint64_t seed, uint64_t subseq, uint64_t first, int64_t n, int64_t O,
+                                int64_t KK, int64_t C, nb_stream_t s)
+{
+    const char *who = "nb_sample_conv_philox16_i64";
+    if (O < 0 || KK < 1) return nb::fail(NB_ERR_SHAPE, "%s: bad shape O=%lld KK=%lld", who, (long long)O, (long long)KK);
+    if (n * O * KK * C > 0 && !out_conv) return nb::fail(NB_ERR_NULL, "%s: out_conv is NULL", who);
+    return nb::sample16_impl<uint64_t>(U64(out_rows), CU64(base), thresh, ts, nb::PhiloxKey{seed, subseq, first}, n,
+                                       O * KK, C, s, who, U64(out_conv), KK);
+}
+int nb_sample_conv_philox16_i32(int32_t *out_conv, int32_t *out_rows, const int32_t *base, const uint32_t *thresh,
+                                uint32_t ts, uint64_t seed, uint64_t subseq, uint64_t first, int64_t n, int64_t O,
+                                int64_t KK, int64_t C, nb_stream_t s)
+{
+    const char *who = "nb_sample_conv_philox16_i32";
+    if (O < 0 || KK < 1) return nb::fail(NB_ERR_SHAPE, "%s: bad shape O=%lld KK=%lld", who, (long long)O, (long long)KK);
+    if (n * O * KK * C > 0 && !out_conv) return nb::fail(NB_ERR_NULL, "%s: out_conv is NULL", who);
+    return nb::sample16_impl<uint32_t>(U32(out_rows), CU32(base), thresh, ts, nb::PhiloxKey{seed, subseq, first}, n,
+                                       O * KK, C, s, who, U32(out_conv), KK);
 }
 int nb_sample_conv_from_words_i64(int64_t *out_conv, int64_t *out_rows, const int64_t *base, const uint32_t *thresh,
                                   uint32_t ts, const uint32_t *words, int64_t n, int64_t O, int64_t KK, int64_t C,

@@ -1,6 +1,6 @@
 // The small steps around weighted_sum in a layer's update (modules/binary.py:67-77), one kernel each instead of
 // three to four tensor expressions: the fitness vector centred in fp16, the l1 / l2 terms added to the gradient
-// estimate, and the bias gradient fitness @ bias_noise.
+// estimate, and the bias gradient fitness @ bias_noise; and set_noise's scaling of the uniform bias draw.
 #include "nb_common.hpp"
 #include "nb_conv_common.hpp"
 
@@ -50,6 +50,18 @@ __global__ __launch_bounds__(256) void grad_regularize_kernel(_Float16 *__restri
         }
         if (l2 != 0.f) g = (_Float16)((float)g + (float)(_Float16)(l2 * x));
         grad[i] = g;
+    }
+}
+
+// x = (x - 0.5) * 6 with the roundings of the fp16 tensor expression of modules/binary.py:63-64 (the uniform draw itself
+// stays torch.rand on the device's global generator, as in the reference): fp16(fp16(x - 0.5) * 6), in place.
+__global__ __launch_bounds__(256) void bias_noise_scale_kernel(_Float16 *__restrict__ x, int64_t n)
+{
+    NB_FLAT_LOOP(i, n)
+    {
+        if (i >= n) continue;
+        const _Float16 c = (_Float16)((float)x[i] - 0.5f);
+        x[i] = (_Float16)((float)c * 6.0f);
     }
 }
 
@@ -113,6 +125,17 @@ int nb_grad_regularize(uint16_t *grad, const uint16_t *weight, float l1, float l
     nb::grad_regularize_kernel<<<dim3(nb::grid_for(n)), dim3(256), 0, nb::as_stream(stream)>>>(
         reinterpret_cast<_Float16 *>(grad), reinterpret_cast<const _Float16 *>(weight), l1, l2, n);
     return nb::check_launch("nb_grad_regularize");
+}
+
+int nb_bias_noise_scale(uint16_t *x, int64_t n, nb_stream_t stream)
+{
+    NB_REQUIRE(n >= 0, "nb_bias_noise_scale: negative length");
+    if (n == 0) return NB_OK;
+    NB_REQUIRE_PTR(x);
+    NB_REQUIRE_ALIGNED(x, 2);
+    nb::bias_noise_scale_kernel<<<dim3(nb::grid_for(n)), dim3(256), 0, nb::as_stream(stream)>>>(
+        reinterpret_cast<_Float16 *>(x), n);
+    return nb::check_launch("nb_bias_noise_scale");
 }
 
 int nb_bias_grad(uint16_t *out, const uint16_t *centered, const uint16_t *bias_noise, int64_t n, int64_t O,

@@ -28,7 +28,7 @@ __all__ = [
     "philox_words", "conv_act_pack", "conv_popc_sums", "conv_bn_thresholds_from_input", "tap_pack_filter", "tap_packing_applies", "conv_engine", "conv_last_engine",
     "bmv_act_pack", "bmv_bn_act", "ExpandedRows", "expand_rows", "bmm_nt", "FlipRows", "flip_rows_from_weights",
     "bmv_flip", "bmv_flip_act_pack", "skip_table", "flip_rows_skip", "flip_rows_to_weights",
-    "center_fitness", "grad_regularize_", "bias_grad", "sample_bits_skip",
+    "center_fitness", "grad_regularize_", "bias_grad", "sample_bits_skip", "half_draws_apply", "bias_noise_scale_",
 ]
 
 
@@ -540,6 +540,16 @@ def grad_regularize_(grad, weight, l1=0.0, l2=0.0):
     return grad
 
 
+def bias_noise_scale_(uniform):
+    """In place ``(uniform - .5) * 6`` with the roundings of that fp16 tensor expression (modules/binary.py:63-64), one
+    kernel; returns its argument."""
+    assert uniform.dtype == torch.float16 and uniform.is_contiguous()
+    _check(uniform, "uniform")
+    with _on(uniform):
+        _lib.call("nb_bias_noise_scale", uniform.data_ptr(), uniform.numel(), _stream(uniform))
+    return uniform
+
+
 def bias_grad(centered, bias_noise):
     """fp16 [out] = ``centered @ bias_noise`` (modules/binary.py:77) with fp32 accumulation in a fixed order; centered
     fp16 [n], bias_noise fp16 [n, out]."""
@@ -672,11 +682,25 @@ def flip_from_words(base_packed, words, threshold):
     return sample_bits_from_words(threshold, words, base_packed.dtype, base=base_packed)
 
 
+def half_draws_apply(C, dtype, first=0, threshold=None):
+    """Whether :func:`sample_bits_philox` can draw this shape from 16-bit half-words: rows of whole words, a stream
+    offset that is a multiple of 8, and (tensor thresholds) 16-byte aligned ones."""
+    bits = torch.iinfo(dtype).bits
+    ok = C > 0 and C % bits == 0 and int(first) % 8 == 0
+    if isinstance(threshold, torch.Tensor):
+        ok = ok and threshold.data_ptr() % 16 == 0
+    return ok
+
+
 def sample_bits_philox(threshold, n, dtype, seed, subsequence=0, first=0, base=None, shape=None, conv_taps=None,
-                       rows_too=True):
+                       rows_too=True, half_draws=False):
     """Like :func:`sample_bits_from_words` with the words generated in-kernel: word (m,r,c) is element
     ``first + (m*R+r)*C + c`` of the Philox4x32-10 stream (seed, subsequence) -- exactly what
-    :func:`philox_words` returns, so both forms agree bit for bit."""
+    :func:`philox_words` returns, so both forms agree bit for bit.
+
+    ``half_draws=True``: the same law from 16-bit draws, two columns per generated word, with a second stream
+    (subsequence ^ 2**63) deciding ties exactly (about 1.4 times as fast: the generator's instructions bound these
+    samplers); other bits than the default draws from the same seed; shapes as :func:`half_draws_apply` says."""
     suf, bits = _suffix(dtype)
     if isinstance(threshold, torch.Tensor):
         R, C = threshold.shape
@@ -687,16 +711,19 @@ def sample_bits_philox(threshold, n, dtype, seed, subsequence=0, first=0, base=N
     keep, tptr, ts = _thr_args(threshold, R, C, device)
     Rw = ceil_div(C, bits)
     bptr = _base_check(base, R, Rw, dtype, device)
+    if half_draws and not half_draws_apply(C, dtype, first, threshold if isinstance(threshold, torch.Tensor) else None):
+        raise ValueError("16-bit draws take rows of whole words and a stream offset that is a multiple of 8")
+    kind = "philox16" if half_draws else "philox"
     if conv_taps is not None:
         conv, rows, O = _conv_outputs(conv_taps, rows_too, n, R, Rw, dtype, device)
         with torch.cuda.device(device):
-            _lib.call("nb_sample_conv_philox" + suf, conv.data_ptr(), None if rows is None else rows.data_ptr(), bptr,
+            _lib.call("nb_sample_conv_" + kind + suf, conv.data_ptr(), None if rows is None else rows.data_ptr(), bptr,
                       tptr, ts, int(seed) & (2 ** 64 - 1), int(subsequence), int(first), n, O, int(conv_taps), C,
                       torch.cuda.current_stream(device).cuda_stream)
         return rows, conv
     ret = torch.empty((n, R, Rw), dtype=dtype, device=device)
     with torch.cuda.device(device):
-        _lib.call("nb_sample_philox" + suf, ret.data_ptr(), bptr, tptr, ts, int(seed) & (2 ** 64 - 1),
+        _lib.call("nb_sample_" + kind + suf, ret.data_ptr(), bptr, tptr, ts, int(seed) & (2 ** 64 - 1),
                   int(subsequence), int(first), n, R, C, torch.cuda.current_stream(device).cuda_stream)
     return ret
 

@@ -14,7 +14,8 @@ global one, and ``BinarizedConv2d(pack_output=True[, pool_output=True])`` return
 already packed along channels (and 2x2 OR-pooled) from one fused kernel instead of a bool map;
 ``fuse_packed_outputs(model)`` switches those on wherever a reference-style ``nn.Sequential`` allows it.
 ``flip_probability=p`` (any layer) replaces the law sigmoid(5 w / mean|w|) by "sign of the latent weight, flipped with
-probability p" (base XOR Bernoulli(p) flip mask).  ``BinarizedLinear(sparse=...)`` keeps ``weight_noise`` as the
+probability p" (base XOR Bernoulli(p) flip mask).  ``set_noise`` draws with 16 bits per weight bit where the rows are
+whole words (``half_draws``, a class attribute; same law, exact, see ``booleanOperations.sample_bits_philox``).  ``BinarizedLinear(sparse=...)`` keeps ``weight_noise`` as the
 shared base plus per-member flip lists (:class:`booleanOperations.FlipRows`) instead of materialised weights: the ops
 the layer calls (``bmm``, ``bmv_act_pack``, ``weighted_sum``) take either form and give the same results.
 """
@@ -140,15 +141,20 @@ class Binarized(Perturbed, nn.Module):
             # near p = 0.07; rows of a few bits gain nothing
             skip = (self.flip_probability <= 0.05 and self.weight.size(1) >= 32
                     and words <= booleanOperations.SKIP_DENSE_MAX_WORDS)
-            sampler = booleanOperations.sample_bits_skip if skip else booleanOperations.sample_bits_philox
-            sampled = sampler(T, self.directions, self.dtype, self.seed, base=self.sign_base(),
-                              shape=tuple(self.weight.shape), conv_taps=self.conv_taps)
+            if skip:
+                sampled = booleanOperations.sample_bits_skip(T, self.directions, self.dtype, self.seed,
+                                                             base=self.sign_base(), shape=tuple(self.weight.shape),
+                                                             conv_taps=self.conv_taps)
+            else:
+                sampled = booleanOperations.sample_bits_philox(T, self.directions, self.dtype, self.seed,
+                                                               base=self.sign_base(), shape=tuple(self.weight.shape),
+                                                               conv_taps=self.conv_taps, half_draws=self._half_draws())
         elif self.weight.is_cuda:
             # sample_bits(P, directions, dtype, seed) of modules/binary.py:62 with the thresholds taken straight from
             # the latent weights
             sampled = booleanOperations.sample_bits_philox(booleanOperations.thresholds_from_weights(self.weight),
                                                            self.directions, self.dtype, self.seed,
-                                                           conv_taps=self.conv_taps)
+                                                           conv_taps=self.conv_taps, half_draws=self._half_draws())
         else:
             sampled = booleanOperations.sample_bits(self.probabilities(), self.directions, self.dtype, self.seed,
                                                     conv_taps=self.conv_taps)
@@ -157,11 +163,20 @@ class Binarized(Perturbed, nn.Module):
         else:
             # one kernel wrote both layouts: rows (what update sums over) and [D, kx*ky*Cw, out] (what conv multiplies)
             self.weight_noise, self.weight_noise_reshaped = sampled
-        self.bias_noise = (torch.rand(size=(self.directions, self.out_degree), dtype=torch.float16,
-                                      device=self.weight.device, generator=bias_generator) - .5) * 6
+        # (torch.rand(...) - .5) * 6 of the reference, the arithmetic in one kernel with the same roundings
+        self.bias_noise = booleanOperations.bias_noise_scale_(
+            torch.rand(size=(self.directions, self.out_degree), dtype=torch.float16, device=self.weight.device,
+                       generator=bias_generator))
 
     def _sparse_now(self):
         return False
+
+    # Generator draws of 16 bits per weight bit (two per generated word, ties decided exactly by a second stream)
+    # wherever the rows are whole words: the generator's instructions bound set_noise.  False: one 32-bit draw per bit.
+    half_draws = True
+
+    def _half_draws(self):
+        return self.half_draws and booleanOperations.half_draws_apply(self.weight.size(1), self.dtype)
 
     def int_thresholds(self, offset, floor=False):
         """int32 [directions, out] thresholds ``(bias + bias_noise) -> int + offset`` of the integer compare

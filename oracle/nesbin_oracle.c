@@ -24,6 +24,9 @@
  *                        (Python integers); per-column flip rates against their own probabilities,
  *                        neighbouring columns uncorrelated, reduction to skip_flips' law when all
  *                        probabilities equal the largest one
+ *   draws16              an independent numpy evaluation from the (pinned) Philox words of the two streams,
+ *                        with thresholds that force ties; rates of columns whose thresholds have non-zero
+ *                        low halves; neighbouring columns (the two halves of one word) uncorrelated
  * The cuRAND XORWOW stream of the reference samplers (sample_bits.cu:23-25,54) is NOT
  * reproduced anywhere: parity unpinned for that stream; supplied-word parity replaces it.
  *
@@ -137,6 +140,40 @@ void nbo_philox_words(uint32_t *out, uint64_t seed, uint64_t subseq, uint64_t fi
         uint32_t o[4];
         nbo_philox4x32_10(o, ctr, key);
         out[i] = o[g & 3];
+    }
+}
+
+/* Bernoulli draws from 16-bit half-words: the contract of nb_sample_philox16_* (no counterpart in the reference,
+ * whose sampler compares a 32-bit uniform per bit, extensions/src/sample_bits.cu:47-57).  Column g = first + row*C + c
+ * (rows flat over members and rows) takes half-word g % 2 (low half first) of element g / 2 of the stream
+ * (seed, subseq): h; with T the column's threshold (thresh[(row % R)*C + c] or thr_scalar) the bit is set iff
+ * h < T >> 16, or h == T >> 16 and l < (T & 0xFFFF), l = the low 16 bits of element g of the stream
+ * (seed, subseq ^ 2^63).  P(bit) = T / 2^32 exactly.  bit: [rows, C] bytes. */
+void nbo_draws16(uint8_t *bit, const uint32_t *thresh, uint32_t thr_scalar, uint64_t seed, uint64_t subseq,
+                 uint64_t first, int64_t rows, int64_t R, int64_t C)
+{
+    const uint32_t key[2] = {(uint32_t)seed, (uint32_t)(seed >> 32)};
+    const uint64_t sub2 = subseq ^ 0x8000000000000000ull;
+#pragma omp parallel for schedule(static)
+    for (int64_t row = 0; row < rows; row++) {
+        for (int64_t c = 0; c < C; c++) {
+            const uint64_t g = first + (uint64_t)row * (uint64_t)C + (uint64_t)c;
+            const uint64_t e = g >> 1, blk = e >> 2;
+            const uint32_t ctr[4] = {(uint32_t)blk, (uint32_t)(blk >> 32), (uint32_t)subseq, (uint32_t)(subseq >> 32)};
+            uint32_t o[4];
+            nbo_philox4x32_10(o, ctr, key);
+            const uint32_t w = o[e & 3];
+            const uint32_t h = (g & 1) ? w >> 16 : w & 0xFFFFu;
+            const uint32_t t = thresh ? thresh[(row % R) * C + c] : thr_scalar;
+            uint8_t b = h < (t >> 16);
+            if (h == (t >> 16)) {
+                const uint64_t blk2 = g >> 2;
+                const uint32_t ctr2[4] = {(uint32_t)blk2, (uint32_t)(blk2 >> 32), (uint32_t)sub2, (uint32_t)(sub2 >> 32)};
+                nbo_philox4x32_10(o, ctr2, key);
+                b = (o[g & 3] & 0xFFFFu) < (t & 0xFFFFu);
+            }
+            bit[row * C + c] = b;
+        }
     }
 }
 

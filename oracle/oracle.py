@@ -236,6 +236,23 @@ def skip_cdf(T, cap=4096):
     return v[:n].astype(np.uint32)
 
 
+def sample_philox16(thresh, n, R, C, seed, subseq=0, first=0, dtype=np.int64, base=None):
+    """Packed [n, R, ceil(C/bits)] draws from 16-bit half-words (see nbo_draws16): ``thresh`` uint32 [R, C] or a
+    scalar; optional base [R, Rw] is XORed on."""
+    suf, wb, wt = _suf(dtype)
+    tarr, tsc = _thr_args(thresh)
+    if tarr is not None:
+        assert tarr.shape == (R, C)
+    bits = np.empty((int(n) * int(R), int(C)), dtype=np.uint8)
+    lib().nbo_draws16(_p(bits), _p(tarr), tsc, ctypes.c_uint64(int(seed)), ctypes.c_uint64(int(subseq)),
+                      ctypes.c_uint64(int(first)), _i64(n * R), _i64(R), _i64(C))
+    pad = (-int(C)) % wb
+    words = np.packbits(np.pad(bits, ((0, 0), (0, pad))), axis=1, bitorder="little").view(wt).reshape(int(n), int(R), -1)
+    if base is not None:
+        words = words ^ _c(base)[None]
+    return np.ascontiguousarray(words)
+
+
 def skip_flips(cdf, seed, subseq, first, rows, C):
     """Flip masks [rows, ceil(C/64)] int64 by gap sampling (see nbo_skip_flips_i64)."""
     cdf = _c(cdf, np.uint32)

@@ -75,6 +75,11 @@ def test_bad_arguments_are_rejected_without_a_launch(lib):
     assert lib.nb_center_fitness_f32(one, ctypes.c_void_p(10), 4, None) == 3
     assert lib.nb_grad_regularize(one, one, 0.1, 0.1, -1, None) == 2
     assert lib.nb_bias_grad(one, one, one, -1, 4, None) == 2
+    assert lib.nb_bias_noise_scale(one, -1, None) == 2
+    # 16-bit draws: rows that are not whole words, a stream offset that is not a multiple of 8
+    assert lib.nb_sample_philox16_i64(one, None, None, 5, 1, 0, 0, 2, 3, 70, None) == 4
+    assert lib.nb_sample_philox16_i32(one, None, None, 5, 1, 0, 4, 2, 3, 64, None) == 4
+    assert lib.nb_sample_conv_philox16_i64(None, one, None, None, 5, 1, 0, 0, 2, 3, 9, 64, None) == 1
     # conv batch-norm thresholds: a pixel count below one, a misaligned fp16 pointer
     assert lib.nb_conv_bn_thresholds(one, one, one, one, 2, 3, 144, 0, None) == 2
     assert lib.nb_conv_bn_thresholds(one, one, ctypes.c_void_p(9), one, 2, 3, 144, 64, None) == 3

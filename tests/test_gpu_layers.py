@@ -511,6 +511,9 @@ def test_update_helper_kernels_against_the_tensor_expressions(binary):
                 want += l2 * w
             got = ops.grad_regularize_(grad0.clone(), w, l1, l2)
             assert torch.equal(got, want), (shape, l1, l2)
+    for shape in [(1024, 64), (7, 3), (1, 1)]:
+        u = torch.rand(shape, device="cuda", generator=g, dtype=torch.float16)
+        assert torch.equal(ops.bias_noise_scale_(u.clone()), (u - .5) * 6)           # modules/binary.py:63-64
     for n, O in [(1024, 64), (1000, 10), (16, 256), (3, 1), (2048, 130)]:
         c = torch.randn(n, device="cuda", generator=g).half()
         noise = ((torch.rand((n, O), device="cuda", generator=g) - 0.5) * 6).half()

@@ -56,6 +56,15 @@ def f16(t):
     return t.detach().cpu().numpy().astype(np.float16)
 
 
+def host_weights(oracle, layer, D, R, C):
+    """The members' weights as set_noise draws them, regenerated on the host from the Philox stream (seed of the
+    layer, subsequence 0): 16-bit draws where the rows are whole words, one 32-bit draw per bit elsewhere."""
+    if layer._half_draws():
+        return oracle.sample_philox16(thresholds(layer), D, R, C, layer.seed, 0, 0, np.int64)
+    words = oracle.philox_words(layer.seed, 0, 0, D * R * C).reshape(D, R, C)
+    return oracle.sample_from_words(thresholds(layer), words, np.int64)
+
+
 def host_forward(oracle, layers, images_bits, D):
     """The forward of modules/binary.py replayed with the oracle's ops: weights regenerated from the Philox stream
     (seed of the layer, subsequence 0), fp16 threshold arithmetic in numpy in the reference's order."""
@@ -64,8 +73,7 @@ def host_forward(oracle, layers, images_bits, D):
     for conv in (conv1, conv2):
         C, O = conv.in_channels, conv.out_channels
         K = 9 * C
-        words = oracle.philox_words(conv.seed, 0, 0, D * O * 9 * C).reshape(D, O * 9, C)
-        Wn = oracle.sample_from_words(thresholds(conv), words, np.int64)              # [D, O*9, Cw]
+        Wn = host_weights(oracle, conv, D, O * 9, C)                                  # [D, O*9, Cw]
         np.testing.assert_array_equal(conv.weight_noise.cpu().numpy(), Wn)
         Cw = Wn.shape[2]
         filt = np.ascontiguousarray(Wn.reshape(D, O, 3, 3, Cw).transpose(0, 2, 3, 4, 1).reshape(D, 9 * Cw, O))
@@ -79,8 +87,7 @@ def host_forward(oracle, layers, images_bits, D):
         a = oracle.max_pool2d(oracle.pack(bits.reshape(-1, O), np.int64).reshape(D, H, H, -1), 2, 2, 0, 0, 2, 2)
     feats = a.reshape(D, -1)                                                          # nn.Flatten: (h, w, word) order
     Kin = lin.in_features
-    words = oracle.philox_words(lin.seed, 0, 0, D * lin.out_features * Kin).reshape(D, lin.out_features, Kin)
-    Wn = oracle.sample_from_words(thresholds(lin), words, np.int64)
+    Wn = host_weights(oracle, lin, D, lin.out_features, Kin)
     np.testing.assert_array_equal(lin.weight_noise.cpu().numpy(), Wn)
     act = 2 * oracle.bmm(Wn, feats.reshape(D, -1, 1))[:, :, 0].astype(np.int64) - Kin  # :97
     # :99-102 literally: the int32 activations go through fp16 (16384 input bits: beyond fp16's exact integers)

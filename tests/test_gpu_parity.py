@@ -434,6 +434,49 @@ def test_sample_bits_law_and_layout(ops):
 
 
 @pytest.mark.parametrize("dtype", [torch.int64, torch.int32])
+def test_sampler_from_half_word_draws_vs_oracle(ops, oracle, dtype):
+    """sample_bits_philox(half_draws=True) == the oracle's restatement of the 16-bit draws: scalar and per-element
+    thresholds (small probabilities: non-zero low halves), base, conv layout, few and many members (two and eight per
+    lane), stream offsets, and thresholds built from the stream itself so that one member ties in every third column
+    (the second stream decides those)."""
+    nd = NDT[dtype]
+    wb = np.dtype(nd).itemsize * 8
+    g = rng(41)
+    for n, R, C, first in [(3, 5, 2 * wb, 0), (9, 4, wb, 8), (40, 130, 3 * wb, 16), (2, 1, wb, 0), (600, 64, 4 * wb, 0)]:
+        seed, sub = 1234 + n, 3
+        Rw = C // wb
+        base = rand_words(g, (R, Rw), nd)
+        # per-element thresholds: probabilities from 1e-6 to 1, and every third column tied for member 1
+        P = 10.0 ** (-6 * g.random((R, C)))
+        T = np.minimum(np.floor(P * 2.0 ** 32), 2.0 ** 32 - 1).astype(np.uint32)
+        gi = first + R * C + np.arange(R * C, dtype=np.uint64)                       # member 1's flat indices
+        w1 = oracle.philox_words(seed, sub, int(gi[0]) // 2, R * C // 2 + 2)
+        w = w1[((gi >> np.uint64(1)) - np.uint64(int(gi[0]) // 2)).astype(np.int64)]
+        h = np.where(gi & np.uint64(1), w >> np.uint32(16), w & np.uint32(0xFFFF)).astype(np.uint32).reshape(R, C)
+        tie = np.arange(C) % 3 == 0
+        T[:, tie] = (h[:, tie] << np.uint32(16)) | (T[:, tie] & np.uint32(0xFFFF))
+        Td = torch.from_numpy(T.view(np.int32)).cuda().view(torch.uint32)
+        want = oracle.sample_philox16(T, n, R, C, seed, sub, first, nd, base=base)
+        got = ops.sample_bits_philox(Td, n, dtype, seed, sub, first, base=dev(base), half_draws=True)
+        np.testing.assert_array_equal(host(got), want, err_msg=str((n, R, C, first)))
+        want_s = oracle.sample_philox16(0x03000001, n, R, C, seed, sub, first, nd)
+        got_s = ops.sample_bits_philox(0x03000001, n, dtype, seed, sub, first, shape=(R, C), half_draws=True)
+        np.testing.assert_array_equal(host(got_s), want_s)
+        if R % 5 == 0:
+            KK, O = 5, R // 5
+            rows, conv = ops.sample_bits_philox(Td, n, dtype, seed, sub, first, base=dev(base), conv_taps=KK, half_draws=True)
+            np.testing.assert_array_equal(host(rows), want)
+            np.testing.assert_array_equal(host(conv), want.reshape(n, O, KK, Rw).transpose(0, 2, 3, 1).reshape(n, KK * Rw, O))
+    assert ops.half_draws_apply(64, torch.int64) and not ops.half_draws_apply(24, torch.int64)
+    assert not ops.half_draws_apply(64, torch.int64, first=4)
+    with pytest.raises(ValueError, match="whole words"):
+        ops.sample_bits_philox(1 << 30, 2, dtype, 1, shape=(3, wb + 8), half_draws=True)
+    with pytest.raises(RuntimeError, match="16-bit draws"):
+        out = torch.empty((2, 3, 1), dtype=dtype, device="cuda")
+        ops._lib.call("nb_sample_philox16" + ("_i64" if wb == 64 else "_i32"), out.data_ptr(), None, None, 1 << 30, 1, 0, 4, 2, 3, wb, None)
+
+
+@pytest.mark.parametrize("dtype", [torch.int64, torch.int32])
 def test_weighted_sum_vs_oracle(ops, oracle, dtype):
     g = rng(21)
     # the second line: rows that are whole 32-byte pieces (a wave per piece), also with fewer output bits than the

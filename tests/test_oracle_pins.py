@@ -356,3 +356,49 @@ def test_skip_flips_thin_against_a_numpy_walk_and_the_per_column_law(oracle):
         want = np.zeros(got.shape[1], np.uint8)
         want[pos[(pos < 300) & (rank < len(cdf3))]] = 1
         np.testing.assert_array_equal(got[q], want)
+
+
+def test_draws16_against_a_numpy_evaluation_ties_and_rates(oracle):
+    """Bernoulli draws from 16-bit half-words: the C restatement against an evaluation in numpy from the pinned
+    Philox words (first stream: half-words; second stream, subsequence ^ 2**63: the tie-breaking low halves), with
+    thresholds chosen so that a third of the columns tie; then what the law fixes: P(bit) = T / 2**32 also where T
+    has a non-zero low half, and the two halves of one word give uncorrelated bits."""
+    seed, sub = 0xC0FFEE, 7
+    n, R, C = 3, 5, 96
+    for first in (0, 8, 5):
+        g = first + np.arange(n * R * C, dtype=np.uint64)
+        w1 = oracle.philox_words(seed, sub, first // 2, (n * R * C + 3) // 2 + 2)
+        e = (g >> np.uint64(1)) - np.uint64(first // 2)
+        w = w1[e.astype(np.int64)]
+        h = np.where(g & np.uint64(1), w >> np.uint32(16), w & np.uint32(0xFFFF)).astype(np.uint32).reshape(n, R, C)
+        low = (oracle.philox_words(seed, sub ^ (1 << 63), first, n * R * C) & np.uint32(0xFFFF)).reshape(n, R, C)
+        rng = np.random.default_rng(first)
+        T = rng.integers(0, 2 ** 32, size=(R, C), dtype=np.uint64).astype(np.uint32)
+        # every third column: the high half of the threshold equals member 1's half-word there, so that member ties
+        tie_cols = (np.arange(C) % 3 == 0)
+        T[:, tie_cols] = (h[1][:, tie_cols] << np.uint32(16)) | (T[:, tie_cols] & np.uint32(0xFFFF))
+        thi, tlo = T >> np.uint32(16), T & np.uint32(0xFFFF)
+        want = (h < thi[None]) | ((h == thi[None]) & (low < tlo[None]))
+        assert ((h == thi[None]).sum()) >= R * tie_cols.sum()
+        got = oracle.sample_philox16(T, n, R, C, seed, sub, first, np.int64)
+        bits = np.unpackbits(got.view(np.uint8), axis=2, bitorder="little")[:, :, :C].astype(bool)
+        np.testing.assert_array_equal(bits, want, err_msg="first=%d" % first)
+        assert not np.unpackbits(got.view(np.uint8), axis=2, bitorder="little")[:, :, C:].any()
+        got32 = oracle.sample_philox16(T, n, R, C, seed, sub, first, np.int32)
+        np.testing.assert_array_equal(np.unpackbits(got32.view(np.uint8), axis=2, bitorder="little")[:, :, :C].astype(bool), want)
+    # rates: thresholds below 2**16 (only ties can set the bit), around 2**-10, and 1/3, over 200 000 draws a column
+    Tr = np.array([[40000, 3 << 20 | 12345, 0x55555555, 0]], dtype=np.uint32)
+    n2 = 200000
+    b = oracle.sample_philox16(Tr, n2, 1, 4, 99, 0, 0, np.int64)
+    cols = np.unpackbits(b.view(np.uint8), axis=2, bitorder="little")[:, 0, :4].astype(np.float64)
+    p = Tr[0].astype(np.float64) / 2.0 ** 32
+    assert (np.abs(cols.mean(axis=0) - p) <= 5 * np.sqrt(p * (1 - p) / n2) + 1e-12).all()
+    assert cols[:, 3].sum() == 0
+    # the two halves of a word: columns 0 and 1 of rows of two columns at p = 1/2
+    b2 = oracle.sample_philox16(1 << 31, n2, 1, 2, 5, 1, 0, np.int64)
+    c2 = np.unpackbits(b2.view(np.uint8), axis=2, bitorder="little")[:, 0, :2].astype(np.float64)
+    assert abs((c2[:, 0] * c2[:, 1]).mean() - 0.25) < 5 * np.sqrt(0.25 * 0.75 / n2)
+    # base is XORed on
+    base = np.array([[0x0F0F]], dtype=np.int64)
+    np.testing.assert_array_equal(oracle.sample_philox16(1 << 31, 4, 1, 16, 5, 1, 0, np.int64, base=base),
+                                  oracle.sample_philox16(1 << 31, 4, 1, 16, 5, 1, 0, np.int64) ^ base[None])
