@@ -63,6 +63,13 @@ int nb_bmm_i64(int32_t *C, const int64_t *A, const int64_t *B, int64_t Z, int64_
                nb_stream_t stream);
 int nb_bmm_i32(int32_t *C, const int32_t *A, const int32_t *B, int64_t Z, int64_t M, int64_t Kw, int64_t N,
                nb_stream_t stream);
+/* The linear layer's activations in one kernel: C[z, x] (int32 [Z, M]) = 2 * sum_k popc(A[z,x,k] ^ x[z,k]) - K, K the
+ * true number of input bits (modules/binary.py:97: `2 * bmm(...) - in_features`); A [Z, M, Kw], x [Z, Kw].  The
+ * matrix-vector kernels of nb_bmm (N = 1) with the affine map applied as the sums are stored. */
+int nb_bmv_pm1_i64(int32_t *C, const int64_t *A, const int64_t *x, int64_t Z, int64_t M, int64_t Kw, int64_t K,
+                   nb_stream_t stream);
+int nb_bmv_pm1_i32(int32_t *C, const int32_t *A, const int32_t *x, int64_t Z, int64_t M, int64_t Kw, int64_t K,
+                   nb_stream_t stream);
 /* same with the output (2*popc > thresh[z,y]) as bool bytes; thresh [Z,N] int32.
  *   replaces extensions/booleanOperations.py:131-158 (extensions/src/bmm_act.cu:5-63). */
 int nb_bmm_act_i64(uint8_t *C, const int64_t *A, const int64_t *B, const int32_t *thresh, int64_t Z, int64_t M,

@@ -23,6 +23,7 @@ _SUFFIXED = {
     "nb_unpack": [_PTR, _PTR, _I64, _I64, _PTR],
     "nb_int8pack": [_PTR, _PTR, _I64, _I64, _PTR],
     "nb_bmm": [_PTR, _PTR, _PTR, _I64, _I64, _I64, _I64, _PTR],
+    "nb_bmv_pm1": [_PTR, _PTR, _PTR, _I64, _I64, _I64, _I64, _PTR],
     "nb_bmm_act": [_PTR, _PTR, _PTR, _PTR, _I64, _I64, _I64, _I64, _PTR],
     "nb_bmv_act_pack": [_PTR, _PTR, _PTR, _PTR, _I64, _I64, _I64, _PTR],
     "nb_im2col": [_PTR, _PTR, _I64, _I64, _I64, _I64] + _GEOM + [_PTR],

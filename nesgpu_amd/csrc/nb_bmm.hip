@@ -12,7 +12,8 @@ namespace nb {
 
 template <typename W, int L, int V, int RPG, int BS>
 __global__ __launch_bounds__(BS) void bmv_kernel(int32_t *__restrict__ C, const W *__restrict__ A,
-                                                 const W *__restrict__ X, int64_t rows, int64_t M, int Kw)
+                                                 const W *__restrict__ X, int64_t rows, int64_t M, int Kw,
+                                                 int omul, int osub)
 {
     typedef W WV __attribute__((ext_vector_type(V == 2 ? 2 : 1)));
     const int64_t gid = ((int64_t)blockIdx.x * BS + threadIdx.x) / L;
@@ -59,7 +60,7 @@ __global__ __launch_bounds__(BS) void bmv_kernel(int32_t *__restrict__ C, const 
     if (sub == 0) {
 #pragma unroll
         for (int q = 0; q < RPG; q++)
-            if (r0 + q < rows) C[r0 + q] = acc[q];
+            if (r0 + q < rows) C[r0 + q] = acc[q] * omul - osub;
     }
 }
 
@@ -69,7 +70,8 @@ __global__ __launch_bounds__(BS) void bmv_kernel(int32_t *__restrict__ C, const 
 // member's input vector (the same few bytes for all lanes of a run, or two neighbouring ones) comes through the cache.
 template <int VPR, int Q>
 __global__ __launch_bounds__(256) void bmv_short_kernel(int32_t *__restrict__ C, const uint4 *__restrict__ A,
-                                                        const uint4 *__restrict__ X, uint32_t rows, uint32_t M)
+                                                        const uint4 *__restrict__ X, uint32_t rows, uint32_t M,
+                                                        int omul, int osub)
 {
     const uint32_t wave_first = (blockIdx.x * 256u + (threadIdx.x & ~63u)) * Q;
     const uint32_t lane = threadIdx.x & 63u;
@@ -96,16 +98,17 @@ __global__ __launch_bounds__(256) void bmv_short_kernel(int32_t *__restrict__ C,
             acc = bcnt_acc(a[q][v].z ^ x[q][v].z, acc);
             acc = bcnt_acc(a[q][v].w ^ x[q][v].w, acc);
         }
-        if (row[q] < rows) C[row[q]] = acc;
+        if (row[q] < rows) C[row[q]] = acc * omul - osub;
     }
 }
 
 template <int VPR>
-static void launch_bmv_short(int32_t *C, const void *A, const void *X, int64_t rows, int64_t M, hipStream_t s)
+static void launch_bmv_short(int32_t *C, const void *A, const void *X, int64_t rows, int64_t M, hipStream_t s, int omul,
+                             int osub)
 {
     constexpr int Q = 4;
     bmv_short_kernel<VPR, Q><<<dim3((unsigned)ceil_div(rows, 256 * Q)), dim3(256), 0, s>>>(
-        C, static_cast<const uint4 *>(A), static_cast<const uint4 *>(X), (uint32_t)rows, (uint32_t)M);
+        C, static_cast<const uint4 *>(A), static_cast<const uint4 *>(X), (uint32_t)rows, (uint32_t)M, omul, osub);
 }
 
 // Matrix-vector form for long rows: L lanes (16, 32 or 64) walk FOUR rows of one member with 16-byte streaming
@@ -123,7 +126,8 @@ static void launch_bmv_short(int32_t *C, const void *A, const void *X, int64_t r
 template <int L, int U, int BS, bool PACK = false>
 __global__ __launch_bounds__(BS) void bmv_quad_kernel(int32_t *__restrict__ C, const uint4 *__restrict__ A,
                                                       const uint4 *__restrict__ X, int64_t quads, int64_t M,
-                                                      int rowvecs, const int32_t *__restrict__ thresh = nullptr)
+                                                      int rowvecs, const int32_t *__restrict__ thresh = nullptr,
+                                                      int omul = 1, int osub = 0)
 {
     constexpr int RPB = 4 * BS / L;  // rows of a workgroup
     __shared__ uint32_t pieces[PACK ? RPB / 32 : 1];
@@ -173,7 +177,7 @@ __global__ __launch_bounds__(BS) void bmv_quad_kernel(int32_t *__restrict__ C, c
     // lane q < 4 of the group now holds row 2*(q&1) + (q>>1); streaming stores: the results are read by another
     // kernel, and ordinary stores between the row loads cost this kernel 2 % of its bandwidth (measured)
     if (!PACK) {
-        if (live && sub < 4) __builtin_nontemporal_store(v, C + r0 + 2 * (sub & 1) + (sub >> 1));
+        if (live && sub < 4) __builtin_nontemporal_store(v * omul - osub, C + r0 + 2 * (sub & 1) + (sub >> 1));
     } else {
         if (live && sub < 4) {
             const int64_t row = r0 + 2 * (sub & 1) + (sub >> 1);
@@ -188,7 +192,7 @@ __global__ __launch_bounds__(BS) void bmv_quad_kernel(int32_t *__restrict__ C, c
 
 template <int L, int U>
 static void launch_bmv_quad(int32_t *C, const void *A, const void *X, int64_t rows, int64_t M, int rowvecs, hipStream_t s,
-                            const int32_t *thresh = nullptr)
+                            const int32_t *thresh = nullptr, int omul = 1, int osub = 0)
 {
     constexpr int BS = 1024;
     const int64_t quads = rows / 4;
@@ -197,8 +201,8 @@ static void launch_bmv_quad(int32_t *C, const void *A, const void *X, int64_t ro
         bmv_quad_kernel<L, U, BS, true><<<dim3((unsigned)blocks), dim3(BS), 0, s>>>(
             C, static_cast<const uint4 *>(A), static_cast<const uint4 *>(X), quads, M, rowvecs, thresh);
     else
-        bmv_quad_kernel<L, U, BS><<<dim3((unsigned)blocks), dim3(BS), 0, s>>>(C, static_cast<const uint4 *>(A),
-                                                                            static_cast<const uint4 *>(X), quads, M, rowvecs);
+        bmv_quad_kernel<L, U, BS><<<dim3((unsigned)blocks), dim3(BS), 0, s>>>(
+            C, static_cast<const uint4 *>(A), static_cast<const uint4 *>(X), quads, M, rowvecs, nullptr, omul, osub);
 }
 
 // Any shape: one wave per output word, its rows one after the other (lanes stride over the row's words).
@@ -238,25 +242,27 @@ __global__ __launch_bounds__(256) void bmm_rowlane_kernel(RowsA<W> al, const W *
 }
 
 template <typename W, int L, int V>
-static void launch_bmv(int32_t *C, const W *A, const W *X, int64_t rows, int64_t M, int Kw, hipStream_t s)
+static void launch_bmv(int32_t *C, const W *A, const W *X, int64_t rows, int64_t M, int Kw, hipStream_t s, int omul,
+                       int osub)
 {
     constexpr int RPG = 4, BS = 1024;  // 8 rows per group measured slower (fewer waves fit)
     const int64_t groups = ceil_div(rows, RPG);
     const int64_t blocks = ceil_div(groups * L, BS);
-    bmv_kernel<W, L, V, RPG, BS><<<dim3((unsigned)blocks), dim3(BS), 0, s>>>(C, A, X, rows, M, Kw);
+    bmv_kernel<W, L, V, RPG, BS><<<dim3((unsigned)blocks), dim3(BS), 0, s>>>(C, A, X, rows, M, Kw, omul, osub);
 }
 
 template <typename W, int V>
-static void dispatch_bmv(int32_t *C, const W *A, const W *X, int64_t rows, int64_t M, int Kw, hipStream_t s)
+static void dispatch_bmv(int32_t *C, const W *A, const W *X, int64_t rows, int64_t M, int Kw, hipStream_t s, int omul,
+                         int osub)
 {
     const int per = (Kw + V - 1) / V;  // lane-steps needed to cover a row once
-    if (per <= 1) launch_bmv<W, 1, V>(C, A, X, rows, M, Kw, s);
-    else if (per <= 2) launch_bmv<W, 2, V>(C, A, X, rows, M, Kw, s);
-    else if (per <= 4) launch_bmv<W, 4, V>(C, A, X, rows, M, Kw, s);
-    else if (per <= 8) launch_bmv<W, 8, V>(C, A, X, rows, M, Kw, s);
-    else if (per <= 16) launch_bmv<W, 16, V>(C, A, X, rows, M, Kw, s);
-    else if (per <= 32) launch_bmv<W, 32, V>(C, A, X, rows, M, Kw, s);
-    else launch_bmv<W, 64, V>(C, A, X, rows, M, Kw, s);
+    if (per <= 1) launch_bmv<W, 1, V>(C, A, X, rows, M, Kw, s, omul, osub);
+    else if (per <= 2) launch_bmv<W, 2, V>(C, A, X, rows, M, Kw, s, omul, osub);
+    else if (per <= 4) launch_bmv<W, 4, V>(C, A, X, rows, M, Kw, s, omul, osub);
+    else if (per <= 8) launch_bmv<W, 8, V>(C, A, X, rows, M, Kw, s, omul, osub);
+    else if (per <= 16) launch_bmv<W, 16, V>(C, A, X, rows, M, Kw, s, omul, osub);
+    else if (per <= 32) launch_bmv<W, 32, V>(C, A, X, rows, M, Kw, s, omul, osub);
+    else launch_bmv<W, 64, V>(C, A, X, rows, M, Kw, s, omul, osub);
 }
 
 template <typename W, class Epi>
@@ -297,7 +303,7 @@ static int bmm_check(const void *C, const W *A, const W *B, int64_t Z, int64_t M
 
 template <typename W>
 int bmm_impl(int32_t *C, const W *A, const W *B, int64_t Z, int64_t M, int64_t Kw, int64_t N, nb_stream_t stream,
-             const char *who)
+             const char *who, int omul = 1, int osub = 0)  // N == 1 only: the sums leave as sum * omul - osub
 {
     bool empty;
     if (int rc = bmm_check<W>(C, A, B, Z, M, Kw, N, who, &empty)) return rc;
@@ -311,23 +317,23 @@ int bmm_impl(int32_t *C, const W *A, const W *B, int64_t Z, int64_t M, int64_t K
         const int64_t rowbytes = Kw * (int64_t)sizeof(W);
         if ((rowbytes == 16 || rowbytes == 32 || rowbytes == 64) && rows < (1LL << 31) && aligned(A, 16) &&
             aligned(B, 16)) {
-            if (rowbytes == 16) launch_bmv_short<1>(C, A, B, rows, M, s);
-            else if (rowbytes == 32) launch_bmv_short<2>(C, A, B, rows, M, s);
-            else launch_bmv_short<4>(C, A, B, rows, M, s);
+            if (rowbytes == 16) launch_bmv_short<1>(C, A, B, rows, M, s, omul, osub);
+            else if (rowbytes == 32) launch_bmv_short<2>(C, A, B, rows, M, s, omul, osub);
+            else launch_bmv_short<4>(C, A, B, rows, M, s, omul, osub);
         } else if (rowbytes % 16 == 0 && rowbytes >= 256 && M % 4 == 0 && aligned(A, 16) && aligned(B, 16)) {
             const int rowvecs = (int)(rowbytes / 16);
             // as many row steps in flight as divide the row (up to 16 loads of 16 bytes per lane), fewest lanes per row
-            if (rowvecs % 256 == 0) launch_bmv_quad<64, 4>(C, A, B, rows, M, rowvecs, s);
-            else if (rowvecs % 128 == 0) launch_bmv_quad<32, 4>(C, A, B, rows, M, rowvecs, s);
-            else if (rowvecs % 64 == 0) launch_bmv_quad<16, 4>(C, A, B, rows, M, rowvecs, s);
-            else if (rowvecs % 32 == 0) launch_bmv_quad<16, 2>(C, A, B, rows, M, rowvecs, s);
-            else if (rowvecs >= 64) launch_bmv_quad<64, 1>(C, A, B, rows, M, rowvecs, s);
-            else if (rowvecs >= 32) launch_bmv_quad<32, 1>(C, A, B, rows, M, rowvecs, s);
-            else launch_bmv_quad<16, 1>(C, A, B, rows, M, rowvecs, s);
+            if (rowvecs % 256 == 0) launch_bmv_quad<64, 4>(C, A, B, rows, M, rowvecs, s, nullptr, omul, osub);
+            else if (rowvecs % 128 == 0) launch_bmv_quad<32, 4>(C, A, B, rows, M, rowvecs, s, nullptr, omul, osub);
+            else if (rowvecs % 64 == 0) launch_bmv_quad<16, 4>(C, A, B, rows, M, rowvecs, s, nullptr, omul, osub);
+            else if (rowvecs % 32 == 0) launch_bmv_quad<16, 2>(C, A, B, rows, M, rowvecs, s, nullptr, omul, osub);
+            else if (rowvecs >= 64) launch_bmv_quad<64, 1>(C, A, B, rows, M, rowvecs, s, nullptr, omul, osub);
+            else if (rowvecs >= 32) launch_bmv_quad<32, 1>(C, A, B, rows, M, rowvecs, s, nullptr, omul, osub);
+            else launch_bmv_quad<16, 1>(C, A, B, rows, M, rowvecs, s, nullptr, omul, osub);
         } else if ((Kw & 1) == 0 && aligned(A, 2 * sizeof(W)) && aligned(B, 2 * sizeof(W)))
-            dispatch_bmv<W, 2>(C, A, B, rows, M, (int)Kw, s);
+            dispatch_bmv<W, 2>(C, A, B, rows, M, (int)Kw, s, omul, osub);
         else
-            dispatch_bmv<W, 1>(C, A, B, rows, M, (int)Kw, s);
+            dispatch_bmv<W, 1>(C, A, B, rows, M, (int)Kw, s, omul, osub);
     } else {
         RowsA<W> al{A, M, (int)Kw};
         EpiI32 epi{C, (N & 3) == 0 && aligned(C, 16)};
@@ -422,6 +428,24 @@ int nb_bmm_i32(int32_t *C, const int32_t *A, const int32_t *B, int64_t Z, int64_
 {
     return nb::bmm_impl<uint32_t>(C, reinterpret_cast<const uint32_t *>(A), reinterpret_cast<const uint32_t *>(B), Z,
                                   M, Kw, N, s, "nb_bmm_i32");
+}
+int nb_bmv_pm1_i64(int32_t *C, const int64_t *A, const int64_t *x, int64_t Z, int64_t M, int64_t Kw, int64_t K,
+                   nb_stream_t s)
+{
+    NB_REQUIRE(K >= 0 && K <= Kw * 64, "nb_bmv_pm1_i64: K = %lld bits does not fit the rows' %lld words", (long long)K,
+               (long long)Kw);
+    if (Kw == 0) return nb::fail(NB_ERR_SHAPE, "nb_bmv_pm1_i64: empty rows");
+    return nb::bmm_impl<uint64_t>(C, reinterpret_cast<const uint64_t *>(A), reinterpret_cast<const uint64_t *>(x), Z, M, Kw, 1, s,
+                                  "nb_bmv_pm1_i64", 2, (int)K);
+}
+int nb_bmv_pm1_i32(int32_t *C, const int32_t *A, const int32_t *x, int64_t Z, int64_t M, int64_t Kw, int64_t K,
+                   nb_stream_t s)
+{
+    NB_REQUIRE(K >= 0 && K <= Kw * 32, "nb_bmv_pm1_i32: K = %lld bits does not fit the rows' %lld words", (long long)K,
+               (long long)Kw);
+    if (Kw == 0) return nb::fail(NB_ERR_SHAPE, "nb_bmv_pm1_i32: empty rows");
+    return nb::bmm_impl<uint32_t>(C, reinterpret_cast<const uint32_t *>(A), reinterpret_cast<const uint32_t *>(x), Z, M, Kw, 1, s,
+                                  "nb_bmv_pm1_i32", 2, (int)K);
 }
 int nb_bmm_act_i64(uint8_t *C, const int64_t *A, const int64_t *B, const int32_t *thresh, int64_t Z, int64_t M,
                    int64_t Kw, int64_t N, nb_stream_t s)

@@ -28,7 +28,7 @@ __all__ = [
     "philox_words", "conv_act_pack", "conv_popc_sums", "conv_bn_thresholds_from_input", "tap_pack_filter", "tap_packing_applies", "conv_engine", "conv_last_engine",
     "bmv_act_pack", "bmv_bn_act", "ExpandedRows", "expand_rows", "bmm_nt", "FlipRows", "flip_rows_from_weights",
     "bmv_flip", "bmv_flip_act_pack", "skip_table", "flip_rows_skip", "flip_rows_to_weights",
-    "center_fitness", "grad_regularize_", "bias_grad", "sample_bits_skip", "half_draws_apply", "bias_noise_scale_",
+    "center_fitness", "grad_regularize_", "bias_grad", "sample_bits_skip", "half_draws_apply", "bias_noise_scale_", "bmv_pm1",
 ]
 
 
@@ -169,6 +169,28 @@ def bmm_act(A, B, threshold):
         _lib.call("nb_bmm_act" + suf, C.data_ptr(), A.data_ptr(), B.data_ptr(), threshold.data_ptr(), A.size(0),
                   A.size(1), A.size(2), B.size(2), _stream(A))
     return C
+
+
+def bmv_pm1(A, x, in_bits):
+    """int32 [Z, M] = ``2 * bmm(A, x.view(Z, Kw, 1)).squeeze(2) - in_bits``: a linear layer's activations
+    (modules/binary.py:97) in one kernel; A [Z, M, Kw] packed weights, x [Z, Kw] one packed input row per member."""
+    assert len(A.shape) == 3 and len(x.shape) == 2
+    assert A.size(0) == x.size(0) and A.size(2) == x.size(1)
+    _check(A, "A")
+    _check(x, "x")
+    _same_device(A, x)
+    assert A.dtype == x.dtype
+    suf, bits = _suffix(A.dtype)
+    assert 0 <= in_bits <= A.size(2) * bits
+    out = torch.empty((A.size(0), A.size(1)), dtype=torch.int32, device=A.device)
+    if out.numel() == 0:
+        return out
+    if A.size(2) == 0:
+        return out.fill_(-int(in_bits))
+    with _on(A):
+        _lib.call("nb_bmv_pm1" + suf, out.data_ptr(), A.data_ptr(), x.data_ptr(), A.size(0), A.size(1), A.size(2),
+                  int(in_bits), _stream(A))
+    return out
 
 
 def bmv_act_pack(A, x, threshold):

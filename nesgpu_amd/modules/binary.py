@@ -304,8 +304,12 @@ class BinarizedLinear(Binarized):
             # activation > t  <=>  2*popc - K > floor(t)  <=>  2*popc > floor(t) + K  (activation is an integer)
             thresh = self.int_thresholds(self.in_features, floor=True)
             return booleanOperations.bmv_act_pack(self.weight_noise, packed_input.view(self.directions, -1), thresh)
-        popc = booleanOperations.bmm(self.weight_noise, packed_input.view(self.directions, -1, 1))
-        activation = 2 * popc.squeeze(dim=2) - self.in_features
+        if dense:
+            activation = booleanOperations.bmv_pm1(self.weight_noise, packed_input.view(self.directions, -1),
+                                                   self.in_features)                       # :97 in one kernel
+        else:
+            popc = booleanOperations.bmm(self.weight_noise, packed_input.view(self.directions, -1, 1))
+            activation = 2 * popc.squeeze(dim=2) - self.in_features
         if self.threshold:
             thresh = (self.bias + self.bias_noise)
             if self.batch_norm:
@@ -504,19 +508,24 @@ class CapturedForward:
     brings the integer thresholds that depend on ``bias`` up to date.  Shapes must not change between draws (a
     flip-list layer keeps its capacity as long as its latent weights give the same one; otherwise capture again).
     ``forward(input)`` copies ``input`` into the graph's input tensor, replays, and returns the graph's output tensor
-    (overwritten by the next replay)."""
+    (overwritten by the next replay).  ``batches=K``: ``example_input`` is [K, ...], K input batches evaluated on the same
+    noise (a fitness evaluation over several minibatches per draw); the graph holds the K forwards and ``forward``
+    returns the list of their K outputs from ONE replay, which matters for small networks: launching a graph from
+    Python costs about 15 us whatever it holds."""
 
-    def __init__(self, model, example_input, warmup=2):
+    def __init__(self, model, example_input, warmup=2, batches=None):
         self.model = model if isinstance(model, PerturbedModel) else PerturbedModel(model, None)
         self.layers = [m for m in self.model.perturbed_layers if isinstance(m, Binarized)]
         self.input = example_input.clone()
+        self.batches = batches
         self._updates = {}
+        run = self._forward_all
         with torch.no_grad():
             side = torch.cuda.Stream()
             side.wait_stream(torch.cuda.current_stream())
             with torch.cuda.stream(side):
                 for _ in range(max(1, warmup)):          # also fills the layers' threshold caches
-                    self.model.forward(self.input)
+                    run()
             torch.cuda.current_stream().wait_stream(side)
             self._static = [_noise_state(m) for m in self.layers]
             self._thresh_args = [m._cache["thresh"][0][3:5] if "thresh" in m._cache else None for m in self.layers]
@@ -524,7 +533,12 @@ class CapturedForward:
                               getattr(m, "weight_noise_tap", None), m.bias_noise) for m in self.layers]
             self.graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(self.graph):
-                self.output = self.model.forward(self.input)
+                self.output = run()
+
+    def _forward_all(self):
+        if self.batches is None:
+            return self.model.forward(self.input)
+        return [self.model.forward(self.input[b]) for b in range(self.batches)]
 
     def forward(self, input=None):
         if input is not None:
@@ -591,6 +605,6 @@ class CapturedForward:
                     m.bias.grad = gb
 
 
-def capture(model, example_input, warmup=2):
+def capture(model, example_input, warmup=2, batches=None):
     """See :class:`CapturedForward`."""
-    return CapturedForward(model, example_input, warmup)
+    return CapturedForward(model, example_input, warmup, batches)

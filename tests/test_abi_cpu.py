@@ -76,6 +76,9 @@ def test_bad_arguments_are_rejected_without_a_launch(lib):
     assert lib.nb_grad_regularize(one, one, 0.1, 0.1, -1, None) == 2
     assert lib.nb_bias_grad(one, one, one, -1, 4, None) == 2
     assert lib.nb_bias_noise_scale(one, -1, None) == 2
+    # the linear layer's activation: more input bits than the rows hold
+    assert lib.nb_bmv_pm1_i64(one, one, one, 1, 1, 1, 65, None) == 2
+    assert lib.nb_bmv_pm1_i32(one, one, one, 1, 1, 2, 65, None) == 2
     # 16-bit draws: rows that are not whole words, a stream offset that is not a multiple of 8
     assert lib.nb_sample_philox16_i64(one, None, None, 5, 1, 0, 0, 2, 3, 70, None) == 4
     assert lib.nb_sample_philox16_i32(one, None, None, 5, 1, 0, 4, 2, 3, 64, None) == 4

@@ -297,3 +297,28 @@ def test_captured_forward_follows_the_eager_one(binary, kind):
                 assert torch.equal(l.weight.grad, gw), (it, type(l).__name__)
                 if gb is not None:
                     assert torch.equal(l.bias.grad, gb), (it, type(l).__name__)
+
+
+def test_captured_forward_over_several_batches(binary):
+    """binary.capture(batches=K): one replay evaluates K input batches on the same noise; every output equals the
+    eager forward of its batch, also after new noise and new inputs."""
+    D, K = 32, 5
+    g = torch.Generator(device="cuda")
+    g.manual_seed(3)
+    model = torch.nn.Sequential(binary.BinarizedLinear(256, 256, D, threshold=False, flip_probability=0.01))
+    randomise(model, 4)
+    pm = binary.PerturbedModel(model, D)
+    pm.set_seed(1)
+    pm.set_noise()
+    xs = torch.randint(0, 2, (K, D, 256), device="cuda", generator=g).bool()
+    cap = binary.capture(pm, xs, batches=K)
+    with torch.no_grad():
+        for it in range(3):
+            outs = [o.clone() for o in cap(xs)]
+            torch.cuda.synchronize()
+            assert len(outs) == K
+            for b in range(K):
+                assert torch.equal(outs[b], pm.forward(xs[b])), (it, b)
+            xs = torch.randint(0, 2, (K, D, 256), device="cuda", generator=g).bool()
+            pm.set_seed(10 + it)
+            cap.set_noise()

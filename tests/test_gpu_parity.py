@@ -503,6 +503,28 @@ def test_weighted_sum_vs_oracle(ops, oracle, dtype):
         np.testing.assert_array_equal(got, want.astype(np.float16).astype(np.float32))
 
 
+@pytest.mark.parametrize("dtype", [torch.int64, torch.int32])
+def test_bmv_pm1_is_the_linear_layers_activation(ops, oracle, dtype):
+    """bmv_pm1(A, x, K) == 2 * bmm(A, x) - K (modules/binary.py:97), on every matrix-vector kernel: rows of 16 / 32 /
+    64 bytes, long rows of whole 16-byte vectors, odd rows, unaligned word counts."""
+    nd = NDT[dtype]
+    wb = np.dtype(nd).itemsize * 8
+    g = rng(5)
+    for Z, M, Kw in [(5, 7, 64 // (wb // 8) // 4 or 1), (3, 256, 2), (4, 64, 4), (2, 8, 8), (3, 12, 32 * 64 // wb),
+                     (2, 16, 512 * 64 // wb), (3, 5, 3), (2, 9, 37), (1, 1, 1), (6, 1000, 16)]:
+        A = rand_words(g, (Z, M, Kw), nd)
+        x = rand_words(g, (Z, Kw), nd)
+        K = Kw * wb - 5 if Kw * wb > 5 else Kw * wb
+        want = 2 * oracle.bmm(A, x.reshape(Z, Kw, 1))[:, :, 0].astype(np.int64) - K
+        got = ops.bmv_pm1(dev(A), dev(x), K)
+        assert got.dtype == torch.int32 and tuple(got.shape) == (Z, M)
+        np.testing.assert_array_equal(host(got).astype(np.int64), want, err_msg=str((Z, M, Kw)))
+        # the plain product is untouched by the map
+        np.testing.assert_array_equal(host(ops.bmm(dev(A), dev(x).view(Z, Kw, 1)))[:, :, 0], oracle.bmm(A, x.reshape(Z, Kw, 1))[:, :, 0])
+    with pytest.raises(RuntimeError, match="does not fit"):
+        ops._lib.call("nb_bmv_pm1" + ("_i64" if wb == 64 else "_i32"), 8, 8, 8, 1, 1, 1, wb + 1, None)
+
+
 def _fp16_interval(exact, slack):
     """The fp16 values a correctly rounded result may take when `exact` is known to within `slack`."""
     with np.errstate(over="ignore"):
