@@ -296,6 +296,37 @@ __device__ __forceinline__ void transpose_bits_32x32(uint32_t (&a)[32])
     transpose_stage<1>(a);
 }
 
+// The 8 tables of a chunk of 64 members (tbl[g * 256 + byte] = sum of the weights of the members 8 g + j whose bit j
+// is set in byte), built by the wave that uses them.
+__device__ __forceinline__ void lut_build_tables(float *tbl, const uint16_t *wr, int64_t m0, int64_t n, int lane)
+{
+    // lane (g, s): group g of the chunk, the entries whose bits 2..4 are s; bits 0, 1, 5, 6 by doubling
+    const int g = lane >> 3, s = lane & 7;
+    float wj[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        const int64_t m = m0 + 8 * g + j;
+        wj[j] = m < n ? (float)__builtin_bit_cast(_Float16, wr[m]) : 0.f;
+    }
+    // 16 entries at a time (bit 7 clear, then set) to keep the registers for the members' words
+    float e[16];
+    e[0] = ((s & 1) ? wj[2] : 0.f) + ((s & 2) ? wj[3] : 0.f) + ((s & 4) ? wj[4] : 0.f);
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const float wk = wj[k < 2 ? k : k + 3];
+#pragma unroll
+        for (int t = 0; t < (1 << k); t++) e[t + (1 << k)] = e[t] + wk;
+    }
+    // register index = (bits 5, 6) << 2 | bits 0..1: the eight lanes of a group write 128 contiguous bytes
+    float4 *dst = reinterpret_cast<float4 *>(tbl + g * 256 + 4 * s);
+#pragma unroll
+    for (int i = 0; i < 4; i++) dst[8 * i] = make_float4(e[4 * i], e[4 * i + 1], e[4 * i + 2], e[4 * i + 3]);
+#pragma unroll
+    for (int t = 0; t < 16; t++) e[t] += wj[7];
+#pragma unroll
+    for (int i = 0; i < 4; i++) dst[8 * (i + 4)] = make_float4(e[4 * i], e[4 * i + 1], e[4 * i + 2], e[4 * i + 3]);
+}
+
 template <int SPLIT>
 __global__ __launch_bounds__(1024) void weighted_sum_lut_kernel(_Float16 *__restrict__ ret,
                                                                  const uint32_t *__restrict__ in,
@@ -331,34 +362,7 @@ __global__ __launch_bounds__(1024) void weighted_sum_lut_kernel(_Float16 *__rest
                 a[j] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)qoff, (int)(j * (uint32_t)Q * 4u), 2);
         };
         fetch(m0);
-        {
-            // lane (g, s): group g of the chunk, the entries whose bits 2..4 are s; bits 0, 1, 5, 6 by doubling
-            const int g = lane >> 3, s = lane & 7;
-            float wj[8];
-#pragma unroll
-            for (int j = 0; j < 8; j++) {
-                const int64_t m = m0 + 8 * g + j;
-                wj[j] = m < n ? (float)__builtin_bit_cast(_Float16, wr[m]) : 0.f;
-            }
-            // 16 entries at a time (bit 7 clear, then set) to keep the registers for the members' words
-            float e[16];
-            e[0] = ((s & 1) ? wj[2] : 0.f) + ((s & 2) ? wj[3] : 0.f) + ((s & 4) ? wj[4] : 0.f);
-#pragma unroll
-            for (int k = 0; k < 4; k++) {
-                const float wk = wj[k < 2 ? k : k + 3];
-#pragma unroll
-                for (int t = 0; t < (1 << k); t++) e[t + (1 << k)] = e[t] + wk;
-            }
-            // register index = (bits 5, 6) << 2 | bits 0..1: the eight lanes of a group write 128 contiguous bytes
-            float4 *dst = reinterpret_cast<float4 *>(tbl + g * 256 + 4 * s);
-#pragma unroll
-            for (int i = 0; i < 4; i++) dst[8 * i] = make_float4(e[4 * i], e[4 * i + 1], e[4 * i + 2], e[4 * i + 3]);
-#pragma unroll
-            for (int t = 0; t < 16; t++) e[t] += wj[7];
-#pragma unroll
-            for (int i = 0; i < 4; i++)
-                dst[8 * (i + 4)] = make_float4(e[4 * i], e[4 * i + 1], e[4 * i + 2], e[4 * i + 3]);
-        }
+        lut_build_tables(tbl, wr, m0, n, lane);
         // the tables are read by other lanes of this wave only: LDS accesses of a wave are served in order
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
@@ -438,6 +442,93 @@ __global__ __launch_bounds__(1024) void weighted_sum_lut_kernel(_Float16 *__rest
     }
 }
 
+// The same for small outputs: a wave takes 32 columns and its two halves take the two blocks of 32 members of a
+// chunk, so that twice as many waves share the work (a small layer's sum is bound by the pace of one wave over its
+// chunk, not by the machine).  Lane = (half h, column): members m0 + 32 h .., tables 4 h .. 4 h + 3; the halves are two
+// more shares in the final addition.
+template <int SPLIT>
+__global__ __launch_bounds__(1024) void weighted_sum_lut_half_kernel(_Float16 *__restrict__ ret,
+                                                                      const uint32_t *__restrict__ in,
+                                                                      const _Float16 *__restrict__ w, int64_t n, int64_t Q,
+                                                                      int rowdw, int zbits, int whole_rows)
+{
+    extern __shared__ __align__(16) float lds[];
+    constexpr int SHARES = 1 << SPLIT, SETS = 16 >> SPLIT;
+    const int lane = threadIdx.x & 63, hb = lane >> 5;
+    const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int ms = wv & (SHARES - 1), cs = wv >> SPLIT;
+    const int64_t q = ((int64_t)blockIdx.x * SETS + cs) * 32 + (lane & 31);
+    float *tbl = lds + wv * 2048;
+    const float *mine = tbl + hb * 1024;
+    const uint16_t *wr = reinterpret_cast<const uint16_t *>(w);
+    float acc[32];
+#pragma unroll
+    for (int k = 0; k < 32; k++) acc[k] = 0.f;
+    const int64_t nchunks = (n + 63) >> 6;
+    // the lane's column and its half's first member of a chunk, as one byte offset into the chunk's buffer
+    const uint32_t off = (uint32_t)(q < Q ? q : Q - 1) * 4u + (uint32_t)hb * 32u * (uint32_t)Q * 4u;
+    for (int64_t c = ms; c < nchunks; c += SHARES) {
+        const int64_t m0 = c * 64;
+        uint32_t a[32];
+        const int64_t left = n - m0;
+        // one buffer per chunk that ends with the last member: members past n read as zero words
+        const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<uint32_t *>(in + m0 * Q), (short)0, (int)((left < 64 ? left : 64) * Q * 4), 0x00020000);
+#pragma unroll
+        for (int j = 0; j < 32; j++)
+            a[j] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)off, (int)(j * (uint32_t)Q * 4u), 2);
+        lut_build_tables(tbl, wr, m0, n, lane);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        transpose_bits_32x32(a);
+#pragma unroll
+        for (int k = 0; k < 32; k++) {
+            const float t0 = mine[0 * 256 + (a[k] & 255u)];
+            const float t1 = mine[1 * 256 + ((a[k] >> 8) & 255u)];
+            const float t2 = mine[2 * 256 + ((a[k] >> 16) & 255u)];
+            const float t3 = mine[3 * 256 + (a[k] >> 24)];
+            acc[k] += (t0 + t1) + (t2 + t3);
+            if ((k & 3) == 3) __builtin_amdgcn_sched_barrier(0);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+    }
+    __syncthreads();  // every wave is done with its tables
+#pragma unroll
+    for (int k = 0; k < 32; k++) lds[(wv * 64 + lane) * kLutRedStride + k] = acc[k];
+    __syncthreads();
+    // thread t < 512 adds the 2 * SHARES partial sums of 32 / SHARES consecutive output bits of one column
+    constexpr int KP = 32 >> SPLIT;
+    const int col = threadIdx.x >> SPLIT, part = threadIdx.x & (SHARES - 1);
+    const int cs2 = col >> 5, l2 = col & 31;
+    const int64_t q2 = ((int64_t)blockIdx.x * SETS + cs2) * 32 + l2;
+    if (col >= SETS * 32 || q2 >= Q) return;
+    float sum[KP];
+#pragma unroll
+    for (int i = 0; i < KP; i++) sum[i] = 0.f;
+#pragma unroll
+    for (int m = 0; m < SHARES; m++)
+#pragma unroll
+        for (int h = 0; h < 2; h++)
+#pragma unroll
+            for (int i = 0; i < KP; i++)
+                sum[i] += lds[(((cs2 << SPLIT) + m) * 64 + h * 32 + l2) * kLutRedStride + part * KP + i];
+    const int64_t r = q2 / rowdw;
+    const int z0 = (int)(q2 - r * rowdw) * 32 + part * KP;
+    if (whole_rows) {
+        uint32_t *o = reinterpret_cast<uint32_t *>(ret + q2 * 32 + part * KP);
+#pragma unroll
+        for (int i = 0; i < KP; i += 2)
+            o[i >> 1] = (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)sum[i]) |
+                        ((uint32_t)__builtin_bit_cast(uint16_t, (_Float16)sum[i + 1]) << 16);
+    } else {
+#pragma unroll
+        for (int i = 0; i < KP; i++)
+            if (z0 + i < zbits) ret[r * zbits + z0 + i] = (_Float16)sum[i];
+    }
+}
+
 template <typename W>
 int weighted_sum_fast_impl(uint16_t *ret, const W *in, const uint16_t *w, int64_t n, int64_t R, int64_t Rw,
                            int64_t zbits, nb_stream_t stream, const char *who)
@@ -467,14 +558,19 @@ int weighted_sum_fast_impl(uint16_t *ret, const W *in, const uint16_t *w, int64_
     const int whole = zbits == rowdw * 32 && aligned(ret, 16);
     const int64_t blocks = ceil_div(sets, 16 >> split);
     NB_REQUIRE(blocks <= kMaxGridX, "%s: output exceeds one launch", who);
+    // small outputs: 32 columns per wave, the wave's halves on the two blocks of a chunk (twice the waves)
+    bool halves = split == 4 && (sets << split) < 2048 && nchunks >= 1 && Q < (1LL << 23);
+    if (const char *v = getenv("NESBIN_WSUM_HALVES")) halves = atoi(v) != 0 && split >= 3 && Q < (1LL << 23);
     static std::once_flag once;
     static hipError_t attr = hipSuccess;
     std::call_once(once, [] {
-        const void *fns[5] = {reinterpret_cast<const void *>(weighted_sum_lut_kernel<0>),
+        const void *fns[7] = {reinterpret_cast<const void *>(weighted_sum_lut_kernel<0>),
                               reinterpret_cast<const void *>(weighted_sum_lut_kernel<1>),
                               reinterpret_cast<const void *>(weighted_sum_lut_kernel<2>),
                               reinterpret_cast<const void *>(weighted_sum_lut_kernel<3>),
-                              reinterpret_cast<const void *>(weighted_sum_lut_kernel<4>)};
+                              reinterpret_cast<const void *>(weighted_sum_lut_kernel<4>),
+                              reinterpret_cast<const void *>(weighted_sum_lut_half_kernel<3>),
+                              reinterpret_cast<const void *>(weighted_sum_lut_half_kernel<4>)};
         for (const void *f : fns) {
             const hipError_t e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, kLutLdsBytes);
             if (e != hipSuccess) attr = e;
@@ -484,11 +580,17 @@ int weighted_sum_fast_impl(uint16_t *ret, const W *in, const uint16_t *w, int64_
         (void)hipGetLastError();
         return fail(NB_ERR_UNSUPPORTED, "%s: cannot raise the kernel's LDS limit: %s", who, hipGetErrorString(attr));
     }
+    const int64_t nblocks = halves ? ceil_div(ceil_div(Q, 32), 16 >> split) : blocks;
     auto launch = [&](auto kern) {
-        kern<<<dim3((unsigned)blocks), dim3(1024), kLutLdsBytes, as_stream(stream)>>>(
+        kern<<<dim3((unsigned)nblocks), dim3(1024), kLutLdsBytes, as_stream(stream)>>>(
             reinterpret_cast<_Float16 *>(ret), reinterpret_cast<const uint32_t *>(in),
             reinterpret_cast<const _Float16 *>(w), n, Q, (int)rowdw, (int)zbits, whole);
     };
+    if (halves) {
+        if (split == 3) launch(weighted_sum_lut_half_kernel<3>);
+        else launch(weighted_sum_lut_half_kernel<4>);
+        return check_launch(who);
+    }
     switch (split) {
         case 0: launch(weighted_sum_lut_kernel<0>); break;
         case 1: launch(weighted_sum_lut_kernel<1>); break;

@@ -3,6 +3,8 @@ include/nesbin.h), against the committed golden fixtures and the CPU oracle on t
 Integer / bit results must match exactly."""
 import itertools
 
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -543,10 +545,17 @@ def test_weighted_sum_fast_mode_within_fp16_rounding_of_the_exact_sum(ops, dtype
     for n, R, C in [(1024, 64, 1024), (1000, 7, 200), (64, 3, 256), (65, 2, 330), (33, 5, 100), (32, 4, 64),
                     (31, 1, 31), (1, 1, 1), (200, 9, 576), (130, 700, 64), (257, 1, 1024), (2100, 3, 96),
                     (96, 1300, 128), (70, 16, 2048), (40, 4200, 64), (512, 300, 1152), (0, 3, 100), (5, 2, 40)]:
-        for extra in (0, 1):  # rows with a word that holds no output bit
-            words = rand_words(g, (n, R, (C + wb - 1) // wb + extra), nd)
+        for extra in (0, 1, 2):  # rows with a word that holds no output bit; 2: the other kernel for small outputs
+            words = rand_words(g, (n, R, (C + wb - 1) // wb + (extra & 1)), nd)
             w = (g.standard_normal(n) * (3.0 if n % 2 else 0.05)).astype(np.float16)
-            got = host(ops.weighted_sum(dev(words), dev(w), C, fast=True)).astype(np.float64)
+            if extra == 2:      # force / forbid the kernel whose waves split into two member halves
+                os.environ["NESBIN_WSUM_HALVES"] = "0" if n >= 961 else "1"
+                os.environ["NESBIN_WSUM_SPLIT"] = "4" if n % 2 else "3"
+            try:
+                got = host(ops.weighted_sum(dev(words), dev(w), C, fast=True)).astype(np.float64)
+            finally:
+                os.environ.pop("NESBIN_WSUM_HALVES", None)
+                os.environ.pop("NESBIN_WSUM_SPLIT", None)
             bits = np.unpackbits(np.ascontiguousarray(words).view(np.uint8), axis=-1, bitorder="little")[:, :, :C]
             exact = np.einsum("m,mrc->rc", w.astype(np.float64), bits.astype(np.float64))
             lo, hi = _fp16_interval(exact, 1e-6 * float(np.abs(w.astype(np.float64)).sum()) + 1e-30)
