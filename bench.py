@@ -445,6 +445,14 @@ def hbm_kernels(torch, steps, warmup, graph=True, core=False):
         lambda: ops.sample_bits_philox(workloads.T_P01, 4096, torch.int64, 0, 11, base=bc, shape=(1152, 64), conv_taps=9),
         2 * 4096 * 1152 * 8)
     del bc
+    # a layer's set_noise from the generator, per-element thresholds: conv 64 -> 256 (3x3) for 1024 members, one 32-bit
+    # draw per weight bit against 16-bit draws (two per generated word)
+    thr = torch.randint(0, 2 ** 31, (2304, 64), device=dev, generator=g, dtype=torch.int64).to(torch.int32).view(torch.uint32)
+    for half in (False, True):
+        run("sample_bits_philox D=1024 x [2304 rows x 64], per-element thresholds, %s (bytes written)"
+            % ("16-bit draws" if half else "32-bit draws"),
+            lambda: ops.sample_bits_philox(thr, 1024, torch.int64, 0, 12, half_draws=half), 1024 * 2304 * 8)
+    del thr
     # first-layer filters of an RGB network: rows of 3 columns, one lane per row
     b1 = torch.randint(0, 8, (576, 1), device=dev, generator=g, dtype=torch.int64)
     run("sample (3-column rows) D=4096 x 576 rows, generator mode",
