@@ -571,6 +571,14 @@ def main():
                                       "generated word (a Philox round is two v_mad_u64_u32 and two v_bitop3_b32), "
                                       "so the vector ALUs are the limit, not HBM"}
     del wg
+    # the same with 16 bits of the stream per weight bit (two per generated word; ties decided by a second stream)
+    wh = workloads.linear_flip_generated(half_draws=True)
+    ph, _ = time_steps(torch, wh.step, max(3, args.steps // 4), 1)
+    line["generator_mode"]["half_draws"] = {
+        "workload": wh.name, "ms_per_step": round(ph * 1e3, 4), "binary_TOPS": round(2 * wh.bit_macs / ph / 1e12, 3),
+        "note": "same law (every bit flips with probability exactly T / 2^32, independently), other bits than the "
+                "headline workload"}
+    del wh
     if not args.no_step:
         # the layer API end to end: one NES step of a SmallNet-shaped network (population 1024), phase by phase
         sn, fw, up = workloads.small_net_step()

@@ -428,6 +428,14 @@ int nb_seeded_bmv_philox_i64(int32_t *C, const int64_t *base, const uint32_t *th
 int nb_seeded_bmv_philox_i32(int32_t *C, const int32_t *base, const uint32_t *thresh, uint32_t thr_scalar,
                              const int32_t *x, uint64_t seed, uint64_t subseq, uint64_t first, int64_t n, int64_t R,
                              int64_t Cbits, nb_stream_t stream);
+/* The same product over the 16-bit draws of nb_sample_philox16 (C[m,r] = what nb_bmm gives on nb_sample_philox16's
+ * output and x): needs Cbits % 8 == 0, first % 8 == 0 and 16-byte aligned thresholds, NB_ERR_UNSUPPORTED otherwise. */
+int nb_seeded_bmv_philox16_i64(int32_t *C, const int64_t *base, const uint32_t *thresh, uint32_t thr_scalar,
+                               const int64_t *x, uint64_t seed, uint64_t subseq, uint64_t first, int64_t n, int64_t R,
+                               int64_t Cbits, nb_stream_t stream);
+int nb_seeded_bmv_philox16_i32(int32_t *C, const int32_t *base, const uint32_t *thresh, uint32_t thr_scalar,
+                               const int32_t *x, uint64_t seed, uint64_t subseq, uint64_t first, int64_t n, int64_t R,
+                               int64_t Cbits, nb_stream_t stream);
 
 /* ---- weighted sum of packed masks (update step) ---------------------------------------------------
  * ret[r,z] = fp16( sum_m float(w[m]) * bit(in[m,r,z/bits], z%bits) ), fp32 accumulation in member

@@ -43,6 +43,7 @@ _SUFFIXED = {
     "nb_sample_conv_philox": [_PTR, _PTR, _PTR, _PTR, _U32, _U64, _U64, _U64, _I64, _I64, _I64, _I64, _PTR],
     "nb_seeded_bmv_from_words": [_PTR, _PTR, _PTR, _U32, _PTR, _PTR, _I64, _I64, _I64, _PTR],
     "nb_seeded_bmv_philox": [_PTR, _PTR, _PTR, _U32, _PTR, _U64, _U64, _U64, _I64, _I64, _I64, _PTR],
+    "nb_seeded_bmv_philox16": [_PTR, _PTR, _PTR, _U32, _PTR, _U64, _U64, _U64, _I64, _I64, _I64, _PTR],
     "nb_sample_skip": [_PTR, _PTR, _PTR, _U64, _U64, _U64, _I64, _I64, _I64, _PTR],
     "nb_sample_conv_skip": [_PTR, _PTR, _PTR, _PTR, _U64, _U64, _U64, _I64, _I64, _I64, _I64, _PTR],
     "nb_weighted_sum": [_PTR, _PTR, _PTR, _I64, _I64, _I64, _I64, _PTR],

@@ -680,6 +680,103 @@ int sample16_impl(W *out, const W *base, const uint32_t *thresh, uint32_t ts, Ph
     return check_launch(who);
 }
 
+// ---- fused sample + XOR-popcount with 16-bit draws -----------------------------------------------------------------
+// C[m, r] = sum_k popcount(w(m, r, k) ^ x[m, k]) with w what sample_word_philox16_kernel would have written.  A wave
+// takes RPW rows of one member (they share the member's input bytes); a lane takes 8 columns per step, i.e. one
+// generator block per row: eight borrow/shift pairs, an XOR with the byte of base ^ x, one v_bcnt.  Needs C % 8 == 0
+// and first % 8 == 0 (blocks do not straddle rows), thresholds 16-byte aligned.
+template <typename W, int RPW, bool HAS_THR, bool HAS_BASE>
+__global__ __launch_bounds__(256) void seeded_bmv_philox16_kernel(int32_t *__restrict__ Cout, const W *__restrict__ base,
+                                                                  const uint32_t *__restrict__ thresh, uint32_t ts,
+                                                                  const W *__restrict__ x, PhiloxKey key, int64_t n,
+                                                                  int R, int C8, int Rw, int groups_per_member)
+{
+    constexpr int bits = WordTraits<W>::bits;
+    constexpr int BPW = bits / 8;  // bytes (blocks of 8 columns) per word
+    const int lane = threadIdx.x & 63;
+    const int64_t wave = (int64_t)blockIdx.x * 4 + __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int64_t m = wave / groups_per_member;
+    if (m >= n) return;
+    const int r0 = (int)(wave - m * groups_per_member) * RPW;
+    int rows[RPW];
+#pragma unroll
+    for (int q = 0; q < RPW; q++) rows[q] = r0 + q < R ? r0 + q : R - 1;  // tail rows are recomputed, not stored
+    int acc[RPW];
+#pragma unroll
+    for (int q = 0; q < RPW; q++) acc[q] = 0;
+    const uint64_t blk0 = key.first >> 3;
+    // every lane runs the same number of steps (the tie test below is a wave-wide vote); lanes past the row's end
+    // compute on the last block and add nothing
+    for (int c0 = 0; c0 < C8; c0 += 64) {
+        const bool live = c0 + lane < C8;
+        const int c8 = live ? c0 + lane : C8 - 1;
+        const int wi = c8 / BPW, sh = 8 * (c8 - wi * BPW);
+        const W xw = x[m * Rw + wi];
+#pragma unroll
+        for (int q = 0; q < RPW; q++) {
+            const int r = rows[q];
+            const uint32_t bx = (uint32_t)((HAS_BASE ? (W)(xw ^ base[(int64_t)r * Rw + wi]) : xw) >> sh) & 0xFFu;
+            const uint4 *tq = reinterpret_cast<const uint4 *>(thresh + ((int64_t)r * C8 + c8) * 8);
+            const uint4 ta = HAS_THR ? tq[0] : make_uint4(ts, ts, ts, ts);
+            const uint4 tb = HAS_THR ? tq[1] : ta;
+            const uint4 ha = make_uint4(ta.x & 0xFFFF0000u, ta.y & 0xFFFF0000u, ta.z & 0xFFFF0000u, ta.w & 0xFFFF0000u);
+            const uint4 hb = make_uint4(tb.x & 0xFFFF0000u, tb.y & 0xFFFF0000u, tb.z & 0xFFFF0000u, tb.w & 0xFFFF0000u);
+            const uint64_t b = blk0 + (uint64_t)((m * R + r) * C8 + c8);
+            const uint4 w = philox_block(key, b);
+            uint32_t zmin = 0xFFFFFFFFu;
+            uint32_t byte = byte_lt16(w, ha, hb, zmin);
+            if (__any(zmin < 65536u)) {
+                if (zmin < 65536u) byte = byte_ties16(byte, w, ta, tb, key, b << 3);
+            }
+            acc[q] += live ? __popc(byte ^ bx) : 0;
+        }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+#pragma unroll
+        for (int q = 0; q < RPW; q++) acc[q] += __shfl_xor(acc[q], off);
+    }
+    if (lane == 0) {
+#pragma unroll
+        for (int q = 0; q < RPW; q++)
+            if (r0 + q < R) Cout[m * R + r0 + q] = acc[q];
+    }
+}
+
+template <typename W>
+int seeded_bmv16_impl(int32_t *Cout, const W *base, const uint32_t *thresh, uint32_t ts, const W *x, PhiloxKey key,
+                      int64_t n, int64_t R, int64_t C, nb_stream_t stream, const char *who)
+{
+    constexpr int bits = WordTraits<W>::bits;
+    NB_REQUIRE(n >= 0 && R >= 0 && C >= 0, "%s: negative shape n=%lld R=%lld C=%lld", who, (long long)n, (long long)R,
+               (long long)C);
+    if (n * R == 0) return NB_OK;
+    NB_REQUIRE_PTR(Cout);
+    NB_REQUIRE_ALIGNED(Cout, 4);
+    NB_REQUIRE(C > 0 && C <= (1 << 30) && R < (1LL << 31), "%s: C=%lld, R=%lld out of range", who, (long long)C, (long long)R);
+    NB_REQUIRE_PTR(x);
+    NB_REQUIRE_ALIGNED(x, sizeof(W));
+    if (base) NB_REQUIRE_ALIGNED(base, sizeof(W));
+    if (C % 8 != 0 || (key.first & 7) != 0 || (thresh && !aligned(thresh, 16)))
+        return fail(NB_ERR_UNSUPPORTED,
+                    "%s: 16-bit draws take C %% 8 == 0, first %% 8 == 0 and 16-byte aligned thresholds", who);
+    constexpr int RPW = 4;
+    const int64_t gpm = ceil_div(R, RPW), waves = n * gpm;
+    NB_REQUIRE(ceil_div(waves, 4) <= kMaxGridX, "%s: n*R=%lld rows exceed one launch", who, (long long)(n * R));
+    const dim3 grid((unsigned)ceil_div(waves, 4)), block(256);
+    const int Rw = (int)ceil_div(C, bits);
+    hipStream_t s = as_stream(stream);
+#define NB_LAUNCH16(T, B)                                                                                              \
+    seeded_bmv_philox16_kernel<W, RPW, T, B><<<grid, block, 0, s>>>(Cout, base, thresh, ts, x, key, n, (int)R, (int)(C / 8), \
+                                                                    Rw, (int)gpm)
+    if (thresh && base) NB_LAUNCH16(true, true);
+    else if (thresh) NB_LAUNCH16(true, false);
+    else if (base) NB_LAUNCH16(false, true);
+    else NB_LAUNCH16(false, false);
+#undef NB_LAUNCH16
+    return check_launch(who);
+}
+
 template <typename W, class Src>
 int seeded_bmv_impl(int32_t *Cout, const W *base, const uint32_t *thresh, uint32_t ts, const W *x, Src src,
                     bool src_vec_ok, int64_t n, int64_t R, int64_t C, nb_stream_t stream, const char *who)
@@ -877,6 +974,20 @@ int nb_seeded_bmv_from_words_i32(int32_t *C, const int32_t *base, const uint32_t
     return nb::seeded_bmv_impl<uint32_t, WordsSrc>(C, CU32(base), thresh, ts, CU32(x), WordsSrc{words},
                                                    nb::aligned(words, 16), n, R, Cbits, s,
                                                    "nb_seeded_bmv_from_words_i32");
+}
+int nb_seeded_bmv_philox16_i64(int32_t *C, const int64_t *base, const uint32_t *thresh, uint32_t ts, const int64_t *x,
+                               uint64_t seed, uint64_t subseq, uint64_t first, int64_t n, int64_t R, int64_t Cbits,
+                               nb_stream_t s)
+{
+    return nb::seeded_bmv16_impl<uint64_t>(C, CU64(base), thresh, ts, CU64(x), nb::PhiloxKey{seed, subseq, first}, n, R,
+                                           Cbits, s, "nb_seeded_bmv_philox16_i64");
+}
+int nb_seeded_bmv_philox16_i32(int32_t *C, const int32_t *base, const uint32_t *thresh, uint32_t ts, const int32_t *x,
+                               uint64_t seed, uint64_t subseq, uint64_t first, int64_t n, int64_t R, int64_t Cbits,
+                               nb_stream_t s)
+{
+    return nb::seeded_bmv16_impl<uint32_t>(C, CU32(base), thresh, ts, CU32(x), nb::PhiloxKey{seed, subseq, first}, n, R,
+                                           Cbits, s, "nb_seeded_bmv_philox16_i32");
 }
 int nb_seeded_bmv_philox_i64(int32_t *C, const int64_t *base, const uint32_t *thresh, uint32_t ts, const int64_t *x,
                              uint64_t seed, uint64_t subseq, uint64_t first, int64_t n, int64_t R, int64_t Cbits,

@@ -775,8 +775,10 @@ def seeded_bmv_from_words(threshold, x_packed, words, base=None):
     return out
 
 
-def seeded_bmv_philox(threshold, x_packed, rows, in_bits, seed, subsequence=0, first=0, base=None):
-    """:func:`seeded_bmv_from_words` with in-kernel Philox words."""
+def seeded_bmv_philox(threshold, x_packed, rows, in_bits, seed, subsequence=0, first=0, base=None, half_draws=False):
+    """:func:`seeded_bmv_from_words` with in-kernel Philox words.  ``half_draws=True``: the 16-bit draws of
+    :func:`sample_bits_philox` (``in_bits`` and ``first`` multiples of 8): the product over exactly the weights that
+    ``sample_bits_philox(..., half_draws=True)`` writes."""
     _check(x_packed, "x_packed")
     suf, bits = _suffix(x_packed.dtype)
     n = x_packed.size(0)
@@ -787,8 +789,9 @@ def seeded_bmv_philox(threshold, x_packed, rows, in_bits, seed, subsequence=0, f
     bptr = _base_check(base, R, Rw, x_packed.dtype, x_packed.device)
     out = torch.empty((n, R), dtype=torch.int32, device=x_packed.device)
     with _on(x_packed):
-        _lib.call("nb_seeded_bmv_philox" + suf, out.data_ptr(), bptr, tptr, ts, x_packed.data_ptr(),
-                  int(seed) & (2 ** 64 - 1), int(subsequence), int(first), n, R, C, _stream(x_packed))
+        _lib.call("nb_seeded_bmv_philox" + ("16" if half_draws else "") + suf, out.data_ptr(), bptr, tptr, ts,
+                  x_packed.data_ptr(), int(seed) & (2 ** 64 - 1), int(subsequence), int(first), n, R, C,
+                  _stream(x_packed))
     return out
 
 

@@ -88,20 +88,25 @@ def linear_flip_fused(D=1024, out_f=1024, in_f=1024, T=T_P05, seed=0, dtype=torc
     return w
 
 
-def linear_flip_generated(D=1024, out_f=1024, in_f=1024, T=T_P05, seed=0, dtype=torch.int64, device="cuda"):
+def linear_flip_generated(D=1024, out_f=1024, in_f=1024, T=T_P05, seed=0, dtype=torch.int64, device="cuda",
+                          half_draws=False):
     """Config 2 in generator mode: the same product with the random words produced inside the kernel by
     Philox4x32-10 (seed, subsequence 2) instead of being read: no 4 GiB operand, the generator's arithmetic is the
-    limit.  Bit for bit the same output as :func:`linear_flip_fused` (same stream)."""
+    limit.  Bit for bit the same output as :func:`linear_flip_fused` (same stream).  ``half_draws``: 16 bits of the
+    stream per weight bit (same law, other bits: the output then equals the product over
+    ``sample_bits_philox(..., half_draws=True)``'s weights)."""
     g = _gen(seed)
     base_bits = _bits(g, (out_f, in_f))
     x_bits = _bits(g, (D, in_f))
     base = ops.pack(base_bits.to(device), dtype)
     x = ops.pack(x_bits.to(device), dtype)
     return Workload(
-        name="linear %dx%d D=%d N=1 p=0.05 flips from in-kernel Philox words, fused" % (out_f, in_f, D),
+        name="linear %dx%d D=%d N=1 p=0.05 flips from in-kernel Philox %s, fused"
+             % (out_f, in_f, D, "half-words (16-bit draws)" if half_draws else "words"),
         population=D, bit_macs=D * out_f * in_f,
         algo_bytes=base.numel() * base.element_size() + x.numel() * x.element_size() + D * out_f * 4,
-        bound="generator", step=lambda: ops.seeded_bmv_philox(T, x, out_f, in_f, seed, subsequence=2, base=base),
+        bound="generator", step=lambda: ops.seeded_bmv_philox(T, x, out_f, in_f, seed, subsequence=2, base=base,
+                                                              half_draws=half_draws),
         tensors=dict(base=base, x=x), meta=dict(T=T, seed=seed, subsequence=2, in_f=in_f, out_f=out_f))
 
 

@@ -479,6 +479,46 @@ def test_sampler_from_half_word_draws_vs_oracle(ops, oracle, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.int64, torch.int32])
+def test_fused_product_over_half_word_draws_vs_oracle(ops, oracle, dtype):
+    """seeded_bmv_philox(half_draws=True) == bmm of the weights the oracle's 16-bit draws give, also for rows that are
+    whole bytes but not whole words, with ties forced for one member, and == bmm on what the sampler itself writes."""
+    nd = NDT[dtype]
+    wb = np.dtype(nd).itemsize * 8
+    g = rng(43)
+    for n, R, C, first in [(3, 5, 2 * wb, 0), (5, 9, 1024, 8), (2, 7, wb + 8, 0), (4, 130, 520, 16), (1, 1, 8, 0), (70, 3, 4096, 0)]:
+        seed, sub = 77 + n, 2
+        Rw = (C + wb - 1) // wb
+        base = rand_words(g, (R, Rw), nd)
+        x = rand_words(g, (n, Rw), nd)
+        if C % wb:                                       # tail bits are zero on every operand
+            keep = np.array((1 << (C % wb)) - 1).astype(np.uint64).astype(np.dtype("u%d" % (wb // 8))).view(nd)
+            base[:, -1] &= keep
+            x[:, -1] &= keep
+        P = 10.0 ** (-4 * g.random((R, C)))
+        T = np.minimum(np.floor(P * 2.0 ** 32), 2.0 ** 32 - 1).astype(np.uint32)
+        if n > 1:                                        # member 1 ties in every third column
+            gi = first + R * C + np.arange(R * C, dtype=np.uint64)
+            w1 = oracle.philox_words(seed, sub, int(gi[0]) // 2, R * C // 2 + 2)
+            w = w1[((gi >> np.uint64(1)) - np.uint64(int(gi[0]) // 2)).astype(np.int64)]
+            h = np.where(gi & np.uint64(1), w >> np.uint32(16), w & np.uint32(0xFFFF)).astype(np.uint32).reshape(R, C)
+            tie = np.arange(C) % 3 == 0
+            T[:, tie] = (h[:, tie] << np.uint32(16)) | (T[:, tie] & np.uint32(0xFFFF))
+        Td = torch.from_numpy(T.view(np.int32)).cuda().view(torch.uint32)
+        W = oracle.sample_philox16(T, n, R, C, seed, sub, first, nd, base=base)
+        want = oracle.bmm(W, x.reshape(n, Rw, 1))[:, :, 0]
+        got = ops.seeded_bmv_philox(Td, dev(x), R, C, seed, sub, first, base=dev(base), half_draws=True)
+        np.testing.assert_array_equal(host(got), want, err_msg=str((n, R, C, first)))
+        Ws = oracle.sample_philox16(0x10000001, n, R, C, seed, sub, first, nd)
+        got_s = ops.seeded_bmv_philox(0x10000001, dev(x), R, C, seed, sub, first, half_draws=True)
+        np.testing.assert_array_equal(host(got_s), oracle.bmm(Ws, x.reshape(n, Rw, 1))[:, :, 0])
+        if C % wb == 0:
+            Wg = ops.sample_bits_philox(Td, n, dtype, seed, sub, first, base=dev(base), half_draws=True)
+            assert torch.equal(ops.bmm(Wg, dev(x).view(n, Rw, 1)).squeeze(2), got)
+    with pytest.raises(RuntimeError, match="16-bit draws"):
+        ops.seeded_bmv_philox(5, dev(rand_words(g, (2, 1), nd)), 3, 12, 1, half_draws=True)
+
+
+@pytest.mark.parametrize("dtype", [torch.int64, torch.int32])
 def test_weighted_sum_vs_oracle(ops, oracle, dtype):
     g = rng(21)
     # the second line: rows that are whole 32-byte pieces (a wave per piece), also with fewer output bits than the
