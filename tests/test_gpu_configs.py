@@ -75,6 +75,25 @@ def test_config2_linear_1024_fused_from_words(wk, ops, oracle):
     assert abs(rate - 0.05) < 5e-4
 
 
+def test_config2_generator_mode_with_half_word_draws(wk, ops, oracle):
+    """Configuration 2 with 16-bit draws: the fused product equals bmm on what the sampler writes from the same
+    stream, over the whole population; members regenerated on the host; the flip rate."""
+    w = wk.linear_flip_generated(half_draws=True)
+    out = w.step()
+    assert tuple(out.shape) == (1024, 1024) and out.dtype == torch.int32
+    base, x = w.tensors["base"], w.tensors["x"]
+    W = ops.sample_bits_philox(wk.T_P05, 1024, torch.int64, 0, 2, base=base, shape=(1024, 1024), half_draws=True)
+    assert torch.equal(ops.bmm(W, x.view(1024, -1, 1)).squeeze(2), out)
+    bh, xh = base.cpu().numpy(), x.cpu().numpy()
+    for m in MEMBERS:
+        Wm = oracle.sample_philox16(wk.T_P05, 1, 1024, 1024, 0, 2, m * 1024 * 1024, np.int64, base=bh)
+        np.testing.assert_array_equal(W[m].cpu().numpy(), Wm[0])
+        np.testing.assert_array_equal(out[m].cpu().numpy(), oracle.bmm(Wm, xh[m:m + 1].reshape(1, -1, 1))[0, :, 0])
+    rate = ops.unpack((W[:64] ^ base).view(-1, 16)).float().mean().item()
+    assert abs(rate - 0.05) < 2e-4
+    assert not torch.equal(out, wk.linear_flip_generated().step())          # other bits than the 32-bit draws
+
+
 def test_config3_conv_64_int32(wk, ops, oracle):
     w = wk.conv_int32()
     out = w.step()
