@@ -156,7 +156,9 @@ int nb_conv_bn_thresholds_from_input_i32(int32_t *thresh, const int32_t *in, con
  *
  * Flip lists ("fixed slices"): with S = ceil(R / 64) and a capacity of `cap` 16-byte pieces per row, piece j of row
  * r of member d sits at dword offset (((d * S + r / 64) * cap + j) * 64 + r % 64) * 4 of entries (16-byte aligned,
- * D * S * cap * 256 dwords): the row's flips 8j .. 8j+7 in column order (low half of a dword first), 16 bits each:
+ * D * S * cap * 256 dwords): the row's flips 8j .. 8j+7 (in column order from every producer but
+ * nb_flip_skip_layered, which lists them class by class; no consumer needs an order, each column at most once is
+ * what counts), low half of a dword first, 16 bits each:
  * [4:0] = column % 32, [15:5] = 2 * (column / 32) + b with b the base bit at that column; the last piece is padded
  * with the sentinel (4Kw) << 5, which may also stand between flips.  info[d, r] (uint32) = flips | pieces << 16: only the
  * first `pieces` pieces of a row are ever written or read.  Every row has a fixed place, so lists are written in one
@@ -200,6 +202,20 @@ int nb_conv_bn_thresholds_from_input_i32(int32_t *thresh, const int32_t *in, con
  *                the largest Tf of the layer (T_max = table[2]).  The words of a row come in pairs: word 2i is a gap as
  *                above, and the column it reaches flips only if word 2i+1 times T_max is below Tf * 2^32 (64-bit
  *                integers): each column flips with probability Tf / 2^32, independently.
+ * nb_flip_skip_layered: per-element probabilities class by class, for laws whose largest probability is far above
+ *                their mean (thinning draws C * p_max pairs per row, this about twice the row's flips plus one or
+ *                two per class).  nb_flip_law_layers sorts a law [R, C] (as nb_flip_skip_thin takes it; the base
+ *                bit travels along) into pl [R, C] uint32 = column | law << 16, the columns of class k
+ *                (2^(30-k) < Tf <= 2^(31-k) for k < 15, 0 < Tf <= 2^16 for k = 15; Tf = 0 is left out, the tail of
+ *                pl holds 0xFFFF) at pl[r, cls[r, k] .. cls[r, k+1]) in increasing column order; cls [R, 17]
+ *                uint32.  tables: nb_flip_layer_table_words() uint32 of device memory filled once by
+ *                nb_flip_layer_tables: 16 tables as nb_skip_table makes them, class k's for the threshold
+ *                2^(31-k), of which the walk uses the first 512 entries.  The words of a row come in pairs as for
+ *                nb_flip_skip_thin, class after class without a break: in class k the gap's rank in that table
+ *                (a rank of 512 = beyond it) moves the position in the class's stretch of pl (start: -1), the
+ *                column reached flips iff the second word is below Tf * 2^(k+1); a position past the stretch ends
+ *                the class and the next class that has columns starts with the next pair.  Same law as
+ *                nb_flip_skip_thin (every column flips with probability Tf / 2^32, independently), other masks.
  * The layers' law (modules/binary.py:59-60), P = sigmoid(5 w / (mean|w| + 1e-5)), rounded to fp16 wherever the tensor
  * expression rounds; mean|w| = the exact sum over the count, rounded once to fp16.  workspace: nb_law_workspace_bytes()
  * bytes of device memory, 8-byte aligned.
@@ -215,6 +231,12 @@ int nb_flip_skip_i64(uint32_t *entries, uint32_t *info, uint32_t *overflow, cons
 int nb_flip_skip_thin_i64(uint32_t *entries, uint32_t *info, uint32_t *overflow, const uint16_t *law,
                           const uint32_t *table, uint64_t seed, uint64_t subseq, uint64_t first, int64_t D, int64_t R,
                           int64_t C, int64_t cap, nb_stream_t stream);
+int64_t nb_flip_layer_table_words(void);
+int nb_flip_layer_tables(uint32_t *tables, nb_stream_t stream);
+int nb_flip_law_layers(uint32_t *pl, uint32_t *cls, const uint16_t *law, int64_t R, int64_t C, nb_stream_t stream);
+int nb_flip_skip_layered_i64(uint32_t *entries, uint32_t *info, uint32_t *overflow, const uint32_t *pl,
+                             const uint32_t *cls, const uint32_t *tables, uint64_t seed, uint64_t subseq, uint64_t first,
+                             int64_t D, int64_t R, int64_t C, int64_t cap, nb_stream_t stream);
 /* The skip sampler's masks as packed words, for short rows (at most 8 words): out = base ^ mask (base NULL: the mask
  * alone), the mask of row q = m*R + r being exactly the flips nb_flip_skip_i64 lists for it (same table, same words
  * first + q*C + i of the stream), i.e. what nb_flip_to_dense_i64 makes of those lists.  Same layouts as the per-bit

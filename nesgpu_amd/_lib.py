@@ -61,6 +61,9 @@ _PLAIN = {
     "nb_skip_table": [_PTR, _PTR, _PTR],
     "nb_flip_skip_i64": [_PTR, _PTR, _PTR, _PTR, _PTR, _U64, _U64, _U64, _I64, _I64, _I64, _I64, _PTR],
     "nb_flip_skip_thin_i64": [_PTR, _PTR, _PTR, _PTR, _PTR, _U64, _U64, _U64, _I64, _I64, _I64, _I64, _PTR],
+    "nb_flip_layer_tables": [_PTR, _PTR],
+    "nb_flip_law_layers": [_PTR, _PTR, _PTR, _I64, _I64, _PTR],
+    "nb_flip_skip_layered_i64": [_PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _U64, _U64, _U64, _I64, _I64, _I64, _I64, _PTR],
     "nb_thresholds_from_weights": [_PTR, _PTR, _I64, _PTR, _PTR],
     "nb_probabilities_from_weights": [_PTR, _PTR, _I64, _PTR, _PTR],
     "nb_flip_law_from_weights": [_PTR, _PTR, _PTR, _PTR, _I64, _I64, _PTR, _PTR],
@@ -82,6 +85,7 @@ _SIZES = {
     "nb_bmv_bn_workspace_bytes": [_I64, _I64],
     "nb_bmv_bn_static_bytes": [],
     "nb_skip_table_words": [],
+    "nb_flip_layer_table_words": [],
     "nb_law_workspace_bytes": [],
 }
 

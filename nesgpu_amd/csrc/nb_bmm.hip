@@ -432,7 +432,7 @@ int nb_bmm_i32(int32_t *C, const int32_t *A, const int32_t *B, int64_t Z, int64_
 int nb_bmv_pm1_i64(int32_t *C, const int64_t *A, const int64_t *x, int64_t Z, int64_t M, int64_t Kw, int64_t K,
                    nb_stream_t s)
 {
-    NB_REQUIRE(K >= 0 && K <= Kw * 64, "nb_bmv_pm1_i64: K = %lld bits does not fit the rows' %lld words", (long long)K,
+    NB_REQUIRE(K >= 0 && K <= Kw * 64 && K < (1LL << 31), "nb_bmv_pm1_i64: K = %lld bits does not fit the rows' %lld words", (long long)K,
                (long long)Kw);
     if (Kw == 0) return nb::fail(NB_ERR_SHAPE, "nb_bmv_pm1_i64: empty rows");
     return nb::bmm_impl<uint64_t>(C, reinterpret_cast<const uint64_t *>(A), reinterpret_cast<const uint64_t *>(x), Z, M, Kw, 1, s,
@@ -441,7 +441,7 @@ int nb_bmv_pm1_i64(int32_t *C, const int64_t *A, const int64_t *x, int64_t Z, in
 int nb_bmv_pm1_i32(int32_t *C, const int32_t *A, const int32_t *x, int64_t Z, int64_t M, int64_t Kw, int64_t K,
                    nb_stream_t s)
 {
-    NB_REQUIRE(K >= 0 && K <= Kw * 32, "nb_bmv_pm1_i32: K = %lld bits does not fit the rows' %lld words", (long long)K,
+    NB_REQUIRE(K >= 0 && K <= Kw * 32 && K < (1LL << 31), "nb_bmv_pm1_i32: K = %lld bits does not fit the rows' %lld words", (long long)K,
                (long long)Kw);
     if (Kw == 0) return nb::fail(NB_ERR_SHAPE, "nb_bmv_pm1_i32: empty rows");
     return nb::bmm_impl<uint32_t>(C, reinterpret_cast<const uint32_t *>(A), reinterpret_cast<const uint32_t *>(x), Z, M, Kw, 1, s,

@@ -269,7 +269,8 @@ __global__ __launch_bounds__(256) void fl_fill_kernel(uint32_t *__restrict__ ent
 }
 
 // Flip lists -> materialised weights: W must hold the base in every member on entry; every flip is XOR-ed in.  A
-// lane owns its row, so plain read-modify-writes suffice (flips come in column order: one write per touched word).
+// lane owns its row, so plain read-modify-writes suffice (flips in column order: one write per touched word; any
+// other order just writes more often).
 __global__ __launch_bounds__(256) void fl_to_dense_kernel(uint64_t *__restrict__ W, const uint32_t *__restrict__ entries,
                                                           const uint32_t *__restrict__ info, int64_t nslices, int S,
                                                           int64_t R, int Kw, int cap)

@@ -549,6 +549,284 @@ static int gen_launch(GenArgs a, bool thin, bool force_walk, hipStream_t s, cons
     return check_launch(who);
 }
 
+// ---- per-element probabilities by layers ---------------------------------------------------------------------------
+// Thinning at the largest probability of a layer draws C * p_max candidates per row whatever the mean: a law with a long
+// tail pays for its tail.  Here the columns of a row are sorted into 16 classes by the size of their flip threshold Tf,
+// class k holding 2^(30-k) < Tf <= 2^(31-k) (class 15: everything down to Tf = 1; Tf = 0 never flips and is left out),
+// and the walk goes class by class over the class's columns at the class's own rate 2^-(k+1): a column it reaches flips
+// iff accept < Tf * 2^(k+1), i.e. with probability Tf / 2^(31-k) >= 1/2 (class 15 aside).  The candidates of a row
+// are then at most twice its flips plus a step or two per class.
+//
+// Contract (restated in oracle/nesbin_oracle.c, nbo_skip_flips_layered_i64): pl[r, i] = column | law << 16 lists the row's
+// columns class by class, in increasing column order inside a class; cls[r, k] is where class k starts (cls[r, 16]:
+// the end).  Row q = d*R + r reads the Philox words first + q*C + 2i (gap) and + 2i + 1 (accept), i = 0, 1, ...: the
+// walk starts at position -1 of the first non-empty class; a gap word's rank in the class's table (the first
+// kLayerTab entries of the gap table of threshold 2^(31-k)) moves it on by rank + 1 positions to a candidate, or,
+// beyond the table, by the table's length without one; past the class's end the next non-empty class starts at -1
+// with the next word pair; the row ends with the last class.
+constexpr int kLayers = 16, kLayerTab = 512, kLayerStride = kLayerTab + 2, kLayerWords = kSkipTableWords;
+
+__device__ __forceinline__ uint32_t law_threshold16(uint32_t law16)
+{
+    const float y = (float)__builtin_bit_cast(_Float16, (uint16_t)(law16 & 0x7FFFu));
+    return (uint32_t)fminf(y * 4294967296.0f, 4294967040.0f);
+}
+
+// class of a flip threshold: 0 .. 15, or 16 for Tf = 0 (never flips)
+__device__ __forceinline__ int law_class(uint32_t tf)
+{
+    if (tf == 0) return kLayers;
+    const int k = __clz((int)(tf - 1u)) - 1;   // __clz(0) = 32
+    return k < 0 ? 0 : (k > kLayers - 1 ? kLayers - 1 : k);
+}
+
+// The 16 gap tables, whole (kSkipTableWords each; the walk keeps the first kLayerTab entries): class k's is the table of
+// threshold 2^(31-k).  A workgroup per class.
+__global__ __launch_bounds__(1024) void fl_layer_tables_kernel(uint32_t *tables)
+{
+    __shared__ uint32_t thr;
+    if (threadIdx.x == 0) thr = 0x80000000u >> blockIdx.x;
+    __syncthreads();
+    skip_table_build(tables + (size_t)blockIdx.x * kLayerWords, &thr);
+}
+
+// One wave per row: count the classes, then place every column (stable: increasing column inside a class).
+__global__ __launch_bounds__(256) void law_layers_kernel(uint32_t *__restrict__ pl, uint32_t *__restrict__ cls,
+                                                         const uint16_t *__restrict__ law, int64_t R, int C)
+{
+    const int lane = threadIdx.x & 63;
+    const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (r >= R) return;
+    const uint16_t *row = law + r * C;
+    uint32_t count[kLayers];
+#pragma unroll
+    for (int k = 0; k < kLayers; k++) count[k] = 0;
+    for (int c0 = 0; c0 < C; c0 += 64) {
+        const int c = c0 + lane;
+        const int k = c < C ? law_class(law_threshold16(row[c])) : kLayers;
+#pragma unroll
+        for (int kk = 0; kk < kLayers; kk++) count[kk] += (uint32_t)__popcll(__ballot(k == kk));
+    }
+    uint32_t offs[kLayers];
+    uint32_t run = 0;
+#pragma unroll
+    for (int k = 0; k < kLayers; k++) {
+        offs[k] = run;
+        if (lane == 0) cls[r * (kLayers + 1) + k] = run;
+        run += count[k];
+    }
+    if (lane == 0) cls[r * (kLayers + 1) + kLayers] = run;
+    const unsigned long long below = (1ull << lane) - 1ull;
+    uint32_t *out = pl + r * C;
+    for (int c0 = 0; c0 < C; c0 += 64) {
+        const int c = c0 + lane;
+        const uint32_t l = c < C ? row[c] : 0u;
+        const int k = c < C ? law_class(law_threshold16(l)) : kLayers;
+#pragma unroll
+        for (int kk = 0; kk < kLayers; kk++) {
+            const unsigned long long m = __ballot(k == kk);
+            if (k == kk) out[offs[kk] + (uint32_t)__popcll(m & below)] = (uint32_t)c | (l << 16);
+            offs[kk] += (uint32_t)__popcll(m);
+        }
+    }
+    // the columns that never flip fill the rest of the row (never read by the walk)
+    for (uint32_t i = run + lane; i < (uint32_t)C; i += 64) out[i] = 0xFFFFu;
+}
+
+struct LayerArgs {
+    uint4 *entries;
+    uint32_t *info, *overflow;
+    const uint32_t *pl, *cls, *tables;   // [R, C], [R, 17], [16, kLayerWords]
+    PhiloxKey key;
+    int64_t D, R;
+    int C, Kw, S, cap, MC, rb_shift;
+};
+
+// INLDS: the workgroup's rows of pl are staged in LDS; else (rows too long for that) read where they lie.
+template <bool ALIGNED, bool INLDS>
+__global__ __launch_bounds__(1024) void fl_gen_layered_kernel(const LayerArgs a)
+{
+    extern __shared__ uint32_t gen_lds[];
+    uint32_t *tabs = gen_lds;                                                 // kLayers tables of kLayerStride words
+    int *kts = reinterpret_cast<int *>(tabs + kLayers * kLayerStride);        // entries of each
+    float *hints = reinterpret_cast<float *>(kts + kLayers);                  // 1 / log2(1 - p_k)
+    const int RB = 1 << a.rb_shift;
+    uint32_t *cl = reinterpret_cast<uint32_t *>(hints + kLayers);             // RB x (kLayers + 1) class starts
+    uint32_t *rowdata = cl + 8 * (kLayers + 1);                               // RB x C (column | law << 16)
+    const int nrg = (int)((a.R + RB - 1) >> a.rb_shift);
+    const int rg = (int)(blockIdx.x % (unsigned)nrg), mc = (int)(blockIdx.x / (unsigned)nrg);
+    const int64_t r0 = (int64_t)rg << a.rb_shift;
+    for (int idx = threadIdx.x; idx < kLayers * kLayerStride; idx += blockDim.x) {
+        const int k = idx / kLayerStride, i = idx - k * kLayerStride;
+        const uint32_t *t = a.tables + k * kLayerWords;
+        const int kt = (int)t[0] < kLayerTab ? (int)t[0] : kLayerTab;
+        tabs[idx] = i == 0 ? 0u : (i <= kt ? t[kSkipHeader + i - 1] : 0xFFFFFFFFu);
+        if (i == 0) {
+            kts[k] = kt;
+            hints[k] = __uint_as_float(t[1]);
+        }
+    }
+    for (int rr = 0; rr < RB && r0 + rr < a.R; rr++) {
+        if (INLDS)
+            for (int i = threadIdx.x; i < a.C; i += blockDim.x) rowdata[rr * a.C + i] = a.pl[(r0 + rr) * a.C + i];
+        for (int i = threadIdx.x; i <= kLayers; i += blockDim.x) cl[rr * (kLayers + 1) + i] = a.cls[(r0 + rr) * (kLayers + 1) + i];
+    }
+    __syncthreads();
+    const int rr = (int)threadIdx.x & (RB - 1);
+    const int64_t r = r0 + rr;
+    const int slots = (int)blockDim.x >> a.rb_shift;
+    const int64_t dend = (int64_t)(mc + 1) * a.MC < a.D ? (int64_t)(mc + 1) * a.MC : a.D;
+    int64_t d = (int64_t)mc * a.MC + ((int)threadIdx.x >> a.rb_shift);
+    const uint32_t *myrow = INLDS ? rowdata + rr * a.C : a.pl + (r < a.R ? r : 0) * a.C;
+    const uint32_t *mycl = cl + rr * (kLayers + 1);
+    const uint32_t sentinel = (uint32_t)(4 * a.Kw) << 5;
+    if (r >= a.R) d = dend;
+    // the lane keeps its row for all its members: which classes have columns, once
+    uint32_t nonempty = 0;
+    if (r < a.R)
+        for (int c = 0; c < kLayers; c++) nonempty |= (mycl[c + 1] != mycl[c] ? 1u : 0u) << c;
+    bool live = d < dend;
+    int64_t q = 0;
+    uint64_t blk = 0;
+    SkipChain chain(a.key, 0);
+    uint4 *dst = a.entries;
+    int cur = 0, pos = -1, nk = 0, startk = 0, n = 0, k = 0, piece = 0;
+    // the current class's table: where it starts in LDS, its length, the hint of its look-ups
+    const uint32_t *tab1 = tabs;
+    int kt = 0;
+    float hint = -1.0f;
+    uint32_t q0 = 0, q1 = 0, q2 = 0, q3 = 0;
+    auto insert = [&](uint32_t e) {
+        q0 = __builtin_amdgcn_alignbit(q1, q0, 16);
+        q1 = __builtin_amdgcn_alignbit(q2, q1, 16);
+        q2 = __builtin_amdgcn_alignbit(q3, q2, 16);
+        q3 = (q3 >> 16) | (e << 16);
+    };
+    auto flush = [&]() {
+        if (piece < a.cap) dst[(int64_t)piece * 64] = make_uint4(q0, q1, q2, q3);
+        piece++;
+        k = 0;
+    };
+    // the next class that has columns, from `from` on; kLayers: none left
+    auto enter_class = [&](int from) {
+        const uint32_t left = from < kLayers ? nonempty >> from : 0u;
+        cur = left ? from + (int)__builtin_ctz(left) : kLayers;
+        const int c = cur < kLayers ? cur : 0;
+        startk = (int)mycl[c];
+        nk = (int)mycl[c + 1] - startk;
+        kt = kts[c];
+        hint = hints[c];
+        tab1 = tabs + c * kLayerStride;
+        pos = -1;
+    };
+    auto start_row = [&]() {
+        live = d < dend;
+        if (live) {
+            q = d * a.R + r;
+            const uint64_t g0 = a.key.first + (uint64_t)q * (uint64_t)a.C;
+            if (ALIGNED) blk = g0 >> 2;
+            else chain.restart(g0);
+            dst = a.entries + ((d * a.S + (r >> 6)) * (int64_t)a.cap) * 64 + (r & 63);
+            enter_class(0);
+        } else {
+            cur = kLayers;
+        }
+        n = 0;
+        k = 0;
+        piece = 0;
+    };
+    auto finish_row = [&]() {
+        if (k) {
+            for (; k < 8; k++) insert(sentinel);
+            flush();
+        }
+        const bool over = piece > a.cap;
+        a.info[q] = over ? flip_info((uint32_t)(8 * a.cap), (uint32_t)a.cap) : flip_info((uint32_t)n, (uint32_t)piece);
+        if (over) atomicAdd(a.overflow, 1u);
+        d += slots;
+        start_row();
+    };
+    auto rank_of = [&](uint32_t gap) {
+        const uint32_t u[1] = {gap};
+        int rank[1];
+        skip_ranks<1>(rank, tab1, kt, u, hint, -32.0f * hint);
+        return rank[0];
+    };
+    // one step of the walk in the lane's current class: the rank of a gap word and the pair's accept word
+    auto step = [&](int rank, uint32_t acc) {
+        pos += rank < kt ? rank + 1 : kt;
+        if (pos >= nk) {
+            enter_class(cur + 1);
+        } else if (rank < kt) {
+            const uint32_t e = myrow[startk + pos];
+            const uint32_t col = e & 0xFFFFu, l = e >> 16;
+            if ((uint64_t)acc < ((uint64_t)law_threshold16(l) << (cur + 1))) {
+                insert((((2u * (col >> 5)) + (l >> 15)) << 5) | (col & 31u));
+                n++;
+                if (++k == 8) flush();
+            }
+        }
+    };
+    start_row();
+    while (__any(live)) {
+        if (live) {
+            if (cur >= kLayers) {
+                finish_row();      // also rows without a column that can flip
+            } else if (ALIGNED) {
+                const uint4 w = philox_block(a.key, blk++);
+                step(rank_of(w.x), w.y);
+                if (cur < kLayers) step(rank_of(w.z), w.w);
+            } else {
+                const uint32_t gap = chain.next();
+                const uint32_t acc = chain.next();
+                step(rank_of(gap), acc);
+            }
+        }
+    }
+}
+
+static int layered_launch(LayerArgs a, hipStream_t s, const char *who)
+{
+    const bool aligned = a.C % 4 == 0 && a.key.first % 4 == 0;
+    const size_t fixed = (size_t)(kLayers * kLayerStride + 2 * kLayers + 8 * (kLayers + 1)) * 4;
+    const size_t row_bytes = (size_t)a.C * 4;
+    // rows per workgroup: eight (a 128-byte line of every piece) where LDS holds them; two at least, else none in LDS
+    int shift = 3;
+    while (shift > 1 && fixed + (row_bytes << shift) > 150 * 1024) shift--;
+    bool inlds = fixed + (row_bytes << shift) <= 150 * 1024;
+    if (const char *e = getenv("NESBIN_LAYERED_LDS")) inlds = inlds && atoi(e) != 0;
+    if (!inlds) shift = 3;
+    a.rb_shift = shift;
+    const size_t lds = fixed + (inlds ? row_bytes << shift : 0);
+    const int threads = 1024;
+    const int slots = threads >> shift;
+    int64_t MC = (int64_t)slots * 8;
+    if (MC > a.D) MC = ceil_div(a.D, slots) * slots;
+    a.MC = (int)MC;
+    const int64_t nrg = ceil_div(a.R, (int64_t)1 << shift), nmc = ceil_div(a.D, MC);
+    NB_REQUIRE(nrg * nmc <= kMaxGridX, "%s: too many rows for one launch", who);
+    static std::once_flag once;
+    static hipError_t attr = hipSuccess;
+    std::call_once(once, [] {
+        const void *fns[2] = {reinterpret_cast<const void *>(fl_gen_layered_kernel<false, true>),
+                              reinterpret_cast<const void *>(fl_gen_layered_kernel<true, true>)};
+        for (const void *f : fns) {
+            const hipError_t e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
+            if (e != hipSuccess) attr = e;
+        }
+    });
+    if (attr != hipSuccess) {
+        (void)hipGetLastError();
+        return fail(NB_ERR_UNSUPPORTED, "%s: cannot raise the kernel's LDS limit: %s", who, hipGetErrorString(attr));
+    }
+    const dim3 grid((unsigned)(nrg * nmc)), block((unsigned)threads);
+    if (aligned && inlds) fl_gen_layered_kernel<true, true><<<grid, block, lds, s>>>(a);
+    else if (aligned) fl_gen_layered_kernel<true, false><<<grid, block, lds, s>>>(a);
+    else if (inlds) fl_gen_layered_kernel<false, true><<<grid, block, lds, s>>>(a);
+    else fl_gen_layered_kernel<false, false><<<grid, block, lds, s>>>(a);
+    return check_launch(who);
+}
+
 static int gen_check(const uint32_t *entries, const uint32_t *info, const uint32_t *overflow, const void *rows,
                      const uint32_t *table, int64_t D, int64_t R, int64_t C, int64_t cap, const char *who)
 {
@@ -725,7 +1003,7 @@ static int sample_skip_launch(W *out_conv, W *out_rows, const W *base, const uin
     if (Rw > 8)
         return fail(NB_ERR_UNSUPPORTED, "%s: rows of more than 8 words (%lld): use the flip lists or the per-bit sampler",
                     who, (long long)Rw);
-    NB_REQUIRE(KK * Rw <= 4096 && R * Rw < (1LL << 31) && n < (1LL << 40), "%s: shape too large", who);
+    NB_REQUIRE(KK * Rw <= 2048 && R * Rw < (1LL << 31) && n < (1LL << 40), "%s: shape too large", who);
     // rows per chunk: whole output channels, about 2048 words of staging at most; members per workgroup: enough rows
     // to spread the table's load over, while the launch keeps a few thousand workgroups
     int64_t oc = std::max<int64_t>(1, 2048 / (KK * Rw));
@@ -825,6 +1103,65 @@ int nb_flip_skip_thin_i64(uint32_t *entries, uint32_t *info, uint32_t *overflow,
     a.S = (int)((R + 63) / 64);
     a.cap = (int)cap;
     return nb::gen_launch(a, true, false, nb::as_stream(stream), who);
+}
+
+int64_t nb_flip_layer_table_words(void) { return nb::kLayers * nb::kLayerWords; }
+
+int nb_flip_layer_tables(uint32_t *tables, nb_stream_t stream)
+{
+    const char *who = "nb_flip_layer_tables";
+    NB_REQUIRE_PTR(tables);
+    NB_REQUIRE_ALIGNED(tables, 4);
+    nb::fl_layer_tables_kernel<<<dim3(nb::kLayers), dim3(1024), 0, nb::as_stream(stream)>>>(tables);
+    return nb::check_launch(who);
+}
+
+int nb_flip_law_layers(uint32_t *pl, uint32_t *cls, const uint16_t *law, int64_t R, int64_t C, nb_stream_t stream)
+{
+    const char *who = "nb_flip_law_layers";
+    NB_REQUIRE(R >= 0 && C >= 0 && C <= 65535 && R <= (1LL << 31), "%s: R=%lld, C=%lld out of range (C at most 65535)", who,
+               (long long)R, (long long)C);
+    if (R == 0) return NB_OK;
+    NB_REQUIRE_PTR(cls);
+    NB_REQUIRE_ALIGNED(cls, 4);
+    if (C > 0) {
+        NB_REQUIRE_PTR(pl);
+        NB_REQUIRE_PTR(law);
+        NB_REQUIRE_ALIGNED(pl, 4);
+        NB_REQUIRE_ALIGNED(law, 2);
+    }
+    const int64_t blocks = nb::ceil_div(R, 4);
+    NB_REQUIRE(blocks <= nb::kMaxGridX, "%s: too many rows for one launch", who);
+    nb::law_layers_kernel<<<dim3((unsigned)blocks), dim3(256), 0, nb::as_stream(stream)>>>(pl, cls, law, R, (int)C);
+    return nb::check_launch(who);
+}
+
+int nb_flip_skip_layered_i64(uint32_t *entries, uint32_t *info, uint32_t *overflow, const uint32_t *pl,
+                             const uint32_t *cls, const uint32_t *tables, uint64_t seed, uint64_t subseq, uint64_t first,
+                             int64_t D, int64_t R, int64_t C, int64_t cap, nb_stream_t stream)
+{
+    const char *who = "nb_flip_skip_layered_i64";
+    if (int rc = nb::gen_check(entries, info, overflow, pl, tables, D, R, C, cap, who)) return rc;
+    if (D * R == 0) return NB_OK;
+    NB_REQUIRE(C <= 65535, "%s: C=%lld, at most 65535 columns", who, (long long)C);
+    NB_REQUIRE_PTR(cls);
+    NB_REQUIRE_ALIGNED(pl, 4);
+    NB_REQUIRE_ALIGNED(cls, 4);
+    nb::LayerArgs a{};
+    a.entries = reinterpret_cast<uint4 *>(entries);
+    a.info = info;
+    a.overflow = overflow;
+    a.pl = pl;
+    a.cls = cls;
+    a.tables = tables;
+    a.key = nb::PhiloxKey{seed, subseq, first};
+    a.D = D;
+    a.R = R;
+    a.C = (int)C;
+    a.Kw = (int)((C + 63) / 64);
+    a.S = (int)((R + 63) / 64);
+    a.cap = (int)cap;
+    return nb::layered_launch(a, nb::as_stream(stream), who);
 }
 
 int nb_sample_skip_i64(int64_t *out, const int64_t *base, const uint32_t *table, uint64_t seed, uint64_t subseq,

@@ -27,7 +27,7 @@ __all__ = [
     "flip_from_words", "sample_bits_philox", "flip_philox", "seeded_bmv_from_words", "seeded_bmv_philox",
     "philox_words", "conv_act_pack", "conv_popc_sums", "conv_bn_thresholds_from_input", "tap_pack_filter", "tap_packing_applies", "conv_engine", "conv_last_engine",
     "bmv_act_pack", "bmv_bn_act", "ExpandedRows", "expand_rows", "bmm_nt", "FlipRows", "flip_rows_from_weights",
-    "bmv_flip", "bmv_flip_act_pack", "skip_table", "flip_rows_skip", "flip_rows_to_weights",
+    "bmv_flip", "bmv_flip_act_pack", "skip_table", "flip_rows_skip", "flip_rows_layered", "layer_tables", "flip_rows_to_weights",
     "center_fitness", "grad_regularize_", "bias_grad", "sample_bits_skip", "half_draws_apply", "bias_noise_scale_", "bmv_pm1",
 ]
 
@@ -1081,6 +1081,20 @@ class FlipLaw:
 
     def __init__(self, law, base, table, in_bits):
         self.law, self.base, self.table, self.in_bits = law, base, table, in_bits
+        self._layers = None
+
+    def layers(self):
+        """The law sorted for :func:`flip_rows_layered`, made on first use and kept: (``pl`` uint32 [R, C] = column |
+        law << 16, the columns class by class; ``cls`` uint32 [R, 17], where each class starts).  One kernel."""
+        if self._layers is None:
+            R, C = self.law.shape
+            pl = torch.empty((R, C), dtype=torch.uint32, device=self.law.device)
+            cls = torch.empty((R, 17), dtype=torch.uint32, device=self.law.device)
+            with _on(self.law):
+                _lib.call("nb_flip_law_layers", pl.data_ptr(), cls.data_ptr(), self.law.data_ptr(), R, C,
+                          _stream(self.law))
+            self._layers = (pl, cls)
+        return self._layers
 
     def max_flip_probability(self):
         """The largest flip probability of the layer (a device read-back)."""
@@ -1150,6 +1164,40 @@ def flip_rows_thin(law, n, seed, cap, subsequence=0, first=0):
         _lib.call("nb_flip_skip_thin_i64", entries.data_ptr(), info.data_ptr(), overflow.data_ptr(), law.law.data_ptr(),
                   law.table.data_ptr(), int(seed) & (2 ** 64 - 1), int(subsequence), int(first), n, R, C, int(cap),
                   _stream(law.law))
+    return FlipRows(law.base, n, R, law.base.size(1), C, info, entries, int(cap), overflow)
+
+
+_layer_tables = {}
+
+
+def layer_tables(device):
+    """The 16 gap tables of :func:`flip_rows_layered` in device memory (constants: made once per device and kept)."""
+    device = torch.device(device)
+    key = (device.type, torch.cuda.current_device() if device.index is None else device.index)
+    buf = _layer_tables.get(key)
+    if buf is None:
+        buf = torch.empty((int(_lib.load().nb_flip_layer_table_words()),), dtype=torch.uint32, device=device)
+        with _on(buf):
+            _lib.call("nb_flip_layer_tables", buf.data_ptr(), _stream(buf))
+        _layer_tables[key] = buf
+    return buf
+
+
+def flip_rows_layered(law, n, seed, cap, subsequence=0, first=0):
+    """:class:`FlipRows` for ``n`` members under a per-element law (:class:`FlipLaw`), for laws with a long tail: the
+    columns of a row are walked class by class (classes by the binary size of the flip probability, 2**-(k+2) < y <=
+    2**-(k+1)), each class at its own rate 2**-(k+1), so that a row costs about two word pairs per flip whatever the
+    layer's largest probability is, where :func:`flip_rows_thin` pays for that largest one in every column.  Same
+    law (every bit differs from the base with its own probability, independently), other masks."""
+    R, C = law.law.shape
+    dev = law.law.device
+    pl, cls = law.layers()
+    tables = layer_tables(dev)
+    entries, info, overflow = _flip_alloc(n, R, int(cap), dev)
+    with _on(law.law):
+        _lib.call("nb_flip_skip_layered_i64", entries.data_ptr(), info.data_ptr(), overflow.data_ptr(), pl.data_ptr(),
+                  cls.data_ptr(), tables.data_ptr(), int(seed) & (2 ** 64 - 1), int(subsequence), int(first), n, R, C,
+                  int(cap), _stream(law.law))
     return FlipRows(law.base, n, R, law.base.size(1), C, info, entries, int(cap), overflow)
 
 

@@ -24,6 +24,10 @@
  *                        (Python integers); per-column flip rates against their own probabilities,
  *                        neighbouring columns uncorrelated, reduction to skip_flips' law when all
  *                        probabilities equal the largest one
+ *   skip_flips_layered   rows whose columns all share a class: equal to skip_flips_thin on the same words with the
+ *                        class's table and tmax = 2^(31-k) (every class); mixed rows: an independent numpy walk
+ *                        per class over the (pinned) Philox words; per-column flip rates against their own
+ *                        probabilities over a law spanning many classes, neighbouring columns uncorrelated
  *   draws16              an independent numpy evaluation from the (pinned) Philox words of the two streams,
  *                        with thresholds that force ties; rates of columns whose thresholds have non-zero
  *                        low halves; neighbouring columns (the two halves of one word) uncorrelated
@@ -271,6 +275,63 @@ void nbo_skip_flips_thin_i64(uint64_t *mask, const uint16_t *law, const uint32_t
             if (!(t <= 4294967040.0f)) t = 4294967040.0f;
             const uint64_t tf = (uint64_t)(uint32_t)t;
             if ((uint64_t)pair[1] * (uint64_t)tmax < (tf << 32)) row[pos >> 6] |= (uint64_t)1 << (pos & 63);
+        }
+    }
+}
+
+/* Flip masks under a per-element law, class by class: the contract of nb_flip_skip_layered_i64 (no counterpart in the
+ * reference, as above).  The columns of row r that can flip are listed in pl[r, :] = column | law << 16, sorted by the
+ * class of their flip threshold Tf (class k: 2^(30-k) < Tf <= 2^(31-k), k < 15; class 15: 0 < Tf <= 2^16), in
+ * increasing column order inside a class; cls[r, k] .. cls[r, k+1] is class k's stretch of the list.  Row q = d*R + r
+ * reads the Philox words first + q*C + 2i (a gap) and + 2i + 1 (accept), i = 0, 1, ..., without a break from class to
+ * class: in class k the gap is ranked in cdfs[k] (kts[k] entries of the gap table of threshold 2^(31-k)) and moves the
+ * position in the class's stretch (start: -1) as in nbo_skip_flips_i64; the column reached flips iff
+ * accept < Tf * 2^(k+1); a position past the stretch ends the class, and the next class that has columns starts with
+ * the next pair.  cdfs is [16, tabw] uint32.  mask is [D*R, ceil(C/64)] 64-bit words, LSB first. */
+void nbo_skip_flips_layered_i64(uint64_t *mask, const uint32_t *pl, const uint32_t *cls, const uint32_t *cdfs,
+                                const int32_t *kts, int64_t tabw, uint64_t seed, uint64_t subseq, uint64_t first,
+                                int64_t D, int64_t R, int64_t C)
+{
+    const uint32_t key[2] = {(uint32_t)seed, (uint32_t)(seed >> 32)};
+    const int64_t Kw = (C + 63) / 64;
+#pragma omp parallel for schedule(static)
+    for (int64_t q = 0; q < D * R; q++) {
+        uint64_t *row = mask + q * Kw;
+        const uint32_t *list = pl + (q % R) * C;
+        const uint32_t *starts = cls + (q % R) * 17;
+        memset(row, 0, (size_t)Kw * 8);
+        uint64_t g = first + (uint64_t)q * (uint64_t)C; /* the next word of the row */
+        for (int k = 0; k < 16; k++) {
+            const int64_t nk = (int64_t)starts[k + 1] - (int64_t)starts[k];
+            const uint32_t *cdf = cdfs + (int64_t)k * tabw;
+            const int64_t Kt = kts[k];
+            if (nk <= 0) continue;
+            int64_t pos = -1;
+            for (;;) {
+                uint32_t pair[2];
+                for (int h = 0; h < 2; h++, g++) {
+                    const uint64_t blk = g >> 2;
+                    const uint32_t ctr[4] = {(uint32_t)blk, (uint32_t)(blk >> 32), (uint32_t)subseq, (uint32_t)(subseq >> 32)};
+                    uint32_t o[4];
+                    nbo_philox4x32_10(o, ctr, key);
+                    pair[h] = o[g & 3];
+                }
+                int64_t lo = 0, hi = Kt;
+                while (lo < hi) {
+                    const int64_t mid = (lo + hi) / 2;
+                    if (cdf[mid] <= pair[0]) lo = mid + 1;
+                    else hi = mid;
+                }
+                pos += lo < Kt ? 1 + lo : Kt;
+                if (pos >= nk) break;
+                if (lo >= Kt) continue;
+                const uint32_t e = list[starts[k] + pos];
+                float t = nbo_half_bits_to_float((uint16_t)((e >> 16) & 0x7FFFu)) * 4294967296.0f;
+                if (!(t <= 4294967040.0f)) t = 4294967040.0f;
+                const uint64_t tf = (uint64_t)(uint32_t)t;
+                const uint32_t col = e & 0xFFFFu;
+                if ((uint64_t)pair[1] < (tf << (k + 1))) row[col >> 6] |= (uint64_t)1 << (col & 63);
+            }
         }
     }
 }

@@ -275,6 +275,65 @@ def skip_flips_thin(law, cdf, tmax, seed, subseq, first, D):
     return out
 
 
+LAYERS, LAYER_TABLE = 16, 512
+
+
+def law_thresholds(law):
+    """Flip thresholds Tf = floor(y * 2**32) (at most 2**32 - 256) of a uint16 law array: y = the fp16 number of bits
+    14:0."""
+    y = (_c(law, np.uint16) & 0x7FFF).view(np.float16).astype(np.float32)
+    return np.minimum(y * np.float32(4294967296.0), np.float32(4294967040.0)).astype(np.uint32)
+
+
+def law_layers(law):
+    """The per-element law uint16 [R, C] sorted for the class-by-class walk (see nbo_skip_flips_layered_i64):
+    (pl uint32 [R, C], cls uint32 [R, 17]).  Class of a column: k with 2**(30-k) < Tf <= 2**(31-k), at most 15;
+    Tf == 0: left out (the tail of pl holds 0xFFFF)."""
+    law = _c(law, np.uint16)
+    R, C = law.shape
+    tf = law_thresholds(law).astype(np.int64)
+    k = np.full((R, C), LAYERS, dtype=np.int64)
+    nz = tf > 0
+    # bit length of (tf - 1): clz32 = 32 - bit_length
+    bl = np.zeros((R, C), dtype=np.int64)
+    v = np.maximum(tf - 1, 0)
+    for b in range(32):
+        bl = np.where(v >> b, b + 1, bl)
+    k[nz] = np.clip(32 - bl[nz] - 1, 0, LAYERS - 1)
+    order = np.argsort(k, axis=1, kind="stable")
+    ks = np.take_along_axis(k, order, axis=1)
+    pl = (order.astype(np.uint32) | (np.take_along_axis(law, order, axis=1).astype(np.uint32) << 16))
+    pl = np.where(ks == LAYERS, np.uint32(0xFFFF), pl).astype(np.uint32)
+    cls = np.stack([(ks < c).sum(axis=1) for c in range(LAYERS + 1)], axis=1).astype(np.uint32)
+    return np.ascontiguousarray(pl), np.ascontiguousarray(cls)
+
+
+def layer_tables(cap=LAYER_TABLE):
+    """The 16 gap tables of the class-by-class walk: (cdfs uint32 [16, cap], kts int32 [16]); class k's table is the
+    first ``cap`` entries of skip_cdf(2**(31-k))."""
+    cdfs = np.full((LAYERS, cap), 0xFFFFFFFF, dtype=np.uint32)
+    kts = np.zeros(LAYERS, dtype=np.int32)
+    for k in range(LAYERS):
+        t = skip_cdf(1 << (31 - k), cap=cap)
+        kts[k] = t.shape[0]
+        cdfs[k, :t.shape[0]] = t
+    return cdfs, kts
+
+
+def skip_flips_layered(pl, cls, seed, subseq, first, D, tables=None):
+    """Flip masks [D*R, ceil(C/64)] int64 under a per-element law sorted by law_layers (see
+    nbo_skip_flips_layered_i64)."""
+    pl, cls = _c(pl, np.uint32), _c(cls, np.uint32)
+    R, C = pl.shape
+    cdfs, kts = layer_tables() if tables is None else tables
+    cdfs, kts = _c(cdfs, np.uint32), _c(kts, np.int32)
+    out = np.empty((int(D) * R, (C + 63) // 64), dtype=np.int64)
+    lib().nbo_skip_flips_layered_i64(_p(out), _p(pl), _p(cls), _p(cdfs), _p(kts), _i64(cdfs.shape[1]),
+                                     ctypes.c_uint64(int(seed)), ctypes.c_uint64(int(subseq)),
+                                     ctypes.c_uint64(int(first)), _i64(D), _i64(R), _i64(C))
+    return out
+
+
 def flip_law(P):
     """fp16 probabilities [R, C] -> (law uint16 [R, C], base bool [R, C], tmax): base = P >= 1/2, flip probability
     y = min(P, 1 - P) (exact in fp16), law = base << 15 | fp16 bits of y, tmax = the largest floor(y * 2**32)."""

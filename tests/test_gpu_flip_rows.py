@@ -68,8 +68,9 @@ def test_expand_rows_codes(ops):
     assert not c[2:].any()
 
 
-def decode_flip_rows(rows):
-    """FlipRows -> boolean flip mask [D, R, 64 * Kw] and the base bit every entry claims, read back entry by entry."""
+def decode_flip_rows(rows, ordered=True):
+    """FlipRows -> boolean flip mask [D, R, 64 * Kw] and the base bit every entry claims, read back entry by entry.
+    ``ordered``: the entries of a row come in column order (else: every column at most once)."""
     D, R, Kw, cap = rows.D, rows.R, rows.Kw, rows.cap
     S = (R + 63) // 64
     ent = host(rows.entries).astype(np.uint32)
@@ -91,7 +92,7 @@ def decode_flip_rows(rows):
                         piece, bit = e >> 5, e & 31
                         assert piece < 4 * Kw
                         col = (piece >> 1) * 32 + bit
-                        assert col > col_prev                                            # column order
+                        assert col > col_prev if ordered else not mask[d, r, col]
                         col_prev = col
                         seen += 1
                         mask[d, r, col] = True
@@ -323,6 +324,87 @@ def test_thinning_sampler_vs_oracle(ops, oracle, D, R, C, first, spread):
         np.testing.assert_array_equal(mask, fb)
         bb = np.unpackbits(base.view(np.uint8), axis=1, bitorder="little").astype(bool)
         np.testing.assert_array_equal(bflag, mask & bb[None])
+
+
+def long_tailed_law(g, R, C, mean):
+    """fp16 probabilities whose flip probabilities span five orders of magnitude, a few of them near 1/2."""
+    y = mean * 0.3 * 10.0 ** (g.random((R, C)) * 1.0)
+    y = np.where(g.random((R, C)) < 0.02, g.random((R, C)) * 0.5, y)
+    y = np.where(g.random((R, C)) < 0.3, y * 10.0 ** -(3 * g.random((R, C))), y)
+    y = np.minimum(y, 0.5)
+    return np.where(g.random((R, C)) < 0.5, y, 1.0 - y).astype(np.float16)
+
+
+@pytest.mark.parametrize("D,R,C,first,mean", [(3, 64, 64, 0, 0.1), (2, 100, 200, 8, 0.05), (3, 1024, 2048, 0, 0.01),
+                                              (2, 70, 300, 3, 0.05), (40, 130, 72, 0, 0.1), (2, 9, 8192, 4, 0.005),
+                                              (3, 5, 77, 1, 0.05), (2, 16, 16384, 0, 0.004), (2, 3, 32704, 0, 0.002),
+                                              (600, 2, 1024, 0, 0.02)])
+def test_layered_sampler_vs_oracle(ops, oracle, D, R, C, first, mean):
+    """Flip lists under a per-element law drawn class by class == the oracle's restatement of that walk: the sort of
+    the law (made on the device) against the oracle's stable sort, the 16 tables against the host formula, then the
+    lists, bit for bit, and the sums from them."""
+    g = np.random.default_rng(D + R + C)
+    Kw = (C + 63) // 64
+    P = long_tailed_law(g, R, C, mean)
+    if R > 2:
+        P[1, : C // 2] = 1.0                                               # columns that never flip
+        P[2, :] = 0.0                                                      # a row that never flips
+    law_np, base_bits, tmax = oracle.flip_law(P)
+    base = oracle.pack(base_bits, np.int64)
+    law = ops.FlipLaw(dev(law_np.view(np.int16)).view(torch.uint16), dev(base), None, C)
+    pl, cls = law.layers()
+    want_pl, want_cls = oracle.law_layers(law_np)
+    np.testing.assert_array_equal(host(cls.view(torch.int32)).view(np.uint32), want_cls)
+    live = np.arange(C)[None, :] < want_cls[:, 16:17]
+    np.testing.assert_array_equal(np.where(live, host(pl.view(torch.int32)).view(np.uint32), 0xFFFF), want_pl)
+    words = int(ops._lib.load().nb_skip_table_words())
+    tb = host(ops.layer_tables("cuda").view(torch.int32)).view(np.uint32).reshape(16, words)
+    cdfs, kts = oracle.layer_tables()
+    for k in range(16):
+        assert int(tb[k, 2]) == 1 << (31 - k) and min(int(tb[k, 0]), 512) == kts[k]
+        assert np.abs(tb[k, 4:4 + kts[k]].astype(np.int64) - cdfs[k, :kts[k]].astype(np.int64)).max() <= 1   # another libm
+        cdfs[k, :kts[k]] = tb[k, 4:4 + kts[k]]                             # the table is input data of the contract
+    seed, sub = 0xFEED + C, 5
+    want_flips = oracle.skip_flips_layered(want_pl, want_cls, seed, sub, first, D, tables=(cdfs, kts)).reshape(D, R, Kw)
+    y = (law_np & 0x7FFF).view(np.float16).astype(np.float64)
+    cap = ops.flip_capacity(C, float(y.mean(axis=1).max()))
+    rows = ops.flip_rows_layered(law, D, seed, cap, subsequence=sub, first=first)
+    assert rows.overflowed() == 0
+    W = ops.flip_rows_to_weights(rows)
+    np.testing.assert_array_equal(host(W), base[None] ^ want_flips)
+    np.testing.assert_array_equal(host(rows.cnt).astype(np.int64),
+                                  np.unpackbits(want_flips.view(np.uint8), axis=2, bitorder="little").sum(axis=2))
+    x = sparse_mask(g, (D, C), 0.5)
+    want = oracle.bmm(base[None] ^ want_flips, x.reshape(D, Kw, 1))[:, :, 0]
+    np.testing.assert_array_equal(host(ops.bmm(rows, dev(x).view(D, Kw, 1)))[:, :, 0], want)
+    if D * R * C <= 500000:
+        mask, bflag = decode_flip_rows(rows, ordered=False)
+        fb = np.unpackbits(want_flips.view(np.uint8), axis=2, bitorder="little").astype(bool)
+        np.testing.assert_array_equal(mask, fb)
+        bb = np.unpackbits(base.view(np.uint8), axis=1, bitorder="little").astype(bool)
+        np.testing.assert_array_equal(bflag, mask & bb[None])
+
+
+def test_layered_sampler_flip_rates_at_size(ops, oracle):
+    """4096 members of a 64 x 8192 layer: every column's flip count against its own probability (binomial tails),
+    and the lists stay inside the capacity chosen from the largest row mean."""
+    g = np.random.default_rng(3)
+    D, R, C = 4096, 64, 8192
+    P = long_tailed_law(g, R, C, 0.007)
+    law_np, base_bits, tmax = oracle.flip_law(P)
+    base = oracle.pack(base_bits, np.int64)
+    law = ops.FlipLaw(dev(law_np.view(np.int16)).view(torch.uint16), dev(base), None, C)
+    y = (law_np & 0x7FFF).view(np.float16).astype(np.float64)
+    cap = ops.flip_capacity(C, float(y.mean(axis=1).max()))
+    rows = ops.flip_rows_layered(law, D, 99, cap)
+    assert rows.overflowed() == 0
+    flips = ops.flip_rows_to_weights(rows) ^ dev(base)[None]
+    count = np.stack([host(((flips >> b) & 1).sum(dim=0)) for b in range(64)], axis=2).reshape(R, C).astype(np.float64)
+    pq = oracle.law_thresholds(law_np).astype(np.float64) / 2.0 ** 32
+    from scipy.stats import binom
+    tail = np.minimum(binom.cdf(count, D, pq), binom.sf(count - 1, D, pq))       # exact: the small means are not normal
+    assert tail.min() > 1e-10, (float(tail.min()), np.unravel_index(tail.argmin(), tail.shape))
+    assert abs(count.sum() - D * pq.sum()) <= 5 * np.sqrt(D * pq.sum())
 
 
 @pytest.mark.parametrize("D,R,C,p", [(64, 8, 64, 0.1), (300, 70, 200, 0.05), (1024, 16, 8192, 0.01), (5, 1, 1, 0.5),

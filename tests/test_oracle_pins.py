@@ -358,6 +358,106 @@ def test_skip_flips_thin_against_a_numpy_walk_and_the_per_column_law(oracle):
         np.testing.assert_array_equal(got[q], want)
 
 
+def _fp16_law(y):
+    """uint16 law (base bit 0) of flip probabilities y <= 1/2."""
+    return np.ascontiguousarray(np.asarray(y, dtype=np.float16)).view(np.uint16) & np.uint16(0x7FFF)
+
+
+def test_skip_flips_layered_against_thinning_a_numpy_walk_and_the_per_column_law(oracle):
+    """The class-by-class walk.  (1) The sort: classes from the thresholds' binary size, by Python integers.  (2) A row
+    whose columns share one class k is the thinned walk (pinned above) with class k's table and tmax = 2^(31-k): same
+    words, same columns.  (3) Mixed rows against an evaluation in numpy, one searchsorted + cumsum per class over the
+    pinned Philox words, each class starting at the pair after the one that ended the class before.  (4) What the law
+    fixes: every column flips at its own rate across five orders of magnitude, neighbours uncorrelated."""
+    g = np.random.default_rng(5)
+    cdfs, kts = oracle.layer_tables()
+    assert cdfs.shape == (16, 512) and kts[0] < 40 and (kts[5:] == 512).all()
+    # (1) the sort
+    y = np.concatenate([[0.0, 0.5, 0.25, 0.25 + 2 ** -12, 2.0 ** -16, 2.0 ** -17, 2.0 ** -24, 6e-8, 0.3, 0.0],
+                        g.random(54) * 0.5 * 10.0 ** -g.integers(0, 6, 54)])
+    law = _fp16_law(y)[None, :]
+    pl, cls = oracle.law_layers(law)
+    tf = [int(min(float(np.float16(v)) * 2.0 ** 32, 4294967040.0)) for v in y]
+    def klass(t):
+        for k in range(15):
+            if (1 << (30 - k)) < t <= (1 << (31 - k)):
+                return k
+        return 15 if t > 0 else 16
+    ks = [klass(t) for t in tf]
+    assert klass(1 << 31) == 0 and klass((1 << 30) + 1) == 0 and klass(1 << 30) == 1 and klass(1) == 15
+    want = sorted(range(len(y)), key=lambda c: (ks[c], c))
+    n_live = sum(k < 16 for k in ks)
+    assert [int(e & 0xFFFF) for e in pl[0, :n_live]] == want[:n_live]
+    assert all(int(pl[0, i] >> 16) == int(law[0, want[i]]) for i in range(n_live))
+    assert (pl[0, n_live:] == 0xFFFF).all()
+    assert [int(c) for c in cls[0]] == [sum(k < c for k in ks) for c in range(17)]
+    # (2) one class per row: the thinned walk with the class's table
+    C, D = 333, 3
+    for k in (0, 1, 3, 6, 11, 15):
+        lo = 2.0 ** -(k + 2) * (1 + 2.0 ** -9) if k < 15 else 2.0 ** -24   # the boundary itself is class k + 1
+        yk = (lo + (2.0 ** -(k + 1) - lo) * g.random((2, C))).astype(np.float16)
+        yk[0, :5] = 2.0 ** -(k + 1)                                      # the class's upper end: always accepted
+        lawk = _fp16_law(yk)
+        plk, clsk = oracle.law_layers(lawk)
+        assert (clsk[:, k] == 0).all() and (clsk[:, k + 1] == C).all(), k
+        for first in (0, 3):
+            got = oracle.skip_flips_layered(plk, clsk, 11, 2, first, D)
+            thin = oracle.skip_flips_thin(lawk, cdfs[k, :kts[k]], 1 << (31 - k), 11, 2, first, D)
+            np.testing.assert_array_equal(got, thin, err_msg="class %d first %d" % (k, first))
+    # (3) mixed rows
+    R, C, D = 3, 700, 3
+    y = (g.random((R, C)) * 0.5 * 10.0 ** -g.integers(0, 5, (R, C))).astype(np.float16)
+    y[1, ::7] = 0.0
+    law = _fp16_law(y)
+    pl, cls = oracle.law_layers(law)
+    tfs = oracle.law_thresholds(law).astype(np.uint64)
+    seed, sub = 0xABCDE, 1
+    for first in (0, 2, 5):
+        got = np.unpackbits(oracle.skip_flips_layered(pl, cls, seed, sub, first, D).view(np.uint8), axis=1,
+                            bitorder="little")
+        assert not got[:, C:].any()
+        for q in range(D * R):
+            r = q % R
+            words = oracle.philox_words(seed, sub, first + q * C, 2 * C + 64)
+            want = np.zeros(got.shape[1], np.uint8)
+            at = 0                                                        # pairs used so far
+            for k in range(16):
+                s0, s1 = int(cls[r, k]), int(cls[r, k + 1])
+                if s1 == s0:
+                    continue
+                gap, acc = words[2 * at::2], words[2 * at + 1::2]
+                cdf = cdfs[k, :kts[k]]
+                rank = np.searchsorted(cdf, gap, side="right").astype(np.int64)
+                pos = np.cumsum(np.where(rank < len(cdf), rank + 1, len(cdf))) - 1
+                used = int(np.argmax(pos >= s1 - s0)) + 1                 # the pair that leaves the class is used up
+                for i in range(used - 1):
+                    if rank[i] < len(cdf):
+                        col = int(pl[r, s0 + pos[i]] & 0xFFFF)
+                        if int(acc[i]) < (int(tfs[r, col]) << (k + 1)):
+                            want[col] = 1
+                at += used
+            np.testing.assert_array_equal(got[q], want, err_msg="first=%d row %d" % (first, q))
+    # (4) rates
+    C2, D2 = 256, 20000
+    levels = np.array([0.4, 0.11, 0.03, 0.004, 0.0003, 0.26, 0.0625, 0.001], dtype=np.float16)
+    y2 = levels[np.arange(C2) % 8]
+    pl2, cls2 = oracle.law_layers(_fp16_law(y2)[None, :])
+    bits = np.unpackbits(oracle.skip_flips_layered(pl2, cls2, 9, 0, 0, D2).view(np.uint8), axis=1,
+                         bitorder="little")[:, :C2].astype(np.float64)
+    p2 = y2.astype(np.float64)
+    rate = bits.mean(axis=0)
+    assert (np.abs(rate - p2) < 5 * np.sqrt(p2 * (1 - p2) / D2)).all()
+    for j in range(8):
+        pj = float(levels[j])
+        assert abs(rate[j::8].mean() - pj) < 4.5 * np.sqrt(pj * (1 - pj) / (D2 * C2 / 8)), j
+    a, b = bits[:, 0::8], bits[:, 5::8]                                   # columns of the same class (0.4 and 0.26)
+    pa, pb = float(levels[0]), float(levels[5])
+    assert abs((a * b).mean() - pa * pb) < 5 * np.sqrt(pa * pb / a.size)
+    a, b = bits[:, 1::8], bits[:, 2::8]                                   # of neighbouring classes
+    pa, pb = float(levels[1]), float(levels[2])
+    assert abs((a * b).mean() - pa * pb) < 5 * np.sqrt(pa * pb / a.size)
+
+
 def test_draws16_against_a_numpy_evaluation_ties_and_rates(oracle):
     """Bernoulli draws from 16-bit half-words: the C restatement against an evaluation in numpy from the pinned
     Philox words (first stream: half-words; second stream, subsequence ^ 2**63: the tie-breaking low halves), with
