@@ -435,6 +435,18 @@ def hbm_kernels(torch, steps, warmup, graph=True, core=False):
     run("flip_rows_skip D=4096 [1024 x 8192], p=0.01 (bytes written)",
         lambda: ops.flip_rows_skip(b4, 8192, 4096, workloads.T_P01, 0, subsequence=13), rows.nbytes())
     del rows, x4, thr4, ex, G
+    # the same layer's lists under the per-element law of latent weights whose magnitudes spread by 10 % (flip
+    # probabilities of 0.8 % on average, 8 % at most): one walk at the largest probability against class by class
+    sign = torch.randint(0, 2, (1024, 8192), device=dev, generator=g) * 2 - 1
+    law = ops.flip_law_from_weights((sign * (1.0 + 0.1 * torch.randn((1024, 8192), device=dev, generator=g))).half())
+    cap = ops.flip_capacity(8192, 0.009)
+    rows = ops.flip_rows_layered(law, 4096, 0, cap)
+    assert rows.overflowed() == 0
+    run("flip_rows_thin D=4096 [1024 x 8192], per-element law (bytes written)",
+        lambda: ops.flip_rows_thin(law, 4096, 0, cap), rows.nbytes())
+    run("flip_rows_layered D=4096 [1024 x 8192], per-element law (bytes written)",
+        lambda: ops.flip_rows_layered(law, 4096, 0, cap), rows.nbytes())
+    del rows, law, sign
     # a conv layer's filters (128 x 3x3 taps of 64 channels) at p = 0.01 for 4096 members, both layouts: the skip
     # sampler as packed words against one draw per bit
     bc = torch.randint(-2 ** 62, 2 ** 62, (1152, 1), device=dev, generator=g, dtype=torch.int64)

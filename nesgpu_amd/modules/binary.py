@@ -227,6 +227,9 @@ class BinarizedLinear(Binarized):
         if sparse not in (True, False, "auto"):
             raise ValueError("sparse must be True, False or 'auto'")
         self.sparse = sparse
+        # per-element laws in the sparse form: "thin" (one walk at the largest probability), "layered" (class by class)
+        # or "auto" (whichever takes fewer steps)
+        self.sparse_walk = "auto"
         if pack_output and not threshold:
             raise NotImplementedError("packed output needs threshold=True")
         self.pack_output = pack_output    # not in the reference: return the thresholded row packed, from one kernel
@@ -267,9 +270,9 @@ class BinarizedLinear(Binarized):
         if self.in_features < 2048:
             return False
         plan = self._sparse_plan()
-        # two bytes per flip against a bit per weight: worth it below one flip in sixteen bits; the thinned walk draws
-        # two words per candidate, at the largest probability of the layer
-        return plan["mean"] <= 0.04 and plan["peak"] <= 0.25
+        # a row's lists cost a few steps per flip where the dense sampler draws every bit: worth it below about one
+        # flip in twenty-five bits, whatever the largest probability (a law with a long tail is walked class by class)
+        return plan["mean"] <= 0.04
 
     def _sample_sparse(self):
         plan = self._sparse_plan()
@@ -280,7 +283,19 @@ class BinarizedLinear(Binarized):
                 "antibase", self.weight, lambda: booleanOperations.pack(self.weight.detach() < 0, self.dtype))
             T = min(int(min(p, 1.0 - p) * 4294967296.0), 0xFFFFFFFF)
             return booleanOperations.flip_rows_skip(base, self.in_features, self.directions, T, self.seed, cap=cap)
+        if self._sparse_walk_now() == "layered":
+            return booleanOperations.flip_rows_layered(plan["law"], self.directions, self.seed, cap)
         return booleanOperations.flip_rows_thin(plan["law"], self.directions, self.seed, cap)
+
+    def _sparse_walk_now(self):
+        """Which walk draws the lists of a per-element law: ``sparse_walk``, or for "auto" the one with fewer steps
+        per row: thinning walks at the layer's largest probability; the class-by-class walk takes about three steps
+        for two flips (every class accepts at least every second candidate) and a few per class."""
+        if self.sparse_walk != "auto":
+            return self.sparse_walk
+        plan = self._sparse_plan()
+        C = self.in_features
+        return "layered" if C * plan["peak"] > 1.5 * C * plan["mean"] + 12 else "thin"
 
     def forward(self, input):
         if not self.perturbed_flag:

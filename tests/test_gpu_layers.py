@@ -384,7 +384,7 @@ def _saturated(shape, g, lo=0.9, hi=1.6):
     return w.to(torch.float16)
 
 
-@pytest.mark.parametrize("mode", ["law", "flip_probability"])
+@pytest.mark.parametrize("mode", ["law", "law_layered", "flip_probability"])
 @pytest.mark.parametrize("threshold,batch_norm,pack_output", [(True, False, True), (True, False, False),
                                                               (False, False, False), (True, True, False)])
 def test_wide_linear_layer_in_sparse_form(binary, oracle, mode, threshold, batch_norm, pack_output):
@@ -401,19 +401,30 @@ def test_wide_linear_layer_in_sparse_form(binary, oracle, mode, threshold, batch
         lin.weight.copy_(_saturated((M, K), g))
         if threshold:
             lin.bias.copy_((torch.randn(M, device="cuda", generator=g) * 20).to(torch.float16))
+    if mode.startswith("law"):
+        assert lin.sparse_walk == "auto" and lin._sparse_walk_now() == "layered"   # largest probability: 4 x the mean
+        lin.sparse_walk = "layered" if mode == "law_layered" else "thin"
     lin.set_seed(77)
     lin.set_noise()
     rows = lin.weight_noise
     assert isinstance(rows, ops.FlipRows) and rows.overflowed() == 0
     # the members' weights, regenerated on the host
-    if mode == "law":
+    if mode.startswith("law"):
         P = lin.probabilities().cpu().numpy()
         law_np, base_bits, tmax = oracle.flip_law(P)
         plan = lin._sparse_plan()
         np.testing.assert_array_equal(plan["law"].law.view(torch.int16).cpu().numpy().view(np.uint16), law_np)
         th = plan["law"].table.view(torch.int32).cpu().numpy().view(np.uint32)
         assert int(th[2]) == tmax
-        flips = oracle.skip_flips_thin(law_np, th[4:4 + int(th[0])].copy(), tmax, 77, 0, 0, D)
+        if mode == "law":
+            flips = oracle.skip_flips_thin(law_np, th[4:4 + int(th[0])].copy(), tmax, 77, 0, 0, D)
+        else:
+            words = int(ops._lib.load().nb_skip_table_words())
+            tb = ops.layer_tables("cuda").view(torch.int32).cpu().numpy().view(np.uint32).reshape(16, words)
+            cdfs, kts = oracle.layer_tables()
+            for k in range(16):
+                cdfs[k, :kts[k]] = tb[k, 4:4 + kts[k]]                           # the tables are input data
+            flips = oracle.skip_flips_layered(*oracle.law_layers(law_np), 77, 0, 0, D, tables=(cdfs, kts))
         base = oracle.pack(base_bits, np.int64)
     else:
         base = oracle.pack(lin.weight.detach().cpu().numpy() >= 0, np.int64)
@@ -461,8 +472,17 @@ def test_sparse_form_is_chosen_by_the_flip_probabilities(binary):
         lin.weight.copy_(_saturated((16, 2048), g))
     lin.set_noise()
     assert isinstance(lin.weight_noise, ops.FlipRows)
+    assert lin._sparse_walk_now() == "layered"               # probabilities between 0.2 % and 3 %
     with torch.no_grad():
-        lin.weight[3, 5] = 0.0                               # one undecided weight: walking at 1/2 would not pay
+        lin.weight.copy_(torch.sign(lin.weight))             # one magnitude: one probability, one walk at it
+    lin.set_noise()
+    assert isinstance(lin.weight_noise, ops.FlipRows) and lin._sparse_walk_now() == "thin"
+    with torch.no_grad():
+        lin.weight[3, 5] = 0.0                               # one undecided weight: a class of its own
+    lin.set_noise()
+    assert isinstance(lin.weight_noise, ops.FlipRows) and lin._sparse_walk_now() == "layered"
+    with torch.no_grad():
+        lin.weight[:, ::4] *= 0.125                          # a quarter of the weights near 1/2: too many flips
     lin.set_noise()
     assert isinstance(lin.weight_noise, torch.Tensor)
     narrow = binary.BinarizedLinear(1024, 16, 8)
