@@ -404,14 +404,28 @@ __device__ __forceinline__ void skip_table_build(uint32_t *table, const uint32_t
 // P = fp16(sigmoid(float(fp16(fp16(w / m) * 5)))) with m = fp16(mean|w| + 1e-5), every step rounded to fp16 where the
 // tensor expression of modules/binary.py:59-60 rounds it.  mean|w| is the exact sum (fp16 values add exactly in a
 // double) divided by the count and rounded once to fp16.
-constexpr int kLawBlocks = 256;   // partial sums
+constexpr int kLawBlocks = 256;   // doubles of workspace: up to 255 partial sums, then the denominator
 
 __global__ __launch_bounds__(256) void law_abs_sum_kernel(double *__restrict__ partial, uint32_t *__restrict__ table,
                                                           const _Float16 *__restrict__ w, int64_t n)
 {
     __shared__ double red[4];
     double s = 0.0;
-    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256)
+    // eight weights per load where the array allows it
+    const int64_t n8 = (reinterpret_cast<uintptr_t>(w) & 15u) == 0 ? n >> 3 : 0;
+    const uint4 *w8 = reinterpret_cast<const uint4 *>(w);
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n8; i += (int64_t)gridDim.x * 256) {
+        const uint4 v = w8[i];
+        const uint32_t d[4] = {v.x, v.y, v.z, v.w};
+        double t = 0.0, u = 0.0;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            t += (double)fabsf((float)__builtin_bit_cast(_Float16, (uint16_t)(d[e] & 0xFFFFu)));
+            u += (double)fabsf((float)__builtin_bit_cast(_Float16, (uint16_t)(d[e] >> 16)));
+        }
+        s += t + u;
+    }
+    for (int64_t i = 8 * n8 + (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256)
         s += (double)fabsf((float)w[i]);
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o);
@@ -423,12 +437,23 @@ __global__ __launch_bounds__(256) void law_abs_sum_kernel(double *__restrict__ p
     }
 }
 
-__device__ __forceinline__ _Float16 law_denominator(const double *partial, int nparts, int64_t n)
+// The partial sums added in index order, by one thread, into the denominator fp16(mean|w| + 1e-5); it is left in the
+// workspace's last slot (as a double: exact) for the kernels that follow.
+__global__ __launch_bounds__(256) void law_denominator_kernel(double *partial, int nparts, int64_t n)
 {
+    __shared__ double part[kLawBlocks];
+    part[threadIdx.x] = (int)threadIdx.x < nparts ? partial[threadIdx.x] : 0.0;
+    __syncthreads();
+    if (threadIdx.x != 0) return;
     double s = 0.0;
-    for (int i = 0; i < nparts; i++) s += partial[i];   // the same order in every thread: all agree
+    for (int i = 0; i < nparts; i++) s += part[i];
     const _Float16 mean = double_round_once_fp16(s / (double)n);
-    return (_Float16)((float)mean + 1e-5f);
+    partial[kLawBlocks - 1] = (double)(float)(_Float16)((float)mean + 1e-5f);
+}
+
+__device__ __forceinline__ _Float16 law_denominator(const double *partial)
+{
+    return (_Float16)(float)partial[kLawBlocks - 1];
 }
 
 __device__ __forceinline__ _Float16 law_probability(_Float16 w, _Float16 denom)
@@ -448,9 +473,9 @@ __device__ __forceinline__ uint32_t law_threshold(_Float16 p)   // min(floor(p *
 template <int MODE>
 __global__ __launch_bounds__(256) void law_dense_kernel(uint32_t *__restrict__ out32, _Float16 *__restrict__ out16,
                                                         const _Float16 *__restrict__ w, const double *__restrict__ partial,
-                                                        int nparts, int64_t n)
+                                                        int64_t n)
 {
-    const _Float16 denom = law_denominator(partial, nparts, n);
+    const _Float16 denom = law_denominator(partial);
     NB_FLAT_LOOP(t, n)
     {
         if (t < n) {
@@ -466,10 +491,10 @@ __global__ __launch_bounds__(256) void law_dense_kernel(uint32_t *__restrict__ o
 // kernel).  One wave per 64 columns of a row: the ballot of the base bits is the packed word.
 __global__ __launch_bounds__(256) void law_sparse_kernel(uint16_t *__restrict__ law, uint64_t *__restrict__ base,
                                                          uint32_t *__restrict__ table, const _Float16 *__restrict__ w,
-                                                         const double *__restrict__ partial, int nparts, int64_t R,
+                                                         const double *__restrict__ partial, int64_t R,
                                                          int C, int Kw)
 {
-    const _Float16 denom = law_denominator(partial, nparts, R * (int64_t)C);
+    const _Float16 denom = law_denominator(partial);
     const int lane = threadIdx.x & 63;
     uint32_t tmax = 0;
     for (int64_t wd = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6); wd < R * Kw; wd += (int64_t)gridDim.x * 4) {
@@ -493,7 +518,14 @@ __global__ __launch_bounds__(256) void law_sparse_kernel(uint16_t *__restrict__ 
         const uint32_t other = (uint32_t)__shfl_xor((int)tmax, o);
         tmax = tmax > other ? tmax : other;
     }
-    if (lane == 0 && tmax) atomicMax(table + 2, tmax);
+    // one atomic per workgroup: they all go to the same word
+    __shared__ uint32_t wave_tmax[4];
+    if (lane == 0) wave_tmax[threadIdx.x >> 6] = tmax;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < 4; w++) tmax = tmax > wave_tmax[w] ? tmax : wave_tmax[w];
+        if (tmax) atomicMax(table + 2, tmax);
+    }
 }
 
 // thr may be table + 2 (the threshold read before anything is written, and written back unchanged)
@@ -590,47 +622,76 @@ __global__ __launch_bounds__(1024) void fl_layer_tables_kernel(uint32_t *tables)
     skip_table_build(tables + (size_t)blockIdx.x * kLayerWords, &thr);
 }
 
-// One wave per row: count the classes, then place every column (stable: increasing column inside a class).
-__global__ __launch_bounds__(256) void law_layers_kernel(uint32_t *__restrict__ pl, uint32_t *__restrict__ cls,
-                                                         const uint16_t *__restrict__ law, int64_t R, int C)
+// One workgroup of 16 waves per row, a wave per stretch of its columns: count the classes, then place every column
+// (stable: increasing column inside a class; a class's columns of an earlier stretch come first).
+__global__ __launch_bounds__(1024) void law_layers_kernel(uint32_t *__restrict__ pl, uint32_t *__restrict__ cls,
+                                                          const uint16_t *__restrict__ law, int C)
 {
-    const int lane = threadIdx.x & 63;
-    const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (r >= R) return;
+    extern __shared__ uint32_t gen_lds[];
+    uint32_t *sorted = gen_lds;                                         // the row in its new order: C words
+    __shared__ uint32_t cnt[16][kLayers];
+    __shared__ uint32_t cstart[kLayers + 1];
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const int64_t r = blockIdx.x;
     const uint16_t *row = law + r * C;
+    const int per = ((C + 63) / 64 + 15) / 16 * 64;                    // columns of a stretch
+    const int cbeg = wv * per, cend = cbeg + per < C ? cbeg + per : C;
     uint32_t count[kLayers];
 #pragma unroll
     for (int k = 0; k < kLayers; k++) count[k] = 0;
-    for (int c0 = 0; c0 < C; c0 += 64) {
+    for (int c0 = cbeg; c0 < cend; c0 += 64) {
         const int c = c0 + lane;
-        const int k = c < C ? law_class(law_threshold16(row[c])) : kLayers;
+        const int k = c < cend ? law_class(law_threshold16(row[c])) : kLayers;
 #pragma unroll
         for (int kk = 0; kk < kLayers; kk++) count[kk] += (uint32_t)__popcll(__ballot(k == kk));
     }
-    uint32_t offs[kLayers];
-    uint32_t run = 0;
 #pragma unroll
-    for (int k = 0; k < kLayers; k++) {
-        offs[k] = run;
-        if (lane == 0) cls[r * (kLayers + 1) + k] = run;
-        run += count[k];
+    for (int k = 0; k < kLayers; k++)
+        if (lane == 0) cnt[wv][k] = count[k];
+    __syncthreads();
+    // thread k < 16: where each wave's columns of class k go, inside the class; then where the classes start
+    if (threadIdx.x < kLayers) {
+        uint32_t acc = 0;
+        for (int w = 0; w < 16; w++) {
+            const uint32_t v = cnt[w][threadIdx.x];
+            cnt[w][threadIdx.x] = acc;
+            acc += v;
+        }
+        cstart[threadIdx.x] = acc;
     }
-    if (lane == 0) cls[r * (kLayers + 1) + kLayers] = run;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        uint32_t acc = 0;
+        for (int k = 0; k < kLayers; k++) {
+            const uint32_t v = cstart[k];
+            cstart[k] = acc;
+            cls[r * (kLayers + 1) + k] = acc;
+            acc += v;
+        }
+        cstart[kLayers] = acc;
+        cls[r * (kLayers + 1) + kLayers] = acc;
+    }
+    __syncthreads();
+    uint32_t offs[kLayers];
+#pragma unroll
+    for (int k = 0; k < kLayers; k++) offs[k] = cstart[k] + cnt[wv][k];
+    const uint32_t run = cstart[kLayers];
     const unsigned long long below = (1ull << lane) - 1ull;
-    uint32_t *out = pl + r * C;
-    for (int c0 = 0; c0 < C; c0 += 64) {
+    for (int c0 = cbeg; c0 < cend; c0 += 64) {
         const int c = c0 + lane;
-        const uint32_t l = c < C ? row[c] : 0u;
-        const int k = c < C ? law_class(law_threshold16(l)) : kLayers;
+        const uint32_t l = c < cend ? row[c] : 0u;
+        const int k = c < cend ? law_class(law_threshold16(l)) : kLayers;
 #pragma unroll
         for (int kk = 0; kk < kLayers; kk++) {
             const unsigned long long m = __ballot(k == kk);
-            if (k == kk) out[offs[kk] + (uint32_t)__popcll(m & below)] = (uint32_t)c | (l << 16);
+            if (k == kk) sorted[offs[kk] + (uint32_t)__popcll(m & below)] = (uint32_t)c | (l << 16);
             offs[kk] += (uint32_t)__popcll(m);
         }
     }
-    // the columns that never flip fill the rest of the row (never read by the walk)
-    for (uint32_t i = run + lane; i < (uint32_t)C; i += 64) out[i] = 0xFFFFu;
+    __syncthreads();
+    // the row leaves in whole lines; the columns that never flip fill its end (never read by the walk)
+    uint32_t *out = pl + r * C;
+    for (uint32_t i = threadIdx.x; i < (uint32_t)C; i += 1024) out[i] = i < run ? sorted[i] : 0xFFFFu;
 }
 
 struct LayerArgs {
@@ -640,6 +701,7 @@ struct LayerArgs {
     PhiloxKey key;
     int64_t D, R;
     int C, Kw, S, cap, MC, rb_shift;
+    int batch;   // lanes of a wave that end their rows together
 };
 
 // INLDS: the workgroup's rows of pl are staged in LDS; else (rows too long for that) read where they lie.
@@ -769,10 +831,14 @@ __global__ __launch_bounds__(1024) void fl_gen_layered_kernel(const LayerArgs a)
     };
     start_row();
     while (__any(live)) {
-        if (live) {
-            if (cur >= kLayers) {
-                finish_row();      // also rows without a column that can flip
-            } else if (ALIGNED) {
+        // A lane whose row has ended waits until `batch` lanes of the wave have (or none is walking): the wave then
+        // goes through the end of a row and the start of the next once for all of them, not in every turn.
+        const bool ended = live && cur >= kLayers;   // also rows without a column that can flip
+        if (__popcll(__ballot(ended)) >= a.batch || !__any(live && !ended)) {
+            if (ended) finish_row();
+        }
+        if (live && cur < kLayers) {
+            if (ALIGNED) {
                 const uint4 w = philox_block(a.key, blk++);
                 step(rank_of(w.x), w.y);
                 if (cur < kLayers) step(rank_of(w.z), w.w);
@@ -797,6 +863,8 @@ static int layered_launch(LayerArgs a, hipStream_t s, const char *who)
     if (const char *e = getenv("NESBIN_LAYERED_LDS")) inlds = inlds && atoi(e) != 0;
     if (!inlds) shift = 3;
     a.rb_shift = shift;
+    a.batch = 4;
+    if (const char *e = getenv("NESBIN_LAYERED_BATCH")) a.batch = std::max(1, std::min(64, atoi(e)));
     const size_t lds = fixed + (inlds ? row_bytes << shift : 0);
     const int threads = 1024;
     const int slots = threads >> shift;
@@ -1119,8 +1187,7 @@ int nb_flip_layer_tables(uint32_t *tables, nb_stream_t stream)
 int nb_flip_law_layers(uint32_t *pl, uint32_t *cls, const uint16_t *law, int64_t R, int64_t C, nb_stream_t stream)
 {
     const char *who = "nb_flip_law_layers";
-    NB_REQUIRE(R >= 0 && C >= 0 && C <= 65535 && R <= (1LL << 31), "%s: R=%lld, C=%lld out of range (C at most 65535)", who,
-               (long long)R, (long long)C);
+    NB_REQUIRE(R >= 0 && C >= 0, "%s: negative shape R=%lld, C=%lld", who, (long long)R, (long long)C);
     if (R == 0) return NB_OK;
     NB_REQUIRE_PTR(cls);
     NB_REQUIRE_ALIGNED(cls, 4);
@@ -1130,9 +1197,19 @@ int nb_flip_law_layers(uint32_t *pl, uint32_t *cls, const uint16_t *law, int64_t
         NB_REQUIRE_ALIGNED(pl, 4);
         NB_REQUIRE_ALIGNED(law, 2);
     }
-    const int64_t blocks = nb::ceil_div(R, 4);
-    NB_REQUIRE(blocks <= nb::kMaxGridX, "%s: too many rows for one launch", who);
-    nb::law_layers_kernel<<<dim3((unsigned)blocks), dim3(256), 0, nb::as_stream(stream)>>>(pl, cls, law, R, (int)C);
+    NB_REQUIRE(R <= nb::kMaxGridX, "%s: too many rows for one launch", who);
+    NB_REQUIRE(C <= 511 * 64, "%s: rows of %lld columns, at most %d", who, (long long)C, 511 * 64);
+    static std::once_flag once;
+    static hipError_t attr = hipSuccess;
+    std::call_once(once, [] {
+        attr = hipFuncSetAttribute(reinterpret_cast<const void *>(nb::law_layers_kernel),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, 511 * 64 * 4);
+    });
+    if (attr != hipSuccess) {
+        (void)hipGetLastError();
+        return nb::fail(NB_ERR_UNSUPPORTED, "%s: cannot raise the kernel's LDS limit: %s", who, hipGetErrorString(attr));
+    }
+    nb::law_layers_kernel<<<dim3((unsigned)R), dim3(1024), (size_t)C * 4, nb::as_stream(stream)>>>(pl, cls, law, (int)C);
     return nb::check_launch(who);
 }
 
@@ -1206,9 +1283,11 @@ static int law_sum(double *ws, uint32_t *table, const uint16_t *w, int64_t n, hi
     NB_REQUIRE_ALIGNED(ws, 8);
     NB_REQUIRE_PTR(w);
     NB_REQUIRE_ALIGNED(w, 2);
-    const int64_t blocks = std::min<int64_t>(nb::kLawBlocks, nb::ceil_div(n, 2048));
+    const int64_t blocks = std::min<int64_t>(nb::kLawBlocks - 1, nb::ceil_div(n, 2048));
     *nparts = (int)blocks;
     nb::law_abs_sum_kernel<<<dim3((unsigned)blocks), dim3(256), 0, s>>>(ws, table, reinterpret_cast<const _Float16 *>(w), n);
+    if (int rc = nb::check_launch(who)) return rc;
+    nb::law_denominator_kernel<<<dim3(1), dim3(nb::kLawBlocks), 0, s>>>(ws, (int)blocks, n);
     return nb::check_launch(who);
 }
 
@@ -1224,7 +1303,7 @@ int nb_thresholds_from_weights(uint32_t *thresholds, const uint16_t *weights, in
     if (int rc = law_sum(static_cast<double *>(workspace), nullptr, weights, n, nb::as_stream(stream), &nparts, who))
         return rc;
     nb::law_dense_kernel<0><<<dim3(nb::grid_for(n)), dim3(256), 0, nb::as_stream(stream)>>>(
-        thresholds, nullptr, reinterpret_cast<const _Float16 *>(weights), static_cast<const double *>(workspace), nparts, n);
+        thresholds, nullptr, reinterpret_cast<const _Float16 *>(weights), static_cast<const double *>(workspace), n);
     return nb::check_launch(who);
 }
 
@@ -1240,7 +1319,7 @@ int nb_probabilities_from_weights(uint16_t *p, const uint16_t *weights, int64_t 
         return rc;
     nb::law_dense_kernel<1><<<dim3(nb::grid_for(n)), dim3(256), 0, nb::as_stream(stream)>>>(
         nullptr, reinterpret_cast<_Float16 *>(p), reinterpret_cast<const _Float16 *>(weights),
-        static_cast<const double *>(workspace), nparts, n);
+        static_cast<const double *>(workspace), n);
     return nb::check_launch(who);
 }
 
@@ -1261,10 +1340,10 @@ int nb_flip_law_from_weights(uint16_t *law, int64_t *base, uint32_t *table, cons
     int nparts = 0;
     if (int rc = law_sum(static_cast<double *>(workspace), table, weights, R * C, nb::as_stream(stream), &nparts, who))
         return rc;
-    const int64_t blocks = std::min<int64_t>(nb::ceil_div(R * Kw, 4), 65536);
+    const int64_t blocks = std::min<int64_t>(nb::ceil_div(R * Kw, 4), 2048);
     nb::law_sparse_kernel<<<dim3((unsigned)blocks), dim3(256), 0, nb::as_stream(stream)>>>(
         law, reinterpret_cast<uint64_t *>(base), table, reinterpret_cast<const _Float16 *>(weights),
-        static_cast<const double *>(workspace), nparts, R, (int)C, (int)Kw);
+        static_cast<const double *>(workspace), R, (int)C, (int)Kw);
     if (int rc = nb::check_launch(who)) return rc;
     nb::fl_skip_table_kernel<<<dim3(1), dim3(1024), 0, nb::as_stream(stream)>>>(table, table + 2);
     return nb::check_launch(who);

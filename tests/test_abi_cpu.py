@@ -114,7 +114,7 @@ def test_bad_arguments_are_rejected_without_a_launch(lib):
     assert lib.nb_flip_skip_layered_i64(big, one, one, ctypes.c_void_p(6), one, one, 1, 0, 0, 2, 64, 64, 4, None) == 3
     assert lib.nb_flip_skip_layered_i64(big, one, one, one, one, one, 1, 0, 0, 2, 64, 512 * 64, 4, None) == 2  # row too long
     assert lib.nb_flip_law_layers(one, None, one, 4, 64, None) == 1
-    assert lib.nb_flip_law_layers(one, one, one, 4, 70000, None) == 2
+    assert lib.nb_flip_law_layers(one, one, one, 4, 512 * 64, None) == 2
     assert lib.nb_flip_law_layers(None, None, None, 0, 64, None) == 0
     assert lib.nb_flip_layer_tables(None, None) == 1
     assert lib.nb_flip_layer_table_words() == 16 * 4100
