@@ -633,6 +633,26 @@ def main():
                         "kernels' own time"}
             del cap, cap1, cap16, pm1
         del sn, fw, up
+        # configuration 5's wide layer under the reference's own per-weight law, through the layer: base + flip lists
+        # drawn class by class against the materialised form (every bit drawn)
+        law = {"workload": "BinarizedLinear(8192, 1024, 4096) under P = sigmoid(5 w / mean|w|), latent weights "
+                           "+-(1 + 0.1 N(0,1)): one NES step, ms (eager launches)"}
+        for name, kw in (("flip_lists_class_by_class", dict(sparse=True, walk="layered")),
+                         ("flip_lists_thinning", dict(sparse=True, walk="thin")),
+                         ("materialised", dict(sparse=False))):
+            lin, sn, fw, up = workloads.wide_linear_law_step(**kw)
+            law[name] = {"set_noise_ms": round(time_steps(torch, sn, 5, 2)[0] * 1e3, 3),
+                         "forward_ms": round(time_steps(torch, fw, 5, 2)[0] * 1e3, 3),
+                         "update_ms": round(time_steps(torch, up, 5, 2)[0] * 1e3, 3)}
+            if kw.get("sparse"):
+                plan = lin._sparse_plan()
+                law["mean_flip_probability"], law["largest_flip_probability"] = round(plan["mean"], 5), round(plan["peak"], 4)
+                lin.sparse_walk = "auto"
+                law["walk_chosen_by_the_layer"] = lin._sparse_walk_now()
+            lin.free_memory()
+            del lin, sn, fw, up
+            torch.cuda.empty_cache()
+        line["per_weight_law_layer"] = law
     # the helper kernels the 70 %-of-HBM target names, each alone, after everything above has warmed the clocks
     line["hbm_kernels"] = [{"kernel": k["kernel"], "us": k["us"], "hbm_frac": k["hbm_frac"], "timing": k["timing"]}
                            for k in hbm_kernels(torch, max(10, args.steps // 4), 5, not args.no_graph, core=True)]

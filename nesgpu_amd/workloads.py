@@ -385,3 +385,32 @@ def linear_layer_config1(D=1024, device="cuda", seed=0):
 
 
 BUILDERS = {1: linear_flip_materialised, 2: linear_flip_fused, 3: conv_int32, 4: conv_sign_pool, 5: cifar_net}
+
+
+def wide_linear_law_step(D=4096, in_features=8192, out_features=1024, spread=0.1, sparse="auto", walk="auto", seed=0,
+                         device="cuda"):
+    """One NES step of configuration 5's 8192 -> 1024 layer under the reference's OWN law (per-weight probabilities
+    sigmoid(5 w / mean|w|), modules/binary.py:59-60) through ``BinarizedLinear``: latent weights +-(1 + spread *
+    N(0,1)), i.e. flip probabilities of 0.7 % and up with a tail that grows with ``spread``.  ``sparse`` / ``walk``:
+    the layer's ``sparse`` argument and ``sparse_walk`` attribute.  Returns (layer, set_noise, forward, update)."""
+    from .modules import binary
+    g = _gen(seed)
+    lin = binary.BinarizedLinear(in_features, out_features, D, threshold=True, pack_output=True, sparse=sparse,
+                                 device=device)
+    lin.sparse_walk = walk
+    shape = (out_features, in_features)
+    sign = torch.randint(0, 2, shape, generator=g) * 2 - 1
+    with torch.no_grad():
+        lin.weight.copy_((sign * (1.0 + spread * torch.randn(shape, generator=g))).to(torch.float16).to(device))
+    lin.set_seed(seed + 1)
+    lin.perturbed_flag = True
+    x = torch.randint(-2 ** 62, 2 ** 62, (D, (in_features + 63) // 64), generator=g, dtype=torch.int64).to(device)
+    fitness = torch.randn(D, generator=g).to(device)
+
+    def forward():
+        with torch.no_grad():
+            return lin(x)
+
+    lin.set_noise()
+    return lin, lin.set_noise, forward, lambda: lin.update(fitness)
+

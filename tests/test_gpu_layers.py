@@ -501,6 +501,29 @@ def test_sparse_form_is_chosen_by_the_flip_probabilities(binary):
     assert abs(flips - 0.01) < 0.002
 
 
+def test_wide_layer_workload_under_the_per_weight_law(binary, oracle):
+    """The bench's wide-layer workload at a small size: both walks give lists, the materialised form a tensor, and
+    each form's forward is the oracle's product on that form's own weights."""
+    from nesgpu_amd import workloads
+    from nesgpu_amd.extensions import booleanOperations as ops
+    D, K, M = 8, 2048, 16
+    for kw in (dict(sparse=True, walk="layered"), dict(sparse=True, walk="thin"), dict(sparse=False)):
+        lin, set_noise, forward, update = workloads.wide_linear_law_step(D=D, in_features=K, out_features=M, **kw)
+        sparse = isinstance(lin.weight_noise, ops.FlipRows)
+        assert sparse == bool(kw["sparse"])
+        W = (ops.flip_rows_to_weights(lin.weight_noise) if sparse else lin.weight_noise).cpu().numpy()
+        out = forward()
+        # the input the workload drew is not handed out: take the product on a fresh one
+        x = torch.randint(-2 ** 62, 2 ** 62, (D, K // 64), dtype=torch.int64, device="cuda")
+        with torch.no_grad():
+            got = lin(x)
+        act = 2 * oracle.bmm(W, x.cpu().numpy().reshape(D, -1, 1))[:, :, 0].astype(np.int64) - K
+        want = torch.from_numpy(act.astype(np.int32)).cuda() > (lin.bias + lin.bias_noise).detach()
+        assert torch.equal(got, ops.pack(want, torch.int64)) and got.shape == out.shape
+        update()
+        assert lin.weight.grad is not None and torch.isfinite(lin.weight.grad.float()).all()
+
+
 def test_update_helper_kernels_against_the_tensor_expressions(binary):
     """center_fitness, grad_regularize_ and bias_grad against the lines of modules/binary.py:67-77 they replace:
     the elementwise ones bit for bit (given the same mean), the two reductions against float64."""
