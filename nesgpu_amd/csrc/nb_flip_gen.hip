@@ -822,7 +822,8 @@ __global__ __launch_bounds__(1024) void fl_gen_layered_kernel(const LayerArgs a)
         } else if (rank < kt) {
             const uint32_t e = myrow[startk + pos];
             const uint32_t col = e & 0xFFFFu, l = e >> 16;
-            if ((uint64_t)acc < ((uint64_t)law_threshold16(l) << (cur + 1))) {
+            // accept < Tf * 2^(k+1) in 32 bits: the right side is even, so halve both (Tf * 2^k <= 2^31)
+            if ((acc >> 1) < (law_threshold16(l) << cur)) {
                 insert((((2u * (col >> 5)) + (l >> 15)) << 5) | (col & 31u));
                 n++;
                 if (++k == 8) flush();
