@@ -216,6 +216,10 @@ int nb_conv_bn_thresholds_from_input_i32(int32_t *thresh, const int32_t *in, con
  *                column reached flips iff the second word is below Tf * 2^(k+1); a position past the stretch ends
  *                the class and the next class that has columns starts with the next pair.  Same law as
  *                nb_flip_skip_thin (every column flips with probability Tf / 2^32, independently), other masks.
+ * Both per-element walks give row q the words from first + q*C on and use two per step, so a row that takes more than
+ * C/2 steps reads into the words of row q + 1 and the two rows' draws are no longer independent: they are meant for
+ * sparse laws (thinning takes about C * p_max steps, the class-by-class walk about 1.5 per flip plus 16;
+ * BinarizedLinear uses them for mean flip probabilities of at most 0.04).
  * The layers' law (modules/binary.py:59-60), P = sigmoid(5 w / (mean|w| + 1e-5)), rounded to fp16 wherever the tensor
  * expression rounds; mean|w| = the exact sum over the count, rounded once to fp16.  workspace: nb_law_workspace_bytes()
  * bytes of device memory, 8-byte aligned.

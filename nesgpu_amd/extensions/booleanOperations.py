@@ -1188,7 +1188,9 @@ def flip_rows_layered(law, n, seed, cap, subsequence=0, first=0):
     columns of a row are walked class by class (classes by the binary size of the flip probability, 2**-(k+2) < y <=
     2**-(k+1)), each class at its own rate 2**-(k+1), so that a row costs about two word pairs per flip whatever the
     layer's largest probability is, where :func:`flip_rows_thin` pays for that largest one in every column.  Same
-    law (every bit differs from the base with its own probability, independently), other masks."""
+    law (every bit differs from the base with its own probability, independently), other masks.  For sparse laws:
+    a row owns C words of the stream and uses two per step (about 1.5 steps per flip plus 16); a row that needs more
+    than its C words reads on into the next row's."""
     R, C = law.law.shape
     dev = law.law.device
     pl, cls = law.layers()
