@@ -385,6 +385,40 @@ def test_layered_sampler_vs_oracle(ops, oracle, D, R, C, first, mean):
         np.testing.assert_array_equal(bflag, mask & bb[None])
 
 
+@pytest.mark.parametrize("walk", ["layered", "thin"])
+def test_per_element_walks_report_rows_beyond_the_capacity(ops, oracle, walk):
+    """The per-element walks with a capacity below what some rows need: those rows are cut to capacity * 8 flips and
+    counted, the others are what they are with room to spare; and shapes at the edges (one row, one member, no
+    column that can flip) come out as empty or short lists."""
+    g = np.random.default_rng(8)
+    R, C, D = 70, 512, 9
+    P = long_tailed_law(g, R, C, 0.05)
+    law_np, base_bits, tmax = oracle.flip_law(P)
+    law = ops.flip_law_from_weights(torch.zeros((R, C), dtype=torch.float16, device="cuda"))   # for its table's place
+    law.law.copy_(dev(law_np.view(np.int16)).view(torch.uint16))
+    law.base.copy_(dev(oracle.pack(base_bits, np.int64)))
+    thr = torch.tensor([tmax], dtype=torch.int64, device="cuda").to(torch.int32)
+    ops._lib.call("nb_skip_table", law.table.data_ptr(), thr.data_ptr(), None)
+    draw = ops.flip_rows_layered if walk == "layered" else ops.flip_rows_thin
+    full = draw(law, D, 11, 64)
+    assert full.overflowed() == 0
+    need = (full.cnt + 7) // 8
+    cap = int(need.max().item()) - 1
+    cut = draw(law, D, 11, cap)
+    assert cut.overflowed() == int((need > cap).sum().item()) > 0
+    fine = (need <= cap)
+    assert torch.equal(cut.cnt[fine], full.cnt[fine]) and bool((cut.cnt[~fine] == 8 * cap).all())
+    Wc, Wf = ops.flip_rows_to_weights(cut), ops.flip_rows_to_weights(full)
+    assert torch.equal(Wc[fine], Wf[fine])
+    # nothing can flip: empty lists, the base itself
+    never = ops.FlipLaw(torch.zeros((3, 128), dtype=torch.uint16, device="cuda"),
+                        dev(sparse_mask(g, (3, 128), 0.5)), law.table, 128)
+    if walk == "layered":
+        rows = ops.flip_rows_layered(never, 5, 1, 2)
+        assert int(rows.cnt.sum().item()) == 0 and rows.overflowed() == 0
+        assert torch.equal(ops.flip_rows_to_weights(rows), never.base[None].expand(5, 3, 2))
+
+
 def test_layered_sampler_flip_rates_at_size(ops, oracle):
     """4096 members of a 64 x 8192 layer: every column's flip count against its own probability (binomial tails),
     and the lists stay inside the capacity chosen from the largest row mean."""
