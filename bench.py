@@ -65,6 +65,8 @@ def parse_args():
     ap.add_argument("--only", type=int, default=0, help="time just this configuration (for profiler runs)")
     ap.add_argument("--no-graph", action="store_true", help="skip the graph-replay timings of the other configurations")
     ap.add_argument("--no-step", action="store_true", help="skip the NES step of the SmallNet-shaped network")
+    ap.add_argument("--only-step", action="store_true",
+                    help="time just the NES step of the SmallNet-shaped network, phase after phase (for profiler runs)")
     ap.add_argument("--kernels", action="store_true",
                     help="time the HBM-bound helper kernels (pack, unpack, samplers, max-pool, im2col) on their own")
     return ap.parse_args()
@@ -518,6 +520,13 @@ def main():
 
     if args.kernels:
         print(json.dumps({"hbm_kernels": hbm_kernels(torch, args.steps, args.warmup, not args.no_graph)}))
+        return 0
+    if args.only_step:
+        sn, fw, up = workloads.small_net_step()
+        out = {}
+        for name, fn in (("set_noise_ms", sn), ("forward_ms", fw), ("update_ms", up)):
+            out[name] = round(time_steps(torch, fn, args.steps, args.warmup)[0] * 1e3, 4)
+        print(json.dumps({"nes_step_smallnet": out}))
         return 0
     if args.only:
         w = workloads.BUILDERS[args.only]()

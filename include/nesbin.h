@@ -235,6 +235,12 @@ int nb_flip_skip_i64(uint32_t *entries, uint32_t *info, uint32_t *overflow, cons
 int nb_flip_skip_thin_i64(uint32_t *entries, uint32_t *info, uint32_t *overflow, const uint16_t *law,
                           const uint32_t *table, uint64_t seed, uint64_t subseq, uint64_t first, int64_t D, int64_t R,
                           int64_t C, int64_t cap, nb_stream_t stream);
+/* stats[0..2] (doubles, device memory) = the mean flip probability of a law [R, C], the largest mean of a row, the
+ * largest flip probability (table[2] / 2^32, table as nb_flip_law_from_weights left it): what a host needs to choose
+ * between the dense and the sparse form, between the two walks, and the lists' capacity, in one read-back.
+ * row_sums: R floats of workspace. */
+int nb_flip_law_stats(double *stats, float *row_sums, const uint16_t *law, const uint32_t *table, int64_t R, int64_t C,
+                      nb_stream_t stream);
 int64_t nb_flip_layer_table_words(void);
 int nb_flip_layer_tables(uint32_t *tables, nb_stream_t stream);
 int nb_flip_law_layers(uint32_t *pl, uint32_t *cls, const uint16_t *law, int64_t R, int64_t C, nb_stream_t stream);

@@ -61,6 +61,7 @@ _PLAIN = {
     "nb_skip_table": [_PTR, _PTR, _PTR],
     "nb_flip_skip_i64": [_PTR, _PTR, _PTR, _PTR, _PTR, _U64, _U64, _U64, _I64, _I64, _I64, _I64, _PTR],
     "nb_flip_skip_thin_i64": [_PTR, _PTR, _PTR, _PTR, _PTR, _U64, _U64, _U64, _I64, _I64, _I64, _I64, _PTR],
+    "nb_flip_law_stats": [_PTR, _PTR, _PTR, _PTR, _I64, _I64, _PTR],
     "nb_flip_layer_tables": [_PTR, _PTR],
     "nb_flip_law_layers": [_PTR, _PTR, _PTR, _I64, _I64, _PTR],
     "nb_flip_skip_layered_i64": [_PTR, _PTR, _PTR, _PTR, _PTR, _PTR, _U64, _U64, _U64, _I64, _I64, _I64, _I64, _PTR],

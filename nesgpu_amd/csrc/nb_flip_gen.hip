@@ -528,6 +528,50 @@ __global__ __launch_bounds__(256) void law_sparse_kernel(uint16_t *__restrict__ 
     }
 }
 
+// What the host decides from (sparse form or not, which walk, the lists' capacity), in one read-back of three
+// doubles: the mean flip probability of the layer, the largest mean of a row, the largest flip probability.
+__global__ __launch_bounds__(256) void law_row_sums_kernel(float *__restrict__ rows, const uint16_t *__restrict__ law, int C)
+{
+    __shared__ float red[4];
+    const uint16_t *row = law + (int64_t)blockIdx.x * C;
+    float s = 0.f;
+    for (int c = threadIdx.x; c < C; c += 256) s += (float)__builtin_bit_cast(_Float16, (uint16_t)(row[c] & 0x7FFFu));
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = s;
+    __syncthreads();
+    if (threadIdx.x == 0) rows[blockIdx.x] = (red[0] + red[1]) + (red[2] + red[3]);
+}
+
+__global__ __launch_bounds__(256) void law_stats_kernel(double *__restrict__ stats, const float *__restrict__ rows,
+                                                        const uint32_t *__restrict__ table, int64_t R, int C)
+{
+    __shared__ double sum_sh[4];
+    __shared__ float max_sh[4];
+    double s = 0.0;
+    float m = 0.f;
+    for (int64_t r = threadIdx.x; r < R; r += 256) {
+        const float v = rows[r];
+        s += (double)v;
+        m = fmaxf(m, v);
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        s += __shfl_xor(s, o);
+        m = fmaxf(m, __shfl_xor(m, o));
+    }
+    if ((threadIdx.x & 63) == 0) {
+        sum_sh[threadIdx.x >> 6] = s;
+        max_sh[threadIdx.x >> 6] = m;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        stats[0] = ((sum_sh[0] + sum_sh[1]) + (sum_sh[2] + sum_sh[3])) / ((double)R * (double)C);
+        stats[1] = (double)fmaxf(fmaxf(max_sh[0], max_sh[1]), fmaxf(max_sh[2], max_sh[3])) / (double)C;
+        stats[2] = (double)table[2] / 4294967296.0;
+    }
+}
+
 // thr may be table + 2 (the threshold read before anything is written, and written back unchanged)
 __global__ __launch_bounds__(1024) void fl_skip_table_kernel(uint32_t *table, const uint32_t *thr)
 {
@@ -1321,6 +1365,26 @@ int nb_probabilities_from_weights(uint16_t *p, const uint16_t *weights, int64_t 
     nb::law_dense_kernel<1><<<dim3(nb::grid_for(n)), dim3(256), 0, nb::as_stream(stream)>>>(
         nullptr, reinterpret_cast<_Float16 *>(p), reinterpret_cast<const _Float16 *>(weights),
         static_cast<const double *>(workspace), n);
+    return nb::check_launch(who);
+}
+
+int nb_flip_law_stats(double *stats, float *row_sums, const uint16_t *law, const uint32_t *table, int64_t R, int64_t C,
+                      nb_stream_t stream)
+{
+    const char *who = "nb_flip_law_stats";
+    NB_REQUIRE(R > 0 && C > 0 && C <= 511 * 64 && R <= nb::kMaxGridX, "%s: bad shape R=%lld C=%lld", who, (long long)R,
+               (long long)C);
+    NB_REQUIRE_PTR(stats);
+    NB_REQUIRE_PTR(row_sums);
+    NB_REQUIRE_PTR(law);
+    NB_REQUIRE_PTR(table);
+    NB_REQUIRE_ALIGNED(stats, 8);
+    NB_REQUIRE_ALIGNED(row_sums, 4);
+    NB_REQUIRE_ALIGNED(law, 2);
+    NB_REQUIRE_ALIGNED(table, 4);
+    nb::law_row_sums_kernel<<<dim3((unsigned)R), dim3(256), 0, nb::as_stream(stream)>>>(row_sums, law, (int)C);
+    if (int rc = nb::check_launch(who)) return rc;
+    nb::law_stats_kernel<<<dim3(1), dim3(256), 0, nb::as_stream(stream)>>>(stats, row_sums, table, R, (int)C);
     return nb::check_launch(who);
 }
 

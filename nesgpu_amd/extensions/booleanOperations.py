@@ -1096,6 +1096,18 @@ class FlipLaw:
             self._layers = (pl, cls)
         return self._layers
 
+    def stats(self):
+        """(mean flip probability of the layer, largest mean of a row, largest flip probability): two small kernels
+        and ONE device read-back."""
+        R, C = self.law.shape
+        out = torch.empty((3,), dtype=torch.float64, device=self.law.device)
+        rows = torch.empty((R,), dtype=torch.float32, device=self.law.device)
+        with _on(self.law):
+            _lib.call("nb_flip_law_stats", out.data_ptr(), rows.data_ptr(), self.law.data_ptr(), self.table.data_ptr(),
+                      R, C, _stream(self.law))
+        mean, row, peak = out.tolist()
+        return mean, row, peak
+
     def max_flip_probability(self):
         """The largest flip probability of the layer (a device read-back)."""
         return float(self.table[2:3].view(torch.int32).to(torch.int64).item() & 0xFFFFFFFF) / 4294967296.0

@@ -230,6 +230,9 @@ class BinarizedLinear(Binarized):
         # per-element laws in the sparse form: "thin" (one walk at the largest probability), "layered" (class by class)
         # or "auto" (whichever takes fewer steps)
         self.sparse_walk = "auto"
+        # sparse="auto": how many versions of the weights a clearly dense law (mean flip probability of 0.06 or more)
+        # stands before it is looked at again; 1: every version
+        self.sparse_recheck = 8
         if pack_output and not threshold:
             raise NotImplementedError("packed output needs threshold=True")
         self.pack_output = pack_output    # not in the reference: return the thresholded row packed, from one kernel
@@ -254,9 +257,8 @@ class BinarizedLinear(Binarized):
                 p = min(self.flip_probability, 1.0 - self.flip_probability)
                 return dict(law=None, mean=p, peak=p, row=p)
             law = booleanOperations.flip_law_from_weights(self.weight)
-            y = (law.law.view(torch.int16) & 0x7FFF).view(torch.float16).float()
-            stats = torch.stack([y.mean(), y.mean(dim=1).max()]).tolist()          # the one read-back
-            return dict(law=law, mean=stats[0], peak=law.max_flip_probability(), row=stats[1])
+            mean, row, peak = law.stats()                                           # the one read-back
+            return dict(law=law, mean=mean, peak=peak, row=row)
         return self._cached("sparse_plan", self.weight, make)
 
     def _sparse_now(self):
@@ -269,10 +271,25 @@ class BinarizedLinear(Binarized):
             return True
         if self.in_features < 2048:
             return False
+        if self.flip_probability is None:
+            # a law that was far from sparse is not looked at again for the next sparse_recheck - 1 versions of the
+            # weights (looking costs a few kernels and a read-back per version; staying dense a few steps too long
+            # costs nothing but time)
+            tag = (self.weight._version, self.weight.data_ptr())
+            wait = self._cache.get("dense_for")
+            if wait is not None and wait[0] != tag and wait[1] > 1:
+                self._cache["dense_for"] = (tag, wait[1] - 1)
+                return False
+            if wait is not None and wait[0] == tag:
+                return False
         plan = self._sparse_plan()
         # a row's lists cost a few steps per flip where the dense sampler draws every bit: worth it below about one
         # flip in twenty-five bits, whatever the largest probability (a law with a long tail is walked class by class)
-        return plan["mean"] <= 0.04
+        sparse = plan["mean"] <= 0.04
+        self._cache.pop("dense_for", None)
+        if not sparse and plan["mean"] >= 0.06 and self.sparse_recheck > 1 and self.flip_probability is None:
+            self._cache["dense_for"] = ((self.weight._version, self.weight.data_ptr()), self.sparse_recheck)
+        return sparse
 
     def _sample_sparse(self):
         plan = self._sparse_plan()

@@ -117,6 +117,8 @@ def test_bad_arguments_are_rejected_without_a_launch(lib):
     assert lib.nb_flip_law_layers(one, one, one, 4, 512 * 64, None) == 2
     assert lib.nb_flip_law_layers(None, None, None, 0, 64, None) == 0
     assert lib.nb_flip_layer_tables(None, None) == 1
+    assert lib.nb_flip_law_stats(one, one, one, None, 4, 64, None) == 1
+    assert lib.nb_flip_law_stats(one, one, one, one, 0, 64, None) == 2
     assert lib.nb_flip_layer_table_words() == 16 * 4100
     assert lib.nb_flip_law_from_weights(one, one, None, one, 4, 64, one, None) == 1
     assert lib.nb_thresholds_from_weights(one, one, 4, ctypes.c_void_p(4), None) == 3

@@ -326,6 +326,21 @@ def test_thinning_sampler_vs_oracle(ops, oracle, D, R, C, first, spread):
         np.testing.assert_array_equal(bflag, mask & bb[None])
 
 
+def test_law_statistics_in_one_read_back(ops, oracle):
+    """FlipLaw.stats(): mean / largest row mean / largest flip probability of the law the library made from latent
+    weights, against numpy on the law read back."""
+    g = torch.Generator(device="cuda")
+    g.manual_seed(12)
+    for R, C in ((16, 2048), (70, 333), (1, 64), (1024, 8192)):
+        w = (torch.randn((R, C), device="cuda", generator=g) * (0.2 + torch.rand((R, 1), device="cuda", generator=g))).half()
+        law = ops.flip_law_from_weights(w)
+        y = (host(law.law.view(torch.int16)).view(np.uint16) & 0x7FFF).view(np.float16).astype(np.float64)
+        mean, row, peak = law.stats()
+        assert abs(mean - y.mean()) <= 1e-6 * y.mean() + 1e-12
+        assert abs(row - y.mean(axis=1).max()) <= 1e-5 * row
+        assert peak == float(np.floor(y.max() * 2.0 ** 32)) / 2.0 ** 32 == law.max_flip_probability()
+
+
 def long_tailed_law(g, R, C, mean):
     """fp16 probabilities whose flip probabilities span five orders of magnitude, a few of them near 1/2."""
     y = mean * 0.3 * 10.0 ** (g.random((R, C)) * 1.0)

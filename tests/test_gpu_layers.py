@@ -465,6 +465,7 @@ def test_sparse_form_is_chosen_by_the_flip_probabilities(binary):
     g = torch.Generator(device="cuda")
     g.manual_seed(3)
     lin = binary.BinarizedLinear(2048, 16, 8)
+    lin.sparse_recheck = 1                                   # look at the law at every version of the weights
     lin.set_seed(1)
     lin.set_noise()                                          # zero latent weights: every probability 1/2
     assert isinstance(lin.weight_noise, torch.Tensor) and tuple(lin.weight_noise.shape) == (8, 16, 32)
@@ -485,6 +486,18 @@ def test_sparse_form_is_chosen_by_the_flip_probabilities(binary):
         lin.weight[:, ::4] *= 0.125                          # a quarter of the weights near 1/2: too many flips
     lin.set_noise()
     assert isinstance(lin.weight_noise, torch.Tensor)
+    # a clearly dense law stands for sparse_recheck versions of the weights before it is looked at again
+    slow = binary.BinarizedLinear(2048, 16, 8)
+    assert slow.sparse_recheck == 8
+    slow.set_seed(1)
+    slow.set_noise()
+    assert isinstance(slow.weight_noise, torch.Tensor) and "sparse_plan" in slow._cache
+    for version in range(1, 9):
+        with torch.no_grad():
+            slow.weight.copy_(_saturated((16, 2048), g))
+        slow.set_noise()
+        slow.set_noise()                                     # the same version again: counted once
+        assert isinstance(slow.weight_noise, ops.FlipRows) == (version == 8), version
     narrow = binary.BinarizedLinear(1024, 16, 8)
     with torch.no_grad():
         narrow.weight.copy_(_saturated((16, 1024), g))
