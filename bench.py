@@ -610,6 +610,25 @@ def main():
             "set_noise_ms": round(time_steps(torch, sn, reps, 2)[0] * 1e3, 4),
             "forward_ms": round(time_steps(torch, fw, reps, 2)[0] * 1e3, 4),
             "update_ms": round(time_steps(torch, up, reps, 2)[0] * 1e3, 4)}
+        # the three phases in a loop that changes the weights every step (plain SGD on the estimated gradients), so
+        # that whatever a layer keeps per version of its weights is made anew every step
+        from nesgpu_amd.modules import binary as _binary
+        _mods = [m for m in fw.model.modules() if isinstance(m, _binary.Binarized)]
+        _opt = torch.optim.SGD(fw.model.parameters(), lr=1e-3)
+        _count = [0]
+
+        def loop_step():
+            _count[0] += 1
+            for j, m in enumerate(_mods):
+                m.set_seed(1000 * _count[0] + j)
+            sn()
+            fw()
+            up()
+            _opt.step()
+        line["nes_step_smallnet"]["training_loop_ms_per_step"] = round(time_steps(torch, loop_step, reps, 3)[0] * 1e3, 4)
+        line["nes_step_smallnet"]["training_loop_note"] = ("set_seed, set_noise, forward, update and torch's SGD step, "
+                                                          "new weights every step")
+        del _opt, _mods
         if not args.no_graph:
             fg = time_graph(torch, fw, reps)                 # the same forward without the host's launch pacing
             if fg:
