@@ -818,8 +818,9 @@ __global__ __launch_bounds__(1024) void fl_gen_layered_kernel(const LayerArgs a)
         const uint32_t left = from < kLayers ? nonempty >> from : 0u;
         cur = left ? from + (int)__builtin_ctz(left) : kLayers;
         const int c = cur < kLayers ? cur : 0;
-        startk = (int)mycl[c];
-        nk = (int)mycl[c + 1] - startk;
+        // (class starts beyond the row, which only a caller's own faulty sort can hold, end the class at once)
+        startk = (int)(mycl[c] < (uint32_t)a.C ? mycl[c] : (uint32_t)a.C);
+        nk = (int)(mycl[c + 1] < (uint32_t)a.C ? mycl[c + 1] : (uint32_t)a.C) - startk;
         kt = kts[c];
         hint = hints[c];
         tab1 = tabs + c * kLayerStride;
