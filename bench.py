@@ -436,6 +436,9 @@ def hbm_kernels(torch, steps, warmup, graph=True, core=False):
         lambda: ops.bmv_flip_act_pack(rows, x4, thr4, G=G), rows.nbytes() + G.numel() * 4 + thr4.numel() * 4 + x4.numel() * 8)
     run("flip_rows_skip D=4096 [1024 x 8192], p=0.01 (bytes written)",
         lambda: ops.flip_rows_skip(b4, 8192, 4096, workloads.T_P01, 0, subsequence=13), rows.nbytes())
+    fit4 = torch.randn(4096, device=dev, generator=g).half()
+    run("weighted_sum over the flip lists D=4096 [1024 x 8192], p=0.01 (lists + row info + fp16 out)",
+        lambda: ops.weighted_sum(rows, fit4, 8192), rows.nbytes() + 1024 * 8192 * 2)
     del rows, x4, thr4, ex, G
     # the same layer's lists under the per-element law of latent weights whose magnitudes spread by 10 % (flip
     # probabilities of 0.8 % on average, 8 % at most): one walk at the largest probability against class by class

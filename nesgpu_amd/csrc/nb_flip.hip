@@ -418,15 +418,17 @@ __global__ __launch_bounds__(1024) void fl_bmv_kernel(void *__restrict__ out, co
 // room: 64 bytes of every piece, whole sectors) and keeps their columns' sums in LDS as 32-bit fixed-point integers
 // (weights scaled by a power of two chosen from sum |w[d]|, so that no sum can overflow, populations below 2^30
 // members: integer adds commute, the result does not depend on the order in which the members arrive);
-// lane = (row, member), 64 / RB members per wave and step; a lane asks for its next piece before it adds the current.
+// lane = (row, member), 64 / RB members per wave and step; a lane asks for four pieces at a time, the next four
+// before it adds the current ones.  Bound by how the lists are read (64-byte halves of lines a kilobyte apart).
 __global__ __launch_bounds__(1024) void fl_wsum_kernel(_Float16 *__restrict__ out, const uint32_t *__restrict__ entries,
                                                        const uint32_t *__restrict__ info,
                                                        const uint64_t *__restrict__ base,
                                                        const _Float16 *__restrict__ wts, int64_t D, int64_t R, int C,
                                                        int Kw, int S, int cap, int RB)
 {
-    extern __shared__ int32_t fl_ws_acc[];  // [RB][64 * Kw] column sums, then 16 x 8 bytes of scratch
+    extern __shared__ int32_t fl_ws_acc[];  // [RB][64 * Kw] column sums, 16 x 8 bytes of scratch, 64 spare words
     float *red = reinterpret_cast<float *>(fl_ws_acc + RB * 64 * Kw);
+    int32_t *spare = fl_ws_acc + RB * 64 * Kw + 32 + (threadIdx.x & 63);   // after the scratch: a word per lane
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int cols = 64 * Kw;
     for (int i = tid; i < RB * cols; i += 1024) fl_ws_acc[i] = 0;
@@ -445,32 +447,62 @@ __global__ __launch_bounds__(1024) void fl_wsum_kernel(_Float16 *__restrict__ ou
     (void)frexpf(A + 1.0f, &ex);  // A + 1 < 2^ex
     const int k = 29 - ex;
     const float scale = ldexpf(1.0f, k), inv_scale = ldexpf(1.0f, -k);
+    // Workgroups go round the eight XCDs in turn; the 64 / RB workgroups that share a slice of 64 rows (their rows'
+    // pieces lie next to each other, two workgroups to a 128-byte line) should share an L2: XCD x takes a contiguous
+    // eighth of the row groups.
+    int bid = (int)blockIdx.x;
+    if ((gridDim.x & 7u) == 0) bid = (bid & 7) * (int)(gridDim.x >> 3) + (bid >> 3);
     const int row = lane & (RB - 1);
-    const int64_t r = (int64_t)blockIdx.x * RB + row;
+    const int64_t r = (int64_t)bid * RB + row;
     const bool rvalid = r < R;
     const int s = (int)(r >> 6), l = (int)(r & 63);
     int32_t *acc = fl_ws_acc + row * cols;
     const uint32_t npieces = (uint32_t)(4 * Kw);
     long long total = 0;  // sum of the scaled weights (this lane's members)
     const int per_wave = 64 / RB, shift = RB == 4 ? 2 : (RB == 2 ? 1 : 0);
-    for (int64_t d = (int64_t)wave * per_wave + (lane >> shift); d < D; d += 16 * per_wave) {
+    // Four pieces of a row are asked for together and the next four while those are added (a lane with one request in
+    // flight leaves the memory system idle: 16 KB per compute unit); the next member's row info comes a member ahead.
+    // Plain loads, not streaming ones: a 128-byte line holds a piece of eight rows, i.e. of two workgroups, and should
+    // stay in L2 until the second has read its half.
+    constexpr int U = 4;
+    const int64_t dstep = 16 * per_wave;
+    int64_t d = (int64_t)wave * per_wave + (lane >> shift);
+    uint32_t inf = (rvalid && d < D) ? info[d * R + r] : 0u;
+    for (; d < D; d += dstep) {
+        const uint32_t inf_next = (rvalid && d + dstep < D) ? info[(d + dstep) * R + r] : 0u;
         const int wq = (int)rintf((float)wts[d] * scale);
         if (row == 0) total += wq;
-        if (!rvalid) continue;
-        int pieces = (int)(info[d * R + r] >> 16);
+        int pieces = (int)(inf >> 16);
         pieces = pieces < cap ? pieces : cap;
+        inf = inf_next;
+        if (!rvalid) continue;
         const uint4 *src = reinterpret_cast<const uint4 *>(entries) + (d * S + s) * (int64_t)cap * 64 + l;
-        uint4 nxt = make_uint4(0u, 0u, 0u, 0u);
-        if (pieces > 0) nxt = load_stream16(src);
-        for (int j = 0; j < pieces; j++) {
-            const uint4 q = nxt;
-            if (j + 1 < pieces) nxt = load_stream16(src + (int64_t)(j + 1) * 64);
-            const uint32_t e[4] = {q.x, q.y, q.z, q.w};
+        uint4 cur[U], nxt[U];
 #pragma unroll
-            for (int h = 0; h < 8; h++) {
-                const uint32_t v = (h & 1) ? e[h >> 1] >> 16 : e[h >> 1] & 0xFFFFu;
-                const uint32_t piece = v >> 5;
-                if (piece < npieces) atomicAdd(acc + (piece >> 1) * 32 + (v & 31u), (piece & 1u) ? -wq : wq);
+        for (int u = 0; u < U; u++) {
+            cur[u] = make_uint4(0u, 0u, 0u, 0u);
+            if (u < pieces) cur[u] = src[(int64_t)u * 64];
+        }
+        for (int j0 = 0; j0 < pieces; j0 += U) {
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                nxt[u] = make_uint4(0u, 0u, 0u, 0u);
+                if (j0 + U + u < pieces) nxt[u] = src[(int64_t)(j0 + U + u) * 64];
+            }
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                if (j0 + u < pieces) {
+                    const uint32_t e[4] = {cur[u].x, cur[u].y, cur[u].z, cur[u].w};
+#pragma unroll
+                    for (int h = 0; h < 8; h++) {
+                        // no branch per entry: a sentinel adds zero to a word of the lane's own
+                        const uint32_t v = (h & 1) ? e[h >> 1] >> 16 : e[h >> 1] & 0xFFFFu;
+                        const bool flip = (v >> 5) < npieces;
+                        const uint32_t col = ((v >> 1) & 0xFFE0u) | (v & 31u);   // 32 * (piece / 2) + bit
+                        atomicAdd(flip ? acc + col : spare, flip ? ((v & 32u) ? -wq : wq) : 0);
+                    }
+                }
+                cur[u] = nxt[u];
             }
         }
     }
@@ -486,7 +518,7 @@ __global__ __launch_bounds__(1024) void fl_wsum_kernel(_Float16 *__restrict__ ou
     for (int w = 0; w < 16; w++) F += tred[w];
     for (int i = tid; i < RB * C; i += 1024) {
         const int rr = i / C, c = i - rr * C;
-        const int64_t ro = (int64_t)blockIdx.x * RB + rr;
+        const int64_t ro = (int64_t)bid * RB + rr;
         if (ro < R) {
             const long long b = (long long)((base[ro * Kw + (c >> 6)] >> (c & 63)) & 1ull);
             out[ro * C + c] = (_Float16)((float)(b * F + (long long)fl_ws_acc[rr * cols + c]) * inv_scale);
@@ -682,8 +714,8 @@ int nb_flip_weighted_sum_i64(uint16_t *out, const uint32_t *entries, const uint3
     NB_REQUIRE_ALIGNED(weights, 2);
     // rows per workgroup: as many of 4, 2, 1 as LDS (160 KB per workgroup on this part) holds
     int RB = 4;
-    while (RB > 1 && (size_t)RB * 64 * Kw * 4 + 128 > 150 * 1024) RB >>= 1;
-    const size_t lds = (size_t)RB * 64 * Kw * 4 + 128;
+    while (RB > 1 && (size_t)RB * 64 * Kw * 4 + 384 > 150 * 1024) RB >>= 1;
+    const size_t lds = (size_t)RB * 64 * Kw * 4 + 384;   // sums, 128 bytes of scratch, a spare word per lane
     static std::once_flag once;
     static hipError_t attr = hipSuccess;
     std::call_once(once, [] {
