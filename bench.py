@@ -213,11 +213,17 @@ def extend_entry(torch, args, cfg, w, entry, steps):
         pg = None if args.no_graph else time_graph(torch, step, n)
         sw, se = time_steps(torch, set_noise, 5, 2)
         fc = model.perturbed_layers[3].weight_noise
+        fitness = torch.randn(model.directions, device=fc.device)
+
+        def update():
+            for layer in model.perturbed_layers:
+                layer.update(fitness)
+        uw, ue = time_steps(torch, update, 5, 2)
         entry["layer_api"] = {
             "workload": "the same network from BinarizedConv2d / BinarizedMaxPool2d / BinarizedLinear "
                         "(flip_probability=0.01) through PerturbedModel, fuse_packed_outputs",
             "ms_per_step": round(pw * 1e3, 4), "ms_per_step_graph": round(pg * 1e3, 4) if pg else None,
-            "set_noise_ms": round(sw * 1e3, 4),
+            "set_noise_ms": round(sw * 1e3, 4), "update_ms": round(uw * 1e3, 4),
             "fc_8192_1024": type(fc).__name__,
             "ratio_to_ops_level": round(pw * 1e3 / entry["ms_per_step"], 3)}
         del model, step, set_noise
