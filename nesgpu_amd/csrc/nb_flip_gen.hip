@@ -404,7 +404,7 @@ __device__ __forceinline__ void skip_table_build(uint32_t *table, const uint32_t
 // P = fp16(sigmoid(float(fp16(fp16(w / m) * 5)))) with m = fp16(mean|w| + 1e-5), every step rounded to fp16 where the
 // tensor expression of modules/binary.py:59-60 rounds it.  mean|w| is the exact sum (fp16 values add exactly in a
 // double) divided by the count and rounded once to fp16.
-constexpr int kLawBlocks = 256;   // doubles of workspace: up to 255 partial sums, then the denominator
+constexpr int kLawBlocks = 256;   // partial sums (doubles of workspace)
 
 __global__ __launch_bounds__(256) void law_abs_sum_kernel(double *__restrict__ partial, uint32_t *__restrict__ table,
                                                           const _Float16 *__restrict__ w, int64_t n)
@@ -437,23 +437,22 @@ __global__ __launch_bounds__(256) void law_abs_sum_kernel(double *__restrict__ p
     }
 }
 
-// The partial sums added in index order, by one thread, into the denominator fp16(mean|w| + 1e-5); it is left in the
-// workspace's last slot (as a double: exact) for the kernels that follow.
-__global__ __launch_bounds__(256) void law_denominator_kernel(double *partial, int nparts, int64_t n)
+// The denominator fp16(mean|w| + 1e-5), made by every workgroup for itself: the partial sums are fetched by as many
+// threads, added in index order by one (the same additions in every workgroup: all agree), and handed round in LDS.
+__device__ __forceinline__ _Float16 law_denominator(const double *partial, int nparts, int64_t n)
 {
     __shared__ double part[kLawBlocks];
-    part[threadIdx.x] = (int)threadIdx.x < nparts ? partial[threadIdx.x] : 0.0;
+    __shared__ float denom_sh;
+    for (int i = threadIdx.x; i < nparts; i += blockDim.x) part[i] = partial[i];
     __syncthreads();
-    if (threadIdx.x != 0) return;
-    double s = 0.0;
-    for (int i = 0; i < nparts; i++) s += part[i];
-    const _Float16 mean = double_round_once_fp16(s / (double)n);
-    partial[kLawBlocks - 1] = (double)(float)(_Float16)((float)mean + 1e-5f);
-}
-
-__device__ __forceinline__ _Float16 law_denominator(const double *partial)
-{
-    return (_Float16)(float)partial[kLawBlocks - 1];
+    if (threadIdx.x == 0) {
+        double s = 0.0;
+        for (int i = 0; i < nparts; i++) s += part[i];
+        const _Float16 mean = double_round_once_fp16(s / (double)n);
+        denom_sh = (float)(_Float16)((float)mean + 1e-5f);
+    }
+    __syncthreads();
+    return (_Float16)denom_sh;
 }
 
 __device__ __forceinline__ _Float16 law_probability(_Float16 w, _Float16 denom)
@@ -473,9 +472,9 @@ __device__ __forceinline__ uint32_t law_threshold(_Float16 p)   // min(floor(p *
 template <int MODE>
 __global__ __launch_bounds__(256) void law_dense_kernel(uint32_t *__restrict__ out32, _Float16 *__restrict__ out16,
                                                         const _Float16 *__restrict__ w, const double *__restrict__ partial,
-                                                        int64_t n)
+                                                        int nparts, int64_t n)
 {
-    const _Float16 denom = law_denominator(partial);
+    const _Float16 denom = law_denominator(partial, nparts, n);
     NB_FLAT_LOOP(t, n)
     {
         if (t < n) {
@@ -491,10 +490,10 @@ __global__ __launch_bounds__(256) void law_dense_kernel(uint32_t *__restrict__ o
 // kernel).  One wave per 64 columns of a row: the ballot of the base bits is the packed word.
 __global__ __launch_bounds__(256) void law_sparse_kernel(uint16_t *__restrict__ law, uint64_t *__restrict__ base,
                                                          uint32_t *__restrict__ table, const _Float16 *__restrict__ w,
-                                                         const double *__restrict__ partial, int64_t R,
+                                                         const double *__restrict__ partial, int nparts, int64_t R,
                                                          int C, int Kw)
 {
-    const _Float16 denom = law_denominator(partial);
+    const _Float16 denom = law_denominator(partial, nparts, R * (int64_t)C);
     const int lane = threadIdx.x & 63;
     uint32_t tmax = 0;
     for (int64_t wd = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6); wd < R * Kw; wd += (int64_t)gridDim.x * 4) {
@@ -1329,11 +1328,9 @@ static int law_sum(double *ws, uint32_t *table, const uint16_t *w, int64_t n, hi
     NB_REQUIRE_ALIGNED(ws, 8);
     NB_REQUIRE_PTR(w);
     NB_REQUIRE_ALIGNED(w, 2);
-    const int64_t blocks = std::min<int64_t>(nb::kLawBlocks - 1, nb::ceil_div(n, 2048));
+    const int64_t blocks = std::min<int64_t>(nb::kLawBlocks, nb::ceil_div(n, 2048));
     *nparts = (int)blocks;
     nb::law_abs_sum_kernel<<<dim3((unsigned)blocks), dim3(256), 0, s>>>(ws, table, reinterpret_cast<const _Float16 *>(w), n);
-    if (int rc = nb::check_launch(who)) return rc;
-    nb::law_denominator_kernel<<<dim3(1), dim3(nb::kLawBlocks), 0, s>>>(ws, (int)blocks, n);
     return nb::check_launch(who);
 }
 
@@ -1349,7 +1346,7 @@ int nb_thresholds_from_weights(uint32_t *thresholds, const uint16_t *weights, in
     if (int rc = law_sum(static_cast<double *>(workspace), nullptr, weights, n, nb::as_stream(stream), &nparts, who))
         return rc;
     nb::law_dense_kernel<0><<<dim3(nb::grid_for(n)), dim3(256), 0, nb::as_stream(stream)>>>(
-        thresholds, nullptr, reinterpret_cast<const _Float16 *>(weights), static_cast<const double *>(workspace), n);
+        thresholds, nullptr, reinterpret_cast<const _Float16 *>(weights), static_cast<const double *>(workspace), nparts, n);
     return nb::check_launch(who);
 }
 
@@ -1365,7 +1362,7 @@ int nb_probabilities_from_weights(uint16_t *p, const uint16_t *weights, int64_t 
         return rc;
     nb::law_dense_kernel<1><<<dim3(nb::grid_for(n)), dim3(256), 0, nb::as_stream(stream)>>>(
         nullptr, reinterpret_cast<_Float16 *>(p), reinterpret_cast<const _Float16 *>(weights),
-        static_cast<const double *>(workspace), n);
+        static_cast<const double *>(workspace), nparts, n);
     return nb::check_launch(who);
 }
 
@@ -1409,7 +1406,7 @@ int nb_flip_law_from_weights(uint16_t *law, int64_t *base, uint32_t *table, cons
     const int64_t blocks = std::min<int64_t>(nb::ceil_div(R * Kw, 4), 2048);
     nb::law_sparse_kernel<<<dim3((unsigned)blocks), dim3(256), 0, nb::as_stream(stream)>>>(
         law, reinterpret_cast<uint64_t *>(base), table, reinterpret_cast<const _Float16 *>(weights),
-        static_cast<const double *>(workspace), R, (int)C, (int)Kw);
+        static_cast<const double *>(workspace), nparts, R, (int)C, (int)Kw);
     if (int rc = nb::check_launch(who)) return rc;
     nb::fl_skip_table_kernel<<<dim3(1), dim3(1024), 0, nb::as_stream(stream)>>>(table, table + 2);
     return nb::check_launch(who);

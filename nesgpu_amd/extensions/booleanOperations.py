@@ -1123,7 +1123,7 @@ def _law_workspace(device):
 
 def thresholds_from_weights(weight):
     """Latent fp16 weights -> uint32 sampler thresholds of P = sigmoid(5 w / (mean|w| + 1e-5)) (modules/binary.py:59-60):
-    the tensor expression's roundings, in three small kernels (the sum of |w|, its rounding into the denominator, the law) instead of nine."""
+    the tensor expression's roundings, in two small kernels (partial sums of |w|, the law) instead of nine."""
     w = weight.detach()
     _check(w, "weight")
     assert w.dtype == torch.float16
@@ -1149,7 +1149,7 @@ def probabilities_from_weights(weight):
 def flip_law_from_weights(weight):
     """Latent fp16 weights [R, C] -> :class:`FlipLaw` of P = sigmoid(5 w / (mean|w| + 1e-5)): base bit = P >= 1/2,
     flip probability min(P, 1 - P), and the skip sampler's table for the layer's largest flip probability, all made
-    on the device (four kernels, nothing read back)."""
+    on the device (three kernels, nothing read back)."""
     w = weight.detach()
     _check(w, "weight")
     assert w.dtype == torch.float16 and len(w.shape) == 2

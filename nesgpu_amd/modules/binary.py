@@ -91,7 +91,7 @@ class Binarized(Perturbed, nn.Module):
 
     def probabilities(self):
         """fp16 [rows, in_degree] per-bit probabilities of a 1 (modules/binary.py:59-60): the tensor expression
-        ``sigmoid((w / (w.abs().mean() + 1e-5) * 5).float()).half()`` with its roundings, in three small kernels (the mean of
+        ``sigmoid((w / (w.abs().mean() + 1e-5) * 5).float()).half()`` with its roundings, in two small kernels (the mean of
         |w| is the exact one rounded once to fp16, where torch's adds in fp32 in its own order).  With
         ``flip_probability`` p: 1 - p where the latent weight is >= 0, p elsewhere."""
         with torch.no_grad():
